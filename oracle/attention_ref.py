@@ -1,0 +1,360 @@
+"""numpy restatement of the CudaDnnDLL primitives and the C# attention layers.
+
+TEST INFRASTRUCTURE ONLY (parity checker).  Every function names the reference
+routine whose index arithmetic / call order it follows; paths are relative to
+the reference tree.  ``dtype`` selects the arithmetic type (float32 mirrors the
+reference's ``Kernel<float>``, float64 gives a tighter mathematical reference).
+
+Pins (tests/test_oracle_layers.py): the inline vectors of
+MyCaffe.test/TestCudaDnn.cs (gemm, gemv, mask, mask_batch, channel_copy), the
+``gpt-pico-csa*`` golden tensors held by the reference test data (q after
+transpose, softmax probabilities, y), scipy/torch library routines (softmax,
+scaled_dot_product_attention) and closed forms (RoPE as a complex rotation).
+"""
+import numpy as np
+
+MASKED = -1e29  # CausalSelfAttentionLayer.cs:60, attn.cu:307,324
+
+
+# ----------------------------------------------------------------------------
+# BLAS-like primitives
+# ----------------------------------------------------------------------------
+
+def gemm(transA, transB, m, n, k, alpha, A, B, beta, C=None, dtype=np.float32):
+    """Row-major C[m,n] = alpha*op(A)*op(B) + beta*C.
+
+    CudaDnnDLL/Cuda Files/math.cu:1481-1505: A is stored (m,k) or, transposed,
+    (k,m); B is stored (k,n) or, transposed, (n,k).
+    """
+    A = np.asarray(A, dtype).reshape(-1)
+    B = np.asarray(B, dtype).reshape(-1)
+    a = A[:m * k].reshape((k, m)).T if transA else A[:m * k].reshape((m, k))
+    b = B[:k * n].reshape((n, k)).T if transB else B[:k * n].reshape((k, n))
+    out = dtype(alpha) * (a @ b)
+    if beta != 0:
+        out = out + dtype(beta) * np.asarray(C, dtype).reshape(-1)[:m * n].reshape(m, n)
+    return out.astype(dtype)
+
+
+def gemv(transA, m, n, alpha, A, x, beta, y=None, dtype=np.float32):
+    """A is row-major (m,n); y = alpha*A*x + beta*y, or with transA y = alpha*A^T*x.
+
+    math.cu:2101-2121 (cublasSgemv with the operation flag inverted because the
+    row-major matrix is a column-major (n,m) matrix).
+    """
+    a = np.asarray(A, dtype).reshape(-1)[:m * n].reshape(m, n)
+    xv = np.asarray(x, dtype).reshape(-1)
+    out = dtype(alpha) * ((a.T @ xv[:m]) if transA else (a @ xv[:n]))
+    if beta != 0:
+        out = out + dtype(beta) * np.asarray(y, dtype).reshape(-1)[:out.size]
+    return out.astype(dtype)
+
+
+def gemm2_colmajor(transA, transB, m, n, k, alpha, A, B, beta, C, lda, ldb, ldc,
+                   strideA=0, strideB=0, strideC=0, batch=1, dtype=np.float32):
+    """cublasSgemmStridedBatched semantics on flat buffers (math.cu:1750-1788).
+
+    Column-major: op(A) is (m,k), op(B) is (k,n), C is (m,n) with leading
+    dimensions lda/ldb/ldc.  Returns the updated flat C.
+    """
+    A = np.asarray(A, dtype).reshape(-1)
+    B = np.asarray(B, dtype).reshape(-1)
+    C = np.array(C, dtype, copy=True).reshape(-1)
+
+    def colview(buf, off, rows, cols, ld):
+        idx = off + np.arange(rows)[:, None] + ld * np.arange(cols)[None, :]
+        return idx
+
+    for b in range(batch):
+        ar, ac = (k, m) if transA else (m, k)
+        br, bc = (n, k) if transB else (k, n)
+        a = A[colview(A, b * strideA, ar, ac, lda)]
+        bb = B[colview(B, b * strideB, br, bc, ldb)]
+        a = a.T if transA else a
+        bb = bb.T if transB else bb
+        ci = colview(C, b * strideC, m, n, ldc)
+        C[ci] = dtype(alpha) * (a @ bb) + (dtype(beta) * C[ci] if beta != 0 else 0)
+    return C
+
+
+def matmul(outer, m, n, k, A, B, scale=1.0, transA=False, transB=False, dtype=np.float32):
+    """Row-major batched C[outer,m,n] = scale * op(A) @ op(B).
+
+    MyCaffe/common/CudaDnn.cs:7513-7524: implemented by the host as a
+    column-major gemm2 with the operands swapped.
+    """
+    lda = m if transA else k
+    ldb = k if transB else n
+    C = np.zeros(outer * m * n, dtype)
+    C = gemm2_colmajor(transB, transA, n, m, k, scale, B, A, 0.0, C, ldb, lda, n,
+                       k * n, m * k, m * n, outer, dtype=dtype)
+    return C.reshape(outer, m, n)
+
+
+def mask(n, mask_dim, search, replace, x, msk, dtype=np.float32):
+    """y[i] = replace if mask[i % mask_dim] == search else x[i] (math.cu:2995-3002)."""
+    x = np.asarray(x, dtype).reshape(-1)[:n]
+    msk = np.asarray(msk, dtype).reshape(-1)
+    idx = np.arange(n) % mask_dim
+    return np.where(msk[idx] == dtype(search), dtype(replace), x).astype(dtype)
+
+
+def mask_batch(n, batch, mask_dim, search, replace, x, msk, dtype=np.float32):
+    """math.cu:3046-3056: mask index = i % (mask_dim/batch) + (i / (n/batch)) * (mask_dim/batch)."""
+    x = np.asarray(x, dtype).reshape(-1)[:n]
+    msk = np.asarray(msk, dtype).reshape(-1)
+    md1 = mask_dim // batch
+    dd1 = n // batch
+    i = np.arange(n)
+    idx = i % md1 + (i // dd1) * md1
+    return np.where(msk[idx] == dtype(search), dtype(replace), x).astype(dtype)
+
+
+def channel_copy_fwd(count, num, channels, blocks, inner, offset, x, dtype=np.float32):
+    """Y[n,c,:] = X[n,c,offset,:] for X of shape (num, channels, blocks, inner) (math.cu:7510-7523)."""
+    x = np.asarray(x, dtype).reshape(-1)
+    i = np.arange(count)
+    nn = i // (channels * inner)
+    c = (i % (channels * inner)) // inner
+    b = i % inner
+    src = nn * channels * blocks * inner + c * blocks * inner + offset * inner + b
+    return x[src].astype(dtype)
+
+
+def channel_copy_bwd(count, num, channels, blocks, inner, offset, x, y, dtype=np.float32):
+    """X[n,c,offset,:] = Y[n,c,:] (math.cu:7525-7539); returns the updated flat X."""
+    x = np.array(x, dtype, copy=True).reshape(-1)
+    y = np.asarray(y, dtype).reshape(-1)
+    i = np.arange(count)
+    nn = i // (channels * inner)
+    c = (i % (channels * inner)) // inner
+    b = i % inner
+    dst = nn * channels * blocks * inner + c * blocks * inner + offset * inner + b
+    x[dst] = y[:count]
+    return x
+
+
+def transpose(x, x_strides, y_strides, mapping, dtype=np.float32):
+    """Generic permute of math.cu:4545-4571.
+
+    ``x_strides[i]``/``y_strides[i]`` are the element strides of axis i of the
+    source / destination (what the host passes as the "counts" blobs) and
+    ``mapping[i]`` is the source axis that becomes destination axis i.
+    """
+    x = np.asarray(x, dtype).reshape(-1)
+    n = x.size
+    y = np.zeros(n, dtype)
+    idx = np.arange(n)
+    rem = idx.copy()
+    from_inds = []
+    for s in x_strides:
+        from_inds.append(rem // int(s))
+        rem = rem % int(s)
+    to = np.zeros(n, np.int64)
+    for i, s in enumerate(y_strides):
+        to += from_inds[int(mapping[i])] * int(s)
+    y[to] = x[idx]
+    return y
+
+
+def transpose_hw(n, c, h, w, x, dtype=np.float32):
+    """(n,c,h,w) -> (n,c,w,h) (math.cu:4618-4654)."""
+    return np.asarray(x, dtype).reshape(n * c, h, w).transpose(0, 2, 1).copy().reshape(-1)
+
+
+def softmax_lastaxis(x, dtype=np.float32):
+    """Max-subtracted softmax over the last axis (cudnnSoftmaxForward ACCURATE,
+    memory.cu:2266-2288; CAFFE-engine chain SoftmaxLayer.cs:230-273)."""
+    x = np.asarray(x, dtype)
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return (e / e.sum(axis=-1, keepdims=True)).astype(dtype)
+
+
+def silu(x, dtype=np.float32):
+    """x * sigmoid(x) (math.cu:11699-11707)."""
+    x = np.asarray(x, dtype)
+    return (x * (dtype(1) / (dtype(1) + np.exp(-x)))).astype(dtype)
+
+
+def embed_fwd(ids, weight, dtype=np.float32):
+    """top[n,:] = weight[(int)ids[n],:] (math.cu:9314-9330)."""
+    w = np.asarray(weight, dtype)
+    return w[np.asarray(ids).astype(np.int64).reshape(-1)]
+
+
+def rmsnorm_layer(x, weight=None, eps=1e-5, dtype=np.float32):
+    """RMSNormLayer.cs:156-180: x / sqrt(mean(x^2, last axis) + eps) [* weight].
+
+    channel_mean accumulates in double in the reference kernel
+    (math.cu:6816-6830) and casts the mean to T.
+    """
+    x = np.asarray(x, dtype)
+    ms = (x.astype(np.float64) ** 2).mean(axis=-1, keepdims=True).astype(dtype)
+    inv = dtype(1) / np.sqrt(ms + dtype(eps))
+    out = x * inv
+    if weight is not None:
+        out = out * np.asarray(weight, dtype)
+    return out.astype(dtype)
+
+
+# ----------------------------------------------------------------------------
+# RoPE, CudaDnnDLL form
+# ----------------------------------------------------------------------------
+
+def rope_tables(seq_len, hs, theta=10000.0):
+    """cos/sin tables [seq_len, hs/2] as RopeDataGpu<float>::Initialize builds
+    them on the host (rope.cu:535-553): freq_j = 1/powf(theta, 2j/hs) in fp32,
+    angle = freq_j * pos in fp32, cosf/sinf."""
+    j = np.arange(0, hs, 2, dtype=np.float32)
+    power = (j / np.float32(hs)).astype(np.float32)
+    freq = (np.float32(1.0) / np.power(np.float32(theta), power, dtype=np.float32)).astype(np.float32)
+    pos = np.arange(seq_len, dtype=np.float32)[:, None]
+    ang = (freq[None, :] * pos).astype(np.float32)
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+def rope_forward(x, seq_len, heads, hs, theta=10000.0, freq_offset=-1, dtype=np.float32):
+    """RopeDataGpu<T>::Forward (rope.cu:725-825).
+
+    x is flat with an even count; consecutive (even, odd) elements form a pair.
+    Pair i uses table entry ((i % (seq_len*heads*hs/2)) / (heads*hs/2)) * hs/2
+    + i % (hs/2), shifted by freq_offset when freq_offset > 0.
+    """
+    x = np.asarray(x, dtype).reshape(-1)
+    half = hs // 2
+    full = half * heads
+    cos, sin = rope_tables(seq_len, hs, theta)
+    cos = cos.reshape(-1).astype(dtype)
+    sin = sin.reshape(-1).astype(dtype)
+    off = freq_offset if freq_offset > 0 else 0
+    i = np.arange(x.size // 2)
+    base = i % (seq_len * full)
+    t = (base // full) * half + base % half + off
+    re, im = x[0::2], x[1::2]
+    y = np.empty_like(x)
+    y[0::2] = re * cos[t] - im * sin[t]
+    y[1::2] = re * sin[t] + im * cos[t]
+    return y
+
+
+# ----------------------------------------------------------------------------
+# attention
+# ----------------------------------------------------------------------------
+
+def attn_forward(q, k, v, mask_data=None, batch_mask=False, dtype=np.float32):
+    """attnHandle<T>::Forward (attn.cu:518-602).
+
+    q, k, v: (B,H,T,hs).  mask (1,1,T,T) when batch_mask is False (zero entries
+    are filled with -1e29), (B,T) key mask when True.  Returns (y, probs).
+    """
+    q = np.asarray(q, dtype)
+    k = np.asarray(k, dtype)
+    v = np.asarray(v, dtype)
+    B, H, T, hs = q.shape
+    scale = dtype(1.0 / np.sqrt(float(hs)))
+    att = (q @ k.transpose(0, 1, 3, 2)) * scale
+    if mask_data is not None:
+        m = np.asarray(mask_data, dtype)
+        if batch_mask:
+            att = mask_batch(att.size, B, m.size, 0.0, MASKED, att, m, dtype).reshape(att.shape)
+        else:
+            att = mask(att.size, m.size, 0.0, MASKED, att, m, dtype).reshape(att.shape)
+    p = softmax_lastaxis(att, dtype)
+    return (p @ v).astype(dtype), p
+
+
+def inner_product(x, w, b=None, dtype=np.float32):
+    """InnerProductLayer.forward (InnerProductLayer.cs:372-417): y = x W^T [+ 1 b],
+    W stored (num_output, K)."""
+    x = np.asarray(x, dtype)
+    y = x @ np.asarray(w, dtype).T
+    if b is not None:
+        y = y + np.asarray(b, dtype)
+    return y.astype(dtype)
+
+
+def causal_mask(T, dtype=np.float32):
+    """fillMask (CausalSelfAttentionLayer.cs:276-291): ones on and below the diagonal."""
+    return np.tril(np.ones((T, T), dtype))
+
+
+def causal_self_attention(x, w_attn, b_attn, w_proj, b_proj, heads, rope=None, dtype=np.float32):
+    """CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-628).
+
+    x (B,T,C); fused QKV InnerProduct (3C,C); q,k,v are consecutive thirds of
+    the fused output; heads split as (B,T,H,hs)->(B,H,T,hs); causal mask;
+    softmax; @v; merge heads; output projection.  ``rope`` = (seq_len, theta)
+    applies rope_forward to q and k before the head transpose.
+    Returns dict with intermediates.
+    """
+    x = np.asarray(x, dtype)
+    B, T, C = x.shape
+    hs = C // heads
+    qkv = inner_product(x, w_attn, b_attn, dtype)
+    q, k, v = qkv[..., :C], qkv[..., C:2 * C], qkv[..., 2 * C:]
+    if rope is not None:
+        q = rope_forward(q, rope[0], heads, hs, rope[1], dtype=dtype).reshape(B, T, C)
+        k = rope_forward(k, rope[0], heads, hs, rope[1], dtype=dtype).reshape(B, T, C)
+    qt = q.reshape(B, T, heads, hs).transpose(0, 2, 1, 3)
+    kt = k.reshape(B, T, heads, hs).transpose(0, 2, 1, 3)
+    vt = v.reshape(B, T, heads, hs).transpose(0, 2, 1, 3)
+    work, att = attn_forward(qt, kt, vt, causal_mask(T, dtype), False, dtype)
+    ymerged = work.transpose(0, 2, 1, 3).reshape(B, T, C)
+    y = inner_product(ymerged, w_proj, b_proj, dtype)
+    return {"qt": qt, "kt": kt, "vt": vt, "att": att, "work": work, "y": y}
+
+
+def multihead_attention(xq, xk, xv, wq, bq, wk, bk, wv, bv, wo, bo, heads, mask_data=None,
+                        mask_kind="none", rope=None, position=-1, dtype=np.float32):
+    """MultiheadAttentionLayer.forward without KV cache (MultiheadAttentionLayer.cs:643-811).
+
+    mask_kind: "none", "causal" ((1,1,T,T) tril), "key" ((B,T_k) key padding,
+    broadcast over heads and query rows) or "full" ((B,T_q,T_k), broadcast over
+    heads): the last two go through mask_batch.  Cross attention may use
+    T_q != T_k here (the reference layer assumes equal lengths; the closed form
+    is the same).
+    """
+    xq = np.asarray(xq, dtype)
+    xk = np.asarray(xk, dtype)
+    xv = np.asarray(xv, dtype)
+    B, Tq, C = xq.shape
+    Tk = xk.shape[1]
+    hs = C // heads
+    q = inner_product(xq, wq, bq, dtype)
+    k = inner_product(xk, wk, bk, dtype)
+    v = inner_product(xv, wv, bv, dtype)
+    if rope is not None:
+        off = position * hs // 2 if position > 0 else -1
+        q = rope_forward(q, rope[0], heads, hs, rope[1], off, dtype).reshape(B, Tq, C)
+        k = rope_forward(k, rope[0], heads, hs, rope[1], off, dtype).reshape(B, Tk, C)
+    qt = q.reshape(B, Tq, heads, hs).transpose(0, 2, 1, 3)
+    kt = k.reshape(B, Tk, heads, hs).transpose(0, 2, 1, 3)
+    vt = v.reshape(B, Tk, heads, hs).transpose(0, 2, 1, 3)
+    scale = dtype(1.0 / np.sqrt(float(hs)))
+    att = (qt @ kt.transpose(0, 1, 3, 2)) * scale
+    if mask_kind == "causal":
+        m = np.asarray(mask_data, dtype)
+        att = mask(att.size, m.size, 0.0, MASKED, att, m, dtype).reshape(att.shape)
+    elif mask_kind in ("key", "full"):
+        m = np.asarray(mask_data, dtype)
+        att = mask_batch(att.size, B, m.size, 0.0, MASKED, att, m, dtype).reshape(att.shape)
+    p = softmax_lastaxis(att, dtype)
+    work = p @ vt
+    y = inner_product(work.transpose(0, 2, 1, 3).reshape(B, Tq, C), wo, bo, dtype)
+    return {"qt": qt, "kt": kt, "vt": vt, "att": p, "work": work, "y": y}
+
+
+def kv_cache_attention(q, kcache, vcache, dtype=np.float32):
+    """KV-cache branch of MultiheadAttentionLayer (MultiheadAttentionLayer.cs:713-730,
+    759-777) and the per-head loop of llama2_cpu.cpp:306-341: one query per head,
+    scores = q.k_t/sqrt(hs) over all cached t, softmax without a mask, sum_t p_t v_t.
+
+    q (B,H,hs); kcache, vcache (B,H,L,hs).  Returns (B,H,hs).
+    """
+    q = np.asarray(q, dtype)
+    kc = np.asarray(kcache, dtype)
+    vc = np.asarray(vcache, dtype)
+    hs = q.shape[-1]
+    s = np.einsum("bhd,bhld->bhl", q, kc) / dtype(np.sqrt(float(hs)))
+    p = softmax_lastaxis(s, dtype)
+    return np.einsum("bhl,bhld->bhd", p, vc).astype(dtype)

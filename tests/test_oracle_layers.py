@@ -1,0 +1,218 @@
+"""Pins the numpy checker (oracle/attention_ref.py) against reference-held
+golden vectors, library routines and closed forms.  CPU only."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import attention_ref as R
+from tests.conftest import GOLDEN, load_txt
+
+INL = json.load(open(os.path.join(GOLDEN, "inline_vectors.json")))
+
+
+# ---- inline known-answer vectors of TestCudaDnn.cs --------------------------------
+
+def test_gemm_inline_all_transposes():
+    g = INL["gemm"]
+    A, B = g["data"][:6], g["data"]
+    exp = np.array(g["result"], np.float32).reshape(2, 4)
+    for tA, tB, a, b in [(0, 0, A, B), (1, 0, g["A_T"], B), (1, 1, g["A_T"], g["B_T"]), (0, 1, A, g["B_T"])]:
+        out = R.gemm(bool(tA), bool(tB), 2, 4, 3, 1.0, a, b, 0.0)
+        assert np.array_equal(out, exp), (tA, tB)
+
+
+def test_gemv_inline():
+    g = INL["gemv"]
+    assert np.array_equal(R.gemv(False, 2, 3, 1.0, g["data"], g["data"][:3], 0.0), np.array(g["result_notrans"], np.float32))
+    assert np.array_equal(R.gemv(True, 2, 3, 1.0, g["data"], g["data"][:2], 0.0), np.array(g["result_trans"], np.float32))
+
+
+def test_mask_inline():
+    x = np.array(INL["mask"]["x"], np.float32)
+    n = x.size
+    for i in range(n):
+        m = np.ones(n, np.float32)
+        m[i:] = 0
+        exp = x.copy()
+        exp[i:] = -np.inf
+        assert np.array_equal(R.mask(n, n, 0.0, -np.inf, x, m), exp)
+
+
+def test_mask2_inline_wraps_mask():
+    x = np.array(INL["mask2"]["x"], np.float32)
+    n, nm = x.size, x.size // 2
+    for i in range(n):
+        m = np.ones(nm, np.float32)
+        m[i:] = 0
+        exp = x.copy()
+        for j in range(i, n):
+            if m[j % nm] == 0:
+                exp[j] = -np.inf
+        assert np.array_equal(R.mask(n, nm, 0.0, -np.inf, x, m), exp)
+
+
+def test_mask_batch_inline():
+    g = INL["mask_batch"]
+    x = np.array(g["x"], np.float32)
+    exp = x.copy()
+    exp[g["masked_positions"]] = -np.inf
+    out = R.mask_batch(x.size, g["batch"], len(g["mask"]), 0.0, -np.inf, x, g["mask"])
+    assert np.array_equal(out, exp)
+
+
+def test_channel_copy_inline():
+    g = INL["channel_copy"]
+    cnt = g["num"] * g["channels"] * g["inner"]
+    allx = np.array(g["all"], np.float32)
+    rebuilt = np.zeros_like(allx)
+    for off, key in enumerate("ABC"):
+        y = R.channel_copy_fwd(cnt, g["num"], g["channels"], g["blocks"], g["inner"], off, allx)
+        assert np.array_equal(y, np.array(g[key], np.float32))
+        rebuilt = R.channel_copy_bwd(cnt, g["num"], g["channels"], g["blocks"], g["inner"], off, rebuilt, y)
+    assert np.array_equal(rebuilt, allx)
+
+
+# ---- library routines / closed forms ----------------------------------------------
+
+def test_gemm2_matmul_matches_numpy():
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((6, 5, 7))
+    B = rng.standard_normal((6, 7, 3))
+    out = R.matmul(6, 5, 3, 7, A, B, scale=0.5, dtype=np.float64)
+    assert np.allclose(out, 0.5 * (A @ B), rtol=1e-13, atol=1e-13)
+    Bt = B.transpose(0, 2, 1).copy()
+    out = R.matmul(6, 5, 3, 7, A, Bt, transB=True, dtype=np.float64)
+    assert np.allclose(out, A @ B, rtol=1e-13, atol=1e-13)
+    At = A.transpose(0, 2, 1).copy()
+    out = R.matmul(6, 5, 3, 7, At, B, transA=True, dtype=np.float64)
+    assert np.allclose(out, A @ B, rtol=1e-13, atol=1e-13)
+
+
+def test_softmax_matches_scipy():
+    from scipy.special import softmax
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((3, 4, 9)) * 5
+    assert np.allclose(R.softmax_lastaxis(x, np.float64), softmax(x, axis=-1), rtol=1e-13)
+
+
+def test_transpose_matches_numpy_permute():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 5, 3, 4)).astype(np.float32)
+    perm = (0, 2, 1, 3)
+    y = np.transpose(x, perm)
+    xs = [5 * 3 * 4, 3 * 4, 4, 1]
+    ys = [int(np.prod(y.shape[i + 1:])) for i in range(4)]
+    out = R.transpose(x, xs, ys, perm)
+    assert np.array_equal(out.reshape(y.shape), y)
+    assert np.array_equal(R.transpose_hw(2, 5, 3, 4, x).reshape(2, 5, 4, 3), x.transpose(0, 1, 3, 2))
+
+
+def test_rope_is_complex_rotation_with_explicit_positions():
+    # closed form: (re + i im) * exp(i * pos * theta^(-2j/hs)); T == seq_len so the
+    # kernel's index-derived position equals the true token position for every batch
+    B, T, H, hs, theta = 2, 6, 3, 8, 10000.0
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((B, T, H, hs))
+    out = R.rope_forward(x, T, H, hs, theta, dtype=np.float64).reshape(B, T, H, hs // 2, 2)
+    z = x.reshape(B, T, H, hs // 2, 2)
+    zc = z[..., 0] + 1j * z[..., 1]
+    j = np.arange(hs // 2)
+    ang = np.arange(T)[:, None] * theta ** (-2.0 * j / hs)[None, :]
+    rot = zc * np.exp(1j * ang)[None, :, None, :]
+    # tables are built in fp32 by the reference host code
+    assert np.allclose(out[..., 0], rot.real, atol=2e-6)
+    assert np.allclose(out[..., 1], rot.imag, atol=2e-6)
+    # invariants: pair norms preserved; position 0 is the identity
+    assert np.allclose(np.hypot(out[..., 0], out[..., 1]), np.abs(zc), atol=1e-6)
+    assert np.allclose(out[:, 0].reshape(B, H, hs), x[:, 0], atol=0)
+
+
+def test_rope_freq_offset_selects_position_row():
+    H, hs, S = 2, 8, 16
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((1, 1, H, hs))
+    full = rng.standard_normal((1, S, H, hs))
+    full[0, 5] = x[0, 0]
+    whole = R.rope_forward(full, S, H, hs, dtype=np.float64).reshape(1, S, H, hs)
+    one = R.rope_forward(x, S, H, hs, freq_offset=5 * hs // 2, dtype=np.float64).reshape(H, hs)
+    assert np.allclose(one, whole[0, 5], atol=1e-12)
+    # offset <= 0 means "no shift" (rope.cu:808-814)
+    assert np.array_equal(R.rope_forward(x, S, H, hs, freq_offset=0), R.rope_forward(x, S, H, hs, freq_offset=-1))
+
+
+def test_attention_matches_torch_sdpa():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(5)
+    B, H, T, hs = 2, 3, 7, 8
+    q, k, v = (rng.standard_normal((B, H, T, hs)) for _ in range(3))
+    y, p = R.attn_forward(q, k, v, R.causal_mask(T, np.float64), False, np.float64)
+    ref = F.scaled_dot_product_attention(*(torch.from_numpy(a) for a in (q, k, v)), is_causal=True).numpy()
+    assert np.allclose(y, ref, rtol=1e-12, atol=1e-12)
+    assert np.all(np.triu(p, 1) == 0) and np.allclose(p.sum(-1), 1)
+    # key-padding mask (B,T): torch boolean mask broadcast over heads and rows
+    lens = [4, 7]
+    km = np.zeros((B, T))
+    for b, n in enumerate(lens):
+        km[b, :n] = 1
+    y2, _ = R.attn_forward(q, k, v, km, True, np.float64)
+    ref2 = F.scaled_dot_product_attention(*(torch.from_numpy(a) for a in (q, k, v)),
+                                          attn_mask=torch.from_numpy(km.astype(bool))[:, None, None, :]).numpy()
+    assert np.allclose(y2, ref2, rtol=1e-12, atol=1e-12)
+
+
+def test_fully_masked_row_is_uniform_not_nan():
+    q = np.zeros((1, 1, 2, 4), np.float32)
+    k = np.ones((1, 1, 2, 4), np.float32)
+    v = np.arange(8, dtype=np.float32).reshape(1, 1, 2, 4)
+    y, p = R.attn_forward(q, k, v, np.zeros((1, 2), np.float32), True)
+    assert np.allclose(p, 0.5) and np.allclose(y[0, 0, 0], v[0, 0].mean(0))
+
+
+def test_kv_cache_attention_equals_last_row_of_causal():
+    rng = np.random.default_rng(6)
+    B, H, L, hs = 2, 3, 9, 8
+    q, k, v = (rng.standard_normal((B, H, L, hs)) for _ in range(3))
+    full, _ = R.attn_forward(q, k, v, R.causal_mask(L, np.float64), False, np.float64)
+    dec = R.kv_cache_attention(q[:, :, -1], k, v, np.float64)
+    assert np.allclose(dec, full[:, :, -1], rtol=1e-12, atol=1e-12)
+
+
+def test_rmsnorm_silu_match_torch():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((3, 5, 16))
+    w = rng.standard_normal(16)
+    ref = F.rms_norm(torch.from_numpy(x), (16,), torch.from_numpy(w), eps=1e-5).numpy()
+    assert np.allclose(R.rmsnorm_layer(x, w, 1e-5, np.float64), ref, rtol=1e-12)
+    assert np.allclose(R.silu(x, np.float64), F.silu(torch.from_numpy(x)).numpy(), rtol=1e-12)
+
+
+# ---- reference-held golden tensors (minGPT CausalSelfAttention dumps) --------------
+
+@pytest.mark.parametrize("name,heads", [("gpt-pico-csa", 1), ("gpt-pico-csa3", 3), ("gpt-pico-csa3B", 3), ("gpt-pico-csaB", 1)])
+def test_causal_self_attention_golden(name, heads):
+    d = os.path.join(GOLDEN, name)
+    x = load_txt(os.path.join(d, "x.txt"))
+    out = R.causal_self_attention(
+        x, load_txt(os.path.join(d, "attn_weight.txt")), load_txt(os.path.join(d, "attn_bias.txt")),
+        load_txt(os.path.join(d, "attn_proj_weight.txt")), load_txt(os.path.join(d, "attn_proj_bias.txt")),
+        heads, dtype=np.float64)
+    y = load_txt(os.path.join(d, "y.txt"))
+    assert np.abs(out["y"] - y.reshape(out["y"].shape)).max() < 2e-7
+    qt = load_txt(os.path.join(d, "qt.txt"))
+    assert np.abs(out["qt"] - qt.reshape(out["qt"].shape)).max() < 2e-7
+    if os.path.exists(os.path.join(d, "var_att.npy")):
+        att = np.load(os.path.join(d, "var_att.npy"))
+        assert np.abs(out["att"] - att).max() < 2e-7
+        assert np.all(np.triu(att, 1) == 0)
+        assert np.abs(out["vt"] - np.load(os.path.join(d, "var_vt.npy"))).max() < 2e-7
+        assert np.abs(out["work"] - np.load(os.path.join(d, "var_y.npy"))).max() < 2e-7
+    # fp32 arithmetic stays within the fp32 parity tolerance of the fp64 result
+    out32 = R.causal_self_attention(
+        x, load_txt(os.path.join(d, "attn_weight.txt")), load_txt(os.path.join(d, "attn_bias.txt")),
+        load_txt(os.path.join(d, "attn_proj_weight.txt")), load_txt(os.path.join(d, "attn_proj_bias.txt")), heads)
+    assert np.abs(out32["y"] - out["y"]).max() < 1e-6

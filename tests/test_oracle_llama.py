@@ -1,0 +1,145 @@
+"""Pins the C checker (oracle/llama2_oracle.c) against library routines and an
+independent library implementation of the Llama-2 architecture.  CPU only."""
+import numpy as np
+import pytest
+
+from oracle import llama2 as O
+
+TINY = dict(dim=48, hidden_dim=128, n_layers=3, n_heads=6, n_kv_heads=6, vocab_size=200, seq_len=32)
+TINY_GQA = dict(dim=48, hidden_dim=96, n_layers=2, n_heads=6, n_kv_heads=2, vocab_size=120, seq_len=24)
+
+
+def test_softmax_vs_scipy():
+    from scipy.special import softmax
+    x = np.random.default_rng(0).standard_normal(777).astype(np.float32) * 4
+    assert np.allclose(O.softmax(x), softmax(x.astype(np.float64)), rtol=2e-6, atol=1e-9)
+    assert O.softmax(np.float32([3.0]))[0] == 1.0
+
+
+def test_rmsnorm_vs_torch():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(288).astype(np.float32)
+    w = rng.standard_normal(288).astype(np.float32)
+    ref = F.rms_norm(torch.from_numpy(x).double(), (288,), torch.from_numpy(w).double(), eps=1e-5).numpy()
+    assert np.allclose(O.rmsnorm(x, w), ref, rtol=3e-6, atol=1e-7)
+
+
+def test_matvec_vs_numpy_and_row_major_layout():
+    rng = np.random.default_rng(2)
+    w = rng.standard_normal((37, 53)).astype(np.float32)
+    x = rng.standard_normal(53).astype(np.float32)
+    assert np.allclose(O.matvec(w, x), w.astype(np.float64) @ x, rtol=1e-5, atol=1e-5)
+    e = np.zeros(53, np.float32)
+    e[7] = 1
+    assert np.array_equal(O.matvec(w, e), w[:, 7])
+
+
+def test_freq_tables_and_rope_closed_form():
+    hs, S, H = 16, 40, 3
+    c, s = O.freq_tables(hs, S)
+    j = np.arange(hs // 2)
+    ang = np.arange(S)[:, None] * 10000.0 ** (-2.0 * j / hs)[None, :]
+    assert np.allclose(c, np.cos(ang), atol=3e-6) and np.allclose(s, np.sin(ang), atol=3e-6)
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((H, hs)).astype(np.float32)
+    k = rng.standard_normal((H, hs)).astype(np.float32)
+    for pos in (0, 1, 17, 39):
+        q2, k2 = O.rope_pairs(q, k, c, s, pos)
+        for src, out in ((q, q2), (k, k2)):
+            z = (src[:, 0::2] + 1j * src[:, 1::2]) * np.exp(1j * ang[pos])[None, :]
+            assert np.allclose(out[:, 0::2], z.real, atol=1e-5)
+            assert np.allclose(out[:, 1::2], z.imag, atol=1e-5)
+    q0, k0 = O.rope_pairs(q, k, c, s, 0)
+    assert np.array_equal(q0, q) and np.array_equal(k0, k)
+
+
+def test_argmax_first_max_wins():
+    assert O.argmax(np.float32([1, 5, 5, 2])) == 1
+    assert O.argmax(np.float32([-3, -3, -3])) == 0
+    assert O.argmax(np.float32([0, 1, 2, 9])) == 3
+
+
+def _hf_model(cfg, views, shared):
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+    hc = LlamaConfig(hidden_size=cfg["dim"], intermediate_size=cfg["hidden_dim"],
+                     num_hidden_layers=cfg["n_layers"], num_attention_heads=cfg["n_heads"],
+                     num_key_value_heads=cfg["n_kv_heads"], vocab_size=cfg["vocab_size"],
+                     max_position_embeddings=cfg["seq_len"], rms_norm_eps=1e-5, rope_theta=10000.0,
+                     tie_word_embeddings=False, attention_bias=False, mlp_bias=False)
+    hc._attn_implementation = "eager"
+    m = LlamaForCausalLM(hc).double().eval()
+    hs = cfg["dim"] // cfg["n_heads"]
+    # adjacent-pair rotary -> half-split rotary: reorder q/k output rows inside each head
+    perm = np.concatenate([np.arange(0, hs, 2), np.arange(1, hs, 2)])
+
+    def rot(w, nh):
+        return w.reshape(nh, hs, -1)[:, perm, :].reshape(nh * hs, -1)
+
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).double()
+    sd = {"model.embed_tokens.weight": t(views["tok_emb"]), "model.norm.weight": t(views["rms_final"]),
+          "lm_head.weight": t(views["tok_emb"] if shared else views["wcls"])}
+    for l in range(cfg["n_layers"]):
+        p = "model.layers.%d." % l
+        sd[p + "input_layernorm.weight"] = t(views["rms_att"][l])
+        sd[p + "post_attention_layernorm.weight"] = t(views["rms_ffn"][l])
+        sd[p + "self_attn.q_proj.weight"] = t(rot(views["wq"][l], cfg["n_heads"]))
+        sd[p + "self_attn.k_proj.weight"] = t(rot(views["wk"][l], cfg["n_kv_heads"]))
+        sd[p + "self_attn.v_proj.weight"] = t(views["wv"][l])
+        sd[p + "self_attn.o_proj.weight"] = t(views["wo"][l])
+        sd[p + "mlp.gate_proj.weight"] = t(views["w1"][l])
+        sd[p + "mlp.down_proj.weight"] = t(views["w2"][l])
+        sd[p + "mlp.up_proj.weight"] = t(views["w3"][l])
+    missing = m.load_state_dict(sd, strict=False)
+    assert not [k for k in missing.missing_keys if "rotary" not in k], missing
+    return m
+
+
+@pytest.mark.parametrize("cfg,shared", [(TINY, False), (TINY, True), (TINY_GQA, False)])
+def test_forward_vs_transformers_llama(cfg, shared):
+    """Incremental KV-cache decode of the checker == full-sequence forward of
+    transformers.LlamaForCausalLM (fp64) on the same weights, every position."""
+    import torch
+    blob, views = O.random_weights(cfg, seed=11, shared_classifier=shared, std=0.2)
+    # non-trivial norm weights so a dropped weight multiply would show
+    rng = np.random.default_rng(5)
+    for k in ("rms_att", "rms_ffn", "rms_final"):
+        views[k][...] = 1.0 + 0.3 * rng.standard_normal(views[k].shape).astype(np.float32)
+    toks = rng.integers(0, cfg["vocab_size"], 20)
+    m = O.Llama(cfg, blob, shared)
+    mine = np.stack([m.forward(int(t), i) for i, t in enumerate(toks)])
+    hf = _hf_model(cfg, views, shared)
+    with torch.no_grad():
+        ref = hf(torch.from_numpy(toks)[None]).logits[0].numpy()
+    err = np.abs(mine - ref).max() / np.abs(ref).max()
+    assert err < 2e-5, err
+    assert np.array_equal(mine.argmax(-1), ref.argmax(-1))
+
+
+def test_generate_greedy_feeds_back_argmax_and_is_deterministic():
+    blob, _ = O.random_weights(TINY, seed=3, std=0.2)
+    m = O.Llama(TINY, blob)
+    prompt = np.array([5, 17, 3, 99], np.int32)
+    ids, lg = m.generate_greedy(prompt, 24, want_logits=True)
+    assert np.array_equal(ids, lg.argmax(-1))
+    m2 = O.Llama(TINY, blob)
+    seq = list(prompt)
+    for pos in range(24):
+        tok = seq[pos] if pos < len(prompt) else int(ids[pos - 1])
+        l2 = m2.forward(tok, pos)
+        assert np.array_equal(l2, lg[pos])
+    assert np.array_equal(O.Llama(TINY, blob).generate_greedy(prompt, 24), ids)
+
+
+def test_checkpoint_v1_header(tmp_path):
+    import struct
+    blob, _ = O.random_weights(TINY, seed=1)
+    p = tmp_path / "m.bin"
+    O.write_checkpoint_v1(str(p), TINY, blob, shared_classifier=False)
+    raw = p.read_bytes()
+    assert struct.unpack("<Ii", raw[:8]) == (0x616B3432, 1)
+    assert struct.unpack("<7i", raw[8:36]) == tuple(TINY[k] for k in O.CONFIG_FIELDS)
+    assert raw[36] == 0 and len(raw) == 256 + blob.size * 4
+    assert np.array_equal(np.frombuffer(raw[256:], np.float32), blob)
