@@ -1,0 +1,232 @@
+/*
+ * C ABI of libmycaffe_hip.so - the gfx950 (MI355X) replacement for the
+ * attention hot path of MyCaffe's CudaDnnDLL.
+ *
+ * The exported names, argument order and argument meaning are those of the
+ * reference's native DLL (CudaDnnDLL/CudaDnnDLL.11.8.def:5-18,
+ * CudaDnnDLL/CudaDnnDLL.cpp:57-1161), with the Win64 typedefs replaced by
+ * fixed-width types: LONG = int32_t, LONGLONG = int64_t, LPTSTR = UTF-16 text
+ * (char16_t*).  Device memory is only ever named by integer handles; no
+ * pointer to device memory crosses this boundary.
+ *
+ * Only the function ids listed below are dispatched; every other id returns
+ * MCH_ERROR_NOT_IMPLEMENTED with a message naming the id.  The Double entry
+ * points exist and return MCH_ERROR_NOT_IMPLEMENTED (the hot path is fp32 and
+ * 16-bit storage).
+ */
+#ifndef MYCAFFE_HIP_ABI_H
+#define MYCAFFE_HIP_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t MCH_LONG;
+typedef int64_t MCH_LONGLONG;
+typedef uint16_t MCH_TCHAR; /* UTF-16 code unit */
+
+/* ---- error codes (CudaDnnDLL/Cuda Files/util.h:128-228) ------------------- */
+enum {
+    MCH_ERROR_DLL_NOT_INIT = 89999,
+    MCH_ERROR_PARAM = 90000,
+    MCH_ERROR_PARAM_OUT_OF_RANGE = 90001,
+    MCH_ERROR_PARAM_NULL = 90002,
+    MCH_ERROR_FILE_READ = 90004,
+    MCH_ERROR_FILE_OPEN = 90005,
+    MCH_ERROR_MEMORY_OUT = 90007,
+    MCH_ERROR_MEMORY_NULL = 90008,
+    MCH_ERROR_NOT_IMPLEMENTED = 90009,
+    MCH_ERROR_MEMORY_RANGE_EXCEEDED = 90010,
+    MCH_ERROR_MEMORY_MIXED_HALF_TYPES = 90011,
+    MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED = 90012,
+    MCH_ERROR_MEMORY_NOT_FOUND = 90014,
+    MCH_ERROR_MEMORY_TOO_SMALL = 90016,
+    MCH_ERROR_DEVICE_NOT_INITIALIZED = 90017,
+    MCH_ERROR_ROPE_NOT_INITIALIZED = 90201,
+    MCH_ERROR_ATTN_NOT_INITIALIZED = 90281,
+    MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE = 90284,
+    MCH_ERROR_ATTN_INVALID_BLOCK_SIZE = 90285,
+    MCH_ERROR_EXTENSION_NOT_INITIALIZED = 90401,
+    /* llama2 extension (CudaExtension.llm32.llama2/Files/llm.h:15-19) */
+    MCH_ERROR_LLM_LOAD_MODEL = 10001,
+    MCH_ERROR_LLM_MISSING_MODEL_FILE = 10002,
+    MCH_ERROR_LLM_MISSING_TOKENIZER_FILE = 10003,
+    MCH_ERROR_LLM_GENERATE = 10004
+};
+
+/* ---- function ids (CudaDnnDLL/inc/FunctionIDs.h:71-551, main.h:23-40) ------ */
+enum {
+    MCH_DLL_FREEMEM = -1,
+    MCH_DLL_INITIALIZE = -2,
+    MCH_DLL_CLEANUP = -3,
+
+    MCH_FN_SETDEVICE = 1,
+    MCH_FN_GETDEVICE = 3,
+    MCH_FN_SYNCHRONIZEDEVICE = 5,
+    MCH_FN_CREATE_MEMORYPOINTER = 16,
+    MCH_FN_FREE_MEMORYPOINTER = 17,
+    MCH_FN_ALLOCMEM_HALF = 19,
+    MCH_FN_ALLOCMEM = 20,
+    MCH_FN_FREEMEM = 21,
+    MCH_FN_GETMEM = 22,
+    MCH_FN_SETMEM = 23,
+    MCH_FN_CREATE_CUDNN = 47,
+    MCH_FN_FREE_CUDNN = 48,
+    MCH_FN_CREATE_TENSORDESC = 50,
+    MCH_FN_FREE_TENSORDESC = 51,
+    MCH_FN_SET_TENSORDESC = 52,
+    MCH_FN_CREATE_EXTENSION = 67,
+    MCH_FN_FREE_EXTENSION = 68,
+    MCH_FN_EXTENSION_RUN = 69,
+    MCH_FN_SOFTMAX_FWD = 111,
+    MCH_FN_ATTN_CREATE = 160,
+    MCH_FN_ATTN_FREE = 161,
+    MCH_FN_ATTN_SET = 162,
+    MCH_FN_ATTN_FWD = 163,
+    MCH_FN_SET = 200,
+    MCH_FN_COPY = 202,
+    MCH_FN_GEMM2 = 219,
+    MCH_FN_GEMM = 220,
+    MCH_FN_GEMV = 221,
+    MCH_FN_AXPY = 222,
+    MCH_FN_SCAL = 224,
+    MCH_FN_SCALE = 227,
+    MCH_FN_ADD = 229,
+    MCH_FN_MUL = 231,
+    MCH_FN_TRANSPOSE = 261,
+    MCH_FN_MASK = 264,
+    MCH_FN_MASK_BATCH = 266,
+    MCH_FN_TRANSPOSE_HW = 267,
+    MCH_FN_CHANNEL_COPY = 300,
+    MCH_FN_EMBED_FWD = 390,
+    MCH_FN_SILU_FWD = 605,
+    MCH_FN_CREATE_ROPE = 980,
+    MCH_FN_FREE_ROPE = 981,
+    MCH_FN_ROPE_FWD = 982,
+    MCH_QRY_DEVICE_NAME = 1000,
+    MCH_QRY_EXTENSION_STRING = 1003,
+
+    /* Ids with no counterpart in the reference: single-call replacements for
+     * host-side loops of the reference's C# layers.  A maintainer adds one
+     * CudaDnn<T> wrapper per id.
+     *
+     * ATTN_DECODE_FWD replaces the O(pos) loop of the KV-cache branch of
+     * MultiheadAttentionLayer.forward (MultiheadAttentionLayer.cs:713-730,
+     * 759-777) and Primitives::attention (primitives.cu:158-202,389-403).
+     *   f{scale (0 = 1/sqrt(hs))}
+     *   l{batch, heads, kvHeads, hs, len, hQ, hKcache, hVcache, hY,
+     *     strideKvBatch, strideKvHead, strideKvPos [, hRope, hKnew, hVnew]}
+     * With hRope != 0 the call first rotates q and k_new at position len-1
+     * with that rope handle's tables and stores k_new/v_new into the caches
+     * at position len-1.
+     *
+     * RMSNORM_FWD replaces the six-call chain of RMSNormLayer.forward
+     * (RMSNormLayer.cs:156-180):  f{eps}  l{outer, dim, hX, hWeight(0=none), hY}
+     *
+     * SWIGLU_FWD = silu(a)*b (TransformerBlockLayer.cs:860-875):  l{n, hA, hB, hY}
+     */
+    MCH_FN_ATTN_DECODE_FWD = 2001,
+    MCH_FN_RMSNORM_FWD = 2002,
+    MCH_FN_SWIGLU_FWD = 2003
+};
+
+/* DEVINIT flags (CudaDnnDLL/Cuda Files/device.h:18-22) */
+enum { MCH_DEVINIT_CUBLAS = 1, MCH_DEVINIT_CURAND = 2, MCH_DEVINIT_SETSEED = 4, MCH_DEVINIT_RESETDEVICE = 8 };
+
+/* ---- reference entry points ------------------------------------------------ */
+
+/* CudaDnnDLL.cpp:134-312.  Legacy packing: every argument (ints and handles
+ * included) travels as float in pInput. */
+MCH_LONG DLL_InvokeFloat(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
+                         float** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:314-492.  Scalars in pInput, integers and handles in plInput. */
+MCH_LONG DLL_InvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
+                            MCH_LONGLONG* plInput, MCH_LONG llInput, float** ppOutput, MCH_LONG* plOutput,
+                            MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:1017-1100.  As DLL_InvokeFloat plus one UTF-16 input string
+ * (CREATE_EXTENSION: library path; EXTENSION_RUN: text handed to the extension). */
+MCH_LONG DLL_InvokeFloatEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
+                           MCH_TCHAR* pszInput, float** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr,
+                           MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:494-853: double twins; return MCH_ERROR_NOT_IMPLEMENTED here. */
+MCH_LONG DLL_InvokeDouble(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,
+                          double** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,
+                             MCH_LONGLONG* plInput, MCH_LONG llInput, double** ppOutput, MCH_LONG* plOutput,
+                             MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+MCH_LONG DLL_InvokeDoubleEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,
+                            MCH_TCHAR* pszInput, double** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr,
+                            MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:855-933.  *ppOutput receives a malloc'ed UTF-16 string that the
+ * caller returns through DLL_QueryString(.., MCH_DLL_FREEMEM, ..). */
+MCH_LONG DLL_QueryString(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, MCH_LONG* pInput, MCH_LONG lInput,
+                         MCH_TCHAR** ppOutput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:935-1015.  Text is written into the caller's buffer. */
+MCH_LONG DLL_QueryStringFloatEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, MCH_LONG* pInput, MCH_LONG lInput,
+                                MCH_TCHAR* pszOutput, MCH_LONG lOutputMax, MCH_TCHAR* szErr,
+                                MCH_LONG lszErrMax);
+MCH_LONG DLL_QueryStringDoubleEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, MCH_LONG* pInput, MCH_LONG lInput,
+                                 MCH_TCHAR* pszOutput, MCH_LONG lOutputMax, MCH_TCHAR* szErr,
+                                 MCH_LONG lszErrMax);
+
+/* CudaDnnDLL.cpp:57-128.  Used by extension libraries: device pointer behind a
+ * memory handle, and host result buffers owned by the parent. */
+MCH_LONG Internal_GetPointerFloat(int32_t ht, MCH_LONG lKernelIdx, MCH_LONG hHandle, void** ppPtr);
+MCH_LONG Internal_GetPointerDouble(int32_t ht, MCH_LONG lKernelIdx, MCH_LONG hHandle, void** ppPtr);
+MCH_LONG Internal_AllocHostFloat(MCH_LONG lKernelIdx, MCH_LONG lCount, float** ppfDst, float* pfSrc,
+                                 bool bSrcOnDevice);
+MCH_LONG Internal_AllocHostDouble(MCH_LONG lKernelIdx, MCH_LONG lCount, double** ppfDst, double* pfSrc,
+                                  bool bSrcOnDevice);
+
+/* ---- extension ABI (libmycaffe_hip_llama2.so) ------------------------------
+ * CudaExtension.llm32.llama2/CudaExtension.llm32.11.8.def:5-11,
+ * CudaExtension.llm32.cpp:67-268.  hParent is the dlopen handle of the parent
+ * library (HMODULE in the reference). */
+enum {
+    MCH_LLM_CREATE = 1,         /* f{temperature, topp, seed} -> f{hLlm} */
+    MCH_LLM_DESTROY = 2,        /* f{hLlm} */
+    MCH_LLM_LOAD = 3,           /* Ex: f{hLlm}, "model.bin;tokenizer.bin" */
+    MCH_LLM_QUERYSTATUS = 4,    /* f{hLlm} -> f{pct, status} */
+    MCH_LLM_GENERATE = 5,       /* Ex: f{hLlm}, prompt text */
+    MCH_LLM_QUERYRESPONSE = 6,  /* Ex: f{hLlm} -> text in szOutput, *ppOutput = end flag */
+    MCH_LLM_ABORT = 7,          /* f{hLlm} */
+    /* No counterpart in the reference: token-id front door used where no
+     * tokenizer file exists (synthetic checkpoints).
+     *   GENERATE_IDS  f{hLlm, nSteps, wantLogits(0|1), id0, id1, ...}
+     *                 -> f{next id after each position [, logits of every step]}
+     *   SET_OPTION    f{hLlm, option, value}; option 1 = weight storage
+     *                 (0 fp32, 1 bf16), applied at the next LOAD
+     *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
+     *                 -> f{batch x nSteps next ids} */
+    MCH_LLM_GENERATE_IDS = 100,
+    MCH_LLM_SET_OPTION = 101,
+    MCH_LLM_GENERATE_BATCH = 102
+};
+
+MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);
+MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG lfnIdx, float* pInput, MCH_LONG lInput, float** ppOutput,
+                                        MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lErrMax);
+MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG lfnIdx, float* pInput, MCH_LONG lInput, float** ppOutput,
+                                          MCH_LONG* plOutput, MCH_TCHAR* szInput, MCH_TCHAR* szOutput,
+                                          MCH_LONG lOutputMax, MCH_TCHAR* szErr, MCH_LONG lErrMax);
+
+/* ---- measurement hook (no counterpart in the reference) --------------------
+ * Runs the same Ex2 dispatch `nWarmup` + `nReps` times on the kernel's stream
+ * and returns the mean duration of the timed launches in milliseconds,
+ * measured with HIP events recorded on that stream.  Only for calls whose
+ * result does not depend on how often they run. */
+MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
+                                MCH_LONGLONG* plInput, MCH_LONG llInput, MCH_LONG nWarmup, MCH_LONG nReps,
+                                float* pfMs, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MYCAFFE_HIP_ABI_H */

@@ -1,0 +1,477 @@
+// Elementwise, layout, softmax, RoPE and RMSNorm kernels for gfx950.
+// All are HBM-bound: one pass over the data, 64-wide wavefronts, 128-bit
+// accesses where the layout allows, grid sized to a few waves per CU.
+#include "kernels.h"
+
+namespace mch {
+
+static constexpr int TPB = 256;
+
+static inline int grid_for(size_t n, int per_thread = 1)
+{
+    size_t blocks = (n + (size_t)TPB * per_thread - 1) / ((size_t)TPB * per_thread);
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256 * 16) blocks = 256 * 16;  // 256 CUs x 16 resident workgroups
+    return (int)blocks;
+}
+
+template <typename T> __device__ inline float ld(const T* p, size_t i);
+template <> __device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ inline float ld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+template <typename T> __device__ inline void st(T* p, size_t i, float v);
+template <> __device__ inline void st<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ inline void st<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+#define GRID_STRIDE(i, n) \
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (n); i += (size_t)blockDim.x * gridDim.x)
+
+#define DISPATCH_DT(dt, CALL)            \
+    do {                                 \
+        if ((dt) == F32) { typedef float T; CALL; } else { typedef bf16_t T; CALL; } \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+template <typename T> __global__ void set_kernel(T* y, size_t n, float v) { GRID_STRIDE(i, n) st(y, i, v); }
+
+hipError_t k_set(hipStream_t s, DType dt, void* y, size_t n, float v)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(set_kernel<T>, grid_for(n), TPB, 0, s, (T*)y, n, v));
+    return hipGetLastError();
+}
+
+template <typename S, typename D> __global__ void convert_kernel(const S* x, D* y, size_t n)
+{
+    GRID_STRIDE(i, n) st(y, i, ld(x, i));
+}
+
+hipError_t k_convert(hipStream_t s, DType sdt, const void* src, DType ddt, void* dst, size_t n)
+{
+    if (n == 0) return hipSuccess;
+    int g = grid_for(n);
+    if (sdt == F32 && ddt == F32)
+        return hipMemcpyAsync(dst, src, n * sizeof(float), hipMemcpyDeviceToDevice, s);
+    if (sdt == BF16 && ddt == BF16)
+        return hipMemcpyAsync(dst, src, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, s);
+    if (sdt == F32)
+        hipLaunchKernelGGL((convert_kernel<float, bf16_t>), g, TPB, 0, s, (const float*)src, (bf16_t*)dst, n);
+    else
+        hipLaunchKernelGGL((convert_kernel<bf16_t, float>), g, TPB, 0, s, (const bf16_t*)src, (float*)dst, n);
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void axpy_kernel(size_t n, float a, const T* x, T* y)
+{
+    GRID_STRIDE(i, n) st(y, i, a * ld(x, i) + ld(y, i));
+}
+hipError_t k_axpy(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(axpy_kernel<T>, grid_for(n), TPB, 0, s, n, alpha, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void scale_kernel(size_t n, float a, const T* x, T* y)
+{
+    GRID_STRIDE(i, n) st(y, i, a * ld(x, i));
+}
+hipError_t k_scale(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(scale_kernel<T>, grid_for(n), TPB, 0, s, n, alpha, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void add_kernel(size_t n, const T* a, const T* b, T* y, float alpha)
+{
+    GRID_STRIDE(i, n) st(y, i, ld(a, i) + ld(b, i) * alpha);
+}
+hipError_t k_add(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, float alpha)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(add_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y, alpha));
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void mul_kernel(size_t n, const T* a, const T* b, T* y)
+{
+    GRID_STRIDE(i, n) st(y, i, ld(a, i) * ld(b, i));
+}
+hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(mul_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y));
+    return hipGetLastError();
+}
+
+__device__ inline float silu_f(float x) { return x * (1.0f / (1.0f + expf(-x))); }
+
+template <typename T> __global__ void silu_kernel(size_t n, const T* x, T* y) { GRID_STRIDE(i, n) st(y, i, silu_f(ld(x, i))); }
+hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(silu_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void swiglu_kernel(size_t n, const T* a, const T* b, T* y)
+{
+    GRID_STRIDE(i, n) st(y, i, silu_f(ld(a, i)) * ld(b, i));
+}
+hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(swiglu_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y));
+    return hipGetLastError();
+}
+
+// y[i] = mask[i % maskDim] == search ? replace : x[i]
+template <typename T>
+__global__ void mask_kernel(size_t n, int maskDim, const T* x, const T* mask, T* y, float search, float replace)
+{
+    GRID_STRIDE(i, n) st(y, i, ld(mask, i % (size_t)maskDim) == search ? replace : ld(x, i));
+}
+hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
+                  const void* mask, void* y)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(mask_kernel<T>, grid_for(n), TPB, 0, s, n, maskDim, (const T*)x, (const T*)mask,
+                                       (T*)y, search, replace));
+    return hipGetLastError();
+}
+
+// mask index = i % (maskDim/batch) + (i / (n/batch)) * (maskDim/batch)
+template <typename T>
+__global__ void mask_batch_kernel(size_t n, int md1, size_t dd1, const T* x, const T* mask, T* y, float search,
+                                  float replace)
+{
+    GRID_STRIDE(i, n)
+    {
+        size_t mi = i % (size_t)md1 + (i / dd1) * (size_t)md1;
+        st(y, i, ld(mask, mi) == search ? replace : ld(x, i));
+    }
+}
+hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDim, float search, float replace,
+                        const void* x, const void* mask, void* y)
+{
+    if (n == 0) return hipSuccess;
+    int md1 = maskDim / batch;
+    size_t dd1 = n / (size_t)batch;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(mask_batch_kernel<T>, grid_for(n), TPB, 0, s, n, md1, dd1, (const T*)x,
+                                       (const T*)mask, (T*)y, search, replace));
+    return hipGetLastError();
+}
+
+// Generic permute: xc / yc hold the element strides of the source / destination
+// axes as floats, map[i] the source axis feeding destination axis i.  The
+// per-element index scratch of the reference kernel is replaced by registers.
+struct PermuteArgs { int xs[8]; int ys[8]; int map[8]; int axes; };
+
+template <typename T> __global__ void transpose_kernel(size_t n, const T* x, T* y, PermuteArgs a)
+{
+    GRID_STRIDE(i, n)
+    {
+        int from[8];
+        size_t rem = i;
+        for (int d = 0; d < a.axes; d++) {
+            from[d] = (int)(rem / (size_t)a.xs[d]);
+            rem = rem % (size_t)a.xs[d];
+        }
+        size_t to = 0;
+        for (int d = 0; d < a.axes; d++) to += (size_t)from[a.map[d]] * (size_t)a.ys[d];
+        y[to] = x[i];
+    }
+}
+
+// (B, d1, d2, inner) -> (B, d2, d1, inner): the head split / merge of the attention layers
+template <typename T>
+__global__ void transpose12_kernel(const T* __restrict__ x, T* __restrict__ y, int d1, int d2, int inner, size_t n)
+{
+    GRID_STRIDE(o, n)
+    {
+        int in = (int)(o % inner);
+        size_t r = o / inner;
+        int a1 = (int)(r % d1);
+        r /= d1;
+        int a2 = (int)(r % d2);
+        size_t b = r / d2;
+        y[o] = x[((b * d1 + a1) * d2 + a2) * (size_t)inner + in];
+    }
+}
+
+hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
+                       const float* map, int axes)
+{
+    if (n == 0) return hipSuccess;
+    if (axes < 1 || axes > 8) return hipErrorInvalidValue;
+    float hx[8], hy[8], hm[8];
+    hipError_t e;
+    // the three tiny float blobs live on the device; fetch them once per call
+    if ((e = hipMemcpyAsync(hx, xc, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
+    if ((e = hipMemcpyAsync(hy, yc, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
+    if ((e = hipMemcpyAsync(hm, map, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
+    if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
+    PermuteArgs a;
+    a.axes = axes;
+    for (int i = 0; i < axes; i++) {
+        a.xs[i] = (int)hx[i];
+        a.ys[i] = (int)hy[i];
+        a.map[i] = (int)hm[i];
+        if (a.xs[i] < 1 || a.ys[i] < 1 || a.map[i] < 0 || a.map[i] >= axes) return hipErrorInvalidValue;
+    }
+    // fast path: 4 axes, axes 1 and 2 swapped, coalesced along the untouched inner axis
+    if (axes == 4 && a.map[0] == 0 && a.map[1] == 2 && a.map[2] == 1 && a.map[3] == 3 && a.xs[3] == 1 && a.ys[3] == 1) {
+        int inner = a.xs[2];
+        int d2 = a.xs[1] / a.xs[2];
+        int d1 = a.xs[0] / a.xs[1];
+        if (a.ys[2] == inner && a.ys[1] == inner * d1 && a.ys[0] == inner * d1 * d2) {
+            DISPATCH_DT(dt, hipLaunchKernelGGL(transpose12_kernel<T>, grid_for(n), TPB, 0, s, (const T*)x, (T*)y, d1, d2,
+                                               inner, n));
+            return hipGetLastError();
+        }
+    }
+    DISPATCH_DT(dt, hipLaunchKernelGGL(transpose_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, a));
+    return hipGetLastError();
+}
+
+// (nc, h, w) -> (nc, w, h) through a padded LDS tile so both sides are coalesced
+template <typename T> __global__ void transpose_hw_kernel(const T* __restrict__ x, T* __restrict__ y, int h, int w)
+{
+    __shared__ T tile[32][33];
+    size_t base = (size_t)blockIdx.z * h * w;
+    int x0 = blockIdx.x * 32, y0 = blockIdx.y * 32;
+    int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int j = ty; j < 32; j += 8)
+        if (y0 + j < h && x0 + tx < w) tile[j][tx] = x[base + (size_t)(y0 + j) * w + x0 + tx];
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8)
+        if (x0 + j < w && y0 + tx < h) y[base + (size_t)(x0 + j) * h + y0 + tx] = tile[tx][j];
+}
+
+hipError_t k_transpose_hw(hipStream_t s, DType dt, int nc, int h, int w, const void* x, void* y)
+{
+    if (nc <= 0 || h <= 0 || w <= 0) return hipSuccess;
+    dim3 grid((w + 31) / 32, (h + 31) / 32, nc);
+    if (grid.z > 65535 || grid.y > 65535) return hipErrorInvalidValue;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(transpose_hw_kernel<T>, grid, TPB, 0, s, (const T*)x, (T*)y, h, w));
+    return hipGetLastError();
+}
+
+// X viewed as (num, channels, blocks, inner), Y as (num, channels, inner);
+// dir 0: Y = X[:, :, offset, :], else X[:, :, offset, :] = Y
+template <typename T>
+__global__ void channel_copy_kernel(size_t n, int channels, int blocks, int inner, int offset, T* x, T* y, int dir)
+{
+    GRID_STRIDE(i, n)
+    {
+        size_t nn = i / ((size_t)channels * inner);
+        size_t c = (i % ((size_t)channels * inner)) / inner;
+        size_t b = i % inner;
+        size_t xi = (nn * channels + c) * (size_t)blocks * inner + (size_t)offset * inner + b;
+        if (dir == 0) y[i] = x[xi];
+        else x[xi] = y[i];
+    }
+}
+hipError_t k_channel_copy(hipStream_t s, DType dt, size_t n, int channels, int blocks, int inner, int offset, void* x,
+                          void* y, int dir)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_copy_kernel<T>, grid_for(n), TPB, 0, s, n, channels, blocks, inner, offset,
+                                       (T*)x, (T*)y, dir));
+    return hipGetLastError();
+}
+
+template <typename T> __global__ void embed_kernel(size_t count, const float* ids, const T* w, int N, T* top)
+{
+    GRID_STRIDE(i, count)
+    {
+        size_t nn = i / N;
+        int d = (int)(i % N);
+        long long idx = (long long)ids[nn];
+        long long wi = idx * N + d;
+        if (wi < 0) wi = -wi;
+        top[i] = w[wi];
+    }
+}
+hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, const void* w, int N, void* top)
+{
+    if (count == 0) return hipSuccess;
+    DISPATCH_DT(wdt, hipLaunchKernelGGL(embed_kernel<T>, grid_for(count), TPB, 0, s, count, ids, (const T*)w, N, (T*)top));
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// reductions
+__device__ inline float wave_max(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ inline float wave_sum(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+template <int NW> __device__ inline float block_max(float v, float* red)
+{
+    v = wave_max(v);
+    int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int i = 1; i < NW; i++) r = fmaxf(r, red[i]);
+    return r;
+}
+template <int NW> __device__ inline float block_sum(float v, float* red)
+{
+    v = wave_sum(v);
+    int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int i = 1; i < NW; i++) r += red[i];
+    return r;
+}
+
+// one workgroup per row (inner == 1); the row is read once into registers when it
+// fits (len <= 256*8) and re-read from L2 otherwise
+template <typename T> __global__ void softmax_rows_kernel(const T* x, T* y, int len, bool logsm)
+{
+    __shared__ float red[4];
+    const T* xr = x + (size_t)blockIdx.x * len;
+    T* yr = y + (size_t)blockIdx.x * len;
+    constexpr int R = 8;
+    float v[R];
+    bool cached = len <= TPB * R;
+    float mx = -INFINITY;
+    if (cached) {
+        for (int j = 0; j < R; j++) {
+            int i = threadIdx.x + j * TPB;
+            v[j] = i < len ? ld(xr, i) : -INFINITY;
+            mx = fmaxf(mx, v[j]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < len; i += TPB) mx = fmaxf(mx, ld(xr, i));
+    }
+    mx = block_max<4>(mx, red);
+    float sum = 0.f;
+    if (cached) {
+        for (int j = 0; j < R; j++) {
+            int i = threadIdx.x + j * TPB;
+            if (i < len) {
+                v[j] = expf(v[j] - mx);
+                sum += v[j];
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < len; i += TPB) sum += expf(ld(xr, i) - mx);
+    }
+    sum = block_sum<4>(sum, red);
+    if (logsm) {
+        float ls = logf(sum);
+        for (int i = threadIdx.x; i < len; i += TPB) st(yr, i, ld(xr, i) - mx - ls);
+        return;
+    }
+    if (cached) {
+        for (int j = 0; j < R; j++) {
+            int i = threadIdx.x + j * TPB;
+            if (i < len) st(yr, i, v[j] / sum);
+        }
+    } else {
+        for (int i = threadIdx.x; i < len; i += TPB) st(yr, i, expf(ld(xr, i) - mx) / sum);
+    }
+}
+
+// general (outer, len, inner): one thread per series
+template <typename T> __global__ void softmax_strided_kernel(const T* x, T* y, size_t series, int len, int inner, bool logsm)
+{
+    GRID_STRIDE(sidx, series)
+    {
+        size_t o = sidx / inner, in = sidx % inner;
+        size_t base = o * (size_t)len * inner + in;
+        float mx = -INFINITY;
+        for (int l = 0; l < len; l++) mx = fmaxf(mx, ld(x, base + (size_t)l * inner));
+        float sum = 0.f;
+        for (int l = 0; l < len; l++) sum += expf(ld(x, base + (size_t)l * inner) - mx);
+        float ls = logf(sum);
+        for (int l = 0; l < len; l++) {
+            float d = ld(x, base + (size_t)l * inner) - mx;
+            st(y, base + (size_t)l * inner, logsm ? d - ls : expf(d) / sum);
+        }
+    }
+}
+
+hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm)
+{
+    if (outer == 0 || len <= 0 || inner <= 0) return hipSuccess;
+    if (inner == 1) {
+        if (outer > 0x7fffffffu) return hipErrorInvalidValue;
+        DISPATCH_DT(dt, hipLaunchKernelGGL(softmax_rows_kernel<T>, (int)outer, TPB, 0, s, (const T*)x, (T*)y, len, logsm));
+    } else {
+        size_t series = outer * (size_t)inner;
+        DISPATCH_DT(dt, hipLaunchKernelGGL(softmax_strided_kernel<T>, grid_for(series), TPB, 0, s, (const T*)x, (T*)y, series,
+                                           len, inner, logsm));
+    }
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// RoPE: pair p = (x[2p], x[2p+1]); table row = (p % (seqLen*heads*half)) / (heads*half),
+// column = p % half; one fused pass replaces the reference's three kernels.
+template <typename T>
+__global__ void rope_kernel(size_t pairs, const T* x, T* y, const float* __restrict__ fcos, const float* __restrict__ fsin,
+                            int seqLen, int heads, int half, int tableOff)
+{
+    size_t full = (size_t)heads * half;
+    size_t wrap = (size_t)seqLen * full;
+    GRID_STRIDE(p, pairs)
+    {
+        size_t base = p % wrap;
+        size_t t = (base / full) * half + base % half + tableOff;
+        float c = fcos[t], sn = fsin[t];
+        float re = ld(x, 2 * p), im = ld(x, 2 * p + 1);
+        st(y, 2 * p, re * c - im * sn);
+        st(y, 2 * p + 1, re * sn + im * c);
+    }
+}
+
+hipError_t k_rope(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* fcos, const float* fsin,
+                  int seqLen, int heads, int hs, int tableOff)
+{
+    size_t pairs = n / 2;
+    if (pairs == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(rope_kernel<T>, grid_for(pairs), TPB, 0, s, pairs, (const T*)x, (T*)y, fcos, fsin,
+                                       seqLen, heads, hs / 2, tableOff));
+    return hipGetLastError();
+}
+
+// y = w * (x / sqrt(mean(x^2) + eps)); one workgroup per row
+template <typename T> __global__ void rmsnorm_kernel(int dim, const T* x, const T* w, T* y, float eps)
+{
+    __shared__ float red[4];
+    const T* xr = x + (size_t)blockIdx.x * dim;
+    T* yr = y + (size_t)blockIdx.x * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += TPB) {
+        float v = ld(xr, i);
+        ss += v * v;
+    }
+    ss = block_sum<4>(ss, red);
+    float inv = 1.0f / sqrtf(ss / dim + eps);
+    for (int i = threadIdx.x; i < dim; i += TPB) {
+        float v = inv * ld(xr, i);
+        st(yr, i, w ? ld(w, i) * v : v);
+    }
+}
+
+hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps)
+{
+    if (outer <= 0 || dim <= 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(rmsnorm_kernel<T>, outer, TPB, 0, s, dim, (const T*)x, (const T*)w, (T*)y, eps));
+    return hipGetLastError();
+}
+
+}  // namespace mch

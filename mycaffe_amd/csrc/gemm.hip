@@ -1,0 +1,419 @@
+// GEMM / GEMV kernels for gfx950.
+//
+//  * gemm_nt_f32_mfma  : C = alpha*A[M,K]*B[N,K]^T + beta*C, fp32 in, fp32 MFMA
+//                        (v_mfma_f32_32x32x2_f32), 128x128x16 LDS-staged tiles.
+//                        This is the InnerProduct shape (weights stored [N,K]).
+//  * gemm_nt_bf16_mfma : same contraction on bf16 storage with
+//                        v_mfma_f32_32x32x16_bf16, fp32 accumulate, 128x128x32 tiles.
+//  * gemm_generic      : any transpose / stride combination (row-major gemm with
+//                        transposed operands, column-major strided-batched gemm2),
+//                        64x64x16 LDS tiles, fp32 FMA.
+//  * gemv              : HBM-bound y = A x, one wavefront per row, 128-bit loads.
+#include "kernels.h"
+
+namespace mch {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T> __device__ inline float ldf(const T* p, size_t i);
+template <> __device__ inline float ldf<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ inline float ldf<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+template <typename T> __device__ inline void stf(T* p, size_t i, float v);
+template <> __device__ inline void stf<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ inline void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+// ---------------------------------------------------------------------------
+// generic strided GEMM: C(i,j) = alpha * sum_k A(i,k) B(k,j) + beta * C(i,j)
+// element addresses: A[i*ai + k*ak], B[k*bk + j*bj], C[i*ci + j*cj]; blockIdx.z = batch
+struct GemmStrides { long long ai, ak, bk, bj, ci, cj, sA, sB, sC; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
+                                                           const T* __restrict__ B, float beta, T* __restrict__ C,
+                                                           GemmStrides st)
+{
+    constexpr int BM = 64, BN = 64, BK = 16;
+    __shared__ float As[BK][BM + 4];
+    __shared__ float Bs[BK][BN + 4];
+    A += (size_t)blockIdx.z * st.sA;
+    B += (size_t)blockIdx.z * st.sB;
+    C += (size_t)blockIdx.z * st.sC;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int tid = threadIdx.x;
+    const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+    // pick the load order that walks the unit-stride axis with consecutive threads
+    const bool a_k_fast = st.ak == 1;
+    const bool b_k_fast = st.bk == 1;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        for (int e = tid; e < BM * BK; e += 256) {
+            int i, k;
+            if (a_k_fast) { i = e / BK; k = e % BK; } else { k = e / BM; i = e % BM; }
+            float v = 0.f;
+            if (m0 + i < M && k0 + k < K) v = ldf(A, (size_t)((long long)(m0 + i) * st.ai + (long long)(k0 + k) * st.ak));
+            As[k][i] = v;
+        }
+        for (int e = tid; e < BN * BK; e += 256) {
+            int j, k;
+            if (b_k_fast) { j = e / BK; k = e % BK; } else { k = e / BN; j = e % BN; }
+            float v = 0.f;
+            if (n0 + j < N && k0 + k < K) v = ldf(B, (size_t)((long long)(k0 + k) * st.bk + (long long)(n0 + j) * st.bj));
+            Bs[k][j] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; k++) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = As[k][tm + i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = Bs[k][tn + j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++) {
+            int r = m0 + tm + i, c = n0 + tn + j;
+            if (r < M && c < N) {
+                size_t ci = (size_t)((long long)r * st.ci + (long long)c * st.cj);
+                float v = alpha * acc[i][j];
+                if (beta != 0.f) v += beta * ldf(C, ci);
+                stf(C, ci, v);
+            }
+        }
+}
+
+template <typename T>
+static hipError_t launch_generic(hipStream_t s, int M, int N, int K, float alpha, const T* A, const T* B, float beta, T* C,
+                                 GemmStrides st, int batch)
+{
+    if (M <= 0 || N <= 0 || batch <= 0) return hipSuccess;
+    dim3 grid((N + 63) / 64, (M + 63) / 64, batch);
+    if (grid.y > 65535 || grid.z > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gemm_generic_kernel<T>, grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// fp32 MFMA, NT.  4 wavefronts in a 2x2 arrangement, each owning 64x64 of the
+// 128x128 tile as 2x2 MFMA 32x32 blocks.  One 128-bit LDS read feeds four
+// MFMA steps: lane group g (= lane/32) holds k = kk+4g .. kk+4g+3, and MFMA step
+// j contracts the two slots {kk+j, kk+4+j}; the slot-to-k assignment is free as
+// long as A and B use the same one.
+__global__ __launch_bounds__(256) void gemm_nt_f32_mfma_kernel(int M, int N, int K, float alpha,
+                                                               const float* __restrict__ A,
+                                                               const float* __restrict__ B, float beta,
+                                                               float* __restrict__ C)
+{
+    constexpr int BM = 128, BN = 128, BK = 16, LDK = BK + 4;
+    __shared__ __attribute__((aligned(16))) float As[2][BM * LDK];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN * LDK];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int lr = tid >> 2, lc = (tid & 3) * 4;  // 64 rows x 4 float4 per pass, 2 passes
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    float4 ra[2], rb[2];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int r = lr + p * 64;
+            ra[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            rb[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m0 + r < M && k0 + lc < K) ra[p] = *(const float4*)(A + (size_t)(m0 + r) * K + k0 + lc);
+            if (n0 + r < N && k0 + lc < K) rb[p] = *(const float4*)(B + (size_t)(n0 + r) * K + k0 + lc);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int r = lr + p * 64;
+            *(float4*)(&As[buf][r * LDK + lc]) = ra[p];
+            *(float4*)(&Bs[buf][r * LDK + lc]) = rb[p];
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    gload(0);
+    sstore(0);
+    __syncthreads();
+    const int fr = lane & 31, fg = (lane >> 5) * 4;
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 8) {
+            float4 a[2], b[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                a[t] = *(const float4*)(&As[buf][(wm + t * 32 + fr) * LDK + kk + fg]);
+                b[t] = *(const float4*)(&Bs[buf][(wn + t * 32 + fr) * LDK + kk + fg]);
+            }
+            const float* af0 = (const float*)&a[0];
+            const float* af1 = (const float*)&a[1];
+            const float* bf0 = (const float*)&b[0];
+            const float* bf1 = (const float*)&b[1];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af0[j], bf0[j], acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af0[j], bf1[j], acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af1[j], bf0[j], acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af1[j], bf1[j], acc[1][1], 0, 0, 0);
+            }
+        }
+        if (kt + 1 < nk) sstore(buf ^ 1);
+        __syncthreads();
+    }
+    // accumulator register v of a 32x32 block: row = 8*(v/4) + 4*(lane/32) + v%4, col = lane%32
+    const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            int c = n0 + wn + j * 32 + col_l;
+            if (c >= N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                int r = m0 + wm + i * 32 + (v >> 2) * 8 + row_l + (v & 3);
+                if (r < M) {
+                    size_t ci = (size_t)r * N + c;
+                    float o = alpha * acc[i][j][v];
+                    if (beta != 0.f) o += beta * C[ci];
+                    C[ci] = o;
+                }
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
+// bf16 MFMA, NT, 128x128x32 tiles, 4 wavefronts each 64x64 (2x2 MFMA 32x32x16).
+// Lane l feeds row l%32 with the eight k values 8*(l/32) .. 8*(l/32)+7 of a
+// 16-wide MFMA step: one 128-bit LDS read per operand block and step.
+__global__ __launch_bounds__(256) void gemm_nt_bf16_mfma_kernel(int M, int N, int K, float alpha,
+                                                                const bf16_t* __restrict__ A,
+                                                                const bf16_t* __restrict__ B, float beta,
+                                                                bf16_t* __restrict__ C)
+{
+    constexpr int BM = 128, BN = 128, BK = 32, LDK = BK + 8;  // row stride 80 B
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BN * LDK];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int lr = tid >> 2, lc = (tid & 3) * 8;  // 64 rows x 4 x (8 bf16) per pass, 2 passes
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    uint4 ra[2], rb[2];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int r = lr + p * 64;
+            ra[p] = make_uint4(0, 0, 0, 0);
+            rb[p] = make_uint4(0, 0, 0, 0);
+            if (m0 + r < M && k0 + lc < K) ra[p] = *(const uint4*)(A + (size_t)(m0 + r) * K + k0 + lc);
+            if (n0 + r < N && k0 + lc < K) rb[p] = *(const uint4*)(B + (size_t)(n0 + r) * K + k0 + lc);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            int r = lr + p * 64;
+            *(uint4*)(&As[buf][r * LDK + lc]) = ra[p];
+            *(uint4*)(&Bs[buf][r * LDK + lc]) = rb[p];
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    gload(0);
+    sstore(0);
+    __syncthreads();
+    const int fr = lane & 31, fg = (lane >> 5) * 8;
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            bf16x8 a[2], b[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                a[t] = *(const bf16x8*)(&As[buf][(wm + t * 32 + fr) * LDK + kk + fg]);
+                b[t] = *(const bf16x8*)(&Bs[buf][(wn + t * 32 + fr) * LDK + kk + fg]);
+            }
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[1], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[0], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[1], acc[1][1], 0, 0, 0);
+        }
+        if (kt + 1 < nk) sstore(buf ^ 1);
+        __syncthreads();
+    }
+    const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            int c = n0 + wn + j * 32 + col_l;
+            if (c >= N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                int r = m0 + wm + i * 32 + (v >> 2) * 8 + row_l + (v & 3);
+                if (r < M) {
+                    size_t ci = (size_t)r * N + c;
+                    float o = alpha * acc[i][j][v];
+                    if (beta != 0.f) o += beta * bf16_to_f32(C[ci]);
+                    C[ci] = f32_to_bf16(o);
+                }
+            }
+        }
+}
+
+hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
+                  const void* B, float beta, void* C)
+{
+    if (m <= 0 || n <= 0) return hipSuccess;
+    if (k <= 0) k = 0;
+    // MFMA fast path: A (m,k) and B (n,k) both k-contiguous, 16-byte aligned rows
+    const int vec = dt == F32 ? 4 : 8;
+    bool aligned = (k % vec == 0) && (((uintptr_t)A | (uintptr_t)B) % 16 == 0) && k >= vec;
+    if (!tA && tB && aligned) {
+        dim3 grid((n + 127) / 128, (m + 127) / 128);
+        if (grid.y > 65535) return hipErrorInvalidValue;
+        if (dt == F32)
+            hipLaunchKernelGGL(gemm_nt_f32_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const float*)A, (const float*)B,
+                               beta, (float*)C);
+        else
+            hipLaunchKernelGGL(gemm_nt_bf16_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const bf16_t*)A,
+                               (const bf16_t*)B, beta, (bf16_t*)C);
+        return hipGetLastError();
+    }
+    GemmStrides st;
+    st.ai = tA ? 1 : k;  st.ak = tA ? m : 1;   // A stored (m,k) or (k,m)
+    st.bk = tB ? 1 : n;  st.bj = tB ? k : 1;   // B stored (k,n) or (n,k)
+    st.ci = n;           st.cj = 1;
+    st.sA = st.sB = st.sC = 0;
+    if (dt == F32)
+        return launch_generic<float>(s, m, n, k, alpha, (const float*)A, (const float*)B, beta, (float*)C, st, 1);
+    return launch_generic<bf16_t>(s, m, n, k, alpha, (const bf16_t*)A, (const bf16_t*)B, beta, (bf16_t*)C, st, 1);
+}
+
+hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
+                   float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch)
+{
+    // column-major: op(A)(i,kk) = tA ? A[kk + i*lda] : A[i + kk*lda]
+    GemmStrides st;
+    st.ai = tA ? lda : 1;  st.ak = tA ? 1 : lda;
+    st.bk = tB ? ldb : 1;  st.bj = tB ? 1 : ldb;
+    st.ci = 1;             st.cj = ldc;
+    st.sA = sA; st.sB = sB; st.sC = sC;
+    return launch_generic<float>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+}
+
+// ---------------------------------------------------------------------------
+// GEMV, not transposed: one wavefront per row, 128-bit loads along the row.
+template <typename T> struct VecLoad;
+template <> struct VecLoad<float> {
+    static constexpr int W = 4;
+    __device__ static inline float dot(const float* a, const float* x)
+    {
+        float4 av = *(const float4*)a, xv = *(const float4*)x;
+        return av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
+    }
+};
+template <> struct VecLoad<bf16_t> {
+    static constexpr int W = 8;
+    __device__ static inline float dot(const bf16_t* a, const float* x)
+    {
+        uint4 av = *(const uint4*)a;
+        float4 x0 = *(const float4*)x, x1 = *(const float4*)(x + 4);
+        const uint32_t u[4] = {av.x, av.y, av.z, av.w};
+        const float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            acc += __uint_as_float(u[i] << 16) * xs[2 * i];
+            acc += __uint_as_float(u[i] & 0xffff0000u) * xs[2 * i + 1];
+        }
+        return acc;
+    }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_n_kernel(int m, int n, float alpha, const T* __restrict__ A,
+                                                     const float* __restrict__ x, float beta, float* __restrict__ y)
+{
+    constexpr int W = VecLoad<T>::W;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= m) return;
+    const T* a = A + (size_t)row * n;
+    float acc = 0.f;
+    const bool vec_ok = (n % W == 0) && (((uintptr_t)a % 16) == 0) && (((uintptr_t)x % 16) == 0);
+    if (vec_ok) {
+        for (int j = lane * W; j < n; j += 64 * W) acc += VecLoad<T>::dot(a + j, x + j);
+    } else {
+        for (int j = lane; j < n; j += 64) acc += ldf(a, j) * x[j];
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) {
+        float v = alpha * acc;
+        if (beta != 0.f) v += beta * y[row];
+        y[row] = v;
+    }
+}
+
+// transposed: y[j] = sum_i A[i,j] x[i]; consecutive threads walk consecutive columns
+template <typename T>
+__global__ void gemv_t_kernel(int m, int n, float alpha, const T* __restrict__ A, const float* __restrict__ x, float beta,
+                              float* __restrict__ y)
+{
+    int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    float acc = 0.f;
+    for (int i = 0; i < m; i++) acc += ldf(A, (size_t)i * n + j) * x[i];
+    float v = alpha * acc;
+    if (beta != 0.f) v += beta * y[j];
+    y[j] = v;
+}
+
+hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x, float beta,
+                  float* y)
+{
+    if (m <= 0 || n <= 0) return hipSuccess;
+    if (!tA) {
+        int grid = (m + 3) / 4;
+        if (adt == F32)
+            hipLaunchKernelGGL(gemv_n_kernel<float>, grid, 256, 0, s, m, n, alpha, (const float*)A, x, beta, y);
+        else
+            hipLaunchKernelGGL(gemv_n_kernel<bf16_t>, grid, 256, 0, s, m, n, alpha, (const bf16_t*)A, x, beta, y);
+    } else {
+        int grid = (n + 255) / 256;
+        if (adt == F32)
+            hipLaunchKernelGGL(gemv_t_kernel<float>, grid, 256, 0, s, m, n, alpha, (const float*)A, x, beta, y);
+        else
+            hipLaunchKernelGGL(gemv_t_kernel<bf16_t>, grid, 256, 0, s, m, n, alpha, (const bf16_t*)A, x, beta, y);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace mch

@@ -1,0 +1,90 @@
+// Host-side launchers of the gfx950 kernels.  Every launcher enqueues on the
+// given stream and returns the launch status; none of them synchronises.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mch {
+
+// storage type of a device buffer: fp32 or bf16 (the library's 16-bit storage)
+enum DType { F32 = 0, BF16 = 1 };
+
+typedef uint16_t bf16_t;
+
+__host__ __device__ inline float bf16_to_f32(bf16_t v)
+{
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)v) << 16;
+    return c.f;
+}
+
+// round to nearest even; NaN stays NaN
+__host__ __device__ inline bf16_t f32_to_bf16(float f)
+{
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    if ((c.u & 0x7fffffffu) > 0x7f800000u)
+        return (bf16_t)((c.u >> 16) | 0x40);
+    uint32_t r = 0x7fffu + ((c.u >> 16) & 1u);
+    return (bf16_t)((c.u + r) >> 16);
+}
+
+// ---- elementwise and layout kernels (ew_kernels.hip) ----------------------
+hipError_t k_set(hipStream_t s, DType dt, void* y, size_t n, float v);
+hipError_t k_convert(hipStream_t s, DType sdt, const void* src, DType ddt, void* dst, size_t n);
+hipError_t k_axpy(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y);
+hipError_t k_scale(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y);
+hipError_t k_add(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, float alpha);
+hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y);
+hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y);
+hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y);
+hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
+                  const void* mask, void* y);
+hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDim, float search, float replace,
+                        const void* x, const void* mask, void* y);
+hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
+                       const float* map, int axes);
+hipError_t k_transpose_hw(hipStream_t s, DType dt, int nc, int h, int w, const void* x, void* y);
+hipError_t k_channel_copy(hipStream_t s, DType dt, size_t n, int channels, int blocks, int inner, int offset,
+                          void* x, void* y, int dir);
+hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, const void* w, int N, void* top);
+// softmax over `len` for outer x inner independent series; element (o, l, i) at (o*len + l)*inner + i
+hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm);
+// adjacent-pair rotary embedding with the CudaDnnDLL index rule; x == y allowed
+hipError_t k_rope(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* fcos, const float* fsin,
+                  int seqLen, int heads, int hs, int tableOff);
+hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps);
+
+// ---- GEMM family (gemm.hip) ------------------------------------------------
+// row-major C[m,n] = alpha*op(A)*op(B) + beta*C; A, B, C all of storage type dt
+hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
+                  const void* B, float beta, void* C);
+// column-major strided batched gemm with BLAS semantics (fp32)
+hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
+                   float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
+                   int batch);
+// A row-major (m,n) of type adt; x, y fp32.  y = alpha*A*x + beta*y, or with tA y = alpha*A^T*x + beta*y
+hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x,
+                  float beta, float* y);
+
+// ---- attention (attn_prefill.hip, attn_decode.hip) --------------------------
+enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAUSAL = 4 };
+// q (B,H,Tq,hs), k/v (B,H,Tk,hs), y (B,H,Tq,hs), all dt.  mask is fp32:
+//   MASK_QK (Tq,Tk) shared, MASK_KEY (B,Tk), MASK_BQK (B,Tq,Tk); zero entries are filled with -1e29.
+//   MASK_CAUSAL needs no mask buffer (lower triangle kept).
+hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind);
+// returns true if mask (Tq,Tk) on the device equals the lower-triangular ones matrix; cached by the caller
+size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
+// one query per (b,h): q (B,H,hs), caches addressed as
+//   cache[b*strideB + (h/kvMul)*strideH + t*strideT + i], y (B,H,hs).  All dt.
+hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc, const void* vc, void* y, int B, int H,
+                         int kvH, int hs, int len, long long strideB, long long strideH, long long strideT,
+                         float scale, void* workspace, size_t workspaceBytes);
+// rotate q (B,H,hs) and knew (B,kvH,hs) at position pos and append knew/vnew to the caches at pos
+hipError_t k_rope_append(hipStream_t s, DType dt, void* q, void* knew, const void* vnew, void* kc, void* vc, int B,
+                         int H, int kvH, int hs, int pos, long long strideB, long long strideH, long long strideT,
+                         const float* fcos, const float* fsin);
+
+}  // namespace mch

@@ -1,0 +1,1417 @@
+// libmycaffe_hip.so: exported C ABI, kernel table, argument unmarshalling.
+//
+// Every case of Kernel::run reproduces the argument positions of the reference's
+// Device<T> unmarshaller for that function id (CudaDnnDLL/Cuda Files/device.cu,
+// device.h; positions are quoted per case) and then enqueues hand-written gfx950
+// kernels on the kernel's own HIP stream.  Compute calls return without waiting;
+// calls that hand data to the host (GETMEM, SYNCHRONIZEDEVICE, extension results)
+// wait for the stream, so "returned means visible" holds for everything the host
+// can observe.
+#include <dlfcn.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <climits>
+
+#include "runtime.h"
+
+namespace mch {
+
+#define HIPCHK(x) do { hipError_t _e = (x); if (_e != hipSuccess) return (long)_e; } while (0)
+#define ERRCHK(x) do { long _e = (x); if (_e) return _e; } while (0)
+
+// ---------------------------------------------------------------------------
+std::string utf16_to_utf8(const MCH_TCHAR* s)
+{
+    std::string out;
+    if (!s) return out;
+    for (; *s; s++) {
+        uint32_t c = *s;
+        if (c >= 0xD800 && c <= 0xDBFF && s[1] >= 0xDC00 && s[1] <= 0xDFFF) {
+            c = 0x10000 + ((c - 0xD800) << 10) + (s[1] - 0xDC00);
+            s++;
+        }
+        if (c < 0x80) out += (char)c;
+        else if (c < 0x800) { out += (char)(0xC0 | (c >> 6)); out += (char)(0x80 | (c & 0x3F)); }
+        else if (c < 0x10000) { out += (char)(0xE0 | (c >> 12)); out += (char)(0x80 | ((c >> 6) & 0x3F)); out += (char)(0x80 | (c & 0x3F)); }
+        else { out += (char)(0xF0 | (c >> 18)); out += (char)(0x80 | ((c >> 12) & 0x3F)); out += (char)(0x80 | ((c >> 6) & 0x3F)); out += (char)(0x80 | (c & 0x3F)); }
+    }
+    return out;
+}
+
+void utf8_to_utf16(const std::string& s, MCH_TCHAR* out, long max)
+{
+    if (!out || max <= 0) return;
+    long o = 0;
+    for (size_t i = 0; i < s.size() && o < max - 1;) {
+        uint32_t c = (unsigned char)s[i];
+        int n = c < 0x80 ? 1 : (c >> 5) == 6 ? 2 : (c >> 4) == 14 ? 3 : 4;
+        if (n == 2) c &= 0x1F; else if (n == 3) c &= 0x0F; else if (n == 4) c &= 0x07;
+        for (int j = 1; j < n && i + j < s.size(); j++) c = (c << 6) | ((unsigned char)s[i + j] & 0x3F);
+        i += n;
+        if (c >= 0x10000) {
+            if (o >= max - 2) break;
+            c -= 0x10000;
+            out[o++] = (MCH_TCHAR)(0xD800 + (c >> 10));
+            out[o++] = (MCH_TCHAR)(0xDC00 + (c & 0x3FF));
+        } else out[o++] = (MCH_TCHAR)c;
+    }
+    out[o] = 0;
+}
+
+// ---------------------------------------------------------------------------
+long MemTable::new_slot()
+{
+    if (!m_free.empty()) { long h = m_free.back(); m_free.pop_back(); return h; }
+    m_items.emplace_back();
+    return (long)m_items.size() - 1;
+}
+
+long MemTable::alloc(size_t count, bool half, hipStream_t s, long* h)
+{
+    void* p = nullptr;
+    size_t bytes = count * (half ? 2 : 4);
+    if (bytes == 0) bytes = 4;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return e == hipErrorOutOfMemory ? (long)MCH_ERROR_MEMORY_OUT : (long)e;
+    // every device allocation starts zero-filled (memorycol.h:75-107); callers rely on it
+    e = hipMemsetAsync(p, 0, bytes, s);
+    if (e != hipSuccess) { (void)hipFree(p); return (long)e; }
+    long slot = new_slot();
+    MemItem& it = m_items[slot];
+    it = MemItem();
+    it.ptr = p; it.count = count; it.half = half; it.used = true;
+    *h = slot;
+    return 0;
+}
+
+long MemTable::alloc_view(long hBase, size_t offset, size_t count, long* h)
+{
+    MemItem* b;
+    ERRCHK(get(hBase, &b));
+    if (offset + count > b->count) return MCH_ERROR_MEMORY_RANGE_EXCEEDED;
+    long root = b->view ? b->base : hBase;
+    char* p = (char*)b->ptr + offset * b->esize();
+    bool half = b->half;
+    long slot = new_slot();
+    MemItem& it = m_items[slot];  // b may dangle after new_slot(); not used below
+    it = MemItem();
+    it.ptr = p; it.count = count; it.half = half; it.used = true; it.view = true; it.base = root;
+    *h = slot;
+    return 0;
+}
+
+long MemTable::get(long h, MemItem** it)
+{
+    if (h <= 0 || (size_t)h >= m_items.size() || !m_items[h].used) return MCH_ERROR_MEMORY_NOT_FOUND;
+    *it = &m_items[h];
+    return 0;
+}
+
+long MemTable::free(long h)
+{
+    MemItem* it;
+    ERRCHK(get(h, &it));
+    if (!it->view) {
+        // views of this allocation die with it
+        for (size_t i = 1; i < m_items.size(); i++)
+            if (m_items[i].used && m_items[i].view && m_items[i].base == h) { m_items[i] = MemItem(); m_free.push_back((long)i); }
+        hipError_t e = hipFree(it->ptr);
+        if (e != hipSuccess) return (long)e;
+    }
+    *it = MemItem();
+    m_free.push_back(h);
+    return 0;
+}
+
+void MemTable::touch(long h)
+{
+    MemItem* it;
+    if (get(h, &it)) return;
+    it->version++;
+    if (it->view && !get(it->base, &it)) it->version++;
+}
+
+uint64_t MemTable::version(long h)
+{
+    MemItem* it;
+    if (get(h, &it)) return 0;
+    uint64_t v = it->version;
+    if (it->view && !get(it->base, &it)) v += it->version << 20;
+    return v;
+}
+
+void MemTable::free_all()
+{
+    for (size_t i = 1; i < m_items.size(); i++)
+        if (m_items[i].used && !m_items[i].view) (void)hipFree(m_items[i].ptr);
+    m_items.assign(1, MemItem());
+    m_free.clear();
+}
+
+ExtensionState::~ExtensionState()
+{
+    if (lib) dlclose(lib);
+}
+
+// ---------------------------------------------------------------------------
+Kernel::Kernel() {}
+
+Kernel::~Kernel()
+{
+    if (m_stream) (void)hipStreamSynchronize(m_stream);
+    m_ext.clear();
+    m_rope.clear();
+    m_mem.free_all();
+    if (m_ws) (void)hipFree(m_ws);
+    if (m_stage) (void)hipHostFree(m_stage);
+    for (float* p : m_hostAllocs) (void)hipHostFree(p);
+    if (m_stream) (void)hipStreamDestroy(m_stream);
+}
+
+long Kernel::initialize(const float* pf, long n)
+{
+    // SetDevice: f{deviceId, flags[, seed]} (device.cu:772-795)
+    if (n < 2 || n > 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    if (!pf) return MCH_ERROR_PARAM_NULL;
+    int count = 0;
+    HIPCHK(hipGetDeviceCount(&count));
+    int dev = (int)pf[0];
+    if (dev < 0 || dev >= count) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    m_device = dev;
+    HIPCHK(hipSetDevice(dev));
+    if (!m_stream) HIPCHK(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking));
+    return 0;
+}
+
+std::string Kernel::device_name()
+{
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, m_device) != hipSuccess) return "unknown";
+    char buf[512];
+    snprintf(buf, sizeof(buf), "%s (%s, %d CUs, %.1f GB)", p.name, p.gcnArchName, p.multiProcessorCount,
+             (double)p.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+    return buf;
+}
+
+long Kernel::workspace(size_t bytes, void** p)
+{
+    if (bytes > m_wsBytes) {
+        if (m_ws) { HIPCHK(hipStreamSynchronize(m_stream)); HIPCHK(hipFree(m_ws)); m_ws = nullptr; m_wsBytes = 0; }
+        size_t want = bytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : bytes + bytes / 4;
+        HIPCHK(hipMalloc(&m_ws, want));
+        m_wsBytes = want;
+    }
+    *p = m_ws;
+    return 0;
+}
+
+long Kernel::staging(size_t bytes, void** p)
+{
+    if (bytes > m_stageBytes) {
+        if (m_stage) { HIPCHK(hipStreamSynchronize(m_stream)); HIPCHK(hipHostFree(m_stage)); m_stage = nullptr; m_stageBytes = 0; }
+        size_t want = bytes < (size_t)(4u << 20) ? (size_t)(4u << 20) : bytes + bytes / 4;
+        HIPCHK(hipHostMalloc(&m_stage, want, hipHostMallocDefault));
+        m_stageBytes = want;
+    }
+    *p = m_stage;
+    return 0;
+}
+
+long Kernel::alloc_host(long count, float** dst, const float* src, bool srcOnDevice)
+{
+    if (count < 0 || !dst) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    float* p = nullptr;
+    HIPCHK(hipHostMalloc((void**)&p, (size_t)(count > 0 ? count : 1) * sizeof(float), hipHostMallocDefault));
+    if (src && count > 0) {
+        if (srcOnDevice) {
+            hipError_t e = hipMemcpyAsync(p, src, (size_t)count * 4, hipMemcpyDeviceToHost, m_stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(m_stream);
+            if (e != hipSuccess) { (void)hipHostFree(p); return (long)e; }
+        } else memcpy(p, src, (size_t)count * 4);
+    }
+    std::lock_guard<std::mutex> g(m_hostLock);
+    m_hostAllocs.push_back(p);
+    *dst = p;
+    return 0;
+}
+
+long Kernel::free_host(float* p)
+{
+    std::lock_guard<std::mutex> g(m_hostLock);
+    for (size_t i = 0; i < m_hostAllocs.size(); i++)
+        if (m_hostAllocs[i] == p) {
+            m_hostAllocs.erase(m_hostAllocs.begin() + i);
+            HIPCHK(hipHostFree(p));
+            return 0;
+        }
+    return MCH_ERROR_MEMORY_NOT_FOUND;
+}
+
+long Kernel::get_pointer(long h, void** pp)
+{
+    MemItem* it;
+    ERRCHK(mem(h, &it));
+    *pp = it->ptr;
+    return 0;
+}
+
+static inline long verify(long n, const void* p, long lo, long hi)
+{
+    // verifyInput (device.h:712-745)
+    if (n < lo || n > hi) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    if (lo == 0 && hi == 0) return 0;
+    if (!p) return MCH_ERROR_PARAM_NULL;
+    return 0;
+}
+
+static inline long set_out(float v, float** ppOut, MCH_LONG* plOut)
+{
+    if (!plOut || !ppOut || !*ppOut) return MCH_ERROR_PARAM_NULL;
+    if (*plOut < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    *plOut = 1;
+    (*ppOut)[0] = v;
+    return 0;
+}
+
+__global__ void check_tril_kernel(const float* m, int T, int* bad)
+{
+    size_t n = (size_t)T * T;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)blockDim.x * gridDim.x) {
+        int r = (int)(i / T), c = (int)(i % T);
+        float want = c <= r ? 1.f : 0.f;
+        // any non-zero on/below the diagonal keeps the entry, so only zero-ness matters
+        if ((m[i] == 0.f) != (want == 0.f)) *bad = 1;
+    }
+}
+
+// true when the (T,T) mask keeps exactly the lower triangle; result cached per
+// (handle, content version, T) so the scan and its host read-back happen once
+bool Kernel::mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T)
+{
+    uint64_t ver = m_mem.version(hMask);
+    if (st->maskHandle == hMask && st->maskVersion == ver && st->maskT == T) return st->maskCausal;
+    void* ws;
+    if (workspace(256, &ws)) return false;
+    int* flag = (int*)ws;
+    if (hipMemsetAsync(flag, 0, sizeof(int), m_stream) != hipSuccess) return false;
+    size_t n = (size_t)T * T;
+    int grid = (int)((n + 255) / 256);
+    if (grid > 2048) grid = 2048;
+    hipLaunchKernelGGL(check_tril_kernel, grid, 256, 0, m_stream, (const float*)mask->ptr, T, flag);
+    int bad = 1;
+    if (hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, m_stream) != hipSuccess) return false;
+    if (hipStreamSynchronize(m_stream) != hipSuccess) return false;
+    st->maskHandle = hMask; st->maskVersion = ver; st->maskT = T; st->maskCausal = (bad == 0);
+    return st->maskCausal;
+}
+
+#define NEED_L(lo, hi) ERRCHK(verify(ll, pl, lo, hi))
+#define NEED_F(lo, hi) ERRCHK(verify(lf, pf, lo, hi))
+#define RANGE(item, off, n) do { if ((long long)(off) < 0 || (long long)(n) < 0 || (size_t)(off) + (size_t)(n) > (item)->count) { \
+        last_detail = "range exceeds the allocation behind the memory handle"; return MCH_ERROR_MEMORY_RANGE_EXCEEDED; } } while (0)
+#define PTR(item, off) ((char*)(item)->ptr + (size_t)(off) * (item)->esize())
+
+long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float** ppOut, MCH_LONG* plOut, bool timing)
+{
+    (void)timing;
+    last_detail.clear();
+    hipStream_t s = m_stream;
+    if (!s) return MCH_ERROR_DEVICE_NOT_INITIALIZED;
+    HIPCHK(hipSetDevice(m_device));
+
+    switch (fn) {
+    case MCH_FN_SETDEVICE:
+        return initialize(pf, lf);
+
+    case MCH_FN_GETDEVICE:
+        return set_out((float)m_device, ppOut, plOut);
+
+    case MCH_FN_SYNCHRONIZEDEVICE:
+        HIPCHK(hipStreamSynchronize(s));
+        return 0;
+
+    // ---- memory ------------------------------------------------------------
+    case MCH_FN_ALLOCMEM:
+    case MCH_FN_ALLOCMEM_HALF: {
+        // l{count[,stream]}; optional f{count,[stream,] data...} (device.cu:854-949)
+        NEED_L(1, 2);
+        if (pl[0] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        size_t count = (size_t)pl[0];
+        const float* src = nullptr;
+        if (lf > 1) {
+            if (!pf) return MCH_ERROR_PARAM_NULL;
+            if ((size_t)lf == count + 1) src = pf + 1;
+            else if ((size_t)lf == count + 2) src = pf + 2;
+            else return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        bool half = fn == MCH_FN_ALLOCMEM_HALF;
+        long h = 0;
+        ERRCHK(m_mem.alloc(count, half, s, &h));
+        if (src && count) {
+            MemItem* it;
+            ERRCHK(mem(h, &it));
+            long e = 0;
+            if (!half) {
+                hipError_t he = hipMemcpyAsync(it->ptr, src, count * 4, hipMemcpyHostToDevice, s);
+                if (he == hipSuccess) he = hipStreamSynchronize(s);
+                e = (long)he;
+            } else {
+                void* ws;
+                e = workspace(count * 4, &ws);
+                if (!e) {
+                    hipError_t he = hipMemcpyAsync(ws, src, count * 4, hipMemcpyHostToDevice, s);
+                    if (he == hipSuccess) he = k_convert(s, F32, ws, BF16, it->ptr, count);
+                    if (he == hipSuccess) he = hipStreamSynchronize(s);
+                    e = (long)he;
+                }
+            }
+            if (e) { m_mem.free(h); return e; }
+        }
+        return set_out((float)h, ppOut, plOut);
+    }
+
+    case MCH_FN_FREEMEM:
+        NEED_L(1, 1);
+        HIPCHK(hipStreamSynchronize(s));
+        return m_mem.free((long)pl[0]);
+
+    case MCH_FN_CREATE_MEMORYPOINTER: {
+        // l{hData, offset, count} (device.h:1000-1020)
+        NEED_L(3, 3);
+        if (pl[1] < 0 || pl[2] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        long h = 0;
+        ERRCHK(m_mem.alloc_view((long)pl[0], (size_t)pl[1], (size_t)pl[2], &h));
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_MEMORYPOINTER:
+        NEED_L(1, 1);
+        return m_mem.free((long)pl[0]);
+
+    case MCH_FN_GETMEM: {
+        // l{h, count(-1 = all)} (device.cu:973-1022)
+        NEED_L(1, 2);
+        if (!plOut || !ppOut) return MCH_ERROR_PARAM_NULL;
+        MemItem* it;
+        ERRCHK(mem((long)pl[0], &it));
+        long long count = ll > 1 ? pl[1] : 0;
+        if (count < 0) count = (long long)it->count;
+        else if ((size_t)count > it->count) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (count > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const void* dsrc = it->ptr;
+        if (it->half && count) {
+            void* ws;
+            ERRCHK(workspace((size_t)count * 4, &ws));
+            HIPCHK(k_convert(s, BF16, it->ptr, F32, ws, (size_t)count));
+            dsrc = ws;
+        }
+        if (count <= *plOut && *ppOut) {
+            if (count) HIPCHK(hipMemcpyAsync(*ppOut, dsrc, (size_t)count * 4, hipMemcpyDeviceToHost, s));
+            HIPCHK(hipStreamSynchronize(s));
+        } else {
+            float* host = nullptr;
+            ERRCHK(alloc_host((long)count, &host, (const float*)dsrc, true));
+            *ppOut = host;
+        }
+        *plOut = (MCH_LONG)count;
+        return 0;
+    }
+
+    case MCH_FN_SETMEM: {
+        // f{h, count, [stream,] data...}, l{h, count} (device.cu:1029-1091)
+        NEED_F(2, INT_MAX);
+        NEED_L(2, 2);
+        if (pl[1] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        size_t count = (size_t)pl[1];
+        const float* data;
+        if (count == (size_t)lf - 2) data = pf + 2;
+        else if (count == (size_t)lf - 3) data = pf + 3;
+        else return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem* it;
+        ERRCHK(mem((long)pl[0], &it));
+        RANGE(it, 0, count);
+        if (count == 0) return 0;
+        if (!it->half) {
+            HIPCHK(hipMemcpyAsync(it->ptr, data, count * 4, hipMemcpyHostToDevice, s));
+        } else {
+            void* ws;
+            ERRCHK(workspace(count * 4, &ws));
+            HIPCHK(hipMemcpyAsync(ws, data, count * 4, hipMemcpyHostToDevice, s));
+            HIPCHK(k_convert(s, F32, ws, BF16, it->ptr, count));
+        }
+        HIPCHK(hipStreamSynchronize(s));  // the caller may reuse its buffer immediately
+        m_mem.touch((long)pl[0]);
+        return 0;
+    }
+
+    case MCH_FN_SET: {
+        // f{val}, l{n, h, 0, idx, xOff} (device.h:6038-6061, math.cu:431-495)
+        NEED_F(1, 1);
+        NEED_L(3, 5);
+        long long n = pl[0];
+        long long idx = ll > 3 ? pl[3] : -1;
+        long long off = ll > 4 ? pl[4] : 0;
+        MemItem* it;
+        ERRCHK(mem((long)pl[1], &it));
+        m_mem.touch((long)pl[1]);
+        if (pf[0] == 0.f && idx == -1 && off == 0) {
+            HIPCHK(hipMemsetAsync(it->ptr, 0, it->count * it->esize(), s));
+            return 0;
+        }
+        if (off < 0) off = 0;
+        if (idx >= 0) {
+            RANGE(it, off + idx, 1);
+            HIPCHK(k_set(s, it->dt(), PTR(it, off + idx), 1, pf[0]));
+        } else {
+            RANGE(it, off, n);
+            HIPCHK(k_set(s, it->dt(), PTR(it, off), (size_t)n, pf[0]));
+        }
+        return 0;
+    }
+
+    case MCH_FN_COPY: {
+        // l{n, hSrc, hDst, srcOff, dstOff, hStream, srcHalfOverride, dstHalfOverride} (device.h:6063-6095)
+        NEED_L(3, 8);
+        long long n = pl[0];
+        long long so = ll > 3 ? pl[3] : 0, dofs = ll > 4 ? pl[4] : 0;
+        MemItem *src, *dst;
+        ERRCHK(mem((long)pl[1], &src));
+        ERRCHK(mem((long)pl[2], &dst));
+        if (so < 0) so = 0;
+        if (dofs < 0) dofs = 0;
+        RANGE(src, so, n);
+        RANGE(dst, dofs, n);
+        HIPCHK(k_convert(s, src->dt(), PTR(src, so), dst->dt(), PTR(dst, dofs), (size_t)n));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
+    // ---- BLAS-like -----------------------------------------------------------
+    case MCH_FN_GEMM: {
+        // f{alpha,beta}, l{tA,tB,m,n,k,0,hA,hB,0,hC,aOff,bOff,cOff,groups,gA,gB,gC} (device.cu:1636-1685)
+        NEED_F(2, 2);
+        NEED_L(10, 17);
+        bool tA = pl[0] != 0, tB = pl[1] != 0;
+        int m = (int)pl[2], n = (int)pl[3], k = (int)pl[4];
+        long long aOff = ll > 10 ? pl[10] : 0, bOff = ll > 11 ? pl[11] : 0, cOff = ll > 12 ? pl[12] : 0;
+        int groups = ll > 13 ? (int)pl[13] : 1;
+        long long gA = ll > 14 ? pl[14] : 0, gB = ll > 15 ? pl[15] : 0, gC = ll > 16 ? pl[16] : 0;
+        if (m < 0 || n < 0 || k < 0 || groups < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *A, *B, *C;
+        ERRCHK(mem((long)pl[6], &A));
+        ERRCHK(mem((long)pl[7], &B));
+        ERRCHK(mem((long)pl[9], &C));
+        if (A->half != B->half || A->half != C->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (aOff < 0) aOff = 0;
+        if (bOff < 0) bOff = 0;
+        if (cOff < 0) cOff = 0;
+        for (int g = 0; g < groups; g++) {
+            long long ao = aOff + gA * g, bo = bOff + gB * g, co = cOff + gC * g;
+            RANGE(A, ao, (long long)m * k);
+            RANGE(B, bo, (long long)k * n);
+            RANGE(C, co, (long long)m * n);
+            HIPCHK(k_gemm(s, A->dt(), tA, tB, m, n, k, pf[0], PTR(A, ao), PTR(B, bo), pf[1], PTR(C, co)));
+        }
+        m_mem.touch((long)pl[9]);
+        return 0;
+    }
+
+    case MCH_FN_GEMM2: {
+        // f{alpha,beta}, l{tA,tB,m,n,k,0,hA,hB,0,hC,lda,ldb,ldc[,sA,sB,sC,batch]}: BLAS column-major (device.cu:1691-1726)
+        NEED_F(2, 2);
+        NEED_L(13, 17);
+        if (ll != 13 && ll != 17) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        bool tA = pl[0] != 0, tB = pl[1] != 0;
+        int m = (int)pl[2], n = (int)pl[3], k = (int)pl[4];
+        int lda = (int)pl[10], ldb = (int)pl[11], ldc = (int)pl[12];
+        long long sA = 0, sB = 0, sC = 0;
+        int batch = 1;
+        if (ll == 17) { sA = pl[13]; sB = pl[14]; sC = pl[15]; batch = (int)pl[16]; }
+        if (m < 0 || n < 0 || k < 0 || batch < 1 || lda < 1 || ldb < 1 || ldc < 1 || sA < 0 || sB < 0 || sC < 0)
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *A, *B, *C;
+        ERRCHK(mem((long)pl[6], &A));
+        ERRCHK(mem((long)pl[7], &B));
+        ERRCHK(mem((long)pl[9], &C));
+        if (A->half || B->half || C->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;  // math.cu:1777-1778
+        if (m == 0 || n == 0) return 0;
+        long long ac = tA ? m : k, bc = tB ? k : n;  // stored column counts
+        long long ar = tA ? k : m, br = tB ? n : k;
+        RANGE(A, 0, (batch - 1) * sA + (ac - 1) * lda + ar);
+        RANGE(B, 0, (batch - 1) * sB + (bc - 1) * ldb + br);
+        RANGE(C, 0, (batch - 1) * sC + (long long)(n - 1) * ldc + m);
+        HIPCHK(k_gemm2(s, tA, tB, m, n, k, pf[0], (const float*)A->ptr, (const float*)B->ptr, pf[1], (float*)C->ptr, lda,
+                       ldb, ldc, sA, sB, sC, batch));
+        m_mem.touch((long)pl[9]);
+        return 0;
+    }
+
+    case MCH_FN_GEMV: {
+        // f{alpha,beta}, l{tA,m,n,0,hA,hX,0,hY,aOff,xOff,yOff} (device.cu:1733-1767)
+        NEED_F(2, 2);
+        NEED_L(8, 11);
+        bool tA = pl[0] != 0;
+        int m = (int)pl[1], n = (int)pl[2];
+        long long aOff = ll > 8 ? pl[8] : 0, xOff = ll > 9 ? pl[9] : 0, yOff = ll > 10 ? pl[10] : 0;
+        if (m < 0 || n < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *A, *X, *Y;
+        ERRCHK(mem((long)pl[4], &A));
+        ERRCHK(mem((long)pl[5], &X));
+        ERRCHK(mem((long)pl[7], &Y));
+        if (X->half || Y->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+        if (aOff < 0) aOff = 0;
+        if (xOff < 0) xOff = 0;
+        if (yOff < 0) yOff = 0;
+        RANGE(A, aOff, (long long)m * n);
+        RANGE(X, xOff, tA ? m : n);
+        RANGE(Y, yOff, tA ? n : m);
+        HIPCHK(k_gemv(s, A->dt(), tA, m, n, pf[0], PTR(A, aOff), (const float*)PTR(X, xOff), pf[1], (float*)PTR(Y, yOff)));
+        m_mem.touch((long)pl[7]);
+        return 0;
+    }
+
+    case MCH_FN_AXPY: {
+        // f{alpha}, l{n,0,hX,hY,xOff,yOff} (device.cu:1830-1857)
+        NEED_F(1, 1);
+        NEED_L(4, 6);
+        long long n = pl[0], xo = ll > 4 ? pl[4] : 0, yo = ll > 5 ? pl[5] : 0;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_axpy(s, X->dt(), (size_t)n, pf[0], PTR(X, xo), PTR(Y, yo)));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_SCAL: {
+        // f{alpha}, l{n,0,hX,xOff} (device.cu:1887-1905)
+        NEED_F(1, 1);
+        NEED_L(3, 4);
+        long long n = pl[0], xo = ll > 3 ? pl[3] : 0;
+        MemItem* X;
+        ERRCHK(mem((long)pl[2], &X));
+        RANGE(X, xo, n);
+        HIPCHK(k_scale(s, X->dt(), (size_t)n, pf[0], PTR(X, xo), PTR(X, xo)));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
+    case MCH_FN_SCALE: {
+        // f{alpha}, l{n,0,hX,hY,xOff,yOff} (device.cu:2028-2051)
+        NEED_F(1, 1);
+        NEED_L(4, 6);
+        long long n = pl[0], xo = ll > 4 ? pl[4] : 0, yo = ll > 5 ? pl[5] : 0;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_scale(s, X->dt(), (size_t)n, pf[0], PTR(X, xo), PTR(Y, yo)));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_ADD: {
+        // [f{alpha}], l{n,hA,hB,hY}: y = a + alpha*b (device.cu:2208-2236, math.cu:3363-3369)
+        if (lf > 0 && pf) NEED_F(1, 1);
+        NEED_L(4, 5);
+        long long n = pl[0];
+        float alpha = (lf > 0 && pf) ? pf[0] : 1.f;
+        MemItem *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != B->half || A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_add(s, A->dt(), (size_t)n, A->ptr, B->ptr, Y->ptr, alpha));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_MUL: {
+        // l{n,hA,hB,hY,aOff,bOff,yOff} (device.cu:2398-2423)
+        NEED_L(4, 7);
+        long long n = pl[0], ao = ll > 4 ? pl[4] : 0, bo = ll > 5 ? pl[5] : 0, yo = ll > 6 ? pl[6] : 0;
+        MemItem *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != B->half || A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, ao, n);
+        RANGE(B, bo, n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_mul(s, A->dt(), (size_t)n, PTR(A, ao), PTR(B, bo), PTR(Y, yo)));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_MASK: {
+        // f{search,replace}, l{n,maskDim,0,0,hX,hMask,hY} (device.cu:2101-2120)
+        NEED_F(2, 2);
+        NEED_L(7, 7);
+        long long n = pl[0];
+        int md = (int)pl[1];
+        if (md < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *M, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &M));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (X->half != M->half || X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        RANGE(M, 0, md);
+        HIPCHK(k_mask(s, X->dt(), (size_t)n, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr));
+        m_mem.touch((long)pl[6]);
+        return 0;
+    }
+
+    case MCH_FN_MASK_BATCH: {
+        // f{search,replace}, l{n,batch,maskDim,0,0,hX,hMask,hY} (device.cu:2125-2145)
+        NEED_F(2, 2);
+        NEED_L(8, 8);
+        long long n = pl[0];
+        int batch = (int)pl[1], md = (int)pl[2];
+        if (batch < 1 || md < batch || n < batch) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *M, *Y;
+        ERRCHK(mem((long)pl[5], &X));
+        ERRCHK(mem((long)pl[6], &M));
+        ERRCHK(mem((long)pl[7], &Y));
+        if (X->half != M->half || X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        // largest mask index = (md/batch - 1) + ((n-1)/(n/batch)) * (md/batch)
+        {
+            long long md1 = md / batch, dd1 = n / batch;
+            RANGE(M, 0, (md1 - 1) + ((n - 1) / dd1) * md1 + 1);
+        }
+        HIPCHK(k_mask_batch(s, X->dt(), (size_t)n, batch, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr));
+        m_mem.touch((long)pl[7]);
+        return 0;
+    }
+
+    case MCH_FN_TRANSPOSE: {
+        // l{n,hX,hY,hXCounts,hYCounts,hMapping,numAxes,hBuffer} (device.cu:3088-3107)
+        NEED_L(8, 8);
+        long long n = pl[0];
+        int axes = (int)pl[6];
+        MemItem *X, *Y, *XC, *YC, *MP;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        ERRCHK(mem((long)pl[3], &XC));
+        ERRCHK(mem((long)pl[4], &YC));
+        ERRCHK(mem((long)pl[5], &MP));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (XC->half || YC->half || MP->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+        if (axes < 1 || axes > 8) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        RANGE(XC, 0, axes);
+        RANGE(YC, 0, axes);
+        RANGE(MP, 0, axes);
+        HIPCHK(k_transpose(s, X->dt(), (size_t)n, X->ptr, Y->ptr, (const float*)XC->ptr, (const float*)YC->ptr,
+                           (const float*)MP->ptr, axes));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
+    case MCH_FN_TRANSPOSE_HW: {
+        // l{n,c,h,w,hSrc,hDst} (device.cu:3110-3127)
+        NEED_L(6, 6);
+        long long nn = pl[0], c = pl[1], h = pl[2], w = pl[3];
+        if (nn < 0 || c < 0 || h < 0 || w < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, nn * c * h * w);
+        RANGE(Y, 0, nn * c * h * w);
+        HIPCHK(k_transpose_hw(s, X->dt(), (int)(nn * c), (int)h, (int)w, X->ptr, Y->ptr));
+        m_mem.touch((long)pl[5]);
+        return 0;
+    }
+
+    case MCH_FN_CHANNEL_COPY: {
+        // l{count,outer,channels,blocks,inner,offset,hX,hY,dir} (device.cu:3730-3748)
+        NEED_L(9, 9);
+        long long n = pl[0], chn = pl[2], blocks = pl[3], inner = pl[4], off = pl[5];
+        int dir = (int)pl[8];
+        if (n < 0 || chn < 1 || blocks < 1 || inner < 1 || off < 0 || off >= blocks) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[6], &X));
+        ERRCHK(mem((long)pl[7], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(Y, 0, n);
+        if (n > 0) {
+            long long last = n - 1;
+            long long xi = ((last / (chn * inner)) * chn + (last % (chn * inner)) / inner) * blocks * inner + off * inner + last % inner;
+            // the last element has the largest n and c, so together with inner-1 this bounds every index
+            RANGE(X, 0, xi + (inner - 1 - last % inner) + 1);
+        }
+        HIPCHK(k_channel_copy(s, X->dt(), (size_t)n, (int)chn, (int)blocks, (int)inner, (int)off, X->ptr, Y->ptr, dir));
+        m_mem.touch(dir == 0 ? (long)pl[7] : (long)pl[6]);
+        return 0;
+    }
+
+    case MCH_FN_EMBED_FWD: {
+        // l{count,hBtm,hWeight,M,N,K,hTop} (CudaDnn.cs:9751; math.cu:9314-9330)
+        NEED_L(7, 7);
+        long long n = pl[0], N = pl[4], K = pl[5];
+        if (n < 0 || N < 1 || K < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *I, *W, *T;
+        ERRCHK(mem((long)pl[1], &I));
+        ERRCHK(mem((long)pl[2], &W));
+        ERRCHK(mem((long)pl[6], &T));
+        if (I->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+        if (W->half != T->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(T, 0, n);
+        RANGE(I, 0, (n + N - 1) / N);
+        RANGE(W, 0, K * N);
+        HIPCHK(k_embed(s, W->dt(), (size_t)n, (const float*)I->ptr, W->ptr, (int)N, T->ptr));
+        m_mem.touch((long)pl[6]);
+        return 0;
+    }
+
+    case MCH_FN_SILU_FWD: {
+        // l{count,hBtm,hTop} (CudaDnn.cs:10152)
+        NEED_L(3, 3);
+        long long n = pl[0];
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_silu(s, X->dt(), (size_t)n, X->ptr, Y->ptr));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
+    case MCH_FN_SWIGLU_FWD: {
+        NEED_L(4, 4);
+        long long n = pl[0];
+        MemItem *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != B->half || A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_swiglu(s, A->dt(), (size_t)n, A->ptr, B->ptr, Y->ptr));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_RMSNORM_FWD: {
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        long long outer = pl[0], dim = pl[1];
+        if (outer < 0 || dim < 1 || outer > INT_MAX || dim > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *W = nullptr, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        if (pl[3]) ERRCHK(mem((long)pl[3], &W));
+        ERRCHK(mem((long)pl[4], &Y));
+        if (X->half != Y->half || (W && W->half != X->half)) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, outer * dim);
+        RANGE(Y, 0, outer * dim);
+        if (W) RANGE(W, 0, dim);
+        HIPCHK(k_rmsnorm(s, X->dt(), (int)outer, (int)dim, X->ptr, W ? W->ptr : nullptr, Y->ptr, pf[0]));
+        m_mem.touch((long)pl[4]);
+        return 0;
+    }
+
+    // ---- cuDNN-shaped handles: opaque records here ---------------------------
+    case MCH_FN_CREATE_CUDNN: {
+        // f{[stream]} (device.h:1201-1221)
+        ERRCHK(verify(lf, pf, 0, 1));
+        long h;
+        ERRCHK(m_cudnn.create(&h));
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_CUDNN:
+        NEED_F(1, 1);
+        return m_cudnn.free((long)pf[0]);
+    case MCH_FN_CREATE_TENSORDESC: {
+        long h;
+        ERRCHK(m_tdesc.create(&h));
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_TENSORDESC:
+        NEED_F(1, 1);
+        return m_tdesc.free((long)pf[0]);
+    case MCH_FN_SET_TENSORDESC: {
+        // l{h,half,n,c,h,w[,sn,sc,sh,sw]} (device.cu:1426-1464)
+        NEED_L(6, 10);
+        if (ll != 6 && ll != 10) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        TensorDesc* d = m_tdesc.get((long)pl[0]);
+        if (!d) return MCH_ERROR_PARAM_NULL;
+        d->half = pl[1] == 1;
+        d->n = (int)pl[2]; d->c = (int)pl[3]; d->h = (int)pl[4]; d->w = (int)pl[5];
+        if (ll == 6) { d->sw = 1; d->sh = d->w; d->sc = d->h * d->sh; d->sn = d->c * d->sc; }
+        else { d->sn = (int)pl[6]; d->sc = (int)pl[7]; d->sh = (int)pl[8]; d->sw = (int)pl[9]; }
+        return 0;
+    }
+
+    case MCH_FN_SOFTMAX_FWD: {
+        // f{alpha,beta}, l{hCudnn,0,hBtmDesc,hBtm,0,hTopDesc,hTop,alg,mode} (device.h:4778-4798)
+        NEED_F(2, 2);
+        NEED_L(9, 9);
+        if (!m_cudnn.get((long)pl[0])) return MCH_ERROR_PARAM_NULL;
+        TensorDesc* bd = m_tdesc.get((long)pl[2]);
+        TensorDesc* td = m_tdesc.get((long)pl[5]);
+        if (!bd || !td) return MCH_ERROR_PARAM_NULL;
+        if (pf[0] != 1.f || pf[1] != 0.f) { last_detail = "softmax supports alpha=1, beta=0 only"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        int alg = (int)pl[7], mode = (int)pl[8];  // alg 0 fast, 1 accurate, 2 log; mode 0 instance, 1 channel
+        if (alg < 0 || alg > 2 || mode < 0 || mode > 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (bd->n != td->n || bd->c != td->c || bd->h != td->h || bd->w != td->w) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        bool packed = bd->sw == 1 && bd->sh == bd->w && bd->sc == bd->h * bd->w && bd->sn == bd->c * bd->h * bd->w &&
+                      td->sw == 1 && td->sh == td->w && td->sc == td->h * td->w && td->sn == td->c * td->h * td->w;
+        if (!packed) { last_detail = "softmax needs fully packed NCHW descriptors"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[3], &X));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        long long total = (long long)bd->n * bd->c * bd->h * bd->w;
+        RANGE(X, 0, total);
+        RANGE(Y, 0, total);
+        size_t outer = bd->n;
+        int len = mode == 0 ? bd->c * bd->h * bd->w : bd->c;
+        int inner = mode == 0 ? 1 : bd->h * bd->w;
+        HIPCHK(k_softmax(s, X->dt(), X->ptr, Y->ptr, outer, len, inner, alg == 2));
+        m_mem.touch((long)pl[6]);
+        return 0;
+    }
+
+    // ---- attention -------------------------------------------------------------
+    case MCH_FN_ATTN_CREATE: {
+        long h;
+        ERRCHK(m_attn.create(&h));
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_ATTN_FREE:
+        NEED_F(1, 1);
+        return m_attn.free((long)pf[0]);
+    case MCH_FN_ATTN_SET: {
+        // f{dropout}, l{hCudnn,hAttn,gpuId,training,batch,blockSize,heads,hs,seed} (device.h:2463-2485)
+        NEED_L(9, 9);
+        NEED_F(1, 1);
+        AttnState* st = m_attn.get((long)pl[1]);
+        if (!st) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        if (pl[4] < 1 || pl[5] < 1 || pl[6] < 1 || pl[7] < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        st->training = pl[3] != 0;
+        st->batch = (int)pl[4]; st->block = (int)pl[5]; st->heads = (int)pl[6]; st->hs = (int)pl[7];
+        st->dropout = pf[0];
+        st->scale = (float)(1.0 / sqrt((double)st->hs));  // attn.cu:427
+        st->set = true;
+        st->maskHandle = 0;
+        return 0;
+    }
+    case MCH_FN_ATTN_FWD: {
+        // l{hCudnn,hAttn,blockSize,hQ,hK,hV,hMask,hY,batchMask[,blockSizeK]} (device.h:2488-2506, attn.cu:518-602)
+        // The optional 10th value (key length when it differs from the query length) has no
+        // counterpart in the reference, whose handle needs T_q == T_k.
+        NEED_L(9, 10);
+        AttnState* st = m_attn.get((long)pl[1]);
+        if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        int T = (int)pl[2];
+        int Tk = ll > 9 ? (int)pl[9] : T;
+        if (T > st->block || Tk > st->block) return MCH_ERROR_ATTN_INVALID_BLOCK_SIZE;
+        if (T < 1 || Tk < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (st->training && st->dropout > 0.f) { last_detail = "attention dropout (training) is not part of the inference path"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        MemItem *Q, *K, *V, *Y, *M = nullptr;
+        ERRCHK(mem((long)pl[3], &Q));
+        ERRCHK(mem((long)pl[4], &K));
+        ERRCHK(mem((long)pl[5], &V));
+        ERRCHK(mem((long)pl[7], &Y));
+        long hMask = (long)pl[6];
+        bool batchMask = pl[8] != 0;
+        if (hMask) ERRCHK(mem(hMask, &M));
+        if (Q->half != K->half || Q->half != V->half || Q->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        long long qn = (long long)st->batch * st->heads * T * st->hs, kn = (long long)st->batch * st->heads * Tk * st->hs;
+        if ((long long)Q->count < qn || (long long)Y->count < qn || (long long)K->count < kn || (long long)V->count < kn)
+            return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+        MaskKind kind = MASK_NONE;
+        if (M) {
+            if (M->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+            if (batchMask) {
+                if ((long long)M->count < (long long)st->batch * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = MASK_KEY;
+            } else {
+                if ((long long)M->count < (long long)T * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = (T == Tk && mask_is_causal(st, hMask, M, T)) ? MASK_CAUSAL : MASK_QK;
+            }
+        }
+        HIPCHK(k_attn_prefill(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, st->batch, st->heads, T, Tk, st->hs, st->scale,
+                              M ? (const float*)M->ptr : nullptr, kind));
+        m_mem.touch((long)pl[7]);
+        return 0;
+    }
+
+    case MCH_FN_ATTN_DECODE_FWD: {
+        // f{scale}, l{batch,heads,kvHeads,hs,len,hQ,hKc,hVc,hY,strideB,strideH,strideT[,hRope,hKnew,hVnew]}
+        NEED_F(1, 1);
+        NEED_L(12, 15);
+        if (ll != 12 && ll != 15) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        long long B = pl[0], H = pl[1], KVH = pl[2], hs = pl[3], len = pl[4];
+        long long sB = pl[9], sH = pl[10], sT = pl[11];
+        if (B < 1 || H < 1 || KVH < 1 || hs < 1 || len < 1 || H % KVH || sB < 0 || sH < 0 || sT < 1 || (hs & 1))
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *Q, *KC, *VC, *Y;
+        ERRCHK(mem((long)pl[5], &Q));
+        ERRCHK(mem((long)pl[6], &KC));
+        ERRCHK(mem((long)pl[7], &VC));
+        ERRCHK(mem((long)pl[8], &Y));
+        if (Q->half != KC->half || Q->half != VC->half || Q->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(Q, 0, B * H * hs);
+        RANGE(Y, 0, B * H * hs);
+        long long need = (B - 1) * sB + (KVH - 1) * sH + (len - 1) * sT + hs;
+        RANGE(KC, 0, need);
+        RANGE(VC, 0, need);
+        float scale = pf[0] != 0.f ? pf[0] : (float)(1.0 / sqrt((double)hs));
+        if (ll == 15 && (pl[12] || pl[13] || pl[14])) {
+            RopeState* rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
+            if (pl[12] && (!rp || !rp->set)) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+            if (rp && (rp->hs != hs || len > rp->seq)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            MemItem *KN, *VN;
+            ERRCHK(mem((long)pl[13], &KN));
+            ERRCHK(mem((long)pl[14], &VN));
+            if (KN->half != Q->half || VN->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+            RANGE(KN, 0, B * KVH * hs);
+            RANGE(VN, 0, B * KVH * hs);
+            HIPCHK(k_rope_append(s, Q->dt(), Q->ptr, KN->ptr, VN->ptr, KC->ptr, VC->ptr, (int)B, (int)H, (int)KVH, (int)hs,
+                                 (int)len - 1, sB, sH, sT, rp ? (const float*)rp->dcos.get() : nullptr,
+                                 rp ? (const float*)rp->dsin.get() : nullptr));
+            m_mem.touch((long)pl[5]);
+            m_mem.touch((long)pl[6]);
+            m_mem.touch((long)pl[7]);
+            m_mem.touch((long)pl[13]);
+        }
+        size_t wsb = attn_decode_workspace_bytes((int)B, (int)H, (int)hs, (int)len);
+        void* ws;
+        ERRCHK(workspace(wsb, &ws));
+        HIPCHK(k_attn_decode(s, Q->dt(), Q->ptr, KC->ptr, VC->ptr, Y->ptr, (int)B, (int)H, (int)KVH, (int)hs, (int)len, sB, sH,
+                             sT, scale, ws, m_wsBytes));
+        m_mem.touch((long)pl[8]);
+        return 0;
+    }
+
+    // ---- RoPE ------------------------------------------------------------------
+    case MCH_FN_CREATE_ROPE: {
+        // f{theta}, l{sharedIdx,gpuId,count,batch,seqLen,heads,hs} (device.h:4201-4229, rope.cu:502-607)
+        NEED_F(1, 1);
+        NEED_L(7, 7);
+        long long seq = pl[4], heads = pl[5], hs = pl[6];
+        if (seq < 1 || heads < 1 || hs < 2 || (hs & 1) || seq * hs > (1ll << 30)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        long h;
+        ERRCHK(m_rope.create(&h));
+        RopeState* r = m_rope.get(h);
+        r->sharedIdx = (int)pl[0]; r->count = (int)pl[2]; r->batch = (int)pl[3];
+        r->seq = (int)seq; r->heads = (int)heads; r->hs = (int)hs; r->theta = pf[0];
+        int half = (int)hs / 2;
+        // host tables exactly as the reference builds them: powf, then fp32 product, then cosf/sinf
+        std::vector<float> freq(half), hc((size_t)seq * half), hsn((size_t)seq * half);
+        int idx = 0;
+        for (int i = 0; i < hs; i += 2) {
+            float power = (float)(i / (float)hs);
+            power = powf(r->theta, power);
+            freq[idx++] = 1.0f / power;
+        }
+        for (int pos = 0; pos < seq; pos++)
+            for (int i = 0; i < half; i++) {
+                float fp = freq[i] * pos;
+                hc[(size_t)pos * half + i] = cosf(fp);
+                hsn[(size_t)pos * half + i] = sinf(fp);
+            }
+        size_t bytes = (size_t)seq * half * sizeof(float);
+        void *dc = nullptr, *ds = nullptr;
+        hipError_t e = hipMalloc(&dc, bytes);
+        if (e == hipSuccess) e = hipMalloc(&ds, bytes);
+        if (e == hipSuccess) e = hipMemcpyAsync(dc, hc.data(), bytes, hipMemcpyHostToDevice, s);
+        if (e == hipSuccess) e = hipMemcpyAsync(ds, hsn.data(), bytes, hipMemcpyHostToDevice, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e != hipSuccess) {
+            if (dc) (void)hipFree(dc);
+            if (ds) (void)hipFree(ds);
+            m_rope.free(h);
+            return (long)e;
+        }
+        r->dcos = std::shared_ptr<void>(dc, [](void* p) { (void)hipFree(p); });
+        r->dsin = std::shared_ptr<void>(ds, [](void* p) { (void)hipFree(p); });
+        r->set = true;
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_ROPE:
+        NEED_F(1, 1);
+        HIPCHK(hipStreamSynchronize(s));
+        return m_rope.free((long)pf[0]);
+    case MCH_FN_ROPE_FWD: {
+        // l{hRope,n,hX,hY[,freqOffset]} (device.h:4232-4255, rope.cu:785-825)
+        NEED_L(4, 5);
+        RopeState* r = m_rope.get((long)pl[0]);
+        if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+        long long n = pl[1];
+        long long off = ll > 4 ? pl[4] : -1;
+        if (off < 0) off = 0;  // offsets <= 0 mean "no shift" (rope.cu:808-814)
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (n < 0 || (n & 1)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        {
+            // largest table index any pair can reach must stay inside the [seq, hs/2] tables
+            long long half = r->hs / 2, full = half * r->heads, wrap = (long long)r->seq * full;
+            long long pairs = n / 2;
+            long long maxbase = (pairs < wrap ? pairs : wrap) - 1;
+            if (pairs > 0 && (maxbase / full) * half + (half - 1) + off >= (long long)r->seq * half) {
+                last_detail = "rope table offset reaches past the last position of the table";
+                return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            }
+        }
+        HIPCHK(k_rope(s, X->dt(), (size_t)n, X->ptr, Y->ptr, (const float*)r->dcos.get(), (const float*)r->dsin.get(), r->seq,
+                      r->heads, r->hs, (int)off));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_FREE_EXTENSION:
+        NEED_F(1, 1);
+        return m_ext.free((long)pf[0]);
+
+    default:
+        break;
+    }
+    char buf[96];
+    snprintf(buf, sizeof(buf), "function id %ld is outside the attention hot path and is not dispatched", fn);
+    last_detail = buf;
+    return MCH_ERROR_NOT_IMPLEMENTED;
+}
+
+// ---- extensions (extension.cu:17-179) ---------------------------------------------
+typedef MCH_LONG (*FnExtInit)(void*, MCH_LONG);
+typedef MCH_LONG (*FnExtInvoke)(MCH_LONG, float*, MCH_LONG, float**, MCH_LONG*, MCH_TCHAR*, MCH_LONG);
+typedef MCH_LONG (*FnExtInvokeEx)(MCH_LONG, float*, MCH_LONG, float**, MCH_LONG*, MCH_TCHAR*, MCH_TCHAR*, MCH_LONG, MCH_TCHAR*,
+                                  MCH_LONG);
+
+static void* self_handle()
+{
+    Dl_info info;
+    if (!dladdr((void*)&self_handle, &info) || !info.dli_fname) return nullptr;
+    return dlopen(info.dli_fname, RTLD_NOW | RTLD_NOLOAD);
+}
+
+long Kernel::create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut)
+{
+    if (!path) return MCH_ERROR_PARAM_NULL;
+    std::string p = utf16_to_utf8(path);
+    void* lib = dlopen(p.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!lib) { last_detail = std::string("cannot load extension: ") + dlerror(); return MCH_ERROR_FILE_OPEN; }
+    FnExtInit init = (FnExtInit)dlsym(lib, "DLL_InitFloatCustomExtension");
+    void* inv = dlsym(lib, "DLL_InvokeFloatCustomExtension");
+    if (!init || !inv) { dlclose(lib); last_detail = "extension lacks DLL_InitFloatCustomExtension / DLL_InvokeFloatCustomExtension"; return MCH_ERROR_NOT_IMPLEMENTED; }
+    long e = init(self_handle(), (MCH_LONG)kernelIdx);
+    if (e) { dlclose(lib); return e; }
+    long h;
+    ERRCHK(m_ext.create(&h));
+    ExtensionState* st = m_ext.get(h);
+    st->lib = lib;
+    st->fnInvoke = inv;
+    st->fnInvokeEx = dlsym(lib, "DLL_InvokeFloatCustomExtensionEx");
+    return set_out((float)h, ppOut, plOut);
+}
+
+long Kernel::run_extension(long hExt, long fn, float* pf, long lf, MCH_TCHAR* szIn, float** ppOut, MCH_LONG* plOut,
+                           MCH_TCHAR* szErr, long errMax)
+{
+    ExtensionState* st = m_ext.get(hExt);
+    if (!st) return MCH_ERROR_EXTENSION_NOT_INITIALIZED;
+    if (lf == 0) pf = nullptr;
+    if (szIn == nullptr)
+        return ((FnExtInvoke)st->fnInvoke)((MCH_LONG)fn, pf, (MCH_LONG)lf, ppOut, plOut, szErr, (MCH_LONG)errMax);
+    if (!st->fnInvokeEx) return MCH_ERROR_NOT_IMPLEMENTED;
+    return ((FnExtInvokeEx)st->fnInvokeEx)((MCH_LONG)fn, pf, (MCH_LONG)lf, ppOut, plOut, szIn, nullptr, 0, szErr, (MCH_LONG)errMax);
+}
+
+long Kernel::query_extension(MCH_LONG* pIn, long n, MCH_TCHAR* out, long outMax, MCH_TCHAR* err, long errMax)
+{
+    // LONG{hExt, fnIdx, args...} (device.h:4590-4603); at most 5 args are forwarded as floats (extension.cu:153-179)
+    if (n < 2) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    if (!pIn) return MCH_ERROR_PARAM_NULL;
+    ExtensionState* st = m_ext.get(pIn[0]);
+    if (!st) return MCH_ERROR_EXTENSION_NOT_INITIALIZED;
+    if (!st->fnInvokeEx) return MCH_ERROR_NOT_IMPLEMENTED;
+    long cnt = n - 2;
+    if (cnt > 5) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    float args[5];
+    for (long i = 0; i < cnt; i++) args[i] = (float)pIn[2 + i];
+    float* o = nullptr;
+    MCH_LONG lo = 0;
+    if (out && outMax > 0) out[0] = 0;
+    long e = ((FnExtInvokeEx)st->fnInvokeEx)(pIn[1], args, (MCH_LONG)cnt, &o, &lo, nullptr, out, (MCH_LONG)outMax, err, (MCH_LONG)errMax);
+    if (e) return e;
+    if (o != nullptr && out) {
+        // the extension passes its "finished" flag through the output pointer; the parent appends the end marker
+        std::string cur = utf16_to_utf8(out) + "\n[END]";
+        utf8_to_utf16(cur, out, outMax);
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// kernel table (dllmain.cpp:6-14, CudaDnnDLL.cpp:1747-1805): 2048 slots, slot 0 reserved
+static const int MAX_KERNELS = 2048;
+static Kernel* g_kernels[MAX_KERNELS];
+static std::mutex g_tableLock;
+
+static const char* error_text(long e)
+{
+    switch (e) {
+    case MCH_ERROR_DLL_NOT_INIT: return "The library is not initialized.";
+    case MCH_ERROR_PARAM: return "General parameter error.";
+    case MCH_ERROR_PARAM_OUT_OF_RANGE: return "A parameter is out of range.";
+    case MCH_ERROR_PARAM_NULL: return "A parameter is NULL (or the kernel/handle does not exist).";
+    case MCH_ERROR_FILE_OPEN: return "Failed to open the file.";
+    case MCH_ERROR_MEMORY_OUT: return "Out of device memory.";
+    case MCH_ERROR_MEMORY_NULL: return "The memory is NULL.";
+    case MCH_ERROR_NOT_IMPLEMENTED: return "The function is not implemented.";
+    case MCH_ERROR_MEMORY_RANGE_EXCEEDED: return "The memory range was exceeded.";
+    case MCH_ERROR_MEMORY_MIXED_HALF_TYPES: return "Half and full size memory types were mixed.";
+    case MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED: return "Half size memory is not supported by this function.";
+    case MCH_ERROR_MEMORY_NOT_FOUND: return "The memory handle was not found.";
+    case MCH_ERROR_DEVICE_NOT_INITIALIZED: return "The device is not initialized.";
+    case MCH_ERROR_ROPE_NOT_INITIALIZED: return "The RoPE handle is not initialized.";
+    case MCH_ERROR_ATTN_NOT_INITIALIZED: return "The attention handle is not initialized.";
+    case MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE: return "A blob passed to the attention handle has an incompatible size.";
+    case MCH_ERROR_ATTN_INVALID_BLOCK_SIZE: return "The block size exceeds the one the attention handle was set for.";
+    case MCH_ERROR_EXTENSION_NOT_INITIALIZED: return "The extension is not initialized.";
+    default: return nullptr;
+    }
+}
+
+static void put_error(Kernel* k, long e, MCH_TCHAR* szErr, long max)
+{
+    if (!szErr || max <= 0) return;
+    std::string msg;
+    const char* t = error_text(e);
+    if (t) msg = t;
+    else if (e > 0 && e < 2000) msg = std::string("HIP runtime error: ") + hipGetErrorString((hipError_t)e);
+    else msg = "Unknown error.";
+    if (k && !k->last_detail.empty()) msg += " " + k->last_detail;
+    char code[32];
+    snprintf(code, sizeof(code), " (%ld)", e);
+    msg += code;
+    utf8_to_utf16(msg, szErr, max);
+}
+
+static Kernel* kernel_at(long idx)
+{
+    if (idx < 0 || idx >= MAX_KERNELS) return nullptr;
+    std::lock_guard<std::mutex> g(g_tableLock);
+    return g_kernels[idx];
+}
+
+static long invoke(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, MCH_TCHAR* szIn, float** ppOut,
+                   MCH_LONG* plOut, MCH_TCHAR* szErr, long errMax, bool ex)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    if (kIdx < 0 || kIdx >= MAX_KERNELS) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long e = 0;
+    Kernel* k = nullptr;
+    switch (fn) {
+    case MCH_DLL_INITIALIZE: {
+        // creates a kernel, returns its index in (*ppOutput)[0] (CudaDnnDLL.cpp:154-176)
+        if (!ppOut || !*ppOut || !plOut) return MCH_ERROR_PARAM_NULL;
+        k = new Kernel();
+        e = k->initialize(pf, lf);
+        if (e) { put_error(k, e, szErr, errMax); delete k; return e; }
+        long slot = -1;
+        {
+            std::lock_guard<std::mutex> g(g_tableLock);
+            for (int i = 1; i < MAX_KERNELS; i++)
+                if (!g_kernels[i]) { g_kernels[i] = k; slot = i; break; }
+        }
+        if (slot < 0) { delete k; e = MCH_ERROR_MEMORY_OUT; put_error(nullptr, e, szErr, errMax); return e; }
+        (*ppOut)[0] = (float)slot;
+        *plOut = 1;
+        return 0;
+    }
+    case MCH_DLL_CLEANUP: {
+        std::lock_guard<std::mutex> g(g_tableLock);
+        k = g_kernels[kIdx];
+        g_kernels[kIdx] = nullptr;
+        delete k;
+        return 0;
+    }
+    case MCH_DLL_FREEMEM:
+        if (!(k = kernel_at(kIdx))) { e = MCH_ERROR_PARAM_NULL; put_error(nullptr, e, szErr, errMax); return e; }
+        e = k->free_host(pf);
+        if (e) put_error(k, e, szErr, errMax);
+        return e;
+    default:
+        break;
+    }
+    if (!(k = kernel_at(kIdx))) { e = MCH_ERROR_PARAM_NULL; put_error(nullptr, e, szErr, errMax); return e; }
+    if (ex && fn == MCH_FN_CREATE_EXTENSION) {
+        e = k->create_extension(kIdx, szIn, ppOut, plOut);
+    } else if (fn == MCH_FN_EXTENSION_RUN) {
+        // f{hExt, fnIdx, args...} (device.h:4569-4588)
+        if (lf < 2) e = MCH_ERROR_PARAM_OUT_OF_RANGE;
+        else if (!pf) e = MCH_ERROR_PARAM_NULL;
+        else {
+            e = k->run_extension((long)pf[0], (long)pf[1], pf + 2, lf - 2, ex ? szIn : nullptr, ppOut, plOut, szErr, errMax);
+            if (e && szErr && szErr[0]) return e;  // the extension wrote its own message
+        }
+    } else if (ex) {
+        e = MCH_ERROR_PARAM_OUT_OF_RANGE;
+    } else {
+        e = k->run(fn, pf, lf, pl, ll, ppOut, plOut, false);
+    }
+    if (e) put_error(k, e, szErr, errMax);
+    return e;
+}
+
+}  // namespace mch
+
+using namespace mch;
+
+extern "C" {
+
+MCH_LONG DLL_InvokeFloat(MCH_LONG k, MCH_LONG fn, float* pIn, MCH_LONG lIn, float** ppOut, MCH_LONG* plOut, MCH_TCHAR* szErr,
+                         MCH_LONG errMax)
+{
+    // the legacy entry point forwards no integer array (CudaDnnDLL.cpp:303)
+    return (MCH_LONG)invoke(k, fn, pIn, lIn, nullptr, 0, nullptr, ppOut, plOut, szErr, errMax, false);
+}
+
+MCH_LONG DLL_InvokeFloatEx2(MCH_LONG k, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn, float** ppOut,
+                            MCH_LONG* plOut, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return (MCH_LONG)invoke(k, fn, pIn, lIn, plIn, llIn, nullptr, ppOut, plOut, szErr, errMax, false);
+}
+
+MCH_LONG DLL_InvokeFloatEx(MCH_LONG k, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_TCHAR* pszIn, float** ppOut, MCH_LONG* plOut,
+                           MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return (MCH_LONG)invoke(k, fn, pIn, lIn, nullptr, 0, pszIn, ppOut, plOut, szErr, errMax, true);
+}
+
+static MCH_LONG double_unsupported(MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    utf8_to_utf16("The double base type is not built: the attention hot path runs in fp32 and 16-bit storage. (90009)", szErr, errMax);
+    return MCH_ERROR_NOT_IMPLEMENTED;
+}
+
+MCH_LONG DLL_InvokeDouble(MCH_LONG, MCH_LONG, double*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return double_unsupported(szErr, errMax);
+}
+MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG, MCH_LONG, double*, MCH_LONG, MCH_LONGLONG*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR* szErr,
+                             MCH_LONG errMax)
+{
+    return double_unsupported(szErr, errMax);
+}
+MCH_LONG DLL_InvokeDoubleEx(MCH_LONG, MCH_LONG, double*, MCH_LONG, MCH_TCHAR*, double**, MCH_LONG*, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return double_unsupported(szErr, errMax);
+}
+
+MCH_LONG DLL_QueryString(MCH_LONG kIdx, MCH_LONG fn, MCH_LONG* pIn, MCH_LONG lIn, MCH_TCHAR** ppOut, MCH_TCHAR* szErr,
+                         MCH_LONG errMax)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    if (kIdx < 0 || kIdx >= MAX_KERNELS) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    Kernel* k = kernel_at(kIdx);
+    if (!k) { put_error(nullptr, MCH_ERROR_PARAM_OUT_OF_RANGE, szErr, errMax); return MCH_ERROR_PARAM_OUT_OF_RANGE; }
+    if (fn == MCH_DLL_FREEMEM) {
+        if (ppOut && *ppOut) { free(*ppOut); *ppOut = nullptr; }
+        return 0;
+    }
+    if (ppOut) *ppOut = nullptr;
+    if (fn == MCH_QRY_DEVICE_NAME) {
+        (void)pIn; (void)lIn;
+        if (!ppOut) return MCH_ERROR_PARAM_NULL;
+        std::string name = k->device_name();
+        long cap = (long)name.size() + 1;
+        MCH_TCHAR* buf = (MCH_TCHAR*)malloc(cap * sizeof(MCH_TCHAR));
+        if (!buf) return MCH_ERROR_MEMORY_OUT;
+        utf8_to_utf16(name, buf, cap);
+        *ppOut = buf;
+        return 0;
+    }
+    put_error(nullptr, MCH_ERROR_NOT_IMPLEMENTED, szErr, errMax);
+    return MCH_ERROR_NOT_IMPLEMENTED;
+}
+
+MCH_LONG DLL_QueryStringFloatEx(MCH_LONG kIdx, MCH_LONG fn, MCH_LONG* pIn, MCH_LONG lIn, MCH_TCHAR* pszOut, MCH_LONG outMax,
+                                MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    if (kIdx < 0 || kIdx >= MAX_KERNELS) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    Kernel* k = kernel_at(kIdx);
+    if (!k) { put_error(nullptr, MCH_ERROR_PARAM_OUT_OF_RANGE, szErr, errMax); return MCH_ERROR_PARAM_OUT_OF_RANGE; }
+    long e = fn == MCH_QRY_EXTENSION_STRING ? k->query_extension(pIn, lIn, pszOut, outMax, szErr, errMax)
+                                            : (long)MCH_ERROR_PARAM_OUT_OF_RANGE;
+    if (e && szErr && szErr[0] == 0) put_error(k, e, szErr, errMax);
+    return (MCH_LONG)e;
+}
+
+MCH_LONG DLL_QueryStringDoubleEx(MCH_LONG, MCH_LONG, MCH_LONG*, MCH_LONG, MCH_TCHAR*, MCH_LONG, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return double_unsupported(szErr, errMax);
+}
+
+MCH_LONG Internal_GetPointerFloat(int32_t ht, MCH_LONG kIdx, MCH_LONG h, void** pp)
+{
+    if (ht != 0 || !pp) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    Kernel* k = kernel_at(kIdx);
+    if (!k) return MCH_ERROR_PARAM_NULL;
+    return (MCH_LONG)k->get_pointer(h, pp);
+}
+MCH_LONG Internal_GetPointerDouble(int32_t, MCH_LONG, MCH_LONG, void**) { return MCH_ERROR_NOT_IMPLEMENTED; }
+
+MCH_LONG Internal_AllocHostFloat(MCH_LONG kIdx, MCH_LONG count, float** dst, float* src, bool srcOnDevice)
+{
+    if (kIdx < 0 || kIdx >= MAX_KERNELS) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    Kernel* k = kernel_at(kIdx);
+    if (!k) return MCH_ERROR_PARAM_NULL;
+    return (MCH_LONG)k->alloc_host(count, dst, src, srcOnDevice);
+}
+MCH_LONG Internal_AllocHostDouble(MCH_LONG, MCH_LONG, double**, double*, bool) { return MCH_ERROR_NOT_IMPLEMENTED; }
+
+MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG kIdx, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn,
+                                MCH_LONG nWarmup, MCH_LONG nReps, float* pfMs, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    Kernel* k = kernel_at(kIdx);
+    if (!k || !pfMs || nReps < 1 || nWarmup < 0) return MCH_ERROR_PARAM_NULL;
+    float dummy[4];
+    float* po = dummy;
+    MCH_LONG lo = 4;
+    long e = 0;
+    for (int i = 0; i < nWarmup && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, plIn, llIn, &po, &lo, true); }
+    hipEvent_t a = nullptr, b = nullptr;
+    if (!e) e = (long)hipEventCreate(&a);
+    if (!e) e = (long)hipEventCreate(&b);
+    if (!e) e = (long)hipEventRecord(a, k->stream());
+    for (int i = 0; i < nReps && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, plIn, llIn, &po, &lo, true); }
+    if (!e) e = (long)hipEventRecord(b, k->stream());
+    if (!e) e = (long)hipEventSynchronize(b);
+    float ms = 0.f;
+    if (!e) e = (long)hipEventElapsedTime(&ms, a, b);
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+    if (e) { put_error(k, e, szErr, errMax); return (MCH_LONG)e; }
+    *pfMs = ms / (float)nReps;
+    return 0;
+}
+
+}  // extern "C"

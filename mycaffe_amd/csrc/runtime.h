@@ -1,0 +1,138 @@
+// Handle tables and per-kernel state of libmycaffe_hip.so.
+//
+// Mirrors the object model the reference DLL exposes through its C ABI: a table
+// of "kernels" (one device context each, CudaDnnDLL/dllmain.cpp:6-14), and inside
+// each kernel integer-handle tables for device memory and for the cuDNN /
+// tensor-descriptor / attention / RoPE / extension objects
+// (CudaDnnDLL/Cuda Files/memorycol.h:282-370, handlecol.h:21-113).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/mycaffe_hip_abi.h"
+#include "kernels.h"
+
+namespace mch {
+
+struct MemItem {
+    void* ptr = nullptr;
+    size_t count = 0;     // elements
+    bool half = false;    // 16-bit (bf16) storage
+    bool used = false;
+    bool view = false;    // aliases part of another item (memory pointer)
+    long base = 0;        // owning handle when view
+    uint64_t version = 0; // bumped on every write through the ABI
+    DType dt() const { return half ? BF16 : F32; }
+    size_t esize() const { return half ? 2 : 4; }
+};
+
+// Device memory by handle.  Handles are 1-based; 0 is the null handle.
+class MemTable {
+public:
+    long alloc(size_t count, bool half, hipStream_t s, long* h);
+    long alloc_view(long hBase, size_t offset, size_t count, long* h);
+    long free(long h);
+    long get(long h, MemItem** it);
+    void touch(long h);               // mark written
+    uint64_t version(long h);
+    void free_all();
+private:
+    long new_slot();
+    std::vector<MemItem> m_items{1};  // slot 0 unused
+    std::vector<long> m_free;
+};
+
+template <class S> class HandleTable {
+public:
+    long create(long* h)
+    {
+        for (size_t i = 1; i < m_items.size(); i++)
+            if (!m_items[i]) { m_items[i].reset(new S()); *h = (long)i; return 0; }
+        m_items.emplace_back(new S());
+        *h = (long)m_items.size() - 1;
+        return 0;
+    }
+    S* get(long h) { return (h > 0 && (size_t)h < m_items.size()) ? m_items[h].get() : nullptr; }
+    long free(long h)
+    {
+        if (h <= 0 || (size_t)h >= m_items.size() || !m_items[h]) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        m_items[h].reset();
+        return 0;
+    }
+    void clear() { m_items.clear(); m_items.emplace_back(nullptr); }
+private:
+    std::vector<std::unique_ptr<S>> m_items{1};
+};
+
+struct CudnnState { long stream = 0; };
+struct TensorDesc { bool half = false; int n = 0, c = 0, h = 0, w = 0, sn = 0, sc = 0, sh = 0, sw = 0; };
+struct AttnState {
+    bool set = false, training = false;
+    int batch = 0, block = 0, heads = 0, hs = 0;
+    float dropout = 0.f, scale = 1.f;
+    // cache of "the (T,T) mask is the lower-triangular ones matrix"
+    long maskHandle = 0; uint64_t maskVersion = 0; int maskT = 0; bool maskCausal = false;
+};
+struct RopeState {
+    bool set = false;
+    int sharedIdx = 0, count = 0, batch = 0, seq = 0, heads = 0, hs = 0;
+    float theta = 10000.f;
+    std::shared_ptr<void> dcos, dsin;  // device tables [seq, hs/2] fp32, shared by sharedIdx
+};
+struct ExtensionState {
+    void* lib = nullptr;
+    void* fnInvoke = nullptr;
+    void* fnInvokeEx = nullptr;
+    ~ExtensionState();
+};
+
+class Kernel {
+public:
+    Kernel();
+    ~Kernel();
+    long initialize(const float* pf, long n);
+    long run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float** ppOut, MCH_LONG* plOut, bool timing);
+    long run_extension(long hExt, long fn, float* pf, long lf, MCH_TCHAR* szIn, float** ppOut, MCH_LONG* plOut,
+                       MCH_TCHAR* szErr, long errMax);
+    long create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut);
+    long query_extension(MCH_LONG* pIn, long n, MCH_TCHAR* out, long outMax, MCH_TCHAR* err, long errMax);
+    long alloc_host(long count, float** dst, const float* src, bool srcOnDevice);
+    long free_host(float* p);
+    long get_pointer(long h, void** pp);
+    hipStream_t stream() const { return m_stream; }
+    int device() const { return m_device; }
+    std::string device_name();
+    std::string last_detail;  // human-readable detail of the last failure
+
+private:
+    long workspace(size_t bytes, void** p);
+    long staging(size_t bytes, void** p);
+    long mem(long h, MemItem** it) { return m_mem.get(h, it); }
+    bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
+
+    int m_device = 0;
+    hipStream_t m_stream = nullptr;
+    MemTable m_mem;
+    HandleTable<CudnnState> m_cudnn;
+    HandleTable<TensorDesc> m_tdesc;
+    HandleTable<AttnState> m_attn;
+    HandleTable<RopeState> m_rope;
+    HandleTable<ExtensionState> m_ext;
+    std::map<int, std::weak_ptr<void>> m_ropeSharedCos, m_ropeSharedSin;
+    void* m_ws = nullptr; size_t m_wsBytes = 0;          // device scratch (split-K partials, conversions)
+    void* m_stage = nullptr; size_t m_stageBytes = 0;    // pinned host staging
+    std::mutex m_stageLock;
+    std::vector<float*> m_hostAllocs;
+    std::mutex m_hostLock;
+};
+
+// UTF-16 helpers
+std::string utf16_to_utf8(const MCH_TCHAR* s);
+void utf8_to_utf16(const std::string& s, MCH_TCHAR* out, long max);
+
+}  // namespace mch

@@ -1,0 +1,370 @@
+"""Host-side mirrors of the MyCaffe layers that call the attention hot path.
+
+These follow the C# ``forward`` methods call for call (cited per class), so that a
+forward pass here issues the same sequence of ``CudaDnn`` calls, with the same
+argument packing, as the unchanged C# host would issue against the native library.
+Inference only: dropout layers are identity and backward is not mirrored.
+"""
+import math
+
+import numpy as np
+
+from .cudadnn import DIR, SOFTMAX_ALGORITHM, SOFTMAX_MODE
+
+
+class Blob:
+    """Shape + device handle, the part of MyCaffe/common/Blob.cs the layers use."""
+
+    def __init__(self, cuda, shape=None, half=False):
+        self.cuda = cuda
+        self.half = half
+        self.shape_ = []
+        self.gpu_data = 0
+        self._capacity = 0
+        if shape is not None:
+            self.Reshape(*shape)
+
+    def Reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (list, tuple)):
+            shape = tuple(shape[0])
+        self.shape_ = [int(s) for s in shape]
+        n = self.count()
+        if n > self._capacity:
+            if self.gpu_data:
+                self.cuda.FreeMemory(self.gpu_data)
+            self.gpu_data = self.cuda.AllocMemory(n, bHalfSize=self.half)
+            self._capacity = n
+
+    def ReshapeLike(self, other):
+        self.Reshape(*other.shape_)
+
+    def count(self, start=0, end=None):
+        s = self.shape_[start:end]
+        return int(np.prod(s)) if s else 1
+
+    def shape(self, i):
+        return self.shape_[i]
+
+    num = property(lambda self: self.shape_[0])
+    channels = property(lambda self: self.shape_[1] if len(self.shape_) > 1 else 1)
+    height = property(lambda self: self.shape_[2] if len(self.shape_) > 2 else 1)
+    width = property(lambda self: self.shape_[3] if len(self.shape_) > 3 else 1)
+    num_axes = property(lambda self: len(self.shape_))
+    mutable_gpu_data = property(lambda self: self.gpu_data)
+
+    @property
+    def mutable_cpu_data(self):
+        return self.cuda.GetMemoryFloat(self.gpu_data, self.count()).reshape(self.shape_)
+
+    @mutable_cpu_data.setter
+    def mutable_cpu_data(self, values):
+        self.cuda.SetMemory(self.gpu_data, np.asarray(values, np.float32).reshape(-1), nCount=self.count())
+
+    def SetData(self, value):
+        self.cuda.set(self.count(), self.gpu_data, float(value))
+
+    def CopyFrom(self, src):
+        self.ReshapeLike(src)
+        self.cuda.copy(self.count(), src.gpu_data, self.gpu_data)
+
+    def MatMul(self, blobA, blobB, bReshape=False, bTransA=False, bTransB=False, dfScale=1.0):
+        """Blob.cs:4229-4269: batched row-major matmul over the two leading axes."""
+        outer = blobA.count(0, 2)
+        m = blobA.shape(3) if bTransA else blobA.shape(2)
+        n = blobB.shape(2) if bTransB else blobB.shape(3)
+        k = blobA.shape(2) if bTransA else blobA.shape(3)
+        shape = [blobA.shape(0), blobB.shape(1), m, n]
+        if bReshape:
+            self.Reshape(*shape)
+        elif self.shape_ != shape:
+            raise ValueError("This (resulting) blob does not have the correct shape! Expected %s" % shape)
+        self.cuda.matmul(outer, m, n, k, blobA.gpu_data, blobB.gpu_data, self.gpu_data, dfScale, bTransA, bTransB)
+
+    def scale_data(self, df):
+        self.cuda.scal(self.count(), df, self.gpu_data)
+
+    def Dispose(self):
+        if self.gpu_data:
+            self.cuda.FreeMemory(self.gpu_data)
+            self.gpu_data = 0
+            self._capacity = 0
+
+
+class InnerProductLayer:
+    """MyCaffe/layers/InnerProductLayer.cs:372-417.  Weights are (num_output, K)."""
+
+    def __init__(self, cuda, num_output, bias_term=True, axis=2, half=False):
+        self.cuda, self.N, self.bias_term, self.axis, self.half = cuda, num_output, bias_term, axis, half
+        self.blobs = []
+        self.bias_multiplier = None
+
+    def Setup(self, bottom, weight=None, bias=None):
+        self.K = bottom.count(self.axis)
+        w = Blob(self.cuda, (self.N, self.K), self.half)
+        if weight is not None:
+            w.mutable_cpu_data = weight
+        self.blobs = [w]
+        if self.bias_term:
+            b = Blob(self.cuda, (self.N,), self.half)
+            if bias is not None:
+                b.mutable_cpu_data = bias
+            self.blobs.append(b)
+
+    def Forward(self, bottom, top):
+        M = bottom.count(0, self.axis)
+        top.Reshape(*(bottom.shape_[:self.axis] + [self.N]))
+        hW = self.blobs[0].gpu_data
+        if M == 1 and not self.half:
+            self.cuda.gemv(False, self.N, self.K, 1.0, hW, bottom.gpu_data, 0.0, top.gpu_data)
+            if self.bias_term:
+                self.cuda.axpy(self.N, 1.0, self.blobs[1].gpu_data, top.gpu_data)
+        else:
+            self.cuda.gemm(False, True, M, self.N, self.K, 1.0, bottom.gpu_data, hW, 0.0, top.gpu_data)
+            if self.bias_term:
+                if self.bias_multiplier is None or self.bias_multiplier.count() < M:
+                    self.bias_multiplier = Blob(self.cuda, (M,), self.half)
+                    self.bias_multiplier.SetData(1.0)
+                self.cuda.gemm(False, False, M, self.N, 1, 1.0, self.bias_multiplier.gpu_data, self.blobs[1].gpu_data, 1.0,
+                               top.gpu_data)
+
+
+class TransposeLayer:
+    """MyCaffe.layers.beta/layers.beta/TransposeLayer.cs:127-213."""
+
+    def __init__(self, cuda, dim):
+        self.cuda, self.dim = cuda, list(dim)
+        self._key = None
+
+    def Forward(self, bottom, top):
+        shape = bottom.shape_
+        top_shape = [shape[d] for d in self.dim]
+        if bottom.gpu_data == top.gpu_data:
+            raise ValueError("The Transpose layer does not support in-place computation.")
+        top.Reshape(*top_shape)
+        key = (tuple(shape), tuple(self.dim))
+        if key != self._key:
+            n = len(shape)
+            bc = [int(np.prod(shape[i + 1:])) for i in range(n)]
+            tc = [int(np.prod(top_shape[i + 1:])) for i in range(n)]
+            self.counts_b = self.cuda.AllocMemory(np.float32(bc))
+            self.counts_t = self.cuda.AllocMemory(np.float32(tc))
+            self.fmap = self.cuda.AllocMemory(np.float32(self.dim))
+            self.buffer = self.cuda.AllocMemory(bottom.count() * n)
+            self._key = key
+        self.cuda.transpose(bottom.count(), bottom.gpu_data, top.gpu_data, self.counts_b, self.counts_t, self.fmap,
+                            len(shape), self.buffer)
+
+
+class SoftmaxLayer:
+    """MyCaffe/layers/SoftmaxLayer.cs:172-181, 339-345 (cuDNN engine)."""
+
+    def __init__(self, cuda, axis=-1):
+        self.cuda, self.axis = cuda, axis
+        self.hCudnn = cuda.CreateCuDNN()
+        self.hBottomDesc = cuda.CreateTensorDesc()
+        self.hTopDesc = cuda.CreateTensorDesc()
+
+    def Forward(self, bottom, top):
+        axis = self.axis % bottom.num_axes
+        nN, nK, nH = bottom.count(0, axis), bottom.shape(axis), bottom.count(axis + 1)
+        mode = SOFTMAX_MODE.INSTANCE if nH == 1 else SOFTMAX_MODE.CHANNEL
+        top.ReshapeLike(bottom)
+        self.cuda.SetTensorDesc(self.hBottomDesc, nN, nK, nH, 1, bottom.half)
+        self.cuda.SetTensorDesc(self.hTopDesc, nN, nK, nH, 1, top.half)
+        self.cuda.SoftmaxForward(self.hCudnn, SOFTMAX_ALGORITHM.ACCURATE, mode, 1.0, self.hBottomDesc, bottom.gpu_data, 0.0,
+                                 self.hTopDesc, top.gpu_data)
+
+
+class CausalSelfAttentionLayer:
+    """MyCaffe.layers.gpt/layers.gpt/CausalSelfAttentionLayer.cs (setup :96-250, forward :526-628).
+
+    ``enable_cuda_scaled_dot_product_attention`` selects the fused attention handle
+    (ids 160-163); otherwise the explicit transpose / MatMul / scale / mask /
+    softmax / MatMul chain runs, as in the reference.
+    """
+
+    def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
+        self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
+        self.nSize = embed // heads
+        self.bias_term, self.half = bias_term, half
+        self.enable_sdpa = enable_cuda_scaled_dot_product_attention
+        self.enable_rope, self.rope_theta = enable_rotary_positional_embedding, rope_theta
+        self.dfIgnoreVal = -1e29
+        self.c_attn = InnerProductLayer(cuda, 3 * embed, bias_term, 2, half)
+        self.c_proj = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.transpose = TransposeLayer(cuda, (0, 2, 1, 3))
+        self.transposeQ = TransposeLayer(cuda, (0, 1, 3, 2))
+        self.softmax = SoftmaxLayer(cuda, -1)
+        names = "IpAttn Q K V Qt Kt Vt Kt1 AttA AttB Work Y".split()
+        self.b = {n: Blob(cuda, half=half) for n in names}
+        self.blobMask = Blob(cuda, (1, 1, block_size, block_size))
+        mask = np.tril(np.ones((block_size, block_size), np.float32))  # fillMask :276-291
+        self.blobMask.mutable_cpu_data = mask
+        self.hCudnn = self.hAttn = self.hRope = 0
+        self._set_for = None
+
+    def Setup(self, bottom, w_attn, b_attn, w_proj, b_proj):
+        self.c_attn.Setup(bottom, w_attn, b_attn)
+        y = Blob(self.cuda, bottom.shape_, self.half)
+        self.c_proj.Setup(y, w_proj, b_proj)
+        y.Dispose()
+
+    def _reshape(self, B, T):
+        if self._set_for == (B, T):
+            return
+        if self.enable_sdpa:
+            if not self.hCudnn:
+                self.hCudnn = self.cuda.CreateCuDNN()
+                self.hAttn = self.cuda.CreateAttn()
+            self.cuda.SetAttn(self.hCudnn, self.hAttn, 0, False, B, self.nBlockSize, self.nHeads, self.nSize, 0.0)
+        if self.enable_rope:
+            if self.hRope:
+                self.cuda.FreeRope(self.hRope)
+            self.hRope = self.cuda.CreateRope(0, 0, B * T * self.nEmbed, B, T, self.nHeads, self.nSize, self.rope_theta)
+        if T != self.nBlockSize and not self.enable_sdpa:
+            m = Blob(self.cuda, (1, 1, T, T))
+            m.mutable_cpu_data = np.tril(np.ones((T, T), np.float32))
+            self.blobMaskT = m
+        self._set_for = (B, T)
+
+    def Forward(self, blobX, top):
+        B, T, C = blobX.shape_[:3]
+        if T > self.nBlockSize:
+            raise ValueError("sequence longer than block_size")
+        self._reshape(B, T)
+        b, cuda, H, hs = self.b, self.cuda, self.nHeads, self.nSize
+        # q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
+        self.c_attn.Forward(blobX, b["IpAttn"])
+        for name in "QKV":
+            b[name].Reshape(B, T, H, hs)
+        nCount = b["Q"].count()
+        ip = b["IpAttn"]
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 0, ip.gpu_data, b["Q"].gpu_data, DIR.FWD)
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 1, ip.gpu_data, b["K"].gpu_data, DIR.FWD)
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 2, ip.gpu_data, b["V"].gpu_data, DIR.FWD)
+        if self.hRope:
+            cuda.RopeForward(self.hRope, b["Q"].count(), b["Q"].gpu_data, b["Q"].gpu_data)
+            cuda.RopeForward(self.hRope, b["K"].count(), b["K"].gpu_data, b["K"].gpu_data)
+        # (B, T, nh, hs) -> (B, nh, T, hs)
+        self.transpose.Forward(b["Q"], b["Qt"])
+        self.transpose.Forward(b["K"], b["Kt"])
+        self.transpose.Forward(b["V"], b["Vt"])
+        if self.enable_sdpa:
+            b["Work"].ReshapeLike(b["Vt"])
+            mask = self.blobMask
+            if T != self.nBlockSize:
+                # the handle reads a (1,1,T,T) mask for the block size it is run with
+                if getattr(self, "_sdpa_mask_T", None) != T:
+                    self.blobMaskSdpa = Blob(cuda, (1, 1, T, T))
+                    self.blobMaskSdpa.mutable_cpu_data = np.tril(np.ones((T, T), np.float32))
+                    self._sdpa_mask_T = T
+                mask = self.blobMaskSdpa
+            cuda.AttnScaledDotProductForward(self.hCudnn, self.hAttn, T, b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data,
+                                             mask.gpu_data, b["Work"].gpu_data, False)
+        else:
+            self.transposeQ.Forward(b["Kt"], b["Kt1"])
+            dfScale = 1.0 / math.sqrt(hs)
+            b["AttA"].MatMul(b["Qt"], b["Kt1"], bReshape=True)
+            b["AttA"].scale_data(dfScale)
+            mask = self.blobMask if T == self.nBlockSize else self.blobMaskT
+            cuda.mask(b["AttA"].count(), mask.count(), 0.0, self.dfIgnoreVal, b["AttA"].gpu_data, mask.gpu_data, b["AttA"].gpu_data)
+            self.softmax.Forward(b["AttA"], b["AttB"])
+            b["Work"].MatMul(b["AttB"], b["Vt"], bReshape=True)
+        # y.transpose(1, 2).contiguous().view(B, T, C)
+        self.transpose.Forward(b["Work"], b["Y"])
+        b["Y"].Reshape(B, T, C)
+        self.c_proj.Forward(b["Y"], top)
+
+
+class MultiheadAttentionLayer:
+    """MyCaffe.layers.gpt/layers.gpt/MultiheadAttentionLayer.cs:643-811 (no KV cache:
+    the cached decode branch is served by :meth:`CudaDnn.AttnDecodeForward`).
+
+    ``Forward(q, k, v, mask)``: mask is ``None``, a (1,1,T,T) blob (causal), a
+    (B,T_k) key-padding blob or a (B,T_q,T_k) blob; the last two take the
+    mask_batch route, as in the reference.
+    """
+
+    def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
+        self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
+        self.nSize = embed // heads
+        self.half = half
+        self.enable_sdpa = enable_cuda_scaled_dot_product_attention
+        self.enable_rope, self.rope_theta = enable_rotary_positional_embedding, rope_theta
+        self.c_attnQ = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.c_attnK = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.c_attnV = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.c_proj = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.transpose = TransposeLayer(cuda, (0, 2, 1, 3))
+        self.transposeK = TransposeLayer(cuda, (0, 2, 1, 3))
+        self.transposeQ = TransposeLayer(cuda, (0, 1, 3, 2))
+        self.softmax = SoftmaxLayer(cuda, -1)
+        self.b = {n: Blob(cuda, half=half) for n in "Q K V Qt Kt Vt Kt1 AttA AttB Work Y".split()}
+        self.hCudnn = self.hAttn = self.hRope = 0
+        self._set_for = None
+        self.options = {}
+
+    def SetLayerOption(self, name, value):
+        self.options[name] = value
+
+    def Setup(self, q, k, v, weights):
+        """weights: dict with wq,bq,wk,bk,wv,bv,wo,bo ([out,in] matrices)."""
+        self.c_attnQ.Setup(q, weights["wq"], weights.get("bq"))
+        self.c_attnK.Setup(k, weights["wk"], weights.get("bk"))
+        self.c_attnV.Setup(v, weights["wv"], weights.get("bv"))
+        self.c_proj.Setup(q, weights["wo"], weights.get("bo"))
+
+    def Forward(self, q, k, v, blobMask, top):
+        cuda, H, hs, b = self.cuda, self.nHeads, self.nSize, self.b
+        B, Tq, C = q.shape_[:3]
+        Tk = k.shape_[1]
+        nPos = int(self.options.get("position", -1))
+        self.c_attnQ.Forward(q, b["Q"])
+        self.c_attnK.Forward(k, b["K"])
+        self.c_attnV.Forward(v, b["V"])
+        b["Q"].Reshape(B, Tq, H, hs)
+        b["K"].Reshape(B, Tk, H, hs)
+        b["V"].Reshape(B, Tk, H, hs)
+        if self.enable_rope:
+            if not self.hRope:
+                self.hRope = cuda.CreateRope(0, 0, B * self.nBlockSize * C, B, self.nBlockSize, H, hs, self.rope_theta)
+            nFreqOffset = nPos * hs // 2 if nPos > 0 else -1
+            cuda.RopeForward(self.hRope, b["Q"].count(), b["Q"].gpu_data, b["Q"].gpu_data, nFreqOffset)
+            cuda.RopeForward(self.hRope, b["K"].count(), b["K"].gpu_data, b["K"].gpu_data, nFreqOffset)
+        self.transpose.Forward(b["Q"], b["Qt"])
+        self.transposeK.Forward(b["K"], b["Kt"])
+        self.transposeK.Forward(b["V"], b["Vt"])
+        is_qk_mask = (blobMask is not None and blobMask.num_axes == 4 and blobMask.num == 1 and blobMask.channels == 1
+                      and blobMask.height == Tq and blobMask.width == Tk)
+        full_mask = blobMask is not None and not is_qk_mask and blobMask.count() == B * Tq * Tk and Tq > 1
+        if self.enable_sdpa and not full_mask:
+            if self._set_for != B:
+                if not self.hCudnn:
+                    self.hCudnn = cuda.CreateCuDNN()
+                    self.hAttn = cuda.CreateAttn()
+                cuda.SetAttn(self.hCudnn, self.hAttn, 0, False, B, self.nBlockSize, H, hs, 0.0)
+                self._set_for = B
+            b["Work"].ReshapeLike(b["Qt"])
+            cuda.AttnScaledDotProductForward(self.hCudnn, self.hAttn, Tq, b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data,
+                                             blobMask.gpu_data if blobMask is not None else 0, b["Work"].gpu_data,
+                                             not is_qk_mask, Tk if Tk != Tq else None)
+        else:
+            # the fused handle only understands (1,1,T,T) or (B,T) masks (attn.cu:544-556); a
+            # (B,T_q,T_k) mask goes through the explicit chain (MultiheadAttentionLayer.cs:733-742)
+            self.transposeQ.Forward(b["Kt"], b["Kt1"])
+            dfScale = 1.0 / math.sqrt(hs)
+            b["AttA"].MatMul(b["Qt"], b["Kt1"], bReshape=True)
+            b["AttA"].scale_data(dfScale)
+            if blobMask is not None:
+                if is_qk_mask:
+                    cuda.mask(b["AttA"].count(), blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data, blobMask.gpu_data, b["AttA"].gpu_data)
+                else:
+                    cuda.mask_batch(b["AttA"].count(), b["AttA"].num, blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data,
+                                    blobMask.gpu_data, b["AttA"].gpu_data)
+            self.softmax.Forward(b["AttA"], b["AttB"])
+            b["Work"].MatMul(b["AttB"], b["Vt"], bReshape=True)
+        self.transpose.Forward(b["Work"], b["Y"])
+        b["Y"].Reshape(B, Tq, C)
+        self.c_proj.Forward(b["Y"], top)

@@ -1,0 +1,359 @@
+"""GPU parity of the CudaDnn primitives on the attention path, called through the
+C ABI exactly as the C# host packs them, checked against the CPU checker and the
+reference's inline known-answer vectors."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mycaffe_amd.cudadnn import CudaDnnError, DIR, ERROR, SOFTMAX_ALGORITHM, SOFTMAX_MODE
+from oracle import attention_ref as R
+from tests.conftest import BF16_RTOL, FP32_RTOL, GOLDEN, assert_close, bf16_round
+
+pytestmark = pytest.mark.gpu
+INL = json.load(open(os.path.join(GOLDEN, "inline_vectors.json")))
+
+
+def test_device_name_and_alloc_is_zero_filled(dev):
+    assert "gfx950" in dev.cuda.GetDeviceName(0)
+    h = dev.zeros(1000)
+    assert np.all(dev.get(h) == 0)
+    hh = dev.zeros(1000, half=True)
+    assert np.all(dev.get(hh) == 0)
+
+
+def test_set_get_memory_round_trip_and_half_storage(dev):
+    x = np.random.default_rng(0).standard_normal(5000).astype(np.float32)
+    h = dev.put(x)
+    assert np.array_equal(dev.get(h), x)
+    dev.cuda.SetMemory(h, x[::-1].copy())
+    assert np.array_equal(dev.get(h), x[::-1])
+    assert np.array_equal(dev.cuda.GetMemoryFloat(h, 7), x[::-1][:7])
+    hh = dev.put(x, half=True)
+    assert np.array_equal(dev.get(hh), bf16_round(x))
+    # copy converts between storage types
+    h2 = dev.zeros(5000)
+    dev.cuda.copy(5000, hh, h2)
+    assert np.array_equal(dev.get(h2), bf16_round(x))
+    dev.cuda.copy(100, h, h2, 10, 20)
+    exp = bf16_round(x)
+    exp[20:120] = x[::-1][10:110]
+    assert np.array_equal(dev.get(h2), exp)
+
+
+def test_memory_pointer_views_alias_the_allocation(dev):
+    x = np.arange(64, dtype=np.float32)
+    h = dev.put(x)
+    v = dev.cuda.CreateMemoryPointer(h, 16, 8)
+    assert np.array_equal(dev.cuda.GetMemoryFloat(v), x[16:24])
+    dev.cuda.set(8, v, 5.0)
+    assert np.array_equal(dev.get(h)[16:24], np.full(8, 5, np.float32))
+    dev.cuda.FreeMemoryPointer(v)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.CreateMemoryPointer(h, 60, 8)
+    assert e.value.code == ERROR.MEMORY_RANGE_EXCEEDED
+
+
+def test_error_codes_bad_handle_and_arg_count(dev):
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.GetMemoryFloat(9999)
+    assert e.value.code == ERROR.MEMORY_NOT_FOUND
+    with pytest.raises(CudaDnnError) as e:   # mask needs exactly 7 longs (device.cu:2108)
+        dev.cuda._ex2(264, [0.0, 1.0], [4, 4, 0, 0, 1, 1])
+    assert e.value.code == ERROR.PARAM_OUT_OF_RANGE
+    with pytest.raises(CudaDnnError) as e:   # Ex2-style id through the legacy entry point has no long array
+        dev.cuda.RunFloat(dev.cuda.m_hKernel, 264, [0.0, 1.0])
+    assert e.value.code == ERROR.PARAM_OUT_OF_RANGE
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda._ex2(321, None, [1])
+    assert e.value.code == ERROR.NOT_IMPLEMENTED
+    h = dev.put(np.zeros(4, np.float32))
+    hh = dev.put(np.zeros(4, np.float32), half=True)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.add(4, h, hh, h)
+    assert e.value.code == ERROR.MEMORY_MIXED_HALF_TYPES
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.add(5, h, h, h)
+    assert e.value.code == ERROR.MEMORY_RANGE_EXCEEDED
+
+
+def test_gemm_inline_vectors_all_transposes(dev):
+    g = INL["gemm"]
+    exp = np.array(g["result"], np.float32)
+    hC = dev.zeros(8)
+    for tA, tB, a, b in [(0, 0, g["data"][:6], g["data"]), (1, 0, g["A_T"], g["data"]), (1, 1, g["A_T"], g["B_T"]),
+                         (0, 1, g["data"][:6], g["B_T"])]:
+        hA, hB = dev.put(a), dev.put(b)
+        for _ in range(2):
+            dev.cuda.gemm(bool(tA), bool(tB), 2, 4, 3, 1.0, hA, hB, 0.0, hC)
+            assert np.array_equal(dev.get(hC), exp), (tA, tB)
+
+
+def test_gemv_inline_vectors(dev):
+    g = INL["gemv"]
+    hA = dev.put(g["data"])
+    hx, hy = dev.put(g["data"][:3]), dev.zeros(2)
+    dev.cuda.gemv(False, 2, 3, 1.0, hA, hx, 0.0, hy)
+    assert np.array_equal(dev.get(hy), np.float32(g["result_notrans"]))
+    hy2, hx2 = dev.put(g["data"][:2]), dev.zeros(3)
+    dev.cuda.gemv(True, 2, 3, 1.0, hA, hy2, 0.0, hx2)
+    assert np.array_equal(dev.get(hx2), np.float32(g["result_trans"]))
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(200, 136, 96), (128, 128, 64), (37, 53, 29), (8, 2304, 768), (513, 260, 20)])
+def test_gemm_fp32_vs_checker(dev, tA, tB, m, n, k):
+    rng = np.random.default_rng(m * 7 + n)
+    A = rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32)
+    B = rng.standard_normal((n, k) if tB else (k, n)).astype(np.float32)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    hA, hB, hC = dev.put(A), dev.put(B), dev.put(C0)
+    dev.cuda.gemm(tA, tB, m, n, k, 0.5, hA, hB, 2.0, hC)
+    ref = R.gemm(tA, tB, m, n, k, 0.5, A, B, 2.0, C0, dtype=np.float64)
+    assert_close(dev.get(hC), ref, FP32_RTOL, "gemm fp32")
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 128), (200, 136, 96), (100, 72, 40)])
+def test_gemm_bf16_inner_product_shape(dev, m, n, k):
+    rng = np.random.default_rng(n)
+    A = bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    B = bf16_round((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    hA, hB, hC = dev.put(A, True), dev.put(B, True), dev.zeros(m * n, True)
+    dev.cuda.gemm(False, True, m, n, k, 1.0, hA, hB, 0.0, hC)
+    ref = R.gemm(False, True, m, n, k, 1.0, A, B, 0.0, dtype=np.float64)
+    assert_close(dev.get(hC), ref, BF16_RTOL, "gemm bf16")
+
+
+def test_gemm_offsets_and_bias_rank1_update(dev):
+    # InnerProductLayer.cs:411-415: y = x W^T, then y += ones(M,1) * bias(1,N) through gemm with K = 1
+    rng = np.random.default_rng(3)
+    M, N, K = 96, 80, 64
+    x, W, b = rng.standard_normal((M, K)), rng.standard_normal((N, K)), rng.standard_normal(N)
+    hx, hW, hb, hones, hy = dev.put(x), dev.put(W), dev.put(b), dev.put(np.ones(M)), dev.zeros(M * N)
+    dev.cuda.gemm(False, True, M, N, K, 1.0, hx, hW, 0.0, hy)
+    dev.cuda.gemm(False, False, M, N, 1, 1.0, hones, hb, 1.0, hy)
+    assert_close(dev.get(hy), R.inner_product(x, W, b, np.float64), FP32_RTOL, "inner product")
+    # offsets: second half of A rows
+    hy2 = dev.zeros(M * N)
+    dev.cuda.gemm(False, True, M // 2, N, K, 1.0, hx, hW, 0.0, hy2, nAOffset=(M // 2) * K, nCOffset=(M // 2) * N)
+    out = dev.get(hy2, (M, N))
+    assert np.all(out[:M // 2] == 0)
+    assert_close(out[M // 2:], (x @ W.T)[M // 2:], FP32_RTOL, "gemm offsets")
+
+
+def test_matmul_batched_is_gemm2_with_swapped_operands(dev):
+    rng = np.random.default_rng(4)
+    outer, m, n, k = 6, 50, 24, 40
+    A, B = rng.standard_normal((outer, m, k)), rng.standard_normal((outer, k, n))
+    hA, hB, hC = dev.put(A), dev.put(B), dev.zeros(outer * m * n)
+    dev.cuda.matmul(outer, m, n, k, hA, hB, hC, 0.125)
+    assert_close(dev.get(hC), 0.125 * (A @ B), FP32_RTOL, "matmul")
+    Bt = B.transpose(0, 2, 1).copy()
+    hBt = dev.put(Bt)
+    dev.cuda.matmul(outer, m, n, k, hA, hBt, hC, 1.0, bTransB=True)
+    assert_close(dev.get(hC), A @ B, FP32_RTOL, "matmul transB")
+    assert_close(dev.get(hC), R.matmul(outer, m, n, k, A, Bt, transB=True, dtype=np.float64), FP32_RTOL, "matmul vs checker")
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_gemv_decode_shapes(dev, half):
+    rng = np.random.default_rng(5)
+    for d, n in [(288, 288), (768, 288), (288, 768), (1000, 52), (3, 7)]:
+        W = (rng.standard_normal((d, n)) * 0.02).astype(np.float32)
+        if half:
+            W = bf16_round(W)
+        x = rng.standard_normal(n).astype(np.float32)
+        y0 = rng.standard_normal(d).astype(np.float32)
+        hW, hx, hy = dev.put(W, half), dev.put(x), dev.put(y0)
+        dev.cuda.gemv(False, d, n, 1.0, hW, hx, 0.0, hy)
+        assert_close(dev.get(hy), W.astype(np.float64) @ x, FP32_RTOL, "gemv")
+        dev.cuda.gemv(False, d, n, 2.0, hW, hx, 1.0, hy)
+        assert_close(dev.get(hy), 3 * (W.astype(np.float64) @ x), FP32_RTOL, "gemv beta")
+        hx2 = dev.zeros(n)
+        dev.cuda.gemv(True, d, n, 1.0, hW, hy, 0.0, hx2)
+        assert_close(dev.get(hx2), W.astype(np.float64).T @ dev.get(hy), FP32_RTOL, "gemv transposed")
+
+
+def test_mask_inline_vectors(dev):
+    x = np.array(INL["mask"]["x"], np.float32)
+    n = x.size
+    hx, hm, hy = dev.put(x), dev.zeros(n), dev.zeros(n)
+    for i in range(n):
+        m = np.ones(n, np.float32)
+        m[i:] = 0
+        dev.cuda.SetMemory(hm, m)
+        dev.cuda.set(n, hy, 0)
+        dev.cuda.mask(n, n, 0.0, -np.inf, hx, hm, hy)
+        exp = x.copy()
+        exp[i:] = -np.inf
+        assert np.array_equal(dev.get(hy), exp)
+    x2 = np.array(INL["mask2"]["x"], np.float32)
+    hx2, hm2, hy2 = dev.put(x2), dev.put([1, 0, 1, 0]), dev.zeros(8)
+    dev.cuda.mask(8, 4, 0.0, -1e29, hx2, hm2, hy2)
+    assert np.array_equal(dev.get(hy2), R.mask(8, 4, 0.0, -1e29, x2, [1, 0, 1, 0]))
+
+
+def test_mask_batch_inline_vectors(dev):
+    g = INL["mask_batch"]
+    x = np.array(g["x"], np.float32)
+    hx, hm, hy = dev.put(x), dev.put(g["mask"]), dev.zeros(x.size)
+    dev.cuda.mask_batch(x.size, g["batch"], len(g["mask"]), 0.0, -np.inf, hx, hm, hy)
+    exp = x.copy()
+    exp[g["masked_positions"]] = -np.inf
+    assert np.array_equal(dev.get(hy), exp)
+
+
+def test_channel_copy_inline_vectors(dev):
+    g = INL["channel_copy"]
+    cnt = g["num"] * g["channels"] * g["inner"]
+    hall = dev.put(g["all"])
+    hs = []
+    for off, key in enumerate("ABC"):
+        h = dev.zeros(cnt)
+        dev.cuda.channel_copy(cnt, g["num"], g["channels"], g["blocks"], g["inner"], off, hall, h, DIR.FWD)
+        assert np.array_equal(dev.get(h), np.float32(g[key]))
+        hs.append(h)
+    hback = dev.zeros(len(g["all"]))
+    for off, h in enumerate(hs):
+        dev.cuda.channel_copy(cnt, g["num"], g["channels"], g["blocks"], g["inner"], off, hback, h, DIR.BWD)
+    assert np.array_equal(dev.get(hback), np.float32(g["all"]))
+
+
+def test_channel_copy_splits_fused_qkv(dev):
+    # CausalSelfAttentionLayer.cs:537-539: (B,T,3C) -> q,k,v (B,T,C)
+    rng = np.random.default_rng(6)
+    B, T, Cc = 3, 17, 48
+    x = rng.standard_normal((B, T, 3 * Cc)).astype(np.float32)
+    hx = dev.put(x)
+    for off in range(3):
+        h = dev.zeros(B * T * Cc)
+        dev.cuda.channel_copy(B * T * Cc, B, T, 3, Cc, off, hx, h, DIR.FWD)
+        assert np.array_equal(dev.get(h, (B, T, Cc)), x[..., off * Cc:(off + 1) * Cc])
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_transpose_head_split_and_generic(dev, half):
+    rng = np.random.default_rng(7)
+    shape = (2, 9, 4, 16)
+    x = bf16_round(rng.standard_normal(shape).astype(np.float32))
+    for perm in [(0, 2, 1, 3), (0, 1, 3, 2), (3, 2, 1, 0)]:
+        y = np.transpose(x, perm)
+        xs = [int(np.prod(shape[i + 1:])) for i in range(4)]
+        ys = [int(np.prod(y.shape[i + 1:])) for i in range(4)]
+        hx, hy = dev.put(x, half), dev.zeros(x.size, half)
+        hxc, hyc, hmap, hbuf = dev.put(xs), dev.put(ys), dev.put(perm), dev.zeros(x.size * 4)
+        dev.cuda.transpose(x.size, hx, hy, hxc, hyc, hmap, 4, hbuf)
+        assert np.array_equal(dev.get(hy, y.shape), y), perm
+        assert np.array_equal(dev.get(hy), R.transpose(x, xs, ys, perm))
+    hx, hy = dev.put(x, half), dev.zeros(x.size, half)
+    dev.cuda.transposeHW(2, 9, 4, 16, hx, hy)
+    assert np.array_equal(dev.get(hy, (2, 9, 16, 4)), x.transpose(0, 1, 3, 2))
+    big = rng.standard_normal((3, 2, 70, 45)).astype(np.float32)
+    hb, hb2 = dev.put(big), dev.zeros(big.size)
+    dev.cuda.transposeHW(3, 2, 70, 45, hb, hb2)
+    assert np.array_equal(dev.get(hb2, (3, 2, 45, 70)), big.transpose(0, 1, 3, 2))
+
+
+def test_softmax_forward_through_tensor_descriptors(dev):
+    rng = np.random.default_rng(8)
+    hc = dev.cuda.CreateCuDNN()
+    for rows, length in [(24, 200), (7, 3000), (5, 1)]:
+        x = (rng.standard_normal((rows, length)) * 4).astype(np.float32)
+        hx, hy = dev.put(x), dev.zeros(x.size)
+        bd, td = dev.cuda.CreateTensorDesc(), dev.cuda.CreateTensorDesc()
+        dev.cuda.SetTensorDesc(bd, rows, length, 1, 1)
+        dev.cuda.SetTensorDesc(td, rows, length, 1, 1)
+        dev.cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, bd, hx, 0.0, td, hy)
+        assert_close(dev.get(hy), R.softmax_lastaxis(x, np.float64), FP32_RTOL, "softmax")
+        dev.cuda.FreeTensorDesc(bd)
+        dev.cuda.FreeTensorDesc(td)
+    # channel mode with an inner axis: softmax over c for every (n, h)
+    x = rng.standard_normal((3, 10, 6)).astype(np.float32)
+    hx, hy = dev.put(x), dev.zeros(x.size)
+    bd, td = dev.cuda.CreateTensorDesc(), dev.cuda.CreateTensorDesc()
+    dev.cuda.SetTensorDesc(bd, 3, 10, 6, 1)
+    dev.cuda.SetTensorDesc(td, 3, 10, 6, 1)
+    dev.cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.CHANNEL, 1.0, bd, hx, 0.0, td, hy)
+    ref = R.softmax_lastaxis(x.transpose(0, 2, 1), np.float64).transpose(0, 2, 1)
+    assert_close(dev.get(hy), ref, FP32_RTOL, "softmax channel")
+    # masked rows of -1e29 stay finite and uniform
+    x = np.full((2, 8), -1e29, np.float32)
+    hx, hy = dev.put(x), dev.zeros(16)
+    dev.cuda.SetTensorDesc(bd, 2, 8, 1, 1)
+    dev.cuda.SetTensorDesc(td, 2, 8, 1, 1)
+    dev.cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, bd, hx, 0.0, td, hy)
+    assert np.allclose(dev.get(hy), 0.125)
+    dev.cuda.FreeCuDNN(hc)
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_rope_forward_vs_checker(dev, half):
+    rng = np.random.default_rng(9)
+    B, T, H, hs = 2, 12, 3, 16
+    x = bf16_round(rng.standard_normal((B, T, H, hs)).astype(np.float32))
+    h = dev.cuda.CreateRope(0, 0, x.size, B, T, H, hs, 10000.0)
+    hx, hy = dev.put(x, half), dev.zeros(x.size, half)
+    dev.cuda.RopeForward(h, x.size, hx, hy)
+    ref = R.rope_forward(x, T, H, hs, 10000.0)
+    assert_close(dev.get(hy), ref, BF16_RTOL if half else 2e-6, "rope")
+    # in place, as the layers call it
+    dev.cuda.RopeForward(h, x.size, hx, hx)
+    assert_close(dev.get(hx), ref, BF16_RTOL if half else 2e-6, "rope in place")
+    # decode form: one position, table offset pos*hs/2 (MultiheadAttentionLayer.cs:678-683)
+    one = x[:1, 5:6].copy()
+    h1, h1y = dev.put(one, half), dev.zeros(one.size, half)
+    dev.cuda.RopeForward(h, one.size, h1, h1y, 5 * hs // 2)
+    assert_close(dev.get(h1y), ref.reshape(B, T, H, hs)[0, 5], BF16_RTOL if half else 2e-6, "rope offset")
+    with pytest.raises(CudaDnnError) as e:   # offset that would leave the table
+        dev.cuda.RopeForward(h, one.size, h1, h1y, T * hs // 2)
+    assert e.value.code == ERROR.PARAM_OUT_OF_RANGE
+    dev.cuda.FreeRope(h)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.RopeForward(h, one.size, h1, h1y)
+    assert e.value.code == ERROR.ROPE_NOT_INITIALIZED
+
+
+def test_elementwise_family(dev):
+    rng = np.random.default_rng(10)
+    n = 10007
+    a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    ha, hb, hy = dev.put(a), dev.put(b), dev.zeros(n)
+    dev.cuda.add(n, ha, hb, hy)
+    assert np.array_equal(dev.get(hy), a + b)
+    dev.cuda.add(n, ha, hb, hy, 0.5)
+    assert_close(dev.get(hy), a + 0.5 * b, 1e-6, "add alpha")
+    dev.cuda.mul(n, ha, hb, hy)
+    assert np.array_equal(dev.get(hy), a * b)
+    dev.cuda.scale(n, 3.0, ha, hy)
+    assert np.array_equal(dev.get(hy), 3 * a)
+    dev.cuda.scal(n, 0.25, hy)
+    assert np.array_equal(dev.get(hy), 0.75 * a)
+    dev.cuda.axpy(n, 2.0, hb, hy)
+    assert_close(dev.get(hy), 0.75 * a + 2 * b, 1e-6, "axpy")
+    dev.cuda.silu_fwd(n, ha, hy)
+    assert_close(dev.get(hy), R.silu(a, np.float64), 1e-6, "silu")
+    dev.cuda.SwigluForward(n, ha, hb, hy)
+    assert_close(dev.get(hy), R.silu(a, np.float64) * b, 1e-6, "swiglu")
+    dev.cuda.set(n, hy, 7.0)
+    assert np.all(dev.get(hy) == 7)
+    dev.cuda.set(1, hy, 9.0, 3)
+    out = dev.get(hy)
+    assert out[3] == 9 and out[2] == 7 and out[4] == 7
+
+
+def test_embed_and_rmsnorm(dev):
+    rng = np.random.default_rng(11)
+    V, D = 50, 24
+    W = rng.standard_normal((V, D)).astype(np.float32)
+    ids = rng.integers(0, V, 13)
+    hW, hi, ht = dev.put(W), dev.put(ids.astype(np.float32)), dev.zeros(13 * D)
+    dev.cuda.embed_fwd(13 * D, hi, hW, 13, D, V, ht)
+    assert np.array_equal(dev.get(ht, (13, D)), W[ids])
+    x = rng.standard_normal((9, 288)).astype(np.float32)
+    w = rng.standard_normal(288).astype(np.float32)
+    hx, hw, hy = dev.put(x), dev.put(w), dev.zeros(x.size)
+    dev.cuda.RmsNormForward(9, 288, hx, hw, hy, 1e-5)
+    assert_close(dev.get(hy), R.rmsnorm_layer(x, w, 1e-5, np.float64), 1e-5, "rmsnorm")
+    dev.cuda.RmsNormForward(9, 288, hx, 0, hy, 1e-5)
+    assert_close(dev.get(hy), R.rmsnorm_layer(x, None, 1e-5, np.float64), 1e-5, "rmsnorm no weight")
