@@ -468,7 +468,7 @@ class CudaDnn:
     # ---- cuDNN-shaped handles ---------------------------------------------------------
     def CreateCuDNN(self, hStream=0):
         """CudaDnn.cs:3509-3520."""
-        return int(self.RunFloat(self.m_hKernel, CUDAFN.CREATE_CUDNN, [hStream] if hStream else None)[0])
+        return int(self.RunFloat(self.m_hKernel, CUDAFN.CREATE_CUDNN, [hStream])[0])
 
     def FreeCuDNN(self, h):
         """CudaDnn.cs:3527-3533."""
