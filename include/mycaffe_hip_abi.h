@@ -202,12 +202,16 @@ enum {
      *   GENERATE_IDS  f{hLlm, nSteps, wantLogits(0|1), id0, id1, ...}
      *                 -> f{next id after each position [, logits of every step]}
      *   SET_OPTION    f{hLlm, option, value}; option 1 = weight storage
-     *                 (0 fp32, 1 bf16), applied at the next LOAD
+     *                 (0 fp32, 1 bf16), applied at the next LOAD; option 2 = first
+     *                 step of the timed span; option 3 = replay one captured
+     *                 HIP graph per step (1, default) or launch eagerly (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
-     *                 -> f{batch x nSteps next ids} */
+     *                 -> f{batch x nSteps next ids}
+     *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it} */
     MCH_LLM_GENERATE_IDS = 100,
     MCH_LLM_SET_OPTION = 101,
-    MCH_LLM_GENERATE_BATCH = 102
+    MCH_LLM_GENERATE_BATCH = 102,
+    MCH_LLM_QUERY_TIMING = 103
 };
 
 MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);

@@ -48,7 +48,23 @@ struct DecodeArgs {
     int B, H, kvMul, hs, len, splits, chunk;
     long long strideB, strideH, strideT;
     float scale;
+    // when dlen is set the number of cached positions is read on the device (so one
+    // captured launch serves every decode step) and the per-split chunk is derived from it
+    const int* dlen;
+    int rowsPerIter;
 };
+
+__device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int* t1)
+{
+    int len = a.len, chunk = a.chunk;
+    if (a.dlen) {
+        len = *a.dlen;
+        chunk = (len + a.splits - 1) / a.splits;
+        chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
+    }
+    *t0 = split * chunk;
+    *t1 = min(len, *t0 + chunk);
+}
 
 // partial layout: part[((b*H + h)*splits + s) * (hs + 2)] = {m, l, acc[hs]}
 template <typename T, int LPR>
@@ -78,8 +94,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
         for (int i = 0; i < W; i++) qv[i] *= a.scale;
     }
 
-    const int t0 = split * a.chunk;
-    const int t1 = min(a.len, t0 + a.chunk);
+    int t0, t1;
+    decode_range(a, split, &t0, &t1);
 
     float m = -INFINITY, l = 0.f, acc[W];
 #pragma unroll
@@ -167,7 +183,8 @@ template <typename T> __global__ __launch_bounds__(64) void attn_decode_scalar_k
     const size_t base = (size_t)b * a.strideB + (size_t)(h / a.kvMul) * a.strideH;
     const T* kc = (const T*)a.kc + base;
     const T* vc = (const T*)a.vc + base;
-    const int t0 = split * a.chunk, t1 = min(a.len, t0 + a.chunk);
+    int t0, t1;
+    decode_range(a, split, &t0, &t1);
     constexpr int DPL = 8;  // output dims per lane: hs <= 512
     float m = -INFINITY, l = 0.f, acc[DPL];
     for (int i = 0; i < DPL; i++) acc[i] = 0.f;
@@ -268,6 +285,7 @@ static hipError_t launch_decode(hipStream_t s, DecodeArgs a, int kvH)
                 (((uintptr_t)a.q | (uintptr_t)a.kc | (uintptr_t)a.vc) % 16 == 0);
     if (fast) {
         int rpi = 4 * (64 / lprp) * 4;
+        a.rowsPerIter = rpi;
         pick_splits(a.B, a.H, a.len, rpi, &a.splits, &a.chunk);
         dim3 grid(a.splits, a.H, a.B);
         switch (lprp) {
@@ -277,6 +295,7 @@ static hipError_t launch_decode(hipStream_t s, DecodeArgs a, int kvH)
         }
     } else {
         if (a.hs > 512) return hipErrorInvalidValue;
+        a.rowsPerIter = 64;
         pick_splits(a.B, a.H, a.len, 64, &a.splits, &a.chunk);
         dim3 grid(a.splits, a.H, a.B);
         hipLaunchKernelGGL(attn_decode_scalar_kernel<T>, grid, 64, 0, s, a);
@@ -290,7 +309,7 @@ static hipError_t launch_decode(hipStream_t s, DecodeArgs a, int kvH)
 
 hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc, const void* vc, void* y, int B, int H,
                          int kvH, int hs, int len, long long strideB, long long strideH, long long strideT, float scale,
-                         void* workspace, size_t workspaceBytes)
+                         void* workspace, size_t workspaceBytes, const int* dlen)
 {
     if (B <= 0 || H <= 0 || hs <= 0 || len <= 0) return hipSuccess;
     if (kvH <= 0 || H % kvH != 0) return hipErrorInvalidValue;
@@ -300,6 +319,7 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
     a.q = q; a.kc = kc; a.vc = vc; a.y = y; a.part = (float*)workspace;
     a.B = B; a.H = H; a.kvMul = H / kvH; a.hs = hs; a.len = len; a.splits = 1; a.chunk = len;
     a.strideB = strideB; a.strideH = strideH; a.strideT = strideT; a.scale = scale;
+    a.dlen = dlen; a.rowsPerIter = 64;
     if (dt == F32) return launch_decode<float>(s, a, kvH);
     return launch_decode<bf16_t>(s, a, kvH);
 }

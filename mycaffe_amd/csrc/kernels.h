@@ -79,9 +79,11 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
 // one query per (b,h): q (B,H,hs), caches addressed as
 //   cache[b*strideB + (h/kvMul)*strideH + t*strideT + i], y (B,H,hs).  All dt.
+// With dlen set, `len` is only the upper bound used to size the launch and the
+// actual number of cached positions is read from *dlen on the device.
 hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc, const void* vc, void* y, int B, int H,
                          int kvH, int hs, int len, long long strideB, long long strideH, long long strideT,
-                         float scale, void* workspace, size_t workspaceBytes);
+                         float scale, void* workspace, size_t workspaceBytes, const int* dlen = nullptr);
 // rotate q (B,H,hs) and knew (B,kvH,hs) at position pos and append knew/vnew to the caches at pos
 hipError_t k_rope_append(hipStream_t s, DType dt, void* q, void* knew, const void* vnew, void* kc, void* vc, int B,
                          int H, int kvH, int hs, int pos, long long strideB, long long strideH, long long strideT,

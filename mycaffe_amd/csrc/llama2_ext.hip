@@ -1,0 +1,844 @@
+// libmycaffe_hip_llama2.so: the llama2 inference extension for gfx950.
+//
+// Drop-in for the reference's CudaExtension.llm32.llama2 DLL: same three exports
+// and function ids (CudaExtension.llm32.cpp:20-26, 67-268), loaded by the parent
+// library through CREATE_EXTENSION.  The forward pass computes what
+// TransformerGpu::forward / TransformerCpu::forward compute
+// (llama2_gpu.cpp:32-111, llama2_cpu.cpp:264-386) but is organised for MI355X:
+//
+//  * weights are repacked once at load (wq|wk|wv and w1|w3 row-concatenated per
+//    layer, optionally stored as bf16) so one token needs 7 launches per layer;
+//  * RMSNorm is fused into the prologue of the QKV and W1/W3 mat-vecs, SwiGLU and
+//    the residual adds into their epilogues;
+//  * position, current token and sampled token live in device memory, so a whole
+//    greedy generation runs without any host round trip, and one decode step is
+//    captured into a HIP graph that is replayed per token;
+//  * attention over the KV cache is the split-K decode kernel of the parent.
+//
+// KV cache layout: [layer][batch][seq_len][kv_dim] fp32, position-major inside a
+// sequence as in the reference (llama2_gpu.cpp:67-71).
+#include <dlfcn.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <atomic>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/mycaffe_hip_abi.h"
+#include "kernels.h"
+
+namespace mch {
+
+#define HIPCHK(x) do { hipError_t _e = (x); if (_e != hipSuccess) return (long)_e; } while (0)
+
+struct Config { int dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab_size, seq_len; };
+
+// ---- device-side generation state ---------------------------------------------------
+struct GenState {
+    int pos;        // position of the token being processed
+    int n_prompt;   // prompt length (same for all sequences of a batch)
+    int len;        // pos + 1, read by the attention kernel
+    int pad;
+};
+
+template <typename T> __device__ inline float wld(const T* p, size_t i);
+template <> __device__ inline float wld<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ inline float wld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+
+__device__ inline float wsum(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// x[b,:] = emb[token,:] where token is the forced prompt id while pos < n_prompt and
+// the previously sampled id afterwards (generate loop, llm.cpp:208-228)
+template <typename T>
+__global__ void embed_step_kernel(const GenState* st, const int* prompt, int promptStride, const int* next, const T* emb,
+                                  float* x, int dim, int* cur)
+{
+    const int b = blockIdx.x;
+    const int pos = st->pos;
+    const int tok = pos < st->n_prompt ? prompt[(size_t)b * promptStride + pos] : next[b];
+    if (threadIdx.x == 0) cur[b] = tok;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) x[(size_t)b * dim + i] = wld(emb, (size_t)tok * dim + i);
+}
+
+__global__ void advance_kernel(GenState* st)
+{
+    st->pos += 1;
+    st->len = st->pos + 1;
+}
+
+// 4 weight values of one row against 4 activations
+template <typename T> struct Row4;
+template <> struct Row4<float> {
+    __device__ static inline float4 load(const float* p) { return *(const float4*)p; }
+};
+template <> struct Row4<bf16_t> {
+    __device__ static inline float4 load(const bf16_t* p)
+    {
+        uint2 u = *(const uint2*)p;
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                           __uint_as_float(u.y & 0xffff0000u));
+    }
+};
+
+// Mat-vec family for one token per sequence.  One wavefront owns ROWS output rows
+// of W (n columns, n % 4 == 0) and walks them with 128-bit (fp32) / 64-bit (bf16)
+// loads; the activation chunk a lane needs is the same for every row, so it is
+// loaded (and, when NORM, RMS-normalised) once per batch entry.
+//   MODE 0: y[b,r]  = W[r,:] . xn[b,:]
+//   MODE 1: y[b,r] += W[r,:] . x[b,:]                      (residual epilogue)
+//   MODE 2: y[b,r]  = silu(W[r,:] . xn) * (W[r+half,:] . xn)   (SwiGLU epilogue, half = rows)
+// NORM: xn = g * x / sqrt(mean(x^2) + 1e-5), recomputed per wavefront from the
+// chunks it already holds (x is L2 resident; it saves a launch and a barrier).
+template <typename T, int MODE, bool NORM, int CH>
+__global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, const float* __restrict__ x,
+                                                     const float* __restrict__ g, float* __restrict__ y, int rows, int n,
+                                                     int B, int ldy)
+{
+    constexpr int ROWS = 2;
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int r0 = wave * ROWS;
+    if (r0 >= rows) return;
+    // weight chunks of this wavefront's rows stay in registers across the batch loop
+    float4 w[(MODE == 2 ? 2 : 1) * ROWS][CH];
+#pragma unroll
+    for (int rr = 0; rr < ROWS; rr++) {
+        const int r = min(r0 + rr, rows - 1);
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int j = (c * 64 + lane) * 4;
+            if (j < n) {
+                w[rr][c] = Row4<T>::load(W + (size_t)r * n + j);
+                if (MODE == 2) w[ROWS + rr][c] = Row4<T>::load(W + (size_t)(r + rows) * n + j);
+            } else {
+                w[rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (MODE == 2) w[ROWS + rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+    for (int b = 0; b < B; b++) {
+        const float* xb = x + (size_t)b * n;
+        float4 xv[CH];
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int j = (c * 64 + lane) * 4;
+            xv[c] = j < n ? *(const float4*)(xb + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (NORM) ss += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
+        }
+        if (NORM) {
+            ss = wsum(ss);
+            const float inv = 1.0f / sqrtf(ss / n + 1e-5f);
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const int j = (c * 64 + lane) * 4;
+                if (j < n) {
+                    const float4 gv = *(const float4*)(g + j);
+                    xv[c].x = gv.x * (inv * xv[c].x);
+                    xv[c].y = gv.y * (inv * xv[c].y);
+                    xv[c].z = gv.z * (inv * xv[c].z);
+                    xv[c].w = gv.w * (inv * xv[c].w);
+                }
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < ROWS; rr++) {
+            float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                a0 += w[rr][c].x * xv[c].x + w[rr][c].y * xv[c].y + w[rr][c].z * xv[c].z + w[rr][c].w * xv[c].w;
+                if (MODE == 2)
+                    a1 += w[ROWS + rr][c].x * xv[c].x + w[ROWS + rr][c].y * xv[c].y + w[ROWS + rr][c].z * xv[c].z +
+                          w[ROWS + rr][c].w * xv[c].w;
+            }
+            a0 = wsum(a0);
+            if (MODE == 2) a1 = wsum(a1);
+            const int r = r0 + rr;
+            if (lane == 0 && r < rows) {
+                float* out = y + (size_t)b * ldy + r;
+                if (MODE == 0) *out = a0;
+                else if (MODE == 1) *out += a0;
+                else *out = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
+            }
+        }
+    }
+}
+
+// rotate q and k at the device-side position, store k, v into the caches (rope + cache
+// write of llama2_cpu.cpp:288-296) and compact the rotated q into qc (B, dim);
+// qkv holds one row [q | k | v] of dim + 2*kvd floats per sequence
+__global__ void rope_store_kernel(const GenState* st, const float* qkv, float* qc, float* kc, float* vc, const float* fcos,
+                                  const float* fsin, int B, int dim, int kvd, int hs, int seqLen)
+{
+    const int pos = st->pos;
+    const int half = hs / 2;
+    const int ld = dim + 2 * kvd;
+    const int nq = dim / 2, nk = kvd / 2;
+    const int per = nq + nk + kvd;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < B * per; i += blockDim.x * gridDim.x) {
+        const int b = i / per, e = i % per;
+        const float* row = qkv + (size_t)b * ld;
+        const size_t coff = ((size_t)b * seqLen + pos) * kvd;
+        if (e < nq + nk) {
+            const bool isq = e < nq;
+            const int p = isq ? e : e - nq;
+            const float* v = (isq ? row : row + dim) + 2 * p;
+            const int j = p % half;
+            const float c = fcos[(size_t)pos * half + j], sn = fsin[(size_t)pos * half + j];
+            const float re = v[0], im = v[1];
+            const float r0 = re * c - im * sn, r1 = re * sn + im * c;
+            float* dst = isq ? qc + (size_t)b * dim + 2 * p : kc + coff + 2 * p;
+            dst[0] = r0;
+            dst[1] = r1;
+        } else {
+            const int d = e - nq - nk;
+            vc[coff + d] = row[dim + kvd + d];
+        }
+    }
+}
+
+// first-max argmax over the logits of each sequence (sample_argmax, llama2_sampler.cpp:25-36:
+// strict '>' so the lowest index wins ties), then record and feed back
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* logits, int V, const GenState* st, int* next, int* out_ids,
+                                                       int outStride)
+{
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const int b = blockIdx.x;
+    const float* lg = logits + (size_t)b * V;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        float v = lg[i];
+        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(bv, o, 64);
+        int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { sv[w] = bv; si[w] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < (int)(blockDim.x >> 6); i++)
+            if (sv[i] > bv || (sv[i] == bv && si[i] < bi)) { bv = sv[i]; bi = si[i]; }
+        if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0, as a scan that never finds a larger value would give
+        next[b] = bi;
+        out_ids[(size_t)b * outStride + st->pos] = bi;
+    }
+}
+
+__global__ void save_logits_kernel(const float* logits, float* all, const GenState* st, int V, int nSteps)
+{
+    const int b = blockIdx.y;
+    float* dst = all + ((size_t)b * nSteps + st->pos) * V;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < V; i += blockDim.x * gridDim.x) dst[i] = logits[(size_t)b * V + i];
+}
+
+// ---------------------------------------------------------------------------
+template <typename T> struct LayerW { T *wqkv, *wo, *w13, *w2; float *rms_att, *rms_ffn; };
+
+class Engine {
+public:
+    Config cfg{};
+    bool loaded = false;
+    bool bf16_weights = false;
+    bool use_graph = true;
+    int shared_classifier = 0;
+    int timedFrom = -1;          // first step of the timed span (-1: first step after the prompt)
+    float lastTimedMs = 0.f;     // HIP-event duration of the timed span of the last generate
+    int lastTimedSteps = 0;
+
+    ~Engine() { release(); }
+    long load(const char* path);
+    long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
+                  std::vector<float>* logits, std::atomic<bool>* cancel);
+    void release();
+
+private:
+    template <typename T> long upload(const float* blob);
+    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits);
+    long ensure_state(int B, int nSteps);
+
+    hipStream_t stream = nullptr;
+    std::vector<void*> allocs;
+    void* dalloc(size_t bytes)
+    {
+        void* p = nullptr;
+        if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) return nullptr;
+        allocs.push_back(p);
+        return p;
+    }
+    // weights
+    void* emb = nullptr; void* wcls = nullptr; float* rms_final = nullptr;
+    std::vector<LayerW<void>> layers;
+    float *fcos = nullptr, *fsin = nullptr;
+    // run state (sized for stateB sequences)
+    int stateB = 0, stateSteps = 0;
+    std::vector<void*> stateAllocs;
+    float *x = nullptr, *xb = nullptr, *qkv = nullptr, *qc = nullptr, *hb = nullptr, *logits = nullptr, *kc = nullptr, *vc = nullptr;
+    void* ws = nullptr; size_t wsBytes = 0;
+    GenState* dstate = nullptr;
+    int *dprompt = nullptr, *dnext = nullptr, *dcur = nullptr, *dout = nullptr;
+    hipGraphExec_t graphExec = nullptr;
+    int graphB = 0; bool graphLogits = false; float* graphAll = nullptr;
+};
+
+void Engine::release()
+{
+    if (stream) (void)hipStreamSynchronize(stream);
+    if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
+    for (void* p : stateAllocs) (void)hipFree(p);
+    stateAllocs.clear();
+    for (void* p : allocs) (void)hipFree(p);
+    allocs.clear();
+    layers.clear();
+    if (stream) { (void)hipStreamDestroy(stream); stream = nullptr; }
+    loaded = false;
+    stateB = 0;
+}
+
+// host fp32 -> device T
+template <typename T> static long put(void* dst, const float* src, size_t n, hipStream_t s, std::vector<bf16_t>& tmp);
+template <> long put<float>(void* dst, const float* src, size_t n, hipStream_t s, std::vector<bf16_t>&)
+{
+    HIPCHK(hipMemcpyAsync(dst, src, n * 4, hipMemcpyHostToDevice, s));
+    HIPCHK(hipStreamSynchronize(s));
+    return 0;
+}
+template <> long put<bf16_t>(void* dst, const float* src, size_t n, hipStream_t s, std::vector<bf16_t>& tmp)
+{
+    tmp.resize(n);
+    for (size_t i = 0; i < n; i++) tmp[i] = f32_to_bf16(src[i]);
+    HIPCHK(hipMemcpyAsync(dst, tmp.data(), n * 2, hipMemcpyHostToDevice, s));
+    HIPCHK(hipStreamSynchronize(s));
+    return 0;
+}
+
+template <typename T> long Engine::upload(const float* p)
+{
+    // file order (llama2_cpu.cpp:74-106): rms_att, rms_ffn, rms_final, tok_emb, wq, wk, wv, wo, w1, w2, w3[, wcls]
+    const size_t L = cfg.n_layers, dim = cfg.dim, hid = cfg.hidden_dim;
+    const size_t hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
+    const float* rms_att = p;   p += L * dim;
+    const float* rms_ffn = p;   p += L * dim;
+    const float* rmsf = p;      p += dim;
+    const float* tok = p;       p += V * dim;
+    const float* wq = p;        p += L * dim * dim;
+    const float* wk = p;        p += L * dim * kvd;
+    const float* wv = p;        p += L * dim * kvd;
+    const float* wo = p;        p += L * dim * dim;
+    const float* w1 = p;        p += L * dim * hid;
+    const float* w2 = p;        p += L * hid * dim;
+    const float* w3 = p;        p += L * dim * hid;
+    const float* wc = shared_classifier ? tok : p;
+    std::vector<bf16_t> tmp;
+    const size_t es = sizeof(T);
+    long e;
+    if (!(emb = dalloc(V * dim * es))) return MCH_ERROR_MEMORY_OUT;
+    if ((e = put<T>(emb, tok, V * dim, stream, tmp))) return e;
+    if (shared_classifier) wcls = emb;
+    else {
+        if (!(wcls = dalloc(V * dim * es))) return MCH_ERROR_MEMORY_OUT;
+        if ((e = put<T>(wcls, wc, V * dim, stream, tmp))) return e;
+    }
+    if (!(rms_final = (float*)dalloc(dim * 4))) return MCH_ERROR_MEMORY_OUT;
+    HIPCHK(hipMemcpy(rms_final, rmsf, dim * 4, hipMemcpyHostToDevice));
+    layers.resize(L);
+    for (size_t l = 0; l < L; l++) {
+        LayerW<void>& w = layers[l];
+        const size_t qkvRows = dim + 2 * kvd;
+        if (!(w.wqkv = dalloc(qkvRows * dim * es)) || !(w.wo = dalloc(dim * dim * es)) || !(w.w13 = dalloc(2 * hid * dim * es)) ||
+            !(w.w2 = dalloc(dim * hid * es)) || !(w.rms_att = (float*)dalloc(dim * 4)) || !(w.rms_ffn = (float*)dalloc(dim * 4)))
+            return MCH_ERROR_MEMORY_OUT;
+        char* q = (char*)w.wqkv;
+        if ((e = put<T>(q, wq + l * dim * dim, dim * dim, stream, tmp))) return e;
+        if ((e = put<T>(q + dim * dim * es, wk + l * dim * kvd, kvd * dim, stream, tmp))) return e;
+        if ((e = put<T>(q + (dim + kvd) * dim * es, wv + l * dim * kvd, kvd * dim, stream, tmp))) return e;
+        if ((e = put<T>(w.wo, wo + l * dim * dim, dim * dim, stream, tmp))) return e;
+        if ((e = put<T>(w.w13, w1 + l * dim * hid, hid * dim, stream, tmp))) return e;
+        if ((e = put<T>((char*)w.w13 + hid * dim * es, w3 + l * dim * hid, hid * dim, stream, tmp))) return e;
+        if ((e = put<T>(w.w2, w2 + l * hid * dim, dim * hid, stream, tmp))) return e;
+        HIPCHK(hipMemcpy(w.rms_att, rms_att + l * dim, dim * 4, hipMemcpyHostToDevice));
+        HIPCHK(hipMemcpy(w.rms_ffn, rms_ffn + l * dim, dim * 4, hipMemcpyHostToDevice));
+    }
+    return 0;
+}
+
+long Engine::load(const char* path)
+{
+    release();
+    FILE* f = fopen(path, "rb");
+    if (!f) return MCH_ERROR_LLM_MISSING_MODEL_FILE;
+    // header (llama2_cpu.cpp:108-147): magic "ak42", version 1, Config, shared-classifier byte, 256 bytes in all
+    uint32_t magic = 0;
+    int version = 0;
+    uint8_t shared = 0;
+    bool ok = fread(&magic, 4, 1, f) == 1 && magic == 0x616b3432 && fread(&version, 4, 1, f) == 1 && version == 1 &&
+              fread(&cfg, sizeof(Config), 1, f) == 1 && fread(&shared, 1, 1, f) == 1;
+    if (!ok) { fclose(f); return MCH_ERROR_LLM_LOAD_MODEL; }
+    shared_classifier = shared;
+    if (cfg.seq_len > 20480) cfg.seq_len = 20480;
+    if (cfg.dim <= 0 || cfg.n_heads <= 0 || cfg.n_kv_heads <= 0 || cfg.n_layers <= 0 || cfg.vocab_size <= 0 || cfg.seq_len <= 0 ||
+        cfg.hidden_dim <= 0 || cfg.dim % cfg.n_heads || cfg.n_heads % cfg.n_kv_heads || (cfg.dim / cfg.n_heads) % 2 ||
+        cfg.dim % 4 || cfg.hidden_dim % 4 || cfg.dim > 64 * 4 * 16 || cfg.hidden_dim > 64 * 4 * 16) {
+        fclose(f);
+        return MCH_ERROR_LLM_LOAD_MODEL;
+    }
+    const size_t L = cfg.n_layers, dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
+    size_t need = 2 * L * dim + dim + (size_t)cfg.vocab_size * dim + 2 * L * dim * dim + 2 * L * dim * kvd + 3 * L * dim * hid;
+    if (!shared) need += (size_t)cfg.vocab_size * dim;
+    fseek(f, 0, SEEK_END);
+    long fsize = ftell(f);
+    if (fsize < 0 || (size_t)fsize < 256 + need * 4) { fclose(f); return MCH_ERROR_LLM_LOAD_MODEL; }
+    fseek(f, 256, SEEK_SET);
+    std::vector<float> blob(need);
+    size_t got = fread(blob.data(), 4, need, f);
+    fclose(f);
+    if (got != need) return MCH_ERROR_LLM_LOAD_MODEL;
+
+    HIPCHK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    long e = bf16_weights ? upload<bf16_t>(blob.data()) : upload<float>(blob.data());
+    if (e) { release(); return e; }
+    // rotary tables as precompute_freqs_cis builds them (llama2_cpu.cpp:388-414)
+    const int half = (int)hs / 2;
+    std::vector<float> fr(half), hc((size_t)cfg.seq_len * half), hsn((size_t)cfg.seq_len * half);
+    for (int i = 0; i < (int)hs; i += 2) {
+        float v = i / (float)hs;
+        float d = powf(10000.0f, v);
+        fr[i / 2] = (d == 0.0) ? 0 : 1.0f / d;
+    }
+    for (size_t i = 0; i < (size_t)cfg.seq_len; i++)
+        for (int j = 0; j < half; j++) {
+            hc[i * half + j] = cosf(i * fr[j]);
+            hsn[i * half + j] = sinf(i * fr[j]);
+        }
+    if (!(fcos = (float*)dalloc(hc.size() * 4)) || !(fsin = (float*)dalloc(hc.size() * 4))) { release(); return MCH_ERROR_MEMORY_OUT; }
+    HIPCHK(hipMemcpy(fcos, hc.data(), hc.size() * 4, hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(fsin, hsn.data(), hc.size() * 4, hipMemcpyHostToDevice));
+    loaded = true;
+    return 0;
+}
+
+long Engine::ensure_state(int B, int nSteps)
+{
+    if (B == stateB && nSteps <= stateSteps) return 0;
+    HIPCHK(hipStreamSynchronize(stream));
+    if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
+    for (void* p : stateAllocs) (void)hipFree(p);
+    stateAllocs.clear();
+    stateB = 0;
+    const size_t dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
+    auto sa = [&](size_t bytes) -> void* {
+        void* p = nullptr;
+        if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) return nullptr;
+        stateAllocs.push_back(p);
+        return p;
+    };
+    const size_t cacheN = (size_t)cfg.n_layers * B * cfg.seq_len * kvd;
+    wsBytes = attn_decode_workspace_bytes(B, cfg.n_heads, (int)hs, cfg.seq_len);
+    x = (float*)sa(B * dim * 4);
+    xb = (float*)sa(B * dim * 4);
+    qkv = (float*)sa(B * (dim + 2 * kvd) * 4);
+    qc = (float*)sa(B * dim * 4);
+    hb = (float*)sa(B * hid * 4);
+    logits = (float*)sa((size_t)B * cfg.vocab_size * 4);
+    kc = (float*)sa(cacheN * 4);
+    vc = (float*)sa(cacheN * 4);
+    ws = sa(wsBytes);
+    dstate = (GenState*)sa(sizeof(GenState));
+    dprompt = (int*)sa((size_t)B * cfg.seq_len * 4);
+    dnext = (int*)sa(B * 4);
+    dcur = (int*)sa(B * 4);
+    dout = (int*)sa((size_t)B * cfg.seq_len * 4);
+    if (!x || !xb || !qkv || !qc || !hb || !logits || !kc || !vc || !ws || !dstate || !dprompt || !dnext || !dcur || !dout)
+        return MCH_ERROR_MEMORY_OUT;
+    stateB = B;
+    stateSteps = cfg.seq_len;
+    return 0;
+}
+
+template <int MODE, bool NORM, typename T>
+static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int B,
+                                int ldy)
+{
+    const int waves = (rows + 1) / 2;
+    const int grid = (waves + 3) / 4;
+    const int ch = (n / 4 + 63) / 64;
+#define MV(C) hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy)
+    if (ch <= 2) MV(2);
+    else if (ch <= 3) MV(3);
+    else if (ch <= 4) MV(4);
+    else if (ch <= 8) MV(8);
+    else if (ch <= 16) MV(16);
+    else return hipErrorInvalidValue;
+#undef MV
+    return hipGetLastError();
+}
+
+// enqueue one decode step for B sequences at the device-side position
+template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits)
+{
+    const int dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
+    const int ldq = dim + 2 * kvd;
+    hipLaunchKernelGGL(embed_step_kernel<T>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const T*)emb, x, dim, dcur);
+    HIPCHK(hipGetLastError());
+    const float scale = 1.0f / sqrtf((float)hs);
+    for (int l = 0; l < cfg.n_layers; l++) {
+        const LayerW<void>& w = layers[l];
+        float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
+        float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
+        // qkv = [Wq;Wk;Wv] rmsnorm(x)
+        HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq)));
+        {
+            const int n = B * (dim / 2 + kvd / 2 + kvd);
+            hipLaunchKernelGGL(rope_store_kernel, (n + 255) / 256, 256, 0, s, dstate, qkv, qc, kcl, vcl, fcos, fsin, B, dim, kvd, hs,
+                               cfg.seq_len);
+            HIPCHK(hipGetLastError());
+        }
+        // xb = attention(q, cache[0..pos])
+        HIPCHK(k_attn_decode(s, F32, qc, kcl, vcl, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len,
+                             (long long)cfg.seq_len * kvd, hs, kvd, scale, ws, wsBytes, &dstate->len));
+        // x += Wo xb
+        HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim)));
+        // hb = silu(W1 rmsnorm(x)) * (W3 rmsnorm(x))
+        HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid)));
+        // x += W2 hb
+        HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim)));
+    }
+    // logits = Wcls rmsnorm(x)
+    HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V)));
+    if (allLogits) {
+        hipLaunchKernelGGL(save_logits_kernel, dim3((V + 255) / 256 > 64 ? 64 : (V + 255) / 256, B), 256, 0, s, logits, allLogits,
+                           dstate, V, nSteps);
+        HIPCHK(hipGetLastError());
+    }
+    hipLaunchKernelGGL(argmax_kernel, B, 1024, 0, s, logits, V, dstate, dnext, dout, cfg.seq_len);
+    HIPCHK(hipGetLastError());
+    hipLaunchKernelGGL(advance_kernel, 1, 1, 0, s, dstate);
+    HIPCHK(hipGetLastError());
+    return 0;
+}
+
+long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
+                      std::vector<float>* outLogits, std::atomic<bool>* cancel)
+{
+    if (!loaded) return MCH_ERROR_LLM_GENERATE;
+    if (B < 1 || B > 64 || nSteps < 1 || nSteps > cfg.seq_len || nPrompt < 1 || nPrompt > cfg.seq_len) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    for (int i = 0; i < B * nPrompt; i++)
+        if (prompts[i] < 0 || prompts[i] >= cfg.vocab_size) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long e = ensure_state(B, nSteps);
+    if (e) return e;
+    hipStream_t s = stream;
+    std::vector<int> hp((size_t)B * cfg.seq_len, 0);
+    for (int b = 0; b < B; b++) memcpy(&hp[(size_t)b * cfg.seq_len], prompts + (size_t)b * nPrompt, nPrompt * sizeof(int));
+    HIPCHK(hipMemcpyAsync(dprompt, hp.data(), hp.size() * 4, hipMemcpyHostToDevice, s));
+    GenState st0 = {0, nPrompt, 1, 0};
+    HIPCHK(hipMemcpyAsync(dstate, &st0, sizeof(st0), hipMemcpyHostToDevice, s));
+    HIPCHK(hipStreamSynchronize(s));
+    float* allLogits = nullptr;
+    if (wantLogits) {
+        HIPCHK(hipMalloc((void**)&allLogits, (size_t)B * nSteps * cfg.vocab_size * 4));
+    }
+    auto enqueue = [&]() -> long {
+        return bf16_weights ? step<bf16_t>(s, B, nSteps, allLogits) : step<float>(s, B, nSteps, allLogits);
+    };
+    hipEvent_t evA = nullptr, evB = nullptr;
+    (void)hipEventCreate(&evA);
+    (void)hipEventCreate(&evB);
+    const int t0 = timedFrom < 0 ? nPrompt : timedFrom;
+    bool graph = use_graph && !wantLogits;
+    if (graph && (!graphExec || graphB != B)) {
+        // one decode step, captured once; position / tokens are device-side so the graph is replayed as is
+        if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
+        hipGraph_t g = nullptr;
+        hipError_t he = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+        if (he == hipSuccess) {
+            e = enqueue();
+            he = hipStreamEndCapture(s, &g);
+            if (e == 0 && he == hipSuccess) he = hipGraphInstantiate(&graphExec, g, nullptr, nullptr, 0);
+            if (g) (void)hipGraphDestroy(g);
+        }
+        if (e || he != hipSuccess || !graphExec) { graphExec = nullptr; graph = false; e = 0; }
+        graphB = B;
+    }
+    int done = 0;
+    for (int i = 0; i < nSteps && !e; i++) {
+        if (i == t0) (void)hipEventRecord(evA, s);
+        if (graph) {
+            hipError_t he = hipGraphLaunch(graphExec, s);
+            if (he != hipSuccess) e = (long)he;
+        } else e = enqueue();
+        done++;
+        if (cancel && (i & 15) == 15 && cancel->load()) break;
+    }
+    (void)hipEventRecord(evB, s);
+    hipError_t he = hipStreamSynchronize(s);
+    if (!e && he != hipSuccess) e = (long)he;
+    lastTimedMs = 0.f;
+    lastTimedSteps = 0;
+    if (!e && done > t0 && t0 >= 0) {
+        (void)hipEventElapsedTime(&lastTimedMs, evA, evB);
+        lastTimedSteps = done - t0;
+    }
+    (void)hipEventDestroy(evA);
+    (void)hipEventDestroy(evB);
+    if (!e) {
+        ids->assign((size_t)B * nSteps, 0);
+        std::vector<int> tmp((size_t)B * cfg.seq_len);
+        he = hipMemcpy(tmp.data(), dout, tmp.size() * 4, hipMemcpyDeviceToHost);
+        if (he != hipSuccess) e = (long)he;
+        for (int b = 0; b < B && !e; b++) memcpy(&(*ids)[(size_t)b * nSteps], &tmp[(size_t)b * cfg.seq_len], done * sizeof(int));
+        if (!e && wantLogits && outLogits) {
+            outLogits->resize((size_t)B * nSteps * cfg.vocab_size);
+            he = hipMemcpy(outLogits->data(), allLogits, outLogits->size() * 4, hipMemcpyDeviceToHost);
+            if (he != hipSuccess) e = (long)he;
+        }
+    }
+    if (allLogits) (void)hipFree(allLogits);
+    return e;
+}
+
+// ---------------------------------------------------------------------------
+// one LLM object per CREATE (CudaExtension.llm32.cpp:100-130, llm.cpp:20-60)
+struct Llm {
+    float temperature = 1.0f, topp = 0.9f;
+    long seed = 0;
+    Engine engine;
+    std::atomic<bool> cancel{false};
+    std::atomic<bool> busy{false};
+    std::atomic<bool> loaded{false};
+    std::atomic<bool> end{false};
+    std::string response;
+    std::mutex responseLock;
+    std::mutex runLock;
+};
+
+typedef MCH_LONG (*FnInvoke)(MCH_LONG, MCH_LONG, float*, MCH_LONG, float**, MCH_LONG*, MCH_TCHAR*, MCH_LONG);
+typedef MCH_LONG (*FnAllocHost)(MCH_LONG, MCH_LONG, float**, float*, bool);
+
+static FnInvoke g_parentInvoke = nullptr;
+static FnAllocHost g_parentAllocHost = nullptr;
+static MCH_LONG g_kernelIdx = 0;
+static std::map<long, Llm*> g_llms;
+static std::mutex g_mapLock;
+
+static Llm* find_llm(long h)
+{
+    std::lock_guard<std::mutex> g(g_mapLock);
+    auto it = g_llms.find(h);
+    return it == g_llms.end() ? nullptr : it->second;
+}
+
+static void put_text(MCH_TCHAR* out, long max, const char* s)
+{
+    if (!out || max <= 0) return;
+    long i = 0;
+    for (; s[i] && i < max - 1; i++) out[i] = (MCH_TCHAR)(unsigned char)s[i];
+    out[i] = 0;
+}
+
+static std::string narrow(const MCH_TCHAR* s)
+{
+    std::string o;
+    if (s) for (; *s; s++) o += (char)(*s < 0x80 ? *s : '?');
+    return o;
+}
+
+static long give(const std::vector<float>& v, float** ppOut, MCH_LONG* plOut)
+{
+    // results are handed over in memory owned by the parent (CudaExtension.llm32.cpp:123)
+    long e = g_parentAllocHost(g_kernelIdx, (MCH_LONG)v.size(), ppOut, const_cast<float*>(v.data()), false);
+    if (e) return e;
+    *plOut = (MCH_LONG)v.size();
+    return 0;
+}
+
+}  // namespace mch
+
+using namespace mch;
+
+extern "C" {
+
+MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx)
+{
+    if (!hParent) return MCH_ERROR_PARAM_NULL;
+    g_parentInvoke = (FnInvoke)dlsym(hParent, "DLL_InvokeFloat");
+    g_parentAllocHost = (FnAllocHost)dlsym(hParent, "Internal_AllocHostFloat");
+    if (!g_parentInvoke || !g_parentAllocHost) return MCH_ERROR_PARAM;
+    g_kernelIdx = lKernelIdx;
+    return 0;
+}
+
+MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, float** ppOut, MCH_LONG* plOut, MCH_TCHAR* szErr,
+                                        MCH_LONG errMax)
+{
+    if (!g_parentInvoke) return MCH_ERROR_EXTENSION_NOT_INITIALIZED;
+    switch (fn) {
+    case MCH_LLM_CREATE: {
+        Llm* m = new Llm();
+        if (lIn > 0) m->temperature = pIn[0];
+        if (lIn > 1) m->topp = pIn[1];
+        if (lIn > 2) m->seed = (long)pIn[2];
+        long h;
+        {
+            std::lock_guard<std::mutex> g(g_mapLock);
+            h = g_llms.empty() ? 1 : g_llms.rbegin()->first + 1;
+            g_llms[h] = m;
+        }
+        long e = give({(float)h}, ppOut, plOut);
+        if (e) {
+            std::lock_guard<std::mutex> g(g_mapLock);
+            g_llms.erase(h);
+            delete m;
+        }
+        return (MCH_LONG)e;
+    }
+    case MCH_LLM_DESTROY: {
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = nullptr;
+        {
+            std::lock_guard<std::mutex> g(g_mapLock);
+            auto it = g_llms.find((long)pIn[0]);
+            if (it != g_llms.end()) { m = it->second; g_llms.erase(it); }
+        }
+        if (m) {
+            m->cancel.store(true);
+            std::lock_guard<std::mutex> run(m->runLock);  // wait for a running generate to notice the flag
+            delete m;
+        }
+        return 0;
+    }
+    case MCH_LLM_ABORT: {
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (m) m->cancel.store(true);
+        return 0;
+    }
+    case MCH_LLM_QUERYSTATUS: {
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        float v = m->loaded.load() ? 1.f : 0.f;
+        return (MCH_LONG)give({v, v}, ppOut, plOut);
+    }
+    case MCH_LLM_SET_OPTION: {
+        if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        std::lock_guard<std::mutex> run(m->runLock);
+        int opt = (int)pIn[1];
+        if (opt == 1) m->engine.bf16_weights = pIn[2] != 0.f;
+        else if (opt == 2) m->engine.timedFrom = (int)pIn[2];
+        else if (opt == 3) m->engine.use_graph = pIn[2] != 0.f;
+        else return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        return 0;
+    }
+    case MCH_LLM_QUERY_TIMING: {
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps}, ppOut, plOut);
+    }
+    case MCH_LLM_GENERATE_IDS:
+    case MCH_LLM_GENERATE_BATCH: {
+        // GENERATE_IDS   f{hLlm, nSteps, wantLogits, ids...}
+        // GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of sequence 0 .., sequence 1 ..}
+        const bool batch = fn == MCH_LLM_GENERATE_BATCH;
+        const int head = batch ? 4 : 3;
+        if (lIn < head + 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        std::lock_guard<std::mutex> run(m->runLock);
+        const int nSteps = (int)pIn[1];
+        const int B = batch ? (int)pIn[2] : 1;
+        const int nPrompt = batch ? (int)pIn[3] : lIn - head;
+        const bool wantLogits = !batch && pIn[2] != 0.f;
+        if (B < 1 || nPrompt < 1 || (long long)B * nPrompt != lIn - head) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        std::vector<int> prompts((size_t)B * nPrompt);
+        for (size_t i = 0; i < prompts.size(); i++) prompts[i] = (int)pIn[head + i];
+        std::vector<int> ids;
+        std::vector<float> logits;
+        m->cancel.store(false);
+        m->busy.store(true);
+        long e = m->engine.generate(prompts.data(), B, nPrompt, nSteps, wantLogits, &ids, &logits, &m->cancel);
+        m->busy.store(false);
+        if (e) {
+            if (e == MCH_ERROR_LLM_GENERATE) put_text(szErr, errMax, "The model is not loaded.");
+            return (MCH_LONG)e;
+        }
+        std::vector<float> out(ids.size() + logits.size());
+        for (size_t i = 0; i < ids.size(); i++) out[i] = (float)ids[i];
+        if (!logits.empty()) memcpy(out.data() + ids.size(), logits.data(), logits.size() * 4);
+        return (MCH_LONG)give(out, ppOut, plOut);
+    }
+    default:
+        put_text(szErr, errMax, "The function specified is not supported.");
+        return MCH_ERROR_NOT_IMPLEMENTED;
+    }
+}
+
+MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn, float** ppOut, MCH_LONG* plOut, MCH_TCHAR* szIn,
+                                          MCH_TCHAR* szOut, MCH_LONG outMax, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    if (!g_parentInvoke) return MCH_ERROR_EXTENSION_NOT_INITIALIZED;
+    switch (fn) {
+    case MCH_LLM_LOAD: {
+        // "model.bin;tokenizer.bin" (llm.cpp:78-98).  An empty tokenizer part selects the token-id front door.
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return 0;
+        std::string in = narrow(szIn), model = in, tok;
+        size_t p = in.find(';');
+        if (p != std::string::npos) { model = in.substr(0, p); tok = in.substr(p + 1); }
+        FILE* f = fopen(model.c_str(), "rb");
+        if (!f) return MCH_ERROR_LLM_MISSING_MODEL_FILE;
+        fclose(f);
+        if (!tok.empty()) {
+            f = fopen(tok.c_str(), "rb");
+            if (!f) return MCH_ERROR_LLM_MISSING_TOKENIZER_FILE;
+            fclose(f);
+        }
+        std::lock_guard<std::mutex> run(m->runLock);
+        m->busy.store(true);
+        long e = m->engine.load(model.c_str());
+        m->busy.store(false);
+        m->loaded.store(e == 0);
+        return (MCH_LONG)e;
+    }
+    case MCH_LLM_GENERATE:
+        // text prompts need the BPE tokenizer of the reference (llama2_tokenizer.cpp), which is not
+        // part of the attention path; token ids go through MCH_LLM_GENERATE_IDS
+        put_text(szErr, errMax, "Text generation needs the tokenizer, which this build does not include; use the token-id entry.");
+        return MCH_ERROR_NOT_IMPLEMENTED;
+    case MCH_LLM_QUERYRESPONSE: {
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        long end = 1;
+        if (m) {
+            std::lock_guard<std::mutex> g(m->responseLock);
+            put_text(szOut, outMax, m->response.c_str());
+            m->response.clear();
+            end = m->end.load() ? 1 : 0;
+            m->end.store(false);
+        }
+        if (ppOut) *ppOut = (float*)end;  // the end flag travels through the pointer (CudaExtension.llm32.cpp:257-258)
+        return 0;
+    }
+    default:
+        put_text(szErr, errMax, "The function specified is not supported.");
+        return MCH_ERROR_NOT_IMPLEMENTED;
+    }
+}
+
+}  // extern "C"
