@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one greedy decode step (one new token) of the Llama-2 110M-shape
+decoder (dim 768, 12 layers, 12 heads x 64, FFN 2048 SwiGLU, vocab 32000, seq 1024;
+random-init N(0, 0.02) fp32 weights, 128 seeded prompt ids), run by the llama2
+extension library through the C ABI.  After the prompt and W untimed decode steps,
+exactly K decode steps are timed with HIP events on the engine's stream.
+
+The single JSON line also carries:
+  roofline      the dominant kernel of that workload (the fused mat-vec family that
+                streams the weights), timed live with HIP event pairs around every
+                launch of eager decode steps;
+  cpu_baseline  the CPU checker (restatement of the reference's llama2 C++ forward)
+                timed on this host's cores on a bounded sample of the same workload;
+  also          the other named kernels at their benchmark shapes, each with its own
+                roofline entry: fused prefill attention (B=8, T=1024, 12 x 64), decode
+                attention over a KV cache (32 x 128, L up to 4096, batch up to 32), the
+                QKV / projection GEMMs, batch-16 and bf16-weight decode.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+
+C4 = dict(dim=768, hidden_dim=2048, n_layers=12, n_heads=12, n_kv_heads=12, vocab_size=32000, seq_len=1024)
+N_PROMPT = 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_checkpoint(cfg, seed, path):
+    from oracle import llama2 as O   # checkpoint writer + the CPU baseline live with the checker
+    blob, _ = O.random_weights(cfg, seed=seed, shared_classifier=False, std=0.02)
+    if not os.path.exists(path):
+        O.write_checkpoint_v1(path, cfg, blob, False)
+    return blob
+
+
+def weight_bytes(cfg, es):
+    L, dim, hid, V = cfg["n_layers"], cfg["dim"], cfg["hidden_dim"], cfg["vocab_size"]
+    kvd = dim // cfg["n_heads"] * cfg["n_kv_heads"]
+    return (L * ((dim + 2 * kvd) * dim + dim * dim + 3 * hid * dim) + V * dim) * es
+
+
+def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
+    from mycaffe_amd.llm_inference import LlmInference
+    inf = LlmInference(cuda)
+    inf.Initialize(fTemperature=0.0)
+    inf.SetOption(1, 1 if bf16 else 0)
+    inf.SetOption(3, 1 if graph else 0)
+    inf.Load(path)
+    rng = np.random.default_rng(seed)
+    total = N_PROMPT + warmup + steps
+    inf.SetOption(2, N_PROMPT + warmup)
+    t0 = time.perf_counter()
+    if batch == 1:
+        prompt = rng.integers(3, C4["vocab_size"], N_PROMPT)
+        ids = inf.GenerateIds(prompt, total)
+    else:
+        prompt = rng.integers(3, C4["vocab_size"], (batch, N_PROMPT))
+        ids = inf.GenerateBatch(prompt, total)
+    wall = time.perf_counter() - t0
+    ms, nsteps = inf.QueryTiming()
+    assert nsteps == steps, (nsteps, steps)
+    res = {"ms_per_step": ms / steps, "tokens_per_s": batch * steps / (ms / 1e3), "wall_s_whole_generation": wall,
+           "prompt": prompt, "ids": ids}
+    return inf, res
+
+
+def matvec_roofline(inf, pos, bf16):
+    prof = inf.ProfileStep(pos, 8)
+    mv = [k for k in prof if k.startswith("matvec")]
+    ms = sum(prof[k][0] for k in mv)
+    launches = sum(prof[k][1] for k in mv)
+    nbytes = sum(prof[k][2] for k in mv)
+    achieved = nbytes / (ms / 1e3) / 1e9
+    detail = {k: {"ms_per_step": round(v[0], 5), "launches": v[1], "GBps": round(v[2] / (v[0] / 1e3) / 1e9, 1) if v[0] > 0 and v[2] > 0 else None}
+              for k, v in prof.items()}
+    return {"kernel": "matvec_kernel (fused RMSNorm / SwiGLU / residual mat-vec, all instantiations of one step)",
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "algorithmic_bytes_per_launch": round(nbytes / launches), "avg_launch_us": round(ms / launches * 1e3, 3),
+            "launches_per_step": launches, "per_class": detail}
+
+
+def cpu_baseline(blob, budget_s=20.0):
+    """The CPU checker on this host: same model, same prompt convention, bounded sample."""
+    from oracle import llama2 as O
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    m = O.Llama(C4, blob, False)
+    prompt = np.random.default_rng(1).integers(3, C4["vocab_size"], N_PROMPT)
+    t0 = time.perf_counter()
+    m.generate_greedy(prompt[:4], 4)
+    per = (time.perf_counter() - t0) / 4
+    n = int(max(8, min(N_PROMPT, budget_s / max(per, 1e-6))))
+    m2 = O.Llama(C4, blob, False)
+    t0 = time.perf_counter()
+    m2.generate_greedy(prompt, n)
+    dt = time.perf_counter() - t0
+    return {"value": round(n / dt, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": "first %d positions of the same 128-id prompt, fp32, batch 1 (%.1f s of CPU work); the GPU "
+                      "figure times positions %d.. where attention reads a longer cache" % (n, dt, N_PROMPT)}
+
+
+def bench_prefill_attention(cuda, reps):
+    """Fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_FWD (id 163)."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    B, H, T, hs = 8, 12, 1024, 64
+    rng = np.random.default_rng(0)
+    out = {}
+    mask = cuda.AllocMemory(np.tril(np.ones((T, T), np.float32)))
+    hc, ha = cuda.CreateCuDNN(), cuda.CreateAttn()
+    cuda.SetAttn(hc, ha, 0, False, B, T, H, hs, 0.0)
+    for name, half in (("bf16", True), ("f32", False)):
+        hs_ = [cuda.AllocMemory(rng.standard_normal(B * H * T * hs).astype(np.float32), bHalfSize=half) for _ in range(3)]
+        hy = cuda.AllocMemory(B * H * T * hs, bHalfSize=half)
+        rgl = [hc, ha, T, hs_[0], hs_[1], hs_[2], mask, hy, 0]
+        cuda.AttnScaledDotProductForward(hc, ha, T, hs_[0], hs_[1], hs_[2], mask, hy, False)
+        ms = cuda.TimeFunction(CUDAFN.CUDA_ATTN_FWD, None, rgl, 5, reps)
+        useful = 2.0 * B * H * T * T * hs          # causal half of the 4*B*H*T*T*hs full-square flops
+        tf = useful / (ms / 1e3) / 1e12
+        out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2), "TFLOPs_full_square": round(2 * tf, 2),
+                     "roofline": {"kernel": "fused causal attention forward", "bound": "mfma", "achieved": round(tf, 2),
+                                  "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s",
+                                  "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4), "traffic": None}}
+        for h in hs_ + [hy]:
+            cuda.FreeMemory(h)
+    cuda.FreeMemory(mask)
+    return out
+
+
+def bench_decode_attention(cuda, reps):
+    """KV-cache attention, 32 heads x 128, one query token per sequence (id 2001)."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    H, hs = 32, 128
+    out = {}
+    rng = np.random.default_rng(0)
+    for name, half, es in (("bf16", True, 2), ("f32", False, 4)):
+        for B in (1, 8, 32):
+            for L in (512, 2048, 4096):
+                n = B * H * L * hs
+                kc = cuda.AllocMemory(n, bHalfSize=half)
+                vc = cuda.AllocMemory(n, bHalfSize=half)
+                # fill on the device: a seeded block repeated (values only matter for parity tests)
+                blk = rng.standard_normal(min(n, 1 << 20)).astype(np.float32)
+                src = cuda.AllocMemory(blk, bHalfSize=half)
+                for off in range(0, n, blk.size):
+                    c = min(blk.size, n - off)
+                    cuda.copy(c, src, kc, 0, off)
+                    cuda.copy(c, src, vc, 0, off)
+                q = cuda.AllocMemory(rng.standard_normal(B * H * hs).astype(np.float32), bHalfSize=half)
+                y = cuda.AllocMemory(B * H * hs, bHalfSize=half)
+                rgl = [B, H, H, hs, L, q, kc, vc, y, H * L * hs, L * hs, hs]
+                ms = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl, 5, reps)
+                nbytes = 2.0 * n * es
+                gbs = nbytes / (ms / 1e3) / 1e9
+                out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+                for h in (kc, vc, src, q, y):
+                    cuda.FreeMemory(h)
+    best = out["bf16_B32_L4096"]
+    out["roofline"] = {"kernel": "attn_decode_kernel (bf16, batch 32, L 4096, 32 x 128)", "bound": "hbm", "achieved": best["GBps"],
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_hbm"], "traffic": None}
+    return out
+
+
+def bench_gemm(cuda, reps):
+    """QKV (8192 x 2304 x 768) and output projection (8192 x 768 x 768) GEMMs, weights [N, K]."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    out = {}
+    rng = np.random.default_rng(0)
+    for name, half in (("bf16", True), ("f32", False)):
+        for tag, (M, N, K) in (("qkv", (8192, 2304, 768)), ("proj", (8192, 768, 768))):
+            a = cuda.AllocMemory(rng.standard_normal(M * K).astype(np.float32), bHalfSize=half)
+            w = cuda.AllocMemory((rng.standard_normal(N * K) * 0.02).astype(np.float32), bHalfSize=half)
+            c = cuda.AllocMemory(M * N, bHalfSize=half)
+            rgl = [0, 1, M, N, K, 0, a, w, 0, c]
+            ms = cuda.TimeFunction(CUDAFN.CUDA_GEMM, [1.0, 0.0], rgl, 3, reps)
+            tf = 2.0 * M * N * K / (ms / 1e3) / 1e12
+            out["%s_%s" % (name, tag)] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS[name], 4)}
+            for h in (a, w, c):
+                cuda.FreeMemory(h)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-graph", action="store_true", help="launch every decode kernel eagerly instead of replaying a HIP graph "
+                    "(kernel tracing tools see the individual kernels this way)")
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,gemm")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: every box of this build has one MI355X and the path has no multi-GPU part; "
+            "run with --gpus 1")
+        sys.exit(2)
+    if N_PROMPT + args.warmup + args.steps > C4["seq_len"]:
+        log("prompt (128) + warmup + steps must fit the 1024-token context")
+        sys.exit(2)
+
+    from mycaffe_amd.cudadnn import CudaDnn
+    cuda = CudaDnn(0)
+    dev_name = cuda.GetDeviceName(0)
+    log("device:", dev_name)
+    path = os.path.join(os.environ.get("TMPDIR", "/tmp"), "mycaffe_amd_llama110m_seed1234.bin")
+    t0 = time.perf_counter()
+    blob = make_checkpoint(C4, 1234, path)
+    log("checkpoint ready in %.1f s" % (time.perf_counter() - t0))
+
+    inf, head = run_decode(cuda, path, False, 1, args.steps, args.warmup, graph=not args.no_graph)
+    log("fp32 batch 1: %.1f tokens/s (%.4f ms/step)" % (head["tokens_per_s"], head["ms_per_step"]))
+    roof = matvec_roofline(inf, N_PROMPT + args.warmup, False)
+    step_bytes = weight_bytes(C4, 4)
+    inf.CleanUp()
+
+    also = {}
+    only = set(x for x in args.only.split(",") if x)
+    want = lambda name: not args.no_also and (not only or name in only)
+    also["decode_whole_step_GBps_fp32_b1"] = round(step_bytes / (head["ms_per_step"] / 1e3) / 1e9, 1)
+    if want("decode"):
+        for tag, bf16, batch in (("bf16_weights_b1", True, 1), ("fp32_b16", False, 16), ("bf16_weights_b16", True, 16)):
+            i2, r = run_decode(cuda, path, bf16, batch, args.steps, args.warmup, graph=not args.no_graph)
+            also["decode_" + tag] = {"tokens_per_s": round(r["tokens_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4)}
+            log("decode %s: %.1f tokens/s" % (tag, r["tokens_per_s"]))
+            i2.CleanUp()
+    if want("prefill"):
+        also["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 50)
+        log("prefill attention:", json.dumps(also["prefill_attention_B8_T1024_H12x64"]))
+    if want("decode_attn"):
+        also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
+        log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
+    if want("gemm"):
+        also["gemm_inner_product"] = bench_gemm(cuda, 10)
+        log("gemm:", json.dumps(also["gemm_inner_product"]))
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(blob)
+        log("cpu baseline:", json.dumps(cpu))
+
+    line = {
+        "metric": "decode_tokens_per_sec", "value": round(head["tokens_per_s"], 2), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "Llama-2 110M-shape greedy decode (dim 768, 12 layers, 12 heads x 64, ffn 2048, vocab 32000, "
+                               "seq 1024), batch 1, fp32 weights N(0,0.02), 128-id seeded prompt then decode",
+                   "prompt_tokens": N_PROMPT, "batch": 1, "device": dev_name},
+        "roofline": roof, "cpu_baseline": cpu, "also": also,
+    }
+    print(json.dumps(line), flush=True)
+    cuda.Dispose()
+
+
+if __name__ == "__main__":
+    main()

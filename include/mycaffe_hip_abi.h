@@ -207,11 +207,16 @@ enum {
      *                 HIP graph per step (1, default) or launch eagerly (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids}
-     *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it} */
+     *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it}
+     *   PROFILE_STEP  f{hLlm, pos, reps} -> per kernel class of one decode step
+     *                 f{ms per step, launches per step, algorithmic bytes per step}, classes in
+     *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,
+     *                 w2, classifier, embed+argmax */
     MCH_LLM_GENERATE_IDS = 100,
     MCH_LLM_SET_OPTION = 101,
     MCH_LLM_GENERATE_BATCH = 102,
-    MCH_LLM_QUERY_TIMING = 103
+    MCH_LLM_QUERY_TIMING = 103,
+    MCH_LLM_PROFILE_STEP = 104
 };
 
 MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);

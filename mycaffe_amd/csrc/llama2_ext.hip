@@ -246,6 +246,23 @@ __global__ void save_logits_kernel(const float* logits, float* all, const GenSta
 }
 
 // ---------------------------------------------------------------------------
+// per-kernel-class timing of one decode step: a HIP event pair around every launch
+enum StepClass { SC_MATVEC_QKV = 0, SC_ROPE_STORE, SC_ATTN_DECODE, SC_MATVEC_WO, SC_MATVEC_W13, SC_MATVEC_W2, SC_MATVEC_CLS,
+                 SC_SAMPLE, SC_COUNT };
+struct StepProfile {
+    std::vector<std::pair<int, std::pair<hipEvent_t, hipEvent_t>>> spans;
+    hipError_t begin(int cls, hipStream_t s)
+    {
+        hipEvent_t a, b;
+        hipError_t e = hipEventCreate(&a);
+        if (e == hipSuccess) e = hipEventCreate(&b);
+        if (e != hipSuccess) return e;
+        spans.push_back({cls, {a, b}});
+        return hipEventRecord(a, s);
+    }
+    hipError_t end(hipStream_t s) { return hipEventRecord(spans.back().second.second, s); }
+};
+
 template <typename T> struct LayerW { T *wqkv, *wo, *w13, *w2; float *rms_att, *rms_ffn; };
 
 class Engine {
@@ -264,10 +281,11 @@ public:
     long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
                   std::vector<float>* logits, std::atomic<bool>* cancel);
     void release();
+    long profile_step(int pos, int reps, std::vector<float>* out);
 
 private:
     template <typename T> long upload(const float* blob);
-    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits);
+    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr);
     long ensure_state(int B, int nSteps);
 
     hipStream_t stream = nullptr;
@@ -291,7 +309,7 @@ private:
     GenState* dstate = nullptr;
     int *dprompt = nullptr, *dnext = nullptr, *dcur = nullptr, *dout = nullptr;
     hipGraphExec_t graphExec = nullptr;
-    int graphB = 0; bool graphLogits = false; float* graphAll = nullptr;
+    int graphB = 0;
 };
 
 void Engine::release()
@@ -487,46 +505,114 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
 }
 
 // enqueue one decode step for B sequences at the device-side position
-template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits)
+template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof)
 {
     const int dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
     const int ldq = dim + 2 * kvd;
+#define SPAN_BEGIN(cls) do { if (prof) HIPCHK(prof->begin(cls, s)); } while (0)
+#define SPAN_END() do { if (prof) HIPCHK(prof->end(s)); } while (0)
+    SPAN_BEGIN(SC_SAMPLE);
     hipLaunchKernelGGL(embed_step_kernel<T>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const T*)emb, x, dim, dcur);
     HIPCHK(hipGetLastError());
+    SPAN_END();
     const float scale = 1.0f / sqrtf((float)hs);
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
         float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
         float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
         // qkv = [Wq;Wk;Wv] rmsnorm(x)
+        SPAN_BEGIN(SC_MATVEC_QKV);
         HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq)));
+        SPAN_END();
+        SPAN_BEGIN(SC_ROPE_STORE);
         {
             const int n = B * (dim / 2 + kvd / 2 + kvd);
             hipLaunchKernelGGL(rope_store_kernel, (n + 255) / 256, 256, 0, s, dstate, qkv, qc, kcl, vcl, fcos, fsin, B, dim, kvd, hs,
                                cfg.seq_len);
             HIPCHK(hipGetLastError());
         }
+        SPAN_END();
         // xb = attention(q, cache[0..pos])
+        SPAN_BEGIN(SC_ATTN_DECODE);
         HIPCHK(k_attn_decode(s, F32, qc, kcl, vcl, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len,
                              (long long)cfg.seq_len * kvd, hs, kvd, scale, ws, wsBytes, &dstate->len));
+        SPAN_END();
         // x += Wo xb
+        SPAN_BEGIN(SC_MATVEC_WO);
         HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim)));
+        SPAN_END();
         // hb = silu(W1 rmsnorm(x)) * (W3 rmsnorm(x))
+        SPAN_BEGIN(SC_MATVEC_W13);
         HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid)));
+        SPAN_END();
         // x += W2 hb
+        SPAN_BEGIN(SC_MATVEC_W2);
         HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim)));
+        SPAN_END();
     }
     // logits = Wcls rmsnorm(x)
+    SPAN_BEGIN(SC_MATVEC_CLS);
     HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V)));
+    SPAN_END();
     if (allLogits) {
         hipLaunchKernelGGL(save_logits_kernel, dim3((V + 255) / 256 > 64 ? 64 : (V + 255) / 256, B), 256, 0, s, logits, allLogits,
                            dstate, V, nSteps);
         HIPCHK(hipGetLastError());
     }
+    SPAN_BEGIN(SC_SAMPLE);
     hipLaunchKernelGGL(argmax_kernel, B, 1024, 0, s, logits, V, dstate, dnext, dout, cfg.seq_len);
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(advance_kernel, 1, 1, 0, s, dstate);
     HIPCHK(hipGetLastError());
+    SPAN_END();
+#undef SPAN_BEGIN
+#undef SPAN_END
+    return 0;
+}
+
+// Runs `reps` eager decode steps of one sequence starting at position `pos` (the cache
+// content before `pos` is whatever earlier generations left; only timing matters here) and
+// returns, per kernel class: {milliseconds per step, launches per step, algorithmic bytes per step}.
+long Engine::profile_step(int pos, int reps, std::vector<float>* out)
+{
+    if (!loaded) return MCH_ERROR_LLM_GENERATE;
+    if (reps < 1 || pos < 0 || pos + reps > cfg.seq_len) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long e = ensure_state(1, cfg.seq_len);
+    if (e) return e;
+    hipStream_t s = stream;
+    std::vector<int> hp(cfg.seq_len, 1);
+    HIPCHK(hipMemcpyAsync(dprompt, hp.data(), hp.size() * 4, hipMemcpyHostToDevice, s));
+    GenState st0 = {pos, cfg.seq_len, pos + 1, 0};
+    HIPCHK(hipMemcpyAsync(dstate, &st0, sizeof(st0), hipMemcpyHostToDevice, s));
+    HIPCHK(hipStreamSynchronize(s));
+    StepProfile prof;
+    for (int i = 0; i < reps && !e; i++) e = bf16_weights ? step<bf16_t>(s, 1, cfg.seq_len, nullptr, &prof) : step<float>(s, 1, cfg.seq_len, nullptr, &prof);
+    hipError_t he = hipStreamSynchronize(s);
+    if (!e && he != hipSuccess) e = (long)he;
+    std::vector<double> ms(SC_COUNT, 0.0), cnt(SC_COUNT, 0.0);
+    for (auto& sp : prof.spans) {
+        float t = 0.f;
+        if (!e && hipEventElapsedTime(&t, sp.second.first, sp.second.second) == hipSuccess) { ms[sp.first] += t; cnt[sp.first] += 1; }
+        (void)hipEventDestroy(sp.second.first);
+        (void)hipEventDestroy(sp.second.second);
+    }
+    if (e) return e;
+    const double es = bf16_weights ? 2.0 : 4.0;
+    const double L = cfg.n_layers, dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
+    const double meanLen = pos + 1 + (reps - 1) / 2.0;
+    double bytes[SC_COUNT] = {0};
+    bytes[SC_MATVEC_QKV] = L * (dim + 2 * kvd) * dim * es;
+    bytes[SC_MATVEC_WO] = L * dim * dim * es;
+    bytes[SC_MATVEC_W13] = L * 2 * hid * dim * es;
+    bytes[SC_MATVEC_W2] = L * dim * hid * es;
+    bytes[SC_MATVEC_CLS] = (double)cfg.vocab_size * dim * es;
+    bytes[SC_ATTN_DECODE] = L * 2 * meanLen * kvd * 4.0;
+    out->clear();
+    for (int c = 0; c < SC_COUNT; c++) {
+        out->push_back((float)(ms[c] / reps));
+        out->push_back((float)(cnt[c] / reps));
+        out->push_back((float)bytes[c]);
+    }
     return 0;
 }
 
@@ -749,6 +835,16 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         Llm* m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps}, ppOut, plOut);
+    }
+    case MCH_LLM_PROFILE_STEP: {
+        if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        std::lock_guard<std::mutex> run(m->runLock);
+        std::vector<float> out;
+        long e = m->engine.profile_step((int)pIn[1], (int)pIn[2], &out);
+        if (e) return (MCH_LONG)e;
+        return (MCH_LONG)give(out, ppOut, plOut);
     }
     case MCH_LLM_GENERATE_IDS:
     case MCH_LLM_GENERATE_BATCH: {

@@ -23,6 +23,10 @@ class CUDAFN_EXTENSION_LLM:
     SET_OPTION = 101
     GENERATE_BATCH = 102
     QUERY_TIMING = 103
+    PROFILE_STEP = 104
+
+
+STEP_CLASSES = ("matvec_qkv", "rope_store", "attn_decode", "matvec_wo", "matvec_w13", "matvec_w2", "matvec_cls", "embed_argmax")
 
 
 class LlmInference:
@@ -94,3 +98,9 @@ class LlmInference:
         """(milliseconds, steps) of the timed span of the last generation, from HIP events."""
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
         return float(rg[0]), int(rg[1])
+
+    def ProfileStep(self, pos, reps=8):
+        """Per-kernel-class timing of eager decode steps at ``pos`` (HIP event pairs around
+        every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}."""
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.PROFILE_STEP, self.m_rgLlm + [pos, reps])
+        return {name: (float(rg[3 * i]), float(rg[3 * i + 1]), float(rg[3 * i + 2])) for i, name in enumerate(STEP_CLASSES)}
