@@ -113,37 +113,40 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 }
 
 // ---------------------------------------------------------------------------
-// MFMA flash attention, bf16 storage, head size 64.
+// MFMA flash attention for head sizes 64 and 128, bf16 and fp32 storage.
 //
 // One workgroup = NW wavefronts; each wavefront owns QT tiles of 32 query rows and walks
 // the keys in LDS blocks of 64, consumed as two 32-key online-softmax steps.  Per step:
 //
-//   S^T = K Q^T   v_mfma_f32_32x32x16_bf16, A = K rows from LDS (128-bit reads), B = Q
-//                 fragments held in registers for the whole kernel.  Computing the
-//                 TRANSPOSED scores puts one query per lane (lane%32) and its keys
-//                 in that lane's accumulator registers, so the row max / row sum of
-//                 the online softmax are in-register reductions plus ONE cross-lane
-//                 exchange (lane ^ 32), and the per-row rescale factor is a per-lane
-//                 scalar.
-//   P^T           exp2 with the softmax scale folded into one fma per score, packed
-//                 to bf16 in registers in exactly the order the next MFMA wants.
-//   O^T += V^T P^T  A = V^T from LDS (V is transposed while it is stored to LDS, two
-//                 64-bit reads per fragment), B = P^T from registers.
+//   S^T = K Q^T   A = K rows from LDS (128-bit reads), B = Q fragments held in registers for
+//                 the whole kernel.  Computing the TRANSPOSED scores puts one query per
+//                 lane (lane%32) and its keys in that lane's accumulator registers, so the
+//                 row max / row sum of the online softmax are in-register reductions plus
+//                 ONE cross-lane exchange (lane ^ 32), and the per-row rescale factor is a
+//                 per-lane scalar.
+//   P^T           exp2 with the softmax scale folded into one fma per score; for bf16 the
+//                 weights are packed in registers in exactly the order the next MFMA wants.
+//   O^T += V^T P^T  A = V^T from LDS (V is transposed while it is stored to LDS), B = P^T
+//                 straight from registers.
 //
-// K and V blocks are shared by the wavefronts of a workgroup through LDS and prefetched
-// into registers one block ahead.  The kernel is bound by the softmax VALU work (about
-// eight issue slots per score against 256 MFMA flops per score at head size 64), so the
-// configuration is chosen for wavefronts per SIMD: that is what lets one wavefront's MFMAs
-// run under another's exp2/fma/add stream.  Causal: key blocks past the workgroup's last
-// row are never visited, wavefronts skip steps past their own rows, only diagonal steps
-// pay for the element mask, and the heaviest query blocks are scheduled first.
+// bf16 uses v_mfma_f32_32x32x16_bf16 (a 16-byte fragment per lane covers 16 contraction
+// indices); fp32 uses v_mfma_f32_32x32x2_f32 four times per 16-byte fragment: lane half h
+// holds indices 4h..4h+3 of an 8-index group and step e contracts the pair {e, 4+e}, which
+// is legal because the slot-to-index assignment only has to agree between A and B.
+//
+// The bf16 kernel is bound by the softmax VALU work (v_exp_f32 is quarter rate: about 27
+// cycles per score against 8 MFMA cycles per score at head size 64); the fp32 kernel is
+// MFMA bound.  Causal: key blocks past the workgroup's last row are never visited,
+// wavefronts skip steps past their own rows, only diagonal steps pay for the element mask,
+// and the heaviest query blocks are scheduled first.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // one 16-byte MFMA operand fragment
 
 struct FlashArgs {
-    const bf16_t* q; const bf16_t* k; const bf16_t* v; bf16_t* y;
+    const void* q; const void* k; const void* v; void* y;
     const float* mask;   // (B, Tk) key mask for KIND 2
     int B, H, Tq, Tk;
     float c;             // softmax scale * log2(e)
@@ -157,15 +160,78 @@ __device__ inline uint32_t pack_bf16x2(float a, float b)
     return *reinterpret_cast<uint32_t*>(&r);
 }
 
+template <typename T> struct FlashTraits;
+template <> struct FlashTraits<bf16_t> {
+    static constexpr int EPC = 8;    // elements per 16-byte chunk
+    static constexpr int CPF = 16;   // contraction indices covered by one fragment (both lane halves)
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&a), *reinterpret_cast<bf16x8*>(&b), c, 0, 0, 0);
+    }
+    // V^T fragment t of a 32-key step: keys 16t + 4h .. +3 and 16t + 8 + 4h .. +3
+    __device__ static inline u32x4 load_vt(const bf16_t* row, int t, int half)
+    {
+        const bf16_t* p = row + 16 * t + 4 * half;
+        uint2 lo = *(const uint2*)p, hi = *(const uint2*)(p + 8);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+    // P^T fragment t: the weights held in accumulator registers 8t .. 8t+7
+    __device__ static inline u32x4 pack_p(const floatx16& p, int t)
+    {
+        return u32x4{pack_bf16x2(p[8 * t], p[8 * t + 1]), pack_bf16x2(p[8 * t + 2], p[8 * t + 3]),
+                     pack_bf16x2(p[8 * t + 4], p[8 * t + 5]), pack_bf16x2(p[8 * t + 6], p[8 * t + 7])};
+    }
+    __device__ static inline void store4(bf16_t* dst, float a, float b, float c, float d)
+    {
+        uint2 w;
+        w.x = pack_bf16x2(a, b);
+        w.y = pack_bf16x2(c, d);
+        *(uint2*)dst = w;
+    }
+    __device__ static inline void scatter_chunk(bf16_t* d, int ld, u32x4 r)
+    {
+        d[0 * ld] = (bf16_t)(r.x & 0xffffu); d[1 * ld] = (bf16_t)(r.x >> 16);
+        d[2 * ld] = (bf16_t)(r.y & 0xffffu); d[3 * ld] = (bf16_t)(r.y >> 16);
+        d[4 * ld] = (bf16_t)(r.z & 0xffffu); d[5 * ld] = (bf16_t)(r.z >> 16);
+        d[6 * ld] = (bf16_t)(r.w & 0xffffu); d[7 * ld] = (bf16_t)(r.w >> 16);
+    }
+};
+template <> struct FlashTraits<float> {
+    static constexpr int EPC = 4;
+    static constexpr int CPF = 8;
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+        return c;
+    }
+    // V^T fragment t of a 32-key step: keys 8t + 4h .. +3
+    __device__ static inline u32x4 load_vt(const float* row, int t, int half) { return *(const u32x4*)(row + 8 * t + 4 * half); }
+    // P^T fragment t: the weights held in accumulator registers 4t .. 4t+3
+    __device__ static inline u32x4 pack_p(const floatx16& p, int t)
+    {
+        return u32x4{__float_as_uint(p[4 * t]), __float_as_uint(p[4 * t + 1]), __float_as_uint(p[4 * t + 2]),
+                     __float_as_uint(p[4 * t + 3])};
+    }
+    __device__ static inline void store4(float* dst, float a, float b, float c, float d) { *(float4*)dst = make_float4(a, b, c, d); }
+    __device__ static inline void scatter_chunk(float* d, int ld, u32x4 r)
+    {
+        d[0 * ld] = __uint_as_float(r.x); d[1 * ld] = __uint_as_float(r.y);
+        d[2 * ld] = __uint_as_float(r.z); d[3 * ld] = __uint_as_float(r.w);
+    }
+};
+
 // One 32-key online-softmax step for all query tiles of a wavefront, written as a single
 // branch-free block (apart from the wavefront-uniform rescale test) so the tiles'
-// dependency chains interleave.  MASKED: scores equal to `sentinel` stand for the
-// reference's -1e29 fill; their weight is decided by comparison (1 while the row maximum
-// is still the sentinel, else exactly 0) because exp2 of a difference of two huge
-// products would not cancel exactly.
+// dependency chains interleave.  On return s holds the weights p.  MASKED: scores equal to
+// `sentinel` stand for the reference's -1e29 fill; their weight is decided by comparison (1
+// while the row maximum is still the sentinel, else exactly 0) because exp2 of a difference
+// of two huge products would not cancel exactly.
 template <bool MASKED, int DT, int QT>
 __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (&o)[DT][QT], float (&m)[QT], float (&l)[QT],
-                                                   bf16x8 (&pf)[QT][2], float c, float sentinel)
+                                                   float c, float sentinel)
 {
     float mx[QT], mnew[QT], alpha[QT], mc[QT];
 #pragma unroll
@@ -185,15 +251,15 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
         m[qt] = mnew[qt];
         same = same && (alpha[qt] == 1.0f);
     }
-    float p[QT][16];
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
         float rs = 0.f;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            p[qt][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][v], c, -mc[qt]));
-            if (MASKED && s[qt][v] == sentinel) p[qt][v] = (mnew[qt] == sentinel) ? 1.0f : 0.0f;
-            rs += p[qt][v];
+            float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][v], c, -mc[qt]));
+            if (MASKED && s[qt][v] == sentinel) pv = (mnew[qt] == sentinel) ? 1.0f : 0.0f;
+            s[qt][v] = pv;
+            rs += pv;
         }
         l[qt] = l[qt] * alpha[qt] + rs;
     }
@@ -205,30 +271,27 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
 #pragma unroll
                 for (int v = 0; v < 16; v++) o[dt][qt][v] *= alpha[qt];
     }
-    // MFMA step t contracts the 16 keys held in registers 8t..8t+7
-#pragma unroll
-    for (int qt = 0; qt < QT; qt++)
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            uint32_t w[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) w[j] = pack_bf16x2(p[qt][8 * t + 2 * j], p[qt][8 * t + 2 * j + 1]);
-            pf[qt][t] = *reinterpret_cast<bf16x8*>(w);
-        }
 }
 
 // KIND: 0 no mask, 1 causal, 2 per-key mask (B, Tk).  OCC: workgroups per CU the register budget is set for.
-template <int KIND, int QT, int NW, int OCC>
-__global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(FlashArgs a)
+// PREFETCH: hold the next K / V block in registers while computing on the current one.
+template <typename T, int HS, int KIND, int QT, int NW, int OCC, bool PREFETCH>
+__global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 {
-    constexpr int HS = 64, NT = NW * 64, BM = NW * 32 * QT, BN = 64;
-    constexpr int KS = HS / 16, DT = HS / 32;
-    constexpr int LDK = HS + 8, LDV = BN + 8;
-    constexpr int KPT = (BN * HS / 8) / NT;   // 16-byte K chunks per thread (512 chunks per block)
-    constexpr int VPW = 8 / NW;               // 8-dim V chunks per wavefront
-    static_assert(KPT >= 1 && VPW >= 1, "at most 8 wavefronts");
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * LDK];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[HS * LDV];
+    typedef FlashTraits<T> TR;
+    constexpr int NT = NW * 64, BM = NW * 32 * QT, BN = 64;
+    constexpr int EPC = TR::EPC, CPF = TR::CPF;
+    constexpr int KF = HS / CPF;              // fragments along the head dimension (S^T contraction)
+    constexpr int PF = 32 / CPF;              // fragments along a 32-key step (P V contraction)
+    constexpr int DT = HS / 32;
+    constexpr int PAD = 16 / (int)sizeof(T);
+    constexpr int LDK = HS + PAD, LDV = BN + PAD;
+    constexpr int CHR = HS / EPC;             // 16-byte chunks per K / V row
+    constexpr int KPT = (BN * CHR) / NT;      // K chunks per thread per block
+    constexpr int VPW = CHR / NW;             // V chunks per wavefront (one key per lane)
+    static_assert(KPT >= 1 && VPW >= 1 && (BN * CHR) % NT == 0 && CHR % NW == 0, "tile / thread mismatch");
+    __shared__ __attribute__((aligned(16))) T Ks[BN * LDK];
+    __shared__ __attribute__((aligned(16))) T Vt[HS * LDV];
     __shared__ float Ms[BN];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -237,17 +300,17 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
     const int h = blockIdx.y, b = blockIdx.z;
     const size_t bh = (size_t)b * a.H + h;
     const int q0 = qblock * BM + wave * 32 * QT;      // first row of this wavefront
-    const bf16_t* qp = a.q + bh * a.Tq * HS;
-    const bf16_t* kp = a.k + bh * a.Tk * HS;
-    const bf16_t* vp = a.v + bh * a.Tk * HS;
+    const T* qp = (const T*)a.q + bh * a.Tq * HS;
+    const T* kp = (const T*)a.k + bh * a.Tk * HS;
+    const T* vp = (const T*)a.v + bh * a.Tk * HS;
 
-    // Q fragments: lane (query l32 of tile qt, half) holds dims 16*ks + 8*half .. +7
-    bf16x8 qf[QT][KS];
+    // Q fragments: lane (query l32 of tile qt, half) holds elements f*CPF + half*CPF/2 .. of its row
+    u32x4 qf[QT][KF];
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
         int row = min(q0 + qt * 32 + l32, a.Tq - 1);
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) qf[qt][ks] = *(const bf16x8*)(qp + (size_t)row * HS + ks * 16 + half * 8);
+        for (int f = 0; f < KF; f++) qf[qt][f] = *(const u32x4*)(qp + (size_t)row * HS + f * CPF + half * (CPF / 2));
     }
     floatx16 o[DT][QT];
 #pragma unroll
@@ -264,36 +327,29 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
     if (KIND == 1) kend = min(a.Tk, qblock * BM + BM);
     const int nkb = (kend + BN - 1) / BN;
 
-    // global -> register prefetch of one K / V block.  K: 8 threads per key row; V: one key per
-    // lane and 8-dim chunks per wavefront, so that the transposing 16-bit LDS stores of a
-    // wavefront hit consecutive addresses.
-    uint4 kreg[KPT], vreg[VPW];
+    // global -> (register ->) LDS movement of one K / V block.  K: consecutive threads take
+    // consecutive 16-byte chunks; V: one key per lane and whole chunks per wavefront, so that the
+    // transposing LDS stores of a wavefront hit consecutive addresses.
+    u32x4 kreg[KPT], vreg[VPW];
     auto gload = [&](int kb) {
         const int kbase = kb * BN;
 #pragma unroll
         for (int i = 0; i < KPT; i++) {
             const int e = tid + i * NT;
-            kreg[i] = *(const uint4*)(kp + (size_t)min(kbase + (e >> 3), a.Tk - 1) * HS + (e & 7) * 8);
+            kreg[i] = *(const u32x4*)(kp + (size_t)min(kbase + e / CHR, a.Tk - 1) * HS + (e % CHR) * EPC);
         }
         const size_t vrow = (size_t)min(kbase + lane, a.Tk - 1) * HS;
 #pragma unroll
-        for (int i = 0; i < VPW; i++) vreg[i] = *(const uint4*)(vp + vrow + (wave + NW * i) * 8);
+        for (int i = 0; i < VPW; i++) vreg[i] = *(const u32x4*)(vp + vrow + (wave + NW * i) * EPC);
     };
     auto sstore = [&](int kb) {
 #pragma unroll
         for (int i = 0; i < KPT; i++) {
             const int e = tid + i * NT;
-            *(uint4*)(&Ks[(e >> 3) * LDK + (e & 7) * 8]) = kreg[i];
+            *(u32x4*)(&Ks[(e / CHR) * LDK + (e % CHR) * EPC]) = kreg[i];
         }
 #pragma unroll
-        for (int i = 0; i < VPW; i++) {
-            bf16_t* d = &Vt[(wave + NW * i) * 8 * LDV + lane];
-            const uint4 r = vreg[i];
-            d[0 * LDV] = (bf16_t)(r.x & 0xffffu); d[1 * LDV] = (bf16_t)(r.x >> 16);
-            d[2 * LDV] = (bf16_t)(r.y & 0xffffu); d[3 * LDV] = (bf16_t)(r.y >> 16);
-            d[4 * LDV] = (bf16_t)(r.z & 0xffffu); d[5 * LDV] = (bf16_t)(r.z >> 16);
-            d[6 * LDV] = (bf16_t)(r.w & 0xffffu); d[7 * LDV] = (bf16_t)(r.w >> 16);
-        }
+        for (int i = 0; i < VPW; i++) TR::scatter_chunk(&Vt[(wave + NW * i) * EPC * LDV + lane], LDV, vreg[i]);
         if (KIND == 2 && tid < BN) {
             const int key = kb * BN + tid;
             Ms[tid] = key < a.Tk ? a.mask[(size_t)b * a.Tk + key] : 1.f;
@@ -307,12 +363,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
 #pragma unroll
     for (int qt = 0; qt < QT; qt++)
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[qt][ks]));
+        for (int f = 0; f < KF; f++) asm volatile("" : "+v"(qf[qt][f]));
     __syncthreads();
 
     const float c = a.c;
     for (int kb = 0; kb < nkb; kb++) {
-        if (kb + 1 < nkb) gload(kb + 1);
+        if (PREFETCH && kb + 1 < nkb) gload(kb + 1);
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const int k0 = kb * BN + 32 * sub;
@@ -325,14 +381,13 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
 #pragma unroll
                     for (int v = 0; v < 16; v++) s[qt][v] = 0.f;
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    bf16x8 kf = *(const bf16x8*)(&Ks[(sub * 32 + l32) * LDK + ks * 16 + half * 8]);
+                for (int f = 0; f < KF; f++) {
+                    const u32x4 kf = *(const u32x4*)(&Ks[(sub * 32 + l32) * LDK + f * CPF + half * (CPF / 2)]);
 #pragma unroll
-                    for (int qt = 0; qt < QT; qt++) s[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qt][ks], s[qt], 0, 0, 0);
+                    for (int qt = 0; qt < QT; qt++) s[qt] = TR::mma(kf, qf[qt][f], s[qt]);
                 }
                 // register v holds key k0 + 8*(v/4) + 4*half + v%4 for query q0 + 32*qt + l32
                 const bool maskedBlock = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk) || KIND == 2;   // wavefront-uniform
-                bf16x8 pf[QT][2];
                 if (maskedBlock) {
 #pragma unroll
                     for (int qt = 0; qt < QT; qt++) {
@@ -348,27 +403,32 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
                             s[qt][v] = sv;
                         }
                     }
-                    flash_softmax_step<true, DT, QT>(s, o, m, l, pf, c, a.maskedRaw);
+                    flash_softmax_step<true, DT, QT>(s, o, m, l, c, a.maskedRaw);
                 } else {
-                    flash_softmax_step<false, DT, QT>(s, o, m, l, pf, c, a.maskedRaw);
+                    flash_softmax_step<false, DT, QT>(s, o, m, l, c, a.maskedRaw);
                 }
-                // O^T += V^T P^T; slot j of step t is key 16t + 4*half + j (j < 4) or 16t + 8 + 4*half + j - 4
+                // O^T += V^T P^T
+                u32x4 pf[QT][PF];
 #pragma unroll
-                for (int t = 0; t < 2; t++)
+                for (int qt = 0; qt < QT; qt++) {
+#pragma unroll
+                    for (int t = 0; t < PF; t++) pf[qt][t] = TR::pack_p(s[qt], t);
+                }
+#pragma unroll
+                for (int t = 0; t < PF; t++)
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
-                        const bf16_t* vrow = &Vt[(dt * 32 + l32) * LDV + 32 * sub + 16 * t + 4 * half];
-                        uint2 lo = *(const uint2*)vrow;
-                        uint2 hi = *(const uint2*)(vrow + 8);
-                        uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
-                        bf16x8 vf = *reinterpret_cast<bf16x8*>(w);
+                        const u32x4 vf = TR::load_vt(&Vt[(dt * 32 + l32) * LDV + 32 * sub], t, half);
 #pragma unroll
-                        for (int qt = 0; qt < QT; qt++) o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qt][t], o[dt][qt], 0, 0, 0);
+                        for (int qt = 0; qt < QT; qt++) o[dt][qt] = TR::mma(vf, pf[qt][t], o[dt][qt]);
                     }
             }
         }
         __syncthreads();
-        if (kb + 1 < nkb) sstore(kb + 1);
+        if (kb + 1 < nkb) {
+            if (!PREFETCH) gload(kb + 1);
+            sstore(kb + 1);
+        }
         __syncthreads();
     }
 
@@ -379,53 +439,51 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_bf16_hs64_kernel(Flash
         const float lt = l[qt] + __shfl_xor(l[qt], 32, 64);
         const float inv = 1.0f / lt;
         if (qrow < a.Tq) {
-            bf16_t* yr = a.y + (bh * a.Tq + qrow) * HS;
+            T* yr = (T*)a.y + (bh * a.Tq + qrow) * HS;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    uint2 w;
-                    w.x = pack_bf16x2(o[dt][qt][4 * g] * inv, o[dt][qt][4 * g + 1] * inv);
-                    w.y = pack_bf16x2(o[dt][qt][4 * g + 2] * inv, o[dt][qt][4 * g + 3] * inv);
-                    *(uint2*)(yr + 32 * dt + 8 * g + 4 * half) = w;
-                }
+                for (int g = 0; g < 4; g++)
+                    TR::store4(yr + 32 * dt + 8 * g + 4 * half, o[dt][qt][4 * g] * inv, o[dt][qt][4 * g + 1] * inv,
+                               o[dt][qt][4 * g + 2] * inv, o[dt][qt][4 * g + 3] * inv);
         }
     }
 }
 
-template <int QT, int NW, int OCC>
+template <typename T, int HS, int QT, int NW, int OCC, bool PREFETCH>
 static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
 {
     constexpr int BM = NW * 32 * QT;
     dim3 grid((f.Tq + BM - 1) / BM, f.H, f.B);
-    if (kind == MASK_NONE) hipLaunchKernelGGL((flash_fwd_bf16_hs64_kernel<0, QT, NW, OCC>), grid, NW * 64, 0, s, f);
-    else if (kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_fwd_bf16_hs64_kernel<1, QT, NW, OCC>), grid, NW * 64, 0, s, f);
-    else hipLaunchKernelGGL((flash_fwd_bf16_hs64_kernel<2, QT, NW, OCC>), grid, NW * 64, 0, s, f);
+    if (kind == MASK_NONE) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 0, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
+    else if (kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 1, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
+    else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 2, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     return hipGetLastError();
 }
 
 hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* handled)
 {
     *handled = false;
-    if (dt != BF16 || a.hs != 64) return hipSuccess;
+    if (a.hs != 64 && a.hs != 128) return hipSuccess;
     if (a.kind != MASK_NONE && a.kind != MASK_CAUSAL && a.kind != MASK_KEY) return hipSuccess;
     if ((((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.y) & 15) != 0) return hipSuccess;
     FlashArgs f;
-    f.q = (const bf16_t*)a.q; f.k = (const bf16_t*)a.k; f.v = (const bf16_t*)a.v; f.y = (bf16_t*)a.y;
+    f.q = a.q; f.k = a.k; f.v = a.v; f.y = a.y;
     f.mask = a.mask; f.B = a.B; f.H = a.H; f.Tq = a.Tq; f.Tk = a.Tk;
     f.c = a.scale * 1.4426950408889634f;
     f.maskedRaw = MASKED / a.scale;
     *handled = true;
-    static int cfg = getenv("MCH_FLASH_CFG") ? atoi(getenv("MCH_FLASH_CFG")) : 0;
-    switch (cfg) {
-    case 1: return flash_launch_cfg<1, 4, 3>(s, f, a.kind);
-    case 2: return flash_launch_cfg<1, 4, 4>(s, f, a.kind);
-    case 3: return flash_launch_cfg<1, 8, 2>(s, f, a.kind);
-    case 4: return flash_launch_cfg<2, 8, 1>(s, f, a.kind);
-    case 5: return flash_launch_cfg<1, 8, 1>(s, f, a.kind);
-    case 6: return flash_launch_cfg<2, 2, 4>(s, f, a.kind);
-    default: return flash_launch_cfg<2, 4, 2>(s, f, a.kind);
+    if (dt == BF16) {
+        if (a.hs == 64) {
+            // causal work is triangular: 32-row wavefront tiles in 256-row workgroups keep the diagonal
+            // waste small; square work prefers the 64-row wavefront tile (each LDS fragment feeds two MFMAs)
+            if (a.kind == MASK_CAUSAL) return flash_launch_cfg<bf16_t, 64, 1, 8, 2, true>(s, f, a.kind);
+            return flash_launch_cfg<bf16_t, 64, 2, 4, 2, true>(s, f, a.kind);
+        }
+        return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
     }
+    if (a.hs == 64) return flash_launch_cfg<float, 64, 2, 4, 2, false>(s, f, a.kind);
+    return flash_launch_cfg<float, 128, 1, 8, 1, false>(s, f, a.kind);
 }
 
 }  // namespace mch
