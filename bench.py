@@ -6,8 +6,11 @@
 One "step" is one greedy decode step (one new token) of the Llama-2 110M-shape
 decoder (dim 768, 12 layers, 12 heads x 64, FFN 2048 SwiGLU, vocab 32000, seq 1024;
 random-init N(0, 0.02) fp32 weights, 128 seeded prompt ids), run by the llama2
-extension library through the C ABI.  After the prompt and W untimed decode steps,
-exactly K decode steps are timed with HIP events on the engine's stream.
+extension library through the C ABI.  A generation forces the 128 prompt ids, runs W
+untimed greedy steps and then timed greedy steps up to position 1023; the defaults
+(W = 16, K = 880) are exactly one generation to 1024 tokens.  A larger K continues with
+further generations (fresh seeded prompts) until exactly K steps have been timed with
+HIP events on the engine's stream.
 
 The single JSON line also carries:
   roofline      the dominant kernel of that workload (the fused mat-vec family that
@@ -57,32 +60,44 @@ def weight_bytes(cfg, es):
 
 
 def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
+    """Times exactly `steps` greedy decode steps (see the module docstring); returns the engine and the figures."""
     from mycaffe_amd.llm_inference import LlmInference
     inf = LlmInference(cuda)
     inf.Initialize(fTemperature=0.0)
     inf.SetOption(1, 1 if bf16 else 0)
     inf.SetOption(3, 1 if graph else 0)
     inf.Load(path)
-    rng = np.random.default_rng(seed)
-    total = N_PROMPT + warmup + steps
-    inf.SetOption(2, N_PROMPT + warmup)
-    t0 = time.perf_counter()
-    if batch == 1:
-        prompt = rng.integers(3, C4["vocab_size"], N_PROMPT)
-        ids = inf.GenerateIds(prompt, total)
-    else:
-        prompt = rng.integers(3, C4["vocab_size"], (batch, N_PROMPT))
-        ids = inf.GenerateBatch(prompt, total)
-    wall = time.perf_counter() - t0
-    ms, nsteps = inf.QueryTiming()
-    assert nsteps == steps, (nsteps, steps)
-    res = {"ms_per_step": ms / steps, "tokens_per_s": batch * steps / (ms / 1e3), "wall_s_whole_generation": wall,
-           "prompt": prompt, "ids": ids}
+    per_gen = C4["seq_len"] - N_PROMPT - warmup
+    left, ms_total, wall, gen = steps, 0.0, 0.0, 0
+    first = None
+    while left > 0:
+        k = min(left, per_gen)
+        rng = np.random.default_rng(seed + gen)
+        total = N_PROMPT + warmup + k
+        inf.SetOption(2, N_PROMPT + warmup)
+        t0 = time.perf_counter()
+        if batch == 1:
+            prompt = rng.integers(3, C4["vocab_size"], N_PROMPT)
+            ids = inf.GenerateIds(prompt, total)
+        else:
+            prompt = rng.integers(3, C4["vocab_size"], (batch, N_PROMPT))
+            ids = inf.GenerateBatch(prompt, total)
+        wall += time.perf_counter() - t0
+        ms, nsteps = inf.QueryTiming()
+        assert nsteps == k, (nsteps, k)
+        ms_total += ms
+        left -= k
+        if first is None:
+            first = (prompt, ids)
+        gen += 1
+    res = {"ms_per_step": ms_total / steps, "tokens_per_s": batch * steps / (ms_total / 1e3), "wall_s_whole_generation": wall,
+           "prompt": first[0], "ids": first[1], "generations": gen}
     return inf, res
 
 
 def matvec_roofline(inf, pos, bf16):
-    prof = inf.ProfileStep(pos, 8)
+    prof = inf.ProfileStep(pos, 16)
+    pair_ms = prof.pop("_event_pair_ms")
     mv = [k for k in prof if k.startswith("matvec")]
     ms = sum(prof[k][0] for k in mv)
     launches = sum(prof[k][1] for k in mv)
@@ -94,26 +109,34 @@ def matvec_roofline(inf, pos, bf16):
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
             "algorithmic_bytes_per_launch": round(nbytes / launches), "avg_launch_us": round(ms / launches * 1e3, 3),
-            "launches_per_step": launches, "per_class": detail}
+            "launches_per_step": launches, "event_pair_around_empty_kernel_us": round(pair_ms * 1e3, 3), "per_class": detail}
 
 
-def cpu_baseline(blob, budget_s=20.0):
-    """The CPU checker on this host: same model, same prompt convention, bounded sample."""
+def cpu_baseline(blob, gpu_prompt, gpu_ids, budget_s=12.0):
+    """The CPU checker on this host's cores: whole generations of the same workload (128 forced ids, then greedy
+    to 1024 positions), repeated until about `budget_s` seconds of CPU work; every position counts as one token
+    (the reference loop spends the same work on a forced position as on a sampled one)."""
     from oracle import llama2 as O
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    m = O.Llama(C4, blob, False)
-    prompt = np.random.default_rng(1).integers(3, C4["vocab_size"], N_PROMPT)
-    t0 = time.perf_counter()
-    m.generate_greedy(prompt[:4], 4)
-    per = (time.perf_counter() - t0) / 4
-    n = int(max(8, min(N_PROMPT, budget_s / max(per, 1e-6))))
-    m2 = O.Llama(C4, blob, False)
-    t0 = time.perf_counter()
-    m2.generate_greedy(prompt, n)
-    dt = time.perf_counter() - t0
-    return {"value": round(n / dt, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": "first %d positions of the same 128-id prompt, fp32, batch 1 (%.1f s of CPU work); the GPU "
-                      "figure times positions %d.. where attention reads a longer cache" % (n, dt, N_PROMPT)}
+    n = C4["seq_len"]
+    tokens, dt, runs, same = 0, 0.0, 0, None
+    while dt < budget_s and runs < 8:
+        m = O.Llama(C4, blob, False)
+        prompt = gpu_prompt if runs == 0 else np.random.default_rng(100 + runs).integers(3, C4["vocab_size"], N_PROMPT)
+        t0 = time.perf_counter()
+        ids = m.generate_greedy(prompt, n)
+        dt += time.perf_counter() - t0
+        tokens += n
+        if runs == 0 and gpu_ids is not None:
+            k = min(len(gpu_ids), len(ids))
+            diff = np.nonzero(np.asarray(ids[:k]) != np.asarray(gpu_ids[:k]).reshape(-1)[:k])[0]
+            same = {"positions_compared": int(k), "first_mismatch": int(diff[0]) if diff.size else None}
+        runs += 1
+        del m
+    return {"value": round(tokens / dt, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": "%d whole generation(s) of the same workload (128 forced prompt ids, then greedy to 1024 positions; "
+                      "fp32, batch 1), %d positions in %.1f s, every position counted" % (runs, tokens, dt),
+            "ids_vs_gpu_first_generation": same}
 
 
 def bench_prefill_attention(cuda, reps):
@@ -196,23 +219,38 @@ def bench_gemm(cuda, reps):
     return out
 
 
+def bench_copy(cuda, reps):
+    """Plain device copy of 64 Mi floats (reads 256 MiB, writes 256 MiB): the known-size kernel that the
+    FETCH_SIZE / WRITE_SIZE counter readings of the other kernels are scaled by."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    n = 64 << 20
+    a = cuda.AllocMemory(n)
+    b = cuda.AllocMemory(n)
+    ms = cuda.TimeFunction(CUDAFN.CUDA_COPY, [], [n, a, b], 2, reps)
+    cuda.FreeMemory(a)
+    cuda.FreeMemory(b)
+    return {"kernel": "convert_kernel<float, float>", "bytes_read": n * 4, "bytes_written": n * 4, "ms": round(ms, 4),
+            "GBps": round(2 * n * 4 / (ms / 1e3) / 1e9, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--steps", type=int, default=880)
+    ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="only the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="launch every decode kernel eagerly instead of replaying a HIP graph "
                     "(kernel tracing tools see the individual kernels this way)")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,gemm")
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,gemm "
+                    "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: every box of this build has one MI355X and the path has no multi-GPU part; "
             "run with --gpus 1")
         sys.exit(2)
-    if N_PROMPT + args.warmup + args.steps > C4["seq_len"]:
-        log("prompt (128) + warmup + steps must fit the 1024-token context")
+    if args.steps < 1 or args.warmup < 0 or N_PROMPT + args.warmup >= C4["seq_len"]:
+        log("need steps >= 1 and prompt (128) + warmup < 1024")
         sys.exit(2)
 
     from mycaffe_amd.cudadnn import CudaDnn
@@ -246,21 +284,23 @@ def main():
     if want("decode_attn"):
         also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
         log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
+    if "copy" in only:
+        also["copy_256MiB"] = bench_copy(cuda, 10)
     if want("gemm"):
         also["gemm_inner_product"] = bench_gemm(cuda, 10)
         log("gemm:", json.dumps(also["gemm_inner_product"]))
 
     cpu = None
     if not args.no_cpu:
-        cpu = cpu_baseline(blob)
+        cpu = cpu_baseline(blob, head["prompt"], head["ids"])
         log("cpu baseline:", json.dumps(cpu))
 
     line = {
-        "metric": "decode_tokens_per_sec", "value": round(head["tokens_per_s"], 2), "unit": "tokens/s",
+        "metric": "decode tokens/sec", "value": round(head["tokens_per_s"], 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "Llama-2 110M-shape greedy decode (dim 768, 12 layers, 12 heads x 64, ffn 2048, vocab 32000, "
-                               "seq 1024), batch 1, fp32 weights N(0,0.02), 128-id seeded prompt then decode",
+                               "seq 1024), batch 1, fp32 weights N(0,0.02), 128-id seeded prompt then greedy decode to 1024 tokens",
                    "prompt_tokens": N_PROMPT, "batch": 1, "device": dev_name},
         "roofline": roof, "cpu_baseline": cpu, "also": also,
     }

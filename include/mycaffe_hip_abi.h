@@ -204,7 +204,9 @@ enum {
      *   SET_OPTION    f{hLlm, option, value}; option 1 = weight storage
      *                 (0 fp32, 1 bf16), applied at the next LOAD; option 2 = first
      *                 step of the timed span; option 3 = replay one captured
-     *                 HIP graph per step (1, default) or launch eagerly (0)
+     *                 HIP graph per step (1, default) or launch eagerly (0);
+     *                 option 4 = weight rows per wavefront of the mat-vec
+     *                 kernels (1 or 2; 0 = library's choice)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it}

@@ -52,6 +52,7 @@ struct DecodeArgs {
     // captured launch serves every decode step) and the per-split chunk is derived from it
     const int* dlen;
     int rowsPerIter;
+    int* counters;   // one zero-initialised ticket per (batch, head): enables the in-kernel merge
 };
 
 __device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int* t1)
@@ -66,41 +67,17 @@ __device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int
     *t1 = min(len, *t0 + chunk);
 }
 
-// partial layout: part[((b*H + h)*splits + s) * (hs + 2)] = {m, l, acc[hs]}
+// Streams cache rows [t0, t1) for one (batch, head): every lane group of LPR lanes keeps its own
+// running max m, sum l and output slice acc[W] (dims gl*W ..).  qv holds the query slice, pre-scaled.
 template <typename T, int LPR>
-__global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
+__device__ __forceinline__ void decode_stream(const T* __restrict__ kc, const T* __restrict__ vc, long long strideT, int t0, int t1,
+                                              int wave, int grp, int d0, bool active, const float (&qv)[Vec16<T>::W], float& m,
+                                              float& l, float (&acc)[Vec16<T>::W])
 {
     constexpr int W = Vec16<T>::W;
     constexpr int RPW = 64 / LPR;  // rows per wavefront load
     constexpr int U = 4;           // row groups in flight per operand
     constexpr int NW = 4;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int grp = lane / LPR, gl = lane % LPR;
-    const int d0 = gl * W;
-    const bool active = d0 < a.hs;  // lanes beyond hs idle when hs/W is not a power of two
-
-    const T* q = (const T*)a.q + ((size_t)b * a.H + h) * a.hs;
-    const size_t base = (size_t)b * a.strideB + (size_t)(h / a.kvMul) * a.strideH;
-    const T* kc = (const T*)a.kc + base;
-    const T* vc = (const T*)a.vc + base;
-
-    float qv[W];
-#pragma unroll
-    for (int i = 0; i < W; i++) qv[i] = 0.f;
-    if (active) {
-        Vec16<T>::load(q + d0, qv);
-#pragma unroll
-        for (int i = 0; i < W; i++) qv[i] *= a.scale;
-    }
-
-    int t0, t1;
-    decode_range(a, split, &t0, &t1);
-
-    float m = -INFINITY, l = 0.f, acc[W];
-#pragma unroll
-    for (int i = 0; i < W; i++) acc[i] = 0.f;
-
     for (int tb = t0 + wave * RPW * U; tb < t1; tb += NW * RPW * U) {
         float kv[U][W], vv[U][W];
         bool ok[U];
@@ -110,12 +87,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
             ok[u] = t < t1;
 #pragma unroll
             for (int i = 0; i < W; i++) { kv[u][i] = 0.f; vv[u][i] = 0.f; }
-            if (ok[u] && active) Vec16<T>::load(kc + (size_t)t * a.strideT + d0, kv[u]);
+            if (ok[u] && active) Vec16<T>::load(kc + (size_t)t * strideT + d0, kv[u]);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             int t = tb + u * RPW + grp;
-            if (ok[u] && active) Vec16<T>::load(vc + (size_t)t * a.strideT + d0, vv[u]);
+            if (ok[u] && active) Vec16<T>::load(vc + (size_t)t * strideT + d0, vv[u]);
         }
         float s[U];
 #pragma unroll
@@ -145,8 +122,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
             m = mn;
         }
     }
+}
 
-    // merge the NW * RPW lane groups through LDS
+// Partials cross workgroups (and XCDs, whose L2 caches are not coherent with each other) inside one
+// launch, so they are written and read with device-scope relaxed atomics, which go to the coherent
+// level of the memory system, instead of a device-scope fence, which would write back and invalidate
+// the whole L2 on every call.
+__device__ __forceinline__ void part_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float part_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// Merges the 4 * (64/LPR) lane groups of a workgroup through LDS and writes {M, L, acc[hs]} to `out`.
+template <typename T, int LPR>
+__device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (&acc)[Vec16<T>::W], int wave, int grp, int gl,
+                                                 int d0, bool active, int hs, float* __restrict__ out)
+{
+    constexpr int W = Vec16<T>::W;
+    constexpr int RPW = 64 / LPR, NW = 4;
     __shared__ float sm[NW * RPW];
     __shared__ float sl[NW * RPW];
     __shared__ float sacc[NW * RPW][LPR * W + 1];
@@ -159,19 +150,185 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
     __syncthreads();
     float M = -INFINITY;
     for (int i = 0; i < NW * RPW; i++) M = fmaxf(M, sm[i]);
-    float* out = a.part + (((size_t)b * a.H + h) * a.splits + split) * (a.hs + 2);
     if (threadIdx.x == 0) {
         float L = 0.f;
         for (int i = 0; i < NW * RPW; i++) L += (sm[i] > -INFINITY) ? sl[i] * __expf(sm[i] - M) : 0.f;
-        out[0] = M;
-        out[1] = L;
+        part_store(out, M);
+        part_store(out + 1, L);
     }
-    for (int d = threadIdx.x; d < a.hs; d += 256) {
+    for (int d = threadIdx.x; d < hs; d += 256) {
         float v = 0.f;
         for (int i = 0; i < NW * RPW; i++)
             if (sm[i] > -INFINITY) v += sacc[i][d] * __expf(sm[i] - M);
-        out[2 + d] = v;
+        part_store(out + 2 + d, v);
     }
+}
+
+// The workgroup that takes the last ticket of a (batch, head) merges all split partials (splits <= 256,
+// 256 threads).  Every wavefront waits for its own partial stores to be acknowledged before the barrier
+// that precedes the ticket, so a workgroup that sees ticket == splits - 1 can read every partial.
+template <typename T>
+__device__ __forceinline__ void decode_merge_last(const float* part, int* counter, int splits, int hs, T* __restrict__ y)
+{
+    __shared__ int ticket;
+    __shared__ float sw[256];
+    __shared__ float sred[256];
+    __shared__ float swv[8];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != splits - 1) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int stride = hs + 2;
+    float ms = -INFINITY, ls = 0.f;
+    if (tid < splits) {
+        ms = part_load(part + (size_t)tid * stride);
+        ls = part_load(part + (size_t)tid * stride + 1);
+    }
+    float M = ms;
+    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+    if (lane == 0) swv[wave] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(swv[0], swv[1]), fmaxf(swv[2], swv[3]));
+    const float w = ms > -INFINITY ? __expf(ms - M) : 0.f;
+    sw[tid] = w;
+    float L = ls * w;
+    for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+    if (lane == 0) swv[4 + wave] = L;
+    __syncthreads();
+    L = (swv[4] + swv[5]) + (swv[6] + swv[7]);
+    // G groups of hs threads; group g sums splits g, g + G, ...
+    const int G = hs >= 256 ? 1 : 256 / hs;
+    const int g = tid / hs;
+    if (G == 1) {
+        if (g == 0 || hs > 256)
+            for (int d = tid; d < hs; d += 256) {
+                float v = 0.f;
+                for (int s = 0; s < splits; s++) v += part_load(part + (size_t)s * stride + 2 + d) * sw[s];
+                st1(y + d, v / L);
+            }
+    } else {
+        const int d = tid - g * hs;
+        float v = 0.f;
+        if (g < G)
+            for (int s = g; s < splits; s += G) v += part_load(part + (size_t)s * stride + 2 + d) * sw[s];
+        sred[tid] = v;
+        __syncthreads();
+        if (g == 0) {
+            for (int k = 1; k < G; k++) v += sred[k * hs + d];
+            st1(y + d, v / L);
+        }
+    }
+    if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+}
+
+// partial layout: part[((b*H + h)*splits + s) * (hs + 2)] = {m, l, acc[hs]}
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
+{
+    constexpr int W = Vec16<T>::W;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int grp = lane / LPR, gl = lane % LPR;
+    const int d0 = gl * W;
+    const bool active = d0 < a.hs;  // lanes beyond hs idle when hs/W is not a power of two
+
+    const T* q = (const T*)a.q + ((size_t)b * a.H + h) * a.hs;
+    const size_t base = (size_t)b * a.strideB + (size_t)(h / a.kvMul) * a.strideH;
+    const T* kc = (const T*)a.kc + base;
+    const T* vc = (const T*)a.vc + base;
+
+    float qv[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) qv[i] = 0.f;
+    if (active) {
+        Vec16<T>::load(q + d0, qv);
+#pragma unroll
+        for (int i = 0; i < W; i++) qv[i] *= a.scale;
+    }
+
+    int t0, t1;
+    decode_range(a, split, &t0, &t1);
+
+    float m = -INFINITY, l = 0.f, acc[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) acc[i] = 0.f;
+    decode_stream<T, LPR>(kc, vc, a.strideT, t0, t1, wave, grp, d0, active, qv, m, l, acc);
+
+    const size_t bh = (size_t)b * a.H + h;
+    float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+    decode_reduce_wg<T, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+    if (a.counters)
+        decode_merge_last<T>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, a.splits, a.hs, (T*)a.y + bh * a.hs);
+}
+
+// Engine form (fp32): one launch per layer does what the reference's decode step does between the QKV
+// mat-vecs and the output projection (llama2_cpu.cpp:288-341): rotate q and k at the current position,
+// store k and v into the cache, attend over positions 0..pos, write the head outputs.  qkv holds one
+// row [q | k | v] of dim + 2*kvd raw projections per sequence; caches are [B][seqLen][kvd].
+struct FusedDecodeArgs {
+    const float* qkv; float* kc; float* vc; float* y; float* part; int* counters;
+    const float* fcos; const float* fsin; const int* dlen;
+    int B, H, kvMul, hs, dim, kvd, seqLen, splits, rowsPerIter;
+    float scale;
+};
+
+template <int LPR>
+__global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs a)
+{
+    constexpr int W = 4;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int grp = lane / LPR, gl = lane % LPR;
+    const int d0 = gl * W;
+    const bool active = d0 < a.hs;
+    const int len = *a.dlen, pos = len - 1;
+    const int half = a.hs / 2;
+    const int kvh = h / a.kvMul;
+    const int ldq = a.dim + 2 * a.kvd;
+    const float* row = a.qkv + (size_t)b * ldq;
+    float* kc = a.kc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    float* vc = a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+
+    int chunk = (len + a.splits - 1) / a.splits;
+    chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
+    const int t0 = split * chunk, t1 = min(len, t0 + chunk);
+
+    // rotation factors of this lane's two adjacent pairs (dims d0, d0+1 and d0+2, d0+3) at `pos`
+    float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
+    if (active) {
+        const size_t ti = (size_t)pos * half + d0 / 2;
+        c0 = a.fcos[ti]; s0 = a.fsin[ti]; c1 = a.fcos[ti + 1]; s1 = a.fsin[ti + 1];
+    }
+    float qv[W] = {0.f, 0.f, 0.f, 0.f};
+    if (active) {
+        const float4 r = *(const float4*)(row + (size_t)h * a.hs + d0);
+        qv[0] = (r.x * c0 - r.y * s0) * a.scale;
+        qv[1] = (r.x * s0 + r.y * c0) * a.scale;
+        qv[2] = (r.z * c1 - r.w * s1) * a.scale;
+        qv[3] = (r.z * s1 + r.w * c1) * a.scale;
+    }
+    // the split that owns the current position appends the rotated key and the value first
+    if (t0 <= pos && pos < t1) {
+        if (wave == 0 && grp == 0 && active) {
+            const float4 kr = *(const float4*)(row + a.dim + (size_t)kvh * a.hs + d0);
+            const float4 vr = *(const float4*)(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0);
+            float4 ko;
+            ko.x = kr.x * c0 - kr.y * s0; ko.y = kr.x * s0 + kr.y * c0;
+            ko.z = kr.z * c1 - kr.w * s1; ko.w = kr.z * s1 + kr.w * c1;
+            *(float4*)(kc + (size_t)pos * a.kvd + d0) = ko;
+            *(float4*)(vc + (size_t)pos * a.kvd + d0) = vr;
+        }
+        __syncthreads();   // the row is read back by this workgroup only (other heads of the group write their own copy)
+    }
+    float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
+    decode_stream<float, LPR>(kc, vc, a.kvd, t0, t1, wave, grp, d0, active, qv, m, l, acc);
+    const size_t bh = (size_t)b * a.H + h;
+    float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+    decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, a.splits, a.hs,
+                             a.y + (size_t)b * a.dim + (size_t)h * a.hs);
 }
 
 // any head size / alignment: scalar loads, one wavefront per (b, h, split)
@@ -302,6 +459,7 @@ static hipError_t launch_decode(hipStream_t s, DecodeArgs a, int kvH)
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if (fast && a.counters) return hipSuccess;   // the last workgroup of every (batch, head) merged in-kernel
     int mt = a.hs <= 64 ? 64 : (a.hs <= 128 ? 128 : 256);
     hipLaunchKernelGGL(attn_decode_merge_kernel<T>, a.B * a.H, mt, 0, s, a.part, (T*)a.y, a.hs, a.splits);
     return hipGetLastError();
@@ -309,7 +467,7 @@ static hipError_t launch_decode(hipStream_t s, DecodeArgs a, int kvH)
 
 hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc, const void* vc, void* y, int B, int H,
                          int kvH, int hs, int len, long long strideB, long long strideH, long long strideT, float scale,
-                         void* workspace, size_t workspaceBytes, const int* dlen)
+                         void* workspace, size_t workspaceBytes, const int* dlen, int* counters)
 {
     if (B <= 0 || H <= 0 || hs <= 0 || len <= 0) return hipSuccess;
     if (kvH <= 0 || H % kvH != 0) return hipErrorInvalidValue;
@@ -319,9 +477,36 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
     a.q = q; a.kc = kc; a.vc = vc; a.y = y; a.part = (float*)workspace;
     a.B = B; a.H = H; a.kvMul = H / kvH; a.hs = hs; a.len = len; a.splits = 1; a.chunk = len;
     a.strideB = strideB; a.strideH = strideH; a.strideT = strideT; a.scale = scale;
-    a.dlen = dlen; a.rowsPerIter = 64;
+    a.dlen = dlen; a.rowsPerIter = 64; a.counters = counters;
     if (dt == F32) return launch_decode<float>(s, a, kvH);
     return launch_decode<bf16_t>(s, a, kvH);
+}
+
+hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float* vc, float* y, int B, int H, int kvH, int hs,
+                               int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
+                               size_t workspaceBytes, int* counters)
+{
+    if (B <= 0 || H <= 0 || hs <= 0 || seqLen <= 0) return hipSuccess;
+    if (kvH <= 0 || H % kvH != 0 || (hs % 4) != 0 || B > 65535 || H > 65535 || !counters || !dlen) return hipErrorInvalidValue;
+    int lpr = hs / 4, lprp = 1;
+    while (lprp < lpr) lprp <<= 1;
+    if (lprp > 64) return hipErrorInvalidValue;
+    if (workspaceBytes < attn_decode_workspace_bytes(B, H, hs, seqLen)) return hipErrorInvalidValue;
+    FusedDecodeArgs a;
+    a.qkv = qkv; a.kc = kc; a.vc = vc; a.y = y; a.part = (float*)workspace; a.counters = counters;
+    a.fcos = fcos; a.fsin = fsin; a.dlen = dlen;
+    a.B = B; a.H = H; a.kvMul = H / kvH; a.hs = hs; a.dim = H * hs; a.kvd = kvH * hs; a.seqLen = seqLen;
+    a.rowsPerIter = 4 * (64 / lprp) * 4;
+    int chunk;
+    pick_splits(B, H, seqLen, a.rowsPerIter, &a.splits, &chunk);
+    a.scale = scale;
+    dim3 grid(a.splits, H, B);
+    switch (lprp) {
+#define CASE(L) case L: hipLaunchKernelGGL((attn_decode_fused_kernel<L>), grid, 256, 0, s, a); break;
+        CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
+#undef CASE
+    }
+    return hipGetLastError();
 }
 
 // rotate q and the new key at `pos` (adjacent-pair convention) and store the new

@@ -75,7 +75,6 @@ enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAU
 //   MASK_CAUSAL needs no mask buffer (lower triangle kept).
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
                           int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind);
-// returns true if mask (Tq,Tk) on the device equals the lower-triangular ones matrix; cached by the caller
 size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
 // one query per (b,h): q (B,H,hs), caches addressed as
 //   cache[b*strideB + (h/kvMul)*strideH + t*strideT + i], y (B,H,hs).  All dt.
@@ -83,7 +82,17 @@ size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
 // actual number of cached positions is read from *dlen on the device.
 hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc, const void* vc, void* y, int B, int H,
                          int kvH, int hs, int len, long long strideB, long long strideH, long long strideT,
-                         float scale, void* workspace, size_t workspaceBytes, const int* dlen = nullptr);
+                         float scale, void* workspace, size_t workspaceBytes, const int* dlen = nullptr,
+                         int* counters = nullptr);
+// `counters`: B*H zero-initialised ints that stay zero between launches; when given, the last
+// workgroup of every (batch, head) merges the split partials inside the kernel (no second launch).
+//
+// fp32 decode step of the llama2 engine in one launch: rotate q / k at position *dlen - 1, append k, v
+// to the caches ([B][seqLen][kvH*hs]), attend over positions 0 .. *dlen - 1.  qkv: [B][(H + 2 kvH) hs]
+// raw projections, y: [B][H*hs].
+hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float* vc, float* y, int B, int H, int kvH, int hs,
+                               int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
+                               size_t workspaceBytes, int* counters);
 // rotate q (B,H,hs) and knew (B,kvH,hs) at position pos and append knew/vnew to the caches at pos
 hipError_t k_rope_append(hipStream_t s, DType dt, void* q, void* knew, const void* vnew, void* kc, void* vc, int B,
                          int H, int kvH, int hs, int pos, long long strideB, long long strideH, long long strideT,

@@ -166,6 +166,7 @@ Kernel::~Kernel()
     m_rope.clear();
     m_mem.free_all();
     if (m_ws) (void)hipFree(m_ws);
+    if (m_tickets) (void)hipFree(m_tickets);
     if (m_stage) (void)hipHostFree(m_stage);
     for (float* p : m_hostAllocs) (void)hipHostFree(p);
     if (m_stream) (void)hipStreamDestroy(m_stream);
@@ -205,6 +206,19 @@ long Kernel::workspace(size_t bytes, void** p)
         m_wsBytes = want;
     }
     *p = m_ws;
+    return 0;
+}
+
+long Kernel::tickets(size_t count, int** p)
+{
+    if (count > m_ticketCount) {
+        if (m_tickets) { HIPCHK(hipStreamSynchronize(m_stream)); HIPCHK(hipFree(m_tickets)); m_tickets = nullptr; m_ticketCount = 0; }
+        size_t want = count < 4096 ? 4096 : count * 2;
+        HIPCHK(hipMalloc((void**)&m_tickets, want * sizeof(int)));
+        HIPCHK(hipMemsetAsync(m_tickets, 0, want * sizeof(int), m_stream));
+        m_ticketCount = want;
+    }
+    *p = m_tickets;
     return 0;
 }
 
@@ -997,8 +1011,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         size_t wsb = attn_decode_workspace_bytes((int)B, (int)H, (int)hs, (int)len);
         void* ws;
         ERRCHK(workspace(wsb, &ws));
+        int* tk;
+        ERRCHK(tickets((size_t)(B * H), &tk));
         HIPCHK(k_attn_decode(s, Q->dt(), Q->ptr, KC->ptr, VC->ptr, Y->ptr, (int)B, (int)H, (int)KVH, (int)hs, (int)len, sB, sH,
-                             sT, scale, ws, m_wsBytes));
+                             sT, scale, ws, m_wsBytes, nullptr, tk));
         m_mem.touch((long)pl[8]);
         return 0;
     }

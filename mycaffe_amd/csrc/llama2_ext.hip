@@ -27,6 +27,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <algorithm>
 #include <vector>
 
 #include "../../include/mycaffe_hip_abi.h"
@@ -69,12 +70,6 @@ __global__ void embed_step_kernel(const GenState* st, const int* prompt, int pro
     for (int i = threadIdx.x; i < dim; i += blockDim.x) x[(size_t)b * dim + i] = wld(emb, (size_t)tok * dim + i);
 }
 
-__global__ void advance_kernel(GenState* st)
-{
-    st->pos += 1;
-    st->len = st->pos + 1;
-}
-
 // 4 weight values of one row against 4 activations
 template <typename T> struct Row4;
 template <> struct Row4<float> {
@@ -98,12 +93,11 @@ template <> struct Row4<bf16_t> {
 //   MODE 2: y[b,r]  = silu(W[r,:] . xn) * (W[r+half,:] . xn)   (SwiGLU epilogue, half = rows)
 // NORM: xn = g * x / sqrt(mean(x^2) + 1e-5), recomputed per wavefront from the
 // chunks it already holds (x is L2 resident; it saves a launch and a barrier).
-template <typename T, int MODE, bool NORM, int CH>
+template <typename T, int MODE, bool NORM, int CH, int ROWS>
 __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, const float* __restrict__ x,
                                                      const float* __restrict__ g, float* __restrict__ y, int rows, int n,
                                                      int B, int ldy)
 {
-    constexpr int ROWS = 2;
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int r0 = wave * ROWS;
@@ -173,53 +167,46 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
     }
 }
 
-// rotate q and k at the device-side position, store k, v into the caches (rope + cache
-// write of llama2_cpu.cpp:288-296) and compact the rotated q into qc (B, dim);
-// qkv holds one row [q | k | v] of dim + 2*kvd floats per sequence
-__global__ void rope_store_kernel(const GenState* st, const float* qkv, float* qc, float* kc, float* vc, const float* fcos,
-                                  const float* fsin, int B, int dim, int kvd, int hs, int seqLen)
-{
-    const int pos = st->pos;
-    const int half = hs / 2;
-    const int ld = dim + 2 * kvd;
-    const int nq = dim / 2, nk = kvd / 2;
-    const int per = nq + nk + kvd;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < B * per; i += blockDim.x * gridDim.x) {
-        const int b = i / per, e = i % per;
-        const float* row = qkv + (size_t)b * ld;
-        const size_t coff = ((size_t)b * seqLen + pos) * kvd;
-        if (e < nq + nk) {
-            const bool isq = e < nq;
-            const int p = isq ? e : e - nq;
-            const float* v = (isq ? row : row + dim) + 2 * p;
-            const int j = p % half;
-            const float c = fcos[(size_t)pos * half + j], sn = fsin[(size_t)pos * half + j];
-            const float re = v[0], im = v[1];
-            const float r0 = re * c - im * sn, r1 = re * sn + im * c;
-            float* dst = isq ? qc + (size_t)b * dim + 2 * p : kc + coff + 2 * p;
-            dst[0] = r0;
-            dst[1] = r1;
-        } else {
-            const int d = e - nq - nk;
-            vc[coff + d] = row[dim + kvd + d];
-        }
-    }
-}
-
-// first-max argmax over the logits of each sequence (sample_argmax, llama2_sampler.cpp:25-36:
-// strict '>' so the lowest index wins ties), then record and feed back
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* logits, int V, const GenState* st, int* next, int* out_ids,
-                                                       int outStride)
+// End of a decode step, one workgroup per sequence: first-max argmax over the logits
+// (sample_argmax, llama2_sampler.cpp:25-36: strict '>' so the lowest index wins ties), record
+// the id, embed the token of the next position (forced prompt id while pos + 1 < n_prompt,
+// generate loop llm.cpp:208-228) and, in the workgroup that takes the last ticket, advance the
+// position.  Every workgroup reads the position before it takes its ticket.
+template <typename T>
+__global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __restrict__ logits, int V, GenState* st, int* ticket,
+                                                               const int* __restrict__ prompt, int promptStride, int* next,
+                                                               int* out_ids, const T* __restrict__ emb, float* __restrict__ x,
+                                                               int dim, int* cur)
 {
     __shared__ float sv[16];
     __shared__ int si[16];
+    __shared__ int stok;
     const int b = blockIdx.x;
+    const int pos = st->pos, nPrompt = st->n_prompt;
     const float* lg = logits + (size_t)b * V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        float v = lg[i];
+    auto take = [&](float v, int i) {
         if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    };
+    if ((V & 3) == 0) {
+        const int n4 = V >> 2;
+        constexpr int U = 8;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += 1024 * U) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = i0 + u * 1024;
+                v[u] = i < n4 ? *(const float4*)(lg + (size_t)i * 4) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = (i0 + u * 1024) * 4;
+                take(v[u].x, i); take(v[u].y, i + 1); take(v[u].z, i + 2); take(v[u].w, i + 3);
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += 1024) take(lg[i], i);
     }
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64);
@@ -230,11 +217,25 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* logits, int V
     if ((threadIdx.x & 63) == 0) { sv[w] = bv; si[w] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < (int)(blockDim.x >> 6); i++)
+        for (int i = 1; i < 16; i++)
             if (sv[i] > bv || (sv[i] == bv && si[i] < bi)) { bv = sv[i]; bi = si[i]; }
         if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0, as a scan that never finds a larger value would give
         next[b] = bi;
-        out_ids[(size_t)b * outStride + st->pos] = bi;
+        out_ids[(size_t)b * promptStride + pos] = bi;
+        const int np = pos + 1;
+        const int tok = (np < nPrompt && np < promptStride) ? prompt[(size_t)b * promptStride + np] : bi;
+        cur[b] = tok;
+        stok = tok;
+    }
+    __syncthreads();
+    const int tok = stok;
+    for (int i = threadIdx.x; i < dim; i += 1024) x[(size_t)b * dim + i] = wld(emb, (size_t)tok * dim + i);
+    if (threadIdx.x == 0) {
+        if (atomicAdd(ticket, 1) == (int)gridDim.x - 1) {
+            *ticket = 0;
+            st->pos = pos + 1;
+            st->len = pos + 2;
+        }
     }
 }
 
@@ -271,6 +272,8 @@ public:
     bool loaded = false;
     bool bf16_weights = false;
     bool use_graph = true;
+    int mvRows = 0;              // weight rows per wavefront in the mat-vec kernels (0: chosen per shape)
+    void set_mv_rows(int r) { mvRows = r; graphB = -1; }   // the captured step is rebuilt at the next generation
     int shared_classifier = 0;
     int timedFrom = -1;          // first step of the timed span (-1: first step after the prompt)
     float lastTimedMs = 0.f;     // HIP-event duration of the timed span of the last generate
@@ -287,6 +290,7 @@ private:
     template <typename T> long upload(const float* blob);
     template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr);
     long ensure_state(int B, int nSteps);
+    hipError_t embed_first(hipStream_t s, int B);
 
     hipStream_t stream = nullptr;
     std::vector<void*> allocs;
@@ -308,6 +312,7 @@ private:
     void* ws = nullptr; size_t wsBytes = 0;
     GenState* dstate = nullptr;
     int *dprompt = nullptr, *dnext = nullptr, *dcur = nullptr, *dout = nullptr;
+    int *dcount = nullptr, *dticket = nullptr;   // attention merge tickets (B * heads) and the step ticket; zero between launches
     hipGraphExec_t graphExec = nullptr;
     int graphB = 0;
 };
@@ -479,8 +484,11 @@ long Engine::ensure_state(int B, int nSteps)
     dnext = (int*)sa(B * 4);
     dcur = (int*)sa(B * 4);
     dout = (int*)sa((size_t)B * cfg.seq_len * 4);
-    if (!x || !xb || !qkv || !qc || !hb || !logits || !kc || !vc || !ws || !dstate || !dprompt || !dnext || !dcur || !dout)
+    dcount = (int*)sa(((size_t)B * cfg.n_heads + 1) * 4);
+    if (!x || !xb || !qkv || !qc || !hb || !logits || !kc || !vc || !ws || !dstate || !dprompt || !dnext || !dcur || !dout || !dcount)
         return MCH_ERROR_MEMORY_OUT;
+    dticket = dcount + (size_t)B * cfg.n_heads;
+    HIPCHK(hipMemset(dcount, 0, ((size_t)B * cfg.n_heads + 1) * 4));
     stateB = B;
     stateSteps = cfg.seq_len;
     return 0;
@@ -488,12 +496,18 @@ long Engine::ensure_state(int B, int nSteps)
 
 template <int MODE, bool NORM, typename T>
 static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int B,
-                                int ldy)
+                                int ldy, int rowsPerWave)
 {
-    const int waves = (rows + 1) / 2;
+    // one row per wavefront fills the chip for the layer matrices; the classifier has rows to spare
+    const bool two = rowsPerWave ? rowsPerWave == 2 : rows >= 16384;
+    const int waves = two ? (rows + 1) / 2 : rows;
     const int grid = (waves + 3) / 4;
     const int ch = (n / 4 + 63) / 64;
-#define MV(C) hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy)
+#define MV(C)                                                                                                              \
+    do {                                                                                                                   \
+        if (two) hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 2>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy); \
+        else hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 1>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy);     \
+    } while (0)
     if (ch <= 2) MV(2);
     else if (ch <= 3) MV(3);
     else if (ch <= 4) MV(4);
@@ -504,6 +518,16 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     return hipGetLastError();
 }
 
+// x = embedding of the token at the starting position; later steps get theirs from the previous step's tail kernel
+hipError_t Engine::embed_first(hipStream_t s, int B)
+{
+    if (bf16_weights)
+        hipLaunchKernelGGL(embed_step_kernel<bf16_t>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const bf16_t*)emb, x, cfg.dim, dcur);
+    else
+        hipLaunchKernelGGL(embed_step_kernel<float>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const float*)emb, x, cfg.dim, dcur);
+    return hipGetLastError();
+}
+
 // enqueue one decode step for B sequences at the device-side position
 template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof)
 {
@@ -511,10 +535,6 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
     const int ldq = dim + 2 * kvd;
 #define SPAN_BEGIN(cls) do { if (prof) HIPCHK(prof->begin(cls, s)); } while (0)
 #define SPAN_END() do { if (prof) HIPCHK(prof->end(s)); } while (0)
-    SPAN_BEGIN(SC_SAMPLE);
-    hipLaunchKernelGGL(embed_step_kernel<T>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const T*)emb, x, dim, dcur);
-    HIPCHK(hipGetLastError());
-    SPAN_END();
     const float scale = 1.0f / sqrtf((float)hs);
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
@@ -522,37 +542,29 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
         float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
         // qkv = [Wq;Wk;Wv] rmsnorm(x)
         SPAN_BEGIN(SC_MATVEC_QKV);
-        HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq)));
+        HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq, mvRows)));
         SPAN_END();
-        SPAN_BEGIN(SC_ROPE_STORE);
-        {
-            const int n = B * (dim / 2 + kvd / 2 + kvd);
-            hipLaunchKernelGGL(rope_store_kernel, (n + 255) / 256, 256, 0, s, dstate, qkv, qc, kcl, vcl, fcos, fsin, B, dim, kvd, hs,
-                               cfg.seq_len);
-            HIPCHK(hipGetLastError());
-        }
-        SPAN_END();
-        // xb = attention(q, cache[0..pos])
+        // xb = attention(rope(q), cache[0..pos] with rope(k), v appended)
         SPAN_BEGIN(SC_ATTN_DECODE);
-        HIPCHK(k_attn_decode(s, F32, qc, kcl, vcl, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len,
-                             (long long)cfg.seq_len * kvd, hs, kvd, scale, ws, wsBytes, &dstate->len));
+        HIPCHK(k_attn_decode_fused(s, qkv, kcl, vcl, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len, scale, fcos, fsin,
+                                   &dstate->len, ws, wsBytes, dcount));
         SPAN_END();
         // x += Wo xb
         SPAN_BEGIN(SC_MATVEC_WO);
-        HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim)));
+        HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim, mvRows)));
         SPAN_END();
         // hb = silu(W1 rmsnorm(x)) * (W3 rmsnorm(x))
         SPAN_BEGIN(SC_MATVEC_W13);
-        HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid)));
+        HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid, mvRows)));
         SPAN_END();
         // x += W2 hb
         SPAN_BEGIN(SC_MATVEC_W2);
-        HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim)));
+        HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim, mvRows)));
         SPAN_END();
     }
     // logits = Wcls rmsnorm(x)
     SPAN_BEGIN(SC_MATVEC_CLS);
-    HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V)));
+    HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V, mvRows)));
     SPAN_END();
     if (allLogits) {
         hipLaunchKernelGGL(save_logits_kernel, dim3((V + 255) / 256 > 64 ? 64 : (V + 255) / 256, B), 256, 0, s, logits, allLogits,
@@ -560,9 +572,8 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
         HIPCHK(hipGetLastError());
     }
     SPAN_BEGIN(SC_SAMPLE);
-    hipLaunchKernelGGL(argmax_kernel, B, 1024, 0, s, logits, V, dstate, dnext, dout, cfg.seq_len);
-    HIPCHK(hipGetLastError());
-    hipLaunchKernelGGL(advance_kernel, 1, 1, 0, s, dstate);
+    hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
+                       (const T*)emb, x, dim, dcur);
     HIPCHK(hipGetLastError());
     SPAN_END();
 #undef SPAN_BEGIN
@@ -570,9 +581,13 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
     return 0;
 }
 
+__global__ void noop_kernel() {}
+
 // Runs `reps` eager decode steps of one sequence starting at position `pos` (the cache
 // content before `pos` is whatever earlier generations left; only timing matters here) and
-// returns, per kernel class: {milliseconds per step, launches per step, algorithmic bytes per step}.
+// returns, per kernel class: {milliseconds per step, launches per step, algorithmic bytes per step}, followed by one
+// more value: the median milliseconds an event pair measures around an empty kernel (dispatch + event cost that
+// every pair above includes).
 long Engine::profile_step(int pos, int reps, std::vector<float>* out)
 {
     if (!loaded) return MCH_ERROR_LLM_GENERATE;
@@ -585,6 +600,24 @@ long Engine::profile_step(int pos, int reps, std::vector<float>* out)
     GenState st0 = {pos, cfg.seq_len, pos + 1, 0};
     HIPCHK(hipMemcpyAsync(dstate, &st0, sizeof(st0), hipMemcpyHostToDevice, s));
     HIPCHK(hipStreamSynchronize(s));
+    HIPCHK(embed_first(s, 1));
+    std::vector<float> empty;
+    {
+        StepProfile cal;
+        for (int i = 0; i < 33; i++) {
+            HIPCHK(cal.begin(0, s));
+            hipLaunchKernelGGL(noop_kernel, 1, 64, 0, s);
+            HIPCHK(cal.end(s));
+        }
+        HIPCHK(hipStreamSynchronize(s));
+        for (auto& sp : cal.spans) {
+            float t = 0.f;
+            if (hipEventElapsedTime(&t, sp.second.first, sp.second.second) == hipSuccess) empty.push_back(t);
+            (void)hipEventDestroy(sp.second.first);
+            (void)hipEventDestroy(sp.second.second);
+        }
+        std::sort(empty.begin(), empty.end());
+    }
     StepProfile prof;
     for (int i = 0; i < reps && !e; i++) e = bf16_weights ? step<bf16_t>(s, 1, cfg.seq_len, nullptr, &prof) : step<float>(s, 1, cfg.seq_len, nullptr, &prof);
     hipError_t he = hipStreamSynchronize(s);
@@ -613,6 +646,7 @@ long Engine::profile_step(int pos, int reps, std::vector<float>* out)
         out->push_back((float)(cnt[c] / reps));
         out->push_back((float)bytes[c]);
     }
+    out->push_back(empty.empty() ? 0.f : empty[empty.size() / 2]);
     return 0;
 }
 
@@ -658,6 +692,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         if (e || he != hipSuccess || !graphExec) { graphExec = nullptr; graph = false; e = 0; }
         graphB = B;
     }
+    HIPCHK(embed_first(s, B));
     int done = 0;
     for (int i = 0; i < nSteps && !e; i++) {
         if (i == t0) (void)hipEventRecord(evA, s);
@@ -827,6 +862,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         if (opt == 1) m->engine.bf16_weights = pIn[2] != 0.f;
         else if (opt == 2) m->engine.timedFrom = (int)pIn[2];
         else if (opt == 3) m->engine.use_graph = pIn[2] != 0.f;
+        else if (opt == 4) m->engine.set_mv_rows(pIn[2] == 1.f ? 1 : (pIn[2] == 2.f ? 2 : 0));
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }

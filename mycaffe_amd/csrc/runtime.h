@@ -112,6 +112,7 @@ public:
 private:
     long workspace(size_t bytes, void** p);
     long staging(size_t bytes, void** p);
+    long tickets(size_t count, int** p);
     long mem(long h, MemItem** it) { return m_mem.get(h, it); }
     bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
 
@@ -125,6 +126,7 @@ private:
     HandleTable<ExtensionState> m_ext;
     std::map<int, std::weak_ptr<void>> m_ropeSharedCos, m_ropeSharedSin;
     void* m_ws = nullptr; size_t m_wsBytes = 0;          // device scratch (split-K partials, conversions)
+    int* m_tickets = nullptr; size_t m_ticketCount = 0;  // split-K merge tickets; zero whenever no kernel is running
     void* m_stage = nullptr; size_t m_stageBytes = 0;    // pinned host staging
     std::mutex m_stageLock;
     std::vector<float*> m_hostAllocs;

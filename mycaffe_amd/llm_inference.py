@@ -101,6 +101,9 @@ class LlmInference:
 
     def ProfileStep(self, pos, reps=8):
         """Per-kernel-class timing of eager decode steps at ``pos`` (HIP event pairs around
-        every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}."""
+        every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}, plus
+        "_event_pair_ms": what such a pair measures around an empty kernel."""
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.PROFILE_STEP, self.m_rgLlm + [pos, reps])
-        return {name: (float(rg[3 * i]), float(rg[3 * i + 1]), float(rg[3 * i + 2])) for i, name in enumerate(STEP_CLASSES)}
+        out = {name: (float(rg[3 * i]), float(rg[3 * i + 1]), float(rg[3 * i + 2])) for i, name in enumerate(STEP_CLASSES)}
+        out["_event_pair_ms"] = float(rg[3 * len(STEP_CLASSES)])
+        return out
