@@ -13,6 +13,9 @@
 
 namespace mch {
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes of a cache row: W elements
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
     static constexpr int W = 4;
@@ -20,6 +23,11 @@ template <> struct Vec16<float> {
     {
         float4 v = *(const float4*)p;
         out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    }
+    __device__ static inline void unpack(u32x4 r, float* out)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = __uint_as_float(r[i]);
     }
 };
 template <> struct Vec16<bf16_t> {
@@ -32,6 +40,14 @@ template <> struct Vec16<bf16_t> {
         for (int i = 0; i < 4; i++) {
             out[2 * i] = __uint_as_float(u[i] << 16);
             out[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+        }
+    }
+    __device__ static inline void unpack(u32x4 r, float* out)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            out[2 * i] = __uint_as_float(r[i] << 16);
+            out[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
         }
     }
 };
@@ -69,58 +85,98 @@ __device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int
 
 // Streams cache rows [t0, t1) for one (batch, head): every lane group of LPR lanes keeps its own
 // running max m, sum l and output slice acc[W] (dims gl*W ..).  qv holds the query slice, pre-scaled.
-template <typename T, int LPR>
-__device__ __forceinline__ void decode_stream(const T* __restrict__ kc, const T* __restrict__ vc, long long strideT, int t0, int t1,
-                                              int wave, int grp, int d0, bool active, const float (&qv)[Vec16<T>::W], float& m,
-                                              float& l, float (&acc)[Vec16<T>::W])
+// A stage is U row groups of K and of V per wavefront, kept as loaded (16 bytes per lane and row);
+// the loads of the next stage are issued before the current one is consumed.
+template <int U> struct DecodeStage { u32x4 k[U], v[U]; };
+
+template <typename T, int LPR, int U>
+__device__ __forceinline__ void decode_issue(DecodeStage<U>& st, const T* __restrict__ kc, const T* __restrict__ vc, long long strideT,
+                                             int tb, int t1, int grp, int d0, bool active)
+{
+    constexpr int RPW = 64 / LPR;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = tb + u * RPW + grp;
+        u32x4 z = {0u, 0u, 0u, 0u};
+        st.k[u] = z;
+        if (t < t1 && active) st.k[u] = *(const u32x4*)(kc + (size_t)t * strideT + d0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int t = tb + u * RPW + grp;
+        u32x4 z = {0u, 0u, 0u, 0u};
+        st.v[u] = z;
+        if (t < t1 && active) st.v[u] = *(const u32x4*)(vc + (size_t)t * strideT + d0);
+    }
+}
+
+template <typename T, int LPR, int U>
+__device__ __forceinline__ void decode_consume(const DecodeStage<U>& st, int tb, int t1, int grp, const float (&qv)[Vec16<T>::W],
+                                               float& m, float& l, float (&acc)[Vec16<T>::W])
 {
     constexpr int W = Vec16<T>::W;
+    constexpr int RPW = 64 / LPR;
+    float s[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float kv[W];
+        Vec16<T>::unpack(st.k[u], kv);
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < W; i++) d += qv[i] * kv[i];
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        s[u] = (tb + u * RPW + grp) < t1 ? d : -INFINITY;
+    }
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < U; u++) mn = fmaxf(mn, s[u]);
+    if (mn > -INFINITY) {
+        const float corr = __expf(m - mn);  // m == -inf gives 0
+        l *= corr;
+#pragma unroll
+        for (int i = 0; i < W; i++) acc[i] *= corr;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float p = __expf(s[u] - mn);  // masked rows: exp(-inf) = 0
+            l += p;
+            float vv[W];
+            Vec16<T>::unpack(st.v[u], vv);
+#pragma unroll
+            for (int i = 0; i < W; i++) acc[i] += p * vv[i];
+        }
+        m = mn;
+    }
+}
+
+template <typename T, int LPR>
+__device__ __forceinline__ void decode_stream(const T* __restrict__ kc, const T* __restrict__ vc, long long strideT, int t0, int t1,
+                                              unsigned rot, int wave, int grp, int d0, bool active,
+                                              const float (&qv)[Vec16<T>::W], float& m, float& l, float (&acc)[Vec16<T>::W])
+{
     constexpr int RPW = 64 / LPR;  // rows per wavefront load
-    constexpr int U = 4;           // row groups in flight per operand
+    constexpr int U = 4;           // row groups per stage and operand
     constexpr int NW = 4;
-    for (int tb = t0 + wave * RPW * U; tb < t1; tb += NW * RPW * U) {
-        float kv[U][W], vv[U][W];
-        bool ok[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int t = tb + u * RPW + grp;
-            ok[u] = t < t1;
-#pragma unroll
-            for (int i = 0; i < W; i++) { kv[u][i] = 0.f; vv[u][i] = 0.f; }
-            if (ok[u] && active) Vec16<T>::load(kc + (size_t)t * strideT + d0, kv[u]);
+    constexpr int STEP = NW * RPW * U;
+    // The online softmax does not care about row order, so every workgroup starts at its own rotation of the
+    // range instead of all of them walking their caches in lockstep.
+    const int nIt = (t1 - t0 + STEP - 1) / STEP;
+    if (nIt <= 0) return;
+    int j = (int)(rot % (unsigned)nIt);
+    auto next = [&](int x) { return x + 1 == nIt ? 0 : x + 1; };
+    const int w0 = t0 + wave * RPW * U;
+    DecodeStage<U> A, B;
+    decode_issue<T, LPR, U>(A, kc, vc, strideT, w0 + j * STEP, t1, grp, d0, active);
+    for (int it = 0; it < nIt; it += 2) {
+        const int j1 = next(j), j2 = next(j1);
+        const bool has1 = it + 1 < nIt, has2 = it + 2 < nIt;
+        if (has1) decode_issue<T, LPR, U>(B, kc, vc, strideT, w0 + j1 * STEP, t1, grp, d0, active);
+        decode_consume<T, LPR, U>(A, w0 + j * STEP, t1, grp, qv, m, l, acc);
+        if (has1) {
+            if (has2) decode_issue<T, LPR, U>(A, kc, vc, strideT, w0 + j2 * STEP, t1, grp, d0, active);
+            decode_consume<T, LPR, U>(B, w0 + j1 * STEP, t1, grp, qv, m, l, acc);
         }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int t = tb + u * RPW + grp;
-            if (ok[u] && active) Vec16<T>::load(vc + (size_t)t * strideT + d0, vv[u]);
-        }
-        float s[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            float d = 0.f;
-#pragma unroll
-            for (int i = 0; i < W; i++) d += qv[i] * kv[u][i];
-#pragma unroll
-            for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-            s[u] = ok[u] ? d : -INFINITY;
-        }
-        float mn = m;
-#pragma unroll
-        for (int u = 0; u < U; u++) mn = fmaxf(mn, s[u]);
-        if (mn > -INFINITY) {
-            float corr = __expf(m - mn);  // m == -inf gives 0
-            l *= corr;
-#pragma unroll
-            for (int i = 0; i < W; i++) acc[i] *= corr;
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                float p = __expf(s[u] - mn);  // masked rows: exp(-inf) = 0
-                l += p;
-#pragma unroll
-                for (int i = 0; i < W; i++) acc[i] += p * vv[u][i];
-            }
-            m = mn;
-        }
+        j = j2;
     }
 }
 
@@ -254,7 +310,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
     float m = -INFINITY, l = 0.f, acc[W];
 #pragma unroll
     for (int i = 0; i < W; i++) acc[i] = 0.f;
-    decode_stream<T, LPR>(kc, vc, a.strideT, t0, t1, wave, grp, d0, active, qv, m, l, acc);
+    decode_stream<T, LPR>(kc, vc, a.strideT, t0, t1, (unsigned)((b * a.H + h) * 37 + split * 11), wave, grp, d0, active, qv, m, l, acc);
 
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
@@ -323,7 +379,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
         __syncthreads();   // the row is read back by this workgroup only (other heads of the group write their own copy)
     }
     float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
-    decode_stream<float, LPR>(kc, vc, a.kvd, t0, t1, wave, grp, d0, active, qv, m, l, acc);
+    decode_stream<float, LPR>(kc, vc, a.kvd, t0, t1, (unsigned)((b * a.H + h) * 37 + split * 11), wave, grp, d0, active, qv, m, l, acc);
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
     decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
