@@ -946,7 +946,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         ERRCHK(mem((long)pl[5], &V));
         ERRCHK(mem((long)pl[7], &Y));
         long hMask = (long)pl[6];
-        bool batchMask = pl[8] != 0;
+        // batchMask: 0 = (1,1,T,T), 1 = (B,T,1,1) as in the reference; 2 = (B,T,T) per-sequence mask (an
+        // extension that lets MultiheadAttentionLayer keep its decoder mask on the fused route)
+        const long long batchMask = pl[8];
+        if (batchMask < 0 || batchMask > 2) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         if (hMask) ERRCHK(mem(hMask, &M));
         if (Q->half != K->half || Q->half != V->half || Q->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         long long qn = (long long)st->batch * st->heads * T * st->hs, kn = (long long)st->batch * st->heads * Tk * st->hs;
@@ -955,7 +958,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         MaskKind kind = MASK_NONE;
         if (M) {
             if (M->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
-            if (batchMask) {
+            if (batchMask == 2) {
+                if ((long long)M->count < (long long)st->batch * T * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = MASK_BQK;
+            } else if (batchMask == 1) {
                 if ((long long)M->count < (long long)st->batch * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
                 kind = MASK_KEY;
             } else {

@@ -507,7 +507,8 @@ class CudaDnn:
     def AttnScaledDotProductForward(self, hCuDnn, hAttn, nBlockSize, hQdata, hKdata, hVdata, hMaskdata, hYdata,
                                     bBatchMask=True, nBlockSizeK=None):
         """CudaDnn.cs:5673-5679.  ``nBlockSizeK`` (key length, when it differs from the
-        query length) is an optional tenth value with no counterpart in the reference."""
+        query length) is an optional tenth value with no counterpart in the reference, and so
+        is ``bBatchMask=2`` (a (B,T_q,T_k) mask)."""
         rgl = [hCuDnn, hAttn, nBlockSize, hQdata, hKdata, hVdata, hMaskdata, hYdata, int(bBatchMask)]
         if nBlockSizeK is not None:
             rgl.append(nBlockSizeK)

@@ -184,8 +184,9 @@ class CausalSelfAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, fuse_batch_qk_mask=False):
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
+        self.fuse_batch_qk_mask = fuse_batch_qk_mask
         self.nSize = embed // heads
         self.bias_term, self.half = bias_term, half
         self.enable_sdpa = enable_cuda_scaled_dot_product_attention
@@ -283,7 +284,9 @@ class MultiheadAttentionLayer:
 
     ``Forward(q, k, v, mask)``: mask is ``None``, a (1,1,T,T) blob (causal), a
     (B,T_k) key-padding blob or a (B,T_q,T_k) blob; the last two take the
-    mask_batch route, as in the reference.
+    mask_batch route, as in the reference (``fuse_batch_qk_mask`` sends the
+    (B,T_q,T_k) mask to the fused handle instead, which the reference's handle
+    cannot do).
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
@@ -339,7 +342,7 @@ class MultiheadAttentionLayer:
         is_qk_mask = (blobMask is not None and blobMask.num_axes == 4 and blobMask.num == 1 and blobMask.channels == 1
                       and blobMask.height == Tq and blobMask.width == Tk)
         full_mask = blobMask is not None and not is_qk_mask and blobMask.count() == B * Tq * Tk and Tq > 1
-        if self.enable_sdpa and not full_mask:
+        if self.enable_sdpa and (not full_mask or self.fuse_batch_qk_mask):
             if self._set_for != B:
                 if not self.hCudnn:
                     self.hCudnn = cuda.CreateCuDNN()
@@ -349,7 +352,7 @@ class MultiheadAttentionLayer:
             b["Work"].ReshapeLike(b["Qt"])
             cuda.AttnScaledDotProductForward(self.hCudnn, self.hAttn, Tq, b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data,
                                              blobMask.gpu_data if blobMask is not None else 0, b["Work"].gpu_data,
-                                             not is_qk_mask, Tk if Tk != Tq else None)
+                                             2 if full_mask else (not is_qk_mask), Tk if Tk != Tq else None)
         else:
             # the fused handle only understands (1,1,T,T) or (B,T) masks (attn.cu:544-556); a
             # (B,T_q,T_k) mask goes through the explicit chain (MultiheadAttentionLayer.cs:733-742)

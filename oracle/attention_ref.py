@@ -9,7 +9,10 @@ Pins (tests/test_oracle_layers.py): the inline vectors of
 MyCaffe.test/TestCudaDnn.cs (gemm, gemv, mask, mask_batch, channel_copy), the
 ``gpt-pico-csa*`` golden tensors held by the reference test data (q after
 transpose, softmax probabilities, y), scipy/torch library routines (softmax,
-scaled_dot_product_attention) and closed forms (RoPE as a complex rotation).
+scaled_dot_product_attention, BLAS dgemm on column-major views for gemm2,
+embedding, linear, multi_head_attention_forward for the whole multi-head layer
+with causal / key-padding / per-batch masks) and closed forms (RoPE as a complex
+rotation, the cos/sin tables).  Every function of this file has such a check.
 """
 import numpy as np
 

@@ -216,6 +216,12 @@ def test_multihead_attention_encoder_decoder_masks(dev, sdpa):
     ref = R.multihead_attention(tgt, tgt, tgt, W["wq"], W["bq"], W["wk"], W["bk"], W["wv"], W["bv"], W["wo"], W["bo"], H,
                                 dec_mask, "full", dtype=np.float64)
     assert_close(top.mutable_cpu_data, ref["y"], FP32_RTOL, "decoder self attention")
+    if sdpa:
+        # the same (B,T,T) mask kept on the fused handle (batch-mask code 2)
+        dec2 = MultiheadAttentionLayer(dev.cuda, H, C, Tt, True, True, fuse_batch_qk_mask=True)
+        dec2.Setup(bt, bt, bt, W)
+        dec2.Forward(bt, bt, bt, bdm, top)
+        assert_close(top.mutable_cpu_data, ref["y"], FP32_RTOL, "decoder self attention, fused per-sequence mask")
     # cross attention: queries from the target, keys / values from the source, source key padding
     if sdpa:
         cross = MultiheadAttentionLayer(dev.cuda, H, C, Ts, True, True)

@@ -216,3 +216,99 @@ def test_causal_self_attention_golden(name, heads):
         x, load_txt(os.path.join(d, "attn_weight.txt")), load_txt(os.path.join(d, "attn_bias.txt")),
         load_txt(os.path.join(d, "attn_proj_weight.txt")), load_txt(os.path.join(d, "attn_proj_bias.txt")), heads)
     assert np.abs(out32["y"] - out["y"]).max() < 1e-6
+
+
+# ---- remaining primitives against independent library routines -----------------------
+
+def test_gemm2_colmajor_matches_blas_sgemm_strided():
+    """Column-major strided-batched semantics against scipy's BLAS dgemm on Fortran-ordered views,
+    with padded leading dimensions, both transposes and beta != 0."""
+    from scipy.linalg import blas
+    rng = np.random.default_rng(5)
+    m, n, k, batch = 4, 3, 5, 3
+    for tA in (False, True):
+        for tB in (False, True):
+            ar, ac = (k, m) if tA else (m, k)
+            br, bc = (n, k) if tB else (k, n)
+            lda, ldb, ldc = ar + 2, br + 1, m + 3
+            sA, sB, sC = lda * ac + 4, ldb * bc + 2, ldc * n + 1
+            A = rng.standard_normal(sA * batch)
+            B = rng.standard_normal(sB * batch)
+            C = rng.standard_normal(sC * batch)
+            out = R.gemm2_colmajor(tA, tB, m, n, k, 0.7, A, B, -0.3, C, lda, ldb, ldc, sA, sB, sC, batch, dtype=np.float64)
+            exp = C.copy()
+            for b in range(batch):
+                a = A[b * sA:b * sA + lda * ac].reshape((lda, ac), order="F")[:ar]
+                bb = B[b * sB:b * sB + ldb * bc].reshape((ldb, bc), order="F")[:br]
+                c = exp[b * sC:b * sC + ldc * n].reshape((ldc, n), order="F")
+                c[:m] = blas.dgemm(0.7, a, bb, beta=-0.3, c=np.asfortranarray(c[:m]), trans_a=tA, trans_b=tB)
+            assert np.allclose(out, exp, rtol=1e-13, atol=1e-13), (tA, tB)
+
+
+def test_embed_inner_product_match_torch():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(6)
+    w = rng.standard_normal((11, 5)).astype(np.float32)
+    ids = np.array([3.0, 0.0, 10.0, 3.0, 7.0], np.float32)   # the reference passes indices as floats
+    assert np.array_equal(R.embed_fwd(ids, w), F.embedding(torch.tensor(ids).long(), torch.tensor(w)).numpy())
+    x = rng.standard_normal((2, 3, 5))
+    wt = rng.standard_normal((4, 5))
+    b = rng.standard_normal(4)
+    exp = F.linear(torch.tensor(x), torch.tensor(wt), torch.tensor(b)).numpy()
+    assert np.allclose(R.inner_product(x, wt, b, dtype=np.float64), exp, rtol=1e-13, atol=1e-13)
+    assert np.allclose(R.inner_product(x, wt, None, dtype=np.float64), exp - b, rtol=1e-12, atol=1e-12)
+
+
+def test_rope_tables_closed_form():
+    """cos/sin(pos * theta^(-2j/hs)) in float64; the fp32 table may differ by the rounding of the angle
+    (|d angle| <= 2^-24 * pos), nothing more."""
+    S, hs, theta = 64, 16, 10000.0
+    c, s = R.rope_tables(S, hs, theta)
+    assert c.shape == (S, hs // 2) and s.shape == (S, hs // 2)
+    pos = np.arange(S, dtype=np.float64)[:, None]
+    ang = pos * theta ** (-np.arange(0, hs, 2, dtype=np.float64) / hs)[None, :]
+    tol = 4e-7 * (1 + pos)
+    assert np.all(np.abs(c - np.cos(ang)) <= tol) and np.all(np.abs(s - np.sin(ang)) <= tol)
+    assert np.all(c[0] == 1) and np.all(s[0] == 0)
+    assert c[1, 0] == np.float32(np.cos(np.float32(1.0))) and s[1, 0] == np.float32(np.sin(np.float32(1.0)))
+
+
+@pytest.mark.parametrize("kind", ["none", "causal", "key", "full"])
+def test_multihead_attention_matches_torch_mha(kind):
+    """The whole layer (four projections, head split, scaled scores, mask fill, softmax, merge) against
+    torch.nn.functional.multi_head_attention_forward with separate projection weights; self attention for
+    the causal / full masks, cross attention (T_q != T_k) with a key padding mask."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(8)
+    B, Tq, C, H = 3, 5, 8, 2
+    Tk = 7 if kind in ("none", "key") else Tq
+    xq = rng.standard_normal((B, Tq, C))
+    xk = rng.standard_normal((B, Tk, C)) if Tk != Tq else xq
+    W = [rng.standard_normal((C, C)) * 0.4 for _ in range(4)]
+    b = [rng.standard_normal(C) * 0.1 for _ in range(4)]
+    mask_data = None
+    attn_mask = None
+    kpm = None
+    if kind == "causal":
+        mask_data = R.causal_mask(Tq, np.float64)
+        attn_mask = torch.tensor(mask_data.reshape(Tq, Tq) == 0)
+    elif kind == "key":
+        lens = np.array([7, 3, 5])
+        mask_data = (np.arange(Tk)[None, :] < lens[:, None]).astype(np.float64)
+        kpm = torch.tensor(mask_data == 0)
+    elif kind == "full":
+        lens = np.array([5, 2, 4])
+        keep = (np.arange(Tq)[None, None, :] < lens[:, None, None]) & np.tril(np.ones((Tq, Tq), bool))[None]
+        mask_data = keep.astype(np.float64)
+        attn_mask = torch.tensor(np.repeat(~keep, H, axis=0))           # (B*H, Tq, Tk), batch-major like torch
+    out = R.multihead_attention(xq, xk, xk, W[0], b[0], W[1], b[1], W[2], b[2], W[3], b[3], H, mask_data, kind, dtype=np.float64)
+    t = lambda a: torch.tensor(a)
+    exp, _ = F.multi_head_attention_forward(
+        t(xq).transpose(0, 1), t(xk).transpose(0, 1), t(xk).transpose(0, 1), C, H, None,
+        torch.cat([t(b[0]), t(b[1]), t(b[2])]), None, None, False, 0.0, t(W[3]), t(b[3]), training=False,
+        key_padding_mask=kpm, need_weights=False, attn_mask=attn_mask, use_separate_proj_weight=True,
+        q_proj_weight=t(W[0]), k_proj_weight=t(W[1]), v_proj_weight=t(W[2]))
+    assert np.allclose(out["y"], exp.transpose(0, 1).numpy(), rtol=1e-10, atol=1e-10)
+    assert np.allclose(out["att"].sum(-1), 1.0)
