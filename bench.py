@@ -95,6 +95,21 @@ def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
     return inf, res
 
 
+def recorded_traffic(key):
+    """HBM bytes per launch from the committed counter summary (FETCH_SIZE + WRITE_SIZE runs, calibrated on a
+    known-size kernel); None when the summary has no entry for `key`."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")):
+            if line.startswith("traffic_bytes_per_launch:"):
+                for item in line.split(":", 1)[1].split():
+                    k, v = item.split("=")
+                    if k == key:
+                        return int(v)
+    except OSError:
+        pass
+    return None
+
+
 def step_roofline(inf, head, steps, warmup):
     """Roofline of the timed unit, one decode step (one replay of the captured graph: 62 dispatches that stream
     every weight once and the KV cache of the current length), from the HIP-event time of the timed region.
@@ -115,7 +130,8 @@ def step_roofline(inf, head, steps, warmup):
     return {"kernel": "decode step = one replay of the captured graph (49 matvec_kernel, 12 attn_decode_fused_kernel, "
                       "1 sample_advance_kernel)",
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic("decode_step"),
+            "traffic_note": "counter runs cover a step at position 512 (475.9 MB algorithmic there)",
             "algorithmic_bytes_per_launch": round(nbytes), "avg_launch_us": round(us, 3), "dispatches_per_launch": 62,
             "event_pair_around_empty_kernel_us": round(pair_ms * 1e3, 3), "per_class_event_pairs": detail}
 
@@ -147,7 +163,7 @@ def cpu_baseline(blob, gpu_prompt, gpu_ids, budget_s=12.0):
             "ids_vs_gpu_first_generation": same}
 
 
-def bench_prefill_attention(cuda, reps):
+def bench_prefill_attention(cuda, reps, warm=5):
     """Fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_FWD (id 163)."""
     from mycaffe_amd.cudadnn import CUDAFN
     B, H, T, hs = 8, 12, 1024, 64
@@ -161,20 +177,21 @@ def bench_prefill_attention(cuda, reps):
         hy = cuda.AllocMemory(B * H * T * hs, bHalfSize=half)
         rgl = [hc, ha, T, hs_[0], hs_[1], hs_[2], mask, hy, 0]
         cuda.AttnScaledDotProductForward(hc, ha, T, hs_[0], hs_[1], hs_[2], mask, hy, False)
-        ms = cuda.TimeFunction(CUDAFN.CUDA_ATTN_FWD, None, rgl, 5, reps)
+        ms = cuda.TimeFunction(CUDAFN.CUDA_ATTN_FWD, None, rgl, warm, reps)
         useful = 2.0 * B * H * T * T * hs          # causal half of the 4*B*H*T*T*hs full-square flops
         tf = useful / (ms / 1e3) / 1e12
         out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2), "TFLOPs_full_square": round(2 * tf, 2),
                      "roofline": {"kernel": "fused causal attention forward", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s",
-                                  "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4), "traffic": None}}
+                                  "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
+                                  "traffic": recorded_traffic("flash_" + name)}}
         for h in hs_ + [hy]:
             cuda.FreeMemory(h)
     cuda.FreeMemory(mask)
     return out
 
 
-def bench_decode_attention(cuda, reps):
+def bench_decode_attention(cuda, reps, warm=5, cases=None):
     """KV-cache attention, 32 heads x 128, one query token per sequence (id 2001)."""
     from mycaffe_amd.cudadnn import CUDAFN
     H, hs = 32, 128
@@ -183,28 +200,36 @@ def bench_decode_attention(cuda, reps):
     for name, half, es in (("bf16", True, 2), ("f32", False, 4)):
         for B in (1, 8, 32):
             for L in (512, 2048, 4096):
+                if cases is not None and (name, B, L) not in cases:
+                    continue
                 n = B * H * L * hs
                 kc = cuda.AllocMemory(n, bHalfSize=half)
                 vc = cuda.AllocMemory(n, bHalfSize=half)
-                # fill on the device: a seeded block repeated (values only matter for parity tests)
+                # fill on the device: a seeded block, then doubled in place (values only matter for parity tests)
                 blk = rng.standard_normal(min(n, 1 << 20)).astype(np.float32)
                 src = cuda.AllocMemory(blk, bHalfSize=half)
-                for off in range(0, n, blk.size):
-                    c = min(blk.size, n - off)
-                    cuda.copy(c, src, kc, 0, off)
-                    cuda.copy(c, src, vc, 0, off)
+                for dst in (kc, vc):
+                    cuda.copy(blk.size, src, dst, 0, 0)
+                    have = blk.size
+                    while have < n:
+                        c = min(have, n - have)
+                        cuda.copy(c, dst, dst, 0, have)
+                        have += c
                 q = cuda.AllocMemory(rng.standard_normal(B * H * hs).astype(np.float32), bHalfSize=half)
                 y = cuda.AllocMemory(B * H * hs, bHalfSize=half)
                 rgl = [B, H, H, hs, L, q, kc, vc, y, H * L * hs, L * hs, hs]
-                ms = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl, 5, reps)
+                ms = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl, warm, reps)
                 nbytes = 2.0 * n * es
                 gbs = nbytes / (ms / 1e3) / 1e9
                 out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
                 for h in (kc, vc, src, q, y):
                     cuda.FreeMemory(h)
+    if "bf16_B32_L4096" not in out:
+        return out
     best = out["bf16_B32_L4096"]
     out["roofline"] = {"kernel": "attn_decode_kernel (bf16, batch 32, L 4096, 32 x 128)", "bound": "hbm", "achieved": best["GBps"],
-                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_hbm"], "traffic": None}
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_hbm"],
+                       "traffic": recorded_traffic("attn_decode_bf16_B32_L4096")}
     return out
 
 
@@ -227,18 +252,39 @@ def bench_gemm(cuda, reps):
     return out
 
 
-def bench_copy(cuda, reps):
-    """Plain device copy of 64 Mi floats (reads 256 MiB, writes 256 MiB): the known-size kernel that the
-    FETCH_SIZE / WRITE_SIZE counter readings of the other kernels are scaled by."""
+def bench_copy(cuda, reps, warm=2):
+    """Plain streaming kernel of known size (y = 1.0 * x over 64 Mi floats: reads 256 MiB, writes 256 MiB): the kernel
+    that the FETCH_SIZE / WRITE_SIZE counter readings of the other kernels are scaled by."""
     from mycaffe_amd.cudadnn import CUDAFN
     n = 64 << 20
     a = cuda.AllocMemory(n)
     b = cuda.AllocMemory(n)
-    ms = cuda.TimeFunction(CUDAFN.CUDA_COPY, [], [n, a, b], 2, reps)
+    ms = cuda.TimeFunction(CUDAFN.CUDA_SCALE, [1.0], [n, 0, a, b, 0, 0], warm, reps)
     cuda.FreeMemory(a)
     cuda.FreeMemory(b)
-    return {"kernel": "convert_kernel<float, float>", "bytes_read": n * 4, "bytes_written": n * 4, "ms": round(ms, 4),
+    return {"kernel": "scale_kernel<float>", "bytes_read": n * 4, "bytes_written": n * 4, "ms": round(ms, 4),
             "GBps": round(2 * n * 4 / (ms / 1e3) / 1e9, 1)}
+
+
+def counter_pass(cuda, path):
+    """A short run for hardware-counter collection (rocprofv3 --pmc serialises and slows every dispatch):
+    two eager decode steps at position 512, two dispatches each of the fused prefill attention (bf16, fp32),
+    the decode attention at batch 32 / L 4096 (bf16, fp32) and the 256 MiB copy that calibrates the counters."""
+    from mycaffe_amd.llm_inference import LlmInference
+    inf = LlmInference(cuda)
+    inf.Initialize(fTemperature=0.0)
+    inf.SetOption(3, 0)
+    inf.Load(path)
+    log("counter pass: decode steps")
+    inf.ProfileStep(512, 2)
+    inf.CleanUp()
+    log("counter pass: copy")
+    out = {"copy_256MiB": bench_copy(cuda, 2, 0)}
+    log("counter pass: prefill attention")
+    out["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 2, 0)
+    log("counter pass: decode attention")
+    out["decode_attention_H32x128"] = bench_decode_attention(cuda, 2, 0, cases=(("bf16", 32, 4096), ("f32", 32, 4096)))
+    return out
 
 
 def main():
@@ -250,6 +296,8 @@ def main():
     ap.add_argument("--no-also", action="store_true", help="only the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="launch every decode kernel eagerly instead of replaying a HIP graph "
                     "(kernel tracing tools see the individual kernels this way)")
+    ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
+                    "prints what ran instead of the benchmark line")
     ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
@@ -270,6 +318,10 @@ def main():
     blob = make_checkpoint(C4, 1234, path)
     log("checkpoint ready in %.1f s" % (time.perf_counter() - t0))
 
+    if args.counter_pass:
+        print(json.dumps({"counter_pass": counter_pass(cuda, path)}), flush=True)
+        cuda.Dispose()
+        return
     inf, head = run_decode(cuda, path, False, 1, args.steps, args.warmup, graph=not args.no_graph)
     log("fp32 batch 1: %.1f tokens/s (%.4f ms/step)" % (head["tokens_per_s"], head["ms_per_step"]))
     roof = step_roofline(inf, head, args.steps, args.warmup)
