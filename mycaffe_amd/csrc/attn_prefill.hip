@@ -138,7 +138,7 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 // cycles per score against 8 MFMA cycles per score at head size 64); the fp32 kernel is
 // MFMA bound.  Causal: key blocks past the workgroup's last row are never visited,
 // wavefronts skip steps past their own rows, only diagonal steps pay for the element mask,
-// and the heaviest query blocks are scheduled first.
+// and workgroups are launched heaviest query block first across all heads.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -151,6 +151,7 @@ struct FlashArgs {
     int B, H, Tq, Tk;
     float c;             // softmax scale * log2(e)
     float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
+    float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
 };
 
 __device__ inline uint32_t pack_bf16x2(float a, float b)
@@ -231,7 +232,7 @@ template <> struct FlashTraits<float> {
 // of two huge products would not cancel exactly.
 template <bool MASKED, int DT, int QT>
 __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (&o)[DT][QT], float (&m)[QT], float (&l)[QT],
-                                                   float c, float sentinel)
+                                                   float c, float sentinel, float lazy)
 {
     float mx[QT], mnew[QT], alpha[QT], mc[QT];
 #pragma unroll
@@ -245,7 +246,10 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
     bool same = true;
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
-        mnew[qt] = fmaxf(m[qt], mx[qt]);
+        // the reference maximum only moves when a score exceeds it by more than the slack: weights are then
+        // at most 2^8 (exact in the final normalisation, since l uses the same reference) and the rescale of
+        // the output accumulators below is skipped on most steps
+        mnew[qt] = (mx[qt] > m[qt] + lazy) ? mx[qt] : m[qt];
         alpha[qt] = __builtin_amdgcn_exp2f((m[qt] - mnew[qt]) * c);
         mc[qt] = mnew[qt] * c;
         m[qt] = mnew[qt];
@@ -296,8 +300,23 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
-    const int qblock = gridDim.x - 1 - blockIdx.x;   // heavy (late) query blocks first
-    const int h = blockIdx.y, b = blockIdx.z;
+    // Causal work grows with the query block, so the launch is one-dimensional and ordered heaviest block
+    // first across ALL (batch, head) pairs: workgroups are dispatched in index order as slots free up, which
+    // makes the hardware dispatcher a longest-job-first scheduler.  Consecutive indices share a query block
+    // and differ in (batch, head), so with B*H a multiple of 8 every head's blocks land on one XCD's L2.
+    int qblock, h, b;
+    if (KIND == 1) {
+        const int nbh = a.B * a.H;
+        const int nqb = (a.Tq + BM - 1) / BM;
+        qblock = nqb - 1 - (int)(blockIdx.x / nbh);
+        const int ibh = blockIdx.x % nbh;
+        b = ibh / a.H;
+        h = ibh % a.H;
+    } else {
+        qblock = blockIdx.x;
+        h = blockIdx.y;
+        b = blockIdx.z;
+    }
     const size_t bh = (size_t)b * a.H + h;
     const int q0 = qblock * BM + wave * 32 * QT;      // first row of this wavefront
     const T* qp = (const T*)a.q + bh * a.Tq * HS;
@@ -403,9 +422,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                             s[qt][v] = sv;
                         }
                     }
-                    flash_softmax_step<true, DT, QT>(s, o, m, l, c, a.maskedRaw);
+                    flash_softmax_step<true, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
                 } else {
-                    flash_softmax_step<false, DT, QT>(s, o, m, l, c, a.maskedRaw);
+                    flash_softmax_step<false, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
                 }
                 // O^T += V^T P^T
                 u32x4 pf[QT][PF];
@@ -455,6 +474,7 @@ static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
 {
     constexpr int BM = NW * 32 * QT;
     dim3 grid((f.Tq + BM - 1) / BM, f.H, f.B);
+    if (kind == MASK_CAUSAL) grid = dim3(((f.Tq + BM - 1) / BM) * f.H * f.B, 1, 1);
     if (kind == MASK_NONE) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 0, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     else if (kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 1, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 2, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
@@ -472,17 +492,16 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     f.mask = a.mask; f.B = a.B; f.H = a.H; f.Tq = a.Tq; f.Tk = a.Tk;
     f.c = a.scale * 1.4426950408889634f;
     f.maskedRaw = MASKED / a.scale;
+    f.lazy = 8.0f / f.c;
     *handled = true;
+    // Tile shapes picked by measurement on MI355X.  Head size 64: four wavefronts with one 32-row tile each
+    // (128-row workgroups) give enough equal-sized workgroups to balance 256 CUs at T = 1024; head size 128
+    // keeps eight wavefronts per workgroup so that each staged K / V block serves more rows.
     if (dt == BF16) {
-        if (a.hs == 64) {
-            // causal work is triangular: 32-row wavefront tiles in 256-row workgroups keep the diagonal
-            // waste small; square work prefers the 64-row wavefront tile (each LDS fragment feeds two MFMAs)
-            if (a.kind == MASK_CAUSAL) return flash_launch_cfg<bf16_t, 64, 1, 8, 2, true>(s, f, a.kind);
-            return flash_launch_cfg<bf16_t, 64, 2, 4, 2, true>(s, f, a.kind);
-        }
+        if (a.hs == 64) return flash_launch_cfg<bf16_t, 64, 1, 4, 3, true>(s, f, a.kind);
         return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
     }
-    if (a.hs == 64) return flash_launch_cfg<float, 64, 2, 4, 2, false>(s, f, a.kind);
+    if (a.hs == 64) return flash_launch_cfg<float, 64, 1, 4, 2, false>(s, f, a.kind);
     return flash_launch_cfg<float, 128, 1, 8, 1, false>(s, f, a.kind);
 }
 

@@ -184,9 +184,8 @@ class CausalSelfAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, fuse_batch_qk_mask=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
-        self.fuse_batch_qk_mask = fuse_batch_qk_mask
         self.nSize = embed // heads
         self.bias_term, self.half = bias_term, half
         self.enable_sdpa = enable_cuda_scaled_dot_product_attention
@@ -290,8 +289,9 @@ class MultiheadAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, fuse_batch_qk_mask=False):
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
+        self.fuse_batch_qk_mask = fuse_batch_qk_mask
         self.nSize = embed // heads
         self.half = half
         self.enable_sdpa = enable_cuda_scaled_dot_product_attention
