@@ -16,6 +16,16 @@ namespace mch {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+typedef float floatx2v __attribute__((ext_vector_type(2)));
+
+__device__ inline uint32_t pack2_bf16(float a, float b)
+{
+    floatx2v f = {a, b};
+    bf16x2v r = __builtin_convertvector(f, bf16x2v);
+    return *reinterpret_cast<uint32_t*>(&r);
+}
 
 template <typename T> __device__ inline float ldf(const T* p, size_t i);
 template <> __device__ inline float ldf<float>(const float* p, size_t i) { return p[i]; }
@@ -288,6 +298,205 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_mfma_kernel(int M, int N, in
         }
 }
 
+// ---------------------------------------------------------------------------
+// bf16 MFMA, NT, large tiles: 2 x 2 wavefronts, each owning WM x WN MFMA 32x32 tiles, so a workgroup
+// covers (64 WM) x (64 WN) of C.  A 128 x 128 wavefront tile (WM = WN = 4) reads 8 LDS fragments per 16 MFMAs,
+// a quarter of the LDS traffic per flop of the 64 x 64 wavefront tile above, which is what keeps the matrix
+// cores fed; its 256 accumulators live in the accumulation registers.  K is walked in steps of 32 through a
+// double-buffered LDS stage (one barrier per step); the next stage travels global -> registers -> LDS while
+// the current one is consumed.  Tiles are numbered so that each XCD (workgroup index mod 8) works on a
+// contiguous band of tile rows and re-uses its A rows out of its own L2.
+template <int WM, int WN, int BK, int OCC>
+__global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N, int K, float alpha, const bf16_t* __restrict__ A,
+                                                                    const bf16_t* __restrict__ B, float beta, bf16_t* __restrict__ C,
+                                                                    int tilesN, int tilesTotal)
+{
+    constexpr int BM = 64 * WM, BN = 64 * WN, LDK = BK + 8;   // row stride 16 B past a power of two: conflict-free 128-bit reads
+    constexpr int CPR = BK / 8;                               // 16-byte chunks per tile row
+    constexpr int RPP = 256 / CPR;                            // rows covered by one pass of the 256 threads
+    constexpr int PA = BM / RPP, PB = BN / RPP;               // passes (16-byte chunks per thread) per operand
+    constexpr int KS = BK / 16;                               // MFMA k-steps per stage
+    constexpr int NMF = WM * WN;                              // MFMAs per k-step
+    static_assert(KS >= 2 && (KS % 2) == 0, "stage = an even number of k-steps");
+    static_assert(NMF >= WM + WN && NMF * (KS / 2) >= PA + PB, "not enough MFMAs per k-step to carry the memory instructions");
+    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+    bf16_t* As = smem;                        // [2][BM * LDK]
+    bf16_t* Bs = smem + 2 * BM * LDK;         // [2][BN * LDK]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per = (tilesTotal + 7) / 8;
+    const int tile = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+    if (tile >= tilesTotal) return;
+    const int m0 = (tile / tilesN) * BM, n0 = (tile % tilesN) * BN;
+    const int wm = (wave >> 1) * (32 * WM), wn = (wave & 1) * (32 * WN);
+    const int lr = tid / CPR, lc = (tid % CPR) * 8;
+
+    floatx16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; i++)
+#pragma unroll
+        for (int j = 0; j < WN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    // rows past the matrix edge are clamped: they are loaded (valid memory) and never stored
+    const bf16_t* ga[PA];
+    const bf16_t* gb[PB];
+#pragma unroll
+    for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * K + lc;
+#pragma unroll
+    for (int p = 0; p < PB; p++) gb[p] = B + (size_t)min(n0 + lr + p * RPP, N - 1) * K + lc;
+    bf16_t* sa = As + lr * LDK + lc;
+    bf16_t* sb = Bs + lr * LDK + lc;
+    u32x4 ra[PA], rb[PB];
+
+    const int nk = K / BK;
+    // stage 0 -> LDS buffer 0, stage 1 -> registers
+#pragma unroll
+    for (int p = 0; p < PA; p++) ra[p] = *(const u32x4*)(ga[p]);
+#pragma unroll
+    for (int p = 0; p < PB; p++) rb[p] = *(const u32x4*)(gb[p]);
+#pragma unroll
+    for (int p = 0; p < PA; p++) *(u32x4*)(sa + p * RPP * LDK) = ra[p];
+#pragma unroll
+    for (int p = 0; p < PB; p++) *(u32x4*)(sb + p * RPP * LDK) = rb[p];
+    {
+        const int k1 = min(1, nk - 1) * BK;
+#pragma unroll
+        for (int p = 0; p < PA; p++) ra[p] = *(const u32x4*)(ga[p] + k1);
+#pragma unroll
+        for (int p = 0; p < PB; p++) rb[p] = *(const u32x4*)(gb[p] + k1);
+    }
+    __syncthreads();
+    const int fr = lane & 31, fg = (lane >> 5) * 8;
+    const bf16_t* fa = As + (wm + fr) * LDK + fg;
+    const bf16_t* fb = Bs + (wn + fr) * LDK + fg;
+    bf16x8 a[2][WM], b[2][WN];
+    // One stage: KS k-steps of NMF MFMAs on LDS buffer kt & 1.  Riding along between the MFMAs (the wavefront is
+    // alone on its SIMD, so whatever it issues between two MFMAs is hidden behind the first one's 8 passes, and
+    // whatever it issues in a block of its own is not):
+    //   first half of the k-steps : the registers holding stage kt + 1 go to the other LDS buffer
+    //   second half               : stage kt + 2 is fetched from global memory into those registers
+    //   every k-step but the last : the fragments of the next k-step are read from LDS
+    // Past the end of K the extra fetches re-read the last stage (valid memory, never consumed).
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        const bf16_t* pa = fa + buf * BM * LDK;
+        const bf16_t* pb = fb + buf * BN * LDK;
+        bf16_t* wa = sa + (buf ^ 1) * BM * LDK;
+        bf16_t* wb = sb + (buf ^ 1) * BN * LDK;
+        const int k2 = min(kt + 2, nk - 1) * BK;
+#pragma unroll
+        for (int t = 0; t < WM; t++) a[0][t] = *(const bf16x8*)(pa + t * 32 * LDK);
+#pragma unroll
+        for (int t = 0; t < WN; t++) b[0][t] = *(const bf16x8*)(pb + t * 32 * LDK);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            // this k-step's share of the staging traffic: chunks [c0, c1) of the PA + PB chunks per thread
+            constexpr int HALF = KS / 2;
+            const int part = ks % HALF;
+            const int c0 = (PA + PB) * part / HALF, c1 = (PA + PB) * (part + 1) / HALF;
+            // written in issue order, one small scheduling region per MFMA so that the order stays as written:
+            // MFMA q, then the q-th fragment read of the next k-step, then the q-th staging instruction
+#pragma unroll
+            for (int q = 0; q < NMF; q++) {
+                const int i = q / WN, j = q % WN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[cur][j], a[cur][i], acc[i][j], 0, 0, 0);
+                if (ks + 1 < KS) {
+                    if (q < WM) a[nxt][q] = *(const bf16x8*)(pa + q * 32 * LDK + (ks + 1) * 16);
+                    else if (q < WM + WN) b[nxt][q - WM] = *(const bf16x8*)(pb + (q - WM) * 32 * LDK + (ks + 1) * 16);
+                }
+                const int c = c0 + q;
+                if (c < c1) {
+                    if (ks < HALF) {
+                        if (c < PA) *(u32x4*)(wa + c * RPP * LDK) = ra[c];
+                        else *(u32x4*)(wb + (c - PA) * RPP * LDK) = rb[c - PA];
+                    } else {
+                        if (c < PA) ra[c] = *(const u32x4*)(ga[c] + k2);
+                        else rb[c - PA] = *(const u32x4*)(gb[c - PA] + k2);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+    }
+    // The MFMAs above compute the TRANSPOSED 32x32 tiles (B fragment as the row operand), so a lane owns one
+    // row of C (lane%32) and register v is column 8*(v/4) + 4*(lane/32) + v%4: four consecutive columns per
+    // register quad.
+    const int row_l = lane & 31, col_l = (lane >> 5) * 4;
+    if (m0 + BM <= M && n0 + BN <= N && beta == 0.f && (N & 7) == 0 && (((uintptr_t)C) & 15) == 0) {
+        // interior tile: each wavefront passes its tile through its own slice of LDS (free after the last
+        // barrier) and writes whole 16-byte pieces of rows, 64 lanes covering full cache lines
+        constexpr int CW = 32 * WN, LDC = CW + 8;
+        constexpr int LPR = CW / 8, RPI = 64 / LPR;            // lanes per row, rows per store instruction
+        bf16_t* cs = smem + wave * (32 * WM) * LDC;
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    uint2 w;
+                    w.x = pack2_bf16(alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1]);
+                    w.y = pack2_bf16(alpha * acc[i][j][4 * g + 2], alpha * acc[i][j][4 * g + 3]);
+                    *(uint2*)(cs + (i * 32 + row_l) * LDC + j * 32 + 8 * g + col_l) = w;
+                }
+        // same wavefront wrote and reads: LDS operations of one wavefront complete in order
+        const int rr = lane / LPR, cc = (lane % LPR) * 8;
+        bf16_t* cg = C + (size_t)(m0 + wm + rr) * N + n0 + wn + cc;
+        constexpr int NIT = (32 * WM + RPI - 1) / RPI;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            // lanes past RPI * LPR (row widths that do not divide 64) and rows past the tile stay idle
+            if (rr < RPI && it * RPI + rr < 32 * WM) {
+                const u32x4 v = *(const u32x4*)(cs + (it * RPI + rr) * LDC + cc);
+                *(u32x4*)(cg + (size_t)it * RPI * N) = v;
+            }
+        }
+        return;
+    }
+    // edge tiles, beta != 0: element-wise (unrolled, so the accumulators are never indexed dynamically)
+#pragma unroll
+    for (int i = 0; i < WM; i++)
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+            const int r = m0 + wm + i * 32 + row_l;
+            if (r >= M) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int c = n0 + wn + j * 32 + (v >> 2) * 8 + col_l + (v & 3);
+                if (c < N) {
+                    const size_t ci = (size_t)r * N + c;
+                    float o = alpha * acc[i][j][v];
+                    if (beta != 0.f) o += beta * bf16_to_f32(C[ci]);
+                    C[ci] = f32_to_bf16(o);
+                }
+            }
+        }
+}
+
+template <int WM, int WN, int BK, int OCC>
+static hipError_t launch_big_bf16(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C)
+{
+    const int tm = (m + 64 * WM - 1) / (64 * WM), tn = (n + 64 * WN - 1) / (64 * WN);
+    const long long total = (long long)tm * tn;
+    if (total > (1ll << 30)) return hipErrorInvalidValue;
+    const int per = (int)((total + 7) / 8);
+    size_t lds = (size_t)2 * (64 * WM + 64 * WN) * (BK + 8) * sizeof(bf16_t);
+    const size_t ldsEpilogue = (size_t)4 * (32 * WM) * (32 * WN + 8) * sizeof(bf16_t);
+    if (ldsEpilogue > lds) lds = ldsEpilogue;
+    static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_bf16_big_kernel<WM, WN, BK, OCC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    hipLaunchKernelGGL((gemm_nt_bf16_big_kernel<WM, WN, BK, OCC>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const bf16_t*)A,
+                       (const bf16_t*)B, beta, (bf16_t*)C, tn, (int)total);
+    return hipGetLastError();
+}
+
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
                   const void* B, float beta, void* C)
 {
@@ -302,9 +511,21 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
         if (dt == F32)
             hipLaunchKernelGGL(gemm_nt_f32_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const float*)A, (const float*)B,
                                beta, (float*)C);
-        else
+        else {
+            if (k % 64 == 0 && ((uintptr_t)C % 4) == 0) {
+                // 256 x 256 tiles (one wavefront per SIMD, 128 x 128 per wavefront) win once K is long enough to
+                // amortise their prologue and the tile count fills the 256 CUs evenly; 128 x 128 tiles with two
+                // workgroups per CU otherwise, 128 x 192 when that gives at most one round of workgroups.
+                const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+                const double fill = (double)t256 / (double)(((t256 + 255) / 256) * 256);
+                if (k >= 2048 && fill >= 0.85) return launch_big_bf16<4, 4, 64, 1>(s, m, n, k, alpha, A, B, beta, C);
+                const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+                if (n % 192 == 0 && t128 <= 512) return launch_big_bf16<2, 3, 64, 2>(s, m, n, k, alpha, A, B, beta, C);
+                return launch_big_bf16<2, 2, 64, 2>(s, m, n, k, alpha, A, B, beta, C);
+            }
             hipLaunchKernelGGL(gemm_nt_bf16_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const bf16_t*)A,
                                (const bf16_t*)B, beta, (bf16_t*)C);
+        }
         return hipGetLastError();
     }
     GemmStrides st;

@@ -125,6 +125,24 @@ def test_gemm_bf16_inner_product_shape(dev, m, n, k):
     assert_close(dev.get(hC), ref, BF16_RTOL, "gemm bf16")
 
 
+@pytest.mark.parametrize("m,n,k,alpha,beta", [
+    (300, 200, 128, 1.0, 0.0),      # edge tiles in both directions
+    (512, 768, 192, 0.5, 0.0),      # interior only, 128 x 192 tiles, alpha
+    (384, 256, 64, 1.0, 2.0),       # beta != 0: read-modify-write epilogue
+    (1024, 1024, 2048, 1.0, 0.0),   # long K: 256 x 256 tiles
+    (260, 132, 64, 0.25, -1.0),     # ragged, both scalars
+])
+def test_gemm_bf16_large_tile_paths(dev, m, n, k, alpha, beta):
+    rng = np.random.default_rng(m + n + k)
+    A = bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    B = bf16_round((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+    C0 = bf16_round(rng.standard_normal((m, n)).astype(np.float32))
+    hA, hB, hC = dev.put(A, True), dev.put(B, True), dev.put(C0, True)
+    dev.cuda.gemm(False, True, m, n, k, alpha, hA, hB, beta, hC)
+    ref = R.gemm(False, True, m, n, k, alpha, A, B, beta, C0, dtype=np.float64)
+    assert_close(dev.get(hC, (m, n)), ref, BF16_RTOL, "gemm bf16 large tiles")
+
+
 def test_gemm_offsets_and_bias_rank1_update(dev):
     # InnerProductLayer.cs:411-415: y = x W^T, then y += ones(M,1) * bias(1,N) through gemm with K = 1
     rng = np.random.default_rng(3)
