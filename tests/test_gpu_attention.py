@@ -77,6 +77,40 @@ def test_attn_forward_arbitrary_qk_mask_and_no_mask(dev):
     assert_close(out, ref, FP32_RTOL, "attn no mask")
 
 
+@pytest.mark.parametrize("half", [True, False])
+@pytest.mark.parametrize("B,H,Tq,Tk,hs", [(2, 3, 64, 64, 64), (1, 2, 100, 100, 64), (2, 2, 257, 257, 64), (1, 4, 1024, 1024, 64),
+                                          (2, 2, 128, 320, 64), (1, 2, 33, 500, 64), (1, 2, 192, 192, 128)])
+def test_attn_forward_unmasked(dev, half, B, H, Tq, Tk, hs):
+    # no mask: bf16 / head size 64 takes the software-pipelined kernel (steady-state phases need > 3 key steps,
+    # ragged lengths end in its sequential phases); T_q != T_k is cross attention
+    rng = np.random.default_rng(Tq + Tk)
+    q = bf16_round(rng.standard_normal((B, H, Tq, hs)).astype(np.float32))
+    k, v = (bf16_round(rng.standard_normal((B, H, Tk, hs)).astype(np.float32)) for _ in range(2))
+    out = _attn(dev, q, k, v, None, False, half)
+    ref, _ = R.attn_forward(q, k, v, None, False, np.float64)
+    assert_close(out, ref, BF16_RTOL if half else FP32_RTOL, "attn unmasked")
+
+
+def test_attn_forward_large_scores_lazy_rescale(dev):
+    # a score that jumps far above the running maximum late in the key range forces the rescale of the output
+    # accumulators; scores within the slack must not
+    rng = np.random.default_rng(5)
+    B, H, T, hs = 1, 2, 512, 64
+    q = rng.standard_normal((B, H, T, hs)).astype(np.float32)
+    k = rng.standard_normal((B, H, T, hs)).astype(np.float32)
+    v = rng.standard_normal((B, H, T, hs)).astype(np.float32)
+    k[:, :, 300] = 6.0 * q[:, :, 17]          # huge score for query 17 (and large ones for similar queries) at key 300
+    k[:, :, 40] = 0.6 * q[:, :, 99]
+    for half in (False, True):
+        qq, kk, vv = (bf16_round(x) for x in (q, k, v))
+        out = _attn(dev, qq, kk, vv, None, False, half)
+        ref, _ = R.attn_forward(qq, kk, vv, None, False, np.float64)
+        assert_close(out, ref, BF16_RTOL if half else FP32_RTOL, "attn with late large scores")
+        out = _attn(dev, qq, kk, vv, R.causal_mask(T), False, half)
+        ref, _ = R.attn_forward(qq, kk, vv, R.causal_mask(T, np.float64), False, np.float64)
+        assert_close(out, ref, BF16_RTOL if half else FP32_RTOL, "causal attn with late large scores")
+
+
 def test_attn_mask_content_change_is_seen(dev):
     # a causal mask that is later overwritten through the ABI must stop being treated as causal
     rng = np.random.default_rng(13)
