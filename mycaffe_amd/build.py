@@ -5,6 +5,8 @@
 Outputs (next to this file, git-ignored):
     libmycaffe_hip.so          the CudaDnnDLL-compatible C ABI (include/mycaffe_hip_abi.h)
     libmycaffe_hip_llama2.so   the llama2 extension library loaded through CREATE_EXTENSION
+and, beside its source, tests/cpp/host_parity: the C++ host-side parity program built on
+include/mycaffe_hip_host.hpp (plain g++, it only dlopens the libraries).
 """
 import os
 import subprocess
@@ -80,7 +82,24 @@ def build(force=False, verbose=True):
         built.append(out)
         if verbose:
             print("built", out)
+    built.append(build_host_program(force, verbose))
     return built
+
+
+def host_program_path():
+    return os.path.join(HERE, "..", "tests", "cpp", "host_parity")
+
+
+def build_host_program(force=False, verbose=True):
+    src = os.path.join(HERE, "..", "tests", "cpp", "host_parity.cpp")
+    out = host_program_path()
+    inc = os.path.join(HERE, "..", "include")
+    deps = [src, os.path.join(inc, "mycaffe_hip_host.hpp"), os.path.join(inc, "mycaffe_hip_abi.h")]
+    if force or _stale(out, deps):
+        subprocess.check_call([os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-o", out, src, "-ldl"])
+    if verbose:
+        print("built", os.path.normpath(out))
+    return out
 
 
 if __name__ == "__main__":
