@@ -21,7 +21,8 @@ The single JSON line also carries:
   also          the other named kernels at their benchmark shapes, each with its own
                 roofline entry: fused prefill attention (B=8, T=1024, 12 x 64), decode
                 attention over a KV cache (32 x 128, L up to 4096, batch up to 32), the
-                QKV / projection GEMMs, batch-16 and bf16-weight decode.
+                encoder-decoder attention shapes with padding masks, the QKV / projection
+                GEMMs, batch-16 and bf16-weight decode.
 """
 import argparse
 import json
@@ -233,6 +234,41 @@ def bench_decode_attention(cuda, reps, warm=5, cases=None):
     return out
 
 
+def bench_encdec_attention(cuda, reps, warm=5):
+    """Encoder-decoder attention shapes (d_model 512, 8 heads x 64, batch 32, source 256, target 128), bf16, through
+    ATTN_FWD: encoder self attention with a (B,T) key-padding mask, decoder self attention with a (B,T,T)
+    causal-and-padding mask, cross attention (T_q 128, T_k 256) with the source key-padding mask.  Valid lengths per
+    sequence are uniform in [32,256] / [16,128] (seed 7).  Padded keys are computed and masked, not skipped: TFLOP/s
+    is quoted on the full rectangle 4*B*H*T_q*T_k*64."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    B, H, hs, Ts, Tt = 32, 8, 64, 256, 128
+    rng = np.random.default_rng(7)
+    slen, tlen = rng.integers(32, Ts + 1, B), rng.integers(16, Tt + 1, B)
+    enc_mask = (np.arange(Ts)[None, :] < slen[:, None]).astype(np.float32)
+    dec_mask = ((np.arange(Tt)[None, :] < tlen[:, None])[:, None, :] * np.tril(np.ones((Tt, Tt)))[None]).astype(np.float32)
+    hme, hmd = cuda.AllocMemory(enc_mask), cuda.AllocMemory(dec_mask)
+    out = {}
+    for name, Tq, Tk, hm, code in (("encoder_self_T256_keymask", Ts, Ts, hme, 1), ("decoder_self_T128_batch_qk_mask", Tt, Tt, hmd, 2),
+                                   ("cross_Tq128_Tk256_keymask", Tt, Ts, hme, 1)):
+        hc, ha = cuda.CreateCuDNN(), cuda.CreateAttn()
+        cuda.SetAttn(hc, ha, 0, False, B, max(Tq, Tk), H, hs, 0.0)
+        hq = cuda.AllocMemory(rng.standard_normal(B * H * Tq * hs).astype(np.float32), bHalfSize=True)
+        hk = cuda.AllocMemory(rng.standard_normal(B * H * Tk * hs).astype(np.float32), bHalfSize=True)
+        hv = cuda.AllocMemory(rng.standard_normal(B * H * Tk * hs).astype(np.float32), bHalfSize=True)
+        hy = cuda.AllocMemory(B * H * Tq * hs, bHalfSize=True)
+        rgl = [hc, ha, Tq, hq, hk, hv, hm, hy, code] + ([Tk] if Tk != Tq else [])
+        ms = cuda.TimeFunction(CUDAFN.CUDA_ATTN_FWD, None, rgl, warm, reps)
+        tf = 4.0 * B * H * Tq * Tk * hs / (ms / 1e3) / 1e12
+        out[name] = {"us": round(ms * 1e3, 2), "TFLOPs_full_rectangle": round(tf, 1), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS["bf16"], 4)}
+        for h in (hq, hk, hv, hy):
+            cuda.FreeMemory(h)
+        cuda.FreeAttn(ha)
+        cuda.FreeCuDNN(hc)
+    cuda.FreeMemory(hme)
+    cuda.FreeMemory(hmd)
+    return out
+
+
 def bench_gemm(cuda, reps):
     """QKV (8192 x 2304 x 768) and output projection (8192 x 768 x 768) GEMMs, weights [N, K]."""
     from mycaffe_amd.cudadnn import CUDAFN
@@ -298,7 +334,7 @@ def main():
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
                     "prints what ran instead of the benchmark line")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -343,6 +379,9 @@ def main():
     if want("decode_attn"):
         also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
         log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
+    if want("encdec"):
+        also["encdec_attention_B32_H8x64_bf16"] = bench_encdec_attention(cuda, 50)
+        log("enc-dec attention:", json.dumps(also["encdec_attention_B32_H8x64_bf16"]))
     if "copy" in only:
         also["copy_256MiB"] = bench_copy(cuda, 10)
     if want("gemm"):

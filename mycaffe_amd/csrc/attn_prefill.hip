@@ -147,7 +147,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // one 16-byte MFM
 
 struct FlashArgs {
     const void* q; const void* k; const void* v; void* y;
-    const float* mask;   // (B, Tk) key mask for KIND 2
+    const float* mask;   // (B, Tk) key mask for KIND 2, (B, Tq, Tk) mask for KIND 3
     int B, H, Tq, Tk;
     float c;             // softmax scale * log2(e)
     float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
@@ -277,7 +277,7 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
     }
 }
 
-// KIND: 0 no mask, 1 causal, 2 per-key mask (B, Tk).  OCC: workgroups per CU the register budget is set for.
+// KIND: 0 no mask, 1 causal, 2 per-key mask (B, Tk), 3 per-sequence mask (B, Tq, Tk).  OCC: workgroups per CU the register budget is set for.
 // PREFETCH: hold the next K / V block in registers while computing on the current one.
 template <typename T, int HS, int KIND, int QT, int NW, int OCC, bool PREFETCH>
 __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                     for (int qt = 0; qt < QT; qt++) s[qt] = TR::mma(kf, qf[qt][f], s[qt]);
                 }
                 // register v holds key k0 + 8*(v/4) + 4*half + v%4 for query q0 + 32*qt + l32
-                const bool maskedBlock = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk) || KIND == 2;   // wavefront-uniform
+                const bool maskedBlock = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk) || KIND >= 2;   // wavefront-uniform
                 if (maskedBlock) {
 #pragma unroll
                     for (int qt = 0; qt < QT; qt++) {
@@ -418,6 +418,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                             float sv = s[qt][v];
                             if (KIND == 1 && key > qrow) sv = a.maskedRaw;
                             if (KIND == 2 && Ms[32 * sub + kl] == 0.f) sv = a.maskedRaw;
+                            if (KIND == 3 && qrow < a.Tq && key < a.Tk && a.mask[((size_t)b * a.Tq + qrow) * a.Tk + key] == 0.f)
+                                sv = a.maskedRaw;
                             if (key >= a.Tk) sv = -INFINITY;
                             s[qt][v] = sv;
                         }
@@ -798,7 +800,8 @@ static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
     if (kind == MASK_CAUSAL) grid = dim3(((f.Tq + BM - 1) / BM) * f.H * f.B, 1, 1);
     if (kind == MASK_NONE) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 0, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     else if (kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 1, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
-    else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 2, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
+    else if (kind == MASK_KEY) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 2, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
+    else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 3, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     return hipGetLastError();
 }
 
@@ -806,7 +809,7 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
 {
     *handled = false;
     if (a.hs != 64 && a.hs != 128) return hipSuccess;
-    if (a.kind != MASK_NONE && a.kind != MASK_CAUSAL && a.kind != MASK_KEY) return hipSuccess;
+    if (a.kind != MASK_NONE && a.kind != MASK_CAUSAL && a.kind != MASK_KEY && a.kind != MASK_BQK) return hipSuccess;
     if ((((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.y) & 15) != 0) return hipSuccess;
     FlashArgs f;
     f.q = a.q; f.k = a.k; f.v = a.v; f.y = a.y;
