@@ -210,7 +210,7 @@ enum {
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it}
-     *   PROFILE_STEP  f{hLlm, pos, reps} -> per kernel class of one decode step
+     *   PROFILE_STEP  f{hLlm, pos, reps[, batch]} -> per kernel class of one decode step
      *                 f{ms per step, launches per step, algorithmic bytes per step}, classes in
      *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,
      *                 w2, classifier, embed+argmax */

@@ -167,6 +167,127 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
     }
 }
 
+// Batched form of the mat-vec family (2 or more sequences): the same three epilogues, computed on the matrix
+// cores so that a decode step stays bound by the weight stream instead of by vector ALU work.  A workgroup owns
+// 16 rows of W; its wavefronts take the 32-column slabs of K round robin.  Per slab a lane (row i = lane % 16,
+// group kk = lane / 16) loads W[i][k0 + 8 kk .. + 7] and, as the other operand, x[j = lane % 16][k0 + 8 kk .. + 7],
+// and issues eight v_mfma_f32_16x16x4_f32, step e contracting column k0 + 8 kk + e of the four groups: the slot to
+// column assignment only has to agree between the two operands.  Weights stored as bf16 are widened in
+// registers; activations and accumulation stay fp32.  NORM: the RMS factor of every sequence is a per-column
+// scale of the result, so the sum of squares is gathered from the x values that pass through anyway and g is
+// folded into x.  Partial tiles of the wavefronts meet in LDS; wavefront 0 finishes.
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+    __device__ static inline void load(const float* p, float* w)
+    {
+        const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+    }
+};
+template <> struct Row8<bf16_t> {
+    __device__ static inline void load(const bf16_t* p, float* w)
+    {
+        const uint4 u = *(const uint4*)p;
+        const uint32_t v[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[2 * i] = __uint_as_float(v[i] << 16);
+            w[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+        }
+    }
+};
+
+template <typename T, int MODE, bool NORM>
+__global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
+                                                          const float* __restrict__ g, float* __restrict__ y, int rows, int n,
+                                                          int B, int ldy, int b0)
+{
+    __shared__ float part[8][(MODE == 2 ? 2 : 1) * 256];
+    __shared__ float sspart[8][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NS = blockDim.x >> 6;
+    const int i = lane & 15, kk = lane >> 4;
+    const int r0 = blockIdx.x * 16;
+    const T* wr = W + (size_t)min(r0 + i, rows - 1) * n + kk * 8;
+    const bool jv = b0 + i < B;                 // this lane's batch column exists
+    const float* xr = x + (size_t)min(b0 + i, B - 1) * n + kk * 8;
+    floatx4v acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+    const int nit = n >> 5;
+    constexpr int U = 4;   // slabs whose loads are in flight together
+    for (int base = wave; base < nit; base += NS * U) {
+        float w[U][8], w2[MODE == 2 ? U : 1][8], xv[U][8], gv[NORM ? U : 1][8];
+#pragma unroll
+        for (int t = 0; t < U; t++) {
+            const int k0 = min(base + t * NS, nit - 1) << 5;   // past the end: re-read the last slab, not used
+            Row8<T>::load(wr + k0, w[t]);
+            if (MODE == 2) Row8<T>::load(wr + (size_t)rows * n + k0, w2[MODE == 2 ? t : 0]);
+            Row8<float>::load(xr + k0, xv[t]);
+            if (NORM) Row8<float>::load(g + kk * 8 + k0, gv[NORM ? t : 0]);
+        }
+#pragma unroll
+        for (int t = 0; t < U; t++) {
+            if (base + t * NS >= nit) break;
+            if (NORM) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    ss += xv[t][e] * xv[t][e];
+                    xv[t][e] *= gv[NORM ? t : 0][e];
+                }
+            }
+            if (!jv) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) xv[t][e] = 0.f;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[t][e], xv[t][e], acc, 0, 0, 0);
+                if (MODE == 2) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(w2[MODE == 2 ? t : 0][e], xv[t][e], acc2, 0, 0, 0);
+            }
+        }
+    }
+    if (NORM) {
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        if (kk == 0) sspart[wave][i] = ss;
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        part[wave][lane * 4 + v] = acc[v];
+        if (MODE == 2) part[wave][256 + lane * 4 + v] = acc2[v];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // accumulator register v of lane l is row 4 * (l / 16) + v, batch column l % 16
+    float d[4], d2[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        d[v] = 0.f;
+        d2[v] = 0.f;
+        for (int w_ = 0; w_ < NS; w_++) {
+            d[v] += part[w_][lane * 4 + v];
+            if (MODE == 2) d2[v] += part[w_][256 + lane * 4 + v];
+        }
+    }
+    if (!jv) return;
+    float inv = 1.f;
+    if (NORM) {
+        float t = 0.f;
+        for (int w_ = 0; w_ < NS; w_++) t += sspart[w_][i];
+        inv = 1.0f / sqrtf(t / n + 1e-5f);
+    }
+    float* out = y + (size_t)(b0 + i) * ldy + r0 + 4 * kk;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        if (r0 + 4 * kk + v >= rows) break;
+        const float a0 = d[v] * inv;
+        if (MODE == 0) out[v] = a0;
+        else if (MODE == 1) out[v] += a0;
+        else out[v] = a0 * (1.0f / (1.0f + expf(-a0))) * (d2[v] * inv);
+    }
+}
+
 // End of a decode step, one workgroup per sequence: first-max argmax over the logits
 // (sample_argmax, llama2_sampler.cpp:25-36: strict '>' so the lowest index wins ties), record
 // the id, embed the token of the next position (forced prompt id while pos + 1 < n_prompt,
@@ -284,7 +405,7 @@ public:
     long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
                   std::vector<float>* logits, std::atomic<bool>* cancel);
     void release();
-    long profile_step(int pos, int reps, std::vector<float>* out);
+    long profile_step(int pos, int reps, int B, std::vector<float>* out);
 
 private:
     template <typename T> long upload(const float* blob);
@@ -498,6 +619,14 @@ template <int MODE, bool NORM, typename T>
 static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int B,
                                 int ldy, int rowsPerWave)
 {
+    if (B >= 2 && n % 32 == 0) {
+        // batched: matrix-core kernel, 16 sequences per pass over the weights
+        const int ns = rows >= 8192 ? 4 : 8;   // fewer, longer wavefronts once the rows alone fill the chip
+        for (int b0 = 0; b0 < B; b0 += 16) {
+            hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM>), (rows + 15) / 16, ns * 64, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, b0);
+        }
+        return hipGetLastError();
+    }
     // one row per wavefront fills the chip for the layer matrices; the classifier has rows to spare
     const bool two = rowsPerWave ? rowsPerWave == 2 : rows >= 16384;
     const int waves = two ? (rows + 1) / 2 : rows;
@@ -588,19 +717,19 @@ __global__ void noop_kernel() {}
 // returns, per kernel class: {milliseconds per step, launches per step, algorithmic bytes per step}, followed by one
 // more value: the median milliseconds an event pair measures around an empty kernel (dispatch + event cost that
 // every pair above includes).
-long Engine::profile_step(int pos, int reps, std::vector<float>* out)
+long Engine::profile_step(int pos, int reps, int B, std::vector<float>* out)
 {
     if (!loaded) return MCH_ERROR_LLM_GENERATE;
-    if (reps < 1 || pos < 0 || pos + reps > cfg.seq_len) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-    long e = ensure_state(1, cfg.seq_len);
+    if (reps < 1 || pos < 0 || pos + reps > cfg.seq_len || B < 1 || B > 64) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long e = ensure_state(B, cfg.seq_len);
     if (e) return e;
     hipStream_t s = stream;
-    std::vector<int> hp(cfg.seq_len, 1);
+    std::vector<int> hp((size_t)B * cfg.seq_len, 1);
     HIPCHK(hipMemcpyAsync(dprompt, hp.data(), hp.size() * 4, hipMemcpyHostToDevice, s));
     GenState st0 = {pos, cfg.seq_len, pos + 1, 0};
     HIPCHK(hipMemcpyAsync(dstate, &st0, sizeof(st0), hipMemcpyHostToDevice, s));
     HIPCHK(hipStreamSynchronize(s));
-    HIPCHK(embed_first(s, 1));
+    HIPCHK(embed_first(s, B));
     std::vector<float> empty;
     {
         StepProfile cal;
@@ -619,7 +748,7 @@ long Engine::profile_step(int pos, int reps, std::vector<float>* out)
         std::sort(empty.begin(), empty.end());
     }
     StepProfile prof;
-    for (int i = 0; i < reps && !e; i++) e = bf16_weights ? step<bf16_t>(s, 1, cfg.seq_len, nullptr, &prof) : step<float>(s, 1, cfg.seq_len, nullptr, &prof);
+    for (int i = 0; i < reps && !e; i++) e = bf16_weights ? step<bf16_t>(s, B, cfg.seq_len, nullptr, &prof) : step<float>(s, B, cfg.seq_len, nullptr, &prof);
     hipError_t he = hipStreamSynchronize(s);
     if (!e && he != hipSuccess) e = (long)he;
     std::vector<double> ms(SC_COUNT, 0.0), cnt(SC_COUNT, 0.0);
@@ -639,7 +768,7 @@ long Engine::profile_step(int pos, int reps, std::vector<float>* out)
     bytes[SC_MATVEC_W13] = L * 2 * hid * dim * es;
     bytes[SC_MATVEC_W2] = L * dim * hid * es;
     bytes[SC_MATVEC_CLS] = (double)cfg.vocab_size * dim * es;
-    bytes[SC_ATTN_DECODE] = L * 2 * meanLen * kvd * 4.0;
+    bytes[SC_ATTN_DECODE] = B * L * 2 * meanLen * kvd * 4.0;
     out->clear();
     for (int c = 0; c < SC_COUNT; c++) {
         out->push_back((float)(ms[c] / reps));
@@ -878,7 +1007,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         if (!m) return MCH_ERROR_PARAM;
         std::lock_guard<std::mutex> run(m->runLock);
         std::vector<float> out;
-        long e = m->engine.profile_step((int)pIn[1], (int)pIn[2], &out);
+        long e = m->engine.profile_step((int)pIn[1], (int)pIn[2], lIn > 3 ? (int)pIn[3] : 1, &out);
         if (e) return (MCH_LONG)e;
         return (MCH_LONG)give(out, ppOut, plOut);
     }

@@ -99,11 +99,11 @@ class LlmInference:
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
         return float(rg[0]), int(rg[1])
 
-    def ProfileStep(self, pos, reps=8):
+    def ProfileStep(self, pos, reps=8, batch=1):
         """Per-kernel-class timing of eager decode steps at ``pos`` (HIP event pairs around
         every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}, plus
         "_event_pair_ms": what such a pair measures around an empty kernel."""
-        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.PROFILE_STEP, self.m_rgLlm + [pos, reps])
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.PROFILE_STEP, self.m_rgLlm + [pos, reps, batch])
         out = {name: (float(rg[3 * i]), float(rg[3 * i + 1]), float(rg[3 * i + 2])) for i, name in enumerate(STEP_CLASSES)}
         out["_event_pair_ms"] = float(rg[3 * len(STEP_CLASSES)])
         return out
