@@ -187,10 +187,11 @@ __device__ __forceinline__ void decode_stream(const T* __restrict__ kc, const T*
 __device__ __forceinline__ void part_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float part_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-// Merges the 4 * (64/LPR) lane groups of a workgroup through LDS and writes {M, L, acc[hs]} to `out`.
+// Merges the 4 * (64/LPR) lane groups of a workgroup through LDS and writes {M, L, acc[hs]} to `out`, or, when
+// this workgroup saw every cached row (yfinal set), the normalised result straight to yfinal.
 template <typename T, int LPR>
 __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (&acc)[Vec16<T>::W], int wave, int grp, int gl,
-                                                 int d0, bool active, int hs, float* __restrict__ out)
+                                                 int d0, bool active, int hs, float* __restrict__ out, T* __restrict__ yfinal = nullptr)
 {
     constexpr int W = Vec16<T>::W;
     constexpr int RPW = 64 / LPR, NW = 4;
@@ -206,6 +207,17 @@ __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (
     __syncthreads();
     float M = -INFINITY;
     for (int i = 0; i < NW * RPW; i++) M = fmaxf(M, sm[i]);
+    if (yfinal) {
+        float L = 0.f;
+        for (int i = 0; i < NW * RPW; i++) L += (sm[i] > -INFINITY) ? sl[i] * __expf(sm[i] - M) : 0.f;
+        for (int d = threadIdx.x; d < hs; d += 256) {
+            float v = 0.f;
+            for (int i = 0; i < NW * RPW; i++)
+                if (sm[i] > -INFINITY) v += sacc[i][d] * __expf(sm[i] - M);
+            st1(yfinal + d, v / L);
+        }
+        return;
+    }
     if (threadIdx.x == 0) {
         float L = 0.f;
         for (int i = 0; i < NW * RPW; i++) L += (sm[i] > -INFINITY) ? sl[i] * __expf(sm[i] - M) : 0.f;
@@ -227,53 +239,65 @@ template <typename T>
 __device__ __forceinline__ void decode_merge_last(const float* part, int* counter, int splits, int hs, T* __restrict__ y)
 {
     __shared__ int ticket;
-    __shared__ float sw[256];
-    __shared__ float sred[256];
-    __shared__ float swv[8];
+    __shared__ float sM[256], sL[256], sA[256];
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (ticket != splits - 1) return;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // One round trip: thread (g, d) merges splits g, g + G, ... for output dimension d with its own running
+    // maximum, four splits' {m, l, value} loads in flight at a time; the G groups then meet in LDS.
+    const int tid = threadIdx.x;
     const int stride = hs + 2;
-    float ms = -INFINITY, ls = 0.f;
-    if (tid < splits) {
-        ms = part_load(part + (size_t)tid * stride);
-        ls = part_load(part + (size_t)tid * stride + 1);
-    }
-    float M = ms;
-    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
-    if (lane == 0) swv[wave] = M;
-    __syncthreads();
-    M = fmaxf(fmaxf(swv[0], swv[1]), fmaxf(swv[2], swv[3]));
-    const float w = ms > -INFINITY ? __expf(ms - M) : 0.f;
-    sw[tid] = w;
-    float L = ls * w;
-    for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
-    if (lane == 0) swv[4 + wave] = L;
-    __syncthreads();
-    L = (swv[4] + swv[5]) + (swv[6] + swv[7]);
-    // G groups of hs threads; group g sums splits g, g + G, ...
     const int G = hs >= 256 ? 1 : 256 / hs;
     const int g = tid / hs;
-    if (G == 1) {
-        if (g == 0 || hs > 256)
-            for (int d = tid; d < hs; d += 256) {
-                float v = 0.f;
-                for (int s = 0; s < splits; s++) v += part_load(part + (size_t)s * stride + 2 + d) * sw[s];
-                st1(y + d, v / L);
+    for (int dbase = 0; dbase < hs; dbase += 256) {
+        const int d = dbase + tid - g * hs;
+        const bool mine = g < G && d < hs;
+        float M = -INFINITY, L = 0.f, A = 0.f;
+        for (int s0 = g; s0 < splits && mine; s0 += 4 * G) {
+            float ms[4], ls[4], vs[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int sp = s0 + k * G;
+                const bool ok = sp < splits;
+                const float* p = part + (size_t)(ok ? sp : s0) * stride;
+                ms[k] = part_load(p);
+                ls[k] = part_load(p + 1);
+                vs[k] = part_load(p + 2 + d);
+                if (!ok) ms[k] = -INFINITY;
             }
-    } else {
-        const int d = tid - g * hs;
-        float v = 0.f;
-        if (g < G)
-            for (int s = g; s < splits; s += G) v += part_load(part + (size_t)s * stride + 2 + d) * sw[s];
-        sred[tid] = v;
-        __syncthreads();
-        if (g == 0) {
-            for (int k = 1; k < G; k++) v += sred[k * hs + d];
-            st1(y + d, v / L);
+            float Mn = fmaxf(fmaxf(fmaxf(M, ms[0]), fmaxf(ms[1], ms[2])), ms[3]);
+            if (Mn > -INFINITY) {
+                const float c = __expf(M - Mn);   // M == -inf gives 0
+                L *= c;
+                A *= c;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float w = ms[k] > -INFINITY ? __expf(ms[k] - Mn) : 0.f;
+                    L += ls[k] * w;
+                    A += vs[k] * w;
+                }
+                M = Mn;
+            }
+        }
+        if (G == 1) {
+            if (mine) st1(y + d, A / L);
+        } else {
+            sM[tid] = M; sL[tid] = L; sA[tid] = A;
+            __syncthreads();
+            if (g == 0 && d < hs) {
+                for (int k = 1; k < G; k++) {
+                    const float m2 = sM[k * hs + d];
+                    if (m2 > -INFINITY) {
+                        const float Mn = fmaxf(M, m2), c1 = __expf(M - Mn), c2 = __expf(m2 - Mn);
+                        L = L * c1 + sL[k * hs + d] * c2;
+                        A = A * c1 + sA[k * hs + d] * c2;
+                        M = Mn;
+                    }
+                }
+                st1(y + d, A / L);
+            }
         }
     }
     if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -306,6 +330,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
 
     int t0, t1;
     decode_range(a, split, &t0, &t1);
+    // splits that hold rows: with a device-side length the launch is sized for the longest cache and the rest idle
+    int nAct = a.splits;
+    if (a.dlen) {
+        const int len = *a.dlen;
+        int chunk = (len + a.splits - 1) / a.splits;
+        chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
+        nAct = (len + chunk - 1) / chunk;
+        if (a.counters && split >= nAct) return;
+    }
 
     float m = -INFINITY, l = 0.f, acc[W];
 #pragma unroll
@@ -314,9 +347,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
 
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+    if (a.counters && nAct == 1) {
+        decode_reduce_wg<T, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, (T*)a.y + bh * a.hs);
+        return;
+    }
     decode_reduce_wg<T, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
     if (a.counters)
-        decode_merge_last<T>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, a.splits, a.hs, (T*)a.y + bh * a.hs);
+        decode_merge_last<T>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, (T*)a.y + bh * a.hs);
 }
 
 // Engine form (fp32): one launch per layer does what the reference's decode step does between the QKV
@@ -350,6 +387,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     int chunk = (len + a.splits - 1) / a.splits;
     chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
     const int t0 = split * chunk, t1 = min(len, t0 + chunk);
+    const int nAct = (len + chunk - 1) / chunk;      // splits that hold rows; the rest of the launch idles
+    if (split >= nAct) return;
 
     // rotation factors of this lane's two adjacent pairs (dims d0, d0+1 and d0+2, d0+3) at `pos`
     float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
@@ -382,9 +421,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     decode_stream<float, LPR>(kc, vc, a.kvd, t0, t1, (unsigned)((b * a.H + h) * 37 + split * 11), wave, grp, d0, active, qv, m, l, acc);
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+    float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
+    if (nAct == 1) {
+        decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
+        return;
+    }
     decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
-    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, a.splits, a.hs,
-                             a.y + (size_t)b * a.dim + (size_t)h * a.hs);
+    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
 }
 
 // any head size / alignment: scalar loads, one wavefront per (b, h, split)
