@@ -299,36 +299,73 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_mfma_kernel(int M, int N, in
 }
 
 // ---------------------------------------------------------------------------
-// bf16 MFMA, NT, large tiles: 2 x 2 wavefronts, each owning WM x WN MFMA 32x32 tiles, so a workgroup
-// covers (64 WM) x (64 WN) of C.  A 128 x 128 wavefront tile (WM = WN = 4) reads 8 LDS fragments per 16 MFMAs,
-// a quarter of the LDS traffic per flop of the 64 x 64 wavefront tile above, which is what keeps the matrix
-// cores fed; its 256 accumulators live in the accumulation registers.  K is walked in steps of 32 through a
-// double-buffered LDS stage (one barrier per step); the next stage travels global -> registers -> LDS while
-// the current one is consumed.  Tiles are numbered so that each XCD (workgroup index mod 8) works on a
-// contiguous band of tile rows and re-uses its A rows out of its own L2.
-template <int WM, int WN, int BK, int OCC>
-__global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N, int K, float alpha, const bf16_t* __restrict__ A,
-                                                                    const bf16_t* __restrict__ B, float beta, bf16_t* __restrict__ C,
-                                                                    int tilesN, int tilesTotal)
+// MFMA, NT, large tiles, bf16 and fp32: 2 x 2 wavefronts, each owning WM x WN MFMA 32x32 tiles, so a workgroup
+// covers (64 WM) x (64 WN) of C.  A 128 x 128 wavefront tile (WM = WN = 4) reads 8 LDS fragments per 16 tile
+// products, a quarter of the LDS traffic per flop of the 64 x 64 wavefront tile, which is what keeps the matrix
+// cores fed; its 256 accumulators live in the accumulation registers.  K is walked in stages of 128 bytes per
+// row through a double-buffered LDS stage (one barrier per stage).  A k-step is one 16-byte fragment per lane
+// and operand: one v_mfma_f32_32x32x16_bf16, or four v_mfma_f32_32x32x2_f32 (lane half h holds k = 4h .. 4h+3 of
+// a group of eight and step e contracts {e, 4 + e}; the slot assignment only has to agree between A and B).
+// Tiles are numbered so that each XCD (workgroup index mod 8) works on a contiguous band of tile rows and
+// re-uses its A rows out of its own L2.
+template <typename T> struct BigTraits;
+template <> struct BigTraits<bf16_t> {
+    static constexpr int E = 8;   // elements per 16-byte chunk
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&a), *reinterpret_cast<bf16x8*>(&b), c, 0, 0, 0);
+    }
+    __device__ static inline float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+    __device__ static inline void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+    __device__ static inline void st4(bf16_t* p, float a, float b, float c, float d)
+    {
+        uint2 w;
+        w.x = pack2_bf16(a, b);
+        w.y = pack2_bf16(c, d);
+        *(uint2*)p = w;
+    }
+};
+template <> struct BigTraits<float> {
+    static constexpr int E = 4;
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+        return c;
+    }
+    __device__ static inline float ld(const float* p) { return *p; }
+    __device__ static inline void st(float* p, float v) { *p = v; }
+    __device__ static inline void st4(float* p, float a, float b, float c, float d) { *(float4*)p = make_float4(a, b, c, d); }
+};
+
+template <typename T, int WM, int WN, int OCC>
+__global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
+                                                               const T* __restrict__ B, float beta, T* __restrict__ C, int tilesN,
+                                                               int tilesTotal)
 {
-    constexpr int BM = 64 * WM, BN = 64 * WN, LDK = BK + 8;   // row stride 16 B past a power of two: conflict-free 128-bit reads
-    constexpr int CPR = BK / 8;                               // 16-byte chunks per tile row
+    typedef BigTraits<T> TR;
+    constexpr int E = TR::E;
+    constexpr int BK = 8 * E;                                 // elements per stage and row (128 bytes)
+    constexpr int BM = 64 * WM, BN = 64 * WN, LDK = BK + E;   // row stride 16 B past a power of two: conflict-free 128-bit reads
+    constexpr int CPR = 8;                                    // 16-byte chunks per tile row
     constexpr int RPP = 256 / CPR;                            // rows covered by one pass of the 256 threads
     constexpr int PA = BM / RPP, PB = BN / RPP;               // passes (16-byte chunks per thread) per operand
-    constexpr int KS = BK / 16;                               // MFMA k-steps per stage
-    constexpr int NMF = WM * WN;                              // MFMAs per k-step
-    static_assert(KS >= 2 && (KS % 2) == 0, "stage = an even number of k-steps");
-    static_assert(NMF >= WM + WN && NMF * (KS / 2) >= PA + PB, "not enough MFMAs per k-step to carry the memory instructions");
-    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
-    bf16_t* As = smem;                        // [2][BM * LDK]
-    bf16_t* Bs = smem + 2 * BM * LDK;         // [2][BN * LDK]
+    constexpr int KS = 4;                                     // k-steps (fragments of 2 E elements) per stage
+    constexpr int NMF = WM * WN;                              // tile products per k-step
+    static_assert(NMF >= WM + WN && NMF * (KS / 2) >= PA + PB, "not enough tile products per k-step to carry the memory instructions");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    T* As = smem;                        // [2][BM * LDK]
+    T* Bs = smem + 2 * BM * LDK;         // [2][BN * LDK]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int per = (tilesTotal + 7) / 8;
     const int tile = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
     if (tile >= tilesTotal) return;
     const int m0 = (tile / tilesN) * BM, n0 = (tile % tilesN) * BN;
     const int wm = (wave >> 1) * (32 * WM), wn = (wave & 1) * (32 * WN);
-    const int lr = tid / CPR, lc = (tid % CPR) * 8;
+    const int lr = tid / CPR, lc = (tid % CPR) * E;
 
     floatx16 acc[WM][WN];
 #pragma unroll
@@ -339,14 +376,14 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     // rows past the matrix edge are clamped: they are loaded (valid memory) and never stored
-    const bf16_t* ga[PA];
-    const bf16_t* gb[PB];
+    const T* ga[PA];
+    const T* gb[PB];
 #pragma unroll
     for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * K + lc;
 #pragma unroll
     for (int p = 0; p < PB; p++) gb[p] = B + (size_t)min(n0 + lr + p * RPP, N - 1) * K + lc;
-    bf16_t* sa = As + lr * LDK + lc;
-    bf16_t* sb = Bs + lr * LDK + lc;
+    T* sa = As + lr * LDK + lc;
+    T* sb = Bs + lr * LDK + lc;
     u32x4 ra[PA], rb[PB];
 
     const int nk = K / BK;
@@ -367,12 +404,12 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
         for (int p = 0; p < PB; p++) rb[p] = *(const u32x4*)(gb[p] + k1);
     }
     __syncthreads();
-    const int fr = lane & 31, fg = (lane >> 5) * 8;
-    const bf16_t* fa = As + (wm + fr) * LDK + fg;
-    const bf16_t* fb = Bs + (wn + fr) * LDK + fg;
-    bf16x8 a[2][WM], b[2][WN];
-    // One stage: KS k-steps of NMF MFMAs on LDS buffer kt & 1.  Riding along between the MFMAs (the wavefront is
-    // alone on its SIMD, so whatever it issues between two MFMAs is hidden behind the first one's 8 passes, and
+    const int fr = lane & 31, fg = (lane >> 5) * E;
+    const T* fa = As + (wm + fr) * LDK + fg;
+    const T* fb = Bs + (wn + fr) * LDK + fg;
+    u32x4 a[2][WM], b[2][WN];
+    // One stage: KS k-steps of NMF tile products on LDS buffer kt & 1.  Riding along between them (the wavefront
+    // is alone on its SIMD, so whatever it issues between two MFMAs is hidden behind the first one's passes, and
     // whatever it issues in a block of its own is not):
     //   first half of the k-steps : the registers holding stage kt + 1 go to the other LDS buffer
     //   second half               : stage kt + 2 is fetched from global memory into those registers
@@ -380,15 +417,15 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
     // Past the end of K the extra fetches re-read the last stage (valid memory, never consumed).
     for (int kt = 0; kt < nk; kt++) {
         const int buf = kt & 1;
-        const bf16_t* pa = fa + buf * BM * LDK;
-        const bf16_t* pb = fb + buf * BN * LDK;
-        bf16_t* wa = sa + (buf ^ 1) * BM * LDK;
-        bf16_t* wb = sb + (buf ^ 1) * BN * LDK;
+        const T* pa = fa + buf * BM * LDK;
+        const T* pb = fb + buf * BN * LDK;
+        T* wa = sa + (buf ^ 1) * BM * LDK;
+        T* wb = sb + (buf ^ 1) * BN * LDK;
         const int k2 = min(kt + 2, nk - 1) * BK;
 #pragma unroll
-        for (int t = 0; t < WM; t++) a[0][t] = *(const bf16x8*)(pa + t * 32 * LDK);
+        for (int t = 0; t < WM; t++) a[0][t] = *(const u32x4*)(pa + t * 32 * LDK);
 #pragma unroll
-        for (int t = 0; t < WN; t++) b[0][t] = *(const bf16x8*)(pb + t * 32 * LDK);
+        for (int t = 0; t < WN; t++) b[0][t] = *(const u32x4*)(pb + t * 32 * LDK);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int cur = ks & 1, nxt = cur ^ 1;
@@ -396,15 +433,15 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
             constexpr int HALF = KS / 2;
             const int part = ks % HALF;
             const int c0 = (PA + PB) * part / HALF, c1 = (PA + PB) * (part + 1) / HALF;
-            // written in issue order, one small scheduling region per MFMA so that the order stays as written:
-            // MFMA q, then the q-th fragment read of the next k-step, then the q-th staging instruction
+            // written in issue order, one small scheduling region per tile product so that the order stays as
+            // written: product q, then the q-th fragment read of the next k-step, then the q-th staging instruction
 #pragma unroll
             for (int q = 0; q < NMF; q++) {
                 const int i = q / WN, j = q % WN;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[cur][j], a[cur][i], acc[i][j], 0, 0, 0);
+                acc[i][j] = TR::mma(b[cur][j], a[cur][i], acc[i][j]);
                 if (ks + 1 < KS) {
-                    if (q < WM) a[nxt][q] = *(const bf16x8*)(pa + q * 32 * LDK + (ks + 1) * 16);
-                    else if (q < WM + WN) b[nxt][q - WM] = *(const bf16x8*)(pb + (q - WM) * 32 * LDK + (ks + 1) * 16);
+                    if (q < WM) a[nxt][q] = *(const u32x4*)(pa + q * 32 * LDK + (ks + 1) * 2 * E);
+                    else if (q < WM + WN) b[nxt][q - WM] = *(const u32x4*)(pb + (q - WM) * 32 * LDK + (ks + 1) * 2 * E);
                 }
                 const int c = c0 + q;
                 if (c < c1) {
@@ -421,37 +458,35 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
         }
         __syncthreads();
     }
-    // The MFMAs above compute the TRANSPOSED 32x32 tiles (B fragment as the row operand), so a lane owns one
+    // The tile products above are the TRANSPOSED 32x32 tiles (B fragment as the row operand), so a lane owns one
     // row of C (lane%32) and register v is column 8*(v/4) + 4*(lane/32) + v%4: four consecutive columns per
     // register quad.
     const int row_l = lane & 31, col_l = (lane >> 5) * 4;
-    if (m0 + BM <= M && n0 + BN <= N && beta == 0.f && (N & 7) == 0 && (((uintptr_t)C) & 15) == 0) {
-        // interior tile: each wavefront passes its tile through its own slice of LDS (free after the last
-        // barrier) and writes whole 16-byte pieces of rows, 64 lanes covering full cache lines
-        constexpr int CW = 32 * WN, LDC = CW + 8;
-        constexpr int LPR = CW / 8, RPI = 64 / LPR;            // lanes per row, rows per store instruction
-        bf16_t* cs = smem + wave * (32 * WM) * LDC;
+    if (m0 + BM <= M && n0 + BN <= N && beta == 0.f && (N % E) == 0 && (((uintptr_t)C) & 15) == 0) {
+        // interior tile: each wavefront passes its tile, 32 rows at a time, through its own slice of LDS (free
+        // after the last barrier) and writes whole 16-byte pieces of rows, the lanes covering full cache lines
+        constexpr int CW = 32 * WN, LDC = CW + E;
+        constexpr int LPR = CW / E, RPI = 64 / LPR;            // lanes per row, rows per store instruction
+        constexpr int NIT = (32 + RPI - 1) / RPI;
+        T* cs = smem + wave * 32 * LDC;
+        const int rr = lane / LPR, cc = (lane % LPR) * E;
 #pragma unroll
-        for (int i = 0; i < WM; i++)
+        for (int i = 0; i < WM; i++) {
 #pragma unroll
             for (int j = 0; j < WN; j++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    uint2 w;
-                    w.x = pack2_bf16(alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1]);
-                    w.y = pack2_bf16(alpha * acc[i][j][4 * g + 2], alpha * acc[i][j][4 * g + 3]);
-                    *(uint2*)(cs + (i * 32 + row_l) * LDC + j * 32 + 8 * g + col_l) = w;
-                }
-        // same wavefront wrote and reads: LDS operations of one wavefront complete in order
-        const int rr = lane / LPR, cc = (lane % LPR) * 8;
-        bf16_t* cg = C + (size_t)(m0 + wm + rr) * N + n0 + wn + cc;
-        constexpr int NIT = (32 * WM + RPI - 1) / RPI;
+                for (int g = 0; g < 4; g++)
+                    TR::st4(cs + row_l * LDC + j * 32 + 8 * g + col_l, alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1],
+                            alpha * acc[i][j][4 * g + 2], alpha * acc[i][j][4 * g + 3]);
+            // same wavefront wrote and reads: LDS operations of one wavefront complete in order
+            T* cg = C + (size_t)(m0 + wm + i * 32 + rr) * N + n0 + wn + cc;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            // lanes past RPI * LPR (row widths that do not divide 64) and rows past the tile stay idle
-            if (rr < RPI && it * RPI + rr < 32 * WM) {
-                const u32x4 v = *(const u32x4*)(cs + (it * RPI + rr) * LDC + cc);
-                *(u32x4*)(cg + (size_t)it * RPI * N) = v;
+            for (int it = 0; it < NIT; it++) {
+                // lanes past RPI * LPR (row widths that do not divide 64) and rows past the block stay idle
+                if (rr < RPI && it * RPI + rr < 32) {
+                    const u32x4 v = *(const u32x4*)(cs + (it * RPI + rr) * LDC + cc);
+                    *(u32x4*)(cg + (size_t)it * RPI * N) = v;
+                }
             }
         }
         return;
@@ -469,31 +504,32 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_bf16_big_kernel(int M, int N
                 if (c < N) {
                     const size_t ci = (size_t)r * N + c;
                     float o = alpha * acc[i][j][v];
-                    if (beta != 0.f) o += beta * bf16_to_f32(C[ci]);
-                    C[ci] = f32_to_bf16(o);
+                    if (beta != 0.f) o += beta * TR::ld(C + ci);
+                    TR::st(C + ci, o);
                 }
             }
         }
 }
 
-template <int WM, int WN, int BK, int OCC>
-static hipError_t launch_big_bf16(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C)
+template <typename T, int WM, int WN, int OCC>
+static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C)
 {
+    constexpr int E = BigTraits<T>::E;
     const int tm = (m + 64 * WM - 1) / (64 * WM), tn = (n + 64 * WN - 1) / (64 * WN);
     const long long total = (long long)tm * tn;
     if (total > (1ll << 30)) return hipErrorInvalidValue;
     const int per = (int)((total + 7) / 8);
-    size_t lds = (size_t)2 * (64 * WM + 64 * WN) * (BK + 8) * sizeof(bf16_t);
-    const size_t ldsEpilogue = (size_t)4 * (32 * WM) * (32 * WN + 8) * sizeof(bf16_t);
+    size_t lds = (size_t)2 * (64 * WM + 64 * WN) * (9 * E) * sizeof(T);
+    const size_t ldsEpilogue = (size_t)4 * 32 * (32 * WN + E) * sizeof(T);
     if (ldsEpilogue > lds) lds = ldsEpilogue;
     static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
     if (!attr) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_bf16_big_kernel<WM, WN, BK, OCC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr = true;
     }
-    hipLaunchKernelGGL((gemm_nt_bf16_big_kernel<WM, WN, BK, OCC>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const bf16_t*)A,
-                       (const bf16_t*)B, beta, (bf16_t*)C, tn, (int)total);
+    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
+                       (T*)C, tn, (int)total);
     return hipGetLastError();
 }
 
@@ -508,20 +544,26 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
     if (!tA && tB && aligned) {
         dim3 grid((n + 127) / 128, (m + 127) / 128);
         if (grid.y > 65535) return hipErrorInvalidValue;
-        if (dt == F32)
+        // Large-tile kernels need whole 128-byte stages along K.  256 x 256 tiles (one wavefront per SIMD, 128 x 128
+        // per wavefront) win once K is long enough to amortise their prologue and the tile count fills the 256 CUs
+        // evenly; 128 x 128 tiles with two workgroups per CU otherwise, 128 x 192 when that gives at most one round
+        // of workgroups.
+        const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+        const double fill = (double)t256 / (double)(((t256 + 255) / 256) * 256);
+        const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+        if (dt == F32) {
+            if (k % 32 == 0) {
+                if (k >= 1024 && fill >= 0.85) return launch_big<float, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
+                if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
+                return launch_big<float, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
+            }
             hipLaunchKernelGGL(gemm_nt_f32_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const float*)A, (const float*)B,
                                beta, (float*)C);
-        else {
-            if (k % 64 == 0 && ((uintptr_t)C % 4) == 0) {
-                // 256 x 256 tiles (one wavefront per SIMD, 128 x 128 per wavefront) win once K is long enough to
-                // amortise their prologue and the tile count fills the 256 CUs evenly; 128 x 128 tiles with two
-                // workgroups per CU otherwise, 128 x 192 when that gives at most one round of workgroups.
-                const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
-                const double fill = (double)t256 / (double)(((t256 + 255) / 256) * 256);
-                if (k >= 2048 && fill >= 0.85) return launch_big_bf16<4, 4, 64, 1>(s, m, n, k, alpha, A, B, beta, C);
-                const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-                if (n % 192 == 0 && t128 <= 512) return launch_big_bf16<2, 3, 64, 2>(s, m, n, k, alpha, A, B, beta, C);
-                return launch_big_bf16<2, 2, 64, 2>(s, m, n, k, alpha, A, B, beta, C);
+        } else {
+            if (k % 64 == 0) {
+                if (k >= 2048 && fill >= 0.85) return launch_big<bf16_t, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
+                if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
+                return launch_big<bf16_t, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }
             hipLaunchKernelGGL(gemm_nt_bf16_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const bf16_t*)A,
                                (const bf16_t*)B, beta, (bf16_t*)C);

@@ -132,6 +132,24 @@ def test_gemm_bf16_inner_product_shape(dev, m, n, k):
     (1024, 1024, 2048, 1.0, 0.0),   # long K: 256 x 256 tiles
     (260, 132, 64, 0.25, -1.0),     # ragged, both scalars
 ])
+def test_gemm_fp32_large_tile_paths(dev, m, n, k, alpha, beta):
+    rng = np.random.default_rng(m + n + k + 1)
+    A = rng.standard_normal((m, k)).astype(np.float32)
+    B = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    hA, hB, hC = dev.put(A), dev.put(B), dev.put(C0)
+    dev.cuda.gemm(False, True, m, n, k, alpha, hA, hB, beta, hC)
+    ref = R.gemm(False, True, m, n, k, alpha, A, B, beta, C0, dtype=np.float64)
+    assert_close(dev.get(hC, (m, n)), ref, FP32_RTOL, "gemm fp32 large tiles")
+
+
+@pytest.mark.parametrize("m,n,k,alpha,beta", [
+    (300, 200, 128, 1.0, 0.0),
+    (512, 768, 192, 0.5, 0.0),
+    (384, 256, 64, 1.0, 2.0),
+    (1024, 1024, 2048, 1.0, 0.0),
+    (260, 132, 64, 0.25, -1.0),
+])
 def test_gemm_bf16_large_tile_paths(dev, m, n, k, alpha, beta):
     rng = np.random.default_rng(m + n + k)
     A = bf16_round(rng.standard_normal((m, k)).astype(np.float32))
