@@ -50,6 +50,7 @@ enum {
     MCH_ERROR_ATTN_INVALID_BLOCK_SIZE = 90285,
     MCH_ERROR_EXTENSION_NOT_INITIALIZED = 90401,
     /* llama2 extension (CudaExtension.llm32.llama2/Files/llm.h:15-19) */
+    MCH_ERROR_LLM_RENDERED_PROMPT_TO_LONG = 10000,
     MCH_ERROR_LLM_LOAD_MODEL = 10001,
     MCH_ERROR_LLM_MISSING_MODEL_FILE = 10002,
     MCH_ERROR_LLM_MISSING_TOKENIZER_FILE = 10003,
@@ -194,7 +195,7 @@ enum {
     MCH_LLM_DESTROY = 2,        /* f{hLlm} */
     MCH_LLM_LOAD = 3,           /* Ex: f{hLlm}, "model.bin;tokenizer.bin" */
     MCH_LLM_QUERYSTATUS = 4,    /* f{hLlm} -> f{pct, status} */
-    MCH_LLM_GENERATE = 5,       /* Ex: f{hLlm}, prompt text */
+    MCH_LLM_GENERATE = 5,       /* Ex: f{hLlm}, prompt text (needs a tokenizer file at LOAD; greedy only) */
     MCH_LLM_QUERYRESPONSE = 6,  /* Ex: f{hLlm} -> text in szOutput, *ppOutput = end flag */
     MCH_LLM_ABORT = 7,          /* f{hLlm} */
     /* No counterpart in the reference: token-id front door used where no
@@ -213,12 +214,15 @@ enum {
      *   PROFILE_STEP  f{hLlm, pos, reps[, batch]} -> per kernel class of one decode step
      *                 f{ms per step, launches per step, algorithmic bytes per step}, classes in
      *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,
-     *                 w2, classifier, embed+argmax */
+     *                 w2, classifier, embed+argmax
+     *   TOKENIZE      Ex: f{hLlm, bos(0|1), eos(0|1)} + text -> f{token ids};
+     *                 f{hLlm, -1, prevToken, token} -> the token's piece in szOutput */
     MCH_LLM_GENERATE_IDS = 100,
     MCH_LLM_SET_OPTION = 101,
     MCH_LLM_GENERATE_BATCH = 102,
     MCH_LLM_QUERY_TIMING = 103,
-    MCH_LLM_PROFILE_STEP = 104
+    MCH_LLM_PROFILE_STEP = 104,
+    MCH_LLM_TOKENIZE = 105
 };
 
 MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);

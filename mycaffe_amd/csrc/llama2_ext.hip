@@ -24,6 +24,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <string>
@@ -31,6 +32,7 @@
 #include <vector>
 
 #include "../../include/mycaffe_hip_abi.h"
+#include "bpe_tokenizer.h"
 #include "kernels.h"
 
 namespace mch {
@@ -403,7 +405,8 @@ public:
     ~Engine() { release(); }
     long load(const char* path);
     long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
-                  std::vector<float>* logits, std::atomic<bool>* cancel);
+                  std::vector<float>* logits, std::atomic<bool>* cancel, int chunk = 0,
+                  const std::function<bool(const int*, int, int)>& onChunk = nullptr);
     void release();
     long profile_step(int pos, int reps, int B, std::vector<float>* out);
 
@@ -780,7 +783,8 @@ long Engine::profile_step(int pos, int reps, int B, std::vector<float>* out)
 }
 
 long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
-                      std::vector<float>* outLogits, std::atomic<bool>* cancel)
+                      std::vector<float>* outLogits, std::atomic<bool>* cancel, int chunk,
+                      const std::function<bool(const int*, int, int)>& onChunk)
 {
     if (!loaded) return MCH_ERROR_LLM_GENERATE;
     if (B < 1 || B > 64 || nSteps < 1 || nSteps > cfg.seq_len || nPrompt < 1 || nPrompt > cfg.seq_len) return MCH_ERROR_PARAM_OUT_OF_RANGE;
@@ -831,6 +835,15 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         } else e = enqueue();
         done++;
         if (cancel && (i & 15) == 15 && cancel->load()) break;
+        if (onChunk && chunk > 0 && (done % chunk == 0 || done == nSteps)) {
+            // hand the ids of sequence 0 chosen so far to the caller, who may stop the generation (end of text)
+            const int from = done - ((done % chunk == 0) ? chunk : done % chunk);
+            std::vector<int> part((size_t)done);
+            hipError_t hc = hipStreamSynchronize(s);
+            if (hc == hipSuccess) hc = hipMemcpy(part.data(), dout, part.size() * 4, hipMemcpyDeviceToHost);
+            if (hc != hipSuccess) { e = (long)hc; break; }
+            if (!onChunk(part.data(), from, done)) break;
+        }
     }
     (void)hipEventRecord(evB, s);
     hipError_t he = hipStreamSynchronize(s);
@@ -865,6 +878,7 @@ struct Llm {
     float temperature = 1.0f, topp = 0.9f;
     long seed = 0;
     Engine engine;
+    BpeTokenizer tokenizer;
     std::atomic<bool> cancel{false};
     std::atomic<bool> busy{false};
     std::atomic<bool> loaded{false};
@@ -890,19 +904,73 @@ static Llm* find_llm(long h)
     return it == g_llms.end() ? nullptr : it->second;
 }
 
+// UTF-8 -> UTF-16 into a caller buffer (malformed bytes become U+FFFD).  The reference converts through the ANSI
+// code page (A2T / T2A); UTF-8 keeps every prompt and response byte intact instead.
 static void put_text(MCH_TCHAR* out, long max, const char* s)
 {
     if (!out || max <= 0) return;
-    long i = 0;
-    for (; s[i] && i < max - 1; i++) out[i] = (MCH_TCHAR)(unsigned char)s[i];
-    out[i] = 0;
+    long o = 0;
+    const unsigned char* p = (const unsigned char*)s;
+    while (*p && o < max - 1) {
+        // one code point, or U+FFFD for the longest prefix of an ill-formed sequence (the usual decoder practice)
+        uint32_t cp = 0xFFFD;
+        int n = 1;
+        const unsigned char b0 = *p;
+        int need = 0;
+        unsigned char lo = 0x80, hi = 0xBF;
+        if (b0 < 0x80) cp = b0;
+        else if (b0 >= 0xC2 && b0 <= 0xDF) need = 1;
+        else if (b0 >= 0xE0 && b0 <= 0xEF) { need = 2; if (b0 == 0xE0) lo = 0xA0; if (b0 == 0xED) hi = 0x9F; }
+        else if (b0 >= 0xF0 && b0 <= 0xF4) { need = 3; if (b0 == 0xF0) lo = 0x90; if (b0 == 0xF4) hi = 0x8F; }
+        if (need) {
+            uint32_t v = b0 & (need == 1 ? 0x1Fu : need == 2 ? 0x0Fu : 0x07u);
+            int k = 1;
+            for (; k <= need; k++) {
+                const unsigned char bk = p[k];
+                const unsigned char l = k == 1 ? lo : 0x80, h = k == 1 ? hi : 0xBF;
+                if (bk < l || bk > h) break;
+                v = (v << 6) | (bk & 0x3Fu);
+            }
+            if (k > need) { cp = v; n = need + 1; }
+            else n = k;      // the bytes before the offending one form the ill-formed prefix
+        }
+        if (cp >= 0x10000) {
+            if (o >= max - 2) break;
+            cp -= 0x10000;
+            out[o++] = (MCH_TCHAR)(0xD800 + (cp >> 10));
+            out[o++] = (MCH_TCHAR)(0xDC00 + (cp & 0x3FF));
+        } else out[o++] = (MCH_TCHAR)cp;
+        p += n;
+    }
+    out[o] = 0;
 }
 
+// UTF-16 -> UTF-8
 static std::string narrow(const MCH_TCHAR* s)
 {
     std::string o;
-    if (s) for (; *s; s++) o += (char)(*s < 0x80 ? *s : '?');
+    if (!s) return o;
+    for (; *s; s++) {
+        uint32_t cp = *s;
+        if (cp >= 0xD800 && cp < 0xDC00 && s[1] >= 0xDC00 && s[1] < 0xE000) { cp = 0x10000 + ((cp - 0xD800) << 10) + (s[1] - 0xDC00); s++; }
+        if (cp < 0x80) o += (char)cp;
+        else if (cp < 0x800) { o += (char)(0xC0 | (cp >> 6)); o += (char)(0x80 | (cp & 0x3F)); }
+        else if (cp < 0x10000) { o += (char)(0xE0 | (cp >> 12)); o += (char)(0x80 | ((cp >> 6) & 0x3F)); o += (char)(0x80 | (cp & 0x3F)); }
+        else { o += (char)(0xF0 | (cp >> 18)); o += (char)(0x80 | ((cp >> 12) & 0x3F)); o += (char)(0x80 | ((cp >> 6) & 0x3F)); o += (char)(0x80 | (cp & 0x3F)); }
+    }
     return o;
+}
+
+// number of leading bytes of s that end on a code-point boundary (a trailing incomplete sequence is left out)
+static size_t utf8_complete_prefix(const std::string& s)
+{
+    size_t n = s.size(), i = n;
+    int back = 0;
+    while (i > 0 && back < 4 && ((unsigned char)s[i - 1] & 0xC0) == 0x80) { i--; back++; }
+    if (i == 0) return n;
+    const unsigned char lead = (unsigned char)s[i - 1];
+    int need = lead < 0x80 ? 1 : (lead & 0xE0) == 0xC0 ? 2 : (lead & 0xF0) == 0xE0 ? 3 : (lead & 0xF8) == 0xF0 ? 4 : 1;
+    return (int)(n - (i - 1)) < need ? i - 1 : n;
 }
 
 static long give(const std::vector<float>& v, float** ppOut, MCH_LONG* plOut)
@@ -1073,25 +1141,94 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         std::lock_guard<std::mutex> run(m->runLock);
         m->busy.store(true);
         long e = m->engine.load(model.c_str());
+        if (!e && !tok.empty() && !m->tokenizer.load(tok.c_str(), m->engine.cfg.vocab_size)) e = MCH_ERROR_LLM_LOAD_MODEL;
         m->busy.store(false);
         m->loaded.store(e == 0);
         return (MCH_LONG)e;
     }
-    case MCH_LLM_GENERATE:
-        // text prompts need the BPE tokenizer of the reference (llama2_tokenizer.cpp), which is not
-        // part of the attention path; token ids go through MCH_LLM_GENERATE_IDS
-        put_text(szErr, errMax, "Text generation needs the tokenizer, which this build does not include; use the token-id entry.");
-        return MCH_ERROR_NOT_IMPLEMENTED;
+    case MCH_LLM_GENERATE: {
+        // LLMData::Generate (llm.cpp:193-263): encode the rendered prompt with BOS, force its tokens, then feed
+        // back the sampled token; from the last prompt position on every sampled token that is not EOS (2)
+        // appends its piece to the response; stop at EOS, at the step limit or on ABORT.  The device loop runs
+        // in chunks of 32 positions, so the response grows while the caller polls QUERY_RESPONSE.
+        if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
+        if (!m->tokenizer.loaded()) {
+            put_text(szErr, errMax, "No tokenizer file was given at LOAD; use the token-id entry.");
+            return MCH_ERROR_LLM_MISSING_TOKENIZER_FILE;
+        }
+        if (m->temperature != 0.f) {
+            put_text(szErr, errMax, "Only greedy decoding (temperature 0) is implemented.");
+            return MCH_ERROR_NOT_IMPLEMENTED;
+        }
+        const std::string prompt = narrow(szIn);
+        if (prompt.size() > 4096) return MCH_ERROR_LLM_RENDERED_PROMPT_TO_LONG;
+        std::lock_guard<std::mutex> run(m->runLock);
+        m->end.store(false);
+        m->cancel.store(false);
+        m->busy.store(true);
+        const std::vector<int> toks = m->tokenizer.encode(prompt, true, false);
+        const int nP = (int)toks.size();
+        const int steps = std::min(2048, m->engine.cfg.seq_len);
+        long e = 0;
+        if (nP > steps) e = MCH_ERROR_LLM_RENDERED_PROMPT_TO_LONG;
+        for (int t : toks)
+            if (t < 0 || t >= m->engine.cfg.vocab_size) e = MCH_ERROR_LLM_GENERATE;   // e.g. a vocabulary without the " " entry
+        if (!e) {
+            std::vector<int> ids;
+            auto onChunk = [&](const int* out, int from, int to) -> bool {
+                for (int pos = from; pos < to; pos++) {
+                    const int token = pos < nP ? toks[pos] : out[pos - 1];
+                    const int next = out[pos];
+                    if (pos + 1 >= nP && next != 2) {
+                        const std::string piece = m->tokenizer.decode(token, next);
+                        std::lock_guard<std::mutex> g(m->responseLock);
+                        m->response += piece;
+                    }
+                    if (token == 2 || next == 2) return false;
+                }
+                return !m->cancel.load();
+            };
+            e = m->engine.generate(toks.data(), 1, nP, steps, false, &ids, nullptr, &m->cancel, 32, onChunk);
+            if (m->cancel.load()) {
+                std::lock_guard<std::mutex> g(m->responseLock);
+                m->response.clear();
+            }
+        }
+        m->busy.store(false);
+        m->end.store(true);
+        return (MCH_LONG)e;
+    }
+    case MCH_LLM_TOKENIZE: {
+        // f{hLlm, bos, eos} + text -> token ids; f{hLlm, -1, prev, token} -> the piece in szOutput
+        if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        if (!m->tokenizer.loaded()) return MCH_ERROR_LLM_MISSING_TOKENIZER_FILE;
+        if (pIn[1] < 0.f) {
+            if (lIn < 4) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            put_text(szOut, outMax, m->tokenizer.decode((int)pIn[2], (int)pIn[3]).c_str());
+            return 0;
+        }
+        const std::vector<int> toks = m->tokenizer.encode(narrow(szIn), pIn[1] != 0.f, pIn[2] != 0.f);
+        return (MCH_LONG)give(std::vector<float>(toks.begin(), toks.end()), ppOut, plOut);
+    }
     case MCH_LLM_QUERYRESPONSE: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         Llm* m = find_llm((long)pIn[0]);
         long end = 1;
         if (m) {
             std::lock_guard<std::mutex> g(m->responseLock);
-            put_text(szOut, outMax, m->response.c_str());
-            m->response.clear();
             end = m->end.load() ? 1 : 0;
-            m->end.store(false);
+            // hand out whole code points only while the generation is still running (byte tokens arrive one at a time),
+            // and no more than fits the caller's buffer (llm.cpp:272-283)
+            size_t n = end ? m->response.size() : utf8_complete_prefix(m->response);
+            if (outMax > 0 && n > (size_t)(outMax - 1)) { n = utf8_complete_prefix(m->response.substr(0, (size_t)(outMax - 1))); end = 0; }
+            put_text(szOut, outMax, m->response.substr(0, n).c_str());
+            m->response.erase(0, n);
+            if (end) m->end.store(false);
         }
         if (ppOut) *ppOut = (float*)end;  // the end flag travels through the pointer (CudaExtension.llm32.cpp:257-258)
         return 0;

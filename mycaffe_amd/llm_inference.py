@@ -24,6 +24,7 @@ class CUDAFN_EXTENSION_LLM:
     GENERATE_BATCH = 102
     QUERY_TIMING = 103
     PROFILE_STEP = 104
+    TOKENIZE = 105
 
 
 STEP_CLASSES = ("matvec_qkv", "rope_store", "attn_decode", "matvec_wo", "matvec_w13", "matvec_w2", "matvec_cls", "embed_argmax")
@@ -76,6 +77,16 @@ class LlmInference:
         text = self.m_cuda.QueryExtensionStrings(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_RESPONSE, [int(self.m_rgLlm[0])])[0]
         end = text.endswith("\n[END]")
         return (text[:-6] if end else text), end
+
+    def Tokenize(self, strText, bBos=True, bEos=False):
+        """Token ids of ``strText`` from the tokenizer given at Load (addition of this library)."""
+        rg = self.m_cuda.RunExtensionEx(self.m_hExtension, CUDAFN_EXTENSION_LLM.TOKENIZE, self.m_rgLlm + [int(bBos), int(bEos)], strText)
+        return rg.astype(np.int32)
+
+    def DecodePiece(self, nPrevToken, nToken):
+        """The text piece a token contributes after ``nPrevToken`` (addition of this library)."""
+        return self.m_cuda.QueryExtensionStrings(self.m_hExtension, CUDAFN_EXTENSION_LLM.TOKENIZE,
+                                                 [int(self.m_rgLlm[0]), -1, int(nPrevToken), int(nToken)])[0]
 
     def GenerateIds(self, prompt_ids, nSteps, want_logits=False, vocab_size=None):
         """Greedy decode from token ids; returns the id sampled after every position

@@ -134,3 +134,85 @@ def test_error_paths(llm, tmp_path):
     text, end = llm.QueryResponse()
     assert text == "" and not end or end
     llm.CancelGenerate()
+
+
+# ---- tokenizer and the text entry points (GENERATE / QUERY_RESPONSE) -------------------------------------
+
+def _vocab(n):
+    """259 specials + byte tokens, then words and word pieces, padded to n entries."""
+    vocab = [b"<unk>", b"<s>", b"</s>"] + [("<0x%02X>" % b).encode() for b in range(256)]
+    scores = [0.0] * len(vocab)
+    pieces = [b" ", b"e", b"t", b"a", b"o", b"h", b"l", b"r", b"w", b"d", b"th", b"he", b"ll", b"lo", b" w", b" h", b"the", b" the",
+              b"hello", b" hello", b"wor", b"world", b" world", b"ld", "é".encode(), b"!", b"?", b",", b" a", b"at", b" cat", b"c"]
+    for i, p in enumerate(pieces):
+        vocab.append(p)
+        scores.append(-1.0 - 0.37 * ((i * 7) % 11) - 0.01 * i)
+    i = 0
+    while len(vocab) < n:
+        vocab.append(b"~pad%d" % i)
+        scores.append(-50.0 - i)
+        i += 1
+    return vocab[:n], scores[:n]
+
+
+def test_text_generation_matches_checker(llm, tmp_path):
+    from oracle import tokenizer_ref as TK
+    cfg = dict(dim=64, hidden_dim=172, n_layers=2, n_heads=4, n_kv_heads=4, vocab_size=320, seq_len=96)
+    vocab, scores = _vocab(cfg["vocab_size"])
+    tok_path = str(tmp_path / "tok.bin")
+    TK.write_tokenizer(tok_path, vocab, scores)
+    tok = TK.Tokenizer(vocab, scores)
+    prompts = ["hello world", "the cat, hello?", "héllo wörld ☃!", ""]
+    # pick weights whose greedy continuation of the first prompt reaches the end-of-text id inside the context,
+    # so the early stop is exercised (searched on the CPU checker)
+    chosen = None
+    for seed in range(60):
+        blob, _ = O.random_weights(cfg, seed=seed, shared_classifier=False, std=0.3)
+        ids = O.Llama(cfg, blob, False).generate_greedy(tok.encode(prompts[0], True, False), cfg["seq_len"])
+        n = len(tok.encode(prompts[0], True, False))
+        if chosen is None:
+            chosen = (seed, blob)
+        if 2 in list(ids[n - 1:]):
+            chosen = (seed, blob)
+            break
+    seed, blob = chosen
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, cfg, blob, False)
+    inf = llm
+    inf.Load(ckpt, tok_path)
+    if True:
+        for text in prompts + ["ab\tc déjà vu", " leading and  double  spaces "]:
+            assert list(inf.Tokenize(text, True, False)) == tok.encode(text, True, False), text
+            assert list(inf.Tokenize(text, False, True)) == tok.encode(text, False, True), text
+        for prev, t in [(1, 259), (5, 259), (0, 3 + 0x41), (0, 270), (1, 280)]:
+            assert inf.DecodePiece(prev, t).encode("utf-8") == tok.decode(prev, t)
+        for text in prompts:
+            ref = TK.generate_text(O.Llama(cfg, blob, False), tok, text, cfg["seq_len"])
+            inf.Generate(text)
+            got, end, polls = "", False, 0
+            while not end and polls < 50:
+                part, end = inf.QueryResponse()
+                got += part
+                polls += 1
+            assert end
+            assert got.encode("utf-8") == ref.decode("utf-8", errors="replace").encode("utf-8"), (text, got, ref)
+
+
+def test_text_generation_errors(llm, tmp_path):
+    cfg = dict(TINY)
+    blob, _ = O.random_weights(cfg, seed=1, shared_classifier=False, std=0.3)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, cfg, blob, False)
+    inf = llm
+    inf.Load(ckpt)                       # no tokenizer file: token-id front door only
+    with pytest.raises(CudaDnnError) as e:
+        inf.Generate("hello")
+    assert e.value.code == 10003         # ERROR_LLM_LOAD_MODEL_MISSING_TOKENIZER_FILE
+    with pytest.raises(CudaDnnError) as e:
+        inf.Load(ckpt, str(tmp_path / "absent.bin"))
+    assert e.value.code == 10003
+    short = str(tmp_path / "short.bin")
+    open(short, "wb").write(b"\x04\x00\x00\x00abc")
+    with pytest.raises(CudaDnnError) as e:
+        inf.Load(ckpt, short)
+    assert e.value.code == 10001         # ERROR_LLM_LOAD_MODEL
