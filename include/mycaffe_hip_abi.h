@@ -44,6 +44,7 @@ enum {
     MCH_ERROR_MEMORY_NOT_FOUND = 90014,
     MCH_ERROR_MEMORY_TOO_SMALL = 90016,
     MCH_ERROR_DEVICE_NOT_INITIALIZED = 90017,
+    MCH_ERROR_LAYERNORM_NOT_INITIALIZED = 90161,
     MCH_ERROR_ROPE_NOT_INITIALIZED = 90201,
     MCH_ERROR_ATTN_NOT_INITIALIZED = 90281,
     MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE = 90284,
@@ -102,10 +103,20 @@ enum {
     MCH_FN_TRANSPOSE_HW = 267,
     MCH_FN_CHANNEL_COPY = 300,
     MCH_FN_EMBED_FWD = 390,
+    MCH_FN_RELU_FWD = 428,
+    MCH_FN_RELU_BWD = 429,
+    MCH_FN_GELU_FWD = 600,
+    MCH_FN_GELU_BWD = 601,
     MCH_FN_SILU_FWD = 605,
+    MCH_FN_SILU_BWD = 606,
+    MCH_FN_CREATE_LAYERNORM = 970,
+    MCH_FN_FREE_LAYERNORM = 971,
+    MCH_FN_LAYERNORM_FWD = 975,
+    MCH_FN_LAYERNORM_BWD = 976,
     MCH_FN_CREATE_ROPE = 980,
     MCH_FN_FREE_ROPE = 981,
     MCH_FN_ROPE_FWD = 982,
+    MCH_FN_ROPE_BWD = 983,
     MCH_QRY_DEVICE_NAME = 1000,
     MCH_QRY_EXTENSION_STRING = 1003,
 

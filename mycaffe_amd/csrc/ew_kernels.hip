@@ -420,10 +420,11 @@ hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t out
 
 // ---------------------------------------------------------------------------
 // RoPE: pair p = (x[2p], x[2p+1]); table row = (p % (seqLen*heads*half)) / (heads*half),
-// column = p % half; one fused pass replaces the reference's three kernels.
+// column = p % half; one fused pass replaces the reference's three kernels.  sinSign = -1 gives the gradient
+// (rotation by the opposite angle, rope.cu:754-770).
 template <typename T>
 __global__ void rope_kernel(size_t pairs, const T* x, T* y, const float* __restrict__ fcos, const float* __restrict__ fsin,
-                            int seqLen, int heads, int half, int tableOff)
+                            int seqLen, int heads, int half, int tableOff, float sinSign)
 {
     size_t full = (size_t)heads * half;
     size_t wrap = (size_t)seqLen * full;
@@ -431,7 +432,7 @@ __global__ void rope_kernel(size_t pairs, const T* x, T* y, const float* __restr
     {
         size_t base = p % wrap;
         size_t t = (base / full) * half + base % half + tableOff;
-        float c = fcos[t], sn = fsin[t];
+        float c = fcos[t], sn = sinSign * fsin[t];
         float re = ld(x, 2 * p), im = ld(x, 2 * p + 1);
         st(y, 2 * p, re * c - im * sn);
         st(y, 2 * p + 1, re * sn + im * c);
@@ -439,12 +440,12 @@ __global__ void rope_kernel(size_t pairs, const T* x, T* y, const float* __restr
 }
 
 hipError_t k_rope(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* fcos, const float* fsin,
-                  int seqLen, int heads, int hs, int tableOff)
+                  int seqLen, int heads, int hs, int tableOff, bool grad)
 {
     size_t pairs = n / 2;
     if (pairs == 0) return hipSuccess;
     DISPATCH_DT(dt, hipLaunchKernelGGL(rope_kernel<T>, grid_for(pairs), TPB, 0, s, pairs, (const T*)x, (T*)y, fcos, fsin,
-                                       seqLen, heads, hs / 2, tableOff));
+                                       seqLen, heads, hs / 2, tableOff, grad ? -1.0f : 1.0f));
     return hipGetLastError();
 }
 
@@ -471,6 +472,164 @@ hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x,
 {
     if (outer <= 0 || dim <= 0) return hipSuccess;
     DISPATCH_DT(dt, hipLaunchKernelGGL(rmsnorm_kernel<T>, outer, TPB, 0, s, dim, (const T*)x, (const T*)w, (T*)y, eps));
+    return hipGetLastError();
+}
+
+
+// ---------------------------------------------------------------------------
+// LayerNorm (no affine part; the reference chain of layernorm.cu:219-262 in one pass): per row of `inner` values
+// y = (x - mean) / sqrt(var + eps); the row's sqrt(var + eps) is kept for the backward pass.  One workgroup per
+// row; the row stays in L2 between the three sweeps, so HBM sees one read and one write.
+template <typename T> __global__ void layernorm_fwd_kernel(int inner, const T* x, T* y, float* stdev, float eps)
+{
+    __shared__ float red[4];
+    const T* xr = x + (size_t)blockIdx.x * inner;
+    T* yr = y + (size_t)blockIdx.x * inner;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < inner; i += TPB) sum += ld(xr, i);
+    const float mean = block_sum<4>(sum, red) / inner;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < inner; i += TPB) {
+        float d = ld(xr, i) - mean;
+        sq += d * d;
+    }
+    const float sd = sqrtf(block_sum<4>(sq, red) / inner + eps);
+    if (threadIdx.x == 0) stdev[blockIdx.x] = sd;
+    for (int i = threadIdx.x; i < inner; i += TPB) st(yr, i, (ld(xr, i) - mean) / sd);
+}
+
+hipError_t k_layernorm_fwd(hipStream_t s, DType dt, int rows, int inner, const void* x, void* y, float* stdev, float eps)
+{
+    if (rows <= 0 || inner <= 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_fwd_kernel<T>, rows, TPB, 0, s, inner, (const T*)x, (T*)y, stdev, eps));
+    return hipGetLastError();
+}
+
+// dx = (dy - (y * mean(y*dy) + mean(dy))) / divisor (layernorm.cu:268-312).  The divisor is the row's stdev; the
+// reference adds eps to the first `rows` entries of its row-expanded stdev array on every backward call, which is
+// reproduced through `bump` = eps x (backward calls since the last forward), applied to flat indices < rows.
+template <typename T>
+__global__ void layernorm_bwd_kernel(int rows, int inner, const T* y, const T* dy, T* dx, const float* stdev, float bump)
+{
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * inner;
+    float a = 0.f, b = 0.f;
+    for (int i = threadIdx.x; i < inner; i += TPB) {
+        float g = ld(dy, base + i);
+        a += ld(y, base + i) * g;
+        b += g;
+    }
+    const float m1 = block_sum<4>(a, red) / inner;
+    const float m2 = block_sum<4>(b, red) / inner;
+    const float sd = stdev[blockIdx.x];
+    for (int i = threadIdx.x; i < inner; i += TPB) {
+        float w = ld(y, base + i) * m1 + m2;
+        float div = base + i < (size_t)rows ? sd + bump : sd;
+        st(dx, base + i, (ld(dy, base + i) - w) / div);
+    }
+}
+
+hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const void* y, const void* dy, void* dx,
+                           const float* stdev, float bump)
+{
+    if (rows <= 0 || inner <= 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_bwd_kernel<T>, rows, TPB, 0, s, rows, inner, (const T*)y, (const T*)dy, (T*)dx,
+                                       stdev, bump));
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// GELU (math.cu:11348-11376) and its gradient (math.cu:11412-11448).  The tanh ("bert") forward evaluates in double
+// as the reference's expression does; the erf forward and both gradients are single precision there.
+__device__ inline float gelu_fwd_f(float x, bool bert)
+{
+    if (bert) {
+        const float k = (float)sqrt(2.0 / M_PI);
+        const float x3 = x * x * x;
+        return (float)(0.5 * x * (1.0 + tanh(k * (x + 0.044715 * x3))));
+    }
+    const float r2 = (float)sqrt(2.0);
+    return x * (0.5f * (1.0f + erff(x / r2)));
+}
+__device__ inline float gelu_grad_f(float x, bool bert)
+{
+    if (bert) {
+        const float x3 = x * x * x;
+        const float t = 0.797885f * (x + 0.044715f * x3);
+        const float vx = 0.0535161f * x3 + 0.398942f * x;
+        const float ch = coshf(t);
+        return 0.5f * tanhf(t) + vx * (1.0f / (ch * ch)) + 0.5f;
+    }
+    const float r2pi = (float)sqrt(2.0 * M_PI), r2 = (float)sqrt(2.0);
+    const float cdf = 0.5f * (1.0f + erff(x / r2));
+    const float pdf = 1.0f / r2pi * expf(-0.5f * (x * x));
+    return cdf + x * pdf;
+}
+template <typename T> __global__ void gelu_fwd_kernel(size_t n, const T* x, T* y, bool bert)
+{
+    GRID_STRIDE(i, n) st(y, i, gelu_fwd_f(ld(x, i), bert));
+}
+template <typename T> __global__ void gelu_bwd_kernel(size_t n, const T* dy, const T* x, T* dx, bool bert)
+{
+    GRID_STRIDE(i, n) st(dx, i, ld(dy, i) * gelu_grad_f(ld(x, i), bert));
+}
+hipError_t k_gelu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, bool bert)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(gelu_fwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, bert));
+    return hipGetLastError();
+}
+hipError_t k_gelu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx, bool bert)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(gelu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)x, (T*)dx, bert));
+    return hipGetLastError();
+}
+
+// SiLU gradient: dx = dy * s(x) (1 + x (1 - s(x))) (math.cu:11740-11749)
+template <typename T> __global__ void silu_bwd_kernel(size_t n, const T* dy, const T* x, T* dx)
+{
+    GRID_STRIDE(i, n)
+    {
+        const float v = ld(x, i);
+        const float sg = 1.0f / (1.0f + expf(-v));
+        st(dx, i, ld(dy, i) * (sg * (1.0f + v * (1.0f - sg))));
+    }
+}
+hipError_t k_silu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(silu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)x, (T*)dx));
+    return hipGetLastError();
+}
+
+// ReLU with negative slope (math.cu:12038-12044) and its gradient, which looks at the TOP data (math.cu:12072-12078)
+template <typename T> __global__ void relu_fwd_kernel(size_t n, const T* x, T* y, float slope)
+{
+    GRID_STRIDE(i, n)
+    {
+        const float v = ld(x, i);
+        st(y, i, v > 0.f ? v : v * slope);
+    }
+}
+template <typename T> __global__ void relu_bwd_kernel(size_t n, const T* dy, const T* y, T* dx, float slope)
+{
+    GRID_STRIDE(i, n)
+    {
+        const float v = ld(y, i);
+        st(dx, i, ld(dy, i) * ((v > 0.f ? 1.f : 0.f) + (v <= 0.f ? 1.f : 0.f) * slope));
+    }
+}
+hipError_t k_relu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, float slope)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(relu_fwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, slope));
+    return hipGetLastError();
+}
+hipError_t k_relu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* y, void* dx, float slope)
+{
+    if (n == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(relu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)y, (T*)dx, slope));
     return hipGetLastError();
 }
 

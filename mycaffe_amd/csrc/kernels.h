@@ -53,7 +53,16 @@ hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, con
 hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm);
 // adjacent-pair rotary embedding with the CudaDnnDLL index rule; x == y allowed
 hipError_t k_rope(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* fcos, const float* fsin,
-                  int seqLen, int heads, int hs, int tableOff);
+                  int seqLen, int heads, int hs, int tableOff, bool grad = false);
+// LayerNorm without affine part over rows x inner; stdev[rows] keeps sqrt(var + eps) of every row for the gradient
+hipError_t k_layernorm_fwd(hipStream_t s, DType dt, int rows, int inner, const void* x, void* y, float* stdev, float eps);
+hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const void* y, const void* dy, void* dx,
+                           const float* stdev, float bump);
+hipError_t k_gelu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, bool bert);
+hipError_t k_gelu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx, bool bert);
+hipError_t k_relu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, float slope);
+hipError_t k_relu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* y, void* dx, float slope);
+hipError_t k_silu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx);
 hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps);
 
 // ---- GEMM family (gemm.hip) ------------------------------------------------

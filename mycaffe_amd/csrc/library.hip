@@ -164,6 +164,7 @@ Kernel::~Kernel()
     if (m_stream) (void)hipStreamSynchronize(m_stream);
     m_ext.clear();
     m_rope.clear();
+    m_layernorm.clear();
     m_mem.free_all();
     if (m_ws) (void)hipFree(m_ws);
     if (m_tickets) (void)hipFree(m_tickets);
@@ -808,6 +809,136 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
+    case MCH_FN_SILU_BWD:
+    case MCH_FN_GELU_BWD: {
+        // l{count,hTopDiff,hTopData,hBtmDiff,hBtmData[,bert]} (CudaDnn.cs:10132-10180, device.h:3269-3316)
+        const bool gelu = fn == MCH_FN_GELU_BWD;
+        NEED_L(gelu ? 6 : 5, gelu ? 6 : 5);
+        long long n = pl[0];
+        MemItem *dY, *dX, *X;
+        ERRCHK(mem((long)pl[1], &dY));
+        ERRCHK(mem((long)pl[3], &dX));
+        ERRCHK(mem((long)pl[4], &X));
+        if (dY->half != dX->half || X->half != dX->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(dY, 0, n);
+        RANGE(dX, 0, n);
+        RANGE(X, 0, n);
+        if (gelu) HIPCHK(k_gelu_bwd(s, X->dt(), (size_t)n, dY->ptr, X->ptr, dX->ptr, pl[5] != 0));
+        else HIPCHK(k_silu_bwd(s, X->dt(), (size_t)n, dY->ptr, X->ptr, dX->ptr));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_RELU_FWD: {
+        // f{negativeSlope}, l{count,hBtm,hTop,0} (CudaDnn.cs:10417-10423, device.h:4925-4940)
+        NEED_F(1, 1);
+        NEED_L(4, 4);
+        long long n = pl[0];
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_relu_fwd(s, X->dt(), (size_t)n, X->ptr, Y->ptr, pf[0]));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_RELU_BWD: {
+        // f{negativeSlope}, l{count,hTopDiff,hTopData,hBtmDiff,0} (CudaDnn.cs:10438-10444, device.h:4943-4959)
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        long long n = pl[0];
+        MemItem *dY, *Y, *dX;
+        ERRCHK(mem((long)pl[1], &dY));
+        ERRCHK(mem((long)pl[2], &Y));
+        ERRCHK(mem((long)pl[3], &dX));
+        if (dY->half != Y->half || dX->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(dY, 0, n);
+        RANGE(Y, 0, n);
+        RANGE(dX, 0, n);
+        HIPCHK(k_relu_bwd(s, Y->dt(), (size_t)n, dY->ptr, Y->ptr, dX->ptr, pf[0]));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_GELU_FWD: {
+        // l{count,hBtm,hTop,bert} (CudaDnn.cs:10098-10104, device.h:3253-3266)
+        NEED_L(4, 4);
+        long long n = pl[0];
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_gelu_fwd(s, X->dt(), (size_t)n, X->ptr, Y->ptr, pl[3] != 0));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
+    case MCH_FN_CREATE_LAYERNORM: {
+        // f{eps}, l{gpuId,count,outer,channels,inner} (CudaDnn.cs:6307-6319, device.h:4123-4147)
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        long long count = pl[1], outer = pl[2], channels = pl[3], inner = pl[4];
+        if (outer < 1 || channels < 1 || inner < 1 || count > INT_MAX || outer * channels > INT_MAX ||
+            count != outer * channels * inner)
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;   // layernorm.cu:141-142
+        long h;
+        ERRCHK(m_layernorm.create(&h));
+        LayerNormState* ln = m_layernorm.get(h);
+        ln->count = (int)count; ln->outer = (int)outer; ln->channels = (int)channels; ln->inner = (int)inner;
+        ln->eps = pf[0];
+        hipError_t e = hipMalloc((void**)&ln->stdev, (size_t)(outer * channels) * sizeof(float));
+        if (e != hipSuccess) {
+            ln->stdev = nullptr;
+            m_layernorm.free(h);
+            return (long)e;
+        }
+        ln->set = true;
+        return set_out((float)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_LAYERNORM:
+        NEED_F(1, 1);
+        HIPCHK(hipStreamSynchronize(s));
+        return m_layernorm.free((long)pf[0]);
+    case MCH_FN_LAYERNORM_FWD: {
+        // l{hLayerNorm,hX,hY} (CudaDnn.cs:6339-6345, layernorm.cu:219-262)
+        NEED_L(3, 3);
+        LayerNormState* ln = m_layernorm.get((long)pl[0]);
+        if (!ln || !ln->set) return MCH_ERROR_LAYERNORM_NOT_INITIALIZED;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, ln->count);
+        RANGE(Y, 0, ln->count);
+        HIPCHK(k_layernorm_fwd(s, X->dt(), ln->outer * ln->channels, ln->inner, X->ptr, Y->ptr, ln->stdev, ln->eps));
+        ln->backwards = 0;
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_LAYERNORM_BWD: {
+        // l{hLayerNorm,hYdata,hYdiff,hXdiff} (CudaDnn.cs:6354-6360, layernorm.cu:268-312)
+        NEED_L(4, 4);
+        LayerNormState* ln = m_layernorm.get((long)pl[0]);
+        if (!ln || !ln->set) return MCH_ERROR_LAYERNORM_NOT_INITIALIZED;
+        MemItem *Y, *dY, *dX;
+        ERRCHK(mem((long)pl[1], &Y));
+        ERRCHK(mem((long)pl[2], &dY));
+        ERRCHK(mem((long)pl[3], &dX));
+        if (Y->half != dY->half || Y->half != dX->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(Y, 0, ln->count);
+        RANGE(dY, 0, ln->count);
+        RANGE(dX, 0, ln->count);
+        ln->backwards++;
+        HIPCHK(k_layernorm_bwd(s, Y->dt(), ln->outer * ln->channels, ln->inner, Y->ptr, dY->ptr, dX->ptr, ln->stdev,
+                               ln->eps * (float)ln->backwards));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
     case MCH_FN_SWIGLU_FWD: {
         NEED_L(4, 4);
         long long n = pl[0];
@@ -1102,6 +1233,25 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         HIPCHK(k_rope(s, X->dt(), (size_t)n, X->ptr, Y->ptr, (const float*)r->dcos.get(), (const float*)r->dsin.get(), r->seq,
                       r->heads, r->hs, (int)off));
         m_mem.touch((long)pl[3]);
+        return 0;
+    }
+
+    case MCH_FN_ROPE_BWD: {
+        // l{hRope,n,hXdata,hYdiff,hXdiff}: the rotation by the opposite angle, never shifted (device.h:4266-4283, rope.cu:832-864)
+        NEED_L(5, 5);
+        RopeState* r = m_rope.get((long)pl[0]);
+        if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+        long long n = pl[1];
+        MemItem *dY, *dX;
+        ERRCHK(mem((long)pl[3], &dY));
+        ERRCHK(mem((long)pl[4], &dX));
+        if (dY->half != dX->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (n < 0 || (n & 1)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(dY, 0, n);
+        RANGE(dX, 0, n);
+        HIPCHK(k_rope(s, dY->dt(), (size_t)n, dY->ptr, dX->ptr, (const float*)r->dcos.get(), (const float*)r->dsin.get(), r->seq,
+                      r->heads, r->hs, 0, true));
+        m_mem.touch((long)pl[4]);
         return 0;
     }
 

@@ -84,6 +84,14 @@ struct RopeState {
     float theta = 10000.f;
     std::shared_ptr<void> dcos, dsin;  // device tables [seq, hs/2] fp32, shared by sharedIdx
 };
+struct LayerNormState {
+    bool set = false;
+    int count = 0, outer = 0, channels = 0, inner = 0;
+    float eps = 1e-10f;
+    float* stdev = nullptr;   // [outer*channels] sqrt(var + eps) of the last forward
+    int backwards = 0;        // backward calls since the last forward
+    ~LayerNormState() { if (stdev) (void)hipFree(stdev); }
+};
 struct ExtensionState {
     void* lib = nullptr;
     void* fnInvoke = nullptr;
@@ -123,6 +131,7 @@ private:
     HandleTable<TensorDesc> m_tdesc;
     HandleTable<AttnState> m_attn;
     HandleTable<RopeState> m_rope;
+    HandleTable<LayerNormState> m_layernorm;
     HandleTable<ExtensionState> m_ext;
     std::map<int, std::weak_ptr<void>> m_ropeSharedCos, m_ropeSharedSin;
     void* m_ws = nullptr; size_t m_wsBytes = 0;          // device scratch (split-K partials, conversions)

@@ -71,10 +71,20 @@ class CUDAFN:
     CUDA_TRANSPOSE_HW = 267
     CUDA_CHANNEL_COPY = 300
     CUDA_EMBED_FWD = 390
+    CUDA_RELU_FWD = 428
+    CUDA_RELU_BWD = 429
+    CUDA_GELU_FWD = 600
+    CUDA_GELU_BWD = 601
     CUDA_SILU_FWD = 605
+    CUDA_SILU_BWD = 606
+    CUDA_CREATE_LAYERNORM = 970
+    CUDA_FREE_LAYERNORM = 971
+    CUDA_LAYERNORM_FWD = 975
+    CUDA_LAYERNORM_BWD = 976
     CUDA_CREATE_ROPE = 980
     CUDA_FREE_ROPE = 981
     CUDA_ROPE_FWD = 982
+    CUDA_ROPE_BWD = 983
     # additions of this library (no counterpart in the reference)
     ATTN_DECODE_FWD = 2001
     RMSNORM_FWD = 2002
@@ -117,6 +127,7 @@ class ERROR:
     MEMORY_RANGE_EXCEEDED = 90010
     MEMORY_MIXED_HALF_TYPES = 90011
     MEMORY_NOT_FOUND = 90014
+    LAYERNORM_NOT_INITIALIZED = 90161
     ROPE_NOT_INITIALIZED = 90201
     ATTN_NOT_INITIALIZED = 90281
     ATTN_INCOMPATIBLE_BLOB_SIZE = 90284
@@ -465,6 +476,43 @@ class CudaDnn:
         """CudaDnn.cs:10152-10158."""
         self._ex2(CUDAFN.CUDA_SILU_FWD, None, [nCount, hBottomData, hTopData])
 
+    def relu_fwd(self, nCount, hBottomData, hTopData, fNegativeSlope=0.0):
+        """CudaDnn.cs:10417-10423."""
+        self._ex2(CUDAFN.CUDA_RELU_FWD, [fNegativeSlope], [nCount, hBottomData, hTopData, 0])
+
+    def relu_bwd(self, nCount, hTopDiff, hTopData, hBottomDiff, fNegativeSlope=0.0):
+        """CudaDnn.cs:10438-10444."""
+        self._ex2(CUDAFN.CUDA_RELU_BWD, [fNegativeSlope], [nCount, hTopDiff, hTopData, hBottomDiff, 0])
+
+    def silu_bwd(self, nCount, hTopDiff, hTopData, hBottomDiff, hBottomData):
+        """CudaDnn.cs:10174-10180."""
+        self._ex2(CUDAFN.CUDA_SILU_BWD, None, [nCount, hTopDiff, hTopData, hBottomDiff, hBottomData])
+
+    def gelu_fwd(self, nCount, hBottomData, hTopData, bEnableBertVersion):
+        """CudaDnn.cs:10098-10104."""
+        self._ex2(CUDAFN.CUDA_GELU_FWD, None, [nCount, hBottomData, hTopData, 1 if bEnableBertVersion else 0])
+
+    def gelu_bwd(self, nCount, hTopDiff, hTopData, hBottomDiff, hBottomData, bEnableBertVersion):
+        """CudaDnn.cs:10132-10138."""
+        self._ex2(CUDAFN.CUDA_GELU_BWD, None, [nCount, hTopDiff, hTopData, hBottomDiff, hBottomData, 1 if bEnableBertVersion else 0])
+
+    # ---- LayerNorm ------------------------------------------------------------------------------
+    def CreateLayerNorm(self, nGpuID, nCount, nOuterNum, nChannels, nInnerNum, fEps=1e-10):
+        """CudaDnn.cs:6307-6319."""
+        return int(self._ex2(CUDAFN.CUDA_CREATE_LAYERNORM, [fEps], [nGpuID, nCount, nOuterNum, nChannels, nInnerNum])[0])
+
+    def FreeLayerNorm(self, hLayerNorm):
+        """CudaDnn.cs:6325-6331."""
+        self.RunFloat(self.m_hKernel, CUDAFN.CUDA_FREE_LAYERNORM, [hLayerNorm])
+
+    def LayerNormForward(self, hLayerNorm, hXdata, hYdata):
+        """CudaDnn.cs:6339-6345."""
+        self._ex2(CUDAFN.CUDA_LAYERNORM_FWD, None, [hLayerNorm, hXdata, hYdata])
+
+    def LayerNormBackward(self, hLayerNorm, hYdata, hYdiff, hXdiff):
+        """CudaDnn.cs:6354-6360."""
+        self._ex2(CUDAFN.CUDA_LAYERNORM_BWD, None, [hLayerNorm, hYdata, hYdiff, hXdiff])
+
     # ---- cuDNN-shaped handles ---------------------------------------------------------
     def CreateCuDNN(self, hStream=0):
         """CudaDnn.cs:3509-3520."""
@@ -544,6 +592,10 @@ class CudaDnn:
     def RopeForward(self, hRope, n, hXdata, hYdata, nFreqOffset=-1):
         """CudaDnn.cs:6409-6415."""
         self._ex2(CUDAFN.CUDA_ROPE_FWD, None, [hRope, n, hXdata, hYdata, nFreqOffset])
+
+    def RopeBackward(self, hRope, n, hXdata, hYdiff, hXdiff):
+        """CudaDnn.cs:6425-6431."""
+        self._ex2(CUDAFN.CUDA_ROPE_BWD, None, [hRope, n, hXdata, hYdiff, hXdiff])
 
     # ---- extensions ---------------------------------------------------------------------------------
     def CreateExtension(self, strExtensionDllPath):

@@ -371,3 +371,89 @@ class MultiheadAttentionLayer:
         self.transpose.Forward(b["Work"], b["Y"])
         b["Y"].Reshape(B, Tq, C)
         self.c_proj.Forward(b["Y"], top)
+
+
+class LayerNormLayer:
+    """MyCaffe.layers.gpt/layers.gpt/LayerNormLayer.cs with ``enable_cuda_impl`` (reshape :153-166, forward :211-212,
+    backward :285-286): normalisation over the last axis through the LayerNorm handle (ids 970-976)."""
+
+    def __init__(self, cuda, epsilon=1e-10):
+        self.cuda, self.epsilon = cuda, epsilon
+        self.hLayerNorm = 0
+        self._shape = None
+
+    def _reshape(self, bottom):
+        if self._shape == bottom.shape_:
+            return
+        if self.hLayerNorm:
+            self.cuda.FreeLayerNorm(self.hLayerNorm)
+        nAxis = len(bottom.shape_) - 1
+        outer, channels, inner = bottom.shape_[0], bottom.count(1, nAxis), bottom.count(nAxis)
+        self.hLayerNorm = self.cuda.CreateLayerNorm(0, bottom.count(), outer, channels, inner, self.epsilon)
+        self._shape = list(bottom.shape_)
+
+    def Forward(self, bottom, top):
+        self._reshape(bottom)
+        top.ReshapeLike(bottom)
+        self.cuda.LayerNormForward(self.hLayerNorm, bottom.gpu_data, top.gpu_data)
+
+    def Backward(self, top, hTopDiff, hBottomDiff):
+        self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, hTopDiff, hBottomDiff)
+
+
+class ActivationLayer:
+    """ReLU (MyCaffe/layers/ReLULayer.cs), GELU (MyCaffe.layers.gpt/layers.gpt/GeluLayer.cs, ``enable_bert_version``) or
+    SiLU (MyCaffe/layers/SiLULayer.cs) as TransformerBlockLayer selects them (TransformerBlockLayer.cs:316-337)."""
+
+    def __init__(self, cuda, kind="relu"):
+        if kind not in ("relu", "gelu", "gelu_bert", "silu"):
+            raise ValueError(kind)
+        self.cuda, self.kind = cuda, kind
+
+    def Forward(self, bottom, top):
+        top.ReshapeLike(bottom)
+        n = bottom.count()
+        if self.kind == "relu":
+            self.cuda.relu_fwd(n, bottom.gpu_data, top.gpu_data, 0.0)
+        elif self.kind == "silu":
+            self.cuda.silu_fwd(n, bottom.gpu_data, top.gpu_data)
+        else:
+            self.cuda.gelu_fwd(n, bottom.gpu_data, top.gpu_data, self.kind == "gelu_bert")
+
+
+class TransformerBlockLayer:
+    """MyCaffe.layers.gpt/layers.gpt/TransformerBlockLayer.cs, block type CAUSAL_SELF_ATTENTION (setup :99-130, 252-340,
+    forward :810-902): x + attn(ln1(x)), then + proj(act(fc(ln2(.)))).  Dropout is the identity at inference."""
+
+    def __init__(self, cuda, heads, embed, block_size, activation="relu", bias_term=True, epsilon=1e-10,
+                 enable_cuda_scaled_dot_product_attention=True):
+        self.cuda = cuda
+        self.norm1 = LayerNormLayer(cuda, epsilon)
+        self.norm2 = LayerNormLayer(cuda, epsilon)
+        self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention)
+        self.fc1 = InnerProductLayer(cuda, 4 * embed, bias_term, 2)
+        self.proj = InnerProductLayer(cuda, embed, bias_term, 2)
+        self.act = ActivationLayer(cuda, activation)
+        self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 Mlp1 MlpOut".split()}
+
+    def Setup(self, bottom, p):
+        """``p``: attn_weight, attn_bias, attn_proj_weight, attn_proj_bias, fc_weight, fc_bias, proj_weight, proj_bias."""
+        self.attn1.Setup(bottom, p["attn_weight"], p.get("attn_bias"), p["attn_proj_weight"], p.get("attn_proj_bias"))
+        self.fc1.Setup(bottom, p["fc_weight"], p.get("fc_bias"))
+        hidden = Blob(self.cuda, bottom.shape_[:2] + [self.fc1.N])
+        self.proj.Setup(hidden, p["proj_weight"], p.get("proj_bias"))
+        hidden.Dispose()
+
+    def Forward(self, blobX, top):
+        b, cuda = self.b, self.cuda
+        nCount = blobX.count()
+        self.norm1.Forward(blobX, b["Norm1"])
+        self.attn1.Forward(b["Norm1"], b["Attn1"])
+        b["X"].ReshapeLike(blobX)
+        cuda.add(nCount, blobX.gpu_data, b["Attn1"].gpu_data, b["X"].gpu_data)
+        self.norm2.Forward(b["X"], b["Norm2"])
+        self.fc1.Forward(b["Norm2"], b["Mlp1"])
+        self.act.Forward(b["Mlp1"], b["Mlp1"])
+        self.proj.Forward(b["Mlp1"], b["MlpOut"])
+        top.ReshapeLike(blobX)
+        cuda.add(nCount, b["X"].gpu_data, b["MlpOut"].gpu_data, top.gpu_data)

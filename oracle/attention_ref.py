@@ -361,3 +361,145 @@ def kv_cache_attention(q, kcache, vcache, dtype=np.float32):
     s = np.einsum("bhd,bhld->bhl", q, kc) / dtype(np.sqrt(float(hs)))
     p = softmax_lastaxis(s, dtype)
     return np.einsum("bhl,bhld->bhd", p, vc).astype(dtype)
+
+
+# ----------------------------------------------------------------------------
+# LayerNorm handle, GELU / SiLU, gradients
+# ----------------------------------------------------------------------------
+
+def layernorm_forward(x, inner, eps=1e-10, dtype=np.float32):
+    """LayerNormData::Forward (CudaDnnDLL/Cuda Files/layernorm.cu:219-262): per row of ``inner`` values
+    mean -> xmu = x - mean -> var = mean(xmu^2) -> stdev = sqrt(var + eps) -> y = xmu / stdev.  No affine part.
+    Returns (y, stdev[rows])."""
+    x = np.asarray(x, dtype)
+    r = x.reshape(-1, inner)
+    mu = (r.astype(np.float64).sum(1) / inner).astype(dtype)          # channel_mean accumulates in double (math.cu:6817-6831)
+    xmu = r - mu[:, None]
+    var = ((xmu * xmu).astype(np.float64).sum(1) / inner).astype(dtype)
+    stdev = np.sqrt(var + dtype(eps)).astype(dtype)
+    return (xmu / stdev[:, None]).astype(dtype).reshape(x.shape), stdev
+
+
+def layernorm_backward(y, dy, stdev, inner, eps=1e-10, backward_calls=1, dtype=np.float32):
+    """LayerNormData::Backward (layernorm.cu:268-312): dx = (dy - (y * mean(y*dy) + mean(dy))) / stdev_full.
+
+    stdev_full is the row-expanded stdev array of the forward pass; before the division the reference adds eps to
+    its first ``rows`` flat entries (``add_scalar(outer*channels, eps, stdevfull)``, layernorm.cu:306), once per
+    backward call and cumulatively until the next forward refills the array."""
+    y = np.asarray(y, dtype)
+    r = y.reshape(-1, inner)
+    g = np.asarray(dy, dtype).reshape(-1, inner)
+    rows = r.shape[0]
+    m1 = ((r * g).astype(np.float64).sum(1) / inner).astype(dtype)
+    m2 = (g.astype(np.float64).sum(1) / inner).astype(dtype)
+    work = g - (r * m1[:, None] + m2[:, None])
+    full = np.repeat(np.asarray(stdev, dtype), inner)
+    for _ in range(backward_calls):
+        full[:rows] = full[:rows] + dtype(eps)
+    return (work / full.reshape(rows, inner)).astype(dtype).reshape(y.shape)
+
+
+def gelu(x, bert, dtype=np.float32):
+    """gelu_fwd_kernel / gelu_fwd_kernel_bert (math.cu:11348-11376).  The tanh form is evaluated in double on the
+    T-typed input and constant and cast back; the erf form stays in T."""
+    from scipy.special import erf
+    x = np.asarray(x, dtype)
+    if bert:
+        k = np.float64(dtype(np.sqrt(2.0 / np.pi)))
+        x3 = (x * x * x).astype(np.float64)
+        xd = x.astype(np.float64)
+        return (0.5 * xd * (1.0 + np.tanh(k * (xd + 0.044715 * x3)))).astype(dtype)
+    return (x * (dtype(0.5) * (dtype(1.0) + erf(x / dtype(np.sqrt(2.0))).astype(dtype)))).astype(dtype)
+
+
+def gelu_grad(x, dy, bert, dtype=np.float32):
+    """gelu_bwd_kernel / gelu_bwd_kernel_bert (math.cu:11412-11448) with the reference's rounded constants."""
+    from scipy.special import erf
+    x = np.asarray(x, dtype)
+    dy = np.asarray(dy, dtype)
+    if bert:
+        x3 = x * x * x
+        t = dtype(0.797885) * (x + dtype(0.044715) * x3)
+        vx = dtype(0.0535161) * x3 + dtype(0.398942) * x
+        ch = np.cosh(t)
+        grad = dtype(0.5) * np.tanh(t) + vx * (dtype(1.0) / (ch * ch)) + dtype(0.5)
+    else:
+        cdf = dtype(0.5) * (dtype(1.0) + erf(x / dtype(np.sqrt(2.0))).astype(dtype))
+        pdf = dtype(1.0) / dtype(np.sqrt(2.0 * np.pi)) * np.exp(dtype(-0.5) * (x * x))
+        grad = cdf + x * pdf
+    return (dy * grad).astype(dtype)
+
+
+def relu(x, slope=0.0, dtype=np.float32):
+    """relu_fwd_kernel (math.cu:12038-12044)."""
+    x = np.asarray(x, dtype)
+    return np.where(x > 0, x, x * dtype(slope)).astype(dtype)
+
+
+def relu_grad(y, dy, slope=0.0, dtype=np.float32):
+    """relu_bwd_kernel (math.cu:12072-12078): the gate is read from the TOP data."""
+    y = np.asarray(y, dtype)
+    return (np.asarray(dy, dtype) * ((y > 0).astype(dtype) + (y <= 0).astype(dtype) * dtype(slope))).astype(dtype)
+
+
+def silu_grad(x, dy, dtype=np.float32):
+    """silu_bwd_kernel (math.cu:11740-11749): dy * s (1 + x (1 - s)), s = sigmoid(x)."""
+    x = np.asarray(x, dtype)
+    s = dtype(1.0) / (dtype(1.0) + np.exp(-x))
+    return (np.asarray(dy, dtype) * (s * (dtype(1.0) + x * (dtype(1.0) - s)))).astype(dtype)
+
+
+def rope_backward(dy, seq_len, heads, hs, theta=10000.0, dtype=np.float32):
+    """RopeDataGpu::Backward (rope.cu:832-864, copy_computeRI_grad_kernel :754-770): the rotation by the opposite
+    angle with the unshifted tables (the backward pass takes no frequency offset)."""
+    dy = np.asarray(dy, dtype)
+    flat = dy.reshape(-1)
+    pairs = flat.size // 2
+    half = hs // 2
+    full = half * heads
+    fcos, fsin = rope_tables(seq_len, hs, theta)
+    p = np.arange(pairs)
+    base = p % (seq_len * full)
+    idx = (base // full) * half + base % half
+    c = fcos.reshape(-1)[idx].astype(dtype)
+    s = fsin.reshape(-1)[idx].astype(dtype)
+    re, im = flat[0::2], flat[1::2]
+    out = np.empty_like(flat)
+    out[0::2] = re * c + im * s
+    out[1::2] = -re * s + im * c
+    return out.reshape(dy.shape)
+
+
+def attn_backward(q, k, v, att, dy, dtype=np.float32):
+    """attnHandle::Backward (attn.cu:608-661) without dropout, on the probabilities ``att`` saved by the forward pass:
+    dV = att^T dY, dAtt = dY V^T (matmulgrad :380-397); softmax backward dS = att * (dAtt - rowsum(dAtt * att));
+    dS *= 1/sqrt(hs); dQ = dS K, dK = dS^T Q.  Masked entries need no special case: their probability is exactly 0.
+    All of q, k, v, dy (B,H,T,hs); returns (dq, dk, dv)."""
+    q = np.asarray(q, dtype); k = np.asarray(k, dtype); v = np.asarray(v, dtype)
+    att = np.asarray(att, dtype); dy = np.asarray(dy, dtype)
+    scale = dtype(1.0 / np.sqrt(np.float64(q.shape[-1])))
+    dv = np.swapaxes(att, -1, -2) @ dy
+    datt = dy @ np.swapaxes(v, -1, -2)
+    ds = att * (datt - (datt * att).sum(-1, keepdims=True))
+    ds = ds * scale
+    dq = ds @ k
+    dk = np.swapaxes(ds, -1, -2) @ q
+    return dq.astype(dtype), dk.astype(dtype), dv.astype(dtype)
+
+
+def transformer_block_gpt(x, p, heads, activation="relu", eps=1e-10, dtype=np.float32):
+    """TransformerBlockLayer.forward, CAUSAL_SELF_ATTENTION block type (TransformerBlockLayer.cs:810-902):
+    xB = x + attn(ln1(x)); y = xB + proj(gelu(fc(ln2(xB)))).  ``p`` maps attn_weight, attn_bias, attn_proj_weight,
+    attn_proj_bias, fc_weight, fc_bias, proj_weight, proj_bias; ``activation`` is "relu" (the layer's default,
+    TransformerBlockLayer.cs:316), "gelu" or "gelu_bert".  Returns dict with the intermediates."""
+    x = np.asarray(x, dtype)
+    C = x.shape[-1]
+    ln1, _ = layernorm_forward(x, C, eps, dtype)
+    attn = causal_self_attention(ln1, p["attn_weight"], p["attn_bias"], p["attn_proj_weight"], p["attn_proj_bias"], heads,
+                                 dtype=dtype)["y"]
+    xb = (x + attn).astype(dtype)
+    ln2, _ = layernorm_forward(xb, C, eps, dtype)
+    fc = inner_product(ln2, p["fc_weight"], p["fc_bias"], dtype)
+    act = relu(fc, 0.0, dtype) if activation == "relu" else gelu(fc, activation == "gelu_bert", dtype)
+    mlp = inner_product(act, p["proj_weight"], p["proj_bias"], dtype)
+    return {"ln1": ln1, "attn": attn, "xb": xb, "ln2": ln2, "fc": fc, "act": act, "mlp": mlp, "y": (xb + mlp).astype(dtype)}

@@ -1,0 +1,160 @@
+"""GPU parity of the per-block ops around attention (LayerNorm handle, GELU / ReLU / SiLU and their gradients, RoPE
+gradient, the GPT transformer block) through the C ABI, against the numpy checker and the reference-held fixtures."""
+import os
+
+import numpy as np
+import pytest
+
+from mycaffe_amd.cudadnn import CudaDnnError, ERROR
+from mycaffe_amd.layers import Blob, TransformerBlockLayer
+from oracle import attention_ref as R
+from tests.conftest import BF16_RTOL, FP32_RTOL, GOLDEN, assert_close, bf16_round, load_txt
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name", ["gpt-pico-ln", "gpt-pico-ln3B"])
+def test_layernorm_handle_golden(dev, name):
+    d = os.path.join(GOLDEN, name)
+    x = load_txt(os.path.join(d, "x.txt"))
+    B, T, C = x.shape
+    h = dev.cuda.CreateLayerNorm(0, x.size, B, T, C, 1e-10)
+    hx, hy = dev.put(x), dev.zeros(x.size)
+    dev.cuda.LayerNormForward(h, hx, hy)
+    y = dev.get(hy)
+    assert_close(y, load_txt(os.path.join(d, "y.txt")), 2e-6, "layernorm fwd")
+    hdy, hdx = dev.put(load_txt(os.path.join(d, "grad_1a_y.txt"))), dev.zeros(x.size)
+    dev.cuda.LayerNormBackward(h, hy, hdy, hdx)
+    assert_close(dev.get(hdx), load_txt(os.path.join(d, "grad_9_x.txt")), 2e-5, "layernorm bwd")
+    dev.cuda.FreeLayerNorm(h)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.LayerNormForward(h, hx, hy)
+    assert e.value.code == ERROR.LAYERNORM_NOT_INITIALIZED
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("shape", [(3, 7, 768), (2, 5, 1000), (4, 3, 24), (1, 2, 5000)])
+def test_layernorm_vs_checker(dev, shape, half):
+    rng = np.random.default_rng(21)
+    x = bf16_round((rng.standard_normal(shape) * 2 + 0.5).astype(np.float32))
+    dy = bf16_round(rng.standard_normal(shape).astype(np.float32))
+    B, T, C = shape
+    eps = 1e-5
+    h = dev.cuda.CreateLayerNorm(0, x.size, B, T, C, eps)
+    hx, hy, hdy, hdx = dev.put(x, half), dev.zeros(x.size, half), dev.put(dy, half), dev.zeros(x.size, half)
+    dev.cuda.LayerNormForward(h, hx, hy)
+    y, sd = R.layernorm_forward(x, C, eps, np.float64)
+    tol = BF16_RTOL if half else 1e-5
+    got_y = dev.get(hy)
+    assert_close(got_y, y, tol, "layernorm fwd")
+    # the gradient is checked on the y the device holds (bf16 storage rounds it)
+    yy = got_y.reshape(shape).astype(np.float64)
+    for calls in (1, 2):   # the divisor of the first rows grows by eps per backward call until the next forward
+        dev.cuda.LayerNormBackward(h, hy, hdy, hdx)
+        ref = R.layernorm_backward(yy, dy, sd, C, eps, calls, np.float64)
+        assert_close(dev.get(hdx), ref, tol, "layernorm bwd call %d" % calls)
+    dev.cuda.LayerNormForward(h, hx, hy)
+    dev.cuda.LayerNormBackward(h, hy, hdy, hdx)
+    assert_close(dev.get(hdx), R.layernorm_backward(yy, dy, sd, C, eps, 1, np.float64), tol, "layernorm bwd after forward")
+    dev.cuda.FreeLayerNorm(h)
+
+
+def test_layernorm_bad_arguments(dev):
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.CreateLayerNorm(0, 100, 2, 5, 11, 1e-5)   # count != outer*channels*inner
+    assert e.value.code == ERROR.PARAM_OUT_OF_RANGE
+    h = dev.cuda.CreateLayerNorm(0, 110, 2, 5, 11, 1e-5)
+    hx, hy = dev.zeros(100), dev.zeros(110)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.LayerNormForward(h, hx, hy)
+    assert e.value.code == ERROR.MEMORY_RANGE_EXCEEDED
+    dev.cuda.FreeLayerNorm(h)
+
+
+def test_gelu_golden(dev):
+    d = os.path.join(GOLDEN, "gpt-pico-gelu")
+    x = load_txt(os.path.join(d, "1_x.txt"))
+    hx, hy = dev.put(x), dev.zeros(x.size)
+    dev.cuda.gelu_fwd(x.size, hx, hy, True)
+    assert_close(dev.get(hy), load_txt(os.path.join(d, "2_y.txt")), 1e-6, "gelu fwd")
+    hdy, hdx = dev.put(load_txt(os.path.join(d, "grad_1_y.txt"))), dev.zeros(x.size)
+    dev.cuda.gelu_bwd(x.size, hdy, hy, hdx, hx, True)
+    assert_close(dev.get(hdx), load_txt(os.path.join(d, "grad_2_x.txt")), 1e-6, "gelu bwd")
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_activations_and_gradients_vs_checker(dev, half):
+    rng = np.random.default_rng(22)
+    n = 70001
+    x = bf16_round((rng.standard_normal(n) * 3).astype(np.float32))
+    g = bf16_round(rng.standard_normal(n).astype(np.float32))
+    hx, hg, hy, hdx = dev.put(x, half), dev.put(g, half), dev.zeros(n, half), dev.zeros(n, half)
+    tol = BF16_RTOL if half else 2e-6
+    for bert in (True, False):
+        dev.cuda.gelu_fwd(n, hx, hy, bert)
+        assert_close(dev.get(hy), R.gelu(x, bert, np.float64), tol, "gelu bert=%s" % bert)
+        dev.cuda.gelu_bwd(n, hg, hy, hdx, hx, bert)
+        assert_close(dev.get(hdx), R.gelu_grad(x, g, bert, np.float64), tol, "gelu grad bert=%s" % bert)
+    dev.cuda.silu_bwd(n, hg, hy, hdx, hx)
+    assert_close(dev.get(hdx), R.silu_grad(x, g, np.float64), tol, "silu grad")
+    for slope in (0.0, 0.1):
+        dev.cuda.relu_fwd(n, hx, hy, slope)
+        y = dev.get(hy)
+        assert_close(y, R.relu(x, slope, np.float64), tol, "relu")
+        dev.cuda.relu_bwd(n, hg, hy, hdx, slope)
+        assert_close(dev.get(hdx), R.relu_grad(y, g, slope, np.float64), tol, "relu grad")
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_rope_backward_vs_checker(dev, half):
+    rng = np.random.default_rng(23)
+    B, T, H, hs = 2, 12, 3, 16
+    x = bf16_round(rng.standard_normal((B, T, H, hs)).astype(np.float32))
+    dy = bf16_round(rng.standard_normal((B, T, H, hs)).astype(np.float32))
+    h = dev.cuda.CreateRope(0, 0, x.size, B, T, H, hs, 10000.0)
+    hx, hdy, hdx = dev.put(x, half), dev.put(dy, half), dev.zeros(x.size, half)
+    dev.cuda.RopeBackward(h, x.size, hx, hdy, hdx)
+    assert_close(dev.get(hdx), R.rope_backward(dy, T, H, hs, dtype=np.float64), BF16_RTOL if half else 2e-6, "rope bwd")
+    if not half:   # backward undoes forward
+        hy = dev.zeros(x.size)
+        dev.cuda.RopeForward(h, x.size, hx, hy)
+        dev.cuda.RopeBackward(h, x.size, hx, hy, hdx)
+        assert_close(dev.get(hdx), x, 2e-6, "rope round trip")
+    dev.cuda.FreeRope(h)
+
+
+@pytest.mark.parametrize("sdpa", [True, False])
+@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3B", 3)])
+def test_transformer_block_golden(dev, name, heads, sdpa):
+    d = os.path.join(GOLDEN, name)
+    p = {k: load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias",
+                                                             "fc_weight", "fc_bias", "proj_weight", "proj_bias")}
+    x = load_txt(os.path.join(d, "1_x.txt"))
+    B, T, C = x.shape
+    layer = TransformerBlockLayer(dev.cuda, heads, C, T, "relu", True, 1e-10, sdpa)
+    bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    assert_close(top.mutable_cpu_data, load_txt(os.path.join(d, "10_y.txt")), 2e-6, "block y")
+    assert_close(layer.b["Norm1"].mutable_cpu_data, load_txt(os.path.join(d, "2_x_ln11.txt")), 2e-6, "ln1")
+    assert_close(layer.b["X"].mutable_cpu_data, load_txt(os.path.join(d, "4_x_p_attn.txt")), 2e-6, "x + attn")
+    assert_close(layer.b["MlpOut"].mutable_cpu_data, load_txt(os.path.join(d, "8_x_c_proj.txt")), 2e-5, "mlp")
+
+
+@pytest.mark.parametrize("activation", ["gelu_bert", "gelu", "relu"])
+def test_transformer_block_gpt2_shape_vs_checker(dev, activation):
+    rng = np.random.default_rng(24)
+    B, T, C, H = 2, 64, 128, 2
+    p = {"attn_weight": rng.standard_normal((3 * C, C)) * 0.05, "attn_bias": rng.standard_normal(3 * C) * 0.02,
+         "attn_proj_weight": rng.standard_normal((C, C)) * 0.05, "attn_proj_bias": rng.standard_normal(C) * 0.02,
+         "fc_weight": rng.standard_normal((4 * C, C)) * 0.05, "fc_bias": rng.standard_normal(4 * C) * 0.02,
+         "proj_weight": rng.standard_normal((C, 4 * C)) * 0.05, "proj_bias": rng.standard_normal(C) * 0.02}
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    layer = TransformerBlockLayer(dev.cuda, H, C, T, activation, True, 1e-5, True)
+    bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    ref = R.transformer_block_gpt(x, {k: v.astype(np.float32) for k, v in p.items()}, H, activation, 1e-5, np.float64)
+    assert_close(top.mutable_cpu_data, ref["y"], FP32_RTOL, "block %s" % activation)

@@ -312,3 +312,121 @@ def test_multihead_attention_matches_torch_mha(kind):
         q_proj_weight=t(W[0]), k_proj_weight=t(W[1]), v_proj_weight=t(W[2]))
     assert np.allclose(out["y"], exp.transpose(0, 1).numpy(), rtol=1e-10, atol=1e-10)
     assert np.allclose(out["att"].sum(-1), 1.0)
+
+
+# ---- LayerNorm / GELU / SiLU / RoPE / attention gradients -----------------------------------
+
+@pytest.mark.parametrize("name", ["gpt-pico-ln", "gpt-pico-ln3B"])
+def test_layernorm_golden_forward_backward(name):
+    d = os.path.join(GOLDEN, name)
+    x = load_txt(os.path.join(d, "x.txt"))
+    y, sd = R.layernorm_forward(x, x.shape[-1], 1e-10, np.float64)
+    assert np.abs(y - load_txt(os.path.join(d, "y.txt"))).max() < 3e-7
+    dx = R.layernorm_backward(y, load_txt(os.path.join(d, "grad_1a_y.txt")), sd, x.shape[-1], 1e-10, 1, np.float64)
+    assert np.abs(dx - load_txt(os.path.join(d, "grad_9_x.txt"))).max() < 3e-8
+
+
+def test_layernorm_matches_torch_and_autograd():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 5, 24))
+    dy = rng.standard_normal((2, 5, 24))
+    eps = 1e-5
+    xt = torch.tensor(x, requires_grad=True)
+    yt = F.layer_norm(xt, (24,), eps=eps)
+    yt.backward(torch.tensor(dy))
+    y, sd = R.layernorm_forward(x, 24, eps, np.float64)
+    assert np.allclose(y, yt.detach().numpy(), rtol=1e-12, atol=1e-13)
+    # eps = 0 in the divisor bump: the exact gradient
+    dx = R.layernorm_backward(y, dy, sd, 24, eps, 0, np.float64)
+    assert np.allclose(dx, xt.grad.numpy(), rtol=1e-10, atol=1e-12)
+    # the bump touches the first rows (=10) flat entries only, once per backward call
+    dx2 = R.layernorm_backward(y, dy, sd, 24, eps, 2, np.float64)
+    flat, flat2 = dx.reshape(-1), dx2.reshape(-1)
+    assert np.array_equal(flat[10:], flat2[10:])
+    assert np.allclose(flat2[:10], flat[:10] * sd[0] / (sd[0] + 2 * eps), rtol=1e-12)
+
+
+def test_gelu_golden_and_library():
+    import torch
+    import torch.nn.functional as F
+    d = os.path.join(GOLDEN, "gpt-pico-gelu")
+    x = load_txt(os.path.join(d, "1_x.txt"))
+    y = load_txt(os.path.join(d, "2_y.txt"))
+    dy = load_txt(os.path.join(d, "grad_1_y.txt"))
+    dx = load_txt(os.path.join(d, "grad_2_x.txt"))
+    assert np.abs(R.gelu(x, True, np.float64) - y).max() < 1e-8
+    assert np.abs(R.gelu_grad(x, dy, True, np.float64) - dx).max() < 1e-8
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal(500) * 3
+    g = rng.standard_normal(500)
+    for bert, approx in ((True, "tanh"), (False, "none")):
+        xt = torch.tensor(x, requires_grad=True)
+        yt = F.gelu(xt, approximate=approx)
+        yt.backward(torch.tensor(g))
+        assert np.allclose(R.gelu(x, bert, np.float64), yt.detach().numpy(), rtol=1e-7, atol=1e-9)
+        # the reference's gradient constants are rounded to six digits
+        assert np.allclose(R.gelu_grad(x, g, bert, np.float64), xt.grad.numpy(), rtol=2e-5, atol=2e-6)
+        assert np.allclose(R.gelu(x, bert), R.gelu(x, bert, np.float64), rtol=1e-6, atol=1e-7)
+
+
+def test_silu_grad_and_rope_backward():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal(300) * 4
+    g = rng.standard_normal(300)
+    xt = torch.tensor(x, requires_grad=True)
+    F.silu(xt).backward(torch.tensor(g))
+    assert np.allclose(R.silu_grad(x, g, np.float64), xt.grad.numpy(), rtol=1e-12)
+    # the rotation is orthogonal: <rope(x), dy> == <x, rope_backward(dy)> and backward(forward(x)) == x
+    B, T, H, hs = 2, 5, 3, 8
+    x = rng.standard_normal((B, T, H, hs))
+    dy = rng.standard_normal((B, T, H, hs))
+    y = R.rope_forward(x, T, H, hs, dtype=np.float64)
+    dx = R.rope_backward(dy, T, H, hs, dtype=np.float64)
+    assert abs((y * dy.reshape(y.shape)).sum() - (x * dx.reshape(x.shape)).sum()) < 1e-6
+    assert np.allclose(R.rope_backward(y, T, H, hs, dtype=np.float64).reshape(x.shape), x, atol=1e-6)
+
+
+@pytest.mark.parametrize("name,heads", [("gpt-pico-csa", 1), ("gpt-pico-csa3", 3), ("gpt-pico-csa3B", 3), ("gpt-pico-csaB", 1)])
+def test_attention_backward_golden(name, heads):
+    d = os.path.join(GOLDEN, name)
+    out = R.causal_self_attention(
+        load_txt(os.path.join(d, "x.txt")), load_txt(os.path.join(d, "attn_weight.txt")), load_txt(os.path.join(d, "attn_bias.txt")),
+        load_txt(os.path.join(d, "attn_proj_weight.txt")), load_txt(os.path.join(d, "attn_proj_bias.txt")), heads, dtype=np.float64)
+    g = os.path.join(d, "iter_0")
+    dy = load_txt(os.path.join(g, "grad_y_pre_transpose.txt"))
+    dq, dk, dv = R.attn_backward(out["qt"], out["kt"], out["vt"], out["att"], dy, np.float64)
+    for got, f in ((dq, "grad_qt.txt"), (dk, "grad_kt.txt"), (dv, "grad_vt.txt")):
+        exp = load_txt(os.path.join(g, f))
+        assert np.abs(got - exp.reshape(got.shape)).max() < 1e-8 + 2e-7 * np.abs(exp).max(), f
+
+
+def test_attention_backward_matches_autograd():
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(8)
+    B, H, T, hs = 2, 3, 9, 8
+    q, k, v, dy = (rng.standard_normal((B, H, T, hs)) for _ in range(4))
+    for causal in (True, False):
+        qt, kt, vt = (torch.tensor(a, requires_grad=True) for a in (q, k, v))
+        F.scaled_dot_product_attention(qt, kt, vt, is_causal=causal).backward(torch.tensor(dy))
+        _, att = R.attn_forward(q, k, v, R.causal_mask(T, np.float64) if causal else None, False, np.float64)
+        dq, dk, dv = R.attn_backward(q, k, v, att, dy, np.float64)
+        assert np.allclose(dq, qt.grad.numpy(), rtol=1e-9, atol=1e-11)
+        assert np.allclose(dk, kt.grad.numpy(), rtol=1e-9, atol=1e-11)
+        assert np.allclose(dv, vt.grad.numpy(), rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3B", 3)])
+def test_transformer_block_golden(name, heads):
+    d = os.path.join(GOLDEN, name)
+    p = {k: load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias",
+                                                             "fc_weight", "fc_bias", "proj_weight", "proj_bias")}
+    out = R.transformer_block_gpt(load_txt(os.path.join(d, "1_x.txt")), p, heads, "relu", 1e-10, np.float64)
+    for key, f in (("ln1", "2_x_ln11"), ("attn", "3_x_attn"), ("xb", "4_x_p_attn"), ("ln2", "5_x_ln2"), ("fc", "6_x_c_fc"),
+                   ("act", "7_x_act"), ("mlp", "8_x_c_proj"), ("y", "10_y")):
+        exp = load_txt(os.path.join(d, f + ".txt"))
+        assert np.abs(out[key] - exp.reshape(out[key].shape)).max() < 5e-7, f
