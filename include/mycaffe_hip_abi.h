@@ -87,6 +87,7 @@ enum {
     MCH_FN_ATTN_FREE = 161,
     MCH_FN_ATTN_SET = 162,
     MCH_FN_ATTN_FWD = 163,
+    MCH_FN_ATTN_BWD = 164,
     MCH_FN_SET = 200,
     MCH_FN_COPY = 202,
     MCH_FN_GEMM2 = 219,

@@ -25,7 +25,7 @@ FLAGS = [
     "-I", os.path.join(HERE, "..", "include"),
 ]
 
-KERNEL_SOURCES = ["ew_kernels.hip", "gemm.hip", "attn_prefill.hip", "attn_decode.hip"]
+KERNEL_SOURCES = ["ew_kernels.hip", "gemm.hip", "attn_prefill.hip", "attn_decode.hip", "attn_backward.hip"]
 LIBS = {
     "libmycaffe_hip.so": KERNEL_SOURCES + ["library.hip"],
     "libmycaffe_hip_llama2.so": KERNEL_SOURCES + ["llama2_ext.hip"],

@@ -29,6 +29,7 @@ struct AttnArgs {
     const float* mask;
     int B, H, Tq, Tk, hs, kind;
     float scale;
+    float* lse2;   // optional [B*H*Tq]: log2 of the row's softmax denominator (-inf marks a fully masked row)
 };
 
 // 4 wavefronts per workgroup, one query row each
@@ -89,19 +90,21 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
         int d = lane + i * 64;
         if (d < a.hs) stp(y, d, acc[i] / l);
     }
+    // a causal row's maximum is never the fill value, so the shortened key range above changes nothing here
+    if (a.lse2 && lane == 0) a.lse2[bh * a.Tq + row] = (m == MASKED) ? -INFINITY : (m + __logf(l)) * 1.4426950408889634f;
 }
 
 hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* handled);
 
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
-                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind)
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2)
 {
     if (B <= 0 || H <= 0 || Tq <= 0 || Tk <= 0 || hs <= 0) return hipSuccess;
     if (B > 65535 || H > 65535) return hipErrorInvalidValue;
     if (kind != MASK_NONE && kind != MASK_CAUSAL && mask == nullptr) return hipErrorInvalidValue;
     AttnArgs a;
     a.q = q; a.k = k; a.v = v; a.y = y; a.mask = mask;
-    a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale;
+    a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale; a.lse2 = lse2;
     bool handled = false;
     hipError_t e = attn_flash_launch(s, dt, a, &handled);
     if (e != hipSuccess || handled) return e;
@@ -152,6 +155,7 @@ struct FlashArgs {
     float c;             // softmax scale * log2(e)
     float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
     float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
+    float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
 };
 
 __device__ inline uint32_t pack_bf16x2(float a, float b)
@@ -459,6 +463,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
         const int qrow = q0 + qt * 32 + l32;
         const float lt = l[qt] + __shfl_xor(l[qt], 32, 64);
         const float inv = 1.0f / lt;
+        if (a.lse2 && qrow < a.Tq && half == 0)
+            a.lse2[bh * a.Tq + qrow] = (m[qt] == a.maskedRaw) ? -INFINITY : __builtin_fmaf(m[qt], a.c, __log2f(lt));
         if (qrow < a.Tq) {
             T* yr = (T*)a.y + (bh * a.Tq + qrow) * HS;
 #pragma unroll
@@ -817,6 +823,7 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     f.c = a.scale * 1.4426950408889634f;
     f.maskedRaw = MASKED / a.scale;
     f.lazy = 8.0f / f.c;
+    f.lse2 = a.lse2;
     *handled = true;
     // Tile shapes picked by measurement on MI355X.  Head size 64: four wavefronts with one 32-row tile each
     // (128-row workgroups) give enough equal-sized workgroups to balance 256 CUs at T = 1024; head size 128
@@ -826,7 +833,7 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
             // Unmasked attention runs the software-pipelined kernel (+15..30 %).  Causal launches measure the same
             // or slightly better with the plain kernel (ragged per-wavefront ranges leave the pipeline in its
             // sequential phases more often), so they stay there.
-            if (a.kind == MASK_NONE) {
+            if (a.kind == MASK_NONE && !a.lse2) {   // the pipelined kernel does not keep the row statistics
                 hipLaunchKernelGGL(flash_pipe_bf16_64_kernel<0>, dim3((f.Tq + 127) / 128, f.H, f.B), 256, 0, s, f);
                 return hipGetLastError();
             }

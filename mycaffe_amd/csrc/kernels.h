@@ -83,7 +83,16 @@ enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAU
 //   MASK_QK (Tq,Tk) shared, MASK_KEY (B,Tk), MASK_BQK (B,Tq,Tk); zero entries are filled with -1e29.
 //   MASK_CAUSAL needs no mask buffer (lower triangle kept).
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
-                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind);
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2 = nullptr);
+// With lse2 ([B*H*Tq] fp32) the forward pass also stores log2 of every row's softmax denominator (scores scaled, masked
+// ones at -1e29; -inf marks a row whose keys are all masked), which is all the backward pass needs of the probabilities.
+//
+// Gradients of the same attention: dq, dk, dv from dy (attn_backward.hip).  lse2 as stored by the forward pass, or
+// nullptr to have it recomputed (slow path).  workspace: attn_backward_workspace_bytes(B, H, Tq).
+size_t attn_backward_workspace_bytes(int B, int H, int Tq);
+hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k, const void* v, const void* y, const void* dy,
+                           void* dq, void* dk, void* dv, int B, int H, int Tq, int Tk, int hs, float scale, const float* mask,
+                           MaskKind kind, const float* lse2, void* workspace, size_t workspaceBytes);
 size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
 // one query per (b,h): q (B,H,hs), caches addressed as
 //   cache[b*strideB + (h/kvMul)*strideH + t*strideT + i], y (B,H,hs).  All dt.

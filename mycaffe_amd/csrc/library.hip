@@ -1057,6 +1057,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         st->scale = (float)(1.0 / sqrt((double)st->hs));  // attn.cu:427
         st->set = true;
         st->maskHandle = 0;
+        st->lseValid = false;
+        st->lastTq = st->lastTk = 0;
         return 0;
     }
     case MCH_FN_ATTN_FWD: {
@@ -1100,8 +1102,75 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 kind = (T == Tk && mask_is_causal(st, hMask, M, T)) ? MASK_CAUSAL : MASK_QK;
             }
         }
+        float* lse = nullptr;
+        st->lseValid = false;
+        if (st->training) {
+            // training mode: keep one number per query row for ATTN_BWD (the reference keeps the T x T probabilities)
+            const size_t rows = (size_t)st->batch * st->heads * T;
+            if (st->lseCap < rows) {
+                if (st->lse) { HIPCHK(hipStreamSynchronize(s)); (void)hipFree(st->lse); st->lse = nullptr; st->lseCap = 0; }
+                HIPCHK(hipMalloc((void**)&st->lse, rows * sizeof(float)));
+                st->lseCap = rows;
+            }
+            lse = st->lse;
+        }
         HIPCHK(k_attn_prefill(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, st->batch, st->heads, T, Tk, st->hs, st->scale,
-                              M ? (const float*)M->ptr : nullptr, kind));
+                              M ? (const float*)M->ptr : nullptr, kind, lse));
+        st->lseValid = lse != nullptr;
+        st->lastTq = T; st->lastTk = Tk; st->lastBatchMask = batchMask;
+        m_mem.touch((long)pl[7]);
+        return 0;
+    }
+    case MCH_FN_ATTN_BWD: {
+        // l{hCudnn,hAttn,hQ,hdQ,hK,hdK,hV,hdV,hMask,hY,hdY} (CudaDnn.cs:5695-5701, device.h:2509-2529, attn.cu:608-661).
+        // Sequence lengths and the mask layout are those of the handle's last forward call (the reference reads
+        // the probabilities that call left behind); without one, the block size given to ATTN_SET is used.
+        NEED_L(11, 11);
+        AttnState* st = m_attn.get((long)pl[1]);
+        if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        if (st->dropout > 0.f && st->training) { last_detail = "attention dropout is not part of this path"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const int T = st->lastTq > 0 ? st->lastTq : st->block, Tk = st->lastTq > 0 ? st->lastTk : st->block;
+        const long long batchMask = st->lastTq > 0 ? st->lastBatchMask : 0;
+        MemItem *Q, *dQ, *K, *dK, *V, *dV, *Y, *dY, *M = nullptr;
+        ERRCHK(mem((long)pl[2], &Q));
+        ERRCHK(mem((long)pl[3], &dQ));
+        ERRCHK(mem((long)pl[4], &K));
+        ERRCHK(mem((long)pl[5], &dK));
+        ERRCHK(mem((long)pl[6], &V));
+        ERRCHK(mem((long)pl[7], &dV));
+        ERRCHK(mem((long)pl[9], &Y));
+        ERRCHK(mem((long)pl[10], &dY));
+        long hMask = (long)pl[8];
+        if (hMask) ERRCHK(mem(hMask, &M));
+        for (MemItem* it : {dQ, K, dK, V, dV, Y, dY})
+            if (it->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        long long qn = (long long)st->batch * st->heads * T * st->hs, kn = (long long)st->batch * st->heads * Tk * st->hs;
+        if ((long long)Q->count < qn || (long long)dQ->count < qn || (long long)Y->count < qn || (long long)dY->count < qn ||
+            (long long)K->count < kn || (long long)dK->count < kn || (long long)V->count < kn || (long long)dV->count < kn)
+            return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+        MaskKind kind = MASK_NONE;
+        if (M) {
+            if (M->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+            if (batchMask == 2) {
+                if ((long long)M->count < (long long)st->batch * T * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = MASK_BQK;
+            } else if (batchMask == 1) {
+                if ((long long)M->count < (long long)st->batch * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = MASK_KEY;
+            } else {
+                if ((long long)M->count < (long long)T * Tk) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+                kind = (T == Tk && mask_is_causal(st, hMask, M, T)) ? MASK_CAUSAL : MASK_QK;
+            }
+        }
+        void* ws;
+        const size_t wsBytes = attn_backward_workspace_bytes(st->batch, st->heads, T);
+        ERRCHK(workspace(wsBytes, &ws));
+        const bool haveLse = st->lseValid && st->lseCap >= (size_t)st->batch * st->heads * T;
+        HIPCHK(k_attn_backward(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, dY->ptr, dQ->ptr, dK->ptr, dV->ptr, st->batch, st->heads,
+                               T, Tk, st->hs, st->scale, M ? (const float*)M->ptr : nullptr, kind, haveLse ? st->lse : nullptr,
+                               ws, wsBytes));
+        m_mem.touch((long)pl[3]);
+        m_mem.touch((long)pl[5]);
         m_mem.touch((long)pl[7]);
         return 0;
     }

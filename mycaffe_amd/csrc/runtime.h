@@ -77,6 +77,10 @@ struct AttnState {
     float dropout = 0.f, scale = 1.f;
     // cache of "the (T,T) mask is the lower-triangular ones matrix"
     long maskHandle = 0; uint64_t maskVersion = 0; int maskT = 0; bool maskCausal = false;
+    // what the backward pass needs of the last training-mode forward: log2 of every row's softmax denominator
+    float* lse = nullptr; size_t lseCap = 0; bool lseValid = false;
+    int lastTq = 0, lastTk = 0; long long lastBatchMask = 0;
+    ~AttnState() { if (lse) (void)hipFree(lse); }
 };
 struct RopeState {
     bool set = false;

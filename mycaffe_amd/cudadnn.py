@@ -55,6 +55,7 @@ class CUDAFN:
     CUDA_ATTN_FREE = 161
     CUDA_ATTN_SET = 162
     CUDA_ATTN_FWD = 163
+    CUDA_ATTN_BWD = 164
     CUDA_SET = 200
     CUDA_COPY = 202
     CUDA_GEMM2 = 219
@@ -561,6 +562,10 @@ class CudaDnn:
         if nBlockSizeK is not None:
             rgl.append(nBlockSizeK)
         self._ex2(CUDAFN.CUDA_ATTN_FWD, None, rgl)
+
+    def AttnScaledDotProductBackward(self, hCuDnn, hAttn, hQdata, hQdiff, hKdata, hKdiff, hVdata, hVdiff, hMaskdata, hYData, hYdiff):
+        """CudaDnn.cs:5695-5701."""
+        self._ex2(CUDAFN.CUDA_ATTN_BWD, None, [hCuDnn, hAttn, hQdata, hQdiff, hKdata, hKdiff, hVdata, hVdiff, hMaskdata, hYData, hYdiff])
 
     def AttnDecodeForward(self, nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead,
                           nStridePos, fScale=0.0, hRope=0, hKNew=0, hVNew=0):
