@@ -192,6 +192,37 @@ def bench_prefill_attention(cuda, reps, warm=5):
     return out
 
 
+def bench_attention_backward(cuda, reps, warm=5):
+    """Gradients of the fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_BWD (id 164): the statistics
+    kernel plus the dK/dV and dQ kernels of one call."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    B, H, T, hs = 8, 12, 1024, 64
+    rng = np.random.default_rng(0)
+    out = {}
+    mask = cuda.AllocMemory(np.tril(np.ones((T, T), np.float32)))
+    hc, ha = cuda.CreateCuDNN(), cuda.CreateAttn()
+    cuda.SetAttn(hc, ha, 0, True, B, T, H, hs, 0.0)
+    n = B * H * T * hs
+    for name, half in (("bf16", True), ("f32", False)):
+        q, k, v, dy = (cuda.AllocMemory(rng.standard_normal(n).astype(np.float32), bHalfSize=half) for _ in range(4))
+        y, dq, dk, dv = (cuda.AllocMemory(n, bHalfSize=half) for _ in range(4))
+        cuda.AttnScaledDotProductForward(hc, ha, T, q, k, v, mask, y, False)
+        rgl = [hc, ha, q, dq, k, dk, v, dv, mask, y, dy]
+        cuda.AttnScaledDotProductBackward(hc, ha, q, dq, k, dk, v, dv, mask, y, dy)
+        ms = cuda.TimeFunction(CUDAFN.CUDA_ATTN_BWD, None, rgl, warm, reps)
+        # five T x T x hs products are the mathematical minimum (dV, dP, dQ, dK and the recomputed scores); causal half
+        useful = 5.0 * B * H * T * T * hs
+        tf = useful / (ms / 1e3) / 1e12
+        out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2),
+                     "roofline": {"kernel": "fused causal attention backward (3 kernels)", "bound": "mfma", "achieved": round(tf, 2),
+                                  "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
+                                  "traffic": None}}
+        for h in (q, k, v, dy, y, dq, dk, dv):
+            cuda.FreeMemory(h)
+    cuda.FreeMemory(mask)
+    return out
+
+
 def bench_decode_attention(cuda, reps, warm=5, cases=None):
     """KV-cache attention, 32 heads x 128, one query token per sequence (id 2001)."""
     from mycaffe_amd.cudadnn import CUDAFN
@@ -334,7 +365,7 @@ def main():
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
                     "prints what ran instead of the benchmark line")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,decode_attn,encdec,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -379,6 +410,9 @@ def main():
     if want("decode_attn"):
         also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
         log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
+    if want("backward"):
+        also["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 30)
+        log("attention backward:", json.dumps(also["attention_backward_B8_T1024_H12x64"]))
     if want("encdec"):
         also["encdec_attention_B32_H8x64_bf16"] = bench_encdec_attention(cuda, 50)
         log("enc-dec attention:", json.dumps(also["encdec_attention_B32_H8x64_bf16"]))

@@ -17,6 +17,7 @@
 //    per query row (per key row), lanes over the other sequence axis.  No atomics: every output row has one owner, so
 //    results do not depend on scheduling.
 //  * MFMA tiles for head sizes 64 and 128 (further down).
+#include "flash_traits.h"
 #include "kernels.h"
 
 namespace mch {
@@ -261,11 +262,407 @@ hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k
 }
 
 // ---------------------------------------------------------------------------
-// MFMA path (placeholder dispatch until the tiles below are enabled per shape)
-hipError_t attn_bwd_mfma_launch(hipStream_t, DType, const AttnBwdArgs&, bool* handled)
+// MFMA tiles for head sizes 64 and 128, bf16 and fp32 storage (fragment conventions: flash_traits.h).
+//
+// A 32x32 accumulator keeps its column in the lane and its rows in the registers, and it can feed the next MFMA only
+// as an operand whose contraction runs over those rows.  So each gradient is computed in the orientation whose
+// contraction index is the one the probabilities have in registers:
+//
+//   dK, dV (attn_bwd_dkv_mfma_kernel): a wavefront owns 32 keys (lane = key) and walks the queries.
+//       S  = Q K^T        A = Q rows from LDS,  B = K fragments held in registers
+//       dP = dY V^T       A = dY rows from LDS, B = V fragments held in registers
+//       P  = exp2(S c - lse2[query]),  dS = P (dP - D[query])       query = register row: lse2, D come from LDS
+//       dV^T += dY^T P    A = dY^T from LDS (transposed while staged), B = P from registers
+//       dK^T += Q^T dS    A = Q^T  from LDS (transposed while staged), B = dS from registers
+//   dQ (attn_bwd_dq_mfma_kernel): a wavefront owns 32 queries (lane = query) and walks the keys.
+//       S^T  = K Q^T      A = K rows from LDS,  B = Q fragments held in registers
+//       dP^T = V dY^T     A = V rows from LDS,  B = dY fragments held in registers
+//       P^T, dS^T as above with lse2, D per lane
+//       dQ^T += K^T dS^T  A = K^T from LDS (transposed while staged), B = dS^T from registers
+//
+// The softmax scale is applied once to the dQ / dK accumulators at the end.  Every output row has exactly one owner
+// and the order of accumulation is fixed, so results are reproducible run to run.  Causal launches skip the tiles above
+// the diagonal and are ordered heaviest workgroup first.
+template <typename T, int HS, int BS> struct BwdTile {
+    typedef FlashTraits<T> TR;
+    static constexpr int NT = 256;
+    static constexpr int EPC = TR::EPC, CPF = TR::CPF;
+    static constexpr int KF = HS / CPF;          // fragments along the head dimension
+    static constexpr int PF = 32 / CPF;          // fragments along a 32-row step
+    static constexpr int DT = HS / 32;
+    static constexpr int PAD = 16 / (int)sizeof(T);
+    static constexpr int LDR = HS + PAD;         // row-major LDS stride
+    static constexpr int LDT = BS + PAD;         // transposed LDS stride
+    static constexpr int CHR = HS / EPC;         // 16-byte chunks per row
+    static constexpr int TPR = NT / BS;          // threads per staged row
+    static constexpr int CPT = CHR / TPR;        // chunks per thread per staged array
+    static_assert(CHR % TPR == 0 && CPT >= 1 && BS % 32 == 0, "stage / thread mismatch");
+};
+
+template <int KIND> __device__ inline bool bwd_masked(const AttnBwdArgs& a, int b, int mb, int qrow, int key, bool keyMasked)
+{
+    if (KIND == 1) return key > qrow;
+    if (KIND == 2) return keyMasked;
+    if (KIND == 3) return qrow < a.Tq && key < a.Tk && a.mask[((size_t)b * mb * a.Tq + qrow) * a.Tk + key] == 0.f;
+    return false;
+}
+
+// KIND: 0 none, 1 causal, 2 key mask (B,Tk), 3 mask (B,Tq,Tk) or, with mb = 0, one (Tq,Tk) mask for all sequences
+template <typename T, int HS, int KIND, int BQ, int OCC>
+__global__ __launch_bounds__(256, OCC) void attn_bwd_dkv_mfma_kernel(AttnBwdArgs a, int mb)
+{
+    typedef BwdTile<T, HS, BQ> TL;
+    typedef FlashTraits<T> TR;
+    constexpr int NW = 4, BK = NW * 32;
+    constexpr int EPC = TL::EPC, CPF = TL::CPF, KF = TL::KF, PF = TL::PF, DT = TL::DT, LDR = TL::LDR, LDT = TL::LDT;
+    constexpr int TPR = TL::TPR, CPT = TL::CPT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    T* Qs = (T*)bwd_smem;
+    T* Gs = Qs + BQ * LDR;
+    T* Qt = Gs + BQ * LDR;
+    T* Gt = Qt + HS * LDT;
+    float* Ls = (float*)(Gt + HS * LDT);
+    float* Ds = Ls + BQ;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int nbh = a.B * a.H;
+    const int kblock = blockIdx.x / nbh;            // causal: low key blocks see the most queries and start first
+    const int ibh = blockIdx.x % nbh;
+    const int b = ibh / a.H, h = ibh % a.H;
+    const size_t bh = (size_t)b * a.H + h;
+    const int kw = kblock * BK + wave * 32;          // first key of this wavefront
+    const int key = kw + l32;
+    const bool waveActive = kw < a.Tk;
+    const T* qp = (const T*)a.q + bh * a.Tq * HS;
+    const T* gp = (const T*)a.dy + bh * a.Tq * HS;
+    const T* kp = (const T*)a.k + bh * a.Tk * HS;
+    const T* vp = (const T*)a.v + bh * a.Tk * HS;
+    const float* lse = a.lse2 + bh * a.Tq;
+    const float* dsm = a.dsum + bh * a.Tq;
+
+    u32x4 kf[KF], vf[KF];
+    {
+        const size_t r = (size_t)min(key, a.Tk - 1) * HS;
+#pragma unroll
+        for (int f = 0; f < KF; f++) {
+            kf[f] = *(const u32x4*)(kp + r + f * CPF + half * (CPF / 2));
+            vf[f] = *(const u32x4*)(vp + r + f * CPF + half * (CPF / 2));
+        }
+    }
+    bool keyMasked = false;
+    if (KIND == 2) keyMasked = a.mask[(size_t)b * a.Tk + min(key, a.Tk - 1)] == 0.f;
+    floatx16 ak[DT], av[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { ak[dt][v] = 0.f; av[dt][v] = 0.f; }
+
+    const int srow = tid % BQ, cg = tid / BQ;
+    u32x4 qreg[CPT], greg[CPT];
+    float lreg = 0.f, dreg = 0.f;
+    auto gload = [&](int q0) {
+        const size_t r = (size_t)min(q0 + srow, a.Tq - 1) * HS;
+#pragma unroll
+        for (int i = 0; i < CPT; i++) {
+            qreg[i] = *(const u32x4*)(qp + r + (cg + TPR * i) * EPC);
+            greg[i] = *(const u32x4*)(gp + r + (cg + TPR * i) * EPC);
+        }
+        if (tid < BQ) {
+            const int qq = q0 + tid;
+            // rows past the end get lse2 = +inf: their probabilities come out as exactly 0
+            lreg = qq < a.Tq ? lse[qq] : INFINITY;
+            dreg = qq < a.Tq ? dsm[qq] : 0.f;
+        }
+    };
+    auto sstore = [&]() {
+#pragma unroll
+        for (int i = 0; i < CPT; i++) {
+            const int c = cg + TPR * i;
+            *(u32x4*)(&Qs[srow * LDR + c * EPC]) = qreg[i];
+            *(u32x4*)(&Gs[srow * LDR + c * EPC]) = greg[i];
+            TR::scatter_chunk(&Qt[c * EPC * LDT + srow], LDT, qreg[i]);
+            TR::scatter_chunk(&Gt[c * EPC * LDT + srow], LDT, greg[i]);
+        }
+        if (tid < BQ) { Ls[tid] = lreg; Ds[tid] = dreg; }
+    };
+
+    const float c = a.scale * LOG2E;
+    const float uniform = 1.0f / a.Tk;
+    const int qbegin = (KIND == 1) ? (kblock * BK / BQ) * BQ : 0;   // causal: earlier queries see none of these keys
+    if (qbegin < a.Tq) {
+        gload(qbegin);
+        sstore();
+    }
+#pragma unroll
+    for (int f = 0; f < KF; f++) { asm volatile("" : "+v"(kf[f])); asm volatile("" : "+v"(vf[f])); }
+    __syncthreads();
+    for (int q0 = qbegin; q0 < a.Tq; q0 += BQ) {
+        const bool more = q0 + BQ < a.Tq;
+        if (more) gload(q0 + BQ);
+        if (waveActive) {
+#pragma unroll
+            for (int sub = 0; sub < BQ / 32; sub++) {
+                const int qs0 = q0 + 32 * sub;
+                if (qs0 >= a.Tq) continue;
+                if (KIND == 1 && qs0 + 31 < kw) continue;     // every (query, key) pair of the tile is masked
+                floatx16 s, dp;
+#pragma unroll
+                for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+                for (int f = 0; f < KF; f++) {
+                    const u32x4 qa = *(const u32x4*)(&Qs[(sub * 32 + l32) * LDR + f * CPF + half * (CPF / 2)]);
+                    s = TR::mma(qa, kf[f], s);
+                    const u32x4 ga = *(const u32x4*)(&Gs[(sub * 32 + l32) * LDR + f * CPF + half * (CPF / 2)]);
+                    dp = TR::mma(ga, vf[f], dp);
+                }
+                // register v: query qs0 + 8*(v/4) + 4*half + v%4, key = this lane's
+                const bool maskedTile = (KIND >= 2) || (KIND == 1 && qs0 < kw + 31);   // wavefront-uniform
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4 l4 = *(const float4*)(&Ls[sub * 32 + 8 * g + 4 * half]);
+                    const float4 d4 = *(const float4*)(&Ds[sub * 32 + 8 * g + 4 * half]);
+                    const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dv4[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int v = 4 * g + j;
+                        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -lv[j]));
+                        if (maskedTile) {
+                            const int qrow = qs0 + 8 * g + 4 * half + j;
+                            if (bwd_masked<KIND>(a, b, mb, qrow, key, keyMasked)) p = 0.f;
+                            if (KIND >= 2 && lv[j] == -INFINITY) p = uniform;   // fully masked row: uniform over all keys
+                        }
+                        s[v] = p;
+                        dp[v] = p * (dp[v] - dv4[j]);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < PF; t++) {
+                    const u32x4 pp = TR::pack_p(s, t), dd = TR::pack_p(dp, t);
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        const u32x4 gt = TR::load_vt(&Gt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        av[dt] = TR::mma(gt, pp, av[dt]);
+                        const u32x4 qt = TR::load_vt(&Qt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        ak[dt] = TR::mma(qt, dd, ak[dt]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (more) sstore();
+        __syncthreads();
+    }
+    // dk[key, d] = scale * dK^T[d, key]; register v of tile dt is d = 32*dt + 8*(v/4) + 4*half + v%4
+    if (waveActive && key < a.Tk) {
+        T* dkr = (T*)a.dk + (bh * a.Tk + key) * HS;
+        T* dvr = (T*)a.dv + (bh * a.Tk + key) * HS;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = 32 * dt + 8 * g + 4 * half;
+                TR::store4(dkr + d, ak[dt][4 * g] * a.scale, ak[dt][4 * g + 1] * a.scale, ak[dt][4 * g + 2] * a.scale,
+                           ak[dt][4 * g + 3] * a.scale);
+                TR::store4(dvr + d, av[dt][4 * g], av[dt][4 * g + 1], av[dt][4 * g + 2], av[dt][4 * g + 3]);
+            }
+    }
+}
+
+template <typename T, int HS, int KIND, int BKS, int OCC>
+__global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs a, int mb)
+{
+    typedef BwdTile<T, HS, BKS> TL;
+    typedef FlashTraits<T> TR;
+    constexpr int NW = 4, BM = NW * 32;
+    constexpr int EPC = TL::EPC, CPF = TL::CPF, KF = TL::KF, PF = TL::PF, DT = TL::DT, LDR = TL::LDR, LDT = TL::LDT;
+    constexpr int TPR = TL::TPR, CPT = TL::CPT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    T* Ks = (T*)bwd_smem;
+    T* Vs = Ks + BKS * LDR;
+    T* Kt = Vs + BKS * LDR;
+    float* Ms = (float*)(Kt + HS * LDT);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int nbh = a.B * a.H;
+    const int nqb = (a.Tq + BM - 1) / BM;
+    const int qblock = (KIND == 1) ? nqb - 1 - (int)(blockIdx.x / nbh) : (int)(blockIdx.x / nbh);   // causal: heaviest first
+    const int ibh = blockIdx.x % nbh;
+    const int b = ibh / a.H, h = ibh % a.H;
+    const size_t bh = (size_t)b * a.H + h;
+    const int q0w = qblock * BM + wave * 32;
+    const int qrow = q0w + l32;
+    const bool waveActive = q0w < a.Tq;
+    const T* qp = (const T*)a.q + bh * a.Tq * HS;
+    const T* gp = (const T*)a.dy + bh * a.Tq * HS;
+    const T* kp = (const T*)a.k + bh * a.Tk * HS;
+    const T* vp = (const T*)a.v + bh * a.Tk * HS;
+
+    u32x4 qf[KF], gf[KF];
+    {
+        const size_t r = (size_t)min(qrow, a.Tq - 1) * HS;
+#pragma unroll
+        for (int f = 0; f < KF; f++) {
+            qf[f] = *(const u32x4*)(qp + r + f * CPF + half * (CPF / 2));
+            gf[f] = *(const u32x4*)(gp + r + f * CPF + half * (CPF / 2));
+        }
+    }
+    const float lrow = qrow < a.Tq ? a.lse2[bh * a.Tq + qrow] : INFINITY;
+    const float drow = qrow < a.Tq ? a.dsum[bh * a.Tq + qrow] : 0.f;
+    floatx16 aq[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) aq[dt][v] = 0.f;
+
+    const int srow = tid % BKS, cg = tid / BKS;
+    u32x4 kreg[CPT], vreg[CPT];
+    float mreg = 1.f;
+    auto gload = [&](int k0) {
+        const size_t r = (size_t)min(k0 + srow, a.Tk - 1) * HS;
+#pragma unroll
+        for (int i = 0; i < CPT; i++) {
+            kreg[i] = *(const u32x4*)(kp + r + (cg + TPR * i) * EPC);
+            vreg[i] = *(const u32x4*)(vp + r + (cg + TPR * i) * EPC);
+        }
+        if (KIND == 2 && tid < BKS) mreg = (k0 + tid < a.Tk) ? a.mask[(size_t)b * a.Tk + k0 + tid] : 1.f;
+    };
+    auto sstore = [&]() {
+#pragma unroll
+        for (int i = 0; i < CPT; i++) {
+            const int c = cg + TPR * i;
+            *(u32x4*)(&Ks[srow * LDR + c * EPC]) = kreg[i];
+            *(u32x4*)(&Vs[srow * LDR + c * EPC]) = vreg[i];
+            TR::scatter_chunk(&Kt[c * EPC * LDT + srow], LDT, kreg[i]);
+        }
+        if (KIND == 2 && tid < BKS) Ms[tid] = mreg;
+    };
+
+    const float c = a.scale * LOG2E;
+    const float uniform = 1.0f / a.Tk;
+    int kend = a.Tk;
+    if (KIND == 1) kend = min(a.Tk, qblock * BM + BM);
+    gload(0);
+    sstore();
+#pragma unroll
+    for (int f = 0; f < KF; f++) { asm volatile("" : "+v"(qf[f])); asm volatile("" : "+v"(gf[f])); }
+    __syncthreads();
+    for (int kb = 0; kb < kend; kb += BKS) {
+        const bool more = kb + BKS < kend;
+        if (more) gload(kb + BKS);
+        if (waveActive) {
+#pragma unroll
+            for (int sub = 0; sub < BKS / 32; sub++) {
+                const int k0 = kb + 32 * sub;
+                if (k0 >= a.Tk) continue;
+                if (KIND == 1 && k0 > q0w + 31) continue;     // keys past this wavefront's last row
+                floatx16 s, dp;
+#pragma unroll
+                for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+                for (int f = 0; f < KF; f++) {
+                    const u32x4 ka = *(const u32x4*)(&Ks[(sub * 32 + l32) * LDR + f * CPF + half * (CPF / 2)]);
+                    s = TR::mma(ka, qf[f], s);
+                    const u32x4 va = *(const u32x4*)(&Vs[(sub * 32 + l32) * LDR + f * CPF + half * (CPF / 2)]);
+                    dp = TR::mma(va, gf[f], dp);
+                }
+                // register v: key k0 + 8*(v/4) + 4*half + v%4, query = this lane's
+                const bool maskedTile = (KIND >= 2) || (KIND == 1 && k0 + 31 > q0w) || (k0 + 32 > a.Tk);   // wavefront-uniform
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -lrow));
+                    if (maskedTile) {
+                        const int kl = 8 * (v >> 2) + 4 * half + (v & 3);
+                        const int key = k0 + kl;
+                        if (bwd_masked<KIND>(a, b, mb, qrow, key, KIND == 2 && Ms[32 * sub + kl] == 0.f)) p = 0.f;
+                        if (KIND >= 2 && lrow == -INFINITY) p = uniform;
+                        if (key >= a.Tk) p = 0.f;
+                    }
+                    dp[v] = p * (dp[v] - drow);
+                }
+#pragma unroll
+                for (int t = 0; t < PF; t++) {
+                    const u32x4 dd = TR::pack_p(dp, t);
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        const u32x4 kt = TR::load_vt(&Kt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        aq[dt] = TR::mma(kt, dd, aq[dt]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (more) sstore();
+        __syncthreads();
+    }
+    if (waveActive && qrow < a.Tq) {
+        T* dqr = (T*)a.dq + (bh * a.Tq + qrow) * HS;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                TR::store4(dqr + 32 * dt + 8 * g + 4 * half, aq[dt][4 * g] * a.scale, aq[dt][4 * g + 1] * a.scale,
+                           aq[dt][4 * g + 2] * a.scale, aq[dt][4 * g + 3] * a.scale);
+    }
+}
+
+template <typename T, int HS, int BS, int OCC, int KIND>
+static hipError_t bwd_launch_kind(hipStream_t s, const AttnBwdArgs& a, int mb)
+{
+    typedef BwdTile<T, HS, BS> TL;
+    const size_t kvBytes = ((size_t)2 * BS * TL::LDR + (size_t)2 * HS * TL::LDT) * sizeof(T) + 2 * BS * sizeof(float);
+    const size_t qBytes = ((size_t)2 * BS * TL::LDR + (size_t)HS * TL::LDT) * sizeof(T) + BS * sizeof(float);
+    auto kkv = attn_bwd_dkv_mfma_kernel<T, HS, KIND, BS, OCC>;
+    auto kq = attn_bwd_dq_mfma_kernel<T, HS, KIND, BS, OCC>;
+    static bool configured = false;   // per instantiation; the attribute is idempotent, so a race only repeats the call
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kkv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kvBytes);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)kq, hipFuncAttributeMaxDynamicSharedMemorySize, (int)qBytes);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const int nbh = a.B * a.H;
+    const long long gkv = (long long)((a.Tk + 127) / 128) * nbh, gq = (long long)((a.Tq + 127) / 128) * nbh;
+    if (gkv > 0x7fffffffll || gq > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kkv, dim3((unsigned)gkv), 256, kvBytes, s, a, mb);
+    hipLaunchKernelGGL(kq, dim3((unsigned)gq), 256, qBytes, s, a, mb);
+    return hipGetLastError();
+}
+
+template <typename T, int HS, int BS, int OCC> static hipError_t bwd_launch_cfg(hipStream_t s, const AttnBwdArgs& a, int kind, int mb)
+{
+    switch (kind) {
+    case 0: return bwd_launch_kind<T, HS, BS, OCC, 0>(s, a, mb);
+    case 1: return bwd_launch_kind<T, HS, BS, OCC, 1>(s, a, mb);
+    case 2: return bwd_launch_kind<T, HS, BS, OCC, 2>(s, a, mb);
+    default: return bwd_launch_kind<T, HS, BS, OCC, 3>(s, a, mb);
+    }
+}
+
+hipError_t attn_bwd_mfma_launch(hipStream_t s, DType dt, const AttnBwdArgs& a, bool* handled)
 {
     *handled = false;
-    return hipSuccess;
+    if (a.hs != 64 && a.hs != 128) return hipSuccess;
+    if ((((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.dy | (uintptr_t)a.dq | (uintptr_t)a.dk | (uintptr_t)a.dv) & 15) != 0)
+        return hipSuccess;
+    int kind, mb = 1;
+    switch (a.kind) {
+    case MASK_NONE: kind = 0; break;
+    case MASK_CAUSAL: kind = 1; break;
+    case MASK_KEY: kind = 2; break;
+    case MASK_BQK: kind = 3; break;
+    case MASK_QK: kind = 3; mb = 0; break;     // one (Tq,Tk) mask for every sequence
+    default: return hipSuccess;
+    }
+    *handled = true;
+    if (dt == BF16) {
+        if (a.hs == 64) return bwd_launch_cfg<bf16_t, 64, 64, 2>(s, a, kind, mb);
+        return bwd_launch_cfg<bf16_t, 128, 32, 1>(s, a, kind, mb);
+    }
+    if (a.hs == 64) return bwd_launch_cfg<float, 64, 32, 2>(s, a, kind, mb);
+    return bwd_launch_cfg<float, 128, 32, 1>(s, a, kind, mb);
 }
 
 }  // namespace mch

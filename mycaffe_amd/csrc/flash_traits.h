@@ -1,0 +1,90 @@
+// MFMA operand fragments shared by the attention forward and backward kernels (gfx950).
+//
+// One fragment is 16 bytes per lane.  bf16: v_mfma_f32_32x32x16_bf16, a fragment covers 16 contraction indices (lane half
+// h holds 8 of them).  fp32: v_mfma_f32_32x32x2_f32 four times per fragment; lane half h holds indices 4h..4h+3 of an
+// 8-index group and step e contracts the pair {e, 4+e}, which is legal because the slot-to-index assignment only has to
+// agree between the A and the B operand.  Accumulator register v of a lane holds row 8*(v/4) + 4*(lane/32) + v%4,
+// column lane%32 of the 32x32 result.
+#pragma once
+#include "kernels.h"
+
+namespace mch {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // one 16-byte MFMA operand fragment
+
+__device__ inline uint32_t pack_bf16x2(float a, float b)
+{
+    floatx2 f = {a, b};
+    bf16x2 r = __builtin_convertvector(f, bf16x2);
+    return *reinterpret_cast<uint32_t*>(&r);
+}
+
+template <typename T> struct FlashTraits;
+template <> struct FlashTraits<bf16_t> {
+    static constexpr int EPC = 8;    // elements per 16-byte chunk
+    static constexpr int CPF = 16;   // contraction indices covered by one fragment (both lane halves)
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&a), *reinterpret_cast<bf16x8*>(&b), c, 0, 0, 0);
+    }
+    // V^T fragment t of a 32-key step: keys 16t + 4h .. +3 and 16t + 8 + 4h .. +3
+    __device__ static inline u32x4 load_vt(const bf16_t* row, int t, int half)
+    {
+        const bf16_t* p = row + 16 * t + 4 * half;
+        uint2 lo = *(const uint2*)p, hi = *(const uint2*)(p + 8);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+    // P^T fragment t: the weights held in accumulator registers 8t .. 8t+7
+    __device__ static inline u32x4 pack_p(const floatx16& p, int t)
+    {
+        return u32x4{pack_bf16x2(p[8 * t], p[8 * t + 1]), pack_bf16x2(p[8 * t + 2], p[8 * t + 3]),
+                     pack_bf16x2(p[8 * t + 4], p[8 * t + 5]), pack_bf16x2(p[8 * t + 6], p[8 * t + 7])};
+    }
+    __device__ static inline void store4(bf16_t* dst, float a, float b, float c, float d)
+    {
+        uint2 w;
+        w.x = pack_bf16x2(a, b);
+        w.y = pack_bf16x2(c, d);
+        *(uint2*)dst = w;
+    }
+    __device__ static inline void scatter_chunk(bf16_t* d, int ld, u32x4 r)
+    {
+        d[0 * ld] = (bf16_t)(r.x & 0xffffu); d[1 * ld] = (bf16_t)(r.x >> 16);
+        d[2 * ld] = (bf16_t)(r.y & 0xffffu); d[3 * ld] = (bf16_t)(r.y >> 16);
+        d[4 * ld] = (bf16_t)(r.z & 0xffffu); d[5 * ld] = (bf16_t)(r.z >> 16);
+        d[6 * ld] = (bf16_t)(r.w & 0xffffu); d[7 * ld] = (bf16_t)(r.w >> 16);
+    }
+};
+template <> struct FlashTraits<float> {
+    static constexpr int EPC = 4;
+    static constexpr int CPF = 8;
+    __device__ static inline floatx16 mma(u32x4 a, u32x4 b, floatx16 c)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+        return c;
+    }
+    // V^T fragment t of a 32-key step: keys 8t + 4h .. +3
+    __device__ static inline u32x4 load_vt(const float* row, int t, int half) { return *(const u32x4*)(row + 8 * t + 4 * half); }
+    // P^T fragment t: the weights held in accumulator registers 4t .. 4t+3
+    __device__ static inline u32x4 pack_p(const floatx16& p, int t)
+    {
+        return u32x4{__float_as_uint(p[4 * t]), __float_as_uint(p[4 * t + 1]), __float_as_uint(p[4 * t + 2]),
+                     __float_as_uint(p[4 * t + 3])};
+    }
+    __device__ static inline void store4(float* dst, float a, float b, float c, float d) { *(float4*)dst = make_float4(a, b, c, d); }
+    __device__ static inline void scatter_chunk(float* d, int ld, u32x4 r)
+    {
+        d[0 * ld] = __uint_as_float(r.x); d[1 * ld] = __uint_as_float(r.y);
+        d[2 * ld] = __uint_as_float(r.z); d[3 * ld] = __uint_as_float(r.w);
+    }
+};
+
+
+}  // namespace mch

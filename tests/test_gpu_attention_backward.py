@@ -114,6 +114,18 @@ def test_attn_backward_masks(dev, hs, half):
     _check(out, q, k, v, dy, m, 0, tol, "(T,T) mask")
 
 
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attn_backward_gpt2_sequence_length(dev, causal, half):
+    """T = 1024, 64-wide heads (the shape the prefill benchmark uses), fewer sequences so the fp64 checker stays small."""
+    rng = np.random.default_rng(51)
+    B, H, T, hs = 1, 3, 1024, 64
+    q, k, v, dy = (bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(4))
+    mask = R.causal_mask(T) if causal else None
+    out = _fwd_bwd(dev, q, k, v, dy, mask, 0, half)
+    _check(out, q, k, v, dy, mask, 0, BF16_RTOL if half else FP32_RTOL, "T=1024")
+
+
 def test_attn_backward_without_training_forward_recomputes_row_statistics(dev):
     rng = np.random.default_rng(41)
     B, H, T, hs = 2, 2, 96, 64
