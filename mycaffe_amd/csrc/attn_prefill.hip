@@ -146,6 +146,7 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 struct FlashArgs {
     const void* q; const void* k; const void* v; void* y;
     const float* mask;   // (B, Tk) key mask for KIND 2, (B, Tq, Tk) mask for KIND 3
+    int maskBatch;       // KIND 3: 1 = one (Tq, Tk) mask per sequence, 0 = one mask shared by all sequences
     int B, H, Tq, Tk;
     float c;             // softmax scale * log2(e)
     float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                             float sv = s[qt][v];
                             if (KIND == 1 && key > qrow) sv = a.maskedRaw;
                             if (KIND == 2 && Ms[32 * sub + kl] == 0.f) sv = a.maskedRaw;
-                            if (KIND == 3 && qrow < a.Tq && key < a.Tk && a.mask[((size_t)b * a.Tq + qrow) * a.Tk + key] == 0.f)
+                            if (KIND == 3 && qrow < a.Tq && key < a.Tk && a.mask[((size_t)b * a.maskBatch * a.Tq + qrow) * a.Tk + key] == 0.f)
                                 sv = a.maskedRaw;
                             if (key >= a.Tk) sv = -INFINITY;
                             s[qt][v] = sv;
@@ -732,7 +733,7 @@ static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
     if (kind == MASK_NONE) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 0, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     else if (kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 1, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
     else if (kind == MASK_KEY) hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 2, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
-    else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 3, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);
+    else hipLaunchKernelGGL((flash_fwd_kernel<T, HS, 3, QT, NW, OCC, PREFETCH>), grid, NW * 64, 0, s, f);   // MASK_BQK, MASK_QK
     return hipGetLastError();
 }
 
@@ -740,9 +741,9 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
 {
     *handled = false;
     if (a.hs != 64 && a.hs != 128) return hipSuccess;
-    if (a.kind != MASK_NONE && a.kind != MASK_CAUSAL && a.kind != MASK_KEY && a.kind != MASK_BQK) return hipSuccess;
     if ((((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.y) & 15) != 0) return hipSuccess;
     FlashArgs f;
+    f.maskBatch = a.kind == MASK_QK ? 0 : 1;   // a shared (Tq,Tk) mask is the per-sequence form with batch stride 0
     f.q = a.q; f.k = a.k; f.v = a.v; f.y = a.y;
     f.mask = a.mask; f.B = a.B; f.H = a.H; f.Tq = a.Tq; f.Tk = a.Tk;
     f.c = a.scale * 1.4426950408889634f;

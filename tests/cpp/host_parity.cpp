@@ -170,7 +170,7 @@ int main(int argc, char** argv)
             report("unknown memory handle -> ERROR_MEMORY_NOT_FOUND", code == MCH_ERROR_MEMORY_NOT_FOUND);
             code = 0;
             try {
-                cuda.Raw().RunFloatEx2(cuda.KernelHandle(), 970 /* a LayerNorm id, outside the path */, {}, {1});
+                cuda.Raw().RunFloatEx2(cuda.KernelHandle(), 480 /* CUDA_FN_LSTM_FWD, outside the path */, {}, {1});
             } catch (const CudaDnnError& e) {
                 code = e.code();
             }
