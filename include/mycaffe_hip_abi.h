@@ -29,6 +29,10 @@ typedef uint16_t MCH_TCHAR; /* UTF-16 code unit */
 
 /* ---- error codes (CudaDnnDLL/Cuda Files/util.h:128-228) ------------------- */
 enum {
+    /* Win32 codes the reference's blob loader returns as they are (blobloader.cu:30-42, 83-99) */
+    MCH_ERROR_WIN_FILE_NOT_FOUND = 2,
+    MCH_ERROR_WIN_INVALID_PARAMETER = 87,
+    MCH_ERROR_WIN_INSUFFICIENT_BUFFER = 122,
     MCH_ERROR_DLL_NOT_INIT = 89999,
     MCH_ERROR_PARAM = 90000,
     MCH_ERROR_PARAM_OUT_OF_RANGE = 90001,
@@ -49,6 +53,7 @@ enum {
     MCH_ERROR_ATTN_NOT_INITIALIZED = 90281,
     MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE = 90284,
     MCH_ERROR_ATTN_INVALID_BLOCK_SIZE = 90285,
+    MCH_ERROR_BLOBLOADER_NOT_INITIALIZED = 90321,
     MCH_ERROR_EXTENSION_NOT_INITIALIZED = 90401,
     /* llama2 extension (CudaExtension.llm32.llama2/Files/llm.h:15-19) */
     MCH_ERROR_LLM_RENDERED_PROMPT_TO_LONG = 10000,
@@ -118,6 +123,11 @@ enum {
     MCH_FN_FREE_ROPE = 981,
     MCH_FN_ROPE_FWD = 982,
     MCH_FN_ROPE_BWD = 983,
+    MCH_FN_CREATE_BLOBLOADER = 990,       /* DLL_InvokeFloatEx: file path -> handle */
+    MCH_FN_FREE_BLOBLOADER = 991,
+    MCH_FN_BLOBLOADER_LOAD = 992,
+    MCH_FN_BLOBLOADER_RESETOFFSET = 993,
+    MCH_FN_BLOBLOADER_ADDTOOFFSET = 994,
     MCH_QRY_DEVICE_NAME = 1000,
     MCH_QRY_EXTENSION_STRING = 1003,
 

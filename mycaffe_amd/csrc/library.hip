@@ -8,11 +8,16 @@
 // wait for the stream, so "returned means visible" holds for everything the host
 // can observe.
 #include <dlfcn.h>
+#include <fcntl.h>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
+#include <algorithm>
 #include <climits>
 
 #include "runtime.h"
@@ -151,6 +156,12 @@ void MemTable::free_all()
     m_free.clear();
 }
 
+BlobLoaderState::~BlobLoaderState()
+{
+    if (data) munmap((void*)data, fileSize);
+    if (fd >= 0) close(fd);
+}
+
 ExtensionState::~ExtensionState()
 {
     if (lib) dlclose(lib);
@@ -163,6 +174,7 @@ Kernel::~Kernel()
 {
     if (m_stream) (void)hipStreamSynchronize(m_stream);
     m_ext.clear();
+    m_blobLoader.clear();
     m_rope.clear();
     m_layernorm.clear();
     m_mem.free_all();
@@ -1324,6 +1336,69 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
+    case MCH_FN_FREE_BLOBLOADER:
+        NEED_F(1, 1);
+        return m_blobLoader.free((long)pf[0]);
+    case MCH_FN_BLOBLOADER_RESETOFFSET: {
+        // l{hBlobLoader, offsetInBytes} (device.h:4651-4662, blobloader.h:56-61)
+        NEED_L(2, 2);
+        BlobLoaderState* bl = m_blobLoader.get((long)pl[0]);
+        if (!bl) return MCH_ERROR_BLOBLOADER_NOT_INITIALIZED;
+        if (pl[1] < 0) return MCH_ERROR_WIN_INVALID_PARAMETER;
+        bl->offsetBytes = (size_t)pl[1];
+        bl->offsetItems = 0;
+        return 0;
+    }
+    case MCH_FN_BLOBLOADER_ADDTOOFFSET: {
+        // l{hBlobLoader, offsetInItems} (device.h:4665-4676, blobloader.h:63-67)
+        NEED_L(2, 2);
+        BlobLoaderState* bl = m_blobLoader.get((long)pl[0]);
+        if (!bl) return MCH_ERROR_BLOBLOADER_NOT_INITIALIZED;
+        if (pl[1] < 0) return MCH_ERROR_WIN_INVALID_PARAMETER;
+        bl->offsetItems += (size_t)pl[1];
+        return 0;
+    }
+    case MCH_FN_BLOBLOADER_LOAD: {
+        // l{hBlobLoader, count, hData, localItemOffset} (device.h:4635-4648, blobloader.cu:83-126): copy `count` fp32
+        // items starting at byte offsetBytes + 4 * (offsetItems + localItemOffset) of the file into the blob.  The
+        // reference does not look at the file size; reading past the end is refused here instead of faulting.
+        NEED_L(4, 4);
+        BlobLoaderState* bl = m_blobLoader.get((long)pl[0]);
+        if (!bl || !bl->data) return MCH_ERROR_BLOBLOADER_NOT_INITIALIZED;
+        if (pl[3] < 0) return MCH_ERROR_WIN_INVALID_PARAMETER;
+        if (pl[1] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem* D;
+        ERRCHK(mem((long)pl[2], &D));
+        const size_t count = (size_t)pl[1];
+        if (count > D->count) return MCH_ERROR_WIN_INSUFFICIENT_BUFFER;
+        const size_t start = bl->offsetBytes + (bl->offsetItems + (size_t)pl[3]) * sizeof(float);
+        if (start > bl->fileSize || count * sizeof(float) > bl->fileSize - start) {
+            last_detail = "the requested items lie past the end of the weight file";
+            return MCH_ERROR_MEMORY_RANGE_EXCEEDED;
+        }
+        const unsigned char* src = bl->data + start;
+        // through pinned staging in slices, so that one blob of any size needs a bounded host buffer
+        const size_t slice = (size_t)16 << 20;   // items per slice (64 MiB)
+        void* ws = nullptr;
+        if (D->half) ERRCHK(workspace(std::min(count, slice) * sizeof(float), &ws));
+        std::lock_guard<std::mutex> g(m_stageLock);
+        for (size_t done = 0; done < count; done += slice) {
+            const size_t n = std::min(slice, count - done);
+            void* st;
+            ERRCHK(staging(n * sizeof(float), &st));
+            memcpy(st, src + done * sizeof(float), n * sizeof(float));
+            if (!D->half) {
+                HIPCHK(hipMemcpyAsync((float*)D->ptr + done, st, n * sizeof(float), hipMemcpyHostToDevice, s));
+            } else {
+                HIPCHK(hipMemcpyAsync(ws, st, n * sizeof(float), hipMemcpyHostToDevice, s));
+                HIPCHK(k_convert(s, F32, ws, BF16, (bf16_t*)D->ptr + done, n));
+            }
+            HIPCHK(hipStreamSynchronize(s));   // the staging buffer is reused by the next slice
+        }
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+
     case MCH_FN_FREE_EXTENSION:
         NEED_F(1, 1);
         return m_ext.free((long)pf[0]);
@@ -1367,6 +1442,25 @@ long Kernel::create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MC
     st->lib = lib;
     st->fnInvoke = inv;
     st->fnInvokeEx = dlsym(lib, "DLL_InvokeFloatCustomExtensionEx");
+    return set_out((float)h, ppOut, plOut);
+}
+
+// CUDA_FN_CREATE_BLOBLOADER (CudaDnn.cs:6438-6450, device.h:4606-4618, blobloader.cu:24-52): map the file read-only
+long Kernel::create_blobloader(MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut)
+{
+    if (!path) return MCH_ERROR_PARAM_NULL;
+    if (!plOut || !ppOut || !*ppOut) return MCH_ERROR_PARAM_NULL;
+    const std::string p = utf16_to_utf8(path);
+    const int fd = open(p.c_str(), O_RDONLY);
+    if (fd < 0) { last_detail = "cannot open " + p; return MCH_ERROR_WIN_FILE_NOT_FOUND; }
+    struct stat sb;
+    if (fstat(fd, &sb) != 0 || sb.st_size <= 0) { close(fd); last_detail = "cannot size " + p; return MCH_ERROR_WIN_FILE_NOT_FOUND; }
+    void* m = mmap(nullptr, (size_t)sb.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    if (m == MAP_FAILED) { close(fd); last_detail = "cannot map " + p; return MCH_ERROR_WIN_FILE_NOT_FOUND; }
+    long h;
+    ERRCHK(m_blobLoader.create(&h));
+    BlobLoaderState* st = m_blobLoader.get(h);
+    st->fd = fd; st->data = (const unsigned char*)m; st->fileSize = (size_t)sb.st_size;
     return set_out((float)h, ppOut, plOut);
 }
 
@@ -1503,6 +1597,8 @@ static long invoke(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, lon
     if (!(k = kernel_at(kIdx))) { e = MCH_ERROR_PARAM_NULL; put_error(nullptr, e, szErr, errMax); return e; }
     if (ex && fn == MCH_FN_CREATE_EXTENSION) {
         e = k->create_extension(kIdx, szIn, ppOut, plOut);
+    } else if (ex && fn == MCH_FN_CREATE_BLOBLOADER) {
+        e = k->create_blobloader(szIn, ppOut, plOut);
     } else if (fn == MCH_FN_EXTENSION_RUN) {
         // f{hExt, fnIdx, args...} (device.h:4569-4588)
         if (lf < 2) e = MCH_ERROR_PARAM_OUT_OF_RANGE;

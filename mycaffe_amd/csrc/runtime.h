@@ -96,6 +96,15 @@ struct LayerNormState {
     int backwards = 0;        // backward calls since the last forward
     ~LayerNormState() { if (stdev) (void)hipFree(stdev); }
 };
+// read-only mapping of a weight file (CudaDnnDLL/Cuda Files/blobloader.h:25-70)
+struct BlobLoaderState {
+    int fd = -1;
+    const unsigned char* data = nullptr;   // start of the mapping
+    size_t fileSize = 0;
+    size_t offsetBytes = 0;                // set by RESETOFFSET
+    size_t offsetItems = 0;                // advanced by ADDTOOFFSET, cleared by RESETOFFSET
+    ~BlobLoaderState();
+};
 struct ExtensionState {
     void* lib = nullptr;
     void* fnInvoke = nullptr;
@@ -112,6 +121,7 @@ public:
     long run_extension(long hExt, long fn, float* pf, long lf, MCH_TCHAR* szIn, float** ppOut, MCH_LONG* plOut,
                        MCH_TCHAR* szErr, long errMax);
     long create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut);
+    long create_blobloader(MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut);
     long query_extension(MCH_LONG* pIn, long n, MCH_TCHAR* out, long outMax, MCH_TCHAR* err, long errMax);
     long alloc_host(long count, float** dst, const float* src, bool srcOnDevice);
     long free_host(float* p);
@@ -137,6 +147,7 @@ private:
     HandleTable<RopeState> m_rope;
     HandleTable<LayerNormState> m_layernorm;
     HandleTable<ExtensionState> m_ext;
+    HandleTable<BlobLoaderState> m_blobLoader;
     std::map<int, std::weak_ptr<void>> m_ropeSharedCos, m_ropeSharedSin;
     void* m_ws = nullptr; size_t m_wsBytes = 0;          // device scratch (split-K partials, conversions)
     int* m_tickets = nullptr; size_t m_ticketCount = 0;  // split-K merge tickets; zero whenever no kernel is running

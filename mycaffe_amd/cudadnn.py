@@ -86,6 +86,11 @@ class CUDAFN:
     CUDA_FREE_ROPE = 981
     CUDA_ROPE_FWD = 982
     CUDA_ROPE_BWD = 983
+    CUDA_CREATE_BLOBLOADER = 990
+    CUDA_FREE_BLOBLOADER = 991
+    CUDA_BLOBLOADER_LOAD = 992
+    CUDA_BLOBLOADER_RESETOFFSET = 993
+    CUDA_BLOBLOADER_ADDTOOFFSET = 994
     # additions of this library (no counterpart in the reference)
     ATTN_DECODE_FWD = 2001
     RMSNORM_FWD = 2002
@@ -133,7 +138,11 @@ class ERROR:
     ATTN_NOT_INITIALIZED = 90281
     ATTN_INCOMPATIBLE_BLOB_SIZE = 90284
     ATTN_INVALID_BLOCK_SIZE = 90285
+    BLOBLOADER_NOT_INITIALIZED = 90321
     EXTENSION_NOT_INITIALIZED = 90401
+    FILE_NOT_FOUND = 2              # Win32 codes the reference's blob loader returns unchanged
+    INVALID_PARAMETER = 87
+    INSUFFICIENT_BUFFER = 122
 
 
 _c_float_p = ctypes.POINTER(ctypes.c_float)
@@ -601,6 +610,27 @@ class CudaDnn:
     def RopeBackward(self, hRope, n, hXdata, hYdiff, hXdiff):
         """CudaDnn.cs:6425-6431."""
         self._ex2(CUDAFN.CUDA_ROPE_BWD, None, [hRope, n, hXdata, hYdiff, hXdiff])
+
+    # ---- blob loader (weights from very large files) ------------------------------------------------
+    def CreateBlobLoader(self, strFile):
+        """CudaDnn.cs:6438-6450."""
+        return int(self.RunFloatEx(self.m_hKernel, CUDAFN.CUDA_CREATE_BLOBLOADER, None, strFile)[0])
+
+    def FreeBlobLoader(self, hBlobLoader):
+        """CudaDnn.cs:6456-6462."""
+        self.RunFloat(self.m_hKernel, CUDAFN.CUDA_FREE_BLOBLOADER, [hBlobLoader])
+
+    def LoadBlob(self, hBlobLoader, lCount, hDst, lLocalOffsetInItems):
+        """CudaDnn.cs:6472-6478."""
+        self._ex2(CUDAFN.CUDA_BLOBLOADER_LOAD, None, [hBlobLoader, lCount, hDst, lLocalOffsetInItems])
+
+    def BlobLoaderResetOffset(self, hBlobLoader, lOffsetInBytes):
+        """CudaDnn.cs:6485-6491."""
+        self._ex2(CUDAFN.CUDA_BLOBLOADER_RESETOFFSET, None, [hBlobLoader, lOffsetInBytes])
+
+    def BlobLoaderAddToOffset(self, hBlobLoader, lOffsetInItems):
+        """CudaDnn.cs:6498-6504."""
+        self._ex2(CUDAFN.CUDA_BLOBLOADER_ADDTOOFFSET, None, [hBlobLoader, lOffsetInItems])
 
     # ---- extensions ---------------------------------------------------------------------------------
     def CreateExtension(self, strExtensionDllPath):

@@ -158,3 +158,62 @@ def test_transformer_block_gpt2_shape_vs_checker(dev, activation):
     layer.Forward(bx, top)
     ref = R.transformer_block_gpt(x, {k: v.astype(np.float32) for k, v in p.items()}, H, activation, 1e-5, np.float64)
     assert_close(top.mutable_cpu_data, ref["y"], FP32_RTOL, "block %s" % activation)
+
+
+def test_blob_loader_reads_a_llama_checkpoint_like_the_model_builder(dev, tmp_path):
+    """The call sequence of LlamaModelBuilder.loadWeights_kpth0 (MyCaffe.model/LlamaModelBuilder.cs:239-420) against the
+    legacy llama2.c file layout: 28-byte header, then tok_emb, rms_att, wq, wk, wv, wo, rms_ffn, w1, w2, w3, rms_final."""
+    import struct
+    rng = np.random.default_rng(61)
+    dim, hid, L, H, V, S = 24, 40, 3, 4, 50, 16
+    order = [("tok_emb", (V, dim)), ("rms_att", (L, dim)), ("wq", (L, dim, dim)), ("wk", (L, dim, dim)), ("wv", (L, dim, dim)),
+             ("wo", (L, dim, dim)), ("rms_ffn", (L, dim)), ("w1", (L, hid, dim)), ("w2", (L, dim, hid)), ("w3", (L, hid, dim)),
+             ("rms_final", (dim,))]
+    w = {n: rng.standard_normal(s).astype(np.float32) for n, s in order}
+    path = str(tmp_path / "legacy.bin")
+    with open(path, "wb") as f:
+        f.write(struct.pack("<7i", dim, hid, L, H, H, V, S))
+        for n, _ in order:
+            w[n].tofile(f)
+    cuda = dev.cuda
+    hdr = 28
+    h = cuda.CreateBlobLoader(path)
+    cuda.BlobLoaderResetOffset(h, hdr)
+    hemb = dev.zeros(V * dim)
+    cuda.LoadBlob(h, V * dim, hemb, 0)
+    assert np.array_equal(dev.get(hemb, (V, dim)), w["tok_emb"])
+    start = hdr + V * dim * 4
+    per_layer = ["rms_att", "wq", "wk", "wv", "wo", "rms_ffn", "w1", "w2", "w3"]
+    for i in range(L):
+        cuda.BlobLoaderResetOffset(h, start)
+        for n in per_layer:
+            total = w[n].size
+            one = total // L
+            hd = dev.zeros(one, half=(n == "w1"))          # one blob kept in 16-bit storage
+            cuda.LoadBlob(h, one, hd, i * one)
+            cuda.BlobLoaderAddToOffset(h, total)
+            got = dev.get(hd).reshape(w[n][i].shape)
+            if n == "w1":
+                assert np.array_equal(got, bf16_round(w[n][i])), (i, n)
+            else:
+                assert np.array_equal(got, w[n][i]), (i, n)
+        hf = dev.zeros(dim)
+        cuda.LoadBlob(h, dim, hf, 0)                          # after the last AddToOffset the cursor is at rms_final
+        assert np.array_equal(dev.get(hf), w["rms_final"])
+    # error behaviour
+    with pytest.raises(CudaDnnError) as e:
+        cuda.LoadBlob(h, dim + 1, hf, 0)                      # blob smaller than the request
+    assert e.value.code == ERROR.INSUFFICIENT_BUFFER
+    with pytest.raises(CudaDnnError) as e:
+        cuda.LoadBlob(h, dim, hf, -1)
+    assert e.value.code == ERROR.INVALID_PARAMETER
+    with pytest.raises(CudaDnnError) as e:
+        cuda.LoadBlob(h, dim, hf, 1)                          # one item past the end of the file
+    assert e.value.code == ERROR.MEMORY_RANGE_EXCEEDED
+    cuda.FreeBlobLoader(h)
+    with pytest.raises(CudaDnnError) as e:
+        cuda.LoadBlob(h, dim, hf, 0)
+    assert e.value.code == ERROR.BLOBLOADER_NOT_INITIALIZED
+    with pytest.raises(CudaDnnError) as e:
+        cuda.CreateBlobLoader(str(tmp_path / "missing.bin"))
+    assert e.value.code == ERROR.FILE_NOT_FOUND
