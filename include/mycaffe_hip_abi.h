@@ -217,7 +217,7 @@ enum {
     MCH_LLM_DESTROY = 2,        /* f{hLlm} */
     MCH_LLM_LOAD = 3,           /* Ex: f{hLlm}, "model.bin;tokenizer.bin" */
     MCH_LLM_QUERYSTATUS = 4,    /* f{hLlm} -> f{pct, status} */
-    MCH_LLM_GENERATE = 5,       /* Ex: f{hLlm}, prompt text (needs a tokenizer file at LOAD; greedy only) */
+    MCH_LLM_GENERATE = 5,       /* Ex: f{hLlm}, prompt text (needs a tokenizer file at LOAD) */
     MCH_LLM_QUERYRESPONSE = 6,  /* Ex: f{hLlm} -> text in szOutput, *ppOutput = end flag */
     MCH_LLM_ABORT = 7,          /* f{hLlm} */
     /* No counterpart in the reference: token-id front door used where no
@@ -229,7 +229,9 @@ enum {
      *                 step of the timed span; option 3 = replay one captured
      *                 HIP graph per step (1, default) or launch eagerly (0);
      *                 option 4 = weight rows per wavefront of the mat-vec
-     *                 kernels (1 or 2; 0 = library's choice)
+     *                 kernels (1 or 2; 0 = library's choice); option 5 = GENERATE_IDS /
+     *                 GENERATE_BATCH draw from the handle's sampler (temperature, top-p,
+     *                 seed of CREATE) instead of the argmax (0, default)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it}
@@ -238,13 +240,16 @@ enum {
      *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,
      *                 w2, classifier, embed+argmax
      *   TOKENIZE      Ex: f{hLlm, bos(0|1), eos(0|1)} + text -> f{token ids};
-     *                 f{hLlm, -1, prevToken, token} -> the token's piece in szOutput */
+     *                 f{hLlm, -1, prevToken, token} -> the token's piece in szOutput
+     *   SAMPLE        f{hLlm, logits...} -> f{id}: one call of the handle's sampler
+     *                 (llama2_sampler.cpp:126-151); advances its random state unless greedy */
     MCH_LLM_GENERATE_IDS = 100,
     MCH_LLM_SET_OPTION = 101,
     MCH_LLM_GENERATE_BATCH = 102,
     MCH_LLM_QUERY_TIMING = 103,
     MCH_LLM_PROFILE_STEP = 104,
-    MCH_LLM_TOKENIZE = 105
+    MCH_LLM_TOKENIZE = 105,
+    MCH_LLM_SAMPLE = 106
 };
 
 MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);

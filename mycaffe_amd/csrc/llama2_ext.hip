@@ -295,11 +295,12 @@ __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ 
 // the id, embed the token of the next position (forced prompt id while pos + 1 < n_prompt,
 // generate loop llm.cpp:208-228) and, in the workgroup that takes the last ticket, advance the
 // position.  Every workgroup reads the position before it takes its ticket.
+// With `given` the id of every sequence comes from the host sampler instead of the scan.
 template <typename T>
 __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __restrict__ logits, int V, GenState* st, int* ticket,
                                                                const int* __restrict__ prompt, int promptStride, int* next,
                                                                int* out_ids, const T* __restrict__ emb, float* __restrict__ x,
-                                                               int dim, int* cur)
+                                                               int dim, int* cur, const int* __restrict__ given)
 {
     __shared__ float sv[16];
     __shared__ int si[16];
@@ -309,6 +310,7 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
     const float* lg = logits + (size_t)b * V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
+    if (given) V = 0;   // the host sampler chose the id: nothing to scan
     auto take = [&](float v, int i) {
         if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
     };
@@ -343,6 +345,7 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
         for (int i = 1; i < 16; i++)
             if (sv[i] > bv || (sv[i] == bv && si[i] < bi)) { bv = sv[i]; bi = si[i]; }
         if (bi == 0x7fffffff) bi = 0;  // all NaN: index 0, as a scan that never finds a larger value would give
+        if (given) bi = given[b];
         next[b] = bi;
         out_ids[(size_t)b * promptStride + pos] = bi;
         const int np = pos + 1;
@@ -389,6 +392,86 @@ struct StepProfile {
 
 template <typename T> struct LayerW { T *wqkv, *wo, *w13, *w2; float *rms_att, *rms_ffn; };
 
+// The sampler of the reference engine (CudaExtension.llm32.llama2/Files/llama2_sampler.cpp), on the host as there:
+// temperature, softmax (llama2_cpu.cpp:204-222), one 24-bit coin from xorshift64* per call, then the inverse CDF over
+// all tokens or over the top-p nucleus.  Sums run sequentially in fp32, in the reference's order.
+struct HostSampler {
+    float temperature = 1.0f, topp = 0.9f;
+    unsigned long long state = 0;
+    std::vector<std::pair<float, int>> probindex;
+
+    void build(float temp, float p, unsigned long long seed) { temperature = temp; topp = p; state = seed; }   // :102-109
+    bool greedy() const { return temperature == 0.0f; }
+    unsigned int random_u32()                                     // :115-121
+    {
+        state ^= state >> 12;
+        state ^= state << 25;
+        state ^= state >> 27;
+        return (unsigned int)((state * 0x2545F4914F6CDD1Dull) >> 32);
+    }
+    float random_f32() { return (random_u32() >> 8) / 16777216.0f; }   // :122-124
+    static int argmax(const float* p, int n)                     // :25-36
+    {
+        int best = 0;
+        for (int i = 1; i < n; i++)
+            if (p[i] > p[best]) best = i;
+        return best;
+    }
+    static int sample_mult(const float* p, int n, float coin)    // :38-49
+    {
+        float cdf = 0.0f;
+        for (int i = 0; i < n; i++) {
+            cdf += p[i];
+            if (coin < cdf) return i;
+        }
+        return n - 1;
+    }
+    int sample_topp(const float* p, int n, float coin)           // :59-100
+    {
+        probindex.clear();
+        const float cutoff = (1.0f - topp) / (n - 1);
+        for (int i = 0; i < n; i++)
+            if (p[i] >= cutoff) probindex.push_back({p[i], i});
+        // descending by probability; the reference's qsort leaves the order of equal probabilities to the C library,
+        // here the lower index comes first
+        std::sort(probindex.begin(), probindex.end(), [](const std::pair<float, int>& a, const std::pair<float, int>& b) {
+            return a.first > b.first || (a.first == b.first && a.second < b.second);
+        });
+        const int n0 = (int)probindex.size();
+        float cum = 0.0f;
+        int last = n0 - 1;
+        for (int i = 0; i < n0; i++) {
+            cum += probindex[i].first;
+            if (cum > topp) { last = i; break; }
+        }
+        const float r = coin * cum;
+        float cdf = 0.0f;
+        for (int i = 0; i <= last; i++) {
+            cdf += probindex[i].first;
+            if (r < cdf) return probindex[i].second;
+        }
+        return probindex[last].second;
+    }
+    // overwrites the logits with the probabilities unless greedy (:126-151)
+    int sample(float* logits, int n)
+    {
+        if (greedy()) return argmax(logits, n);
+        for (int q = 0; q < n; q++) logits[q] /= temperature;
+        float mx = logits[0];
+        for (int i = 1; i < n; i++)
+            if (logits[i] > mx) mx = logits[i];
+        float sum = 0.0f;
+        for (int i = 0; i < n; i++) {
+            logits[i] = expf(logits[i] - mx);
+            sum += logits[i];
+        }
+        for (int i = 0; i < n; i++) logits[i] /= sum;
+        const float coin = random_f32();
+        if (topp <= 0 || topp >= 1) return sample_mult(logits, n, coin);
+        return sample_topp(logits, n, coin);
+    }
+};
+
 class Engine {
 public:
     Config cfg{};
@@ -406,13 +489,14 @@ public:
     long load(const char* path);
     long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
                   std::vector<float>* logits, std::atomic<bool>* cancel, int chunk = 0,
-                  const std::function<bool(const int*, int, int)>& onChunk = nullptr);
+                  const std::function<bool(const int*, int, int)>& onChunk = nullptr, HostSampler* sampler = nullptr);
     void release();
     long profile_step(int pos, int reps, int B, std::vector<float>* out);
 
 private:
     template <typename T> long upload(const float* blob);
-    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr);
+    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr, bool deviceArgmax = true);
+    template <typename T> long advance_given(hipStream_t s, int B);
     long ensure_state(int B, int nSteps);
     hipError_t embed_first(hipStream_t s, int B);
 
@@ -439,12 +523,17 @@ private:
     int *dcount = nullptr, *dticket = nullptr;   // attention merge tickets (B * heads) and the step ticket; zero between launches
     hipGraphExec_t graphExec = nullptr;
     int graphB = 0;
+    bool graphArgmax = true;                     // whether the captured step ends with the device argmax
+    int* dgiven = nullptr;                       // ids chosen by the host sampler (one per sequence)
+    float* hLogits = nullptr; int* hGiven = nullptr; size_t hLogitsCount = 0;   // pinned staging of the sampled path
 };
 
 void Engine::release()
 {
     if (stream) (void)hipStreamSynchronize(stream);
     if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
+    if (hLogits) { (void)hipHostFree(hLogits); hLogits = nullptr; hLogitsCount = 0; }
+    if (hGiven) { (void)hipHostFree(hGiven); hGiven = nullptr; }
     for (void* p : stateAllocs) (void)hipFree(p);
     stateAllocs.clear();
     for (void* p : allocs) (void)hipFree(p);
@@ -582,6 +671,8 @@ long Engine::ensure_state(int B, int nSteps)
     if (B == stateB && nSteps <= stateSteps) return 0;
     HIPCHK(hipStreamSynchronize(stream));
     if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
+    if (hLogits) { (void)hipHostFree(hLogits); hLogits = nullptr; hLogitsCount = 0; }
+    if (hGiven) { (void)hipHostFree(hGiven); hGiven = nullptr; }
     for (void* p : stateAllocs) (void)hipFree(p);
     stateAllocs.clear();
     stateB = 0;
@@ -607,6 +698,7 @@ long Engine::ensure_state(int B, int nSteps)
     dprompt = (int*)sa((size_t)B * cfg.seq_len * 4);
     dnext = (int*)sa(B * 4);
     dcur = (int*)sa(B * 4);
+    dgiven = (int*)sa(B * 4);
     dout = (int*)sa((size_t)B * cfg.seq_len * 4);
     dcount = (int*)sa(((size_t)B * cfg.n_heads + 1) * 4);
     if (!x || !xb || !qkv || !qc || !hb || !logits || !kc || !vc || !ws || !dstate || !dprompt || !dnext || !dcur || !dout || !dcount)
@@ -661,7 +753,7 @@ hipError_t Engine::embed_first(hipStream_t s, int B)
 }
 
 // enqueue one decode step for B sequences at the device-side position
-template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof)
+template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof, bool deviceArgmax)
 {
     const int dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
     const int ldq = dim + 2 * kvd;
@@ -703,13 +795,24 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
                            dstate, V, nSteps);
         HIPCHK(hipGetLastError());
     }
-    SPAN_BEGIN(SC_SAMPLE);
-    hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
-                       (const T*)emb, x, dim, dcur);
-    HIPCHK(hipGetLastError());
-    SPAN_END();
+    if (deviceArgmax) {
+        SPAN_BEGIN(SC_SAMPLE);
+        hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
+                           (const T*)emb, x, dim, dcur, (const int*)nullptr);
+        HIPCHK(hipGetLastError());
+        SPAN_END();
+    }
 #undef SPAN_BEGIN
 #undef SPAN_END
+    return 0;
+}
+
+// tail of a step whose ids were chosen on the host (dgiven): record, embed the next token, advance the position
+template <typename T> long Engine::advance_given(hipStream_t s, int B)
+{
+    hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, cfg.vocab_size, dstate, dticket, dprompt, cfg.seq_len, dnext,
+                       dout, (const T*)emb, x, cfg.dim, dcur, (const int*)dgiven);
+    HIPCHK(hipGetLastError());
     return 0;
 }
 
@@ -784,7 +887,7 @@ long Engine::profile_step(int pos, int reps, int B, std::vector<float>* out)
 
 long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
                       std::vector<float>* outLogits, std::atomic<bool>* cancel, int chunk,
-                      const std::function<bool(const int*, int, int)>& onChunk)
+                      const std::function<bool(const int*, int, int)>& onChunk, HostSampler* sampler)
 {
     if (!loaded) return MCH_ERROR_LLM_GENERATE;
     if (B < 1 || B > 64 || nSteps < 1 || nSteps > cfg.seq_len || nPrompt < 1 || nPrompt > cfg.seq_len) return MCH_ERROR_PARAM_OUT_OF_RANGE;
@@ -803,15 +906,29 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     if (wantLogits) {
         HIPCHK(hipMalloc((void**)&allLogits, (size_t)B * nSteps * cfg.vocab_size * 4));
     }
+    // With a sampler whose temperature is not 0 the id of every step is chosen on the host, as in the reference: the
+    // step's kernels stop at the logits, which are copied out, sampled, and the chosen id goes back for the step's tail.
+    const bool hostSample = sampler && !sampler->greedy();
+    const size_t V = (size_t)cfg.vocab_size;
+    if (hostSample) {
+        if (hLogitsCount < (size_t)B * V) {
+            if (hLogits) (void)hipHostFree(hLogits);
+            hLogits = nullptr;
+            HIPCHK(hipHostMalloc((void**)&hLogits, (size_t)B * V * sizeof(float), hipHostMallocDefault));
+            hLogitsCount = (size_t)B * V;
+        }
+        if (!hGiven) HIPCHK(hipHostMalloc((void**)&hGiven, 64 * sizeof(int), hipHostMallocDefault));
+    }
     auto enqueue = [&]() -> long {
-        return bf16_weights ? step<bf16_t>(s, B, nSteps, allLogits) : step<float>(s, B, nSteps, allLogits);
+        return bf16_weights ? step<bf16_t>(s, B, nSteps, allLogits, nullptr, !hostSample)
+                            : step<float>(s, B, nSteps, allLogits, nullptr, !hostSample);
     };
     hipEvent_t evA = nullptr, evB = nullptr;
     (void)hipEventCreate(&evA);
     (void)hipEventCreate(&evB);
     const int t0 = timedFrom < 0 ? nPrompt : timedFrom;
     bool graph = use_graph && !wantLogits;
-    if (graph && (!graphExec || graphB != B)) {
+    if (graph && (!graphExec || graphB != B || graphArgmax != !hostSample)) {
         // one decode step, captured once; position / tokens are device-side so the graph is replayed as is
         if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
         hipGraph_t g = nullptr;
@@ -824,6 +941,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         }
         if (e || he != hipSuccess || !graphExec) { graphExec = nullptr; graph = false; e = 0; }
         graphB = B;
+        graphArgmax = !hostSample;
     }
     HIPCHK(embed_first(s, B));
     int done = 0;
@@ -833,6 +951,16 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
             hipError_t he = hipGraphLaunch(graphExec, s);
             if (he != hipSuccess) e = (long)he;
         } else e = enqueue();
+        if (hostSample && !e) {
+            hipError_t hc = hipMemcpyAsync(hLogits, logits, (size_t)B * V * sizeof(float), hipMemcpyDeviceToHost, s);
+            if (hc == hipSuccess) hc = hipStreamSynchronize(s);
+            if (hc != hipSuccess) { e = (long)hc; break; }
+            for (int b = 0; b < B; b++) hGiven[b] = sampler->sample(hLogits + (size_t)b * V, (int)V);
+            hc = hipMemcpyAsync(dgiven, hGiven, (size_t)B * sizeof(int), hipMemcpyHostToDevice, s);
+            if (hc != hipSuccess) { e = (long)hc; break; }
+            e = bf16_weights ? advance_given<bf16_t>(s, B) : advance_given<float>(s, B);
+            if (e) break;
+        }
         done++;
         if (cancel && (i & 15) == 15 && cancel->load()) break;
         if (onChunk && chunk > 0 && (done % chunk == 0 || done == nSteps)) {
@@ -879,6 +1007,8 @@ struct Llm {
     long seed = 0;
     Engine engine;
     BpeTokenizer tokenizer;
+    HostSampler sampler;         // built at LOAD from the CREATE arguments, state kept across generations (llm.cpp:140)
+    bool sampleIds = false;      // GENERATE_IDS / GENERATE_BATCH draw from the sampler instead of the device argmax
     std::atomic<bool> cancel{false};
     std::atomic<bool> busy{false};
     std::atomic<bool> loaded{false};
@@ -1060,6 +1190,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 2) m->engine.timedFrom = (int)pIn[2];
         else if (opt == 3) m->engine.use_graph = pIn[2] != 0.f;
         else if (opt == 4) m->engine.set_mv_rows(pIn[2] == 1.f ? 1 : (pIn[2] == 2.f ? 2 : 0));
+        else if (opt == 5) m->sampleIds = pIn[2] != 0.f;
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }
@@ -1078,6 +1209,16 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         long e = m->engine.profile_step((int)pIn[1], (int)pIn[2], lIn > 3 ? (int)pIn[3] : 1, &out);
         if (e) return (MCH_LONG)e;
         return (MCH_LONG)give(out, ppOut, plOut);
+    }
+    case MCH_LLM_SAMPLE: {
+        // f{hLlm, logits...} -> f{id}: one call of the handle's sampler (advances its random state unless greedy)
+        if (lIn < 2) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        Llm* m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
+        std::lock_guard<std::mutex> run(m->runLock);
+        std::vector<float> lg(pIn + 1, pIn + lIn);
+        return (MCH_LONG)give({(float)m->sampler.sample(lg.data(), (int)lg.size())}, ppOut, plOut);
     }
     case MCH_LLM_GENERATE_IDS:
     case MCH_LLM_GENERATE_BATCH: {
@@ -1100,7 +1241,8 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         std::vector<float> logits;
         m->cancel.store(false);
         m->busy.store(true);
-        long e = m->engine.generate(prompts.data(), B, nPrompt, nSteps, wantLogits, &ids, &logits, &m->cancel);
+        long e = m->engine.generate(prompts.data(), B, nPrompt, nSteps, wantLogits, &ids, &logits, &m->cancel, 0, nullptr,
+                                    m->sampleIds ? &m->sampler : nullptr);
         m->busy.store(false);
         if (e) {
             if (e == MCH_ERROR_LLM_GENERATE) put_text(szErr, errMax, "The model is not loaded.");
@@ -1143,6 +1285,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         long e = m->engine.load(model.c_str());
         if (!e && !tok.empty() && !m->tokenizer.load(tok.c_str(), m->engine.cfg.vocab_size)) e = MCH_ERROR_LLM_LOAD_MODEL;
         m->busy.store(false);
+        if (!e) m->sampler.build(m->temperature, m->topp, (unsigned long long)m->seed);
         m->loaded.store(e == 0);
         return (MCH_LONG)e;
     }
@@ -1158,10 +1301,6 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         if (!m->tokenizer.loaded()) {
             put_text(szErr, errMax, "No tokenizer file was given at LOAD; use the token-id entry.");
             return MCH_ERROR_LLM_MISSING_TOKENIZER_FILE;
-        }
-        if (m->temperature != 0.f) {
-            put_text(szErr, errMax, "Only greedy decoding (temperature 0) is implemented.");
-            return MCH_ERROR_NOT_IMPLEMENTED;
         }
         const std::string prompt = narrow(szIn);
         if (prompt.size() > 4096) return MCH_ERROR_LLM_RENDERED_PROMPT_TO_LONG;
@@ -1191,7 +1330,10 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
                 }
                 return !m->cancel.load();
             };
-            e = m->engine.generate(toks.data(), 1, nP, steps, false, &ids, nullptr, &m->cancel, 32, onChunk);
+            // greedy: ids are looked at every 32 steps; sampled: after every step, so that the generation stops on the very
+            // step that draws the end-of-text id and the random stream stays where the reference's would be
+            e = m->engine.generate(toks.data(), 1, nP, steps, false, &ids, nullptr, &m->cancel, m->sampler.greedy() ? 32 : 1, onChunk,
+                                   &m->sampler);
             if (m->cancel.load()) {
                 std::lock_guard<std::mutex> g(m->responseLock);
                 m->response.clear();

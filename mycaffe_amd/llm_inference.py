@@ -25,6 +25,7 @@ class CUDAFN_EXTENSION_LLM:
     QUERY_TIMING = 103
     PROFILE_STEP = 104
     TOKENIZE = 105
+    SAMPLE = 106
 
 
 STEP_CLASSES = ("matvec_qkv", "rope_store", "attn_decode", "matvec_wo", "matvec_w13", "matvec_w2", "matvec_cls", "embed_argmax")
@@ -87,6 +88,11 @@ class LlmInference:
         """The text piece a token contributes after ``nPrevToken`` (addition of this library)."""
         return self.m_cuda.QueryExtensionStrings(self.m_hExtension, CUDAFN_EXTENSION_LLM.TOKENIZE,
                                                  [int(self.m_rgLlm[0]), -1, int(nPrevToken), int(nToken)])[0]
+
+    def Sample(self, logits):
+        """One call of the handle's sampler on the given logits (advances its random state unless temperature is 0)."""
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.SAMPLE, self.m_rgLlm + [float(v) for v in logits])
+        return int(rg[0])
 
     def GenerateIds(self, prompt_ids, nSteps, want_logits=False, vocab_size=None):
         """Greedy decode from token ids; returns the id sampled after every position

@@ -58,6 +58,20 @@ def lib():
         L.orc_llama_forward.restype = fp
         L.orc_llama_generate_greedy.argtypes = [ctypes.c_void_p, ip, ctypes.c_int, ctypes.c_int, ip, fp]
         L.orc_llama_generate_greedy.restype = ctypes.c_int
+        u64p = ctypes.POINTER(ctypes.c_ulonglong)
+        L.orc_random_u32.argtypes = [u64p]
+        L.orc_random_u32.restype = ctypes.c_uint
+        L.orc_random_f32.argtypes = [u64p]
+        L.orc_random_f32.restype = ctypes.c_float
+        L.orc_sample_mult.argtypes = [fp, ctypes.c_int, ctypes.c_float]
+        L.orc_sample_mult.restype = ctypes.c_int
+        L.orc_sample_topp.argtypes = [fp, ctypes.c_int, ctypes.c_float, ctypes.c_float]
+        L.orc_sample_topp.restype = ctypes.c_int
+        L.orc_sample.argtypes = [fp, ctypes.c_int, ctypes.c_float, ctypes.c_float, u64p]
+        L.orc_sample.restype = ctypes.c_int
+        L.orc_llama_generate_sampled.argtypes = [ctypes.c_void_p, ip, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float,
+                                                 u64p, ip]
+        L.orc_llama_generate_sampled.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -110,6 +124,34 @@ def rope_pairs(q, k, fcos, fsin, pos):
 def argmax(p):
     p = np.ascontiguousarray(p, np.float32)
     return int(lib().orc_argmax(_fp(p), p.size))
+
+
+class Sampler:
+    """llama2_sampler.cpp: build_sampler / sample with the xorshift64* state kept across calls."""
+
+    def __init__(self, temperature, topp, seed):
+        self.temperature, self.topp = float(temperature), float(topp)
+        self.state = ctypes.c_ulonglong(int(seed) & 0xFFFFFFFFFFFFFFFF)
+
+    def random_u32(self):
+        return int(lib().orc_random_u32(ctypes.byref(self.state)))
+
+    def random_f32(self):
+        return float(lib().orc_random_f32(ctypes.byref(self.state)))
+
+    def sample(self, logits):
+        lg = np.array(logits, np.float32)   # copy: the routine overwrites its input
+        return int(lib().orc_sample(_fp(lg), lg.size, self.temperature, self.topp, ctypes.byref(self.state)))
+
+
+def sample_mult(p, coin):
+    p = np.ascontiguousarray(p, np.float32)
+    return int(lib().orc_sample_mult(_fp(p), p.size, float(coin)))
+
+
+def sample_topp(p, topp, coin):
+    p = np.ascontiguousarray(p, np.float32)
+    return int(lib().orc_sample_topp(_fp(p), p.size, float(topp), float(coin)))
 
 
 # ----------------------------------------------------------------------------
@@ -186,6 +228,15 @@ class Llama:
         lib().orc_llama_generate_greedy(self._h, prompt.ctypes.data_as(ip), prompt.size, n_steps,
                                         out.ctypes.data_as(ip), _fp(lg) if want_logits else None)
         return (out, lg) if want_logits else out
+
+    def generate_sampled(self, prompt, n_steps, sampler):
+        """The generate loop with ``sampler`` (its state advances at every position, prompt included)."""
+        prompt = np.ascontiguousarray(prompt, np.int32)
+        out = np.empty(n_steps, np.int32)
+        ip = ctypes.POINTER(ctypes.c_int)
+        lib().orc_llama_generate_sampled(self._h, prompt.ctypes.data_as(ip), prompt.size, n_steps, sampler.temperature,
+                                         sampler.topp, ctypes.byref(sampler.state), out.ctypes.data_as(ip))
+        return out
 
     def close(self):
         if self._h:

@@ -306,3 +306,93 @@ int orc_llama_generate_greedy(OrcLlama *m, const int *prompt, int n_prompt, int 
     }
     return n_steps;
 }
+
+/* ---------------------------------------------------------------------------
+ * Sampler (llama2_sampler.cpp): temperature, softmax, a 24-bit coin from xorshift64*, then either the inverse CDF over
+ * all tokens or nucleus (top-p) sampling.  All accumulations are sequential fp32, as there.
+ */
+unsigned int orc_random_u32(unsigned long long *state)   /* llama2_sampler.cpp:115-121 */
+{
+    *state ^= *state >> 12;
+    *state ^= *state << 25;
+    *state ^= *state >> 27;
+    return (unsigned int)((*state * 0x2545F4914F6CDD1Dull) >> 32);
+}
+
+float orc_random_f32(unsigned long long *state)          /* llama2_sampler.cpp:122-124: [0, 1) in steps of 2^-24 */
+{
+    return (orc_random_u32(state) >> 8) / 16777216.0f;
+}
+
+int orc_sample_mult(const float *p, int n, float coin)   /* llama2_sampler.cpp:38-49 */
+{
+    float cdf = 0.0f;
+    for (int i = 0; i < n; i++) {
+        cdf += p[i];
+        if (coin < cdf) return i;
+    }
+    return n - 1;
+}
+
+typedef struct { float prob; int index; } OrcProbIndex;
+
+/* descending by probability; equal probabilities keep the lower index first (the reference's qsort leaves their
+ * order to the C library) */
+static int orc_cmp_prob(const void *a, const void *b)
+{
+    const OrcProbIndex *x = (const OrcProbIndex *)a, *y = (const OrcProbIndex *)b;
+    if (x->prob > y->prob) return -1;
+    if (x->prob < y->prob) return 1;
+    return (x->index > y->index) - (x->index < y->index);
+}
+
+int orc_sample_topp(const float *p, int n, float topp, float coin)   /* llama2_sampler.cpp:59-100 */
+{
+    OrcProbIndex *pi = (OrcProbIndex *)malloc((size_t)n * sizeof(OrcProbIndex));
+    int n0 = 0;
+    const float cutoff = (1.0f - topp) / (n - 1);
+    for (int i = 0; i < n; i++)
+        if (p[i] >= cutoff) { pi[n0].index = i; pi[n0].prob = p[i]; n0++; }
+    qsort(pi, n0, sizeof(OrcProbIndex), orc_cmp_prob);
+    float cum = 0.0f;
+    int last = n0 - 1;
+    for (int i = 0; i < n0; i++) {
+        cum += pi[i].prob;
+        if (cum > topp) { last = i; break; }
+    }
+    const float r = coin * cum;
+    float cdf = 0.0f;
+    int res = pi[last].index;
+    for (int i = 0; i <= last; i++) {
+        cdf += pi[i].prob;
+        if (r < cdf) { res = pi[i].index; break; }
+    }
+    free(pi);
+    return res;
+}
+
+/* sample (llama2_sampler.cpp:126-151); logits are overwritten with the probabilities when temperature != 0 */
+int orc_sample(float *logits, int n, float temperature, float topp, unsigned long long *state)
+{
+    if (temperature == 0.0f) return orc_argmax(logits, n);
+    for (int q = 0; q < n; q++) logits[q] /= temperature;
+    orc_softmax(logits, n);
+    const float coin = orc_random_f32(state);
+    if (topp <= 0 || topp >= 1) return orc_sample_mult(logits, n, coin);
+    return orc_sample_topp(logits, n, topp, coin);
+}
+
+/* generate loop of llm.cpp:208-245 with the sampler: sample() runs at every position, prompt positions included (its
+ * result is discarded there but the random state advances). */
+int orc_llama_generate_sampled(OrcLlama *m, const int *prompt, int n_prompt, int n_steps, float temperature, float topp,
+                               unsigned long long *state, int *out_ids)
+{
+    int next = 0;
+    for (int pos = 0; pos < n_steps; pos++) {
+        int token = pos < n_prompt ? prompt[pos] : next;
+        float *lg = orc_llama_forward(m, token, pos);
+        next = orc_sample(lg, m->cfg.vocab_size, temperature, topp, state);
+        out_ids[pos] = next;
+    }
+    return n_steps;
+}

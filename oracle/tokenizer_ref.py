@@ -114,3 +114,22 @@ def generate_text(model, tok, prompt, steps):
         if token == 2 or nxt == 2:
             break
     return resp
+
+
+def generate_text_sampled(model, tok, prompt, steps, sampler):
+    """LLMData::Generate (llm.cpp:193-263) with the engine's sampler: ``model.forward(token, pos)`` gives the logits,
+    ``sampler.sample(logits)`` is called at every position (the prompt's included), and the loop ends on the step that
+    feeds or draws the end-of-text id, so the sampler's random state carries over to the next call as in the reference.
+    Returns the response bytes."""
+    toks = tok.encode(prompt, True, False)
+    n = len(toks)
+    resp = b""
+    nxt = 0
+    for pos in range(steps):
+        token = toks[pos] if pos < n else nxt
+        nxt = sampler.sample(model.forward(token, pos))
+        if pos + 1 >= n and nxt != 2:
+            resp += tok.decode(token, nxt)
+        if token == 2 or nxt == 2:
+            break
+    return resp

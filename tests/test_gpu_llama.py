@@ -216,3 +216,80 @@ def test_text_generation_errors(llm, tmp_path):
     with pytest.raises(CudaDnnError) as e:
         inf.Load(ckpt, short)
     assert e.value.code == 10001         # ERROR_LLM_LOAD_MODEL
+
+
+def test_sampler_entry_matches_checker_on_given_logits():
+    """SAMPLE (the engine's host sampler, llama2_sampler.cpp) against the C checker on the same logits and seed: the
+    same coin stream and the same ids, for plain multinomial and for top-p."""
+    rng = np.random.default_rng(71)
+    blob, _ = O.random_weights(TINY, seed=2, std=0.2)
+    for topp, temp, seed in ((0.9, 0.8, 1234), (0.0, 1.3, 99), (0.5, 0.3, 7), (0.9, 0.0, 5)):
+        cuda = CudaDnn(0)
+        inf = LlmInference(cuda)
+        inf.Initialize(fTemperature=temp, fTopp=topp, lSeed=seed)
+        import tempfile, os
+        with tempfile.TemporaryDirectory() as d:
+            ckpt = os.path.join(d, "m.bin")
+            O.write_checkpoint_v1(ckpt, TINY, blob, False)
+            inf.Load(ckpt)
+        ref = O.Sampler(temp, topp, seed)
+        for _ in range(200):
+            logits = (rng.standard_normal(TINY["vocab_size"]) * 3).astype(np.float32)
+            assert inf.Sample(logits) == ref.sample(logits)
+        inf.CleanUp()
+        cuda.Dispose()
+
+
+@pytest.mark.parametrize("topp", [0.9, 0.0])
+def test_sampled_generation_matches_checker(topp, tmp_path):
+    """Token-id generation with temperature 0.8: ids equal to the checker's sampled loop with the same seed, graph replay
+    and eager launches, and the random state carries over from one generation to the next."""
+    blob, _ = O.random_weights(TINY, seed=4, shared_classifier=False, std=0.25)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, TINY, blob, False)
+    prompt = [1, 17, 300, 42, 7]
+    for graph in (1, 0):
+        cuda = CudaDnn(0)
+        inf = LlmInference(cuda)
+        inf.Initialize(fTemperature=0.8, fTopp=topp, lSeed=2024)
+        inf.SetOption(3, graph)
+        inf.SetOption(5, 1)
+        inf.Load(ckpt)
+        ref_sampler = O.Sampler(0.8, topp, 2024)
+        for rnd in range(2):
+            ref = O.Llama(TINY, blob, False).generate_sampled(prompt, 48, ref_sampler)
+            ids = inf.GenerateIds(prompt, 48)
+            assert np.array_equal(ids, ref), (graph, rnd, ids, ref)
+        # greedy ids are a different sequence: the sampler really ran
+        assert not np.array_equal(ref, O.Llama(TINY, blob, False).generate_greedy(prompt, 48))
+        inf.CleanUp()
+        cuda.Dispose()
+
+
+def test_sampled_text_generation_matches_checker(tmp_path):
+    from oracle import tokenizer_ref as TK
+    cfg = dict(dim=64, hidden_dim=172, n_layers=2, n_heads=4, n_kv_heads=4, vocab_size=320, seq_len=96)
+    vocab, scores = _vocab(cfg["vocab_size"])
+    tok_path = str(tmp_path / "tok.bin")
+    TK.write_tokenizer(tok_path, vocab, scores)
+    tok = TK.Tokenizer(vocab, scores)
+    blob, _ = O.random_weights(cfg, seed=9, shared_classifier=False, std=0.3)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, cfg, blob, False)
+    cuda = CudaDnn(0)
+    inf = LlmInference(cuda)
+    inf.Initialize(fTemperature=0.9, fTopp=0.9, lSeed=31337)
+    inf.Load(ckpt, tok_path)
+    ref_sampler = O.Sampler(0.9, 0.9, 31337)
+    for text in ["hello world", "the cat, hello?", "hello world"]:       # the third call continues the random stream
+        ref = TK.generate_text_sampled(O.Llama(cfg, blob, False), tok, text, cfg["seq_len"], ref_sampler)
+        inf.Generate(text)
+        got, end, polls = "", False, 0
+        while not end and polls < 50:
+            part, end = inf.QueryResponse()
+            got += part
+            polls += 1
+        assert end
+        assert got.encode("utf-8") == ref.decode("utf-8", errors="replace").encode("utf-8"), (text, got, ref)
+    inf.CleanUp()
+    cuda.Dispose()

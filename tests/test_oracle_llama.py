@@ -143,3 +143,121 @@ def test_checkpoint_v1_header(tmp_path):
     assert struct.unpack("<7i", raw[8:36]) == tuple(TINY[k] for k in O.CONFIG_FIELDS)
     assert raw[36] == 0 and len(raw) == 256 + blob.size * 4
     assert np.array_equal(np.frombuffer(raw[256:], np.float32), blob)
+
+
+# ---- sampler (llama2_sampler.cpp) -------------------------------------------------------------------
+
+def _xorshift64star(state):
+    """xorshift64* on Python integers (unbounded, masked to 64 bits): an independent arithmetic for the same recurrence."""
+    M = (1 << 64) - 1
+    state ^= state >> 12
+    state ^= (state << 25) & M
+    state ^= state >> 27
+    return state, ((state * 0x2545F4914F6CDD1D) & M) >> 32
+
+
+def test_rng_recurrence_range_and_uniformity():
+    # worked by hand for state 1: no bit reaches the >> shifts, so the new state is 1 | 1 << 25
+    s = O.Sampler(1.0, 0.9, 1)
+    assert s.random_u32() == ((33554433 * 0x2545F4914F6CDD1D) & ((1 << 64) - 1)) >> 32
+    assert s.state.value == 33554433
+    for seed in (1, 2, 1234567, 0xDEADBEEFCAFEF00D):
+        s = O.Sampler(1.0, 0.9, seed)
+        st = seed
+        for _ in range(200):
+            st, u = _xorshift64star(st)
+            assert s.random_u32() == u and s.state.value == st
+    s = O.Sampler(1.0, 0.9, 0)            # the all-zero state is a fixed point: every coin is 0
+    assert s.random_u32() == 0 and s.random_f32() == 0.0
+    s = O.Sampler(1.0, 0.9, 42)
+    f = np.array([s.random_f32() for _ in range(100000)])
+    assert f.min() >= 0.0 and f.max() < 1.0
+    assert np.all(f * 16777216 == np.floor(f * 16777216))            # 24-bit coins
+    hist = np.bincount((f * 16).astype(int), minlength=16)
+    chi2 = ((hist - 6250.0) ** 2 / 6250.0).sum()
+    assert chi2 < 45                                                    # 15 degrees of freedom, p ~ 1e-4
+
+
+def test_sample_mult_is_the_inverse_cdf():
+    rng = np.random.default_rng(7)
+    for n in (2, 17, 1000):
+        p = rng.random(n).astype(np.float32)
+        p /= p.sum()
+        cdf = np.cumsum(p.astype(np.float64))
+        for coin in rng.random(300):
+            j = int(np.searchsorted(cdf, coin, side="right"))
+            if j < n and min(abs(cdf - coin)) > 1e-5:                   # away from the rounding of the boundaries
+                assert O.sample_mult(p, coin) == j
+        assert O.sample_mult(p, 0.0) == 0
+        assert O.sample_mult(p, 1.5) == n - 1                           # past the end: the last index
+    p = np.array([0, 0, 0.5, 0.5], np.float32)
+    assert O.sample_mult(p, 0.0) == 2                                   # strict '<': zero-probability entries are skipped
+
+
+def test_sample_topp_nucleus_and_frequencies():
+    rng = np.random.default_rng(8)
+    n, topp = 50, 0.8
+    p = rng.random(n).astype(np.float32) ** 4
+    p /= p.sum()
+    order = np.argsort(-p.astype(np.float64), kind="stable")
+    cum = np.cumsum(p[order].astype(np.float64))
+    k = int(np.searchsorted(cum, topp, side="right")) + 1               # smallest prefix whose mass exceeds topp
+    nucleus = set(order[:k].tolist())
+    coins = (np.arange(20000) + 0.5) / 20000                            # a regular grid of coins = exact quantiles
+    got = np.array([O.sample_topp(p, topp, c) for c in coins])
+    assert set(got.tolist()) == nucleus
+    freq = np.bincount(got, minlength=n) / len(coins)
+    want = np.zeros(n)
+    want[order[:k]] = p[order[:k]] / cum[k - 1]
+    assert np.abs(freq - want).max() < 2e-4                             # grid resolution 5e-5 per boundary
+    # a nucleus of one token: always the most likely one; probabilities below (1-topp)/(n-1) never appear
+    assert all(O.sample_topp(p, 1e-6, c) == order[0] for c in (0.0, 0.3, 0.999))
+    cut = (1 - topp) / (n - 1)
+    assert all(p[i] >= cut for i in set(got.tolist()))
+
+
+def test_sample_temperature_softmax_and_random_stream():
+    rng = np.random.default_rng(9)
+    logits = (rng.standard_normal(64) * 2).astype(np.float32)
+    assert O.Sampler(0.0, 0.9, 5).sample(logits) == int(logits.argmax())          # temperature 0: greedy, no coin drawn
+    s = O.Sampler(0.0, 0.9, 5)
+    s.sample(logits)
+    assert s.state.value == 5
+    assert all(O.Sampler(1e-3, 0.0, seed).sample(logits) == int(logits.argmax()) for seed in range(1, 20))
+    T = 0.7
+    s = O.Sampler(T, 0.0, 99)                                                        # topp <= 0: plain multinomial
+    draws = np.array([s.sample(logits) for _ in range(40000)])
+    z = logits.astype(np.float64) / T
+    want = np.exp(z - z.max())
+    want /= want.sum()
+    freq = np.bincount(draws, minlength=64) / len(draws)
+    assert np.abs(freq - want).max() < 4 * np.sqrt(want.max() / len(draws)) + 1e-3
+    # one coin per call, taken from the same stream as random_f32
+    a, b = O.Sampler(T, 0.0, 7), O.Sampler(T, 0.0, 7)
+    p = np.exp((logits / np.float32(T)) - (logits / np.float32(T)).max())
+    for _ in range(50):
+        coin = b.random_f32()
+        tok = a.sample(logits)
+        assert a.state.value == b.state.value
+        pf = (p / p.sum(dtype=np.float32)).astype(np.float32)
+        cdf = np.cumsum(pf.astype(np.float64))
+        if min(abs(cdf - coin)) > 1e-5:
+            assert tok == int(np.searchsorted(cdf, coin, side="right"))
+
+
+def test_generate_sampled_loop_draws_a_coin_at_every_position():
+    blob, _ = O.random_weights(TINY, seed=3, std=0.2)
+    prompt = np.array([5, 17, 3, 99], np.int32)
+    greedy = O.Llama(TINY, blob).generate_greedy(prompt, 24)
+    assert np.array_equal(O.Llama(TINY, blob).generate_sampled(prompt, 24, O.Sampler(0.0, 0.9, 11)), greedy)
+    for topp in (0.9, 0.0):
+        ids = O.Llama(TINY, blob).generate_sampled(prompt, 24, O.Sampler(0.8, topp, 11))
+        assert np.array_equal(ids, O.Llama(TINY, blob).generate_sampled(prompt, 24, O.Sampler(0.8, topp, 11)))
+        assert not np.array_equal(ids, greedy)
+        # step by step: forward, then one sample() per position, the prompt positions included
+        m, s = O.Llama(TINY, blob), O.Sampler(0.8, topp, 11)
+        nxt = 0
+        for pos in range(24):
+            tok = int(prompt[pos]) if pos < len(prompt) else nxt
+            nxt = s.sample(m.forward(tok, pos))
+            assert nxt == ids[pos]
