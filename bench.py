@@ -193,8 +193,8 @@ def bench_prefill_attention(cuda, reps, warm=5):
 
 
 def bench_attention_backward(cuda, reps, warm=5):
-    """Gradients of the fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_BWD (id 164): the statistics
-    kernel plus the dK/dV and dQ kernels of one call."""
+    """Gradients of the fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_BWD (id 164): the dQ kernel (which also
+    produces the per-row dY.Y sums) and the dK/dV kernel of one call."""
     from mycaffe_amd.cudadnn import CUDAFN
     B, H, T, hs = 8, 12, 1024, 64
     rng = np.random.default_rng(0)
@@ -214,7 +214,7 @@ def bench_attention_backward(cuda, reps, warm=5):
         useful = 5.0 * B * H * T * T * hs
         tf = useful / (ms / 1e3) / 1e12
         out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2),
-                     "roofline": {"kernel": "fused causal attention backward (3 kernels)", "bound": "mfma", "achieved": round(tf, 2),
+                     "roofline": {"kernel": "fused causal attention backward (dQ kernel + dK/dV kernel)", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
                                   "traffic": None}}
         for h in (q, k, v, dy, y, dq, dk, dv):

@@ -296,6 +296,48 @@ public:
         ex2(MCH_FN_EMBED_FWD, {}, {nCount, hBottom, hWeight, nM, nN, nK, hTop});
     }
     void silu_fwd(long long nCount, long hBottom, long hTop) { ex2(MCH_FN_SILU_FWD, {}, {nCount, hBottom, hTop}); }            // :10152
+    void silu_bwd(long long nCount, long hTopDiff, long hTopData, long hBottomDiff, long hBottomData)                          // :10174
+    {
+        ex2(MCH_FN_SILU_BWD, {}, {nCount, hTopDiff, hTopData, hBottomDiff, hBottomData});
+    }
+    void gelu_fwd(long long nCount, long hBottom, long hTop, bool bEnableBertVersion)                                           // :10098
+    {
+        ex2(MCH_FN_GELU_FWD, {}, {nCount, hBottom, hTop, bEnableBertVersion ? 1 : 0});
+    }
+    void gelu_bwd(long long nCount, long hTopDiff, long hTopData, long hBottomDiff, long hBottomData, bool bEnableBertVersion)  // :10132
+    {
+        ex2(MCH_FN_GELU_BWD, {}, {nCount, hTopDiff, hTopData, hBottomDiff, hBottomData, bEnableBertVersion ? 1 : 0});
+    }
+    void relu_fwd(long long nCount, long hBottom, long hTop, float fNegativeSlope = 0.f)                                        // :10417
+    {
+        ex2(MCH_FN_RELU_FWD, {fNegativeSlope}, {nCount, hBottom, hTop, 0});
+    }
+    void relu_bwd(long long nCount, long hTopDiff, long hTopData, long hBottomDiff, float fNegativeSlope = 0.f)                 // :10438
+    {
+        ex2(MCH_FN_RELU_BWD, {fNegativeSlope}, {nCount, hTopDiff, hTopData, hBottomDiff, 0});
+    }
+
+    // ---- LayerNorm handle (CudaDnn.cs:6307-6360) ---------------------------------------------------------------------
+    long CreateLayerNorm(int nGpuID, long long nCount, int nOuterNum, int nChannels, int nInnerNum, float fEps = 1e-10f)
+    {
+        return (long)ex2(MCH_FN_CREATE_LAYERNORM, {fEps}, {nGpuID, nCount, nOuterNum, nChannels, nInnerNum}).at(0);
+    }
+    void FreeLayerNorm(long h) { m_cuda.RunFloat(m_hKernel, MCH_FN_FREE_LAYERNORM, {(float)h}); }
+    void LayerNormForward(long hLayerNorm, long hXdata, long hYdata) { ex2(MCH_FN_LAYERNORM_FWD, {}, {hLayerNorm, hXdata, hYdata}); }
+    void LayerNormBackward(long hLayerNorm, long hYdata, long hYdiff, long hXdiff)
+    {
+        ex2(MCH_FN_LAYERNORM_BWD, {}, {hLayerNorm, hYdata, hYdiff, hXdiff});
+    }
+
+    // ---- blob loader (CudaDnn.cs:6438-6504) ---------------------------------------------------------------------------
+    long CreateBlobLoader(const std::string& strFile) { return (long)m_cuda.RunFloatEx(m_hKernel, MCH_FN_CREATE_BLOBLOADER, {}, strFile).at(0); }
+    void FreeBlobLoader(long h) { m_cuda.RunFloat(m_hKernel, MCH_FN_FREE_BLOBLOADER, {(float)h}); }
+    void LoadBlob(long hBlobLoader, long long lCount, long hDst, long long lLocalOffsetInItems)
+    {
+        ex2(MCH_FN_BLOBLOADER_LOAD, {}, {hBlobLoader, lCount, hDst, lLocalOffsetInItems});
+    }
+    void BlobLoaderResetOffset(long hBlobLoader, long long lOffsetInBytes) { ex2(MCH_FN_BLOBLOADER_RESETOFFSET, {}, {hBlobLoader, lOffsetInBytes}); }
+    void BlobLoaderAddToOffset(long hBlobLoader, long long lOffsetInItems) { ex2(MCH_FN_BLOBLOADER_ADDTOOFFSET, {}, {hBlobLoader, lOffsetInItems}); }
 
     // ---- cuDNN-shaped handles, softmax (CudaDnn.cs:3509-3527, 3819-3900, 4919)
     long CreateCuDNN(long hStream = 0) { return (long)m_cuda.RunFloat(m_hKernel, MCH_FN_CREATE_CUDNN, {(float)hStream}).at(0); }
@@ -324,6 +366,11 @@ public:
         ex2(MCH_FN_ATTN_FWD, {}, {hCuDnn, hAttn, nBlockSize, hQ, hK, hV, hMask, hY, nBatchMask});
     }
     // additions of this library (no counterpart in the reference)
+    void AttnScaledDotProductBackward(long hCuDnn, long hAttn, long hQ, long hdQ, long hK, long hdK, long hV, long hdV, long hMask, long hY,
+                                      long hdY)                                                                                // :5695
+    {
+        ex2(MCH_FN_ATTN_BWD, {}, {hCuDnn, hAttn, hQ, hdQ, hK, hdK, hV, hdV, hMask, hY, hdY});
+    }
     void AttnDecodeForward(int nBatch, int nHeads, int nKvHeads, int nSize, int nLen, long hQ, long hKCache, long hVCache, long hY,
                            long long nStrideBatch, long long nStrideHead, long long nStridePos, float fScale = 0.f)
     {
@@ -341,6 +388,7 @@ public:
     }
     void FreeRope(long h) { m_cuda.RunFloat(m_hKernel, MCH_FN_FREE_ROPE, {(float)h}); }
     void RopeForward(long hRope, long long n, long hX, long hY, int nFreqOffset = -1) { ex2(MCH_FN_ROPE_FWD, {}, {hRope, n, hX, hY, nFreqOffset}); }
+    void RopeBackward(long hRope, long long n, long hXdata, long hYdiff, long hXdiff) { ex2(MCH_FN_ROPE_BWD, {}, {hRope, n, hXdata, hYdiff, hXdiff}); }   // :6425
 
     // ---- extensions (CudaDnn.cs:3703-3811)
     long CreateExtension(const std::string& strExtensionDllPath)

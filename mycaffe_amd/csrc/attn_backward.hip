@@ -12,7 +12,8 @@
 // over all keys there (all scores equal) and is marked here by lse2 = -inf.
 //
 // Kernels:
-//  * attn_bwd_stats_kernel: D for every row and, when the forward pass left no lse2, lse2 as well (one wavefront a row).
+//  * attn_bwd_stats_kernel: D for every row and, when the forward pass left no lse2, lse2 as well (one wavefront a row);
+//    skipped when the MFMA kernels run on a stored lse2 (the dQ kernel then computes D on the way).
 //  * attn_bwd_dq_rows_kernel / attn_bwd_dkv_rows_kernel: any head size up to 256, any mask kind, Tq != Tk: one wavefront
 //    per query row (per key row), lanes over the other sequence axis.  No atomics: every output row has one owner, so
 //    results do not depend on scheduling.
@@ -41,6 +42,7 @@ struct AttnBwdArgs {
     int B, H, Tq, Tk, hs, kind;
     float scale;
     int computeLse;
+    int computeD;     // MFMA path: the dQ kernel computes D itself (no statistics kernel ran)
 };
 
 __device__ inline bool attn_masked(const AttnBwdArgs& a, int b, int row, int key)
@@ -227,7 +229,8 @@ template <typename T> __global__ __launch_bounds__(256) void attn_bwd_dkv_rows_k
     }
 }
 
-hipError_t attn_bwd_mfma_launch(hipStream_t s, DType dt, const AttnBwdArgs& a, bool* handled);
+bool attn_bwd_mfma_usable(DType dt, const AttnBwdArgs& a);
+hipError_t attn_bwd_mfma_launch(hipStream_t s, DType dt, const AttnBwdArgs& a);
 
 size_t attn_backward_workspace_bytes(int B, int H, int Tq) { return (size_t)B * H * Tq * 2 * sizeof(float); }
 
@@ -246,11 +249,14 @@ hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k
     a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale;
     a.computeLse = lse2 ? 0 : 1;
     dim3 gq((Tq + 3) / 4, H, B), gk((Tk + 3) / 4, H, B);
-    if (dt == F32) hipLaunchKernelGGL(attn_bwd_stats_kernel<float>, gq, 256, 0, s, a);
-    else hipLaunchKernelGGL(attn_bwd_stats_kernel<bf16_t>, gq, 256, 0, s, a);
-    bool handled = false;
-    hipError_t e = attn_bwd_mfma_launch(s, dt, a, &handled);
-    if (e != hipSuccess || handled) return e;
+    const bool mfma = attn_bwd_mfma_usable(dt, a);
+    // the statistics kernel is needed for lse2 when the forward pass left none, and for D whenever the row kernels run
+    a.computeD = (mfma && lse2) ? 1 : 0;
+    if (!a.computeD) {
+        if (dt == F32) hipLaunchKernelGGL(attn_bwd_stats_kernel<float>, gq, 256, 0, s, a);
+        else hipLaunchKernelGGL(attn_bwd_stats_kernel<bf16_t>, gq, 256, 0, s, a);
+    }
+    if (mfma) return attn_bwd_mfma_launch(s, dt, a);
     if (dt == F32) {
         hipLaunchKernelGGL(attn_bwd_dq_rows_kernel<float>, gq, 256, 0, s, a);
         hipLaunchKernelGGL(attn_bwd_dkv_rows_kernel<float>, gk, 256, 0, s, a);
@@ -509,7 +515,19 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs 
         }
     }
     const float lrow = qrow < a.Tq ? a.lse2[bh * a.Tq + qrow] : INFINITY;
-    const float drow = qrow < a.Tq ? a.dsum[bh * a.Tq + qrow] : 0.f;
+    // D[row] = sum_d dY * Y.  When the statistics kernel did not run (the forward pass left lse2), it is computed here from
+    // the dY fragments already in registers and stored for the dK/dV kernel, which is launched after this one.
+    float drow = 0.f;
+    if (a.computeD) {
+        const T* yp = (const T*)a.y + bh * a.Tq * HS + (size_t)min(qrow, a.Tq - 1) * HS;
+#pragma unroll
+        for (int f = 0; f < KF; f++) drow += TR::dot(*(const u32x4*)(yp + f * CPF + half * (CPF / 2)), gf[f]);
+        drow += __shfl_xor(drow, 32, 64);
+        if (qrow < a.Tq && half == 0) a.dsum[bh * a.Tq + qrow] = drow;
+        if (qrow >= a.Tq) drow = 0.f;
+    } else if (qrow < a.Tq) {
+        drow = a.dsum[bh * a.Tq + qrow];
+    }
     floatx16 aq[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
@@ -626,8 +644,8 @@ static hipError_t bwd_launch_kind(hipStream_t s, const AttnBwdArgs& a, int mb)
     const int nbh = a.B * a.H;
     const long long gkv = (long long)((a.Tk + 127) / 128) * nbh, gq = (long long)((a.Tq + 127) / 128) * nbh;
     if (gkv > 0x7fffffffll || gq > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kq, dim3((unsigned)gq), 256, qBytes, s, a, mb);      // first: it may produce D for the other kernel
     hipLaunchKernelGGL(kkv, dim3((unsigned)gkv), 256, kvBytes, s, a, mb);
-    hipLaunchKernelGGL(kq, dim3((unsigned)gq), 256, qBytes, s, a, mb);
     return hipGetLastError();
 }
 
@@ -641,22 +659,23 @@ template <typename T, int HS, int BS, int OCC> static hipError_t bwd_launch_cfg(
     }
 }
 
-hipError_t attn_bwd_mfma_launch(hipStream_t s, DType dt, const AttnBwdArgs& a, bool* handled)
+bool attn_bwd_mfma_usable(DType, const AttnBwdArgs& a)
 {
-    *handled = false;
-    if (a.hs != 64 && a.hs != 128) return hipSuccess;
-    if ((((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.dy | (uintptr_t)a.dq | (uintptr_t)a.dk | (uintptr_t)a.dv) & 15) != 0)
-        return hipSuccess;
-    int kind, mb = 1;
+    if (a.hs != 64 && a.hs != 128) return false;
+    return (((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.y | (uintptr_t)a.dy | (uintptr_t)a.dq | (uintptr_t)a.dk |
+             (uintptr_t)a.dv) & 15) == 0;
+}
+
+hipError_t attn_bwd_mfma_launch(hipStream_t s, DType dt, const AttnBwdArgs& a)
+{
+    int kind = 0, mb = 1;
     switch (a.kind) {
     case MASK_NONE: kind = 0; break;
     case MASK_CAUSAL: kind = 1; break;
     case MASK_KEY: kind = 2; break;
     case MASK_BQK: kind = 3; break;
-    case MASK_QK: kind = 3; mb = 0; break;     // one (Tq,Tk) mask for every sequence
-    default: return hipSuccess;
+    default: kind = 3; mb = 0; break;          // MASK_QK: one (Tq,Tk) mask for every sequence
     }
-    *handled = true;
     if (dt == BF16) {
         if (a.hs == 64) return bwd_launch_cfg<bf16_t, 64, 64, 2>(s, a, kind, mb);
         return bwd_launch_cfg<bf16_t, 128, 32, 1>(s, a, kind, mb);

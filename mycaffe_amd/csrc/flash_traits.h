@@ -44,6 +44,18 @@ template <> struct FlashTraits<bf16_t> {
         return u32x4{pack_bf16x2(p[8 * t], p[8 * t + 1]), pack_bf16x2(p[8 * t + 2], p[8 * t + 3]),
                      pack_bf16x2(p[8 * t + 4], p[8 * t + 5]), pack_bf16x2(p[8 * t + 6], p[8 * t + 7])};
     }
+    // sum of the eight products of two fragments
+    __device__ static inline float dot(u32x4 a, u32x4 b)
+    {
+        float r = 0.f;
+        const uint32_t av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r += __uint_as_float(av[i] << 16) * __uint_as_float(bv[i] << 16);
+            r += __uint_as_float(av[i] & 0xffff0000u) * __uint_as_float(bv[i] & 0xffff0000u);
+        }
+        return r;
+    }
     __device__ static inline void store4(bf16_t* dst, float a, float b, float c, float d)
     {
         uint2 w;
@@ -77,6 +89,11 @@ template <> struct FlashTraits<float> {
     {
         return u32x4{__float_as_uint(p[4 * t]), __float_as_uint(p[4 * t + 1]), __float_as_uint(p[4 * t + 2]),
                      __float_as_uint(p[4 * t + 3])};
+    }
+    __device__ static inline float dot(u32x4 a, u32x4 b)
+    {
+        return __uint_as_float(a.x) * __uint_as_float(b.x) + __uint_as_float(a.y) * __uint_as_float(b.y) +
+               __uint_as_float(a.z) * __uint_as_float(b.z) + __uint_as_float(a.w) * __uint_as_float(b.w);
     }
     __device__ static inline void store4(float* dst, float a, float b, float c, float d) { *(float4*)dst = make_float4(a, b, c, d); }
     __device__ static inline void scatter_chunk(float* d, int ld, u32x4 r)

@@ -116,7 +116,7 @@ static void csa_golden(CudaDnn& cuda, const std::string& dir, int heads)
     tr.Forward({B, T, heads, hs}, hK, hKt);
     tr.Forward({B, T, heads, hs}, hV, hVt);
     long hCudnn = cuda.CreateCuDNN(), hAttn = cuda.CreateAttn();
-    cuda.SetAttn(hCudnn, hAttn, 0, false, B, T, heads, hs, 0.f);
+    cuda.SetAttn(hCudnn, hAttn, 0, true, B, T, heads, hs, 0.f);    // training: the forward call keeps what ATTN_BWD needs
     cuda.AttnScaledDotProductForward(hCudnn, hAttn, T, hQt, hKt, hVt, hMask, hWork, 0);
     // y.transpose(1, 2).contiguous().view(B, T, C), then the output projection
     TransposeLayer tb(cuda, {0, 2, 1, 3});
@@ -125,9 +125,52 @@ static void csa_golden(CudaDnn& cuda, const std::string& dir, int heads)
     std::vector<float> out = cuda.GetMemoryFloat(hTop, (long long)M * C);
     const double err = max_rel_err(out, y.data);
     report(("causal self attention layer vs " + dir.substr(dir.find_last_of('/') + 1) + "/y.txt").c_str(), err <= 1e-4, err);
+    // gradients of the attention core against the reference's dump of the same layer (iter_0): dY (B,H,T,hs) -> dQ, dK, dV
+    {
+        Tensor gy = load_txt(dir + "/iter_0/grad_y_pre_transpose.txt");
+        long hdY = cuda.AllocMemory(gy.data), hdQ = cuda.AllocMemory((long long)M * C), hdK = cuda.AllocMemory((long long)M * C);
+        long hdV = cuda.AllocMemory((long long)M * C);
+        cuda.AttnScaledDotProductBackward(hCudnn, hAttn, hQt, hdQ, hKt, hdK, hVt, hdV, hMask, hWork, hdY);
+        double worst = 0;
+        const char* names[3] = {"/iter_0/grad_qt.txt", "/iter_0/grad_kt.txt", "/iter_0/grad_vt.txt"};
+        const long hs3[3] = {hdQ, hdK, hdV};
+        for (int i = 0; i < 3; i++) worst = std::max(worst, max_rel_err(cuda.GetMemoryFloat(hs3[i], (long long)M * C), load_txt(dir + names[i]).data));
+        report(("attention backward vs " + dir.substr(dir.find_last_of('/') + 1) + "/iter_0 grad_qt, grad_kt, grad_vt").c_str(), worst <= 1e-4, worst);
+        for (long h : {hdY, hdQ, hdK, hdV}) cuda.FreeMemory(h);
+    }
     cuda.FreeAttn(hAttn);
     cuda.FreeCuDNN(hCudnn);
     for (long h : {hX, hWa, hBa, hWp, hBp, hOnes, hIp, hQ, hK, hV, hQt, hKt, hVt, hWork, hY, hTop, hMask}) cuda.FreeMemory(h);
+}
+
+// LayerNorm handle forward and gradient on the reference's dump (x, y, grad_1a_y -> grad_9_x), eps 1e-10
+static void layernorm_golden(CudaDnn& cuda, const std::string& dir)
+{
+    Tensor x = load_txt(dir + "/x.txt"), y = load_txt(dir + "/y.txt"), gy = load_txt(dir + "/grad_1a_y.txt"), gx = load_txt(dir + "/grad_9_x.txt");
+    const int B = x.shape[0], T = x.shape[1], C = x.shape[2];
+    const long long n = (long long)B * T * C;
+    long h = cuda.CreateLayerNorm(0, n, B, T, C, 1e-10f);
+    long hX = cuda.AllocMemory(x.data), hY = cuda.AllocMemory(n), hdY = cuda.AllocMemory(gy.data), hdX = cuda.AllocMemory(n);
+    cuda.LayerNormForward(h, hX, hY);
+    const double e1 = max_rel_err(cuda.GetMemoryFloat(hY, n), y.data);
+    cuda.LayerNormBackward(h, hY, hdY, hdX);
+    const double e2 = max_rel_err(cuda.GetMemoryFloat(hdX, n), gx.data);
+    report(("layer norm forward + backward vs " + dir.substr(dir.find_last_of('/') + 1)).c_str(), e1 <= 1e-4 && e2 <= 1e-4, std::max(e1, e2));
+    cuda.FreeLayerNorm(h);
+    for (long m : {hX, hY, hdY, hdX}) cuda.FreeMemory(m);
+}
+
+static void gelu_golden(CudaDnn& cuda, const std::string& dir)
+{
+    Tensor x = load_txt(dir + "/1_x.txt"), y = load_txt(dir + "/2_y.txt"), gy = load_txt(dir + "/grad_1_y.txt"), gx = load_txt(dir + "/grad_2_x.txt");
+    const long long n = (long long)x.data.size();
+    long hX = cuda.AllocMemory(x.data), hY = cuda.AllocMemory(n), hdY = cuda.AllocMemory(gy.data), hdX = cuda.AllocMemory(n);
+    cuda.gelu_fwd(n, hX, hY, true);
+    const double e1 = max_rel_err(cuda.GetMemoryFloat(hY, n), y.data);
+    cuda.gelu_bwd(n, hdY, hY, hdX, hX, true);
+    const double e2 = max_rel_err(cuda.GetMemoryFloat(hdX, n), gx.data);
+    report("gelu forward + backward vs gpt-pico-gelu", e1 <= 1e-4 && e2 <= 1e-4, std::max(e1, e2));
+    for (long m : {hX, hY, hdY, hdX}) cuda.FreeMemory(m);
 }
 
 int main(int argc, char** argv)
@@ -182,6 +225,9 @@ int main(int argc, char** argv)
         csa_golden(cuda, g + "/gpt-pico-csaB", 1);
         csa_golden(cuda, g + "/gpt-pico-csa3", 3);
         csa_golden(cuda, g + "/gpt-pico-csa3B", 3);
+        layernorm_golden(cuda, g + "/gpt-pico-ln");
+        layernorm_golden(cuda, g + "/gpt-pico-ln3B");
+        gelu_golden(cuda, g + "/gpt-pico-gelu");
         // 4. llama2 extension
         if (argc >= 7) {
             LlmInference llm(cuda, argv[3]);
