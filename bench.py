@@ -319,6 +319,42 @@ def bench_gemm(cuda, reps):
     return out
 
 
+def bench_block_ops(cuda, reps, warm=3):
+    """The per-block elementwise ops at the GPT-2 shape of the prefill benchmark (8192 rows x 768, MLP width 3072):
+    LayerNorm handle forward / backward, GELU forward / backward.  HBM bound: algorithmic bytes = tensors read + written."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    rows, C = 8192, 768
+    out = {}
+    rng = np.random.default_rng(0)
+    for name, half, es in (("bf16", True, 2), ("f32", False, 4)):
+        n = rows * C
+        x = cuda.AllocMemory(rng.standard_normal(n).astype(np.float32), bHalfSize=half)
+        y, dy, dx = (cuda.AllocMemory(n, bHalfSize=half) for _ in range(3))
+        h = cuda.CreateLayerNorm(0, n, 8, 1024, C, 1e-5)
+        cuda.LayerNormForward(h, x, y)
+        res = {}
+        for key, fn, rgl, tensors in (("layernorm_fwd", CUDAFN.CUDA_LAYERNORM_FWD, [h, x, y], 2),
+                                      ("layernorm_bwd", CUDAFN.CUDA_LAYERNORM_BWD, [h, y, dy, dx], 3)):
+            ms = cuda.TimeFunction(fn, None, rgl, warm, reps)
+            gbs = tensors * n * es / (ms / 1e3) / 1e9
+            res[key] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+        cuda.FreeLayerNorm(h)
+        for hh in (x, y, dy, dx):
+            cuda.FreeMemory(hh)
+        n = rows * 4 * C
+        x = cuda.AllocMemory(rng.standard_normal(n).astype(np.float32), bHalfSize=half)
+        y, dy, dx = (cuda.AllocMemory(n, bHalfSize=half) for _ in range(3))
+        for key, fn, rgl, tensors in (("gelu_tanh_fwd", CUDAFN.CUDA_GELU_FWD, [n, x, y, 1], 2),
+                                      ("gelu_tanh_bwd", CUDAFN.CUDA_GELU_BWD, [n, dy, y, dx, x, 1], 3)):
+            ms = cuda.TimeFunction(fn, None, rgl, warm, reps)
+            gbs = tensors * n * es / (ms / 1e3) / 1e9
+            res[key] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+        for hh in (x, y, dy, dx):
+            cuda.FreeMemory(hh)
+        out[name] = res
+    return out
+
+
 def bench_copy(cuda, reps, warm=2):
     """Plain streaming kernel of known size (y = 1.0 * x over 64 Mi floats: reads 256 MiB, writes 256 MiB): the kernel
     that the FETCH_SIZE / WRITE_SIZE counter readings of the other kernels are scaled by."""
@@ -365,7 +401,7 @@ def main():
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
                     "prints what ran instead of the benchmark line")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,decode_attn,encdec,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -413,6 +449,9 @@ def main():
     if want("backward"):
         also["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 30)
         log("attention backward:", json.dumps(also["attention_backward_B8_T1024_H12x64"]))
+    if want("block_ops"):
+        also["block_ops_8192x768"] = bench_block_ops(cuda, 20)
+        log("block ops:", json.dumps(also["block_ops_8192x768"]))
     if want("encdec"):
         also["encdec_attention_B32_H8x64_bf16"] = bench_encdec_attention(cuda, 50)
         log("enc-dec attention:", json.dumps(also["encdec_attention_B32_H8x64_bf16"]))

@@ -31,6 +31,78 @@ template <> __device__ inline void st<bf16_t>(bf16_t* p, size_t i, float v) { p[
     } while (0)
 
 // ---------------------------------------------------------------------------
+// Elementwise maps y = f(a, b): eight elements per thread and trip (one 16-byte access for bf16, two for fp32) when all
+// operands are 16-byte aligned, one element per thread otherwise and for the tail.
+typedef __bf16 ew_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ew_floatx2 __attribute__((ext_vector_type(2)));
+// two fp32 -> packed bf16 pair with the hardware conversion (round to nearest even)
+__device__ inline uint32_t pack2_bf16_hw(float a, float b)
+{
+    ew_floatx2 f = {a, b};
+    ew_bf16x2 r = __builtin_convertvector(f, ew_bf16x2);
+    return *reinterpret_cast<uint32_t*>(&r);
+}
+
+template <typename T> struct Vec8;
+template <> struct Vec8<float> {
+    __device__ static inline void load(const float* p, float (&v)[8])
+    {
+        const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    __device__ static inline void store(float* p, const float (&v)[8])
+    {
+        *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+        *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+template <> struct Vec8<bf16_t> {
+    __device__ static inline void load(const bf16_t* p, float (&v)[8])
+    {
+        const uint4 a = *(const uint4*)p;
+        const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    __device__ static inline void store(bf16_t* p, const float (&v)[8])
+    {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = pack2_bf16_hw(v[2 * i], v[2 * i + 1]);
+        *(uint4*)p = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+};
+
+template <typename T, bool TWO, typename F> __global__ void map_kernel(size_t n, size_t chunks, const T* a, const T* b, T* y, F f)
+{
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)blockDim.x * gridDim.x;
+    for (size_t c = gid; c < chunks; c += stride) {
+        float va[8], vb[8], r[8];
+        Vec8<T>::load(a + c * 8, va);
+        if (TWO) Vec8<T>::load(b + c * 8, vb);
+#pragma unroll
+        for (int j = 0; j < 8; j++) r[j] = f(va[j], TWO ? vb[j] : 0.f);
+        Vec8<T>::store(y + c * 8, r);
+    }
+    for (size_t i = chunks * 8 + gid; i < n; i += stride) st(y, i, f(ld(a, i), TWO ? ld(b, i) : 0.f));
+}
+
+// y = f(a) (b == nullptr) or y = f(a, b)
+template <typename F> static hipError_t launch_map(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, F f)
+{
+    if (n == 0) return hipSuccess;
+    const bool aligned = ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15) == 0);
+    const size_t chunks = aligned ? n / 8 : 0;
+    const int g = grid_for(chunks ? chunks : n);
+    if (b) DISPATCH_DT(dt, hipLaunchKernelGGL((map_kernel<T, true, F>), g, TPB, 0, s, n, chunks, (const T*)a, (const T*)b, (T*)y, f));
+    else DISPATCH_DT(dt, hipLaunchKernelGGL((map_kernel<T, false, F>), g, TPB, 0, s, n, chunks, (const T*)a, (const T*)a, (T*)y, f));
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 template <typename T> __global__ void set_kernel(T* y, size_t n, float v) { GRID_STRIDE(i, n) st(y, i, v); }
 
 hipError_t k_set(hipStream_t s, DType dt, void* y, size_t n, float v)
@@ -60,70 +132,20 @@ hipError_t k_convert(hipStream_t s, DType sdt, const void* src, DType ddt, void*
     return hipGetLastError();
 }
 
-template <typename T> __global__ void axpy_kernel(size_t n, float a, const T* x, T* y)
-{
-    GRID_STRIDE(i, n) st(y, i, a * ld(x, i) + ld(y, i));
-}
-hipError_t k_axpy(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(axpy_kernel<T>, grid_for(n), TPB, 0, s, n, alpha, (const T*)x, (T*)y));
-    return hipGetLastError();
-}
-
-template <typename T> __global__ void scale_kernel(size_t n, float a, const T* x, T* y)
-{
-    GRID_STRIDE(i, n) st(y, i, a * ld(x, i));
-}
-hipError_t k_scale(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(scale_kernel<T>, grid_for(n), TPB, 0, s, n, alpha, (const T*)x, (T*)y));
-    return hipGetLastError();
-}
-
-template <typename T> __global__ void add_kernel(size_t n, const T* a, const T* b, T* y, float alpha)
-{
-    GRID_STRIDE(i, n) st(y, i, ld(a, i) + ld(b, i) * alpha);
-}
-hipError_t k_add(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, float alpha)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(add_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y, alpha));
-    return hipGetLastError();
-}
-
-template <typename T> __global__ void mul_kernel(size_t n, const T* a, const T* b, T* y)
-{
-    GRID_STRIDE(i, n) st(y, i, ld(a, i) * ld(b, i));
-}
-hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(mul_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y));
-    return hipGetLastError();
-}
-
+struct AxpyF { float a; __device__ float operator()(float x, float y) const { return a * x + y; } };
+struct ScaleF { float a; __device__ float operator()(float x, float) const { return a * x; } };
+struct AddF { float alpha; __device__ float operator()(float a, float b) const { return a + b * alpha; } };
+struct MulF { __device__ float operator()(float a, float b) const { return a * b; } };
 __device__ inline float silu_f(float x) { return x * (1.0f / (1.0f + expf(-x))); }
+struct SiluF { __device__ float operator()(float x, float) const { return silu_f(x); } };
+struct SwigluF { __device__ float operator()(float a, float b) const { return silu_f(a) * b; } };
 
-template <typename T> __global__ void silu_kernel(size_t n, const T* x, T* y) { GRID_STRIDE(i, n) st(y, i, silu_f(ld(x, i))); }
-hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(silu_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y));
-    return hipGetLastError();
-}
-
-template <typename T> __global__ void swiglu_kernel(size_t n, const T* a, const T* b, T* y)
-{
-    GRID_STRIDE(i, n) st(y, i, silu_f(ld(a, i)) * ld(b, i));
-}
-hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(swiglu_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y));
-    return hipGetLastError();
-}
+hipError_t k_axpy(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y) { return launch_map(s, dt, n, x, y, y, AxpyF{alpha}); }
+hipError_t k_scale(hipStream_t s, DType dt, size_t n, float alpha, const void* x, void* y) { return launch_map(s, dt, n, x, nullptr, y, ScaleF{alpha}); }
+hipError_t k_add(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, float alpha) { return launch_map(s, dt, n, a, b, y, AddF{alpha}); }
+hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y) { return launch_map(s, dt, n, a, b, y, MulF{}); }
+hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y) { return launch_map(s, dt, n, x, nullptr, y, SiluF{}); }
+hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y) { return launch_map(s, dt, n, a, b, y, SwigluF{}); }
 
 // y[i] = mask[i % maskDim] == search ? replace : x[i]
 template <typename T>
@@ -498,10 +520,127 @@ template <typename T> __global__ void layernorm_fwd_kernel(int inner, const T* x
     for (int i = threadIdx.x; i < inner; i += TPB) st(yr, i, (ld(xr, i) - mean) / sd);
 }
 
+// Rows of up to 2048 values, a multiple of 4: one wavefront per row, the row lives in registers (chunks of four values,
+// lane l takes chunks l, l + 64, ...), reductions stay inside the wavefront.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    __device__ static inline void load(const float* p, float (&v)[4]) { const float4 a = *(const float4*)p; v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; }
+    __device__ static inline void store(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4<bf16_t> {
+    __device__ static inline void load(const bf16_t* p, float (&v)[4])
+    {
+        const uint2 a = *(const uint2*)p;
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    }
+    __device__ static inline void store(bf16_t* p, const float (&v)[4])
+    {
+        *(uint2*)p = make_uint2(pack2_bf16_hw(v[0], v[1]), pack2_bf16_hw(v[2], v[3]));
+    }
+};
+
+template <typename T, int R> __global__ __launch_bounds__(256) void layernorm_fwd_wave_kernel(int rows, int inner, const T* x, T* y, float* stdev, float eps)
+{
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = inner >> 2;
+    const T* xr = x + (size_t)row * inner;
+    T* yr = y + (size_t)row * inner;
+    float v[R][4];
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + 64 * r;
+        if (c < chunks) {
+            Vec4<T>::load(xr + 4 * c, v[r]);
+            sum += (v[r][0] + v[r][1]) + (v[r][2] + v[r][3]);
+        }
+    }
+    const float mean = wave_sum(sum) / inner;
+    float sq = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (lane + 64 * r < chunks) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[r][j] -= mean;
+                sq += v[r][j] * v[r][j];
+            }
+        }
+    const float sd = sqrtf(wave_sum(sq) / inner + eps);
+    if (lane == 0) stdev[row] = sd;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + 64 * r;
+        if (c < chunks) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[r][j] /= sd;
+            Vec4<T>::store(yr + 4 * c, v[r]);
+        }
+    }
+}
+
+template <typename T, int R>
+__global__ __launch_bounds__(256) void layernorm_bwd_wave_kernel(int rows, int inner, const T* y, const T* dy, T* dx, const float* stdev, float bump)
+{
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = inner >> 2;
+    const size_t base = (size_t)row * inner;
+    float vy[R][4], vg[R][4];
+    float a = 0.f, b = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + 64 * r;
+        if (c < chunks) {
+            Vec4<T>::load(y + base + 4 * c, vy[r]);
+            Vec4<T>::load(dy + base + 4 * c, vg[r]);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                a += vy[r][j] * vg[r][j];
+                b += vg[r][j];
+            }
+        }
+    }
+    const float m1 = wave_sum(a) / inner, m2 = wave_sum(b) / inner;
+    const float sd = stdev[row];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + 64 * r;
+        if (c < chunks) {
+            float o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float div = base + 4 * c + j < (size_t)rows ? sd + bump : sd;
+                o[j] = (vg[r][j] - (vy[r][j] * m1 + m2)) / div;
+            }
+            Vec4<T>::store(dx + base + 4 * c, o);
+        }
+    }
+}
+
+// register budget per lane: R chunks of four values
+static inline int layernorm_wave_chunks(int inner, const void* a, const void* b, const void* c, size_t esize)
+{
+    if (inner % 4 != 0 || inner > 2048) return 0;
+    if ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & (4 * esize - 1)) != 0) return 0;
+    const int r = (inner / 4 + 63) / 64;
+    return r <= 1 ? 1 : (r <= 2 ? 2 : (r <= 4 ? 4 : 8));
+}
+
 hipError_t k_layernorm_fwd(hipStream_t s, DType dt, int rows, int inner, const void* x, void* y, float* stdev, float eps)
 {
     if (rows <= 0 || inner <= 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_fwd_kernel<T>, rows, TPB, 0, s, inner, (const T*)x, (T*)y, stdev, eps));
+    const int R = layernorm_wave_chunks(inner, x, y, y, dt == F32 ? 4 : 2);
+    const int g = (rows + 3) / 4;
+#define LN_FWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((layernorm_fwd_wave_kernel<T, RR>), g, 256, 0, s, rows, inner, (const T*)x, (T*)y, stdev, eps))
+    if (R == 1) LN_FWD(1);
+    else if (R == 2) LN_FWD(2);
+    else if (R == 4) LN_FWD(4);
+    else if (R == 8) LN_FWD(8);
+    else DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_fwd_kernel<T>, rows, TPB, 0, s, inner, (const T*)x, (T*)y, stdev, eps));
+#undef LN_FWD
     return hipGetLastError();
 }
 
@@ -533,104 +672,78 @@ hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const v
                            const float* stdev, float bump)
 {
     if (rows <= 0 || inner <= 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_bwd_kernel<T>, rows, TPB, 0, s, rows, inner, (const T*)y, (const T*)dy, (T*)dx,
-                                       stdev, bump));
+    const int R = layernorm_wave_chunks(inner, y, dy, dx, dt == F32 ? 4 : 2);
+    const int g = (rows + 3) / 4;
+#define LN_BWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((layernorm_bwd_wave_kernel<T, RR>), g, 256, 0, s, rows, inner, (const T*)y, (const T*)dy, (T*)dx, stdev, bump))
+    if (R == 1) LN_BWD(1);
+    else if (R == 2) LN_BWD(2);
+    else if (R == 4) LN_BWD(4);
+    else if (R == 8) LN_BWD(8);
+    else DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_bwd_kernel<T>, rows, TPB, 0, s, rows, inner, (const T*)y, (const T*)dy, (T*)dx,
+                                            stdev, bump));
+#undef LN_BWD
     return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
-// GELU (math.cu:11348-11376) and its gradient (math.cu:11412-11448).  The tanh ("bert") forward evaluates in double
-// as the reference's expression does; the erf forward and both gradients are single precision there.
-__device__ inline float gelu_fwd_f(float x, bool bert)
-{
-    if (bert) {
-        const float k = (float)sqrt(2.0 / M_PI);
-        const float x3 = x * x * x;
-        return (float)(0.5 * x * (1.0 + tanh(k * (x + 0.044715 * x3))));
+// GELU (math.cu:11348-11376) and its gradient (math.cu:11412-11448).  The reference evaluates the tanh ("bert") forward
+// in double and rounds to T; here everything is single precision with tanh through one exp (difference: a few 1e-7 of |x|).
+// tanh through one v_exp_f32: 1 - 2 / (e^{2u} + 1); exact limits at +-inf, absolute error about one float ulp of 1
+__device__ inline float tanh_fast(float u) { return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f); }
+
+struct GeluF {
+    bool bert;
+    __device__ float operator()(float x, float) const
+    {
+        if (bert) {
+            const float k = 0.7978845608028654f;   // sqrt(2 / pi)
+            // 0.5 x (1 + tanh u) = x (1 - 1 / (e^{2u} + 1))
+            return x * (1.0f - __builtin_amdgcn_rcpf(__expf(2.0f * k * (x + 0.044715f * (x * x * x))) + 1.0f));
+        }
+        return x * (0.5f * (1.0f + erff(x * 0.7071067811865475f)));
     }
-    const float r2 = (float)sqrt(2.0);
-    return x * (0.5f * (1.0f + erff(x / r2)));
-}
-__device__ inline float gelu_grad_f(float x, bool bert)
-{
-    if (bert) {
-        const float x3 = x * x * x;
-        const float t = 0.797885f * (x + 0.044715f * x3);
-        const float vx = 0.0535161f * x3 + 0.398942f * x;
-        const float ch = coshf(t);
-        return 0.5f * tanhf(t) + vx * (1.0f / (ch * ch)) + 0.5f;
+};
+struct GeluGradF {   // f(dy, x)
+    bool bert;
+    __device__ float operator()(float dy, float x) const
+    {
+        float grad;
+        if (bert) {
+            const float x3 = x * x * x;
+            const float t = tanh_fast(0.797885f * (x + 0.044715f * x3));      // the reference's rounded constants
+            grad = 0.5f * t + (0.0535161f * x3 + 0.398942f * x) * (1.0f - t * t) + 0.5f;   // 1 / cosh^2 = 1 - tanh^2
+        } else {
+            const float cdf = 0.5f * (1.0f + erff(x * 0.7071067811865475f));
+            const float pdf = 0.3989422804014327f * __expf(-0.5f * (x * x));   // 1 / sqrt(2 pi)
+            grad = cdf + x * pdf;
+        }
+        return dy * grad;
     }
-    const float r2pi = (float)sqrt(2.0 * M_PI), r2 = (float)sqrt(2.0);
-    const float cdf = 0.5f * (1.0f + erff(x / r2));
-    const float pdf = 1.0f / r2pi * expf(-0.5f * (x * x));
-    return cdf + x * pdf;
-}
-template <typename T> __global__ void gelu_fwd_kernel(size_t n, const T* x, T* y, bool bert)
-{
-    GRID_STRIDE(i, n) st(y, i, gelu_fwd_f(ld(x, i), bert));
-}
-template <typename T> __global__ void gelu_bwd_kernel(size_t n, const T* dy, const T* x, T* dx, bool bert)
-{
-    GRID_STRIDE(i, n) st(dx, i, ld(dy, i) * gelu_grad_f(ld(x, i), bert));
-}
-hipError_t k_gelu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, bool bert)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(gelu_fwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, bert));
-    return hipGetLastError();
-}
+};
+struct SiluGradF {   // f(dy, x) = dy * s (1 + x (1 - s)) (math.cu:11740-11749)
+    __device__ float operator()(float dy, float x) const
+    {
+        const float sg = 1.0f / (1.0f + expf(-x));
+        return dy * (sg * (1.0f + x * (1.0f - sg)));
+    }
+};
+// ReLU with negative slope (math.cu:12038-12044) and its gradient, which looks at the TOP data (math.cu:12072-12078)
+struct ReluF { float slope; __device__ float operator()(float x, float) const { return x > 0.f ? x : x * slope; } };
+struct ReluGradF {   // f(dy, y)
+    float slope;
+    __device__ float operator()(float dy, float y) const { return dy * ((y > 0.f ? 1.f : 0.f) + (y <= 0.f ? 1.f : 0.f) * slope); }
+};
+
+hipError_t k_gelu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, bool bert) { return launch_map(s, dt, n, x, nullptr, y, GeluF{bert}); }
 hipError_t k_gelu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx, bool bert)
 {
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(gelu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)x, (T*)dx, bert));
-    return hipGetLastError();
+    return launch_map(s, dt, n, dy, x, dx, GeluGradF{bert});
 }
-
-// SiLU gradient: dx = dy * s(x) (1 + x (1 - s(x))) (math.cu:11740-11749)
-template <typename T> __global__ void silu_bwd_kernel(size_t n, const T* dy, const T* x, T* dx)
-{
-    GRID_STRIDE(i, n)
-    {
-        const float v = ld(x, i);
-        const float sg = 1.0f / (1.0f + expf(-v));
-        st(dx, i, ld(dy, i) * (sg * (1.0f + v * (1.0f - sg))));
-    }
-}
-hipError_t k_silu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(silu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)x, (T*)dx));
-    return hipGetLastError();
-}
-
-// ReLU with negative slope (math.cu:12038-12044) and its gradient, which looks at the TOP data (math.cu:12072-12078)
-template <typename T> __global__ void relu_fwd_kernel(size_t n, const T* x, T* y, float slope)
-{
-    GRID_STRIDE(i, n)
-    {
-        const float v = ld(x, i);
-        st(y, i, v > 0.f ? v : v * slope);
-    }
-}
-template <typename T> __global__ void relu_bwd_kernel(size_t n, const T* dy, const T* y, T* dx, float slope)
-{
-    GRID_STRIDE(i, n)
-    {
-        const float v = ld(y, i);
-        st(dx, i, ld(dy, i) * ((v > 0.f ? 1.f : 0.f) + (v <= 0.f ? 1.f : 0.f) * slope));
-    }
-}
-hipError_t k_relu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, float slope)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(relu_fwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, slope));
-    return hipGetLastError();
-}
+hipError_t k_silu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx) { return launch_map(s, dt, n, dy, x, dx, SiluGradF{}); }
+hipError_t k_relu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, float slope) { return launch_map(s, dt, n, x, nullptr, y, ReluF{slope}); }
 hipError_t k_relu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* y, void* dx, float slope)
 {
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(relu_bwd_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)dy, (const T*)y, (T*)dx, slope));
-    return hipGetLastError();
+    return launch_map(s, dt, n, dy, y, dx, ReluGradF{slope});
 }
 
 }  // namespace mch
