@@ -1071,6 +1071,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         st->maskHandle = 0;
         st->lseValid = false;
         st->lastTq = st->lastTk = 0;
+        st->lastMask = 0;
         return 0;
     }
     case MCH_FN_ATTN_FWD: {
@@ -1125,18 +1126,29 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 st->lseCap = rows;
             }
             lse = st->lse;
+            const size_t ybytes = (size_t)qn * Y->esize();
+            if (st->ysaveBytes < ybytes) {
+                if (st->ysave) { HIPCHK(hipStreamSynchronize(s)); (void)hipFree(st->ysave); st->ysave = nullptr; st->ysaveBytes = 0; }
+                HIPCHK(hipMalloc(&st->ysave, ybytes));
+                st->ysaveBytes = ybytes;
+            }
         }
         HIPCHK(k_attn_prefill(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, st->batch, st->heads, T, Tk, st->hs, st->scale,
                               M ? (const float*)M->ptr : nullptr, kind, lse));
+        // the backward pass needs this output (dY . Y per row); the C# layer hands ATTN_BWD a Y buffer that holds the
+        // head-merged layout by then (CausalSelfAttentionLayer.cs:668-672), so a copy stays with the handle
+        if (lse) HIPCHK(hipMemcpyAsync(st->ysave, Y->ptr, (size_t)qn * Y->esize(), hipMemcpyDeviceToDevice, s));
         st->lseValid = lse != nullptr;
-        st->lastTq = T; st->lastTk = Tk; st->lastBatchMask = batchMask;
+        st->lastTq = T; st->lastTk = Tk; st->lastBatchMask = batchMask; st->lastMask = hMask;
         m_mem.touch((long)pl[7]);
         return 0;
     }
     case MCH_FN_ATTN_BWD: {
         // l{hCudnn,hAttn,hQ,hdQ,hK,hdK,hV,hdV,hMask,hY,hdY} (CudaDnn.cs:5695-5701, device.h:2509-2529, attn.cu:608-661).
-        // Sequence lengths and the mask layout are those of the handle's last forward call (the reference reads
-        // the probabilities that call left behind); without one, the block size given to ATTN_SET is used.
+        // Sequence lengths, the mask and its layout are those of the handle's last forward call: the reference reads
+        // the probabilities that call left behind and never looks at hMask here (CausalSelfAttentionLayer.cs:672 passes
+        // 0), so the probabilities are recomputed under the forward call's mask.  Without a forward call the block
+        // size given to ATTN_SET and the hMask argument are used.
         NEED_L(11, 11);
         AttnState* st = m_attn.get((long)pl[1]);
         if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
@@ -1152,7 +1164,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         ERRCHK(mem((long)pl[7], &dV));
         ERRCHK(mem((long)pl[9], &Y));
         ERRCHK(mem((long)pl[10], &dY));
-        long hMask = (long)pl[8];
+        long hMask = st->lastTq > 0 ? st->lastMask : (long)pl[8];
         if (hMask) ERRCHK(mem(hMask, &M));
         for (MemItem* it : {dQ, K, dK, V, dV, Y, dY})
             if (it->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
@@ -1178,7 +1190,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         const size_t wsBytes = attn_backward_workspace_bytes(st->batch, st->heads, T);
         ERRCHK(workspace(wsBytes, &ws));
         const bool haveLse = st->lseValid && st->lseCap >= (size_t)st->batch * st->heads * T;
-        HIPCHK(k_attn_backward(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, dY->ptr, dQ->ptr, dK->ptr, dV->ptr, st->batch, st->heads,
+        const bool haveY = haveLse && st->ysave && st->ysaveBytes >= (size_t)qn * Y->esize();
+        HIPCHK(k_attn_backward(s, Q->dt(), Q->ptr, K->ptr, V->ptr, haveY ? st->ysave : Y->ptr, dY->ptr, dQ->ptr, dK->ptr, dV->ptr, st->batch, st->heads,
                                T, Tk, st->hs, st->scale, M ? (const float*)M->ptr : nullptr, kind, haveLse ? st->lse : nullptr,
                                ws, wsBytes));
         m_mem.touch((long)pl[3]);

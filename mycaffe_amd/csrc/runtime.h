@@ -79,8 +79,9 @@ struct AttnState {
     long maskHandle = 0; uint64_t maskVersion = 0; int maskT = 0; bool maskCausal = false;
     // what the backward pass needs of the last training-mode forward: log2 of every row's softmax denominator
     float* lse = nullptr; size_t lseCap = 0; bool lseValid = false;
-    int lastTq = 0, lastTk = 0; long long lastBatchMask = 0;
-    ~AttnState() { if (lse) (void)hipFree(lse); }
+    void* ysave = nullptr; size_t ysaveBytes = 0;   // copy of that forward's output (the caller's Y buffer may be reused)
+    int lastTq = 0, lastTk = 0; long long lastBatchMask = 0; long lastMask = 0;
+    ~AttnState() { if (lse) (void)hipFree(lse); if (ysave) (void)hipFree(ysave); }
 };
 struct RopeState {
     bool set = false;

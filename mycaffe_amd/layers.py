@@ -3,7 +3,8 @@
 These follow the C# ``forward`` methods call for call (cited per class), so that a
 forward pass here issues the same sequence of ``CudaDnn`` calls, with the same
 argument packing, as the unchanged C# host would issue against the native library.
-Inference only: dropout layers are identity and backward is not mirrored.
+Dropout layers are the identity (inference, or training with ratio 0).  ``Backward`` is mirrored for the GPT block
+(InnerProduct, Transpose, LayerNorm, activations, CausalSelfAttention with the fused attention handle, TransformerBlock).
 """
 import math
 
@@ -21,6 +22,8 @@ class Blob:
         self.shape_ = []
         self.gpu_data = 0
         self._capacity = 0
+        self._gpu_diff = 0
+        self._diff_capacity = 0
         if shape is not None:
             self.Reshape(*shape)
 
@@ -53,6 +56,27 @@ class Blob:
     mutable_gpu_data = property(lambda self: self.gpu_data)
 
     @property
+    def gpu_diff(self):
+        """Gradient buffer of the same size, allocated (zero filled) on first use."""
+        n = self.count()
+        if n > self._diff_capacity:
+            if self._gpu_diff:
+                self.cuda.FreeMemory(self._gpu_diff)
+            self._gpu_diff = self.cuda.AllocMemory(n, bHalfSize=self.half)
+            self._diff_capacity = n
+        return self._gpu_diff
+
+    mutable_gpu_diff = gpu_diff
+
+    @property
+    def mutable_cpu_diff(self):
+        return self.cuda.GetMemoryFloat(self.gpu_diff, self.count()).reshape(self.shape_)
+
+    @mutable_cpu_diff.setter
+    def mutable_cpu_diff(self, values):
+        self.cuda.SetMemory(self.gpu_diff, np.asarray(values, np.float32).reshape(-1), nCount=self.count())
+
+    @property
     def mutable_cpu_data(self):
         return self.cuda.GetMemoryFloat(self.gpu_data, self.count()).reshape(self.shape_)
 
@@ -63,9 +87,14 @@ class Blob:
     def SetData(self, value):
         self.cuda.set(self.count(), self.gpu_data, float(value))
 
-    def CopyFrom(self, src):
-        self.ReshapeLike(src)
-        self.cuda.copy(self.count(), src.gpu_data, self.gpu_data)
+    def CopyFrom(self, src, bCopyDiff=False, bReshape=True):
+        """Blob.cs CopyFrom(src, bCopyDiff, bReshape): copies the data, or with bCopyDiff the diff."""
+        if bReshape:
+            self.ReshapeLike(src)
+        if bCopyDiff:
+            self.cuda.copy(self.count(), src.gpu_diff, self.gpu_diff)
+        else:
+            self.cuda.copy(self.count(), src.gpu_data, self.gpu_data)
 
     def MatMul(self, blobA, blobB, bReshape=False, bTransA=False, bTransB=False, dfScale=1.0):
         """Blob.cs:4229-4269: batched row-major matmul over the two leading axes."""
@@ -88,6 +117,10 @@ class Blob:
             self.cuda.FreeMemory(self.gpu_data)
             self.gpu_data = 0
             self._capacity = 0
+        if self._gpu_diff:
+            self.cuda.FreeMemory(self._gpu_diff)
+            self._gpu_diff = 0
+            self._diff_capacity = 0
 
 
 class InnerProductLayer:
@@ -128,31 +161,63 @@ class InnerProductLayer:
                                top.gpu_data)
 
 
+    def Backward(self, top, bottom):
+        """InnerProductLayer.cs:429-494: weight gradient accumulates into the weight diff, bias gradient through gemv with
+        the ones vector, data gradient = top diff x W."""
+        M = bottom.count(0, self.axis)
+        hTopDiff, hW = top.gpu_diff, self.blobs[0].gpu_data
+        self.cuda.gemm(True, False, self.N, self.K, M, 1.0, hTopDiff, bottom.gpu_data, 1.0, self.blobs[0].gpu_diff)
+        if self.bias_term:
+            if self.bias_multiplier is None or self.bias_multiplier.count() < M:
+                self.bias_multiplier = Blob(self.cuda, (M,), self.half)
+                self.bias_multiplier.SetData(1.0)
+            self.cuda.gemv(True, M, self.N, 1.0, hTopDiff, self.bias_multiplier.gpu_data, 1.0, self.blobs[1].gpu_diff)
+        self.cuda.gemm(False, False, M, self.K, self.N, 1.0, hTopDiff, hW, 0.0, bottom.gpu_diff)
+
+
 class TransposeLayer:
-    """MyCaffe.layers.beta/layers.beta/TransposeLayer.cs:127-213."""
+    """MyCaffe.layers.beta/layers.beta/TransposeLayer.cs:127-232."""
 
     def __init__(self, cuda, dim):
         self.cuda, self.dim = cuda, list(dim)
         self._key = None
+        self._handles = []
 
-    def Forward(self, bottom, top):
-        shape = bottom.shape_
-        top_shape = [shape[d] for d in self.dim]
-        if bottom.gpu_data == top.gpu_data:
-            raise ValueError("The Transpose layer does not support in-place computation.")
-        top.Reshape(*top_shape)
+    def _reshape(self, shape):
+        """Reshape (TransposeLayer.cs:127-200): stride arrays of bottom and top, forward and backward axis maps."""
         key = (tuple(shape), tuple(self.dim))
+        top_shape = [shape[d] for d in self.dim]
         if key != self._key:
+            for h in self._handles:
+                self.cuda.FreeMemory(h)
             n = len(shape)
             bc = [int(np.prod(shape[i + 1:])) for i in range(n)]
             tc = [int(np.prod(top_shape[i + 1:])) for i in range(n)]
+            bmap = [0] * n
+            for i, d in enumerate(self.dim):
+                bmap[d] = i
             self.counts_b = self.cuda.AllocMemory(np.float32(bc))
             self.counts_t = self.cuda.AllocMemory(np.float32(tc))
             self.fmap = self.cuda.AllocMemory(np.float32(self.dim))
-            self.buffer = self.cuda.AllocMemory(bottom.count() * n)
+            self.bmap = self.cuda.AllocMemory(np.float32(bmap))
+            self.buffer = self.cuda.AllocMemory(int(np.prod(shape)) * n)
+            self._handles = [self.counts_b, self.counts_t, self.fmap, self.bmap, self.buffer]
             self._key = key
+        return top_shape
+
+    def Forward(self, bottom, top):
+        if bottom.gpu_data == top.gpu_data:
+            raise ValueError("The Transpose layer does not support in-place computation.")
+        top.Reshape(*self._reshape(bottom.shape_))
         self.cuda.transpose(bottom.count(), bottom.gpu_data, top.gpu_data, self.counts_b, self.counts_t, self.fmap,
-                            len(shape), self.buffer)
+                            len(bottom.shape_), self.buffer)
+
+    def Backward(self, top, bottom):
+        """TransposeLayer.cs:223-232: reshape for this bottom, then the same kernel with the count arrays swapped and the
+        inverse axis map."""
+        self._reshape(bottom.shape_)
+        self.cuda.transpose(bottom.count(), top.gpu_diff, bottom.gpu_diff, self.counts_t, self.counts_b, self.bmap,
+                            len(bottom.shape_), self.buffer)
 
 
 class SoftmaxLayer:
@@ -184,7 +249,8 @@ class CausalSelfAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, training=False):
+        self.training = training
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
         self.nSize = embed // heads
         self.bias_term, self.half = bias_term, half
@@ -217,7 +283,7 @@ class CausalSelfAttentionLayer:
             if not self.hCudnn:
                 self.hCudnn = self.cuda.CreateCuDNN()
                 self.hAttn = self.cuda.CreateAttn()
-            self.cuda.SetAttn(self.hCudnn, self.hAttn, 0, False, B, self.nBlockSize, self.nHeads, self.nSize, 0.0)
+            self.cuda.SetAttn(self.hCudnn, self.hAttn, 0, self.training, B, self.nBlockSize, self.nHeads, self.nSize, 0.0)
         if self.enable_rope:
             if self.hRope:
                 self.cuda.FreeRope(self.hRope)
@@ -273,8 +339,36 @@ class CausalSelfAttentionLayer:
             b["Work"].MatMul(b["AttB"], b["Vt"], bReshape=True)
         # y.transpose(1, 2).contiguous().view(B, T, C)
         self.transpose.Forward(b["Work"], b["Y"])
+        self._y_shape = list(b["Y"].shape_)
         b["Y"].Reshape(B, T, C)
         self.c_proj.Forward(b["Y"], top)
+
+    def Backward(self, top, blobX):
+        """CausalSelfAttentionLayer.cs:641-747 with the fused attention handle: top.gpu_diff -> blobX.gpu_diff, parameter
+        gradients accumulate in the InnerProduct weight diffs.  The handle's backward call gets mask handle 0, as there."""
+        if not self.enable_sdpa:
+            raise NotImplementedError("the explicit chain's backward (softmax gradient) is not mirrored")
+        b, cuda = self.b, self.cuda
+        B, T, C = blobX.shape_[:3]
+        self.c_proj.Backward(top, b["Y"])
+        b["Y"].Reshape(*self._y_shape)
+        self.transpose.Backward(b["Y"], b["Work"])
+        b["Y"].CopyFrom(b["Work"], True, True)
+        cuda.AttnScaledDotProductBackward(self.hCudnn, self.hAttn, b["Qt"].gpu_data, b["Qt"].gpu_diff, b["Kt"].gpu_data,
+                                          b["Kt"].gpu_diff, b["Vt"].gpu_data, b["Vt"].gpu_diff, 0, b["Y"].gpu_data, b["Y"].gpu_diff)
+        self.transpose.Backward(b["Kt"], b["K"])
+        self.transpose.Backward(b["Qt"], b["Q"])
+        self.transpose.Backward(b["Vt"], b["V"])
+        if self.hRope:
+            cuda.RopeBackward(self.hRope, b["Q"].count(), b["Q"].gpu_data, b["Q"].gpu_diff, b["Q"].gpu_diff)
+            cuda.RopeBackward(self.hRope, b["K"].count(), b["K"].gpu_data, b["K"].gpu_diff, b["K"].gpu_diff)
+        nCount = b["Q"].count()
+        ip = b["IpAttn"]
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 0, ip.gpu_diff, b["Q"].gpu_diff, DIR.BWD)
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 1, ip.gpu_diff, b["K"].gpu_diff, DIR.BWD)
+        cuda.channel_copy(nCount, ip.num, ip.channels, 3, self.nEmbed, 2, ip.gpu_diff, b["V"].gpu_diff, DIR.BWD)
+        b["Y"].Reshape(B, T, C)
+        self.c_attn.Backward(ip, blobX)
 
 
 class MultiheadAttentionLayer:
@@ -397,8 +491,8 @@ class LayerNormLayer:
         top.ReshapeLike(bottom)
         self.cuda.LayerNormForward(self.hLayerNorm, bottom.gpu_data, top.gpu_data)
 
-    def Backward(self, top, hTopDiff, hBottomDiff):
-        self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, hTopDiff, hBottomDiff)
+    def Backward(self, top, bottom):
+        self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, top.gpu_diff, bottom.gpu_diff)
 
 
 class ActivationLayer:
@@ -409,16 +503,34 @@ class ActivationLayer:
         if kind not in ("relu", "gelu", "gelu_bert", "silu"):
             raise ValueError(kind)
         self.cuda, self.kind = cuda, kind
+        self.blobX = Blob(cuda)     # GeluLayer.cs:84-87: the input is kept when the layer runs in place
 
     def Forward(self, bottom, top):
         top.ReshapeLike(bottom)
         n = bottom.count()
+        hBottom = bottom.gpu_data
+        if self.kind != "relu" and bottom.gpu_data == top.gpu_data:
+            self.blobX.CopyFrom(bottom)
+            hBottom = self.blobX.gpu_data
         if self.kind == "relu":
-            self.cuda.relu_fwd(n, bottom.gpu_data, top.gpu_data, 0.0)
+            self.cuda.relu_fwd(n, hBottom, top.gpu_data, 0.0)
         elif self.kind == "silu":
-            self.cuda.silu_fwd(n, bottom.gpu_data, top.gpu_data)
+            self.cuda.silu_fwd(n, hBottom, top.gpu_data)
         else:
-            self.cuda.gelu_fwd(n, bottom.gpu_data, top.gpu_data, self.kind == "gelu_bert")
+            self.cuda.gelu_fwd(n, hBottom, top.gpu_data, self.kind == "gelu_bert")
+
+    def Backward(self, top, bottom):
+        """ReLULayer.cs:203, GeluLayer.cs:110-121, SiLULayer.cs backward."""
+        n = bottom.count()
+        hBottomData = bottom.gpu_data
+        if top.gpu_data == bottom.gpu_data:
+            hBottomData = self.blobX.gpu_data
+        if self.kind == "relu":
+            self.cuda.relu_bwd(n, top.gpu_diff, top.gpu_data, bottom.gpu_diff, 0.0)
+        elif self.kind == "silu":
+            self.cuda.silu_bwd(n, top.gpu_diff, top.gpu_data, bottom.gpu_diff, hBottomData)
+        else:
+            self.cuda.gelu_bwd(n, top.gpu_diff, top.gpu_data, bottom.gpu_diff, hBottomData, self.kind == "gelu_bert")
 
 
 class TransformerBlockLayer:
@@ -426,11 +538,12 @@ class TransformerBlockLayer:
     forward :810-902): x + attn(ln1(x)), then + proj(act(fc(ln2(.)))).  Dropout is the identity at inference."""
 
     def __init__(self, cuda, heads, embed, block_size, activation="relu", bias_term=True, epsilon=1e-10,
-                 enable_cuda_scaled_dot_product_attention=True):
+                 enable_cuda_scaled_dot_product_attention=True, training=False):
         self.cuda = cuda
         self.norm1 = LayerNormLayer(cuda, epsilon)
         self.norm2 = LayerNormLayer(cuda, epsilon)
-        self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention)
+        self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention,
+                                              training=training)
         self.fc1 = InnerProductLayer(cuda, 4 * embed, bias_term, 2)
         self.proj = InnerProductLayer(cuda, embed, bias_term, 2)
         self.act = ActivationLayer(cuda, activation)
@@ -457,3 +570,21 @@ class TransformerBlockLayer:
         self.proj.Forward(b["Mlp1"], b["MlpOut"])
         top.ReshapeLike(blobX)
         cuda.add(nCount, b["X"].gpu_data, b["MlpOut"].gpu_data, top.gpu_data)
+
+    def Backward(self, top, blobX):
+        """TransformerBlockLayer.cs:924-1040, CAUSAL_SELF_ATTENTION block: top.gpu_diff -> blobX.gpu_diff."""
+        b, cuda = self.b, self.cuda
+        nCount = blobX.count()
+        cuda.copy(nCount, top.gpu_diff, b["MlpOut"].gpu_diff)
+        cuda.copy(nCount, top.gpu_diff, b["X"].gpu_diff)
+        self.proj.Backward(b["MlpOut"], b["Mlp1"])
+        self.act.Backward(b["Mlp1"], b["Mlp1"])
+        self.fc1.Backward(b["Mlp1"], b["Norm2"])
+        # x_2 = ln_2(xB): keep xB's own gradient aside, add the one that comes through the norm
+        b["Attn1"].CopyFrom(b["X"], True)
+        self.norm2.Backward(b["Norm2"], b["X"])
+        cuda.add(nCount, b["Attn1"].gpu_diff, b["X"].gpu_diff, b["X"].gpu_diff)
+        b["Attn1"].CopyFrom(b["X"], True)
+        self.attn1.Backward(b["Attn1"], b["Norm1"])
+        self.norm1.Backward(b["Norm1"], blobX)
+        cuda.add(nCount, b["X"].gpu_diff, blobX.gpu_diff, blobX.gpu_diff)
