@@ -319,6 +319,32 @@ def bench_gemm(cuda, reps):
     return out
 
 
+def bench_matmul_chain(cuda, reps, warm=3):
+    """The two strided-batched MatMul calls of the explicit (not fused) attention chain at B=8, T=1024, 12 x 64, fp32
+    (ids 219): Q K^T -> (B,H,T,T) and P V -> (B,H,T,hs), the route the C# layers take when the fused handle is off."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    outer, T, hs = 96, 1024, 64
+    rng = np.random.default_rng(0)
+    q = cuda.AllocMemory(rng.standard_normal(outer * T * hs).astype(np.float32))
+    kt = cuda.AllocMemory(rng.standard_normal(outer * T * hs).astype(np.float32))
+    v = cuda.AllocMemory(rng.standard_normal(outer * T * hs).astype(np.float32))
+    att = cuda.AllocMemory(outer * T * T)
+    y = cuda.AllocMemory(outer * T * hs)
+    out = {}
+    # matmul(outer, m, n, k, A, B, C) = gemm2(false, false, n, m, k, 1, B, A, 0, C, n, k, n, k*n, m*k, m*n, outer)
+    for name, (m, n, k, hA, hB, hC) in (("qk_t", (T, T, hs, q, kt, att)), ("p_v", (T, hs, T, att, v, y))):
+        rgl = [0, 0, n, m, k, 0, hB, hA, 0, hC, n, k, n, k * n, m * k, m * n, outer]
+        ms = cuda.TimeFunction(CUDAFN.CUDA_GEMM2, [1.0, 0.0], rgl, warm, reps)
+        fl = 2.0 * outer * m * n * k
+        nbytes = 4.0 * outer * (m * k + k * n + m * n)
+        tf = fl / (ms / 1e3) / 1e12
+        out[name] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_PEAK_TFLOPS["f32"], 4),
+                     "GBps": round(nbytes / (ms / 1e3) / 1e9, 1), "frac_hbm": round(nbytes / (ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4)}
+    for h in (q, kt, v, att, y):
+        cuda.FreeMemory(h)
+    return out
+
+
 def bench_block_ops(cuda, reps, warm=3):
     """The per-block elementwise ops at the GPT-2 shape of the prefill benchmark (8192 rows x 768, MLP width 3072):
     LayerNorm handle forward / backward, GELU forward / backward.  HBM bound: algorithmic bytes = tensors read + written."""
@@ -401,7 +427,7 @@ def main():
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
                     "prints what ran instead of the benchmark line")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,block_ops,decode_attn,encdec,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,matmul_chain,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -449,6 +475,9 @@ def main():
     if want("backward"):
         also["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 30)
         log("attention backward:", json.dumps(also["attention_backward_B8_T1024_H12x64"]))
+    if want("matmul_chain"):
+        also["matmul_chain_B8_T1024_H12x64_f32"] = bench_matmul_chain(cuda, 10)
+        log("matmul chain:", json.dumps(also["matmul_chain_B8_T1024_H12x64_f32"]))
     if want("block_ops"):
         also["block_ops_8192x768"] = bench_block_ops(cuda, 20)
         log("block ops:", json.dumps(also["block_ops_8192x768"]))

@@ -580,6 +580,156 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
     return launch_generic<bf16_t>(s, m, n, k, alpha, (const bf16_t*)A, (const bf16_t*)B, beta, (bf16_t*)C, st, 1);
 }
 
+// ---------------------------------------------------------------------------
+// fp32 MFMA for the strided-batched gemm2 (the Blob.MatMul route of the explicit attention chain: Q K^T and P V per
+// (batch, head), math.cu:1750-1788).  Column-major operands with any leading dimension: A(i,k) has either i or k at unit
+// stride, B(k,j) either k or j, C(i,j) has i at unit stride.  Both operands are staged into LDS as [row][k] (a
+// transposing scatter when the row index is the unit-stride one), so that one 128-bit LDS read feeds four
+// v_mfma_f32_32x32x2_f32 steps (slot trick as in gemm_nt_f32_mfma_kernel).  The MFMA row operand is B and the column
+// operand is A: the accumulator then has i in the lane and every store instruction of a wavefront writes two 128-byte
+// runs of C.  TI x TJ tile (i x j), four wavefronts 2 x 2.
+template <bool A_IFAST, bool B_KFAST, int TI, int TJ>
+__global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K, float alpha, const float* __restrict__ A,
+                                                             const float* __restrict__ B, float beta, float* __restrict__ C,
+                                                             GemmStrides st)
+{
+    constexpr int BK = 16, LDK = BK + 4;
+    constexpr int NI = TI / 64, NJ = TJ / 64;        // 32x32 blocks per wavefront along i and j
+    __shared__ __attribute__((aligned(16))) float Is[2][TI * LDK];   // A: [i][k]
+    __shared__ __attribute__((aligned(16))) float Js[2][TJ * LDK];   // B: [j][k]
+    A += (size_t)blockIdx.z * st.sA;
+    B += (size_t)blockIdx.z * st.sB;
+    C += (size_t)blockIdx.z * st.sC;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wi = (wave & 1) * (TI / 2), wj = (wave >> 1) * (TJ / 2);
+    const int i0 = blockIdx.x * TI, j0 = blockIdx.y * TJ;
+    const long long lda = A_IFAST ? st.ak : st.ai, ldb = B_KFAST ? st.bj : st.bk;
+
+    floatx16 acc[NJ][NI];
+#pragma unroll
+    for (int a = 0; a < NJ; a++)
+#pragma unroll
+        for (int b = 0; b < NI; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+    // staging: TI*BK/4 float4 of A and TJ*BK/4 of B per stage, 256 threads
+    constexpr int PA = TI * BK / 4 / 256, PB = TJ * BK / 4 / 256;
+    float4 ra[PA], rb[PB];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < PA; p++) {
+            const int e = tid + p * 256;
+            ra[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (A_IFAST) {   // four consecutive i at one k
+                const int ig = e % (TI / 4), k = e / (TI / 4);
+                if (i0 + 4 * ig < M && k0 + k < K) ra[p] = *(const float4*)(A + (size_t)(i0 + 4 * ig) + (size_t)(k0 + k) * lda);
+            } else {         // four consecutive k at one i
+                const int kg = e % (BK / 4), i = e / (BK / 4);
+                if (i0 + i < M && k0 + 4 * kg < K) ra[p] = *(const float4*)(A + (size_t)(i0 + i) * lda + (size_t)(k0 + 4 * kg));
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PB; p++) {
+            const int e = tid + p * 256;
+            rb[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (B_KFAST) {
+                const int kg = e % (BK / 4), j = e / (BK / 4);
+                if (j0 + j < N && k0 + 4 * kg < K) rb[p] = *(const float4*)(B + (size_t)(j0 + j) * ldb + (size_t)(k0 + 4 * kg));
+            } else {
+                const int jg = e % (TJ / 4), k = e / (TJ / 4);
+                if (j0 + 4 * jg < N && k0 + k < K) rb[p] = *(const float4*)(B + (size_t)(j0 + 4 * jg) + (size_t)(k0 + k) * ldb);
+            }
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < PA; p++) {
+            const int e = tid + p * 256;
+            if (A_IFAST) {
+                const int ig = e % (TI / 4), k = e / (TI / 4);
+                float* d = &Is[buf][(4 * ig) * LDK + k];
+                d[0] = ra[p].x; d[LDK] = ra[p].y; d[2 * LDK] = ra[p].z; d[3 * LDK] = ra[p].w;
+            } else {
+                const int kg = e % (BK / 4), i = e / (BK / 4);
+                *(float4*)(&Is[buf][i * LDK + 4 * kg]) = ra[p];
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PB; p++) {
+            const int e = tid + p * 256;
+            if (B_KFAST) {
+                const int kg = e % (BK / 4), j = e / (BK / 4);
+                *(float4*)(&Js[buf][j * LDK + 4 * kg]) = rb[p];
+            } else {
+                const int jg = e % (TJ / 4), k = e / (TJ / 4);
+                float* d = &Js[buf][(4 * jg) * LDK + k];
+                d[0] = rb[p].x; d[LDK] = rb[p].y; d[2 * LDK] = rb[p].z; d[3 * LDK] = rb[p].w;
+            }
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    gload(0);
+    sstore(0);
+    __syncthreads();
+    const int fr = lane & 31, fg = (lane >> 5) * 4;
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 8) {
+            float4 fj[NJ], fi[NI];
+#pragma unroll
+            for (int t = 0; t < NJ; t++) fj[t] = *(const float4*)(&Js[buf][(wj + t * 32 + fr) * LDK + kk + fg]);
+#pragma unroll
+            for (int t = 0; t < NI; t++) fi[t] = *(const float4*)(&Is[buf][(wi + t * 32 + fr) * LDK + kk + fg]);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int a = 0; a < NJ; a++)
+#pragma unroll
+                    for (int b = 0; b < NI; b++)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(((const float*)&fj[a])[e], ((const float*)&fi[b])[e], acc[a][b], 0, 0, 0);
+        }
+        if (kt + 1 < nk) sstore(buf ^ 1);
+        __syncthreads();
+    }
+    // accumulator register v of a block: j = 8*(v/4) + 4*(lane/32) + v%4, i = lane%32
+    const int il = lane & 31, jl = (lane >> 5) * 4;
+#pragma unroll
+    for (int a = 0; a < NJ; a++)
+#pragma unroll
+        for (int b = 0; b < NI; b++) {
+            const int i = i0 + wi + b * 32 + il;
+            if (i >= M) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int j = j0 + wj + a * 32 + (v >> 2) * 8 + jl + (v & 3);
+                if (j < N) {
+                    const size_t ci = (size_t)i + (size_t)j * st.cj;
+                    float o = alpha * acc[a][b][v];
+                    if (beta != 0.f) o += beta * C[ci];
+                    C[ci] = o;
+                }
+            }
+        }
+}
+
+template <bool A_IFAST, bool B_KFAST>
+static hipError_t launch_gemm2_mfma(hipStream_t s, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                                    float* C, const GemmStrides& st, int batch)
+{
+    const bool si = M <= 64, sj = N <= 64;
+    dim3 grid((M + (si ? 63 : 127)) / (si ? 64 : 128), (N + (sj ? 63 : 127)) / (sj ? 64 : 128), batch);
+    if (grid.y > 65535 || grid.z > 65535) return hipErrorInvalidValue;
+    if (si && sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    else if (si) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    else if (sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    else hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    return hipGetLastError();
+}
+
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch)
 {
@@ -589,6 +739,17 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
     st.bk = tB ? ldb : 1;  st.bj = tB ? 1 : ldb;
     st.ci = 1;             st.cj = ldc;
     st.sA = sA; st.sB = sB; st.sC = sC;
+    if (m <= 0 || n <= 0 || batch <= 0) return hipSuccess;
+    // MFMA path: every float4 the staging loads must be aligned and whole (the unit-stride extent a multiple of 4)
+    const bool aligned = ((((uintptr_t)A | (uintptr_t)B) & 15) == 0) && lda % 4 == 0 && ldb % 4 == 0 && sA % 4 == 0 && sB % 4 == 0;
+    const bool aOk = tA ? (k % 4 == 0) : (m % 4 == 0);
+    const bool bOk = tB ? (n % 4 == 0) : (k % 4 == 0);
+    if (aligned && aOk && bOk && k > 0 && (long long)m * n >= 1024) {
+        if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+        if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+        if (tA && !tB) return launch_gemm2_mfma<false, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+        return launch_gemm2_mfma<false, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+    }
     return launch_generic<float>(s, m, n, k, alpha, A, B, beta, C, st, batch);
 }
 

@@ -192,6 +192,46 @@ def test_matmul_batched_is_gemm2_with_swapped_operands(dev):
     assert_close(dev.get(hC), R.matmul(outer, m, n, k, A, Bt, transB=True, dtype=np.float64), FP32_RTOL, "matmul vs checker")
 
 
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+@pytest.mark.parametrize("m,n,k,batch", [(64, 256, 64, 6), (256, 64, 256, 4), (132, 200, 76, 3), (36, 36, 8, 2), (128, 128, 20, 2)])
+def test_gemm2_strided_batched_blas_semantics(dev, tA, tB, m, n, k, batch):
+    """Column-major strided-batched gemm with padded leading dimensions and strides (cublasSgemmStridedBatched
+    semantics, math.cu:1750-1788), alpha / beta, every transpose combination; sizes that take the matrix-core kernel
+    (all extents multiples of 4) including ragged tiles."""
+    rng = np.random.default_rng(m + n + k)
+    ar, ac = (k, m) if tA else (m, k)
+    br, bc = (n, k) if tB else (k, n)
+    lda, ldb, ldc = ar + 4, br + 8, m + 4
+    sA, sB, sC = lda * ac + 8, ldb * bc + 4, ldc * n + 4
+    A = rng.standard_normal(sA * batch).astype(np.float32)
+    B = rng.standard_normal(sB * batch).astype(np.float32)
+    C = rng.standard_normal(sC * batch).astype(np.float32)
+    hA, hB, hC = dev.put(A), dev.put(B), dev.put(C)
+    dev.cuda.gemm2(tA, tB, m, n, k, 0.7, hA, hB, -0.3, hC, lda, ldb, ldc, sA, sB, sC, batch)
+    ref = R.gemm2_colmajor(tA, tB, m, n, k, 0.7, A, B, -0.3, C, lda, ldb, ldc, sA, sB, sC, batch, dtype=np.float64)
+    assert_close(dev.get(hC), ref, FP32_RTOL, "gemm2 tA=%s tB=%s" % (tA, tB))
+    # the padding of C between columns and batches is untouched
+    got = dev.get(hC)
+    for b in range(batch):
+        blk = got[b * sC:(b + 1) * sC]
+        assert np.array_equal(blk[ldc * n:], C[b * sC + ldc * n:(b + 1) * sC])
+        assert np.array_equal(blk[:ldc * n].reshape(n, ldc)[:, m:], C[b * sC:b * sC + ldc * n].reshape(n, ldc)[:, m:])
+
+
+def test_matmul_attention_chain_shapes(dev):
+    """The two MatMul calls of the explicit attention chain (CausalSelfAttentionLayer.cs:583-603) at 64-wide heads."""
+    rng = np.random.default_rng(44)
+    outer, T, hs = 6, 256, 64
+    q, kt, v = rng.standard_normal((outer, T, hs)), rng.standard_normal((outer, hs, T)), rng.standard_normal((outer, T, hs))
+    hq, hkt, hv, hatt, hy = dev.put(q), dev.put(kt), dev.put(v), dev.zeros(outer * T * T), dev.zeros(outer * T * hs)
+    dev.cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    att = q @ kt
+    assert_close(dev.get(hatt), att, FP32_RTOL, "q @ k^T")
+    dev.cuda.matmul(outer, T, hs, T, hatt, hv, hy)
+    assert_close(dev.get(hy), att @ v, FP32_RTOL, "att @ v")
+
+
 @pytest.mark.parametrize("half", [False, True])
 def test_gemv_decode_shapes(dev, half):
     rng = np.random.default_rng(5)
