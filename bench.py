@@ -319,6 +319,36 @@ def bench_gemm(cuda, reps):
     return out
 
 
+def bench_csa_layer(cuda, reps, warm=2):
+    """CausalSelfAttentionLayer.forward at B=8, T=1024, C=768, 12 heads through the layer mirror (the C# call sequence
+    over the C ABI), fp32: with the fused attention handle and with the explicit MatMul / mask / softmax chain that the
+    layer's default parameters select.  Wall clock around `reps` forwards, device synchronised before and after."""
+    from mycaffe_amd.layers import Blob, CausalSelfAttentionLayer
+    B, T, C, H = 8, 1024, 768, 12
+    rng = np.random.default_rng(0)
+    x = Blob(cuda, (B, T, C))
+    x.mutable_cpu_data = rng.standard_normal((B, T, C)).astype(np.float32)
+    wa, ba = rng.standard_normal((3 * C, C)).astype(np.float32) * 0.02, np.zeros(3 * C, np.float32)
+    wp, bp = rng.standard_normal((C, C)).astype(np.float32) * 0.02, np.zeros(C, np.float32)
+    out = {}
+    for name, sdpa in (("fused_handle", True), ("explicit_chain", False)):
+        layer = CausalSelfAttentionLayer(cuda, H, C, T, True, sdpa)
+        top = Blob(cuda)
+        layer.Setup(x, wa, ba, wp, bp)
+        for _ in range(warm):
+            layer.Forward(x, top)
+        cuda.SynchronizeDevice()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            layer.Forward(x, top)
+        cuda.SynchronizeDevice()
+        out[name] = {"ms_per_forward": round((time.perf_counter() - t0) / reps * 1e3, 3)}
+        for b in list(layer.b.values()) + [top, layer.blobMask]:
+            b.Dispose()
+    x.Dispose()
+    return out
+
+
 def bench_matmul_chain(cuda, reps, warm=3):
     """The two strided-batched MatMul calls of the explicit (not fused) attention chain at B=8, T=1024, 12 x 64, fp32
     (ids 219): Q K^T -> (B,H,T,T) and P V -> (B,H,T,hs), the route the C# layers take when the fused handle is off."""
@@ -427,7 +457,7 @@ def main():
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
                     "prints what ran instead of the benchmark line")
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,matmul_chain,block_ops,decode_attn,encdec,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,csa_layer,matmul_chain,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -475,6 +505,9 @@ def main():
     if want("backward"):
         also["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 30)
         log("attention backward:", json.dumps(also["attention_backward_B8_T1024_H12x64"]))
+    if want("csa_layer"):
+        also["csa_layer_B8_T1024_C768_f32"] = bench_csa_layer(cuda, 5)
+        log("csa layer:", json.dumps(also["csa_layer_B8_T1024_C768_f32"]))
     if want("matmul_chain"):
         also["matmul_chain_B8_T1024_H12x64_f32"] = bench_matmul_chain(cuda, 10)
         log("matmul chain:", json.dumps(also["matmul_chain_B8_T1024_H12x64_f32"]))

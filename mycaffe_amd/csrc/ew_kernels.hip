@@ -153,16 +153,7 @@ __global__ void mask_kernel(size_t n, int maskDim, const T* x, const T* mask, T*
 {
     GRID_STRIDE(i, n) st(y, i, ld(mask, i % (size_t)maskDim) == search ? replace : ld(x, i));
 }
-hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
-                  const void* mask, void* y)
-{
-    if (n == 0) return hipSuccess;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(mask_kernel<T>, grid_for(n), TPB, 0, s, n, maskDim, (const T*)x, (const T*)mask,
-                                       (T*)y, search, replace));
-    return hipGetLastError();
-}
-
-// mask index = i % (maskDim/batch) + (i / (n/batch)) * (maskDim/batch)
+// mask index = i % md1 + (i / dd1) * md1 (md1 = maskDim / batch, dd1 = n / batch); the plain mask is the case dd1 = n
 template <typename T>
 __global__ void mask_batch_kernel(size_t n, int md1, size_t dd1, const T* x, const T* mask, T* y, float search,
                                   float replace)
@@ -173,21 +164,54 @@ __global__ void mask_batch_kernel(size_t n, int md1, size_t dd1, const T* x, con
         st(y, i, ld(mask, mi) == search ? replace : ld(x, i));
     }
 }
+// eight elements per thread: needs md1 and dd1 to be multiples of 8 (a chunk never wraps) and 16-byte aligned operands
+template <typename T>
+__global__ void mask_vec_kernel(size_t chunks, size_t md8, size_t dd8, const T* x, const T* mask, T* y, float search, float replace)
+{
+    GRID_STRIDE(c, chunks)
+    {
+        const size_t mc = c % md8 + (c / dd8) * md8;
+        float vx[8], vm[8];
+        Vec8<T>::load(x + c * 8, vx);
+        Vec8<T>::load(mask + mc * 8, vm);
+#pragma unroll
+        for (int k = 0; k < 8; k++) vx[k] = vm[k] == search ? replace : vx[k];
+        Vec8<T>::store(y + c * 8, vx);
+    }
+}
+static hipError_t launch_mask(hipStream_t s, DType dt, size_t n, int md1, size_t dd1, float search, float replace, const void* x,
+                              const void* mask, void* y)
+{
+    const bool vec = md1 % 8 == 0 && dd1 % 8 == 0 && n % 8 == 0 && ((((uintptr_t)x | (uintptr_t)mask | (uintptr_t)y) & 15) == 0);
+    if (vec) {
+        DISPATCH_DT(dt, hipLaunchKernelGGL(mask_vec_kernel<T>, grid_for(n / 8), TPB, 0, s, n / 8, (size_t)md1 / 8, dd1 / 8, (const T*)x,
+                                           (const T*)mask, (T*)y, search, replace));
+    } else {
+        DISPATCH_DT(dt, hipLaunchKernelGGL(mask_batch_kernel<T>, grid_for(n), TPB, 0, s, n, md1, dd1, (const T*)x, (const T*)mask,
+                                           (T*)y, search, replace));
+    }
+    return hipGetLastError();
+}
+hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
+                  const void* mask, void* y)
+{
+    if (n == 0) return hipSuccess;
+    if (maskDim % 8 == 0 && n % (size_t)maskDim == 0)
+        return launch_mask(s, dt, n, maskDim, n, search, replace, x, mask, y);   // i % maskDim with dd1 = n: one "batch"
+    DISPATCH_DT(dt, hipLaunchKernelGGL(mask_kernel<T>, grid_for(n), TPB, 0, s, n, maskDim, (const T*)x, (const T*)mask,
+                                       (T*)y, search, replace));
+    return hipGetLastError();
+}
 hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDim, float search, float replace,
                         const void* x, const void* mask, void* y)
 {
     if (n == 0) return hipSuccess;
-    int md1 = maskDim / batch;
-    size_t dd1 = n / (size_t)batch;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(mask_batch_kernel<T>, grid_for(n), TPB, 0, s, n, md1, dd1, (const T*)x,
-                                       (const T*)mask, (T*)y, search, replace));
-    return hipGetLastError();
+    return launch_mask(s, dt, n, maskDim / batch, n / (size_t)batch, search, replace, x, mask, y);
 }
 
 // Generic permute: xc / yc hold the element strides of the source / destination
 // axes as floats, map[i] the source axis feeding destination axis i.  The
 // per-element index scratch of the reference kernel is replaced by registers.
-struct PermuteArgs { int xs[8]; int ys[8]; int map[8]; int axes; };
 
 template <typename T> __global__ void transpose_kernel(size_t n, const T* x, T* y, PermuteArgs a)
 {
@@ -221,39 +245,85 @@ __global__ void transpose12_kernel(const T* __restrict__ x, T* __restrict__ y, i
     }
 }
 
-hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
-                       const float* map, int axes)
+// the same with 16-byte chunks along the inner axis (inner counts chunks)
+__global__ void transpose12_vec_kernel(const uint4* __restrict__ x, uint4* __restrict__ y, int d1, int d2, int inner, size_t n)
 {
-    if (n == 0) return hipSuccess;
+    GRID_STRIDE(o, n)
+    {
+        int in = (int)(o % inner);
+        size_t r = o / inner;
+        int a1 = (int)(r % d1);
+        r /= d1;
+        int a2 = (int)(r % d2);
+        size_t b = r / d2;
+        y[o] = x[((b * d1 + a1) * d2 + a2) * (size_t)inner + in];
+    }
+}
+
+hipError_t k_transpose_hw(hipStream_t s, DType dt, int nc, int h, int w, const void* x, void* y);
+
+// reads the three small float blobs (source strides, destination strides, axis map) from the device: one round trip
+hipError_t k_transpose_fetch(hipStream_t s, const float* xc, const float* yc, const float* map, int axes, PermuteArgs* out)
+{
     if (axes < 1 || axes > 8) return hipErrorInvalidValue;
     float hx[8], hy[8], hm[8];
     hipError_t e;
-    // the three tiny float blobs live on the device; fetch them once per call
     if ((e = hipMemcpyAsync(hx, xc, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(hy, yc, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(hm, map, axes * sizeof(float), hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
     if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
-    PermuteArgs a;
-    a.axes = axes;
+    out->axes = axes;
     for (int i = 0; i < axes; i++) {
-        a.xs[i] = (int)hx[i];
-        a.ys[i] = (int)hy[i];
-        a.map[i] = (int)hm[i];
-        if (a.xs[i] < 1 || a.ys[i] < 1 || a.map[i] < 0 || a.map[i] >= axes) return hipErrorInvalidValue;
+        out->xs[i] = (int)hx[i];
+        out->ys[i] = (int)hy[i];
+        out->map[i] = (int)hm[i];
+        if (out->xs[i] < 1 || out->ys[i] < 1 || out->map[i] < 0 || out->map[i] >= axes) return hipErrorInvalidValue;
     }
+    return hipSuccess;
+}
+
+hipError_t k_transpose_run(hipStream_t s, DType dt, size_t n, const void* x, void* y, const PermuteArgs& a)
+{
+    if (n == 0) return hipSuccess;
+    const int axes = a.axes;
+    const size_t es = dt == F32 ? 4 : 2;
     // fast path: 4 axes, axes 1 and 2 swapped, coalesced along the untouched inner axis
     if (axes == 4 && a.map[0] == 0 && a.map[1] == 2 && a.map[2] == 1 && a.map[3] == 3 && a.xs[3] == 1 && a.ys[3] == 1) {
         int inner = a.xs[2];
         int d2 = a.xs[1] / a.xs[2];
         int d1 = a.xs[0] / a.xs[1];
         if (a.ys[2] == inner && a.ys[1] == inner * d1 && a.ys[0] == inner * d1 * d2) {
+            const int vec = (int)(16 / es);
+            if (inner % vec == 0 && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
+                hipLaunchKernelGGL(transpose12_vec_kernel, grid_for(n / vec), TPB, 0, s, (const uint4*)x, (uint4*)y, d1, d2, inner / vec,
+                                   n / vec);
+                return hipGetLastError();
+            }
             DISPATCH_DT(dt, hipLaunchKernelGGL(transpose12_kernel<T>, grid_for(n), TPB, 0, s, (const T*)x, (T*)y, d1, d2,
                                                inner, n));
             return hipGetLastError();
         }
     }
+    // fast path: the last two axes swapped, everything in front untouched: tiled transpose through LDS
+    if (axes >= 2 && a.xs[axes - 1] == 1 && a.ys[axes - 1] == 1) {
+        bool lead = a.map[axes - 1] == axes - 2 && a.map[axes - 2] == axes - 1;
+        for (int i = 0; i + 2 < axes; i++) lead = lead && a.map[i] == i && a.xs[i] == a.ys[i];
+        const int w = a.xs[axes - 2], h = a.ys[axes - 2];   // source rows have w elements, destination rows h
+        if (lead && w > 0 && h > 0 && n % ((size_t)w * h) == 0 && (axes < 3 || a.xs[axes - 3] == w * h) && n / ((size_t)w * h) <= 65535)
+            return k_transpose_hw(s, dt, (int)(n / ((size_t)w * h)), h, w, x, y);
+    }
     DISPATCH_DT(dt, hipLaunchKernelGGL(transpose_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)x, (T*)y, a));
     return hipGetLastError();
+}
+
+hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
+                       const float* map, int axes)
+{
+    if (n == 0) return hipSuccess;
+    PermuteArgs a;
+    hipError_t e = k_transpose_fetch(s, xc, yc, map, axes, &a);
+    if (e != hipSuccess) return e;
+    return k_transpose_run(s, dt, n, x, y, a);
 }
 
 // (nc, h, w) -> (nc, w, h) through a padded LDS tile so both sides are coalesced
@@ -294,10 +364,29 @@ __global__ void channel_copy_kernel(size_t n, int channels, int blocks, int inne
         else x[xi] = y[i];
     }
 }
+// the same on 16-byte chunks (inner counts chunks)
+__global__ void channel_copy_vec_kernel(size_t n, int channels, int blocks, int inner, int offset, uint4* x, uint4* y, int dir)
+{
+    GRID_STRIDE(i, n)
+    {
+        size_t nn = i / ((size_t)channels * inner);
+        size_t c = (i % ((size_t)channels * inner)) / inner;
+        size_t b = i % inner;
+        size_t xi = (nn * channels + c) * (size_t)blocks * inner + (size_t)offset * inner + b;
+        if (dir == 0) y[i] = x[xi];
+        else x[xi] = y[i];
+    }
+}
 hipError_t k_channel_copy(hipStream_t s, DType dt, size_t n, int channels, int blocks, int inner, int offset, void* x,
                           void* y, int dir)
 {
     if (n == 0) return hipSuccess;
+    const int vec = dt == F32 ? 4 : 8;
+    if (inner % vec == 0 && n % vec == 0 && ((((uintptr_t)x | (uintptr_t)y) & 15) == 0)) {
+        hipLaunchKernelGGL(channel_copy_vec_kernel, grid_for(n / vec), TPB, 0, s, n / vec, channels, blocks, inner / vec, offset,
+                           (uint4*)x, (uint4*)y, dir);
+        return hipGetLastError();
+    }
     DISPATCH_DT(dt, hipLaunchKernelGGL(channel_copy_kernel<T>, grid_for(n), TPB, 0, s, n, channels, blocks, inner, offset,
                                        (T*)x, (T*)y, dir));
     return hipGetLastError();

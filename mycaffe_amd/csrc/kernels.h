@@ -45,6 +45,10 @@ hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDi
                         const void* x, const void* mask, void* y);
 hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
                        const float* map, int axes);
+// the two halves of k_transpose: fetching the stride / map blobs costs a device round trip, so callers keep the result
+struct PermuteArgs { int xs[8]; int ys[8]; int map[8]; int axes; };
+hipError_t k_transpose_fetch(hipStream_t s, const float* xc, const float* yc, const float* map, int axes, PermuteArgs* out);
+hipError_t k_transpose_run(hipStream_t s, DType dt, size_t n, const void* x, void* y, const PermuteArgs& a);
 hipError_t k_transpose_hw(hipStream_t s, DType dt, int nc, int h, int w, const void* x, void* y);
 hipError_t k_channel_copy(hipStream_t s, DType dt, size_t n, int channels, int blocks, int inner, int offset,
                           void* x, void* y, int dir);

@@ -88,6 +88,7 @@ long MemTable::alloc(size_t count, bool half, hipStream_t s, long* h)
     MemItem& it = m_items[slot];
     it = MemItem();
     it.ptr = p; it.count = count; it.half = half; it.used = true;
+    it.version = ++m_clock;
     *h = slot;
     return 0;
 }
@@ -104,6 +105,7 @@ long MemTable::alloc_view(long hBase, size_t offset, size_t count, long* h)
     MemItem& it = m_items[slot];  // b may dangle after new_slot(); not used below
     it = MemItem();
     it.ptr = p; it.count = count; it.half = half; it.used = true; it.view = true; it.base = root;
+    it.version = ++m_clock;
     *h = slot;
     return 0;
 }
@@ -135,8 +137,9 @@ void MemTable::touch(long h)
 {
     MemItem* it;
     if (get(h, &it)) return;
-    it->version++;
-    if (it->view && !get(it->base, &it)) it->version++;
+    // one clock for the whole table: a (handle, version) pair never repeats, also after the handle is freed and reused
+    it->version = ++m_clock;
+    if (it->view && !get(it->base, &it)) it->version = m_clock;
 }
 
 uint64_t MemTable::version(long h)
@@ -144,7 +147,7 @@ uint64_t MemTable::version(long h)
     MemItem* it;
     if (get(h, &it)) return 0;
     uint64_t v = it->version;
-    if (it->view && !get(it->base, &it)) v += it->version << 20;
+    if (it->view && !get(it->base, &it) && it->version > v) v = it->version;   // a write through the base changes the view
     return v;
 }
 
@@ -743,8 +746,25 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(XC, 0, axes);
         RANGE(YC, 0, axes);
         RANGE(MP, 0, axes);
-        HIPCHK(k_transpose(s, X->dt(), (size_t)n, X->ptr, Y->ptr, (const float*)XC->ptr, (const float*)YC->ptr,
-                           (const float*)MP->ptr, axes));
+        {
+            // the stride / map blobs sit on the device; reading them costs a round trip, so the decoded form is kept per
+            // (handles, content versions) - a layer passes the same three blobs on every call
+            const uint64_t key[6] = {(uint64_t)pl[3], (uint64_t)pl[4], (uint64_t)pl[5], m_mem.version((long)pl[3]),
+                                     m_mem.version((long)pl[4]), m_mem.version((long)pl[5])};
+            const PermuteArgs* pa = nullptr;
+            for (const PermuteCacheEntry& e : m_permuteCache)
+                if (e.axes == axes && memcmp(e.key, key, sizeof(key)) == 0) { pa = &e.args; break; }
+            if (!pa) {
+                PermuteCacheEntry e;
+                memcpy(e.key, key, sizeof(key));
+                e.axes = axes;
+                HIPCHK(k_transpose_fetch(s, (const float*)XC->ptr, (const float*)YC->ptr, (const float*)MP->ptr, axes, &e.args));
+                if (m_permuteCache.size() >= 64) m_permuteCache.erase(m_permuteCache.begin());
+                m_permuteCache.push_back(e);
+                pa = &m_permuteCache.back().args;
+            }
+            HIPCHK(k_transpose_run(s, X->dt(), (size_t)n, X->ptr, Y->ptr, *pa));
+        }
         m_mem.touch((long)pl[2]);
         return 0;
     }

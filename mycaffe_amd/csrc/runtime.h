@@ -45,6 +45,7 @@ private:
     long new_slot();
     std::vector<MemItem> m_items{1};  // slot 0 unused
     std::vector<long> m_free;
+    uint64_t m_clock = 0;             // source of content versions
 };
 
 template <class S> class HandleTable {
@@ -106,6 +107,7 @@ struct BlobLoaderState {
     size_t offsetItems = 0;                // advanced by ADDTOOFFSET, cleared by RESETOFFSET
     ~BlobLoaderState();
 };
+struct PermuteCacheEntry { uint64_t key[6]; int axes; PermuteArgs args; };
 struct ExtensionState {
     void* lib = nullptr;
     void* fnInvoke = nullptr;
@@ -154,6 +156,7 @@ private:
     int* m_tickets = nullptr; size_t m_ticketCount = 0;  // split-K merge tickets; zero whenever no kernel is running
     void* m_stage = nullptr; size_t m_stageBytes = 0;    // pinned host staging
     std::mutex m_stageLock;
+    std::vector<PermuteCacheEntry> m_permuteCache;   // decoded TRANSPOSE arguments by (blob handles, versions)
     std::vector<float*> m_hostAllocs;
     std::mutex m_hostLock;
 };
