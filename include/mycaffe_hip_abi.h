@@ -101,13 +101,23 @@ enum {
     MCH_FN_AXPY = 222,
     MCH_FN_SCAL = 224,
     MCH_FN_SCALE = 227,
+    MCH_FN_ADD_SCALAR = 228,
     MCH_FN_ADD = 229,
+    MCH_FN_SUB = 230,
     MCH_FN_MUL = 231,
+    MCH_FN_DIV = 233,
+    MCH_FN_POWX = 237,
+    MCH_FN_SQRT = 239,
     MCH_FN_TRANSPOSE = 261,
     MCH_FN_MASK = 264,
     MCH_FN_MASK_BATCH = 266,
     MCH_FN_TRANSPOSE_HW = 267,
+    MCH_FN_INVERT = 273,
+    MCH_FN_CHANNEL_MEAN = 287,
     MCH_FN_CHANNEL_COPY = 300,
+    MCH_FN_CHANNEL_FILLFROM = 301,
+    MCH_FN_CHANNEL_COPYALL = 302,
+    MCH_FN_CHANNEL_DUP = 303,
     MCH_FN_EMBED_FWD = 390,
     MCH_FN_RELU_FWD = 428,
     MCH_FN_RELU_BWD = 429,

@@ -835,4 +835,90 @@ hipError_t k_relu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const v
     return launch_map(s, dt, n, dy, y, dx, ReluGradF{slope});
 }
 
+// ---------------------------------------------------------------------------
+// The elementwise / per-row primitives that the C# RMSNormLayer and LayerNormLayer chains are made of
+// (RMSNormLayer.cs:156-180, LayerNormLayer.cs:223-264).
+struct PowxF {   // powx_kernel (math.cu:5955-5961); the square, the only exponent those layers use, is exact
+    float alpha;
+    __device__ float operator()(float a, float) const { return alpha == 2.0f ? a * a : powf(a, alpha); }
+};
+struct SqrtF { float eps; __device__ float operator()(float x, float) const { return sqrtf(x + eps); } };   // math.cu:6211-6217
+struct InvertF {   // invert_kernel and its _n / _d / _nd forms (math.cu:6018-6082): 0 stays 0; factors 0 and 1 are ignored
+    float num, den;
+    __device__ float operator()(float x, float) const { return x == 0.f ? 0.f : num / (x * den); }
+};
+struct SubF { __device__ float operator()(float a, float b) const { return a - b; } };
+struct AddScalarF { float alpha; __device__ float operator()(float y, float) const { return y + alpha; } };
+struct DivF { __device__ float operator()(float a, float b) const { return b == 0.f ? 0.f : a / b; } };   // math.cu:5681-5687
+
+hipError_t k_powx(hipStream_t s, DType dt, size_t n, const void* a, float alpha, void* y) { return launch_map(s, dt, n, a, nullptr, y, PowxF{alpha}); }
+hipError_t k_sqrt(hipStream_t s, DType dt, size_t n, const void* x, void* y, float eps) { return launch_map(s, dt, n, x, nullptr, y, SqrtF{eps}); }
+hipError_t k_invert(hipStream_t s, DType dt, size_t n, const void* x, void* y, float num, float den)
+{
+    const bool un = num != 0.f && num != 1.f, ud = den != 0.f && den != 1.f;
+    return launch_map(s, dt, n, x, nullptr, y, InvertF{un ? num : 1.0f, ud ? den : 1.0f});
+}
+hipError_t k_add_scalar(hipStream_t s, DType dt, size_t n, float alpha, void* y) { return launch_map(s, dt, n, y, nullptr, y, AddScalarF{alpha}); }
+hipError_t k_div(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y) { return launch_map(s, dt, n, a, b, y, DivF{}); }
+
+// y[i] = a[i] - b[i % nB] (sub_kernel, math.cu:5064-5090); nB == 0: plain difference
+template <typename T> __global__ void sub_mod_kernel(size_t n, const T* a, const T* b, T* y, size_t nB)
+{
+    GRID_STRIDE(i, n) st(y, i, ld(a, i) - ld(b, i % nB));
+}
+hipError_t k_sub(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, size_t nB)
+{
+    if (n == 0) return hipSuccess;
+    if (nB == 0) return launch_map(s, dt, n, a, b, y, SubF{});
+    DISPATCH_DT(dt, hipLaunchKernelGGL(sub_mod_kernel<T>, grid_for(n), TPB, 0, s, n, (const T*)a, (const T*)b, (T*)y, nB));
+    return hipGetLastError();
+}
+
+// mean of every row of `inner` values (channel_mean_kernel, math.cu:6817-6831): four rows per workgroup, one wavefront each
+template <typename T> __global__ __launch_bounds__(256) void channel_mean_kernel(size_t rows, int inner, const T* x, T* y)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * inner;
+    float acc = 0.f;
+    for (int i = lane; i < inner; i += 64) acc += ld(xr, i);
+    acc = wave_sum(acc);
+    if (lane == 0) st(y, row, acc / inner);
+}
+hipError_t k_channel_mean(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y)
+{
+    if (rows == 0 || inner <= 0) return hipSuccess;
+    const size_t g = (rows + 3) / 4;
+    if (g > 0x7fffffffu) return hipErrorInvalidValue;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_mean_kernel<T>, (int)g, 256, 0, s, rows, inner, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+
+// MODE 0: y[i] = x[i / spatial]                               (channel_fillfrom forward, math.cu:7465-7472)
+// MODE 1: x[i] = y[i * spatial], i < rows                     (channel_fillfrom backward, math.cu:7474-7481)
+// MODE 2: y[i] = x[i % period]                                (channel_copyall, math.cu:7630-7639)
+// MODE 3: y[i] = x[(i / period) * channels + i % channels]    (channel_duplicate, math.cu:7667-7676)
+template <typename T, int MODE> __global__ void channel_spread_kernel(size_t n, size_t spatial, size_t period, size_t channels, T* x, T* y)
+{
+    GRID_STRIDE(i, n)
+    {
+        if (MODE == 0) y[i] = x[i / spatial];
+        else if (MODE == 1) x[i] = y[i * spatial];
+        else if (MODE == 2) y[i] = x[i % period];
+        else y[i] = x[(i / period) * channels + i % channels];
+    }
+}
+hipError_t k_channel_spread(hipStream_t s, DType dt, int mode, size_t n, size_t spatial, size_t period, size_t channels, void* x, void* y)
+{
+    if (n == 0) return hipSuccess;
+#define SPREAD(M) DISPATCH_DT(dt, hipLaunchKernelGGL((channel_spread_kernel<T, M>), grid_for(n), TPB, 0, s, n, spatial, period, channels, (T*)x, (T*)y))
+    if (mode == 0) SPREAD(0);
+    else if (mode == 1) SPREAD(1);
+    else if (mode == 2) SPREAD(2);
+    else SPREAD(3);
+#undef SPREAD
+    return hipGetLastError();
+}
+
 }  // namespace mch

@@ -67,6 +67,16 @@ hipError_t k_gelu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const v
 hipError_t k_relu_fwd(hipStream_t s, DType dt, size_t n, const void* x, void* y, float slope);
 hipError_t k_relu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* y, void* dx, float slope);
 hipError_t k_silu_bwd(hipStream_t s, DType dt, size_t n, const void* dy, const void* x, void* dx);
+// primitives of the C# RMSNormLayer / LayerNormLayer chains
+hipError_t k_powx(hipStream_t s, DType dt, size_t n, const void* a, float alpha, void* y);
+hipError_t k_sqrt(hipStream_t s, DType dt, size_t n, const void* x, void* y, float eps);
+hipError_t k_invert(hipStream_t s, DType dt, size_t n, const void* x, void* y, float num, float den);
+hipError_t k_add_scalar(hipStream_t s, DType dt, size_t n, float alpha, void* y);
+hipError_t k_div(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y);
+hipError_t k_sub(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, size_t nB);
+hipError_t k_channel_mean(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y);
+// mode 0 fillfrom forward, 1 fillfrom backward, 2 copyall, 3 duplicate (index rules in ew_kernels.hip)
+hipError_t k_channel_spread(hipStream_t s, DType dt, int mode, size_t n, size_t spatial, size_t period, size_t channels, void* x, void* y);
 hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps);
 
 // ---- GEMM family (gemm.hip) ------------------------------------------------

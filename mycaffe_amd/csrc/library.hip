@@ -683,6 +683,144 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
+    case MCH_FN_SUB: {
+        // l{n,hA,hB,hY[,aOff,bOff,yOff,nB]}: y = a - b[i % nB] when nB > 0 (CudaDnn.cs:8132-8138, device.cu:2294-2331)
+        NEED_L(4, 8);
+        long long n = pl[0], ao = ll > 4 ? pl[4] : 0, bo = ll > 5 ? pl[5] : 0, yo = ll > 6 ? pl[6] : 0, nB = ll > 7 ? pl[7] : 0;
+        MemItem *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != B->half || A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (nB < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(A, ao, n);
+        RANGE(B, bo, nB > 0 ? (nB < n ? nB : n) : n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_sub(s, A->dt(), (size_t)n, PTR(A, ao), PTR(B, bo), PTR(Y, yo), (size_t)nB));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+    case MCH_FN_DIV: {
+        // l{n,hA,hB,hY}: y = b == 0 ? 0 : a / b (CudaDnn.cs:8281-8287, device.cu:2492-2505)
+        NEED_L(4, 4);
+        long long n = pl[0];
+        MemItem *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != B->half || A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_div(s, A->dt(), (size_t)n, A->ptr, B->ptr, Y->ptr));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+    case MCH_FN_ADD_SCALAR: {
+        // f{alpha}, l{n,0,hY[,yOff]} (CudaDnn.cs:8010-8016, device.cu:2183-2201)
+        NEED_F(1, 1);
+        NEED_L(3, 4);
+        long long n = pl[0], yo = ll > 3 ? pl[3] : 0;
+        MemItem* Y;
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(Y, yo, n);
+        HIPCHK(k_add_scalar(s, Y->dt(), (size_t)n, pf[0], PTR(Y, yo)));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_POWX: {
+        // f{alpha}, l{n,hA,0,hY[,aOff,yOff]} (CudaDnn.cs:8419-8425, device.cu:2595-2618)
+        NEED_F(1, 1);
+        NEED_L(4, 6);
+        long long n = pl[0], ao = ll > 4 ? pl[4] : 0, yo = ll > 5 ? pl[5] : 0;
+        MemItem *A, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, ao, n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_powx(s, A->dt(), (size_t)n, PTR(A, ao), pf[0], PTR(Y, yo)));
+        m_mem.touch((long)pl[3]);
+        return 0;
+    }
+    case MCH_FN_SQRT: {
+        // [f{epsilon}], l{n,hX,hY}: y = sqrt(x + epsilon) (CudaDnn.cs:8520-8526, device.cu:2712-2728)
+        NEED_L(3, 3);
+        long long n = pl[0];
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        HIPCHK(k_sqrt(s, X->dt(), (size_t)n, X->ptr, Y->ptr, (lf > 0 && pf) ? pf[0] : 0.f));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_INVERT: {
+        // [f{numerator, denominator}], l{n,hX,hY[,xOff,yOff]} (CudaDnn.cs:8453-8459, device.cu:2624-2655)
+        NEED_L(3, 5);
+        long long n = pl[0], xo = ll > 3 ? pl[3] : 0, yo = ll > 4 ? pl[4] : 0;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        HIPCHK(k_invert(s, X->dt(), (size_t)n, PTR(X, xo), PTR(Y, yo), (lf > 0 && pf) ? pf[0] : 1.f, (lf > 1 && pf) ? pf[1] : 1.f));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_CHANNEL_MEAN: {
+        // l{count,outer,channels,inner,hX,hY[,xOff]}: y[outer*channels] = row means (CudaDnn.cs:9030-9036, device.cu:3386-3405)
+        NEED_L(6, 7);
+        long long outer = pl[1], ch = pl[2], inner = pl[3], xo = ll > 6 ? pl[6] : 0;
+        if (outer < 0 || ch < 0 || inner < 1 || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, xo, outer * ch * inner);
+        RANGE(Y, 0, outer * ch);
+        HIPCHK(k_channel_mean(s, X->dt(), (size_t)(outer * ch), (int)inner, PTR(X, xo), Y->ptr));
+        m_mem.touch((long)pl[5]);
+        return 0;
+    }
+    case MCH_FN_CHANNEL_FILLFROM:
+    case MCH_FN_CHANNEL_COPYALL:
+    case MCH_FN_CHANNEL_DUP: {
+        // l{count,outer,channels,inner,hX,hY[,dir]} (CudaDnn.cs:9086-9092, 9443-9449, 9312-9318; math.cu:7465-7481, 7630-7639, 7667-7676)
+        const bool fill = fn == MCH_FN_CHANNEL_FILLFROM;
+        NEED_L(fill ? 7 : 6, fill ? 7 : 6);
+        long long n = pl[0], outer = pl[1], ch = pl[2], inner = pl[3];
+        if (n < 0 || outer < 1 || ch < 1 || inner < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (fill && pl[6] != 0) {
+            // backward: x[i] = y[i * inner], i < outer * channels
+            RANGE(X, 0, outer * ch);
+            RANGE(Y, 0, (outer * ch - 1) * inner + 1);
+            HIPCHK(k_channel_spread(s, X->dt(), 1, (size_t)(outer * ch), (size_t)inner, 1, 1, X->ptr, Y->ptr));
+            m_mem.touch((long)pl[4]);
+            return 0;
+        }
+        RANGE(Y, 0, n);
+        if (fill) {
+            RANGE(X, 0, n > 0 ? (n - 1) / inner + 1 : 0);
+            HIPCHK(k_channel_spread(s, X->dt(), 0, (size_t)n, (size_t)inner, 1, 1, X->ptr, Y->ptr));
+        } else if (fn == MCH_FN_CHANNEL_COPYALL) {
+            RANGE(X, 0, n < ch * inner ? n : ch * inner);
+            HIPCHK(k_channel_spread(s, X->dt(), 2, (size_t)n, 1, (size_t)(ch * inner), 1, X->ptr, Y->ptr));
+        } else {
+            RANGE(X, 0, n > 0 ? ((n - 1) / (ch * inner)) * ch + ch : 0);
+            HIPCHK(k_channel_spread(s, X->dt(), 3, (size_t)n, 1, (size_t)(ch * inner), (size_t)ch, X->ptr, Y->ptr));
+        }
+        m_mem.touch((long)pl[5]);
+        return 0;
+    }
+
     case MCH_FN_MASK: {
         // f{search,replace}, l{n,maskDim,0,0,hX,hMask,hY} (device.cu:2101-2120)
         NEED_F(2, 2);

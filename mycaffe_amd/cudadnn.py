@@ -64,13 +64,23 @@ class CUDAFN:
     CUDA_AXPY = 222
     CUDA_SCAL = 224
     CUDA_SCALE = 227
+    CUDA_ADD_SCALAR = 228
     CUDA_ADD = 229
+    CUDA_SUB = 230
     CUDA_MUL = 231
+    CUDA_DIV = 233
+    CUDA_POWX = 237
+    CUDA_SQRT = 239
     CUDA_TRANSPOSE = 261
     CUDA_MASK = 264
     CUDA_MASK_BATCH = 266
     CUDA_TRANSPOSE_HW = 267
+    CUDA_INVERT = 273
+    CUDA_CHANNEL_MEAN = 287
     CUDA_CHANNEL_COPY = 300
+    CUDA_CHANNEL_FILLFROM = 301
+    CUDA_CHANNEL_COPYALL = 302
+    CUDA_CHANNEL_DUP = 303
     CUDA_EMBED_FWD = 390
     CUDA_RELU_FWD = 428
     CUDA_RELU_BWD = 429
@@ -457,6 +467,46 @@ class CudaDnn:
     def mul(self, n, hA, hB, hY, nAOff=0, nBOff=0, nYOff=0):
         """CudaDnn.cs:8154-8160."""
         self._ex2(CUDAFN.CUDA_MUL, None, [n, hA, hB, hY, nAOff, nBOff, nYOff])
+
+    def sub(self, n, hA, hB, hY, nAOff=0, nBOff=0, nYOff=0, nB=0):
+        """CudaDnn.cs:8132-8138."""
+        self._ex2(CUDAFN.CUDA_SUB, None, [n, hA, hB, hY, nAOff, nBOff, nYOff, nB])
+
+    def div(self, n, hA, hB, hY):
+        """CudaDnn.cs:8281-8287."""
+        self._ex2(CUDAFN.CUDA_DIV, None, [n, hA, hB, hY])
+
+    def add_scalar(self, n, fAlpha, hY, nYOff=0):
+        """CudaDnn.cs:8010-8016."""
+        self._ex2(CUDAFN.CUDA_ADD_SCALAR, [fAlpha], [n, 0, hY, nYOff])
+
+    def powx(self, n, hA, fAlpha, hY, nAOff=0, nYOff=0):
+        """CudaDnn.cs:8419-8425."""
+        self._ex2(CUDAFN.CUDA_POWX, [fAlpha], [n, hA, 0, hY, nAOff, nYOff])
+
+    def sqrt(self, n, hX, hY, dfEpsilon=0.0):
+        """CudaDnn.cs:8520-8526."""
+        self._ex2(CUDAFN.CUDA_SQRT, [dfEpsilon], [n, hX, hY])
+
+    def invert(self, n, hX, hY, nXOff=0, nYOff=0, dfScaleNumerator=1.0, dfScaleDenom=1.0):
+        """CudaDnn.cs:8453-8459."""
+        self._ex2(CUDAFN.CUDA_INVERT, [dfScaleNumerator, dfScaleDenom], [n, hX, hY, nXOff, nYOff])
+
+    def channel_mean(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff=0):
+        """CudaDnn.cs:9030-9036."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_MEAN, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff])
+
+    def channel_fillfrom(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, dir):
+        """CudaDnn.cs:9086-9092."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_FILLFROM, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, dir])
+
+    def channel_copyall(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY):
+        """CudaDnn.cs:9443-9449."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_COPYALL, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY])
+
+    def channel_duplicate(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY):
+        """CudaDnn.cs:9312-9318."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_DUP, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY])
 
     def mask(self, n, nMaskDim, fSearch, fReplace, hX, hMask, hY):
         """CudaDnn.cs:7850-7856."""

@@ -468,31 +468,99 @@ class MultiheadAttentionLayer:
 
 
 class LayerNormLayer:
-    """MyCaffe.layers.gpt/layers.gpt/LayerNormLayer.cs with ``enable_cuda_impl`` (reshape :153-166, forward :211-212,
-    backward :285-286): normalisation over the last axis through the LayerNorm handle (ids 970-976)."""
+    """MyCaffe.layers.gpt/layers.gpt/LayerNormLayer.cs.  ``enable_cuda_impl`` runs the LayerNorm handle (ids 970-976;
+    reshape :153-166, forward :211-212, backward :285-286); otherwise the explicit chain of :223-264 runs (channel_mean,
+    channel_fillfrom, sub, powx, channel_mean, add_scalar, sqrt, channel_fillfrom, div)."""
 
-    def __init__(self, cuda, epsilon=1e-10):
-        self.cuda, self.epsilon = cuda, epsilon
+    def __init__(self, cuda, epsilon=1e-10, enable_cuda_impl=True):
+        self.cuda, self.epsilon, self.enable_cuda_impl = cuda, epsilon, enable_cuda_impl
         self.hLayerNorm = 0
         self._shape = None
+        self.b = {n: Blob(cuda) for n in "Mu Xmu XmuSq Var Stdev StdevFull".split()}
 
     def _reshape(self, bottom):
+        nAxis = len(bottom.shape_) - 1
+        self.nCount = bottom.count()
+        self.nOuterNum, self.nChannels, self.nInnerNum = bottom.shape_[0], bottom.count(1, nAxis), bottom.count(nAxis)
         if self._shape == bottom.shape_:
             return
-        if self.hLayerNorm:
-            self.cuda.FreeLayerNorm(self.hLayerNorm)
-        nAxis = len(bottom.shape_) - 1
-        outer, channels, inner = bottom.shape_[0], bottom.count(1, nAxis), bottom.count(nAxis)
-        self.hLayerNorm = self.cuda.CreateLayerNorm(0, bottom.count(), outer, channels, inner, self.epsilon)
+        if self.enable_cuda_impl:
+            if self.hLayerNorm:
+                self.cuda.FreeLayerNorm(self.hLayerNorm)
+            self.hLayerNorm = self.cuda.CreateLayerNorm(0, self.nCount, self.nOuterNum, self.nChannels, self.nInnerNum, self.epsilon)
+        else:
+            for n in ("Xmu", "XmuSq", "StdevFull"):
+                self.b[n].ReshapeLike(bottom)
+            for n in ("Mu", "Var", "Stdev"):
+                self.b[n].Reshape(self.nOuterNum, self.nChannels, 1, 1)
         self._shape = list(bottom.shape_)
 
     def Forward(self, bottom, top):
         self._reshape(bottom)
         top.ReshapeLike(bottom)
-        self.cuda.LayerNormForward(self.hLayerNorm, bottom.gpu_data, top.gpu_data)
+        cuda, b = self.cuda, self.b
+        if self.enable_cuda_impl:
+            cuda.LayerNormForward(self.hLayerNorm, bottom.gpu_data, top.gpu_data)
+            return
+        n, o, c, i = self.nCount, self.nOuterNum, self.nChannels, self.nInnerNum
+        cuda.channel_mean(n, o, c, i, bottom.gpu_data, b["Mu"].gpu_data)
+        cuda.channel_fillfrom(n, o, c, i, b["Mu"].gpu_data, b["Xmu"].gpu_data, DIR.FWD)
+        cuda.sub(n, bottom.gpu_data, b["Xmu"].gpu_data, b["Xmu"].gpu_data)
+        cuda.powx(n, b["Xmu"].gpu_data, 2.0, b["XmuSq"].gpu_data)
+        cuda.channel_mean(n, o, c, i, b["XmuSq"].gpu_data, b["Var"].gpu_data)
+        cuda.add_scalar(o * c, self.epsilon, b["Var"].gpu_data)
+        cuda.sqrt(o * c, b["Var"].gpu_data, b["Stdev"].gpu_data)
+        cuda.channel_fillfrom(n, o, c, i, b["Stdev"].gpu_data, b["StdevFull"].gpu_data, DIR.FWD)
+        cuda.div(n, b["Xmu"].gpu_data, b["StdevFull"].gpu_data, top.gpu_data)
 
     def Backward(self, top, bottom):
+        if not self.enable_cuda_impl:
+            raise NotImplementedError("the explicit chain's backward is not mirrored")
         self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, top.gpu_diff, bottom.gpu_diff)
+
+
+class RMSNormLayer:
+    """MyCaffe.layers.gpt/layers.gpt/RMSNormLayer.cs:96-180, the layer's own chain: powx(2), channel_mean, sqrt(+eps),
+    invert, channel_duplicate, mul, and with weights channel_copyall + mul.  ``fused`` replaces the chain by the
+    single call RMSNORM_FWD (id 2002), which has no counterpart in the reference."""
+
+    def __init__(self, cuda, epsilon=1e-5, enable_weights=True, fused=False):
+        self.cuda, self.epsilon, self.enable_weights, self.fused = cuda, epsilon, enable_weights, fused
+        self.blobs = []
+        self.b = {n: Blob(cuda) for n in "Rms Rms1 Out Rms1Full".split()}
+
+    def Setup(self, bottom, weight=None):
+        nAxis = len(bottom.shape_) - 1
+        if self.enable_weights:
+            w = Blob(self.cuda, (bottom.count(nAxis),))
+            w.mutable_cpu_data = np.ones(bottom.count(nAxis), np.float32) if weight is None else weight
+            self.blobs = [w]
+
+    def Forward(self, bottom, top):
+        cuda, b = self.cuda, self.b
+        nAxis = len(bottom.shape_) - 1
+        n, inner = bottom.count(), bottom.count(nAxis)
+        channels, outer = bottom.shape_[nAxis - 1], bottom.count(0, nAxis - 1)
+        top.ReshapeLike(bottom)
+        if self.fused:
+            cuda.RmsNormForward(outer * channels, inner, bottom.gpu_data, self.blobs[0].gpu_data if self.enable_weights else 0,
+                                top.gpu_data, self.epsilon)
+            return
+        b["Rms"].Reshape(outer, channels, 1, 1)
+        b["Rms1"].Reshape(outer, channels, 1, 1)
+        b["Out"].ReshapeLike(bottom)
+        b["Rms1Full"].ReshapeLike(bottom)
+        cuda.powx(n, bottom.gpu_data, 2.0, top.gpu_data)
+        cuda.channel_mean(n, outer, channels, inner, top.gpu_data, b["Rms"].gpu_data)
+        cuda.sqrt(b["Rms"].count(), b["Rms"].gpu_data, b["Rms"].gpu_data, self.epsilon)
+        cuda.invert(b["Rms1"].count(), b["Rms"].gpu_data, b["Rms1"].gpu_data)
+        cuda.channel_duplicate(n, outer * channels, 1, inner, b["Rms1"].gpu_data, b["Rms1Full"].gpu_data)
+        cuda.mul(n, bottom.gpu_data, b["Rms1Full"].gpu_data, b["Out"].gpu_data)
+        if self.enable_weights:
+            cuda.channel_copyall(n, outer * channels, 1, inner, self.blobs[0].gpu_data, b["Out"].gpu_diff)
+            cuda.mul(n, b["Out"].gpu_diff, b["Out"].gpu_data, top.gpu_data)
+        else:
+            top.CopyFrom(b["Out"])
 
 
 class ActivationLayer:
@@ -538,21 +606,37 @@ class TransformerBlockLayer:
     forward :810-902): x + attn(ln1(x)), then + proj(act(fc(ln2(.)))).  Dropout is the identity at inference."""
 
     def __init__(self, cuda, heads, embed, block_size, activation="relu", bias_term=True, epsilon=1e-10,
-                 enable_cuda_scaled_dot_product_attention=True, training=False):
+                 enable_cuda_scaled_dot_product_attention=True, training=False, enable_llama_style_head=False, hidden_dim=0,
+                 multiple_of=64, enable_layernorm_cuda_impl=True, fused_rmsnorm=False):
         self.cuda = cuda
-        self.norm1 = LayerNormLayer(cuda, epsilon)
-        self.norm2 = LayerNormLayer(cuda, epsilon)
+        self.llama = enable_llama_style_head
+        if self.llama:
+            # RMSNorm, rotary attention without bias, SiLU-gated MLP (TransformerBlockLayer.cs:86-98, 239-247, 860-875)
+            self.norm1 = RMSNormLayer(cuda, epsilon, True, fused_rmsnorm)
+            self.norm2 = RMSNormLayer(cuda, epsilon, True, fused_rmsnorm)
+            if hidden_dim == 0:
+                hidden_dim = 2 * (4 * embed) // 3
+                hidden_dim = multiple_of * ((hidden_dim + multiple_of - 1) // multiple_of)
+        else:
+            self.norm1 = LayerNormLayer(cuda, epsilon, enable_layernorm_cuda_impl)
+            self.norm2 = LayerNormLayer(cuda, epsilon, enable_layernorm_cuda_impl)
+            hidden_dim = hidden_dim or 4 * embed
         self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention,
-                                              training=training)
-        self.fc1 = InnerProductLayer(cuda, 4 * embed, bias_term, 2)
+                                              enable_rotary_positional_embedding=self.llama, training=training)
+        self.fc1 = InnerProductLayer(cuda, hidden_dim, bias_term, 2)
+        self.fc2 = InnerProductLayer(cuda, hidden_dim, bias_term, 2) if self.llama else None
         self.proj = InnerProductLayer(cuda, embed, bias_term, 2)
         self.act = ActivationLayer(cuda, activation)
-        self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 Mlp1 MlpOut".split()}
+        self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 Mlp1 Mlp2 Mlp3 MlpOut".split()}
 
     def Setup(self, bottom, p):
         """``p``: attn_weight, attn_bias, attn_proj_weight, attn_proj_bias, fc_weight, fc_bias, proj_weight, proj_bias."""
         self.attn1.Setup(bottom, p["attn_weight"], p.get("attn_bias"), p["attn_proj_weight"], p.get("attn_proj_bias"))
         self.fc1.Setup(bottom, p["fc_weight"], p.get("fc_bias"))
+        if self.llama:
+            self.fc2.Setup(bottom, p["fc2_weight"], p.get("fc2_bias"))
+            self.norm1.Setup(bottom, p.get("rms1_weight"))
+            self.norm2.Setup(bottom, p.get("rms2_weight"))
         hidden = Blob(self.cuda, bottom.shape_[:2] + [self.fc1.N])
         self.proj.Setup(hidden, p["proj_weight"], p.get("proj_bias"))
         hidden.Dispose()
@@ -567,12 +651,20 @@ class TransformerBlockLayer:
         self.norm2.Forward(b["X"], b["Norm2"])
         self.fc1.Forward(b["Norm2"], b["Mlp1"])
         self.act.Forward(b["Mlp1"], b["Mlp1"])
-        self.proj.Forward(b["Mlp1"], b["MlpOut"])
+        blobMlp = b["Mlp1"]
+        if self.llama:
+            self.fc2.Forward(b["Norm2"], b["Mlp2"])
+            b["Mlp3"].ReshapeLike(b["Mlp1"])
+            cuda.mul(b["Mlp1"].count(), b["Mlp1"].gpu_data, b["Mlp2"].gpu_data, b["Mlp3"].gpu_data)
+            blobMlp = b["Mlp3"]
+        self.proj.Forward(blobMlp, b["MlpOut"])
         top.ReshapeLike(blobX)
         cuda.add(nCount, b["X"].gpu_data, b["MlpOut"].gpu_data, top.gpu_data)
 
     def Backward(self, top, blobX):
         """TransformerBlockLayer.cs:924-1040, CAUSAL_SELF_ATTENTION block: top.gpu_diff -> blobX.gpu_diff."""
+        if self.llama:
+            raise NotImplementedError("the RMSNorm chain's backward is not mirrored")
         b, cuda = self.b, self.cuda
         nCount = blobX.count()
         cuda.copy(nCount, top.gpu_diff, b["MlpOut"].gpu_diff)

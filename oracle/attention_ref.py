@@ -503,3 +503,16 @@ def transformer_block_gpt(x, p, heads, activation="relu", eps=1e-10, dtype=np.fl
     act = relu(fc, 0.0, dtype) if activation == "relu" else gelu(fc, activation == "gelu_bert", dtype)
     mlp = inner_product(act, p["proj_weight"], p["proj_bias"], dtype)
     return {"ln1": ln1, "attn": attn, "xb": xb, "ln2": ln2, "fc": fc, "act": act, "mlp": mlp, "y": (xb + mlp).astype(dtype)}
+
+
+def transformer_block_llama(x, p, heads, seq_len, theta=10000.0, eps=1e-5, dtype=np.float32):
+    """TransformerBlockLayer.forward with enable_llama_style_head (TransformerBlockLayer.cs:810-902): RMSNorm, causal self
+    attention with rotary q / k and no bias, xB = x + attn; y = xB + proj(silu(fc1(n)) * fc2(n)), n = RMSNorm(xB).
+    ``p``: rms1_weight, rms2_weight, attn_weight, attn_proj_weight, fc_weight, fc2_weight, proj_weight."""
+    x = np.asarray(x, dtype)
+    n1 = rmsnorm_layer(x, p["rms1_weight"], eps, dtype)
+    attn = causal_self_attention(n1, p["attn_weight"], None, p["attn_proj_weight"], None, heads, rope=(seq_len, theta), dtype=dtype)["y"]
+    xb = (x + attn).astype(dtype)
+    n2 = rmsnorm_layer(xb, p["rms2_weight"], eps, dtype)
+    h = silu(inner_product(n2, p["fc_weight"], None, dtype), dtype) * inner_product(n2, p["fc2_weight"], None, dtype)
+    return (xb + inner_product(h.astype(dtype), p["proj_weight"], None, dtype)).astype(dtype)

@@ -265,3 +265,117 @@ def test_transformer_block_backward_golden(dev, name, heads):
     assert_close(layer.b["Norm2"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_6_x_ln2.txt")), 2e-5, "grad ln2 out")
     assert_close(layer.b["Norm1"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_9_ln1.txt")), 5e-5, "grad ln1 out")
     assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(g, "grad_10_x.txt")), 5e-5, "grad x")
+
+
+def test_norm_chain_primitives_vs_numpy(dev):
+    """The elementwise / per-row ids the C# RMSNormLayer and LayerNormLayer chains call, each against its index rule."""
+    rng = np.random.default_rng(81)
+    cuda = dev.cuda
+    outer, ch, inner = 3, 5, 48
+    n = outer * ch * inner
+    x = rng.standard_normal(n).astype(np.float32)
+    x[7] = 0.0
+    hx, hy = dev.put(x), dev.zeros(n)
+    cuda.powx(n, hx, 2.0, hy)
+    assert np.array_equal(dev.get(hy), x * x)
+    cuda.powx(n, hx, 3.0, hy)
+    assert_close(dev.get(hy), x.astype(np.float64) ** 3, 1e-6, "powx 3")
+    cuda.sqrt(n, hy, hy)                                   # of negative values: NaN, as sqrtf gives
+    cuda.powx(n, hx, 2.0, hy)
+    cuda.sqrt(n, hy, hy, 0.25)
+    assert_close(dev.get(hy), np.sqrt(x.astype(np.float64) ** 2 + 0.25), 1e-6, "sqrt eps")
+    cuda.invert(n, hx, hy)
+    ref = np.where(x == 0, 0, 1.0 / np.where(x == 0, 1, x))
+    assert_close(dev.get(hy), ref, 1e-6, "invert")
+    cuda.invert(n, hx, hy, 0, 0, 3.0, 2.0)
+    assert_close(dev.get(hy), 1.5 * ref, 1e-6, "invert n/d")
+    cuda.invert(n, hx, hy, 0, 0, -1.0)
+    assert_close(dev.get(hy), -ref, 1e-6, "invert -1")
+    hm = dev.zeros(outer * ch)
+    cuda.channel_mean(n, outer, ch, inner, hx, hm)
+    assert_close(dev.get(hm), x.reshape(outer * ch, inner).astype(np.float64).mean(1), 1e-6, "channel_mean")
+    cuda.channel_fillfrom(n, outer, ch, inner, hm, hy, 0)
+    assert np.array_equal(dev.get(hy), np.repeat(dev.get(hm), inner))
+    hb = dev.zeros(outer * ch)
+    cuda.channel_fillfrom(n, outer, ch, inner, hb, hx, 1)  # backward: picks the first value of every row
+    assert np.array_equal(dev.get(hb), x.reshape(outer * ch, inner)[:, 0])
+    cuda.channel_duplicate(n, outer * ch, 1, inner, hm, hy)
+    assert np.array_equal(dev.get(hy), np.repeat(dev.get(hm), inner))
+    w = rng.standard_normal(inner).astype(np.float32)
+    hw = dev.put(w)
+    cuda.channel_copyall(n, outer * ch, 1, inner, hw, hy)
+    assert np.array_equal(dev.get(hy), np.tile(w, outer * ch))
+    d2 = rng.standard_normal((2, 3, 4)).astype(np.float32)   # duplicate with more than one channel: (num, dup, channels)
+    hd, hd2 = dev.put(d2[:, 0, :].copy()), dev.zeros(d2.size)
+    cuda.channel_duplicate(d2.size, 2, 4, 3, hd, hd2)
+    assert np.array_equal(dev.get(hd2, d2.shape), np.broadcast_to(d2[:, :1, :], d2.shape))
+    a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    b[11] = 0.0
+    ha, hb2 = dev.put(a), dev.put(b)
+    cuda.sub(n, ha, hb2, hy)
+    assert np.array_equal(dev.get(hy), a - b)
+    cuda.sub(n, ha, hb2, hy, 0, 0, 0, inner)
+    assert np.array_equal(dev.get(hy), a - np.tile(b[:inner], outer * ch))
+    cuda.div(n, ha, hb2, hy)
+    assert_close(dev.get(hy), np.where(b == 0, 0, a / np.where(b == 0, 1, b)), 1e-6, "div")
+    cuda.add_scalar(n, 0.5, ha)
+    assert np.array_equal(dev.get(ha), a + np.float32(0.5))
+    cuda.add_scalar(10, 1.0, ha, 5)
+    exp = a + np.float32(0.5)
+    exp[5:15] += 1
+    assert np.array_equal(dev.get(ha), exp)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_rmsnorm_layer_chain_vs_checker(dev, fused):
+    from mycaffe_amd.layers import RMSNormLayer
+    rng = np.random.default_rng(82)
+    x = rng.standard_normal((2, 9, 288)).astype(np.float32)
+    w = rng.standard_normal(288).astype(np.float32)
+    for weights in (True, False):
+        layer = RMSNormLayer(dev.cuda, 1e-5, weights, fused)
+        bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+        bx.mutable_cpu_data = x
+        layer.Setup(bx, w)
+        layer.Forward(bx, top)
+        assert_close(top.mutable_cpu_data, R.rmsnorm_layer(x, w if weights else None, 1e-5, np.float64), 1e-5, "rmsnorm layer")
+
+
+def test_layernorm_layer_chain_equals_handle(dev):
+    from mycaffe_amd.layers import LayerNormLayer
+    rng = np.random.default_rng(83)
+    x = (rng.standard_normal((2, 6, 96)) * 3 + 1).astype(np.float32)
+    bx = Blob(dev.cuda, x.shape)
+    bx.mutable_cpu_data = x
+    outs = []
+    for impl in (True, False):
+        top = Blob(dev.cuda)
+        LayerNormLayer(dev.cuda, 1e-5, impl).Forward(bx, top)
+        outs.append(top.mutable_cpu_data)
+    ref, _ = R.layernorm_forward(x, 96, 1e-5, np.float64)
+    assert_close(outs[0], ref, 1e-5, "handle")
+    assert_close(outs[1], ref, 1e-5, "chain")
+
+
+@pytest.mark.parametrize("fused_rmsnorm,sdpa", [(False, False), (True, True)])
+def test_transformer_block_llama_style_vs_checker(dev, fused_rmsnorm, sdpa):
+    """The Llama-style block (RMSNorm chain or the fused id, rotary attention without bias, SiLU-gated MLP) through the
+    layer mirrors, against the checker."""
+    rng = np.random.default_rng(84)
+    B, T, C, H = 2, 32, 128, 2
+    layer = TransformerBlockLayer(dev.cuda, H, C, T, "silu", False, 1e-5, sdpa, enable_llama_style_head=True, multiple_of=32,
+                                  fused_rmsnorm=fused_rmsnorm)
+    hid = layer.fc1.N
+    assert hid == 352    # 2 * (4 * 128) / 3 = 341 rounded up to a multiple of 32
+    p = {"rms1_weight": 1 + 0.1 * rng.standard_normal(C), "rms2_weight": 1 + 0.1 * rng.standard_normal(C),
+         "attn_weight": rng.standard_normal((3 * C, C)) * 0.05, "attn_proj_weight": rng.standard_normal((C, C)) * 0.05,
+         "fc_weight": rng.standard_normal((hid, C)) * 0.05, "fc2_weight": rng.standard_normal((hid, C)) * 0.05,
+         "proj_weight": rng.standard_normal((C, hid)) * 0.05}
+    p = {k: v.astype(np.float32) for k, v in p.items()}
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    ref = R.transformer_block_llama(x, p, H, T, 10000.0, 1e-5, np.float64)
+    assert_close(top.mutable_cpu_data, ref, FP32_RTOL, "llama block")

@@ -430,3 +430,36 @@ def test_transformer_block_golden(name, heads):
                    ("act", "7_x_act"), ("mlp", "8_x_c_proj"), ("y", "10_y")):
         exp = load_txt(os.path.join(d, f + ".txt"))
         assert np.abs(out[key] - exp.reshape(out[key].shape)).max() < 5e-7, f
+
+
+def test_transformer_block_llama_matches_torch_composition():
+    """The Llama-style block of the checker against torch library routines: rms_norm, linear, SDPA (causal), silu, with
+    the rotary embedding applied as a complex rotation of adjacent pairs."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(12)
+    B, T, C, H, hid = 2, 7, 24, 3, 40
+    hs = C // H
+    p = {"rms1_weight": rng.standard_normal(C), "rms2_weight": rng.standard_normal(C),
+         "attn_weight": rng.standard_normal((3 * C, C)) * 0.2, "attn_proj_weight": rng.standard_normal((C, C)) * 0.2,
+         "fc_weight": rng.standard_normal((hid, C)) * 0.2, "fc2_weight": rng.standard_normal((hid, C)) * 0.2,
+         "proj_weight": rng.standard_normal((C, hid)) * 0.2}
+    x = rng.standard_normal((B, T, C))
+    got = R.transformer_block_llama(x, p, H, T, 10000.0, 1e-5, np.float64)
+    t = {k: torch.tensor(v) for k, v in p.items()}
+    xt = torch.tensor(x)
+
+    def rope(v):    # (B,T,H,hs): pairs (2j, 2j+1) rotated by pos * theta^(-2j/hs)
+        vc = torch.view_as_complex(v.reshape(B, T, H, hs // 2, 2).contiguous())
+        ang = torch.arange(T, dtype=torch.float64)[:, None] * (10000.0 ** (-torch.arange(0, hs, 2, dtype=torch.float64) / hs))[None, :]
+        return torch.view_as_real(vc * torch.polar(torch.ones_like(ang), ang)[None, :, None, :]).reshape(B, T, H, hs)
+
+    n1 = F.rms_norm(xt, (C,), t["rms1_weight"], 1e-5)
+    q, k, v = F.linear(n1, t["attn_weight"]).split(C, dim=2)
+    q, k, v = rope(q.reshape(B, T, H, hs)), rope(k.reshape(B, T, H, hs)), v.reshape(B, T, H, hs)
+    att = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+    xb = xt + F.linear(att.transpose(1, 2).reshape(B, T, C), t["attn_proj_weight"])
+    n2 = F.rms_norm(xb, (C,), t["rms2_weight"], 1e-5)
+    want = xb + F.linear(F.silu(F.linear(n2, t["fc_weight"])) * F.linear(n2, t["fc2_weight"]), t["proj_weight"])
+    # the table frequencies are rounded to fp32 in the reference (rope.cu:535-553), hence 1e-6 and not 1e-12
+    assert np.allclose(got, want.numpy(), rtol=1e-5, atol=1e-6)
