@@ -9,6 +9,8 @@
 //                        transposed operands, column-major strided-batched gemm2),
 //                        64x64x16 LDS tiles, fp32 FMA.
 //  * gemv              : HBM-bound y = A x, one wavefront per row, 128-bit loads.
+#include <algorithm>
+
 #include "kernels.h"
 
 namespace mch {
@@ -533,9 +535,35 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
     return hipGetLastError();
 }
 
+// K = 1: the rank-1 update C[i,j] = alpha a[i] b[j] + beta C[i,j] that InnerProductLayer uses to add its bias
+// (ones (M,1) x bias (1,N), InnerProductLayer.cs:405-414): one streaming pass over C, four columns per thread
+template <typename T> __global__ void gemm_rank1_kernel(int m, int n, float alpha, const T* __restrict__ a, const T* __restrict__ b, float beta, T* C)
+{
+    const size_t total = (size_t)m * n;
+    const bool vec = (n & 3) == 0;
+    const size_t step = vec ? 4 : 1, items = vec ? total / 4 : total;
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < items; e += (size_t)blockDim.x * gridDim.x) {
+        const size_t idx = e * step;
+        const int i = (int)(idx / n), j = (int)(idx % n);
+        const float ai = alpha * ldf(a, i);
+        for (size_t q = 0; q < step; q++) {
+            float v = ai * ldf(b, j + q);
+            if (beta != 0.f) v += beta * ldf(C, idx + q);
+            stf(C, idx + q, v);
+        }
+    }
+}
+
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
                   const void* B, float beta, void* C)
 {
+    if (k == 1) {
+        const size_t items = ((size_t)m * n + 3) / 4;
+        const int g = (int)std::min<size_t>((items + 255) / 256, 256 * 16);
+        if (dt == F32) hipLaunchKernelGGL(gemm_rank1_kernel<float>, g, 256, 0, s, m, n, alpha, (const float*)A, (const float*)B, beta, (float*)C);
+        else hipLaunchKernelGGL(gemm_rank1_kernel<bf16_t>, g, 256, 0, s, m, n, alpha, (const bf16_t*)A, (const bf16_t*)B, beta, (bf16_t*)C);
+        return hipGetLastError();
+    }
     if (m <= 0 || n <= 0) return hipSuccess;
     if (k <= 0) k = 0;
     // MFMA fast path: A (m,k) and B (n,k) both k-contiguous, 16-byte aligned rows
@@ -575,6 +603,11 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
     st.bk = tB ? 1 : n;  st.bj = tB ? k : 1;   // B stored (k,n) or (n,k)
     st.ci = n;           st.cj = 1;
     st.sA = st.sB = st.sC = 0;
+    if (dt == F32 && k > 0) {
+        // the other transpose combinations (InnerProductLayer backward: weight gradient dY^T X, data gradient dY W) run on
+        // the strided fp32 MFMA kernel: row-major C = op(A) op(B) is column-major C^T = op(B)^T op(A)^T
+        return k_gemm2(s, tB, tA, n, m, k, alpha, (const float*)B, (const float*)A, beta, (float*)C, tB ? k : n, tA ? m : k, n, 0, 0, 0, 1);
+    }
     if (dt == F32)
         return launch_generic<float>(s, m, n, k, alpha, (const float*)A, (const float*)B, beta, (float*)C, st, 1);
     return launch_generic<bf16_t>(s, m, n, k, alpha, (const bf16_t*)A, (const bf16_t*)B, beta, (bf16_t*)C, st, 1);
