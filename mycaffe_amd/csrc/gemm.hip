@@ -537,19 +537,41 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
 
 // K = 1: the rank-1 update C[i,j] = alpha a[i] b[j] + beta C[i,j] that InnerProductLayer uses to add its bias
 // (ones (M,1) x bias (1,N), InnerProductLayer.cs:405-414): one streaming pass over C, four columns per thread
-template <typename T> __global__ void gemm_rank1_kernel(int m, int n, float alpha, const T* __restrict__ a, const T* __restrict__ b, float beta, T* C)
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+    __device__ static inline void load(const float* p, float (&v)[4]) { const float4 a = *(const float4*)p; v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; }
+    __device__ static inline void store(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Quad<bf16_t> {
+    __device__ static inline void load(const bf16_t* p, float (&v)[4])
+    {
+        const uint2 a = *(const uint2*)p;
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    }
+    __device__ static inline void store(bf16_t* p, const float (&v)[4]) { *(uint2*)p = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3])); }
+};
+template <typename T, bool VEC>
+__global__ void gemm_rank1_kernel(int m, int n, float alpha, const T* __restrict__ a, const T* __restrict__ b, float beta, T* C)
 {
     const size_t total = (size_t)m * n;
-    const bool vec = (n & 3) == 0;
-    const size_t step = vec ? 4 : 1, items = vec ? total / 4 : total;
+    const size_t items = VEC ? total / 4 : total;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < items; e += (size_t)blockDim.x * gridDim.x) {
-        const size_t idx = e * step;
-        const int i = (int)(idx / n), j = (int)(idx % n);
-        const float ai = alpha * ldf(a, i);
-        for (size_t q = 0; q < step; q++) {
-            float v = ai * ldf(b, j + q);
-            if (beta != 0.f) v += beta * ldf(C, idx + q);
-            stf(C, idx + q, v);
+        if (VEC) {
+            const size_t idx = e * 4;
+            const int i = (int)(idx / n), j = (int)(idx % n);
+            const float ai = alpha * ldf(a, i);
+            float bv[4], cv[4];
+            Quad<T>::load(b + j, bv);
+            if (beta != 0.f) Quad<T>::load(C + idx, cv);
+#pragma unroll
+            for (int q = 0; q < 4; q++) cv[q] = beta != 0.f ? ai * bv[q] + beta * cv[q] : ai * bv[q];
+            Quad<T>::store(C + idx, cv);
+        } else {
+            const int i = (int)(e / n), j = (int)(e % n);
+            float v = alpha * ldf(a, i) * ldf(b, j);
+            if (beta != 0.f) v += beta * ldf(C, e);
+            stf(C, e, v);
         }
     }
 }
@@ -558,10 +580,14 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
                   const void* B, float beta, void* C)
 {
     if (k == 1) {
-        const size_t items = ((size_t)m * n + 3) / 4;
+        const size_t es = dt == F32 ? 4 : 2;
+        const bool vec = n % 4 == 0 && ((((uintptr_t)B | (uintptr_t)C) & (4 * es - 1)) == 0);
+        const size_t items = vec ? (size_t)m * n / 4 : (size_t)m * n;
         const int g = (int)std::min<size_t>((items + 255) / 256, 256 * 16);
-        if (dt == F32) hipLaunchKernelGGL(gemm_rank1_kernel<float>, g, 256, 0, s, m, n, alpha, (const float*)A, (const float*)B, beta, (float*)C);
-        else hipLaunchKernelGGL(gemm_rank1_kernel<bf16_t>, g, 256, 0, s, m, n, alpha, (const bf16_t*)A, (const bf16_t*)B, beta, (bf16_t*)C);
+#define RANK1(TT, V) hipLaunchKernelGGL((gemm_rank1_kernel<TT, V>), g, 256, 0, s, m, n, alpha, (const TT*)A, (const TT*)B, beta, (TT*)C)
+        if (dt == F32) { if (vec) RANK1(float, true); else RANK1(float, false); }
+        else { if (vec) RANK1(bf16_t, true); else RANK1(bf16_t, false); }
+#undef RANK1
         return hipGetLastError();
     }
     if (m <= 0 || n <= 0) return hipSuccess;
@@ -624,15 +650,20 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
 template <bool A_IFAST, bool B_KFAST, int TI, int TJ>
 __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K, float alpha, const float* __restrict__ A,
                                                              const float* __restrict__ B, float beta, float* __restrict__ C,
-                                                             GemmStrides st)
+                                                             GemmStrides st, int splits, int kChunk)
 {
     constexpr int BK = 16, LDK = BK + 4;
     constexpr int NI = TI / 64, NJ = TJ / 64;        // 32x32 blocks per wavefront along i and j
     __shared__ __attribute__((aligned(16))) float Is[2][TI * LDK];   // A: [i][k]
     __shared__ __attribute__((aligned(16))) float Js[2][TJ * LDK];   // B: [j][k]
-    A += (size_t)blockIdx.z * st.sA;
-    B += (size_t)blockIdx.z * st.sB;
-    C += (size_t)blockIdx.z * st.sC;
+    // blockIdx.z = batch * splits + split; with splits > 1 every workgroup covers kChunk of the contraction and adds its
+    // part to C with float atomics (C holds beta * C already)
+    const int batchIdx = blockIdx.z / splits, split = blockIdx.z % splits;
+    const int kBegin = split * kChunk;
+    if (splits > 1) K = min(K, kBegin + kChunk);
+    A += (size_t)batchIdx * st.sA;
+    B += (size_t)batchIdx * st.sB;
+    C += (size_t)batchIdx * st.sC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave & 1) * (TI / 2), wj = (wave >> 1) * (TJ / 2);
     const int i0 = blockIdx.x * TI, j0 = blockIdx.y * TJ;
@@ -702,14 +733,14 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
         }
     };
 
-    const int nk = (K + BK - 1) / BK;
-    gload(0);
+    const int nk = (K - kBegin + BK - 1) / BK;
+    gload(kBegin);
     sstore(0);
     __syncthreads();
     const int fr = lane & 31, fg = (lane >> 5) * 4;
     for (int kt = 0; kt < nk; kt++) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) gload((kt + 1) * BK);
+        if (kt + 1 < nk) gload(kBegin + (kt + 1) * BK);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 8) {
             float4 fj[NJ], fi[NI];
@@ -742,11 +773,21 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
                 if (j < N) {
                     const size_t ci = (size_t)i + (size_t)j * st.cj;
                     float o = alpha * acc[a][b][v];
-                    if (beta != 0.f) o += beta * C[ci];
-                    C[ci] = o;
+                    if (splits > 1) {
+                        unsafeAtomicAdd(&C[ci], o);
+                    } else {
+                        if (beta != 0.f) o += beta * C[ci];
+                        C[ci] = o;
+                    }
                 }
             }
         }
+}
+
+template <typename T> __global__ void gemm_prescale_kernel(T* c, size_t n, float beta)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)blockDim.x * gridDim.x)
+        c[i] = beta == 0.f ? 0.f : beta * c[i];
 }
 
 template <bool A_IFAST, bool B_KFAST>
@@ -754,12 +795,28 @@ static hipError_t launch_gemm2_mfma(hipStream_t s, int M, int N, int K, float al
                                     float* C, const GemmStrides& st, int batch)
 {
     const bool si = M <= 64, sj = N <= 64;
-    dim3 grid((M + (si ? 63 : 127)) / (si ? 64 : 128), (N + (sj ? 63 : 127)) / (sj ? 64 : 128), batch);
+    const int gi = (M + (si ? 63 : 127)) / (si ? 64 : 128), gj = (N + (sj ? 63 : 127)) / (sj ? 64 : 128);
+    // Split the contraction when one batch of few tiles has a long K (weight gradients: K = batch x sequence): enough
+    // workgroups for two per CU, at least 512 of K each.  Needs a dense C (ldc == M) for the beta pre-pass.
+    int splits = 1, kChunk = K;
+    const long long tiles = (long long)gi * gj;
+    if (batch == 1 && tiles < 256 && K >= 2048 && st.cj == M) {
+        splits = (int)std::min<long long>((512 + tiles - 1) / tiles, K / 512);
+        if (splits > 1) {
+            kChunk = (((K + splits - 1) / splits) + 15) / 16 * 16;
+            splits = (K + kChunk - 1) / kChunk;
+        }
+        if (splits > 1 && beta != 1.f) {
+            const size_t cn = (size_t)M * N;
+            hipLaunchKernelGGL(gemm_prescale_kernel<float>, (int)std::min<size_t>((cn + 255) / 256, 4096), 256, 0, s, C, cn, beta);
+        }
+    }
+    dim3 grid(gi, gj, batch * splits);
     if (grid.y > 65535 || grid.z > 65535) return hipErrorInvalidValue;
-    if (si && sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
-    else if (si) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
-    else if (sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
-    else hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st);
+    if (si && sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
+    else if (si) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
+    else if (sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
+    else hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
     return hipGetLastError();
 }
 

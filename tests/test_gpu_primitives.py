@@ -219,6 +219,22 @@ def test_gemm2_strided_batched_blas_semantics(dev, tA, tB, m, n, k, batch):
         assert np.array_equal(blk[:ldc * n].reshape(n, ldc)[:, m:], C[b * sC:b * sC + ldc * n].reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
+@pytest.mark.parametrize("tA,tB", [(True, False), (False, False)])
+def test_gemm_fp32_long_contraction_few_tiles(dev, tA, tB, beta):
+    """Weight-gradient shape (InnerProductLayer.cs:445-447): few output tiles, a long contraction; the contraction is split
+    over workgroups there, so the result is checked for every beta (the accumulate case is the layer's)."""
+    rng = np.random.default_rng(45)
+    m, n, k = 192, 160, 4096
+    A = rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    C = rng.standard_normal((m, n)).astype(np.float32)
+    hA, hB, hC = dev.put(A), dev.put(B), dev.put(C)
+    dev.cuda.gemm(tA, tB, m, n, k, 0.5, hA, hB, beta, hC)
+    ref = 0.5 * ((A.T if tA else A).astype(np.float64) @ B) + beta * C
+    assert_close(dev.get(hC, (m, n)), ref, FP32_RTOL, "long K")
+
+
 def test_matmul_attention_chain_shapes(dev):
     """The two MatMul calls of the explicit attention chain (CausalSelfAttentionLayer.cs:583-603) at 64-wide heads."""
     rng = np.random.default_rng(44)
