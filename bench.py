@@ -441,7 +441,7 @@ def bench_copy(cuda, reps, warm=2):
     ms = cuda.TimeFunction(CUDAFN.CUDA_SCALE, [1.0], [n, 0, a, b, 0, 0], warm, reps)
     cuda.FreeMemory(a)
     cuda.FreeMemory(b)
-    return {"kernel": "scale_kernel<float>", "bytes_read": n * 4, "bytes_written": n * 4, "ms": round(ms, 4),
+    return {"kernel": "map_kernel<float, false, ScaleF>", "bytes_read": n * 4, "bytes_written": n * 4, "ms": round(ms, 4),
             "GBps": round(2 * n * 4 / (ms / 1e3) / 1e9, 1)}
 
 
