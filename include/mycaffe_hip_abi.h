@@ -17,6 +17,7 @@
 #ifndef MYCAFFE_HIP_ABI_H
 #define MYCAFFE_HIP_ABI_H
 
+#include <stdbool.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -63,83 +64,86 @@ enum {
     MCH_ERROR_LLM_GENERATE = 10004
 };
 
-/* ---- function ids (CudaDnnDLL/inc/FunctionIDs.h:71-551, main.h:23-40) ------ */
+/* ---- function ids (CudaDnnDLL/inc/FunctionIDs.h:71-551, main.h:23-40) ------
+ * f{...} = the float array of the call, l{...} = the 64-bit integer array (DLL_InvokeFloatEx2); ids that take no l{}
+ * go through DLL_InvokeFloat.  [..] = optional trailing values.  Handles are integers.  Each id cites the reference's
+ * unmarshalling code, whose argument order and count checks are reproduced. */
 enum {
     MCH_DLL_FREEMEM = -1,
     MCH_DLL_INITIALIZE = -2,
     MCH_DLL_CLEANUP = -3,
 
-    MCH_FN_SETDEVICE = 1,
-    MCH_FN_GETDEVICE = 3,
+    MCH_FN_SETDEVICE = 1,                   /* f{deviceId[, flags, seed]} (device.cu:772-795) */
+    MCH_FN_GETDEVICE = 3,                   /* -> f{deviceId}  */
     MCH_FN_SYNCHRONIZEDEVICE = 5,
-    MCH_FN_CREATE_MEMORYPOINTER = 16,
-    MCH_FN_FREE_MEMORYPOINTER = 17,
-    MCH_FN_ALLOCMEM_HALF = 19,
-    MCH_FN_ALLOCMEM = 20,
-    MCH_FN_FREEMEM = 21,
-    MCH_FN_GETMEM = 22,
-    MCH_FN_SETMEM = 23,
-    MCH_FN_CREATE_CUDNN = 47,
-    MCH_FN_FREE_CUDNN = 48,
-    MCH_FN_CREATE_TENSORDESC = 50,
-    MCH_FN_FREE_TENSORDESC = 51,
-    MCH_FN_SET_TENSORDESC = 52,
-    MCH_FN_CREATE_EXTENSION = 67,
-    MCH_FN_FREE_EXTENSION = 68,
-    MCH_FN_EXTENSION_RUN = 69,
-    MCH_FN_SOFTMAX_FWD = 111,
-    MCH_FN_ATTN_CREATE = 160,
-    MCH_FN_ATTN_FREE = 161,
-    MCH_FN_ATTN_SET = 162,
-    MCH_FN_ATTN_FWD = 163,
-    MCH_FN_ATTN_BWD = 164,
-    MCH_FN_SET = 200,
-    MCH_FN_COPY = 202,
-    MCH_FN_GEMM2 = 219,
-    MCH_FN_GEMM = 220,
-    MCH_FN_GEMV = 221,
-    MCH_FN_AXPY = 222,
-    MCH_FN_SCAL = 224,
-    MCH_FN_SCALE = 227,
-    MCH_FN_ADD_SCALAR = 228,
-    MCH_FN_ADD = 229,
-    MCH_FN_SUB = 230,
-    MCH_FN_MUL = 231,
-    MCH_FN_DIV = 233,
-    MCH_FN_POWX = 237,
-    MCH_FN_SQRT = 239,
-    MCH_FN_TRANSPOSE = 261,
-    MCH_FN_MASK = 264,
-    MCH_FN_MASK_BATCH = 266,
-    MCH_FN_TRANSPOSE_HW = 267,
-    MCH_FN_INVERT = 273,
-    MCH_FN_CHANNEL_MEAN = 287,
-    MCH_FN_CHANNEL_COPY = 300,
-    MCH_FN_CHANNEL_FILLFROM = 301,
-    MCH_FN_CHANNEL_COPYALL = 302,
-    MCH_FN_CHANNEL_DUP = 303,
-    MCH_FN_EMBED_FWD = 390,
-    MCH_FN_RELU_FWD = 428,
-    MCH_FN_RELU_BWD = 429,
-    MCH_FN_GELU_FWD = 600,
-    MCH_FN_GELU_BWD = 601,
-    MCH_FN_SILU_FWD = 605,
-    MCH_FN_SILU_BWD = 606,
-    MCH_FN_CREATE_LAYERNORM = 970,
-    MCH_FN_FREE_LAYERNORM = 971,
-    MCH_FN_LAYERNORM_FWD = 975,
-    MCH_FN_LAYERNORM_BWD = 976,
-    MCH_FN_CREATE_ROPE = 980,
-    MCH_FN_FREE_ROPE = 981,
-    MCH_FN_ROPE_FWD = 982,
-    MCH_FN_ROPE_BWD = 983,
+    MCH_FN_CREATE_MEMORYPOINTER = 16,       /* l{hData, offset, count} -> view handle (device.h:1000-1020) */
+    MCH_FN_FREE_MEMORYPOINTER = 17,         /* l{hView} */
+    MCH_FN_ALLOCMEM_HALF = 19,              /* as ALLOCMEM, 16-bit storage (bf16 here) */
+    MCH_FN_ALLOCMEM = 20,                   /* l{count[, stream]} [f{count, [stream,] data...}] -> handle (device.cu:854-949) */
+    MCH_FN_FREEMEM = 21,                    /* l{h} (device.cu:956-968) */
+    MCH_FN_GETMEM = 22,                     /* l{h, count(-1 = all)} -> data (device.cu:973-1022) */
+    MCH_FN_SETMEM = 23,                     /* f{h, count, [stream,] data...} l{h, count} (device.cu:1029-1091) */
+    MCH_FN_CREATE_CUDNN = 47,               /* f{[stream]} -> handle (device.h:1201-1221) */
+    MCH_FN_FREE_CUDNN = 48,                 /* f{h} */
+    MCH_FN_CREATE_TENSORDESC = 50,          /* -> handle */
+    MCH_FN_FREE_TENSORDESC = 51,            /* f{h} */
+    MCH_FN_SET_TENSORDESC = 52,             /* l{h, half, n, c, h, w[, strides x4]} (device.cu:1426-1464) */
+    MCH_FN_CREATE_EXTENSION = 67,           /* DLL_InvokeFloatEx: library path -> handle (device.h:4569-4588) */
+    MCH_FN_FREE_EXTENSION = 68,             /* f{h} */
+    MCH_FN_EXTENSION_RUN = 69,              /* f{hExt, fnIdx, args...} [+ text] (device.h:4569-4588) */
+    MCH_FN_SOFTMAX_FWD = 111,               /* f{alpha, beta} l{hCudnn, 0, hBtmDesc, hBtm, 0, hTopDesc, hTop, alg, mode} (device.h:4778-4798) */
+    MCH_FN_ATTN_CREATE = 160,               /* -> handle */
+    MCH_FN_ATTN_FREE = 161,                 /* f{h} */
+    MCH_FN_ATTN_SET = 162,                  /* f{dropout} l{hCudnn, hAttn, gpuId, training, batch, blockSize, heads, hs, seed} (device.h:2463-2485) */
+    MCH_FN_ATTN_FWD = 163,                  /* l{hCudnn, hAttn, blockSize, hQ, hK, hV, hMask, hY, batchMask[, blockSizeK]} (device.h:2488-2506, attn.cu:518-602) */
+    MCH_FN_ATTN_BWD = 164,                  /* l{hCudnn, hAttn, hQ, hdQ, hK, hdK, hV, hdV, hMask, hY, hdY} (device.h:2509-2529, attn.cu:608-661) */
+    MCH_FN_SET = 200,                       /* f{val} l{n, h, 0, idx, xOff} (device.h:6038-6061) */
+    MCH_FN_COPY = 202,                      /* l{n, hSrc, hDst, srcOff, dstOff, hStream, srcHalf, dstHalf} (device.h:6063-6095) */
+    MCH_FN_GEMM2 = 219,                     /* f{alpha, beta} l{tA, tB, m, n, k, 0, hA, hB, 0, hC, lda, ldb, ldc[, sA, sB, sC, batch]}, column-major (device.cu:1691-1726) */
+    MCH_FN_GEMM = 220,                      /* f{alpha, beta} l{tA, tB, m, n, k, 0, hA, hB, 0, hC[, aOff, bOff, cOff, groups, gA, gB, gC]}, row-major (device.cu:1636-1685) */
+    MCH_FN_GEMV = 221,                      /* f{alpha, beta} l{tA, m, n, 0, hA, hX, 0, hY[, aOff, xOff, yOff]} (device.cu:1733-1767) */
+    MCH_FN_AXPY = 222,                      /* f{alpha} l{n, 0, hX, hY[, xOff, yOff]} (device.cu:1830-1857) */
+    MCH_FN_SCAL = 224,                      /* f{alpha} l{n, 0, hX[, xOff]} (device.cu:1887-1905) */
+    MCH_FN_SCALE = 227,                     /* f{alpha} l{n, 0, hX, hY[, xOff, yOff]} (device.cu:2028-2051) */
+    MCH_FN_ADD_SCALAR = 228,                /* f{alpha} l{n, 0, hY[, yOff]} (device.cu:2183-2201) */
+    MCH_FN_ADD = 229,                       /* [f{alpha}] l{n, hA, hB, hY} (device.cu:2208-2236) */
+    MCH_FN_SUB = 230,                       /* l{n, hA, hB, hY[, aOff, bOff, yOff, nB]} (device.cu:2294-2331) */
+    MCH_FN_MUL = 231,                       /* l{n, hA, hB, hY[, aOff, bOff, yOff]} (device.cu:2398-2423) */
+    MCH_FN_DIV = 233,                       /* l{n, hA, hB, hY} (device.cu:2492-2505) */
+    MCH_FN_POWX = 237,                      /* f{alpha} l{n, hA, 0, hY[, aOff, yOff]} (device.cu:2595-2618) */
+    MCH_FN_SQRT = 239,                      /* [f{epsilon}] l{n, hX, hY} (device.cu:2712-2728) */
+    MCH_FN_TRANSPOSE = 261,                 /* l{n, hX, hY, hXCounts, hYCounts, hMapping, numAxes, hBuffer} (device.cu:3088-3107) */
+    MCH_FN_MASK = 264,                      /* f{search, replace} l{n, maskDim, 0, 0, hX, hMask, hY} (device.cu:2101-2120) */
+    MCH_FN_MASK_BATCH = 266,                /* f{search, replace} l{n, batch, maskDim, 0, 0, hX, hMask, hY} (device.cu:2125-2145) */
+    MCH_FN_TRANSPOSE_HW = 267,              /* l{n, c, h, w, hSrc, hDst} (device.cu:3110-3127) */
+    MCH_FN_INVERT = 273,                    /* [f{numerator, denominator}] l{n, hX, hY[, xOff, yOff]} (device.cu:2624-2655) */
+    MCH_FN_CHANNEL_MEAN = 287,              /* l{count, outer, channels, inner, hX, hY[, xOff]} (device.cu:3386-3405) */
+    MCH_FN_CHANNEL_COPY = 300,              /* l{count, outer, channels, blocks, inner, offset, hX, hY, dir} (device.cu:3730-3748) */
+    MCH_FN_CHANNEL_FILLFROM = 301,          /* l{count, outer, channels, inner, hX, hY, dir} (CudaDnn.cs:9086-9092, math.cu:7465-7481) */
+    MCH_FN_CHANNEL_COPYALL = 302,           /* l{count, outer, channels, inner, hX, hY} (CudaDnn.cs:9443-9449, math.cu:7630-7639) */
+    MCH_FN_CHANNEL_DUP = 303,               /* l{count, outer, channels, inner, hX, hY} (CudaDnn.cs:9312-9318, math.cu:7667-7676) */
+    MCH_FN_EMBED_FWD = 390,                 /* l{count, hBtm, hWeight, M, N, K, hTop} (CudaDnn.cs:9751, math.cu:9314-9330) */
+    MCH_FN_RELU_FWD = 428,                  /* f{negativeSlope} l{count, hBtm, hTop, 0} (device.h:4925-4940) */
+    MCH_FN_RELU_BWD = 429,                  /* f{negativeSlope} l{count, hTopDiff, hTopData, hBtmDiff, 0} (device.h:4943-4959) */
+    MCH_FN_GELU_FWD = 600,                  /* l{count, hBtm, hTop, bert} (device.h:3253-3266) */
+    MCH_FN_GELU_BWD = 601,                  /* l{count, hTopDiff, hTopData, hBtmDiff, hBtmData, bert} (device.h:3269-3316) */
+    MCH_FN_SILU_FWD = 605,                  /* l{count, hBtm, hTop} (CudaDnn.cs:10152) */
+    MCH_FN_SILU_BWD = 606,                  /* l{count, hTopDiff, hTopData, hBtmDiff, hBtmData} (CudaDnn.cs:10132-10180, device.h:3269-3316) */
+    MCH_FN_CREATE_LAYERNORM = 970,          /* f{eps} l{gpuId, count, outer, channels, inner} -> handle (device.h:4123-4147) */
+    MCH_FN_FREE_LAYERNORM = 971,            /* f{h} */
+    MCH_FN_LAYERNORM_FWD = 975,             /* l{h, hX, hY} (CudaDnn.cs:6339-6345, layernorm.cu:219-262) */
+    MCH_FN_LAYERNORM_BWD = 976,             /* l{h, hYdata, hYdiff, hXdiff} (CudaDnn.cs:6354-6360, layernorm.cu:268-312) */
+    MCH_FN_CREATE_ROPE = 980,               /* f{theta} l{sharedIdx, gpuId, count, batch, seqLen, heads, hs} -> handle (device.h:4201-4229) */
+    MCH_FN_FREE_ROPE = 981,                 /* f{h} */
+    MCH_FN_ROPE_FWD = 982,                  /* l{hRope, n, hX, hY[, freqOffset]} (device.h:4232-4255, rope.cu:785-825) */
+    MCH_FN_ROPE_BWD = 983,                  /* l{hRope, n, hXdata, hYdiff, hXdiff} (device.h:4266-4283, rope.cu:832-864) */
     MCH_FN_CREATE_BLOBLOADER = 990,       /* DLL_InvokeFloatEx: file path -> handle */
-    MCH_FN_FREE_BLOBLOADER = 991,
-    MCH_FN_BLOBLOADER_LOAD = 992,
-    MCH_FN_BLOBLOADER_RESETOFFSET = 993,
-    MCH_FN_BLOBLOADER_ADDTOOFFSET = 994,
-    MCH_QRY_DEVICE_NAME = 1000,
-    MCH_QRY_EXTENSION_STRING = 1003,
+    MCH_FN_FREE_BLOBLOADER = 991,           /* f{h} */
+    MCH_FN_BLOBLOADER_LOAD = 992,           /* l{h, count, hData, localItemOffset} (device.h:4635-4648, blobloader.cu:83-126) */
+    MCH_FN_BLOBLOADER_RESETOFFSET = 993,    /* l{h, offsetInBytes} (device.h:4651-4662) */
+    MCH_FN_BLOBLOADER_ADDTOOFFSET = 994,    /* l{h, offsetInItems} (device.h:4665-4676) */
+    MCH_QRY_DEVICE_NAME = 1000,             /* DLL_QueryString: LONG{deviceId} */
+    MCH_QRY_EXTENSION_STRING = 1003,        /* DLL_QueryStringFloatEx: LONG{hExt, fnIdx, args...} (device.h:4590-4603) */
 
     /* Ids with no counterpart in the reference: single-call replacements for
      * host-side loops of the reference's C# layers.  A maintainer adds one
