@@ -158,7 +158,22 @@ def cpu_baseline(blob, gpu_prompt, gpu_ids, budget_s=12.0):
             same = {"positions_compared": int(k), "first_mismatch": int(diff[0]) if diff.size else None}
         runs += 1
         del m
+    # the same loop on one thread, over a shorter sample (64 forced ids, then greedy to 96 positions)
+    prev = O.set_threads(1)
+    m = O.Llama(C4, blob, False)
+    t0 = time.perf_counter()
+    m.generate_greedy(np.asarray(gpu_prompt[:64]), 96)
+    one = 96 / (time.perf_counter() - t0)
+    O.set_threads(prev)
+    del m
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), "")
+    except OSError:
+        pass
     return {"value": round(tokens / dt, 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "cpu_model": model, "one_thread_tokens_per_s": round(one, 3), "one_thread_sample": "positions 0..95 of one generation",
             "sample": "%d whole generation(s) of the same workload (128 forced prompt ids, then greedy to 1024 positions; "
                       "fp32, batch 1), %d positions in %.1f s, every position counted" % (runs, tokens, dt),
             "ids_vs_gpu_first_generation": same}
@@ -253,7 +268,10 @@ def bench_decode_attention(cuda, reps, warm=5, cases=None):
                 ms = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl, warm, reps)
                 nbytes = 2.0 * n * es
                 gbs = nbytes / (ms / 1e3) / 1e9
-                out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+                # back-to-back dispatches re-read the same cache: below the 256 MB of last-level cache the figure is
+                # not an HBM rate (and the smallest cases are launch bound)
+                out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                                                    "fits_last_level_cache": bool(nbytes <= 256e6)}
                 for h in (kc, vc, src, q, y):
                     cuda.FreeMemory(h)
     if "bf16_B32_L4096" not in out:
@@ -366,7 +384,30 @@ def bench_csa_layer(cuda, reps, warm=2):
         for b in list(layer.b.values()) + [top, layer.blobMask]:
             b.Dispose()
     x.Dispose()
+    out["compiled_host"] = csa_layer_compiled_host(reps)
     return out
+
+
+def csa_layer_compiled_host(reps):
+    """The same layer forward issued by the compiled C++ host program (a child process with its own device context):
+    per-call host cost of a compiled caller, which is what the C# layer pays, instead of the Python mirror's.
+    Flops of one forward: QKV 29.0 G + causal-useful attention 25.8 G / 2 * 2 + projection 9.7 G = 51.5 G."""
+    import subprocess
+    from mycaffe_amd import build as B
+    exe = B.host_bench_path()
+    if not os.path.exists(exe):
+        return {"error": "host benchmark program not built"}
+    try:
+        r = subprocess.run([exe, os.path.join(ROOT, "mycaffe_amd", "libmycaffe_hip.so"), str(max(reps, 20))], capture_output=True, text=True, timeout=120)
+    except subprocess.TimeoutExpired:
+        return {"error": "timed out"}
+    if r.returncode != 0:
+        return {"error": r.stderr.strip()[-300:]}
+    d = json.loads(r.stdout.strip().splitlines()[-1])
+    flops = 51.5e9
+    for k in ("f32_fused_ms", "f32_explicit_ms", "bf16_fused_ms"):
+        d[k.replace("_ms", "_TFLOPs_causal_useful")] = round(flops / (d[k] / 1e3) / 1e12, 1)
+    return d
 
 
 def bench_matmul_chain(cuda, reps, warm=3):

@@ -5,8 +5,8 @@
 Outputs (next to this file, git-ignored):
     libmycaffe_hip.so          the CudaDnnDLL-compatible C ABI (include/mycaffe_hip_abi.h)
     libmycaffe_hip_llama2.so   the llama2 extension library loaded through CREATE_EXTENSION
-and, beside its source, tests/cpp/host_parity: the C++ host-side parity program built on
-include/mycaffe_hip_host.hpp (plain g++, it only dlopens the libraries).
+and, beside their sources, two C++ host programs built on include/mycaffe_hip_host.hpp (plain g++, they only
+dlopen the libraries): tests/cpp/host_parity (parity) and host_bench/csa_layer_bench (whole-layer wall clock).
 """
 import os
 import subprocess
@@ -83,6 +83,7 @@ def build(force=False, verbose=True):
         if verbose:
             print("built", out)
     built.append(build_host_program(force, verbose))
+    built.append(build_host_program(force, verbose, os.path.join(HERE, "host_bench", "csa_layer_bench.cpp"), host_bench_path()))
     return built
 
 
@@ -90,13 +91,17 @@ def host_program_path():
     return os.path.join(HERE, "..", "tests", "cpp", "host_parity")
 
 
-def build_host_program(force=False, verbose=True):
-    src = os.path.join(HERE, "..", "tests", "cpp", "host_parity.cpp")
-    out = host_program_path()
+def host_bench_path():
+    return os.path.join(HERE, "host_bench", "csa_layer_bench")
+
+
+def build_host_program(force=False, verbose=True, src=None, out=None):
+    src = src or os.path.join(HERE, "..", "tests", "cpp", "host_parity.cpp")
+    out = out or host_program_path()
     inc = os.path.join(HERE, "..", "include")
     deps = [src, os.path.join(inc, "mycaffe_hip_host.hpp"), os.path.join(inc, "mycaffe_hip_abi.h")]
     if force or _stale(out, deps):
-        subprocess.check_call([os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-o", out, src, "-ldl"])
+        subprocess.check_call([os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-I", inc, "-o", out, src, "-ldl"])
     if verbose:
         print("built", os.path.normpath(out))
     return out

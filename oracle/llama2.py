@@ -42,6 +42,8 @@ def lib():
         L = ctypes.CDLL(_LIB)
         fp = ctypes.POINTER(ctypes.c_float)
         ip = ctypes.POINTER(ctypes.c_int)
+        L.orc_set_threads.argtypes = [ctypes.c_int]
+        L.orc_set_threads.restype = ctypes.c_int
         L.orc_rmsnorm.argtypes = [fp, fp, fp, ctypes.c_int]
         L.orc_softmax.argtypes = [fp, ctypes.c_int]
         L.orc_matvec.argtypes = [fp, fp, fp, ctypes.c_int, ctypes.c_int]
@@ -119,6 +121,11 @@ def rope_pairs(q, k, fcos, fsin, pos):
     fsin = np.ascontiguousarray(fsin, np.float32)
     lib().orc_rope_pairs(nh, hs, _fp(q), _fp(k), _fp(fcos), _fp(fsin), pos * hs // 2)
     return q, k
+
+
+def set_threads(n):
+    """Limit the checker's parallel loops to ``n`` threads; returns the previous limit."""
+    return int(lib().orc_set_threads(int(n)))
 
 
 def argmax(p):

@@ -33,6 +33,9 @@
  * stand-ins; no oracle/_ref build exists for it.
  */
 #include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -50,6 +53,19 @@ typedef struct {
     float *x, *xb, *xb2, *hb, *hb2, *q, *k, *v, *att, *logits;
     float *kcache, *vcache, *fcos, *fsin;
 } OrcLlama;
+
+/* worker threads of the parallel loops below (the reference takes OpenMP's default); returns the previous limit */
+int orc_set_threads(int n)
+{
+#ifdef _OPENMP
+    int prev = omp_get_max_threads();
+    if (n > 0) omp_set_num_threads(n);
+    return prev;
+#else
+    (void)n;
+    return 1;
+#endif
+}
 
 void orc_rmsnorm(float *o, const float *x, const float *w, int n)
 {
