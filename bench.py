@@ -231,7 +231,7 @@ def bench_attention_backward(cuda, reps, warm=5):
         out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2),
                      "roofline": {"kernel": "fused causal attention backward (dQ kernel + dK/dV kernel)", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
-                                  "traffic": None}}
+                                  "traffic": recorded_traffic("attn_bwd_" + name)}}
         for h in (q, k, v, dy, y, dq, dk, dv):
             cuda.FreeMemory(h)
     cuda.FreeMemory(mask)
@@ -331,7 +331,9 @@ def bench_gemm(cuda, reps):
             rgl = [0, 1, M, N, K, 0, a, w, 0, c]
             ms = cuda.TimeFunction(CUDAFN.CUDA_GEMM, [1.0, 0.0], rgl, 3, reps)
             tf = 2.0 * M * N * K / (ms / 1e3) / 1e12
-            out["%s_%s" % (name, tag)] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS[name], 4)}
+            out["%s_%s" % (name, tag)] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS[name], 4),
+                                          "algorithmic_bytes": (M * K + N * K + M * N) * (2 if half else 4),
+                                          "traffic": recorded_traffic("gemm_%s_%s" % (tag, name))}
             for h in (a, w, c):
                 cuda.FreeMemory(h)
     # InnerProductLayer backward of the QKV layer (fp32): bias update of the forward pass (K = 1), data gradient
@@ -438,7 +440,8 @@ def bench_matmul_chain(cuda, reps, warm=3):
 
 def bench_block_ops(cuda, reps, warm=3):
     """The per-block elementwise ops at the GPT-2 shape of the prefill benchmark (8192 rows x 768, MLP width 3072):
-    LayerNorm handle forward / backward, GELU forward / backward.  HBM bound: algorithmic bytes = tensors read + written."""
+    LayerNorm handle forward / backward, GELU forward / backward, and the softmax (forward, gradient) of the explicit
+    attention chain.  HBM bound: algorithmic bytes = tensors read + written."""
     from mycaffe_amd.cudadnn import CUDAFN
     rows, C = 8192, 768
     out = {}
@@ -468,6 +471,21 @@ def bench_block_ops(cuda, reps, warm=3):
             res[key] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
         for hh in (x, y, dy, dx):
             cuda.FreeMemory(hh)
+        # softmax of the explicit attention chain's score tensor (B*H*T rows of T = 1024 values) and its gradient
+        srows, slen = 8 * 12 * 1024, 1024
+        n = srows * slen
+        x, y, dy = (cuda.AllocMemory(n, bHalfSize=half) for _ in range(3))
+        hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+        cuda.SetTensorDesc(d, srows, slen, 1, 1, half)
+        for key, fn, rgl, tensors in (("softmax_fwd_98304x1024", CUDAFN.SOFTMAX_FWD, [hc, 0, d, x, 0, d, y, 1, 0], 2),
+                                      ("softmax_bwd_98304x1024", CUDAFN.SOFTMAX_BWD, [hc, 0, d, y, d, dy, 0, d, x, 1, 0], 3)):
+            ms = cuda.TimeFunction(fn, [1.0, 0.0], rgl, warm, max(4, reps // 4))
+            gbs = tensors * n * es / (ms / 1e3) / 1e9
+            res[key] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+        cuda.FreeTensorDesc(d)
+        cuda.FreeCuDNN(hc)
+        for hh in (x, y, dy):
+            cuda.FreeMemory(hh)
         out[name] = res
     return out
 
@@ -488,8 +506,9 @@ def bench_copy(cuda, reps, warm=2):
 
 def counter_pass(cuda, path):
     """A short run for hardware-counter collection (rocprofv3 --pmc serialises and slows every dispatch):
-    two eager decode steps at position 512, two dispatches each of the fused prefill attention (bf16, fp32),
-    the decode attention at batch 32 / L 4096 (bf16, fp32) and the 256 MiB copy that calibrates the counters."""
+    two eager decode steps at position 512, a few dispatches each of the fused prefill attention and its backward pass
+    (bf16, fp32), the decode attention at batch 32 / L 4096 (bf16, fp32), the layer GEMMs and the 256 MiB copy that
+    calibrates the counters."""
     from mycaffe_amd.llm_inference import LlmInference
     inf = LlmInference(cuda)
     inf.Initialize(fTemperature=0.0)
@@ -504,6 +523,10 @@ def counter_pass(cuda, path):
     out["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 2, 0)
     log("counter pass: decode attention")
     out["decode_attention_H32x128"] = bench_decode_attention(cuda, 2, 0, cases=(("bf16", 32, 4096), ("f32", 32, 4096)))
+    log("counter pass: attention backward")
+    out["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 2, 0)
+    log("counter pass: gemm")
+    out["gemm_M8192"] = bench_gemm(cuda, 2)
     return out
 
 

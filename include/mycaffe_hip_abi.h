@@ -92,6 +92,7 @@ enum {
     MCH_FN_FREE_EXTENSION = 68,             /* f{h} */
     MCH_FN_EXTENSION_RUN = 69,              /* f{hExt, fnIdx, args...} [+ text] (device.h:4569-4588) */
     MCH_FN_SOFTMAX_FWD = 111,               /* f{alpha, beta} l{hCudnn, 0, hBtmDesc, hBtm, 0, hTopDesc, hTop, alg, mode} (device.h:4778-4798) */
+    MCH_FN_SOFTMAX_BWD = 112,               /* f{alpha, beta} l{hCudnn, 0, hTopDataDesc, hTopData, hTopDiffDesc, hTopDiff, 0, hBtmDiffDesc, hBtmDiff, alg, mode} (device.h:4801-4823) */
     MCH_FN_ATTN_CREATE = 160,               /* -> handle */
     MCH_FN_ATTN_FREE = 161,                 /* f{h} */
     MCH_FN_ATTN_SET = 162,                  /* f{dropout} l{hCudnn, hAttn, gpuId, training, batch, blockSize, heads, hs, seed} (device.h:2463-2485) */

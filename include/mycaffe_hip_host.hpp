@@ -353,6 +353,12 @@ public:
         ex2(MCH_FN_SOFTMAX_FWD, {1.f, 0.f}, {hCuDnn, 0, hBottomDesc, hBottom, 0, hTopDesc, hTop, alg, mode});
     }
 
+    void SoftmaxBackward(long hCuDnn, long hTopDataDesc, long hTopData, long hTopDiffDesc, long hTopDiff, long hBottomDiffDesc, long hBottomDiff,
+                         int alg = 1, int mode = 1)   // :4941
+    {
+        ex2(MCH_FN_SOFTMAX_BWD, {1.f, 0.f}, {hCuDnn, 0, hTopDataDesc, hTopData, hTopDiffDesc, hTopDiff, 0, hBottomDiffDesc, hBottomDiff, alg, mode});
+    }
+
     // ---- attention handle (CudaDnn.cs:5614-5701)
     long CreateAttn() { return (long)m_cuda.RunFloat(m_hKernel, MCH_FN_ATTN_CREATE, {}).at(0); }
     void FreeAttn(long h) { m_cuda.RunFloat(m_hKernel, MCH_FN_ATTN_FREE, {(float)h}); }

@@ -515,9 +515,12 @@ template <typename T> __global__ void softmax_strided_kernel(const T* x, T* y, s
     }
 }
 
+static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm);
+
 hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm)
 {
     if (outer == 0 || len <= 0 || inner <= 0) return hipSuccess;
+    if (inner == 1 && softmax_fwd_wave_launch(s, dt, x, y, outer, len, logsm)) return hipGetLastError();
     if (inner == 1) {
         if (outer > 0x7fffffffu) return hipErrorInvalidValue;
         DISPATCH_DT(dt, hipLaunchKernelGGL(softmax_rows_kernel<T>, (int)outer, TPB, 0, s, (const T*)x, (T*)y, len, logsm));
@@ -771,6 +774,146 @@ hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const v
     else DISPATCH_DT(dt, hipLaunchKernelGGL(layernorm_bwd_kernel<T>, rows, TPB, 0, s, rows, inner, (const T*)y, (const T*)dy, (T*)dx,
                                             stdev, bump));
 #undef LN_BWD
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Softmax gradient (cudnnSoftmaxBackward as called from SoftmaxLayer.cs:359-367): per series of `len` values
+//   accurate / fast : dx = (dy - sum(dy * y)) * y
+//   log             : dx = dy - exp(y) * sum(dy)
+// inner == 1 and len % 4 == 0, len <= 2048: one wavefront per row, the row kept in registers between the two passes.
+// Forward pass of the same shape class: one wavefront per row, max, exp and sum on the registers that hold the row.
+template <typename T, int R>
+__global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int len, const T* x, T* y, bool logsm)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = len >> 2;
+    const T* xr = x + row * len;
+    T* yr = y + row * len;
+    float v[R][4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + r * 64;
+        if (c < chunks) {
+            Vec4<T>::load(xr + 4 * c, v[r]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) mx = fmaxf(mx, v[r][i]);
+        }
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (lane + r * 64 < chunks) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float d = v[r][i] - mx;
+                const float e = expf(d);
+                sum += e;
+                v[r][i] = logsm ? d : e;
+            }
+        }
+    }
+    sum = wave_sum(sum);
+    const float ls = logf(sum);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + r * 64;
+        if (c < chunks) {
+            float o[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = logsm ? v[r][i] - ls : v[r][i] / sum;
+            Vec4<T>::store(yr + 4 * c, o);
+        }
+    }
+}
+
+static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm)
+{
+    const int R = layernorm_wave_chunks(len, x, y, y, dt == F32 ? 4 : 2);
+    if (R == 0 || (rows + 3) / 4 > 0x7fffffffu) return false;
+    const int g = (int)((rows + 3) / 4);
+#define SM_FWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((softmax_fwd_wave_kernel<T, RR>), g, 256, 0, s, rows, len, (const T*)x, (T*)y, logsm))
+    if (R == 1) SM_FWD(1);
+    else if (R == 2) SM_FWD(2);
+    else if (R == 4) SM_FWD(4);
+    else SM_FWD(8);
+#undef SM_FWD
+    return true;
+}
+
+template <typename T, int R>
+__global__ __launch_bounds__(256) void softmax_bwd_wave_kernel(size_t rows, int len, const T* y, const T* dy, T* dx, bool logsm)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = len >> 2;
+    const T* yr = y + row * len;
+    const T* gr = dy + row * len;
+    T* xr = dx + row * len;
+    float yv[R][4], gv[R][4];
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + r * 64;
+        if (c < chunks) {
+            Vec4<T>::load(yr + 4 * c, yv[r]);
+            Vec4<T>::load(gr + 4 * c, gv[r]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) sum += logsm ? gv[r][i] : gv[r][i] * yv[r][i];
+        }
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int c = lane + r * 64;
+        if (c < chunks) {
+            float o[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = logsm ? gv[r][i] - __expf(yv[r][i]) * sum : (gv[r][i] - sum) * yv[r][i];
+            Vec4<T>::store(xr + 4 * c, o);
+        }
+    }
+}
+
+// any (outer, len, inner): one workgroup per series, two passes over global memory
+template <typename T>
+__global__ void softmax_bwd_kernel(int len, int inner, const T* y, const T* dy, T* dx, bool logsm)
+{
+    __shared__ float red[4];
+    const size_t o = blockIdx.x / inner, in = blockIdx.x % inner;
+    const size_t base = o * (size_t)len * inner + in;
+    float sum = 0.f;
+    for (int l = threadIdx.x; l < len; l += TPB) {
+        const float g = ld(dy, base + (size_t)l * inner);
+        sum += logsm ? g : g * ld(y, base + (size_t)l * inner);
+    }
+    sum = block_sum<4>(sum, red);
+    for (int l = threadIdx.x; l < len; l += TPB) {
+        const size_t i = base + (size_t)l * inner;
+        const float g = ld(dy, i), v = ld(y, i);
+        st(dx, i, logsm ? g - expf(v) * sum : (g - sum) * v);
+    }
+}
+
+hipError_t k_softmax_bwd(hipStream_t s, DType dt, const void* y, const void* dy, void* dx, size_t outer, int len, int inner, bool logsm)
+{
+    if (outer == 0 || len <= 0 || inner <= 0) return hipSuccess;
+    const int R = inner == 1 ? layernorm_wave_chunks(len, y, dy, dx, dt == F32 ? 4 : 2) : 0;
+    const size_t series = outer * (size_t)inner;
+    if (series > 0x7fffffffu) return hipErrorInvalidValue;
+    const int g = (int)((outer + 3) / 4);
+#define SM_BWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((softmax_bwd_wave_kernel<T, RR>), g, 256, 0, s, outer, len, (const T*)y, (const T*)dy, (T*)dx, logsm))
+    if (R == 1) SM_BWD(1);
+    else if (R == 2) SM_BWD(2);
+    else if (R == 4) SM_BWD(4);
+    else if (R == 8) SM_BWD(8);
+    else DISPATCH_DT(dt, hipLaunchKernelGGL(softmax_bwd_kernel<T>, (int)series, TPB, 0, s, len, inner, (const T*)y, (const T*)dy, (T*)dx, logsm));
+#undef SM_BWD
     return hipGetLastError();
 }
 

@@ -345,7 +345,7 @@ template <> struct BigTraits<float> {
 template <typename T, int WM, int WN, int OCC>
 __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
                                                                const T* __restrict__ B, float beta, T* __restrict__ C, int tilesN,
-                                                               int tilesTotal)
+                                                               int tilesTotal, int bandRows, int colBlock)
 {
     typedef BigTraits<T> TR;
     constexpr int E = TR::E;
@@ -363,7 +363,16 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     T* Bs = smem + 2 * BM * LDK;         // [2][BN * LDK]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int per = (tilesTotal + 7) / 8;
-    const int tile = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+    int tile = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+    if (colBlock > 0) {
+        // The XCD's band of bandRows tile rows is walked in blocks of colBlock tile columns, so that the tiles in
+        // flight on the XCD at one time share few enough A and B rows for its L2 to hold them.
+        const int i = (int)(blockIdx.x / 8), nb = (tilesN + colBlock - 1) / colBlock;
+        const int blk = min(i / (bandRows * colBlock), nb - 1);
+        const int rem = i - blk * bandRows * colBlock;
+        const int width = blk == nb - 1 ? tilesN - blk * colBlock : colBlock;
+        tile = ((int)(blockIdx.x % 8) * bandRows + rem / width) * tilesN + blk * colBlock + rem % width;
+    }
     if (tile >= tilesTotal) return;
     const int m0 = (tile / tilesN) * BM, n0 = (tile % tilesN) * BN;
     const int wm = (wave >> 1) * (32 * WM), wn = (wave & 1) * (32 * WN);
@@ -530,8 +539,20 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
         if (e != hipSuccess) return e;
         attr = true;
     }
+    // Bands of whole tile rows per XCD (tm divisible by 8): pick the column block so that the rows of A and B behind
+    // one block of tiles stay under 3 MB of the XCD's 4 MB L2; 0 keeps the plain row-major walk of the band.
+    int bandRows = 0, colBlock = 0;
+    if (tm % 8 == 0 && tn > 1) {
+        bandRows = tm / 8;
+        const double rowBytes = 64.0 * WM * k * sizeof(T), colBytes = 64.0 * WN * k * sizeof(T), budget = 3.0 * 1024 * 1024;
+        const int fit = (int)((budget - bandRows * rowBytes) / colBytes);
+        if (fit >= 1 && fit < tn) {
+            const int nb = (tn + fit - 1) / fit;
+            colBlock = (tn + nb - 1) / nb;   // equal-width blocks
+        }
+    }
     hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
-                       (T*)C, tn, (int)total);
+                       (T*)C, tn, (int)total, bandRows, colBlock);
     return hipGetLastError();
 }
 

@@ -55,6 +55,8 @@ hipError_t k_channel_copy(hipStream_t s, DType dt, size_t n, int channels, int b
 hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, const void* w, int N, void* top);
 // softmax over `len` for outer x inner independent series; element (o, l, i) at (o*len + l)*inner + i
 hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm);
+// gradient with respect to the softmax input from the output y and its gradient dy (dx may alias dy)
+hipError_t k_softmax_bwd(hipStream_t s, DType dt, const void* y, const void* dy, void* dx, size_t outer, int len, int inner, bool logsm);
 // adjacent-pair rotary embedding with the CudaDnnDLL index rule; x == y allowed
 hipError_t k_rope(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* fcos, const float* fsin,
                   int seqLen, int heads, int hs, int tableOff, bool grad = false);

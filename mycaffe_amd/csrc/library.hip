@@ -1205,6 +1205,45 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
+    case MCH_FN_SOFTMAX_BWD: {
+        // f{alpha,beta}, l{hCudnn,0,hTopDataDesc,hTopData,hTopDiffDesc,hTopDiff,0,hBtmDiffDesc,hBtmDiff,alg,mode}
+        // (CudaDnn.cs:4941-4947, device.h:4801-4823)
+        NEED_F(2, 2);
+        NEED_L(11, 11);
+        if (!m_cudnn.get((long)pl[0])) return MCH_ERROR_PARAM_NULL;
+        TensorDesc* yd = m_tdesc.get((long)pl[2]);
+        TensorDesc* gd = m_tdesc.get((long)pl[4]);
+        TensorDesc* bd = m_tdesc.get((long)pl[7]);
+        if (!yd || !gd || !bd) return MCH_ERROR_PARAM_NULL;
+        if (pf[0] != 1.f || pf[1] != 0.f) { last_detail = "softmax supports alpha=1, beta=0 only"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        int alg = (int)pl[9], mode = (int)pl[10];
+        if (alg < 0 || alg > 2 || mode < 0 || mode > 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        for (TensorDesc* d : {gd, bd}) {
+            if (d->n != yd->n || d->c != yd->c || d->h != yd->h || d->w != yd->w) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        for (TensorDesc* d : {yd, gd, bd}) {
+            if (!(d->sw == 1 && d->sh == d->w && d->sc == d->h * d->w && d->sn == d->c * d->h * d->w)) {
+                last_detail = "softmax needs fully packed NCHW descriptors";
+                return MCH_ERROR_NOT_IMPLEMENTED;
+            }
+        }
+        MemItem *Y, *G, *X;
+        ERRCHK(mem((long)pl[3], &Y));
+        ERRCHK(mem((long)pl[5], &G));
+        ERRCHK(mem((long)pl[8], &X));
+        if (Y->half != G->half || Y->half != X->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        long long total = (long long)yd->n * yd->c * yd->h * yd->w;
+        RANGE(Y, 0, total);
+        RANGE(G, 0, total);
+        RANGE(X, 0, total);
+        size_t outer = yd->n;
+        int len = mode == 0 ? yd->c * yd->h * yd->w : yd->c;
+        int inner = mode == 0 ? 1 : yd->h * yd->w;
+        HIPCHK(k_softmax_bwd(s, Y->dt(), Y->ptr, G->ptr, X->ptr, outer, len, inner, alg == 2));
+        m_mem.touch((long)pl[8]);
+        return 0;
+    }
+
     // ---- attention -------------------------------------------------------------
     case MCH_FN_ATTN_CREATE: {
         long h;

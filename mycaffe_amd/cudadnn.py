@@ -51,6 +51,7 @@ class CUDAFN:
     FREE_EXTENSION = 68
     EXTENSION_RUN = 69
     SOFTMAX_FWD = 111
+    SOFTMAX_BWD = 112
     CUDA_ATTN_CREATE = 160
     CUDA_ATTN_FREE = 161
     CUDA_ATTN_SET = 162
@@ -598,6 +599,11 @@ class CudaDnn:
     def SoftmaxForward(self, hCuDnn, alg, mode, fAlpha, hBottomDataDesc, hBottomData, fBeta, hTopDataDesc, hTopData):
         """CudaDnn.cs:4919-4925."""
         self._ex2(CUDAFN.SOFTMAX_FWD, [fAlpha, fBeta], [hCuDnn, 0, hBottomDataDesc, hBottomData, 0, hTopDataDesc, hTopData, alg, mode])
+
+    def SoftmaxBackward(self, hCuDnn, alg, mode, fAlpha, hTopDataDesc, hTopData, hTopDiffDesc, hTopDiff, fBeta, hBottomDiffDesc, hBottomDiff):
+        """CudaDnn.cs:4941-4947."""
+        self._ex2(CUDAFN.SOFTMAX_BWD, [fAlpha, fBeta],
+                  [hCuDnn, 0, hTopDataDesc, hTopData, hTopDiffDesc, hTopDiff, 0, hBottomDiffDesc, hBottomDiff, alg, mode])
 
     # ---- attention -------------------------------------------------------------------------
     def CreateAttn(self):

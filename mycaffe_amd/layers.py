@@ -96,8 +96,9 @@ class Blob:
         else:
             self.cuda.copy(self.count(), src.gpu_data, self.gpu_data)
 
-    def MatMul(self, blobA, blobB, bReshape=False, bTransA=False, bTransB=False, dfScale=1.0):
-        """Blob.cs:4229-4269: batched row-major matmul over the two leading axes."""
+    def MatMul(self, blobA, blobB, bReshape=False, bTransA=False, bTransB=False, dfScale=1.0, bADiff=False, bBDiff=False,
+               bCDiff=False, bAccumulate=False):
+        """Blob.cs:4229-4269: batched row-major matmul over the two leading axes; the flags pick the diff side of each blob."""
         outer = blobA.count(0, 2)
         m = blobA.shape(3) if bTransA else blobA.shape(2)
         n = blobB.shape(2) if bTransB else blobB.shape(3)
@@ -107,10 +108,23 @@ class Blob:
             self.Reshape(*shape)
         elif self.shape_ != shape:
             raise ValueError("This (resulting) blob does not have the correct shape! Expected %s" % shape)
-        self.cuda.matmul(outer, m, n, k, blobA.gpu_data, blobB.gpu_data, self.gpu_data, dfScale, bTransA, bTransB)
+        hA = blobA.gpu_diff if bADiff else blobA.gpu_data
+        hB = blobB.gpu_diff if bBDiff else blobB.gpu_data
+        hC = self.gpu_diff if bCDiff else self.gpu_data
+        self.cuda.matmul(outer, m, n, k, hA, hB, hC, dfScale, bTransA, bTransB, bAccumulate)
+
+    def MatMulGrad(self, blobA, blobB, dfScale=1.0, bAccumulate=False):
+        """Blob.cs:4304-4311: from this blob's diff, A.diff = dC B^T and B.diff = A^T dC."""
+        if dfScale != 1.0:
+            self.scale_diff(dfScale)
+        blobA.MatMul(self, blobB, False, False, True, 1.0, True, False, True, bAccumulate)
+        blobB.MatMul(blobA, self, False, True, False, 1.0, False, True, True, bAccumulate)
 
     def scale_data(self, df):
         self.cuda.scal(self.count(), df, self.gpu_data)
+
+    def scale_diff(self, df):
+        self.cuda.scal(self.count(), df, self.gpu_diff)
 
     def Dispose(self):
         if self.gpu_data:
@@ -238,6 +252,12 @@ class SoftmaxLayer:
         self.cuda.SetTensorDesc(self.hTopDesc, nN, nK, nH, 1, top.half)
         self.cuda.SoftmaxForward(self.hCudnn, SOFTMAX_ALGORITHM.ACCURATE, mode, 1.0, self.hBottomDesc, bottom.gpu_data, 0.0,
                                  self.hTopDesc, top.gpu_data)
+        self._mode = mode
+
+    def Backward(self, top, bottom):
+        """SoftmaxLayer.cs:359-367: bottom.diff from top.data and top.diff (descriptors as set by Forward)."""
+        self.cuda.SoftmaxBackward(self.hCudnn, SOFTMAX_ALGORITHM.ACCURATE, self._mode, 1.0, self.hTopDesc, top.gpu_data, self.hTopDesc,
+                                  top.gpu_diff, 0.0, self.hBottomDesc, bottom.gpu_diff)
 
 
 class CausalSelfAttentionLayer:
@@ -344,18 +364,24 @@ class CausalSelfAttentionLayer:
         self.c_proj.Forward(b["Y"], top)
 
     def Backward(self, top, blobX):
-        """CausalSelfAttentionLayer.cs:641-747 with the fused attention handle: top.gpu_diff -> blobX.gpu_diff, parameter
-        gradients accumulate in the InnerProduct weight diffs.  The handle's backward call gets mask handle 0, as there."""
-        if not self.enable_sdpa:
-            raise NotImplementedError("the explicit chain's backward (softmax gradient) is not mirrored")
+        """CausalSelfAttentionLayer.cs:641-747: top.gpu_diff -> blobX.gpu_diff, parameter gradients accumulate in the
+        InnerProduct weight diffs.  Fused handle: its backward call gets mask handle 0, as there.  Explicit chain: the
+        two MatMulGrad calls around the softmax gradient (no dropout)."""
         b, cuda = self.b, self.cuda
         B, T, C = blobX.shape_[:3]
         self.c_proj.Backward(top, b["Y"])
         b["Y"].Reshape(*self._y_shape)
         self.transpose.Backward(b["Y"], b["Work"])
         b["Y"].CopyFrom(b["Work"], True, True)
-        cuda.AttnScaledDotProductBackward(self.hCudnn, self.hAttn, b["Qt"].gpu_data, b["Qt"].gpu_diff, b["Kt"].gpu_data,
-                                          b["Kt"].gpu_diff, b["Vt"].gpu_data, b["Vt"].gpu_diff, 0, b["Y"].gpu_data, b["Y"].gpu_diff)
+        if self.enable_sdpa:
+            cuda.AttnScaledDotProductBackward(self.hCudnn, self.hAttn, b["Qt"].gpu_data, b["Qt"].gpu_diff, b["Kt"].gpu_data,
+                                              b["Kt"].gpu_diff, b["Vt"].gpu_data, b["Vt"].gpu_diff, 0, b["Y"].gpu_data, b["Y"].gpu_diff)
+        else:
+            # att' = y' @ v^T, vt' = att^T @ y'; softmax gradient; qt' = att' @ kt, kt1' = qt^T @ att' (scaled)
+            b["Y"].MatMulGrad(b["AttB"], b["Vt"])
+            self.softmax.Backward(b["AttB"], b["AttA"])
+            b["AttA"].MatMulGrad(b["Qt"], b["Kt1"], 1.0 / math.sqrt(self.nSize))
+            self.transposeQ.Backward(b["Kt1"], b["Kt"])
         self.transpose.Backward(b["Kt"], b["K"])
         self.transpose.Backward(b["Qt"], b["Q"])
         self.transpose.Backward(b["Vt"], b["V"])

@@ -173,6 +173,16 @@ def softmax_lastaxis(x, dtype=np.float32):
     return (e / e.sum(axis=-1, keepdims=True)).astype(dtype)
 
 
+def softmax_backward(y, dy, axis=-1, log=False, dtype=np.float32):
+    """Gradient with respect to the softmax input along ``axis`` from the output y and its gradient dy
+    (cudnnSoftmaxBackward as SoftmaxLayer.cs:359-367 calls it): (dy - sum(dy * y)) * y, or, for the log form,
+    dy - exp(y) * sum(dy)."""
+    y, dy = np.asarray(y, dtype), np.asarray(dy, dtype)
+    if log:
+        return (dy - np.exp(y) * dy.sum(axis=axis, keepdims=True)).astype(dtype)
+    return ((dy - (dy * y).sum(axis=axis, keepdims=True)) * y).astype(dtype)
+
+
 def silu(x, dtype=np.float32):
     """x * sigmoid(x) (math.cu:11699-11707)."""
     x = np.asarray(x, dtype)

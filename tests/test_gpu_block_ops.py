@@ -223,16 +223,18 @@ def _csa_params(d):
     return [load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias")]
 
 
+@pytest.mark.parametrize("sdpa", [True, False])
 @pytest.mark.parametrize("name,heads", [("gpt-pico-csa", 1), ("gpt-pico-csa3", 3), ("gpt-pico-csa3B", 3), ("gpt-pico-csaB", 1)])
-def test_causal_self_attention_layer_backward_golden(dev, name, heads):
+def test_causal_self_attention_layer_backward_golden(dev, name, heads, sdpa):
     """Forward + backward of the layer through the C ABI against the reference's dump of the same layer: grad_y in, grad_x
-    out, with the gradients of q / k / v checked on the way."""
+    out, with the gradients of q / k / v checked on the way; with the fused attention handle and with the layer's default
+    chain (MatMul gradients around the softmax gradient, id 112)."""
     from mycaffe_amd.layers import CausalSelfAttentionLayer
     d = os.path.join(GOLDEN, name)
     g = os.path.join(d, "iter_0")
     x = load_txt(os.path.join(d, "x.txt"))
     B, T, C = x.shape
-    layer = CausalSelfAttentionLayer(dev.cuda, heads, C, T, training=True)
+    layer = CausalSelfAttentionLayer(dev.cuda, heads, C, T, True, sdpa, training=True)
     bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
     bx.mutable_cpu_data = x
     layer.Setup(bx, *_csa_params(d))
@@ -246,15 +248,16 @@ def test_causal_self_attention_layer_backward_golden(dev, name, heads):
     assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(g, "grad_x.txt")), 2e-5, "grad x")
 
 
+@pytest.mark.parametrize("sdpa", [True, False])
 @pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3B", 3)])
-def test_transformer_block_backward_golden(dev, name, heads):
+def test_transformer_block_backward_golden(dev, name, heads, sdpa):
     d = os.path.join(GOLDEN, name)
     g = os.path.join(d, "iter_0")
     p = {k: load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias",
                                                              "fc_weight", "fc_bias", "proj_weight", "proj_bias")}
     x = load_txt(os.path.join(d, "1_x.txt"))
     B, T, C = x.shape
-    layer = TransformerBlockLayer(dev.cuda, heads, C, T, "relu", True, 1e-10, True, training=True)
+    layer = TransformerBlockLayer(dev.cuda, heads, C, T, "relu", True, 1e-10, sdpa, training=True)
     bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
     bx.mutable_cpu_data = x
     layer.Setup(bx, p)

@@ -347,10 +347,60 @@ def test_transpose_head_split_and_generic(dev, half):
     assert np.array_equal(dev.get(hb2, (3, 2, 45, 70)), big.transpose(0, 1, 3, 2))
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_softmax_backward_through_tensor_descriptors(dev, half):
+    """Id 112 against the checker: row lengths on the one-wavefront path (multiples of four up to 2048) and off it,
+    channel mode with an inner axis, the log form, and the gradient written over dy."""
+    rng = np.random.default_rng(18)
+    hc = dev.cuda.CreateCuDNN()
+    tol = BF16_RTOL if half else FP32_RTOL
+    d = dev.cuda.CreateTensorDesc()
+    for rows, length in [(24, 200), (9, 1024), (3, 2048), (7, 3000), (5, 1), (6, 37), (130, 64)]:
+        y = bf16_round(R.softmax_lastaxis((rng.standard_normal((rows, length)) * 3).astype(np.float32)))
+        dy = bf16_round(rng.standard_normal((rows, length)).astype(np.float32))
+        hy, hg, hx = dev.put(y, half), dev.put(dy, half), dev.zeros(y.size, half)
+        dev.cuda.SetTensorDesc(d, rows, length, 1, 1, half)
+        dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hg, 0.0, d, hx)
+        assert_close(dev.get(hx, y.shape), R.softmax_backward(y, dy, dtype=np.float64), tol, "softmax backward %dx%d" % (rows, length))
+        # in place over the incoming gradient
+        dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hg, 0.0, d, hg)
+        assert np.array_equal(dev.get(hg, y.shape), dev.get(hx, y.shape))
+    # channel mode: series along c for every (n, h)
+    y = bf16_round(R.softmax_lastaxis(rng.standard_normal((3, 6, 10)).astype(np.float32)).transpose(0, 2, 1).copy())   # (3, 10, 6)
+    dy = bf16_round(rng.standard_normal(y.shape).astype(np.float32))
+    hy, hg, hx = dev.put(y, half), dev.put(dy, half), dev.zeros(y.size, half)
+    dev.cuda.SetTensorDesc(d, 3, 10, 6, 1, half)
+    dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.CHANNEL, 1.0, d, hy, d, hg, 0.0, d, hx)
+    assert_close(dev.get(hx, y.shape), R.softmax_backward(y, dy, axis=1, dtype=np.float64), tol, "softmax backward channel")
+    # log form
+    x = (rng.standard_normal((11, 96)) * 2).astype(np.float64)
+    ylog = bf16_round((x - np.log(np.exp(x).sum(-1, keepdims=True))).astype(np.float32))
+    dy = bf16_round(rng.standard_normal(ylog.shape).astype(np.float32))
+    hy, hg, hx = dev.put(ylog, half), dev.put(dy, half), dev.zeros(ylog.size, half)
+    dev.cuda.SetTensorDesc(d, 11, 96, 1, 1, half)
+    dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.LOG, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hg, 0.0, d, hx)
+    assert_close(dev.get(hx, ylog.shape), R.softmax_backward(ylog, dy, log=True, dtype=np.float64), tol, "log softmax backward")
+    # argument checks: scaling factors other than (1, 0), a descriptor of another shape, a short buffer
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hg, 1.0, d, hx)
+    assert e.value.code == ERROR.NOT_IMPLEMENTED
+    d2 = dev.cuda.CreateTensorDesc()
+    dev.cuda.SetTensorDesc(d2, 11, 95, 1, 1, half)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d2, hg, 0.0, d, hx)
+    assert e.value.code == ERROR.PARAM_OUT_OF_RANGE
+    dev.cuda.SetTensorDesc(d, 12, 96, 1, 1, half)
+    with pytest.raises(CudaDnnError):
+        dev.cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hg, 0.0, d, hx)
+    dev.cuda.FreeTensorDesc(d)
+    dev.cuda.FreeTensorDesc(d2)
+    dev.cuda.FreeCuDNN(hc)
+
+
 def test_softmax_forward_through_tensor_descriptors(dev):
     rng = np.random.default_rng(8)
     hc = dev.cuda.CreateCuDNN()
-    for rows, length in [(24, 200), (7, 3000), (5, 1)]:
+    for rows, length in [(24, 200), (7, 3000), (5, 1), (9, 1024), (3, 2048), (130, 64), (6, 37)]:
         x = (rng.standard_normal((rows, length)) * 4).astype(np.float32)
         hx, hy = dev.put(x), dev.zeros(x.size)
         bd, td = dev.cuda.CreateTensorDesc(), dev.cuda.CreateTensorDesc()

@@ -90,6 +90,19 @@ def test_gemm2_matmul_matches_numpy():
     assert np.allclose(out, A @ B, rtol=1e-13, atol=1e-13)
 
 
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("axis", [-1, 1])
+def test_softmax_backward_matches_torch_autograd(axis, log):
+    import torch
+    rng = np.random.default_rng(5)
+    x = torch.tensor(rng.standard_normal((3, 7, 11)) * 3, dtype=torch.float64, requires_grad=True)
+    dy = rng.standard_normal((3, 7, 11))
+    y = torch.log_softmax(x, dim=axis) if log else torch.softmax(x, dim=axis)
+    y.backward(torch.tensor(dy))
+    got = R.softmax_backward(y.detach().numpy(), dy, axis, log, np.float64)
+    assert np.allclose(got, x.grad.numpy(), rtol=1e-11, atol=1e-13)
+
+
 def test_softmax_matches_scipy():
     from scipy.special import softmax
     rng = np.random.default_rng(1)
