@@ -119,10 +119,12 @@ enum {
     MCH_FN_TRANSPOSE_HW = 267,              /* l{n, c, h, w, hSrc, hDst} (device.cu:3110-3127) */
     MCH_FN_INVERT = 273,                    /* [f{numerator, denominator}] l{n, hX, hY[, xOff, yOff]} (device.cu:2624-2655) */
     MCH_FN_CHANNEL_MEAN = 287,              /* l{count, outer, channels, inner, hX, hY[, xOff]} (device.cu:3386-3405) */
+    MCH_FN_CHANNEL_SUM = 292,               /* l{count, outer, channels, inner, hX, hY} (device.cu:3488-3503) */
     MCH_FN_CHANNEL_COPY = 300,              /* l{count, outer, channels, blocks, inner, offset, hX, hY, dir} (device.cu:3730-3748) */
     MCH_FN_CHANNEL_FILLFROM = 301,          /* l{count, outer, channels, inner, hX, hY, dir} (CudaDnn.cs:9086-9092, math.cu:7465-7481) */
     MCH_FN_CHANNEL_COPYALL = 302,           /* l{count, outer, channels, inner, hX, hY} (CudaDnn.cs:9443-9449, math.cu:7630-7639) */
     MCH_FN_CHANNEL_DUP = 303,               /* l{count, outer, channels, inner, hX, hY} (CudaDnn.cs:9312-9318, math.cu:7667-7676) */
+    MCH_FN_CHANNEL_SUM2 = 309,              /* l{count, outer, channels, inner, hX, hY, acrossChannels[, dir, channelsY]} (device.cu:3510-3534) */
     MCH_FN_EMBED_FWD = 390,                 /* l{count, hBtm, hWeight, M, N, K, hTop} (CudaDnn.cs:9751, math.cu:9314-9330) */
     MCH_FN_RELU_FWD = 428,                  /* f{negativeSlope} l{count, hBtm, hTop, 0} (device.h:4925-4940) */
     MCH_FN_RELU_BWD = 429,                  /* f{negativeSlope} l{count, hTopDiff, hTopData, hBtmDiff, 0} (device.h:4943-4959) */

@@ -1017,8 +1017,9 @@ hipError_t k_sub(hipStream_t s, DType dt, size_t n, const void* a, const void* b
     return hipGetLastError();
 }
 
-// mean of every row of `inner` values (channel_mean_kernel, math.cu:6817-6831): four rows per workgroup, one wavefront each
-template <typename T> __global__ __launch_bounds__(256) void channel_mean_kernel(size_t rows, int inner, const T* x, T* y)
+// sum (scale 1) or mean (scale 1 / inner) of every row of `inner` values (channel_mean_kernel, math.cu:6817-6831;
+// channel_sum_kernel_withinchannel, math.cu:6983-6997): four rows per workgroup, one wavefront each
+template <typename T> __global__ __launch_bounds__(256) void channel_rowsum_kernel(size_t rows, int inner, const T* x, T* y, float scale)
 {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -1027,14 +1028,51 @@ template <typename T> __global__ __launch_bounds__(256) void channel_mean_kernel
     float acc = 0.f;
     for (int i = lane; i < inner; i += 64) acc += ld(xr, i);
     acc = wave_sum(acc);
-    if (lane == 0) st(y, row, acc / inner);
+    if (lane == 0) st(y, row, acc * scale);
 }
-hipError_t k_channel_mean(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y)
+hipError_t k_channel_rowsum(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y, float scale)
 {
     if (rows == 0 || inner <= 0) return hipSuccess;
     const size_t g = (rows + 3) / 4;
     if (g > 0x7fffffffu) return hipErrorInvalidValue;
-    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_mean_kernel<T>, (int)g, 256, 0, s, rows, inner, (const T*)x, (T*)y));
+    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_rowsum_kernel<T>, (int)g, 256, 0, s, rows, inner, (const T*)x, (T*)y, scale));
+    return hipGetLastError();
+}
+hipError_t k_channel_mean(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y)
+{
+    return k_channel_rowsum(s, dt, rows, inner, x, y, inner > 0 ? 1.0f / inner : 0.f);
+}
+
+// y[n, s] = sum over c of x[n, c, s] (channel_sum_kernel_acrosschannels, math.cu:6945-6980; the reference accumulates in
+// double, here four fp32 partial sums per column meet in LDS).  A workgroup owns 64 columns s of one n: lane = column,
+// wavefront w takes channels w, w + 4, ..., so every load instruction reads 64 consecutive values.
+template <typename T> __global__ __launch_bounds__(256) void channel_colsum_kernel(int channels, int spatial, const T* x, T* y)
+{
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int sIdx = blockIdx.x * 64 + lane;
+    const size_t n = blockIdx.y;
+    float a0 = 0.f, a1 = 0.f;
+    if (sIdx < spatial) {
+        const T* xc = x + n * channels * (size_t)spatial + sIdx;
+        int c = w;
+        for (; c + 4 < channels; c += 8) {
+            a0 += ld(xc, (size_t)c * spatial);
+            a1 += ld(xc, (size_t)(c + 4) * spatial);
+        }
+        if (c < channels) a0 += ld(xc, (size_t)c * spatial);
+    }
+    part[w][lane] = a0 + a1;
+    __syncthreads();
+    if (w == 0 && sIdx < spatial) st(y, n * spatial + sIdx, (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]));
+}
+hipError_t k_channel_colsum(hipStream_t s, DType dt, size_t outer, int channels, int spatial, const void* x, void* y)
+{
+    if (outer == 0 || channels <= 0 || spatial <= 0) return hipSuccess;
+    if (spatial == 1) return k_channel_rowsum(s, dt, outer, channels, x, y, 1.0f);
+    if (outer > 65535) return hipErrorInvalidValue;
+    dim3 grid((spatial + 63) / 64, (unsigned)outer);
+    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_colsum_kernel<T>, grid, 256, 0, s, channels, spatial, (const T*)x, (T*)y));
     return hipGetLastError();
 }
 

@@ -77,6 +77,9 @@ hipError_t k_add_scalar(hipStream_t s, DType dt, size_t n, float alpha, void* y)
 hipError_t k_div(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y);
 hipError_t k_sub(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y, size_t nB);
 hipError_t k_channel_mean(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y);
+// y[row] = scale * sum of the row's `inner` values; y[n, s] = sum over the channels of x[n, c, s]
+hipError_t k_channel_rowsum(hipStream_t s, DType dt, size_t rows, int inner, const void* x, void* y, float scale);
+hipError_t k_channel_colsum(hipStream_t s, DType dt, size_t outer, int channels, int spatial, const void* x, void* y);
 // mode 0 fillfrom forward, 1 fillfrom backward, 2 copyall, 3 duplicate (index rules in ew_kernels.hip)
 hipError_t k_channel_spread(hipStream_t s, DType dt, int mode, size_t n, size_t spatial, size_t period, size_t channels, void* x, void* y);
 hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps);

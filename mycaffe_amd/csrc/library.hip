@@ -786,6 +786,50 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         m_mem.touch((long)pl[5]);
         return 0;
     }
+    case MCH_FN_CHANNEL_SUM:
+    case MCH_FN_CHANNEL_SUM2: {
+        // 292 l{count,outer,channels,inner,hX,hY}: y[outer,inner] = sum over the channels (CudaDnn.cs:9182-9188,
+        //     device.cu:3488-3503, math.cu:6945-6961)
+        // 309 l{count,outer,channels,inner,hX,hY,acrossChannels[,dir,channelsY]} (CudaDnn.cs:9205-9211, device.cu:3510-3534,
+        //     math.cu:7076-7114): forward sums across the channels (as 292) or within every channel (y[outer,channels] = row
+        //     sums); backward writes X from Y, every Y value spread over what it was summed from.
+        const bool two = fn == MCH_FN_CHANNEL_SUM2;
+        if (two) NEED_L(7, 9); else NEED_L(6, 6);
+        long long outer = pl[1], ch = pl[2], inner = pl[3];
+        const bool across = two ? pl[6] != 0 : true;
+        const int dir = two && ll > 7 ? (int)pl[7] : 0;
+        const long long chY = two && ll > 8 ? pl[8] : -1;
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (!two && outer > 1 && (long long)Y->count < outer * inner && (long long)Y->count >= inner) {
+            // RMSNormLayer.cs:198-199 passes its weight gradient (inner values) as Y with outer = batch: the reference
+            // writes the sums of every batch entry, the later ones past the end of Y.  Only what Y holds is computed.
+            outer = (long long)Y->count / inner;
+        }
+        const long long full = outer * ch * inner, reduced = across ? outer * inner : outer * ch;
+        RANGE(X, 0, full);
+        RANGE(Y, 0, reduced);
+        if (dir == 0) {
+            if (X->ptr == Y->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            if (across) HIPCHK(k_channel_colsum(s, X->dt(), (size_t)outer, (int)ch, (int)inner, X->ptr, Y->ptr));
+            else HIPCHK(k_channel_rowsum(s, X->dt(), (size_t)(outer * ch), (int)inner, X->ptr, Y->ptr, 1.0f));
+            m_mem.touch((long)pl[5]);
+            return 0;
+        }
+        if (chY == 1 && chY != ch) {
+            // the reference's second pair of backward kernels (math.cu:7017-7052) reads Y with an index that runs past
+            // outer * inner for the within-channel form; neither is used by the layers of this path
+            last_detail = "channel_sum backward with channelsY = 1 is not supported";
+            return MCH_ERROR_NOT_IMPLEMENTED;
+        }
+        if (across) HIPCHK(k_channel_spread(s, X->dt(), 3, (size_t)full, 1, (size_t)(ch * inner), (size_t)inner, Y->ptr, X->ptr));
+        else HIPCHK(k_channel_spread(s, X->dt(), 0, (size_t)full, (size_t)inner, 1, 1, Y->ptr, X->ptr));
+        m_mem.touch((long)pl[4]);
+        return 0;
+    }
     case MCH_FN_CHANNEL_FILLFROM:
     case MCH_FN_CHANNEL_COPYALL:
     case MCH_FN_CHANNEL_DUP: {

@@ -78,10 +78,12 @@ class CUDAFN:
     CUDA_TRANSPOSE_HW = 267
     CUDA_INVERT = 273
     CUDA_CHANNEL_MEAN = 287
+    CUDA_CHANNEL_SUM = 292
     CUDA_CHANNEL_COPY = 300
     CUDA_CHANNEL_FILLFROM = 301
     CUDA_CHANNEL_COPYALL = 302
     CUDA_CHANNEL_DUP = 303
+    CUDA_CHANNEL_SUM2 = 309
     CUDA_EMBED_FWD = 390
     CUDA_RELU_FWD = 428
     CUDA_RELU_BWD = 429
@@ -496,6 +498,15 @@ class CudaDnn:
     def channel_mean(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff=0):
         """CudaDnn.cs:9030-9036."""
         self._ex2(CUDAFN.CUDA_CHANNEL_MEAN, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff])
+
+    def channel_sum(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY):
+        """CudaDnn.cs:9182-9188: y[outer, inner] = sum over the channels."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_SUM, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY])
+
+    def channel_sumEx(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, bSumAcrossChannels, dir, nChannelsY=-1):
+        """CudaDnn.cs:9205-9211."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_SUM2, None,
+                  [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, 1 if bSumAcrossChannels else 0, dir, nChannelsY])
 
     def channel_fillfrom(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, dir):
         """CudaDnn.cs:9086-9092."""

@@ -587,6 +587,40 @@ class RMSNormLayer:
             cuda.mul(n, b["Out"].gpu_diff, b["Out"].gpu_data, top.gpu_data)
         else:
             top.CopyFrom(b["Out"])
+        self._dims = (n, outer, channels, inner)
+
+    def Backward(self, top, bottom, freeze_learning=False):
+        """RMSNormLayer.cs:189-232, the layer's own chain (after a Forward through the chain): top.diff -> bottom.diff and,
+        with weights, the weight gradient through channel_sum (which, as there, keeps the sums of the first batch
+        entry: the call passes outer = batch and a gradient blob of `inner` values)."""
+        if self.fused:
+            raise NotImplementedError("the fused forward call keeps none of the chain's intermediates")
+        cuda, b = self.cuda, self.b
+        n, outer, channels, inner = self._dims
+        if self.enable_weights:
+            if not freeze_learning:
+                cuda.mul(n, top.gpu_diff, b["Out"].gpu_data, b["Out"].gpu_data)
+                cuda.channel_sum(n, outer, channels, inner, b["Out"].gpu_data, self.blobs[0].gpu_diff)
+            cuda.mul(n, top.gpu_diff, b["Out"].gpu_diff, b["Out"].gpu_diff)
+        # (without weights the reference reads Out's gradient here although nothing has written it; same here)
+        # x6 = x * x5 -> dx and dx5
+        cuda.mul(n, b["Out"].gpu_diff, b["Rms1Full"].gpu_data, bottom.gpu_diff)
+        cuda.mul(n, b["Out"].gpu_diff, bottom.gpu_data, b["Rms1Full"].gpu_diff)
+        cuda.channel_sumEx(n, outer, channels, inner, b["Rms1Full"].gpu_diff, b["Rms1"].gpu_diff, False, DIR.FWD)
+        # x5 = 1 / x4 -> dx4
+        cuda.powx(b["Rms"].count(), b["Rms"].gpu_data, 2.0, b["Rms"].gpu_diff)
+        cuda.invert(b["Rms"].count(), b["Rms"].gpu_diff, b["Rms"].gpu_diff, 0, 0, -1)
+        cuda.mul(b["Rms1"].count(), b["Rms1"].gpu_diff, b["Rms"].gpu_diff, b["Rms"].gpu_diff)
+        # x4 = sqrt(x2 + eps) -> dx2
+        cuda.invert(b["Rms1"].count(), b["Rms"].gpu_data, b["Rms1"].gpu_diff, 0, 0, 1, 2)
+        cuda.mul(b["Rms"].count(), b["Rms1"].gpu_diff, b["Rms"].gpu_diff, b["Rms"].gpu_diff)
+        # x2 = mean(x1) -> dx1
+        cuda.channel_duplicate(n, outer * channels, 1, inner, b["Rms"].gpu_diff, b["Rms1Full"].gpu_diff)
+        cuda.scal(b["Rms1Full"].count(), 1.0 / inner, b["Rms1Full"].gpu_diff)
+        # x1 = x^2 -> dx, and the sum of both paths
+        cuda.scale(n, 2.0, bottom.gpu_data, b["Out"].gpu_diff)
+        cuda.mul(n, b["Out"].gpu_diff, b["Rms1Full"].gpu_diff, b["Out"].gpu_diff)
+        cuda.add(n, b["Out"].gpu_diff, bottom.gpu_diff, bottom.gpu_diff)
 
 
 class ActivationLayer:
@@ -653,7 +687,7 @@ class TransformerBlockLayer:
         self.fc2 = InnerProductLayer(cuda, hidden_dim, bias_term, 2) if self.llama else None
         self.proj = InnerProductLayer(cuda, embed, bias_term, 2)
         self.act = ActivationLayer(cuda, activation)
-        self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 Mlp1 Mlp2 Mlp3 MlpOut".split()}
+        self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 NormA Mlp1 Mlp2 Mlp3 MlpOut".split()}
 
     def Setup(self, bottom, p):
         """``p``: attn_weight, attn_bias, attn_proj_weight, attn_proj_bias, fc_weight, fc_bias, proj_weight, proj_bias."""
@@ -689,15 +723,23 @@ class TransformerBlockLayer:
 
     def Backward(self, top, blobX):
         """TransformerBlockLayer.cs:924-1040, CAUSAL_SELF_ATTENTION block: top.gpu_diff -> blobX.gpu_diff."""
-        if self.llama:
-            raise NotImplementedError("the RMSNorm chain's backward is not mirrored")
         b, cuda = self.b, self.cuda
         nCount = blobX.count()
         cuda.copy(nCount, top.gpu_diff, b["MlpOut"].gpu_diff)
         cuda.copy(nCount, top.gpu_diff, b["X"].gpu_diff)
-        self.proj.Backward(b["MlpOut"], b["Mlp1"])
+        self.proj.Backward(b["MlpOut"], b["Mlp3"] if self.llama else b["Mlp1"])
+        if self.llama:
+            # gate: Mlp3 = silu(fc1) * fc2; the gradient through fc2 waits in NormA's data until fc1's has arrived
+            n1 = b["Mlp1"].count()
+            cuda.mul(n1, b["Mlp3"].gpu_diff, b["Mlp2"].gpu_data, b["Mlp1"].gpu_diff)
+            cuda.mul(n1, b["Mlp3"].gpu_diff, b["Mlp1"].gpu_data, b["Mlp2"].gpu_diff)
+            self.fc2.Backward(b["Mlp2"], b["Norm2"])
+            b["NormA"].ReshapeLike(b["Norm2"])
+            cuda.copy(b["Norm2"].count(), b["Norm2"].gpu_diff, b["NormA"].gpu_data)
         self.act.Backward(b["Mlp1"], b["Mlp1"])
         self.fc1.Backward(b["Mlp1"], b["Norm2"])
+        if self.llama:
+            cuda.add(b["Norm2"].count(), b["NormA"].gpu_data, b["Norm2"].gpu_diff, b["Norm2"].gpu_diff)
         # x_2 = ln_2(xB): keep xB's own gradient aside, add the one that comes through the norm
         b["Attn1"].CopyFrom(b["X"], True)
         self.norm2.Backward(b["Norm2"], b["X"])

@@ -210,6 +210,28 @@ def rmsnorm_layer(x, weight=None, eps=1e-5, dtype=np.float32):
     return out.astype(dtype)
 
 
+def rmsnorm_layer_backward(x, weight, dy, eps=1e-5, dtype=np.float32):
+    """Gradients of ``rmsnorm_layer`` with weights as RMSNormLayer.cs:189-232 computes them, step by step: returns
+    (dx, dw).  dw is what the layer's channel_sum call leaves in the weight gradient: the call sums over the axis
+    before the last one for every leading index and the gradient blob holds one row, so it is the first leading
+    entry's sum (for an input with one leading entry, the full gradient)."""
+    x, dy, w = np.asarray(x, dtype), np.asarray(dy, dtype), np.asarray(weight, dtype)
+    inner = x.shape[-1]
+    x2 = (x.astype(np.float64) ** 2).mean(axis=-1, keepdims=True).astype(dtype)
+    x4 = np.sqrt(x2 + dtype(eps))
+    x5 = dtype(1) / x4
+    out = x * x5
+    lead = x.reshape((-1,) + x.shape[-2:])                       # (outer, channels, inner)
+    dw = (dy * out).reshape(lead.shape)[0].sum(axis=0)
+    dout = dy * w
+    dx_a = dout * x5
+    dx5 = (dout * x).sum(axis=-1, keepdims=True)
+    dx4 = dx5 * (dtype(-1) / (x4 * x4))
+    dx2 = dx4 * (dtype(1) / (dtype(2) * x4))
+    dx1 = np.broadcast_to(dx2, x.shape) / dtype(inner)
+    return (dx_a + dtype(2) * x * dx1).astype(dtype), dw.astype(dtype)
+
+
 # ----------------------------------------------------------------------------
 # RoPE, CudaDnnDLL form
 # ----------------------------------------------------------------------------

@@ -5,7 +5,7 @@ import os
 import numpy as np
 import pytest
 
-from mycaffe_amd.cudadnn import CudaDnnError, ERROR
+from mycaffe_amd.cudadnn import CudaDnnError, DIR, ERROR
 from mycaffe_amd.layers import Blob, TransformerBlockLayer
 from oracle import attention_ref as R
 from tests.conftest import BF16_RTOL, FP32_RTOL, GOLDEN, assert_close, bf16_round, load_txt
@@ -329,6 +329,65 @@ def test_norm_chain_primitives_vs_numpy(dev):
     assert np.array_equal(dev.get(ha), exp)
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_channel_sum_forms_vs_numpy(dev, half):
+    """Ids 292 and 309: sums across the channels and within every channel, and the backward forms that spread the sums."""
+    rng = np.random.default_rng(83)
+    cuda = dev.cuda
+    tol = BF16_RTOL if half else 1e-6
+    for outer, ch, inner in [(3, 5, 48), (2, 1024, 70), (4, 7, 1), (1, 1, 300), (2, 130, 64)]:
+        n = outer * ch * inner
+        x = bf16_round(rng.standard_normal((outer, ch, inner)).astype(np.float32))
+        hx, ha, hw = dev.put(x, half), dev.zeros(outer * inner, half), dev.zeros(outer * ch, half)
+        cuda.channel_sum(n, outer, ch, inner, hx, ha)
+        assert_close(dev.get(ha, (outer, inner)), x.astype(np.float64).sum(1), tol, "channel_sum %s" % ((outer, ch, inner),))
+        cuda.channel_sumEx(n, outer, ch, inner, hx, ha, True, DIR.FWD)
+        assert_close(dev.get(ha, (outer, inner)), x.astype(np.float64).sum(1), tol, "channel_sumEx across")
+        cuda.channel_sumEx(n, outer, ch, inner, hx, hw, False, DIR.FWD)
+        assert_close(dev.get(hw, (outer, ch)), x.astype(np.float64).sum(2), tol, "channel_sumEx within")
+        across, within = dev.get(ha, (outer, 1, inner)), dev.get(hw, (outer, ch, 1))
+        cuda.channel_sumEx(n, outer, ch, inner, hx, ha, True, DIR.BWD)
+        assert np.array_equal(dev.get(hx, x.shape), np.broadcast_to(across, x.shape))
+        cuda.channel_sumEx(n, outer, ch, inner, hx, hw, False, DIR.BWD)
+        assert np.array_equal(dev.get(hx, x.shape), np.broadcast_to(within, x.shape))
+    # a destination that holds one row of `inner` sums although outer > 1 (the weight gradient of RMSNormLayer): the
+    # first entry's sums, nothing written past the end
+    x = rng.standard_normal((3, 6, 40)).astype(np.float32)
+    hx, hy = dev.put(x), dev.put(np.zeros(40 + 8, np.float32))
+    hv = cuda.CreateMemoryPointer(hy, 0, 40)
+    cuda.channel_sum(x.size, 3, 6, 40, hx, hv)
+    got = dev.get(hy)
+    assert_close(got[:40], x[0].astype(np.float64).sum(0), 1e-6, "channel_sum into one row")
+    assert np.array_equal(got[40:], np.zeros(8, np.float32))
+    cuda.FreeMemoryPointer(hv)
+    with pytest.raises(CudaDnnError):
+        cuda.channel_sum(x.size, 3, 6, 40, hx, dev.zeros(39))
+    with pytest.raises(CudaDnnError) as e:
+        cuda.channel_sumEx(x.size, 3, 6, 40, hx, dev.zeros(3 * 40), True, DIR.BWD, 1)
+    assert e.value.code == ERROR.NOT_IMPLEMENTED
+
+
+def test_rmsnorm_layer_backward_chain_vs_checker(dev):
+    """RMSNormLayer.backward as the C# layer issues it (mul, channel_sum, channel_sumEx, powx, invert, channel_duplicate,
+    scal, scale, add) against the checker's gradients, for one and for several leading entries."""
+    from mycaffe_amd.layers import RMSNormLayer
+    rng = np.random.default_rng(84)
+    for shape in [(1, 9, 288), (3, 5, 64)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        w = (rng.standard_normal(shape[-1]) + 1.0).astype(np.float32)
+        dy = rng.standard_normal(shape).astype(np.float32)
+        layer = RMSNormLayer(dev.cuda, 1e-5, True, False)
+        bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+        bx.mutable_cpu_data = x
+        layer.Setup(bx, w)
+        layer.Forward(bx, top)
+        top.mutable_cpu_diff = dy
+        layer.Backward(top, bx)
+        dx, dw = R.rmsnorm_layer_backward(x, w, dy, 1e-5, np.float64)
+        assert_close(bx.mutable_cpu_diff, dx, 1e-5, "rmsnorm dx %s" % (shape,))
+        assert_close(layer.blobs[0].mutable_cpu_diff, dw, 1e-5, "rmsnorm dw %s" % (shape,))
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_rmsnorm_layer_chain_vs_checker(dev, fused):
     from mycaffe_amd.layers import RMSNormLayer
@@ -382,3 +441,39 @@ def test_transformer_block_llama_style_vs_checker(dev, fused_rmsnorm, sdpa):
     layer.Forward(bx, top)
     ref = R.transformer_block_llama(x, p, H, T, 10000.0, 1e-5, np.float64)
     assert_close(top.mutable_cpu_data, ref, FP32_RTOL, "llama block")
+
+
+@pytest.mark.parametrize("sdpa", [True, False])
+def test_transformer_block_llama_style_backward_vs_finite_differences(dev, sdpa):
+    """Backward of the Llama-style block through the layer mirrors (RMSNorm chain, rotary attention, gated MLP): the input
+    gradient against central differences of the fp64 checker's forward pass, every input element perturbed."""
+    rng = np.random.default_rng(85)
+    B, T, C, H = 2, 6, 16, 2
+    layer = TransformerBlockLayer(dev.cuda, H, C, T, "silu", False, 1e-5, sdpa, training=True, enable_llama_style_head=True,
+                                  multiple_of=8)
+    hid = layer.fc1.N
+    p = {"rms1_weight": 1 + 0.1 * rng.standard_normal(C), "rms2_weight": 1 + 0.1 * rng.standard_normal(C),
+         "attn_weight": rng.standard_normal((3 * C, C)) * 0.3, "attn_proj_weight": rng.standard_normal((C, C)) * 0.3,
+         "fc_weight": rng.standard_normal((hid, C)) * 0.3, "fc2_weight": rng.standard_normal((hid, C)) * 0.3,
+         "proj_weight": rng.standard_normal((C, hid)) * 0.3}
+    p = {k: v.astype(np.float32) for k, v in p.items()}
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    dy = rng.standard_normal((B, T, C)).astype(np.float32)
+    bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    top.mutable_cpu_diff = dy
+    layer.Backward(top, bx)
+    got = bx.mutable_cpu_diff.reshape(x.shape)
+
+    def loss(xx):
+        return float((R.transformer_block_llama(xx, p, H, T, 10000.0, 1e-5, np.float64) * dy).sum())
+
+    x64, num, h = x.astype(np.float64), np.zeros(x.shape, np.float64), 1e-5
+    for i in np.ndindex(*x.shape):
+        xp, xm = x64.copy(), x64.copy()
+        xp[i] += h
+        xm[i] -= h
+        num[i] = (loss(xp) - loss(xm)) / (2 * h)
+    assert_close(got, num, 2e-4, "llama block dx")

@@ -90,6 +90,28 @@ def test_gemm2_matmul_matches_numpy():
     assert np.allclose(out, A @ B, rtol=1e-13, atol=1e-13)
 
 
+def test_rmsnorm_layer_backward_matches_torch_autograd():
+    import torch
+    rng = np.random.default_rng(6)
+    x = torch.tensor(rng.standard_normal((1, 5, 24)), dtype=torch.float64, requires_grad=True)
+    w = torch.tensor(rng.standard_normal(24) + 1.0, dtype=torch.float64, requires_grad=True)
+    dy = rng.standard_normal((1, 5, 24))
+    y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w
+    y.backward(torch.tensor(dy))
+    dx, dw = R.rmsnorm_layer_backward(x.detach().numpy(), w.detach().numpy(), dy, 1e-5, np.float64)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-11, atol=1e-13)
+    assert np.allclose(dw, w.grad.numpy(), rtol=1e-11, atol=1e-13)
+    # more than one leading entry: the input gradient is still the full one, the weight gradient is the first entry's
+    x3 = rng.standard_normal((3, 5, 24))
+    dy3 = rng.standard_normal((3, 5, 24))
+    xt = torch.tensor(x3, requires_grad=True)
+    (xt * torch.rsqrt((xt * xt).mean(-1, keepdim=True) + 1e-5) * w.detach()).backward(torch.tensor(dy3))
+    dx3, dw3 = R.rmsnorm_layer_backward(x3, w.detach().numpy(), dy3, 1e-5, np.float64)
+    assert np.allclose(dx3, xt.grad.numpy(), rtol=1e-11, atol=1e-13)
+    _, dw0 = R.rmsnorm_layer_backward(x3[:1], w.detach().numpy(), dy3[:1], 1e-5, np.float64)
+    assert np.allclose(dw3, dw0)
+
+
 @pytest.mark.parametrize("log", [False, True])
 @pytest.mark.parametrize("axis", [-1, 1])
 def test_softmax_backward_matches_torch_autograd(axis, log):
