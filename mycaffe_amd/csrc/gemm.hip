@@ -663,9 +663,10 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
 // ---------------------------------------------------------------------------
 // fp32 MFMA for the strided-batched gemm2 (the Blob.MatMul route of the explicit attention chain: Q K^T and P V per
 // (batch, head), math.cu:1750-1788).  Column-major operands with any leading dimension: A(i,k) has either i or k at unit
-// stride, B(k,j) either k or j, C(i,j) has i at unit stride.  Both operands are staged into LDS as [row][k] (a
-// transposing scatter when the row index is the unit-stride one), so that one 128-bit LDS read feeds four
-// v_mfma_f32_32x32x2_f32 steps (slot trick as in gemm_nt_f32_mfma_kernel).  The MFMA row operand is B and the column
+// stride, B(k,j) either k or j, C(i,j) has i at unit stride.  An operand with k at unit stride is staged into LDS as
+// [row][k], so that one 128-bit LDS read feeds four v_mfma_f32_32x32x2_f32 steps (slot trick as in
+// gemm_nt_f32_mfma_kernel); one with the row index at unit stride is staged as it lies, [k][row], and a lane gathers its
+// four k with 32-bit reads (consecutive lanes, consecutive words: no bank conflicts on either side).  The MFMA row operand is B and the column
 // operand is A: the accumulator then has i in the lane and every store instruction of a wavefront writes two 128-byte
 // runs of C.  TI x TJ tile (i x j), four wavefronts 2 x 2.
 template <bool A_IFAST, bool B_KFAST, int TI, int TJ>
@@ -674,9 +675,10 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
                                                              GemmStrides st, int splits, int kChunk)
 {
     constexpr int BK = 16, LDK = BK + 4;
+    constexpr int LDI = TI + 4, LDJ = TJ + 4;        // row strides of the [k][row] layouts
     constexpr int NI = TI / 64, NJ = TJ / 64;        // 32x32 blocks per wavefront along i and j
-    __shared__ __attribute__((aligned(16))) float Is[2][TI * LDK];   // A: [i][k]
-    __shared__ __attribute__((aligned(16))) float Js[2][TJ * LDK];   // B: [j][k]
+    __shared__ __attribute__((aligned(16))) float Is[2][A_IFAST ? BK * LDI : TI * LDK];   // A: [k][i] or [i][k]
+    __shared__ __attribute__((aligned(16))) float Js[2][B_KFAST ? TJ * LDK : BK * LDJ];   // B: [j][k] or [k][j]
     // blockIdx.z = batch * splits + split; with splits > 1 every workgroup covers kChunk of the contraction and adds its
     // part to C with float atomics (C holds beta * C already)
     const int batchIdx = blockIdx.z / splits, split = blockIdx.z % splits;
@@ -733,8 +735,7 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
             const int e = tid + p * 256;
             if (A_IFAST) {
                 const int ig = e % (TI / 4), k = e / (TI / 4);
-                float* d = &Is[buf][(4 * ig) * LDK + k];
-                d[0] = ra[p].x; d[LDK] = ra[p].y; d[2 * LDK] = ra[p].z; d[3 * LDK] = ra[p].w;
+                *(float4*)(&Is[buf][k * LDI + 4 * ig]) = ra[p];
             } else {
                 const int kg = e % (BK / 4), i = e / (BK / 4);
                 *(float4*)(&Is[buf][i * LDK + 4 * kg]) = ra[p];
@@ -748,8 +749,7 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
                 *(float4*)(&Js[buf][j * LDK + 4 * kg]) = rb[p];
             } else {
                 const int jg = e % (TJ / 4), k = e / (TJ / 4);
-                float* d = &Js[buf][(4 * jg) * LDK + k];
-                d[0] = rb[p].x; d[LDK] = rb[p].y; d[2 * LDK] = rb[p].z; d[3 * LDK] = rb[p].w;
+                *(float4*)(&Js[buf][k * LDJ + 4 * jg]) = rb[p];
             }
         }
     };
@@ -766,9 +766,23 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
         for (int kk = 0; kk < BK; kk += 8) {
             float4 fj[NJ], fi[NI];
 #pragma unroll
-            for (int t = 0; t < NJ; t++) fj[t] = *(const float4*)(&Js[buf][(wj + t * 32 + fr) * LDK + kk + fg]);
+            for (int t = 0; t < NJ; t++) {
+                if (B_KFAST) {
+                    fj[t] = *(const float4*)(&Js[buf][(wj + t * 32 + fr) * LDK + kk + fg]);
+                } else {   // four k of one j: consecutive lanes read consecutive words
+                    const float* q = &Js[buf][(kk + fg) * LDJ + wj + t * 32 + fr];
+                    fj[t] = make_float4(q[0], q[LDJ], q[2 * LDJ], q[3 * LDJ]);
+                }
+            }
 #pragma unroll
-            for (int t = 0; t < NI; t++) fi[t] = *(const float4*)(&Is[buf][(wi + t * 32 + fr) * LDK + kk + fg]);
+            for (int t = 0; t < NI; t++) {
+                if (A_IFAST) {
+                    const float* q = &Is[buf][(kk + fg) * LDI + wi + t * 32 + fr];
+                    fi[t] = make_float4(q[0], q[LDI], q[2 * LDI], q[3 * LDI]);
+                } else {
+                    fi[t] = *(const float4*)(&Is[buf][(wi + t * 32 + fr) * LDK + kk + fg]);
+                }
+            }
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
