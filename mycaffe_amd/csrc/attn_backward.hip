@@ -333,8 +333,9 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dkv_mfma_kernel(AttnBwdArgs
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int nbh = a.B * a.H;
-    const int kblock = blockIdx.x / nbh;            // causal: low key blocks see the most queries and start first
-    const int ibh = blockIdx.x % nbh;
+    const int rank = KIND == 1 ? flash_causal_rank(OCC) : (int)blockIdx.x;
+    const int kblock = rank / nbh;                  // causal: low key blocks see the most queries and start first
+    const int ibh = rank % nbh;
     const int b = ibh / a.H, h = ibh % a.H;
     const size_t bh = (size_t)b * a.H + h;
     const int kw = kblock * BK + wave * 32;          // first key of this wavefront
@@ -493,8 +494,9 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs 
     const int l32 = lane & 31, half = lane >> 5;
     const int nbh = a.B * a.H;
     const int nqb = (a.Tq + BM - 1) / BM;
-    const int qblock = (KIND == 1) ? nqb - 1 - (int)(blockIdx.x / nbh) : (int)(blockIdx.x / nbh);   // causal: heaviest first
-    const int ibh = blockIdx.x % nbh;
+    const int rank = KIND == 1 ? flash_causal_rank(OCC) : (int)blockIdx.x;
+    const int qblock = (KIND == 1) ? nqb - 1 - rank / nbh : rank / nbh;   // causal: heaviest first
+    const int ibh = rank % nbh;
     const int b = ibh / a.H, h = ibh % a.H;
     const size_t bh = (size_t)b * a.H + h;
     const int q0w = qblock * BM + wave * 32;

@@ -207,21 +207,6 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
     }
 }
 
-// Rank of a workgroup of a causal launch in the heaviest-first order.  Workgroup i goes to XCD i % 8 and, within it, the
-// first launches land on its 32 CUs in turn, `occ` rounds of 32 before the XCD is full.  A CU keeps what it was given in
-// those rounds, so every second one of them is walked backwards: the CU that got the heaviest block of one round gets
-// the lightest of the next.  Later rounds start as slots free up, where plain heaviest-first is the better order.
-// Ranks stay congruent to the workgroup index mod 8 (same XCD, same L2).
-__device__ __forceinline__ int flash_causal_rank(int occ)
-{
-    if ((gridDim.x & 7) != 0) return (int)blockIdx.x;
-    const int x = blockIdx.x & 7, j = blockIdx.x >> 3, per = gridDim.x >> 3;
-    const int r = j >> 5, c = j & 31;
-    if (!(r & 1) || r >= occ) return (int)blockIdx.x;
-    const int width = min(32, per - (r << 5));   // the last round may be short
-    return (((r << 5) + width - 1 - c) << 3) + x;
-}
-
 // KIND: 0 no mask, 1 causal, 2 per-key mask (B, Tk), 3 per-sequence mask (B, Tq, Tk).  OCC: workgroups per CU the register budget is set for.
 // PREFETCH: hold the next K / V block in registers while computing on the current one.
 template <typename T, int HS, int KIND, int QT, int NW, int OCC, bool PREFETCH>
