@@ -47,10 +47,10 @@ def log(*a):
 
 
 def make_checkpoint(cfg, seed, path):
-    from oracle import llama2 as O   # checkpoint writer + the CPU baseline live with the checker
-    blob, _ = O.random_weights(cfg, seed=seed, shared_classifier=False, std=0.02)
+    from mycaffe_amd import checkpoint as C
+    blob = C.random_model(cfg, seed, shared_classifier=False, std=0.02)
     if not os.path.exists(path):
-        O.write_checkpoint_v1(path, cfg, blob, False)
+        C.write_v1(path, cfg, blob, False)
     return blob
 
 

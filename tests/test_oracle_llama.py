@@ -261,3 +261,18 @@ def test_generate_sampled_loop_draws_a_coin_at_every_position():
             tok = int(prompt[pos]) if pos < len(prompt) else nxt
             nxt = s.sample(m.forward(tok, pos))
             assert nxt == ids[pos]
+
+
+def test_package_checkpoint_writer_matches_the_checkers(tmp_path):
+    """The benchmark writes its synthetic model with the package's own writer; the file and the weights are the ones
+    the checker's writer gives for the same seed, so both sides load the same model."""
+    from mycaffe_amd import checkpoint as C
+    cfg = dict(dim=64, hidden_dim=172, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=256, seq_len=32)
+    for shared in (False, True):
+        a, _ = O.random_weights(cfg, seed=3, shared_classifier=shared, std=0.2)
+        b = C.random_model(cfg, 3, shared_classifier=shared, std=0.2)
+        assert np.array_equal(a, b)
+        pa, pb = str(tmp_path / "a.bin"), str(tmp_path / "b.bin")
+        O.write_checkpoint_v1(pa, cfg, a, shared)
+        C.write_v1(pb, cfg, b, shared)
+        assert open(pa, "rb").read() == open(pb, "rb").read()
