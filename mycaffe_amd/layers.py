@@ -398,8 +398,9 @@ class CausalSelfAttentionLayer:
 
 
 class MultiheadAttentionLayer:
-    """MyCaffe.layers.gpt/layers.gpt/MultiheadAttentionLayer.cs:643-811 (no KV cache:
-    the cached decode branch is served by :meth:`CudaDnn.AttnDecodeForward`).
+    """MyCaffe.layers.gpt/layers.gpt/MultiheadAttentionLayer.cs:643-811.  With ``enable_key_value_cache`` and the
+    "position" layer option set, the explicit chain takes the reference's cached decode branch (:713-730, 759-777: one
+    token per call, a loop over the cached positions); :meth:`CudaDnn.AttnDecodeForward` is the one-call replacement.
 
     ``Forward(q, k, v, mask)``: mask is ``None``, a (1,1,T,T) blob (causal), a
     (B,T_k) key-padding blob or a (B,T_q,T_k) blob; the last two take the
@@ -409,9 +410,11 @@ class MultiheadAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, fuse_batch_qk_mask=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, fuse_batch_qk_mask=False,
+                 enable_key_value_cache=False):
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
         self.fuse_batch_qk_mask = fuse_batch_qk_mask
+        self.enable_kv_cache = enable_key_value_cache
         self.nSize = embed // heads
         self.half = half
         self.enable_sdpa = enable_cuda_scaled_dot_product_attention
@@ -424,7 +427,7 @@ class MultiheadAttentionLayer:
         self.transposeK = TransposeLayer(cuda, (0, 2, 1, 3))
         self.transposeQ = TransposeLayer(cuda, (0, 1, 3, 2))
         self.softmax = SoftmaxLayer(cuda, -1)
-        self.b = {n: Blob(cuda, half=half) for n in "Q K V Qt Kt Vt Kt1 AttA AttB Work Y".split()}
+        self.b = {n: Blob(cuda, half=half) for n in "Q K V Qt Kt Vt Kt1 AttA AttB Work Y KeyCache ValCache Work2 Work3".split()}
         self.hCudnn = self.hAttn = self.hRope = 0
         self._set_for = None
         self.options = {}
@@ -478,16 +481,50 @@ class MultiheadAttentionLayer:
             # (B,T_q,T_k) mask goes through the explicit chain (MultiheadAttentionLayer.cs:733-742)
             self.transposeQ.Forward(b["Kt"], b["Kt1"])
             dfScale = 1.0 / math.sqrt(hs)
-            b["AttA"].MatMul(b["Qt"], b["Kt1"], bReshape=True)
-            b["AttA"].scale_data(dfScale)
-            if blobMask is not None:
-                if is_qk_mask:
-                    cuda.mask(b["AttA"].count(), blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data, blobMask.gpu_data, b["AttA"].gpu_data)
-                else:
-                    cuda.mask_batch(b["AttA"].count(), b["AttA"].num, blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data,
-                                    blobMask.gpu_data, b["AttA"].gpu_data)
+            cached = nPos >= 0 and self.enable_kv_cache
+            if cached:
+                # one token: append its key / value to the caches (sized for the block size at the first call, as the
+                # layer's reshape does), then one MatMul per cached position (:713-730)
+                for name in ("KeyCache", "ValCache"):
+                    if b[name]._capacity == 0:
+                        b[name].Reshape(B, H, self.nBlockSize, hs)
+                b["KeyCache"].Reshape(nPos + 1, H, hs, 1)
+                b["ValCache"].Reshape(nPos + 1, H, 1, hs)
+                nK, nV = b["Kt1"].count(), b["Vt"].count()
+                cuda.copy(nK, b["Kt1"].gpu_data, b["KeyCache"].gpu_data, 0, nPos * nK)
+                cuda.copy(nV, b["Vt"].gpu_data, b["ValCache"].gpu_data, 0, nPos * nV)
+                b["AttA"].Reshape(1, H, 1, nPos + 1)
+                for i in range(nPos + 1):
+                    cuda.copy(nK, b["KeyCache"].gpu_data, b["Kt1"].gpu_data, i * nK, 0)
+                    b["Work2"].MatMul(b["Qt"], b["Kt1"], True)
+                    b["Work2"].scale_data(dfScale)
+                    cuda.channel_copy(b["Work2"].count(), 1, H, nPos + 1, 1, i, b["AttA"].gpu_data, b["Work2"].gpu_data, DIR.BWD)
+            else:
+                b["AttA"].MatMul(b["Qt"], b["Kt1"], bReshape=True)
+                b["AttA"].scale_data(dfScale)
+                if blobMask is not None:
+                    if is_qk_mask:
+                        cuda.mask(b["AttA"].count(), blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data, blobMask.gpu_data, b["AttA"].gpu_data)
+                    else:
+                        cuda.mask_batch(b["AttA"].count(), b["AttA"].num, blobMask.count(), 0.0, -1e29, b["AttA"].gpu_data,
+                                        blobMask.gpu_data, b["AttA"].gpu_data)
             self.softmax.Forward(b["AttA"], b["AttB"])
-            b["Work"].MatMul(b["AttB"], b["Vt"], bReshape=True)
+            if cached:
+                # y = sum over the cached positions of weight_i * v_i, one MatMul and one add per position (:759-777)
+                b["Work"].Reshape(1, H, 1, hs)
+                b["Work3"].Reshape(1, H, 1, 1)
+                b["Work2"].Reshape(1, H, 1, hs)
+                nV = b["Vt"].count()
+                for i in range(nPos + 1):
+                    cuda.copy(nV, b["ValCache"].gpu_data, b["Vt"].gpu_data, i * nV, 0)
+                    cuda.channel_copy(b["Work3"].count(), 1, H, nPos + 1, 1, i, b["AttB"].gpu_data, b["Work3"].gpu_data, DIR.FWD)
+                    b["Work2"].MatMul(b["Work3"], b["Vt"], True)
+                    if i == 0:
+                        cuda.copy(b["Work"].count(), b["Work2"].gpu_data, b["Work"].gpu_data)
+                    else:
+                        cuda.add(b["Work"].count(), b["Work2"].gpu_data, b["Work"].gpu_data, b["Work"].gpu_data)
+            else:
+                b["Work"].MatMul(b["AttB"], b["Vt"], bReshape=True)
         self.transpose.Forward(b["Work"], b["Y"])
         b["Y"].Reshape(B, Tq, C)
         self.c_proj.Forward(b["Y"], top)

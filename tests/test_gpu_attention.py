@@ -218,6 +218,30 @@ def test_causal_self_attention_layer_bf16(dev):
     assert_close(top.mutable_cpu_data, ref["y"], BF16_RTOL, "csa bf16")
 
 
+@pytest.mark.parametrize("rope", [False, True])
+def test_multihead_attention_cached_decode_branch_of_the_layer(dev, rope):
+    """The reference layer's own cached decode (MultiheadAttentionLayer.cs:713-730, 759-777: one token per call with the
+    "position" option, a copy / MatMul / channel_copy / add loop over the cached positions) through the unchanged call
+    sequence: the output for token p equals row p of the causal forward over the whole sequence."""
+    rng = np.random.default_rng(29)
+    B, T, C, H = 1, 10, 96, 3
+    W = {k: (rng.standard_normal((C, C)) * 0.2).astype(np.float32) for k in ("wq", "wk", "wv", "wo")}
+    W.update({k: (rng.standard_normal(C) * 0.1).astype(np.float32) for k in ("bq", "bk", "bv", "bo")})
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    ref = R.multihead_attention(x, x, x, W["wq"], W["bq"], W["wk"], W["bk"], W["wv"], W["bv"], W["wo"], W["bo"], H,
+                                R.causal_mask(T), "causal", rope=(T, 10000.0) if rope else None, dtype=np.float64)["y"]
+    layer = MultiheadAttentionLayer(dev.cuda, H, C, T, True, False, enable_rotary_positional_embedding=rope,
+                                    enable_key_value_cache=True)
+    tok, top = Blob(dev.cuda, (B, 1, C)), Blob(dev.cuda)
+    tok.mutable_cpu_data = x[:, :1]
+    layer.Setup(tok, tok, tok, W)
+    for p in range(T):
+        tok.mutable_cpu_data = x[:, p:p + 1]
+        layer.SetLayerOption("position", p)
+        layer.Forward(tok, tok, tok, None, top)
+        assert_close(top.mutable_cpu_data.reshape(B, C), ref[:, p], FP32_RTOL, "cached decode, position %d" % p)
+
+
 @pytest.mark.parametrize("sdpa", [True, False])
 def test_multihead_attention_encoder_decoder_masks(dev, sdpa):
     # scaled-down encoder / decoder / cross attention with padding masks (valid lengths per sequence)
