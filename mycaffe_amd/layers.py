@@ -699,13 +699,19 @@ class ActivationLayer:
 
 
 class TransformerBlockLayer:
-    """MyCaffe.layers.gpt/layers.gpt/TransformerBlockLayer.cs, block type CAUSAL_SELF_ATTENTION (setup :99-130, 252-340,
-    forward :810-902): x + attn(ln1(x)), then + proj(act(fc(ln2(.)))).  Dropout is the identity at inference."""
+    """MyCaffe.layers.gpt/layers.gpt/TransformerBlockLayer.cs, block types CAUSAL_SELF_ATTENTION and ENCODER (setup
+    :99-170, 252-340, forward :800-902): x + attn(ln1(x)), then + proj(act(fc(ln2(.)))).  The ENCODER type attends
+    through MultiheadAttentionLayer(x_1, x_1, x_1, mask), the form the Llama models built by LlamaModelBuilder use
+    (rotary embedding, key / value cache, "position" layer option).  Dropout is the identity at inference."""
 
     def __init__(self, cuda, heads, embed, block_size, activation="relu", bias_term=True, epsilon=1e-10,
                  enable_cuda_scaled_dot_product_attention=True, training=False, enable_llama_style_head=False, hidden_dim=0,
-                 multiple_of=64, enable_layernorm_cuda_impl=True, fused_rmsnorm=False):
+                 multiple_of=64, enable_layernorm_cuda_impl=True, fused_rmsnorm=False, block_type="causal_self_attention",
+                 enable_key_value_cache=False):
+        if block_type not in ("causal_self_attention", "encoder"):
+            raise ValueError(block_type)
         self.cuda = cuda
+        self.block_type = block_type
         self.llama = enable_llama_style_head
         if self.llama:
             # RMSNorm, rotary attention without bias, SiLU-gated MLP (TransformerBlockLayer.cs:86-98, 239-247, 860-875)
@@ -718,8 +724,13 @@ class TransformerBlockLayer:
             self.norm1 = LayerNormLayer(cuda, epsilon, enable_layernorm_cuda_impl)
             self.norm2 = LayerNormLayer(cuda, epsilon, enable_layernorm_cuda_impl)
             hidden_dim = hidden_dim or 4 * embed
-        self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention,
-                                              enable_rotary_positional_embedding=self.llama, training=training)
+        if block_type == "encoder":
+            self.attn1 = MultiheadAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention,
+                                                 enable_rotary_positional_embedding=self.llama,
+                                                 enable_key_value_cache=enable_key_value_cache)
+        else:
+            self.attn1 = CausalSelfAttentionLayer(cuda, heads, embed, block_size, bias_term, enable_cuda_scaled_dot_product_attention,
+                                                  enable_rotary_positional_embedding=self.llama, training=training)
         self.fc1 = InnerProductLayer(cuda, hidden_dim, bias_term, 2)
         self.fc2 = InnerProductLayer(cuda, hidden_dim, bias_term, 2) if self.llama else None
         self.proj = InnerProductLayer(cuda, embed, bias_term, 2)
@@ -727,8 +738,12 @@ class TransformerBlockLayer:
         self.b = {n: Blob(cuda) for n in "Norm1 Attn1 X Norm2 NormA Mlp1 Mlp2 Mlp3 MlpOut".split()}
 
     def Setup(self, bottom, p):
-        """``p``: attn_weight, attn_bias, attn_proj_weight, attn_proj_bias, fc_weight, fc_bias, proj_weight, proj_bias."""
-        self.attn1.Setup(bottom, p["attn_weight"], p.get("attn_bias"), p["attn_proj_weight"], p.get("attn_proj_bias"))
+        """``p``: attn_weight, attn_bias, attn_proj_weight, attn_proj_bias (ENCODER type: wq, bq, wk, bk, wv, bv, wo, bo),
+        fc_weight, fc_bias, proj_weight, proj_bias; Llama style also fc2_weight, rms1_weight, rms2_weight."""
+        if self.block_type == "encoder":
+            self.attn1.Setup(bottom, bottom, bottom, p)
+        else:
+            self.attn1.Setup(bottom, p["attn_weight"], p.get("attn_bias"), p["attn_proj_weight"], p.get("attn_proj_bias"))
         self.fc1.Setup(bottom, p["fc_weight"], p.get("fc_bias"))
         if self.llama:
             self.fc2.Setup(bottom, p["fc2_weight"], p.get("fc2_bias"))
@@ -738,11 +753,19 @@ class TransformerBlockLayer:
         self.proj.Setup(hidden, p["proj_weight"], p.get("proj_bias"))
         hidden.Dispose()
 
-    def Forward(self, blobX, top):
+    def SetLayerOption(self, name, value):
+        """Layer options reach the attention layer (TransformerBlockLayer.cs SetLayerOption override)."""
+        if self.block_type == "encoder":
+            self.attn1.SetLayerOption(name, value)
+
+    def Forward(self, blobX, top, blobXMask=None):
         b, cuda = self.b, self.cuda
         nCount = blobX.count()
         self.norm1.Forward(blobX, b["Norm1"])
-        self.attn1.Forward(b["Norm1"], b["Attn1"])
+        if self.block_type == "encoder":
+            self.attn1.Forward(b["Norm1"], b["Norm1"], b["Norm1"], blobXMask, b["Attn1"])
+        else:
+            self.attn1.Forward(b["Norm1"], b["Attn1"])
         b["X"].ReshapeLike(blobX)
         cuda.add(nCount, blobX.gpu_data, b["Attn1"].gpu_data, b["X"].gpu_data)
         self.norm2.Forward(b["X"], b["Norm2"])
@@ -760,6 +783,8 @@ class TransformerBlockLayer:
 
     def Backward(self, top, blobX):
         """TransformerBlockLayer.cs:924-1040, CAUSAL_SELF_ATTENTION block: top.gpu_diff -> blobX.gpu_diff."""
+        if self.block_type != "causal_self_attention":
+            raise NotImplementedError("backward is mirrored for the CAUSAL_SELF_ATTENTION block type")
         b, cuda = self.b, self.cuda
         nCount = blobX.count()
         cuda.copy(nCount, top.gpu_diff, b["MlpOut"].gpu_diff)

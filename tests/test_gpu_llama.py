@@ -293,3 +293,47 @@ def test_sampled_text_generation_matches_checker(tmp_path):
         assert got.encode("utf-8") == ref.decode("utf-8", errors="replace").encode("utf-8"), (text, got, ref)
     inf.CleanUp()
     cuda.Dispose()
+
+
+def test_llama_decode_through_the_layer_call_sequences_matches_the_checker(dev):
+    """The route the C# model builder's networks take (TestModelBuilder.cs:745-790: "position" layer option, one token
+    per forward): embedding, Llama-style ENCODER transformer blocks (RMSNorm chain, MultiheadAttentionLayer with rotary
+    embedding and its key / value cache loop, SiLU-gated MLP), final RMSNorm, classifier InnerProduct - every step an
+    ABI call of the reference's own sequence - against the CPU checker's logits, token by token."""
+    from mycaffe_amd.layers import Blob, InnerProductLayer, RMSNormLayer, TransformerBlockLayer
+    cfg = dict(dim=96, hidden_dim=256, n_layers=2, n_heads=3, n_kv_heads=3, vocab_size=320, seq_len=16)
+    blob, w = O.random_weights(cfg, seed=11, std=0.2)
+    w["rms_att"][...] = 1 + 0.1 * np.random.default_rng(1).standard_normal(w["rms_att"].shape).astype(np.float32)
+    w["rms_ffn"][...] = 1 + 0.1 * np.random.default_rng(2).standard_normal(w["rms_ffn"].shape).astype(np.float32)
+    w["rms_final"][...] = 1 + 0.1 * np.random.default_rng(3).standard_normal(w["rms_final"].shape).astype(np.float32)
+    ref = O.Llama(cfg, blob, False)
+    cuda, dim, V = dev.cuda, cfg["dim"], cfg["vocab_size"]
+    x, top = Blob(cuda, (1, 1, dim)), Blob(cuda)
+    blocks = []
+    for l in range(cfg["n_layers"]):
+        blk = TransformerBlockLayer(cuda, cfg["n_heads"], dim, cfg["seq_len"], "silu", False, 1e-5, False,
+                                    enable_llama_style_head=True, hidden_dim=cfg["hidden_dim"], block_type="encoder",
+                                    enable_key_value_cache=True)
+        blk.Setup(x, {"wq": w["wq"][l], "wk": w["wk"][l], "wv": w["wv"][l], "wo": w["wo"][l], "rms1_weight": w["rms_att"][l],
+                      "rms2_weight": w["rms_ffn"][l], "fc_weight": w["w1"][l], "fc2_weight": w["w3"][l], "proj_weight": w["w2"][l]})
+        blocks.append(blk)
+    norm = RMSNormLayer(cuda, 1e-5, True)
+    norm.Setup(x, w["rms_final"])
+    cls = InnerProductLayer(cuda, V, False, 2)
+    cls.Setup(x, w["wcls"])
+    hEmb = dev.put(w["tok_emb"])
+    hTok = dev.put(np.zeros(1, np.float32))
+    tokens = [5, 200, 17, 301, 9, 64, 2, 111]
+    a, b, logits = Blob(cuda, (1, 1, dim)), Blob(cuda, (1, 1, dim)), Blob(cuda)
+    for pos, tok in enumerate(tokens):
+        cuda.SetMemory(hTok, np.array([tok], np.float32))
+        cuda.embed_fwd(dim, hTok, hEmb, 1, dim, V, a.gpu_data)
+        for blk in blocks:
+            blk.SetLayerOption("position", pos)
+            blk.Forward(a, b)
+            a, b = b, a
+        norm.Forward(a, top)
+        cls.Forward(top, logits)
+        exp = ref.forward(tok, pos)
+        assert_close(logits.mutable_cpu_data.reshape(-1), exp, FP32_RTOL, "logits at position %d" % pos)
+        assert int(np.argmax(logits.mutable_cpu_data)) == int(np.argmax(exp))
