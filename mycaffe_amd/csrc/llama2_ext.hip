@@ -86,6 +86,27 @@ template <> struct Row4<bf16_t> {
     }
 };
 
+template <typename T> struct Row8;
+template <> struct Row8<float> {
+    __device__ static inline void load(const float* p, float* w)
+    {
+        const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+    }
+};
+template <> struct Row8<bf16_t> {
+    __device__ static inline void load(const bf16_t* p, float* w)
+    {
+        const uint4 u = *(const uint4*)p;
+        const uint32_t v[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[2 * i] = __uint_as_float(v[i] << 16);
+            w[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+        }
+    }
+};
+
 // Mat-vec family for one token per sequence.  One wavefront owns ROWS output rows
 // of W (n columns, n % 4 == 0) and walks them with 128-bit (fp32) / 64-bit (bf16)
 // loads; the activation chunk a lane needs is the same for every row, so it is
@@ -95,11 +116,19 @@ template <> struct Row4<bf16_t> {
 //   MODE 2: y[b,r]  = silu(W[r,:] . xn) * (W[r+half,:] . xn)   (SwiGLU epilogue, half = rows)
 // NORM: xn = g * x / sqrt(mean(x^2) + 1e-5), recomputed per wavefront from the
 // chunks it already holds (x is L2 resident; it saves a launch and a barrier).
-template <typename T, int MODE, bool NORM, int CH, int ROWS>
+// WIDE (bf16 weights, n % 8 == 0): a lane takes 8 consecutive weights per load (16 bytes, two of the CH float4 slots),
+// so 16-bit weights move in as few load instructions per byte as fp32 ones.
+template <bool WIDE> __device__ __forceinline__ int matvec_col(int c, int lane)
+{
+    return WIDE ? ((c >> 1) * 64 + lane) * 8 + (c & 1) * 4 : (c * 64 + lane) * 4;
+}
+
+template <typename T, int MODE, bool NORM, int CH, int ROWS, bool WIDE = false>
 __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, const float* __restrict__ x,
                                                      const float* __restrict__ g, float* __restrict__ y, int rows, int n,
                                                      int B, int ldy)
 {
+    static_assert(!WIDE || (sizeof(T) == 2 && CH % 2 == 0), "wide loads are for 16-bit weights, two slots per load");
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int r0 = wave * ROWS;
@@ -109,15 +138,33 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
 #pragma unroll
     for (int rr = 0; rr < ROWS; rr++) {
         const int r = min(r0 + rr, rows - 1);
+        if (WIDE) {
 #pragma unroll
-        for (int c = 0; c < CH; c++) {
-            const int j = (c * 64 + lane) * 4;
-            if (j < n) {
-                w[rr][c] = Row4<T>::load(W + (size_t)r * n + j);
-                if (MODE == 2) w[ROWS + rr][c] = Row4<T>::load(W + (size_t)(r + rows) * n + j);
-            } else {
-                w[rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (MODE == 2) w[ROWS + rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int c = 0; c < CH; c += 2) {
+                const int j = matvec_col<WIDE>(c, lane);
+                float lo[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, hi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                if (j < n) {
+                    Row8<T>::load(W + (size_t)r * n + j, lo);
+                    if (MODE == 2) Row8<T>::load(W + (size_t)(r + rows) * n + j, hi);
+                }
+                w[rr][c] = make_float4(lo[0], lo[1], lo[2], lo[3]);
+                w[rr][c + 1] = make_float4(lo[4], lo[5], lo[6], lo[7]);
+                if (MODE == 2) {
+                    w[ROWS + rr][c] = make_float4(hi[0], hi[1], hi[2], hi[3]);
+                    w[ROWS + rr][c + 1] = make_float4(hi[4], hi[5], hi[6], hi[7]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const int j = matvec_col<WIDE>(c, lane);
+                if (j < n) {
+                    w[rr][c] = Row4<T>::load(W + (size_t)r * n + j);
+                    if (MODE == 2) w[ROWS + rr][c] = Row4<T>::load(W + (size_t)(r + rows) * n + j);
+                } else {
+                    w[rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (MODE == 2) w[ROWS + rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
             }
         }
     }
@@ -127,7 +174,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
         float ss = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
-            const int j = (c * 64 + lane) * 4;
+            const int j = matvec_col<WIDE>(c, lane);
             xv[c] = j < n ? *(const float4*)(xb + j) : make_float4(0.f, 0.f, 0.f, 0.f);
             if (NORM) ss += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
         }
@@ -136,7 +183,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
             const float inv = 1.0f / sqrtf(ss / n + 1e-5f);
 #pragma unroll
             for (int c = 0; c < CH; c++) {
-                const int j = (c * 64 + lane) * 4;
+                const int j = matvec_col<WIDE>(c, lane);
                 if (j < n) {
                     const float4 gv = *(const float4*)(g + j);
                     xv[c].x = gv.x * (inv * xv[c].x);
@@ -179,27 +226,6 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
 // scale of the result, so the sum of squares is gathered from the x values that pass through anyway and g is
 // folded into x.  Partial tiles of the wavefronts meet in LDS; wavefront 0 finishes.
 typedef float floatx4v __attribute__((ext_vector_type(4)));
-
-template <typename T> struct Row8;
-template <> struct Row8<float> {
-    __device__ static inline void load(const float* p, float* w)
-    {
-        const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
-        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
-    }
-};
-template <> struct Row8<bf16_t> {
-    __device__ static inline void load(const bf16_t* p, float* w)
-    {
-        const uint4 u = *(const uint4*)p;
-        const uint32_t v[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w[2 * i] = __uint_as_float(v[i] << 16);
-            w[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
-        }
-    }
-};
 
 template <typename T, int MODE, bool NORM>
 __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
@@ -726,18 +752,27 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     const bool two = rowsPerWave ? rowsPerWave == 2 : rows >= 16384;
     const int waves = two ? (rows + 1) / 2 : rows;
     const int grid = (waves + 3) / 4;
-    const int ch = (n / 4 + 63) / 64;
+    const bool wide = sizeof(T) == 2 && n % 8 == 0 && (((uintptr_t)W) & 15) == 0;
+    const int ch = wide ? 2 * ((n / 8 + 63) / 64) : (n / 4 + 63) / 64;
+#define MV1(C, WIDE_)                                                                                                      \
+    do {                                                                                                                   \
+        if (two) hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 2, WIDE_>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy); \
+        else hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 1, WIDE_>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy);     \
+    } while (0)
 #define MV(C)                                                                                                              \
     do {                                                                                                                   \
-        if (two) hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 2>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy); \
-        else hipLaunchKernelGGL((matvec_kernel<T, MODE, NORM, C, 1>), grid, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy);     \
+        if constexpr (sizeof(T) == 2 && (C) % 2 == 0) {                                                                    \
+            if (wide) { MV1(C, true); break; }                                                                             \
+        }                                                                                                                  \
+        MV1(C, false);                                                                                                     \
     } while (0)
     if (ch <= 2) MV(2);
-    else if (ch <= 3) MV(3);
+    else if (ch <= 3 && !wide) MV(3);
     else if (ch <= 4) MV(4);
     else if (ch <= 8) MV(8);
     else if (ch <= 16) MV(16);
     else return hipErrorInvalidValue;
+#undef MV1
 #undef MV
     return hipGetLastError();
 }
