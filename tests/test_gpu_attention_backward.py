@@ -141,3 +141,20 @@ def test_attn_backward_large_scores(dev):
     q *= 6.0   # scores in the hundreds: probabilities are nearly one-hot
     out = _fwd_bwd(dev, q, k, v, dy, R.causal_mask(T), 0)
     _check(out, q, k, v, dy, R.causal_mask(T), 0, FP32_RTOL, "large scores")
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_causal_launch_order_does_not_change_results(dev, half):
+    """A causal launch large enough for the reordered dispatch rounds (384 workgroups: the second round of 32 per XCD is
+    dealt backwards) gives, head by head, exactly what small launches of the same heads give (which keep the plain
+    order), forward and backward."""
+    rng = np.random.default_rng(61)
+    B, H, T, hs = 4, 12, 1024, 64
+    q, k, v, dy = (bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(4))
+    mask = R.causal_mask(T)
+    big = _fwd_bwd(dev, q, k, v, dy, mask, 0, half)
+    for b, h0 in ((0, 0), (3, 9), (2, 5)):
+        sl = (slice(b, b + 1), slice(h0, h0 + 3))
+        small = _fwd_bwd(dev, q[sl], k[sl], v[sl], dy[sl], mask, 0, half)
+        for got, exp, name in zip(big, small, ("y", "dq", "dk", "dv")):
+            assert np.array_equal(got[sl], exp), name
