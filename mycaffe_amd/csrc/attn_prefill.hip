@@ -306,6 +306,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
         }
     };
 
+    // Key-padding masks: a 32-key step whose keys are all masked adds exact zeros once the sequence has a valid key
+    // anywhere (its weights underflow against any real maximum), so such steps are skipped, and steps without a masked
+    // key take the unmasked path.  A sequence with no valid key at all keeps every step (uniform weights, as the
+    // reference's -1e29 fill gives).
+    bool seqValid = false;
+    if (KIND == 2) {
+        int any = 0;
+        for (int t = tid; t < a.Tk; t += NT) any |= a.mask[(size_t)b * a.Tk + t] != 0.f;
+        seqValid = __syncthreads_or(any) != 0;
+    }
     gload(0);
     sstore(0);
     // make the Q fragments "used" here, so the wait for their loads sits before the loop and the
@@ -319,12 +329,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
     const float c = a.c;
     for (int kb = 0; kb < nkb; kb++) {
         if (PREFETCH && kb + 1 < nkb) gload(kb + 1);
+        unsigned long long zeros = 0;      // bit = key of this block is masked (KIND 2)
+        if (KIND == 2) zeros = __ballot(Ms[lane] == 0.f);
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const int k0 = kb * BN + 32 * sub;
             // causal: this wavefront's last row is q0 + 32*QT - 1; keys past it contribute nothing
             const bool active = (KIND != 1) || (k0 <= q0 + 32 * QT - 1);
-            if (active && k0 < a.Tk) {
+            const unsigned subZeros = (unsigned)(zeros >> (32 * sub));
+            const bool skip = KIND == 2 && seqValid && subZeros == 0xffffffffu;
+            if (active && k0 < a.Tk && !skip) {
                 floatx16 s[QT];
 #pragma unroll
                 for (int qt = 0; qt < QT; qt++)
@@ -337,7 +351,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                     for (int qt = 0; qt < QT; qt++) s[qt] = TR::mma(kf, qf[qt][f], s[qt]);
                 }
                 // register v holds key k0 + 8*(v/4) + 4*half + v%4 for query q0 + 32*qt + l32
-                const bool maskedBlock = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk) || KIND >= 2;   // wavefront-uniform
+                const bool maskedBlock = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk) || KIND == 3 ||
+                                         (KIND == 2 && subZeros != 0);   // wavefront-uniform
                 if (maskedBlock) {
 #pragma unroll
                     for (int qt = 0; qt < QT; qt++) {
