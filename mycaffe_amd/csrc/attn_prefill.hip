@@ -357,6 +357,24 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 #pragma unroll
                     for (int qt = 0; qt < QT; qt++) {
                         const int qrow = q0 + qt * 32 + l32;
+                        // KIND 3: the lane's 16 keys are four runs of four; with whole, aligned runs each is one
+                        // 16-byte load of the mask row instead of four scalar ones
+                        float mk[16];
+                        if (KIND == 3) {
+                            const float* mrow = a.mask + ((size_t)b * a.maskBatch * a.Tq + min(qrow, a.Tq - 1)) * a.Tk;
+                            const bool vec = (a.Tk & 3) == 0 && k0 + 32 <= a.Tk && (((uintptr_t)a.mask) & 15) == 0;
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                const int kq = k0 + 8 * g + 4 * half;
+                                if (vec) {
+                                    const float4 t = *(const float4*)(mrow + kq);
+                                    mk[4 * g] = t.x; mk[4 * g + 1] = t.y; mk[4 * g + 2] = t.z; mk[4 * g + 3] = t.w;
+                                } else {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) mk[4 * g + e] = kq + e < a.Tk ? mrow[kq + e] : 1.f;
+                                }
+                            }
+                        }
 #pragma unroll
                         for (int v = 0; v < 16; v++) {
                             const int kl = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -364,8 +382,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                             float sv = s[qt][v];
                             if (KIND == 1 && key > qrow) sv = a.maskedRaw;
                             if (KIND == 2 && Ms[32 * sub + kl] == 0.f) sv = a.maskedRaw;
-                            if (KIND == 3 && qrow < a.Tq && key < a.Tk && a.mask[((size_t)b * a.maskBatch * a.Tq + qrow) * a.Tk + key] == 0.f)
-                                sv = a.maskedRaw;
+                            if (KIND == 3 && qrow < a.Tq && key < a.Tk && mk[v] == 0.f) sv = a.maskedRaw;
                             if (key >= a.Tk) sv = -INFINITY;
                             s[qt][v] = sv;
                         }
