@@ -319,12 +319,13 @@ def bench_encdec_attention(cuda, reps, warm=5):
 
 
 def bench_gemm(cuda, reps):
-    """QKV (8192 x 2304 x 768) and output projection (8192 x 768 x 768) GEMMs, weights [N, K]."""
+    """QKV (8192 x 2304 x 768) and output projection (8192 x 768 x 768) GEMMs of the causal self attention layer and one
+    projection of the encoder-decoder attention layer (8192 x 512 x 512), weights [N, K]."""
     from mycaffe_amd.cudadnn import CUDAFN
     out = {}
     rng = np.random.default_rng(0)
     for name, half in (("bf16", True), ("f32", False)):
-        for tag, (M, N, K) in (("qkv", (8192, 2304, 768)), ("proj", (8192, 768, 768))):
+        for tag, (M, N, K) in (("qkv", (8192, 2304, 768)), ("proj", (8192, 768, 768)), ("mha_proj_d512", (8192, 512, 512))):
             a = cuda.AllocMemory(rng.standard_normal(M * K).astype(np.float32), bHalfSize=half)
             w = cuda.AllocMemory((rng.standard_normal(N * K) * 0.02).astype(np.float32), bHalfSize=half)
             c = cuda.AllocMemory(M * N, bHalfSize=half)
