@@ -147,26 +147,27 @@ hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b
 hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y) { return launch_map(s, dt, n, x, nullptr, y, SiluF{}); }
 hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y) { return launch_map(s, dt, n, a, b, y, SwigluF{}); }
 
-// y[i] = mask[i % maskDim] == search ? replace : x[i]
+// y[i] = mask[i % maskDim] == search ? replace : xscale * x[i]   (xscale: a scaling of x that the caller had deferred; 1 otherwise)
 template <typename T>
-__global__ void mask_kernel(size_t n, int maskDim, const T* x, const T* mask, T* y, float search, float replace)
+__global__ void mask_kernel(size_t n, int maskDim, const T* x, const T* mask, T* y, float search, float replace, float xscale)
 {
-    GRID_STRIDE(i, n) st(y, i, ld(mask, i % (size_t)maskDim) == search ? replace : ld(x, i));
+    GRID_STRIDE(i, n) st(y, i, ld(mask, i % (size_t)maskDim) == search ? replace : xscale * ld(x, i));
 }
 // mask index = i % md1 + (i / dd1) * md1 (md1 = maskDim / batch, dd1 = n / batch); the plain mask is the case dd1 = n
 template <typename T>
 __global__ void mask_batch_kernel(size_t n, int md1, size_t dd1, const T* x, const T* mask, T* y, float search,
-                                  float replace)
+                                  float replace, float xscale)
 {
     GRID_STRIDE(i, n)
     {
         size_t mi = i % (size_t)md1 + (i / dd1) * (size_t)md1;
-        st(y, i, ld(mask, mi) == search ? replace : ld(x, i));
+        st(y, i, ld(mask, mi) == search ? replace : xscale * ld(x, i));
     }
 }
 // eight elements per thread: needs md1 and dd1 to be multiples of 8 (a chunk never wraps) and 16-byte aligned operands
 template <typename T>
-__global__ void mask_vec_kernel(size_t chunks, size_t md8, size_t dd8, const T* x, const T* mask, T* y, float search, float replace)
+__global__ void mask_vec_kernel(size_t chunks, size_t md8, size_t dd8, const T* x, const T* mask, T* y, float search, float replace,
+                                float xscale)
 {
     GRID_STRIDE(c, chunks)
     {
@@ -175,38 +176,38 @@ __global__ void mask_vec_kernel(size_t chunks, size_t md8, size_t dd8, const T* 
         Vec8<T>::load(x + c * 8, vx);
         Vec8<T>::load(mask + mc * 8, vm);
 #pragma unroll
-        for (int k = 0; k < 8; k++) vx[k] = vm[k] == search ? replace : vx[k];
+        for (int k = 0; k < 8; k++) vx[k] = vm[k] == search ? replace : xscale * vx[k];
         Vec8<T>::store(y + c * 8, vx);
     }
 }
 static hipError_t launch_mask(hipStream_t s, DType dt, size_t n, int md1, size_t dd1, float search, float replace, const void* x,
-                              const void* mask, void* y)
+                              const void* mask, void* y, float xscale)
 {
     const bool vec = md1 % 8 == 0 && dd1 % 8 == 0 && n % 8 == 0 && ((((uintptr_t)x | (uintptr_t)mask | (uintptr_t)y) & 15) == 0);
     if (vec) {
         DISPATCH_DT(dt, hipLaunchKernelGGL(mask_vec_kernel<T>, grid_for(n / 8), TPB, 0, s, n / 8, (size_t)md1 / 8, dd1 / 8, (const T*)x,
-                                           (const T*)mask, (T*)y, search, replace));
+                                           (const T*)mask, (T*)y, search, replace, xscale));
     } else {
         DISPATCH_DT(dt, hipLaunchKernelGGL(mask_batch_kernel<T>, grid_for(n), TPB, 0, s, n, md1, dd1, (const T*)x, (const T*)mask,
-                                           (T*)y, search, replace));
+                                           (T*)y, search, replace, xscale));
     }
     return hipGetLastError();
 }
 hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
-                  const void* mask, void* y)
+                  const void* mask, void* y, float xscale)
 {
     if (n == 0) return hipSuccess;
     if (maskDim % 8 == 0 && n % (size_t)maskDim == 0)
-        return launch_mask(s, dt, n, maskDim, n, search, replace, x, mask, y);   // i % maskDim with dd1 = n: one "batch"
+        return launch_mask(s, dt, n, maskDim, n, search, replace, x, mask, y, xscale);   // i % maskDim with dd1 = n: one "batch"
     DISPATCH_DT(dt, hipLaunchKernelGGL(mask_kernel<T>, grid_for(n), TPB, 0, s, n, maskDim, (const T*)x, (const T*)mask,
-                                       (T*)y, search, replace));
+                                       (T*)y, search, replace, xscale));
     return hipGetLastError();
 }
 hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDim, float search, float replace,
-                        const void* x, const void* mask, void* y)
+                        const void* x, const void* mask, void* y, float xscale)
 {
     if (n == 0) return hipSuccess;
-    return launch_mask(s, dt, n, maskDim / batch, n / (size_t)batch, search, replace, x, mask, y);
+    return launch_mask(s, dt, n, maskDim / batch, n / (size_t)batch, search, replace, x, mask, y, xscale);
 }
 
 // Generic permute: xc / yc hold the element strides of the source / destination

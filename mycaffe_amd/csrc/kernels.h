@@ -40,9 +40,9 @@ hipError_t k_mul(hipStream_t s, DType dt, size_t n, const void* a, const void* b
 hipError_t k_silu(hipStream_t s, DType dt, size_t n, const void* x, void* y);
 hipError_t k_swiglu(hipStream_t s, DType dt, size_t n, const void* a, const void* b, void* y);
 hipError_t k_mask(hipStream_t s, DType dt, size_t n, int maskDim, float search, float replace, const void* x,
-                  const void* mask, void* y);
+                  const void* mask, void* y, float xscale = 1.0f);
 hipError_t k_mask_batch(hipStream_t s, DType dt, size_t n, int batch, int maskDim, float search, float replace,
-                        const void* x, const void* mask, void* y);
+                        const void* x, const void* mask, void* y, float xscale = 1.0f);
 hipError_t k_transpose(hipStream_t s, DType dt, size_t n, const void* x, void* y, const float* xc, const float* yc,
                        const float* map, int axes);
 // the two halves of k_transpose: fetching the stride / map blobs costs a device round trip, so callers keep the result

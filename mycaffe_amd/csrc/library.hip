@@ -106,6 +106,7 @@ long MemTable::alloc_view(long hBase, size_t offset, size_t count, long* h)
     it = MemItem();
     it.ptr = p; it.count = count; it.half = half; it.used = true; it.view = true; it.base = root;
     it.version = ++m_clock;
+    m_items[root].views++;
     *h = slot;
     return 0;
 }
@@ -127,6 +128,8 @@ long MemTable::free(long h)
             if (m_items[i].used && m_items[i].view && m_items[i].base == h) { m_items[i] = MemItem(); m_free.push_back((long)i); }
         hipError_t e = hipFree(it->ptr);
         if (e != hipSuccess) return (long)e;
+    } else if (it->base > 0 && (size_t)it->base < m_items.size() && m_items[it->base].used) {
+        m_items[it->base].views--;
     }
     *it = MemItem();
     m_free.push_back(h);
@@ -280,6 +283,37 @@ long Kernel::free_host(float* p)
     return MCH_ERROR_MEMORY_NOT_FOUND;
 }
 
+long Kernel::mem(long h, MemItem** it)
+{
+    ERRCHK(m_mem.get(h, it));
+    MemItem* root = *it;
+    if (root->view && m_mem.get(root->base, &root)) return 0;
+    if (root->pending != 1.f) {
+        const float a = root->pending;
+        root->pending = 1.f;
+        HIPCHK(k_scale(m_stream, root->dt(), root->count, a, root->ptr, root->ptr));
+    }
+    return 0;
+}
+
+// Operands of a mask call.  When X carries a deferred scaling and the call masks the whole tensor in place, the factor
+// is handed to the mask kernel (*xscale) instead of being applied in a pass of its own.
+long Kernel::mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale)
+{
+    *xscale = 1.f;
+    ERRCHK(mem(hM, M));
+    MemItem* x;
+    ERRCHK(mem_lazy(hX, &x));
+    if (!x->view && x->pending != 1.f && hX == hY && n > 0 && (size_t)n == x->count) {
+        *xscale = x->pending;   // the caller clears `pending` once its kernel is launched
+        *X = *Y = x;
+        return 0;
+    }
+    ERRCHK(mem(hX, X));
+    ERRCHK(mem(hY, Y));
+    return 0;
+}
+
 long Kernel::get_pointer(long h, void** pp)
 {
     MemItem* it;
@@ -413,6 +447,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         NEED_L(3, 3);
         if (pl[1] < 0 || pl[2] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         long h = 0;
+        MemItem* base;
+        ERRCHK(mem((long)pl[0], &base));   // applies a deferred scaling before the allocation gets an alias
         ERRCHK(m_mem.alloc_view((long)pl[0], (size_t)pl[1], (size_t)pl[2], &h));
         return set_out((float)h, ppOut, plOut);
     }
@@ -626,6 +662,13 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         MemItem* X;
         ERRCHK(mem((long)pl[2], &X));
         RANGE(X, xo, n);
+        if (!timing && !X->view && X->views == 0 && xo == 0 && (size_t)n == X->count && n >= (1 << 20)) {
+            // a large whole tensor: the multiplication waits for the next call that touches the tensor; the mask calls
+            // of the attention chain (scale, then mask in place) do it in their own pass
+            X->pending = pf[0];
+            m_mem.touch((long)pl[2]);
+            return 0;
+        }
         HIPCHK(k_scale(s, X->dt(), (size_t)n, pf[0], PTR(X, xo), PTR(X, xo)));
         m_mem.touch((long)pl[2]);
         return 0;
@@ -873,14 +916,14 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         int md = (int)pl[1];
         if (md < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         MemItem *X, *M, *Y;
-        ERRCHK(mem((long)pl[4], &X));
-        ERRCHK(mem((long)pl[5], &M));
-        ERRCHK(mem((long)pl[6], &Y));
+        float xscale = 1.f;
+        ERRCHK(mask_operands((long)pl[4], (long)pl[5], (long)pl[6], n, &X, &M, &Y, &xscale));
         if (X->half != M->half || X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         RANGE(X, 0, n);
         RANGE(Y, 0, n);
         RANGE(M, 0, md);
-        HIPCHK(k_mask(s, X->dt(), (size_t)n, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr));
+        HIPCHK(k_mask(s, X->dt(), (size_t)n, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
+        if (xscale != 1.f) X->pending = 1.f;
         m_mem.touch((long)pl[6]);
         return 0;
     }
@@ -893,9 +936,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         int batch = (int)pl[1], md = (int)pl[2];
         if (batch < 1 || md < batch || n < batch) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         MemItem *X, *M, *Y;
-        ERRCHK(mem((long)pl[5], &X));
-        ERRCHK(mem((long)pl[6], &M));
-        ERRCHK(mem((long)pl[7], &Y));
+        float xscale = 1.f;
+        ERRCHK(mask_operands((long)pl[5], (long)pl[6], (long)pl[7], n, &X, &M, &Y, &xscale));
         if (X->half != M->half || X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         RANGE(X, 0, n);
         RANGE(Y, 0, n);
@@ -904,7 +946,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             long long md1 = md / batch, dd1 = n / batch;
             RANGE(M, 0, (md1 - 1) + ((n - 1) / dd1) * md1 + 1);
         }
-        HIPCHK(k_mask_batch(s, X->dt(), (size_t)n, batch, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr));
+        HIPCHK(k_mask_batch(s, X->dt(), (size_t)n, batch, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
+        if (xscale != 1.f) X->pending = 1.f;
         m_mem.touch((long)pl[7]);
         return 0;
     }

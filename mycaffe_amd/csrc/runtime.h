@@ -27,6 +27,11 @@ struct MemItem {
     bool view = false;    // aliases part of another item (memory pointer)
     long base = 0;        // owning handle when view
     uint64_t version = 0; // bumped on every write through the ABI
+    int views = 0;        // memory pointers that alias this allocation
+    // A whole-tensor SCAL that has not run yet: the contents are `pending` times what memory holds.  Only set on
+    // allocations without views; every access through Kernel::mem() applies it first, except the mask calls, which
+    // fold it into their own pass (the scale / mask pair of the explicit attention chain becomes one pass).
+    float pending = 1.f;
     DType dt() const { return half ? BF16 : F32; }
     size_t esize() const { return half ? 2 : 4; }
 };
@@ -138,7 +143,9 @@ private:
     long workspace(size_t bytes, void** p);
     long staging(size_t bytes, void** p);
     long tickets(size_t count, int** p);
-    long mem(long h, MemItem** it) { return m_mem.get(h, it); }
+    long mem(long h, MemItem** it);                                            // with any deferred scaling applied
+    long mem_lazy(long h, MemItem** it) { return m_mem.get(h, it); }           // as it is; the caller deals with `pending`
+    long mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale);
     bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
 
     int m_device = 0;

@@ -499,3 +499,71 @@ def test_embed_and_rmsnorm(dev):
     assert_close(dev.get(hy), R.rmsnorm_layer(x, w, 1e-5, np.float64), 1e-5, "rmsnorm")
     dev.cuda.RmsNormForward(9, 288, hx, 0, hy, 1e-5)
     assert_close(dev.get(hy), R.rmsnorm_layer(x, None, 1e-5, np.float64), 1e-5, "rmsnorm no weight")
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_whole_tensor_scal_is_deferred_without_changing_any_result(dev, half):
+    """A SCAL over a large whole tensor is held back until the tensor is next touched (the mask calls fold it into their
+    pass).  Whatever touches the tensor afterwards sees exactly what an immediate multiplication would have left."""
+    rng = np.random.default_rng(71)
+    cuda = dev.cuda
+    n, md = 1 << 20, 4096
+    x = bf16_round(rng.standard_normal(n).astype(np.float32))
+    m = (rng.random(md) > 0.3).astype(np.float32)
+    alpha = np.float32(0.125) if half else np.float32(0.3)
+    scaled = bf16_round(x * alpha) if half else x * alpha
+    hm = dev.put(m, half)
+
+    def fresh():
+        return dev.put(x, half)
+
+    # read back
+    h = fresh()
+    cuda.scal(n, float(alpha), h)
+    assert np.array_equal(dev.get(h), scaled)
+    # mask in place: one pass
+    h = fresh()
+    cuda.scal(n, float(alpha), h)
+    cuda.mask(n, md, 0.0, -1e29, h, hm, h)
+    exp = np.where(np.tile(m, n // md) == 0, np.float32(-1e29), scaled)
+    if half:
+        exp = bf16_round(exp)
+    assert np.array_equal(dev.get(h), exp)
+    # mask_batch in place
+    h = fresh()
+    cuda.scal(n, float(alpha), h)
+    mb = (rng.random(2 * md) > 0.3).astype(np.float32)
+    hmb = dev.put(mb, half)
+    cuda.mask_batch(n, 2, 2 * md, 0.0, -1e29, h, hmb, h)
+    idx = np.arange(n) % md + (np.arange(n) // (n // 2)) * md
+    exp = np.where(mb[idx] == 0, np.float32(-1e29), scaled)
+    assert np.array_equal(dev.get(h), bf16_round(exp) if half else exp)
+    # mask into another tensor: the source ends up scaled as well
+    h, hy = fresh(), dev.zeros(n, half)
+    cuda.scal(n, float(alpha), h)
+    cuda.mask(n, md, 0.0, 7.0, h, hm, hy)
+    assert np.array_equal(dev.get(hy), np.where(np.tile(m, n // md) == 0, np.float32(7.0), scaled))
+    assert np.array_equal(dev.get(h), scaled)
+    # two in a row, a copy, a memory pointer created afterwards, an element-wise consumer
+    h, hc = fresh(), dev.zeros(n, half)
+    cuda.scal(n, float(alpha), h)
+    cuda.scal(n, 2.0, h)
+    twice = bf16_round(scaled * np.float32(2.0)) if half else scaled * np.float32(2.0)
+    cuda.copy(n, h, hc)
+    assert np.array_equal(dev.get(hc), twice)
+    h = fresh()
+    cuda.scal(n, float(alpha), h)
+    hv = cuda.CreateMemoryPointer(h, 16, 64)
+    assert np.array_equal(dev.get(hv), scaled[16:80])
+    # with a memory pointer alive the multiplication is immediate, and visible through the pointer
+    cuda.scal(n, 2.0, h)
+    assert np.array_equal(dev.get(hv), twice[16:80])
+    cuda.FreeMemoryPointer(hv)
+    h, hb = fresh(), dev.put(np.ones(n, np.float32), half)
+    cuda.scal(n, float(alpha), h)
+    cuda.mul(n, h, hb, hb)
+    assert np.array_equal(dev.get(hb), scaled)
+    # freed while the multiplication is still pending
+    h = fresh()
+    cuda.scal(n, float(alpha), h)
+    cuda.FreeMemory(h)
