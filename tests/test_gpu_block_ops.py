@@ -246,6 +246,11 @@ def test_causal_self_attention_layer_backward_golden(dev, name, heads, sdpa):
     assert_close(layer.b["Kt"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_kt.txt")), 2e-5, "grad k")
     assert_close(layer.b["Vt"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_vt.txt")), 2e-5, "grad v")
     assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(g, "grad_x.txt")), 2e-5, "grad x")
+    if not sdpa:
+        # the explicit chain's own intermediates: gradient of the probabilities, of the (scaled) scores, of k^T
+        assert_close(layer.b["AttB"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_att_after_softmax.txt")), 2e-5, "grad att")
+        assert_close(layer.b["AttA"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_qkt.txt")), 2e-5, "grad q k^T")
+        assert_close(layer.b["Kt1"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_kt1.txt")), 2e-5, "grad k^T")
 
 
 @pytest.mark.parametrize("sdpa", [True, False])
