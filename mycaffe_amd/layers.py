@@ -539,7 +539,7 @@ class LayerNormLayer:
         self.cuda, self.epsilon, self.enable_cuda_impl = cuda, epsilon, enable_cuda_impl
         self.hLayerNorm = 0
         self._shape = None
-        self.b = {n: Blob(cuda) for n in "Mu Xmu XmuSq Var Stdev StdevFull".split()}
+        self.b = {n: Blob(cuda) for n in "Mu Xmu XmuSq Var Stdev StdevFull Work".split()}
 
     def _reshape(self, bottom):
         nAxis = len(bottom.shape_) - 1
@@ -577,9 +577,23 @@ class LayerNormLayer:
         cuda.div(n, b["Xmu"].gpu_data, b["StdevFull"].gpu_data, top.gpu_data)
 
     def Backward(self, top, bottom):
-        if not self.enable_cuda_impl:
-            raise NotImplementedError("the explicit chain's backward is not mirrored")
-        self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, top.gpu_diff, bottom.gpu_diff)
+        if self.enable_cuda_impl:
+            self.cuda.LayerNormBackward(self.hLayerNorm, top.gpu_data, top.gpu_diff, bottom.gpu_diff)
+            return
+        # LayerNormLayer.cs:292-320, the layer's own chain: dx = (dy - (y * mean(y * dy) + mean(dy))) / (std + eps)
+        cuda, b = self.cuda, self.b
+        n, o, c, i = self.nCount, self.nOuterNum, self.nChannels, self.nInnerNum
+        b["Work"].ReshapeLike(top)
+        cuda.mul(n, top.gpu_data, top.gpu_diff, b["Work"].gpu_data)
+        cuda.channel_mean(n, o, c, i, b["Work"].gpu_data, b["Var"].gpu_diff)
+        cuda.channel_mean(n, o, c, i, top.gpu_diff, b["Stdev"].gpu_diff)
+        cuda.channel_fillfrom(n, o, c, i, b["Var"].gpu_diff, b["StdevFull"].gpu_diff, DIR.FWD)
+        cuda.mul(n, top.gpu_data, b["StdevFull"].gpu_diff, b["Work"].gpu_data)
+        cuda.channel_fillfrom(n, o, c, i, b["Stdev"].gpu_diff, b["StdevFull"].gpu_diff, DIR.FWD)
+        cuda.add(n, b["Work"].gpu_data, b["StdevFull"].gpu_diff, b["Work"].gpu_data)
+        cuda.sub(n, top.gpu_diff, b["Work"].gpu_data, b["Work"].gpu_data)
+        cuda.add_scalar(b["StdevFull"].count(), self.epsilon, b["StdevFull"].gpu_data)
+        cuda.div(n, b["Work"].gpu_data, b["StdevFull"].gpu_data, bottom.gpu_diff)
 
 
 class RMSNormLayer:

@@ -13,7 +13,7 @@ from tests.conftest import BF16_RTOL, FP32_RTOL, GOLDEN, assert_close, bf16_roun
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name", ["gpt-pico-ln", "gpt-pico-ln3B"])
+@pytest.mark.parametrize("name", ["gpt-pico-ln", "gpt-pico-ln3", "gpt-pico-ln3B"])
 def test_layernorm_handle_golden(dev, name):
     d = os.path.join(GOLDEN, name)
     x = load_txt(os.path.join(d, "x.txt"))
@@ -124,7 +124,7 @@ def test_rope_backward_vs_checker(dev, half):
 
 
 @pytest.mark.parametrize("sdpa", [True, False])
-@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3B", 3)])
+@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3", 3), ("gpt-pico-blk3B", 3)])
 def test_transformer_block_golden(dev, name, heads, sdpa):
     d = os.path.join(GOLDEN, name)
     p = {k: load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias",
@@ -254,7 +254,7 @@ def test_causal_self_attention_layer_backward_golden(dev, name, heads, sdpa):
 
 
 @pytest.mark.parametrize("sdpa", [True, False])
-@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3B", 3)])
+@pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3", 3), ("gpt-pico-blk3B", 3)])
 def test_transformer_block_backward_golden(dev, name, heads, sdpa):
     d = os.path.join(GOLDEN, name)
     g = os.path.join(d, "iter_0")
@@ -482,3 +482,21 @@ def test_transformer_block_llama_style_backward_vs_finite_differences(dev, sdpa)
         xm[i] -= h
         num[i] = (loss(xp) - loss(xm)) / (2 * h)
     assert_close(got, num, 2e-4, "llama block dx")
+
+
+def test_layernorm_layer_chain_intermediates_and_backward_golden(dev):
+    """LayerNormLayer's own chain (no handle) against the reference's dump of every intermediate of a minGPT LayerNorm
+    (mean, x - mean, its square, variance, standard deviation, y) and of its gradient."""
+    from mycaffe_amd.layers import LayerNormLayer
+    d = os.path.join(GOLDEN, "gpt-pico-ln-blk")
+    x = load_txt(os.path.join(d, "x.txt"))
+    layer = LayerNormLayer(dev.cuda, 1e-10, False)
+    bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+    bx.mutable_cpu_data = x
+    layer.Forward(bx, top)
+    for blob, f, tol in (("Mu", "mean", 2e-6), ("Xmu", "xmu", 2e-6), ("XmuSq", "xmusq", 2e-6), ("Var", "var1", 2e-6), ("Stdev", "std", 2e-6)):
+        assert_close(layer.b[blob].mutable_cpu_data, load_txt(os.path.join(d, f + ".txt")), tol, f)
+    assert_close(top.mutable_cpu_data, load_txt(os.path.join(d, "y.txt")), 2e-6, "y")
+    top.mutable_cpu_diff = load_txt(os.path.join(d, "iter_0", "grad_1a_y.txt"))
+    layer.Backward(top, bx)
+    assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(d, "iter_0", "grad_9_x.txt")), 2e-5, "grad x")
