@@ -784,8 +784,13 @@ hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const v
 //   log             : dx = dy - exp(y) * sum(dy)
 // inner == 1 and len % 4 == 0, len <= 2048: one wavefront per row, the row kept in registers between the two passes.
 // Forward pass of the same shape class: one wavefront per row, max, exp and sum on the registers that hold the row.
-template <typename T, int R>
-__global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int len, const T* x, T* y, bool logsm)
+// MASKED: the row is first put through a mask call that was held back for this purpose,
+//   x = mask[mi] == search ? replace : xscale * x,   mi = i % md1 + (i / dd1) * md1   (i = flat index; md1 and dd1 are
+// multiples of the row length, so a row maps to one run of mask values).
+struct SoftmaxMask { const void* mask; size_t md1, dd1; float search, replace, xscale; };
+
+template <typename T, int R, bool MASKED>
+__global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int len, const T* x, T* y, bool logsm, SoftmaxMask mk)
 {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -793,6 +798,11 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
     const int chunks = len >> 2;
     const T* xr = x + row * len;
     T* yr = y + row * len;
+    const T* mr = nullptr;
+    if (MASKED) {
+        const size_t i0 = row * (size_t)len;
+        mr = (const T*)mk.mask + i0 % mk.md1 + (i0 / mk.dd1) * mk.md1;
+    }
     float v[R][4];
     float mx = -INFINITY;
 #pragma unroll
@@ -800,6 +810,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
         const int c = lane + r * 64;
         if (c < chunks) {
             Vec4<T>::load(xr + 4 * c, v[r]);
+            if (MASKED) {
+                float mv[4];
+                Vec4<T>::load(mr + 4 * c, mv);
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[r][i] = mv[i] == mk.search ? mk.replace : mk.xscale * v[r][i];
+            }
 #pragma unroll
             for (int i = 0; i < 4; i++) mx = fmaxf(mx, v[r][i]);
         }
@@ -832,18 +848,36 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
     }
 }
 
-static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm)
+template <bool MASKED>
+static bool softmax_fwd_wave_launch_t(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, SoftmaxMask mk)
 {
-    const int R = layernorm_wave_chunks(len, x, y, y, dt == F32 ? 4 : 2);
+    const int R = layernorm_wave_chunks(len, x, y, MASKED ? mk.mask : y, dt == F32 ? 4 : 2);
     if (R == 0 || (rows + 3) / 4 > 0x7fffffffu) return false;
     const int g = (int)((rows + 3) / 4);
-#define SM_FWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((softmax_fwd_wave_kernel<T, RR>), g, 256, 0, s, rows, len, (const T*)x, (T*)y, logsm))
+#define SM_FWD(RR) DISPATCH_DT(dt, hipLaunchKernelGGL((softmax_fwd_wave_kernel<T, RR, MASKED>), g, 256, 0, s, rows, len, (const T*)x, (T*)y, logsm, mk))
     if (R == 1) SM_FWD(1);
     else if (R == 2) SM_FWD(2);
     else if (R == 4) SM_FWD(4);
     else SM_FWD(8);
 #undef SM_FWD
     return true;
+}
+static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm)
+{
+    return softmax_fwd_wave_launch_t<false>(s, dt, x, y, rows, len, logsm, SoftmaxMask());
+}
+
+// Softmax over rows of `len` of a tensor whose mask call (with its folded-in scaling) has been held back: one pass
+// instead of two.  Returns hipErrorNotSupported when the shape does not fit the one-wavefront-per-row kernel or a row
+// would straddle a wrap of the mask; the caller then runs the mask call first.
+hipError_t k_softmax_masked(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, const void* mask,
+                            size_t md1, size_t dd1, float search, float replace, float xscale)
+{
+    if (rows == 0 || len <= 0) return hipSuccess;
+    if (md1 == 0 || dd1 == 0 || md1 % (size_t)len != 0 || dd1 % (size_t)len != 0) return hipErrorNotSupported;
+    SoftmaxMask mk{mask, md1, dd1, search, replace, xscale};
+    if (!softmax_fwd_wave_launch_t<true>(s, dt, x, y, rows, len, logsm, mk)) return hipErrorNotSupported;
+    return hipGetLastError();
 }
 
 template <typename T, int R>

@@ -283,10 +283,38 @@ long Kernel::free_host(float* p)
     return MCH_ERROR_MEMORY_NOT_FOUND;
 }
 
+long Kernel::flush_pending_mask()
+{
+    const PendingMask p = m_pendingMask;
+    m_pendingMask = PendingMask();
+    if (!p.hX) return 0;
+    MemItem *X, *M;
+    if (m_mem.get(p.hX, &X) || m_mem.get(p.hM, &M)) return 0;   // an operand is gone: nothing left to apply it to
+    if (p.batch == 0) HIPCHK(k_mask(m_stream, X->dt(), (size_t)p.n, p.md, p.search, p.replace, X->ptr, M->ptr, X->ptr, p.xscale));
+    else HIPCHK(k_mask_batch(m_stream, X->dt(), (size_t)p.n, p.batch, p.md, p.search, p.replace, X->ptr, M->ptr, X->ptr, p.xscale));
+    return 0;
+}
+
+// Holds a mask call back when it masks a large whole allocation in place (the attention chain's score tensor), so that
+// the softmax that follows can do both in one pass.  The folded-in scaling of X moves into the record.
+bool Kernel::defer_mask(long hX, long hM, long hY, MemItem* X, MemItem* M, long long n, int md, int batch, float search,
+                        float replace, float xscale, bool timing)
+{
+    if (timing || hX != hY || hX == hM || X->view || X->views != 0 || M->view || (size_t)n != X->count || n < (1 << 20)) return false;
+    m_pendingMask.hX = hX; m_pendingMask.hM = hM; m_pendingMask.n = n; m_pendingMask.md = md; m_pendingMask.batch = batch;
+    m_pendingMask.search = search; m_pendingMask.replace = replace; m_pendingMask.xscale = xscale;
+    X->pending = 1.f;
+    return true;
+}
+
 long Kernel::mem(long h, MemItem** it)
 {
     ERRCHK(m_mem.get(h, it));
     MemItem* root = *it;
+    if (m_pendingMask.hX) {
+        const long hr = root->view ? root->base : h;
+        if (hr == m_pendingMask.hX || hr == m_pendingMask.hM) ERRCHK(flush_pending_mask());
+    }
     if (root->view && m_mem.get(root->base, &root)) return 0;
     if (root->pending != 1.f) {
         const float a = root->pending;
@@ -301,6 +329,7 @@ long Kernel::mem(long h, MemItem** it)
 long Kernel::mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale)
 {
     *xscale = 1.f;
+    if (m_pendingMask.hX) ERRCHK(flush_pending_mask());   // one outstanding mask call at a time
     ERRCHK(mem(hM, M));
     MemItem* x;
     ERRCHK(mem_lazy(hX, &x));
@@ -439,6 +468,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
 
     case MCH_FN_FREEMEM:
         NEED_L(1, 1);
+        if (m_pendingMask.hX == (long)pl[0]) m_pendingMask = PendingMask();       // the tensor goes: nothing to apply
+        else if (m_pendingMask.hM == (long)pl[0]) ERRCHK(flush_pending_mask());   // the mask blob goes: apply it now
         HIPCHK(hipStreamSynchronize(s));
         return m_mem.free((long)pl[0]);
 
@@ -600,7 +631,15 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         MemItem *A, *B, *C;
         ERRCHK(mem((long)pl[6], &A));
         ERRCHK(mem((long)pl[7], &B));
-        ERRCHK(mem((long)pl[9], &C));
+        // When every element of C is overwritten, a held-back scaling or mask call on C has nothing left to act on and is
+        // cancelled (once the arguments have passed their checks) instead of being run first.
+        bool overwrite = false;
+        if ((long)pl[9] != (long)pl[6] && (long)pl[9] != (long)pl[7] && (long)pl[9] != m_pendingMask.hM && pf[1] == 0.f &&
+            !mem_lazy((long)pl[9], &C) && !C->view && ldc == m && (batch == 1 || sC == (long long)m * n) &&
+            (long long)batch * m * n == (long long)C->count)
+            overwrite = true;
+        else
+            ERRCHK(mem((long)pl[9], &C));
         if (A->half || B->half || C->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;  // math.cu:1777-1778
         if (m == 0 || n == 0) return 0;
         long long ac = tA ? m : k, bc = tB ? k : n;  // stored column counts
@@ -608,6 +647,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(A, 0, (batch - 1) * sA + (ac - 1) * lda + ar);
         RANGE(B, 0, (batch - 1) * sB + (bc - 1) * ldb + br);
         RANGE(C, 0, (batch - 1) * sC + (long long)(n - 1) * ldc + m);
+        if (overwrite) {
+            C->pending = 1.f;
+            if (m_pendingMask.hX == (long)pl[9]) m_pendingMask = PendingMask();
+        }
         HIPCHK(k_gemm2(s, tA, tB, m, n, k, pf[0], (const float*)A->ptr, (const float*)B->ptr, pf[1], (float*)C->ptr, lda,
                        ldb, ldc, sA, sB, sC, batch));
         m_mem.touch((long)pl[9]);
@@ -922,6 +965,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(X, 0, n);
         RANGE(Y, 0, n);
         RANGE(M, 0, md);
+        if (defer_mask((long)pl[4], (long)pl[5], (long)pl[6], X, M, n, md, 0, pf[0], pf[1], xscale, timing)) {
+            m_mem.touch((long)pl[6]);
+            return 0;
+        }
         HIPCHK(k_mask(s, X->dt(), (size_t)n, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
         if (xscale != 1.f) X->pending = 1.f;
         m_mem.touch((long)pl[6]);
@@ -945,6 +992,11 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         {
             long long md1 = md / batch, dd1 = n / batch;
             RANGE(M, 0, (md1 - 1) + ((n - 1) / dd1) * md1 + 1);
+        }
+        if (n % batch == 0 && md % batch == 0 &&
+            defer_mask((long)pl[5], (long)pl[6], (long)pl[7], X, M, n, md, batch, pf[0], pf[1], xscale, timing)) {
+            m_mem.touch((long)pl[7]);
+            return 0;
         }
         HIPCHK(k_mask_batch(s, X->dt(), (size_t)n, batch, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
         if (xscale != 1.f) X->pending = 1.f;
@@ -1278,15 +1330,33 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                       td->sw == 1 && td->sh == td->w && td->sc == td->h * td->w && td->sn == td->c * td->h * td->w;
         if (!packed) { last_detail = "softmax needs fully packed NCHW descriptors"; return MCH_ERROR_NOT_IMPLEMENTED; }
         MemItem *X, *Y;
-        ERRCHK(mem((long)pl[3], &X));
-        ERRCHK(mem((long)pl[6], &Y));
-        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         long long total = (long long)bd->n * bd->c * bd->h * bd->w;
-        RANGE(X, 0, total);
-        RANGE(Y, 0, total);
         size_t outer = bd->n;
         int len = mode == 0 ? bd->c * bd->h * bd->w : bd->c;
         int inner = mode == 0 ? 1 : bd->h * bd->w;
+        if (m_pendingMask.hX == (long)pl[3] && (long)pl[6] != (long)pl[3] && (long)pl[6] != m_pendingMask.hM && inner == 1 &&
+            total == m_pendingMask.n) {
+            // the bottom's mask call is still outstanding: mask, scale and softmax in one pass; the bottom stays as it is
+            // (masked only on record) until something else needs it
+            MemItem* M;
+            ERRCHK(mem((long)pl[6], &Y));
+            if (m_pendingMask.hX == (long)pl[3] && !mem_lazy((long)pl[3], &X) && !mem_lazy(m_pendingMask.hM, &M) && X->half == Y->half &&
+                (size_t)total <= Y->count) {
+                const PendingMask& p = m_pendingMask;
+                const size_t md1 = p.batch ? (size_t)(p.md / p.batch) : (size_t)p.md, dd1 = p.batch ? (size_t)(p.n / p.batch) : (size_t)p.n;
+                hipError_t e = k_softmax_masked(s, X->dt(), X->ptr, Y->ptr, outer, len, alg == 2, M->ptr, md1, dd1, p.search, p.replace, p.xscale);
+                if (e == hipSuccess) {
+                    m_mem.touch((long)pl[6]);
+                    return 0;
+                }
+                if (e != hipErrorNotSupported) return (long)e;
+            }
+        }
+        ERRCHK(mem((long)pl[3], &X));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, total);
+        RANGE(Y, 0, total);
         HIPCHK(k_softmax(s, X->dt(), X->ptr, Y->ptr, outer, len, inner, alg == 2));
         m_mem.touch((long)pl[6]);
         return 0;

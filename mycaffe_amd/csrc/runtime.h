@@ -112,6 +112,15 @@ struct BlobLoaderState {
     size_t offsetItems = 0;                // advanced by ADDTOOFFSET, cleared by RESETOFFSET
     ~BlobLoaderState();
 };
+// A whole-tensor, in-place mask call (ids 264 / 266) that has not run yet: X's contents are what that call would leave.
+// At most one is outstanding.  A softmax forward over X takes it into its own pass; anything else that touches X or
+// the mask blob runs it first (Kernel::mem), a call that overwrites all of X or frees it cancels it.
+struct PendingMask {
+    long hX = 0, hM = 0;
+    long long n = 0;
+    int md = 0, batch = 0;      // batch 0: plain mask (index i % md); else mask_batch
+    float search = 0.f, replace = 0.f, xscale = 1.f;
+};
 struct PermuteCacheEntry { uint64_t key[6]; int axes; PermuteArgs args; };
 struct ExtensionState {
     void* lib = nullptr;
@@ -146,6 +155,10 @@ private:
     long mem(long h, MemItem** it);                                            // with any deferred scaling applied
     long mem_lazy(long h, MemItem** it) { return m_mem.get(h, it); }           // as it is; the caller deals with `pending`
     long mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale);
+    long flush_pending_mask();
+    bool defer_mask(long hX, long hM, long hY, MemItem* X, MemItem* M, long long n, int md, int batch, float search, float replace,
+                    float xscale, bool timing);
+    PendingMask m_pendingMask;
     bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
 
     int m_device = 0;

@@ -567,3 +567,84 @@ def test_whole_tensor_scal_is_deferred_without_changing_any_result(dev, half):
     h = fresh()
     cuda.scal(n, float(alpha), h)
     cuda.FreeMemory(h)
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_in_place_mask_is_held_back_for_the_softmax_without_changing_any_result(dev, half):
+    """An in-place mask call over a large whole tensor waits for the next call: a softmax forward over the tensor does
+    mask, folded-in scaling and softmax in one pass; whatever else touches the tensor (or the mask blob) first sees
+    exactly what the immediate call would have left; a MatMul that overwrites the tensor cancels it."""
+    rng = np.random.default_rng(72)
+    cuda = dev.cuda
+    rows, length = 1024, 1024
+    n = rows * length
+    tol = BF16_RTOL if half else FP32_RTOL
+    x = bf16_round(rng.standard_normal((rows, length)).astype(np.float32) * 4)
+    tril = np.tril(np.ones((length, length), np.float32))
+    alpha = np.float32(0.125)
+    hm = dev.put(tril, half)
+    hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+    cuda.SetTensorDesc(d, rows, length, 1, 1, half)
+    masked = np.where(tril == 0, np.float32(-1e29), x * alpha)
+    if half:
+        masked = bf16_round(masked)
+
+    def prepared():
+        h = dev.put(x, half)
+        cuda.scal(n, float(alpha), h)
+        cuda.mask(n, length * length, 0.0, -1e29, h, hm, h)
+        return h
+
+    # softmax straight after: one pass; the probabilities are those of the masked, scaled scores
+    h, hp = prepared(), dev.zeros(n, half)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, h, 0.0, d, hp)
+    assert_close(dev.get(hp, x.shape), R.softmax_lastaxis(masked, np.float64), tol, "softmax of the held-back mask")
+    # ... and the tensor itself, read afterwards, holds the masked scores
+    assert np.array_equal(dev.get(h, x.shape), masked)
+    # read back without a softmax
+    h = prepared()
+    assert np.array_equal(dev.get(h, x.shape), masked)
+    # consumed by another call first
+    h, hy = prepared(), dev.zeros(n, half)
+    cuda.copy(n, h, hy)
+    assert np.array_equal(dev.get(hy, x.shape), masked)
+    # the mask blob changes before anything reads the tensor: the old mask values count
+    hm2 = dev.put(tril, half)
+    h = dev.put(x, half)
+    cuda.mask(n, length * length, 0.0, -1e29, h, hm2, h)
+    cuda.set(length * length, hm2, 1.0)
+    exp = np.where(tril == 0, np.float32(-1e29), x)
+    assert np.array_equal(dev.get(h, x.shape), bf16_round(exp) if half else exp)
+    # the mask blob is freed first
+    hm3 = dev.put(tril, half)
+    h = dev.put(x, half)
+    cuda.mask(n, length * length, 0.0, -1e29, h, hm3, h)
+    cuda.FreeMemory(hm3)
+    assert np.array_equal(dev.get(h, x.shape), bf16_round(exp) if half else exp)
+    # two tensors in a row: the first call runs when the second arrives
+    h1, h2 = dev.put(x, half), dev.put(x, half)
+    cuda.mask(n, length * length, 0.0, -1e29, h1, hm, h1)
+    cuda.mask(n, length * length, 0.0, 5.0, h2, hm, h2)
+    assert np.array_equal(dev.get(h2, x.shape), np.where(tril == 0, np.float32(5.0), x))
+    assert np.array_equal(dev.get(h1, x.shape), bf16_round(exp) if half else exp)
+    # per-sequence masks (mask_batch), two sequences
+    mb = (rng.random((2, length // 2, length)) > 0.3).astype(np.float32)
+    hmb = dev.put(mb, half)
+    h, hp = dev.put(x, half), dev.zeros(n, half)
+    cuda.mask_batch(n, 2, mb.size, 0.0, -1e29, h, hmb, h)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, h, 0.0, d, hp)
+    mexp = np.where(mb.reshape(rows, length) == 0, np.float32(-1e29), x)
+    assert_close(dev.get(hp, x.shape), R.softmax_lastaxis(mexp, np.float64), tol, "softmax of a held-back mask_batch")
+    assert np.array_equal(dev.get(h, x.shape), bf16_round(mexp) if half else mexp)
+    # freed while the mask call is outstanding
+    h = prepared()
+    cuda.FreeMemory(h)
+    if not half:
+        # a MatMul that rewrites the whole tensor cancels the call: (rows x 8) @ (8 x length)
+        a, b = rng.standard_normal((1, 1, rows, 8)).astype(np.float32), rng.standard_normal((1, 1, 8, length)).astype(np.float32)
+        ha, hb = dev.put(a), dev.put(b)
+        h = prepared()
+        cuda.matmul(1, rows, length, 8, ha, hb, h)
+        assert_close(dev.get(h, x.shape), a[0, 0].astype(np.float64) @ b[0, 0].astype(np.float64), FP32_RTOL, "overwritten")
+    cuda.FreeTensorDesc(d)
+    cuda.FreeCuDNN(hc)
