@@ -500,3 +500,34 @@ def test_layernorm_layer_chain_intermediates_and_backward_golden(dev):
     top.mutable_cpu_diff = load_txt(os.path.join(d, "iter_0", "grad_1a_y.txt"))
     layer.Backward(top, bx)
     assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(d, "iter_0", "grad_9_x.txt")), 2e-5, "grad x")
+
+
+def test_explicit_chain_with_held_back_calls_matches_the_fused_handle_at_a_large_shape(dev):
+    """A score tensor of two million elements: the layer's scal / mask / softmax sequence runs through the held-back
+    path (one pass), forward twice in a row (the second MatMul overwrites the tensor that is still masked on record)
+    and backward; everything agrees with the checker and with the same layer on the fused attention handle."""
+    from mycaffe_amd.layers import CausalSelfAttentionLayer
+    rng = np.random.default_rng(91)
+    B, T, C, H = 2, 512, 128, 4
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    dy = rng.standard_normal((B, T, C)).astype(np.float32)
+    wa, ba = (rng.standard_normal((3 * C, C)) * 0.1).astype(np.float32), (rng.standard_normal(3 * C) * 0.1).astype(np.float32)
+    wp, bp = (rng.standard_normal((C, C)) * 0.1).astype(np.float32), (rng.standard_normal(C) * 0.1).astype(np.float32)
+    ref = R.causal_self_attention(x, wa, ba, wp, bp, H, dtype=np.float64)["y"]
+    grads = {}
+    for sdpa in (False, True):
+        layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, True, sdpa, training=True)
+        bx, top = Blob(dev.cuda, x.shape), Blob(dev.cuda)
+        bx.mutable_cpu_data = x
+        layer.Setup(bx, wa, ba, wp, bp)
+        for _ in range(2):
+            layer.Forward(bx, top)
+            assert_close(top.mutable_cpu_data, ref, FP32_RTOL, "layer forward, sdpa=%s" % sdpa)
+        top.mutable_cpu_diff = dy
+        layer.Backward(top, bx)
+        grads[sdpa] = bx.mutable_cpu_diff.copy()
+        if not sdpa:
+            # the score tensor, read after everything else: masked and scaled, as the immediate calls would have left it
+            att = layer.b["AttA"].mutable_cpu_data.reshape(B, H, T, T)
+            assert np.all(att[:, :, 0, 1:] == np.float32(-1e29))
+    assert_close(grads[False], grads[True], 5e-5, "input gradient, explicit chain against fused handle")
