@@ -365,6 +365,7 @@ struct FusedDecodeArgs {
     const float* fcos; const float* fsin; const int* dlen;
     int B, H, kvMul, hs, dim, kvd, seqLen, splits, rowsPerIter;
     float scale;
+    bool oneIter;   // seqLen <= splits * rowsPerIter: a split never holds more than one iteration of rows
 };
 
 template <int LPR>
@@ -384,6 +385,67 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     float* kc = a.kc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
     float* vc = a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
 
+    if (a.oneIter) {
+        // The whole cache fits one iteration per split, so a split's rows do not depend on the length: the cache
+        // rows, the query and the new key / value are requested together with the length itself, and only the
+        // rotation factors wait for it.  The row at `pos` is patched in registers instead of being stored and
+        // read back; arithmetic and its order are those of the general path below.
+        constexpr int RPW = 64 / LPR, U = 4, STEP = 4 * RPW * U;
+        const int t0 = split * STEP;
+        const int tb = t0 + wave * RPW * U;
+        DecodeStage<U> A;
+        decode_issue<float, LPR, U>(A, kc, vc, a.kvd, tb, min(a.seqLen, t0 + STEP), grp, d0, active);
+        float4 r = {0.f, 0.f, 0.f, 0.f}, kr = r, vr = r;
+        if (active) {
+            r = *(const float4*)(row + (size_t)h * a.hs + d0);
+            kr = *(const float4*)(row + a.dim + (size_t)kvh * a.hs + d0);
+            vr = *(const float4*)(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0);
+        }
+        const int nAct = (len + STEP - 1) / STEP;
+        if (split >= nAct) return;
+        const int t1 = min(len, t0 + STEP);
+        float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
+        if (active) {
+            const size_t ti = (size_t)pos * half + d0 / 2;
+            c0 = a.fcos[ti]; s0 = a.fsin[ti]; c1 = a.fcos[ti + 1]; s1 = a.fsin[ti + 1];
+        }
+        float qv[W];
+        qv[0] = (r.x * c0 - r.y * s0) * a.scale;
+        qv[1] = (r.x * s0 + r.y * c0) * a.scale;
+        qv[2] = (r.z * c1 - r.w * s1) * a.scale;
+        qv[3] = (r.z * s1 + r.w * c1) * a.scale;
+        if (t0 <= pos && pos < t1) {
+            float4 ko;
+            ko.x = kr.x * c0 - kr.y * s0; ko.y = kr.x * s0 + kr.y * c0;
+            ko.z = kr.z * c1 - kr.w * s1; ko.w = kr.z * s1 + kr.w * c1;
+            if (wave == 0 && grp == 0 && active) {
+                *(float4*)(kc + (size_t)pos * a.kvd + d0) = ko;
+                *(float4*)(vc + (size_t)pos * a.kvd + d0) = vr;
+            }
+            const u32x4 kb = {__float_as_uint(ko.x), __float_as_uint(ko.y), __float_as_uint(ko.z), __float_as_uint(ko.w)};
+            const u32x4 vb = {__float_as_uint(vr.x), __float_as_uint(vr.y), __float_as_uint(vr.z), __float_as_uint(vr.w)};
+#pragma unroll
+            for (int u = 0; u < U; u++)
+                if (tb + u * RPW + grp == pos && active) { A.k[u] = kb; A.v[u] = vb; }
+        }
+        // rows past the length were requested before it was known and may hold anything: their weight is an exact
+        // zero, and zero times their value has to be zero as well
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (tb + u * RPW + grp >= t1) { const u32x4 z = {0u, 0u, 0u, 0u}; A.v[u] = z; }
+        float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
+        decode_consume<float, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
+        const size_t bh = (size_t)b * a.H + h;
+        float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+        float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
+        if (nAct == 1) {
+            decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
+            return;
+        }
+        decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+        decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
+        return;
+    }
     int chunk = (len + a.splits - 1) / a.splits;
     chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
     const int t0 = split * chunk, t1 = min(len, t0 + chunk);
@@ -599,6 +661,7 @@ hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float
     int chunk;
     pick_splits(B, H, seqLen, a.rowsPerIter, &a.splits, &chunk);
     a.scale = scale;
+    a.oneIter = seqLen <= a.splits * a.rowsPerIter;
     dim3 grid(a.splits, H, B);
     switch (lprp) {
 #define CASE(L) case L: hipLaunchKernelGGL((attn_decode_fused_kernel<L>), grid, 256, 0, s, a); break;
