@@ -386,15 +386,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     float* vc = a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
 
     if (a.oneIter) {
-        // The whole cache fits one iteration per split, so a split's rows do not depend on the length: the cache
-        // rows, the query and the new key / value are requested together with the length itself, and only the
-        // rotation factors wait for it.  The row at `pos` is patched in registers instead of being stored and
-        // read back; arithmetic and its order are those of the general path below.
+        // The whole cache fits one iteration per split: the query and the new key / value are requested together with
+        // the length, the cache rows and the rotation factors as soon as it is known, and the row at `pos` (which the
+        // cache does not hold yet) is patched in registers instead of being stored and read back.  Arithmetic and
+        // its order are those of the general path below.
         constexpr int RPW = 64 / LPR, U = 4, STEP = 4 * RPW * U;
         const int t0 = split * STEP;
         const int tb = t0 + wave * RPW * U;
-        DecodeStage<U> A;
-        decode_issue<float, LPR, U>(A, kc, vc, a.kvd, tb, min(a.seqLen, t0 + STEP), grp, d0, active);
         float4 r = {0.f, 0.f, 0.f, 0.f}, kr = r, vr = r;
         if (active) {
             r = *(const float4*)(row + (size_t)h * a.hs + d0);
@@ -404,6 +402,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
         const int nAct = (len + STEP - 1) / STEP;
         if (split >= nAct) return;
         const int t1 = min(len, t0 + STEP);
+        DecodeStage<U> A;
+        decode_issue<float, LPR, U>(A, kc, vc, a.kvd, tb, t1, grp, d0, active);
         float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
         if (active) {
             const size_t ti = (size_t)pos * half + d0 / 2;
@@ -428,11 +428,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
             for (int u = 0; u < U; u++)
                 if (tb + u * RPW + grp == pos && active) { A.k[u] = kb; A.v[u] = vb; }
         }
-        // rows past the length were requested before it was known and may hold anything: their weight is an exact
-        // zero, and zero times their value has to be zero as well
-#pragma unroll
-        for (int u = 0; u < U; u++)
-            if (tb + u * RPW + grp >= t1) { const u32x4 z = {0u, 0u, 0u, 0u}; A.v[u] = z; }
         float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
         decode_consume<float, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
         const size_t bh = (size_t)b * a.H + h;
