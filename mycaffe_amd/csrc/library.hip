@@ -300,7 +300,7 @@ long Kernel::flush_pending_mask()
 bool Kernel::defer_mask(long hX, long hM, long hY, MemItem* X, MemItem* M, long long n, int md, int batch, float search,
                         float replace, float xscale, bool timing)
 {
-    if (timing || hX != hY || hX == hM || X->view || X->views != 0 || M->view || (size_t)n != X->count || n < (1 << 20)) return false;
+    if (timing || hX != hY || hX == hM || X->view || X->views != 0 || X->exposed || M->view || M->exposed || (size_t)n != X->count || n < (1 << 20)) return false;
     m_pendingMask.hX = hX; m_pendingMask.hM = hM; m_pendingMask.n = n; m_pendingMask.md = md; m_pendingMask.batch = batch;
     m_pendingMask.search = search; m_pendingMask.replace = replace; m_pendingMask.xscale = xscale;
     X->pending = 1.f;
@@ -347,6 +347,9 @@ long Kernel::get_pointer(long h, void** pp)
 {
     MemItem* it;
     ERRCHK(mem(h, &it));
+    it->exposed = true;
+    MemItem* root;
+    if (it->view && !m_mem.get(it->base, &root)) root->exposed = true;
     *pp = it->ptr;
     return 0;
 }
@@ -705,7 +708,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         MemItem* X;
         ERRCHK(mem((long)pl[2], &X));
         RANGE(X, xo, n);
-        if (!timing && !X->view && X->views == 0 && xo == 0 && (size_t)n == X->count && n >= (1 << 20)) {
+        if (!timing && !X->view && X->views == 0 && !X->exposed && xo == 0 && (size_t)n == X->count && n >= (1 << 20)) {
             // a large whole tensor: the multiplication waits for the next call that touches the tensor; the mask calls
             // of the attention chain (scale, then mask in place) do it in their own pass
             X->pending = pf[0];

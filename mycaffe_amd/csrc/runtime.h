@@ -32,6 +32,9 @@ struct MemItem {
     // allocations without views; every access through Kernel::mem() applies it first, except the mask calls, which
     // fold it into their own pass (the scale / mask pair of the explicit attention chain becomes one pass).
     float pending = 1.f;
+    // The raw device address has been handed out (Internal_GetPointerFloat): its holder reads memory without passing
+    // through Kernel::mem(), so nothing is ever held back on this allocation again.
+    bool exposed = false;
     DType dt() const { return half ? BF16 : F32; }
     size_t esize() const { return half ? 2 : 4; }
 };

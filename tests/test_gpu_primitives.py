@@ -569,6 +569,39 @@ def test_whole_tensor_scal_is_deferred_without_changing_any_result(dev, half):
     cuda.FreeMemory(h)
 
 
+def test_nothing_is_held_back_on_a_tensor_whose_device_address_was_handed_out(dev):
+    """Internal_GetPointerFloat (CudaDnnDLL.cpp:57-75) gives an extension library the device address behind a memory
+    handle, and the extension then reads that memory on its own: a SCAL and an in-place mask over such a tensor have
+    to be in the stream when the call returns, where the same calls on an ordinary tensor wait for the next access."""
+    import ctypes
+    rng = np.random.default_rng(73)
+    cuda = dev.cuda
+    n, md = 1 << 20, 4096
+    x = rng.standard_normal(n).astype(np.float32)
+    m = (rng.random(md) > 0.3).astype(np.float32)
+    h, hm = dev.put(x, False), dev.put(m, False)
+    lib = cuda._lib
+    lib.Internal_GetPointerFloat.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_void_p)]
+    lib.Internal_GetPointerFloat.restype = ctypes.c_int32
+    p = ctypes.c_void_p()
+    assert lib.Internal_GetPointerFloat(0, cuda.m_hKernel, h, ctypes.byref(p)) == 0 and p.value
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    hip.hipMemcpy.restype = ctypes.c_int
+
+    def raw():
+        cuda.SynchronizeDevice()
+        out = np.empty(n, np.float32)
+        assert hip.hipMemcpy(out.ctypes.data, p, 4 * n, 2) == 0   # device to host, straight from the address
+        return out
+
+    assert np.array_equal(raw(), x)
+    cuda.scal(n, 0.5, h)
+    assert np.array_equal(raw(), x * np.float32(0.5))
+    cuda.mask(n, md, 0.0, -1e29, h, hm, h)
+    assert np.array_equal(raw(), np.where(np.tile(m, n // md) == 0, np.float32(-1e29), x * np.float32(0.5)))
+
+
 @pytest.mark.parametrize("half", [False, True])
 def test_in_place_mask_is_held_back_for_the_softmax_without_changing_any_result(dev, half):
     """An in-place mask call over a large whole tensor waits for the next call: a softmax forward over the tensor does
