@@ -179,16 +179,16 @@ def cpu_baseline(blob, gpu_prompt, gpu_ids, budget_s=12.0):
             "ids_vs_gpu_first_generation": same}
 
 
-def bench_prefill_attention(cuda, reps, warm=5):
-    """Fused causal attention at B=8, T=1024, 12 heads x 64 through ATTN_FWD (id 163)."""
+def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=(("bf16", True), ("f32", False))):
+    """Fused causal attention through ATTN_FWD (id 163): B=8, T=1024, 12 heads x 64 unless another shape is given."""
     from mycaffe_amd.cudadnn import CUDAFN
-    B, H, T, hs = 8, 12, 1024, 64
+    B, H, T, hs = shape
     rng = np.random.default_rng(0)
     out = {}
     mask = cuda.AllocMemory(np.tril(np.ones((T, T), np.float32)))
     hc, ha = cuda.CreateCuDNN(), cuda.CreateAttn()
     cuda.SetAttn(hc, ha, 0, False, B, T, H, hs, 0.0)
-    for name, half in (("bf16", True), ("f32", False)):
+    for name, half in dtypes:
         hs_ = [cuda.AllocMemory(rng.standard_normal(B * H * T * hs).astype(np.float32), bHalfSize=half) for _ in range(3)]
         hy = cuda.AllocMemory(B * H * T * hs, bHalfSize=half)
         rgl = [hc, ha, T, hs_[0], hs_[1], hs_[2], mask, hy, 0]
@@ -200,7 +200,7 @@ def bench_prefill_attention(cuda, reps, warm=5):
                      "roofline": {"kernel": "fused causal attention forward", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s",
                                   "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
-                                  "traffic": recorded_traffic("flash_" + name)}}
+                                  "traffic": recorded_traffic("flash_" + name) if shape == (8, 12, 1024, 64) else None}}
         for h in hs_ + [hy]:
             cuda.FreeMemory(h)
     cuda.FreeMemory(mask)
@@ -584,6 +584,9 @@ def main():
     if want("prefill"):
         also["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 50)
         log("prefill attention:", json.dumps(also["prefill_attention_B8_T1024_H12x64"]))
+        # the Llama-2 7B head shape at its full context: long enough that launch and tail effects no longer count
+        also["prefill_attention_B4_T4096_H32x128"] = bench_prefill_attention(cuda, 10, 2, (4, 32, 4096, 128), (("bf16", True),))
+        log("prefill attention, 32 x 128 heads, T = 4096:", json.dumps(also["prefill_attention_B4_T4096_H32x128"]))
     if want("decode_attn"):
         also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
         log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
