@@ -170,22 +170,29 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
     }
     for (int b = 0; b < B; b++) {
         const float* xb = x + (size_t)b * n;
-        float4 xv[CH];
+        float4 xv[CH], gq[NORM ? CH : 1];
         float ss = 0.f;
+        // the residual epilogue's old values are requested now, not once the row sums are known
+        float prev[ROWS];
+#pragma unroll
+        for (int rr = 0; rr < ROWS; rr++) prev[rr] = (MODE == 1 && lane == 0 && r0 + rr < rows) ? y[(size_t)b * ldy + r0 + rr] : 0.f;
+        // the norm weights are requested together with the activations, not after the sum of squares has gone round
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int j = matvec_col<WIDE>(c, lane);
             xv[c] = j < n ? *(const float4*)(xb + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-            if (NORM) ss += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
+            if (NORM) gq[c] = j < n ? *(const float4*)(g + j) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
         if (NORM) {
+#pragma unroll
+            for (int c = 0; c < CH; c++) ss += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
             ss = wsum(ss);
             const float inv = 1.0f / sqrtf(ss / n + 1e-5f);
 #pragma unroll
             for (int c = 0; c < CH; c++) {
                 const int j = matvec_col<WIDE>(c, lane);
                 if (j < n) {
-                    const float4 gv = *(const float4*)(g + j);
+                    const float4 gv = gq[c];
                     xv[c].x = gv.x * (inv * xv[c].x);
                     xv[c].y = gv.y * (inv * xv[c].y);
                     xv[c].z = gv.z * (inv * xv[c].z);
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
             if (lane == 0 && r < rows) {
                 float* out = y + (size_t)b * ldy + r;
                 if (MODE == 0) *out = a0;
-                else if (MODE == 1) *out += a0;
+                else if (MODE == 1) *out = prev[rr] + a0;
                 else *out = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
             }
         }
