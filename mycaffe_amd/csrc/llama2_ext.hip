@@ -249,6 +249,13 @@ __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ 
     const float* xr = x + (size_t)min(b0 + i, B - 1) * n + kk * 8;
     floatx4v acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
+    // the residual epilogue's old values (wavefront 0 finishes the tile) are requested with the first weights
+    float prev[4] = {0.f, 0.f, 0.f, 0.f};
+    if (MODE == 1 && wave == 0 && jv) {
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+            if (r0 + 4 * kk + v < rows) prev[v] = y[(size_t)(b0 + i) * ldy + r0 + 4 * kk + v];
+    }
     const int nit = n >> 5;
     constexpr int U = 4;   // slabs whose loads are in flight together
     for (int base = wave; base < nit; base += NS * U) {
@@ -318,7 +325,7 @@ __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ 
         if (r0 + 4 * kk + v >= rows) break;
         const float a0 = d[v] * inv;
         if (MODE == 0) out[v] = a0;
-        else if (MODE == 1) out[v] += a0;
+        else if (MODE == 1) out[v] = prev[v] + a0;
         else out[v] = a0 * (1.0f / (1.0f + expf(-a0))) * (d2[v] * inv);
     }
 }
@@ -341,6 +348,9 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
     const int b = blockIdx.x;
     const int pos = st->pos, nPrompt = st->n_prompt;
     const float* lg = logits + (size_t)b * V;
+    // the forced id of the next position, if there is one, is requested before the scan instead of after it
+    const bool forced = pos + 1 < nPrompt && pos + 1 < promptStride;
+    const int forcedTok = (threadIdx.x == 0 && forced) ? prompt[(size_t)b * promptStride + pos + 1] : 0;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     if (given) V = 0;   // the host sampler chose the id: nothing to scan
@@ -381,8 +391,7 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
         if (given) bi = given[b];
         next[b] = bi;
         out_ids[(size_t)b * promptStride + pos] = bi;
-        const int np = pos + 1;
-        const int tok = (np < nPrompt && np < promptStride) ? prompt[(size_t)b * promptStride + np] : bi;
+        const int tok = forced ? forcedTok : bi;
         cur[b] = tok;
         stok = tok;
     }
