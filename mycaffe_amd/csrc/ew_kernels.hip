@@ -787,7 +787,9 @@ hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const v
 // MASKED: the row is first put through a mask call that was held back for this purpose,
 //   x = mask[mi] == search ? replace : xscale * x,   mi = i % md1 + (i / dd1) * md1   (i = flat index; md1 and dd1 are
 // multiples of the row length, so a row maps to one run of mask values).
-struct SoftmaxMask { const void* mask; size_t md1, dd1; float search, replace, xscale; };
+// causalT != 0: the mask is known to keep exactly the lower triangle of a (causalT, causalT) square and rows are causalT
+// long, so it is not read, and neither are the chunks of x that lie wholly above the diagonal.
+struct SoftmaxMask { const void* mask; size_t md1, dd1; float search, replace, xscale; int causalT; };
 
 template <typename T, int R, bool MASKED>
 __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int len, const T* x, T* y, bool logsm, SoftmaxMask mk)
@@ -799,9 +801,14 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
     const T* xr = x + row * len;
     T* yr = y + row * len;
     const T* mr = nullptr;
+    int qrow = 0;
     if (MASKED) {
-        const size_t i0 = row * (size_t)len;
-        mr = (const T*)mk.mask + i0 % mk.md1 + (i0 / mk.dd1) * mk.md1;
+        if (mk.causalT) {
+            qrow = (int)(row % (size_t)mk.causalT);
+        } else {
+            const size_t i0 = row * (size_t)len;
+            mr = (const T*)mk.mask + i0 % mk.md1 + (i0 / mk.dd1) * mk.md1;
+        }
     }
     float v[R][4];
     float mx = -INFINITY;
@@ -809,8 +816,19 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
     for (int r = 0; r < R; r++) {
         const int c = lane + r * 64;
         if (c < chunks) {
-            Vec4<T>::load(xr + 4 * c, v[r]);
-            if (MASKED) {
+            if (MASKED && mk.causalT) {
+                if (4 * c > qrow) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) v[r][i] = mk.replace;
+                } else {
+                    Vec4<T>::load(xr + 4 * c, v[r]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) v[r][i] = 4 * c + i > qrow ? mk.replace : mk.xscale * v[r][i];
+                }
+            } else {
+                Vec4<T>::load(xr + 4 * c, v[r]);
+            }
+            if (MASKED && !mk.causalT) {
                 float mv[4];
                 Vec4<T>::load(mr + 4 * c, mv);
 #pragma unroll
@@ -871,11 +889,12 @@ static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void
 // instead of two.  Returns hipErrorNotSupported when the shape does not fit the one-wavefront-per-row kernel or a row
 // would straddle a wrap of the mask; the caller then runs the mask call first.
 hipError_t k_softmax_masked(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, const void* mask,
-                            size_t md1, size_t dd1, float search, float replace, float xscale)
+                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal)
 {
     if (rows == 0 || len <= 0) return hipSuccess;
     if (md1 == 0 || dd1 == 0 || md1 % (size_t)len != 0 || dd1 % (size_t)len != 0) return hipErrorNotSupported;
-    SoftmaxMask mk{mask, md1, dd1, search, replace, xscale};
+    if (causal && (md1 != (size_t)len * len || dd1 % md1 != 0)) return hipErrorInvalidValue;
+    SoftmaxMask mk{mask, md1, dd1, search, replace, xscale, causal ? len : 0};
     if (!softmax_fwd_wave_launch_t<true>(s, dt, x, y, rows, len, logsm, mk)) return hipErrorNotSupported;
     return hipGetLastError();
 }

@@ -58,7 +58,7 @@ hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t out
 // softmax of mask(x) in one pass (mask semantics of k_mask / k_mask_batch with md1 = maskDim / batch, dd1 = n / batch);
 // hipErrorNotSupported when the shape does not fit
 hipError_t k_softmax_masked(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, const void* mask,
-                            size_t md1, size_t dd1, float search, float replace, float xscale);
+                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal = false);
 // gradient with respect to the softmax input from the output y and its gradient dy (dx may alias dy)
 hipError_t k_softmax_bwd(hipStream_t s, DType dt, const void* y, const void* dy, void* dx, size_t outer, int len, int inner, bool logsm);
 // adjacent-pair rotary embedding with the CudaDnnDLL index rule; x == y allowed

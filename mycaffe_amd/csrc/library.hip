@@ -389,6 +389,15 @@ bool Kernel::mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T)
 {
     uint64_t ver = m_mem.version(hMask);
     if (st->maskHandle == hMask && st->maskVersion == ver && st->maskT == T) return st->maskCausal;
+    bool causal;
+    if (!tril_scan(mask, T, &causal)) return false;
+    st->maskHandle = hMask; st->maskVersion = ver; st->maskT = T; st->maskCausal = causal;
+    return st->maskCausal;
+}
+
+// one scan of a (T,T) fp32 mask and its host read-back; false when the scan could not be run
+bool Kernel::tril_scan(MemItem* mask, int T, bool* causal)
+{
     void* ws;
     if (workspace(256, &ws)) return false;
     int* flag = (int*)ws;
@@ -400,8 +409,21 @@ bool Kernel::mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T)
     int bad = 1;
     if (hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, m_stream) != hipSuccess) return false;
     if (hipStreamSynchronize(m_stream) != hipSuccess) return false;
-    st->maskHandle = hMask; st->maskVersion = ver; st->maskT = T; st->maskCausal = (bad == 0);
-    return st->maskCausal;
+    *causal = (bad == 0);
+    return true;
+}
+
+// the same question for the mask blob of a held-back mask call (no attention handle to keep the answer on): cached per
+// (handle, content version, T) on the kernel
+bool Kernel::held_mask_is_causal(long hMask, MemItem* mask, int T)
+{
+    if (mask->half || mask->view || mask->count < (size_t)T * T) return false;
+    const uint64_t ver = m_mem.version(hMask);
+    if (m_heldMaskHandle == hMask && m_heldMaskVersion == ver && m_heldMaskT == T) return m_heldMaskCausal;
+    bool causal;
+    if (!tril_scan(mask, T, &causal)) return false;
+    m_heldMaskHandle = hMask; m_heldMaskVersion = ver; m_heldMaskT = T; m_heldMaskCausal = causal;
+    return causal;
 }
 
 #define NEED_L(lo, hi) ERRCHK(verify(ll, pl, lo, hi))
@@ -1347,7 +1369,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 (size_t)total <= Y->count) {
                 const PendingMask& p = m_pendingMask;
                 const size_t md1 = p.batch ? (size_t)(p.md / p.batch) : (size_t)p.md, dd1 = p.batch ? (size_t)(p.n / p.batch) : (size_t)p.n;
-                hipError_t e = k_softmax_masked(s, X->dt(), X->ptr, Y->ptr, outer, len, alg == 2, M->ptr, md1, dd1, p.search, p.replace, p.xscale);
+                // a (len,len) lower-triangle mask with search == 0 is not read at all, and neither are the scores above the diagonal
+                const bool causal = p.batch == 0 && !X->half && p.search == 0.f && md1 == (size_t)len * len && dd1 % md1 == 0 &&
+                                    held_mask_is_causal(p.hM, M, len);
+                hipError_t e = k_softmax_masked(s, X->dt(), X->ptr, Y->ptr, outer, len, alg == 2, M->ptr, md1, dd1, p.search, p.replace, p.xscale, causal);
                 if (e == hipSuccess) {
                     m_mem.touch((long)pl[6]);
                     return 0;

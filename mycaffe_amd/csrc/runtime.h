@@ -163,6 +163,9 @@ private:
                     float xscale, bool timing);
     PendingMask m_pendingMask;
     bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
+    bool tril_scan(MemItem* mask, int T, bool* causal);
+    bool held_mask_is_causal(long hMask, MemItem* mask, int T);
+    long m_heldMaskHandle = 0; uint64_t m_heldMaskVersion = 0; int m_heldMaskT = 0; bool m_heldMaskCausal = false;
 
     int m_device = 0;
     hipStream_t m_stream = nullptr;

@@ -602,6 +602,53 @@ def test_nothing_is_held_back_on_a_tensor_whose_device_address_was_handed_out(de
     assert np.array_equal(raw(), np.where(np.tile(m, n // md) == 0, np.float32(-1e29), x * np.float32(0.5)))
 
 
+def test_held_back_causal_mask_is_not_read_and_still_follows_the_mask_blob(dev):
+    """A held-back (T,T) mask that keeps exactly the lower triangle is recognised once per content version: the
+    softmax then reads neither the mask nor the scores above the diagonal.  Its output equals, bit for bit, that of the
+    immediate calls (forced here by a memory pointer on the tensor, which rules out holding anything back), and a
+    change to the mask blob is seen by the next call."""
+    rng = np.random.default_rng(74)
+    cuda = dev.cuda
+    rows, T = 4096, 256
+    n = rows * T
+    x = (rng.standard_normal((rows, T)) * 4).astype(np.float32)
+    tril = np.tril(np.ones((T, T), np.float32))
+    alpha = np.float32(0.125)
+    hm = dev.put(tril)
+    hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+    cuda.SetTensorDesc(d, rows, T, 1, 1, False)
+
+    def run(immediate):
+        h, hp = dev.put(x), dev.zeros(n)
+        hv = cuda.CreateMemoryPointer(h, 0, n) if immediate else 0
+        cuda.scal(n, float(alpha), h)
+        cuda.mask(n, T * T, 0.0, -1e29, h, hm, h)
+        cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, h, 0.0, d, hp)
+        p, kept = dev.get(hp, x.shape), dev.get(h, x.shape)
+        if hv:
+            cuda.FreeMemoryPointer(hv)
+        cuda.FreeMemory(h)
+        cuda.FreeMemory(hp)
+        return p, kept
+
+    def expect(m):
+        masked = np.where(np.tile(m, (rows // T, 1)) == 0, np.float32(-1e29), x * alpha)
+        return masked, R.softmax_lastaxis(masked, np.float64)
+
+    for m in (tril, None):
+        if m is None:   # one more key kept in row 3 of the same blob: no longer a triangle
+            m = tril.copy()
+            m[3, 200] = 1.0
+            cuda.SetMemory(hm, m)
+        masked, want = expect(m)
+        p_held, kept_held = run(False)
+        p_now, kept_now = run(True)
+        assert np.array_equal(p_held, p_now)
+        assert np.array_equal(kept_held, masked) and np.array_equal(kept_now, masked)
+        assert_close(p_held, want, FP32_RTOL, "softmax of the held-back causal mask")
+    assert p_held[3, 200] > 0 and p_held[4, 200] == 0
+
+
 @pytest.mark.parametrize("half", [False, True])
 def test_in_place_mask_is_held_back_for_the_softmax_without_changing_any_result(dev, half):
     """An in-place mask call over a large whole tensor waits for the next call: a softmax forward over the tensor does
