@@ -387,6 +387,9 @@ __global__ void check_tril_kernel(const float* m, int T, int* bad)
 // (handle, content version, T) so the scan and its host read-back happen once
 bool Kernel::mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T)
 {
+    // a blob whose device address was handed out can change without its version moving: it is read every time
+    MemItem* root = mask;
+    if (mask->exposed || (mask->view && !m_mem.get(mask->base, &root) && root->exposed)) return false;
     uint64_t ver = m_mem.version(hMask);
     if (st->maskHandle == hMask && st->maskVersion == ver && st->maskT == T) return st->maskCausal;
     bool causal;
@@ -417,7 +420,7 @@ bool Kernel::tril_scan(MemItem* mask, int T, bool* causal)
 // (handle, content version, T) on the kernel
 bool Kernel::held_mask_is_causal(long hMask, MemItem* mask, int T)
 {
-    if (mask->half || mask->view || mask->count < (size_t)T * T) return false;
+    if (mask->half || mask->view || mask->exposed || mask->count < (size_t)T * T) return false;
     const uint64_t ver = m_mem.version(hMask);
     if (m_heldMaskHandle == hMask && m_heldMaskVersion == ver && m_heldMaskT == T) return m_heldMaskCausal;
     bool causal;
