@@ -65,6 +65,27 @@ def test_logits_and_ids_tiny(llm, tmp_path, cfg, shared, std):
     assert np.array_equal(llm.GenerateIds(prompt, n), ids)
 
 
+def test_grouped_query_heads_over_several_cache_splits(llm, tmp_path):
+    """Head size 64 with two query heads per key / value head and a cache of 256 positions: the fused decode attention
+    cuts the cache into up to four 64-row splits, the heads of a group append the same rotated key, and the split that
+    owns the current position moves on every 64 steps.  Logits and ids against the checker over 200 positions."""
+    cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256)
+    blob, views = O.random_weights(cfg, seed=11, shared_classifier=False, std=0.08)
+    rng = np.random.default_rng(2)
+    for k in ("rms_att", "rms_ffn", "rms_final"):
+        views[k][...] = 1 + 0.2 * rng.standard_normal(views[k].shape).astype(np.float32)
+    path = str(tmp_path / "gqa.bin")
+    O.write_checkpoint_v1(path, cfg, blob, False)
+    llm.Load(path)
+    prompt = rng.integers(3, cfg["vocab_size"], 8)
+    n = 200
+    ids, logits = llm.GenerateIds(prompt, n, want_logits=True)
+    ref_ids, ref_logits = O.Llama(cfg, blob, False).generate_greedy(prompt, n, want_logits=True)
+    assert_close(logits, ref_logits, FP32_RTOL, "logits")
+    _check_ids(ids, ref_ids, ref_logits, "grouped-query heads")
+    assert np.array_equal(llm.GenerateIds(prompt, n), ids)   # captured-graph path
+
+
 def test_reference_cpu_config_greedy_256_tokens(llm, tmp_path):
     """dim 288 / 6 layers / 6 heads x 48 / ffn 768 / vocab 32000 / seq 256, N(0, 0.02) weights,
     RMSNorm weights 1, unshared classifier; 8 seeded prompt ids, greedy to 256 tokens."""
