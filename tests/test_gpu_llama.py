@@ -131,6 +131,25 @@ def test_batch_generation_matches_independent_sequences(llm, tmp_path):
         _check_ids(out[b], ref_ids, ref_logits, "batch row %d" % b)
 
 
+def test_batch_with_grouped_query_heads_and_multi_iteration_splits(llm, tmp_path):
+    """40 sequences, head size 64, two query heads per key / value head, cache of 512 positions: with 160 (sequence,
+    head) pairs the fused decode attention takes four splits of 128 rows, i.e. two 64-row iterations per split, and
+    appends the new key / value through the cache (the path batch 1 does not take).  Ids of every row against the
+    checker over 300 positions."""
+    cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=512)
+    blob, _ = O.random_weights(cfg, seed=12, shared_classifier=False, std=0.08)
+    path = str(tmp_path / "gqa_batch.bin")
+    O.write_checkpoint_v1(path, cfg, blob, False)
+    llm.Load(path)
+    prompts = np.random.default_rng(3).integers(3, cfg["vocab_size"], (40, 6))
+    n = 300
+    out = llm.GenerateBatch(prompts, n)
+    ref = O.Llama(cfg, blob)
+    for b in range(40):
+        ref_ids, ref_logits = ref.generate_greedy(prompts[b], n, want_logits=True)
+        _check_ids(out[b], ref_ids, ref_logits, "batch row %d" % b)
+
+
 def test_error_paths(llm, tmp_path):
     with pytest.raises(CudaDnnError) as e:
         llm.Load(str(tmp_path / "missing.bin"))
