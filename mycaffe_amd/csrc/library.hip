@@ -211,7 +211,8 @@ std::string Kernel::device_name()
     hipDeviceProp_t p;
     if (hipGetDeviceProperties(&p, m_device) != hipSuccess) return "unknown";
     char buf[512];
-    snprintf(buf, sizeof(buf), "%s (%s, %d CUs, %.1f GB)", p.name, p.gcnArchName, p.multiProcessorCount,
+    // some driver stacks report no marketing name
+    snprintf(buf, sizeof(buf), "%s (%s, %d CUs, %.1f GB)", p.name[0] ? p.name : "AMD GPU", p.gcnArchName, p.multiProcessorCount,
              (double)p.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
     return buf;
 }
