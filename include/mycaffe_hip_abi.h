@@ -242,7 +242,8 @@ enum {
      *   GENERATE_IDS  f{hLlm, nSteps, wantLogits(0|1), id0, id1, ...}
      *                 -> f{next id after each position [, logits of every step]}
      *   SET_OPTION    f{hLlm, option, value}; option 1 = weight storage
-     *                 (0 fp32, 1 bf16), applied at the next LOAD; option 2 = first
+     *                 (0 fp32, 1 bf16), applied at the next LOAD (weights already on the
+     *                 device keep the storage they were loaded in); option 2 = first
      *                 step of the timed span; option 3 = replay one captured
      *                 HIP graph per step (1, default) or launch eagerly (0);
      *                 option 4 = weight rows per wavefront of the mat-vec
@@ -251,7 +252,8 @@ enum {
      *                 seed of CREATE) instead of the argmax (0, default)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids}
-     *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it}
+     *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were
+     *                 replays of the captured graph / 0 if they were launched eagerly}
      *   PROFILE_STEP  f{hLlm, pos, reps[, batch]} -> per kernel class of one decode step
      *                 f{ms per step, launches per step, algorithmic bytes per step}, classes in
      *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,
@@ -275,6 +277,14 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG lfnIdx, float* pInput, MCH_LONG
 MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG lfnIdx, float* pInput, MCH_LONG lInput, float** ppOutput,
                                           MCH_LONG* plOutput, MCH_TCHAR* szInput, MCH_TCHAR* szOutput,
                                           MCH_LONG lOutputMax, MCH_TCHAR* szErr, MCH_LONG lErrMax);
+/* CudaExtension.llm32.cpp:85-89, 180-206, 270-330: double twins; the engine is fp32 / 16-bit storage only, so all
+ * three return MCH_ERROR_NOT_IMPLEMENTED (a double-typed parent fails cleanly at CREATE_EXTENSION). */
+MCH_LONG DLL_InitDoubleCustomExtension(void* hParent, MCH_LONG lKernelIdx);
+MCH_LONG DLL_InvokeDoubleCustomExtension(MCH_LONG lfnIdx, double* pInput, MCH_LONG lInput, double** ppOutput,
+                                         MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lErrMax);
+MCH_LONG DLL_InvokeDoubleCustomExtensionEx(MCH_LONG lfnIdx, double* pInput, MCH_LONG lInput, double** ppOutput,
+                                           MCH_LONG* plOutput, MCH_TCHAR* szInput, MCH_TCHAR* szOutput,
+                                           MCH_LONG lOutputMax, MCH_TCHAR* szErr, MCH_LONG lErrMax);
 
 /* ---- measurement hook (no counterpart in the reference) --------------------
  * Runs the same Ex2 dispatch `nWarmup` + `nReps` times on the kernel's stream
@@ -284,6 +294,18 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG lfnIdx, float* pInput, MCH_LO
 MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
                                 MCH_LONGLONG* plInput, MCH_LONG llInput, MCH_LONG nWarmup, MCH_LONG nReps,
                                 float* pfMs, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+
+/* ---- entry point that allocates nothing (no counterpart in the reference) ----
+ * For callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The call is ATTN_DECODE_FWD (id 2001) with the same f{scale} and l{...} arrays; the
+ * split partials and merge tickets come from a fixed device array inside the library (4 MiB + 16 KiB per GPU,
+ * held until the process ends) instead of the kernel object's growable workspace, and no hipMalloc, hipFree or
+ * other allocating routine is called.  Limits: batch x heads <= 4096 and (batch x heads x splits) x (hs + 2) x 4
+ * bytes <= 4 MiB, where splits = min(256, ceil(1024 / (batch x heads))); larger calls return
+ * MCH_ERROR_PARAM_OUT_OF_RANGE.  All calls on one GPU share the array: calls that overlap on one GPU (two kernel
+ * objects, two host threads) race, so serialise them. */
+MCH_LONG MCH_AttnDecodeForwardNoAlloc(MCH_LONG lKernelIdx, float* pInput, MCH_LONG lInput, MCH_LONGLONG* plInput,
+                                      MCH_LONG llInput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
 
 #ifdef __cplusplus
 }

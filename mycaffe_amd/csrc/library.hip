@@ -174,6 +174,39 @@ ExtensionState::~ExtensionState()
 }
 
 // ---------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing (MCH_AttnDecodeForwardNoAlloc): merge tickets followed by the
+// split-K partials of the decode attention.  Every GPU this library runs on holds its own copy of the array until the
+// process ends; g_scratch below is only the host-side stand-in of the symbol, the device address is looked up once per
+// device and that pointer is what kernels, fills and copies get.
+enum : long long { MCH_NOALLOC_MAX_TICKETS = 4096, MCH_NOALLOC_PARTIAL_BYTES = 4ll << 20 };
+static __device__ __align__(256) unsigned char g_scratch[MCH_NOALLOC_MAX_TICKETS * sizeof(int) + MCH_NOALLOC_PARTIAL_BYTES];
+static char* g_scratchPtr[64];
+static std::mutex g_scratchLock;
+
+// looks the array's address up on `device`, which must be the current device; called when a kernel object is
+// initialised on it
+static long static_scratch_init(int device)
+{
+    if (device < 0 || device >= 64) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    std::lock_guard<std::mutex> g(g_scratchLock);
+    if (g_scratchPtr[device]) return 0;
+    void* p = nullptr;
+    HIPCHK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_scratch)));
+    if (!p) return MCH_ERROR_MEMORY_NULL;
+    g_scratchPtr[device] = (char*)p;
+    return 0;
+}
+
+static long static_scratch(int device, char** p)
+{
+    if (device < 0 || device >= 64) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    std::lock_guard<std::mutex> g(g_scratchLock);
+    if (!g_scratchPtr[device]) return MCH_ERROR_DEVICE_NOT_INITIALIZED;
+    *p = g_scratchPtr[device];
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 Kernel::Kernel() {}
 
 Kernel::~Kernel()
@@ -203,6 +236,7 @@ long Kernel::initialize(const float* pf, long n)
     m_device = dev;
     HIPCHK(hipSetDevice(dev));
     if (!m_stream) HIPCHK(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking));
+    ERRCHK(static_scratch_init(dev));
     return 0;
 }
 
@@ -1586,55 +1620,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
-    case MCH_FN_ATTN_DECODE_FWD: {
-        // f{scale}, l{batch,heads,kvHeads,hs,len,hQ,hKc,hVc,hY,strideB,strideH,strideT[,hRope,hKnew,hVnew]}
-        NEED_F(1, 1);
-        NEED_L(12, 15);
-        if (ll != 12 && ll != 15) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        long long B = pl[0], H = pl[1], KVH = pl[2], hs = pl[3], len = pl[4];
-        long long sB = pl[9], sH = pl[10], sT = pl[11];
-        if (B < 1 || H < 1 || KVH < 1 || hs < 1 || len < 1 || H % KVH || sB < 0 || sH < 0 || sT < 1 || (hs & 1))
-            return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        MemItem *Q, *KC, *VC, *Y;
-        ERRCHK(mem((long)pl[5], &Q));
-        ERRCHK(mem((long)pl[6], &KC));
-        ERRCHK(mem((long)pl[7], &VC));
-        ERRCHK(mem((long)pl[8], &Y));
-        if (Q->half != KC->half || Q->half != VC->half || Q->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
-        RANGE(Q, 0, B * H * hs);
-        RANGE(Y, 0, B * H * hs);
-        long long need = (B - 1) * sB + (KVH - 1) * sH + (len - 1) * sT + hs;
-        RANGE(KC, 0, need);
-        RANGE(VC, 0, need);
-        float scale = pf[0] != 0.f ? pf[0] : (float)(1.0 / sqrt((double)hs));
-        if (ll == 15 && (pl[12] || pl[13] || pl[14])) {
-            RopeState* rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
-            if (pl[12] && (!rp || !rp->set)) return MCH_ERROR_ROPE_NOT_INITIALIZED;
-            if (rp && (rp->hs != hs || len > rp->seq)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-            MemItem *KN, *VN;
-            ERRCHK(mem((long)pl[13], &KN));
-            ERRCHK(mem((long)pl[14], &VN));
-            if (KN->half != Q->half || VN->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
-            RANGE(KN, 0, B * KVH * hs);
-            RANGE(VN, 0, B * KVH * hs);
-            HIPCHK(k_rope_append(s, Q->dt(), Q->ptr, KN->ptr, VN->ptr, KC->ptr, VC->ptr, (int)B, (int)H, (int)KVH, (int)hs,
-                                 (int)len - 1, sB, sH, sT, rp ? (const float*)rp->dcos.get() : nullptr,
-                                 rp ? (const float*)rp->dsin.get() : nullptr));
-            m_mem.touch((long)pl[5]);
-            m_mem.touch((long)pl[6]);
-            m_mem.touch((long)pl[7]);
-            m_mem.touch((long)pl[13]);
-        }
-        size_t wsb = attn_decode_workspace_bytes((int)B, (int)H, (int)hs, (int)len);
-        void* ws;
-        ERRCHK(workspace(wsb, &ws));
-        int* tk;
-        ERRCHK(tickets((size_t)(B * H), &tk));
-        HIPCHK(k_attn_decode(s, Q->dt(), Q->ptr, KC->ptr, VC->ptr, Y->ptr, (int)B, (int)H, (int)KVH, (int)hs, (int)len, sB, sH,
-                             sT, scale, ws, m_wsBytes, nullptr, tk));
-        m_mem.touch((long)pl[8]);
-        return 0;
-    }
+    case MCH_FN_ATTN_DECODE_FWD:
+        return attn_decode_fwd(pf, lf, pl, ll, false);
 
     // ---- RoPE ------------------------------------------------------------------
     case MCH_FN_CREATE_ROPE: {
@@ -1861,6 +1848,87 @@ long Kernel::create_blobloader(MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut)
     BlobLoaderState* st = m_blobLoader.get(h);
     st->fd = fd; st->data = (const unsigned char*)m; st->fileSize = (size_t)sb.st_size;
     return set_out((float)h, ppOut, plOut);
+}
+
+// ATTN_DECODE_FWD: f{scale}, l{batch,heads,kvHeads,hs,len,hQ,hKc,hVc,hY,strideB,strideH,strideT[,hRope,hKnew,hVnew]}.
+// With staticScratch the split partials and merge tickets come from the file-scope device array instead of the
+// kernel object's allocations.
+long Kernel::attn_decode_fwd(float* pf, long lf, MCH_LONGLONG* pl, long ll, bool staticScratch)
+{
+    hipStream_t s = m_stream;
+    NEED_F(1, 1);
+    NEED_L(12, 15);
+    if (ll != 12 && ll != 15) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long long B = pl[0], H = pl[1], KVH = pl[2], hs = pl[3], len = pl[4];
+    long long sB = pl[9], sH = pl[10], sT = pl[11];
+    if (B < 1 || H < 1 || KVH < 1 || hs < 1 || len < 1 || H % KVH || sB < 0 || sH < 0 || sT < 1 || (hs & 1))
+        return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    MemItem *Q, *KC, *VC, *Y;
+    ERRCHK(mem((long)pl[5], &Q));
+    ERRCHK(mem((long)pl[6], &KC));
+    ERRCHK(mem((long)pl[7], &VC));
+    ERRCHK(mem((long)pl[8], &Y));
+    if (Q->half != KC->half || Q->half != VC->half || Q->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+    RANGE(Q, 0, B * H * hs);
+    RANGE(Y, 0, B * H * hs);
+    long long need = (B - 1) * sB + (KVH - 1) * sH + (len - 1) * sT + hs;
+    RANGE(KC, 0, need);
+    RANGE(VC, 0, need);
+    float scale = pf[0] != 0.f ? pf[0] : (float)(1.0 / sqrt((double)hs));
+    if (ll == 15 && (pl[12] || pl[13] || pl[14])) {
+        RopeState* rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
+        if (pl[12] && (!rp || !rp->set)) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+        if (rp && (rp->hs != hs || len > rp->seq)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *KN, *VN;
+        ERRCHK(mem((long)pl[13], &KN));
+        ERRCHK(mem((long)pl[14], &VN));
+        if (KN->half != Q->half || VN->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(KN, 0, B * KVH * hs);
+        RANGE(VN, 0, B * KVH * hs);
+        HIPCHK(k_rope_append(s, Q->dt(), Q->ptr, KN->ptr, VN->ptr, KC->ptr, VC->ptr, (int)B, (int)H, (int)KVH, (int)hs,
+                             (int)len - 1, sB, sH, sT, rp ? (const float*)rp->dcos.get() : nullptr,
+                             rp ? (const float*)rp->dsin.get() : nullptr));
+        m_mem.touch((long)pl[5]);
+        m_mem.touch((long)pl[6]);
+        m_mem.touch((long)pl[7]);
+        m_mem.touch((long)pl[13]);
+    }
+    size_t wsb = attn_decode_workspace_bytes((int)B, (int)H, (int)hs, (int)len);
+    void* ws;
+    size_t wsHave;
+    int* tk;
+    if (staticScratch) {
+        // partials and tickets live in this device's copy of the file-scope array: nothing is allocated
+        char* base = nullptr;
+        ERRCHK(static_scratch(m_device, &base));
+        if (B * H > MCH_NOALLOC_MAX_TICKETS || wsb > MCH_NOALLOC_PARTIAL_BYTES) {
+            last_detail = "the no-allocation decode attention holds at most 4096 (batch x head) pairs and 4 MiB of split partials";
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        tk = (int*)base;
+        ws = base + MCH_NOALLOC_MAX_TICKETS * sizeof(int);
+        wsHave = MCH_NOALLOC_PARTIAL_BYTES;
+        // the array keeps what the last call left: the tickets must start at zero (a fill kernel, so that a caller
+        // may capture the call into a graph)
+        HIPCHK(k_set(s, F32, tk, (size_t)(B * H), 0.f));
+    } else {
+        ERRCHK(workspace(wsb, &ws));
+        wsHave = m_wsBytes;
+        ERRCHK(tickets((size_t)(B * H), &tk));
+    }
+    HIPCHK(k_attn_decode(s, Q->dt(), Q->ptr, KC->ptr, VC->ptr, Y->ptr, (int)B, (int)H, (int)KVH, (int)hs, (int)len, sB, sH,
+                         sT, scale, ws, wsHave, nullptr, tk));
+    m_mem.touch((long)pl[8]);
+    return 0;
+}
+
+// the same call through the entry point that allocates nothing
+long Kernel::attn_decode_no_alloc(float* pf, long lf, MCH_LONGLONG* pl, long ll)
+{
+    last_detail.clear();
+    if (!m_stream) return MCH_ERROR_DEVICE_NOT_INITIALIZED;
+    HIPCHK(hipSetDevice(m_device));
+    return attn_decode_fwd(pf, lf, pl, ll, true);
 }
 
 long Kernel::run_extension(long hExt, long fn, float* pf, long lf, MCH_TCHAR* szIn, float** ppOut, MCH_LONG* plOut,
@@ -2122,6 +2190,18 @@ MCH_LONG Internal_AllocHostFloat(MCH_LONG kIdx, MCH_LONG count, float** dst, flo
     return (MCH_LONG)k->alloc_host(count, dst, src, srcOnDevice);
 }
 MCH_LONG Internal_AllocHostDouble(MCH_LONG, MCH_LONG, double**, double*, bool) { return MCH_ERROR_NOT_IMPLEMENTED; }
+
+MCH_LONG MCH_AttnDecodeForwardNoAlloc(MCH_LONG kIdx, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn, MCH_TCHAR* szErr,
+                                      MCH_LONG errMax)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    if (kIdx < 0 || kIdx >= MAX_KERNELS) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    Kernel* k = kernel_at(kIdx);
+    if (!k) { put_error(nullptr, MCH_ERROR_PARAM_NULL, szErr, errMax); return MCH_ERROR_PARAM_NULL; }
+    long e = k->attn_decode_no_alloc(pIn, lIn, plIn, llIn);
+    if (e) put_error(k, e, szErr, errMax);
+    return (MCH_LONG)e;
+}
 
 MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG kIdx, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn,
                                 MCH_LONG nWarmup, MCH_LONG nReps, float* pfMs, MCH_TCHAR* szErr, MCH_LONG errMax)

@@ -26,6 +26,7 @@
 #include <atomic>
 #include <functional>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <algorithm>
@@ -219,6 +220,69 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
                 else if (MODE == 1) *out = prev[rr] + a0;
                 else *out = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
             }
+        }
+    }
+}
+
+// The same family for rows too long to hold in registers (n > 4096): one wavefront per row walks K in slabs of
+// 64 x 4 columns, four slabs in flight.  With NORM the sum of squares of x (L2 resident) is taken in a first walk.
+template <typename T, int MODE, bool NORM>
+__global__ __launch_bounds__(256) void matvec_loop_kernel(const T* __restrict__ W, const float* __restrict__ x,
+                                                          const float* __restrict__ g, float* __restrict__ y, int rows, int n,
+                                                          int B, int ldy)
+{
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const T* w0 = W + (size_t)r * n;
+    const T* w1 = W + (size_t)(r + rows) * n;   // only read when MODE == 2
+    constexpr int U = 4;
+    for (int b = 0; b < B; b++) {
+        const float* xb = x + (size_t)b * n;
+        const float prev = (MODE == 1 && lane == 0) ? y[(size_t)b * ldy + r] : 0.f;
+        float inv = 1.f;
+        if (NORM) {
+            float ss = 0.f;
+            for (int j = lane * 4; j < n; j += 256) {
+                const float4 v = *(const float4*)(xb + j);
+                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            }
+            ss = wsum(ss);
+            inv = 1.0f / sqrtf(ss / n + 1e-5f);
+        }
+        float a0 = 0.f, a1 = 0.f;
+        for (int j0 = lane * 4; j0 < n; j0 += 256 * U) {
+            float4 wv[U], w2v[MODE == 2 ? U : 1], xv[U], gv[NORM ? U : 1];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int j = j0 + u * 256;
+                const bool in = j < n;
+                wv[u] = in ? Row4<T>::load(w0 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (MODE == 2) w2v[MODE == 2 ? u : 0] = in ? Row4<T>::load(w1 + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+                xv[u] = in ? *(const float4*)(xb + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (NORM) gv[NORM ? u : 0] = in ? *(const float4*)(g + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float4 v = xv[u];
+                if (NORM) {
+                    const float4 gq = gv[NORM ? u : 0];
+                    v.x = gq.x * (inv * v.x); v.y = gq.y * (inv * v.y); v.z = gq.z * (inv * v.z); v.w = gq.w * (inv * v.w);
+                }
+                a0 += wv[u].x * v.x + wv[u].y * v.y + wv[u].z * v.z + wv[u].w * v.w;
+                if (MODE == 2) {
+                    const float4 q = w2v[MODE == 2 ? u : 0];
+                    a1 += q.x * v.x + q.y * v.y + q.z * v.z + q.w * v.w;
+                }
+            }
+        }
+        a0 = wsum(a0);
+        if (MODE == 2) a1 = wsum(a1);
+        if (lane == 0) {
+            float* out = y + (size_t)b * ldy + r;
+            if (MODE == 0) *out = a0;
+            else if (MODE == 1) *out = prev + a0;
+            else *out = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
         }
     }
 }
@@ -518,12 +582,15 @@ class Engine {
 public:
     Config cfg{};
     bool loaded = false;
-    bool bf16_weights = false;
+    bool bf16_weights = false;   // storage the NEXT load uploads the weights in
+    bool stored_bf16 = false;    // storage of the weights that are on the device now: every launch dispatches on this
     bool use_graph = true;
+    bool lastUsedGraph = false;  // whether the last generate replayed a captured graph (false: eager launches)
     int mvRows = 0;              // weight rows per wavefront in the mat-vec kernels (0: chosen per shape)
     void set_mv_rows(int r) { mvRows = r; graphB = -1; }   // the captured step is rebuilt at the next generation
     int shared_classifier = 0;
     int timedFrom = -1;          // first step of the timed span (-1: first step after the prompt)
+    std::string lastError;       // detail of the last failed load, handed to the caller's error text
     float lastTimedMs = 0.f;     // HIP-event duration of the timed span of the last generate
     int lastTimedSteps = 0;
 
@@ -656,21 +723,31 @@ template <typename T> long Engine::upload(const float* p)
 long Engine::load(const char* path)
 {
     release();
+    lastError.clear();
     FILE* f = fopen(path, "rb");
-    if (!f) return MCH_ERROR_LLM_MISSING_MODEL_FILE;
+    if (!f) { lastError = "The model file could not be opened."; return MCH_ERROR_LLM_MISSING_MODEL_FILE; }
     // header (llama2_cpu.cpp:108-147): magic "ak42", version 1, Config, shared-classifier byte, 256 bytes in all
     uint32_t magic = 0;
     int version = 0;
     uint8_t shared = 0;
     bool ok = fread(&magic, 4, 1, f) == 1 && magic == 0x616b3432 && fread(&version, 4, 1, f) == 1 && version == 1 &&
               fread(&cfg, sizeof(Config), 1, f) == 1 && fread(&shared, 1, 1, f) == 1;
-    if (!ok) { fclose(f); return MCH_ERROR_LLM_LOAD_MODEL; }
+    if (!ok) {
+        fclose(f);
+        lastError = "Not a llama2.c version 1 checkpoint (magic 'ak42', version 1, seven-integer configuration).";
+        return MCH_ERROR_LLM_LOAD_MODEL;
+    }
     shared_classifier = shared;
-    if (cfg.seq_len > 20480) cfg.seq_len = 20480;
+    if (cfg.seq_len > 20480) cfg.seq_len = 20480;   // the reference clamps the context the same way (llama2_cpu.cpp:145)
     if (cfg.dim <= 0 || cfg.n_heads <= 0 || cfg.n_kv_heads <= 0 || cfg.n_layers <= 0 || cfg.vocab_size <= 0 || cfg.seq_len <= 0 ||
         cfg.hidden_dim <= 0 || cfg.dim % cfg.n_heads || cfg.n_heads % cfg.n_kv_heads || (cfg.dim / cfg.n_heads) % 2 ||
-        cfg.dim % 4 || cfg.hidden_dim % 4 || cfg.dim > 64 * 4 * 16 || cfg.hidden_dim > 64 * 4 * 16) {
+        cfg.dim % 4 || cfg.hidden_dim % 4) {
         fclose(f);
+        char msg[256];
+        snprintf(msg, sizeof(msg), "Unsupported model shape: dim %d, hidden %d, layers %d, heads %d, kv heads %d, vocabulary %d, "
+                 "context %d (dim and hidden must be multiples of 4, dim a multiple of heads, heads of kv heads, head size even).",
+                 cfg.dim, cfg.hidden_dim, cfg.n_layers, cfg.n_heads, cfg.n_kv_heads, cfg.vocab_size, cfg.seq_len);
+        lastError = msg;
         return MCH_ERROR_LLM_LOAD_MODEL;
     }
     const size_t L = cfg.n_layers, dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
@@ -678,15 +755,20 @@ long Engine::load(const char* path)
     if (!shared) need += (size_t)cfg.vocab_size * dim;
     fseek(f, 0, SEEK_END);
     long fsize = ftell(f);
-    if (fsize < 0 || (size_t)fsize < 256 + need * 4) { fclose(f); return MCH_ERROR_LLM_LOAD_MODEL; }
+    if (fsize < 0 || (size_t)fsize < 256 + need * 4) {
+        fclose(f);
+        lastError = "The model file is shorter than its configuration requires.";
+        return MCH_ERROR_LLM_LOAD_MODEL;
+    }
     fseek(f, 256, SEEK_SET);
     std::vector<float> blob(need);
     size_t got = fread(blob.data(), 4, need, f);
     fclose(f);
-    if (got != need) return MCH_ERROR_LLM_LOAD_MODEL;
+    if (got != need) { lastError = "The model file could not be read."; return MCH_ERROR_LLM_LOAD_MODEL; }
 
     HIPCHK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
-    long e = bf16_weights ? upload<bf16_t>(blob.data()) : upload<float>(blob.data());
+    stored_bf16 = bf16_weights;
+    long e = stored_bf16 ? upload<bf16_t>(blob.data()) : upload<float>(blob.data());
     if (e) { release(); return e; }
     // rotary tables as precompute_freqs_cis builds them (llama2_cpu.cpp:388-414)
     const int half = (int)hs / 2;
@@ -787,7 +869,7 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     else if (ch <= 4) MV(4);
     else if (ch <= 8) MV(8);
     else if (ch <= 16) MV(16);
-    else return hipErrorInvalidValue;
+    else hipLaunchKernelGGL((matvec_loop_kernel<T, MODE, NORM>), (rows + 3) / 4, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy);
 #undef MV1
 #undef MV
     return hipGetLastError();
@@ -796,7 +878,7 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
 // x = embedding of the token at the starting position; later steps get theirs from the previous step's tail kernel
 hipError_t Engine::embed_first(hipStream_t s, int B)
 {
-    if (bf16_weights)
+    if (stored_bf16)
         hipLaunchKernelGGL(embed_step_kernel<bf16_t>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const bf16_t*)emb, x, cfg.dim, dcur);
     else
         hipLaunchKernelGGL(embed_step_kernel<float>, B, 256, 0, s, dstate, dprompt, cfg.seq_len, dnext, (const float*)emb, x, cfg.dim, dcur);
@@ -905,7 +987,7 @@ long Engine::profile_step(int pos, int reps, int B, std::vector<float>* out)
         std::sort(empty.begin(), empty.end());
     }
     StepProfile prof;
-    for (int i = 0; i < reps && !e; i++) e = bf16_weights ? step<bf16_t>(s, B, cfg.seq_len, nullptr, &prof) : step<float>(s, B, cfg.seq_len, nullptr, &prof);
+    for (int i = 0; i < reps && !e; i++) e = stored_bf16 ? step<bf16_t>(s, B, cfg.seq_len, nullptr, &prof) : step<float>(s, B, cfg.seq_len, nullptr, &prof);
     hipError_t he = hipStreamSynchronize(s);
     if (!e && he != hipSuccess) e = (long)he;
     std::vector<double> ms(SC_COUNT, 0.0), cnt(SC_COUNT, 0.0);
@@ -916,7 +998,7 @@ long Engine::profile_step(int pos, int reps, int B, std::vector<float>* out)
         (void)hipEventDestroy(sp.second.second);
     }
     if (e) return e;
-    const double es = bf16_weights ? 2.0 : 4.0;
+    const double es = stored_bf16 ? 2.0 : 4.0;
     const double L = cfg.n_layers, dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
     const double meanLen = pos + 1 + (reps - 1) / 2.0;
     double bytes[SC_COUNT] = {0};
@@ -953,10 +1035,21 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     GenState st0 = {0, nPrompt, 1, 0};
     HIPCHK(hipMemcpyAsync(dstate, &st0, sizeof(st0), hipMemcpyHostToDevice, s));
     HIPCHK(hipStreamSynchronize(s));
-    float* allLogits = nullptr;
+    // owned here so that every early return below releases them
+    struct Scratch {
+        float* allLogits = nullptr;
+        hipEvent_t evA = nullptr, evB = nullptr;
+        ~Scratch()
+        {
+            if (allLogits) (void)hipFree(allLogits);
+            if (evA) (void)hipEventDestroy(evA);
+            if (evB) (void)hipEventDestroy(evB);
+        }
+    } sc;
     if (wantLogits) {
-        HIPCHK(hipMalloc((void**)&allLogits, (size_t)B * nSteps * cfg.vocab_size * 4));
+        HIPCHK(hipMalloc((void**)&sc.allLogits, (size_t)B * nSteps * cfg.vocab_size * 4));
     }
+    float* const allLogits = sc.allLogits;
     // With a sampler whose temperature is not 0 the id of every step is chosen on the host, as in the reference: the
     // step's kernels stop at the logits, which are copied out, sampled, and the chosen id goes back for the step's tail.
     const bool hostSample = sampler && !sampler->greedy();
@@ -971,12 +1064,12 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         if (!hGiven) HIPCHK(hipHostMalloc((void**)&hGiven, 64 * sizeof(int), hipHostMallocDefault));
     }
     auto enqueue = [&]() -> long {
-        return bf16_weights ? step<bf16_t>(s, B, nSteps, allLogits, nullptr, !hostSample)
+        return stored_bf16 ? step<bf16_t>(s, B, nSteps, allLogits, nullptr, !hostSample)
                             : step<float>(s, B, nSteps, allLogits, nullptr, !hostSample);
     };
-    hipEvent_t evA = nullptr, evB = nullptr;
-    (void)hipEventCreate(&evA);
-    (void)hipEventCreate(&evB);
+    HIPCHK(hipEventCreate(&sc.evA));
+    HIPCHK(hipEventCreate(&sc.evB));
+    const hipEvent_t evA = sc.evA, evB = sc.evB;
     const int t0 = timedFrom < 0 ? nPrompt : timedFrom;
     bool graph = use_graph && !wantLogits;
     if (graph && (!graphExec || graphB != B || graphArgmax != !hostSample)) {
@@ -994,6 +1087,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         graphB = B;
         graphArgmax = !hostSample;
     }
+    lastUsedGraph = graph;
     HIPCHK(embed_first(s, B));
     int done = 0;
     for (int i = 0; i < nSteps && !e; i++) {
@@ -1009,7 +1103,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
             for (int b = 0; b < B; b++) hGiven[b] = sampler->sample(hLogits + (size_t)b * V, (int)V);
             hc = hipMemcpyAsync(dgiven, hGiven, (size_t)B * sizeof(int), hipMemcpyHostToDevice, s);
             if (hc != hipSuccess) { e = (long)hc; break; }
-            e = bf16_weights ? advance_given<bf16_t>(s, B) : advance_given<float>(s, B);
+            e = stored_bf16 ? advance_given<bf16_t>(s, B) : advance_given<float>(s, B);
             if (e) break;
         }
         done++;
@@ -1033,8 +1127,6 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         (void)hipEventElapsedTime(&lastTimedMs, evA, evB);
         lastTimedSteps = done - t0;
     }
-    (void)hipEventDestroy(evA);
-    (void)hipEventDestroy(evB);
     if (!e) {
         ids->assign((size_t)B * nSteps, 0);
         std::vector<int> tmp((size_t)B * cfg.seq_len);
@@ -1047,7 +1139,6 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
             if (he != hipSuccess) e = (long)he;
         }
     }
-    if (allLogits) (void)hipFree(allLogits);
     return e;
 }
 
@@ -1075,10 +1166,10 @@ typedef MCH_LONG (*FnAllocHost)(MCH_LONG, MCH_LONG, float**, float*, bool);
 static FnInvoke g_parentInvoke = nullptr;
 static FnAllocHost g_parentAllocHost = nullptr;
 static MCH_LONG g_kernelIdx = 0;
-static std::map<long, Llm*> g_llms;
+static std::map<long, std::shared_ptr<Llm>> g_llms;   // calls in flight hold a reference of their own
 static std::mutex g_mapLock;
 
-static Llm* find_llm(long h)
+static std::shared_ptr<Llm> find_llm(long h)
 {
     std::lock_guard<std::mutex> g(g_mapLock);
     auto it = g_llms.find(h);
@@ -1185,7 +1276,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
     if (!g_parentInvoke) return MCH_ERROR_EXTENSION_NOT_INITIALIZED;
     switch (fn) {
     case MCH_LLM_CREATE: {
-        Llm* m = new Llm();
+        std::shared_ptr<Llm> m = std::make_shared<Llm>();
         if (lIn > 0) m->temperature = pIn[0];
         if (lIn > 1) m->topp = pIn[1];
         if (lIn > 2) m->seed = (long)pIn[2];
@@ -1199,13 +1290,12 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         if (e) {
             std::lock_guard<std::mutex> g(g_mapLock);
             g_llms.erase(h);
-            delete m;
         }
         return (MCH_LONG)e;
     }
     case MCH_LLM_DESTROY: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = nullptr;
+        std::shared_ptr<Llm> m;
         {
             std::lock_guard<std::mutex> g(g_mapLock);
             auto it = g_llms.find((long)pIn[0]);
@@ -1213,27 +1303,29 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         }
         if (m) {
             m->cancel.store(true);
-            std::lock_guard<std::mutex> run(m->runLock);  // wait for a running generate to notice the flag
-            delete m;
+            // wait for a running generate to notice the flag; the lock is released before the object can go away, and
+            // a call that looked the handle up before the erase keeps the object alive until it returns
+            { std::lock_guard<std::mutex> run(m->runLock); }
+            m.reset();
         }
         return 0;
     }
     case MCH_LLM_ABORT: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (m) m->cancel.store(true);
         return 0;
     }
     case MCH_LLM_QUERYSTATUS: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         float v = m->loaded.load() ? 1.f : 0.f;
         return (MCH_LONG)give({v, v}, ppOut, plOut);
     }
     case MCH_LLM_SET_OPTION: {
         if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         std::lock_guard<std::mutex> run(m->runLock);
         int opt = (int)pIn[1];
@@ -1247,13 +1339,13 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
     }
     case MCH_LLM_QUERY_TIMING: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
-        return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps}, ppOut, plOut);
+        return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps, m->engine.lastUsedGraph ? 1.f : 0.f}, ppOut, plOut);
     }
     case MCH_LLM_PROFILE_STEP: {
         if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         std::lock_guard<std::mutex> run(m->runLock);
         std::vector<float> out;
@@ -1264,7 +1356,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
     case MCH_LLM_SAMPLE: {
         // f{hLlm, logits...} -> f{id}: one call of the handle's sampler (advances its random state unless greedy)
         if (lIn < 2) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
         std::lock_guard<std::mutex> run(m->runLock);
@@ -1278,7 +1370,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         const bool batch = fn == MCH_LLM_GENERATE_BATCH;
         const int head = batch ? 4 : 3;
         if (lIn < head + 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         std::lock_guard<std::mutex> run(m->runLock);
         const int nSteps = (int)pIn[1];
@@ -1318,7 +1410,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
     case MCH_LLM_LOAD: {
         // "model.bin;tokenizer.bin" (llm.cpp:78-98).  An empty tokenizer part selects the token-id front door.
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return 0;
         std::string in = narrow(szIn), model = in, tok;
         size_t p = in.find(';');
@@ -1338,6 +1430,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         m->busy.store(false);
         if (!e) m->sampler.build(m->temperature, m->topp, (unsigned long long)m->seed);
         m->loaded.store(e == 0);
+        if (e && !m->engine.lastError.empty()) put_text(szErr, errMax, m->engine.lastError.c_str());
         return (MCH_LONG)e;
     }
     case MCH_LLM_GENERATE: {
@@ -1346,7 +1439,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         // appends its piece to the response; stop at EOS, at the step limit or on ABORT.  The device loop runs
         // in chunks of 32 positions, so the response grows while the caller polls QUERY_RESPONSE.
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
         if (!m->tokenizer.loaded()) {
@@ -1397,7 +1490,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
     case MCH_LLM_TOKENIZE: {
         // f{hLlm, bos, eos} + text -> token ids; f{hLlm, -1, prev, token} -> the piece in szOutput
         if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
         if (!m->tokenizer.loaded()) return MCH_ERROR_LLM_MISSING_TOKENIZER_FILE;
         if (pIn[1] < 0.f) {
@@ -1410,7 +1503,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
     }
     case MCH_LLM_QUERYRESPONSE: {
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        Llm* m = find_llm((long)pIn[0]);
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         long end = 1;
         if (m) {
             std::lock_guard<std::mutex> g(m->responseLock);
@@ -1430,6 +1523,23 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
         put_text(szErr, errMax, "The function specified is not supported.");
         return MCH_ERROR_NOT_IMPLEMENTED;
     }
+}
+
+// Double twins of the three exports (CudaExtension.llm32.11.8.def:8-11): the engine computes in fp32 only.
+static MCH_LONG ext_double_unsupported(MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    put_text(szErr, errMax, "The double base type is not built: the llama2 engine runs in fp32 and 16-bit storage. (90009)");
+    return MCH_ERROR_NOT_IMPLEMENTED;
+}
+MCH_LONG DLL_InitDoubleCustomExtension(void*, MCH_LONG) { return MCH_ERROR_NOT_IMPLEMENTED; }
+MCH_LONG DLL_InvokeDoubleCustomExtension(MCH_LONG, double*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return ext_double_unsupported(szErr, errMax);
+}
+MCH_LONG DLL_InvokeDoubleCustomExtensionEx(MCH_LONG, double*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR*, MCH_TCHAR*, MCH_LONG,
+                                           MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return ext_double_unsupported(szErr, errMax);
 }
 
 }  // extern "C"

@@ -138,6 +138,7 @@ public:
     ~Kernel();
     long initialize(const float* pf, long n);
     long run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float** ppOut, MCH_LONG* plOut, bool timing);
+    long attn_decode_no_alloc(float* pf, long lf, MCH_LONGLONG* pl, long ll);
     long run_extension(long hExt, long fn, float* pf, long lf, MCH_TCHAR* szIn, float** ppOut, MCH_LONG* plOut,
                        MCH_TCHAR* szErr, long errMax);
     long create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut);
@@ -152,6 +153,7 @@ public:
     std::string last_detail;  // human-readable detail of the last failure
 
 private:
+    long attn_decode_fwd(float* pf, long lf, MCH_LONGLONG* pl, long ll, bool staticScratch);
     long workspace(size_t bytes, void** p);
     long staging(size_t bytes, void** p);
     long tickets(size_t count, int** p);

@@ -168,10 +168,11 @@ EXPORTS = (
     "DLL_InvokeFloat", "DLL_InvokeDouble", "DLL_QueryString", "DLL_InvokeFloatEx", "DLL_InvokeDoubleEx",
     "DLL_InvokeFloatEx2", "DLL_InvokeDoubleEx2", "Internal_GetPointerFloat", "Internal_GetPointerDouble",
     "Internal_AllocHostFloat", "Internal_AllocHostDouble", "DLL_QueryStringFloatEx", "DLL_QueryStringDoubleEx",
-    "MCH_TimeInvokeFloatEx2",
+    "MCH_TimeInvokeFloatEx2", "MCH_AttnDecodeForwardNoAlloc",
 )
 EXTENSION_EXPORTS = (
     "DLL_InitFloatCustomExtension", "DLL_InvokeFloatCustomExtension", "DLL_InvokeFloatCustomExtensionEx",
+    "DLL_InitDoubleCustomExtension", "DLL_InvokeDoubleCustomExtension", "DLL_InvokeDoubleCustomExtensionEx",
 )
 
 
@@ -210,6 +211,8 @@ def load_library(path=None):
     lib.MCH_TimeInvokeFloatEx2.argtypes = [_c_long, _c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_long, _c_long,
                                            _c_float_p, _c_tchar_p, _c_long]
     lib.MCH_TimeInvokeFloatEx2.restype = _c_long
+    lib.MCH_AttnDecodeForwardNoAlloc.argtypes = [_c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_tchar_p, _c_long]
+    lib.MCH_AttnDecodeForwardNoAlloc.restype = _c_long
     return lib
 
 
@@ -652,6 +655,20 @@ class CudaDnn:
         if hRope or hKNew or hVNew:
             rgl += [hRope, hKNew, hVNew]
         self._ex2(CUDAFN.ATTN_DECODE_FWD, [fScale], rgl)
+
+    def AttnDecodeForwardNoAlloc(self, nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead,
+                                 nStridePos, fScale=0.0, hRope=0, hKNew=0, hVNew=0):
+        """AttnDecodeForward through the entry point that allocates no device memory (fixed scratch inside the
+        library; for callers that cannot call hipMalloc).  Same arguments, bounded problem size."""
+        rgl = [nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead, nStridePos]
+        if hRope or hKNew or hVNew:
+            rgl += [hRope, hKNew, hVNew]
+        a, n = self._farr([fScale])
+        l, ln = self._larr(rgl)
+        errbuf = (ctypes.c_uint16 * _ERRMAX)()
+        err = self._lib.MCH_AttnDecodeForwardNoAlloc(self.m_hKernel, a.ctypes.data_as(_c_float_p), n, l.ctypes.data_as(_c_longlong_p),
+                                                     ln, errbuf, _ERRMAX)
+        self._check(err, errbuf)
 
     def RmsNormForward(self, nOuter, nDim, hX, hWeight, hY, fEps=1e-5):
         """Fused RMSNorm (replaces the chain of RMSNormLayer.cs:156-180)."""

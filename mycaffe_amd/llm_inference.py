@@ -116,6 +116,12 @@ class LlmInference:
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
         return float(rg[0]), int(rg[1])
 
+    def LastRunUsedGraph(self):
+        """Whether the steps of the last generation were replays of the captured HIP graph (False: eager launches,
+        either asked for with option 3 or because capture failed)."""
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
+        return bool(rg[2] != 0)
+
     def ProfileStep(self, pos, reps=8, batch=1):
         """Per-kernel-class timing of eager decode steps at ``pos`` (HIP event pairs around
         every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}, plus

@@ -42,6 +42,43 @@ def test_double_entry_points_report_not_implemented():
     assert "double" in C._from_utf16(err)
 
 
+def test_extension_double_twins_report_not_implemented():
+    # CudaExtension.llm32.11.8.def:8-11 lists the double twins; they exist and refuse
+    if not os.path.exists(C.llama2_extension_path()):
+        pytest.skip("extension library not built")
+    ext = ctypes.CDLL(C.llama2_extension_path())
+    err = (ctypes.c_uint16 * 256)()
+    assert ext.DLL_InitDoubleCustomExtension(None, 1) == C.ERROR.NOT_IMPLEMENTED
+    assert ext.DLL_InvokeDoubleCustomExtension(1, None, 0, None, None, err, 256) == C.ERROR.NOT_IMPLEMENTED
+    assert "double" in C._from_utf16(err)
+    assert ext.DLL_InvokeDoubleCustomExtensionEx(5, None, 0, None, None, None, None, 0, err, 256) == C.ERROR.NOT_IMPLEMENTED
+
+
+def _def_exports(name):
+    text = open(os.path.join(ROOT, "mycaffe_amd", "csrc", name)).read()
+    body = text.split("EXPORTS", 1)[1]
+    return [l.split()[0] for l in body.splitlines() if l.strip() and not l.strip().startswith(";")]
+
+
+def test_def_files_list_what_the_libraries_export():
+    # the Windows export lists name exactly the header's entry points, library by library
+    decl = set(_declared_symbols())
+    main, ext = _def_exports("mycaffe_hip.def"), _def_exports("mycaffe_hip_llama2.def")
+    assert set(main) == decl - set(C.EXTENSION_EXPORTS)
+    assert set(ext) == set(C.EXTENSION_EXPORTS)
+    assert set(C.EXPORTS) == set(main)
+
+
+def test_no_alloc_entry_rejects_bad_kernel_before_touching_a_device():
+    lib = C.load_library()
+    err = (ctypes.c_uint16 * 256)()
+    l = np.zeros(12, np.int64)
+    f = np.zeros(1, np.float32)
+    fp, lp = f.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), l.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
+    assert lib.MCH_AttnDecodeForwardNoAlloc(77, fp, 1, lp, 12, err, 256) == C.ERROR.PARAM_NULL
+    assert lib.MCH_AttnDecodeForwardNoAlloc(5000, fp, 1, lp, 12, err, 256) == C.ERROR.PARAM_OUT_OF_RANGE
+
+
 def test_uninitialised_kernel_and_bad_index_codes():
     # CudaDnnDLL.cpp:296-301: a null table slot gives ERROR_PARAM_NULL; indices outside the table ERROR_PARAM_OUT_OF_RANGE
     lib = C.load_library()
