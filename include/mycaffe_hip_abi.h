@@ -249,9 +249,10 @@ enum {
      *                 option 4 = weight rows per wavefront of the mat-vec
      *                 kernels (1 or 2; 0 = library's choice); option 5 = GENERATE_IDS /
      *                 GENERATE_BATCH draw from the handle's sampler (temperature, top-p,
-     *                 seed of CREATE) instead of the argmax (0, default)
+     *                 seed of CREATE) instead of the argmax (0, default); option 6 = GENERATE_BATCH
+     *                 appends the logits of every step, batch x nSteps x vocabulary (0, default)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
-     *                 -> f{batch x nSteps next ids}
+     *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were
      *                 replays of the captured graph / 0 if they were launched eagerly}
      *   PROFILE_STEP  f{hLlm, pos, reps[, batch]} -> per kernel class of one decode step

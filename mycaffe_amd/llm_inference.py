@@ -104,12 +104,18 @@ class LlmInference:
             return ids, rg[nSteps:].reshape(nSteps, -1)
         return ids
 
-    def GenerateBatch(self, prompts, nSteps):
-        """prompts: (batch, nPrompt) ids; returns (batch, nSteps) sampled ids."""
+    def GenerateBatch(self, prompts, nSteps, want_logits=False):
+        """prompts: (batch, nPrompt) ids; returns (batch, nSteps) sampled ids (and, on request, the logits of
+        every step, (batch, nSteps, vocabulary))."""
         p = np.asarray(prompts)
         args = self.m_rgLlm + [nSteps, p.shape[0], p.shape[1]] + [float(t) for t in p.reshape(-1)]
+        self.SetOption(6, 1 if want_logits else 0)
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.GENERATE_BATCH, args)
-        return rg.astype(np.int32).reshape(p.shape[0], nSteps)
+        n = p.shape[0] * nSteps
+        ids = rg[:n].astype(np.int32).reshape(p.shape[0], nSteps)
+        if want_logits:
+            return ids, rg[n:].reshape(p.shape[0], nSteps, -1)
+        return ids
 
     def QueryTiming(self):
         """(milliseconds, steps) of the timed span of the last generation, from HIP events."""

@@ -44,20 +44,39 @@ def llm():
     cuda.Dispose()
 
 
-def _rel_gap(logits_row):
-    s = np.sort(logits_row)
-    return (s[-1] - s[-2]) / max(abs(s[-1]), 1e-30)
+def _first_max(logits):
+    """sample_argmax (llama2_sampler.cpp:25-36): strict '>' scan, so the lowest index wins a tie."""
+    return np.argmax(logits, axis=-1)
 
 
-def _ids_match(ids, ref_ids, ref_logits, what):
-    """Greedy ids bit-exact.  Where they first differ the checker's own top-2 gap must be below the fp32 parity
-    tolerance (an undetermined argmax); that is reported as a failure all the same unless it is such a tie."""
+def _ids_match(ids, ref_ids, ref_logits, what, logits=None):
+    """Greedy ids bit-exact against the checker.  Sequences can only part where the checker's own top-2 logits are
+    closer than the fp32 parity tolerance allows the two implementations to differ: anything else fails.  When the
+    device logits are given, every chosen id must also be the first-max argmax of those logits, bit-exact."""
+    ids, ref_ids = np.asarray(ids), np.asarray(ref_ids)
+    if logits is not None:
+        assert np.array_equal(ids, _first_max(logits)), what + ": id is not the first-max argmax of the device logits"
     if np.array_equal(ids, ref_ids):
-        return
-    first = int(np.argmax(np.asarray(ids) != np.asarray(ref_ids)))
-    gap = _rel_gap(ref_logits[first])
+        return True
+    first = int(np.argmax(ids != ref_ids))
+    top2 = np.sort(ref_logits[first])[-2:]
+    gap = (top2[1] - top2[0]) / max(float(np.abs(ref_logits[first]).max()), 1e-30)
+    print("%s: ids part at step %d, checker's relative top-2 gap %.3e" % (what, first, gap), flush=True)
     assert gap < FP32_RTOL, "%s: ids differ at step %d where the checker's top-2 gap is %.3e" % (what, first, gap)
-    pytest.skip("%s: tie at step %d (relative top-2 gap %.2e); ids before it are identical" % (what, first, gap))
+    return False
+
+
+def _batch_rows_against_cpu(cpu, prompts, n, ids, logits, what):
+    """Every sequence of a batched generation against its own CPU run: logits of every step up to the point where the
+    two id streams part (they may only part at a tie of the checker's top-2 logits), ids bit-exact before it."""
+    parted = 0
+    for b in range(len(prompts)):
+        ref_ids, ref_logits = cpu.generate_greedy(prompts[b], n, want_logits=True)
+        same = _ids_match(ids[b], ref_ids, ref_logits, "%s, sequence %d" % (what, b), logits[b])
+        upto = n if same else int(np.argmax(np.asarray(ids[b]) != np.asarray(ref_ids))) + 1
+        assert_close(logits[b, :upto], ref_logits[:upto], FP32_RTOL, "%s, sequence %d logits" % (what, b))
+        parted += 0 if same else 1
+    assert parted <= 2, "%s: %d of %d sequences parted from the checker" % (what, parted, len(prompts))
 
 
 def test_llama110m_batch1_fp32_logits_and_ids(llm, c4_model):
@@ -68,7 +87,7 @@ def test_llama110m_batch1_fp32_logits_and_ids(llm, c4_model):
     ref_ids, ref_logits = O.Llama(C4, blob).generate_greedy(prompt, n, want_logits=True)
     ids, logits = llm.GenerateIds(prompt, n, want_logits=True)   # eager launches
     assert_close(logits, ref_logits, FP32_RTOL, "110M logits, every position")
-    _ids_match(ids, ref_ids, ref_logits, "110M eager")
+    assert _ids_match(ids, ref_ids, ref_logits, "110M eager", logits)
     ids_graph = llm.GenerateIds(prompt, n)                        # one captured graph per step
     assert llm.LastRunUsedGraph()
     assert np.array_equal(ids_graph, ids)
@@ -80,11 +99,11 @@ def test_llama110m_batch16_fp32_every_row_an_independent_cpu_run(llm, c4_model):
     rng = np.random.default_rng(16)
     B, nP, n = 16, 24, 64
     prompts = rng.integers(3, C4["vocab_size"], (B, nP))
-    ids = llm.GenerateBatch(prompts, n)
-    cpu = O.Llama(C4, blob)
-    for b in range(B):
-        ref_ids, ref_logits = cpu.generate_greedy(prompts[b], n, want_logits=True)
-        _ids_match(ids[b], ref_ids, ref_logits, "110M batch 16, sequence %d" % b)
+    ids, logits = llm.GenerateBatch(prompts, n, want_logits=True)   # eager launches
+    ids_graph = llm.GenerateBatch(prompts, n)                        # one captured graph per step
+    assert llm.LastRunUsedGraph()
+    assert np.array_equal(ids_graph, ids)
+    _batch_rows_against_cpu(O.Llama(C4, blob), prompts, n, ids, logits, "110M batch 16")
 
 
 @pytest.mark.parametrize("batch", [1, 16])
@@ -101,7 +120,7 @@ def test_llama110m_bf16_weights_against_checker_on_rounded_weights(llm, c4_model
         ref_ids, ref_logits = cpu.generate_greedy(prompt, n, want_logits=True)
         ids, logits = llm.GenerateIds(prompt, n, want_logits=True)
         assert_close(logits, ref_logits, FP32_RTOL, "bf16-weight logits vs checker on rounded weights")
-        _ids_match(ids, ref_ids, ref_logits, "110M bf16 weights")
+        assert _ids_match(ids, ref_ids, ref_logits, "110M bf16 weights", logits)
         assert np.array_equal(llm.GenerateIds(prompt, n), ids)
         # and the rounding itself stays inside the 16-bit bar against the fp32 model
         _, full = O.Llama(C4, blob).generate_greedy(prompt, 4, want_logits=True)
@@ -109,10 +128,9 @@ def test_llama110m_bf16_weights_against_checker_on_rounded_weights(llm, c4_model
     else:
         prompts = rng.integers(3, C4["vocab_size"], (batch, 16))
         n = 48
-        ids = llm.GenerateBatch(prompts, n)
-        for b in range(batch):
-            ref_ids, ref_logits = cpu.generate_greedy(prompts[b], n, want_logits=True)
-            _ids_match(ids[b], ref_ids, ref_logits, "110M bf16 batch 16, sequence %d" % b)
+        ids, logits = llm.GenerateBatch(prompts, n, want_logits=True)
+        assert np.array_equal(llm.GenerateBatch(prompts, n), ids)
+        _batch_rows_against_cpu(cpu, prompts, n, ids, logits, "110M bf16 batch 16")
 
 
 def test_weight_storage_option_after_load_leaves_the_loaded_model_alone(llm, c4_model):
@@ -124,7 +142,7 @@ def test_weight_storage_option_after_load_leaves_the_loaded_model_alone(llm, c4_
     llm.SetOption(1, 1)
     assert np.array_equal(llm.GenerateIds(prompt, 24), ids)
     ref_ids, ref_logits = O.Llama(C4, blob).generate_greedy(prompt, 24, want_logits=True)
-    _ids_match(ids, ref_ids, ref_logits, "fp32 model after the option flip")
+    assert _ids_match(ids, ref_ids, ref_logits, "fp32 model after the option flip")
 
 
 # ---- decode attention, 32 heads x 128, cache 4096 --------------------------------------------
@@ -194,7 +212,10 @@ def test_attn_decode_7b_head_shape_with_rope_and_append_B32_L4096(dev, half):
         assert_close(y[b, h], _decode_row_ref(rq[b, h], kk, vv), tol, "row (%d,%d)" % (b, h))
     # the caches hold the appended rows
     kc = dev.get(hk, k.shape)
-    assert_close(kc[:, :, L - 1], rk, tol if half else 1e-6, "appended key rows")
+    # the rotation factors at position 4095 come from fp32 angles of up to 4095 radians (rope.cu:544-553): one unit in
+    # the last place of a frequency (powf of the C library against numpy's) moves such an angle by 2.4e-4, and the
+    # rotated key with it.  The bound is that, not fp32 round-off; the attention output above is held to the parity bar.
+    assert_close(kc[:, :, L - 1], rk, tol if half else 4e-4, "appended key rows")
     assert np.array_equal(kc[:, :, L - 2], rnd(k[:, :, L - 2]))
     assert np.array_equal(dev.get(hv, v.shape)[:, :, L - 1], rnd(vn))
 
@@ -227,11 +248,12 @@ def test_encdec_attention_config_bf16(dev):
 
     print("decoder self attention, per-sequence causal-and-padding mask, bf16", flush=True)
     ref = R.multihead_attention(tgt, tgt, tgt, *args, dec_mask, "full", dtype=np.float64)["y"]
-    for fuse in (True, False):
-        dec = MultiheadAttentionLayer(dev.cuda, H, C, Tt, True, fuse, half=True, fuse_batch_qk_mask=fuse)
-        dec.Setup(bt, bt, bt, W)
-        dec.Forward(bt, bt, bt, bdm, top)
-        assert_close(top.mutable_cpu_data, ref, BF16_RTOL, "decoder self attention bf16 (fused handle: %s)" % fuse)
+    # 16-bit storage goes through the fused handle only: the explicit chain's batched MatMul (gemm2) refuses
+    # half-size memory, as the reference's does (math.cu:1777-1778)
+    dec = MultiheadAttentionLayer(dev.cuda, H, C, Tt, True, True, half=True, fuse_batch_qk_mask=True)
+    dec.Setup(bt, bt, bt, W)
+    dec.Forward(bt, bt, bt, bdm, top)
+    assert_close(top.mutable_cpu_data, ref, BF16_RTOL, "decoder self attention bf16")
 
     print("cross attention T_q 128 / T_k 256, source key-padding mask, bf16", flush=True)
     cross = MultiheadAttentionLayer(dev.cuda, H, C, Ts, True, True, half=True)
