@@ -250,11 +250,15 @@ enum {
      *                 kernels (1 or 2; 0 = library's choice); option 5 = GENERATE_IDS /
      *                 GENERATE_BATCH draw from the handle's sampler (temperature, top-p,
      *                 seed of CREATE) instead of the argmax (0, default); option 6 = GENERATE_BATCH
-     *                 appends the logits of every step, batch x nSteps x vocabulary (0, default)
+     *                 appends the logits of every step, batch x nSteps x vocabulary (0, default);
+     *                 option 7 = the forced prompt positions run as one batched pass (1, default: MFMA
+     *                 GEMMs + fused causal attention over sequences x positions rows) or one decode
+     *                 step per position as in the reference's loop (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were
-     *                 replays of the captured graph / 0 if they were launched eagerly}
+     *                 replays of the captured graph / 0 if they were launched eagerly, ms of the batched
+     *                 prompt pass (0 if none ran), sequences x prompt positions it covered}
      *   PROFILE_STEP  f{hLlm, pos, reps[, batch]} -> per kernel class of one decode step
      *                 f{ms per step, launches per step, algorithmic bytes per step}, classes in
      *                 the order qkv mat-vec, rope+cache store, decode attention, wo, w1|w3,

@@ -64,6 +64,7 @@ public:
         m_query = (FnQuery)sym("DLL_QueryString");
         m_queryEx = (FnQueryEx)sym("DLL_QueryStringFloatEx");
         m_time = (FnTime)dlsym(m_lib, "MCH_TimeInvokeFloatEx2");
+        m_decodeNoAlloc = (FnDecodeNoAlloc)dlsym(m_lib, "MCH_AttnDecodeForwardNoAlloc");
     }
     ~Marshaller()
     {
@@ -123,6 +124,14 @@ public:
         return from_utf16(buf.data(), max);
     }
     // mean milliseconds of nReps back-to-back dispatches of one Ex2 call (measurement hook of this library)
+    // id 2001 through the entry point that allocates no device memory (fixed scratch inside the library)
+    void AttnDecodeNoAlloc(long kernel, const std::vector<float>& f, const std::vector<long long>& l)
+    {
+        if (!m_decodeNoAlloc) throw std::runtime_error("MCH_AttnDecodeForwardNoAlloc is not exported");
+        MCH_TCHAR err[kErrMax] = {0};
+        check(m_decodeNoAlloc((MCH_LONG)kernel, const_cast<float*>(f.data()), (MCH_LONG)f.size(),
+                              (MCH_LONGLONG*)const_cast<long long*>(l.data()), (MCH_LONG)l.size(), err, kErrMax), err);
+    }
     float TimeFloatEx2(long kernel, long fn, const std::vector<float>& f, const std::vector<long long>& l, int nWarmup, int nReps)
     {
         if (!m_time) throw std::runtime_error("MCH_TimeInvokeFloatEx2 is not exported");
@@ -142,6 +151,7 @@ private:
     typedef MCH_LONG (*FnInvokeEx2)(MCH_LONG, MCH_LONG, float*, MCH_LONG, MCH_LONGLONG*, MCH_LONG, float**, MCH_LONG*, MCH_TCHAR*, MCH_LONG);
     typedef MCH_LONG (*FnQuery)(MCH_LONG, MCH_LONG, MCH_LONG*, MCH_LONG, MCH_TCHAR**, MCH_TCHAR*, MCH_LONG);
     typedef MCH_LONG (*FnQueryEx)(MCH_LONG, MCH_LONG, MCH_LONG*, MCH_LONG, MCH_TCHAR*, MCH_LONG, MCH_TCHAR*, MCH_LONG);
+    typedef MCH_LONG (*FnDecodeNoAlloc)(MCH_LONG, float*, MCH_LONG, MCH_LONGLONG*, MCH_LONG, MCH_TCHAR*, MCH_LONG);
     typedef MCH_LONG (*FnTime)(MCH_LONG, MCH_LONG, float*, MCH_LONG, MCH_LONGLONG*, MCH_LONG, MCH_LONG, MCH_LONG, float*, MCH_TCHAR*, MCH_LONG);
 
     struct Out {   // caller-owned result buffer, as the C# marshaller passes one
@@ -180,6 +190,7 @@ private:
     FnQuery m_query = nullptr;
     FnQueryEx m_queryEx = nullptr;
     FnTime m_time = nullptr;
+    FnDecodeNoAlloc m_decodeNoAlloc = nullptr;
 };
 
 enum DIR { FWD = 0, BWD = 1 };
@@ -381,6 +392,11 @@ public:
                            long long nStrideBatch, long long nStrideHead, long long nStridePos, float fScale = 0.f)
     {
         ex2(MCH_FN_ATTN_DECODE_FWD, {fScale}, {nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead, nStridePos});
+    }
+    void AttnDecodeForwardNoAlloc(int nBatch, int nHeads, int nKvHeads, int nSize, int nLen, long hQ, long hKCache, long hVCache, long hY,
+                                  long long nStrideBatch, long long nStrideHead, long long nStridePos, float fScale = 0.f)
+    {
+        m_cuda.AttnDecodeNoAlloc(m_hKernel, {fScale}, {nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead, nStridePos});
     }
     void RmsNormForward(int nOuter, int nDim, long hX, long hWeight, long hY, float fEps = 1e-5f)
     {

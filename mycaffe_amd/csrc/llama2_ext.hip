@@ -471,6 +471,119 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
     }
 }
 
+// ---------------------------------------------------------------------------
+// Batched prompt prefill: the P forced prompt positions of every sequence go through the layers as one (B*P)-row
+// matrix (row m = b*P + p) instead of P single-token steps (the reference's loop, llm.cpp:208-231, forward() per
+// token).  The projections run on the MFMA GEMM, attention on the fused causal kernel; the kernels below are the
+// glue between their layouts.
+
+// x[m,:] = emb[prompt[b][p],:]
+template <typename T>
+__global__ void prefill_embed_kernel(const int* __restrict__ prompt, int promptStride, int P, const T* __restrict__ emb,
+                                     float* __restrict__ x, int dim)
+{
+    const int m = blockIdx.x, b = m / P, p = m - b * P;
+    const int tok = prompt[(size_t)b * promptStride + p];
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) x[(size_t)m * dim + i] = wld(emb, (size_t)tok * dim + i);
+}
+
+// One row [q | k | v] of raw projections per (b, p): rotate q and k at position p (adjacent pairs, the arithmetic of
+// the decode kernel), write q as (B,H,P,hs), k and v as (B,H,P,hs) with every key / value head repeated for the query
+// heads that share it, and append the rotated key and the value to the caches [b][pos][kvd].
+__global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float* __restrict__ qh, float* __restrict__ kh,
+                                            float* __restrict__ vh, float* __restrict__ kc, float* __restrict__ vc,
+                                            const float* __restrict__ fcos, const float* __restrict__ fsin, int B, int P, int H,
+                                            int kvH, int hs, int seqLen)
+{
+    const int dim = H * hs, kvd = kvH * hs, ldq = dim + 2 * kvd, half = hs / 2, kvMul = H / kvH;
+    const size_t pairsPerRow = (size_t)ldq / 2;
+    const size_t total = (size_t)B * P * pairsPerRow;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+        const size_t m = i / pairsPerRow;
+        const int col = (int)(i - m * pairsPerRow) * 2;
+        const int b = (int)(m / P), p = (int)(m - (size_t)b * P);
+        const float2 r = *(const float2*)(qkv + m * ldq + col);
+        if (col < dim + kvd) {
+            const int c = col < dim ? col : col - dim;
+            const int h = c / hs, d = c - h * hs;
+            const float cs = fcos[(size_t)p * half + d / 2], sn = fsin[(size_t)p * half + d / 2];
+            float2 o;
+            o.x = r.x * cs - r.y * sn;
+            o.y = r.x * sn + r.y * cs;
+            if (col < dim) {
+                *(float2*)(qh + (((size_t)b * H + h) * P + p) * hs + d) = o;
+            } else {
+                *(float2*)(kc + ((size_t)b * seqLen + p) * kvd + c) = o;
+                for (int g = 0; g < kvMul; g++) *(float2*)(kh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = o;
+            }
+        } else {
+            const int c = col - dim - kvd;
+            const int h = c / hs, d = c - h * hs;
+            *(float2*)(vc + ((size_t)b * seqLen + p) * kvd + c) = r;
+            for (int g = 0; g < kvMul; g++) *(float2*)(vh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = r;
+        }
+    }
+}
+
+// (B,H,P,hs) -> (B*P, H*hs)
+__global__ void prefill_merge_heads_kernel(const float* __restrict__ y, float* __restrict__ out, int B, int P, int H, int hs)
+{
+    const int q = hs / 4;
+    const size_t total = (size_t)B * P * H * q;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+        const int d4 = (int)(i % q);
+        size_t t = i / q;
+        const int h = (int)(t % H);
+        t /= H;
+        const int p = (int)(t % P), b = (int)(t / P);
+        *(float4*)(out + (((size_t)b * P + p) * H + h) * hs + d4 * 4) = *(const float4*)(y + (((size_t)b * H + h) * P + p) * hs + d4 * 4);
+    }
+}
+
+// hb[m, j] = silu(h2[m, j]) * h2[m, hid + j], the epilogue of the decode path's W1|W3 mat-vec
+__global__ void prefill_swiglu_kernel(const float* __restrict__ h2, float* __restrict__ hb, size_t rows, int hid)
+{
+    const size_t total = rows * hid;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+        const size_t m = i / hid;
+        const int j = (int)(i - m * hid);
+        const float a0 = h2[m * 2 * hid + j], a1 = h2[m * 2 * hid + hid + j];
+        hb[i] = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
+    }
+}
+
+// First-max argmax of every logits row (sample_argmax, llama2_sampler.cpp:25-36), one workgroup per row: the id
+// chosen after prompt position p of sequence b goes to out_ids[b][p]; the one after the last prefilled position is
+// also the token the first decode step starts from (next[b]).
+__global__ __launch_bounds__(256) void prefill_argmax_kernel(const float* __restrict__ logits, int V, int row0, int P,
+                                                             int promptStride, int* __restrict__ out_ids, int* __restrict__ next)
+{
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const int m = row0 + blockIdx.x, b = m / P, p = m - b * P;
+    const float* lg = logits + (size_t)blockIdx.x * V;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += 256) {
+        const float v = lg[i];
+        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; i++)
+            if (sv[i] > bv || (sv[i] == bv && si[i] < bi)) { bv = sv[i]; bi = si[i]; }
+        if (bi == 0x7fffffff) bi = 0;
+        out_ids[(size_t)b * promptStride + p] = bi;
+        if (p == P - 1) next[b] = bi;
+    }
+}
+
 __global__ void save_logits_kernel(const float* logits, float* all, const GenState* st, int V, int nSteps)
 {
     const int b = blockIdx.y;
@@ -586,6 +699,9 @@ public:
     bool stored_bf16 = false;    // storage of the weights that are on the device now: every launch dispatches on this
     bool use_graph = true;
     bool lastUsedGraph = false;  // whether the last generate replayed a captured graph (false: eager launches)
+    bool use_prefill = true;     // prompt positions as one batched pass (false: one decode step per position)
+    float lastPrefillMs = 0.f;   // HIP-event duration of the batched prompt pass of the last generate (0: none ran)
+    int lastPrefillRows = 0;     // sequences x prompt positions it covered
     int mvRows = 0;              // weight rows per wavefront in the mat-vec kernels (0: chosen per shape)
     void set_mv_rows(int r) { mvRows = r; graphB = -1; }   // the captured step is rebuilt at the next generation
     int shared_classifier = 0;
@@ -607,6 +723,9 @@ private:
     template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr, bool deviceArgmax = true);
     template <typename T> long advance_given(hipStream_t s, int B);
     long ensure_state(int B, int nSteps);
+    long ensure_prefill(size_t rows);
+    template <typename T> long prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits);
+    template <typename T> const float* as_f32(hipStream_t s, const void* w, size_t n, long* err);
     hipError_t embed_first(hipStream_t s, int B);
 
     hipStream_t stream = nullptr;
@@ -634,7 +753,13 @@ private:
     int graphB = 0;
     bool graphArgmax = true;                     // whether the captured step ends with the device argmax
     int* dgiven = nullptr;                       // ids chosen by the host sampler (one per sequence)
+    int hostNPrompt = 0;                         // prompt length of the running generation
     float* hLogits = nullptr; int* hGiven = nullptr; size_t hLogitsCount = 0;   // pinned staging of the sampled path
+    // batched prompt pass: activations of rows = sequences x prompt positions, sized for pfRows
+    size_t pfRows = 0, pfLogitRows = 0;
+    std::vector<void*> prefillAllocs;
+    float *pfX = nullptr, *pfXn = nullptr, *pfQkv = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfY = nullptr,
+          *pfH2 = nullptr, *pfHb = nullptr, *pfLogits = nullptr, *pfW = nullptr;
 };
 
 void Engine::release()
@@ -645,6 +770,9 @@ void Engine::release()
     if (hGiven) { (void)hipHostFree(hGiven); hGiven = nullptr; }
     for (void* p : stateAllocs) (void)hipFree(p);
     stateAllocs.clear();
+    for (void* p : prefillAllocs) (void)hipFree(p);
+    prefillAllocs.clear();
+    pfRows = 0;
     for (void* p : allocs) (void)hipFree(p);
     allocs.clear();
     layers.clear();
@@ -740,12 +868,13 @@ long Engine::load(const char* path)
     shared_classifier = shared;
     if (cfg.seq_len > 20480) cfg.seq_len = 20480;   // the reference clamps the context the same way (llama2_cpu.cpp:145)
     if (cfg.dim <= 0 || cfg.n_heads <= 0 || cfg.n_kv_heads <= 0 || cfg.n_layers <= 0 || cfg.vocab_size <= 0 || cfg.seq_len <= 0 ||
-        cfg.hidden_dim <= 0 || cfg.dim % cfg.n_heads || cfg.n_heads % cfg.n_kv_heads || (cfg.dim / cfg.n_heads) % 2 ||
+        cfg.hidden_dim <= 0 || cfg.dim % cfg.n_heads || cfg.n_heads % cfg.n_kv_heads || (cfg.dim / cfg.n_heads) % 4 ||
+        cfg.dim / cfg.n_heads > 256 ||
         cfg.dim % 4 || cfg.hidden_dim % 4) {
         fclose(f);
         char msg[256];
         snprintf(msg, sizeof(msg), "Unsupported model shape: dim %d, hidden %d, layers %d, heads %d, kv heads %d, vocabulary %d, "
-                 "context %d (dim and hidden must be multiples of 4, dim a multiple of heads, heads of kv heads, head size even).",
+                 "context %d (dim and hidden must be multiples of 4, dim a multiple of heads, heads of kv heads, head size a multiple of 4 up to 256).",
                  cfg.dim, cfg.hidden_dim, cfg.n_layers, cfg.n_heads, cfg.n_kv_heads, cfg.vocab_size, cfg.seq_len);
         lastError = msg;
         return MCH_ERROR_LLM_LOAD_MODEL;
@@ -831,6 +960,109 @@ long Engine::ensure_state(int B, int nSteps)
     HIPCHK(hipMemset(dcount, 0, ((size_t)B * cfg.n_heads + 1) * 4));
     stateB = B;
     stateSteps = cfg.seq_len;
+    return 0;
+}
+
+long Engine::ensure_prefill(size_t rows)
+{
+    if (rows <= pfRows) return 0;
+    HIPCHK(hipStreamSynchronize(stream));
+    for (void* p : prefillAllocs) (void)hipFree(p);
+    prefillAllocs.clear();
+    pfRows = 0;
+    const size_t dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
+    auto pa = [&](size_t floats) -> float* {
+        void* p = nullptr;
+        if (hipMalloc(&p, floats ? floats * 4 : 4) != hipSuccess) return nullptr;
+        prefillAllocs.push_back(p);
+        return (float*)p;
+    };
+    // the classifier runs over at most 512 MB of logits at a time
+    pfLogitRows = std::max<size_t>(1, std::min(rows, ((size_t)128 << 20) / V));
+    pfX = pa(rows * dim); pfXn = pa(rows * dim); pfQkv = pa(rows * (dim + 2 * kvd));
+    pfQ = pa(rows * dim); pfK = pa(rows * dim); pfV = pa(rows * dim); pfY = pa(rows * dim);
+    pfH2 = pa(rows * 2 * hid); pfHb = pa(rows * hid); pfLogits = pa(pfLogitRows * V);
+    // weights stored as bf16 are widened to fp32 one matrix at a time: room for the largest one
+    pfW = stored_bf16 ? pa(std::max({(dim + 2 * kvd) * dim, 2 * hid * dim, V * dim})) : pfX;
+    if (!pfX || !pfXn || !pfQkv || !pfQ || !pfK || !pfV || !pfY || !pfH2 || !pfHb || !pfLogits || !pfW) return MCH_ERROR_MEMORY_OUT;
+    pfRows = rows;
+    return 0;
+}
+
+// the matrix as fp32: itself, or (16-bit storage) widened into the scratch matrix, which gives the GEMM exactly the
+// values the decode path's mat-vec kernels widen in registers
+template <typename T> const float* Engine::as_f32(hipStream_t s, const void* w, size_t n, long* err)
+{
+    if (sizeof(T) == 4) return (const float*)w;
+    hipError_t e = k_convert(s, BF16, w, F32, pfW, n);
+    if (e != hipSuccess) *err = (long)e;
+    return pfW;
+}
+
+// Positions 0 .. P-1 of all B sequences in one pass.  Leaves what P single-token steps leave: the caches of every
+// layer filled up to P - 1, the id chosen after every position in dout, the id after the last one in dnext, and the
+// generation state at position P.
+template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits)
+{
+    const int dim = cfg.dim, hid = cfg.hidden_dim, H = cfg.n_heads, kvH = cfg.n_kv_heads, hs = dim / H, kvd = hs * kvH, V = cfg.vocab_size;
+    const int ldq = dim + 2 * kvd;
+    const size_t M = (size_t)B * P;
+    long e = ensure_prefill(M);
+    if (e) return e;
+    const float scale = 1.0f / sqrtf((float)hs);
+    auto grid_for = [](size_t items) { return (int)std::min<size_t>((items + 255) / 256, 8192); };
+    hipLaunchKernelGGL(prefill_embed_kernel<T>, (int)M, 256, 0, s, dprompt, cfg.seq_len, P, (const T*)emb, pfX, dim);
+    HIPCHK(hipGetLastError());
+    for (int l = 0; l < cfg.n_layers; l++) {
+        const LayerW<void>& w = layers[l];
+        float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
+        float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
+        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_att, pfXn, 1e-5f));
+        const float* wqkv = as_f32<T>(s, w.wqkv, (size_t)ldq * dim, &e);
+        if (e) return e;
+        HIPCHK(k_gemm(s, F32, false, true, (int)M, ldq, dim, 1.f, pfXn, wqkv, 0.f, pfQkv));
+        hipLaunchKernelGGL(prefill_rope_scatter_kernel, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, kcl, vcl, fcos, fsin, B, P,
+                           H, kvH, hs, cfg.seq_len);
+        HIPCHK(hipGetLastError());
+        HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfY, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL));
+        hipLaunchKernelGGL(prefill_merge_heads_kernel, grid_for(M * dim / 4), 256, 0, s, pfY, pfXn, B, P, H, hs);
+        HIPCHK(hipGetLastError());
+        const float* wo = as_f32<T>(s, w.wo, (size_t)dim * dim, &e);
+        if (e) return e;
+        HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, dim, 1.f, pfXn, wo, 1.f, pfX));          // x += Wo att
+        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_ffn, pfXn, 1e-5f));
+        const float* w13 = as_f32<T>(s, w.w13, (size_t)2 * hid * dim, &e);
+        if (e) return e;
+        HIPCHK(k_gemm(s, F32, false, true, (int)M, 2 * hid, dim, 1.f, pfXn, w13, 0.f, pfH2));
+        hipLaunchKernelGGL(prefill_swiglu_kernel, grid_for(M * hid), 256, 0, s, pfH2, pfHb, M, hid);
+        HIPCHK(hipGetLastError());
+        const float* w2 = as_f32<T>(s, w.w2, (size_t)dim * hid, &e);
+        if (e) return e;
+        HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, hid, 1.f, pfHb, w2, 1.f, pfX));          // x += W2 hb
+    }
+    HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
+    const float* wc = as_f32<T>(s, wcls, (size_t)V * dim, &e);
+    if (e) return e;
+    for (size_t r0 = 0; r0 < M; r0 += pfLogitRows) {
+        const int rows = (int)std::min(pfLogitRows, M - r0);
+        HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
+        hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
+        HIPCHK(hipGetLastError());
+        if (allLogits) {
+            // rows of one sequence are contiguous on both sides: [b][nSteps][V] <- [b*P + p][V]
+            for (size_t m = r0; m < r0 + rows;) {
+                const size_t b = m / P, p = m - b * P;
+                const size_t n = std::min<size_t>(P - p, r0 + rows - m);
+                HIPCHK(hipMemcpyAsync(allLogits + ((size_t)b * nSteps + p) * V, pfLogits + (m - r0) * V, n * V * sizeof(float),
+                                      hipMemcpyDeviceToDevice, s));
+                m += n;
+            }
+        }
+    }
+    GenState st = {P, 0, P + 1, 0};
+    st.n_prompt = hostNPrompt;
+    HIPCHK(hipMemcpyAsync(dstate, &st, sizeof(st), hipMemcpyHostToDevice, s));
+    HIPCHK(hipStreamSynchronize(s));   // `st` lives on this stack frame
     return 0;
 }
 
@@ -1028,6 +1260,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         if (prompts[i] < 0 || prompts[i] >= cfg.vocab_size) return MCH_ERROR_PARAM_OUT_OF_RANGE;
     long e = ensure_state(B, nSteps);
     if (e) return e;
+    hostNPrompt = nPrompt;
     hipStream_t s = stream;
     std::vector<int> hp((size_t)B * cfg.seq_len, 0);
     for (int b = 0; b < B; b++) memcpy(&hp[(size_t)b * cfg.seq_len], prompts + (size_t)b * nPrompt, nPrompt * sizeof(int));
@@ -1038,12 +1271,12 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     // owned here so that every early return below releases them
     struct Scratch {
         float* allLogits = nullptr;
-        hipEvent_t evA = nullptr, evB = nullptr;
+        hipEvent_t evA = nullptr, evB = nullptr, evP0 = nullptr, evP1 = nullptr;
         ~Scratch()
         {
             if (allLogits) (void)hipFree(allLogits);
-            if (evA) (void)hipEventDestroy(evA);
-            if (evB) (void)hipEventDestroy(evB);
+            for (hipEvent_t ev : {evA, evB, evP0, evP1})
+                if (ev) (void)hipEventDestroy(ev);
         }
     } sc;
     if (wantLogits) {
@@ -1088,10 +1321,42 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         graphArgmax = !hostSample;
     }
     lastUsedGraph = graph;
+    // the forced prompt positions in one batched pass (ids chosen on the host need every position's logits in turn,
+    // so a sampled generation keeps the one-step-per-position loop)
+    const int nPre = std::min(nPrompt, nSteps);
+    const bool batched = use_prefill && !hostSample && nPre >= 2;
+    const int start = batched ? nPre : 0;
+    lastPrefillMs = 0.f;
+    lastPrefillRows = 0;
+    bool timing = false;
+    if (t0 < start) { (void)hipEventRecord(evA, s); timing = true; }
+    if (batched) {
+        HIPCHK(hipEventCreate(&sc.evP0));
+        HIPCHK(hipEventCreate(&sc.evP1));
+        HIPCHK(hipEventRecord(sc.evP0, s));
+        e = stored_bf16 ? prefill<bf16_t>(s, B, nPre, nSteps, allLogits) : prefill<float>(s, B, nPre, nSteps, allLogits);
+        if (e) return e;
+        HIPCHK(hipEventRecord(sc.evP1, s));
+        HIPCHK(hipEventSynchronize(sc.evP1));
+        (void)hipEventElapsedTime(&lastPrefillMs, sc.evP0, sc.evP1);
+        lastPrefillRows = B * nPre;
+    }
     HIPCHK(embed_first(s, B));
-    int done = 0;
-    for (int i = 0; i < nSteps && !e; i++) {
-        if (i == t0) (void)hipEventRecord(evA, s);
+    int done = start, reported = 0;
+    // hands the ids of sequence 0 chosen at positions [reported, done) to the caller, who may stop the generation
+    auto report = [&]() -> int {
+        std::vector<int> part((size_t)done);
+        hipError_t hc = hipStreamSynchronize(s);
+        if (hc == hipSuccess) hc = hipMemcpy(part.data(), dout, part.size() * 4, hipMemcpyDeviceToHost);
+        if (hc != hipSuccess) { e = (long)hc; return -1; }
+        const bool go = onChunk(part.data(), reported, done);
+        reported = done;
+        return go ? 1 : 0;
+    };
+    bool stop = false;
+    if (onChunk && chunk > 0 && done > 0) stop = report() != 1;
+    for (int i = start; i < nSteps && !e && !stop; i++) {
+        if (i == t0 && !timing) { (void)hipEventRecord(evA, s); timing = true; }
         if (graph) {
             hipError_t he = hipGraphLaunch(graphExec, s);
             if (he != hipSuccess) e = (long)he;
@@ -1108,22 +1373,14 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         }
         done++;
         if (cancel && (i & 15) == 15 && cancel->load()) break;
-        if (onChunk && chunk > 0 && (done % chunk == 0 || done == nSteps)) {
-            // hand the ids of sequence 0 chosen so far to the caller, who may stop the generation (end of text)
-            const int from = done - ((done % chunk == 0) ? chunk : done % chunk);
-            std::vector<int> part((size_t)done);
-            hipError_t hc = hipStreamSynchronize(s);
-            if (hc == hipSuccess) hc = hipMemcpy(part.data(), dout, part.size() * 4, hipMemcpyDeviceToHost);
-            if (hc != hipSuccess) { e = (long)hc; break; }
-            if (!onChunk(part.data(), from, done)) break;
-        }
+        if (onChunk && chunk > 0 && (done - reported >= chunk || done == nSteps)) stop = report() != 1;
     }
     (void)hipEventRecord(evB, s);
     hipError_t he = hipStreamSynchronize(s);
     if (!e && he != hipSuccess) e = (long)he;
     lastTimedMs = 0.f;
     lastTimedSteps = 0;
-    if (!e && done > t0 && t0 >= 0) {
+    if (!e && done > t0 && t0 >= 0 && timing) {
         (void)hipEventElapsedTime(&lastTimedMs, evA, evB);
         lastTimedSteps = done - t0;
     }
@@ -1151,6 +1408,7 @@ struct Llm {
     BpeTokenizer tokenizer;
     HostSampler sampler;         // built at LOAD from the CREATE arguments, state kept across generations (llm.cpp:140)
     bool sampleIds = false;      // GENERATE_IDS / GENERATE_BATCH draw from the sampler instead of the device argmax
+    bool batchLogits = false;    // GENERATE_BATCH also returns the logits of every step (eager launches)
     std::atomic<bool> cancel{false};
     std::atomic<bool> busy{false};
     std::atomic<bool> loaded{false};
@@ -1334,6 +1592,8 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 3) m->engine.use_graph = pIn[2] != 0.f;
         else if (opt == 4) m->engine.set_mv_rows(pIn[2] == 1.f ? 1 : (pIn[2] == 2.f ? 2 : 0));
         else if (opt == 5) m->sampleIds = pIn[2] != 0.f;
+        else if (opt == 6) m->batchLogits = pIn[2] != 0.f;
+        else if (opt == 7) m->engine.use_prefill = pIn[2] != 0.f;
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }
@@ -1341,7 +1601,8 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         if (lIn < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
         if (!m) return MCH_ERROR_PARAM;
-        return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps, m->engine.lastUsedGraph ? 1.f : 0.f}, ppOut, plOut);
+        return (MCH_LONG)give({m->engine.lastTimedMs, (float)m->engine.lastTimedSteps, m->engine.lastUsedGraph ? 1.f : 0.f,
+                                m->engine.lastPrefillMs, (float)m->engine.lastPrefillRows}, ppOut, plOut);
     }
     case MCH_LLM_PROFILE_STEP: {
         if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
@@ -1367,6 +1628,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
     case MCH_LLM_GENERATE_BATCH: {
         // GENERATE_IDS   f{hLlm, nSteps, wantLogits, ids...}
         // GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of sequence 0 .., sequence 1 ..}
+        //                -> f{batch x nSteps ids [, batch x nSteps x vocabulary logits with option 6]}
         const bool batch = fn == MCH_LLM_GENERATE_BATCH;
         const int head = batch ? 4 : 3;
         if (lIn < head + 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
@@ -1376,7 +1638,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         const int nSteps = (int)pIn[1];
         const int B = batch ? (int)pIn[2] : 1;
         const int nPrompt = batch ? (int)pIn[3] : lIn - head;
-        const bool wantLogits = !batch && pIn[2] != 0.f;
+        const bool wantLogits = batch ? m->batchLogits : pIn[2] != 0.f;
         if (B < 1 || nPrompt < 1 || (long long)B * nPrompt != lIn - head) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         std::vector<int> prompts((size_t)B * nPrompt);
         for (size_t i = 0; i < prompts.size(); i++) prompts[i] = (int)pIn[head + i];

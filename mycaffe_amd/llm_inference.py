@@ -128,6 +128,12 @@ class LlmInference:
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
         return bool(rg[2] != 0)
 
+    def LastPrefill(self):
+        """(milliseconds, rows) of the batched prompt pass of the last generation: HIP-event time on the engine's stream
+        and sequences x prompt positions covered; (0, 0) when the prompt went one decode step per position."""
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.QUERY_TIMING, self.m_rgLlm)
+        return float(rg[3]), int(rg[4])
+
     def ProfileStep(self, pos, reps=8, batch=1):
         """Per-kernel-class timing of eager decode steps at ``pos`` (HIP event pairs around
         every launch): {class: (ms per step, launches per step, algorithmic bytes per step)}, plus

@@ -91,6 +91,13 @@ def test_llama110m_batch1_fp32_logits_and_ids(llm, c4_model):
     ids_graph = llm.GenerateIds(prompt, n)                        # one captured graph per step
     assert llm.LastRunUsedGraph()
     assert np.array_equal(ids_graph, ids)
+    # the 128 prompt positions went through the batched pass; one decode step per position gives the same
+    assert llm.LastPrefill()[1] == 128
+    llm.SetOption(7, 0)
+    ids_loop, logits_loop = llm.GenerateIds(prompt, n, want_logits=True)
+    assert llm.LastPrefill() == (0.0, 0)
+    assert_close(logits_loop, ref_logits, FP32_RTOL, "110M logits, one step per prompt position")
+    assert np.array_equal(ids_loop, ids)
 
 
 def test_llama110m_batch16_fp32_every_row_an_independent_cpu_run(llm, c4_model):

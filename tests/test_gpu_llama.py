@@ -377,3 +377,63 @@ def test_llama_decode_through_the_layer_call_sequences_matches_the_checker(dev):
         exp = ref.forward(tok, pos)
         assert_close(logits.mutable_cpu_data.reshape(-1), exp, FP32_RTOL, "logits at position %d" % pos)
         assert int(np.argmax(logits.mutable_cpu_data)) == int(np.argmax(exp))
+
+
+@pytest.mark.parametrize("name,cfg,std,nP,n", [("tiny", TINY, 0.2, 9, 40), ("gqa", dict(TINY, n_kv_heads=2), 0.2, 17, 48),
+                                               ("hs64", dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256), 0.08, 100, 160),
+                                               ("c1", C1, 0.02, 8, 64)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_batched_prompt_pass_equals_one_step_per_position(llm, tmp_path, name, cfg, std, nP, n, bf16):
+    """The prompt as one batched pass (MFMA GEMMs, fused causal attention, caches written in bulk) against the
+    reference's loop of one forward per prompt token (llm.cpp:208-231): logits of every position against the CPU
+    checker, the same ids, and the same continuation out of the caches it filled."""
+    blob, views = O.random_weights(cfg, seed=21, shared_classifier=False, std=std)
+    rng = np.random.default_rng(4)
+    for k in ("rms_att", "rms_ffn", "rms_final"):
+        # norm weights stay fp32 on the device whatever the matrix storage: keep them exact in bf16 so that the
+        # checker on bf16-rounded weights sees the same values
+        views[k][...] = bf16_round(1 + 0.2 * rng.standard_normal(views[k].shape).astype(np.float32))
+    path = str(tmp_path / (name + ".bin"))
+    O.write_checkpoint_v1(path, cfg, blob, False)
+    if bf16:
+        llm.SetOption(1, 1)
+    llm.Load(path)
+    prompt = rng.integers(3, cfg["vocab_size"], nP)
+    ref_ids, ref_logits = O.Llama(cfg, bf16_round(blob) if bf16 else blob).generate_greedy(prompt, n, want_logits=True)
+    llm.SetOption(7, 0)
+    ids_loop, logits_loop = llm.GenerateIds(prompt, n, want_logits=True)
+    assert llm.LastPrefill() == (0.0, 0)
+    llm.SetOption(7, 1)
+    ids, logits = llm.GenerateIds(prompt, n, want_logits=True)
+    ms, rows = llm.LastPrefill()
+    assert rows == nP and ms > 0
+    assert_close(logits, ref_logits, FP32_RTOL, "logits with the batched prompt pass")
+    assert_close(logits, logits_loop, FP32_RTOL, "batched prompt pass vs one step per position")
+    assert np.array_equal(ids, np.argmax(logits, axis=-1))
+    _check_ids(ids, ref_ids, ref_logits, name)
+    assert np.array_equal(ids, ids_loop)
+    assert np.array_equal(llm.GenerateIds(prompt, n), ids)        # graph replays after the batched pass
+    # a generation that ends inside the prompt
+    short = llm.GenerateIds(prompt, nP - 1)
+    assert np.array_equal(short, ids[:nP - 1])
+
+
+def test_batched_prompt_pass_batch_of_sequences(llm, tmp_path):
+    cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=4, vocab_size=512, seq_len=128)
+    blob, _ = O.random_weights(cfg, seed=5, shared_classifier=False, std=0.08)
+    path = str(tmp_path / "b.bin")
+    O.write_checkpoint_v1(path, cfg, blob, False)
+    llm.Load(path)
+    rng = np.random.default_rng(6)
+    B, nP, n = 5, 33, 70
+    prompts = rng.integers(3, cfg["vocab_size"], (B, nP))
+    ids, logits = llm.GenerateBatch(prompts, n, want_logits=True)
+    assert llm.LastPrefill()[1] == B * nP
+    llm.SetOption(7, 0)
+    ids_loop = llm.GenerateBatch(prompts, n)
+    assert np.array_equal(ids, ids_loop)
+    cpu = O.Llama(cfg, blob)
+    for b in range(B):
+        ref_ids, ref_logits = cpu.generate_greedy(prompts[b], n, want_logits=True)
+        assert_close(logits[b], ref_logits, FP32_RTOL, "sequence %d" % b)
+        assert np.array_equal(ids[b], ref_ids)
