@@ -71,6 +71,9 @@ def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
     per_gen = C4["seq_len"] - N_PROMPT - warmup
     left, ms_total, wall, gen = steps, 0.0, 0.0, 0
     first = None
+    # one short untimed generation first: buffers allocated, kernels loaded, the step graph captured
+    wp = np.random.default_rng(seed + 999).integers(3, C4["vocab_size"], (batch, N_PROMPT))
+    inf.GenerateIds(wp[0], N_PROMPT + 4) if batch == 1 else inf.GenerateBatch(wp, N_PROMPT + 4)
     while left > 0:
         k = min(left, per_gen)
         rng = np.random.default_rng(seed + gen)
@@ -89,11 +92,26 @@ def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
         ms_total += ms
         left -= k
         if first is None:
-            first = (prompt, ids)
+            first = (prompt, ids, inf.LastPrefill(), inf.LastRunUsedGraph())
         gen += 1
     res = {"ms_per_step": ms_total / steps, "tokens_per_s": batch * steps / (ms_total / 1e3), "wall_s_whole_generation": wall,
-           "prompt": first[0], "ids": first[1], "generations": gen}
+           "prompt": first[0], "ids": first[1], "generations": gen, "prefill_ms": first[2][0], "prefill_rows": first[2][1],
+           "graph": first[3]}
     return inf, res
+
+
+def prefill_summary(r, batch, es):
+    """The batched prompt pass of one generation: HIP-event time, prompt tokens per second, and the fraction of the fp32
+    MFMA peak its arithmetic reaches (the pass computes in fp32 whatever the weight storage; flops = 2 x matrix
+    parameters x rows, the classifier included, plus the causal half of the attention products)."""
+    if not r["prefill_rows"]:
+        return None
+    rows, P = r["prefill_rows"], r["prefill_rows"] // batch
+    dim, L, H = C4["dim"], C4["n_layers"], C4["n_heads"]
+    flops = 2.0 * (weight_bytes(C4, 1)) * rows + L * 2.0 * batch * H * P * P * (dim // H)
+    tf = flops / (r["prefill_ms"] / 1e3) / 1e12
+    return {"ms": round(r["prefill_ms"], 4), "prompt_tokens": rows, "prompt_tokens_per_s": round(rows / (r["prefill_ms"] / 1e3), 1),
+            "TFLOPs": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_PEAK_TFLOPS["f32"], 4)}
 
 
 def recorded_traffic(key):
@@ -128,8 +146,9 @@ def step_roofline(inf, head, steps, warmup):
     detail = {k: {"us_per_launch": round(v[0] / v[1] * 1e3, 3), "launches_per_step": v[1],
                   "algorithmic_MB_per_launch": round(v[2] / v[1] / 1e6, 3) if v[2] > 0 else None}
               for k, v in prof.items() if v[1] > 0}
-    return {"kernel": "decode step = one replay of the captured graph (49 matvec_kernel, 12 attn_decode_fused_kernel, "
-                      "1 sample_advance_kernel)",
+    how = "one replay of the captured graph" if head.get("graph") else "62 eager launches (no graph: asked for, or capture failed)"
+    return {"kernel": "decode step = %s (49 matvec_kernel, 12 attn_decode_fused_kernel, 1 sample_advance_kernel)" % how,
+            "graph_replay": bool(head.get("graph")),
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic("decode_step"),
             "traffic_note": "counter runs cover a step at position 512 (475.9 MB algorithmic there)",
@@ -263,21 +282,30 @@ def bench_decode_attention(cuda, reps, warm=5, cases=None):
                         cuda.copy(c, dst, dst, 0, have)
                         have += c
                 q = cuda.AllocMemory(rng.standard_normal(B * H * hs).astype(np.float32), bHalfSize=half)
+                kn = cuda.AllocMemory(rng.standard_normal(B * H * hs).astype(np.float32), bHalfSize=half)
+                vn = cuda.AllocMemory(rng.standard_normal(B * H * hs).astype(np.float32), bHalfSize=half)
                 y = cuda.AllocMemory(B * H * hs, bHalfSize=half)
-                rgl = [B, H, H, hs, L, q, kc, vc, y, H * L * hs, L * hs, hs]
+                hr = cuda.CreateRope(0, 0, B * H * hs, B, L, H, hs, 10000.0)
+                # the whole step the configuration names: rotate q and the newest key at position L - 1 (theta 10000),
+                # append key and value to the caches, attend over the L cached positions.  Repeats rotate q again in
+                # place: its values change, its magnitude and the timing do not.
+                rgl = [B, H, H, hs, L, q, kc, vc, y, H * L * hs, L * hs, hs, hr, kn, vn]
                 ms = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl, warm, reps)
+                ms_attn = cuda.TimeFunction(CUDAFN.ATTN_DECODE_FWD, [0.0], rgl[:12], warm, reps)
                 nbytes = 2.0 * n * es
                 gbs = nbytes / (ms / 1e3) / 1e9
                 # back-to-back dispatches re-read the same cache: below the 256 MB of last-level cache the figure is
                 # not an HBM rate (and the smallest cases are launch bound)
                 out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                                                    "us_attention_kernel_alone": round(ms_attn * 1e3, 2),
                                                     "fits_last_level_cache": bool(nbytes <= 256e6)}
-                for h in (kc, vc, src, q, y):
+                cuda.FreeRope(hr)
+                for h in (kc, vc, src, q, kn, vn, y):
                     cuda.FreeMemory(h)
     if "bf16_B32_L4096" not in out:
         return out
     best = out["bf16_B32_L4096"]
-    out["roofline"] = {"kernel": "attn_decode_kernel (bf16, batch 32, L 4096, 32 x 128)", "bound": "hbm", "achieved": best["GBps"],
+    out["roofline"] = {"kernel": "rope_append_kernel + attn_decode_kernel (bf16, batch 32, L 4096, 32 x 128)", "bound": "hbm", "achieved": best["GBps"],
                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_hbm"],
                        "traffic": recorded_traffic("attn_decode_bf16_B32_L4096")}
     return out
@@ -505,29 +533,44 @@ def bench_copy(cuda, reps, warm=2):
             "GBps": round(2 * n * 4 / (ms / 1e3) / 1e9, 1)}
 
 
-def counter_pass(cuda, path):
-    """A short run for hardware-counter collection (rocprofv3 --pmc serialises and slows every dispatch):
-    two eager decode steps at position 512, a few dispatches each of the fused prefill attention and its backward pass
-    (bf16, fp32), the decode attention at batch 32 / L 4096 (bf16, fp32), the layer GEMMs and the 256 MiB copy that
-    calibrates the counters."""
-    from mycaffe_amd.llm_inference import LlmInference
-    inf = LlmInference(cuda)
-    inf.Initialize(fTemperature=0.0)
-    inf.SetOption(3, 0)
-    inf.Load(path)
-    log("counter pass: decode steps")
-    inf.ProfileStep(512, 2)
-    inf.CleanUp()
-    log("counter pass: copy")
-    out = {"copy_256MiB": bench_copy(cuda, 2, 0)}
-    log("counter pass: prefill attention")
-    out["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 2, 0)
-    log("counter pass: decode attention")
-    out["decode_attention_H32x128"] = bench_decode_attention(cuda, 2, 0, cases=(("bf16", 32, 4096), ("f32", 32, 4096)))
-    log("counter pass: attention backward")
-    out["attention_backward_B8_T1024_H12x64"] = bench_attention_backward(cuda, 2, 0)
-    log("counter pass: gemm")
-    out["gemm_M8192"] = bench_gemm(cuda, 2)
+COUNTER_SECTIONS = ("decode_step", "copy", "prefill", "prefill_7b", "decode_attn", "backward", "gemm", "matmul_chain")
+
+
+def counter_pass(cuda, path, sections):
+    """A short run for hardware-counter collection (rocprofv3 --pmc serialises and slows every dispatch): a few
+    dispatches of the kernels of the named sections only, so that one counter run stays within seconds.
+    decode_step: two eager decode steps at position 512; copy: the 256 MiB streaming kernel that calibrates the traffic
+    counters; prefill / prefill_7b: fused causal attention at B=8 T=1024 12x64 (bf16, fp32) / B=4 T=4096 32x128 (bf16);
+    decode_attn: decode attention at batch 32, L 4096 (bf16, fp32); backward: attention backward; gemm: the layer
+    GEMMs; matmul_chain: the two batched MatMul calls of the explicit attention chain."""
+    out = {}
+    for sec in sections:
+        log("counter pass:", sec)
+        if sec == "decode_step":
+            from mycaffe_amd.llm_inference import LlmInference
+            inf = LlmInference(cuda)
+            inf.Initialize(fTemperature=0.0)
+            inf.SetOption(3, 0)
+            inf.Load(path)
+            inf.ProfileStep(512, 2)
+            inf.CleanUp()
+            out[sec] = "2 eager steps at position 512"
+        elif sec == "copy":
+            out[sec] = bench_copy(cuda, 2, 0)
+        elif sec == "prefill":
+            out[sec] = bench_prefill_attention(cuda, 2, 0)
+        elif sec == "prefill_7b":
+            out[sec] = bench_prefill_attention(cuda, 2, 0, (4, 32, 4096, 128), (("bf16", True),))
+        elif sec == "decode_attn":
+            out[sec] = bench_decode_attention(cuda, 2, 0, cases=(("bf16", 32, 4096), ("f32", 32, 4096)))
+        elif sec == "backward":
+            out[sec] = bench_attention_backward(cuda, 2, 0)
+        elif sec == "gemm":
+            out[sec] = bench_gemm(cuda, 2)
+        elif sec == "matmul_chain":
+            out[sec] = bench_matmul_chain(cuda, 2, 0)
+        else:
+            raise SystemExit("unknown counter-pass section %r (known: %s)" % (sec, ", ".join(COUNTER_SECTIONS)))
     return out
 
 
@@ -540,8 +583,9 @@ def main():
     ap.add_argument("--no-also", action="store_true", help="only the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="launch every decode kernel eagerly instead of replaying a HIP graph "
                     "(kernel tracing tools see the individual kernels this way)")
-    ap.add_argument("--counter-pass", action="store_true", help="few dispatches of every kernel, for rocprofv3 --pmc runs; "
-                    "prints what ran instead of the benchmark line")
+    ap.add_argument("--counter-pass", nargs="?", const="all", default=None, metavar="SECTIONS",
+                    help="few dispatches of the kernels of the named sections (comma list of %s; default all), for rocprofv3 "
+                         "--pmc runs; prints what ran instead of the benchmark line" % ", ".join(COUNTER_SECTIONS))
     ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,csa_layer,matmul_chain,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
@@ -563,7 +607,8 @@ def main():
     log("checkpoint ready in %.1f s" % (time.perf_counter() - t0))
 
     if args.counter_pass:
-        print(json.dumps({"counter_pass": counter_pass(cuda, path)}), flush=True)
+        secs = COUNTER_SECTIONS if args.counter_pass == "all" else tuple(x for x in args.counter_pass.split(",") if x)
+        print(json.dumps({"counter_pass": counter_pass(cuda, path, secs)}), flush=True)
         cuda.Dispose()
         return
     inf, head = run_decode(cuda, path, False, 1, args.steps, args.warmup, graph=not args.no_graph)
@@ -575,11 +620,15 @@ def main():
     only = set(x for x in args.only.split(",") if x)
     want = lambda name: not args.no_also and (not only or name in only)
     also["decode_fp32_b1_wall_s_incl_id_transfers"] = round(head["wall_s_whole_generation"], 4)
+    # the 128-token prompt of the same generation: one batched pass before the timed decode steps
+    also["prefill_128_tokens_fp32_b1"] = prefill_summary(head, 1, 4)
+    log("prompt pass, batch 1:", json.dumps(also["prefill_128_tokens_fp32_b1"]))
     if want("decode"):
         for tag, bf16, batch in (("bf16_weights_b1", True, 1), ("fp32_b16", False, 16), ("bf16_weights_b16", True, 16)):
             i2, r = run_decode(cuda, path, bf16, batch, args.steps, args.warmup, graph=not args.no_graph)
-            also["decode_" + tag] = {"tokens_per_s": round(r["tokens_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4)}
-            log("decode %s: %.1f tokens/s" % (tag, r["tokens_per_s"]))
+            also["decode_" + tag] = {"tokens_per_s": round(r["tokens_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4),
+                                     "graph_replay": bool(r["graph"]), "prefill_128_tokens": prefill_summary(r, batch, 2 if bf16 else 4)}
+            log("decode %s: %.1f tokens/s, prompt pass %s" % (tag, r["tokens_per_s"], json.dumps(also["decode_" + tag]["prefill_128_tokens"])))
             i2.CleanUp()
     if want("prefill"):
         also["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 50)
@@ -615,6 +664,20 @@ def main():
     if not args.no_cpu:
         cpu = cpu_baseline(blob, head["prompt"], head["ids"])
         log("cpu baseline:", json.dumps(cpu))
+
+    # the two kernels the targets are set on (fused prefill attention >= 50 % of the bf16 MFMA peak, decode attention
+    # >= 70 % of HBM peak), inside the roofline object so that they travel with it
+    targets = {}
+    pa = also.get("prefill_attention_B8_T1024_H12x64", {}).get("bf16")
+    if pa:
+        targets["prefill_attention_bf16_causal_B8_T1024_H12x64"] = dict(pa["roofline"], target_frac=0.5, avg_launch_us=round(pa["ms"] * 1e3, 2))
+    pa = also.get("prefill_attention_B4_T4096_H32x128", {}).get("bf16")
+    if pa:
+        targets["prefill_attention_bf16_causal_B4_T4096_H32x128"] = dict(pa["roofline"], target_frac=0.5, avg_launch_us=round(pa["ms"] * 1e3, 2))
+    da = also.get("decode_attention_H32x128", {})
+    if "roofline" in da:
+        targets["decode_attention_bf16_B32_L4096_H32x128"] = dict(da["roofline"], target_frac=0.7, avg_launch_us=da["bf16_B32_L4096"]["us"])
+    roof["targets"] = targets
 
     line = {
         "metric": "decode tokens/sec", "value": round(head["tokens_per_s"], 2), "unit": "tokens/s",

@@ -154,6 +154,13 @@ struct FlashArgs {
     float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
 };
 
+__device__ __forceinline__ float flash_half_max(float v)
+{
+    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // One 32-key online-softmax step for all query tiles of a wavefront, written as a single
 // branch-free block (apart from the wavefront-uniform rescale test) so the tiles'
 // dependency chains interleave.  On return s holds the weights p.  MASKED: scores equal to
@@ -171,8 +178,9 @@ __device__ __forceinline__ void flash_softmax_step(floatx16 (&s)[QT], floatx16 (
 #pragma unroll
         for (int v = 1; v < 16; v++) mx[qt] = fmaxf(mx[qt], s[qt][v]);
     }
+    // the other lane half's maximum comes through a register swap, not a trip through LDS
 #pragma unroll
-    for (int qt = 0; qt < QT; qt++) mx[qt] = fmaxf(mx[qt], __shfl_xor(mx[qt], 32, 64));
+    for (int qt = 0; qt < QT; qt++) mx[qt] = flash_half_max(mx[qt]);
     bool same = true;
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
@@ -222,10 +230,13 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
     constexpr int LDK = HS + PAD, LDV = BN + PAD;
     constexpr int CHR = HS / EPC;             // 16-byte chunks per K / V row
     constexpr int KPT = (BN * CHR) / NT;      // K chunks per thread per block
-    constexpr int VPW = CHR / NW;             // V chunks per wavefront (one key per lane)
-    static_assert(KPT >= 1 && VPW >= 1 && (BN * CHR) % NT == 0 && CHR % NW == 0, "tile / thread mismatch");
+    // 16-bit storage keeps V row-major in LDS, staged exactly like K, and reads the V^T fragments with the transposing
+    // LDS read; fp32 stores V transposed (4-byte scatter stores, which do not collide)
+    constexpr bool VROW = sizeof(T) == 2;
+    constexpr int VPW = VROW ? KPT : CHR / NW;   // V chunks per thread (row-major) / per wavefront, one key per lane (transposed)
+    static_assert(KPT >= 1 && VPW >= 1 && (BN * CHR) % NT == 0 && (VROW || CHR % NW == 0), "tile / thread mismatch");
     __shared__ __attribute__((aligned(16))) T Ks[BN * LDK];
-    __shared__ __attribute__((aligned(16))) T Vt[HS * LDV];
+    __shared__ __attribute__((aligned(16))) T Vt[VROW ? BN * LDK : HS * LDV];
     __shared__ float Ms[BN];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -288,9 +299,17 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
             const int e = tid + i * NT;
             kreg[i] = *(const u32x4*)(kp + (size_t)min(kbase + e / CHR, a.Tk - 1) * HS + (e % CHR) * EPC);
         }
-        const size_t vrow = (size_t)min(kbase + lane, a.Tk - 1) * HS;
+        if (VROW) {
 #pragma unroll
-        for (int i = 0; i < VPW; i++) vreg[i] = *(const u32x4*)(vp + vrow + (wave + NW * i) * EPC);
+            for (int i = 0; i < VPW; i++) {
+                const int e = tid + i * NT;
+                vreg[i] = *(const u32x4*)(vp + (size_t)min(kbase + e / CHR, a.Tk - 1) * HS + (e % CHR) * EPC);
+            }
+        } else {
+            const size_t vrow = (size_t)min(kbase + lane, a.Tk - 1) * HS;
+#pragma unroll
+            for (int i = 0; i < VPW; i++) vreg[i] = *(const u32x4*)(vp + vrow + (wave + NW * i) * EPC);
+        }
     };
     auto sstore = [&](int kb) {
 #pragma unroll
@@ -298,8 +317,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
             const int e = tid + i * NT;
             *(u32x4*)(&Ks[(e / CHR) * LDK + (e % CHR) * EPC]) = kreg[i];
         }
+        if (VROW) {
 #pragma unroll
-        for (int i = 0; i < VPW; i++) TR::scatter_chunk(&Vt[(wave + NW * i) * EPC * LDV + lane], LDV, vreg[i]);
+            for (int i = 0; i < VPW; i++) {
+                const int e = tid + i * NT;
+                *(u32x4*)(&Vt[(e / CHR) * LDK + (e % CHR) * EPC]) = vreg[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < VPW; i++) TR::scatter_chunk(&Vt[(wave + NW * i) * EPC * LDV + lane], LDV, vreg[i]);
+        }
         if (KIND == 2 && tid < BN) {
             const int key = kb * BN + tid;
             Ms[tid] = key < a.Tk ? a.mask[(size_t)b * a.Tk + key] : 1.f;
@@ -402,7 +429,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                 for (int t = 0; t < PF; t++)
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
-                        const u32x4 vf = TR::load_vt(&Vt[(dt * 32 + l32) * LDV + 32 * sub], t, half);
+                        const u32x4 vf = VROW ? TR::load_vt_rowmajor(&Vt[32 * sub * LDK + dt * 32], LDK, t, lane)
+                                              : TR::load_vt(&Vt[(dt * 32 + l32) * LDV + 32 * sub], t, half);
 #pragma unroll
                         for (int qt = 0; qt < QT; qt++) o[dt][qt] = TR::mma(vf, pf[qt][t], o[dt][qt]);
                     }
@@ -450,13 +478,6 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 // keys are double buffered; block kb + 1 of K is written to LDS during phase 2 kb and of V during phase
 // 2 kb + 1, each while the other buffer is being read.  Phases that are not in steady state (the first, the
 // last two, diagonal or ragged steps) take a plain sequential path built from the same pieces.
-__device__ __forceinline__ float flash_half_max(float v)
-{
-    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
-    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-
 struct PipeStage {
     const bf16_t* gk[2];   // global addresses of this thread's two K chunks of block 0 (advance by 64 * 64 per block)
     const bf16_t* gv[2];

@@ -23,6 +23,17 @@ __device__ inline uint32_t pack_bf16x2(float a, float b)
     return *reinterpret_cast<uint32_t*>(&r);
 }
 
+// Transposing LDS read of gfx950 (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane i supplies the address of
+// four consecutive 16-bit elements; the 64 elements form a 4 x 16 matrix whose row r comes from lanes 4r .. 4r+3, and
+// lane c of the group receives column c: {row 0, row 1, row 2, row 3}[c].  A row-major [key][dim] tile is thus read as
+// the [dim][key] fragments the matrix cores want without ever being stored transposed.
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr16(const bf16_t* p)
+{
+    const short4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(p));
+    return *reinterpret_cast<const uint2*>(&r);
+}
+
 template <typename T> struct FlashTraits;
 template <> struct FlashTraits<bf16_t> {
     static constexpr int EPC = 8;    // elements per 16-byte chunk
@@ -36,6 +47,17 @@ template <> struct FlashTraits<bf16_t> {
     {
         const bf16_t* p = row + 16 * t + 4 * half;
         uint2 lo = *(const uint2*)p, hi = *(const uint2*)(p + 8);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+    // The same fragment from a ROW-MAJOR [key][dim] tile (row stride ld elements): `tile` points at key 0, first dim of
+    // the 32-dim tile.  Lane (group g = lane / 16, i = lane % 16) supplies row 4 half + i / 4 of the four-key run, dims
+    // 16 (g & 1) + 4 (i % 4) .. + 3, and receives its own dim lane % 32 for the four keys; the second read is the run
+    // eight keys further on.
+    __device__ static inline u32x4 load_vt_rowmajor(const bf16_t* tile, int ld, int t, int lane)
+    {
+        const int i = lane & 15, half = lane >> 5;
+        const bf16_t* p = tile + (16 * t + 4 * half + (i >> 2)) * ld + 16 * ((lane >> 4) & 1) + 4 * (i & 3);
+        const uint2 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 8 * ld);
         return u32x4{lo.x, lo.y, hi.x, hi.y};
     }
     // P^T fragment t: the weights held in accumulator registers 8t .. 8t+7
@@ -84,6 +106,7 @@ template <> struct FlashTraits<float> {
     }
     // V^T fragment t of a 32-key step: keys 8t + 4h .. +3
     __device__ static inline u32x4 load_vt(const float* row, int t, int half) { return *(const u32x4*)(row + 8 * t + 4 * half); }
+    __device__ static inline u32x4 load_vt_rowmajor(const float*, int, int, int) { return u32x4{0u, 0u, 0u, 0u}; }   // 16-bit storage only
     // P^T fragment t: the weights held in accumulator registers 4t .. 4t+3
     __device__ static inline u32x4 pack_p(const floatx16& p, int t)
     {

@@ -1331,6 +1331,8 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     bool timing = false;
     if (t0 < start) { (void)hipEventRecord(evA, s); timing = true; }
     if (batched) {
+        e = ensure_prefill((size_t)B * nPre);      // allocations stay out of the timed pass
+        if (e) return e;
         HIPCHK(hipEventCreate(&sc.evP0));
         HIPCHK(hipEventCreate(&sc.evP1));
         HIPCHK(hipEventRecord(sc.evP0, s));
