@@ -96,7 +96,7 @@ enum {
     MCH_FN_ATTN_CREATE = 160,               /* -> handle */
     MCH_FN_ATTN_FREE = 161,                 /* f{h} */
     MCH_FN_ATTN_SET = 162,                  /* f{dropout} l{hCudnn, hAttn, gpuId, training, batch, blockSize, heads, hs, seed} (device.h:2463-2485) */
-    MCH_FN_ATTN_FWD = 163,                  /* l{hCudnn, hAttn, blockSize, hQ, hK, hV, hMask, hY, batchMask[, blockSizeK]} (device.h:2488-2506, attn.cu:518-602) */
+    MCH_FN_ATTN_FWD = 163,                  /* l{hCudnn, hAttn, blockSize, hQ, hK, hV, hMask, hY, batchMask[, blockSizeK[, mergedY]]} (device.h:2488-2506, attn.cu:518-602) */
     MCH_FN_ATTN_BWD = 164,                  /* l{hCudnn, hAttn, hQ, hdQ, hK, hdK, hV, hdV, hMask, hY, hdY} (device.h:2509-2529, attn.cu:608-661) */
     MCH_FN_SET = 200,                       /* f{val} l{n, h, 0, idx, xOff} (device.h:6038-6061) */
     MCH_FN_COPY = 202,                      /* l{n, hSrc, hDst, srcOff, dstOff, hStream, srcHalf, dstHalf} (device.h:6063-6095) */
@@ -166,10 +166,18 @@ enum {
      * (RMSNormLayer.cs:156-180):  f{eps}  l{outer, dim, hX, hWeight(0=none), hY}
      *
      * SWIGLU_FWD = silu(a)*b (TransformerBlockLayer.cs:860-875):  l{n, hA, hB, hY}
+     *
+     * QKV_PROJ_HEADS replaces the head of CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-557):
+     * the fused InnerProduct, its bias GEMM, the three channel copies and the three head transposes become one
+     * GEMM whose epilogue adds the bias and writes q, k, v as (batch, heads, T, hs):
+     *   l{batch, T, heads, hs, hX, hWeight (3C x C), hBias (0 = none), hQ, hK, hV}
+     * Together with the 11th value of ATTN_FWD (Y written head-merged) the layer forward is four calls:
+     * QKV_PROJ_HEADS, ATTN_FWD, GEMM and bias GEMM of the output projection.
      */
     MCH_FN_ATTN_DECODE_FWD = 2001,
     MCH_FN_RMSNORM_FWD = 2002,
-    MCH_FN_SWIGLU_FWD = 2003
+    MCH_FN_SWIGLU_FWD = 2003,
+    MCH_FN_QKV_PROJ_HEADS = 2004
 };
 
 /* DEVINIT flags (CudaDnnDLL/Cuda Files/device.h:18-22) */

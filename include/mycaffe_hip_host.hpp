@@ -378,9 +378,12 @@ public:
     {
         ex2(MCH_FN_ATTN_SET, {fDropout}, {hCuDnn, hAttn, nGpuID, bTraining, nBatch, nBlockSize, nHeads, nSize, lSeed});
     }
-    void AttnScaledDotProductForward(long hCuDnn, long hAttn, int nBlockSize, long hQ, long hK, long hV, long hMask, long hY, int nBatchMask = 1)
+    void AttnScaledDotProductForward(long hCuDnn, long hAttn, int nBlockSize, long hQ, long hK, long hV, long hMask, long hY, int nBatchMask = 1,
+                                     bool bMergedY = false)
     {
-        ex2(MCH_FN_ATTN_FWD, {}, {hCuDnn, hAttn, nBlockSize, hQ, hK, hV, hMask, hY, nBatchMask});
+        // the eleventh value (Y written head-merged, (B,T,H,hs)) has no counterpart in the reference
+        if (bMergedY) ex2(MCH_FN_ATTN_FWD, {}, {hCuDnn, hAttn, nBlockSize, hQ, hK, hV, hMask, hY, nBatchMask, nBlockSize, 1});
+        else ex2(MCH_FN_ATTN_FWD, {}, {hCuDnn, hAttn, nBlockSize, hQ, hK, hV, hMask, hY, nBatchMask});
     }
     // additions of this library (no counterpart in the reference)
     void AttnScaledDotProductBackward(long hCuDnn, long hAttn, long hQ, long hdQ, long hK, long hdK, long hV, long hdV, long hMask, long hY,
@@ -397,6 +400,11 @@ public:
                                   long long nStrideBatch, long long nStrideHead, long long nStridePos, float fScale = 0.f)
     {
         m_cuda.AttnDecodeNoAlloc(m_hKernel, {fScale}, {nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead, nStridePos});
+    }
+    // fused QKV projection: q, k, v = X W^T + bias written as (B,H,T,hs) (no counterpart in the reference)
+    void QkvProjHeads(int nBatch, int nT, int nHeads, int nSize, long hX, long hWeight, long hBias, long hQ, long hK, long hV)
+    {
+        ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV});
     }
     void RmsNormForward(int nOuter, int nDim, long hX, long hWeight, long hY, float fEps = 1e-5f)
     {

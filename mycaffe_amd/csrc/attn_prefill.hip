@@ -31,7 +31,14 @@ struct AttnArgs {
     int B, H, Tq, Tk, hs, kind;
     float scale;
     float* lse2;   // optional [B*H*Tq]: log2 of the row's softmax denominator (-inf marks a fully masked row)
+    int yMerged;   // 1: y is written head-merged, (B,Tq,H,hs), the layout the output projection reads; 0: (B,H,Tq,hs)
 };
+
+// offset of output row `row` of head (b, h) in y
+__device__ __forceinline__ size_t attn_y_row(int yMerged, int b, int h, int H, int Tq, int row, int hs)
+{
+    return yMerged ? (((size_t)b * Tq + row) * H + h) * hs : (((size_t)b * H + h) * Tq + row) * hs;
+}
 
 // 4 wavefronts per workgroup, one query row each
 template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(AttnArgs a)
@@ -86,7 +93,7 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
         }
         m = mn;
     }
-    T* y = (T*)a.y + (bh * a.Tq + row) * a.hs;
+    T* y = (T*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, row, a.hs);
     for (int i = 0; i < DPL; i++) {
         int d = lane + i * 64;
         if (d < a.hs) stp(y, d, acc[i] / l);
@@ -98,7 +105,7 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
 hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* handled);
 
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
-                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2)
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2, bool yMerged)
 {
     if (B <= 0 || H <= 0 || Tq <= 0 || Tk <= 0 || hs <= 0) return hipSuccess;
     if (B > 65535 || H > 65535) return hipErrorInvalidValue;
@@ -106,6 +113,7 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
     AttnArgs a;
     a.q = q; a.k = k; a.v = v; a.y = y; a.mask = mask;
     a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale; a.lse2 = lse2;
+    a.yMerged = yMerged ? 1 : 0;
     bool handled = false;
     hipError_t e = attn_flash_launch(s, dt, a, &handled);
     if (e != hipSuccess || handled) return e;
@@ -152,6 +160,7 @@ struct FlashArgs {
     float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
     float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
     float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
+    int yMerged;         // y laid out (B,Tq,H,hs) instead of (B,H,Tq,hs)
 };
 
 __device__ __forceinline__ float flash_half_max(float v)
@@ -453,7 +462,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
         if (a.lse2 && qrow < a.Tq && half == 0)
             a.lse2[bh * a.Tq + qrow] = (m[qt] == a.maskedRaw) ? -INFINITY : __builtin_fmaf(m[qt], a.c, __log2f(lt));
         if (qrow < a.Tq) {
-            T* yr = (T*)a.y + (bh * a.Tq + qrow) * HS;
+            T* yr = (T*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, qrow, HS);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -769,7 +778,7 @@ __global__ __launch_bounds__(256, 3) void flash_pipe_bf16_64_kernel(FlashArgs a)
     const float lt = l[0] + __shfl_xor(l[0], 32, 64);
     const float inv = 1.0f / lt;
     if (qrow < a.Tq) {
-        bf16_t* yr = (bf16_t*)a.y + (bh * a.Tq + qrow) * HS;
+        bf16_t* yr = (bf16_t*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, qrow, HS);
 #pragma unroll
         for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -805,6 +814,7 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     f.maskedRaw = MASKED / a.scale;
     f.lazy = 8.0f / f.c;
     f.lse2 = a.lse2;
+    f.yMerged = a.yMerged;
     *handled = true;
     // Tile shapes picked by measurement on MI355X.  Head size 64: four wavefronts with one 32-row tile each
     // (128-row workgroups) give enough equal-sized workgroups to balance 256 CUs at T = 1024; head size 128

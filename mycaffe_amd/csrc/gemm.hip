@@ -342,10 +342,25 @@ template <> struct BigTraits<float> {
     __device__ static inline void st4(float* p, float a, float b, float c, float d) { *(float4*)p = make_float4(a, b, c, d); }
 };
 
-template <typename T, int WM, int WN, int OCC>
+// Epilogue of the fused QKV projection (HEADS): row r = (b, t) of the M = B*T rows, column c = (which, h, d) of the
+// N = 3*H*hs columns goes, bias added, to element (b, h, t, d) of tensor `which` (q, k, v), i.e. the layout the
+// attention kernels read, instead of to C[r][c].  Replaces the bias GEMM, the three channel copies and the three head
+// transposes that follow the fused InnerProduct in CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-557).
+struct HeadsEpilogue { const void* bias; void* dst[3]; int T, H, hs; };
+
+template <typename T>
+__device__ __forceinline__ T* heads_dst(const HeadsEpilogue& he, int row, int col)
+{
+    const int Cd = he.H * he.hs;
+    const int which = col / Cd, w = col - which * Cd, h = w / he.hs, d = w - h * he.hs;
+    const int b = row / he.T, t = row - b * he.T;
+    return (T*)he.dst[which] + (((size_t)b * he.H + h) * he.T + t) * he.hs + d;
+}
+
+template <typename T, int WM, int WN, int OCC, bool HEADS = false>
 __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
                                                                const T* __restrict__ B, float beta, T* __restrict__ C, int tilesN,
-                                                               int tilesTotal, int bandRows, int colBlock)
+                                                               int tilesTotal, int bandRows, int colBlock, HeadsEpilogue he)
 {
     typedef BigTraits<T> TR;
     constexpr int E = TR::E;
@@ -473,7 +488,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     // row of C (lane%32) and register v is column 8*(v/4) + 4*(lane/32) + v%4: four consecutive columns per
     // register quad.
     const int row_l = lane & 31, col_l = (lane >> 5) * 4;
-    if (m0 + BM <= M && n0 + BN <= N && beta == 0.f && (N % E) == 0 && (((uintptr_t)C) & 15) == 0) {
+    if (m0 + BM <= M && n0 + BN <= N && (HEADS || (beta == 0.f && (((uintptr_t)C) & 15) == 0)) && (N % E) == 0) {
         // interior tile: each wavefront passes its tile, 32 rows at a time, through its own slice of LDS (free
         // after the last barrier) and writes whole 16-byte pieces of rows, the lanes covering full cache lines
         constexpr int CW = 32 * WN, LDC = CW + E;
@@ -486,9 +501,15 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
 #pragma unroll
             for (int j = 0; j < WN; j++)
 #pragma unroll
-                for (int g = 0; g < 4; g++)
-                    TR::st4(cs + row_l * LDC + j * 32 + 8 * g + col_l, alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1],
-                            alpha * acc[i][j][4 * g + 2], alpha * acc[i][j][4 * g + 3]);
+                for (int g = 0; g < 4; g++) {
+                    float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+                    if (HEADS && he.bias) {
+                        const T* bp = (const T*)he.bias + n0 + wn + j * 32 + 8 * g + col_l;
+                        b0 = TR::ld(bp); b1 = TR::ld(bp + 1); b2 = TR::ld(bp + 2); b3 = TR::ld(bp + 3);
+                    }
+                    TR::st4(cs + row_l * LDC + j * 32 + 8 * g + col_l, alpha * acc[i][j][4 * g] + b0, alpha * acc[i][j][4 * g + 1] + b1,
+                            alpha * acc[i][j][4 * g + 2] + b2, alpha * acc[i][j][4 * g + 3] + b3);
+                }
             // same wavefront wrote and reads: LDS operations of one wavefront complete in order
             T* cg = C + (size_t)(m0 + wm + i * 32 + rr) * N + n0 + wn + cc;
 #pragma unroll
@@ -496,7 +517,8 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                 // lanes past RPI * LPR (row widths that do not divide 64) and rows past the block stay idle
                 if (rr < RPI && it * RPI + rr < 32) {
                     const u32x4 v = *(const u32x4*)(cs + (it * RPI + rr) * LDC + cc);
-                    *(u32x4*)(cg + (size_t)it * RPI * N) = v;
+                    if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + i * 32 + it * RPI + rr, n0 + wn + cc) = v;
+                    else *(u32x4*)(cg + (size_t)it * RPI * N) = v;
                 }
             }
         }
@@ -515,16 +537,24 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                 if (c < N) {
                     const size_t ci = (size_t)r * N + c;
                     float o = alpha * acc[i][j][v];
-                    if (beta != 0.f) o += beta * TR::ld(C + ci);
-                    TR::st(C + ci, o);
+                    if (HEADS) {
+                        if (he.bias) o += TR::ld((const T*)he.bias + c);
+                        TR::st(heads_dst<T>(he, r, c), o);
+                    } else {
+                        if (beta != 0.f) o += beta * TR::ld(C + ci);
+                        TR::st(C + ci, o);
+                    }
                 }
             }
         }
 }
 
-template <typename T, int WM, int WN, int OCC>
-static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C)
+template <typename T, int WM, int WN, int OCC, bool HEADS = false>
+static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C,
+                             const HeadsEpilogue* heads = nullptr)
 {
+    HeadsEpilogue he = {};
+    if (heads) he = *heads;
     constexpr int E = BigTraits<T>::E;
     const int tm = (m + 64 * WM - 1) / (64 * WM), tn = (n + 64 * WN - 1) / (64 * WN);
     const long long total = (long long)tm * tn;
@@ -535,7 +565,7 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
     if (ldsEpilogue > lds) lds = ldsEpilogue;
     static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
     if (!attr) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC, HEADS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr = true;
     }
@@ -551,8 +581,8 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
             colBlock = (tn + nb - 1) / nb;   // equal-width blocks
         }
     }
-    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
-                       (T*)C, tn, (int)total, bandRows, colBlock);
+    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
+                       (T*)C, tn, (int)total, bandRows, colBlock, he);
     return hipGetLastError();
 }
 
@@ -597,9 +627,52 @@ __global__ void gemm_rank1_kernel(int m, int n, float alpha, const T* __restrict
     }
 }
 
+// Fallback of the fused QKV projection: the plain product in `tmp` (M x 3C) is split, bias added, into the three
+// (B,H,T,hs) tensors in one pass.
+template <typename T>
+__global__ void qkv_split_heads_kernel(const T* __restrict__ tmp, size_t total, int N, HeadsEpilogue he)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+        const int r = (int)(i / N), c = (int)(i - (size_t)r * N);
+        float o = ldf(tmp, i);
+        if (he.bias) o += ldf((const T*)he.bias, c);
+        stf(heads_dst<T>(he, r, c), 0, o);
+    }
+}
+
+hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
+                            void* q, void* k, void* v, void* tmp)
+{
+    const int m = B * T, C = H * hs, n = 3 * C, kk = C;
+    if (m <= 0 || C <= 0) return hipSuccess;
+    HeadsEpilogue he;
+    he.bias = bias; he.dst[0] = q; he.dst[1] = k; he.dst[2] = v; he.T = T; he.H = H; he.hs = hs;
+    const int vec = dt == F32 ? 4 : 8;
+    const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 == 0) && hs % vec == 0;
+    const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+    if (aligned && dt == F32 && kk % 32 == 0) {
+        if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
+        return launch_big<float, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
+    }
+    if (aligned && dt == BF16 && kk % 64 == 0) {
+        if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
+        return launch_big<bf16_t, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
+    }
+    // any other shape: plain product into the caller's scratch matrix, then one splitting pass
+    if (!tmp) return hipErrorInvalidValue;
+    hipError_t e = k_gemm(s, dt, false, true, m, n, kk, 1.f, X, W, 0.f, tmp);
+    if (e != hipSuccess) return e;
+    const size_t total = (size_t)m * n;
+    const int grid = (int)std::min<size_t>((total + 255) / 256, 8192);
+    if (dt == F32) hipLaunchKernelGGL(qkv_split_heads_kernel<float>, grid, 256, 0, s, (const float*)tmp, total, n, he);
+    else hipLaunchKernelGGL(qkv_split_heads_kernel<bf16_t>, grid, 256, 0, s, (const bf16_t*)tmp, total, n, he);
+    return hipGetLastError();
+}
+
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
                   const void* B, float beta, void* C)
 {
+    if (m <= 0 || n <= 0) return hipSuccess;
     if (k == 1) {
         const size_t es = dt == F32 ? 4 : 2;
         const bool vec = n % 4 == 0 && ((((uintptr_t)B | (uintptr_t)C) & (4 * es - 1)) == 0);

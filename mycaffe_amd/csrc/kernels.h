@@ -92,6 +92,10 @@ hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x,
 // row-major C[m,n] = alpha*op(A)*op(B) + beta*C; A, B, C all of storage type dt
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
                   const void* B, float beta, void* C);
+// Fused QKV projection of CausalSelfAttentionLayer: [q|k|v] = X W^T + bias with X (B*T, C), W (3C, C), C = H*hs, written
+// straight into three (B,H,T,hs) tensors.  tmp: (B*T, 3C) scratch, only used for shapes the fused kernel does not take.
+hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
+                            void* q, void* k, void* v, void* tmp);
 // column-major strided batched gemm with BLAS semantics (fp32)
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
@@ -106,7 +110,9 @@ enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAU
 //   MASK_QK (Tq,Tk) shared, MASK_KEY (B,Tk), MASK_BQK (B,Tq,Tk); zero entries are filled with -1e29.
 //   MASK_CAUSAL needs no mask buffer (lower triangle kept).
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
-                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2 = nullptr);
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2 = nullptr,
+                          bool yMerged = false);
+// yMerged: y is written as (B,Tq,H,hs), the head-merged layout the output projection reads, instead of (B,H,Tq,hs).
 // With lse2 ([B*H*Tq] fp32) the forward pass also stores log2 of every row's softmax denominator (scores scaled, masked
 // ones at -1e29; -inf marks a row whose keys are all masked), which is all the backward pass needs of the probabilities.
 //

@@ -1495,10 +1495,12 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
     case MCH_FN_ATTN_FWD: {
-        // l{hCudnn,hAttn,blockSize,hQ,hK,hV,hMask,hY,batchMask[,blockSizeK]} (device.h:2488-2506, attn.cu:518-602)
-        // The optional 10th value (key length when it differs from the query length) has no
-        // counterpart in the reference, whose handle needs T_q == T_k.
-        NEED_L(9, 10);
+        // l{hCudnn,hAttn,blockSize,hQ,hK,hV,hMask,hY,batchMask[,blockSizeK[,mergedY]]} (device.h:2488-2506, attn.cu:518-602)
+        // The optional 10th value (key length when it differs from the query length) and 11th (1: Y is written
+        // head-merged, (B,T,H,hs), ready for the output projection) have no counterpart in the reference, whose
+        // handle needs T_q == T_k and always writes (B,H,T,hs).
+        NEED_L(9, 11);
+        const bool mergedY = ll > 10 && pl[10] != 0;
         AttnState* st = m_attn.get((long)pl[1]);
         if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
         int T = (int)pl[2];
@@ -1537,6 +1539,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         }
         float* lse = nullptr;
         st->lseValid = false;
+        if (st->training && mergedY) {
+            last_detail = "the head-merged output layout is for inference: the backward pass reads Y as (B,H,T,hs)";
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
         if (st->training) {
             // training mode: keep one number per query row for ATTN_BWD (the reference keeps the T x T probabilities)
             const size_t rows = (size_t)st->batch * st->heads * T;
@@ -1554,7 +1560,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             }
         }
         HIPCHK(k_attn_prefill(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, st->batch, st->heads, T, Tk, st->hs, st->scale,
-                              M ? (const float*)M->ptr : nullptr, kind, lse));
+                              M ? (const float*)M->ptr : nullptr, kind, lse, mergedY));
         // the backward pass needs this output (dY . Y per row); the C# layer hands ATTN_BWD a Y buffer that holds the
         // head-merged layout by then (CausalSelfAttentionLayer.cs:668-672), so a copy stays with the handle
         if (lse) HIPCHK(hipMemcpyAsync(st->ysave, Y->ptr, (size_t)qn * Y->esize(), hipMemcpyDeviceToDevice, s));
@@ -1622,6 +1628,38 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
 
     case MCH_FN_ATTN_DECODE_FWD:
         return attn_decode_fwd(pf, lf, pl, ll, false);
+
+    case MCH_FN_QKV_PROJ_HEADS: {
+        // l{batch, T, heads, hs, hX, hW, hBias(0 = none), hQ, hK, hV}: [q|k|v] = X W^T + bias, X (batch*T, C), W (3C, C),
+        // C = heads*hs, each third written as (batch, heads, T, hs)
+        NEED_L(10, 10);
+        const long long B = pl[0], T = pl[1], H = pl[2], hs = pl[3];
+        if (B < 1 || T < 1 || H < 1 || hs < 1 || B * T > INT_MAX || 3 * H * hs > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const long long C = H * hs, M = B * T;
+        MemItem *X, *W, *Bi = nullptr, *Q, *K, *V;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &W));
+        if (pl[6]) ERRCHK(mem((long)pl[6], &Bi));
+        ERRCHK(mem((long)pl[7], &Q));
+        ERRCHK(mem((long)pl[8], &K));
+        ERRCHK(mem((long)pl[9], &V));
+        if (X->half != W->half || X->half != Q->half || X->half != K->half || X->half != V->half || (Bi && Bi->half != X->half))
+            return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, M * C);
+        RANGE(W, 0, 3 * C * C);
+        if (Bi) RANGE(Bi, 0, 3 * C);
+        RANGE(Q, 0, M * C);
+        RANGE(K, 0, M * C);
+        RANGE(V, 0, M * C);
+        void* ws = nullptr;
+        ERRCHK(workspace((size_t)(M * 3 * C) * X->esize(), &ws));
+        HIPCHK(k_gemm_qkv_heads(s, X->dt(), (int)B, (int)T, (int)H, (int)hs, X->ptr, W->ptr, Bi ? Bi->ptr : nullptr, Q->ptr, K->ptr,
+                                V->ptr, ws));
+        m_mem.touch((long)pl[7]);
+        m_mem.touch((long)pl[8]);
+        m_mem.touch((long)pl[9]);
+        return 0;
+    }
 
     // ---- RoPE ------------------------------------------------------------------
     case MCH_FN_CREATE_ROPE: {

@@ -108,6 +108,7 @@ class CUDAFN:
     ATTN_DECODE_FWD = 2001
     RMSNORM_FWD = 2002
     SWIGLU_FWD = 2003
+    QKV_PROJ_HEADS = 2004
 
 
 class CUDAQRY:
@@ -633,14 +634,23 @@ class CudaDnn:
         self._ex2(CUDAFN.CUDA_ATTN_SET, [fDropout], [hCuDnn, hAttn, nGpuID, int(bTraining), nBatch, nBlockSize, nHeads, nSize, lSeed])
 
     def AttnScaledDotProductForward(self, hCuDnn, hAttn, nBlockSize, hQdata, hKdata, hVdata, hMaskdata, hYdata,
-                                    bBatchMask=True, nBlockSizeK=None):
+                                    bBatchMask=True, nBlockSizeK=None, bMergedY=False):
         """CudaDnn.cs:5673-5679.  ``nBlockSizeK`` (key length, when it differs from the
         query length) is an optional tenth value with no counterpart in the reference, and so
-        is ``bBatchMask=2`` (a (B,T_q,T_k) mask)."""
+        are ``bBatchMask=2`` (a (B,T_q,T_k) mask) and ``bMergedY`` (eleventh value: Y written
+        head-merged, (B,T,H,hs), instead of (B,H,T,hs))."""
         rgl = [hCuDnn, hAttn, nBlockSize, hQdata, hKdata, hVdata, hMaskdata, hYdata, int(bBatchMask)]
-        if nBlockSizeK is not None:
-            rgl.append(nBlockSizeK)
+        if nBlockSizeK is not None or bMergedY:
+            rgl.append(nBlockSizeK if nBlockSizeK is not None else nBlockSize)
+        if bMergedY:
+            rgl.append(1)
         self._ex2(CUDAFN.CUDA_ATTN_FWD, None, rgl)
+
+    def QkvProjHeads(self, nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV):
+        """Fused QKV projection (no counterpart in the reference: replaces the InnerProduct, bias GEMM, three
+        channel copies and three head transposes of CausalSelfAttentionLayer.cs:526-557): q, k, v written as
+        (B,H,T,hs)."""
+        self._ex2(CUDAFN.QKV_PROJ_HEADS, None, [nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV])
 
     def AttnScaledDotProductBackward(self, hCuDnn, hAttn, hQdata, hQdiff, hKdata, hKdiff, hVdata, hVdiff, hMaskdata, hYData, hYdiff):
         """CudaDnn.cs:5695-5701."""

@@ -9,6 +9,8 @@
 //   f32_fused     fp32 storage, fused attention handle (ids 160-163)
 //   f32_explicit  fp32 storage, the layer's default chain: transpose, MatMul, scale, mask, softmax, MatMul
 //   bf16_fused    16-bit storage (ALLOCMEM_HALF), fused attention handle
+//   *_4call       the same forward as four calls: fused QKV projection writing (B,H,T,hs) (id 2004), attention handle
+//                 writing head-merged output, output projection GEMM and its bias GEMM
 // Timed region: `reps` forwards between two device synchronisations (steady_clock).
 #include <chrono>
 #include <cmath>
@@ -59,7 +61,7 @@ std::vector<float> normal(size_t n, float std, unsigned seed)
     return v;
 }
 
-double run(CudaDnn& cuda, bool half, bool fused, int reps)
+double run(CudaDnn& cuda, bool half, bool fused, int reps, bool fourCall = false)
 {
     const int B = 8, T = 1024, C = 768, H = 12, hs = C / H, M = B * T;
     const long long MC = (long long)M * C;
@@ -90,6 +92,13 @@ double run(CudaDnn& cuda, bool half, bool fused, int reps)
         cuda.SetTensorDesc(hTopDesc, B * H * T, T, 1, 1, half);
     }
     auto forward = [&]() {
+        if (fourCall) {
+            cuda.QkvProjHeads(B, T, H, hs, hX, hWa, hBa, hQt, hKt, hVt);
+            cuda.AttnScaledDotProductForward(hCudnn, hAttn, T, hQt, hKt, hVt, hMask, hY, 0, true);
+            cuda.gemm(false, true, M, C, C, 1.f, hY, hWp, 0.f, hTop);
+            cuda.gemm(false, false, M, C, 1, 1.f, hOnes, hBp, 1.f, hTop);
+            return;
+        }
         // q, k, v = c_attn(x).split(n_embd, dim = 2)   (InnerProductLayer.cs:372-417: gemm, then the bias as a rank-1 gemm)
         cuda.gemm(false, true, M, 3 * C, C, 1.f, hX, hWa, 0.f, hIp);
         cuda.gemm(false, false, M, 3 * C, 1, 1.f, hOnes, hBa, 1.f, hIp);
@@ -145,7 +154,10 @@ int main(int argc, char** argv)
         const double a = run(cuda, false, true, reps);
         const double b = run(cuda, false, false, reps);
         const double c = run(cuda, true, true, reps);
-        std::printf("{\"reps\": %d, \"f32_fused_ms\": %.4f, \"f32_explicit_ms\": %.4f, \"bf16_fused_ms\": %.4f}\n", reps, a, b, c);
+        const double d = run(cuda, false, true, reps, true);
+        const double e = run(cuda, true, true, reps, true);
+        std::printf("{\"reps\": %d, \"f32_fused_ms\": %.4f, \"f32_explicit_ms\": %.4f, \"bf16_fused_ms\": %.4f, \"f32_4call_ms\": %.4f, "
+                    "\"bf16_4call_ms\": %.4f}\n", reps, a, b, c, d, e);
     } catch (const std::exception& e) {
         std::fprintf(stderr, "csa_layer_bench: %s\n", e.what());
         return 1;

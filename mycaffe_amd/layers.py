@@ -269,8 +269,13 @@ class CausalSelfAttentionLayer:
     """
 
     def __init__(self, cuda, heads, embed, block_size, bias_term=True, enable_cuda_scaled_dot_product_attention=True,
-                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, training=False):
+                 enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, training=False,
+                 fused_qkv_heads=False):
         self.training = training
+        # four calls per forward instead of seventeen (ids with no counterpart in the reference): the fused QKV
+        # projection writes q, k, v as (B,H,T,hs) and the attention handle writes its output head-merged.  Inference,
+        # fused attention handle, no rotary embedding.
+        self.fused_qkv_heads = fused_qkv_heads
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
         self.nSize = embed // heads
         self.bias_term, self.half = bias_term, half
@@ -320,6 +325,26 @@ class CausalSelfAttentionLayer:
             raise ValueError("sequence longer than block_size")
         self._reshape(B, T)
         b, cuda, H, hs = self.b, self.cuda, self.nHeads, self.nSize
+        if self.fused_qkv_heads:
+            if not self.enable_sdpa or self.hRope or self.training:
+                raise ValueError("fused_qkv_heads needs the fused attention handle, no rotary embedding, inference mode")
+            for name in ("Qt", "Kt", "Vt"):
+                b[name].Reshape(B, H, T, hs)
+            ip = self.c_attn
+            cuda.QkvProjHeads(B, T, H, hs, blobX.gpu_data, ip.blobs[0].gpu_data, ip.blobs[1].gpu_data if ip.bias_term else 0,
+                              b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data)
+            mask = self.blobMask
+            if T != self.nBlockSize:
+                if getattr(self, "_sdpa_mask_T", None) != T:
+                    self.blobMaskSdpa = Blob(cuda, (1, 1, T, T))
+                    self.blobMaskSdpa.mutable_cpu_data = np.tril(np.ones((T, T), np.float32))
+                    self._sdpa_mask_T = T
+                mask = self.blobMaskSdpa
+            b["Y"].Reshape(B, T, C)
+            cuda.AttnScaledDotProductForward(self.hCudnn, self.hAttn, T, b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data,
+                                             mask.gpu_data, b["Y"].gpu_data, False, T, True)
+            self.c_proj.Forward(b["Y"], top)
+            return
         # q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
         self.c_attn.Forward(blobX, b["IpAttn"])
         for name in "QKV":

@@ -343,3 +343,60 @@ def test_attn_decode_with_rope_and_append(dev):
     assert_close(dev.get(hy, q.shape), ref, FP32_RTOL, "decode with rope")
     assert_close(dev.get(hk, kc.shape), kc2, 1e-6, "key cache after append")
     assert np.array_equal(dev.get(hv, vc.shape), vc2)
+
+
+# ---- fused QKV projection (id 2004) and head-merged attention output -----------------------
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("B,T,H,hs,bias", [(2, 128, 4, 64, True), (3, 100, 3, 64, True), (1, 257, 2, 128, False), (2, 40, 3, 16, True),
+                                           (2, 64, 5, 24, True)])
+def test_qkv_proj_heads_against_the_call_sequence_it_replaces(dev, half, B, T, H, hs, bias):
+    """One call against InnerProduct + bias GEMM + three channel copies + three head transposes
+    (CausalSelfAttentionLayer.cs:526-557): bit for bit in fp32, within the 16-bit bar otherwise, and against the checker."""
+    C = H * hs
+    rng = np.random.default_rng(B * 1000 + T)
+    x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    w = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
+    bv = bf16_round((rng.standard_normal(3 * C) * 0.1).astype(np.float32)) if bias else None
+    hx, hw = dev.put(x, half), dev.put(w, half)
+    hb = dev.put(bv, half) if bias else 0
+    hq, hk, hv = (dev.zeros(B * T * C, half) for _ in range(3))
+    dev.cuda.QkvProjHeads(B, T, H, hs, hx, hw, hb, hq, hk, hv)
+    got = [dev.get(h, (B, H, T, hs)) for h in (hq, hk, hv)]
+    # the sequence it replaces, through the layer mirror's own pieces
+    layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, bias, True, half=half)
+    bottom, top = Blob(dev.cuda, x.shape, half=half), Blob(dev.cuda, half=half)
+    bottom.mutable_cpu_data = x
+    layer.Setup(bottom, w, bv if bias else None, np.eye(C, dtype=np.float32), np.zeros(C, np.float32) if bias else None)
+    layer.Forward(bottom, top)
+    seq = [layer.b[n].mutable_cpu_data.reshape(B, H, T, hs) for n in ("Qt", "Kt", "Vt")]
+    ref = R.inner_product(x, w, bv, np.float64).reshape(B, T, 3, H, hs).transpose(2, 0, 3, 1, 4)
+    for i, name in enumerate("qkv"):
+        assert_close(got[i], ref[i], BF16_RTOL if half else FP32_RTOL, name + " vs checker")
+        if not half:
+            assert np.array_equal(got[i], seq[i]), name + " differs from the call sequence"
+        else:
+            assert_close(got[i], seq[i], BF16_RTOL, name + " vs the call sequence")
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("B,T,C,H", [(2, 128, 256, 4), (1, 200, 192, 3), (2, 96, 256, 2), (2, 50, 48, 3)])
+def test_causal_self_attention_layer_as_four_calls(dev, half, B, T, C, H):
+    rng = np.random.default_rng(T)
+    x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    wa = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
+    wp = bf16_round((rng.standard_normal((C, C)) * 0.05).astype(np.float32))
+    ba = bf16_round((rng.standard_normal(3 * C) * 0.1).astype(np.float32))
+    bp = bf16_round((rng.standard_normal(C) * 0.1).astype(np.float32))
+    outs = []
+    for fused in (False, True):
+        layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, True, True, half=half, fused_qkv_heads=fused)
+        bottom, top = Blob(dev.cuda, x.shape, half=half), Blob(dev.cuda, half=half)
+        bottom.mutable_cpu_data = x
+        layer.Setup(bottom, wa, ba, wp, bp)
+        layer.Forward(bottom, top)
+        outs.append(top.mutable_cpu_data.copy())
+    ref = R.causal_self_attention(x, wa, ba, wp, bp, H, dtype=np.float64)["y"]
+    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "four-call layer vs checker")
+    if not half:
+        assert np.array_equal(outs[0], outs[1]), "four-call layer differs from the seventeen-call sequence"
