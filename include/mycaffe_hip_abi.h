@@ -111,6 +111,8 @@ enum {
     MCH_FN_SUB = 230,                       /* l{n, hA, hB, hY[, aOff, bOff, yOff, nB]} (device.cu:2294-2331) */
     MCH_FN_MUL = 231,                       /* l{n, hA, hB, hY[, aOff, bOff, yOff]} (device.cu:2398-2423) */
     MCH_FN_DIV = 233,                       /* l{n, hA, hB, hY} (device.cu:2492-2505) */
+    MCH_FN_EXP = 235,                       /* [f{beta}] l{n, hA, hY[, aOff, yOff, 0]} (device.cu:2531-2557) */
+    MCH_FN_LOG = 236,                       /* [f{beta[, alpha]}] l{n, hA, hY[, 0, 0]} (device.cu:2564-2590) */
     MCH_FN_POWX = 237,                      /* f{alpha} l{n, hA, 0, hY[, aOff, yOff]} (device.cu:2595-2618) */
     MCH_FN_SQRT = 239,                      /* [f{epsilon}] l{n, hX, hY} (device.cu:2712-2728) */
     MCH_FN_TRANSPOSE = 261,                 /* l{n, hX, hY, hXCounts, hYCounts, hMapping, numAxes, hBuffer} (device.cu:3088-3107) */
@@ -119,7 +121,11 @@ enum {
     MCH_FN_TRANSPOSE_HW = 267,              /* l{n, c, h, w, hSrc, hDst} (device.cu:3110-3127) */
     MCH_FN_INVERT = 273,                    /* [f{numerator, denominator}] l{n, hX, hY[, xOff, yOff]} (device.cu:2624-2655) */
     MCH_FN_CHANNEL_MEAN = 287,              /* l{count, outer, channels, inner, hX, hY[, xOff]} (device.cu:3386-3405) */
+    MCH_FN_CHANNEL_MAX = 290,               /* l{count, outer, channels, inner, hX, hY, returnIdx[, acrossChannels]} (device.cu:3359-3380) */
+    MCH_FN_CHANNEL_SUB = 291,               /* l{count, outer, channels, inner, hX, hY[, hA]}: y = a - x[n, s], a = y when absent (device.cu:3438-3457) */
     MCH_FN_CHANNEL_SUM = 292,               /* l{count, outer, channels, inner, hX, hY} (device.cu:3488-3503) */
+    MCH_FN_CHANNEL_DIV = 293,               /* l{count, outer, channels, inner, hX, hY[, method]}: y /= x[n, s] (device.cu:3541-3560) */
+    MCH_FN_CHANNEL_DOT = 294,               /* l{count, outer, channels, inner, hX, hA, hY} (device.cu:3638-3654) */
     MCH_FN_CHANNEL_COPY = 300,              /* l{count, outer, channels, blocks, inner, offset, hX, hY, dir} (device.cu:3730-3748) */
     MCH_FN_CHANNEL_FILLFROM = 301,          /* l{count, outer, channels, inner, hX, hY, dir} (CudaDnn.cs:9086-9092, math.cu:7465-7481) */
     MCH_FN_CHANNEL_COPYALL = 302,           /* l{count, outer, channels, inner, hX, hY} (CudaDnn.cs:9443-9449, math.cu:7630-7639) */

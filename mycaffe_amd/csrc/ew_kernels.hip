@@ -1156,4 +1156,99 @@ hipError_t k_channel_spread(hipStream_t s, DType dt, int mode, size_t n, size_t 
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Primitives of the CAFFE-engine softmax chain (SoftmaxLayer.cs:230-330): exp, log, and the per-(n, s) channel
+// reductions and broadcasts.  x is (num, channels, spatial); the reduced tensors are (num, spatial).
+struct ExpF { float beta; __device__ float operator()(float a, float) const { return expf(beta * a); } };                    // math.cu:5859-5865
+struct LogF { float beta, alpha; __device__ float operator()(float a, float) const { return logf(beta * (a + alpha)); } };   // math.cu:5923-5929
+hipError_t k_exp(hipStream_t s, DType dt, size_t n, const void* a, void* y, float beta) { return launch_map(s, dt, n, a, nullptr, y, ExpF{beta}); }
+hipError_t k_log(hipStream_t s, DType dt, size_t n, const void* a, void* y, float beta, float alpha) { return launch_map(s, dt, n, a, nullptr, y, LogF{beta, alpha}); }
+
+// across channels (math.cu:6697-6713, 6733-6754): y[n, s] = max over c of x[n, c, s], or its first index; within a
+// channel (math.cu:6716-6730, 6757-6778, whose loop runs over num * spatial rows of `spatial` values): y[i] = max of
+// row i.  Lane = s (across) so that a wavefront reads consecutive values; starts from -FLT_MAX as the reference does.
+template <typename T, bool IDX, bool ACROSS>
+__global__ void channel_max_kernel(size_t rows, int channels, int spatial, const T* __restrict__ x, T* __restrict__ y)
+{
+    GRID_STRIDE(i, rows) {
+        float val = -3.402823466e+38f;
+        int idx = 0;
+        if (ACROSS) {
+            const size_t n = i / spatial, sp = i % spatial;
+            const T* xp = x + n * channels * (size_t)spatial + sp;
+            for (int c = 0; c < channels; c++) {
+                const float v = ld(xp, (size_t)c * spatial);
+                if (v > val) { val = v; idx = c; }
+            }
+        } else {
+            const T* xp = x + i * spatial;
+            for (int j = 0; j < spatial; j++) {
+                const float v = ld(xp, j);
+                if (v > val) { val = v; idx = j; }
+            }
+        }
+        st(y, i, IDX ? (float)idx : val);
+    }
+}
+hipError_t k_channel_max(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, void* y, bool idx, bool across)
+{
+    const size_t rows = num * spatial;
+    if (rows == 0) return hipSuccess;
+#define CMAX(I, A) DISPATCH_DT(dt, hipLaunchKernelGGL((channel_max_kernel<T, I, A>), grid_for(rows), TPB, 0, s, rows, channels, spatial, (const T*)x, (T*)y))
+    if (idx) { if (across) CMAX(true, true); else CMAX(true, false); }
+    else { if (across) CMAX(false, true); else CMAX(false, false); }
+#undef CMAX
+    return hipGetLastError();
+}
+
+// MODE 0: y[i] = a[i] - x[n, s] (channel_sub_kernel, math.cu:6908-6916); MODE 1: y[i] /= x[n, s] (channel_div_kernel,
+// math.cu:7160-7168); i = (n, c, s)
+template <typename T, int MODE>
+__global__ void channel_bcast_kernel(size_t count, int channels, int spatial, const T* __restrict__ a, const T* __restrict__ x, T* y)
+{
+    GRID_STRIDE(i, count) {
+        const size_t n = i / channels / spatial, sp = i % spatial;
+        const float r = ld(x, n * spatial + sp);
+        st(y, i, MODE == 0 ? ld(a, i) - r : ld(y, i) / r);
+    }
+}
+hipError_t k_channel_sub(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* a, const void* x, void* y)
+{
+    if (count == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL((channel_bcast_kernel<T, 0>), grid_for(count), TPB, 0, s, count, channels, spatial, (const T*)a, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+hipError_t k_channel_div(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* x, void* y)
+{
+    if (count == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL((channel_bcast_kernel<T, 1>), grid_for(count), TPB, 0, s, count, channels, spatial, (const T*)nullptr, (const T*)x, (T*)y));
+    return hipGetLastError();
+}
+
+// y[n, s] = sum over c of x[n, c, s] * a[n, c, s] (channel_dot_kernel, math.cu:7335-7351, double accumulation there;
+// fp32 here, channel counts of a softmax axis are short)
+template <typename T>
+__global__ void channel_dot_kernel(size_t rows, int channels, int spatial, const T* __restrict__ x, const T* __restrict__ a, T* __restrict__ y)
+{
+    GRID_STRIDE(i, rows) {
+        const size_t n = i / spatial, sp = i % spatial;
+        const size_t base = n * channels * (size_t)spatial + sp;
+        float v0 = 0.f, v1 = 0.f;
+        int c = 0;
+        for (; c + 1 < channels; c += 2) {
+            v0 += ld(x, base + (size_t)c * spatial) * ld(a, base + (size_t)c * spatial);
+            v1 += ld(x, base + (size_t)(c + 1) * spatial) * ld(a, base + (size_t)(c + 1) * spatial);
+        }
+        if (c < channels) v0 += ld(x, base + (size_t)c * spatial) * ld(a, base + (size_t)c * spatial);
+        st(y, i, v0 + v1);
+    }
+}
+hipError_t k_channel_dot(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, const void* a, void* y)
+{
+    const size_t rows = num * spatial;
+    if (rows == 0) return hipSuccess;
+    DISPATCH_DT(dt, hipLaunchKernelGGL(channel_dot_kernel<T>, grid_for(rows), TPB, 0, s, rows, channels, spatial, (const T*)x, (const T*)a, (T*)y));
+    return hipGetLastError();
+}
+
 }  // namespace mch

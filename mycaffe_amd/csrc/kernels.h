@@ -87,6 +87,13 @@ hipError_t k_channel_colsum(hipStream_t s, DType dt, size_t outer, int channels,
 // mode 0 fillfrom forward, 1 fillfrom backward, 2 copyall, 3 duplicate (index rules in ew_kernels.hip)
 hipError_t k_channel_spread(hipStream_t s, DType dt, int mode, size_t n, size_t spatial, size_t period, size_t channels, void* x, void* y);
 hipError_t k_rmsnorm(hipStream_t s, DType dt, int outer, int dim, const void* x, const void* w, void* y, float eps);
+// primitives of the CAFFE-engine softmax chain: x is (num, channels, spatial), reduced tensors (num, spatial)
+hipError_t k_exp(hipStream_t s, DType dt, size_t n, const void* a, void* y, float beta);
+hipError_t k_log(hipStream_t s, DType dt, size_t n, const void* a, void* y, float beta, float alpha);
+hipError_t k_channel_max(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, void* y, bool idx, bool across);
+hipError_t k_channel_sub(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* a, const void* x, void* y);
+hipError_t k_channel_div(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* x, void* y);
+hipError_t k_channel_dot(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, const void* a, void* y);
 
 // ---- GEMM family (gemm.hip) ------------------------------------------------
 // row-major C[m,n] = alpha*op(A)*op(B) + beta*C; A, B, C all of storage type dt

@@ -935,6 +935,91 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         m_mem.touch((long)pl[5]);
         return 0;
     }
+    case MCH_FN_EXP:
+    case MCH_FN_LOG: {
+        // 235 [f{beta}] l{n,hA,hY[,aOff,yOff,0]}: y = exp(beta a) (device.cu:2531-2557, math.cu:5859-5865)
+        // 236 [f{beta[,alpha]}] l{n,hA,hY[,0,0]}: y = log(beta (a + alpha)) (device.cu:2564-2590, math.cu:5923-5929)
+        const bool isExp = fn == MCH_FN_EXP;
+        ERRCHK(verify(lf, pf, 0, isExp ? 1 : 2));
+        if (isExp) NEED_L(3, 6); else NEED_L(3, 5);
+        const long long n = pl[0];
+        long long aOff = isExp && ll > 3 ? pl[3] : 0, yOff = isExp && ll > 4 ? pl[4] : 0;
+        if (n < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (aOff < 0) aOff = 0;
+        if (yOff < 0) yOff = 0;
+        const float beta = lf > 0 ? pf[0] : 1.f, alpha = !isExp && lf > 1 ? pf[1] : 0.f;
+        MemItem *A, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &Y));
+        if (A->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(A, aOff, n);
+        RANGE(Y, yOff, n);
+        if (isExp) HIPCHK(k_exp(s, A->dt(), (size_t)n, PTR(A, aOff), PTR(Y, yOff), beta));
+        else HIPCHK(k_log(s, A->dt(), (size_t)n, A->ptr, Y->ptr, beta, alpha));
+        m_mem.touch((long)pl[2]);
+        return 0;
+    }
+    case MCH_FN_CHANNEL_MAX: {
+        // l{count,outer,channels,inner,hX,hY,returnIdx[,acrossChannels]} (device.cu:3359-3380, math.cu:6697-6810)
+        NEED_L(7, 8);
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        const bool idx = pl[6] != 0, across = ll > 7 ? pl[7] != 0 : true;
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (X->ptr == Y->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        // within a channel the reference's kernel walks outer * inner rows of `inner` values
+        RANGE(X, 0, across ? outer * ch * inner : outer * inner * inner);
+        RANGE(Y, 0, outer * inner);
+        HIPCHK(k_channel_max(s, X->dt(), (size_t)outer, (int)ch, (int)inner, X->ptr, Y->ptr, idx, across));
+        m_mem.touch((long)pl[5]);
+        return 0;
+    }
+    case MCH_FN_CHANNEL_SUB:
+    case MCH_FN_CHANNEL_DIV: {
+        // 291 l{count,outer,channels,inner,hX,hY[,hA]}: y[n,c,s] = a[n,c,s] - x[n,s], a = y when absent (device.cu:3438-3457)
+        // 293 l{count,outer,channels,inner,hX,hY[,method]}: y[n,c,s] /= x[n,s]; method 2 is the same division walked
+        //     from the (n, s) side with count = outer * inner (device.cu:3541-3560, math.cu:7160-7204)
+        NEED_L(6, 7);
+        const bool sub = fn == MCH_FN_CHANNEL_SUB;
+        long long count = pl[0];
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        if (count < 0 || outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (!sub && ll > 6 && pl[6] == 2) count *= ch;
+        if (count > outer * ch * inner) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *Y, *A = nullptr;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (sub && ll > 6) ERRCHK(mem((long)pl[6], &A));
+        if (X->half != Y->half || (A && A->half != Y->half)) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, outer * inner);
+        RANGE(Y, 0, count);
+        if (A) RANGE(A, 0, count);
+        if (sub) HIPCHK(k_channel_sub(s, Y->dt(), (size_t)count, (int)ch, (int)inner, A ? A->ptr : Y->ptr, X->ptr, Y->ptr));
+        else HIPCHK(k_channel_div(s, Y->dt(), (size_t)count, (int)ch, (int)inner, X->ptr, Y->ptr));
+        m_mem.touch((long)pl[5]);
+        return 0;
+    }
+    case MCH_FN_CHANNEL_DOT: {
+        // l{count,outer,channels,inner,hX,hA,hY}: y[n,s] = sum_c x[n,c,s] a[n,c,s] (device.cu:3638-3654, math.cu:7335-7351)
+        NEED_L(7, 7);
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *A, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &A));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (X->half != A->half || X->half != Y->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (Y->ptr == X->ptr || Y->ptr == A->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, outer * ch * inner);
+        RANGE(A, 0, outer * ch * inner);
+        RANGE(Y, 0, outer * inner);
+        HIPCHK(k_channel_dot(s, X->dt(), (size_t)outer, (int)ch, (int)inner, X->ptr, A->ptr, Y->ptr));
+        m_mem.touch((long)pl[6]);
+        return 0;
+    }
     case MCH_FN_CHANNEL_SUM:
     case MCH_FN_CHANNEL_SUM2: {
         // 292 l{count,outer,channels,inner,hX,hY}: y[outer,inner] = sum over the channels (CudaDnn.cs:9182-9188,
@@ -1861,7 +1946,7 @@ long Kernel::create_extension(long kernelIdx, MCH_TCHAR* path, float** ppOut, MC
     long e = init(self_handle(), (MCH_LONG)kernelIdx);
     if (e) { dlclose(lib); return e; }
     long h;
-    ERRCHK(m_ext.create(&h));
+    if ((e = m_ext.create(&h))) { dlclose(lib); return e; }
     ExtensionState* st = m_ext.get(h);
     st->lib = lib;
     st->fnInvoke = inv;
@@ -1882,7 +1967,7 @@ long Kernel::create_blobloader(MCH_TCHAR* path, float** ppOut, MCH_LONG* plOut)
     void* m = mmap(nullptr, (size_t)sb.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
     if (m == MAP_FAILED) { close(fd); last_detail = "cannot map " + p; return MCH_ERROR_WIN_FILE_NOT_FOUND; }
     long h;
-    ERRCHK(m_blobLoader.create(&h));
+    if (long e = m_blobLoader.create(&h)) { munmap(m, (size_t)sb.st_size); close(fd); return e; }
     BlobLoaderState* st = m_blobLoader.get(h);
     st->fd = fd; st->data = (const unsigned char*)m; st->fileSize = (size_t)sb.st_size;
     return set_out((float)h, ppOut, plOut);
@@ -2059,7 +2144,45 @@ static Kernel* kernel_at(long idx)
     return g_kernels[idx];
 }
 
-static long invoke(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, MCH_TCHAR* szIn, float** ppOut,
+// ---------------------------------------------------------------------------
+// Call trace, the counterpart of the reference's _TRACEAPI build (CudaDnnDLL/Cuda Files/main.cu:44-55): with the
+// environment variable MYCAFFE_HIP_TRACE set, every dispatched call appends one line
+//   FLOAT calling CudaDnnDLL FunctionID (220) CUDA_FN_GEMM kernel 1 floats 2 longs 10 -> 0
+// to stderr (value "1" or "stderr") or to the file the variable names.  Off (one pointer test per call) otherwise.
+static const char* api_name(long fn)
+{
+#define N(x) {MCH_FN_##x, "CUDA_FN_" #x}
+    static const struct { long id; const char* name; } table[] = {
+        {MCH_DLL_FREEMEM, "CUDA_DLL_FREEMEM"}, {MCH_DLL_INITIALIZE, "CUDA_DLL_INITIALIZE"}, {MCH_DLL_CLEANUP, "CUDA_DLL_CLEANUP"},
+        N(SETDEVICE), N(GETDEVICE), N(SYNCHRONIZEDEVICE), N(CREATE_MEMORYPOINTER), N(FREE_MEMORYPOINTER), N(ALLOCMEM_HALF), N(ALLOCMEM), N(FREEMEM), N(GETMEM), N(SETMEM), N(CREATE_CUDNN), N(FREE_CUDNN), N(CREATE_TENSORDESC), N(FREE_TENSORDESC), N(SET_TENSORDESC), N(CREATE_EXTENSION), N(FREE_EXTENSION), N(EXTENSION_RUN), N(SOFTMAX_FWD), N(SOFTMAX_BWD), N(ATTN_CREATE), N(ATTN_FREE), N(ATTN_SET), N(ATTN_FWD), N(ATTN_BWD), N(SET), N(COPY), N(GEMM2), N(GEMM), N(GEMV), N(AXPY), N(SCAL), N(SCALE), N(ADD_SCALAR), N(ADD), N(SUB), N(MUL), N(DIV), N(EXP), N(LOG), N(POWX), N(SQRT), N(TRANSPOSE), N(MASK), N(MASK_BATCH), N(TRANSPOSE_HW), N(INVERT), N(CHANNEL_MEAN), N(CHANNEL_MAX), N(CHANNEL_SUB), N(CHANNEL_SUM), N(CHANNEL_DIV), N(CHANNEL_DOT), N(CHANNEL_COPY), N(CHANNEL_FILLFROM), N(CHANNEL_COPYALL), N(CHANNEL_DUP), N(CHANNEL_SUM2), N(EMBED_FWD), N(RELU_FWD), N(RELU_BWD), N(GELU_FWD), N(GELU_BWD), N(SILU_FWD), N(SILU_BWD), N(CREATE_LAYERNORM), N(FREE_LAYERNORM), N(LAYERNORM_FWD), N(LAYERNORM_BWD), N(CREATE_ROPE), N(FREE_ROPE), N(ROPE_FWD), N(ROPE_BWD), N(CREATE_BLOBLOADER), N(FREE_BLOBLOADER), N(BLOBLOADER_LOAD), N(BLOBLOADER_RESETOFFSET), N(BLOBLOADER_ADDTOOFFSET), N(ATTN_DECODE_FWD), N(RMSNORM_FWD), N(SWIGLU_FWD), N(QKV_PROJ_HEADS)};
+#undef N
+    for (const auto& t : table)
+        if (t.id == fn) return t.name;
+    return "(not dispatched)";
+}
+
+static FILE* trace_file()
+{
+    static FILE* f = []() -> FILE* {
+        const char* v = getenv("MYCAFFE_HIP_TRACE");
+        if (!v || !*v || !strcmp(v, "0")) return nullptr;
+        if (!strcmp(v, "1") || !strcmp(v, "stderr")) return stderr;
+        return fopen(v, "a");
+    }();
+    return f;
+}
+
+static void trace_call(long kIdx, long fn, long lf, long ll, long rc)
+{
+    FILE* f = trace_file();
+    if (!f) return;
+    static std::mutex lock;
+    std::lock_guard<std::mutex> g(lock);
+    fprintf(f, "FLOAT calling CudaDnnDLL FunctionID (%ld) %s kernel %ld floats %ld longs %ld -> %ld\n", fn, api_name(fn), kIdx, lf, ll, rc);
+    fflush(f);
+}
+
+static long invoke_untraced(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, MCH_TCHAR* szIn, float** ppOut,
                    MCH_LONG* plOut, MCH_TCHAR* szErr, long errMax, bool ex)
 {
     if (szErr && errMax > 0) szErr[0] = 0;
@@ -2119,6 +2242,14 @@ static long invoke(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, lon
     }
     if (e) put_error(k, e, szErr, errMax);
     return e;
+}
+
+static long invoke(long kIdx, long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, MCH_TCHAR* szIn, float** ppOut,
+                   MCH_LONG* plOut, MCH_TCHAR* szErr, long errMax, bool ex)
+{
+    const long rc = invoke_untraced(kIdx, fn, pf, lf, pl, ll, szIn, ppOut, plOut, szErr, errMax, ex);
+    if (trace_file()) trace_call(kIdx, fn, lf, ll, rc);
+    return rc;
 }
 
 }  // namespace mch

@@ -70,6 +70,8 @@ class CUDAFN:
     CUDA_SUB = 230
     CUDA_MUL = 231
     CUDA_DIV = 233
+    CUDA_EXP = 235
+    CUDA_LOG = 236
     CUDA_POWX = 237
     CUDA_SQRT = 239
     CUDA_TRANSPOSE = 261
@@ -78,7 +80,11 @@ class CUDAFN:
     CUDA_TRANSPOSE_HW = 267
     CUDA_INVERT = 273
     CUDA_CHANNEL_MEAN = 287
+    CUDA_CHANNEL_MAX = 290
+    CUDA_CHANNEL_SUB = 291
     CUDA_CHANNEL_SUM = 292
+    CUDA_CHANNEL_DIV = 293
+    CUDA_CHANNEL_DOT = 294
     CUDA_CHANNEL_COPY = 300
     CUDA_CHANNEL_FILLFROM = 301
     CUDA_CHANNEL_COPYALL = 302
@@ -502,6 +508,32 @@ class CudaDnn:
     def channel_mean(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff=0):
         """CudaDnn.cs:9030-9036."""
         self._ex2(CUDAFN.CUDA_CHANNEL_MEAN, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nXOff])
+
+    def exp(self, n, hA, hY, nAOff=0, nYOff=0, dfBeta=1.0):
+        """CudaDnn.cs:8332-8338: y = exp(beta a)."""
+        self._ex2(CUDAFN.CUDA_EXP, [dfBeta], [n, hA, hY, nAOff, nYOff, 0])
+
+    def log(self, n, hA, hY, dfBeta=1.0, dfAlpha=0.0):
+        """CudaDnn.cs:8365-8371: y = log(beta (a + alpha))."""
+        self._ex2(CUDAFN.CUDA_LOG, [dfBeta, dfAlpha], [n, hA, hY, 0, 0])
+
+    def channel_max(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, bReturnIdx=False, bAcrossChannels=True):
+        """CudaDnn.cs:9012-9018."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_MAX, None,
+                  [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, 1 if bReturnIdx else 0, 1 if bAcrossChannels else 0])
+
+    def channel_sub(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, hA=None):
+        """CudaDnn.cs:9131-9154: y = a - x (x broadcast over the channels); a = y when absent."""
+        rgl = [nCount, nOuterNum, nChannels, nInnerNum, hX, hY] + ([hA] if hA is not None else [])
+        self._ex2(CUDAFN.CUDA_CHANNEL_SUB, None, rgl)
+
+    def channel_div(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nMethod=1):
+        """CudaDnn.cs:9223-9229."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_DIV, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hY, nMethod])
+
+    def channel_dot(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hA, hY):
+        """CudaDnn.cs:9295-9301."""
+        self._ex2(CUDAFN.CUDA_CHANNEL_DOT, None, [nCount, nOuterNum, nChannels, nInnerNum, hX, hA, hY])
 
     def channel_sum(self, nCount, nOuterNum, nChannels, nInnerNum, hX, hY):
         """CudaDnn.cs:9182-9188: y[outer, inner] = sum over the channels."""

@@ -235,15 +235,55 @@ class TransposeLayer:
 
 
 class SoftmaxLayer:
-    """MyCaffe/layers/SoftmaxLayer.cs:172-181, 339-345 (cuDNN engine)."""
+    """MyCaffe/layers/SoftmaxLayer.cs: the cuDNN engine (:172-181, 339-367) or, with ``engine="CAFFE"``, the chain of
+    primitives of forward_cuda / backward_cuda (:230-330; ``algorithm="LOG"`` for the log-softmax variant)."""
 
-    def __init__(self, cuda, axis=-1):
-        self.cuda, self.axis = cuda, axis
+    def __init__(self, cuda, axis=-1, engine="CUDNN", algorithm="ACCURATE"):
+        self.cuda, self.axis, self.engine, self.algorithm = cuda, axis, engine, algorithm
         self.hCudnn = cuda.CreateCuDNN()
         self.hBottomDesc = cuda.CreateTensorDesc()
         self.hTopDesc = cuda.CreateTensorDesc()
+        self.blobScale = None
+
+    def _forward_caffe(self, bottom, top):
+        """SoftmaxLayer.cs:230-273."""
+        cuda = self.cuda
+        axis = self.axis % bottom.num_axes
+        nOuter, nCh, nInner = bottom.count(0, axis), bottom.shape(axis), bottom.count(axis + 1)
+        top.ReshapeLike(bottom)
+        if self.blobScale is None or self.blobScale.count() != nOuter * nInner or self.blobScale.half != bottom.half:
+            self.blobScale = Blob(cuda, (nOuter, nInner), bottom.half)
+        self._dims = (nOuter, nCh, nInner)
+        hB, hT, hSd, hSf = bottom.gpu_data, top.gpu_data, self.blobScale.gpu_data, self.blobScale.gpu_diff
+        n = bottom.count()
+        cuda.copy(n, hB, hT)
+        cuda.channel_max(nOuter * nInner, nOuter, nCh, nInner, hT, hSd)
+        cuda.channel_sub(n, nOuter, nCh, nInner, hSd, hT)
+        cuda.exp(n, hT, hT)
+        cuda.channel_sum(nOuter * nInner, nOuter, nCh, nInner, hT, hSf)
+        if self.algorithm == "LOG":
+            cuda.log(nOuter * nInner, hSf, hSf)
+            cuda.add(nOuter * nInner, hSd, hSf, hSd)
+            cuda.copy(n, hB, hT)
+            cuda.channel_sub(n, nOuter, nCh, nInner, hSd, hT)
+        else:
+            cuda.channel_div(n, nOuter, nCh, nInner, hSf, hT)
+
+    def _backward_caffe(self, top, bottom):
+        """SoftmaxLayer.cs:289-330 (the ACCURATE branch: inner1d(top_diff, top_data), subtract, multiply)."""
+        cuda = self.cuda
+        nOuter, nCh, nInner = self._dims
+        n = top.count()
+        if self.algorithm == "LOG":
+            raise NotImplementedError("log-softmax gradient chain (channel_fillfrom over a reshaped scale blob)")
+        cuda.copy(n, top.gpu_diff, bottom.gpu_diff)
+        cuda.channel_dot(nOuter * nInner, nOuter, nCh, nInner, top.gpu_diff, top.gpu_data, self.blobScale.gpu_data)
+        cuda.channel_sub(n, nOuter, nCh, nInner, self.blobScale.gpu_data, bottom.gpu_diff)
+        cuda.mul(n, bottom.gpu_diff, top.gpu_data, bottom.gpu_diff)
 
     def Forward(self, bottom, top):
+        if self.engine == "CAFFE":
+            return self._forward_caffe(bottom, top)
         axis = self.axis % bottom.num_axes
         nN, nK, nH = bottom.count(0, axis), bottom.shape(axis), bottom.count(axis + 1)
         mode = SOFTMAX_MODE.INSTANCE if nH == 1 else SOFTMAX_MODE.CHANNEL
@@ -256,6 +296,8 @@ class SoftmaxLayer:
 
     def Backward(self, top, bottom):
         """SoftmaxLayer.cs:359-367: bottom.diff from top.data and top.diff (descriptors as set by Forward)."""
+        if self.engine == "CAFFE":
+            return self._backward_caffe(top, bottom)
         self.cuda.SoftmaxBackward(self.hCudnn, SOFTMAX_ALGORITHM.ACCURATE, self._mode, 1.0, self.hTopDesc, top.gpu_data, self.hTopDesc,
                                   top.gpu_diff, 0.0, self.hBottomDesc, bottom.gpu_diff)
 

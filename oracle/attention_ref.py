@@ -183,6 +183,49 @@ def softmax_backward(y, dy, axis=-1, log=False, dtype=np.float32):
     return ((dy - (dy * y).sum(axis=axis, keepdims=True)) * y).astype(dtype)
 
 
+def channel_max(x, num, channels, spatial, return_idx=False, across=True, dtype=np.float32):
+    """channel_max kernels (math.cu:6697-6778).  across: y[n, s] = max_c x[n, c, s] (or the first index of it);
+    within a channel the kernel walks num * spatial rows of `spatial` values: y[i] = max_j x[i * spatial + j]."""
+    x = np.asarray(x, dtype).reshape(-1)
+    if across:
+        v = x[:num * channels * spatial].reshape(num, channels, spatial)
+        return (np.argmax(v, axis=1).astype(dtype) if return_idx else v.max(axis=1)).reshape(-1)
+    v = x[:num * spatial * spatial].reshape(num * spatial, spatial)
+    return np.argmax(v, axis=1).astype(dtype) if return_idx else v.max(axis=1)
+
+
+def channel_sub(a, x, num, channels, spatial, dtype=np.float32):
+    """channel_sub_kernel (math.cu:6908-6916): y[n, c, s] = a[n, c, s] - x[n, s]."""
+    return (np.asarray(a, dtype).reshape(num, channels, spatial) - np.asarray(x, dtype).reshape(num, 1, spatial)).reshape(-1)
+
+
+def channel_div(y, x, num, channels, spatial, dtype=np.float32):
+    """channel_div_kernel (math.cu:7160-7168): y[n, c, s] /= x[n, s]."""
+    return (np.asarray(y, dtype).reshape(num, channels, spatial) / np.asarray(x, dtype).reshape(num, 1, spatial)).reshape(-1)
+
+
+def channel_dot(x, a, num, channels, spatial, dtype=np.float32):
+    """channel_dot_kernel (math.cu:7335-7351): y[n, s] = sum_c x[n, c, s] a[n, c, s], accumulated in double."""
+    v = np.asarray(x, np.float64).reshape(num, channels, spatial) * np.asarray(a, np.float64).reshape(num, channels, spatial)
+    return v.sum(axis=1).astype(dtype).reshape(-1)
+
+
+def softmax_caffe_chain(x, axis, log=False, dtype=np.float32):
+    """SoftmaxLayer.forward_cuda (SoftmaxLayer.cs:230-273) step by step on the primitives above."""
+    x = np.asarray(x, dtype)
+    axis %= x.ndim
+    num, ch, sp = int(np.prod(x.shape[:axis], dtype=np.int64)), x.shape[axis], int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    top = x.reshape(-1).copy()
+    c = channel_max(top, num, ch, sp, dtype=dtype)
+    top = channel_sub(top, c, num, ch, sp, dtype)
+    top = np.exp(top).astype(dtype)
+    ssum = top.reshape(num, ch, sp).sum(axis=1).reshape(-1)
+    if log:
+        logz = c + np.log(ssum).astype(dtype)
+        return channel_sub(x.reshape(-1), logz, num, ch, sp, dtype).reshape(x.shape)
+    return channel_div(top, ssum, num, ch, sp, dtype).reshape(x.shape)
+
+
 def silu(x, dtype=np.float32):
     """x * sigmoid(x) (math.cu:11699-11707)."""
     x = np.asarray(x, dtype)

@@ -98,3 +98,30 @@ def test_uninitialised_kernel_and_bad_index_codes():
 def test_utf16_round_trip_helpers():
     buf = C._utf16("model.bin;tokenizer.bin é中")
     assert C._from_utf16(buf) == "model.bin;tokenizer.bin é中"
+
+
+def test_call_trace_names_the_function(tmp_path):
+    # MYCAFFE_HIP_TRACE=<file>: one line per dispatched call in the reference's _TRACEAPI wording (main.cu:44-55);
+    # the variable is read once per process, so the traced calls run in a child process (no device needed: the
+    # call fails on an uninitialised kernel and is traced all the same)
+    import subprocess
+    import sys
+    log = tmp_path / "trace.txt"
+    code = (
+        "import ctypes, numpy as np\n"
+        "from mycaffe_amd import cudadnn as C\n"
+        "lib = C.load_library()\n"
+        "err = (ctypes.c_uint16 * 256)()\n"
+        "out = (ctypes.c_float * 4)()\n"
+        "pout = ctypes.cast(out, ctypes.POINTER(ctypes.c_float))\n"
+        "n = ctypes.c_int32(4)\n"
+        "l = np.zeros(10, np.int64)\n"
+        "f = np.zeros(2, np.float32)\n"
+        "rc = lib.DLL_InvokeFloatEx2(77, 220, f.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), 2,\n"
+        "                            l.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), 10, ctypes.byref(pout), ctypes.byref(n), err, 256)\n"
+        "assert rc == C.ERROR.PARAM_NULL, rc\n"
+    )
+    env = dict(os.environ, MYCAFFE_HIP_TRACE=str(log), PYTHONPATH=ROOT)
+    subprocess.run([sys.executable, "-c", code], check=True, env=env, cwd=ROOT)
+    text = log.read_text()
+    assert "FLOAT calling CudaDnnDLL FunctionID (220) CUDA_FN_GEMM kernel 77 floats 2 longs 10 -> 90002" in text

@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from mycaffe_amd.cudadnn import CudaDnnError, DIR, ERROR, SOFTMAX_ALGORITHM, SOFTMAX_MODE
+from mycaffe_amd.layers import Blob, SoftmaxLayer
 from oracle import attention_ref as R
 from tests.conftest import BF16_RTOL, FP32_RTOL, GOLDEN, assert_close, bf16_round
 
@@ -728,3 +729,73 @@ def test_in_place_mask_is_held_back_for_the_softmax_without_changing_any_result(
         assert_close(dev.get(h, x.shape), a[0, 0].astype(np.float64) @ b[0, 0].astype(np.float64), FP32_RTOL, "overwritten")
     cuda.FreeTensorDesc(d)
     cuda.FreeCuDNN(hc)
+
+
+# ---- CAFFE-engine softmax chain: exp, log, channel_max / sub / div / dot ----------------------
+
+@pytest.mark.parametrize("half", [False, True])
+def test_channel_primitives_of_the_softmax_chain(dev, half):
+    rng = np.random.default_rng(3)
+    num, ch, sp = 5, 37, 19
+    x = bf16_round(rng.standard_normal((num, ch, sp)).astype(np.float32))
+    a = bf16_round(rng.standard_normal((num, ch, sp)).astype(np.float32))
+    r = bf16_round((rng.random((num, sp)) + 0.5).astype(np.float32))
+    tol = BF16_RTOL if half else 1e-6
+    hx, ha, hr = dev.put(x, half), dev.put(a, half), dev.put(r, half)
+    hy, hfull = dev.zeros(num * sp, half), dev.zeros(x.size, half)
+    n, full = num * sp, x.size
+    dev.cuda.channel_max(n, num, ch, sp, hx, hy)
+    assert np.array_equal(dev.get(hy), R.channel_max(x, num, ch, sp))
+    dev.cuda.channel_max(n, num, ch, sp, hx, hy, True)
+    assert np.array_equal(dev.get(hy), R.channel_max(x, num, ch, sp, return_idx=True))
+    dev.cuda.channel_max(n, num, 1, sp, hx, hy, False, False)                      # within-channel index rule
+    assert np.array_equal(dev.get(hy), R.channel_max(x, num, 1, sp, across=False))
+    dev.cuda.channel_sub(full, num, ch, sp, hr, hfull, ha)
+    assert_close(dev.get(hfull), R.channel_sub(a, r, num, ch, sp), tol, "channel_sub a - x")
+    dev.cuda.copy(full, hx, hfull)
+    dev.cuda.channel_sub(full, num, ch, sp, hr, hfull)
+    assert_close(dev.get(hfull), R.channel_sub(x, r, num, ch, sp), tol, "channel_sub in place")
+    for method, count in ((1, full), (2, n)):
+        dev.cuda.copy(full, hx, hfull)
+        dev.cuda.channel_div(count, num, ch, sp, hr, hfull, method)
+        assert_close(dev.get(hfull), R.channel_div(x, r, num, ch, sp), tol, "channel_div method %d" % method)
+    dev.cuda.channel_dot(n, num, ch, sp, hx, ha, hy)
+    assert_close(dev.get(hy), R.channel_dot(x, a, num, ch, sp), BF16_RTOL if half else 1e-5, "channel_dot")
+    dev.cuda.exp(full, hx, hfull, 0, 0, 0.5)
+    assert_close(dev.get(hfull), np.exp(0.5 * x.astype(np.float64)).reshape(-1), tol, "exp")
+    dev.cuda.log(n, hr, hy, 2.0, 0.25)
+    assert_close(dev.get(hy), np.log(2.0 * (r.astype(np.float64) + 0.25)).reshape(-1), tol, "log")
+
+
+@pytest.mark.parametrize("shape,axis", [((6, 50), -1), ((3, 4, 64, 64), -1), ((4, 9, 33), 1)])
+@pytest.mark.parametrize("algorithm", ["ACCURATE", "LOG"])
+def test_softmax_layer_caffe_engine_chain(dev, shape, axis, algorithm):
+    """SoftmaxLayer with engine CAFFE (SoftmaxLayer.cs:230-330): forward against scipy and against the cuDNN-engine
+    call (id 111), gradient of the ACCURATE form against the softmax gradient id (112)."""
+    from scipy.special import log_softmax, softmax
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    outs = {}
+    for engine in ("CAFFE", "CUDNN"):
+        if engine == "CUDNN" and algorithm == "LOG":
+            continue
+        layer = SoftmaxLayer(dev.cuda, axis, engine, algorithm)
+        bottom, top = Blob(dev.cuda, shape), Blob(dev.cuda)
+        bottom.mutable_cpu_data = x
+        layer.Forward(bottom, top)
+        y = top.mutable_cpu_data.copy()
+        dx = None
+        if algorithm == "ACCURATE":
+            top.mutable_cpu_diff = dy
+            layer.Backward(top, bottom)
+            dx = bottom.mutable_cpu_diff.copy()
+        outs[engine] = (y, dx)
+    ref = (log_softmax if algorithm == "LOG" else softmax)(x.astype(np.float64), axis=axis)
+    assert_close(outs["CAFFE"][0], ref, FP32_RTOL, "CAFFE-engine forward")
+    assert_close(outs["CAFFE"][0], R.softmax_caffe_chain(x, axis, algorithm == "LOG"), 1e-6, "forward vs the checker's chain")
+    if algorithm == "ACCURATE":
+        assert_close(outs["CAFFE"][0], outs["CUDNN"][0], 1e-6, "CAFFE vs cuDNN engine forward")
+        refdx = R.softmax_backward(ref, dy.astype(np.float64), axis=axis, dtype=np.float64)
+        assert_close(outs["CAFFE"][1], refdx, FP32_RTOL, "CAFFE-engine gradient")
+        assert_close(outs["CAFFE"][1], outs["CUDNN"][1], 1e-5, "CAFFE vs cuDNN engine gradient")

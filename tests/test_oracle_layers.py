@@ -499,3 +499,29 @@ def test_transformer_block_llama_matches_torch_composition():
     want = xb + F.linear(F.silu(F.linear(n2, t["fc_weight"])) * F.linear(n2, t["fc2_weight"]), t["proj_weight"])
     # the table frequencies are rounded to fp32 in the reference (rope.cu:535-553), hence 1e-6 and not 1e-12
     assert np.allclose(got, want.numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ---- CAFFE-engine softmax chain (SoftmaxLayer.cs:230-273) -------------------------------------
+
+def test_channel_primitives_against_numpy_and_a_worked_case():
+    # worked by hand: num 1, channels 3, spatial 2, x[c][s] = [[1, 5], [4, 2], [4, -1]]
+    x = np.array([1, 5, 4, 2, 4, -1], np.float32)
+    assert R.channel_max(x, 1, 3, 2).tolist() == [4, 5]
+    assert R.channel_max(x, 1, 3, 2, return_idx=True).tolist() == [1, 0]          # first maximum wins (strict '>')
+    assert R.channel_sub(x, [1, 2], 1, 3, 2).tolist() == [0, 3, 3, 0, 3, -3]
+    assert R.channel_div(x, [2, 4], 1, 3, 2).tolist() == [0.5, 1.25, 2, 0.5, 2, -0.25]
+    assert R.channel_dot(x, x, 1, 3, 2).tolist() == [33, 30]
+    # within a channel: the kernel's own index rule, num * spatial rows of `spatial` values
+    assert R.channel_max(np.arange(8, dtype=np.float32), 2, 1, 2, across=False).tolist() == [1, 3, 5, 7]
+    rng = np.random.default_rng(0)
+    v = rng.standard_normal((3, 5, 7)).astype(np.float32)
+    assert np.array_equal(R.channel_max(v, 3, 5, 7), v.max(1).reshape(-1))
+    assert np.allclose(R.channel_dot(v, 2 * v, 3, 5, 7), np.einsum("ncs,ncs->ns", v, 2 * v).reshape(-1), rtol=1e-6)
+
+
+@pytest.mark.parametrize("axis", [1, 2, -1])
+def test_softmax_chain_equals_scipy(axis):
+    from scipy.special import log_softmax, softmax
+    x = np.random.default_rng(1).standard_normal((4, 6, 5)).astype(np.float32) * 3
+    assert np.allclose(R.softmax_caffe_chain(x, axis, dtype=np.float64), softmax(x.astype(np.float64), axis=axis), rtol=1e-12)
+    assert np.allclose(R.softmax_caffe_chain(x, axis, log=True, dtype=np.float64), log_softmax(x.astype(np.float64), axis=axis), rtol=1e-10, atol=1e-12)
