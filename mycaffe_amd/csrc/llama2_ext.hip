@@ -108,6 +108,24 @@ template <> struct Row8<bf16_t> {
     }
 };
 
+// The 8 of a 32-column slab's values that lane group kk (0..3) of the matrix-core mat-vec contracts.  Which columns a
+// group takes is free as long as both operands agree, so it is chosen for the loads: with fp32 weights a group takes
+// columns 4 kk .. 4 kk + 3 and 16 + 4 kk .. + 3, so that the four groups of a row read 64 contiguous bytes per load
+// instruction; with bf16 weights a group's 16-byte load holds columns 8 kk .. 8 kk + 7 and x follows that.
+template <typename T> struct Slab8;
+template <> struct Slab8<float> {
+    __device__ static inline void w(const float* slab, int kk, float* o) { x(slab, kk, o); }
+    __device__ static inline void x(const float* slab, int kk, float* o)
+    {
+        const float4 a = *(const float4*)(slab + 4 * kk), b = *(const float4*)(slab + 16 + 4 * kk);
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+};
+template <> struct Slab8<bf16_t> {
+    __device__ static inline void w(const bf16_t* slab, int kk, float* o) { Row8<bf16_t>::load(slab + 8 * kk, o); }
+    __device__ static inline void x(const float* slab, int kk, float* o) { Row8<float>::load(slab + 8 * kk, o); }
+};
+
 // Mat-vec family for one token per sequence.  One wavefront owns ROWS output rows
 // of W (n columns, n % 4 == 0) and walks them with 128-bit (fp32) / 64-bit (bf16)
 // loads; the activation chunk a lane needs is the same for every row, so it is
@@ -298,99 +316,130 @@ __global__ __launch_bounds__(256) void matvec_loop_kernel(const T* __restrict__ 
 // folded into x.  Partial tiles of the wavefronts meet in LDS; wavefront 0 finishes.
 typedef float floatx4v __attribute__((ext_vector_type(4)));
 
-template <typename T, int MODE, bool NORM>
+template <typename T, int MODE, bool NORM, int G = 1>
 __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
                                                           const float* __restrict__ g, float* __restrict__ y, int rows, int n,
-                                                          int B, int ldy, int b0)
+                                                          int B, int ldy, int nGroups)
 {
+    // Workgroups go to the chip's 8 dies round robin by their index, and each die has its own L2: the nGroups
+    // workgroups that walk the same 16 rows of W (one per group of 16 G sequences or prompt rows) are given indices
+    // that are equal modulo 8, so a slab of weights is fetched into one L2 instead of all eight.
+    const int die = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int r0 = ((slot / nGroups) * 8 + die) * 16;
+    const int b0 = (slot % nGroups) * 16 * G;
+    if (r0 >= rows) return;   // the grid is padded to a multiple of 8 row tiles
+    // G groups of 16 sequences (or prompt rows) per pass: a slab of weights is loaded once and multiplied into all of
+    // them, so up to 128 rows of x share one walk over W (the batched prompt pass of a single sequence)
     __shared__ float part[8][(MODE == 2 ? 2 : 1) * 256];
     __shared__ float sspart[8][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NS = blockDim.x >> 6;
     const int i = lane & 15, kk = lane >> 4;
-    const int r0 = blockIdx.x * 16;
-    const T* wr = W + (size_t)min(r0 + i, rows - 1) * n + kk * 8;
-    const bool jv = b0 + i < B;                 // this lane's batch column exists
-    const float* xr = x + (size_t)min(b0 + i, B - 1) * n + kk * 8;
-    floatx4v acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-    float ss = 0.f;
+    const T* wr = W + (size_t)min(r0 + i, rows - 1) * n;
+    bool jv[G];                                 // this lane's batch column exists
+    const float* xr[G];
+#pragma unroll
+    for (int q = 0; q < G; q++) {
+        jv[q] = b0 + 16 * q + i < B;
+        xr[q] = x + (size_t)min(b0 + 16 * q + i, B - 1) * n;
+    }
+    floatx4v acc[G], acc2[MODE == 2 ? G : 1];
+    float ss[G];
+#pragma unroll
+    for (int q = 0; q < G; q++) {
+        acc[q] = floatx4v{0.f, 0.f, 0.f, 0.f};
+        if (MODE == 2) acc2[MODE == 2 ? q : 0] = floatx4v{0.f, 0.f, 0.f, 0.f};
+        ss[q] = 0.f;
+    }
     // the residual epilogue's old values (wavefront 0 finishes the tile) are requested with the first weights
-    float prev[4] = {0.f, 0.f, 0.f, 0.f};
-    if (MODE == 1 && wave == 0 && jv) {
+    float prev[G][4];
+#pragma unroll
+    for (int q = 0; q < G; q++)
 #pragma unroll
         for (int v = 0; v < 4; v++)
-            if (r0 + 4 * kk + v < rows) prev[v] = y[(size_t)(b0 + i) * ldy + r0 + 4 * kk + v];
-    }
+            prev[q][v] = (MODE == 1 && wave == 0 && jv[q] && r0 + 4 * kk + v < rows) ? y[(size_t)(b0 + 16 * q + i) * ldy + r0 + 4 * kk + v] : 0.f;
     const int nit = n >> 5;
-    constexpr int U = 4;   // slabs whose loads are in flight together
+    constexpr int U = G == 1 ? 4 : 2;   // slabs whose loads are in flight together
     for (int base = wave; base < nit; base += NS * U) {
-        float w[U][8], w2[MODE == 2 ? U : 1][8], xv[U][8], gv[NORM ? U : 1][8];
+        float w[U][8], w2[MODE == 2 ? U : 1][8], gv[NORM ? U : 1][8];
 #pragma unroll
         for (int t = 0; t < U; t++) {
             const int k0 = min(base + t * NS, nit - 1) << 5;   // past the end: re-read the last slab, not used
-            Row8<T>::load(wr + k0, w[t]);
-            if (MODE == 2) Row8<T>::load(wr + (size_t)rows * n + k0, w2[MODE == 2 ? t : 0]);
-            Row8<float>::load(xr + k0, xv[t]);
-            if (NORM) Row8<float>::load(g + kk * 8 + k0, gv[NORM ? t : 0]);
+            Slab8<T>::w(wr + k0, kk, w[t]);
+            if (MODE == 2) Slab8<T>::w(wr + (size_t)rows * n + k0, kk, w2[MODE == 2 ? t : 0]);
+            if (NORM) Slab8<T>::x(g + k0, kk, gv[NORM ? t : 0]);
         }
 #pragma unroll
-        for (int t = 0; t < U; t++) {
-            if (base + t * NS >= nit) break;
-            if (NORM) {
+        for (int q = 0; q < G; q++) {
+            float xv[U][8];
+#pragma unroll
+            for (int t = 0; t < U; t++) Slab8<T>::x(xr[q] + (min(base + t * NS, nit - 1) << 5), kk, xv[t]);
+#pragma unroll
+            for (int t = 0; t < U; t++) {
+                if (base + t * NS >= nit) break;
+                if (NORM) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        ss[q] += xv[t][e] * xv[t][e];
+                        xv[t][e] *= gv[NORM ? t : 0][e];
+                    }
+                }
+                if (!jv[q]) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) xv[t][e] = 0.f;
+                }
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    ss += xv[t][e] * xv[t][e];
-                    xv[t][e] *= gv[NORM ? t : 0][e];
+                    acc[q] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[t][e], xv[t][e], acc[q], 0, 0, 0);
+                    if (MODE == 2)
+                        acc2[MODE == 2 ? q : 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w2[MODE == 2 ? t : 0][e], xv[t][e], acc2[MODE == 2 ? q : 0], 0, 0, 0);
                 }
             }
-            if (!jv) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) xv[t][e] = 0.f;
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[t][e], xv[t][e], acc, 0, 0, 0);
-                if (MODE == 2) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(w2[MODE == 2 ? t : 0][e], xv[t][e], acc2, 0, 0, 0);
-            }
         }
     }
-    if (NORM) {
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        if (kk == 0) sspart[wave][i] = ss;
-    }
+    // the wavefronts' partial tiles meet in LDS one group at a time; wavefront 0 finishes each
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-        part[wave][lane * 4 + v] = acc[v];
-        if (MODE == 2) part[wave][256 + lane * 4 + v] = acc2[v];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-    // accumulator register v of lane l is row 4 * (l / 16) + v, batch column l % 16
-    float d[4], d2[4];
-#pragma unroll
-    for (int v = 0; v < 4; v++) {
-        d[v] = 0.f;
-        d2[v] = 0.f;
-        for (int w_ = 0; w_ < NS; w_++) {
-            d[v] += part[w_][lane * 4 + v];
-            if (MODE == 2) d2[v] += part[w_][256 + lane * 4 + v];
+    for (int q = 0; q < G; q++) {
+        if (q > 0) __syncthreads();   // wavefront 0 has read the previous group's partials
+        if (NORM) {
+            float t = ss[q];
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            if (kk == 0) sspart[wave][i] = t;
         }
-    }
-    if (!jv) return;
-    float inv = 1.f;
-    if (NORM) {
-        float t = 0.f;
-        for (int w_ = 0; w_ < NS; w_++) t += sspart[w_][i];
-        inv = 1.0f / sqrtf(t / n + 1e-5f);
-    }
-    float* out = y + (size_t)(b0 + i) * ldy + r0 + 4 * kk;
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-        if (r0 + 4 * kk + v >= rows) break;
-        const float a0 = d[v] * inv;
-        if (MODE == 0) out[v] = a0;
-        else if (MODE == 1) out[v] = prev[v] + a0;
-        else out[v] = a0 * (1.0f / (1.0f + expf(-a0))) * (d2[v] * inv);
+        for (int v = 0; v < 4; v++) {
+            part[wave][lane * 4 + v] = acc[q][v];
+            if (MODE == 2) part[wave][256 + lane * 4 + v] = acc2[MODE == 2 ? q : 0][v];
+        }
+        __syncthreads();
+        if (wave != 0) continue;
+        // accumulator register v of lane l is row 4 * (l / 16) + v, batch column l % 16
+        float d[4], d2[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            d[v] = 0.f;
+            d2[v] = 0.f;
+            for (int w_ = 0; w_ < NS; w_++) {
+                d[v] += part[w_][lane * 4 + v];
+                if (MODE == 2) d2[v] += part[w_][256 + lane * 4 + v];
+            }
+        }
+        if (!jv[q]) continue;
+        float inv = 1.f;
+        if (NORM) {
+            float t = 0.f;
+            for (int w_ = 0; w_ < NS; w_++) t += sspart[w_][i];
+            inv = 1.0f / sqrtf(t / n + 1e-5f);
+        }
+        float* out = y + (size_t)(b0 + 16 * q + i) * ldy + r0 + 4 * kk;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            if (r0 + 4 * kk + v >= rows) break;
+            const float a0 = d[v] * inv;
+            if (MODE == 0) out[v] = a0;
+            else if (MODE == 1) out[v] = prev[q][v] + a0;
+            else out[v] = a0 * (1.0f / (1.0f + expf(-a0))) * (d2[v] * inv);
+        }
     }
 }
 
@@ -564,9 +613,28 @@ __global__ __launch_bounds__(256) void prefill_argmax_kernel(const float* __rest
     const float* lg = logits + (size_t)blockIdx.x * V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += 256) {
-        const float v = lg[i];
+    auto take = [&](float v, int i) {
         if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    };
+    if ((V & 3) == 0 && (((uintptr_t)lg) & 15) == 0) {
+        // 16 bytes per lane, eight loads in flight
+        const int n4 = V >> 2;
+        constexpr int U = 8;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += 256 * U) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = i0 + u * 256;
+                v[u] = i < n4 ? *(const float4*)(lg + (size_t)i * 4) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = (i0 + u * 256) * 4;
+                take(v[u].x, i); take(v[u].y, i + 1); take(v[u].z, i + 2); take(v[u].w, i + 3);
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += 256) take(lg[i], i);
     }
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(bv, o, 64);
@@ -963,6 +1031,9 @@ long Engine::ensure_state(int B, int nSteps)
     return 0;
 }
 
+template <int MODE, bool NORM, typename T>
+static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy);
+
 long Engine::ensure_prefill(size_t rows)
 {
     if (rows <= pfRows) return 0;
@@ -1013,10 +1084,24 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
     auto grid_for = [](size_t items) { return (int)std::min<size_t>((items + 255) / 256, 8192); };
     hipLaunchKernelGGL(prefill_embed_kernel<T>, (int)M, 256, 0, s, dprompt, cfg.seq_len, P, (const T*)emb, pfX, dim);
     HIPCHK(hipGetLastError());
+    // Few rows (one or two sequences' prompts): the fused mat-vec family on the matrix cores, all rows sharing one walk
+    // over each matrix, norms / SwiGLU / residuals in its epilogues.  Many rows: 128 x 128-tile GEMMs.
+    const bool skinny = M <= 256 && dim % 32 == 0 && hid % 32 == 0;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
         float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
         float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
+        if (skinny) {
+            HIPCHK((launch_matvec_rows<0, true, T>(s, w.wqkv, pfX, w.rms_att, pfQkv, ldq, dim, (int)M, ldq)));
+            hipLaunchKernelGGL(prefill_rope_scatter_kernel, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, kcl, vcl, fcos, fsin, B, P,
+                               H, kvH, hs, cfg.seq_len);
+            HIPCHK(hipGetLastError());
+            HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
+            HIPCHK((launch_matvec_rows<1, false, T>(s, w.wo, pfXn, nullptr, pfX, dim, dim, (int)M, dim)));          // x += Wo att
+            HIPCHK((launch_matvec_rows<2, true, T>(s, w.w13, pfX, w.rms_ffn, pfHb, hid, dim, (int)M, hid)));
+            HIPCHK((launch_matvec_rows<1, false, T>(s, w.w2, pfHb, nullptr, pfX, dim, hid, (int)M, dim)));           // x += W2 hb
+            continue;
+        }
         HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_att, pfXn, 1e-5f));
         const float* wqkv = as_f32<T>(s, w.wqkv, (size_t)ldq * dim, &e);
         if (e) return e;
@@ -1024,9 +1109,7 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         hipLaunchKernelGGL(prefill_rope_scatter_kernel, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, kcl, vcl, fcos, fsin, B, P,
                            H, kvH, hs, cfg.seq_len);
         HIPCHK(hipGetLastError());
-        HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfY, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL));
-        hipLaunchKernelGGL(prefill_merge_heads_kernel, grid_for(M * dim / 4), 256, 0, s, pfY, pfXn, B, P, H, hs);
-        HIPCHK(hipGetLastError());
+        HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));   // head-merged output
         const float* wo = as_f32<T>(s, w.wo, (size_t)dim * dim, &e);
         if (e) return e;
         HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, dim, 1.f, pfXn, wo, 1.f, pfX));          // x += Wo att
@@ -1040,12 +1123,16 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         if (e) return e;
         HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, hid, 1.f, pfHb, w2, 1.f, pfX));          // x += W2 hb
     }
-    HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
-    const float* wc = as_f32<T>(s, wcls, (size_t)V * dim, &e);
-    if (e) return e;
+    const float* wc = nullptr;
+    if (!skinny) {
+        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
+        wc = as_f32<T>(s, wcls, (size_t)V * dim, &e);
+        if (e) return e;
+    }
     for (size_t r0 = 0; r0 < M; r0 += pfLogitRows) {
         const int rows = (int)std::min(pfLogitRows, M - r0);
-        HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
+        if (skinny) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V)));
+        else HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
         hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
         HIPCHK(hipGetLastError());
         if (allLogits) {
@@ -1073,9 +1160,9 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     if (B >= 2 && n % 32 == 0) {
         // batched: matrix-core kernel, 16 sequences per pass over the weights
         const int ns = rows >= 8192 ? 4 : 8;   // fewer, longer wavefronts once the rows alone fill the chip
-        for (int b0 = 0; b0 < B; b0 += 16) {
-            hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM>), (rows + 15) / 16, ns * 64, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, b0);
-        }
+        // every group of 16 sequences walks the weights in the same launch
+        const int nGroups = (B + 15) / 16, tiles8 = ((rows + 15) / 16 + 7) / 8;
+        hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM>), tiles8 * 8 * nGroups, ns * 64, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
         return hipGetLastError();
     }
     // one row per wavefront fills the chip for the layer matrices; the classifier has rows to spare
@@ -1104,6 +1191,20 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     else hipLaunchKernelGGL((matvec_loop_kernel<T, MODE, NORM>), (rows + 3) / 4, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy);
 #undef MV1
 #undef MV
+    return hipGetLastError();
+}
+
+// The same kernels over the M rows of a prompt pass (row = one position of one sequence): up to 128 rows share one walk
+// over the weights, so a single sequence's prompt streams every matrix once (or a few times) instead of going through
+// 128 x 128 GEMM tiles that would leave most of the chip idle at this height.
+template <int MODE, bool NORM, typename T>
+static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy)
+{
+    const int tiles8 = ((rows + 15) / 16 + 7) / 8;
+    // two groups of 16 rows per workgroup: half the weight traffic from L2 of one group, and still more workgroups than CUs
+#define MVG(G_) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, G_>), tiles8 * 8 * ((M + 16 * G_ - 1) / (16 * G_)), 512, 0, s, (const T*)W, x, g, y, rows, n, M, ldy, (M + 16 * G_ - 1) / (16 * G_))
+    if (M > 16) MVG(2); else MVG(1);
+#undef MVG
     return hipGetLastError();
 }
 
