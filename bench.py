@@ -219,7 +219,8 @@ def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=
                      "roofline": {"kernel": "fused causal attention forward", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s",
                                   "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
-                                  "traffic": recorded_traffic("flash_" + name) if shape == (8, 12, 1024, 64) else None}}
+                                  "traffic": recorded_traffic("flash_" + name if shape == (8, 12, 1024, 64) else
+                                                               "flash_%s_B%d_T%d_%dx%d" % (name, B, T, H, hs))}}
         for h in hs_ + [hy]:
             cuda.FreeMemory(h)
     cuda.FreeMemory(mask)

@@ -237,6 +237,10 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
     constexpr int DT = HS / 32;
     constexpr int PAD = 16 / (int)sizeof(T);
     constexpr int LDK = HS + PAD, LDV = BN + PAD;
+    // Row stride of the row-major V tile.  The transposing read takes 32 contiguous bytes from each of four rows per
+    // 16 lanes, so rows must start 8 banks (32 bytes) apart modulo the bank count: 144 bytes (head size 64) does, 272
+    // (head size 128 with the K padding) puts neighbouring rows 4 banks apart and halves the read rate; 288 does not.
+    constexpr int LDVR = (HS * (int)sizeof(T)) % 256 == 0 ? HS + 2 * PAD : HS + PAD;
     constexpr int CHR = HS / EPC;             // 16-byte chunks per K / V row
     constexpr int KPT = (BN * CHR) / NT;      // K chunks per thread per block
     // 16-bit storage keeps V row-major in LDS, staged exactly like K, and reads the V^T fragments with the transposing
@@ -245,7 +249,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
     constexpr int VPW = VROW ? KPT : CHR / NW;   // V chunks per thread (row-major) / per wavefront, one key per lane (transposed)
     static_assert(KPT >= 1 && VPW >= 1 && (BN * CHR) % NT == 0 && (VROW || CHR % NW == 0), "tile / thread mismatch");
     __shared__ __attribute__((aligned(16))) T Ks[BN * LDK];
-    __shared__ __attribute__((aligned(16))) T Vt[VROW ? BN * LDK : HS * LDV];
+    __shared__ __attribute__((aligned(16))) T Vt[VROW ? BN * LDVR : HS * LDV];
     __shared__ float Ms[BN];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -330,7 +334,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 #pragma unroll
             for (int i = 0; i < VPW; i++) {
                 const int e = tid + i * NT;
-                *(u32x4*)(&Vt[(e / CHR) * LDK + (e % CHR) * EPC]) = vreg[i];
+                *(u32x4*)(&Vt[(e / CHR) * LDVR + (e % CHR) * EPC]) = vreg[i];
             }
         } else {
 #pragma unroll
@@ -438,7 +442,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                 for (int t = 0; t < PF; t++)
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
-                        const u32x4 vf = VROW ? TR::load_vt_rowmajor(&Vt[32 * sub * LDK + dt * 32], LDK, t, lane)
+                        const u32x4 vf = VROW ? TR::load_vt_rowmajor(&Vt[32 * sub * LDVR + dt * 32], LDVR, t, lane)
                                               : TR::load_vt(&Vt[(dt * 32 + l32) * LDV + 32 * sub], t, half);
 #pragma unroll
                         for (int qt = 0; qt < QT; qt++) o[dt][qt] = TR::mma(vf, pf[qt][t], o[dt][qt]);
