@@ -320,7 +320,7 @@ MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, floa
  * split partials and merge tickets come from a fixed device array inside the library (4 MiB + 16 KiB per GPU,
  * held until the process ends) instead of the kernel object's growable workspace, and no hipMalloc, hipFree or
  * other allocating routine is called.  Limits: batch x heads <= 4096 and (batch x heads x splits) x (hs + 2) x 4
- * bytes <= 4 MiB, where splits = min(256, ceil(1024 / (batch x heads))); larger calls return
+ * bytes <= 4 MiB, where splits = ceil(256 / (batch x heads)); larger calls return
  * MCH_ERROR_PARAM_OUT_OF_RANGE.  All calls on one GPU share the array: calls that overlap on one GPU (two kernel
  * objects, two host threads) race, so serialise them. */
 MCH_LONG MCH_AttnDecodeForwardNoAlloc(MCH_LONG lKernelIdx, float* pInput, MCH_LONG lInput, MCH_LONGLONG* plInput,

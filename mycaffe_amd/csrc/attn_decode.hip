@@ -558,11 +558,15 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part, T* __re
     }
 }
 
+// Workgroups a launch aims for: one per CU.  More splits per (batch, head) shorten each workgroup's stream but add
+// partials to store, count and merge, which costs more than it saves from 8 sequences x 32 heads down (measured: 256
+// against 1024 gains up to 20 % at batch 1 and a few per cent at batch 8, and changes nothing at batch 32).
+constexpr int kDecodeTargetWgs = 256;
 static void pick_splits(int B, int H, int len, int rows_per_iter, int* splits, int* chunk)
 {
-    // aim for >= 4 workgroups per CU; never less than one full iteration per split
+    // never less than one full iteration per split
     long long bh = (long long)B * H;
-    int want = (int)((1024 + bh - 1) / bh);
+    int want = (int)((kDecodeTargetWgs + bh - 1) / bh);
     int maxs = (len + rows_per_iter - 1) / rows_per_iter;
     int s = want < 1 ? 1 : want;
     if (s > maxs) s = maxs;
@@ -577,10 +581,10 @@ static void pick_splits(int B, int H, int len, int rows_per_iter, int* splits, i
 
 size_t attn_decode_workspace_bytes(int B, int H, int hs, int len)
 {
-    // pick_splits never asks for more than ceil(1024 / (B*H)) splits (256 at most)
+    // pick_splits never asks for more than ceil(256 / (B*H)) splits
     (void)len;
     long long bh = (long long)B * H;
-    long long want = (1024 + bh - 1) / bh;
+    long long want = (kDecodeTargetWgs + bh - 1) / bh;
     if (want > 256) want = 256;
     if (want < 1) want = 1;
     return (size_t)(bh * want) * (size_t)(hs + 2) * sizeof(float);
