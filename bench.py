@@ -60,13 +60,14 @@ def weight_bytes(cfg, es):
     return (L * ((dim + 2 * kvd) * dim + dim * dim + 3 * hid * dim) + V * dim) * es
 
 
-def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True):
+def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True, kv_bf16=False):
     """Times exactly `steps` greedy decode steps (see the module docstring); returns the engine and the figures."""
     from mycaffe_amd.llm_inference import LlmInference
     inf = LlmInference(cuda)
     inf.Initialize(fTemperature=0.0)
     inf.SetOption(1, 1 if bf16 else 0)
     inf.SetOption(3, 1 if graph else 0)
+    inf.SetOption(8, 1 if kv_bf16 else 0)
     inf.Load(path)
     per_gen = C4["seq_len"] - N_PROMPT - warmup
     left, ms_total, wall, gen = steps, 0.0, 0.0, 0
@@ -625,8 +626,9 @@ def main():
     also["prefill_128_tokens_fp32_b1"] = prefill_summary(head, 1, 4)
     log("prompt pass, batch 1:", json.dumps(also["prefill_128_tokens_fp32_b1"]))
     if want("decode"):
-        for tag, bf16, batch in (("bf16_weights_b1", True, 1), ("fp32_b16", False, 16), ("bf16_weights_b16", True, 16)):
-            i2, r = run_decode(cuda, path, bf16, batch, args.steps, args.warmup, graph=not args.no_graph)
+        for tag, bf16, batch, kv16 in (("bf16_weights_b1", True, 1, False), ("fp32_b16", False, 16, False),
+                                       ("bf16_weights_b16", True, 16, False), ("bf16_weights_and_cache_b16", True, 16, True)):
+            i2, r = run_decode(cuda, path, bf16, batch, args.steps, args.warmup, graph=not args.no_graph, kv_bf16=kv16)
             also["decode_" + tag] = {"tokens_per_s": round(r["tokens_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4),
                                      "graph_replay": bool(r["graph"]), "prefill_128_tokens": prefill_summary(r, batch, 2 if bf16 else 4)}
             log("decode %s: %.1f tokens/s, prompt pass %s" % (tag, r["tokens_per_s"], json.dumps(also["decode_" + tag]["prefill_128_tokens"])))

@@ -267,7 +267,11 @@ enum {
      *                 appends the logits of every step, batch x nSteps x vocabulary (0, default);
      *                 option 7 = the forced prompt positions run as one batched pass (1, default: MFMA
      *                 GEMMs + fused causal attention over sequences x positions rows) or one decode
-     *                 step per position as in the reference's loop (0)
+     *                 step per position as in the reference's loop (0); option 8 = storage of the key /
+     *                 value caches: fp32 (0, default) or bf16 (1: rotated keys and values are rounded to
+     *                 nearest-even when they are appended, every step attends over the rounded rows;
+     *                 activations stay fp32; needs a head size that is a multiple of 8, otherwise the
+     *                 caches stay fp32); takes effect at the next generation
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were

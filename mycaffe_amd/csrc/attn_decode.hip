@@ -29,6 +29,10 @@ template <> struct Vec16<float> {
 #pragma unroll
         for (int i = 0; i < 4; i++) out[i] = __uint_as_float(r[i]);
     }
+    __device__ static inline u32x4 pack(const float* in)
+    {
+        return u32x4{__float_as_uint(in[0]), __float_as_uint(in[1]), __float_as_uint(in[2]), __float_as_uint(in[3])};
+    }
 };
 template <> struct Vec16<bf16_t> {
     static constexpr int W = 8;
@@ -49,6 +53,13 @@ template <> struct Vec16<bf16_t> {
             out[2 * i] = __uint_as_float(r[i] << 16);
             out[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
         }
+    }
+    __device__ static inline u32x4 pack(const float* in)
+    {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = (uint32_t)f32_to_bf16(in[2 * i]) | ((uint32_t)f32_to_bf16(in[2 * i + 1]) << 16);
+        return r;
     }
 };
 
@@ -189,9 +200,9 @@ __device__ __forceinline__ float part_load(const float* p) { return __hip_atomic
 
 // Merges the 4 * (64/LPR) lane groups of a workgroup through LDS and writes {M, L, acc[hs]} to `out`, or, when
 // this workgroup saw every cached row (yfinal set), the normalised result straight to yfinal.
-template <typename T, int LPR>
+template <typename T, int LPR, typename TY = T>
 __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (&acc)[Vec16<T>::W], int wave, int grp, int gl,
-                                                 int d0, bool active, int hs, float* __restrict__ out, T* __restrict__ yfinal = nullptr)
+                                                 int d0, bool active, int hs, float* __restrict__ out, TY* __restrict__ yfinal = nullptr)
 {
     constexpr int W = Vec16<T>::W;
     constexpr int RPW = 64 / LPR, NW = 4;
@@ -361,17 +372,20 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
 // store k and v into the cache, attend over positions 0..pos, write the head outputs.  qkv holds one
 // row [q | k | v] of dim + 2*kvd raw projections per sequence; caches are [B][seqLen][kvd].
 struct FusedDecodeArgs {
-    const float* qkv; float* kc; float* vc; float* y; float* part; int* counters;
+    const float* qkv; void* kc; void* vc; float* y; float* part; int* counters;
     const float* fcos; const float* fsin; const int* dlen;
     int B, H, kvMul, hs, dim, kvd, seqLen, splits, rowsPerIter;
     float scale;
     bool oneIter;   // seqLen <= splits * rowsPerIter: a split never holds more than one iteration of rows
 };
 
-template <int LPR>
+// TC: storage type of the caches (fp32, or bf16: the rotated key and the value are rounded when they are appended, and the
+// step that appends them attends over the rounded row as well, so a position is seen the same way by every later step).
+// Activations (q, the head outputs) stay fp32; a lane owns the W = 16 bytes / sizeof(TC) dimensions d0 .. d0 + W - 1.
+template <int LPR, typename TC>
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs a)
 {
-    constexpr int W = 4;
+    constexpr int W = Vec16<TC>::W;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int grp = lane / LPR, gl = lane % LPR;
@@ -382,8 +396,40 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     const int kvh = h / a.kvMul;
     const int ldq = a.dim + 2 * a.kvd;
     const float* row = a.qkv + (size_t)b * ldq;
-    float* kc = a.kc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
-    float* vc = a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    TC* kc = (TC*)a.kc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    TC* vc = (TC*)a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    auto load_row = [&](const float* p, float* o) {
+#pragma unroll
+        for (int j = 0; j < W / 4; j++) {
+            const float4 t = *(const float4*)(p + 4 * j);
+            o[4 * j] = t.x; o[4 * j + 1] = t.y; o[4 * j + 2] = t.z; o[4 * j + 3] = t.w;
+        }
+    };
+    // rotation factors of this lane's adjacent pairs (dims d0 + 2 j, d0 + 2 j + 1) at `pos`
+    float cs[W / 2], sn[W / 2];
+    auto load_factors = [&]() {
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) { cs[j] = 1.f; sn[j] = 0.f; }
+        if (active) {
+            const size_t ti = (size_t)pos * half + d0 / 2;
+#pragma unroll
+            for (int j = 0; j < W / 2; j++) { cs[j] = a.fcos[ti + j]; sn[j] = a.fsin[ti + j]; }
+        }
+    };
+    auto rotate = [&](const float* in, float* out, float scale) {
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) {
+            out[2 * j] = (in[2 * j] * cs[j] - in[2 * j + 1] * sn[j]) * scale;
+            out[2 * j + 1] = (in[2 * j] * sn[j] + in[2 * j + 1] * cs[j]) * scale;
+        }
+    };
+    auto rotate_key = [&](const float* in, float* out) {
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) {
+            out[2 * j] = in[2 * j] * cs[j] - in[2 * j + 1] * sn[j];
+            out[2 * j + 1] = in[2 * j] * sn[j] + in[2 * j + 1] * cs[j];
+        }
+    };
 
     if (a.oneIter) {
         // The whole cache fits one iteration per split: the query and the new key / value are requested together with
@@ -393,51 +439,46 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
         constexpr int RPW = 64 / LPR, U = 4, STEP = 4 * RPW * U;
         const int t0 = split * STEP;
         const int tb = t0 + wave * RPW * U;
-        float4 r = {0.f, 0.f, 0.f, 0.f}, kr = r, vr = r;
+        float r[W], kr[W], vr[W];
+#pragma unroll
+        for (int i = 0; i < W; i++) { r[i] = 0.f; kr[i] = 0.f; vr[i] = 0.f; }
         if (active) {
-            r = *(const float4*)(row + (size_t)h * a.hs + d0);
-            kr = *(const float4*)(row + a.dim + (size_t)kvh * a.hs + d0);
-            vr = *(const float4*)(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0);
+            load_row(row + (size_t)h * a.hs + d0, r);
+            load_row(row + a.dim + (size_t)kvh * a.hs + d0, kr);
+            load_row(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0, vr);
         }
         const int nAct = (len + STEP - 1) / STEP;
         if (split >= nAct) return;
         const int t1 = min(len, t0 + STEP);
         DecodeStage<U> A;
-        decode_issue<float, LPR, U>(A, kc, vc, a.kvd, tb, t1, grp, d0, active);
-        float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
-        if (active) {
-            const size_t ti = (size_t)pos * half + d0 / 2;
-            c0 = a.fcos[ti]; s0 = a.fsin[ti]; c1 = a.fcos[ti + 1]; s1 = a.fsin[ti + 1];
-        }
+        decode_issue<TC, LPR, U>(A, kc, vc, a.kvd, tb, t1, grp, d0, active);
+        load_factors();
         float qv[W];
-        qv[0] = (r.x * c0 - r.y * s0) * a.scale;
-        qv[1] = (r.x * s0 + r.y * c0) * a.scale;
-        qv[2] = (r.z * c1 - r.w * s1) * a.scale;
-        qv[3] = (r.z * s1 + r.w * c1) * a.scale;
+        rotate(r, qv, a.scale);
         if (t0 <= pos && pos < t1) {
-            float4 ko;
-            ko.x = kr.x * c0 - kr.y * s0; ko.y = kr.x * s0 + kr.y * c0;
-            ko.z = kr.z * c1 - kr.w * s1; ko.w = kr.z * s1 + kr.w * c1;
+            float ko[W];
+            rotate_key(kr, ko);
+            const u32x4 kb = Vec16<TC>::pack(ko), vb = Vec16<TC>::pack(vr);
             if (wave == 0 && grp == 0 && active) {
-                *(float4*)(kc + (size_t)pos * a.kvd + d0) = ko;
-                *(float4*)(vc + (size_t)pos * a.kvd + d0) = vr;
+                *(u32x4*)(kc + (size_t)pos * a.kvd + d0) = kb;
+                *(u32x4*)(vc + (size_t)pos * a.kvd + d0) = vb;
             }
-            const u32x4 kb = {__float_as_uint(ko.x), __float_as_uint(ko.y), __float_as_uint(ko.z), __float_as_uint(ko.w)};
-            const u32x4 vb = {__float_as_uint(vr.x), __float_as_uint(vr.y), __float_as_uint(vr.z), __float_as_uint(vr.w)};
 #pragma unroll
             for (int u = 0; u < U; u++)
                 if (tb + u * RPW + grp == pos && active) { A.k[u] = kb; A.v[u] = vb; }
         }
-        float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
-        decode_consume<float, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
+        float m = -INFINITY, l = 0.f, acc[W];
+#pragma unroll
+        for (int i = 0; i < W; i++) acc[i] = 0.f;
+        decode_consume<TC, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
         const size_t bh = (size_t)b * a.H + h;
         float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
         float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
         if (nAct == 1) {
-            decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
+            decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
             return;
         }
-        decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+        decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
         decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
         return;
     }
@@ -447,43 +488,39 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     const int nAct = (len + chunk - 1) / chunk;      // splits that hold rows; the rest of the launch idles
     if (split >= nAct) return;
 
-    // rotation factors of this lane's two adjacent pairs (dims d0, d0+1 and d0+2, d0+3) at `pos`
-    float c0 = 1.f, s0 = 0.f, c1 = 1.f, s1 = 0.f;
+    load_factors();
+    float qv[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) qv[i] = 0.f;
     if (active) {
-        const size_t ti = (size_t)pos * half + d0 / 2;
-        c0 = a.fcos[ti]; s0 = a.fsin[ti]; c1 = a.fcos[ti + 1]; s1 = a.fsin[ti + 1];
-    }
-    float qv[W] = {0.f, 0.f, 0.f, 0.f};
-    if (active) {
-        const float4 r = *(const float4*)(row + (size_t)h * a.hs + d0);
-        qv[0] = (r.x * c0 - r.y * s0) * a.scale;
-        qv[1] = (r.x * s0 + r.y * c0) * a.scale;
-        qv[2] = (r.z * c1 - r.w * s1) * a.scale;
-        qv[3] = (r.z * s1 + r.w * c1) * a.scale;
+        float r[W];
+        load_row(row + (size_t)h * a.hs + d0, r);
+        rotate(r, qv, a.scale);
     }
     // the split that owns the current position appends the rotated key and the value first
     if (t0 <= pos && pos < t1) {
         if (wave == 0 && grp == 0 && active) {
-            const float4 kr = *(const float4*)(row + a.dim + (size_t)kvh * a.hs + d0);
-            const float4 vr = *(const float4*)(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0);
-            float4 ko;
-            ko.x = kr.x * c0 - kr.y * s0; ko.y = kr.x * s0 + kr.y * c0;
-            ko.z = kr.z * c1 - kr.w * s1; ko.w = kr.z * s1 + kr.w * c1;
-            *(float4*)(kc + (size_t)pos * a.kvd + d0) = ko;
-            *(float4*)(vc + (size_t)pos * a.kvd + d0) = vr;
+            float kr[W], vr[W], ko[W];
+            load_row(row + a.dim + (size_t)kvh * a.hs + d0, kr);
+            load_row(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0, vr);
+            rotate_key(kr, ko);
+            *(u32x4*)(kc + (size_t)pos * a.kvd + d0) = Vec16<TC>::pack(ko);
+            *(u32x4*)(vc + (size_t)pos * a.kvd + d0) = Vec16<TC>::pack(vr);
         }
         __syncthreads();   // the row is read back by this workgroup only (other heads of the group write their own copy)
     }
-    float m = -INFINITY, l = 0.f, acc[W] = {0.f, 0.f, 0.f, 0.f};
-    decode_stream<float, LPR>(kc, vc, a.kvd, t0, t1, (unsigned)((b * a.H + h) * 37 + split * 11), wave, grp, d0, active, qv, m, l, acc);
+    float m = -INFINITY, l = 0.f, acc[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) acc[i] = 0.f;
+    decode_stream<TC, LPR>(kc, vc, a.kvd, t0, t1, (unsigned)((b * a.H + h) * 37 + split * 11), wave, grp, d0, active, qv, m, l, acc);
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
     float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
     if (nAct == 1) {
-        decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
+        decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
         return;
     }
-    decode_reduce_wg<float, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+    decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
     decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
 }
 
@@ -642,13 +679,14 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
     return launch_decode<bf16_t>(s, a, kvH);
 }
 
-hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float* vc, float* y, int B, int H, int kvH, int hs,
-                               int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
+hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* vc, DType cacheType, float* y, int B, int H, int kvH,
+                               int hs, int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
                                size_t workspaceBytes, int* counters)
 {
     if (B <= 0 || H <= 0 || hs <= 0 || seqLen <= 0) return hipSuccess;
-    if (kvH <= 0 || H % kvH != 0 || (hs % 4) != 0 || B > 65535 || H > 65535 || !counters || !dlen) return hipErrorInvalidValue;
-    int lpr = hs / 4, lprp = 1;
+    const int W = cacheType == F32 ? 4 : 8;   // elements per 16-byte cache chunk
+    if (kvH <= 0 || H % kvH != 0 || (hs % W) != 0 || B > 65535 || H > 65535 || !counters || !dlen) return hipErrorInvalidValue;
+    int lpr = hs / W, lprp = 1;
     while (lprp < lpr) lprp <<= 1;
     if (lprp > 64) return hipErrorInvalidValue;
     if (workspaceBytes < attn_decode_workspace_bytes(B, H, hs, seqLen)) return hipErrorInvalidValue;
@@ -663,7 +701,11 @@ hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float
     a.oneIter = seqLen <= a.splits * a.rowsPerIter;
     dim3 grid(a.splits, H, B);
     switch (lprp) {
-#define CASE(L) case L: hipLaunchKernelGGL((attn_decode_fused_kernel<L>), grid, 256, 0, s, a); break;
+#define CASE(L)                                                                                                            \
+    case L:                                                                                                                \
+        if (cacheType == F32) hipLaunchKernelGGL((attn_decode_fused_kernel<L, float>), grid, 256, 0, s, a);                \
+        else hipLaunchKernelGGL((attn_decode_fused_kernel<L, bf16_t>), grid, 256, 0, s, a);                                \
+        break;
         CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
 #undef CASE
     }

@@ -141,11 +141,11 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
 // `counters`: B*H zero-initialised ints that stay zero between launches; when given, the last
 // workgroup of every (batch, head) merges the split partials inside the kernel (no second launch).
 //
-// fp32 decode step of the llama2 engine in one launch: rotate q / k at position *dlen - 1, append k, v
-// to the caches ([B][seqLen][kvH*hs]), attend over positions 0 .. *dlen - 1.  qkv: [B][(H + 2 kvH) hs]
-// raw projections, y: [B][H*hs].
-hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, float* kc, float* vc, float* y, int B, int H, int kvH, int hs,
-                               int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
+// Decode step of the llama2 engine in one launch: rotate q / k at position *dlen - 1, append k, v to the caches
+// ([B][seqLen][kvH*hs], stored as cacheType: fp32, or bf16 with hs a multiple of 8), attend over positions
+// 0 .. *dlen - 1.  qkv: [B][(H + 2 kvH) hs] raw fp32 projections, y: [B][H*hs] fp32.
+hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* vc, DType cacheType, float* y, int B, int H, int kvH,
+                               int hs, int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
                                size_t workspaceBytes, int* counters);
 // rotate q (B,H,hs) and knew (B,kvH,hs) at position pos and append knew/vnew to the caches at pos
 hipError_t k_rope_append(hipStream_t s, DType dt, void* q, void* knew, const void* vnew, void* kc, void* vc, int B,

@@ -536,11 +536,18 @@ __global__ void prefill_embed_kernel(const int* __restrict__ prompt, int promptS
     for (int i = threadIdx.x; i < dim; i += blockDim.x) x[(size_t)m * dim + i] = wld(emb, (size_t)tok * dim + i);
 }
 
+__device__ inline void store_pair(float* p, float2 v) { *(float2*)p = v; }
+__device__ inline void store_pair(bf16_t* p, float2 v) { *(uint32_t*)p = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16); }
+// what a later decode step reads back from a cache of type TC
+template <typename TC> __device__ inline float2 as_stored(float2 v) { return v; }
+template <> __device__ inline float2 as_stored<bf16_t>(float2 v) { return make_float2(bf16_to_f32(f32_to_bf16(v.x)), bf16_to_f32(f32_to_bf16(v.y))); }
+
 // One row [q | k | v] of raw projections per (b, p): rotate q and k at position p (adjacent pairs, the arithmetic of
 // the decode kernel), write q as (B,H,P,hs), k and v as (B,H,P,hs) with every key / value head repeated for the query
 // heads that share it, and append the rotated key and the value to the caches [b][pos][kvd].
+template <typename TC>
 __global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float* __restrict__ qh, float* __restrict__ kh,
-                                            float* __restrict__ vh, float* __restrict__ kc, float* __restrict__ vc,
+                                            float* __restrict__ vh, TC* __restrict__ kc, TC* __restrict__ vc,
                                             const float* __restrict__ fcos, const float* __restrict__ fsin, int B, int P, int H,
                                             int kvH, int hs, int seqLen)
 {
@@ -562,14 +569,16 @@ __global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float
             if (col < dim) {
                 *(float2*)(qh + (((size_t)b * H + h) * P + p) * hs + d) = o;
             } else {
-                *(float2*)(kc + ((size_t)b * seqLen + p) * kvd + c) = o;
+                o = as_stored<TC>(o);   // the pass attends over the values the cache holds, as the decode steps will
+                store_pair(kc + ((size_t)b * seqLen + p) * kvd + c, o);
                 for (int g = 0; g < kvMul; g++) *(float2*)(kh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = o;
             }
         } else {
             const int c = col - dim - kvd;
             const int h = c / hs, d = c - h * hs;
-            *(float2*)(vc + ((size_t)b * seqLen + p) * kvd + c) = r;
-            for (int g = 0; g < kvMul; g++) *(float2*)(vh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = r;
+            const float2 rs = as_stored<TC>(r);
+            store_pair(vc + ((size_t)b * seqLen + p) * kvd + c, rs);
+            for (int g = 0; g < kvMul; g++) *(float2*)(vh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = rs;
         }
     }
 }
@@ -768,6 +777,9 @@ public:
     bool use_graph = true;
     bool lastUsedGraph = false;  // whether the last generate replayed a captured graph (false: eager launches)
     bool use_prefill = true;     // prompt positions as one batched pass (false: one decode step per position)
+    bool kv_bf16 = false;        // caches stored as bf16 (option 8; takes effect when the run state is next allocated)
+    bool state_kv_bf16 = false;  // what the allocated caches hold
+    void set_kv_bf16(bool on) { kv_bf16 = on; if (on != state_kv_bf16) { stateB = -1; graphB = -1; } }
     float lastPrefillMs = 0.f;   // HIP-event duration of the batched prompt pass of the last generate (0: none ran)
     int lastPrefillRows = 0;     // sequences x prompt positions it covered
     int mvRows = 0;              // weight rows per wavefront in the mat-vec kernels (0: chosen per shape)
@@ -812,7 +824,8 @@ private:
     // run state (sized for stateB sequences)
     int stateB = 0, stateSteps = 0;
     std::vector<void*> stateAllocs;
-    float *x = nullptr, *xb = nullptr, *qkv = nullptr, *qc = nullptr, *hb = nullptr, *logits = nullptr, *kc = nullptr, *vc = nullptr;
+    float *x = nullptr, *xb = nullptr, *qkv = nullptr, *qc = nullptr, *hb = nullptr, *logits = nullptr;
+    void *kc = nullptr, *vc = nullptr;             // caches [layer][batch][seq][kv_dim], fp32 or bf16 (state_kv_bf16)
     void* ws = nullptr; size_t wsBytes = 0;
     GenState* dstate = nullptr;
     int *dprompt = nullptr, *dnext = nullptr, *dcur = nullptr, *dout = nullptr;
@@ -1012,8 +1025,9 @@ long Engine::ensure_state(int B, int nSteps)
     qc = (float*)sa(B * dim * 4);
     hb = (float*)sa(B * hid * 4);
     logits = (float*)sa((size_t)B * cfg.vocab_size * 4);
-    kc = (float*)sa(cacheN * 4);
-    vc = (float*)sa(cacheN * 4);
+    state_kv_bf16 = kv_bf16 && hs % 8 == 0;       // a 16-byte chunk of a bf16 row is 8 dims of one head
+    kc = sa(cacheN * (state_kv_bf16 ? 2 : 4));
+    vc = sa(cacheN * (state_kv_bf16 ? 2 : 4));
     ws = sa(wsBytes);
     dstate = (GenState*)sa(sizeof(GenState));
     dprompt = (int*)sa((size_t)B * cfg.seq_len * 4);
@@ -1089,13 +1103,21 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
     const bool skinny = M <= 256 && dim % 32 == 0 && hid % 32 == 0;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
-        float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
-        float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
+        const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
+        void* kcl = (char*)kc + cacheOfs;
+        void* vcl = (char*)vc + cacheOfs;
+        auto rope_scatter = [&]() {
+            if (state_kv_bf16)
+                hipLaunchKernelGGL(prefill_rope_scatter_kernel<bf16_t>, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, (bf16_t*)kcl,
+                                   (bf16_t*)vcl, fcos, fsin, B, P, H, kvH, hs, cfg.seq_len);
+            else
+                hipLaunchKernelGGL(prefill_rope_scatter_kernel<float>, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, (float*)kcl,
+                                   (float*)vcl, fcos, fsin, B, P, H, kvH, hs, cfg.seq_len);
+            return hipGetLastError();
+        };
         if (skinny) {
             HIPCHK((launch_matvec_rows<0, true, T>(s, w.wqkv, pfX, w.rms_att, pfQkv, ldq, dim, (int)M, ldq)));
-            hipLaunchKernelGGL(prefill_rope_scatter_kernel, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, kcl, vcl, fcos, fsin, B, P,
-                               H, kvH, hs, cfg.seq_len);
-            HIPCHK(hipGetLastError());
+            HIPCHK(rope_scatter());
             HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
             HIPCHK((launch_matvec_rows<1, false, T>(s, w.wo, pfXn, nullptr, pfX, dim, dim, (int)M, dim)));          // x += Wo att
             HIPCHK((launch_matvec_rows<2, true, T>(s, w.w13, pfX, w.rms_ffn, pfHb, hid, dim, (int)M, hid)));
@@ -1106,9 +1128,7 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         const float* wqkv = as_f32<T>(s, w.wqkv, (size_t)ldq * dim, &e);
         if (e) return e;
         HIPCHK(k_gemm(s, F32, false, true, (int)M, ldq, dim, 1.f, pfXn, wqkv, 0.f, pfQkv));
-        hipLaunchKernelGGL(prefill_rope_scatter_kernel, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, kcl, vcl, fcos, fsin, B, P,
-                           H, kvH, hs, cfg.seq_len);
-        HIPCHK(hipGetLastError());
+        HIPCHK(rope_scatter());
         HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));   // head-merged output
         const float* wo = as_f32<T>(s, w.wo, (size_t)dim * dim, &e);
         if (e) return e;
@@ -1228,15 +1248,16 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
     const float scale = 1.0f / sqrtf((float)hs);
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
-        float* kcl = kc + (size_t)l * B * cfg.seq_len * kvd;
-        float* vcl = vc + (size_t)l * B * cfg.seq_len * kvd;
+        const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
+        void* kcl = (char*)kc + cacheOfs;
+        void* vcl = (char*)vc + cacheOfs;
         // qkv = [Wq;Wk;Wv] rmsnorm(x)
         SPAN_BEGIN(SC_MATVEC_QKV);
         HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq, mvRows)));
         SPAN_END();
         // xb = attention(rope(q), cache[0..pos] with rope(k), v appended)
         SPAN_BEGIN(SC_ATTN_DECODE);
-        HIPCHK(k_attn_decode_fused(s, qkv, kcl, vcl, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len, scale, fcos, fsin,
+        HIPCHK(k_attn_decode_fused(s, qkv, kcl, vcl, state_kv_bf16 ? BF16 : F32, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len, scale, fcos, fsin,
                                    &dstate->len, ws, wsBytes, dcount));
         SPAN_END();
         // x += Wo xb
@@ -1697,6 +1718,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 5) m->sampleIds = pIn[2] != 0.f;
         else if (opt == 6) m->batchLogits = pIn[2] != 0.f;
         else if (opt == 7) m->engine.use_prefill = pIn[2] != 0.f;
+        else if (opt == 8) m->engine.set_kv_bf16(pIn[2] != 0.f);
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }

@@ -44,6 +44,8 @@ def lib():
         ip = ctypes.POINTER(ctypes.c_int)
         L.orc_set_threads.argtypes = [ctypes.c_int]
         L.orc_set_threads.restype = ctypes.c_int
+        L.orc_set_kv_bf16.argtypes = [ctypes.c_int]
+        L.orc_round_bf16.argtypes = [fp, ctypes.c_int]
         L.orc_rmsnorm.argtypes = [fp, fp, fp, ctypes.c_int]
         L.orc_softmax.argtypes = [fp, ctypes.c_int]
         L.orc_matvec.argtypes = [fp, fp, fp, ctypes.c_int, ctypes.c_int]
@@ -126,6 +128,19 @@ def rope_pairs(q, k, fcos, fsin, pos):
 def set_threads(n):
     """Limit the checker's parallel loops to ``n`` threads; returns the previous limit."""
     return int(lib().orc_set_threads(int(n)))
+
+
+def set_kv_bf16(on):
+    """Checker-only option (no counterpart in the reference): every forward from now on rounds the rotated key and the
+    value of the current position to bfloat16 before they enter the cache and the attention."""
+    lib().orc_set_kv_bf16(int(bool(on)))
+
+
+def round_bf16(x):
+    """fp32 -> nearest bfloat16 (ties to even), as fp32."""
+    x = np.array(x, np.float32).ravel().copy()
+    lib().orc_round_bf16(_fp(x), x.size)
+    return x
 
 
 def argmax(p):

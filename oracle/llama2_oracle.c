@@ -31,6 +31,13 @@
  * for this path includes <io.h> and the CUDA headers (llama2_cpu.h:6,22 via
  * primitives.h:20-27) and so cannot be compiled in this image without
  * stand-ins; no oracle/_ref build exists for it.
+ *
+ * One checker-only option has no counterpart in the reference: orc_set_kv_bf16(1)
+ * makes the forward round the rotated key and the value of the current position
+ * to bfloat16 (round to nearest even) before they enter the cache and the
+ * attention, which is what the HIP engine's 16-bit cache mode does.  The
+ * rounding (orc_round_bf16) is pinned against torch's float32 -> bfloat16
+ * conversion, ties, denormals and infinities included.
  */
 #include <math.h>
 #ifdef _OPENMP
@@ -53,6 +60,25 @@ typedef struct {
     float *x, *xb, *xb2, *hb, *hb2, *q, *k, *v, *att, *logits;
     float *kcache, *vcache, *fcos, *fsin;
 } OrcLlama;
+
+/* checker-only: cache entries rounded to bfloat16 (see the header) */
+static int g_kv_bf16 = 0;
+void orc_set_kv_bf16(int on) { g_kv_bf16 = on; }
+
+/* fp32 -> nearest bfloat16 (ties to even), returned as fp32; NaN stays NaN */
+void orc_round_bf16(float *x, int n)
+{
+    for (int i = 0; i < n; i++) {
+        uint32_t u;
+        memcpy(&u, &x[i], 4);
+        if ((u & 0x7fffffffu) > 0x7f800000u)
+            u |= 0x00400000u;
+        else
+            u += 0x7fffu + ((u >> 16) & 1u);
+        u &= 0xffff0000u;
+        memcpy(&x[i], &u, 4);
+    }
+}
 
 /* worker threads of the parallel loops below (the reference takes OpenMP's default); returns the previous limit */
 int orc_set_threads(int n)
@@ -247,6 +273,10 @@ float *orc_llama_forward(OrcLlama *m, int token, int pos)
 
         orc_rope_pairs(c->n_heads, hs, m->q, m->k, m->fcos, m->fsin, foff);
 
+        if (g_kv_bf16) {
+            orc_round_bf16(m->k, kvd);
+            orc_round_bf16(m->v, kvd);
+        }
         size_t loff = l * c->seq_len * kvd;
         memcpy(m->kcache + loff + (size_t)pos * kvd, m->k, kvd * sizeof(float));
         memcpy(m->vcache + loff + (size_t)pos * kvd, m->v, kvd * sizeof(float));

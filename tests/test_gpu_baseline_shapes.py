@@ -140,6 +140,43 @@ def test_llama110m_bf16_weights_against_checker_on_rounded_weights(llm, c4_model
         _batch_rows_against_cpu(cpu, prompts, n, ids, logits, "110M bf16 batch 16")
 
 
+def test_llama110m_batch16_bf16_weights_and_bf16_cache(llm, c4_model):
+    """The fully 16-bit-storage configuration at the benchmarked shape: bf16 weights and bf16 key / value caches, batch 16,
+    a 128-token prompt per sequence (the batched prompt pass through the GEMM path) and greedy steps after it.  Every row
+    against its own CPU run on the rounded weights with the checker's cache rounding; 3e-3 on the logits: a last-bit
+    difference between the two sides' fp32 key or value next to a rounding boundary moves the cached element by one
+    bfloat16 step, and a sequence caches 3 million elements here (2 x 12 layers x 768 x 160 positions)."""
+    path, blob = c4_model
+    llm.SetOption(1, 1)
+    llm.SetOption(8, 1)
+    llm.Load(path)
+    rb = bf16_round(blob)
+    rng = np.random.default_rng(77)
+    B, nP, n = 16, 128, 160
+    prompts = rng.integers(3, C4["vocab_size"], (B, nP))
+    ids, logits = llm.GenerateBatch(prompts, n, want_logits=True)
+    assert llm.LastPrefill()[1] == B * nP
+    assert np.array_equal(llm.GenerateBatch(prompts, n), ids)
+    assert llm.LastRunUsedGraph()
+    O.set_kv_bf16(True)
+    try:
+        cpu = O.Llama(C4, rb)
+        parted = 0
+        for b in range(0, B, 3):   # six of the sixteen rows: 160 positions of the 110M model take the CPU a second each
+            ref_ids, ref_logits = cpu.generate_greedy(prompts[b], n, want_logits=True)
+            assert np.array_equal(ids[b], _first_max(logits[b]))
+            same = np.array_equal(ids[b], ref_ids)
+            upto = n if same else int(np.argmax(ids[b] != ref_ids)) + 1
+            assert_close(logits[b, :upto], ref_logits[:upto], 3e-3, "110M 16-bit weights and caches, sequence %d" % b)
+            if not same:
+                top2 = np.sort(ref_logits[upto - 1])[-2:]
+                assert (top2[1] - top2[0]) / np.abs(ref_logits[upto - 1]).max() < 3e-3, "sequence %d parts at a decisive step" % b
+                parted += 1
+        assert parted <= 1
+    finally:
+        O.set_kv_bf16(False)
+
+
 def test_weight_storage_option_after_load_leaves_the_loaded_model_alone(llm, c4_model):
     # option 1 names the storage of the NEXT load: flipping it on a loaded fp32 model changes nothing
     path, blob = c4_model

@@ -133,7 +133,7 @@ def test_batch_generation_matches_independent_sequences(llm, tmp_path):
 
 def test_batch_with_grouped_query_heads_and_multi_iteration_splits(llm, tmp_path):
     """40 sequences, head size 64, two query heads per key / value head, cache of 512 positions: with 160 (sequence,
-    head) pairs the fused decode attention takes four splits of 128 rows, i.e. two 64-row iterations per split, and
+    head) pairs the fused decode attention takes two splits of 256 rows, i.e. four 64-row iterations per split, and
     appends the new key / value through the cache (the path batch 1 does not take).  Ids of every row against the
     checker over 300 positions."""
     cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=512)

@@ -276,3 +276,73 @@ def test_package_checkpoint_writer_matches_the_checkers(tmp_path):
         O.write_checkpoint_v1(pa, cfg, a, shared)
         C.write_v1(pb, cfg, b, shared)
         assert open(pa, "rb").read() == open(pb, "rb").read()
+
+
+def test_bf16_rounding_vs_torch():
+    import torch
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.standard_normal(4096).astype(np.float32) * 10.0 ** rng.integers(-30, 30, 4096).astype(np.float32),
+        # exact ties between two bfloat16 neighbours, even and odd kept bit below them
+        np.array([0x3f808000, 0x3f818000, 0xbf808000, 0xbf818000, 0x00008000, 0x00018000, 0x7f7f8000, 0x7f7fffff],
+                 np.uint32).view(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-40, 3.3895314e38], np.float32),
+    ])
+    with np.errstate(over="ignore"):
+        ref = torch.from_numpy(x.copy()).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(O.round_bf16(x).view(np.uint32), ref.view(np.uint32))
+    assert np.isnan(O.round_bf16(np.array([np.nan], np.float32))[0])
+
+
+@pytest.mark.parametrize("cfg", [TINY, TINY_GQA], ids=["mha", "gqa"])
+def test_bf16_cache_option_vs_a_forward_assembled_from_the_pinned_routines(cfg):
+    """The checker-only 16-bit cache option: the same logits as a forward written out here from the individually pinned
+    routines (rmsnorm, matvec, rope, softmax) with torch doing the rounding of every key and value that enters the cache."""
+    import torch
+    blob, w = O.random_weights(cfg, seed=5, std=0.3)
+    dim, H, kvH = cfg["dim"], cfg["n_heads"], cfg["n_kv_heads"]
+    hs, L = dim // H, cfg["n_layers"]
+    fcos, fsin = O.freq_tables(hs, cfg["seq_len"])
+    rnd = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(torch.bfloat16).to(torch.float32).numpy()
+    toks = [3, 77, 12, 5, 41, 9]
+    kc = [[] for _ in range(L)]
+    vc = [[] for _ in range(L)]
+    mine = []
+    for pos, tok in enumerate(toks):
+        x = w["tok_emb"][tok].copy()
+        for l in range(L):
+            xb = O.rmsnorm(x, w["rms_att"][l])
+            q = O.matvec(w["wq"][l], xb).reshape(H, hs)
+            k = O.matvec(w["wk"][l], xb).reshape(kvH, hs)
+            v = O.matvec(w["wv"][l], xb).reshape(kvH, hs)
+            # the checker rotates q and k in one call over n_heads heads of which the first kv heads are k's
+            kpad = np.zeros((H, hs), np.float32)
+            kpad[:kvH] = k
+            q, kpad = O.rope_pairs(q, kpad, fcos, fsin, pos)
+            kc[l].append(rnd(kpad[:kvH]))
+            vc[l].append(rnd(v))
+            o = np.zeros((H, hs), np.float32)
+            for h in range(H):
+                g = h // (H // kvH)
+                s = np.stack([kc[l][t][g] for t in range(pos + 1)]).astype(np.float64) @ q[h].astype(np.float64) / np.sqrt(hs)
+                a = O.softmax(s.astype(np.float32))
+                o[h] = (a[:, None].astype(np.float64) * np.stack([vc[l][t][g] for t in range(pos + 1)])).sum(0)
+            x = x + O.matvec(w["wo"][l], o.ravel())
+            xb = O.rmsnorm(x, w["rms_ffn"][l])
+            h1 = O.matvec(w["w1"][l], xb)
+            h3 = O.matvec(w["w3"][l], xb)
+            x = x + O.matvec(w["w2"][l], (h1 / (1.0 + np.exp(-h1)) * h3).astype(np.float32))
+        x = O.rmsnorm(x, w["rms_final"])
+        mine.append(O.matvec(w.get("wcls", w["tok_emb"]), x))
+    O.set_kv_bf16(True)
+    try:
+        m = O.Llama(cfg, blob)
+        got = np.stack([m.forward(t, p) for p, t in enumerate(toks)])
+    finally:
+        O.set_kv_bf16(False)
+    plain = np.stack([O.Llama(cfg, blob).forward(t, p) for p, t in enumerate(toks)][:1])
+    mine = np.stack(mine)
+    assert np.abs(got - mine).max() / np.abs(mine).max() < 2e-5
+    # the option changes the result (position 0 attends over its own rounded value) and is off again afterwards
+    assert np.abs(got[0] - plain[0]).max() > 1e-6
+    assert np.array_equal(O.Llama(cfg, blob).forward(toks[0], 0), plain[0])
