@@ -95,7 +95,9 @@ enum {
     MCH_FN_SOFTMAX_BWD = 112,               /* f{alpha, beta} l{hCudnn, 0, hTopDataDesc, hTopData, hTopDiffDesc, hTopDiff, 0, hBtmDiffDesc, hBtmDiff, alg, mode} (device.h:4801-4823) */
     MCH_FN_ATTN_CREATE = 160,               /* -> handle */
     MCH_FN_ATTN_FREE = 161,                 /* f{h} */
-    MCH_FN_ATTN_SET = 162,                  /* f{dropout} l{hCudnn, hAttn, gpuId, training, batch, blockSize, heads, hs, seed} (device.h:2463-2485) */
+    MCH_FN_ATTN_SET = 162,                  /* f{dropout} l{hCudnn, hAttn, gpuId, training, batch, blockSize, heads, hs, seed} (device.h:2463-2485);
+                                             * dropout in [0, 1) acts in training mode only (attn.cu:578-583): a new mask per forward call from a
+                                             * counter-based generator seeded with `seed`, repeated by the backward call that follows */
     MCH_FN_ATTN_FWD = 163,                  /* l{hCudnn, hAttn, blockSize, hQ, hK, hV, hMask, hY, batchMask[, blockSizeK[, mergedY]]} (device.h:2488-2506, attn.cu:518-602) */
     MCH_FN_ATTN_BWD = 164,                  /* l{hCudnn, hAttn, hQ, hdQ, hK, hdK, hV, hdV, hMask, hY, hdY} (device.h:2509-2529, attn.cu:608-661) */
     MCH_FN_SET = 200,                       /* f{val} l{n, h, 0, idx, xOff} (device.h:6038-6061) */

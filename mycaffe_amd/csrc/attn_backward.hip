@@ -43,7 +43,20 @@ struct AttnBwdArgs {
     float scale;
     int computeLse;
     int computeD;     // MFMA path: the dQ kernel computes D itself (no statistics kernel ran)
+    int useDropout;   // row kernels only
+    AttnDropout drop;
 };
+
+// factors of probability (bh, row, key) under dropout: pf multiplies P for dV, sf multiplies dS
+__device__ inline void attn_drop_factors(const AttnBwdArgs& a, size_t bh, int row, int key, float* pf, float* sf)
+{
+    *pf = 1.f;
+    *sf = 1.f;
+    if (!a.useDropout) return;
+    const bool keep = attn_dropout_keep(a.drop.seed, (uint64_t)(bh * a.Tq + row) * a.Tk + key, a.drop.threshold);
+    *pf = keep ? a.drop.keepScale : 0.f;
+    *sf = keep ? a.drop.keepScale * a.drop.keepScale : 0.f;
+}
 
 __device__ inline bool attn_masked(const AttnBwdArgs& a, int b, int row, int key)
 {
@@ -148,7 +161,9 @@ template <typename T> __global__ __launch_bounds__(256) void attn_bwd_dq_rows_ke
                 dp += gs[wave][i] * ldb(vr, i);
             }
             const float p = attn_prob(s, attn_masked(a, b, row, j), lse2, uniform);
-            ds = p * (dp - dsum) * a.scale;
+            float pf, sf;
+            attn_drop_factors(a, bh, row, j, &pf, &sf);
+            ds = sf * p * (dp - dsum) * a.scale;
         }
         const int cnt = min(64, kend - kb);
         for (int jj = 0; jj < cnt; jj++) {
@@ -203,7 +218,10 @@ template <typename T> __global__ __launch_bounds__(256) void attn_bwd_dkv_rows_k
                 dp += vs[wave][d] * ldb(gr, d);
             }
             p = attn_prob(s, attn_masked(a, b, i, key), lse[i], uniform);
-            ds = p * (dp - dsm[i]) * a.scale;
+            float pf, sf;
+            attn_drop_factors(a, bh, i, key, &pf, &sf);
+            ds = sf * p * (dp - dsm[i]) * a.scale;
+            p *= pf;
         }
         const int cnt = min(64, a.Tq - qb);
         for (int ii = 0; ii < cnt; ii++) {
@@ -236,7 +254,7 @@ size_t attn_backward_workspace_bytes(int B, int H, int Tq) { return (size_t)B * 
 
 hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k, const void* v, const void* y, const void* dy,
                            void* dq, void* dk, void* dv, int B, int H, int Tq, int Tk, int hs, float scale, const float* mask,
-                           MaskKind kind, const float* lse2, void* workspace, size_t workspaceBytes)
+                           MaskKind kind, const float* lse2, void* workspace, size_t workspaceBytes, const AttnDropout* dropout)
 {
     if (B <= 0 || H <= 0 || Tq <= 0 || Tk <= 0 || hs <= 0) return hipSuccess;
     if (B > 65535 || H > 65535 || hs > 256) return hipErrorInvalidValue;
@@ -249,7 +267,9 @@ hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k
     a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale;
     a.computeLse = lse2 ? 0 : 1;
     dim3 gq((Tq + 3) / 4, H, B), gk((Tk + 3) / 4, H, B);
-    const bool mfma = attn_bwd_mfma_usable(dt, a);
+    a.useDropout = dropout ? 1 : 0;
+    if (dropout) a.drop = *dropout;
+    const bool mfma = !dropout && attn_bwd_mfma_usable(dt, a);
     // the statistics kernel is needed for lse2 when the forward pass left none, and for D whenever the row kernels run
     a.computeD = (mfma && lse2) ? 1 : 0;
     if (!a.computeD) {

@@ -32,6 +32,8 @@ struct AttnArgs {
     float scale;
     float* lse2;   // optional [B*H*Tq]: log2 of the row's softmax denominator (-inf marks a fully masked row)
     int yMerged;   // 1: y is written head-merged, (B,Tq,H,hs), the layout the output projection reads; 0: (B,H,Tq,hs)
+    int useDropout;
+    AttnDropout drop;
 };
 
 // offset of output row `row` of head (b, h) in y
@@ -82,9 +84,13 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
         for (int o = 32; o > 0; o >>= 1) ps += __shfl_xor(ps, o, 64);
         l = l * corr + ps;
         for (int i = 0; i < DPL; i++) acc[i] *= corr;
+        // dropout acts on the normalised probabilities: the denominator keeps every key, the output only the survivors
+        float pd = p;
+        if (a.useDropout && j < kend)
+            pd = attn_dropout_keep(a.drop.seed, (uint64_t)(bh * a.Tq + row) * a.Tk + j, a.drop.threshold) ? p * a.drop.keepScale : 0.f;
         const int cnt = min(64, kend - kb);
         for (int jj = 0; jj < cnt; jj++) {
-            const float pj = __shfl(p, jj, 64);
+            const float pj = __shfl(pd, jj, 64);
             const T* vr = v + (size_t)(kb + jj) * a.hs;
             for (int i = 0; i < DPL; i++) {
                 int d = lane + i * 64;
@@ -105,7 +111,8 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
 hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* handled);
 
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
-                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2, bool yMerged)
+                          int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2, bool yMerged,
+                          const AttnDropout* dropout)
 {
     if (B <= 0 || H <= 0 || Tq <= 0 || Tk <= 0 || hs <= 0) return hipSuccess;
     if (B > 65535 || H > 65535) return hipErrorInvalidValue;
@@ -114,9 +121,13 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
     a.q = q; a.k = k; a.v = v; a.y = y; a.mask = mask;
     a.B = B; a.H = H; a.Tq = Tq; a.Tk = Tk; a.hs = hs; a.kind = (int)kind; a.scale = scale; a.lse2 = lse2;
     a.yMerged = yMerged ? 1 : 0;
+    a.useDropout = dropout ? 1 : 0;
+    if (dropout) a.drop = *dropout;
     bool handled = false;
-    hipError_t e = attn_flash_launch(s, dt, a, &handled);
-    if (e != hipSuccess || handled) return e;
+    if (!dropout) {   // the matrix-core kernels have no dropout: training with a non-zero ratio takes the row kernel
+        hipError_t e = attn_flash_launch(s, dt, a, &handled);
+        if (e != hipSuccess || handled) return e;
+    }
     if (hs > 256) return hipErrorInvalidValue;
     dim3 grid((Tq + 3) / 4, H, B);
     if (dt == F32) hipLaunchKernelGGL(attn_rows_kernel<float>, grid, 256, 0, s, a);

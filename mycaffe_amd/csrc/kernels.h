@@ -116,9 +116,26 @@ enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAU
 // q (B,H,Tq,hs), k/v (B,H,Tk,hs), y (B,H,Tq,hs), all dt.  mask is fp32:
 //   MASK_QK (Tq,Tk) shared, MASK_KEY (B,Tk), MASK_BQK (B,Tq,Tk); zero entries are filled with -1e29.
 //   MASK_CAUSAL needs no mask buffer (lower triangle kept).
+// Attention dropout (training mode of the handle, attn.cu:455-486, 578-583): which probabilities survive is a pure
+// function of (seed, batch*heads index, query, key), so the backward pass regenerates the mask of the forward call
+// instead of storing it.  keep(i) = high 32 bits of splitmix64(seed * 0x9E3779B97F4A7C15 + i) >= threshold, with
+// i = ((b*H + h)*Tq + query)*Tk + key and threshold = ratio * 2^32; survivors are scaled by 1 / (1 - ratio).
+struct AttnDropout {
+    uint64_t seed;
+    uint32_t threshold;
+    float keepScale;
+};
+__host__ __device__ inline bool attn_dropout_keep(uint64_t seed, uint64_t index, uint32_t threshold)
+{
+    uint64_t z = seed * 0x9E3779B97F4A7C15ull + index + 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (uint32_t)(z >> 32) >= threshold;
+}
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
                           int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2 = nullptr,
-                          bool yMerged = false);
+                          bool yMerged = false, const AttnDropout* dropout = nullptr);
 // yMerged: y is written as (B,Tq,H,hs), the head-merged layout the output projection reads, instead of (B,H,Tq,hs).
 // With lse2 ([B*H*Tq] fp32) the forward pass also stores log2 of every row's softmax denominator (scores scaled, masked
 // ones at -1e29; -inf marks a row whose keys are all masked), which is all the backward pass needs of the probabilities.
@@ -128,7 +145,11 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 size_t attn_backward_workspace_bytes(int B, int H, int Tq);
 hipError_t k_attn_backward(hipStream_t s, DType dt, const void* q, const void* k, const void* v, const void* y, const void* dy,
                            void* dq, void* dk, void* dv, int B, int H, int Tq, int Tk, int hs, float scale, const float* mask,
-                           MaskKind kind, const float* lse2, void* workspace, size_t workspaceBytes);
+                           MaskKind kind, const float* lse2, void* workspace, size_t workspaceBytes,
+                           const AttnDropout* dropout = nullptr);
+// With dropout both calls take the general one-row-per-wavefront kernels (no matrix-core path), and the backward pass
+// follows the reference's sequence literally: its softmax backward reads the probabilities AFTER dropout was applied to
+// them in place (attn.cu:578-583, 637-646), which gives dS = M / (1 - ratio)^2 * P * (dP - dY.Y) and dV = (P M')^T dY.
 size_t attn_decode_workspace_bytes(int B, int H, int hs, int len);
 // one query per (b,h): q (B,H,hs), caches addressed as
 //   cache[b*strideB + (h/kvMul)*strideH + t*strideT + i], y (B,H,hs).  All dt.

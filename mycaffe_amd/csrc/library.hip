@@ -1571,6 +1571,9 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         st->training = pl[3] != 0;
         st->batch = (int)pl[4]; st->block = (int)pl[5]; st->heads = (int)pl[6]; st->hs = (int)pl[7];
         st->dropout = pf[0];
+        if (!(st->dropout >= 0.f) || st->dropout >= 1.f) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        st->seed = (uint64_t)pl[8];
+        st->fwdCalls = 0;
         st->scale = (float)(1.0 / sqrt((double)st->hs));  // attn.cu:427
         st->set = true;
         st->maskHandle = 0;
@@ -1592,7 +1595,6 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         int Tk = ll > 9 ? (int)pl[9] : T;
         if (T > st->block || Tk > st->block) return MCH_ERROR_ATTN_INVALID_BLOCK_SIZE;
         if (T < 1 || Tk < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        if (st->training && st->dropout > 0.f) { last_detail = "attention dropout (training) is not part of the inference path"; return MCH_ERROR_NOT_IMPLEMENTED; }
         MemItem *Q, *K, *V, *Y, *M = nullptr;
         ERRCHK(mem((long)pl[3], &Q));
         ERRCHK(mem((long)pl[4], &K));
@@ -1644,8 +1646,16 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 st->ysaveBytes = ybytes;
             }
         }
+        // training with a dropout ratio: a fresh mask per forward call (the reference's generator state advances with
+        // every call), remembered for the backward call that follows
+        const bool drop = st->training && st->dropout > 0.f;
+        if (drop) {
+            st->drop.seed = st->seed + 0xD1B54A32D192ED03ull * (uint64_t)(++st->fwdCalls);
+            st->drop.threshold = (uint32_t)fmin((double)st->dropout * 4294967296.0, 4294967295.0);
+            st->drop.keepScale = 1.0f / (1.0f - st->dropout);
+        }
         HIPCHK(k_attn_prefill(s, Q->dt(), Q->ptr, K->ptr, V->ptr, Y->ptr, st->batch, st->heads, T, Tk, st->hs, st->scale,
-                              M ? (const float*)M->ptr : nullptr, kind, lse, mergedY));
+                              M ? (const float*)M->ptr : nullptr, kind, lse, mergedY, drop ? &st->drop : nullptr));
         // the backward pass needs this output (dY . Y per row); the C# layer hands ATTN_BWD a Y buffer that holds the
         // head-merged layout by then (CausalSelfAttentionLayer.cs:668-672), so a copy stays with the handle
         if (lse) HIPCHK(hipMemcpyAsync(st->ysave, Y->ptr, (size_t)qn * Y->esize(), hipMemcpyDeviceToDevice, s));
@@ -1663,7 +1673,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         NEED_L(11, 11);
         AttnState* st = m_attn.get((long)pl[1]);
         if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
-        if (st->dropout > 0.f && st->training) { last_detail = "attention dropout is not part of this path"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const bool drop = st->training && st->dropout > 0.f;
+        if (drop && !st->lseValid) { last_detail = "ATTN_BWD with dropout needs the training-mode forward call whose mask it repeats"; return MCH_ERROR_ATTN_NOT_INITIALIZED; }
         const int T = st->lastTq > 0 ? st->lastTq : st->block, Tk = st->lastTq > 0 ? st->lastTk : st->block;
         const long long batchMask = st->lastTq > 0 ? st->lastBatchMask : 0;
         MemItem *Q, *dQ, *K, *dK, *V, *dV, *Y, *dY, *M = nullptr;
@@ -1704,7 +1715,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         const bool haveY = haveLse && st->ysave && st->ysaveBytes >= (size_t)qn * Y->esize();
         HIPCHK(k_attn_backward(s, Q->dt(), Q->ptr, K->ptr, V->ptr, haveY ? st->ysave : Y->ptr, dY->ptr, dQ->ptr, dK->ptr, dV->ptr, st->batch, st->heads,
                                T, Tk, st->hs, st->scale, M ? (const float*)M->ptr : nullptr, kind, haveLse ? st->lse : nullptr,
-                               ws, wsBytes));
+                               ws, wsBytes, drop ? &st->drop : nullptr));
         m_mem.touch((long)pl[3]);
         m_mem.touch((long)pl[5]);
         m_mem.touch((long)pl[7]);

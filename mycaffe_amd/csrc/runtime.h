@@ -84,6 +84,8 @@ struct AttnState {
     bool set = false, training = false;
     int batch = 0, block = 0, heads = 0, hs = 0;
     float dropout = 0.f, scale = 1.f;
+    uint64_t seed = 0, fwdCalls = 0;   // dropout: seed of ATTN_SET, training-mode forward calls since
+    AttnDropout drop = {0, 0, 1.f};    // mask parameters of the last training-mode forward call
     // cache of "the (T,T) mask is the lower-triangular ones matrix"
     long maskHandle = 0; uint64_t maskVersion = 0; int maskT = 0; bool maskCausal = false;
     // what the backward pass needs of the last training-mode forward: log2 of every row's softmax denominator

@@ -562,6 +562,62 @@ def attn_backward(q, k, v, att, dy, dtype=np.float32):
     return dq.astype(dtype), dk.astype(dtype), dv.astype(dtype)
 
 
+def splitmix64(state):
+    """One output of the SplitMix64 generator for each 64-bit ``state`` (Steele, Lea, Flood, "Fast splittable
+    pseudorandom number generators", OOPSLA 2014; the increment is folded in: out = mix(state + golden))."""
+    with np.errstate(over="ignore"):
+        z = np.asarray(state, np.uint64) + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+ATTN_DROPOUT_CALL_STRIDE = 0xD1B54A32D192ED03   # the HIP handle adds this to the seed for every training-mode forward call
+
+
+def attn_dropout_keep(seed, B, H, Tq, Tk, ratio, forward_calls=1):
+    """Which probabilities survive attention dropout in the HIP library (the reference draws its mask from cuDNN's
+    generator, attn.cu:261-276, whose stream cannot be restated; only the distribution and the forward / backward
+    consistency carry over).  keep[b,h,i,j] = high 32 bits of splitmix64(seed' * golden + index) >= ratio * 2^32 with
+    index = ((b*H + h)*Tq + i)*Tk + j and seed' = seed + forward_calls * ATTN_DROPOUT_CALL_STRIDE."""
+    with np.errstate(over="ignore"):
+        seed2 = np.uint64((int(seed) + forward_calls * ATTN_DROPOUT_CALL_STRIDE) & 0xFFFFFFFFFFFFFFFF)
+        idx = np.arange(B * H * Tq * Tk, dtype=np.uint64)
+        r = splitmix64(seed2 * np.uint64(0x9E3779B97F4A7C15) + idx) >> np.uint64(32)
+    thr = min(int(float(np.float32(ratio)) * 4294967296.0), 4294967295)
+    return (r >= np.uint64(thr)).reshape(B, H, Tq, Tk)
+
+
+def attn_forward_dropout(q, k, v, keep, ratio, mask_data=None, batch_mask=False, dtype=np.float32):
+    """attnHandle::Forward in training mode with a dropout ratio (attn.cu:518-602): dropout is applied in place to the
+    softmax probabilities (survivors scaled by 1 / (1 - ratio)) before the product with V.  Returns (y, probabilities
+    before dropout, probabilities after)."""
+    _, p = attn_forward(q, k, v, mask_data, batch_mask, dtype)
+    pd = (p * (np.asarray(keep, dtype) * dtype(1.0 / (1.0 - float(np.float32(ratio)))))).astype(dtype)
+    return (pd @ np.asarray(v, dtype)).astype(dtype), p, pd
+
+
+def attn_backward_dropout(q, k, v, att_dropped, keep, ratio, dy, dtype=np.float32):
+    """attnHandle::Backward with dropout, step by step as the reference runs it (attn.cu:608-661).  ``att_dropped`` is
+    what m_blobAttB holds after the forward pass: the probabilities with dropout applied IN PLACE (:578-583).
+      dV = AttB^T dY, dAttB = dY V^T                       (matmulgrad, :632-633)
+      dAttB *= keep / (1 - ratio)                          (apply_dropout_bwd, :637-640)
+      dAttA = AttB * (dAttB - rowsum(dAttB * AttB))        (softmax_bwd with y = the dropped AttB, :643-644)
+      dQ = dAttA K / sqrt(hs), dK = dAttA^T Q / sqrt(hs)   (:647-652)
+    Because the softmax backward reads the dropped probabilities, a dropped entry gets no gradient at all and a kept one
+    carries 1 / (1 - ratio)^2; this is the reference's result, not the derivative of its forward pass."""
+    q = np.asarray(q, dtype); k = np.asarray(k, dtype); v = np.asarray(v, dtype)
+    attb = np.asarray(att_dropped, dtype); dy = np.asarray(dy, dtype)
+    scale = dtype(1.0 / np.sqrt(np.float64(q.shape[-1])))
+    dv = np.swapaxes(attb, -1, -2) @ dy
+    datt = dy @ np.swapaxes(v, -1, -2)
+    datt = datt * (np.asarray(keep, dtype) * dtype(1.0 / (1.0 - float(np.float32(ratio)))))
+    ds = softmax_backward(attb, datt, axis=-1, log=False, dtype=dtype) * scale
+    dq = ds @ k
+    dk = np.swapaxes(ds, -1, -2) @ q
+    return dq.astype(dtype), dk.astype(dtype), dv.astype(dtype)
+
+
 def transformer_block_gpt(x, p, heads, activation="relu", eps=1e-10, dtype=np.float32):
     """TransformerBlockLayer.forward, CAUSAL_SELF_ATTENTION block type (TransformerBlockLayer.cs:810-902):
     xB = x + attn(ln1(x)); y = xB + proj(gelu(fc(ln2(xB)))).  ``p`` maps attn_weight, attn_bias, attn_proj_weight,

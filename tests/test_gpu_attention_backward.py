@@ -158,3 +158,86 @@ def test_causal_launch_order_does_not_change_results(dev, half):
         small = _fwd_bwd(dev, q[sl], k[sl], v[sl], dy[sl], mask, 0, half)
         for got, exp, name in zip(big, small, ("y", "dq", "dk", "dv")):
             assert np.array_equal(got[sl], exp), name
+
+
+# ---- attention dropout: training mode of the handle with a ratio (attn.cu:455-486, 578-583, 637-640) ---------------
+
+def _dropout_case(dev, B, H, Tq, Tk, hs, ratio, seed, mask, batch_mask, half, calls=1):
+    rng = np.random.default_rng(seed)
+    rnd = bf16_round if half else (lambda a: a)
+    q, dy = (rnd(rng.standard_normal((B, H, Tq, hs)).astype(np.float32)) for _ in range(2))
+    k, v = (rnd(rng.standard_normal((B, H, Tk, hs)).astype(np.float32)) for _ in range(2))
+    hc, ha = dev.cuda.CreateCuDNN(), dev.cuda.CreateAttn()
+    dev.cuda.SetAttn(hc, ha, 0, True, B, max(Tq, Tk), H, hs, ratio, seed)
+    hq, hk, hv, hy, hdy = dev.put(q, half), dev.put(k, half), dev.put(v, half), dev.zeros(q.size, half), dev.put(dy, half)
+    hdq, hdk, hdv = dev.zeros(q.size, half), dev.zeros(k.size, half), dev.zeros(k.size, half)
+    hm = dev.put(mask) if mask is not None else 0
+    ys = []
+    for _ in range(calls):
+        dev.cuda.AttnScaledDotProductForward(hc, ha, Tq, hq, hk, hv, hm, hy, batch_mask, Tk if Tk != Tq else None)
+        ys.append(dev.get(hy, q.shape))
+    dev.cuda.AttnScaledDotProductBackward(hc, ha, hq, hdq, hk, hdk, hv, hdv, hm, hy, hdy)
+    got = ys, dev.get(hdq, q.shape), dev.get(hdk, k.shape), dev.get(hdv, k.shape)
+    dev.cuda.FreeAttn(ha)
+    dev.cuda.FreeCuDNN(hc)
+    # checker: probabilities in fp64, the library's mask generator, the reference's step sequence
+    p = _probs(q, k, mask, batch_mask)
+    exp_y, keep = [], None
+    for c in range(1, calls + 1):
+        keep = R.attn_dropout_keep(seed, B, H, Tq, Tk, ratio, forward_calls=c)
+        pd = p * keep / (1.0 - float(np.float32(ratio)))
+        exp_y.append(pd @ np.asarray(v, np.float64))
+    grads = R.attn_backward_dropout(q, k, v, pd, keep, ratio, dy, np.float64)
+    return got, exp_y, grads
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("B,H,Tq,Tk,hs,ratio,kind", [(2, 3, 70, 70, 64, 0.1, "causal"), (1, 2, 130, 130, 128, 0.5, "causal"),
+                                                     (2, 2, 33, 50, 48, 0.25, "none"), (3, 2, 40, 40, 64, 0.3, "key"),
+                                                     (2, 2, 24, 24, 16, 0.2, "bqk")])
+def test_attn_dropout_forward_and_backward(dev, B, H, Tq, Tk, hs, ratio, kind, half):
+    rng = np.random.default_rng(3)
+    mask, bm = None, 0
+    if kind == "causal":
+        mask = np.tril(np.ones((Tq, Tk), np.float32))
+    elif kind == "key":
+        mask, bm = (rng.random((B, Tk)) > 0.3).astype(np.float32), 1
+        mask[:, 0] = 1
+    elif kind == "bqk":
+        mask, bm = (rng.random((B, Tq, Tk)) > 0.3).astype(np.float32), 2
+        mask[:, :, 0] = 1
+    tol = BF16_RTOL if half else FP32_RTOL
+    (ys, dq, dk, dv), exp_y, (edq, edk, edv) = _dropout_case(dev, B, H, Tq, Tk, hs, ratio, 1234, mask, bm, half)
+    what = "dropout %.2f %s hs %d" % (ratio, kind, hs)
+    assert_close(ys[0], exp_y[0], tol, what + " y")
+    assert_close(dq, edq, tol, what + " dq")
+    assert_close(dk, edk, tol, what + " dk")
+    assert_close(dv, edv, tol, what + " dv")
+
+
+def test_attn_dropout_draws_a_new_mask_per_forward_call_and_backward_repeats_the_last(dev):
+    (ys, dq, dk, dv), exp_y, (edq, edk, edv) = _dropout_case(dev, 2, 2, 48, 48, 64, 0.4, 77, np.tril(np.ones((48, 48), np.float32)), 0,
+                                                              False, calls=3)
+    for c in range(3):
+        assert_close(ys[c], exp_y[c], FP32_RTOL, "forward call %d" % (c + 1))
+    assert np.abs(ys[0] - ys[1]).max() > 1e-2 and np.abs(ys[1] - ys[2]).max() > 1e-2
+    assert_close(dq, edq, FP32_RTOL, "dq after three forward calls")
+    assert_close(dk, edk, FP32_RTOL, "dk after three forward calls")
+    assert_close(dv, edv, FP32_RTOL, "dv after three forward calls")
+
+
+def test_attn_dropout_is_ignored_outside_training_and_checked_at_set(dev):
+    rng = np.random.default_rng(5)
+    B, H, T, hs = 2, 2, 40, 64
+    q, k, v = (rng.standard_normal((B, H, T, hs)).astype(np.float32) for _ in range(3))
+    m = np.tril(np.ones((T, T), np.float32))
+    hc, ha = dev.cuda.CreateCuDNN(), dev.cuda.CreateAttn()
+    dev.cuda.SetAttn(hc, ha, 0, False, B, T, H, hs, 0.5, 9)   # inference: the ratio has no effect (attn.cu:578)
+    hq, hk, hv, hy, hm = dev.put(q), dev.put(k), dev.put(v), dev.zeros(q.size), dev.put(m)
+    dev.cuda.AttnScaledDotProductForward(hc, ha, T, hq, hk, hv, hm, hy, False)
+    assert_close(dev.get(hy, q.shape), _probs(q, k, m, 0) @ v.astype(np.float64), FP32_RTOL, "inference with a ratio set")
+    from mycaffe_amd.cudadnn import CudaDnnError
+    with pytest.raises(CudaDnnError):
+        dev.cuda.SetAttn(hc, ha, 0, True, B, T, H, hs, 1.0, 9)
+    dev.cuda.FreeAttn(ha)
+    dev.cuda.FreeCuDNN(hc)

@@ -525,3 +525,66 @@ def test_softmax_chain_equals_scipy(axis):
     x = np.random.default_rng(1).standard_normal((4, 6, 5)).astype(np.float32) * 3
     assert np.allclose(R.softmax_caffe_chain(x, axis, dtype=np.float64), softmax(x.astype(np.float64), axis=axis), rtol=1e-12)
     assert np.allclose(R.softmax_caffe_chain(x, axis, log=True, dtype=np.float64), log_softmax(x.astype(np.float64), axis=axis), rtol=1e-10, atol=1e-12)
+
+
+# ---- attention dropout (training mode of the attention handle) ------------------------------------------------------
+
+def test_splitmix64_known_answers():
+    # the generator's published outputs for seed 1234567 (first five draws; the state advances by the golden increment)
+    G = 0x9E3779B97F4A7C15
+    st = np.array([(1234567 + i * G) & (2 ** 64 - 1) for i in range(5)], np.uint64)
+    assert [int(x) for x in R.splitmix64(st)] == [6457827717110365317, 3203168211198807973, 9817491932198370423,
+                                                  4593380528125082431, 16408922859458223821]
+
+
+@pytest.mark.parametrize("ratio", [0.1, 0.25, 0.5])
+def test_attn_dropout_mask_statistics(ratio):
+    keep = R.attn_dropout_keep(99, 4, 6, 64, 80, ratio)
+    n = keep.size
+    sigma = np.sqrt(ratio * (1 - ratio) / n)
+    assert abs(keep.mean() - (1 - ratio)) < 4 * sigma
+    # rows and columns are not correlated with each other, and another call of the forward pass draws another mask
+    assert abs(np.corrcoef(keep[..., :-1].ravel(), keep[..., 1:].ravel())[0, 1]) < 0.01
+    assert abs(np.corrcoef(keep[:, :, :-1].ravel(), keep[:, :, 1:].ravel())[0, 1]) < 0.01
+    again = R.attn_dropout_keep(99, 4, 6, 64, 80, ratio, forward_calls=2)
+    assert abs(np.corrcoef(keep.ravel(), again.ravel())[0, 1]) < 0.01
+    assert np.array_equal(R.attn_dropout_keep(99, 4, 6, 64, 80, ratio), keep)
+
+
+def test_attn_forward_dropout_is_unbiased_and_reduces_to_the_plain_forward():
+    rng = np.random.default_rng(0)
+    B, H, T, hs = 1, 2, 24, 8
+    q, k, v = (rng.standard_normal((B, H, T, hs)) for _ in range(3))
+    m = R.causal_mask(T, np.float64)
+    y0, p0 = R.attn_forward(q, k, v, m, False, np.float64)
+    y, p, pd = R.attn_forward_dropout(q, k, v, np.ones((B, H, T, T), bool), 0.0, m, False, np.float64)
+    assert np.array_equal(y, y0) and np.array_equal(p, p0) and np.array_equal(pd, p0)
+    acc = np.zeros_like(y0)
+    n = 600
+    for seed in range(n):
+        acc += R.attn_forward_dropout(q, k, v, R.attn_dropout_keep(seed, B, H, T, T, 0.3), 0.3, m, False, np.float64)[0]
+    # the mean over masks is the undropped output (error shrinks as 1 / sqrt(n))
+    assert np.abs(acc / n - y0).max() < 6 * np.abs(v).max() * np.sqrt(0.3 / 0.7 / n)
+
+
+def test_attn_backward_dropout_sequence_and_its_closed_form():
+    """The reference's step sequence (softmax backward on the probabilities dropout was applied to in place) collapses to
+    dS = keep / (1 - r)^2 * P * (dP - dY.Y), dV = (P keep / (1 - r))^T dY, which is what the HIP kernels compute from the
+    regenerated mask; with no dropout it is the plain backward pass (itself pinned on torch autograd)."""
+    rng = np.random.default_rng(1)
+    B, H, T, hs, r = 2, 2, 20, 8, 0.25
+    q, k, v, dy = (rng.standard_normal((B, H, T, hs)) for _ in range(4))
+    m = R.causal_mask(T, np.float64)
+    keep = R.attn_dropout_keep(5, B, H, T, T, r)
+    y, p, pd = R.attn_forward_dropout(q, k, v, keep, r, m, False, np.float64)
+    dq, dk, dv = R.attn_backward_dropout(q, k, v, pd, keep, r, dy, np.float64)
+    dP = dy @ np.swapaxes(v, -1, -2)
+    D = (dy * y).sum(-1, keepdims=True)
+    dS = keep / (1 - r) ** 2 * p * (dP - D) / np.sqrt(hs)
+    assert np.allclose(dq, dS @ k, rtol=1e-12, atol=1e-12)
+    assert np.allclose(dk, np.swapaxes(dS, -1, -2) @ q, rtol=1e-12, atol=1e-12)
+    assert np.allclose(dv, np.swapaxes(pd, -1, -2) @ dy, rtol=1e-12, atol=1e-12)
+    ones = np.ones_like(keep)
+    y1, p1, pd1 = R.attn_forward_dropout(q, k, v, ones, 0.0, m, False, np.float64)
+    for a, b in zip(R.attn_backward_dropout(q, k, v, pd1, ones, 0.0, dy, np.float64), R.attn_backward(q, k, v, p1, dy, np.float64)):
+        assert np.allclose(a, b, rtol=1e-12, atol=1e-12)
