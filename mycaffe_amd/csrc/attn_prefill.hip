@@ -362,12 +362,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
     // key take the unmasked path.  A sequence with no valid key at all keeps every step (uniform weights, as the
     // reference's -1e29 fill gives).
     bool seqValid = false;
+    gload(0);   // requested before the mask scan, so that the two trips to memory overlap
     if (KIND == 2) {
         int any = 0;
         for (int t = tid; t < a.Tk; t += NT) any |= a.mask[(size_t)b * a.Tk + t] != 0.f;
         seqValid = __syncthreads_or(any) != 0;
     }
-    gload(0);
     sstore(0);
     // make the Q fragments "used" here, so the wait for their loads sits before the loop and the
     // loop body never waits on the memory counter that the next block's prefetch shares
@@ -431,14 +431,17 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
                             const int kl = 8 * (v >> 2) + 4 * half + (v & 3);
                             const int key = k0 + kl;
                             float sv = s[qt][v];
-                            if (KIND == 1 && key > qrow) sv = a.maskedRaw;
+                            // causal: every row of a diagonal step keeps at least its own key, so the masked scores
+                            // can simply be -inf (weight exactly 0) and the step takes the plain softmax path
+                            if (KIND == 1 && key > qrow) sv = -INFINITY;
                             if (KIND == 2 && Ms[32 * sub + kl] == 0.f) sv = a.maskedRaw;
                             if (KIND == 3 && qrow < a.Tq && key < a.Tk && mk[v] == 0.f) sv = a.maskedRaw;
                             if (key >= a.Tk) sv = -INFINITY;
                             s[qt][v] = sv;
                         }
                     }
-                    flash_softmax_step<true, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
+                    if (KIND == 1) flash_softmax_step<false, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
+                    else flash_softmax_step<true, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
                 } else {
                     flash_softmax_step<false, DT, QT>(s, o, m, l, c, a.maskedRaw, a.lazy);
                 }

@@ -583,21 +583,6 @@ __global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float
     }
 }
 
-// (B,H,P,hs) -> (B*P, H*hs)
-__global__ void prefill_merge_heads_kernel(const float* __restrict__ y, float* __restrict__ out, int B, int P, int H, int hs)
-{
-    const int q = hs / 4;
-    const size_t total = (size_t)B * P * H * q;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
-        const int d4 = (int)(i % q);
-        size_t t = i / q;
-        const int h = (int)(t % H);
-        t /= H;
-        const int p = (int)(t % P), b = (int)(t / P);
-        *(float4*)(out + (((size_t)b * P + p) * H + h) * hs + d4 * 4) = *(const float4*)(y + (((size_t)b * H + h) * P + p) * hs + d4 * 4);
-    }
-}
-
 // hb[m, j] = silu(h2[m, j]) * h2[m, hid + j], the epilogue of the decode path's W1|W3 mat-vec
 __global__ void prefill_swiglu_kernel(const float* __restrict__ h2, float* __restrict__ hb, size_t rows, int hid)
 {
@@ -839,7 +824,7 @@ private:
     // batched prompt pass: activations of rows = sequences x prompt positions, sized for pfRows
     size_t pfRows = 0, pfLogitRows = 0;
     std::vector<void*> prefillAllocs;
-    float *pfX = nullptr, *pfXn = nullptr, *pfQkv = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr, *pfY = nullptr,
+    float *pfX = nullptr, *pfXn = nullptr, *pfQkv = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr,
           *pfH2 = nullptr, *pfHb = nullptr, *pfLogits = nullptr, *pfW = nullptr;
 };
 
@@ -1065,11 +1050,11 @@ long Engine::ensure_prefill(size_t rows)
     // the classifier runs over at most 512 MB of logits at a time
     pfLogitRows = std::max<size_t>(1, std::min(rows, ((size_t)128 << 20) / V));
     pfX = pa(rows * dim); pfXn = pa(rows * dim); pfQkv = pa(rows * (dim + 2 * kvd));
-    pfQ = pa(rows * dim); pfK = pa(rows * dim); pfV = pa(rows * dim); pfY = pa(rows * dim);
+    pfQ = pa(rows * dim); pfK = pa(rows * dim); pfV = pa(rows * dim);
     pfH2 = pa(rows * 2 * hid); pfHb = pa(rows * hid); pfLogits = pa(pfLogitRows * V);
     // weights stored as bf16 are widened to fp32 one matrix at a time: room for the largest one
     pfW = stored_bf16 ? pa(std::max({(dim + 2 * kvd) * dim, 2 * hid * dim, V * dim})) : pfX;
-    if (!pfX || !pfXn || !pfQkv || !pfQ || !pfK || !pfV || !pfY || !pfH2 || !pfHb || !pfLogits || !pfW) return MCH_ERROR_MEMORY_OUT;
+    if (!pfX || !pfXn || !pfQkv || !pfQ || !pfK || !pfV || !pfH2 || !pfHb || !pfLogits || !pfW) return MCH_ERROR_MEMORY_OUT;
     pfRows = rows;
     return 0;
 }
