@@ -11,6 +11,8 @@
 //  * flash kernels (attn_flash_*.inc) - MFMA tiles for hs in {64, 128}.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "flash_traits.h"
 #include "kernels.h"
 
@@ -172,6 +174,7 @@ struct FlashArgs {
     float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
     float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
     int yMerged;         // y laid out (B,Tq,H,hs) instead of (B,H,Tq,hs)
+    int causalGroup;     // causal launches: heads per group of the workgroup order (0: all heads in one group)
 };
 
 __device__ __forceinline__ float flash_half_max(float v)
@@ -274,8 +277,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
         const int nbh = a.B * a.H;
         const int nqb = (a.Tq + BM - 1) / BM;
         const int rank = flash_causal_rank(OCC);
-        qblock = nqb - 1 - rank / nbh;
-        const int ibh = rank % nbh;
+        int ibh;
+        flash_causal_map(rank, nbh, nqb, a.causalGroup, &qblock, &ibh);
         b = ibh / a.H;
         h = ibh % a.H;
     } else {
@@ -806,6 +809,256 @@ __global__ __launch_bounds__(256, 3) void flash_pipe_bf16_64_kernel(FlashArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same software pipeline for head size 128 (bf16, no mask or causal): eight wavefronts of one 32-row tile each,
+// K and V row-major and double buffered in dynamic LDS (V^T fragments through the transposing read).  A phase is
+// sixteen MFMA slots - eight of O^T += V^T P^T of step t - 1, then eight of S^T of step t + 1 - and the softmax of
+// step t, the fragment reads two slots ahead and the K / V staging traffic ride along, one slice per slot.
+template <int KIND>
+__global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a)
+{
+    typedef FlashTraits<bf16_t> TR;
+    constexpr int HS = 128, BN = 64, NT = 512, BM = 256, LDK = HS + 8, LDVR = HS + 16;
+    constexpr int KBUF = BN * LDK, VBUF = BN * LDVR;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pipe_smem[];
+    bf16_t* Ks = reinterpret_cast<bf16_t*>(pipe_smem);   // [2][KBUF]
+    bf16_t* Vs = Ks + 2 * KBUF;                          // [2][VBUF]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    int qblock, h, b;
+    if (KIND == 1) {
+        const int nbh = a.B * a.H;
+        const int nqb = (a.Tq + BM - 1) / BM;
+        const int rank = flash_causal_rank(1);
+        int ibh;
+        flash_causal_map(rank, nbh, nqb, a.causalGroup, &qblock, &ibh);
+        b = ibh / a.H;
+        h = ibh % a.H;
+    } else {
+        qblock = blockIdx.x;
+        h = blockIdx.y;
+        b = blockIdx.z;
+    }
+    const size_t bh = (size_t)b * a.H + h;
+    const int q0 = qblock * BM + wave * 32;
+    const bf16_t* qp = (const bf16_t*)a.q + bh * a.Tq * HS;
+    const bf16_t* kp = (const bf16_t*)a.k + bh * a.Tk * HS;
+    const bf16_t* vp = (const bf16_t*)a.v + bh * a.Tk * HS;
+
+    u32x4 qf[8];
+    {
+        const int row = min(q0 + l32, a.Tq - 1);
+#pragma unroll
+        for (int f = 0; f < 8; f++) qf[f] = *(const u32x4*)(qp + (size_t)row * HS + f * 16 + half * 8);
+    }
+    int kend = a.Tk;
+    if (KIND == 1) kend = min(a.Tk, qblock * BM + BM);
+    const int nkb = (kend + BN - 1) / BN;
+    int nstw = min(2 * nkb, (a.Tk + 31) / 32);             // steps this wavefront computes
+    if (KIND == 1) nstw = min(nstw, (q0 + 31) / 32 + 1);
+    if (q0 >= a.Tq) nstw = 0;
+
+    // staging: chunk e = tid + 512 i of a block -> key e / 16, 16-byte chunk e % 16 (K and V alike)
+    // two register sets per operand (set = block & 1): a block is requested three phases before it is written to LDS
+    u32x4 kreg[2][2], vreg[2][2];
+    const int srow[2] = {tid / 16, (tid + NT) / 16}, scol = (tid % 16) * 8;
+    auto gaddr = [&](const bf16_t* base, int kb, int i) { return base + (size_t)min(kb * BN + srow[i], a.Tk - 1) * HS + scol; };
+    auto kstore = [&](int buf, const u32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) *(u32x4*)(Ks + buf * KBUF + srow[i] * LDK + scol) = r[i];
+    };
+    auto vstore = [&](int buf, const u32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) *(u32x4*)(Vs + buf * VBUF + srow[i] * LDVR + scol) = r[i];
+    };
+
+    floatx16 o[4][1];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[dt][0][v] = 0.f;
+    float m[1] = {-INFINITY}, l[1] = {0.f};
+    const float c = a.c, lazy = a.lazy;
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const bf16_t* kfrag = Ks + l32 * LDK + half * 8;
+
+    // fragment j of a phase around step t: 0..7 = V^T fragments of step t - 1 (key half j / 4, dim tile j % 4),
+    // 8..15 = K fragments of step t + 1
+    auto frag = [&](int j, int t) -> u32x4 {
+        if (j < 8) {
+            const int tv = t - 1;
+            return TR::load_vt_rowmajor(Vs + ((tv >> 1) & 1) * VBUF + 32 * (tv & 1) * LDVR + (j & 3) * 32, LDVR, j >> 2, lane);
+        }
+        const int ts = t + 1;
+        return *(const u32x4*)(kfrag + ((ts >> 1) & 1) * KBUF + (ts & 1) * 32 * LDK + (j - 8) * 16);
+    };
+    auto smma = [&](int t, floatx16& sn) {      // S^T of step t
+        const bf16_t* kb_ = kfrag + ((t >> 1) & 1) * KBUF + (t & 1) * 32 * LDK;
+        sn = TR::mma(*(const u32x4*)(kb_), qf[0], zero16);
+#pragma unroll
+        for (int f = 1; f < 8; f++) sn = TR::mma(*(const u32x4*)(kb_ + 16 * f), qf[f], sn);
+    };
+    auto pvmma = [&](int t, const u32x4 (&pp)[2]) {   // O^T += V^T P^T of step t
+        const bf16_t* vb_ = Vs + ((t >> 1) & 1) * VBUF + 32 * (t & 1) * LDVR;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) o[dt][0] = TR::mma(TR::load_vt_rowmajor(vb_ + dt * 32, LDVR, tt, lane), pp[tt], o[dt][0]);
+    };
+    // sequential softmax of step t (any masking), leaves the packed weights in pc
+    auto soft_slow = [&](int t, floatx16 (&sc)[1], u32x4 (&pc)[2]) {
+        const int k0 = t * 32;
+        const bool masked = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk);
+        if (masked) {
+            const int qrow = q0 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+                // every row of such a step keeps at least one key (its own, or key k0 < Tk), so -inf is safe
+                if ((KIND == 1 && key > qrow) || key >= a.Tk) sc[0][v] = -INFINITY;
+            }
+        }
+        flash_softmax_step<false, 4, 1>(sc, o, m, l, c, a.maskedRaw, lazy);
+        pc[0] = TR::pack_p(sc[0], 0);
+        pc[1] = TR::pack_p(sc[0], 1);
+    };
+
+    // prologue: K(0), V(0) in LDS, K(1), K(2) and V(1) in registers, S^T of step 0
+#pragma unroll
+    for (int i = 0; i < 2; i++) { kreg[0][i] = *(const u32x4*)gaddr(kp, 0, i); vreg[0][i] = *(const u32x4*)gaddr(vp, 0, i); }
+    kstore(0, kreg[0]);
+    vstore(0, vreg[0]);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        kreg[1][i] = *(const u32x4*)gaddr(kp, 1, i);
+        kreg[0][i] = *(const u32x4*)gaddr(kp, 2, i);
+        vreg[1][i] = *(const u32x4*)gaddr(vp, 1, i);
+    }
+#pragma unroll
+    for (int f = 0; f < 8; f++) asm volatile("" : "+v"(qf[f]));
+    __syncthreads();
+    floatx16 sA[1], sB[1];
+    u32x4 pA[2], pB[2];
+    sA[0] = zero16;
+    sB[0] = zero16;
+    pA[0] = pA[1] = pB[0] = pB[1] = u32x4{0u, 0u, 0u, 0u};
+    if (nstw > 0) smma(0, sA[0]);
+
+    // One phase of block kb = t / 2, P = kb & 1.  ROLE 0 (even phase 2 kb): request V(kb + 2) into set P, write K(kb + 1)
+    // from set 1 - P to LDS; ROLE 1 (odd phase 2 kb + 1): request K(kb + 3) into set 1 - P (just written out), write
+    // V(kb + 1) from set 1 - P.  sc: scores of step t (in), sn: scores of step t + 1 (out), pp: packed weights of step
+    // t - 1 (in), pc: packed weights of step t (out).  Blocks past the end re-read the last rows (never consumed).
+    auto phase = [&](auto role_, auto par_, int t, floatx16 (&sc)[1], floatx16 (&sn)[1], const u32x4 (&pp)[2], u32x4 (&pc)[2]) {
+        constexpr int ROLE = decltype(role_)::value, P = decltype(par_)::value;
+        const int kbn = (ROLE == 0) ? (t >> 1) + 2 : (t >> 1) + 3;     // block requested in this phase
+        const int wbuf = ((t >> 1) + 1) & 1;                           // LDS buffer written in this phase: block kb + 1
+        u32x4 (&fetch)[2] = ROLE == 0 ? vreg[P] : kreg[1 - P];
+        const u32x4 (&put)[2] = ROLE == 0 ? kreg[1 - P] : vreg[1 - P];
+        const bool doSoft = t < nstw, doS = t + 1 < nstw, doPV = t >= 1 && t - 1 < nstw;
+        const bool plain = !((KIND == 1) && (t * 32 + 31 > q0)) && (t * 32 + 32 <= a.Tk);
+        if (doSoft && doS && doPV && plain) {
+            u32x4 fr[16];
+            fr[0] = frag(0, t);
+            fr[1] = frag(1, t);
+            float m1 = 0.f, m2 = 0.f, m3 = 0.f, m4 = 0.f, mx = 0.f, alpha = 1.f, mc = 0.f, rs = 0.f, pw[16];
+            uint32_t pk[8];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                if (j < 8) o[j & 3][0] = TR::mma(fr[j], pp[j >> 2], o[j & 3][0]);
+                else sn[0] = TR::mma(fr[j], qf[j - 8], j == 8 ? zero16 : sn[0]);
+                if (j + 2 < 16) fr[j + 2] = frag(j + 2, t);
+                // softmax of step t, one slice per slot
+                if (j == 0) {
+                    m1 = fmaxf(fmaxf(sc[0][0], sc[0][1]), sc[0][2]);
+                    m2 = fmaxf(fmaxf(sc[0][3], sc[0][4]), sc[0][5]);
+                    m3 = fmaxf(fmaxf(sc[0][6], sc[0][7]), sc[0][8]);
+                    m4 = fmaxf(fmaxf(sc[0][9], sc[0][10]), sc[0][11]);
+                    asm volatile("" : "+v"(m1), "+v"(m2), "+v"(m3), "+v"(m4));
+                } else if (j == 1) {
+                    const float m5 = fmaxf(fmaxf(sc[0][12], sc[0][13]), sc[0][14]);
+                    mx = fmaxf(fmaxf(m1, m2), m3);
+                    mx = fmaxf(fmaxf(mx, m4), m5);
+                    mx = fmaxf(mx, sc[0][15]);
+                    mx = flash_half_max(mx);
+                    asm volatile("" : "+v"(mx));
+                } else if (j == 2) {
+                    const float mnew = (mx > m[0] + lazy) ? mx : m[0];
+                    alpha = __builtin_amdgcn_exp2f((m[0] - mnew) * c);
+                    mc = mnew * c;
+                    m[0] = mnew;
+                    asm volatile("" : "+v"(alpha), "+v"(mc), "+v"(m[0]));
+                } else if (j <= 10) {
+                    const int e = 2 * (j - 3);
+                    pw[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e], c, -mc));
+                    pw[e + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e + 1], c, -mc));
+                    rs += pw[e] + pw[e + 1];
+                    asm volatile("" : "+v"(pw[e]), "+v"(pw[e + 1]), "+v"(rs));
+                } else if (j <= 14) {
+                    const int w = 2 * (j - 11);
+                    pk[w] = pack_bf16x2(pw[2 * w], pw[2 * w + 1]);
+                    pk[w + 1] = pack_bf16x2(pw[2 * w + 2], pw[2 * w + 3]);
+                    asm volatile("" : "+v"(pk[w]), "+v"(pk[w + 1]));
+                } else {
+                    l[0] = l[0] * alpha + rs;
+                    asm volatile("" : "+v"(l[0]));
+                }
+                // K / V staging traffic of this phase
+                if (j == 12 || j == 13) {
+                    const int i = j - 12;
+                    if (ROLE == 0) *(u32x4*)(Ks + wbuf * KBUF + srow[i] * LDK + scol) = put[i];
+                    else *(u32x4*)(Vs + wbuf * VBUF + srow[i] * LDVR + scol) = put[i];
+                } else if (j == 14 || j == 15) {
+                    // the set that ROLE 1 refills is the one ROLE 0 emptied a phase ago; ROLE 0 refills a set that the
+                    // previous odd phase emptied: requests go after this phase's LDS writes in program order
+                    fetch[j - 14] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, j - 14);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            pc[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+            pc[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
+            if (!__all(alpha == 1.0f)) {
+#pragma unroll
+                for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) o[dt][0][v] *= alpha;
+            }
+        } else {
+            if (doPV) pvmma(t - 1, pp);
+            if (doSoft) soft_slow(t, sc, pc);
+            if (doS) smma(t + 1, sn[0]);
+            if (ROLE == 1) vstore(wbuf, put);
+            else kstore(wbuf, put);
+#pragma unroll
+            for (int i = 0; i < 2; i++) fetch[i] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, i);
+        }
+        __syncthreads();
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    for (int kb = 0; kb <= nkb; kb += 2) {
+        phase(I0{}, I0{}, 2 * kb, sA, sB, pB, pA);
+        if (kb < nkb) phase(I1{}, I0{}, 2 * kb + 1, sB, sA, pA, pB);
+        if (kb + 1 <= nkb) phase(I0{}, I1{}, 2 * kb + 2, sA, sB, pB, pA);
+        if (kb + 1 < nkb) phase(I1{}, I1{}, 2 * kb + 3, sB, sA, pA, pB);
+    }
+
+    // epilogue: y[query, dim] = O^T[dim, query] / l
+    const int qrow = q0 + l32;
+    const float lt = l[0] + __shfl_xor(l[0], 32, 64);
+    const float inv = 1.0f / lt;
+    if (qrow < a.Tq) {
+        bf16_t* yr = (bf16_t*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, qrow, HS);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                TR::store4(yr + 32 * dt + 8 * g + 4 * half, o[dt][0][4 * g] * inv, o[dt][0][4 * g + 1] * inv,
+                           o[dt][0][4 * g + 2] * inv, o[dt][0][4 * g + 3] * inv);
+    }
+}
+
 template <typename T, int HS, int QT, int NW, int OCC, bool PREFETCH>
 static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
 {
@@ -833,6 +1086,14 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     f.lazy = 8.0f / f.c;
     f.lse2 = a.lse2;
     f.yMerged = a.yMerged;
+    f.causalGroup = 0;
+    if (a.kind == MASK_CAUSAL && a.hs == 128 && dt == BF16) {
+        // when K and V of all heads together exceed what the caches hold (128 MB taken as the line), walk the heads in
+        // at most four groups of a multiple of 8 heads
+        const long long nbh = (long long)a.B * a.H;
+        const double kvBytes = 2.0 * nbh * a.Tk * a.hs * 2;
+        if (kvBytes > 128e6 && nbh % 8 == 0) f.causalGroup = (int)(((nbh + 3) / 4 + 7) / 8 * 8);
+    }
     *handled = true;
     // Tile shapes picked by measurement on MI355X.  Head size 64: four wavefronts with one 32-row tile each
     // (128-row workgroups) give enough equal-sized workgroups to balance 256 CUs at T = 1024; head size 128
@@ -847,6 +1108,22 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
                 return hipGetLastError();
             }
             return flash_launch_cfg<bf16_t, 64, 1, 4, 3, true>(s, f, a.kind);
+        }
+        // no mask or causal, inference: the software-pipelined kernel (it does not keep the row statistics).  Measured at
+        // B=4, T=4096, 32 heads: unmasked 1.57 -> 1.31 ms, causal 0.80 -> 0.76 ms with the grouped head order.
+        if ((a.kind == MASK_NONE || a.kind == MASK_CAUSAL) && !a.lse2) {
+            constexpr int LDSB = 2 * (64 * 136 + 64 * 144) * 2;
+            static bool attr = false;
+            if (!attr) {
+                hipError_t e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e != hipSuccess) return e;
+                attr = true;
+            }
+            const int nqb = (f.Tq + 255) / 256;
+            if (a.kind == MASK_CAUSAL) hipLaunchKernelGGL(flash_pipe_bf16_128_kernel<1>, dim3(nqb * f.H * f.B), 512, LDSB, s, f);
+            else hipLaunchKernelGGL(flash_pipe_bf16_128_kernel<0>, dim3(nqb, f.H, f.B), 512, LDSB, s, f);
+            return hipGetLastError();
         }
         return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
     }

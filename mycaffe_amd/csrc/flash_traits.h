@@ -142,4 +142,23 @@ __device__ __forceinline__ int flash_causal_rank(int occ)
     return (((r << 5) + width - 1 - c) << 3) + x;
 }
 
+// (query block, head index) of rank r of a causal launch.  Heads are taken in groups of `group` (a multiple of 8, so a
+// head keeps its die): within a group heaviest query block first across the group's heads, then the next group.  Fewer
+// heads in flight at a time keep their K and V in the caches while their query blocks run; with at most four groups the
+// last group's heaviest blocks still start early enough not to stick out at the end.  group >= nbh is the plain
+// heaviest-first order over all heads.
+__device__ __forceinline__ void flash_causal_map(int rank, int nbh, int nqb, int group, int* qblock, int* ibh)
+{
+    if (group <= 0 || group >= nbh) {
+        *qblock = nqb - 1 - rank / nbh;
+        *ibh = rank % nbh;
+        return;
+    }
+    const int per = group * nqb;
+    const int g = rank / per, r = rank - g * per;
+    const int width = min(group, nbh - g * group);   // the last group may be short
+    *qblock = nqb - 1 - r / width;
+    *ibh = g * group + r % width;
+}
+
 }  // namespace mch

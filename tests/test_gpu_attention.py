@@ -40,8 +40,11 @@ def test_attn_forward_causal_fp32(dev, B, H, T, hs):
         assert_close(out, v, 1e-6, "T=1 returns V")
 
 
-@pytest.mark.parametrize("B,H,T,hs", [(3, 8, 200, 64), (2, 4, 256, 64), (2, 2, 256, 128)])
+@pytest.mark.parametrize("B,H,T,hs", [(3, 8, 200, 64), (2, 4, 256, 64), (2, 2, 256, 128), (2, 3, 777, 128), (1, 2, 1024, 128),
+                                      (1, 2, 33, 128), (1, 1, 300, 128)])
 def test_attn_forward_causal_bf16(dev, B, H, T, hs):
+    # head size 128 takes the software-pipelined kernel: 256-row workgroups, so T = 777 has full, diagonal, ragged and
+    # idle wavefronts, T = 33 never reaches a steady-state phase
     rng = np.random.default_rng(T + 1)
     q, k, v = (bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(3))
     out = _attn(dev, q, k, v, R.causal_mask(T), False, half=True)
@@ -79,7 +82,8 @@ def test_attn_forward_arbitrary_qk_mask_and_no_mask(dev):
 
 @pytest.mark.parametrize("half", [True, False])
 @pytest.mark.parametrize("B,H,Tq,Tk,hs", [(2, 3, 64, 64, 64), (1, 2, 100, 100, 64), (2, 2, 257, 257, 64), (1, 4, 1024, 1024, 64),
-                                          (2, 2, 128, 320, 64), (1, 2, 33, 500, 64), (1, 2, 192, 192, 128)])
+                                          (2, 2, 128, 320, 64), (1, 2, 33, 500, 64), (1, 2, 192, 192, 128), (2, 2, 700, 700, 128),
+                                          (1, 3, 130, 777, 128), (1, 2, 520, 95, 128)])
 def test_attn_forward_unmasked(dev, half, B, H, Tq, Tk, hs):
     # no mask: bf16 / head size 64 takes the software-pipelined kernel (steady-state phases need > 3 key steps,
     # ragged lengths end in its sequential phases); T_q != T_k is cross attention
@@ -89,6 +93,22 @@ def test_attn_forward_unmasked(dev, half, B, H, Tq, Tk, hs):
     out = _attn(dev, q, k, v, None, False, half)
     ref, _ = R.attn_forward(q, k, v, None, False, np.float64)
     assert_close(out, ref, BF16_RTOL if half else FP32_RTOL, "attn unmasked")
+
+
+def test_attn_forward_large_scores_rescale_in_the_pipelined_head_size_128_kernel(dev):
+    # as below for bf16, head size 128: a key far above the running maximum late in the range forces the rescale of the
+    # output accumulators inside a steady-state phase of the pipelined kernel
+    rng = np.random.default_rng(6)
+    B, H, T, hs = 1, 2, 640, 128
+    q = bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32))
+    k = bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32))
+    v = bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32))
+    k[:, :, 401] = bf16_round(6.0 * q[:, :, 500])      # a large score for the rows near 500 (and a wide spread elsewhere)
+    k[:, :, 130] = bf16_round(-5.0 * q[:, :, 200])
+    for mask in (None, R.causal_mask(T)):
+        out = _attn(dev, q, k, v, mask, False, True)
+        ref, _ = R.attn_forward(q, k, v, None if mask is None else R.causal_mask(T, np.float64), False, np.float64)
+        assert_close(out, ref, BF16_RTOL, "attn hs128 with score jumps")
 
 
 def test_attn_forward_large_scores_lazy_rescale(dev):

@@ -189,6 +189,53 @@ def test_weight_storage_option_after_load_leaves_the_loaded_model_alone(llm, c4_
     assert _ids_match(ids, ref_ids, ref_logits, "fp32 model after the option flip")
 
 
+# ---- fused causal attention at the long-context shape of the benchmark ---------------------------
+
+def test_flash_attention_bf16_B4_T4096_32x128_causal_sampled_heads(dev):
+    """The Llama-2 7B head shape at full context (the second prefill target of the bench line): the software-pipelined
+    kernel with the grouped head order (K and V of the 128 heads are 268 MB).  Three (batch, head) pairs against the fp64
+    closed form, and the heads between them against a cheap invariant (row 0 of a causal head returns V[0])."""
+    B, H, T, hs = 4, 32, 4096, 128
+    rng = np.random.default_rng(40)
+    blk = bf16_round(rng.standard_normal((3, T, hs)).astype(np.float32))
+    picks = [(0, 0), (1, 17), (3, 31)]
+    n = B * H * T * hs
+    hq, hk, hv, hy = (dev.zeros(n, True) for _ in range(4))
+    # every head gets seeded data cheaply: one random block copied on the device, the picked heads their own q, k, v
+    fill = bf16_round(rng.standard_normal(T * hs).astype(np.float32))
+    hf = dev.put(fill, True)
+    for h_ in (hq, hk, hv):
+        for i in range(B * H):
+            dev.cuda.copy(T * hs, hf, h_, 0, i * T * hs)
+    data = {}
+    for (b, h) in picks:
+        q, k, v = (bf16_round(rng.standard_normal((T, hs)).astype(np.float32)) for _ in range(3))
+        data[(b, h)] = (q, k, v)
+        for arr, hd in ((q, hq), (k, hk), (v, hv)):
+            ht = dev.put(arr, True)
+            dev.cuda.copy(T * hs, ht, hd, 0, (b * H + h) * T * hs)
+    hm = dev.put(np.tril(np.ones((T, T), np.float32)))
+    hc, ha = dev.cuda.CreateCuDNN(), dev.cuda.CreateAttn()
+    dev.cuda.SetAttn(hc, ha, 0, False, B, T, H, hs, 0.0)
+    dev.cuda.AttnScaledDotProductForward(hc, ha, T, hq, hk, hv, hm, hy, False)
+    y = dev.get(hy, (B, H, T, hs))
+    dev.cuda.FreeAttn(ha)
+    dev.cuda.FreeCuDNN(hc)
+    assert np.all(np.isfinite(y))
+    tri = np.tril(np.ones((T, T), bool))
+    for (b, h), (q, k, v) in data.items():
+        s_ = (q.astype(np.float64) @ k.astype(np.float64).T) / np.sqrt(hs)
+        s_ = np.where(tri, s_, -np.inf)
+        p = np.exp(s_ - s_.max(-1, keepdims=True))
+        ref = (p / p.sum(-1, keepdims=True)) @ v.astype(np.float64)
+        assert_close(y[b, h], ref, BF16_RTOL, "long-context causal attention, head (%d, %d)" % (b, h))
+    # every other head holds the same q = k = v block: identical outputs, and row 0 attends to key 0 only
+    same = [(b, h) for b in range(B) for h in range(H) if (b, h) not in data]
+    assert_close(y[same[0]][0], fill.reshape(T, hs)[0], BF16_RTOL, "row 0 returns V[0]")
+    for bh in same[1:]:
+        assert np.array_equal(y[bh], y[same[0]]), "heads with identical inputs differ: %s" % (bh,)
+
+
 # ---- decode attention, 32 heads x 128, cache 4096 --------------------------------------------
 
 def _decode_row_ref(q, k, v):
