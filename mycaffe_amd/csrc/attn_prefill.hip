@@ -1110,7 +1110,7 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
             return flash_launch_cfg<bf16_t, 64, 1, 4, 3, true>(s, f, a.kind);
         }
         // no mask or causal, inference: the software-pipelined kernel (it does not keep the row statistics).  Measured at
-        // B=4, T=4096, 32 heads: unmasked 1.57 -> 1.31 ms, causal 0.80 -> 0.76 ms with the grouped head order.
+        // B=4, T=4096, 32 heads: unmasked 1.57 -> 1.31 ms; causal the same as the plain kernel (0.77 - 0.80 ms).
         if ((a.kind == MASK_NONE || a.kind == MASK_CAUSAL) && !a.lse2) {
             constexpr int LDSB = 2 * (64 * 136 + 64 * 144) * 2;
             static bool attr = false;
