@@ -814,11 +814,12 @@ __global__ __launch_bounds__(256, 3) void flash_pipe_bf16_64_kernel(FlashArgs a)
 // K and V row-major and double buffered in dynamic LDS (V^T fragments through the transposing read).  A phase is
 // sixteen MFMA slots - eight of O^T += V^T P^T of step t - 1, then eight of S^T of step t + 1 - and the softmax of
 // step t, the fragment reads two slots ahead and the K / V staging traffic ride along, one slice per slot.
-template <int KIND>
-__global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a)
+template <int KIND, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(FlashArgs a)
 {
     typedef FlashTraits<bf16_t> TR;
-    constexpr int HS = 128, BN = 64, NT = 512, BM = 256, LDK = HS + 8, LDVR = HS + 16;
+    constexpr int HS = 128, BN = 64, NT = NW * 64, BM = NW * 32, LDK = HS + 8, LDVR = HS + 16;
+    constexpr int CPT = BN * 16 / NT;   // 16-byte chunks of a K (or V) block per thread
     constexpr int KBUF = BN * LDK, VBUF = BN * LDVR;
     extern __shared__ __attribute__((aligned(16))) unsigned char pipe_smem[];
     bf16_t* Ks = reinterpret_cast<bf16_t*>(pipe_smem);   // [2][KBUF]
@@ -830,7 +831,7 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
     if (KIND == 1) {
         const int nbh = a.B * a.H;
         const int nqb = (a.Tq + BM - 1) / BM;
-        const int rank = flash_causal_rank(1);
+        const int rank = flash_causal_rank(8 / NW);
         int ibh;
         flash_causal_map(rank, nbh, nqb, a.causalGroup, &qblock, &ibh);
         b = ibh / a.H;
@@ -861,16 +862,19 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
 
     // staging: chunk e = tid + 512 i of a block -> key e / 16, 16-byte chunk e % 16 (K and V alike)
     // two register sets per operand (set = block & 1): a block is requested three phases before it is written to LDS
-    u32x4 kreg[2][2], vreg[2][2];
-    const int srow[2] = {tid / 16, (tid + NT) / 16}, scol = (tid % 16) * 8;
+    u32x4 kreg[2][CPT], vreg[2][CPT];
+    int srow[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; i++) srow[i] = (tid + i * NT) / 16;
+    const int scol = (tid % 16) * 8;
     auto gaddr = [&](const bf16_t* base, int kb, int i) { return base + (size_t)min(kb * BN + srow[i], a.Tk - 1) * HS + scol; };
-    auto kstore = [&](int buf, const u32x4 (&r)[2]) {
+    auto kstore = [&](int buf, const u32x4 (&r)[CPT]) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) *(u32x4*)(Ks + buf * KBUF + srow[i] * LDK + scol) = r[i];
+        for (int i = 0; i < CPT; i++) *(u32x4*)(Ks + buf * KBUF + srow[i] * LDK + scol) = r[i];
     };
-    auto vstore = [&](int buf, const u32x4 (&r)[2]) {
+    auto vstore = [&](int buf, const u32x4 (&r)[CPT]) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) *(u32x4*)(Vs + buf * VBUF + srow[i] * LDVR + scol) = r[i];
+        for (int i = 0; i < CPT; i++) *(u32x4*)(Vs + buf * VBUF + srow[i] * LDVR + scol) = r[i];
     };
 
     floatx16 o[4][1];
@@ -926,11 +930,11 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
 
     // prologue: K(0), V(0) in LDS, K(1), K(2) and V(1) in registers, S^T of step 0
 #pragma unroll
-    for (int i = 0; i < 2; i++) { kreg[0][i] = *(const u32x4*)gaddr(kp, 0, i); vreg[0][i] = *(const u32x4*)gaddr(vp, 0, i); }
+    for (int i = 0; i < CPT; i++) { kreg[0][i] = *(const u32x4*)gaddr(kp, 0, i); vreg[0][i] = *(const u32x4*)gaddr(vp, 0, i); }
     kstore(0, kreg[0]);
     vstore(0, vreg[0]);
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int i = 0; i < CPT; i++) {
         kreg[1][i] = *(const u32x4*)gaddr(kp, 1, i);
         kreg[0][i] = *(const u32x4*)gaddr(kp, 2, i);
         vreg[1][i] = *(const u32x4*)gaddr(vp, 1, i);
@@ -953,8 +957,8 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
         constexpr int ROLE = decltype(role_)::value, P = decltype(par_)::value;
         const int kbn = (ROLE == 0) ? (t >> 1) + 2 : (t >> 1) + 3;     // block requested in this phase
         const int wbuf = ((t >> 1) + 1) & 1;                           // LDS buffer written in this phase: block kb + 1
-        u32x4 (&fetch)[2] = ROLE == 0 ? vreg[P] : kreg[1 - P];
-        const u32x4 (&put)[2] = ROLE == 0 ? kreg[1 - P] : vreg[1 - P];
+        u32x4 (&fetch)[CPT] = ROLE == 0 ? vreg[P] : kreg[1 - P];
+        const u32x4 (&put)[CPT] = ROLE == 0 ? kreg[1 - P] : vreg[1 - P];
         const bool doSoft = t < nstw, doS = t + 1 < nstw, doPV = t >= 1 && t - 1 < nstw;
         const bool plain = !((KIND == 1) && (t * 32 + 31 > q0)) && (t * 32 + 32 <= a.Tk);
         if (doSoft && doS && doPV && plain) {
@@ -1005,14 +1009,14 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
                     asm volatile("" : "+v"(l[0]));
                 }
                 // K / V staging traffic of this phase
-                if (j == 12 || j == 13) {
-                    const int i = j - 12;
+                if (j >= 16 - 2 * CPT && j < 16 - CPT) {
+                    const int i = j - (16 - 2 * CPT);
                     if (ROLE == 0) *(u32x4*)(Ks + wbuf * KBUF + srow[i] * LDK + scol) = put[i];
                     else *(u32x4*)(Vs + wbuf * VBUF + srow[i] * LDVR + scol) = put[i];
-                } else if (j == 14 || j == 15) {
+                } else if (j >= 16 - CPT) {
                     // the set that ROLE 1 refills is the one ROLE 0 emptied a phase ago; ROLE 0 refills a set that the
                     // previous odd phase emptied: requests go after this phase's LDS writes in program order
-                    fetch[j - 14] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, j - 14);
+                    fetch[j - (16 - CPT)] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, j - (16 - CPT));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1031,7 +1035,7 @@ __global__ __launch_bounds__(512, 1) void flash_pipe_bf16_128_kernel(FlashArgs a
             if (ROLE == 1) vstore(wbuf, put);
             else kstore(wbuf, put);
 #pragma unroll
-            for (int i = 0; i < 2; i++) fetch[i] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, i);
+            for (int i = 0; i < CPT; i++) fetch[i] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, i);
         }
         __syncthreads();
     };
@@ -1115,14 +1119,21 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
             constexpr int LDSB = 2 * (64 * 136 + 64 * 144) * 2;
             static bool attr = false;
             if (!attr) {
-                hipError_t e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
-                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                hipError_t e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<0, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
                 if (e != hipSuccess) return e;
                 attr = true;
             }
+            // launches that leave CUs empty with 256-row workgroups take four wavefronts per workgroup (T = 777, 6 heads:
+            // 28.9 -> 23.8 us); at full size the larger workgroup wins (0.77 against 0.81 ms)
+            if (a.kind == MASK_CAUSAL && (long long)((f.Tq + 255) / 256) * f.H * f.B < 256) {
+                hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<1, 4>), dim3(((f.Tq + 127) / 128) * f.H * f.B), 256, LDSB, s, f);
+                return hipGetLastError();
+            }
             const int nqb = (f.Tq + 255) / 256;
-            if (a.kind == MASK_CAUSAL) hipLaunchKernelGGL(flash_pipe_bf16_128_kernel<1>, dim3(nqb * f.H * f.B), 512, LDSB, s, f);
-            else hipLaunchKernelGGL(flash_pipe_bf16_128_kernel<0>, dim3(nqb, f.H, f.B), 512, LDSB, s, f);
+            if (a.kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<1, 8>), dim3(nqb * f.H * f.B), 512, LDSB, s, f);
+            else hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<0, 8>), dim3(nqb, f.H, f.B), 512, LDSB, s, f);
             return hipGetLastError();
         }
         return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
