@@ -1,10 +1,12 @@
 // Micro-benchmarks of the gfx950 properties that the kernel designs of this library rest on.  Each prints one line per
 // case; none of them touches the library.  Build: mycaffe_amd/build.py; run: mycaffe_amd/host_bench/hw_probes [section]
-// with section in {overlap, lds, graph} (default: all).
+// with section in {overlap, lds, graph, persist} (default: all).
 //   overlap  how much vector-ALU work a wavefront can hide behind its own MFMAs (plain fma and v_exp_f32)
 //   lds      rate of the LDS fragment reads of the attention and GEMM kernels (ds_read_b128 in the K-fragment pattern,
 //            the transposing ds_read_b64_tr_b16 in the row-major V pattern) alone and with one MFMA per fragment
 //   graph    cost of a kernel boundary inside a replayed HIP graph and of a bare mat-vec kernel at several working sets
+//   persist  the same mat-vec chain as one cooperative kernel with bounded grid barriers, with and without the next
+//            phase's weights requested across the barrier
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <string.h>
@@ -210,6 +212,151 @@ static int run_graph()
     return 0;
 }
 
+// ---- persist: the same 62-phase mat-vec chain as ONE kernel with grid-wide barriers -------------------------------------
+// 256 workgroups (one per CU, launched cooperatively so that all are resident), four computing wavefronts each.  A wavefront owns up
+// to three rows of every 2304 x 768 matrix; it requests the NEXT phase's rows before it waits at the barrier, so the trip
+// to HBM overlaps the barrier.  Barrier: arrive on one of 8 counters (workgroup index mod 8, i.e. per die), the last
+// arrival of a die arrives on the global counter, the last of those releases one flag per die, which the die's workgroups poll.  Every wait is bounded: after
+// `spinLimit` polls a workgroup sets the error flag, and once the flag is set nobody waits any more, so the kernel ends.
+struct PersistArgs {
+    const float4* w;        // matrices of 2304 x 192 float4, phase p uses matrix p % nmat
+    float* xy;              // two vectors of 2304 floats (ping-pong); the first 768 of one are the next phase's input
+    int* counters;          // [0..7] per-die arrivals, [8] global arrivals, [9] error flag, [32 + 16 d] release flag of die d; zero at launch
+    int phases, nmat, spinLimit, prefetch;
+};
+__global__ __launch_bounds__(320) void persist_kernel(PersistArgs a)
+{
+    // wavefronts 0..3 compute; wavefront 4 only runs the barrier, so that its polls are not queued behind the weight
+    // requests of a computing wavefront (memory operations of a wavefront complete in order)
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const bool worker = wv < 4;
+    const int wave = blockIdx.x * 4 + wv;   // 1024 computing wavefronts
+    const int die = blockIdx.x & 7;
+    float4 cur[3][3], nxt[3][3];
+    auto request = [&](int p, float4 (&r)[3][3]) {
+        const float4* m = a.w + (size_t)(p % a.nmat) * 2304 * 192;
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            const int row = min(wave + 1024 * k, 2303);
+#pragma unroll
+            for (int c = 0; c < 3; c++) r[k][c] = m[(size_t)row * 192 + c * 64 + lane];
+        }
+    };
+    if (worker) request(0, cur);
+    for (int p = 0; p < a.phases; p++) {
+        if (worker) {
+            const float* x = a.xy + (p & 1) * 2304;
+            float* y = a.xy + ((p + 1) & 1) * 2304;
+            float4 xv[3];
+#pragma unroll
+            for (int c = 0; c < 3; c++) {
+                const float* xp = x + (c * 64 + lane) * 4;
+                xv[c].x = __hip_atomic_load(xp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                xv[c].y = __hip_atomic_load(xp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                xv[c].z = __hip_atomic_load(xp + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                xv[c].w = __hip_atomic_load(xp + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int k = 0; k < 3; k++) {
+                float s = 0.f;
+#pragma unroll
+                for (int c = 0; c < 3; c++)
+                    s += cur[k][c].x * xv[c].x + cur[k][c].y * xv[c].y + cur[k][c].z * xv[c].z + cur[k][c].w * xv[c].w;
+                for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+                const int row = wave + 1024 * k;
+                if (lane == 0 && row < 2304) __hip_atomic_store(y + row, s * 1e-3f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's results have been acknowledged
+        }
+        if (p + 1 == a.phases) break;
+        __syncthreads();   // all results of the workgroup are out
+        if (worker) {
+            if (a.prefetch) request(p + 1, nxt);   // in flight while the barrier wavefront waits
+        } else if (lane == 0) {
+            // arrive on the die's counter; the die's last arrival arrives on the global counter; the last of those
+            // releases the eight per-die flags (one cache line each), which is what the workgroups poll: 32 pollers per
+            // address instead of 256 (same-address accesses at this scope serialise)
+            if (__hip_atomic_fetch_add(a.counters + die, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (p + 1) * 32 - 1) {
+                if (__hip_atomic_fetch_add(a.counters + 8, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (p + 1) * 8 - 1) {
+                    for (int d = 0; d < 8; d++) __hip_atomic_store(a.counters + 32 + 16 * d, p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            int spins = 0;
+            while (__hip_atomic_load(a.counters + 32 + 16 * die, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p + 1) {
+                if ((++spins & 255) == 0 && __hip_atomic_load(a.counters + 9, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                if (spins > a.spinLimit) {
+                    __hip_atomic_store(a.counters + 9, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+            }
+        }
+        __syncthreads();   // the grid barrier has been passed (or given up)
+        if (worker) {
+            if (a.prefetch) {
+#pragma unroll
+                for (int k = 0; k < 3; k++)
+#pragma unroll
+                    for (int c = 0; c < 3; c++) cur[k][c] = nxt[k][c];
+            } else {
+                request(p + 1, cur);
+            }
+        }
+    }
+}
+
+static int run_persist()
+{
+    int dev = 0, coop = 0, cus = 0;
+    CK(hipGetDevice(&dev));
+    CK(hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev));
+    CK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (!coop || cus < 256) {
+        printf("persist  skipped (cooperative launch %d, CUs %d)\n", coop, cus);
+        return 0;
+    }
+    hipStream_t s;
+    CK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    const size_t matBytes = (size_t)2304 * 768 * 4;
+    float *big, *xy;
+    int* counters;
+    CK(hipMalloc(&big, 64 * matBytes));
+    CK(hipMalloc(&xy, 2 * 2304 * 4));
+    CK(hipMalloc(&counters, 1024));
+    CK(hipMemset(big, 0, 64 * matBytes));
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    for (int prefetch = 0; prefetch < 2; prefetch++) {
+        for (int nmat : {4, 64}) {
+            PersistArgs a = {(const float4*)big, xy, counters, 62, nmat, 1 << 20, prefetch};
+            void* args[] = {&a};
+            float best = 1e30f;
+            int err = 0;
+            for (int rep = 0; rep < 6; rep++) {
+                CK(hipMemsetAsync(counters, 0, 1024, s));
+                CK(hipMemsetAsync(xy, 0, 2 * 2304 * 4, s));
+                CK(hipEventRecord(e0, s));
+                CK(hipLaunchCooperativeKernel((const void*)persist_kernel, dim3(256), dim3(320), args, 0, s));
+                CK(hipEventRecord(e1, s));
+                CK(hipEventSynchronize(e1));
+                float ms;
+                CK(hipEventElapsedTime(&ms, e0, e1));
+                int h[16];
+                CK(hipMemcpy(h, counters, 64, hipMemcpyDeviceToHost));
+                err |= h[9];
+                if (rep > 0 && ms < best) best = ms;
+            }
+            printf("persist  62 phases of a 7.1 MB mat-vec in one kernel, weights cycling through %4.0f MB, next phase's rows %s: %5.2f us per phase%s\n",
+                   nmat * matBytes / 1e6, prefetch ? "requested before the barrier" : "requested after the barrier ", best * 1e3 / 62,
+                   err ? "  (a barrier wait hit its spin limit)" : "");
+        }
+    }
+    CK(hipFree(big));
+    CK(hipFree(xy));
+    CK(hipFree(counters));
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     const char* sec = argc > 1 ? argv[1] : "all";
@@ -242,6 +389,9 @@ int main(int argc, char** argv)
     }
     if (all || !strcmp(sec, "graph")) {
         if (run_graph()) return 1;
+    }
+    if (all || !strcmp(sec, "persist")) {
+        if (run_persist()) return 1;
     }
     CK(hipFree(d));
     return 0;
