@@ -495,331 +495,33 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_fwd_kernel(FlashArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// Software-pipelined variant for the hottest case: bf16, head size 64, no mask or causal.
+// Software-pipelined kernel for bf16 inference without mask or with the causal one, head sizes 64 and 128.
 //
-// Same data flow as flash_fwd_kernel with one 32-row tile per wavefront and four wavefronts, but the three
-// parts of a 32-key step run in different phases so that matrix and vector instructions of ONE wavefront
-// overlap (those of different wavefronts on a SIMD do not): during phase t a wavefront issues
+// Same data flow as flash_fwd_kernel with one 32-row tile per wavefront, but the three parts of a 32-key step run
+// in different phases so that matrix and vector instructions of ONE wavefront overlap (those of different
+// wavefronts on a SIMD do not): during phase t a wavefront issues
+//     O^T += V^T P^T of step t - 1     (HS / 16 MFMAs, V^T fragments through the transposing LDS read)
+//     S^T of step t + 1                (HS / 16 MFMAs, K fragments from LDS)
 //     the softmax of step t            (vector ALU: max, exp2, sum, pack)
-//     S^T of step t + 1                (4 MFMAs, K fragments from LDS)
-//     O^T += V^T P^T of step t - 1     (4 MFMAs, V fragments from LDS)
-// in a fixed issue order, one MFMA followed by a slice of the softmax and a slice of the K / V staging
-// traffic, each slice in a scheduling region of its own so that the order is kept.  K and V blocks of 64
-// keys are double buffered; block kb + 1 of K is written to LDS during phase 2 kb and of V during phase
-// 2 kb + 1, each while the other buffer is being read.  Phases that are not in steady state (the first, the
-// last two, diagonal or ragged steps) take a plain sequential path built from the same pieces.
-struct PipeStage {
-    const bf16_t* gk[2];   // global addresses of this thread's two K chunks of block 0 (advance by 64 * 64 per block)
-    const bf16_t* gv[2];
-    bf16_t* sk[2];         // LDS destinations inside buffer 0
-    bf16_t* sv[2];
-    u32x4 kreg[2], vreg[2];
-};
-
-template <int KIND>
-__global__ __launch_bounds__(256, 3) void flash_pipe_bf16_64_kernel(FlashArgs a)
+// in a fixed issue order: a phase is NSLOT MFMA slots, each followed by a slice of the softmax, the fragment
+// read two slots ahead and a slice of the K / V staging traffic, every slice in a scheduling region of its own
+// so that the order is kept.  K and V blocks of 64 keys are row-major and double buffered in dynamic LDS; a
+// block is requested from memory three phases before it is written to LDS, while the other buffer is being
+// read.  Phases that are not in steady state (the first, the last, diagonal or ragged steps) take a plain
+// sequential path built from the same pieces.
+template <int KIND, int NW, int HS, int OCC>
+__global__ __launch_bounds__(NW * 64, OCC) void flash_pipe_bf16_kernel(FlashArgs a)
 {
     typedef FlashTraits<bf16_t> TR;
-    constexpr int HS = 64, BN = 64, BM = 128, LDK = HS + 8, LDV = BN + 8;
-    constexpr int KBUF = BN * LDK, VBUF = HS * LDV;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[2 * KBUF];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[2 * VBUF];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int l32 = lane & 31, half = lane >> 5;
-    int qblock, h, b;
-    if (KIND == 1) {
-        const int nbh = a.B * a.H;
-        const int nqb = (a.Tq + BM - 1) / BM;
-        const int rank = flash_causal_rank(3);
-        qblock = nqb - 1 - rank / nbh;
-        const int ibh = rank % nbh;
-        b = ibh / a.H;
-        h = ibh % a.H;
-    } else {
-        qblock = blockIdx.x;
-        h = blockIdx.y;
-        b = blockIdx.z;
-    }
-    const size_t bh = (size_t)b * a.H + h;
-    const int q0 = qblock * BM + wave * 32;
-    const bf16_t* qp = (const bf16_t*)a.q + bh * a.Tq * HS;
-    const bf16_t* kp = (const bf16_t*)a.k + bh * a.Tk * HS;
-    const bf16_t* vp = (const bf16_t*)a.v + bh * a.Tk * HS;
-
-    u32x4 qf[4];
-    {
-        const int row = min(q0 + l32, a.Tq - 1);
-#pragma unroll
-        for (int f = 0; f < 4; f++) qf[f] = *(const u32x4*)(qp + (size_t)row * HS + f * 16 + half * 8);
-    }
-    int kend = a.Tk;
-    if (KIND == 1) kend = min(a.Tk, qblock * BM + BM);
-    const int nkb = (kend + BN - 1) / BN;
-    const int nst = 2 * nkb;                               // phases 0 .. nst
-    int nstw = min(nst, (a.Tk + 31) / 32);                 // steps this wavefront computes
-    if (KIND == 1) nstw = min(nstw, (q0 + 31) / 32 + 1);
-    if (q0 >= a.Tq) nstw = 0;
-
-    // staging addresses: K chunk e = tid + 256 i -> key e / 8, 16-byte chunk e % 8; V: key = lane, chunks wave + 4 i
-    PipeStage st;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int e = tid + i * 256;
-        st.sk[i] = Ks + (e / 8) * LDK + (e % 8) * 8;
-        st.sv[i] = Vt + (wave + 4 * i) * 8 * LDV + lane;
-    }
-    auto kload = [&](int kb) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int e = tid + i * 256;
-            st.kreg[i] = *(const u32x4*)(kp + (size_t)min(kb * BN + e / 8, a.Tk - 1) * HS + (e % 8) * 8);
-        }
-    };
-    auto vload = [&](int kb) {
-        const size_t vrow = (size_t)min(kb * BN + lane, a.Tk - 1) * HS;
-#pragma unroll
-        for (int i = 0; i < 2; i++) st.vreg[i] = *(const u32x4*)(vp + vrow + (wave + 4 * i) * 8);
-    };
-    auto kstore = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) *(u32x4*)(st.sk[i] + buf * KBUF) = st.kreg[i];
-    };
-    auto vstore = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) TR::scatter_chunk(st.sv[i] + buf * VBUF, LDV, st.vreg[i]);
-    };
-
-    floatx16 o[2][1];
-#pragma unroll
-    for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) o[dt][0][v] = 0.f;
-    float m[1] = {-INFINITY}, l[1] = {0.f};
-    const float c = a.c, lazy = a.lazy;
-    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    // fragment addresses: K rows of a 32-key step (add (step & 1) * 32 * LDK and the buffer), V^T rows per dim tile
-    const bf16_t* kfrag = Ks + l32 * LDK + half * 8;
-    const bf16_t* vfrag = Vt + l32 * LDV;
-
-    auto smma = [&](int t, floatx16& sn) {      // S^T of step t
-        const bf16_t* kb_ = kfrag + ((t >> 1) & 1) * KBUF + (t & 1) * 32 * LDK;
-        sn = TR::mma(*(const u32x4*)(kb_), qf[0], zero16);
-        sn = TR::mma(*(const u32x4*)(kb_ + 16), qf[1], sn);
-        sn = TR::mma(*(const u32x4*)(kb_ + 32), qf[2], sn);
-        sn = TR::mma(*(const u32x4*)(kb_ + 48), qf[3], sn);
-    };
-    auto pvmma = [&](int t, const u32x4 (&pp)[2]) {   // O^T += V^T P^T of step t
-        const bf16_t* vb_ = vfrag + ((t >> 1) & 1) * VBUF + (t & 1) * 32;
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-            for (int dt = 0; dt < 2; dt++) o[dt][0] = TR::mma(TR::load_vt(vb_ + dt * 32 * LDV, tt, half), pp[tt], o[dt][0]);
-    };
-    // sequential softmax of step t (any masking), leaves the packed weights in pc
-    auto soft_slow = [&](int t, floatx16 (&sc)[1], u32x4 (&pc)[2]) {
-        const int k0 = t * 32;
-        const bool masked = ((KIND == 1) && (k0 + 31 > q0)) || (k0 + 32 > a.Tk);
-        if (masked) {
-            const int qrow = q0 + l32;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
-                float sv = sc[0][v];
-                if (KIND == 1 && key > qrow) sv = a.maskedRaw;
-                if (key >= a.Tk) sv = -INFINITY;
-                sc[0][v] = sv;
-            }
-            flash_softmax_step<true, 2, 1>(sc, o, m, l, c, a.maskedRaw, lazy);
-        } else {
-            flash_softmax_step<false, 2, 1>(sc, o, m, l, c, a.maskedRaw, lazy);
-        }
-        pc[0] = TR::pack_p(sc[0], 0);
-        pc[1] = TR::pack_p(sc[0], 1);
-    };
-
-    // prologue: K(0), V(0) in LDS, K(1) in registers, S^T of step 0
-    kload(0);
-    vload(0);
-    kstore(0);
-    vstore(0);
-    kload(min(1, nkb - 1));
-#pragma unroll
-    for (int f = 0; f < 4; f++) asm volatile("" : "+v"(qf[f]));
-    __syncthreads();
-    floatx16 sA[1], sB[1];
-    u32x4 pA[2], pB[2];
-    sA[0] = zero16;
-    sB[0] = zero16;
-    pA[0] = pA[1] = pB[0] = pB[1] = u32x4{0u, 0u, 0u, 0u};
-    if (nstw > 0) smma(0, sA[0]);
-
-// One phase.  ROLE 0 (even phase 2 kb): fetch V(kb + 1), write K(kb + 1) to LDS; ROLE 1 (odd phase 2 kb - 1):
-// fetch K(kb + 1), write V(kb).  SC: scores of step t (in), SN: scores of step t + 1 (out), PP: packed weights
-// of step t - 1 (in), PC: packed weights of step t (out).
-#define PIPE_STAGE_LOAD(ROLE, KBN, I)                                                                                          \
-    do {                                                                                                                       \
-        if (ROLE == 0) {                                                                                                       \
-            const size_t vrow_ = (size_t)min((KBN) * BN + lane, a.Tk - 1) * HS;                                                \
-            st.vreg[I] = *(const u32x4*)(vp + vrow_ + (wave + 4 * (I)) * 8);                                                   \
-        } else {                                                                                                               \
-            const int e_ = tid + (I) * 256;                                                                                    \
-            st.kreg[I] = *(const u32x4*)(kp + (size_t)min((KBN) * BN + e_ / 8, a.Tk - 1) * HS + (e_ % 8) * 8);                 \
-        }                                                                                                                      \
-    } while (0)
-#define PIPE_V_SCATTER2(BUF, I, J)                                                                                             \
-    do {                                                                                                                       \
-        const uint32_t w_ = st.vreg[I][(J)];                                                                                   \
-        bf16_t* d_ = st.sv[I] + (BUF) * VBUF + 2 * (J) * LDV;                                                                  \
-        d_[0] = (bf16_t)(w_ & 0xffffu);                                                                                        \
-        d_[LDV] = (bf16_t)(w_ >> 16);                                                                                          \
-    } while (0)
-// keep a slice's results where the slice is written: code motion before scheduling would otherwise sink them
-// towards their first use, past the scheduling barriers
-#define PIPE_PIN1(A) asm volatile("" : "+v"(A))
-#define PIPE_PIN4(A, B, C, D) asm volatile("" : "+v"(A), "+v"(B), "+v"(C), "+v"(D))
-#define PIPE_EXP4(SC, V0)                                                                                                          \
-    do {                                                                                                                       \
-        pw_[(V0)] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[0][(V0)], c, -mc_));                                              \
-        pw_[(V0) + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[0][(V0) + 1], c, -mc_));                                      \
-        pw_[(V0) + 2] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[0][(V0) + 2], c, -mc_));                                      \
-        pw_[(V0) + 3] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[0][(V0) + 3], c, -mc_));                                      \
-        PIPE_PIN4(pw_[(V0)], pw_[(V0) + 1], pw_[(V0) + 2], pw_[(V0) + 3]);                                                     \
-    } while (0)
-#define PIPE_PHASE(ROLE, T, SC, SN, PP, PC)                                                                                    \
-    do {                                                                                                                       \
-        const int t_ = (T);                                                                                                    \
-        const int kbn_ = (ROLE == 0) ? (t_ >> 1) + 1 : ((t_ + 1) >> 1) + 1; /* block fetched in this phase */                  \
-        const int wbuf_ = (ROLE == 0) ? (((t_ >> 1) + 1) & 1) : (((t_ + 1) >> 1) & 1); /* buffer written in this phase */      \
-        const bool doSoft_ = t_ < nstw, doS_ = t_ + 1 < nstw, doPV_ = t_ >= 1 && t_ - 1 < nstw;                                \
-        const bool plain_ = !((KIND == 1) && (t_ * 32 + 31 > q0)) && (t_ * 32 + 32 <= a.Tk);                                   \
-        if (doSoft_ && doS_ && doPV_ && plain_) {                                                                              \
-            const bf16_t* kb_ = kfrag + (((t_ + 1) >> 1) & 1) * KBUF + ((t_ + 1) & 1) * 32 * LDK;                              \
-            const bf16_t* vb_ = vfrag + (((t_ - 1) >> 1) & 1) * VBUF + ((t_ - 1) & 1) * 32;                                    \
-            const u32x4 kf0_ = *(const u32x4*)(kb_), kf1_ = *(const u32x4*)(kb_ + 16);                                         \
-            const u32x4 kf2_ = *(const u32x4*)(kb_ + 32), kf3_ = *(const u32x4*)(kb_ + 48);                                    \
-            const u32x4 v00_ = TR::load_vt(vb_, 0, half), v01_ = TR::load_vt(vb_ + 32 * LDV, 0, half);                         \
-            const u32x4 v10_ = TR::load_vt(vb_, 1, half), v11_ = TR::load_vt(vb_ + 32 * LDV, 1, half);                         \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 0 */                                                                                                       \
-            o[0][0] = TR::mma(v00_, PP[0], o[0][0]);                                                                           \
-            float m1_ = fmaxf(fmaxf(SC[0][0], SC[0][1]), SC[0][2]), m2_ = fmaxf(fmaxf(SC[0][3], SC[0][4]), SC[0][5]);          \
-            float m3_ = fmaxf(fmaxf(SC[0][6], SC[0][7]), SC[0][8]), m4_ = fmaxf(fmaxf(SC[0][9], SC[0][10]), SC[0][11]);        \
-            PIPE_PIN4(m1_, m2_, m3_, m4_);                                                                                     \
-            PIPE_STAGE_LOAD(ROLE, kbn_, 0);                                                                                    \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 1 */                                                                                                       \
-            o[1][0] = TR::mma(v01_, PP[0], o[1][0]);                                                                           \
-            float m5_ = fmaxf(fmaxf(SC[0][12], SC[0][13]), SC[0][14]);                                                         \
-            float mx_ = fmaxf(fmaxf(m1_, m2_), m3_);                                                                           \
-            mx_ = fmaxf(fmaxf(mx_, m4_), m5_);                                                                                 \
-            mx_ = fmaxf(mx_, SC[0][15]);                                                                                       \
-            mx_ = flash_half_max(mx_);                                                                                         \
-            PIPE_PIN1(mx_);                                                                                                    \
-            PIPE_STAGE_LOAD(ROLE, kbn_, 1);                                                                                    \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 2 */                                                                                                       \
-            o[0][0] = TR::mma(v10_, PP[1], o[0][0]);                                                                           \
-            const float mnew_ = (mx_ > m[0] + lazy) ? mx_ : m[0];                                                              \
-            float alpha_ = __builtin_amdgcn_exp2f((m[0] - mnew_) * c);                                                         \
-            float mc_ = mnew_ * c;                                                                                             \
-            m[0] = mnew_;                                                                                                      \
-            PIPE_PIN4(alpha_, mc_, m[0], mx_);                                                                                 \
-            float pw_[16];                                                                                                     \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 3 */                                                                                                       \
-            o[1][0] = TR::mma(v11_, PP[1], o[1][0]);                                                                           \
-            PIPE_EXP4(SC, 0);                                                                                                      \
-            float rs_ = (pw_[0] + pw_[1]) + (pw_[2] + pw_[3]);                                                                 \
-            PIPE_PIN1(rs_);                                                                                                    \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 4 */                                                                                                       \
-            SN[0] = TR::mma(kf0_, qf[0], zero16);                                                                              \
-            PIPE_EXP4(SC, 4);                                                                                                      \
-            rs_ += (pw_[4] + pw_[5]) + (pw_[6] + pw_[7]);                                                                      \
-            PIPE_PIN1(rs_);                                                                                                    \
-            if (ROLE == 1) { PIPE_V_SCATTER2(wbuf_, 0, 0); PIPE_V_SCATTER2(wbuf_, 0, 1); }                                     \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 5 */                                                                                                       \
-            SN[0] = TR::mma(kf1_, qf[1], SN[0]);                                                                               \
-            PIPE_EXP4(SC, 8);                                                                                                      \
-            rs_ += (pw_[8] + pw_[9]) + (pw_[10] + pw_[11]);                                                                    \
-            PIPE_PIN1(rs_);                                                                                                    \
-            if (ROLE == 1) { PIPE_V_SCATTER2(wbuf_, 0, 2); PIPE_V_SCATTER2(wbuf_, 0, 3); }                                     \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 6 */                                                                                                       \
-            SN[0] = TR::mma(kf2_, qf[2], SN[0]);                                                                               \
-            PIPE_EXP4(SC, 12);                                                                                                     \
-            rs_ += (pw_[12] + pw_[13]) + (pw_[14] + pw_[15]);                                                                  \
-            PIPE_PIN1(rs_);                                                                                                    \
-            if (ROLE == 1) { PIPE_V_SCATTER2(wbuf_, 1, 0); PIPE_V_SCATTER2(wbuf_, 1, 1); }                                     \
-            else *(u32x4*)(st.sk[0] + wbuf_ * KBUF) = st.kreg[0];                                                              \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            /* slot 7 */                                                                                                       \
-            SN[0] = TR::mma(kf3_, qf[3], SN[0]);                                                                               \
-            PC[0] = u32x4{pack_bf16x2(pw_[0], pw_[1]), pack_bf16x2(pw_[2], pw_[3]), pack_bf16x2(pw_[4], pw_[5]),               \
-                          pack_bf16x2(pw_[6], pw_[7])};                                                                        \
-            PC[1] = u32x4{pack_bf16x2(pw_[8], pw_[9]), pack_bf16x2(pw_[10], pw_[11]), pack_bf16x2(pw_[12], pw_[13]),           \
-                          pack_bf16x2(pw_[14], pw_[15])};                                                                      \
-            l[0] = l[0] * alpha_ + rs_;                                                                                        \
-            asm volatile("" : "+v"(PC[0]), "+v"(PC[1]), "+v"(l[0]));                                                           \
-            if (ROLE == 1) { PIPE_V_SCATTER2(wbuf_, 1, 2); PIPE_V_SCATTER2(wbuf_, 1, 3); }                                     \
-            else *(u32x4*)(st.sk[1] + wbuf_ * KBUF) = st.kreg[1];                                                              \
-            __builtin_amdgcn_sched_barrier(0);                                                                                 \
-            if (!__all(alpha_ == 1.0f)) {                                                                                      \
-                _Pragma("unroll") for (int dt = 0; dt < 2; dt++)                                                               \
-                    _Pragma("unroll") for (int v = 0; v < 16; v++) o[dt][0][v] *= alpha_;                                      \
-            }                                                                                                                  \
-        } else {                                                                                                               \
-            PIPE_STAGE_LOAD(ROLE, kbn_, 0);                                                                                    \
-            PIPE_STAGE_LOAD(ROLE, kbn_, 1);                                                                                    \
-            if (doPV_) pvmma(t_ - 1, PP);                                                                                      \
-            if (doSoft_) soft_slow(t_, SC, PC);                                                                                \
-            if (doS_) smma(t_ + 1, SN[0]);                                                                                     \
-            if (ROLE == 1) vstore(wbuf_);                                                                                      \
-            else kstore(wbuf_);                                                                                                \
-        }                                                                                                                      \
-        __syncthreads();                                                                                                       \
-    } while (0)
-
-    for (int kb = 0; kb <= nkb; kb++) {
-        PIPE_PHASE(0, 2 * kb, sA, sB, pB, pA);
-        if (kb < nkb) PIPE_PHASE(1, 2 * kb + 1, sB, sA, pA, pB);
-    }
-#undef PIPE_PHASE
-#undef PIPE_EXP4
-#undef PIPE_PIN4
-#undef PIPE_PIN1
-#undef PIPE_V_SCATTER2
-#undef PIPE_STAGE_LOAD
-
-    // epilogue: y[query, dim] = O^T[dim, query] / l
-    const int qrow = q0 + l32;
-    const float lt = l[0] + __shfl_xor(l[0], 32, 64);
-    const float inv = 1.0f / lt;
-    if (qrow < a.Tq) {
-        bf16_t* yr = (bf16_t*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, qrow, HS);
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-            for (int g = 0; g < 4; g++)
-                TR::store4(yr + 32 * dt + 8 * g + 4 * half, o[dt][0][4 * g] * inv, o[dt][0][4 * g + 1] * inv,
-                           o[dt][0][4 * g + 2] * inv, o[dt][0][4 * g + 3] * inv);
-    }
-}
-
-// ---------------------------------------------------------------------------
-// The same software pipeline for head size 128 (bf16, no mask or causal): eight wavefronts of one 32-row tile each,
-// K and V row-major and double buffered in dynamic LDS (V^T fragments through the transposing read).  A phase is
-// sixteen MFMA slots - eight of O^T += V^T P^T of step t - 1, then eight of S^T of step t + 1 - and the softmax of
-// step t, the fragment reads two slots ahead and the K / V staging traffic ride along, one slice per slot.
-template <int KIND, int NW>
-__global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(FlashArgs a)
-{
-    typedef FlashTraits<bf16_t> TR;
-    constexpr int HS = 128, BN = 64, NT = NW * 64, BM = NW * 32, LDK = HS + 8, LDVR = HS + 16;
-    constexpr int CPT = BN * 16 / NT;   // 16-byte chunks of a K (or V) block per thread
+    constexpr int BN = 64, NT = NW * 64, BM = NW * 32, LDK = HS + 8, LDVR = (HS * 2) % 256 == 0 ? HS + 16 : HS + 8;
+    constexpr int KF = HS / 16, DT = HS / 32, NPV = 2 * DT, NSLOT = NPV + KF;   // 16 slots at head size 128, 8 at 64
+    constexpr int CPR = HS / 8;                  // 16-byte chunks per K (or V) row
+    constexpr int CPT = BN * CPR / NT;           // chunks of a block per thread
+    // slots of the softmax slices: maxima in 0 and 1, new maximum in 2, the exponentials from 3 on, then the packing,
+    // the row sum in the last slot
+    constexpr int NEXP = NSLOT == 16 ? 8 : 3, EPS = NSLOT == 16 ? 2 : 6;   // exponential slots, scores per slot
+    constexpr int PACK0 = 3 + NEXP, NPACK = NSLOT == 16 ? 4 : 1, WPS = 8 / NPACK;   // packing slots, words per slot
+    static_assert(PACK0 + NPACK < NSLOT && 2 * CPT <= NSLOT - 2, "slices do not fit the slots");
     constexpr int KBUF = BN * LDK, VBUF = BN * LDVR;
     extern __shared__ __attribute__((aligned(16))) unsigned char pipe_smem[];
     bf16_t* Ks = reinterpret_cast<bf16_t*>(pipe_smem);   // [2][KBUF]
@@ -831,7 +533,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
     if (KIND == 1) {
         const int nbh = a.B * a.H;
         const int nqb = (a.Tq + BM - 1) / BM;
-        const int rank = flash_causal_rank(8 / NW);
+        const int rank = flash_causal_rank(OCC);
         int ibh;
         flash_causal_map(rank, nbh, nqb, a.causalGroup, &qblock, &ibh);
         b = ibh / a.H;
@@ -847,11 +549,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
     const bf16_t* kp = (const bf16_t*)a.k + bh * a.Tk * HS;
     const bf16_t* vp = (const bf16_t*)a.v + bh * a.Tk * HS;
 
-    u32x4 qf[8];
+    u32x4 qf[KF];
     {
         const int row = min(q0 + l32, a.Tq - 1);
 #pragma unroll
-        for (int f = 0; f < 8; f++) qf[f] = *(const u32x4*)(qp + (size_t)row * HS + f * 16 + half * 8);
+        for (int f = 0; f < KF; f++) qf[f] = *(const u32x4*)(qp + (size_t)row * HS + f * 16 + half * 8);
     }
     int kend = a.Tk;
     if (KIND == 1) kend = min(a.Tk, qblock * BM + BM);
@@ -860,13 +562,13 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
     if (KIND == 1) nstw = min(nstw, (q0 + 31) / 32 + 1);
     if (q0 >= a.Tq) nstw = 0;
 
-    // staging: chunk e = tid + 512 i of a block -> key e / 16, 16-byte chunk e % 16 (K and V alike)
+    // staging: chunk e = tid + NT i of a block -> key e / CPR, 16-byte chunk e % CPR (K and V alike)
     // two register sets per operand (set = block & 1): a block is requested three phases before it is written to LDS
     u32x4 kreg[2][CPT], vreg[2][CPT];
     int srow[CPT];
 #pragma unroll
-    for (int i = 0; i < CPT; i++) srow[i] = (tid + i * NT) / 16;
-    const int scol = (tid % 16) * 8;
+    for (int i = 0; i < CPT; i++) srow[i] = (tid + i * NT) / CPR;
+    const int scol = (tid % CPR) * 8;
     auto gaddr = [&](const bf16_t* base, int kb, int i) { return base + (size_t)min(kb * BN + srow[i], a.Tk - 1) * HS + scol; };
     auto kstore = [&](int buf, const u32x4 (&r)[CPT]) {
 #pragma unroll
@@ -877,9 +579,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
         for (int i = 0; i < CPT; i++) *(u32x4*)(Vs + buf * VBUF + srow[i] * LDVR + scol) = r[i];
     };
 
-    floatx16 o[4][1];
+    floatx16 o[DT][1];
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+    for (int dt = 0; dt < DT; dt++)
 #pragma unroll
         for (int v = 0; v < 16; v++) o[dt][0][v] = 0.f;
     float m[1] = {-INFINITY}, l[1] = {0.f};
@@ -887,28 +589,28 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const bf16_t* kfrag = Ks + l32 * LDK + half * 8;
 
-    // fragment j of a phase around step t: 0..7 = V^T fragments of step t - 1 (key half j / 4, dim tile j % 4),
-    // 8..15 = K fragments of step t + 1
+    // fragment j of a phase around step t: 0 .. NPV - 1 = V^T fragments of step t - 1 (key half j / DT, dim tile j % DT),
+    // the rest = K fragments of step t + 1
     auto frag = [&](int j, int t) -> u32x4 {
-        if (j < 8) {
+        if (j < NPV) {
             const int tv = t - 1;
-            return TR::load_vt_rowmajor(Vs + ((tv >> 1) & 1) * VBUF + 32 * (tv & 1) * LDVR + (j & 3) * 32, LDVR, j >> 2, lane);
+            return TR::load_vt_rowmajor(Vs + ((tv >> 1) & 1) * VBUF + 32 * (tv & 1) * LDVR + (j % DT) * 32, LDVR, j / DT, lane);
         }
         const int ts = t + 1;
-        return *(const u32x4*)(kfrag + ((ts >> 1) & 1) * KBUF + (ts & 1) * 32 * LDK + (j - 8) * 16);
+        return *(const u32x4*)(kfrag + ((ts >> 1) & 1) * KBUF + (ts & 1) * 32 * LDK + (j - NPV) * 16);
     };
     auto smma = [&](int t, floatx16& sn) {      // S^T of step t
         const bf16_t* kb_ = kfrag + ((t >> 1) & 1) * KBUF + (t & 1) * 32 * LDK;
         sn = TR::mma(*(const u32x4*)(kb_), qf[0], zero16);
 #pragma unroll
-        for (int f = 1; f < 8; f++) sn = TR::mma(*(const u32x4*)(kb_ + 16 * f), qf[f], sn);
+        for (int f = 1; f < KF; f++) sn = TR::mma(*(const u32x4*)(kb_ + 16 * f), qf[f], sn);
     };
     auto pvmma = [&](int t, const u32x4 (&pp)[2]) {   // O^T += V^T P^T of step t
         const bf16_t* vb_ = Vs + ((t >> 1) & 1) * VBUF + 32 * (t & 1) * LDVR;
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) o[dt][0] = TR::mma(TR::load_vt_rowmajor(vb_ + dt * 32, LDVR, tt, lane), pp[tt], o[dt][0]);
+            for (int dt = 0; dt < DT; dt++) o[dt][0] = TR::mma(TR::load_vt_rowmajor(vb_ + dt * 32, LDVR, tt, lane), pp[tt], o[dt][0]);
     };
     // sequential softmax of step t (any masking), leaves the packed weights in pc
     auto soft_slow = [&](int t, floatx16 (&sc)[1], u32x4 (&pc)[2]) {
@@ -923,7 +625,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
                 if ((KIND == 1 && key > qrow) || key >= a.Tk) sc[0][v] = -INFINITY;
             }
         }
-        flash_softmax_step<false, 4, 1>(sc, o, m, l, c, a.maskedRaw, lazy);
+        flash_softmax_step<false, DT, 1>(sc, o, m, l, c, a.maskedRaw, lazy);
         pc[0] = TR::pack_p(sc[0], 0);
         pc[1] = TR::pack_p(sc[0], 1);
     };
@@ -940,7 +642,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
         vreg[1][i] = *(const u32x4*)gaddr(vp, 1, i);
     }
 #pragma unroll
-    for (int f = 0; f < 8; f++) asm volatile("" : "+v"(qf[f]));
+    for (int f = 0; f < KF; f++) asm volatile("" : "+v"(qf[f]));
     __syncthreads();
     floatx16 sA[1], sB[1];
     u32x4 pA[2], pB[2];
@@ -962,17 +664,17 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
         const bool doSoft = t < nstw, doS = t + 1 < nstw, doPV = t >= 1 && t - 1 < nstw;
         const bool plain = !((KIND == 1) && (t * 32 + 31 > q0)) && (t * 32 + 32 <= a.Tk);
         if (doSoft && doS && doPV && plain) {
-            u32x4 fr[16];
+            u32x4 fr[NSLOT];
             fr[0] = frag(0, t);
             fr[1] = frag(1, t);
             float m1 = 0.f, m2 = 0.f, m3 = 0.f, m4 = 0.f, mx = 0.f, alpha = 1.f, mc = 0.f, rs = 0.f, pw[16];
             uint32_t pk[8];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                if (j < 8) o[j & 3][0] = TR::mma(fr[j], pp[j >> 2], o[j & 3][0]);
-                else sn[0] = TR::mma(fr[j], qf[j - 8], j == 8 ? zero16 : sn[0]);
-                if (j + 2 < 16) fr[j + 2] = frag(j + 2, t);
+            for (int j = 0; j < NSLOT; j++) {
+                if (j < NPV) o[j % DT][0] = TR::mma(fr[j], pp[j / DT], o[j % DT][0]);
+                else sn[0] = TR::mma(fr[j], qf[j - NPV], j == NPV ? zero16 : sn[0]);
+                if (j + 2 < NSLOT) fr[j + 2] = frag(j + 2, t);
                 // softmax of step t, one slice per slot
                 if (j == 0) {
                     m1 = fmaxf(fmaxf(sc[0][0], sc[0][1]), sc[0][2]);
@@ -993,30 +695,33 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
                     mc = mnew * c;
                     m[0] = mnew;
                     asm volatile("" : "+v"(alpha), "+v"(mc), "+v"(m[0]));
-                } else if (j <= 10) {
-                    const int e = 2 * (j - 3);
-                    pw[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e], c, -mc));
-                    pw[e + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e + 1], c, -mc));
-                    rs += pw[e] + pw[e + 1];
-                    asm volatile("" : "+v"(pw[e]), "+v"(pw[e + 1]), "+v"(rs));
-                } else if (j <= 14) {
-                    const int w = 2 * (j - 11);
-                    pk[w] = pack_bf16x2(pw[2 * w], pw[2 * w + 1]);
-                    pk[w + 1] = pack_bf16x2(pw[2 * w + 2], pw[2 * w + 3]);
-                    asm volatile("" : "+v"(pk[w]), "+v"(pk[w + 1]));
-                } else {
+                } else if (j < 3 + NEXP) {
+#pragma unroll
+                    for (int e = EPS * (j - 3); e < EPS * (j - 2) && e < 16; e += 2) {
+                        pw[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e], c, -mc));
+                        pw[e + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[0][e + 1], c, -mc));
+                        rs += pw[e] + pw[e + 1];
+                        asm volatile("" : "+v"(pw[e]), "+v"(pw[e + 1]), "+v"(rs));
+                    }
+                } else if (j < PACK0 + NPACK) {
+#pragma unroll
+                    for (int w = WPS * (j - PACK0); w < WPS * (j - PACK0 + 1); w++) {
+                        pk[w] = pack_bf16x2(pw[2 * w], pw[2 * w + 1]);
+                        asm volatile("" : "+v"(pk[w]));
+                    }
+                } else if (j == NSLOT - 1) {
                     l[0] = l[0] * alpha + rs;
                     asm volatile("" : "+v"(l[0]));
                 }
                 // K / V staging traffic of this phase
-                if (j >= 16 - 2 * CPT && j < 16 - CPT) {
-                    const int i = j - (16 - 2 * CPT);
+                if (j >= NSLOT - 2 * CPT && j < NSLOT - CPT) {
+                    const int i = j - (NSLOT - 2 * CPT);
                     if (ROLE == 0) *(u32x4*)(Ks + wbuf * KBUF + srow[i] * LDK + scol) = put[i];
                     else *(u32x4*)(Vs + wbuf * VBUF + srow[i] * LDVR + scol) = put[i];
-                } else if (j >= 16 - CPT) {
+                } else if (j >= NSLOT - CPT) {
                     // the set that ROLE 1 refills is the one ROLE 0 emptied a phase ago; ROLE 0 refills a set that the
                     // previous odd phase emptied: requests go after this phase's LDS writes in program order
-                    fetch[j - (16 - CPT)] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, j - (16 - CPT));
+                    fetch[j - (NSLOT - CPT)] = *(const u32x4*)gaddr(ROLE == 0 ? vp : kp, kbn, j - (NSLOT - CPT));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1024,7 +729,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
             pc[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
             if (!__all(alpha == 1.0f)) {
 #pragma unroll
-                for (int dt = 0; dt < 4; dt++)
+                for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int v = 0; v < 16; v++) o[dt][0][v] *= alpha;
             }
@@ -1055,7 +760,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_pipe_bf16_128_kernel(Fl
     if (qrow < a.Tq) {
         bf16_t* yr = (bf16_t*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, qrow, HS);
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int g = 0; g < 4; g++)
                 TR::store4(yr + 32 * dt + 8 * g + 4 * half, o[dt][0][4 * g] * inv, o[dt][0][4 * g + 1] * inv,
@@ -1104,11 +809,13 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     // keeps eight wavefronts per workgroup so that each staged K / V block serves more rows.
     if (dt == BF16) {
         if (a.hs == 64) {
-            // Unmasked attention runs the software-pipelined kernel (+15..30 %).  Causal launches measure the same
-            // or slightly better with the plain kernel (ragged per-wavefront ranges leave the pipeline in its
-            // sequential phases more often), so they stay there.
+            // Unmasked attention runs the software-pipelined kernel (B = 8, T = 1024, 12 heads: 45.7 us; B = 4,
+            // T = 4096, 32 heads: 0.79 ms).  Causal launches measure the same (T = 1024) or up to 10 % slower
+            // (T >= 2048) with it - ragged per-wavefront ranges leave the pipeline in its sequential phases more
+            // often - so they stay with the plain kernel.
             if (a.kind == MASK_NONE && !a.lse2) {   // the pipelined kernel does not keep the row statistics
-                hipLaunchKernelGGL(flash_pipe_bf16_64_kernel<0>, dim3((f.Tq + 127) / 128, f.H, f.B), 256, 0, s, f);
+                constexpr int LDSB = 2 * (64 * 72 + 64 * 72) * 2;
+                hipLaunchKernelGGL((flash_pipe_bf16_kernel<0, 4, 64, 3>), dim3((f.Tq + 127) / 128, f.H, f.B), 256, LDSB, s, f);
                 return hipGetLastError();
             }
             return flash_launch_cfg<bf16_t, 64, 1, 4, 3, true>(s, f, a.kind);
@@ -1119,21 +826,21 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
             constexpr int LDSB = 2 * (64 * 136 + 64 * 144) * 2;
             static bool attr = false;
             if (!attr) {
-                hipError_t e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<0, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
-                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
-                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_128_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                hipError_t e = hipFuncSetAttribute((const void*)flash_pipe_bf16_kernel<0, 8, 128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_kernel<1, 8, 128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)flash_pipe_bf16_kernel<1, 4, 128, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, LDSB);
                 if (e != hipSuccess) return e;
                 attr = true;
             }
             // launches that leave CUs empty with 256-row workgroups take four wavefronts per workgroup (T = 777, 6 heads:
             // 28.9 -> 23.8 us); at full size the larger workgroup wins (0.77 against 0.81 ms)
             if (a.kind == MASK_CAUSAL && (long long)((f.Tq + 255) / 256) * f.H * f.B < 256) {
-                hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<1, 4>), dim3(((f.Tq + 127) / 128) * f.H * f.B), 256, LDSB, s, f);
+                hipLaunchKernelGGL((flash_pipe_bf16_kernel<1, 4, 128, 2>), dim3(((f.Tq + 127) / 128) * f.H * f.B), 256, LDSB, s, f);
                 return hipGetLastError();
             }
             const int nqb = (f.Tq + 255) / 256;
-            if (a.kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<1, 8>), dim3(nqb * f.H * f.B), 512, LDSB, s, f);
-            else hipLaunchKernelGGL((flash_pipe_bf16_128_kernel<0, 8>), dim3(nqb, f.H, f.B), 512, LDSB, s, f);
+            if (a.kind == MASK_CAUSAL) hipLaunchKernelGGL((flash_pipe_bf16_kernel<1, 8, 128, 1>), dim3(nqb * f.H * f.B), 512, LDSB, s, f);
+            else hipLaunchKernelGGL((flash_pipe_bf16_kernel<0, 8, 128, 1>), dim3(nqb, f.H, f.B), 512, LDSB, s, f);
             return hipGetLastError();
         }
         return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
