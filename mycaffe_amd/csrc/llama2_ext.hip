@@ -30,6 +30,7 @@
 #include <mutex>
 #include <string>
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/mycaffe_hip_abi.h"
@@ -54,10 +55,23 @@ template <typename T> __device__ inline float wld(const T* p, size_t i);
 template <> __device__ inline float wld<float>(const float* p, size_t i) { return p[i]; }
 template <> __device__ inline float wld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
 
+// Sum over the 64 lanes of a wavefront, the result in every lane: four DPP steps inside each row of 16 lanes, then the
+// two row-swapping permutes.  All of it runs at vector-ALU latency; the same butterfly through __shfl_xor goes through
+// the LDS crossbar six times and costs 0.1 - 0.2 us at the end of a kernel that is a few microseconds long.
+template <int CTRL> __device__ __forceinline__ float wsum_dpp(float v)
+{
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xf, 0xf, false));
+}
 __device__ inline float wsum(float v)
 {
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += wsum_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += wsum_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += wsum_dpp<0x124>(v);   // row_ror:4
+    v += wsum_dpp<0x128>(v);   // row_ror:8
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
 }
 
 // x[b,:] = emb[token,:] where token is the forced prompt id while pos < n_prompt and
@@ -152,6 +166,26 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int r0 = wave * ROWS;
     if (r0 >= rows) return;
+    // Every load below is unconditional (columns past the end come from a clamped address and meet a zeroed activation):
+    // loads under a branch would make the compiler wait for ALL outstanding loads at the first use of any of them.
+    // The first sequence's activations (and the norm weights) are requested before the weights: loads return in order,
+    // so the sum of squares, its reduction and the square root run while the weights are still on their way.
+    constexpr int LW = WIDE ? 8 : 4;   // columns per load
+    float4 xv[CH], gq[NORM ? CH : 1];
+    float prev[ROWS];
+    auto request_x = [&](int b) {
+        const float* xb = x + (size_t)b * n;
+        // the residual epilogue's old values are requested now, not once the row sums are known
+#pragma unroll
+        for (int rr = 0; rr < ROWS; rr++) prev[rr] = (MODE == 1 && lane == 0) ? y[(size_t)b * ldy + min(r0 + rr, rows - 1)] : 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int jc = min(matvec_col<WIDE>(c, lane), n - 4);
+            xv[c] = *(const float4*)(xb + jc);
+            if (NORM) gq[c] = *(const float4*)(g + jc);
+        }
+    };
+    request_x(0);
     // weight chunks of this wavefront's rows stay in registers across the batch loop
     float4 w[(MODE == 2 ? 2 : 1) * ROWS][CH];
 #pragma unroll
@@ -160,15 +194,13 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
         if (WIDE) {
 #pragma unroll
             for (int c = 0; c < CH; c += 2) {
-                const int j = matvec_col<WIDE>(c, lane);
-                float lo[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, hi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                if (j < n) {
-                    Row8<T>::load(W + (size_t)r * n + j, lo);
-                    if (MODE == 2) Row8<T>::load(W + (size_t)(r + rows) * n + j, hi);
-                }
+                const int jc = min(matvec_col<WIDE>(c, lane), n - LW);
+                float lo[8], hi[8];
+                Row8<T>::load(W + (size_t)r * n + jc, lo);
                 w[rr][c] = make_float4(lo[0], lo[1], lo[2], lo[3]);
                 w[rr][c + 1] = make_float4(lo[4], lo[5], lo[6], lo[7]);
                 if (MODE == 2) {
+                    Row8<T>::load(W + (size_t)(r + rows) * n + jc, hi);
                     w[ROWS + rr][c] = make_float4(hi[0], hi[1], hi[2], hi[3]);
                     w[ROWS + rr][c + 1] = make_float4(hi[4], hi[5], hi[6], hi[7]);
                 }
@@ -176,47 +208,33 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
         } else {
 #pragma unroll
             for (int c = 0; c < CH; c++) {
-                const int j = matvec_col<WIDE>(c, lane);
-                if (j < n) {
-                    w[rr][c] = Row4<T>::load(W + (size_t)r * n + j);
-                    if (MODE == 2) w[ROWS + rr][c] = Row4<T>::load(W + (size_t)(r + rows) * n + j);
-                } else {
-                    w[rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (MODE == 2) w[ROWS + rr][c] = make_float4(0.f, 0.f, 0.f, 0.f);
-                }
+                const int jc = min(matvec_col<WIDE>(c, lane), n - 4);
+                w[rr][c] = Row4<T>::load(W + (size_t)r * n + jc);
+                if (MODE == 2) w[ROWS + rr][c] = Row4<T>::load(W + (size_t)(r + rows) * n + jc);
             }
         }
     }
-    for (int b = 0; b < B; b++) {
-        const float* xb = x + (size_t)b * n;
-        float4 xv[CH], gq[NORM ? CH : 1];
-        float ss = 0.f;
-        // the residual epilogue's old values are requested now, not once the row sums are known
-        float prev[ROWS];
-#pragma unroll
-        for (int rr = 0; rr < ROWS; rr++) prev[rr] = (MODE == 1 && lane == 0 && r0 + rr < rows) ? y[(size_t)b * ldy + r0 + rr] : 0.f;
-        // the norm weights are requested together with the activations, not after the sum of squares has gone round
+    __builtin_amdgcn_sched_barrier(0);   // every request above is issued before any arithmetic below
+    auto sequence = [&](int b, auto first) {
+        if (!decltype(first)::value) request_x(b);
 #pragma unroll
         for (int c = 0; c < CH; c++) {
-            const int j = matvec_col<WIDE>(c, lane);
-            xv[c] = j < n ? *(const float4*)(xb + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-            if (NORM) gq[c] = j < n ? *(const float4*)(g + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float keep = matvec_col<WIDE>(c, lane) < n ? 1.f : 0.f;
+            xv[c].x *= keep; xv[c].y *= keep; xv[c].z *= keep; xv[c].w *= keep;
         }
         if (NORM) {
+            float ss = 0.f;
 #pragma unroll
             for (int c = 0; c < CH; c++) ss += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
             ss = wsum(ss);
             const float inv = 1.0f / sqrtf(ss / n + 1e-5f);
 #pragma unroll
             for (int c = 0; c < CH; c++) {
-                const int j = matvec_col<WIDE>(c, lane);
-                if (j < n) {
-                    const float4 gv = gq[c];
-                    xv[c].x = gv.x * (inv * xv[c].x);
-                    xv[c].y = gv.y * (inv * xv[c].y);
-                    xv[c].z = gv.z * (inv * xv[c].z);
-                    xv[c].w = gv.w * (inv * xv[c].w);
-                }
+                const float4 gv = gq[c];
+                xv[c].x = gv.x * (inv * xv[c].x);
+                xv[c].y = gv.y * (inv * xv[c].y);
+                xv[c].z = gv.z * (inv * xv[c].z);
+                xv[c].w = gv.w * (inv * xv[c].w);
             }
         }
 #pragma unroll
@@ -239,7 +257,10 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
                 else *out = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
             }
         }
-    }
+    };
+    // the first sequence in straight-line code, so that the wait before the norm counts only the loads it needs
+    sequence(0, std::true_type());
+    for (int b = 1; b < B; b++) sequence(b, std::false_type());
 }
 
 // The same family for rows too long to hold in registers (n > 4096): one wavefront per row walks K in slabs of

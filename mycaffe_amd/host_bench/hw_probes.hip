@@ -161,6 +161,17 @@ __global__ __launch_bounds__(256) void matvec_probe_kernel(const float4* __restr
     if (lane == 0) y[wave] = s;
 }
 
+// touches the same bytes as matvec_probe_kernel from the same workgroup index (same die, same L2) and keeps nothing
+__global__ __launch_bounds__(256) void prefetch_probe_kernel(const float4* __restrict__ w, int rows)
+{
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (wave >= rows) return;
+    for (int c = 0; c < 3; c++) {
+        float4 a = w[(size_t)wave * 192 + c * 64 + lane];
+        asm volatile("" :: "v"(a.x), "v"(a.y), "v"(a.z), "v"(a.w));
+    }
+}
+
 static int run_graph()
 {
     hipStream_t s;
@@ -205,6 +216,45 @@ static int run_graph()
     for (int nmat : {4, 8, 16, 32, 64}) {
         if (timeGraph(64, 30, [&](int i) { hipLaunchKernelGGL(matvec_probe_kernel, 576, 256, 0, s, (const float4*)big + (size_t)(i % nmat) * 2304 * 192, x, (i & 1) ? x : y, 2304); }, &us)) return 1;
         printf("graph    64 mat-vec kernels 2304 x 768 (7.1 MB each) cycling through %4.0f MB  %5.2f us per kernel\n", nmat * matBytes / 1e6, us);
+    }
+    // the same chain through all 64 matrices with a second branch of the graph that reads matrix i + ahead while kernel i
+    // runs (the branch forks after kernel i - 1 and joins at the end of the graph)
+    {
+        hipStream_t s2;
+        CK(hipStreamCreateWithFlags(&s2, hipStreamNonBlocking));
+        hipEvent_t fork[64], join;
+        for (int i = 0; i < 64; i++) CK(hipEventCreateWithFlags(&fork[i], hipEventDisableTiming));
+        CK(hipEventCreateWithFlags(&join, hipEventDisableTiming));
+        for (int ahead : {1, 2, 3}) {
+            hipGraph_t g;
+            hipGraphExec_t ge;
+            CK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            for (int i = 0; i < 64; i++) {
+                if (i + ahead < 64) {
+                    CK(hipEventRecord(fork[i], s));
+                    CK(hipStreamWaitEvent(s2, fork[i], 0));
+                    hipLaunchKernelGGL(prefetch_probe_kernel, 576, 256, 0, s2, (const float4*)big + (size_t)(i + ahead) * 2304 * 192, 2304);
+                }
+                hipLaunchKernelGGL(matvec_probe_kernel, 576, 256, 0, s, (const float4*)big + (size_t)i * 2304 * 192, x, (i & 1) ? x : y, 2304);
+            }
+            CK(hipEventRecord(join, s2));
+            CK(hipStreamWaitEvent(s, join, 0));
+            CK(hipStreamEndCapture(s, &g));
+            CK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+            for (int r = 0; r < 5; r++) CK(hipGraphLaunch(ge, s));
+            CK(hipStreamSynchronize(s));
+            CK(hipEventRecord(e0, s));
+            for (int r = 0; r < 30; r++) CK(hipGraphLaunch(ge, s));
+            CK(hipEventRecord(e1, s));
+            CK(hipEventSynchronize(e1));
+            float ms;
+            CK(hipEventElapsedTime(&ms, e0, e1));
+            printf("graph    64 mat-vec kernels 2304 x 768 cycling through  453 MB, matrix i + %d read on a parallel branch  %5.2f us per kernel\n",
+                   ahead, ms * 1e3f / 30 / 64);
+            CK(hipGraphExecDestroy(ge));
+            CK(hipGraphDestroy(g));
+        }
+        CK(hipStreamDestroy(s2));
     }
     CK(hipFree(x));
     CK(hipFree(y));
