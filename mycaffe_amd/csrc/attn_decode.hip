@@ -100,6 +100,44 @@ __device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int
 // the loads of the next stage are issued before the current one is consumed.
 template <int U> struct DecodeStage { u32x4 k[U], v[U]; };
 
+// v + (v of lane ^ O), by DPP inside a row of 16 lanes and by the row-swapping permutes across rows: everything at
+// vector-ALU latency, where __shfl_xor goes through the LDS crossbar (some 50 ns per step for a lone wavefront).  The
+// sums are those of the xor butterfly, bit for bit.
+template <int CTRL, int BANK> __device__ __forceinline__ float dpp_take(float old, float v)
+{
+    return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(old), __float_as_uint(v), CTRL, 0xf, BANK, false));
+}
+template <int O> __device__ __forceinline__ float add_lane_xor(float v)
+{
+    static_assert(O == 1 || O == 2 || O == 4 || O == 8 || O == 16 || O == 32, "one bit of the lane index");
+    if constexpr (O == 1) return v + dpp_take<0xB1, 0xf>(0.f, v);          // quad_perm [1,0,3,2]
+    else if constexpr (O == 2) return v + dpp_take<0x4E, 0xf>(0.f, v);     // quad_perm [2,3,0,1]
+    else if constexpr (O == 4) {
+        // lanes 0-3 and 8-11 of a row take the lane four above (row_shl:4), the others the lane four below (row_shr:4)
+        float t = dpp_take<0x104, 0x5>(0.f, v);
+        t = dpp_take<0x114, 0xA>(t, v);
+        return v + t;
+    } else if constexpr (O == 8) return v + dpp_take<0x128, 0xf>(0.f, v);  // row_ror:8
+    else if constexpr (O == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+}
+// sum over each group of LPR adjacent lanes (a power of two), widest step first
+template <int LPR> __device__ __forceinline__ float group_sum(float v)
+{
+    if constexpr (LPR >= 64) v = add_lane_xor<32>(v);
+    if constexpr (LPR >= 32) v = add_lane_xor<16>(v);
+    if constexpr (LPR >= 16) v = add_lane_xor<8>(v);
+    if constexpr (LPR >= 8) v = add_lane_xor<4>(v);
+    if constexpr (LPR >= 4) v = add_lane_xor<2>(v);
+    if constexpr (LPR >= 2) v = add_lane_xor<1>(v);
+    return v;
+}
+
 template <typename T, int LPR, int U>
 __device__ __forceinline__ void decode_issue(DecodeStage<U>& st, const T* __restrict__ kc, const T* __restrict__ vc, long long strideT,
                                              int tb, int t1, int grp, int d0, bool active)
@@ -135,8 +173,7 @@ __device__ __forceinline__ void decode_consume(const DecodeStage<U>& st, int tb,
         float d = 0.f;
 #pragma unroll
         for (int i = 0; i < W; i++) d += qv[i] * kv[i];
-#pragma unroll
-        for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        d = group_sum<LPR>(d);
         s[u] = (tb + u * RPW + grp) < t1 ? d : -INFINITY;
     }
     float mn = m;
@@ -216,6 +253,33 @@ __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (
         for (int i = 0; i < W; i++) sacc[g][d0 + i] = acc[i];
     }
     __syncthreads();
+    constexpr int NG = NW * RPW;
+    if constexpr (NG <= 32) {
+        // Every LDS read is unconditional and the group weights are computed once, side by side: with the reads under
+        // `if (sm[i] > -inf)` the compiler emits one branch and one LDS round trip after the other.  An empty group has
+        // weight 0 and a zero accumulator, so the sums are those of the loop form below, term for term.
+        float w[NG], M = -INFINITY, L = 0.f;
+#pragma unroll
+        for (int i = 0; i < NG; i++) { w[i] = sm[i]; M = fmaxf(M, w[i]); }
+#pragma unroll
+        for (int i = 0; i < NG; i++) w[i] = w[i] > -INFINITY ? __expf(w[i] - M) : 0.f;
+        if (yfinal || threadIdx.x == 0) {
+#pragma unroll
+            for (int i = 0; i < NG; i++) L += sl[i] * w[i];
+        }
+        if (!yfinal && threadIdx.x == 0) {
+            part_store(out, M);
+            part_store(out + 1, L);
+        }
+        for (int d = threadIdx.x; d < hs; d += 256) {
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < NG; i++) v += sacc[i][d] * w[i];
+            if (yfinal) st1(yfinal + d, v / L);
+            else part_store(out + 2 + d, v);
+        }
+        return;
+    }
     float M = -INFINITY;
     for (int i = 0; i < NW * RPW; i++) M = fmaxf(M, sm[i]);
     if (yfinal) {
@@ -431,57 +495,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
         }
     };
 
-    if (a.oneIter) {
-        // The whole cache fits one iteration per split: the query and the new key / value are requested together with
-        // the length, the cache rows and the rotation factors as soon as it is known, and the row at `pos` (which the
-        // cache does not hold yet) is patched in registers instead of being stored and read back.  Arithmetic and
-        // its order are those of the general path below.
-        constexpr int RPW = 64 / LPR, U = 4, STEP = 4 * RPW * U;
-        const int t0 = split * STEP;
-        const int tb = t0 + wave * RPW * U;
-        float r[W], kr[W], vr[W];
-#pragma unroll
-        for (int i = 0; i < W; i++) { r[i] = 0.f; kr[i] = 0.f; vr[i] = 0.f; }
-        if (active) {
-            load_row(row + (size_t)h * a.hs + d0, r);
-            load_row(row + a.dim + (size_t)kvh * a.hs + d0, kr);
-            load_row(row + a.dim + a.kvd + (size_t)kvh * a.hs + d0, vr);
-        }
-        const int nAct = (len + STEP - 1) / STEP;
-        if (split >= nAct) return;
-        const int t1 = min(len, t0 + STEP);
-        DecodeStage<U> A;
-        decode_issue<TC, LPR, U>(A, kc, vc, a.kvd, tb, t1, grp, d0, active);
-        load_factors();
-        float qv[W];
-        rotate(r, qv, a.scale);
-        if (t0 <= pos && pos < t1) {
-            float ko[W];
-            rotate_key(kr, ko);
-            const u32x4 kb = Vec16<TC>::pack(ko), vb = Vec16<TC>::pack(vr);
-            if (wave == 0 && grp == 0 && active) {
-                *(u32x4*)(kc + (size_t)pos * a.kvd + d0) = kb;
-                *(u32x4*)(vc + (size_t)pos * a.kvd + d0) = vb;
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++)
-                if (tb + u * RPW + grp == pos && active) { A.k[u] = kb; A.v[u] = vb; }
-        }
-        float m = -INFINITY, l = 0.f, acc[W];
-#pragma unroll
-        for (int i = 0; i < W; i++) acc[i] = 0.f;
-        decode_consume<TC, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
-        const size_t bh = (size_t)b * a.H + h;
-        float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
-        float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
-        if (nAct == 1) {
-            decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
-            return;
-        }
-        decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
-        decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
-        return;
-    }
     int chunk = (len + a.splits - 1) / a.splits;
     chunk = ((chunk + a.rowsPerIter - 1) / a.rowsPerIter) * a.rowsPerIter;
     const int t0 = split * chunk, t1 = min(len, t0 + chunk);
@@ -522,6 +535,117 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
     }
     decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
     decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
+}
+
+// The engine form when the whole cache fits one iteration per split (seqLen <= splits * rowsPerIter): a kernel of its
+// own so that the order of its memory requests is the one written here.
+template <int LPR, typename TC>
+__global__ __launch_bounds__(256) void attn_decode_fused_step_kernel(FusedDecodeArgs a)
+{
+    constexpr int W = Vec16<TC>::W;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int grp = lane / LPR, gl = lane % LPR;
+    const int d0 = gl * W;
+    const bool active = d0 < a.hs;
+    const int half = a.hs / 2;
+    const int kvh = h / a.kvMul;
+    const int ldq = a.dim + 2 * a.kvd;
+    const float* row = a.qkv + (size_t)b * ldq;
+    TC* kc = (TC*)a.kc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    TC* vc = (TC*)a.vc + (size_t)b * a.seqLen * a.kvd + (size_t)kvh * a.hs;
+    auto load_row = [&](const float* p, float* o) {
+#pragma unroll
+        for (int j = 0; j < W / 4; j++) {
+            const float4 t = *(const float4*)(p + 4 * j);
+            o[4 * j] = t.x; o[4 * j + 1] = t.y; o[4 * j + 2] = t.z; o[4 * j + 3] = t.w;
+        }
+    };
+    float cs[W / 2], sn[W / 2];   // rotation factors of this lane's adjacent pairs (dims d0 + 2 j, d0 + 2 j + 1) at `pos`
+    auto rotate = [&](const float* in, float* out, float scale) {
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) {
+            out[2 * j] = (in[2 * j] * cs[j] - in[2 * j + 1] * sn[j]) * scale;
+            out[2 * j + 1] = (in[2 * j] * sn[j] + in[2 * j + 1] * cs[j]) * scale;
+        }
+    };
+    auto rotate_key = [&](const float* in, float* out) {
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) {
+            out[2 * j] = in[2 * j] * cs[j] - in[2 * j + 1] * sn[j];
+            out[2 * j + 1] = in[2 * j] * sn[j] + in[2 * j + 1] * cs[j];
+        }
+    };
+    // The whole cache fits one iteration per split.  Everything that does not depend on the length is requested at
+    // once, before the length is looked at: the query, the new key / value and this split's cache rows (rows past
+    // the end of the cache clamped; rows past the length are masked afterwards).  All loads are unconditional -
+    // lanes past the head size read column 0 - because loads under a branch make the compiler wait for every
+    // outstanding load at the first use of any.  The rotation factors follow as soon as the length is known, and
+    // the row at `pos` (which the cache does not hold yet) is patched in registers instead of being stored and
+    // read back.  Arithmetic and its order are those of attn_decode_fused_kernel.
+    constexpr int RPW = 64 / LPR, U = 4, STEP = 4 * RPW * U;
+    const int t0 = split * STEP;
+    const int tb = t0 + wave * RPW * U;
+    const int dc = active ? d0 : 0;
+    float r[W], kr[W], vr[W];
+    load_row(row + (size_t)h * a.hs + dc, r);
+    load_row(row + a.dim + (size_t)kvh * a.hs + dc, kr);
+    load_row(row + a.dim + a.kvd + (size_t)kvh * a.hs + dc, vr);
+    DecodeStage<U> A;
+#pragma unroll
+    for (int u = 0; u < U; u++) A.k[u] = *(const u32x4*)(kc + (size_t)min(tb + u * RPW + grp, a.seqLen - 1) * a.kvd + dc);
+#pragma unroll
+    for (int u = 0; u < U; u++) A.v[u] = *(const u32x4*)(vc + (size_t)min(tb + u * RPW + grp, a.seqLen - 1) * a.kvd + dc);
+    __builtin_amdgcn_sched_barrier(0);   // the requests above are issued before the length is asked for
+    const int len = *a.dlen, pos = len - 1;
+    const int nAct = (len + STEP - 1) / STEP;
+    if (split >= nAct) return;
+    const int t1 = min(len, t0 + STEP);
+    {
+        const size_t ti = (size_t)pos * half + dc / 2;
+#pragma unroll
+        for (int j = 0; j < W / 2; j++) { cs[j] = a.fcos[ti + j]; sn[j] = a.fsin[ti + j]; }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (!active) {
+#pragma unroll
+        for (int i = 0; i < W; i++) r[i] = 0.f;
+    }
+    float qv[W];
+    rotate(r, qv, a.scale);
+    // rows past the length hold whatever the cache memory holds: their scores are masked when they are consumed,
+    // their values are cleared here (0 x NaN would not be 0)
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        if (tb + u * RPW + grp >= t1) A.v[u] = z;
+    }
+    if (t0 <= pos && pos < t1) {
+        float ko[W];
+        rotate_key(kr, ko);
+        const u32x4 kb = Vec16<TC>::pack(ko), vb = Vec16<TC>::pack(vr);
+        if (wave == 0 && grp == 0 && active) {
+            *(u32x4*)(kc + (size_t)pos * a.kvd + d0) = kb;
+            *(u32x4*)(vc + (size_t)pos * a.kvd + d0) = vb;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (tb + u * RPW + grp == pos) { A.k[u] = kb; A.v[u] = vb; }   // every lane: none keeps what the cache held
+    }
+    float m = -INFINITY, l = 0.f, acc[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) acc[i] = 0.f;
+    decode_consume<TC, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
+    const size_t bh = (size_t)b * a.H + h;
+    float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
+    float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
+    if (nAct == 1) {
+        decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out, yout);
+        return;
+    }
+    decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
+    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
+    return;
 }
 
 // any head size / alignment: scalar loads, one wavefront per (b, h, split)
@@ -703,7 +827,10 @@ hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* 
     switch (lprp) {
 #define CASE(L)                                                                                                            \
     case L:                                                                                                                \
-        if (cacheType == F32) hipLaunchKernelGGL((attn_decode_fused_kernel<L, float>), grid, 256, 0, s, a);                \
+        if (a.oneIter) {                                                                                                   \
+            if (cacheType == F32) hipLaunchKernelGGL((attn_decode_fused_step_kernel<L, float>), grid, 256, 0, s, a);       \
+            else hipLaunchKernelGGL((attn_decode_fused_step_kernel<L, bf16_t>), grid, 256, 0, s, a);                       \
+        } else if (cacheType == F32) hipLaunchKernelGGL((attn_decode_fused_kernel<L, float>), grid, 256, 0, s, a);         \
         else hipLaunchKernelGGL((attn_decode_fused_kernel<L, bf16_t>), grid, 256, 0, s, a);                                \
         break;
         CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
