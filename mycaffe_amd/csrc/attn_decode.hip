@@ -378,6 +378,61 @@ __device__ __forceinline__ void decode_merge_last(const float* part, int* counte
     if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 }
 
+// The same for head sizes up to 64, where the first wavefront alone wrote the workgroup's partial (decode_reduce_wg: thread
+// d stores dimension d): it waits for its own stores, takes the ticket and, if it is the last one, merges with one lane
+// per dimension and sixteen splits' loads in flight - no workgroup barrier and no LDS on the way.  The other wavefronts
+// are done.
+template <typename T>
+__device__ __forceinline__ void decode_merge_last_wave(const float* part, int* counter, int splits, int hs, T* __restrict__ y)
+{
+    if (threadIdx.x >= 64) return;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int ticket = 0;
+    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = __builtin_amdgcn_readfirstlane(ticket);
+    if (ticket != splits - 1) return;
+    const int d = threadIdx.x < hs ? threadIdx.x : 0;
+    const int stride = hs + 2;
+    constexpr int NS = 16;
+    float M = -INFINITY, L = 0.f, A = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += NS) {
+        float ms[NS], ls[NS], vs[NS];
+#pragma unroll
+        for (int k = 0; k < NS; k++) {
+            const bool ok = s0 + k < splits;
+            const float* p = part + (size_t)(ok ? s0 + k : s0) * stride;
+            ms[k] = part_load(p);
+            ls[k] = part_load(p + 1);
+            vs[k] = part_load(p + 2 + d);
+            if (!ok) ms[k] = -INFINITY;
+        }
+        float Mn = M;
+#pragma unroll
+        for (int k = 0; k < NS; k++) Mn = fmaxf(Mn, ms[k]);
+        if (Mn > -INFINITY) {
+            const float c = __expf(M - Mn);   // M == -inf gives 0
+            L *= c;
+            A *= c;
+#pragma unroll
+            for (int k = 0; k < NS; k++) {
+                const float w = ms[k] > -INFINITY ? __expf(ms[k] - Mn) : 0.f;
+                L += ls[k] * w;
+                A += vs[k] * w;
+            }
+            M = Mn;
+        }
+    }
+    if ((int)threadIdx.x < hs) st1(y + threadIdx.x, A / L);
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+}
+
+template <typename T>
+__device__ __forceinline__ void decode_merge(const float* part, int* counter, int splits, int hs, T* __restrict__ y)
+{
+    if (hs <= 64) decode_merge_last_wave<T>(part, counter, splits, hs, y);
+    else decode_merge_last<T>(part, counter, splits, hs, y);
+}
+
 // partial layout: part[((b*H + h)*splits + s) * (hs + 2)] = {m, l, acc[hs]}
 template <typename T, int LPR>
 __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
@@ -428,7 +483,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a)
     }
     decode_reduce_wg<T, LPR>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
     if (a.counters)
-        decode_merge_last<T>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, (T*)a.y + bh * a.hs);
+        decode_merge<T>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, (T*)a.y + bh * a.hs);
 }
 
 // Engine form (fp32): one launch per layer does what the reference's decode step does between the QKV
@@ -534,7 +589,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(FusedDecodeArgs 
         return;
     }
     decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
-    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
+    decode_merge<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
 }
 
 // The engine form when the whole cache fits one iteration per split (seqLen <= splits * rowsPerIter): a kernel of its
@@ -644,7 +699,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_step_kernel(FusedDecode
         return;
     }
     decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
-    decode_merge_last<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
+    decode_merge<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
     return;
 }
 
