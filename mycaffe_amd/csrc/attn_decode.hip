@@ -236,10 +236,13 @@ __device__ __forceinline__ void part_store(float* p, float v) { __hip_atomic_sto
 __device__ __forceinline__ float part_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Merges the 4 * (64/LPR) lane groups of a workgroup through LDS and writes {M, L, acc[hs]} to `out`, or, when
-// this workgroup saw every cached row (yfinal set), the normalised result straight to yfinal.
+// this workgroup saw every cached row (yfinal set), the normalised result straight to yfinal.  With plainAcc set the
+// partial is meant for the NEXT kernel of the stream, which merges the splits itself: {M, L} go to `out` and acc[hs] to
+// plainAcc with ordinary stores (the kernel boundary makes them visible).
 template <typename T, int LPR, typename TY = T>
 __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (&acc)[Vec16<T>::W], int wave, int grp, int gl,
-                                                 int d0, bool active, int hs, float* __restrict__ out, TY* __restrict__ yfinal = nullptr)
+                                                 int d0, bool active, int hs, float* __restrict__ out, TY* __restrict__ yfinal = nullptr,
+                                                 float* __restrict__ plainAcc = nullptr)
 {
     constexpr int W = Vec16<T>::W;
     constexpr int RPW = 64 / LPR, NW = 4;
@@ -268,14 +271,15 @@ __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (
             for (int i = 0; i < NG; i++) L += sl[i] * w[i];
         }
         if (!yfinal && threadIdx.x == 0) {
-            part_store(out, M);
-            part_store(out + 1, L);
+            if (plainAcc) { out[0] = M; out[1] = L; }
+            else { part_store(out, M); part_store(out + 1, L); }
         }
         for (int d = threadIdx.x; d < hs; d += 256) {
             float v = 0.f;
 #pragma unroll
             for (int i = 0; i < NG; i++) v += sacc[i][d] * w[i];
             if (yfinal) st1(yfinal + d, v / L);
+            else if (plainAcc) plainAcc[d] = v;
             else part_store(out + 2 + d, v);
         }
         return;
@@ -296,14 +300,15 @@ __device__ __forceinline__ void decode_reduce_wg(float m, float l, const float (
     if (threadIdx.x == 0) {
         float L = 0.f;
         for (int i = 0; i < NW * RPW; i++) L += (sm[i] > -INFINITY) ? sl[i] * __expf(sm[i] - M) : 0.f;
-        part_store(out, M);
-        part_store(out + 1, L);
+        if (plainAcc) { out[0] = M; out[1] = L; }
+        else { part_store(out, M); part_store(out + 1, L); }
     }
     for (int d = threadIdx.x; d < hs; d += 256) {
         float v = 0.f;
         for (int i = 0; i < NW * RPW; i++)
             if (sm[i] > -INFINITY) v += sacc[i][d] * __expf(sm[i] - M);
-        part_store(out + 2 + d, v);
+        if (plainAcc) plainAcc[d] = v;
+        else part_store(out + 2 + d, v);
     }
 }
 
@@ -496,6 +501,9 @@ struct FusedDecodeArgs {
     int B, H, kvMul, hs, dim, kvd, seqLen, splits, rowsPerIter;
     float scale;
     bool oneIter;   // seqLen <= splits * rowsPerIter: a split never holds more than one iteration of rows
+    // B == 1 and oneIter only: leave the merge of the splits to the next kernel.  Split s of head h writes its
+    // accumulator to part[s * dim + h * hs ..] and {m, l} to part[splits * dim + (s * H + h) * 2 ..]; y is not written.
+    bool deferMerge;
 };
 
 // TC: storage type of the caches (fp32, or bf16: the rotated key and the value are rounded when they are appended, and the
@@ -691,6 +699,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_step_kernel(FusedDecode
 #pragma unroll
     for (int i = 0; i < W; i++) acc[i] = 0.f;
     decode_consume<TC, LPR, U>(A, tb, t1, grp, qv, m, l, acc);
+    if (a.deferMerge) {
+        decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs,
+                                         a.part + (size_t)a.splits * a.dim + ((size_t)split * a.H + h) * 2, (float*)nullptr,
+                                         a.part + (size_t)split * a.dim + (size_t)h * a.hs);
+        return;
+    }
     const size_t bh = (size_t)b * a.H + h;
     float* out = a.part + (bh * a.splits + split) * (a.hs + 2);
     float* yout = a.y + (size_t)b * a.dim + (size_t)h * a.hs;
@@ -700,7 +714,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_step_kernel(FusedDecode
     }
     decode_reduce_wg<TC, LPR, float>(m, l, acc, wave, grp, gl, d0, active, a.hs, out);
     decode_merge<float>(a.part + bh * a.splits * (a.hs + 2), a.counters + bh, nAct, a.hs, yout);
-    return;
 }
 
 // any head size / alignment: scalar loads, one wavefront per (b, h, split)
@@ -858,9 +871,26 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
     return launch_decode<bf16_t>(s, a, kvH);
 }
 
+// The splits of a launch that leaves the merge to the next kernel (batch 1, the whole cache in one iteration per split), and
+// the rows each of them covers; 0 when the launch cannot be of that kind.
+int attn_decode_fused_deferred_splits(int B, int H, int hs, int seqLen, DType cacheType, int* rowsPerSplit)
+{
+    const int W = cacheType == F32 ? 4 : 8;
+    if (B != 1 || H <= 0 || hs <= 0 || hs % W != 0 || seqLen <= 0) return 0;
+    int lpr = hs / W, lprp = 1;
+    while (lprp < lpr) lprp <<= 1;
+    if (lprp > 64) return 0;
+    const int rpi = 4 * (64 / lprp) * 4;
+    int splits, chunk;
+    pick_splits(B, H, seqLen, rpi, &splits, &chunk);
+    if (seqLen > splits * rpi) return 0;
+    if (rowsPerSplit) *rowsPerSplit = rpi;
+    return splits;
+}
+
 hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* vc, DType cacheType, float* y, int B, int H, int kvH,
                                int hs, int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
-                               size_t workspaceBytes, int* counters)
+                               size_t workspaceBytes, int* counters, bool deferMerge)
 {
     if (B <= 0 || H <= 0 || hs <= 0 || seqLen <= 0) return hipSuccess;
     const int W = cacheType == F32 ? 4 : 8;   // elements per 16-byte cache chunk
@@ -878,6 +908,8 @@ hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* 
     pick_splits(B, H, seqLen, a.rowsPerIter, &a.splits, &chunk);
     a.scale = scale;
     a.oneIter = seqLen <= a.splits * a.rowsPerIter;
+    a.deferMerge = deferMerge;
+    if (deferMerge && (B != 1 || !a.oneIter)) return hipErrorInvalidValue;
     dim3 grid(a.splits, H, B);
     switch (lprp) {
 #define CASE(L)                                                                                                            \

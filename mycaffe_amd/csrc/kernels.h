@@ -165,9 +165,14 @@ hipError_t k_attn_decode(hipStream_t s, DType dt, const void* q, const void* kc,
 // Decode step of the llama2 engine in one launch: rotate q / k at position *dlen - 1, append k, v to the caches
 // ([B][seqLen][kvH*hs], stored as cacheType: fp32, or bf16 with hs a multiple of 8), attend over positions
 // 0 .. *dlen - 1.  qkv: [B][(H + 2 kvH) hs] raw fp32 projections, y: [B][H*hs] fp32.
+// deferMerge (batch 1 with the whole cache in one iteration of rows per split; attn_decode_fused_deferred_splits says whether
+// and how many splits): y is not written.  Split s leaves its accumulator of head h at workspace[s * H*hs + h * hs ..] and
+// {running maximum, sum} at workspace[splits * H*hs + (s * H + h) * 2 ..] (fp32) for the next kernel of the stream, which
+// merges the ceil(*dlen / rowsPerSplit) splits that hold rows (k_llama_matvec_merge in the engine).
 hipError_t k_attn_decode_fused(hipStream_t s, const float* qkv, void* kc, void* vc, DType cacheType, float* y, int B, int H, int kvH,
                                int hs, int seqLen, float scale, const float* fcos, const float* fsin, const int* dlen, void* workspace,
-                               size_t workspaceBytes, int* counters);
+                               size_t workspaceBytes, int* counters, bool deferMerge = false);
+int attn_decode_fused_deferred_splits(int B, int H, int hs, int seqLen, DType cacheType, int* rowsPerSplit);
 // rotate q (B,H,hs) and knew (B,kvH,hs) at position pos and append knew/vnew to the caches at pos
 hipError_t k_rope_append(hipStream_t s, DType dt, void* q, void* knew, const void* vnew, void* kc, void* vc, int B,
                          int H, int kvH, int hs, int pos, long long strideB, long long strideH, long long strideT,

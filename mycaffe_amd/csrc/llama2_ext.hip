@@ -263,6 +263,85 @@ __global__ __launch_bounds__(256) void matvec_kernel(const T* __restrict__ W, co
     for (int b = 1; b < B; b++) sequence(b, std::false_type());
 }
 
+// Output projection of a decode step whose attention left its split partials unmerged (batch 1):
+//   y[r] += W[r,:] . att,   att[h*hs + d] = sum_s acc[s][h][d] e^(m[s][h] - M[h]) / sum_s l[s][h] e^(m[s][h] - M[h])
+// over the nAct = ceil(*dlen / rowsPerSplit) splits that hold rows.  Thread t of a workgroup merges columns 4t .. 4t + 3
+// (one head: hs % 4 == 0) with all NS splits' loads in flight, the merged vector meets the wavefronts in LDS, and each
+// wavefront then finishes its row of W as matvec_kernel does.  This replaces the attention kernel's own merge - partial
+// stores acknowledged, a ticket, the partials read back: three trips to memory in a row - by loads that travel together
+// with the weights.  Splits beyond nAct hold stale partials: they are masked, not multiplied away.
+template <typename T, int CH, bool WIDE, int NS>
+__global__ __launch_bounds__(256) void matvec_merge_kernel(const T* __restrict__ W, const float* __restrict__ partAcc,
+                                                           const float* __restrict__ partML, const int* __restrict__ dlen,
+                                                           int splits, int rowsPerSplit, int H, int hs, float* __restrict__ y, int rows,
+                                                           int n)
+{
+    __shared__ float4 xs[256];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int r = min(blockIdx.x * 4 + (tid >> 6), rows - 1);   // a wavefront past the end repeats the last row and stores nothing
+    const bool store = blockIdx.x * 4 + (tid >> 6) < rows && lane == 0;
+    constexpr int LW = WIDE ? 8 : 4;
+    // partials first: the longer chain (merge, LDS, barrier) hangs on them
+    const int col = min(tid * 4, n - 4);
+    const int h = col / hs;
+    float4 pa[NS];
+    float2 pm[NS];
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        const int kc = min(k, splits - 1);
+        pa[k] = *(const float4*)(partAcc + (size_t)kc * n + col);
+        pm[k] = *(const float2*)(partML + ((size_t)kc * H + h) * 2);
+    }
+    const float prev = y[r];
+    float4 w[CH];
+    if (WIDE) {
+#pragma unroll
+        for (int c = 0; c < CH; c += 2) {
+            float lo[8];
+            Row8<T>::load(W + (size_t)r * n + min(matvec_col<WIDE>(c, lane), n - LW), lo);
+            w[c] = make_float4(lo[0], lo[1], lo[2], lo[3]);
+            w[c + 1] = make_float4(lo[4], lo[5], lo[6], lo[7]);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < CH; c++) w[c] = Row4<T>::load(W + (size_t)r * n + min(matvec_col<WIDE>(c, lane), n - 4));
+    }
+    __builtin_amdgcn_sched_barrier(0);   // every request above is issued before the length is asked for
+    const int len = *dlen;
+    const int nAct = (len + rowsPerSplit - 1) / rowsPerSplit;
+    float M = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        if (k >= nAct) pm[k].x = -INFINITY;
+        M = fmaxf(M, pm[k].x);
+    }
+    float L = 0.f;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        const bool on = k < nAct;
+        const float e = on ? __expf(pm[k].x - M) : 0.f;
+        L += on ? pm[k].y * e : 0.f;
+        a.x += on ? pa[k].x * e : 0.f;
+        a.y += on ? pa[k].y * e : 0.f;
+        a.z += on ? pa[k].z * e : 0.f;
+        a.w += on ? pa[k].w * e : 0.f;
+    }
+    const float inv = 1.0f / L;
+    xs[tid] = make_float4(a.x * inv, a.y * inv, a.z * inv, a.w * inv);
+    __syncthreads();
+    float a0 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int j = matvec_col<WIDE>(c, lane);
+        float4 xv = xs[min(j, n - 4) >> 2];
+        const float keep = j < n ? 1.f : 0.f;
+        a0 += keep * (w[c].x * xv.x + w[c].y * xv.y + w[c].z * xv.z + w[c].w * xv.w);
+    }
+    a0 = wsum(a0);
+    if (store) y[r] = prev + a0;
+}
+
 // The same family for rows too long to hold in registers (n > 4096): one wavefront per row walks K in slabs of
 // 64 x 4 columns, four slabs in flight.  With NORM the sum of squares of x (L2 resident) is taken in a first walk.
 template <typename T, int MODE, bool NORM>
@@ -790,6 +869,8 @@ public:
     int lastPrefillRows = 0;     // sequences x prompt positions it covered
     int mvRows = 0;              // weight rows per wavefront in the mat-vec kernels (0: chosen per shape)
     void set_mv_rows(int r) { mvRows = r; graphB = -1; }   // the captured step is rebuilt at the next generation
+    bool defer_merge = true;     // batch 1: the output projection merges the attention's splits (when the shapes allow)
+    void set_defer_merge(bool on) { defer_merge = on; graphB = -1; }
     int shared_classifier = 0;
     int timedFrom = -1;          // first step of the timed span (-1: first step after the prompt)
     std::string lastError;       // detail of the last failed load, handed to the caller's error text
@@ -1220,6 +1301,35 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
     return hipGetLastError();
 }
 
+constexpr int kMergeSplits = 16;   // split partials a thread of matvec_merge_kernel holds in flight
+// whether the output projection can merge the attention's splits itself: one float4 of the merged vector per thread
+static bool matvec_merge_usable(int n, int hs, int splits)
+{
+    return n % 4 == 0 && n <= 1024 && hs % 4 == 0 && splits >= 1 && splits <= kMergeSplits;
+}
+template <typename T>
+static hipError_t launch_matvec_merge(hipStream_t s, const void* W, const float* part, int splits, int rowsPerSplit, const int* dlen,
+                                      int H, int hs, float* y, int rows, int n)
+{
+    if (!matvec_merge_usable(n, hs, splits)) return hipErrorInvalidValue;
+    const float* partML = part + (size_t)splits * n;
+    const int grid = (rows + 3) / 4;
+    const bool wide = sizeof(T) == 2 && n % 8 == 0 && (((uintptr_t)W) & 15) == 0;
+    const int ch = wide ? 2 * ((n / 8 + 63) / 64) : (n / 4 + 63) / 64;
+#define MVM(C, WIDE_) hipLaunchKernelGGL((matvec_merge_kernel<T, C, WIDE_, kMergeSplits>), grid, 256, 0, s, (const T*)W, part, partML, dlen, splits, rowsPerSplit, H, hs, y, rows, n)
+    if constexpr (sizeof(T) == 2) {
+        if (wide) {
+            if (ch <= 2) MVM(2, true); else MVM(4, true);
+            return hipGetLastError();
+        }
+    }
+    if (ch <= 2) MVM(2, false);
+    else if (ch <= 3) MVM(3, false);
+    else MVM(4, false);
+#undef MVM
+    return hipGetLastError();
+}
+
 // The same kernels over the M rows of a prompt pass (row = one position of one sequence): up to 128 rows share one walk
 // over the weights, so a single sequence's prompt streams every matrix once (or a few times) instead of going through
 // 128 x 128 GEMM tiles that would leave most of the chip idle at this height.
@@ -1252,6 +1362,10 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
 #define SPAN_BEGIN(cls) do { if (prof) HIPCHK(prof->begin(cls, s)); } while (0)
 #define SPAN_END() do { if (prof) HIPCHK(prof->end(s)); } while (0)
     const float scale = 1.0f / sqrtf((float)hs);
+    // batch 1 with the cache in one iteration of rows per split: the attention leaves its splits to the output projection
+    int deferRows = 0;
+    int deferSplits = defer_merge ? attn_decode_fused_deferred_splits(B, cfg.n_heads, hs, cfg.seq_len, state_kv_bf16 ? BF16 : F32, &deferRows) : 0;
+    if (!matvec_merge_usable(dim, hs, deferSplits)) deferSplits = 0;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
         const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
@@ -1264,11 +1378,12 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
         // xb = attention(rope(q), cache[0..pos] with rope(k), v appended)
         SPAN_BEGIN(SC_ATTN_DECODE);
         HIPCHK(k_attn_decode_fused(s, qkv, kcl, vcl, state_kv_bf16 ? BF16 : F32, xb, B, cfg.n_heads, cfg.n_kv_heads, hs, cfg.seq_len, scale, fcos, fsin,
-                                   &dstate->len, ws, wsBytes, dcount));
+                                   &dstate->len, ws, wsBytes, dcount, deferSplits > 0));
         SPAN_END();
-        // x += Wo xb
+        // x += Wo xb (with the merge of the attention's splits in front when it was left to this kernel)
         SPAN_BEGIN(SC_MATVEC_WO);
-        HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim, mvRows)));
+        if (deferSplits > 0) HIPCHK((launch_matvec_merge<T>(s, w.wo, (const float*)ws, deferSplits, deferRows, &dstate->len, cfg.n_heads, hs, x, dim, dim)));
+        else HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim, mvRows)));
         SPAN_END();
         // hb = silu(W1 rmsnorm(x)) * (W3 rmsnorm(x))
         SPAN_BEGIN(SC_MATVEC_W13);
@@ -1725,6 +1840,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 6) m->batchLogits = pIn[2] != 0.f;
         else if (opt == 7) m->engine.use_prefill = pIn[2] != 0.f;
         else if (opt == 8) m->engine.set_kv_bf16(pIn[2] != 0.f);
+        else if (opt == 9) m->engine.set_defer_merge(pIn[2] != 0.f);
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }

@@ -65,6 +65,34 @@ def test_logits_and_ids_tiny(llm, tmp_path, cfg, shared, std):
     assert np.array_equal(llm.GenerateIds(prompt, n), ids)
 
 
+@pytest.mark.parametrize("name,cfg,std,nP,n", [
+    ("hs16", TINY, 0.2, 5, 56),                                                                   # one split most of the way
+    ("hs48", C1, 0.02, 8, 200),                                                                   # lanes past the head size idle
+    ("hs64_gqa", dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256), 0.08, 70, 180)])
+def test_batch1_split_merge_in_the_output_projection_or_in_the_attention_kernel(llm, tmp_path, name, cfg, std, nP, n):
+    """At batch 1 (cache within one iteration of rows per split) the attention kernel leaves its split partials to the
+    output projection, which merges them in front of its mat-vec; SET_OPTION 9 = 0 keeps the merge in the attention kernel
+    (last-ticket workgroup).  Both against the checker, logits at every position, eager and replayed graph, fp32 and
+    16-bit cache."""
+    blob, _ = O.random_weights(cfg, seed=21, shared_classifier=False, std=std)
+    path = str(tmp_path / (name + ".bin"))
+    O.write_checkpoint_v1(path, cfg, blob, False)
+    llm.Load(path)
+    prompt = np.random.default_rng(4).integers(3, cfg["vocab_size"], nP)
+    ref_ids, ref_logits = O.Llama(cfg, blob, False).generate_greedy(prompt, n, want_logits=True)
+    llm.SetOption(7, 0)   # one step per prompt position: every position goes through the decode attention
+    got = {}
+    for defer in (1, 0):
+        llm.SetOption(9, defer)
+        ids, logits = llm.GenerateIds(prompt, n, want_logits=True)
+        assert_close(logits, ref_logits, FP32_RTOL, "%s logits, merge deferred %d" % (name, defer))
+        assert np.array_equal(llm.GenerateIds(prompt, n), ids)
+        assert llm.LastRunUsedGraph()
+        got[defer] = ids
+    _check_ids(got[1], ref_ids, ref_logits, name)
+    _check_ids(got[0], ref_ids, ref_logits, name)
+
+
 def test_grouped_query_heads_over_several_cache_splits(llm, tmp_path):
     """Head size 64 with two query heads per key / value head and a cache of 256 positions: the fused decode attention
     cuts the cache into up to four 64-row splits, the heads of a group append the same rotated key, and the split that
