@@ -10,6 +10,7 @@
 // such loads per operand are kept in flight.  Each lane group keeps its own
 // running max / sum / output slice; groups are merged through LDS at the end.
 #include "kernels.h"
+#include "lane_ops.h"
 
 namespace mch {
 
@@ -99,44 +100,6 @@ __device__ inline void decode_range(const DecodeArgs& a, int split, int* t0, int
 // A stage is U row groups of K and of V per wavefront, kept as loaded (16 bytes per lane and row);
 // the loads of the next stage are issued before the current one is consumed.
 template <int U> struct DecodeStage { u32x4 k[U], v[U]; };
-
-// v + (v of lane ^ O), by DPP inside a row of 16 lanes and by the row-swapping permutes across rows: everything at
-// vector-ALU latency, where __shfl_xor goes through the LDS crossbar (some 50 ns per step for a lone wavefront).  The
-// sums are those of the xor butterfly, bit for bit.
-template <int CTRL, int BANK> __device__ __forceinline__ float dpp_take(float old, float v)
-{
-    return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(old), __float_as_uint(v), CTRL, 0xf, BANK, false));
-}
-template <int O> __device__ __forceinline__ float add_lane_xor(float v)
-{
-    static_assert(O == 1 || O == 2 || O == 4 || O == 8 || O == 16 || O == 32, "one bit of the lane index");
-    if constexpr (O == 1) return v + dpp_take<0xB1, 0xf>(0.f, v);          // quad_perm [1,0,3,2]
-    else if constexpr (O == 2) return v + dpp_take<0x4E, 0xf>(0.f, v);     // quad_perm [2,3,0,1]
-    else if constexpr (O == 4) {
-        // lanes 0-3 and 8-11 of a row take the lane four above (row_shl:4), the others the lane four below (row_shr:4)
-        float t = dpp_take<0x104, 0x5>(0.f, v);
-        t = dpp_take<0x114, 0xA>(t, v);
-        return v + t;
-    } else if constexpr (O == 8) return v + dpp_take<0x128, 0xf>(0.f, v);  // row_ror:8
-    else if constexpr (O == 16) {
-        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-    } else {
-        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-    }
-}
-// sum over each group of LPR adjacent lanes (a power of two), widest step first
-template <int LPR> __device__ __forceinline__ float group_sum(float v)
-{
-    if constexpr (LPR >= 64) v = add_lane_xor<32>(v);
-    if constexpr (LPR >= 32) v = add_lane_xor<16>(v);
-    if constexpr (LPR >= 16) v = add_lane_xor<8>(v);
-    if constexpr (LPR >= 8) v = add_lane_xor<4>(v);
-    if constexpr (LPR >= 4) v = add_lane_xor<2>(v);
-    if constexpr (LPR >= 2) v = add_lane_xor<1>(v);
-    return v;
-}
 
 template <typename T, int LPR, int U>
 __device__ __forceinline__ void decode_issue(DecodeStage<U>& st, const T* __restrict__ kc, const T* __restrict__ vc, long long strideT,

@@ -36,6 +36,7 @@
 #include "../../include/mycaffe_hip_abi.h"
 #include "bpe_tokenizer.h"
 #include "kernels.h"
+#include "lane_ops.h"
 
 namespace mch {
 
@@ -55,24 +56,8 @@ template <typename T> __device__ inline float wld(const T* p, size_t i);
 template <> __device__ inline float wld<float>(const float* p, size_t i) { return p[i]; }
 template <> __device__ inline float wld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
 
-// Sum over the 64 lanes of a wavefront, the result in every lane: four DPP steps inside each row of 16 lanes, then the
-// two row-swapping permutes.  All of it runs at vector-ALU latency; the same butterfly through __shfl_xor goes through
-// the LDS crossbar six times and costs 0.1 - 0.2 us at the end of a kernel that is a few microseconds long.
-template <int CTRL> __device__ __forceinline__ float wsum_dpp(float v)
-{
-    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xf, 0xf, false));
-}
-__device__ inline float wsum(float v)
-{
-    v += wsum_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
-    v += wsum_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
-    v += wsum_dpp<0x124>(v);   // row_ror:4
-    v += wsum_dpp<0x128>(v);   // row_ror:8
-    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
-    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
-}
+// sum over the 64 lanes of a wavefront, the result in every lane
+__device__ inline float wsum(float v) { return group_sum<64>(v); }
 
 // x[b,:] = emb[token,:] where token is the forced prompt id while pos < n_prompt and
 // the previously sampled id afterwards (generate loop, llm.cpp:208-228)
@@ -589,11 +574,7 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
     } else {
         for (int i = threadIdx.x; i < V; i += 1024) take(lg[i], i);
     }
-    for (int o = 32; o > 0; o >>= 1) {
-        float ov = __shfl_xor(bv, o, 64);
-        int oi = __shfl_xor(bi, o, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    wave_argmax_first(bv, bi);
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) { sv[w] = bv; si[w] = bi; }
     __syncthreads();
@@ -612,8 +593,10 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
     const int tok = stok;
     for (int i = threadIdx.x; i < dim; i += 1024) x[(size_t)b * dim + i] = wld(emb, (size_t)tok * dim + i);
     if (threadIdx.x == 0) {
-        if (atomicAdd(ticket, 1) == (int)gridDim.x - 1) {
-            *ticket = 0;
+        // the last sequence to finish advances the position; a single sequence has no one to wait for (and no atomic
+        // whose answer the kernel would have to wait for before it can end)
+        if (gridDim.x == 1 || atomicAdd(ticket, 1) == (int)gridDim.x - 1) {
+            if (gridDim.x > 1) *ticket = 0;
             st->pos = pos + 1;
             st->len = pos + 2;
         }
