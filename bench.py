@@ -148,7 +148,7 @@ def step_roofline(inf, head, steps, warmup):
                   "algorithmic_MB_per_launch": round(v[2] / v[1] / 1e6, 3) if v[2] > 0 else None}
               for k, v in prof.items() if v[1] > 0}
     how = "one replay of the captured graph" if head.get("graph") else "62 eager launches (no graph: asked for, or capture failed)"
-    return {"kernel": "decode step = %s (49 matvec_kernel, 12 attn_decode_fused_kernel, 1 sample_advance_kernel)" % how,
+    return {"kernel": "decode step = %s (37 matvec_kernel, 12 attn_decode_fused_step_kernel, 12 matvec_merge_kernel, 1 sample_advance_kernel)" % how,
             "graph_replay": bool(head.get("graph")),
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic("decode_step"),

@@ -273,7 +273,10 @@ enum {
      *                 value caches: fp32 (0, default) or bf16 (1: rotated keys and values are rounded to
      *                 nearest-even when they are appended, every step attends over the rounded rows;
      *                 activations stay fp32; needs a head size that is a multiple of 8, otherwise the
-     *                 caches stay fp32); takes effect at the next generation
+     *                 caches stay fp32); takes effect at the next generation; option 9 = where the
+     *                 partial results of a single sequence's attention splits are merged: in front of
+     *                 the output projection's mat-vec (1, default, when dim <= 1024 and the cache fits
+     *                 one pass of rows per split) or inside the attention kernel (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were
