@@ -401,8 +401,8 @@ __global__ __launch_bounds__(256) void matvec_loop_kernel(const T* __restrict__ 
 // folded into x.  Partial tiles of the wavefronts meet in LDS; wavefront 0 finishes.
 typedef float floatx4v __attribute__((ext_vector_type(4)));
 
-template <typename T, int MODE, bool NORM, int G = 1>
-__global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
+template <typename T, int MODE, bool NORM, int G = 1, int NS = 8>
+__global__ __launch_bounds__(NS * 64) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
                                                           const float* __restrict__ g, float* __restrict__ y, int rows, int n,
                                                           int B, int ldy, int nGroups)
 {
@@ -415,9 +415,9 @@ __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ 
     if (r0 >= rows) return;   // the grid is padded to a multiple of 8 row tiles
     // G groups of 16 sequences (or prompt rows) per pass: a slab of weights is loaded once and multiplied into all of
     // them, so up to 128 rows of x share one walk over W (the batched prompt pass of a single sequence)
-    __shared__ float part[8][(MODE == 2 ? 2 : 1) * 256];
-    __shared__ float sspart[8][16];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NS = blockDim.x >> 6;
+    __shared__ __attribute__((aligned(16))) float part[NS][(MODE == 2 ? 2 : 1) * 256];
+    __shared__ float sspart[NS][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;   // NS wavefronts: a compile-time count keeps the final sums unrolled
     const int i = lane & 15, kk = lane >> 4;
     const T* wr = W + (size_t)min(r0 + i, rows - 1) * n;
     bool jv[G];                                 // this lane's batch column exists
@@ -504,15 +504,21 @@ __global__ __launch_bounds__(512) void matvec_mfma_kernel(const T* __restrict__ 
         for (int v = 0; v < 4; v++) {
             d[v] = 0.f;
             d2[v] = 0.f;
-            for (int w_ = 0; w_ < NS; w_++) {
-                d[v] += part[w_][lane * 4 + v];
-                if (MODE == 2) d2[v] += part[w_][256 + lane * 4 + v];
+        }
+#pragma unroll
+        for (int w_ = 0; w_ < NS; w_++) {
+            const float4 p = *(const float4*)&part[w_][lane * 4];
+            d[0] += p.x; d[1] += p.y; d[2] += p.z; d[3] += p.w;
+            if (MODE == 2) {
+                const float4 p2 = *(const float4*)&part[w_][256 + lane * 4];
+                d2[0] += p2.x; d2[1] += p2.y; d2[2] += p2.z; d2[3] += p2.w;
             }
         }
         if (!jv[q]) continue;
         float inv = 1.f;
         if (NORM) {
             float t = 0.f;
+#pragma unroll
             for (int w_ = 0; w_ < NS; w_++) t += sspart[w_][i];
             inv = 1.0f / sqrtf(t / n + 1e-5f);
         }
@@ -1252,7 +1258,8 @@ static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, co
         const int ns = rows >= 8192 ? 4 : 8;   // fewer, longer wavefronts once the rows alone fill the chip
         // every group of 16 sequences walks the weights in the same launch
         const int nGroups = (B + 15) / 16, tiles8 = ((rows + 15) / 16 + 7) / 8;
-        hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM>), tiles8 * 8 * nGroups, ns * 64, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
+        if (ns == 4) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 4>), tiles8 * 8 * nGroups, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
+        else hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 8>), tiles8 * 8 * nGroups, 512, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
         return hipGetLastError();
     }
     // one row per wavefront fills the chip for the layer matrices; the classifier has rows to spare
