@@ -390,6 +390,43 @@ __global__ __launch_bounds__(256) void matvec_loop_kernel(const T* __restrict__ 
     }
 }
 
+// Tile-packed copy of a weight matrix for matvec_mfma_kernel.  In the row-major matrix one load instruction of that kernel
+// touches 16 rows (64 bytes of each): sixteen half-used cache lines.  The packed copy stores, for every tile of 16 rows
+// and every slab of 32 columns, the 2 KB (fp32) or 1 KB (bf16) of the slab in the order the lanes read it, so that an
+// instruction reads 1 KB of consecutive bytes: fp32 [tile][slab][half][lane][4], lane (i = row, kk) holding columns
+// 16 half + 4 kk .. + 3; bf16 [tile][slab][lane][8], columns 8 kk .. 8 kk + 7.  Rows past the end are zero.
+template <typename T> struct PackedSlab;
+template <> struct PackedSlab<float> {
+    __device__ static inline void w(const float* slab, int lane, float* o)
+    {
+        const float4 a = *(const float4*)(slab + lane * 4), b = *(const float4*)(slab + 256 + lane * 4);
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+};
+template <> struct PackedSlab<bf16_t> {
+    __device__ static inline void w(const bf16_t* slab, int lane, float* o) { Row8<bf16_t>::load(slab + lane * 8, o); }
+};
+template <typename T>
+__global__ void pack_tiles_kernel(const T* __restrict__ W, T* __restrict__ P, int rows, int n)
+{
+    constexpr int E = 16 / sizeof(T);                 // elements per 16-byte piece
+    constexpr int PPS = 512 / E;                      // pieces per slab
+    const int nit = n >> 5, tiles = (rows + 15) >> 4;
+    const size_t total = (size_t)tiles * nit * PPS;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+        const int piece = (int)(idx % PPS);
+        const size_t ts = idx / PPS;
+        const int slab = (int)(ts % nit), tile = (int)(ts / nit);
+        const int lane = piece & 63, half = piece >> 6;       // bf16: one piece per lane, half stays 0
+        const int i = lane & 15, kk = lane >> 4;
+        const int r = tile * 16 + i;
+        const int c = slab * 32 + (sizeof(T) == 4 ? 16 * half + 4 * kk : 8 * kk);
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (r < rows) v = *(const uint4*)(W + (size_t)r * n + c);
+        *(uint4*)(P + idx * E) = v;
+    }
+}
+
 // Batched form of the mat-vec family (2 or more sequences): the same three epilogues, computed on the matrix
 // cores so that a decode step stays bound by the weight stream instead of by vector ALU work.  A workgroup owns
 // 16 rows of W; its wavefronts take the 32-column slabs of K round robin.  Per slab a lane (row i = lane % 16,
@@ -401,7 +438,7 @@ __global__ __launch_bounds__(256) void matvec_loop_kernel(const T* __restrict__ 
 // folded into x.  Partial tiles of the wavefronts meet in LDS; wavefront 0 finishes.
 typedef float floatx4v __attribute__((ext_vector_type(4)));
 
-template <typename T, int MODE, bool NORM, int G = 1, int NS = 8>
+template <typename T, int MODE, bool NORM, int G = 1, int NS = 8, bool PACKED = false>
 __global__ __launch_bounds__(NS * 64) void matvec_mfma_kernel(const T* __restrict__ W, const float* __restrict__ x,
                                                           const float* __restrict__ g, float* __restrict__ y, int rows, int n,
                                                           int B, int ldy, int nGroups)
@@ -419,7 +456,10 @@ __global__ __launch_bounds__(NS * 64) void matvec_mfma_kernel(const T* __restric
     __shared__ float sspart[NS][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;   // NS wavefronts: a compile-time count keeps the final sums unrolled
     const int i = lane & 15, kk = lane >> 4;
-    const T* wr = W + (size_t)min(r0 + i, rows - 1) * n;
+    const int nit = n >> 5;
+    // PACKED: W is the tile-packed copy (pack_tiles_kernel); the second matrix of MODE 2 follows the first one's tiles
+    const T* wr = PACKED ? W + (size_t)(r0 >> 4) * nit * 512 : W + (size_t)min(r0 + i, rows - 1) * n;
+    const T* wr2 = PACKED ? wr + (size_t)((rows + 15) >> 4) * nit * 512 : wr + (size_t)rows * n;
     bool jv[G];                                 // this lane's batch column exists
     const float* xr[G];
 #pragma unroll
@@ -442,15 +482,19 @@ __global__ __launch_bounds__(NS * 64) void matvec_mfma_kernel(const T* __restric
 #pragma unroll
         for (int v = 0; v < 4; v++)
             prev[q][v] = (MODE == 1 && wave == 0 && jv[q] && r0 + 4 * kk + v < rows) ? y[(size_t)(b0 + 16 * q + i) * ldy + r0 + 4 * kk + v] : 0.f;
-    const int nit = n >> 5;
     constexpr int U = G == 1 ? 4 : 2;   // slabs whose loads are in flight together
     for (int base = wave; base < nit; base += NS * U) {
         float w[U][8], w2[MODE == 2 ? U : 1][8], gv[NORM ? U : 1][8];
 #pragma unroll
         for (int t = 0; t < U; t++) {
             const int k0 = min(base + t * NS, nit - 1) << 5;   // past the end: re-read the last slab, not used
-            Slab8<T>::w(wr + k0, kk, w[t]);
-            if (MODE == 2) Slab8<T>::w(wr + (size_t)rows * n + k0, kk, w2[MODE == 2 ? t : 0]);
+            if (PACKED) {
+                PackedSlab<T>::w(wr + (size_t)(k0 >> 5) * 512, lane, w[t]);
+                if (MODE == 2) PackedSlab<T>::w(wr2 + (size_t)(k0 >> 5) * 512, lane, w2[MODE == 2 ? t : 0]);
+            } else {
+                Slab8<T>::w(wr + k0, kk, w[t]);
+                if (MODE == 2) Slab8<T>::w(wr2 + k0, kk, w2[MODE == 2 ? t : 0]);
+            }
             if (NORM) Slab8<T>::x(g + k0, kk, gv[NORM ? t : 0]);
         }
 #pragma unroll
@@ -895,6 +939,12 @@ private:
     }
     // weights
     void* emb = nullptr; void* wcls = nullptr; float* rms_final = nullptr;
+    // tile-packed copies of the matrices for the matrix-core mat-vec (batched steps, skinny prompt passes); null pointers
+    // where a matrix cannot be packed (columns not a multiple of 32) or the memory was not to be had
+    std::vector<LayerW<void>> packed;
+    void* wclsP = nullptr;
+    template <typename T> void* pack_matrix(const void* W, size_t rows, size_t n, size_t second = 0);
+    template <typename T> void pack_all();
     std::vector<LayerW<void>> layers;
     float *fcos = nullptr, *fsin = nullptr;
     // run state (sized for stateB sequences)
@@ -933,6 +983,8 @@ void Engine::release()
     for (void* p : allocs) (void)hipFree(p);
     allocs.clear();
     layers.clear();
+    packed.clear();
+    wclsP = nullptr;
     if (stream) { (void)hipStreamDestroy(stream); stream = nullptr; }
     loaded = false;
     stateB = 0;
@@ -1005,6 +1057,36 @@ template <typename T> long Engine::upload(const float* p)
     return 0;
 }
 
+// tile-packed copy of a rows x n matrix (of two stacked ones of `rows` rows each when second != 0: the second one's tiles
+// follow the first one's); nullptr when n is not a multiple of 32 or there is no memory for it
+template <typename T> void* Engine::pack_matrix(const void* W, size_t rows, size_t n, size_t second)
+{
+    if (n % 32 != 0 || rows == 0) return nullptr;
+    const size_t tiles = (rows + 15) / 16, per = tiles * 16 * n;
+    void* P = dalloc((second ? 2 : 1) * per * sizeof(T));
+    if (!P) { (void)hipGetLastError(); return nullptr; }
+    for (int m = 0; m < (second ? 2 : 1); m++) {
+        const size_t pieces = per * sizeof(T) / 16;
+        const int grid = (int)std::min<size_t>((pieces + 255) / 256, 65535);
+        hipLaunchKernelGGL(pack_tiles_kernel<T>, grid, 256, 0, stream, (const T*)W + m * second * n, (T*)P + m * per, (int)rows, (int)n);
+    }
+    return P;
+}
+
+template <typename T> void Engine::pack_all()
+{
+    const size_t dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads;
+    packed.assign(layers.size(), LayerW<void>{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr});
+    for (size_t l = 0; l < layers.size(); l++) {
+        packed[l].wqkv = pack_matrix<T>(layers[l].wqkv, dim + 2 * kvd, dim);
+        packed[l].wo = pack_matrix<T>(layers[l].wo, dim, dim);
+        packed[l].w13 = pack_matrix<T>(layers[l].w13, hid, dim, hid);
+        packed[l].w2 = pack_matrix<T>(layers[l].w2, dim, hid);
+    }
+    wclsP = pack_matrix<T>(wcls, cfg.vocab_size, dim);
+    (void)hipStreamSynchronize(stream);
+}
+
 long Engine::load(const char* path)
 {
     release();
@@ -1056,6 +1138,7 @@ long Engine::load(const char* path)
     stored_bf16 = bf16_weights;
     long e = stored_bf16 ? upload<bf16_t>(blob.data()) : upload<float>(blob.data());
     if (e) { release(); return e; }
+    if (stored_bf16) pack_all<bf16_t>(); else pack_all<float>();
     // rotary tables as precompute_freqs_cis builds them (llama2_cpu.cpp:388-414)
     const int half = (int)hs / 2;
     std::vector<float> fr(half), hc((size_t)cfg.seq_len * half), hsn((size_t)cfg.seq_len * half);
@@ -1122,7 +1205,8 @@ long Engine::ensure_state(int B, int nSteps)
 }
 
 template <int MODE, bool NORM, typename T>
-static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy);
+static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy,
+                                     const void* Wp = nullptr);
 
 long Engine::ensure_prefill(size_t rows)
 {
@@ -1179,6 +1263,7 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
     const bool skinny = M <= 256 && dim % 32 == 0 && hid % 32 == 0;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
+        const LayerW<void>& wp = packed[l];
         const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
         void* kcl = (char*)kc + cacheOfs;
         void* vcl = (char*)vc + cacheOfs;
@@ -1192,12 +1277,12 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
             return hipGetLastError();
         };
         if (skinny) {
-            HIPCHK((launch_matvec_rows<0, true, T>(s, w.wqkv, pfX, w.rms_att, pfQkv, ldq, dim, (int)M, ldq)));
+            HIPCHK((launch_matvec_rows<0, true, T>(s, w.wqkv, pfX, w.rms_att, pfQkv, ldq, dim, (int)M, ldq, wp.wqkv)));
             HIPCHK(rope_scatter());
             HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
-            HIPCHK((launch_matvec_rows<1, false, T>(s, w.wo, pfXn, nullptr, pfX, dim, dim, (int)M, dim)));          // x += Wo att
-            HIPCHK((launch_matvec_rows<2, true, T>(s, w.w13, pfX, w.rms_ffn, pfHb, hid, dim, (int)M, hid)));
-            HIPCHK((launch_matvec_rows<1, false, T>(s, w.w2, pfHb, nullptr, pfX, dim, hid, (int)M, dim)));           // x += W2 hb
+            HIPCHK((launch_matvec_rows<1, false, T>(s, w.wo, pfXn, nullptr, pfX, dim, dim, (int)M, dim, wp.wo)));          // x += Wo att
+            HIPCHK((launch_matvec_rows<2, true, T>(s, w.w13, pfX, w.rms_ffn, pfHb, hid, dim, (int)M, hid, wp.w13)));
+            HIPCHK((launch_matvec_rows<1, false, T>(s, w.w2, pfHb, nullptr, pfX, dim, hid, (int)M, dim, wp.w2)));           // x += W2 hb
             continue;
         }
         HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_att, pfXn, 1e-5f));
@@ -1227,7 +1312,7 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
     }
     for (size_t r0 = 0; r0 < M; r0 += pfLogitRows) {
         const int rows = (int)std::min(pfLogitRows, M - r0);
-        if (skinny) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V)));
+        if (skinny) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V, wclsP)));
         else HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
         hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
         HIPCHK(hipGetLastError());
@@ -1251,14 +1336,18 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
 
 template <int MODE, bool NORM, typename T>
 static hipError_t launch_matvec(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int B,
-                                int ldy, int rowsPerWave)
+                                int ldy, int rowsPerWave, const void* Wp = nullptr)
 {
     if (B >= 2 && n % 32 == 0) {
         // batched: matrix-core kernel, 16 sequences per pass over the weights
         const int ns = rows >= 8192 ? 4 : 8;   // fewer, longer wavefronts once the rows alone fill the chip
         // every group of 16 sequences walks the weights in the same launch
         const int nGroups = (B + 15) / 16, tiles8 = ((rows + 15) / 16 + 7) / 8;
-        if (ns == 4) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 4>), tiles8 * 8 * nGroups, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
+        // Wp: the tile-packed copy of W, when the engine holds one
+        if (Wp) {
+            if (ns == 4) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 4, true>), tiles8 * 8 * nGroups, 256, 0, s, (const T*)Wp, x, g, y, rows, n, B, ldy, nGroups);
+            else hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 8, true>), tiles8 * 8 * nGroups, 512, 0, s, (const T*)Wp, x, g, y, rows, n, B, ldy, nGroups);
+        } else if (ns == 4) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 4>), tiles8 * 8 * nGroups, 256, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
         else hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, 1, 8>), tiles8 * 8 * nGroups, 512, 0, s, (const T*)W, x, g, y, rows, n, B, ldy, nGroups);
         return hipGetLastError();
     }
@@ -1324,12 +1413,14 @@ static hipError_t launch_matvec_merge(hipStream_t s, const void* W, const float*
 // over the weights, so a single sequence's prompt streams every matrix once (or a few times) instead of going through
 // 128 x 128 GEMM tiles that would leave most of the chip idle at this height.
 template <int MODE, bool NORM, typename T>
-static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy)
+static hipError_t launch_matvec_rows(hipStream_t s, const void* W, const float* x, const float* g, float* y, int rows, int n, int M, int ldy,
+                                     const void* Wp)
 {
     const int tiles8 = ((rows + 15) / 16 + 7) / 8;
     // two groups of 16 rows per workgroup: half the weight traffic from L2 of one group, and still more workgroups than CUs
-#define MVG(G_) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, G_>), tiles8 * 8 * ((M + 16 * G_ - 1) / (16 * G_)), 512, 0, s, (const T*)W, x, g, y, rows, n, M, ldy, (M + 16 * G_ - 1) / (16 * G_))
-    if (M > 16) MVG(2); else MVG(1);
+#define MVG(G_, PK_, W_) hipLaunchKernelGGL((matvec_mfma_kernel<T, MODE, NORM, G_, 8, PK_>), tiles8 * 8 * ((M + 16 * G_ - 1) / (16 * G_)), 512, 0, s, (const T*)(W_), x, g, y, rows, n, M, ldy, (M + 16 * G_ - 1) / (16 * G_))
+    if (Wp) { if (M > 16) MVG(2, true, Wp); else MVG(1, true, Wp); }
+    else if (M > 16) MVG(2, false, W); else MVG(1, false, W);
 #undef MVG
     return hipGetLastError();
 }
@@ -1358,12 +1449,13 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
     if (!matvec_merge_usable(dim, hs, deferSplits)) deferSplits = 0;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
+        const LayerW<void>& wp = packed[l];
         const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
         void* kcl = (char*)kc + cacheOfs;
         void* vcl = (char*)vc + cacheOfs;
         // qkv = [Wq;Wk;Wv] rmsnorm(x)
         SPAN_BEGIN(SC_MATVEC_QKV);
-        HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq, mvRows)));
+        HIPCHK((launch_matvec<0, true, T>(s, w.wqkv, x, w.rms_att, qkv, ldq, dim, B, ldq, mvRows, wp.wqkv)));
         SPAN_END();
         // xb = attention(rope(q), cache[0..pos] with rope(k), v appended)
         SPAN_BEGIN(SC_ATTN_DECODE);
@@ -1373,20 +1465,20 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
         // x += Wo xb (with the merge of the attention's splits in front when it was left to this kernel)
         SPAN_BEGIN(SC_MATVEC_WO);
         if (deferSplits > 0) HIPCHK((launch_matvec_merge<T>(s, w.wo, (const float*)ws, deferSplits, deferRows, &dstate->len, cfg.n_heads, hs, x, dim, dim)));
-        else HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim, mvRows)));
+        else HIPCHK((launch_matvec<1, false, T>(s, w.wo, xb, nullptr, x, dim, dim, B, dim, mvRows, wp.wo)));
         SPAN_END();
         // hb = silu(W1 rmsnorm(x)) * (W3 rmsnorm(x))
         SPAN_BEGIN(SC_MATVEC_W13);
-        HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid, mvRows)));
+        HIPCHK((launch_matvec<2, true, T>(s, w.w13, x, w.rms_ffn, hb, hid, dim, B, hid, mvRows, wp.w13)));
         SPAN_END();
         // x += W2 hb
         SPAN_BEGIN(SC_MATVEC_W2);
-        HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim, mvRows)));
+        HIPCHK((launch_matvec<1, false, T>(s, w.w2, hb, nullptr, x, dim, hid, B, dim, mvRows, wp.w2)));
         SPAN_END();
     }
     // logits = Wcls rmsnorm(x)
     SPAN_BEGIN(SC_MATVEC_CLS);
-    HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V, mvRows)));
+    HIPCHK((launch_matvec<0, true, T>(s, wcls, x, rms_final, logits, V, dim, B, V, mvRows, wclsP)));
     SPAN_END();
     if (allLogits) {
         hipLaunchKernelGGL(save_logits_kernel, dim3((V + 255) / 256 > 64 ? 64 : (V + 255) / 256, B), 256, 0, s, logits, allLogits,
