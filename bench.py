@@ -123,6 +123,8 @@ def timed(cuda, fn, rgf, rgl, warm, reps):
     the 28 us causal attention launch measures 28.4 us over the first 2 ms after one and 24.9 us from 40 ms on, the 0.6 ms
     long-context one 0.76 against 0.61 ms.  Every section starts after host-side allocation and upload (such a gap), so
     the timed dispatches follow at least STEADY_MS milliseconds of the same dispatches, untimed."""
+    if STEADY_MS <= 0:
+        return cuda.TimeFunction(fn, rgf, rgl, warm, reps)
     est = cuda.TimeFunction(fn, rgf, rgl, 1, 3)
     chunk = int(min(5000, max(1, 10.0 / max(est, 1e-4))))      # about 10 ms of dispatches per library call
     t0 = time.perf_counter()
@@ -215,13 +217,14 @@ def cpu_baseline(blob, gpu_prompt, gpu_ids, budget_s=12.0):
             "ids_vs_gpu_first_generation": same}
 
 
-def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=(("bf16", True), ("f32", False))):
-    """Fused causal attention through ATTN_FWD (id 163): B=8, T=1024, 12 heads x 64 unless another shape is given."""
+def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=(("bf16", True), ("f32", False)), causal=True):
+    """Fused attention through ATTN_FWD (id 163): B=8, T=1024, 12 heads x 64 unless another shape is given; causal
+    (the (T,T) lower-triangular mask) or without a mask."""
     from mycaffe_amd.cudadnn import CUDAFN
     B, H, T, hs = shape
     rng = np.random.default_rng(0)
     out = {}
-    mask = cuda.AllocMemory(np.tril(np.ones((T, T), np.float32)))
+    mask = cuda.AllocMemory(np.tril(np.ones((T, T), np.float32))) if causal else 0
     hc, ha = cuda.CreateCuDNN(), cuda.CreateAttn()
     cuda.SetAttn(hc, ha, 0, False, B, T, H, hs, 0.0)
     for name, half in dtypes:
@@ -232,6 +235,11 @@ def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=
         ms = timed(cuda, CUDAFN.CUDA_ATTN_FWD, None, rgl, warm, reps)
         useful = 2.0 * B * H * T * T * hs          # causal half of the 4*B*H*T*T*hs full-square flops
         tf = useful / (ms / 1e3) / 1e12
+        if not causal:
+            out[name] = {"ms": round(ms, 4), "TFLOPs": round(2 * tf, 2), "frac_mfma": round(2 * tf / MFMA_PEAK_TFLOPS[name], 4)}
+            for h in hs_ + [hy]:
+                cuda.FreeMemory(h)
+            continue
         out[name] = {"ms": round(ms, 4), "TFLOPs_causal_useful": round(tf, 2), "TFLOPs_full_square": round(2 * tf, 2),
                      "roofline": {"kernel": "fused causal attention forward", "bound": "mfma", "achieved": round(tf, 2),
                                   "peak": MFMA_PEAK_TFLOPS[name], "unit": "TFLOP/s",
@@ -240,7 +248,8 @@ def bench_prefill_attention(cuda, reps, warm=5, shape=(8, 12, 1024, 64), dtypes=
                                                                "flash_%s_B%d_T%d_%dx%d" % (name, B, T, H, hs))}}
         for h in hs_ + [hy]:
             cuda.FreeMemory(h)
-    cuda.FreeMemory(mask)
+    if mask:
+        cuda.FreeMemory(mask)
     return out
 
 
@@ -599,6 +608,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-steady", action="store_true", help="time each section right away instead of after 100 ms of the same "
+                    "dispatches (for traced runs, whose output would otherwise hold thousands of warm-up dispatches)")
     ap.add_argument("--no-graph", action="store_true", help="launch every decode kernel eagerly instead of replaying a HIP graph "
                     "(kernel tracing tools see the individual kernels this way)")
     ap.add_argument("--counter-pass", nargs="?", const="all", default=None, metavar="SECTIONS",
@@ -607,6 +618,9 @@ def main():
     ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,csa_layer,matmul_chain,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
+    if args.no_steady:
+        global STEADY_MS
+        STEADY_MS = 0.0
     if args.gpus != 1:
         log("bench.py measures one GPU: every box of this build has one MI355X and the path has no multi-GPU part; "
             "run with --gpus 1")
@@ -655,6 +669,10 @@ def main():
         # the Llama-2 7B head shape at its full context: long enough that launch and tail effects no longer count
         also["prefill_attention_B4_T4096_H32x128"] = bench_prefill_attention(cuda, 10, 2, (4, 32, 4096, 128), (("bf16", True),))
         log("prefill attention, 32 x 128 heads, T = 4096:", json.dumps(also["prefill_attention_B4_T4096_H32x128"]))
+        also["prefill_attention_unmasked_bf16"] = {
+            "B%d_T%d_H%dx%d" % (sh[0], sh[2], sh[1], sh[3]): bench_prefill_attention(cuda, r, 2, sh, (("bf16", True),), causal=False)["bf16"]
+            for sh, r in (((8, 12, 1024, 64), 50), ((4, 32, 4096, 64), 10), ((4, 32, 4096, 128), 10))}
+        log("prefill attention without a mask:", json.dumps(also["prefill_attention_unmasked_bf16"]))
     if want("decode_attn"):
         also["decode_attention_H32x128"] = bench_decode_attention(cuda, 20)
         log("decode attention roofline:", json.dumps(also["decode_attention_H32x128"]["roofline"]))
