@@ -319,6 +319,9 @@ template <typename T, int HS, int BS> struct BwdTile {
     static constexpr int PAD = 16 / (int)sizeof(T);
     static constexpr int LDR = HS + PAD;         // row-major LDS stride
     static constexpr int LDT = BS + PAD;         // transposed LDS stride
+    // 16-bit storage with 128-byte rows: the transposed operands are read from the ROW-MAJOR tiles with the transposing
+    // LDS read (row stride 144 bytes suits it) instead of being scattered into transposed tiles two bytes at a time
+    static constexpr bool TRR = sizeof(T) == 2 && HS == 64;
     static constexpr int CHR = HS / EPC;         // 16-byte chunks per row
     static constexpr int TPR = NT / BS;          // threads per staged row
     static constexpr int CPT = CHR / TPR;        // chunks per thread per staged array
@@ -345,9 +348,9 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dkv_mfma_kernel(AttnBwdArgs
     extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
     T* Qs = (T*)bwd_smem;
     T* Gs = Qs + BQ * LDR;
-    T* Qt = Gs + BQ * LDR;
+    T* Qt = Gs + BQ * LDR;                       // the transposed tiles are not there with TRR
     T* Gt = Qt + HS * LDT;
-    float* Ls = (float*)(Gt + HS * LDT);
+    float* Ls = TL::TRR ? (float*)Qt : (float*)(Gt + HS * LDT);
     float* Ds = Ls + BQ;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -408,8 +411,10 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dkv_mfma_kernel(AttnBwdArgs
             const int c = cg + TPR * i;
             *(u32x4*)(&Qs[srow * LDR + c * EPC]) = qreg[i];
             *(u32x4*)(&Gs[srow * LDR + c * EPC]) = greg[i];
-            TR::scatter_chunk(&Qt[c * EPC * LDT + srow], LDT, qreg[i]);
-            TR::scatter_chunk(&Gt[c * EPC * LDT + srow], LDT, greg[i]);
+            if (!TL::TRR) {
+                TR::scatter_chunk(&Qt[c * EPC * LDT + srow], LDT, qreg[i]);
+                TR::scatter_chunk(&Gt[c * EPC * LDT + srow], LDT, greg[i]);
+            }
         }
         if (tid < BQ) { Ls[tid] = lreg; Ds[tid] = dreg; }
     };
@@ -468,9 +473,11 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dkv_mfma_kernel(AttnBwdArgs
                     const u32x4 pp = TR::pack_p(s, t), dd = TR::pack_p(dp, t);
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
-                        const u32x4 gt = TR::load_vt(&Gt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        const u32x4 gt = TL::TRR ? TR::load_vt_rowmajor(&Gs[32 * sub * LDR + dt * 32], LDR, t, lane)
+                                                 : TR::load_vt(&Gt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
                         av[dt] = TR::mma(gt, pp, av[dt]);
-                        const u32x4 qt = TR::load_vt(&Qt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        const u32x4 qt = TL::TRR ? TR::load_vt_rowmajor(&Qs[32 * sub * LDR + dt * 32], LDR, t, lane)
+                                                 : TR::load_vt(&Qt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
                         ak[dt] = TR::mma(qt, dd, ak[dt]);
                     }
                 }
@@ -507,8 +514,8 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs 
     extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
     T* Ks = (T*)bwd_smem;
     T* Vs = Ks + BKS * LDR;
-    T* Kt = Vs + BKS * LDR;
-    float* Ms = (float*)(Kt + HS * LDT);
+    T* Kt = Vs + BKS * LDR;                      // not there with TRR
+    float* Ms = TL::TRR ? (float*)Kt : (float*)(Kt + HS * LDT);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -574,7 +581,7 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs 
             const int c = cg + TPR * i;
             *(u32x4*)(&Ks[srow * LDR + c * EPC]) = kreg[i];
             *(u32x4*)(&Vs[srow * LDR + c * EPC]) = vreg[i];
-            TR::scatter_chunk(&Kt[c * EPC * LDT + srow], LDT, kreg[i]);
+            if (!TL::TRR) TR::scatter_chunk(&Kt[c * EPC * LDT + srow], LDT, kreg[i]);
         }
         if (KIND == 2 && tid < BKS) Ms[tid] = mreg;
     };
@@ -626,7 +633,8 @@ __global__ __launch_bounds__(256, OCC) void attn_bwd_dq_mfma_kernel(AttnBwdArgs 
                     const u32x4 dd = TR::pack_p(dp, t);
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
-                        const u32x4 kt = TR::load_vt(&Kt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
+                        const u32x4 kt = TL::TRR ? TR::load_vt_rowmajor(&Ks[32 * sub * LDR + dt * 32], LDR, t, lane)
+                                                 : TR::load_vt(&Kt[(dt * 32 + l32) * LDT + 32 * sub], t, half);
                         aq[dt] = TR::mma(kt, dd, aq[dt]);
                     }
                 }
@@ -651,8 +659,9 @@ template <typename T, int HS, int BS, int OCC, int KIND>
 static hipError_t bwd_launch_kind(hipStream_t s, const AttnBwdArgs& a, int mb)
 {
     typedef BwdTile<T, HS, BS> TL;
-    const size_t kvBytes = ((size_t)2 * BS * TL::LDR + (size_t)2 * HS * TL::LDT) * sizeof(T) + 2 * BS * sizeof(float);
-    const size_t qBytes = ((size_t)2 * BS * TL::LDR + (size_t)HS * TL::LDT) * sizeof(T) + BS * sizeof(float);
+    const size_t nT = TL::TRR ? 0 : 1;   // transposed tiles
+    const size_t kvBytes = ((size_t)2 * BS * TL::LDR + nT * 2 * HS * TL::LDT) * sizeof(T) + 2 * BS * sizeof(float);
+    const size_t qBytes = ((size_t)2 * BS * TL::LDR + nT * HS * TL::LDT) * sizeof(T) + BS * sizeof(float);
     auto kkv = attn_bwd_dkv_mfma_kernel<T, HS, KIND, BS, OCC>;
     auto kq = attn_bwd_dq_mfma_kernel<T, HS, KIND, BS, OCC>;
     static bool configured = false;   // per instantiation; the attribute is idempotent, so a race only repeats the call
