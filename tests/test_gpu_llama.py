@@ -68,7 +68,10 @@ def test_logits_and_ids_tiny(llm, tmp_path, cfg, shared, std):
 @pytest.mark.parametrize("name,cfg,std,nP,n", [
     ("hs16", TINY, 0.2, 5, 56),                                                                   # one split most of the way
     ("hs48", C1, 0.02, 8, 200),                                                                   # lanes past the head size idle
-    ("hs64_gqa", dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256), 0.08, 70, 180)])
+    ("hs64_gqa", dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256), 0.08, 70, 180),
+    # context length that is not a multiple of the 128 rows a split covers at head size 32: the second split's requests
+    # past the end of the cache are clamped to its last row
+    ("hs32_seq200", dict(dim=128, hidden_dim=256, n_layers=2, n_heads=4, n_kv_heads=4, vocab_size=300, seq_len=200), 0.1, 3, 196)])
 def test_batch1_split_merge_in_the_output_projection_or_in_the_attention_kernel(llm, tmp_path, name, cfg, std, nP, n):
     """At batch 1 (cache within one iteration of rows per split) the attention kernel leaves its split partials to the
     output projection, which merges them in front of its mat-vec; SET_OPTION 9 = 0 keeps the merge in the attention kernel
