@@ -2,6 +2,7 @@
 // All are HBM-bound: one pass over the data, 64-wide wavefronts, 128-bit
 // accesses where the layout allows, grid sized to a few waves per CU.
 #include "kernels.h"
+#include "lane_ops.h"
 
 namespace mch {
 
@@ -414,16 +415,9 @@ hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, con
 
 // ---------------------------------------------------------------------------
 // reductions
-__device__ inline float wave_max(float v)
-{
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-__device__ inline float wave_sum(float v)
-{
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+// (DPP and row-swap permutes: the same butterfly as `v += __shfl_xor(v, o)` for o = 32 .. 1, without the LDS crossbar)
+__device__ inline float wave_max(float v) { return group_max<64>(v); }
+__device__ inline float wave_sum(float v) { return group_sum<64>(v); }
 
 template <int NW> __device__ inline float block_max(float v, float* red)
 {

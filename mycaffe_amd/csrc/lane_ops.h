@@ -54,6 +54,24 @@ template <int LPR> __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
+template <int O> __device__ __forceinline__ float max_lane_xor(float v)
+{
+    uint32_t a, b;
+    lane_xor_pair<O>(__float_as_uint(v), a, b);
+    return fmaxf(__uint_as_float(a), __uint_as_float(b));
+}
+// maximum over each group of LPR adjacent lanes, in every lane of the group
+template <int LPR> __device__ __forceinline__ float group_max(float v)
+{
+    if constexpr (LPR >= 64) v = max_lane_xor<32>(v);
+    if constexpr (LPR >= 32) v = max_lane_xor<16>(v);
+    if constexpr (LPR >= 16) v = max_lane_xor<8>(v);
+    if constexpr (LPR >= 8) v = max_lane_xor<4>(v);
+    if constexpr (LPR >= 4) v = max_lane_xor<2>(v);
+    if constexpr (LPR >= 2) v = max_lane_xor<1>(v);
+    return v;
+}
+
 // Largest value of the wavefront with the smallest index among equals, in every lane.
 template <int O> __device__ __forceinline__ void argmax_lane_xor(float& v, int& i)
 {
