@@ -317,11 +317,13 @@ template <typename T, int HS, int BS> struct BwdTile {
     static constexpr int PF = 32 / CPF;          // fragments along a 32-row step
     static constexpr int DT = HS / 32;
     static constexpr int PAD = 16 / (int)sizeof(T);
-    static constexpr int LDR = HS + PAD;         // row-major LDS stride
+    // row-major LDS stride; rows of 256 bytes take two pads with TRR (the transposing read wants rows 32 bytes apart
+    // modulo the banks: 288 bytes, where 272 halves its rate)
+    static constexpr int LDR = (sizeof(T) == 2 && HS == 128) ? HS + 2 * PAD : HS + PAD;
     static constexpr int LDT = BS + PAD;         // transposed LDS stride
-    // 16-bit storage with 128-byte rows: the transposed operands are read from the ROW-MAJOR tiles with the transposing
+    // 16-bit storage, head sizes 64 and 128: the transposed operands are read from the ROW-MAJOR tiles with the transposing
     // LDS read (row stride 144 bytes suits it) instead of being scattered into transposed tiles two bytes at a time
-    static constexpr bool TRR = sizeof(T) == 2 && HS == 64;
+    static constexpr bool TRR = sizeof(T) == 2 && (HS == 64 || HS == 128);
     static constexpr int CHR = HS / EPC;         // 16-byte chunks per row
     static constexpr int TPR = NT / BS;          // threads per staged row
     static constexpr int CPT = CHR / TPR;        // chunks per thread per staged array
