@@ -586,6 +586,166 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// bf16, NT, one 256 x 288 tile per workgroup and one workgroup per CU: 8192 x 2304 (the fused QKV projection of a
+// 768-wide layer over 8192 tokens) is exactly 256 such tiles, one round of the chip, and a stage of K moves half the
+// bytes per flop of the 128 x 128 tile from L2 to LDS.  Eight wavefronts stacked along M, 32 x 288 each (9 MFMA
+// tiles, 144 accumulation registers), two per SIMD.
+//   * Staging goes from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wavefront lands 16 i bytes
+//     past a wavefront-uniform address, so one instruction fills eight 128-byte rows): no staging registers and no
+//     ds_write_b128, whose issue nothing covers when a SIMD holds one or two wavefronts.  Rows therefore lie 128 bytes
+//     apart without padding, and the 16-byte piece c of row r is kept at position c ^ ((r >> 1) & 7) of its row (the
+//     lane that fills position s of row r fetches piece s ^ ((r >> 1) & 7)): a 128-bit read serves sixteen lanes per
+//     cycle out of 64 banks, and sixteen consecutive rows (two per 256 bytes of bank space) then fall on sixteen
+//     different bank groups.
+//   * A k-step is one A fragment and nine B fragments for nine tile products; only RB B fragments are held: fragment
+//     f + RB - 1 of the (k-step, column) sequence is read while fragment f is multiplied.
+// No edge handling: launched only where the tiles divide the matrix (wide_tile_fits).
+template <int WN, bool HEADS>
+__global__ __launch_bounds__(512, 1) void gemm_nt_wide_bf16_kernel(int M, int N, int K, float alpha, const bf16_t* __restrict__ A,
+                                                                    const bf16_t* __restrict__ B, bf16_t* __restrict__ C, int tilesN,
+                                                                    int tilesTotal, HeadsEpilogue he)
+{
+    typedef bf16_t T;
+    typedef BigTraits<bf16_t> TR;
+    constexpr int E = 8, BK = 64, BM = 256, BN = 32 * WN, KS = 4;
+    constexpr int ROWS = BM + BN;                 // rows of one stage: A's 256, then B's 32 WN
+    constexpr int STAGE = ROWS * BK;              // elements of one stage buffer
+    constexpr int NP = (ROWS + 63) / 64;          // fetch instructions per thread and stage (a wavefront fills 8 rows with each)
+    constexpr int RB = 5;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per = (tilesTotal + 7) / 8;         // each XCD (workgroup index mod 8) takes a contiguous run of tiles
+    const int tile = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+    if (tile >= tilesTotal) return;
+    const int m0 = (tile / tilesN) * BM, n0 = (tile % tilesN) * BN;
+    const int wm = wave * 32;
+
+    floatx16 acc[WN];
+#pragma unroll
+    for (int j = 0; j < WN; j++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[j][v] = 0.f;
+
+    // fetch p of a stage: rows 64 p + 8 wave .. + 7 of the stage; this lane fills position tid & 7 of row 64 p + tid / 8.
+    // The last fetch covers the 32 rows past a multiple of 64 only: wavefronts 0 .. 3.
+    const int lr = tid >> 3;
+    const int piece = ((tid & 7) ^ ((lr >> 1) & 7)) * E;
+    const T* srcA = A + (size_t)(m0 + lr) * K + piece;
+    const T* srcB = B + (size_t)(n0 + lr) * K + piece;
+    const size_t passStride = (size_t)64 * K;
+    auto fetch = [&](int p, int k0, T* stage) {
+        if (p * 64 + wave * 8 >= ROWS) return;   // wavefront-uniform
+        const T* src = p < BM / 64 ? srcA + p * passStride + k0 : srcB + (p - BM / 64) * passStride + k0;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(stage + (p * 64 + wave * 8) * BK), 16, 0, 0);
+    };
+    const int nk = K / BK;
+#pragma unroll
+    for (int p = 0; p < NP; p++) fetch(p, 0, smem);
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the fetches have landed in LDS
+    __syncthreads();
+
+    // fragment of rows base + lane % 32, k-step ks: piece 2 ks + lane / 32, kept at position piece ^ ((row >> 1) & 7)
+    const int fr = lane & 31, half = lane >> 5;
+    int koff[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) koff[ks] = ((2 * ks + half) ^ ((fr >> 1) & 7)) * E;
+    const T* fa = smem + (wm + fr) * BK;
+    const T* fb = smem + (BM + fr) * BK;
+    u32x4 a[2], b[RB];
+    for (int kt = 0; kt < nk; kt++) {
+        const T* pa = fa + (kt & 1) * STAGE;
+        const T* pb = fb + (kt & 1) * STAGE;
+        T* next = smem + ((kt & 1) ^ 1) * STAGE;   // read during stage kt - 1; free since the barrier that ended it
+        const int k1 = min(kt + 1, nk - 1) * BK;   // past the end the last stage is fetched again (valid memory, never read)
+        a[0] = *(const u32x4*)(pa + koff[0]);
+#pragma unroll
+        for (int f = 0; f < RB - 1; f++) b[f] = *(const u32x4*)(pb + (f % WN) * 32 * BK + koff[f / WN]);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            // written in issue order, one scheduling region per tile product: the product, a fragment read, and with
+            // each of the stage's first products one fetch of the next stage
+#pragma unroll
+            for (int j = 0; j < WN; j++) {
+                acc[j] = TR::mma(b[(ks * WN + j) % RB], a[ks & 1], acc[j]);
+                const int f = ks * WN + j + RB - 1, fks = f / WN, fj = f % WN;
+                if (fks < KS) b[f % RB] = *(const u32x4*)(pb + fj * 32 * BK + koff[fks]);
+                if (j == WN / 2 && ks + 1 < KS) a[(ks + 1) & 1] = *(const u32x4*)(pa + koff[ks + 1]);
+                const int n = ks * WN + j;
+                if (n < NP) fetch(n, k1, next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+    }
+
+    // Epilogue as in gemm_nt_big_kernel: the products are the transposed 32x32 tiles, a lane owns row lane % 32 and
+    // register v is column 8 (v / 4) + 4 (lane / 32) + v % 4.  Each wavefront passes its 32 rows through its own slice of
+    // LDS (free after the last barrier) and stores 16-byte pieces, dealt to the lanes in row-major order.
+    constexpr int CW = 32 * WN, LDC = CW + E, LPR = CW / E, NIT = (32 * LPR + 63) / 64;
+    const int row_l = lane & 31, col_l = (lane >> 5) * 4;
+    T* cs = smem + wave * 32 * LDC;
+#pragma unroll
+    for (int j = 0; j < WN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+            if (HEADS && he.bias) {
+                const T* bp = (const T*)he.bias + n0 + j * 32 + 8 * g + col_l;
+                b0 = TR::ld(bp); b1 = TR::ld(bp + 1); b2 = TR::ld(bp + 2); b3 = TR::ld(bp + 3);
+            }
+            TR::st4(cs + row_l * LDC + j * 32 + 8 * g + col_l, alpha * acc[j][4 * g] + b0, alpha * acc[j][4 * g + 1] + b1,
+                    alpha * acc[j][4 * g + 2] + b2, alpha * acc[j][4 * g + 3] + b3);
+        }
+    // same wavefront wrote and reads: LDS operations of one wavefront complete in order
+#pragma unroll 6
+    for (int it = 0; it < NIT; it++) {
+        const int id = it * 64 + lane, r = id / LPR, cc = (id - r * LPR) * E;
+        const u32x4 v = *(const u32x4*)(cs + r * LDC + cc);
+        if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + r, n0 + cc) = v;
+        else *(u32x4*)(C + (size_t)(m0 + wm + r) * N + n0 + cc) = v;
+    }
+}
+
+// The wide tiles have no edge handling and one workgroup per CU: they are used where they divide the matrix, fill whole
+// rounds of the 256 CUs to at least 85 % and K is long enough to pay for the larger prologue and epilogue.  Returns the
+// tile width in MFMA tiles (9: 256 x 288, 6: 256 x 192) or 0.
+static int wide_tile_fits(int m, int n, int k, const void* A, const void* B, const void* C)
+{
+    if (m % 256 != 0 || k % 64 != 0 || k < 512) return 0;
+    if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) return 0;
+    for (int wn : {9, 6}) {
+        if (n % (32 * wn) != 0) continue;
+        const long long tiles = (long long)(m / 256) * (n / (32 * wn)), rounds = (tiles + 255) / 256;
+        if (tiles <= (1ll << 30) && tiles * 100 >= rounds * 256 * 85) return wn;
+    }
+    return 0;
+}
+
+template <int WN, bool HEADS>
+static hipError_t launch_wide(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, void* C,
+                              const HeadsEpilogue* heads = nullptr)
+{
+    HeadsEpilogue he = {};
+    if (heads) he = *heads;
+    constexpr int BN = 32 * WN;
+    const int tm = m / 256, tn = n / BN, total = tm * tn, per = (total + 7) / 8;
+    // two stages of (256 + BN) rows x 128 bytes, or the epilogue's eight slices of 32 x (BN + 8) elements, whichever is larger
+    const size_t lds = std::max((size_t)2 * (256 + BN) * 64, (size_t)8 * 32 * (BN + 8)) * sizeof(bf16_t);
+    static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_wide_bf16_kernel<WN, HEADS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    hipLaunchKernelGGL((gemm_nt_wide_bf16_kernel<WN, HEADS>), dim3(per * 8), 512, lds, s, m, n, k, alpha, (const bf16_t*)A, (const bf16_t*)B,
+                       (bf16_t*)C, tn, total, he);
+    return hipGetLastError();
+}
+
 // K = 1: the rank-1 update C[i,j] = alpha a[i] b[j] + beta C[i,j] that InnerProductLayer uses to add its bias
 // (ones (M,1) x bias (1,N), InnerProductLayer.cs:405-414): one streaming pass over C, four columns per thread
 template <typename T> struct Quad;
@@ -655,6 +815,10 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
         return launch_big<float, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
     if (aligned && dt == BF16 && kk % 64 == 0) {
+        switch (wide_tile_fits(m, n, kk, X, W, nullptr)) {
+        case 9: return launch_wide<9, true>(s, m, n, kk, 1.f, X, W, nullptr, &he);
+        case 6: return launch_wide<6, true>(s, m, n, kk, 1.f, X, W, nullptr, &he);
+        }
         if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         return launch_big<bf16_t, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
@@ -710,6 +874,10 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
         } else {
             if (k % 64 == 0) {
                 if (k >= 2048 && fill >= 0.85) return launch_big<bf16_t, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
+                switch (beta == 0.f ? wide_tile_fits(m, n, k, A, B, C) : 0) {
+                case 9: return launch_wide<9, false>(s, m, n, k, alpha, A, B, C);
+                case 6: return launch_wide<6, false>(s, m, n, k, alpha, A, B, C);
+                }
                 if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
                 return launch_big<bf16_t, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }

@@ -357,7 +357,7 @@ def test_encdec_attention_config_bf16(dev):
 # ---- causal self attention layer, B = 8, T = 1024, C = 768 ------------------------------------
 
 @pytest.mark.parametrize("half", [False, True])
-@pytest.mark.parametrize("N", [2304, 768])
+@pytest.mark.parametrize("N", [2304, 768, 1536])
 def test_inner_product_gemm_at_layer_shapes(dev, half, N):
     # InnerProductLayer.forward: gemm(false, true, M, N, K, 1, X, W, 0, Y), W stored [N, K]
     M, K = 8192, 768
@@ -371,6 +371,24 @@ def test_inner_product_gemm_at_layer_shapes(dev, half, N):
     # every tile of the walk was written: no row or column band left at zero
     y = dev.get(hy, (M, N))
     assert np.count_nonzero(np.abs(y).max(axis=1) == 0) == 0 and np.count_nonzero(np.abs(y).max(axis=0) == 0) == 0
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("H,hs", [(12, 64), (8, 64)])
+def test_qkv_proj_heads_at_layer_shapes(dev, half, H, hs):
+    # the fused QKV projection over 8 x 1024 tokens: in 16-bit storage 8192 x 2304 x 768 is 256 tiles of 256 x 288 and
+    # 8192 x 1536 x 512 is 256 tiles of 256 x 192 (one workgroup per CU each); every element of q, k, v against the checker
+    B, T, C = 8, 1024, H * hs
+    rng = np.random.default_rng(C)
+    x = bf16_round(rng.standard_normal((B, T, C), dtype=np.float32))
+    w = bf16_round(rng.standard_normal((3 * C, C), dtype=np.float32) * 0.02)
+    bv = bf16_round(rng.standard_normal(3 * C, dtype=np.float32) * 0.1)
+    hx, hw, hb = dev.put(x, half), dev.put(w, half), dev.put(bv, half)
+    hq, hk, hv = (dev.zeros(B * T * C, half) for _ in range(3))
+    dev.cuda.QkvProjHeads(B, T, H, hs, hx, hw, hb, hq, hk, hv)
+    ref = R.inner_product(x, w, bv, np.float64).reshape(B, T, 3, H, hs).transpose(2, 0, 3, 1, 4)
+    for i, (name, h) in enumerate(zip("qkv", (hq, hk, hv))):
+        assert_close(dev.get(h, (B, H, T, hs)), ref[i], BF16_RTOL if half else FP32_RTOL, name)
 
 
 @pytest.mark.parametrize("half", [False, True])
