@@ -601,14 +601,13 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
 //   * A k-step is one A fragment and nine B fragments for nine tile products; only RB B fragments are held: fragment
 //     f + RB - 1 of the (k-step, column) sequence is read while fragment f is multiplied.
 // No edge handling: launched only where the tiles divide the matrix (wide_tile_fits).
-template <int WN, bool HEADS>
-__global__ __launch_bounds__(512, 1) void gemm_nt_wide_bf16_kernel(int M, int N, int K, float alpha, const bf16_t* __restrict__ A,
-                                                                    const bf16_t* __restrict__ B, bf16_t* __restrict__ C, int tilesN,
-                                                                    int tilesTotal, HeadsEpilogue he)
+template <typename T, int WN, bool HEADS>
+__global__ __launch_bounds__(512, 1) void gemm_nt_wide_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
+                                                               const T* __restrict__ B, T* __restrict__ C, int tilesN,
+                                                               int tilesTotal, HeadsEpilogue he)
 {
-    typedef bf16_t T;
-    typedef BigTraits<bf16_t> TR;
-    constexpr int E = 8, BK = 64, BM = 256, BN = 32 * WN, KS = 4;
+    typedef BigTraits<T> TR;
+    constexpr int E = TR::E, BK = 8 * E, BM = 256, BN = 32 * WN, KS = 4;   // a stage is 128 bytes of every row
     constexpr int ROWS = BM + BN;                 // rows of one stage: A's 256, then B's 32 WN
     constexpr int STAGE = ROWS * BK;              // elements of one stage buffer
     constexpr int NP = (ROWS + 63) / 64;          // fetch instructions per thread and stage (a wavefront fills 8 rows with each)
@@ -683,39 +682,48 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_wide_bf16_kernel(int M, int N,
     }
 
     // Epilogue as in gemm_nt_big_kernel: the products are the transposed 32x32 tiles, a lane owns row lane % 32 and
-    // register v is column 8 (v / 4) + 4 (lane / 32) + v % 4.  Each wavefront passes its 32 rows through its own slice of
-    // LDS (free after the last barrier) and stores 16-byte pieces, dealt to the lanes in row-major order.
-    constexpr int CW = 32 * WN, LDC = CW + E, LPR = CW / E, NIT = (32 * LPR + 63) / 64;
+    // register v is column 8 (v / 4) + 4 (lane / 32) + v % 4.  Each wavefront passes its 32 rows, CH tiles of columns at a
+    // time (all of them in 16-bit storage, three in fp32: eight slices have to fit the LDS), through its own slice of LDS
+    // (free after the last barrier) and stores 16-byte pieces, dealt to the lanes in row-major order.
+    constexpr int CH = sizeof(T) == 2 ? WN : 3;
+    static_assert(WN % CH == 0, "whole column chunks");
+    constexpr int CW = 32 * CH, LDC = CW + E, LPR = CW / E, NIT = (32 * LPR) / 64;
+    static_assert((32 * LPR) % 64 == 0, "the pieces of a 32-row block fill whole store instructions");
     const int row_l = lane & 31, col_l = (lane >> 5) * 4;
     T* cs = smem + wave * 32 * LDC;
 #pragma unroll
-    for (int j = 0; j < WN; j++)
+    for (int c = 0; c < WN / CH; c++) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
-            if (HEADS && he.bias) {
-                const T* bp = (const T*)he.bias + n0 + j * 32 + 8 * g + col_l;
-                b0 = TR::ld(bp); b1 = TR::ld(bp + 1); b2 = TR::ld(bp + 2); b3 = TR::ld(bp + 3);
+        for (int jj = 0; jj < CH; jj++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int j = c * CH + jj;
+                float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+                if (HEADS && he.bias) {
+                    const T* bp = (const T*)he.bias + n0 + j * 32 + 8 * g + col_l;
+                    b0 = TR::ld(bp); b1 = TR::ld(bp + 1); b2 = TR::ld(bp + 2); b3 = TR::ld(bp + 3);
+                }
+                TR::st4(cs + row_l * LDC + jj * 32 + 8 * g + col_l, alpha * acc[j][4 * g] + b0, alpha * acc[j][4 * g + 1] + b1,
+                        alpha * acc[j][4 * g + 2] + b2, alpha * acc[j][4 * g + 3] + b3);
             }
-            TR::st4(cs + row_l * LDC + j * 32 + 8 * g + col_l, alpha * acc[j][4 * g] + b0, alpha * acc[j][4 * g + 1] + b1,
-                    alpha * acc[j][4 * g + 2] + b2, alpha * acc[j][4 * g + 3] + b3);
-        }
-    // same wavefront wrote and reads: LDS operations of one wavefront complete in order
+        // same wavefront wrote and reads, and writes the next chunk after it has read this one: LDS operations of one
+        // wavefront complete in order
 #pragma unroll 6
-    for (int it = 0; it < NIT; it++) {
-        const int id = it * 64 + lane, r = id / LPR, cc = (id - r * LPR) * E;
-        const u32x4 v = *(const u32x4*)(cs + r * LDC + cc);
-        if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + r, n0 + cc) = v;
-        else *(u32x4*)(C + (size_t)(m0 + wm + r) * N + n0 + cc) = v;
+        for (int it = 0; it < NIT; it++) {
+            const int id = it * 64 + lane, r = id / LPR, cc = (id - r * LPR) * E;
+            const u32x4 v = *(const u32x4*)(cs + r * LDC + cc);
+            if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + r, n0 + c * CW + cc) = v;
+            else *(u32x4*)(C + (size_t)(m0 + wm + r) * N + n0 + c * CW + cc) = v;
+        }
     }
 }
 
 // The wide tiles have no edge handling and one workgroup per CU: they are used where they divide the matrix, fill whole
 // rounds of the 256 CUs to at least 85 % and K is long enough to pay for the larger prologue and epilogue.  Returns the
 // tile width in MFMA tiles (9: 256 x 288, 6: 256 x 192) or 0.
-static int wide_tile_fits(int m, int n, int k, const void* A, const void* B, const void* C)
+static int wide_tile_fits(int m, int n, int k, int stageElems, const void* A, const void* B, const void* C)
 {
-    if (m % 256 != 0 || k % 64 != 0 || k < 512) return 0;
+    if (m % 256 != 0 || k % stageElems != 0 || k < 8 * stageElems) return 0;
     if ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) != 0) return 0;
     for (int wn : {9, 6}) {
         if (n % (32 * wn) != 0) continue;
@@ -725,25 +733,46 @@ static int wide_tile_fits(int m, int n, int k, const void* A, const void* B, con
     return 0;
 }
 
-template <int WN, bool HEADS>
+template <typename T, int WN, bool HEADS>
 static hipError_t launch_wide(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, void* C,
                               const HeadsEpilogue* heads = nullptr)
 {
     HeadsEpilogue he = {};
     if (heads) he = *heads;
-    constexpr int BN = 32 * WN;
+    constexpr int BN = 32 * WN, E = BigTraits<T>::E, CH = sizeof(T) == 2 ? WN : 3;
     const int tm = m / 256, tn = n / BN, total = tm * tn, per = (total + 7) / 8;
-    // two stages of (256 + BN) rows x 128 bytes, or the epilogue's eight slices of 32 x (BN + 8) elements, whichever is larger
-    const size_t lds = std::max((size_t)2 * (256 + BN) * 64, (size_t)8 * 32 * (BN + 8)) * sizeof(bf16_t);
+    // two stages of (256 + BN) rows x 128 bytes, or the epilogue's eight slices of 32 x (32 CH + E) elements, whichever is larger
+    const size_t lds = std::max((size_t)2 * (256 + BN) * 128, (size_t)8 * 32 * (32 * CH + E) * sizeof(T));
     static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
     if (!attr) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_wide_bf16_kernel<WN, HEADS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_wide_kernel<T, WN, HEADS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr = true;
     }
-    hipLaunchKernelGGL((gemm_nt_wide_bf16_kernel<WN, HEADS>), dim3(per * 8), 512, lds, s, m, n, k, alpha, (const bf16_t*)A, (const bf16_t*)B,
-                       (bf16_t*)C, tn, total, he);
+    hipLaunchKernelGGL((gemm_nt_wide_kernel<T, WN, HEADS>), dim3(per * 8), 512, lds, s, m, n, k, alpha, (const T*)A, (const T*)B,
+                       (T*)C, tn, total, he);
     return hipGetLastError();
+}
+
+// fp32 keeps the matrix cores busy with 128 x 128 tiles as well (512 of them fill the chip at two workgroups per CU) and
+// measures 3 % faster with them when their rounds are full or half full; the wide tile wins (8192 x 2304 x 768: 232 ->
+// 214 us) where the last round of 128 x 128 tiles would be mostly empty.
+static bool short_last_round(long long t128)
+{
+    const long long rem = t128 % 512;
+    return rem != 0 && rem * 10 < 512 * 4;
+}
+
+// one stage of K is 128 bytes of a row: 64 elements in 16-bit storage, 32 in fp32
+template <typename T, bool HEADS>
+static bool launch_wide_if_fits(hipError_t* e, hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, void* C,
+                                const HeadsEpilogue* heads = nullptr)
+{
+    switch (wide_tile_fits(m, n, k, 8 * BigTraits<T>::E, A, B, C)) {
+    case 9: *e = launch_wide<T, 9, HEADS>(s, m, n, k, alpha, A, B, C, heads); return true;
+    case 6: *e = launch_wide<T, 6, HEADS>(s, m, n, k, alpha, A, B, C, heads); return true;
+    }
+    return false;
 }
 
 // K = 1: the rank-1 update C[i,j] = alpha a[i] b[j] + beta C[i,j] that InnerProductLayer uses to add its bias
@@ -812,13 +841,13 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
     if (aligned && dt == F32 && kk % 32 == 0) {
         if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
+        hipError_t e;
+        if (short_last_round(t128) && launch_wide_if_fits<float, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
         return launch_big<float, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
     if (aligned && dt == BF16 && kk % 64 == 0) {
-        switch (wide_tile_fits(m, n, kk, X, W, nullptr)) {
-        case 9: return launch_wide<9, true>(s, m, n, kk, 1.f, X, W, nullptr, &he);
-        case 6: return launch_wide<6, true>(s, m, n, kk, 1.f, X, W, nullptr, &he);
-        }
+        hipError_t e;
+        if (launch_wide_if_fits<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
         if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         return launch_big<bf16_t, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
@@ -867,6 +896,8 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
             if (k % 32 == 0) {
                 if (k >= 1024 && fill >= 0.85) return launch_big<float, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
                 if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
+                hipError_t e;
+                if (beta == 0.f && short_last_round(t128) && launch_wide_if_fits<float, false>(&e, s, m, n, k, alpha, A, B, C)) return e;
                 return launch_big<float, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }
             hipLaunchKernelGGL(gemm_nt_f32_mfma_kernel, grid, 256, 0, s, m, n, k, alpha, (const float*)A, (const float*)B,
@@ -874,10 +905,8 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
         } else {
             if (k % 64 == 0) {
                 if (k >= 2048 && fill >= 0.85) return launch_big<bf16_t, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
-                switch (beta == 0.f ? wide_tile_fits(m, n, k, A, B, C) : 0) {
-                case 9: return launch_wide<9, false>(s, m, n, k, alpha, A, B, C);
-                case 6: return launch_wide<6, false>(s, m, n, k, alpha, A, B, C);
-                }
+                hipError_t e;
+                if (beta == 0.f && launch_wide_if_fits<bf16_t, false>(&e, s, m, n, k, alpha, A, B, C)) return e;
                 if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
                 return launch_big<bf16_t, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }
