@@ -1304,15 +1304,18 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         if (e) return e;
         HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, hid, 1.f, pfHb, w2, 1.f, pfX));          // x += W2 hb
     }
+    // The classifier has 250 tiles of 128 x 128 per 128 rows, enough for the tiled GEMM even where the layers' matrices
+    // are not: the mat-vec family keeps it only for a handful of rows.
+    const bool clsGemm = !skinny || M >= 64;
     const float* wc = nullptr;
-    if (!skinny) {
+    if (clsGemm) {
         HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
         wc = as_f32<T>(s, wcls, (size_t)V * dim, &e);
         if (e) return e;
     }
     for (size_t r0 = 0; r0 < M; r0 += pfLogitRows) {
         const int rows = (int)std::min(pfLogitRows, M - r0);
-        if (skinny) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V, wclsP)));
+        if (!clsGemm) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V, wclsP)));
         else HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
         hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
         HIPCHK(hipGetLastError());
