@@ -587,10 +587,10 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
 }
 
 // ---------------------------------------------------------------------------
-// bf16, NT, one 256 x 288 tile per workgroup and one workgroup per CU: 8192 x 2304 (the fused QKV projection of a
-// 768-wide layer over 8192 tokens) is exactly 256 such tiles, one round of the chip, and a stage of K moves half the
-// bytes per flop of the 128 x 128 tile from L2 to LDS.  Eight wavefronts stacked along M, 32 x 288 each (9 MFMA
-// tiles, 144 accumulation registers), two per SIMD.
+// NT, one 256 x 288 (WN = 9) or 256 x 192 (WN = 6) tile per workgroup and one workgroup per CU: 8192 x 2304 (the fused
+// QKV projection of a 768-wide layer over 8192 tokens) is exactly 256 tiles of 256 x 288, one round of the chip, and a
+// stage of K moves half the bytes per flop of the 128 x 128 tile from L2 to LDS.  Eight wavefronts stacked along M,
+// 32 rows x 32 WN columns each (WN MFMA tiles, 144 accumulation registers at WN = 9), two per SIMD.
 //   * Staging goes from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wavefront lands 16 i bytes
 //     past a wavefront-uniform address, so one instruction fills eight 128-byte rows): no staging registers and no
 //     ds_write_b128, whose issue nothing covers when a SIMD holds one or two wavefronts.  Rows therefore lie 128 bytes
@@ -598,7 +598,7 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
 //     lane that fills position s of row r fetches piece s ^ ((r >> 1) & 7)): a 128-bit read serves sixteen lanes per
 //     cycle out of 64 banks, and sixteen consecutive rows (two per 256 bytes of bank space) then fall on sixteen
 //     different bank groups.
-//   * A k-step is one A fragment and nine B fragments for nine tile products; only RB B fragments are held: fragment
+//   * A k-step is one A fragment and WN B fragments for WN tile products; only RB B fragments are held: fragment
 //     f + RB - 1 of the (k-step, column) sequence is read while fragment f is multiplied.
 // No edge handling: launched only where the tiles divide the matrix (wide_tile_fits).
 template <typename T, int WN, bool HEADS>
