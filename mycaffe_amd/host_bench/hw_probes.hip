@@ -1,14 +1,18 @@
 // Micro-benchmarks of the gfx950 properties that the kernel designs of this library rest on.  Each prints one line per
 // case; none of them touches the library.  Build: mycaffe_amd/build.py; run: mycaffe_amd/host_bench/hw_probes [section]
-// with section in {overlap, lds, graph, persist} (default: all).
+// with section in {overlap, lds, graph, persist, stage} (default: all).
 //   overlap  how much vector-ALU work a wavefront can hide behind its own MFMAs (plain fma and v_exp_f32)
 //   lds      rate of the LDS fragment reads of the attention and GEMM kernels (ds_read_b128 in the K-fragment pattern,
 //            the transposing ds_read_b64_tr_b16 in the row-major V pattern) alone and with one MFMA per fragment
 //   graph    cost of a kernel boundary inside a replayed HIP graph and of a bare mat-vec kernel at several working sets
 //   persist  the same mat-vec chain as one cooperative kernel with bounded grid barriers, with and without the next
 //            phase's weights requested across the barrier
+//   stage    what the GEMM kernels' operand staging can draw from the caches: where the lanes of a direct global-to-LDS
+//            load (global_load_lds_dwordx4) land, and the rate at which all CUs together stream 16-byte loads out of
+//            their die's L2 and out of the last-level cache, into registers and straight into LDS
 #include <hip/hip_runtime.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -407,6 +411,112 @@ static int run_persist()
     return 0;
 }
 
+
+// ---- stage: direct global-to-LDS loads ---------------------------------------------------------------------------------
+// placement: every thread loads 16 bytes of a counting pattern with four direct-to-LDS instructions; the workgroup then
+// reads LDS back linearly.  If lane i of a wavefront lands 16 i bytes past the wavefront's (uniform) destination, LDS
+// holds the pattern in order.
+__global__ __launch_bounds__(256) void dma_place_kernel(const unsigned* __restrict__ g, unsigned* out)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char dsm[];
+    const int wave = threadIdx.x >> 6;
+    const unsigned* src = g + (size_t)threadIdx.x * 4;
+#pragma unroll
+    for (int p = 0; p < 4; p++)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + p * 1024),
+                                         (__attribute__((address_space(3))) void*)(dsm + p * 4096 + wave * 1024), 16, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+    __syncthreads();
+    for (int i = threadIdx.x; i < 4096; i += 256) out[i] = ((const unsigned*)dsm)[i];
+}
+
+// rate: every workgroup streams from a region that belongs to its die (workgroup index mod 8); a region that fits the
+// die's 4 MB L2 is served from it, a larger one from the last-level cache.  UNR 16-byte loads per thread in flight.
+template <int UNR, bool DIRECT>
+__global__ __launch_bounds__(256) void stage_rate_kernel(const unsigned* __restrict__ g, unsigned* out, size_t regionWords, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char dsm[];
+    const int die = blockIdx.x % 8, idx = blockIdx.x / 8;
+    const unsigned* base = g + (size_t)die * regionWords;
+    const size_t chunkWords = 256 * 4 * UNR, nChunks = regionWords / chunkWords;
+    u32x4 acc = {0, 0, 0, 0};
+    for (int it = 0; it < iters; it++) {
+        const unsigned* p = base + (((size_t)idx * 7 + it) % nChunks) * chunkWords + threadIdx.x * 4;
+        if (DIRECT) {
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p + u * 1024),
+                                                 (__attribute__((address_space(3))) void*)(dsm + (u * 4 + (threadIdx.x >> 6)) * 1024), 16, 0, 0);
+        } else {
+            u32x4 v[UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; u++) v[u] = *(const u32x4*)(p + u * 1024);
+#pragma unroll
+            for (int u = 0; u < UNR; u++) acc ^= v[u];
+        }
+    }
+    if (DIRECT) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        acc = *(const u32x4*)(dsm + threadIdx.x * 16);
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) out[0] = 1;   // keeps the loads alive
+}
+
+template <bool DIRECT> static int run_stage_rate(const unsigned* g, unsigned* out, size_t regionWords, int wgs)
+{
+    constexpr int UNR = 8;
+    const int iters = 400, reps = 10;
+    const size_t lds = DIRECT ? UNR * 4096 : 0;
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    for (int w = 0; w < 3; w++) hipLaunchKernelGGL((stage_rate_kernel<UNR, DIRECT>), wgs, 256, lds, 0, g, out, regionWords, iters);
+    CK(hipEventRecord(e0));
+    for (int r = 0; r < reps; r++) hipLaunchKernelGGL((stage_rate_kernel<UNR, DIRECT>), wgs, 256, lds, 0, g, out, regionWords, iters);
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    float ms = 0;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    const double bytes = (double)wgs * iters * 256 * 16 * UNR * reps;
+    printf("stage    %-22s %4d workgroups, %5.1f MB per die: %6.2f TB/s (%5.1f GB/s per CU)\n", DIRECT ? "straight into LDS," : "into registers,", wgs,
+           regionWords * 4 / 1e6, bytes / ms / 1e9, bytes / ms / 1e6 / 256);
+    CK(hipEventDestroy(e0));
+    CK(hipEventDestroy(e1));
+    return 0;
+}
+
+static int run_stage()
+{
+    const size_t maxRegionWords = (size_t)16 << 20;   // 64 MB per die
+    unsigned *g, *out;
+    CK(hipMalloc(&g, maxRegionWords * 4 * 8));
+    CK(hipMalloc(&out, 4096 * 4));
+    {
+        unsigned* h = (unsigned*)malloc(8192 * 4);
+        for (int i = 0; i < 8192; i++) h[i] = (unsigned)i;
+        CK(hipMemcpy(g, h, 8192 * 4, hipMemcpyHostToDevice));
+        hipLaunchKernelGGL(dma_place_kernel, 1, 256, 16384, 0, g, out);
+        CK(hipMemcpy(h, out, 4096 * 4, hipMemcpyDeviceToHost));
+        int bad = 0;
+        for (int i = 0; i < 4096; i++) bad += h[i] != (unsigned)i;
+        printf("stage    global_load_lds_dwordx4: lane i of a wavefront lands 16 i bytes past the wavefront's LDS address: %s (%d of 4096 words differ)\n",
+               bad ? "NO" : "yes", bad);
+        free(h);
+    }
+    CK(hipMemset(g, 1, maxRegionWords * 4 * 8));
+    for (size_t mb : {2, 16}) {
+        const size_t rw = mb * 1024 * 1024 / 4;
+        for (int wgs : {256, 512}) {
+            if (run_stage_rate<false>(g, out, rw, wgs)) return 1;
+            if (run_stage_rate<true>(g, out, rw, wgs)) return 1;
+        }
+    }
+    CK(hipFree(g));
+    CK(hipFree(out));
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     const char* sec = argc > 1 ? argv[1] : "all";
@@ -442,6 +552,9 @@ int main(int argc, char** argv)
     }
     if (all || !strcmp(sec, "persist")) {
         if (run_persist()) return 1;
+    }
+    if (all || !strcmp(sec, "stage")) {
+        if (run_stage()) return 1;
     }
     CK(hipFree(d));
     return 0;
