@@ -371,7 +371,11 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     constexpr int PA = BM / RPP, PB = BN / RPP;               // passes (16-byte chunks per thread) per operand
     constexpr int KS = 4;                                     // k-steps (fragments of 2 E elements) per stage
     constexpr int NMF = WM * WN;                              // tile products per k-step
-    static_assert(NMF >= WM + WN && NMF * (KS / 2) >= PA + PB, "not enough tile products per k-step to carry the memory instructions");
+    // Memory instructions ride along with the tile products (below): RF fragment reads and SC staging instructions per
+    // product.  One of each where a k-step has at least as many products as fragments (every tile of 128 x 128 and up);
+    // two with the 64-row tiles, whose wavefronts own one or two MFMA tiles.
+    constexpr int RF = (WM + WN + NMF - 1) / NMF;
+    constexpr int SC = ((PA + PB + KS / 2 - 1) / (KS / 2) + NMF - 1) / NMF;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     T* As = smem;                        // [2][BM * LDK]
@@ -466,11 +470,15 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                 const int i = q / WN, j = q % WN;
                 acc[i][j] = TR::mma(b[cur][j], a[cur][i], acc[i][j]);
                 if (ks + 1 < KS) {
-                    if (q < WM) a[nxt][q] = *(const u32x4*)(pa + q * 32 * LDK + (ks + 1) * 2 * E);
-                    else if (q < WM + WN) b[nxt][q - WM] = *(const u32x4*)(pb + (q - WM) * 32 * LDK + (ks + 1) * 2 * E);
+#pragma unroll
+                    for (int r = q * RF; r < (q + 1) * RF; r++) {
+                        if (r < WM) a[nxt][r] = *(const u32x4*)(pa + r * 32 * LDK + (ks + 1) * 2 * E);
+                        else if (r < WM + WN) b[nxt][r - WM] = *(const u32x4*)(pb + (r - WM) * 32 * LDK + (ks + 1) * 2 * E);
+                    }
                 }
-                const int c = c0 + q;
-                if (c < c1) {
+#pragma unroll
+                for (int c = c0 + q * SC; c < c0 + (q + 1) * SC; c++) {
+                    if (c >= c1) break;
                     if (ks < HALF) {
                         if (c < PA) *(u32x4*)(wa + c * RPP * LDK) = ra[c];
                         else *(u32x4*)(wb + (c - PA) * RPP * LDK) = rb[c - PA];
@@ -754,6 +762,20 @@ static hipError_t launch_wide(hipStream_t s, int m, int n, int k, float alpha, c
     return hipGetLastError();
 }
 
+// Fewer 128 x 128 tiles than CUs: 64 x 128 tiles if they give every CU one, 64 x 64 otherwise (three or four of these
+// small workgroups fit a CU, so more tiles than CUs is welcome).
+template <typename T, bool HEADS>
+static bool launch_small_if_few(hipError_t* e, hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C,
+                                const HeadsEpilogue* heads = nullptr)
+{
+    const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+    if (t128 >= 200) return false;
+    const long long t64x128 = (long long)((m + 63) / 64) * ((n + 127) / 128);
+    if (t64x128 >= 200) *e = launch_big<T, 1, 2, 3, HEADS>(s, m, n, k, alpha, A, B, beta, C, heads);
+    else *e = launch_big<T, 1, 1, 3, HEADS>(s, m, n, k, alpha, A, B, beta, C, heads);
+    return true;
+}
+
 // fp32 keeps the matrix cores busy with 128 x 128 tiles as well (512 of them fill the chip at two workgroups per CU) and
 // measures 3 % faster with them when their rounds are full or half full; the wide tile wins (8192 x 2304 x 768: 232 ->
 // 214 us) where the last round of 128 x 128 tiles would be mostly empty.
@@ -840,14 +862,16 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
     const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 == 0) && hs % vec == 0;
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
     if (aligned && dt == F32 && kk % 32 == 0) {
-        if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         hipError_t e;
+        if (launch_small_if_few<float, true>(&e, s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he)) return e;
+        if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (short_last_round(t128) && launch_wide_if_fits<float, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
         return launch_big<float, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
     if (aligned && dt == BF16 && kk % 64 == 0) {
         hipError_t e;
         if (launch_wide_if_fits<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
+        if (launch_small_if_few<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he)) return e;
         if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         return launch_big<bf16_t, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
@@ -895,8 +919,9 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
         if (dt == F32) {
             if (k % 32 == 0) {
                 if (k >= 1024 && fill >= 0.85) return launch_big<float, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
-                if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
                 hipError_t e;
+                if (launch_small_if_few<float, false>(&e, s, m, n, k, alpha, A, B, beta, C)) return e;
+                if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
                 if (beta == 0.f && short_last_round(t128) && launch_wide_if_fits<float, false>(&e, s, m, n, k, alpha, A, B, C)) return e;
                 return launch_big<float, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }
@@ -907,6 +932,7 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
                 if (k >= 2048 && fill >= 0.85) return launch_big<bf16_t, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);
                 hipError_t e;
                 if (beta == 0.f && launch_wide_if_fits<bf16_t, false>(&e, s, m, n, k, alpha, A, B, C)) return e;
+                if (launch_small_if_few<bf16_t, false>(&e, s, m, n, k, alpha, A, B, beta, C)) return e;
                 if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2>(s, m, n, k, alpha, A, B, beta, C);
                 return launch_big<bf16_t, 2, 2, 2>(s, m, n, k, alpha, A, B, beta, C);
             }
