@@ -768,6 +768,116 @@ __global__ __launch_bounds__(NW * 64, OCC) void flash_pipe_bf16_kernel(FlashArgs
     }
 }
 
+// ---------------------------------------------------------------------------
+// Short causal sequences in fp32, head size 64 (the one-sequence prompt pass of the decode engine: 128 positions, 12
+// heads).  flash_fwd_kernel gives such a launch one workgroup per head, and the wavefront that owns the last 32 rows runs
+// its four 32-key steps - 256 fp32 MFMAs of 64 cycles - one after the other.  Here a workgroup owns 32 query rows and
+// its four wavefronts take the 32-key steps in turn (step w, w + 4, ...), each with its own running maximum, sum and
+// output tile; the partial results meet in LDS and are combined as the splits of a decode step are.  K and V go from
+// global memory straight into the fragments (a step's tiles are read by one wavefront only, so LDS would add a
+// round trip and nothing else).
+__global__ __launch_bounds__(256) void flash_short_causal_f32_kernel(FlashArgs a)
+{
+    typedef FlashTraits<float> TR;
+    constexpr int HS = 64, CPF = TR::CPF, KF = HS / CPF, PF = 32 / CPF, DT = HS / 32, LDO = HS + 4;
+    __shared__ __attribute__((aligned(16))) float Os[4][32 * LDO];
+    __shared__ float Ms[4][32], Ls[4][32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int qtile = (int)gridDim.x - 1 - (int)blockIdx.x;   // heaviest first
+    const int h = blockIdx.y, b = blockIdx.z;
+    const size_t bh = (size_t)b * a.H + h;
+    const int q0 = qtile * 32;
+    const float* qp = (const float*)a.q + bh * a.Tq * HS;
+    const float* kp = (const float*)a.k + bh * a.Tk * HS;
+    const float* vp = (const float*)a.v + bh * a.Tk * HS;
+    const int qrow = q0 + l32;
+
+    u32x4 qf[1][KF];
+    {
+        const int row = min(qrow, a.Tq - 1);
+#pragma unroll
+        for (int f = 0; f < KF; f++) qf[0][f] = *(const u32x4*)(qp + (size_t)row * HS + f * CPF + half * (CPF / 2));
+    }
+    floatx16 o[DT][1];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[dt][0][v] = 0.f;
+    float m[1] = {-INFINITY}, l[1] = {0.f};
+
+    const int lastStep = min(qtile, (a.Tk - 1) / 32);   // causal: keys past the tile's last row contribute nothing
+    for (int step = wave; step <= lastStep; step += 4) {
+        const int k0 = step * 32;
+        floatx16 s[1];
+#pragma unroll
+        for (int v = 0; v < 16; v++) s[0][v] = 0.f;
+        const float* krow = kp + (size_t)min(k0 + l32, a.Tk - 1) * HS + half * (CPF / 2);
+        u32x4 kf[KF];
+#pragma unroll
+        for (int f = 0; f < KF; f++) kf[f] = *(const u32x4*)(krow + f * CPF);
+        // V^T fragments: lane (d = 32 dt + l32, half) holds keys k0 + 8 t + 4 half .. + 3 of column d
+        u32x4 vf[PF][DT];
+#pragma unroll
+        for (int t = 0; t < PF; t++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                const float* vc = vp + dt * 32 + l32;
+                const int kb = k0 + 8 * t + 4 * half;
+                vf[t][dt] = u32x4{__float_as_uint(vc[(size_t)min(kb, a.Tk - 1) * HS]), __float_as_uint(vc[(size_t)min(kb + 1, a.Tk - 1) * HS]),
+                                  __float_as_uint(vc[(size_t)min(kb + 2, a.Tk - 1) * HS]), __float_as_uint(vc[(size_t)min(kb + 3, a.Tk - 1) * HS])};
+            }
+#pragma unroll
+        for (int f = 0; f < KF; f++) s[0] = TR::mma(kf[f], qf[0][f], s[0]);
+        // register v holds key k0 + 8 (v / 4) + 4 half + v % 4 for query q0 + l32
+        if (k0 + 31 > q0 || k0 + 32 > a.Tk) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (key > qrow || key >= a.Tk) s[0][v] = -INFINITY;
+            }
+        }
+        flash_softmax_step<false, DT, 1>(s, o, m, l, a.c, a.maskedRaw, a.lazy);
+#pragma unroll
+        for (int t = 0; t < PF; t++) {
+            const u32x4 pf = TR::pack_p(s[0], t);
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) o[dt][0] = TR::mma(vf[t][dt], pf, o[dt][0]);
+        }
+    }
+    // partial results to LDS: register v of tile dt is dim 32 dt + 8 (v / 4) + 4 half + v % 4 of query l32
+    const float lsum = l[0] + __shfl_xor(l[0], 32, 64);
+    if (half == 0) { Ms[wave][l32] = m[0]; Ls[wave][l32] = lsum; }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *(float4*)&Os[wave][l32 * LDO + 32 * dt + 8 * g + 4 * half] =
+                make_float4(o[dt][0][4 * g], o[dt][0][4 * g + 1], o[dt][0][4 * g + 2], o[dt][0][4 * g + 3]);
+    __syncthreads();
+    // thread t combines eight dims of query t / 8.  Wavefront 0 always has a step (key 0 is visible to every row), so
+    // the common maximum is finite; a wavefront without steps has maximum -inf and weight exp2(-inf) = 0.
+    const int q = tid >> 3, d8 = (tid & 7) * 8;
+    float mw[4], M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; w++) { mw[w] = Ms[w][q]; M = fmaxf(M, mw[w]); }
+    float L = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const float sc = __builtin_amdgcn_exp2f((mw[w] - M) * a.c);
+        L += Ls[w][q] * sc;
+        const float4 x0 = *(const float4*)&Os[w][q * LDO + d8], x1 = *(const float4*)&Os[w][q * LDO + d8 + 4];
+        acc[0] += x0.x * sc; acc[1] += x0.y * sc; acc[2] += x0.z * sc; acc[3] += x0.w * sc;
+        acc[4] += x1.x * sc; acc[5] += x1.y * sc; acc[6] += x1.z * sc; acc[7] += x1.w * sc;
+    }
+    if (q0 + q < a.Tq) {
+        const float inv = 1.0f / L;
+        float* yr = (float*)a.y + attn_y_row(a.yMerged, b, h, a.H, a.Tq, q0 + q, HS) + d8;
+        *(float4*)yr = make_float4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+        *(float4*)(yr + 4) = make_float4(acc[4] * inv, acc[5] * inv, acc[6] * inv, acc[7] * inv);
+    }
+}
+
 template <typename T, int HS, int QT, int NW, int OCC, bool PREFETCH>
 static hipError_t flash_launch_cfg(hipStream_t s, const FlashArgs& f, int kind)
 {
@@ -845,7 +955,15 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
         }
         return flash_launch_cfg<bf16_t, 128, 1, 8, 1, true>(s, f, a.kind);
     }
-    if (a.hs == 64) return flash_launch_cfg<float, 64, 1, 4, 2, false>(s, f, a.kind);
+    if (a.hs == 64) {
+        // causal self attention whose 128-row blocks would not give every CU a workgroup: one workgroup per 32 rows,
+        // the key steps dealt to its wavefronts
+        if (a.kind == MASK_CAUSAL && !a.lse2 && a.Tq == a.Tk && (long long)((a.Tq + 127) / 128) * a.H * a.B < 256) {
+            hipLaunchKernelGGL(flash_short_causal_f32_kernel, dim3((a.Tq + 31) / 32, a.H, a.B), 256, 0, s, f);
+            return hipGetLastError();
+        }
+        return flash_launch_cfg<float, 64, 1, 4, 2, false>(s, f, a.kind);
+    }
     return flash_launch_cfg<float, 128, 1, 8, 1, false>(s, f, a.kind);
 }
 

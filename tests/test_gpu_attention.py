@@ -28,7 +28,8 @@ def _attn(dev, q, k, v, mask, batch_mask, half=False, block=None):
     return out
 
 
-@pytest.mark.parametrize("B,H,T,hs", [(3, 8, 200, 64), (2, 4, 128, 64), (1, 2, 77, 48), (2, 2, 256, 128), (1, 1, 1, 64), (2, 3, 130, 32)])
+@pytest.mark.parametrize("B,H,T,hs", [(3, 8, 200, 64), (2, 4, 128, 64), (1, 2, 77, 48), (2, 2, 256, 128), (1, 1, 1, 64), (2, 3, 130, 32), (1, 4, 777, 64), (2, 2, 1000, 64),
+                                      (12, 32, 160, 64)])
 def test_attn_forward_causal_fp32(dev, B, H, T, hs):
     # the shape (3,8,200,64) is the one TestCudaAttentionForward uses (TestGPT_MultiheadAttentionLayer.cs:945-1036)
     rng = np.random.default_rng(T)
