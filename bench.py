@@ -702,8 +702,8 @@ def main():
         cpu = cpu_baseline(blob, head["prompt"], head["ids"])
         log("cpu baseline:", json.dumps(cpu))
 
-    # the two kernels the targets are set on (fused prefill attention >= 50 % of the bf16 MFMA peak, decode attention
-    # >= 70 % of HBM peak), inside the roofline object so that they travel with it
+    # the kernels the targets are set on (fused prefill attention >= 50 % of the bf16 MFMA peak, decode attention
+    # >= 70 % of HBM peak, the 16-bit QKV GEMM >= 40 %), inside the roofline object so that they travel with it
     targets = {}
     pa = also.get("prefill_attention_B8_T1024_H12x64", {}).get("bf16")
     if pa:
@@ -714,6 +714,11 @@ def main():
     da = also.get("decode_attention_H32x128", {})
     if "roofline" in da:
         targets["decode_attention_bf16_B32_L4096_H32x128"] = dict(da["roofline"], target_frac=0.7, avg_launch_us=da["bf16_B32_L4096"]["us"])
+    gq = also.get("gemm_inner_product", {}).get("bf16_qkv")
+    if gq:
+        targets["gemm_bf16_8192x2304x768"] = {"kernel": "QKV projection GEMM, 16-bit storage", "bound": "mfma", "achieved": gq["TFLOPs"],
+                                              "peak": MFMA_PEAK_TFLOPS["bf16"], "unit": "TFLOP/s", "frac": gq["frac_mfma"], "traffic": gq["traffic"],
+                                              "algorithmic_bytes": gq["algorithmic_bytes"], "target_frac": 0.4, "avg_launch_us": round(gq["ms"] * 1e3, 2)}
     roof["targets"] = targets
 
     line = {
