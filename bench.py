@@ -170,7 +170,9 @@ def step_roofline(inf, head, steps, warmup):
             "graph_replay": bool(head.get("graph")),
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic("decode_step"),
-            "traffic_note": "counter runs cover a step at position 512 (475.9 MB algorithmic there)",
+            "traffic_note": "counter runs cover a step at position 512 (475.9 MB algorithmic there); the timed steps ran at the positions given",
+            "traffic_position": 512, "traffic_algorithmic_bytes_at_that_position": 475900000,
+            "timed_positions_first": first, "timed_positions_last": first + n_first - 1,
             "algorithmic_bytes_per_launch": round(nbytes), "avg_launch_us": round(us, 3), "dispatches_per_launch": 62,
             "event_pair_around_empty_kernel_us": round(pair_ms * 1e3, 3), "per_class_event_pairs": detail}
 
@@ -659,7 +661,15 @@ def main():
         for tag, bf16, batch, kv16 in (("bf16_weights_b1", True, 1, False), ("fp32_b16", False, 16, False),
                                        ("bf16_weights_b16", True, 16, False), ("bf16_weights_and_cache_b16", True, 16, True)):
             i2, r = run_decode(cuda, path, bf16, batch, args.steps, args.warmup, graph=not args.no_graph, kv_bf16=kv16)
+            # algorithmic bytes of one step: every weight once, plus each sequence's cache at the mean timed length
+            first = N_PROMPT + args.warmup
+            mean_len = first + 1 + (min(args.steps, C4["seq_len"] - first) - 1) / 2.0
+            kvd = C4["dim"] // C4["n_heads"] * C4["n_kv_heads"]
+            step_bytes = weight_bytes(C4, 2 if bf16 else 4) + batch * C4["n_layers"] * 2 * mean_len * kvd * (2 if kv16 else 4)
+            gbps = step_bytes / (r["ms_per_step"] * 1e-3) / 1e9
             also["decode_" + tag] = {"tokens_per_s": round(r["tokens_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4),
+                                     "algorithmic_bytes_per_step": round(step_bytes), "GBps": round(gbps, 1),
+                                     "frac_hbm": round(gbps / HBM_PEAK_GBS, 4),
                                      "graph_replay": bool(r["graph"]), "prefill_128_tokens": prefill_summary(r, batch, 2 if bf16 else 4)}
             log("decode %s: %.1f tokens/s, prompt pass %s" % (tag, r["tokens_per_s"], json.dumps(also["decode_" + tag]["prefill_128_tokens"])))
             i2.CleanUp()
@@ -720,6 +730,29 @@ def main():
                                               "peak": MFMA_PEAK_TFLOPS["bf16"], "unit": "TFLOP/s", "frac": gq["frac_mfma"], "traffic": gq["traffic"],
                                               "algorithmic_bytes": gq["algorithmic_bytes"], "target_frac": 0.4, "avg_launch_us": round(gq["ms"] * 1e3, 2)}
     roof["targets"] = targets
+    # The same figures once more as flat scalars of the roofline object (a consumer that keeps only scalar keys still
+    # gets them), fractions of the MI355X peak (2.5 PFLOP/s bf16 MFMA, 8 TB/s HBM).
+    flat = {}
+    for key, tag in (("prefill_attention_bf16_causal_B8_T1024_H12x64", "prefill_bf16_causal_B8_T1024"),
+                     ("prefill_attention_bf16_causal_B4_T4096_H32x128", "prefill_bf16_causal_B4_T4096")):
+        if key in targets:
+            flat[tag + "_frac"] = targets[key]["frac"]
+            flat[tag + "_us"] = targets[key]["avg_launch_us"]
+    if "decode_attention_bf16_B32_L4096_H32x128" in targets:
+        t = targets["decode_attention_bf16_B32_L4096_H32x128"]
+        flat["decode_attn_bf16_B32_L4096_frac"] = t["frac"]
+        flat["decode_attn_bf16_B32_L4096_GBps"] = t["achieved"]
+    if "gemm_bf16_8192x2304x768" in targets:
+        flat["gemm_bf16_qkv_frac"] = targets["gemm_bf16_8192x2304x768"]["frac"]
+    for tag, short in (("fp32_b16", "decode_fp32_b16"), ("bf16_weights_b16", "decode_bf16w_b16"),
+                       ("bf16_weights_and_cache_b16", "decode_bf16w_bf16kv_b16"), ("bf16_weights_b1", "decode_bf16w_b1")):
+        d = also.get("decode_" + tag)
+        if d:
+            flat[short + "_frac_hbm"] = d["frac_hbm"]
+            flat[short + "_tokens_per_s"] = d["tokens_per_s"]
+            if d.get("prefill_128_tokens"):
+                flat[short + "_prefill_ms"] = d["prefill_128_tokens"]["ms"]
+    roof.update(flat)
 
     line = {
         "metric": "decode tokens/sec", "value": round(head["tokens_per_s"], 2), "unit": "tokens/s",
@@ -730,6 +763,11 @@ def main():
                    "prompt_tokens": N_PROMPT, "batch": 1, "device": dev_name},
         "roofline": roof, "cpu_baseline": cpu, "also": also,
     }
+    # the north-star figures once more, last on stderr
+    for k in sorted(flat):
+        log("%s = %s" % (k, flat[k]))
+    log("decode fp32 batch 1: %.1f tokens/s, %.4f ms/step, %.4f of HBM peak; cpu baseline %s tokens/s"
+        % (head["tokens_per_s"], head["ms_per_step"], roof["frac"], cpu["value"] if cpu else "not run"))
     print(json.dumps(line), flush=True)
     cuda.Dispose()
 
