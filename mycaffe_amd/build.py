@@ -6,8 +6,7 @@ Outputs (next to this file, git-ignored):
     libmycaffe_hip.so          the CudaDnnDLL-compatible C ABI (include/mycaffe_hip_abi.h)
     libmycaffe_hip_llama2.so   the llama2 extension library loaded through CREATE_EXTENSION
 and, beside their sources, two C++ host programs built on include/mycaffe_hip_host.hpp (plain g++, they only
-dlopen the libraries): tests/cpp/host_parity (parity) and host_bench/csa_layer_bench (whole-layer wall clock), and
-host_bench/hw_probes (hipcc; micro-benchmarks of the hardware properties the kernel designs rest on, no library use).
+dlopen the libraries): tests/cpp/host_parity (parity) and host_bench/csa_layer_bench (whole-layer wall clock).
 """
 import os
 import subprocess
@@ -26,7 +25,7 @@ FLAGS = [
     "-I", os.path.join(HERE, "..", "include"),
 ]
 
-KERNEL_SOURCES = ["ew_kernels.hip", "gemm.hip", "attn_prefill.hip", "attn_decode.hip", "attn_backward.hip"]
+KERNEL_SOURCES = ["ew_kernels.hip", "gemm.hip", "attn_prefill.hip", "attn_flash2.hip", "attn_decode.hip", "attn_backward.hip"]
 LIBS = {
     "libmycaffe_hip.so": KERNEL_SOURCES + ["library.hip"],
     "libmycaffe_hip_llama2.so": KERNEL_SOURCES + ["llama2_ext.hip"],
@@ -85,26 +84,7 @@ def build(force=False, verbose=True):
             print("built", out)
     built.append(build_host_program(force, verbose))
     built.append(build_host_program(force, verbose, os.path.join(HERE, "host_bench", "csa_layer_bench.cpp"), host_bench_path()))
-    built.append(build_hw_probes(force, verbose))
     return built
-
-
-def hw_probes_path():
-    return os.path.join(HERE, "host_bench", "hw_probes")
-
-
-def build_hw_probes(force=False, verbose=True):
-    src, out = os.path.join(HERE, "host_bench", "hw_probes.hip"), hw_probes_path()
-    if force or _stale(out, [src]):
-        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Wall", "-Wno-unused-result",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", src, "-o", out]
-        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
-        if r.returncode != 0:
-            raise RuntimeError("hipcc failed for hw_probes.hip:\n%s" % log)
-    if verbose:
-        print("built", os.path.normpath(out))
-    return out
 
 
 def host_program_path():
