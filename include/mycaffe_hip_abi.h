@@ -325,12 +325,15 @@ MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, floa
 
 /* ---- entry point that allocates nothing (no counterpart in the reference) ----
  * For callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
- * that forbid hipMalloc.  The call is ATTN_DECODE_FWD (id 2001) with the same f{scale} and l{...} arrays; the
+ * that forbid hipMalloc.  (What the entry point guarantees is that nothing is allocated and that its scratch is cleared
+ * by a fill kernel, not a memset node; it still makes host-side calls - hipSetDevice, hipGetLastError - and a capture
+ * of the call itself is not part of its tests.)  The call is ATTN_DECODE_FWD (id 2001) with the same f{scale} and l{...} arrays; the
  * split partials and merge tickets come from a fixed device array inside the library (4 MiB + 16 KiB per GPU,
  * held until the process ends) instead of the kernel object's growable workspace, and no hipMalloc, hipFree or
  * other allocating routine is called.  Limits: batch x heads <= 4096 and (batch x heads x splits) x (hs + 2) x 4
  * bytes <= 4 MiB, where splits = ceil(256 / (batch x heads)); larger calls return
- * MCH_ERROR_PARAM_OUT_OF_RANGE.  All calls on one GPU share the array: calls that overlap on one GPU (two kernel
+ * MCH_ERROR_PARAM_OUT_OF_RANGE before anything is enqueued (q, the new key / value and the caches are untouched, so
+ * the same call can then go through id 2001).  All calls on one GPU share the array: calls that overlap on one GPU (two kernel
  * objects, two host threads) race, so serialise them. */
 MCH_LONG MCH_AttnDecodeForwardNoAlloc(MCH_LONG lKernelIdx, float* pInput, MCH_LONG lInput, MCH_LONGLONG* plInput,
                                       MCH_LONG llInput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);

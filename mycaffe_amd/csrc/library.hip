@@ -987,7 +987,15 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         long long count = pl[0];
         const long long outer = pl[1], ch = pl[2], inner = pl[3];
         if (count < 0 || outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        if (!sub && ll > 6 && pl[6] == 2) count *= ch;
+        if (!sub && ll > 6 && pl[6] == 2) {
+            // the reference's second kernel divides all channels of the first `count` (n, s) pairs; that is the first
+            // kernel's element set only for the full count, the one the layers pass - a partial count is refused
+            if (count != outer * inner) {
+                last_detail = "channel_div method 2 takes count = outer * inner only";
+                return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            }
+            count *= ch;
+        }
         if (count > outer * ch * inner) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         MemItem *X, *Y, *A = nullptr;
         ERRCHK(mem((long)pl[4], &X));
@@ -2009,23 +2017,20 @@ long Kernel::attn_decode_fwd(float* pf, long lf, MCH_LONGLONG* pl, long ll, bool
     RANGE(KC, 0, need);
     RANGE(VC, 0, need);
     float scale = pf[0] != 0.f ? pf[0] : (float)(1.0 / sqrt((double)hs));
-    if (ll == 15 && (pl[12] || pl[13] || pl[14])) {
-        RopeState* rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
+    // Everything that can refuse the call comes before the first kernel: a refused call leaves q, the new key / value and
+    // the caches untouched, so that the caller can repeat it through the other entry point.
+    RopeState* rp = nullptr;
+    MemItem *KN = nullptr, *VN = nullptr;
+    const bool append = ll == 15 && (pl[12] || pl[13] || pl[14]);
+    if (append) {
+        rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
         if (pl[12] && (!rp || !rp->set)) return MCH_ERROR_ROPE_NOT_INITIALIZED;
         if (rp && (rp->hs != hs || len > rp->seq)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        MemItem *KN, *VN;
         ERRCHK(mem((long)pl[13], &KN));
         ERRCHK(mem((long)pl[14], &VN));
         if (KN->half != Q->half || VN->half != Q->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         RANGE(KN, 0, B * KVH * hs);
         RANGE(VN, 0, B * KVH * hs);
-        HIPCHK(k_rope_append(s, Q->dt(), Q->ptr, KN->ptr, VN->ptr, KC->ptr, VC->ptr, (int)B, (int)H, (int)KVH, (int)hs,
-                             (int)len - 1, sB, sH, sT, rp ? (const float*)rp->dcos.get() : nullptr,
-                             rp ? (const float*)rp->dsin.get() : nullptr));
-        m_mem.touch((long)pl[5]);
-        m_mem.touch((long)pl[6]);
-        m_mem.touch((long)pl[7]);
-        m_mem.touch((long)pl[13]);
     }
     size_t wsb = attn_decode_workspace_bytes((int)B, (int)H, (int)hs, (int)len);
     void* ws;
@@ -2042,14 +2047,22 @@ long Kernel::attn_decode_fwd(float* pf, long lf, MCH_LONGLONG* pl, long ll, bool
         tk = (int*)base;
         ws = base + MCH_NOALLOC_MAX_TICKETS * sizeof(int);
         wsHave = MCH_NOALLOC_PARTIAL_BYTES;
-        // the array keeps what the last call left: the tickets must start at zero (a fill kernel, so that a caller
-        // may capture the call into a graph)
-        HIPCHK(k_set(s, F32, tk, (size_t)(B * H), 0.f));
     } else {
         ERRCHK(workspace(wsb, &ws));
         wsHave = m_wsBytes;
         ERRCHK(tickets((size_t)(B * H), &tk));
     }
+    if (append) {
+        HIPCHK(k_rope_append(s, Q->dt(), Q->ptr, KN->ptr, VN->ptr, KC->ptr, VC->ptr, (int)B, (int)H, (int)KVH, (int)hs,
+                             (int)len - 1, sB, sH, sT, rp ? (const float*)rp->dcos.get() : nullptr,
+                             rp ? (const float*)rp->dsin.get() : nullptr));
+        m_mem.touch((long)pl[5]);
+        m_mem.touch((long)pl[6]);
+        m_mem.touch((long)pl[7]);
+        m_mem.touch((long)pl[13]);
+    }
+    // the static array keeps what the last call left: the tickets must start at zero (a fill kernel, not a memset node)
+    if (staticScratch) HIPCHK(k_set(s, F32, tk, (size_t)(B * H), 0.f));
     HIPCHK(k_attn_decode(s, Q->dt(), Q->ptr, KC->ptr, VC->ptr, Y->ptr, (int)B, (int)H, (int)KVH, (int)hs, (int)len, sB, sH,
                          sT, scale, ws, wsHave, nullptr, tk));
     m_mem.touch((long)pl[8]);

@@ -100,6 +100,24 @@ def test_llama110m_batch1_fp32_logits_and_ids(llm, c4_model):
     assert np.array_equal(ids_loop, ids)
 
 
+def test_llama110m_batch1_fp32_whole_generation_to_1024_positions(llm, c4_model):
+    # benchmark configuration 4 at its full length: 128 forced ids, then greedy to position 1023 (cache rows beyond the
+    # first split iteration, every split of the fused decode attention in use)
+    path, blob = c4_model
+    llm.Load(path)
+    prompt = np.random.default_rng(4).integers(3, C4["vocab_size"], 128)
+    n = C4["seq_len"]
+    ref_ids, ref_logits = O.Llama(C4, blob).generate_greedy(prompt, n, want_logits=True)
+    ids, logits = llm.GenerateIds(prompt, n, want_logits=True)   # eager launches
+    same = _ids_match(ids, ref_ids, ref_logits, "110M to 1024 positions", logits)
+    upto = n if same else int(np.argmax(np.asarray(ids) != np.asarray(ref_ids))) + 1
+    assert upto > 900, "ids part from the checker at position %d" % upto
+    assert_close(logits[:upto], ref_logits[:upto], FP32_RTOL, "110M logits up to position %d" % upto)
+    ids_graph = llm.GenerateIds(prompt, n)                        # replays of the captured step
+    assert llm.LastRunUsedGraph()
+    assert np.array_equal(ids_graph, ids)
+
+
 def test_llama110m_batch16_fp32_every_row_an_independent_cpu_run(llm, c4_model):
     path, blob = c4_model
     llm.Load(path)

@@ -130,7 +130,10 @@ def test_gemm_bf16_inner_product_shape(dev, m, n, k):
     (300, 200, 128, 1.0, 0.0),      # edge tiles in both directions
     (512, 768, 192, 0.5, 0.0),      # interior only, 128 x 192 tiles, alpha
     (384, 256, 64, 1.0, 2.0),       # beta != 0: read-modify-write epilogue
-    (1024, 1024, 2048, 1.0, 0.0),   # long K: 256 x 256 tiles
+    (1024, 1024, 2048, 1.0, 0.0),   # fewer 128 x 128 tiles than CUs and fewer than 200 tiles of 64 x 128: 64 x 64 tiles
+    (2048, 768, 2048, 1.0, 0.0),    # the same dispatch at the w2 shape of the batched prompt pass
+    (2048, 1024, 512, 1.0, 0.0),    # 128 tiles of 128 x 128, 256 of 64 x 128: the 64 x 128 tile
+    (2000, 1000, 512, 0.5, 1.0),    # the 64 x 128 tile with ragged edges and a read-modify-write epilogue
     (260, 132, 64, 0.25, -1.0),     # ragged, both scalars
 ])
 def test_gemm_fp32_large_tile_paths(dev, m, n, k, alpha, beta):
@@ -148,7 +151,10 @@ def test_gemm_fp32_large_tile_paths(dev, m, n, k, alpha, beta):
     (300, 200, 128, 1.0, 0.0),
     (512, 768, 192, 0.5, 0.0),
     (384, 256, 64, 1.0, 2.0),
-    (1024, 1024, 2048, 1.0, 0.0),
+    (1024, 1024, 2048, 1.0, 0.0),   # 64 x 64 tiles (see the fp32 list)
+    (2048, 768, 2048, 1.0, 0.0),    # 64 x 64 tiles
+    (2048, 1024, 512, 1.0, 0.0),    # 64 x 128 tiles
+    (2000, 1000, 512, 0.5, 1.0),    # 64 x 128 tiles, ragged, beta != 0
     (260, 132, 64, 0.25, -1.0),
 ])
 def test_gemm_bf16_large_tile_paths(dev, m, n, k, alpha, beta):
@@ -457,6 +463,27 @@ def test_rope_forward_vs_checker(dev, half):
     assert e.value.code == ERROR.ROPE_NOT_INITIALIZED
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_rope_forward_shorter_than_the_handle_keeps_the_reference_index_rule(dev, half):
+    # The reference derives a pair's position from its flat index modulo the HANDLE's sequence length
+    # (rope.cu:741-744), so with T < seq_len and more than one sequence the second sequence does not restart at
+    # position 0: its first rows continue at position T.  Reproduced, not corrected.
+    rng = np.random.default_rng(19)
+    B, T, S, H, hs = 2, 12, 16, 3, 16
+    x = bf16_round(rng.standard_normal((B, T, H, hs)).astype(np.float32))
+    h = dev.cuda.CreateRope(0, 0, B * S * H * hs, B, S, H, hs, 10000.0)
+    hx, hy = dev.put(x, half), dev.zeros(x.size, half)
+    dev.cuda.RopeForward(h, x.size, hx, hy)
+    ref = R.rope_forward(x, S, H, hs, 10000.0)
+    assert_close(dev.get(hy), ref, BF16_RTOL if half else 2e-6, "rope with T < seq_len")
+    # what the quirk amounts to: sequence 1, row 0 is rotated as position 12, and row 4 wraps to position 0
+    per_pos = R.rope_forward(np.broadcast_to(x[1, 0], (S, H, hs)).copy(), S, H, hs, 10000.0).reshape(S, H, hs)
+    assert_close(ref.reshape(B, T, H, hs)[1, 0], per_pos[12], 1e-6, "sequence 1 row 0 sits at position 12")
+    per_pos = R.rope_forward(np.broadcast_to(x[1, 4], (S, H, hs)).copy(), S, H, hs, 10000.0).reshape(S, H, hs)
+    assert_close(ref.reshape(B, T, H, hs)[1, 4], per_pos[0], 1e-6, "sequence 1 row 4 wraps to position 0")
+    dev.cuda.FreeRope(h)
+
+
 def test_elementwise_family(dev):
     rng = np.random.default_rng(10)
     n = 10007
@@ -759,6 +786,17 @@ def test_channel_primitives_of_the_softmax_chain(dev, half):
         dev.cuda.copy(full, hx, hfull)
         dev.cuda.channel_div(count, num, ch, sp, hr, hfull, method)
         assert_close(dev.get(hfull), R.channel_div(x, r, num, ch, sp), tol, "channel_div method %d" % method)
+    # a partial count: method 1 divides the first `count` elements; method 2 would divide all channels of the first
+    # `count` (n, s) pairs (math.cu:7171-7183), a different set, and is refused rather than silently run as method 1
+    dev.cuda.copy(full, hx, hfull)
+    part = (num - 1) * ch * sp
+    dev.cuda.channel_div(part, num, ch, sp, hr, hfull, 1)
+    want = R.channel_div(x, r, num, ch, sp).reshape(-1).copy()
+    want[part:] = x.reshape(-1)[part:]
+    assert_close(dev.get(hfull), want, tol, "channel_div method 1, partial count")
+    with pytest.raises(CudaDnnError) as ei:
+        dev.cuda.channel_div(n - sp, num, ch, sp, hr, hfull, 2)
+    assert ei.value.code == ERROR.PARAM_OUT_OF_RANGE
     dev.cuda.channel_dot(n, num, ch, sp, hx, ha, hy)
     assert_close(dev.get(hy), R.channel_dot(x, a, num, ch, sp), BF16_RTOL if half else 1e-5, "channel_dot")
     dev.cuda.exp(full, hx, hfull, 0, 0, 0.5)

@@ -588,3 +588,22 @@ def test_attn_backward_dropout_sequence_and_its_closed_form():
     y1, p1, pd1 = R.attn_forward_dropout(q, k, v, ones, 0.0, m, False, np.float64)
     for a, b in zip(R.attn_backward_dropout(q, k, v, pd1, ones, 0.0, dy, np.float64), R.attn_backward(q, k, v, p1, dy, np.float64)):
         assert np.allclose(a, b, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("slope", [0.0, 0.1])
+def test_relu_and_its_gradient_against_torch(slope):
+    """relu_fwd / relu_bwd of the checker against torch.nn.functional.leaky_relu and its autograd gradient.  The
+    reference's backward reads its gate from the TOP data (math.cu:12072-12078); for slope >= 0 the output has the sign
+    of the input, so that gate equals the one autograd takes from the input."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((7, 33)).astype(np.float32)
+    x[0, :4] = [0.0, -0.0, 1e-30, -1e-30]
+    dy = rng.standard_normal(x.shape).astype(np.float32)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    yt = torch.nn.functional.leaky_relu(xt, negative_slope=slope)
+    yt.backward(torch.tensor(dy, dtype=torch.float64))
+    y = R.relu(x, slope, np.float64)
+    assert np.allclose(y, yt.detach().numpy(), rtol=0, atol=1e-12)
+    nz = x != 0        # at exactly zero the subgradient is a convention
+    assert np.allclose(R.relu_grad(y, dy, slope, np.float64)[nz], xt.grad.numpy()[nz], rtol=0, atol=1e-12)

@@ -61,3 +61,25 @@ def test_no_alloc_entry_point_rejects_sizes_beyond_its_array(dev):
     assert "4096" in str(ei.value)
     # the ordinary entry point takes the same call
     dev.cuda.AttnDecodeForward(B, H, H, hs, L, hq, hk, hv, hy, H * L * hs, L * hs, hs)
+
+
+def test_no_alloc_entry_point_refuses_an_oversize_call_before_it_rotates_or_appends(dev):
+    # 15-argument form (rotary embedding + new key / value) beyond the array's 4096 (batch x head) pairs: the refusal has
+    # to come before the rotate-and-append kernel, or a caller that falls back to id 2001 would rotate q and k twice
+    rng = np.random.default_rng(9)
+    B, H, hs, L, S = 4097, 1, 8, 3, 4
+    q = rng.standard_normal((B, H, hs)).astype(np.float32)
+    kn, vn = (rng.standard_normal((B, H, hs)).astype(np.float32) for _ in range(2))
+    kc, vc = (rng.standard_normal((B, H, S, hs)).astype(np.float32) for _ in range(2))
+    hr = dev.cuda.CreateRope(0, 0, B * H * hs, B, S, H, hs, 10000.0)
+    hq, hkn, hvn, hk, hv, hy = dev.put(q), dev.put(kn), dev.put(vn), dev.put(kc), dev.put(vc), dev.zeros(q.size)
+    with pytest.raises(CudaDnnError) as ei:
+        dev.cuda.AttnDecodeForwardNoAlloc(B, H, H, hs, L, hq, hk, hv, hy, H * S * hs, S * hs, hs, 0.0, hr, hkn, hvn)
+    assert ei.value.code == ERROR.PARAM_OUT_OF_RANGE
+    for h, ref, name in ((hq, q, "q"), (hkn, kn, "new key"), (hk, kc, "key cache"), (hv, vc, "value cache")):
+        assert np.array_equal(dev.get(h, ref.shape), ref), name + " changed by a refused call"
+    # the fallback the header names: the same call through id 2001 equals a fresh id 2001 call
+    dev.cuda.AttnDecodeForward(B, H, H, hs, L, hq, hk, hv, hy, H * S * hs, S * hs, hs, 0.0, hr, hkn, hvn)
+    hq2, hkn2, hvn2, hk2, hv2, hy2 = dev.put(q), dev.put(kn), dev.put(vn), dev.put(kc), dev.put(vc), dev.zeros(q.size)
+    dev.cuda.AttnDecodeForward(B, H, H, hs, L, hq2, hk2, hv2, hy2, H * S * hs, S * hs, hs, 0.0, hr, hkn2, hvn2)
+    assert np.array_equal(dev.get(hy, q.shape), dev.get(hy2, q.shape))
