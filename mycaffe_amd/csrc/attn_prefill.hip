@@ -38,11 +38,6 @@ struct AttnArgs {
     AttnDropout drop;
 };
 
-// offset of output row `row` of head (b, h) in y
-__device__ __forceinline__ size_t attn_y_row(int yMerged, int b, int h, int H, int Tq, int row, int hs)
-{
-    return yMerged ? (((size_t)b * Tq + row) * H + h) * hs : (((size_t)b * H + h) * Tq + row) * hs;
-}
 
 // 4 wavefronts per workgroup, one query row each
 template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(AttnArgs a)
@@ -111,6 +106,7 @@ template <typename T> __global__ __launch_bounds__(256) void attn_rows_kernel(At
 }
 
 hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* handled);
+hipError_t attn_flash2_launch(hipStream_t s, const FlashArgs& f, int hs, bool causal, bool* handled);
 
 hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k, const void* v, void* y, int B, int H,
                           int Tq, int Tk, int hs, float scale, const float* mask, MaskKind kind, float* lse2, bool yMerged,
@@ -164,18 +160,6 @@ hipError_t k_attn_prefill(hipStream_t s, DType dt, const void* q, const void* k,
 // MFMA bound.  Causal: key blocks past the workgroup's last row are never visited,
 // wavefronts skip steps past their own rows, only diagonal steps pay for the element mask,
 // and workgroups are launched heaviest query block first across all heads.
-struct FlashArgs {
-    const void* q; const void* k; const void* v; void* y;
-    const float* mask;   // (B, Tk) key mask for KIND 2, (B, Tq, Tk) mask for KIND 3
-    int maskBatch;       // KIND 3: 1 = one (Tq, Tk) mask per sequence, 0 = one mask shared by all sequences
-    int B, H, Tq, Tk;
-    float c;             // softmax scale * log2(e)
-    float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
-    float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
-    float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
-    int yMerged;         // y laid out (B,Tq,H,hs) instead of (B,H,Tq,hs)
-    int causalGroup;     // causal launches: heads per group of the workgroup order (0: all heads in one group)
-};
 
 __device__ __forceinline__ float flash_half_max(float v)
 {
@@ -918,6 +902,15 @@ hipError_t attn_flash_launch(hipStream_t s, DType dt, const AttnArgs& a, bool* h
     // (128-row workgroups) give enough equal-sized workgroups to balance 256 CUs at T = 1024; head size 128
     // keeps eight wavefronts per workgroup so that each staged K / V block serves more rows.
     if (dt == BF16) {
+        // 512 keys and more, no mask or the causal one: the kernel with two query tiles per wavefront (attn_flash2.hip),
+        // 7 .. 30 % ahead of the ones below from that length on (B = 8, T = 1024, 12 heads of 64, causal: 26.4 against
+        // 28.6 us; B = 4, T = 4096, 32 heads of 128, causal: 0.52 against 0.62 ms).  Its workgroups own 256 query rows,
+        // too coarse a grain for shorter sequences.
+        if (f.Tk >= 512 && (a.kind == MASK_NONE || a.kind == MASK_CAUSAL)) {
+            bool took = false;
+            const hipError_t e = attn_flash2_launch(s, f, a.hs, a.kind == MASK_CAUSAL, &took);
+            if (e != hipSuccess || took) return e;
+        }
         if (a.hs == 64) {
             // Unmasked attention runs the software-pipelined kernel (B = 8, T = 1024, 12 heads: 45.7 us; B = 4,
             // T = 4096, 32 heads: 0.79 ms).  Causal launches measure the same (T = 1024) or up to 10 % slower

@@ -126,6 +126,26 @@ template <> struct FlashTraits<float> {
     }
 };
 
+// offset of output row `row` of head (b, h) in y
+__device__ __forceinline__ size_t attn_y_row(int yMerged, int b, int h, int H, int Tq, int row, int hs)
+{
+    return yMerged ? (((size_t)b * Tq + row) * H + h) * hs : (((size_t)b * H + h) * Tq + row) * hs;
+}
+
+// arguments of the matrix-core attention forward kernels (attn_prefill.hip, attn_flash2.hip)
+struct FlashArgs {
+    const void* q; const void* k; const void* v; void* y;
+    const float* mask;   // (B, Tk) key mask for KIND 2, (B, Tq, Tk) mask for KIND 3
+    int maskBatch;       // KIND 3: 1 = one (Tq, Tk) mask per sequence, 0 = one mask shared by all sequences
+    int B, H, Tq, Tk;
+    float c;             // softmax scale * log2(e)
+    float maskedRaw;     // raw (unscaled) score that stands for the reference's -1e29
+    float lazy;          // raw-score slack of the running maximum: 8 / c, so weights stay below 2^8
+    float* lse2;         // optional [B*H*Tq]: log2 of the softmax denominator of every row, kept for the backward pass
+    int yMerged;         // y laid out (B,Tq,H,hs) instead of (B,H,Tq,hs)
+    int causalGroup;     // causal launches: heads per group of the workgroup order (0: all heads in one group)
+};
+
 // Rank of a workgroup of a causal launch in the heaviest-first order.  Workgroup i goes to XCD i % 8 and, within it, the
 // first launches land on its 32 CUs in turn, `occ` rounds of 32 before the XCD is full.  A CU keeps what it was given in
 // those rounds, so every second one of them is walked backwards: the CU that got the heaviest block of one round gets

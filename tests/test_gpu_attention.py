@@ -132,6 +132,45 @@ def test_attn_forward_large_scores_lazy_rescale(dev):
         assert_close(out, ref, BF16_RTOL if half else FP32_RTOL, "causal attn with late large scores")
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,T,hs", [(1, 2, 512, 64), (2, 2, 513, 64), (1, 3, 777, 64), (1, 2, 1000, 128), (2, 1, 1024, 64), (1, 1, 1100, 128),
+                                      (1, 2, 1536, 64), (1, 1, 2000, 128), (1, 2, 575, 128), (1, 1, 640, 64)])
+def test_attn_forward_two_tiles_per_wavefront_kernel(dev, causal, B, H, T, hs):
+    # bf16 with 512 keys or more, no mask or the causal one, takes the kernel with two 32-row tiles per wavefront and
+    # 256-row workgroups: the lengths give workgroups with idle tiles (513, 575), a last block of 1 .. 63 keys (513, 777,
+    # 1000, 1100, 2000: the pinned phases stop four blocks before it), whole blocks only (512, 1024, 1536) and an odd
+    # number of 32-key steps (1000 -> 32 steps, 1100 -> 35)
+    rng = np.random.default_rng(T + hs + causal)
+    q, k, v = (bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(3))
+    out = _attn(dev, q, k, v, R.causal_mask(T) if causal else None, False, half=True)
+    ref, _ = R.attn_forward(q, k, v, R.causal_mask(T, np.float64) if causal else None, False, np.float64)
+    assert_close(out, ref, BF16_RTOL, "attn bf16, two tiles per wavefront")
+
+
+@pytest.mark.parametrize("hs", [64, 128])
+@pytest.mark.parametrize("scale", [1.5, 2.0, 3.0, 6.0])
+def test_attn_forward_two_tiles_per_wavefront_kernel_hands_large_scores_to_its_plain_pass(dev, hs, scale):
+    # That kernel takes exp2 of the scaled scores with the reference 0 and accepts a row whose sum of weights ends inside
+    # [2^-18, 2^18]; a workgroup with a row outside computes its rows again with running maxima.  Inputs scaled by 1.5 stay
+    # inside (scaled scores up to about 15), by 2 and more leave it (up to 25 .. 200 and far beyond what exp2 can hold).
+    rng = np.random.default_rng(int(10 * scale) + hs)
+    B, H, T = 1, 2, 640
+    q, k, v = (bf16_round(scale * rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(3))
+    for causal in (True, False):
+        out = _attn(dev, q, k, v, R.causal_mask(T) if causal else None, False, half=True)
+        ref, _ = R.attn_forward(q, k, v, R.causal_mask(T, np.float64) if causal else None, False, np.float64)
+        assert np.isfinite(out).all()
+        assert_close(out, ref, BF16_RTOL, "attn bf16, large scores")
+    # one row far below the range, the others ordinary: every key of query 100 scores about -60
+    q2, k2, v2 = (bf16_round(rng.standard_normal((B, H, T, hs)).astype(np.float32)) for _ in range(3))
+    k2[..., 0] = 8.0
+    q2[:, :, 100, 0] = -60.0 * np.sqrt(hs) / 8.0 / 1.4426950408889634
+    q2, k2 = bf16_round(q2), bf16_round(k2)
+    out = _attn(dev, q2, k2, v2, None, False, half=True)
+    ref, _ = R.attn_forward(q2, k2, v2, None, False, np.float64)
+    assert_close(out, ref, BF16_RTOL, "attn bf16, one row of tiny weights")
+
+
 def test_attn_mask_content_change_is_seen(dev):
     # a causal mask that is later overwritten through the ABI must stop being treated as causal
     rng = np.random.default_rng(13)
