@@ -1,10 +1,13 @@
 // Fused attention forward for 16-bit storage, head sizes 64 and 128, no mask or the causal one (gfx950).
 //
 // What bounds this computation on the part is not the matrix cores alone.  Every MFMA of an attention step takes one
-// 1 KB operand fragment from LDS (K for the scores, V^T for the output; Q and P stay in registers), and the LDS of a CU
-// streams about as many fragments per unit of time as its four SIMDs can multiply; and the softmax between the two
-// products is vector work that one wavefront can only hide behind its OWN MFMAs (a wavefront that issues MFMAs back to
-// back starves the vector instructions of its neighbours on the SIMD).  The kernel is built around both facts:
+// 1 KB operand fragment from LDS (K for the scores, V^T for the output; Q and P stay in registers), the softmax between
+// the two products is vector work, and a wavefront issues one instruction every four to five cycles whatever its kind
+// (an exponential every twelve): per 64 keys a wavefront with 64 query rows issues about as many cycles of other
+// instructions as its MFMAs take.  Vector work of one wavefront does not hide behind the MFMAs of another on the same
+// SIMD, only behind its own; and with every unit busy the part runs into its power limit, where time follows the
+// number of instructions and bytes moved rather than the longest of the parallel streams (the same kernel is a
+// quarter faster on all-zero operands).  The kernel is built around these facts:
 //
 //  * Two 32-row query tiles per wavefront.  Every K / V fragment read from LDS feeds two MFMAs, one per tile, which
 //    halves the LDS traffic per flop.  The fragments are held in registers across the two tiles' phases.
@@ -12,25 +15,33 @@
 //    vector ALU does the softmax of job j, the matrix cores do S^T of job j + 1 and O^T += V^T P^T of job j - 1, in a
 //    pinned issue order (one scheduling region per MFMA, each followed by a slice of the softmax, the fragment reads of
 //    the next phase and a slice of the K / V staging).  Jobs alternate between the two tiles, so a block of 64 keys is
-//    four such phases in straight-line code with fixed registers.  Blocks in which some step of the wavefront needs a
-//    mask (the diagonal of the causal mask, the ragged end of the keys) run the same jobs one after the other instead.
-//  * One wavefront per SIMD with the whole register file: the output tiles and the Q fragments live in accumulation
-//    registers (MFMA operands may come from either file), the score tiles, weights and K / V fragments in vector
-//    registers.  The MFMAs of the pinned phases are inline assembly with the register file of every operand spelled
-//    out, because the compiler's own choice for an MFMA result is an accumulation register, which the vector ALU cannot
-//    read (sixteen copies per score tile).
+//    four such phases in straight-line code with fixed registers.
+//  * The output tiles and the Q fragments live in accumulation registers (MFMA operands may come from either file), the
+//    score tiles, weights and K / V fragments in vector registers.  The MFMAs of the pinned phases are inline assembly
+//    with the register file of every operand spelled out, because the compiler's own choice for an MFMA result is an
+//    accumulation register, which the vector ALU cannot read (sixteen copies per score tile).  Head size 64 fits 256
+//    registers, two workgroups per CU; head size 128 takes the whole file, one wavefront per SIMD.
 //  * A lean softmax.  Q is multiplied by scale * log2(e) once, when its fragments are loaded, and the weights are
-//    exp2(score - m) with the reference m of a row at 0 for as long as every step's sum stays inside [2^-60, 2^60]: bf16
-//    and fp32 share their exponent range, so weights far from 1 lose no precision, and a score then costs one v_exp_f32
-//    and half a v_cvt_pk_bf16_f32.  The row sum is formed from the packed pairs with v_dot2c_f32_bf16 (a two-element dot
-//    product against ones), i.e. from exactly the rounded weights that multiply V.  A workgroup one of whose rows leaves
-//    that range (scaled scores beyond about +-40 in natural units) raises a flag in LDS and, after its pass, computes its
-//    rows again with the usual running maximum, one job after the other: correct for any input, at twice the time for
-//    such a workgroup.
-//  * K and V blocks of 64 keys are staged through registers into three LDS stages, rows unpadded, the 16-byte pieces of
+//    exp2(score) with a fixed reference, 0, instead of a running maximum: bf16 and fp32 share their exponent range, so
+//    weights far from 1 lose no precision, and a score then costs one v_exp_f32 and half a v_perm_b32 (the bf16 pair
+//    is the upper halves of the two floats).  The row sum is formed from the packed pairs with v_dot2c_f32_bf16 (a
+//    two-element dot product against ones), i.e. from exactly the weights that multiply V, so rounding the weights
+//    down cancels between numerator and denominator.  No step needs the result of another: the jobs of a row may run in
+//    any order, and partial sums simply add.
+//  * A workgroup one of whose row sums ends outside [2^-18, 2^18] (scaled scores beyond about +-18: weights that exp2
+//    cannot hold, or scores large enough for the second rounding of Q to show) computes its rows again the plain way:
+//    running maxima, the scale applied to the scores in fp32 (flash2_plain_pass).  Correct for any input, at several
+//    times the cost for such a workgroup.
+//  * K and V blocks of 64 keys are staged through registers into four LDS stages, rows unpadded, the 16-byte pieces of
 //    a row permuted by an XOR of row bits so that both the 128-bit K fragment reads (sixteen rows per access) and the
 //    transposing V reads (four rows x 64 bytes per access) fall on distinct banks.  A block is requested from memory a
-//    whole block (four phases) before it is written to LDS; one workgroup barrier per block.
+//    whole block (four phases) before it is written to LDS, a few pieces per phase; one workgroup barrier per block.
+//  * Blocks in which some step of the wavefront needs a mask (the diagonal of the causal mask, the ragged end of the
+//    keys) run one job after the other.  With the causal mask that block is a different one for every wavefront of the
+//    workgroup, so these blocks are kept in their stages and done behind the loop over the blocks, by all wavefronts at
+//    once, instead of one wavefront at a time with the others waiting at the block's barrier.
+//  * The output leaves through LDS as whole rows, 16 bytes a lane: a lane owns a query, and its own values would be
+//    sixteen scattered 8-byte stores.
 //
 // Scores are computed transposed (S^T = K Q^T), so that a lane owns one query row: register v of a 32 x 32 tile holds
 // key 8 (v / 4) + 4 (lane / 32) + v % 4 of query lane % 32.
