@@ -276,7 +276,12 @@ enum {
      *                 caches stay fp32); takes effect at the next generation; option 9 = where the
      *                 partial results of a single sequence's attention splits are merged: in front of
      *                 the output projection's mat-vec (1, default, when dim <= 1024 and the cache fits
-     *                 one pass of rows per split) or inside the attention kernel (0)
+     *                 one pass of rows per split) or inside the attention kernel (0); option 10 = the
+     *                 batched prompt pass over 16-bit weights (more than 256 prompt rows, widths that are
+     *                 multiples of 64) keeps its activations to sixteen leading bits - two bf16 numbers a
+     *                 value on the bf16 matrix cores, attention in fp32: logits within the fp32 bar of the
+     *                 step-per-position loop (0, default) - or rounds them to bf16 and runs the attention
+     *                 in bf16 (1: half the matrix-core work, logits within the 16-bit bar)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were

@@ -11,6 +11,8 @@
 //  * gemv              : HBM-bound y = A x, one wavefront per row, 128-bit loads.
 #include <algorithm>
 
+#include <type_traits>
+
 #include "kernels.h"
 
 namespace mch {
@@ -357,11 +359,15 @@ __device__ __forceinline__ T* heads_dst(const HeadsEpilogue& he, int row, int co
     return (T*)he.dst[which] + (((size_t)b * he.H + h) * he.T + t) * he.hs + d;
 }
 
-template <typename T, int WM, int WN, int OCC, bool HEADS = false>
+// SPLIT (16-bit operands, fp32 C): a row of A is 2 K long, the upper halves of K fp32 values followed by what the upper
+// halves leave over (see k_gemm_bf16_split), and B is walked twice: C = alpha (A_hi + A_lo) B^T + beta C.
+template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false>
 __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
-                                                               const T* __restrict__ B, float beta, T* __restrict__ C, int tilesN,
+                                                               const T* __restrict__ B, float beta, TC* __restrict__ C, int tilesN,
                                                                int tilesTotal, int bandRows, int colBlock, HeadsEpilogue he)
 {
+    static_assert(std::is_same<T, TC>::value || (!HEADS && std::is_same<TC, float>::value), "C is of the operands' type, or fp32");
+    static_assert(!SPLIT || !std::is_same<T, TC>::value, "the split product writes fp32");
     typedef BigTraits<T> TR;
     constexpr int E = TR::E;
     constexpr int BK = 8 * E;                                 // elements per stage and row (128 bytes)
@@ -409,14 +415,14 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     const T* ga[PA];
     const T* gb[PB];
 #pragma unroll
-    for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * K + lc;
+    for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * (SPLIT ? 2 * K : K) + lc;
 #pragma unroll
     for (int p = 0; p < PB; p++) gb[p] = B + (size_t)min(n0 + lr + p * RPP, N - 1) * K + lc;
     T* sa = As + lr * LDK + lc;
     T* sb = Bs + lr * LDK + lc;
     u32x4 ra[PA], rb[PB];
 
-    const int nk = K / BK;
+    const int nkB = K / BK, nk = SPLIT ? 2 * nkB : nkB;   // stage kt of A goes with stage kt % nkB of B
     // stage 0 -> LDS buffer 0, stage 1 -> registers
 #pragma unroll
     for (int p = 0; p < PA; p++) ra[p] = *(const u32x4*)(ga[p]);
@@ -427,11 +433,11 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
 #pragma unroll
     for (int p = 0; p < PB; p++) *(u32x4*)(sb + p * RPP * LDK) = rb[p];
     {
-        const int k1 = min(1, nk - 1) * BK;
+        const int s1 = min(1, nk - 1), k1 = s1 * BK, k1b = (SPLIT ? s1 % nkB : s1) * BK;
 #pragma unroll
         for (int p = 0; p < PA; p++) ra[p] = *(const u32x4*)(ga[p] + k1);
 #pragma unroll
-        for (int p = 0; p < PB; p++) rb[p] = *(const u32x4*)(gb[p] + k1);
+        for (int p = 0; p < PB; p++) rb[p] = *(const u32x4*)(gb[p] + k1b);
     }
     __syncthreads();
     const int fr = lane & 31, fg = (lane >> 5) * E;
@@ -451,7 +457,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
         const T* pb = fb + buf * BN * LDK;
         T* wa = sa + (buf ^ 1) * BM * LDK;
         T* wb = sb + (buf ^ 1) * BN * LDK;
-        const int k2 = min(kt + 2, nk - 1) * BK;
+        const int s2 = min(kt + 2, nk - 1), k2 = s2 * BK, k2b = (SPLIT ? (s2 >= nkB ? s2 - nkB : s2) : s2) * BK;
 #pragma unroll
         for (int t = 0; t < WM; t++) a[0][t] = *(const u32x4*)(pa + t * 32 * LDK);
 #pragma unroll
@@ -484,7 +490,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                         else *(u32x4*)(wb + (c - PA) * RPP * LDK) = rb[c - PA];
                     } else {
                         if (c < PA) ra[c] = *(const u32x4*)(ga[c] + k2);
-                        else rb[c - PA] = *(const u32x4*)(gb[c - PA] + k2);
+                        else rb[c - PA] = *(const u32x4*)(gb[c - PA] + k2b);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -496,6 +502,36 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     // row of C (lane%32) and register v is column 8*(v/4) + 4*(lane/32) + v%4: four consecutive columns per
     // register quad.
     const int row_l = lane & 31, col_l = (lane >> 5) * 4;
+    if constexpr (!std::is_same<T, TC>::value) {
+        // fp32 C from 16-bit operands: a lane's register quad is four consecutive columns of its row, one 16-byte access
+        const bool vec4 = (N & 3) == 0 && (((uintptr_t)C) & 15) == 0;
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++) {
+                const int r = m0 + wm + i * 32 + row_l;
+                if (r >= M) continue;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int c = n0 + wn + j * 32 + 8 * g + col_l;
+                    float* cp = C + (size_t)r * N + c;
+                    if (vec4 && c + 3 < N) {
+                        float4 o = make_float4(alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1], alpha * acc[i][j][4 * g + 2],
+                                               alpha * acc[i][j][4 * g + 3]);
+                        if (beta != 0.f) {
+                            const float4 old = *(const float4*)cp;
+                            o.x += beta * old.x; o.y += beta * old.y; o.z += beta * old.z; o.w += beta * old.w;
+                        }
+                        *(float4*)cp = o;
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            if (c + q < N) cp[q] = alpha * acc[i][j][4 * g + q] + (beta != 0.f ? beta * cp[q] : 0.f);
+                    }
+                }
+            }
+        return;
+    } else
     if (m0 + BM <= M && n0 + BN <= N && (HEADS || (beta == 0.f && (((uintptr_t)C) & 15) == 0)) && (N % E) == 0) {
         // interior tile: each wavefront passes its tile, 32 rows at a time, through its own slice of LDS (free
         // after the last barrier) and writes whole 16-byte pieces of rows, the lanes covering full cache lines
@@ -533,6 +569,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
         return;
     }
     // edge tiles, beta != 0: element-wise (unrolled, so the accumulators are never indexed dynamically)
+    if constexpr (std::is_same<T, TC>::value) {
 #pragma unroll
     for (int i = 0; i < WM; i++)
 #pragma unroll
@@ -555,9 +592,10 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                 }
             }
         }
+    }
 }
 
-template <typename T, int WM, int WN, int OCC, bool HEADS = false>
+template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false>
 static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C,
                              const HeadsEpilogue* heads = nullptr)
 {
@@ -573,7 +611,7 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
     if (ldsEpilogue > lds) lds = ldsEpilogue;
     static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
     if (!attr) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC, HEADS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr = true;
     }
@@ -589,8 +627,8 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
             colBlock = (tn + nb - 1) / nb;   // equal-width blocks
         }
     }
-    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
-                       (T*)C, tn, (int)total, bandRows, colBlock, he);
+    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
+                       (TC*)C, tn, (int)total, bandRows, colBlock, he);
     return hipGetLastError();
 }
 
@@ -884,6 +922,33 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
     if (dt == F32) hipLaunchKernelGGL(qkv_split_heads_kernel<float>, grid, 256, 0, s, (const float*)tmp, total, n, he);
     else hipLaunchKernelGGL(qkv_split_heads_kernel<bf16_t>, grid, 256, 0, s, (const bf16_t*)tmp, total, n, he);
     return hipGetLastError();
+}
+
+// C (m x n, fp32) = alpha X W^T + beta C for a 16-bit weight matrix W (n x k), on the bf16 matrix cores, C in fp32.
+// split = false: A is X rounded to bf16, m rows of k.  split = true keeps the activations' precision: A holds every row of
+// an fp32 X as two bf16 rows back to back, the bf16 nearest to each of its k values and then the bf16 nearest to what
+// those leave over, and the kernel walks W once for each.  The products are exact and accumulate in fp32, so what is lost
+// is the part of X below its leading sixteen bits: 2^-17 relative, against 2^-9 for activations rounded to bf16.
+// k a multiple of 64, 16-byte aligned operands.
+template <bool SPLIT>
+static hipError_t gemm_bf16_f32_tiles(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* W, float beta, float* C)
+{
+    // Tile shapes as k_gemm picks them for bf16: below 200 tiles of 128 x 128, 64 x 128 tiles where they give every CU
+    // one, else 64 x 64 (2048 x 768: 384 tiles of 64 x 64 measure 27.8 us a product, 192 of 64 x 128 30.1 us).
+    const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+    if (t128 < 200) {
+        const long long t64x128 = (long long)((m + 63) / 64) * ((n + 127) / 128);
+        if (t64x128 >= 200) return launch_big<bf16_t, 1, 2, 3, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+        return launch_big<bf16_t, 1, 1, 3, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+    }
+    if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+    return launch_big<bf16_t, 2, 2, 2, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+}
+hipError_t k_gemm_bf16_f32(hipStream_t s, int m, int n, int k, float alpha, const void* A, bool split, const void* W, float beta, float* C)
+{
+    if (m <= 0 || n <= 0) return hipSuccess;
+    if (k <= 0 || k % 64 != 0 || (((uintptr_t)A | (uintptr_t)W) & 15) != 0) return hipErrorInvalidValue;
+    return split ? gemm_bf16_f32_tiles<true>(s, m, n, k, alpha, A, W, beta, C) : gemm_bf16_f32_tiles<false>(s, m, n, k, alpha, A, W, beta, C);
 }
 
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,

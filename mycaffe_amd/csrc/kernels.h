@@ -104,6 +104,9 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
 hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
                             void* q, void* k, void* v, void* tmp);
 // column-major strided batched gemm with BLAS semantics (fp32)
+// C (fp32) = alpha X W^T + beta C on the bf16 matrix cores: W 16-bit (n x k), k % 64 == 0; A is X as bf16 (m x k) or,
+// split, every row of X as two bf16 rows (nearest bf16, then the bf16 nearest to the remainder; m x 2k)
+hipError_t k_gemm_bf16_f32(hipStream_t s, int m, int n, int k, float alpha, const void* A, bool split, const void* W, float beta, float* C);
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
                    int batch);

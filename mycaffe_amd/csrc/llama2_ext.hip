@@ -678,9 +678,9 @@ template <> __device__ inline float2 as_stored<bf16_t>(float2 v) { return make_f
 // One row [q | k | v] of raw projections per (b, p): rotate q and k at position p (adjacent pairs, the arithmetic of
 // the decode kernel), write q as (B,H,P,hs), k and v as (B,H,P,hs) with every key / value head repeated for the query
 // heads that share it, and append the rotated key and the value to the caches [b][pos][kvd].
-template <typename TC>
-__global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float* __restrict__ qh, float* __restrict__ kh,
-                                            float* __restrict__ vh, TC* __restrict__ kc, TC* __restrict__ vc,
+template <typename TC, typename TQ>
+__global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, TQ* __restrict__ qh, TQ* __restrict__ kh,
+                                            TQ* __restrict__ vh, TC* __restrict__ kc, TC* __restrict__ vc,
                                             const float* __restrict__ fcos, const float* __restrict__ fsin, int B, int P, int H,
                                             int kvH, int hs, int seqLen)
 {
@@ -700,18 +700,18 @@ __global__ void prefill_rope_scatter_kernel(const float* __restrict__ qkv, float
             o.x = r.x * cs - r.y * sn;
             o.y = r.x * sn + r.y * cs;
             if (col < dim) {
-                *(float2*)(qh + (((size_t)b * H + h) * P + p) * hs + d) = o;
+                store_pair(qh + (((size_t)b * H + h) * P + p) * hs + d, o);
             } else {
                 o = as_stored<TC>(o);   // the pass attends over the values the cache holds, as the decode steps will
                 store_pair(kc + ((size_t)b * seqLen + p) * kvd + c, o);
-                for (int g = 0; g < kvMul; g++) *(float2*)(kh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = o;
+                for (int g = 0; g < kvMul; g++) store_pair(kh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d, o);
             }
         } else {
             const int c = col - dim - kvd;
             const int h = c / hs, d = c - h * hs;
             const float2 rs = as_stored<TC>(r);
             store_pair(vc + ((size_t)b * seqLen + p) * kvd + c, rs);
-            for (int g = 0; g < kvMul; g++) *(float2*)(vh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d) = rs;
+            for (int g = 0; g < kvMul; g++) store_pair(vh + (((size_t)b * H + h * kvMul + g) * P + p) * hs + d, rs);
         }
     }
 }
@@ -725,6 +725,66 @@ __global__ void prefill_swiglu_kernel(const float* __restrict__ h2, float* __res
         const int j = (int)(i - m * hid);
         const float a0 = h2[m * 2 * hid + j], a1 = h2[m * 2 * hid + hid + j];
         hb[i] = a0 * (1.0f / (1.0f + expf(-a0))) * a1;
+    }
+}
+
+// The prompt pass over 16-bit weights multiplies its fp32 activations on the bf16 matrix cores.  LO = true: as two bf16
+// numbers each - hi, the bf16 nearest to the value, and lo, the bf16 nearest to what hi leaves over; both products with
+// a bf16 weight are exact and the sums are fp32, so the activations keep sixteen leading bits.  A row of n values then
+// becomes 2 n bf16 values, the n his first.  LO = false: hi alone (activations rounded to bf16), rows of n.
+template <bool LO> __device__ inline void split_store4(bf16_t* row, int n, int i, float4 v)
+{
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    bf16_t hi[4], lo[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        hi[q] = f32_to_bf16(f[q]);
+        lo[q] = f32_to_bf16(f[q] - bf16_to_f32(hi[q]));
+    }
+    *(uint2*)(row + i) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16));
+    if (LO) *(uint2*)(row + n + i) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
+}
+// out[m] = split(g * x[m] / sqrt(mean(x[m]^2) + eps)) (g null: split(x[m])); one workgroup per row, n a multiple of 4
+template <bool LO>
+__global__ __launch_bounds__(256) void prefill_norm_split_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                                 bf16_t* __restrict__ out, int n, float eps)
+{
+    __shared__ float red[4];
+    const float* xr = x + (size_t)blockIdx.x * n;
+    bf16_t* orow = out + (size_t)blockIdx.x * (LO ? 2 : 1) * n;
+    float inv = 1.0f;
+    if (g) {
+        float ss = 0.f;
+        for (int i = threadIdx.x * 4; i < n; i += 1024) {
+            const float4 v = *(const float4*)(xr + i);
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+        ss = group_sum<64>(ss);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        ss = red[0] + red[1] + red[2] + red[3];
+        inv = 1.0f / sqrtf(ss / n + eps);
+    }
+    for (int i = threadIdx.x * 4; i < n; i += 1024) {
+        float4 v = *(const float4*)(xr + i);
+        if (g) {
+            const float4 w = *(const float4*)(g + i);
+            v = make_float4(w.x * (inv * v.x), w.y * (inv * v.y), w.z * (inv * v.z), w.w * (inv * v.w));
+        }
+        split_store4<LO>(orow, n, i, v);
+    }
+}
+// out[m] = split(silu(h2[m, j]) * h2[m, hid + j]), hid a multiple of 4
+template <bool LO>
+__global__ void prefill_swiglu_split_kernel(const float* __restrict__ h2, bf16_t* __restrict__ out, size_t rows, int hid)
+{
+    const size_t total = rows * hid / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+        const size_t m = i * 4 / hid;
+        const int j = (int)(i * 4 - m * hid);
+        const float4 a0 = *(const float4*)(h2 + m * 2 * hid + j), a1 = *(const float4*)(h2 + m * 2 * hid + hid + j);
+        auto f = [](float a, float b) { return a * (1.0f / (1.0f + expf(-a))) * b; };
+        split_store4<LO>(out + m * (LO ? 2 : 1) * hid, hid, j, make_float4(f(a0.x, a1.x), f(a0.y, a1.y), f(a0.z, a1.z), f(a0.w, a1.w)));
     }
 }
 
@@ -895,6 +955,7 @@ public:
     bool use_graph = true;
     bool lastUsedGraph = false;  // whether the last generate replayed a captured graph (false: eager launches)
     bool use_prefill = true;     // prompt positions as one batched pass (false: one decode step per position)
+    bool prefill_act16 = false;  // 16-bit weights, many prompt rows: activations of the pass rounded to bf16 (false: kept to sixteen bits)
     bool kv_bf16 = false;        // caches stored as bf16 (option 8; takes effect when the run state is next allocated)
     bool state_kv_bf16 = false;  // what the allocated caches hold
     void set_kv_bf16(bool on) { kv_bf16 = on; if (on != state_kv_bf16) { stateB = -1; graphB = -1; } }
@@ -925,7 +986,6 @@ private:
     long ensure_state(int B, int nSteps);
     long ensure_prefill(size_t rows);
     template <typename T> long prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits);
-    template <typename T> const float* as_f32(hipStream_t s, const void* w, size_t n, long* err);
     hipError_t embed_first(hipStream_t s, int B);
 
     hipStream_t stream = nullptr;
@@ -967,6 +1027,7 @@ private:
     std::vector<void*> prefillAllocs;
     float *pfX = nullptr, *pfXn = nullptr, *pfQkv = nullptr, *pfQ = nullptr, *pfK = nullptr, *pfV = nullptr,
           *pfH2 = nullptr, *pfHb = nullptr, *pfLogits = nullptr, *pfW = nullptr;
+    bool pfSplit = false;
 };
 
 void Engine::release()
@@ -1227,21 +1288,13 @@ long Engine::ensure_prefill(size_t rows)
     pfX = pa(rows * dim); pfXn = pa(rows * dim); pfQkv = pa(rows * (dim + 2 * kvd));
     pfQ = pa(rows * dim); pfK = pa(rows * dim); pfV = pa(rows * dim);
     pfH2 = pa(rows * 2 * hid); pfHb = pa(rows * hid); pfLogits = pa(pfLogitRows * V);
-    // weights stored as bf16 are widened to fp32 one matrix at a time: room for the largest one
-    pfW = stored_bf16 ? pa(std::max({(dim + 2 * kvd) * dim, 2 * hid * dim, V * dim})) : pfX;
+    // 16-bit weights: the GEMMs read their activations as pairs of bf16 rows (prefill_norm_split_kernel), 2 x 2 bytes a
+    // value; widths that are no multiple of 64 widen one matrix at a time to fp32 instead and need room for the largest
+    pfSplit = dim % 64 == 0 && hid % 64 == 0;
+    pfW = !stored_bf16 ? pfX : pfSplit ? pa(rows * std::max(dim, hid)) : pa(std::max({(dim + 2 * kvd) * dim, 2 * hid * dim, V * dim}));
     if (!pfX || !pfXn || !pfQkv || !pfQ || !pfK || !pfV || !pfH2 || !pfHb || !pfLogits || !pfW) return MCH_ERROR_MEMORY_OUT;
     pfRows = rows;
     return 0;
-}
-
-// the matrix as fp32: itself, or (16-bit storage) widened into the scratch matrix, which gives the GEMM exactly the
-// values the decode path's mat-vec kernels widen in registers
-template <typename T> const float* Engine::as_f32(hipStream_t s, const void* w, size_t n, long* err)
-{
-    if (sizeof(T) == 4) return (const float*)w;
-    hipError_t e = k_convert(s, BF16, w, F32, pfW, n);
-    if (e != hipSuccess) *err = (long)e;
-    return pfW;
 }
 
 // Positions 0 .. P-1 of all B sequences in one pass.  Leaves what P single-token steps leave: the caches of every
@@ -1261,62 +1314,102 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
     // Few rows (one or two sequences' prompts): the fused mat-vec family on the matrix cores, all rows sharing one walk
     // over each matrix, norms / SwiGLU / residuals in its epilogues.  Many rows: 128 x 128-tile GEMMs.
     const bool skinny = M <= 256 && dim % 32 == 0 && hid % 32 == 0;
+    enum { PF_F32, PF_WIDEN, PF_SPLIT, PF_ACT16 };
+    const int mode = sizeof(T) == 4 ? PF_F32 : !pfSplit ? PF_WIDEN : (prefill_act16 && (hs == 64 || hs == 128)) ? PF_ACT16 : PF_SPLIT;
     for (int l = 0; l < cfg.n_layers; l++) {
         const LayerW<void>& w = layers[l];
         const LayerW<void>& wp = packed[l];
         const size_t cacheOfs = (size_t)l * B * cfg.seq_len * kvd * (state_kv_bf16 ? 2 : 4);
         void* kcl = (char*)kc + cacheOfs;
         void* vcl = (char*)vc + cacheOfs;
-        auto rope_scatter = [&]() {
-            if (state_kv_bf16)
-                hipLaunchKernelGGL(prefill_rope_scatter_kernel<bf16_t>, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, (bf16_t*)kcl,
-                                   (bf16_t*)vcl, fcos, fsin, B, P, H, kvH, hs, cfg.seq_len);
-            else
-                hipLaunchKernelGGL(prefill_rope_scatter_kernel<float>, grid_for(M * ldq / 2), 256, 0, s, pfQkv, pfQ, pfK, pfV, (float*)kcl,
-                                   (float*)vcl, fcos, fsin, B, P, H, kvH, hs, cfg.seq_len);
+        // act16: the q / k / v head tensors (and with them the attention) in bf16
+        auto rope_scatter = [&](bool act16) {
+            const int g = grid_for(M * ldq / 2);
+#define ROPE_SCATTER(TC, TQ) hipLaunchKernelGGL((prefill_rope_scatter_kernel<TC, TQ>), g, 256, 0, s, pfQkv, (TQ*)pfQ, (TQ*)pfK, (TQ*)pfV, (TC*)kcl, \
+                                                (TC*)vcl, fcos, fsin, B, P, H, kvH, hs, cfg.seq_len)
+            if (state_kv_bf16) { if (act16) ROPE_SCATTER(bf16_t, bf16_t); else ROPE_SCATTER(bf16_t, float); }
+            else { if (act16) ROPE_SCATTER(float, bf16_t); else ROPE_SCATTER(float, float); }
+#undef ROPE_SCATTER
             return hipGetLastError();
         };
         if (skinny) {
             HIPCHK((launch_matvec_rows<0, true, T>(s, w.wqkv, pfX, w.rms_att, pfQkv, ldq, dim, (int)M, ldq, wp.wqkv)));
-            HIPCHK(rope_scatter());
+            HIPCHK(rope_scatter(false));
             HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
             HIPCHK((launch_matvec_rows<1, false, T>(s, w.wo, pfXn, nullptr, pfX, dim, dim, (int)M, dim, wp.wo)));          // x += Wo att
             HIPCHK((launch_matvec_rows<2, true, T>(s, w.w13, pfX, w.rms_ffn, pfHb, hid, dim, (int)M, hid, wp.w13)));
             HIPCHK((launch_matvec_rows<1, false, T>(s, w.w2, pfHb, nullptr, pfX, dim, hid, (int)M, dim, wp.w2)));           // x += W2 hb
             continue;
         }
-        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_att, pfXn, 1e-5f));
-        const float* wqkv = as_f32<T>(s, w.wqkv, (size_t)ldq * dim, &e);
-        if (e) return e;
-        HIPCHK(k_gemm(s, F32, false, true, (int)M, ldq, dim, 1.f, pfXn, wqkv, 0.f, pfQkv));
-        HIPCHK(rope_scatter());
-        HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));   // head-merged output
-        const float* wo = as_f32<T>(s, w.wo, (size_t)dim * dim, &e);
-        if (e) return e;
-        HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, dim, 1.f, pfXn, wo, 1.f, pfX));          // x += Wo att
-        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_ffn, pfXn, 1e-5f));
-        const float* w13 = as_f32<T>(s, w.w13, (size_t)2 * hid * dim, &e);
-        if (e) return e;
-        HIPCHK(k_gemm(s, F32, false, true, (int)M, 2 * hid, dim, 1.f, pfXn, w13, 0.f, pfH2));
-        hipLaunchKernelGGL(prefill_swiglu_kernel, grid_for(M * hid), 256, 0, s, pfH2, pfHb, M, hid);
+        if (mode == PF_F32 || mode == PF_WIDEN) {
+            // fp32 weights - or 16-bit ones of a width the bf16 GEMM does not take, widened one matrix at a time - on
+            // the fp32 MFMA GEMM
+            auto wf = [&](const void* W, size_t n) -> const float* {
+                if (mode == PF_F32) return (const float*)W;
+                const hipError_t ce = k_convert(s, BF16, W, F32, pfW, n);
+                if (ce != hipSuccess) e = (long)ce;
+                return pfW;
+            };
+            HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_att, pfXn, 1e-5f));
+            HIPCHK(k_gemm(s, F32, false, true, (int)M, ldq, dim, 1.f, pfXn, wf(w.wqkv, (size_t)ldq * dim), 0.f, pfQkv));
+            HIPCHK(rope_scatter(false));
+            HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));   // head-merged output
+            HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, dim, 1.f, pfXn, wf(w.wo, (size_t)dim * dim), 1.f, pfX));          // x += Wo att
+            HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, w.rms_ffn, pfXn, 1e-5f));
+            HIPCHK(k_gemm(s, F32, false, true, (int)M, 2 * hid, dim, 1.f, pfXn, wf(w.w13, (size_t)2 * hid * dim), 0.f, pfH2));
+            hipLaunchKernelGGL(prefill_swiglu_kernel, grid_for(M * hid), 256, 0, s, pfH2, pfHb, M, hid);
+            HIPCHK(hipGetLastError());
+            HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, hid, 1.f, pfHb, wf(w.w2, (size_t)dim * hid), 1.f, pfX));          // x += W2 hb
+            if (e) return e;
+            continue;
+        }
+        // 16-bit weights on the bf16 MFMA GEMM, fp32 results and residual stream.  PF_SPLIT: every activation goes in
+        // as two bf16 numbers (k_gemm_bf16_f32, split), attention in fp32.  PF_ACT16: activations rounded to bf16, q / k /
+        // v and the attention in bf16, whose head-merged output is the next GEMM's operand as it is.
+        const bool split = mode == PF_SPLIT;
+        bf16_t* a16 = (bf16_t*)pfW;
+        auto norm16 = [&](const float* x, const float* g, int k) {
+            if (split) hipLaunchKernelGGL(prefill_norm_split_kernel<true>, (int)M, 256, 0, s, x, g, a16, k, 1e-5f);
+            else hipLaunchKernelGGL(prefill_norm_split_kernel<false>, (int)M, 256, 0, s, x, g, a16, k, 1e-5f);
+            return hipGetLastError();
+        };
+        HIPCHK(norm16(pfX, w.rms_att, dim));
+        HIPCHK(k_gemm_bf16_f32(s, (int)M, ldq, dim, 1.f, a16, split, w.wqkv, 0.f, pfQkv));
+        HIPCHK(rope_scatter(!split));
+        if (split) {
+            HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
+            HIPCHK(norm16(pfXn, nullptr, dim));
+        } else {
+            HIPCHK(k_attn_prefill(s, BF16, pfQ, pfK, pfV, a16, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
+        }
+        HIPCHK(k_gemm_bf16_f32(s, (int)M, dim, dim, 1.f, a16, split, w.wo, 1.f, pfX));                               // x += Wo att
+        HIPCHK(norm16(pfX, w.rms_ffn, dim));
+        HIPCHK(k_gemm_bf16_f32(s, (int)M, 2 * hid, dim, 1.f, a16, split, w.w13, 0.f, pfH2));
+        if (split) hipLaunchKernelGGL(prefill_swiglu_split_kernel<true>, grid_for(M * hid / 4), 256, 0, s, pfH2, a16, M, hid);
+        else hipLaunchKernelGGL(prefill_swiglu_split_kernel<false>, grid_for(M * hid / 4), 256, 0, s, pfH2, a16, M, hid);
         HIPCHK(hipGetLastError());
-        const float* w2 = as_f32<T>(s, w.w2, (size_t)dim * hid, &e);
-        if (e) return e;
-        HIPCHK(k_gemm(s, F32, false, true, (int)M, dim, hid, 1.f, pfHb, w2, 1.f, pfX));          // x += W2 hb
+        HIPCHK(k_gemm_bf16_f32(s, (int)M, dim, hid, 1.f, a16, split, w.w2, 1.f, pfX));                               // x += W2 hb
     }
     // The classifier has 250 tiles of 128 x 128 per 128 rows, enough for the tiled GEMM even where the layers' matrices
     // are not: the mat-vec family keeps it only for a handful of rows.
     const bool clsGemm = !skinny || M >= 64;
-    const float* wc = nullptr;
+    const bool cls16 = mode == PF_SPLIT || mode == PF_ACT16;
+    const int a16Row = mode == PF_SPLIT ? 2 * dim : dim;
     if (clsGemm) {
-        HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
-        wc = as_f32<T>(s, wcls, (size_t)V * dim, &e);
-        if (e) return e;
+        if (!cls16) {
+            HIPCHK(k_rmsnorm(s, F32, (int)M, dim, pfX, rms_final, pfXn, 1e-5f));
+            if (mode == PF_WIDEN) HIPCHK(k_convert(s, BF16, wcls, F32, pfW, (size_t)V * dim));
+        } else {
+            if (mode == PF_SPLIT) hipLaunchKernelGGL(prefill_norm_split_kernel<true>, (int)M, 256, 0, s, pfX, rms_final, (bf16_t*)pfW, dim, 1e-5f);
+            else hipLaunchKernelGGL(prefill_norm_split_kernel<false>, (int)M, 256, 0, s, pfX, rms_final, (bf16_t*)pfW, dim, 1e-5f);
+            HIPCHK(hipGetLastError());
+        }
     }
     for (size_t r0 = 0; r0 < M; r0 += pfLogitRows) {
         const int rows = (int)std::min(pfLogitRows, M - r0);
         if (!clsGemm) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V, wclsP)));
-        else HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, wc, 0.f, pfLogits));
+        else if (!cls16) HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, mode == PF_F32 ? wcls : (const void*)pfW, 0.f, pfLogits));
+        else HIPCHK(k_gemm_bf16_f32(s, rows, V, dim, 1.f, (bf16_t*)pfW + r0 * a16Row, mode == PF_SPLIT, wcls, 0.f, pfLogits));
         hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
         HIPCHK(hipGetLastError());
         if (allLogits) {
@@ -1926,6 +2019,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 7) m->engine.use_prefill = pIn[2] != 0.f;
         else if (opt == 8) m->engine.set_kv_bf16(pIn[2] != 0.f);
         else if (opt == 9) m->engine.set_defer_merge(pIn[2] != 0.f);
+        else if (opt == 10) m->engine.prefill_act16 = pIn[2] != 0.f;
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }
