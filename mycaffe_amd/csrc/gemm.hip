@@ -359,13 +359,84 @@ __device__ __forceinline__ T* heads_dst(const HeadsEpilogue& he, int row, int co
     return (T*)he.dst[which] + (((size_t)b * he.H + h) * he.T + t) * he.hs + d;
 }
 
+// Epilogues of the prompt pass of the Llama engine (fp32 results of 16-bit operands; llama2_ext.hip), which save the
+// round trip of the product through memory and the kernel that would read it back:
+//   EPI 1, SwiGLU of the stacked W1 | W3 product.  Tile column c multiplies weight row (c & 1) hid + c / 2, so that a
+//     lane's register quad holds (w1 x, w3 x) of two consecutive hidden units j: out[j] = silu(w1 x) (w3 x), stored as
+//     bf16 (rows of hid), or as the bf16 nearest to it followed, hid further on, by the bf16 nearest to the remainder
+//     (rows of 2 hid: the operand form of k_gemm_bf16_f32's split product).
+//   EPI 2, rotation and scatter of the stacked Wq | Wk | Wv product (row = sequence b, position p): q and k rotated at p
+//     (adjacent pairs, the decode kernel's arithmetic), q / k / v written as (B, H, P, hs) head tensors - fp32 or bf16,
+//     every key / value head repeated for the query heads that share it - and the rotated key and the value appended to
+//     the caches [b][p][kvd] (fp32 or bf16; the head tensors then carry the values the cache holds).
+struct PromptEpilogue {
+    void* out; int hid; int split;                                   // EPI 1
+    void* q; void* k; void* v; void* kc; void* vc;                   // EPI 2
+    const float* fcos; const float* fsin;
+    int P, H, kvH, hs, seqLen, heads16, cache16, kvMul;
+    float invP, invHs;
+};
+__device__ __forceinline__ uint32_t pe_pack(float a, float b) { return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16); }
+__device__ __forceinline__ float pe_round(float a) { return bf16_to_f32(f32_to_bf16(a)); }
+// four consecutive values to a tensor of fp32 or bf16
+__device__ __forceinline__ void pe_store4(void* base, size_t idx, int is16, const float (&v)[4])
+{
+    if (is16) *(uint2*)((bf16_t*)base + idx) = make_uint2(pe_pack(v[0], v[1]), pe_pack(v[2], v[3]));
+    else *(float4*)((float*)base + idx) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void prompt_epilogue_swiglu(const PromptEpilogue& pe, int r, int c, const float (&a)[4])
+{
+    const int j = c >> 1;   // c is a multiple of 4: hidden units j, j + 1
+    float o[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) o[q] = a[2 * q] * (1.0f / (1.0f + expf(-a[2 * q]))) * a[2 * q + 1];
+    bf16_t* row = (bf16_t*)pe.out + (size_t)r * (pe.split ? 2 : 1) * pe.hid;
+    *(uint32_t*)(row + j) = pe_pack(o[0], o[1]);
+    if (pe.split) *(uint32_t*)(row + pe.hid + j) = pe_pack(o[0] - pe_round(o[0]), o[1] - pe_round(o[1]));
+}
+// x / d for 0 <= x < 2^24, d > 0, through the reciprocal (an integer division is some forty instructions)
+__device__ __forceinline__ int pe_div(int x, int d, float inv)
+{
+    int q = (int)((float)x * inv);
+    if ((q + 1) * d <= x) q++;
+    if (q * d > x) q--;
+    return q;
+}
+__device__ __forceinline__ void prompt_epilogue_rope(const PromptEpilogue& pe, int r, int c, const float (&a)[4])
+{
+    const int dim = pe.H * pe.hs, kvd = pe.kvH * pe.hs, kvMul = pe.kvMul, half = pe.hs >> 1;
+    const int b = pe_div(r, pe.P, pe.invP), p = r - b * pe.P;
+    float o[4] = {a[0], a[1], a[2], a[3]};
+    const int which = c < dim ? 0 : c < dim + kvd ? 1 : 2;
+    const int cc = which == 0 ? c : which == 1 ? c - dim : c - dim - kvd;
+    const int h = pe_div(cc, pe.hs, pe.invHs), d = cc - h * pe.hs;
+    if (which < 2) {
+        const float2 cs = *(const float2*)(pe.fcos + (size_t)p * half + (d >> 1)), sn = *(const float2*)(pe.fsin + (size_t)p * half + (d >> 1));
+        o[0] = a[0] * cs.x - a[1] * sn.x; o[1] = a[0] * sn.x + a[1] * cs.x;
+        o[2] = a[2] * cs.y - a[3] * sn.y; o[3] = a[2] * sn.y + a[3] * cs.y;
+    }
+    if (which == 0) {
+        pe_store4(pe.q, (((size_t)b * pe.H + h) * pe.P + p) * pe.hs + d, pe.heads16, o);
+        return;
+    }
+    if (pe.cache16) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) o[q] = pe_round(o[q]);   // the pass attends over the values the cache holds
+    }
+    pe_store4(which == 1 ? pe.kc : pe.vc, ((size_t)b * pe.seqLen + p) * kvd + cc, pe.cache16, o);
+    for (int g = 0; g < kvMul; g++)
+        pe_store4(which == 1 ? pe.k : pe.v, (((size_t)b * pe.H + h * kvMul + g) * pe.P + p) * pe.hs + d, pe.heads16, o);
+}
+
 // SPLIT (16-bit operands, fp32 C): a row of A is 2 K long, the upper halves of K fp32 values followed by what the upper
 // halves leave over (see k_gemm_bf16_split), and B is walked twice: C = alpha (A_hi + A_lo) B^T + beta C.
-template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false>
+template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false, int EPI = 0>
 __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
                                                                const T* __restrict__ B, float beta, TC* __restrict__ C, int tilesN,
-                                                               int tilesTotal, int bandRows, int colBlock, HeadsEpilogue he)
+                                                               int tilesTotal, int bandRows, int colBlock, HeadsEpilogue he,
+                                                               PromptEpilogue pe)
 {
+    static_assert(EPI == 0 || !std::is_same<T, TC>::value, "the prompt epilogues take the fp32 results of 16-bit operands");
     static_assert(std::is_same<T, TC>::value || (!HEADS && std::is_same<TC, float>::value), "C is of the operands' type, or fp32");
     static_assert(!SPLIT || !std::is_same<T, TC>::value, "the split product writes fp32");
     typedef BigTraits<T> TR;
@@ -417,7 +488,10 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
 #pragma unroll
     for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * (SPLIT ? 2 * K : K) + lc;
 #pragma unroll
-    for (int p = 0; p < PB; p++) gb[p] = B + (size_t)min(n0 + lr + p * RPP, N - 1) * K + lc;
+    for (int p = 0; p < PB; p++) {
+        const int c = min(n0 + lr + p * RPP, N - 1);
+        gb[p] = B + (size_t)(EPI == 1 ? (c & 1) * pe.hid + (c >> 1) : c) * K + lc;
+    }
     T* sa = As + lr * LDK + lc;
     T* sb = Bs + lr * LDK + lc;
     u32x4 ra[PA], rb[PB];
@@ -503,33 +577,53 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     // register quad.
     const int row_l = lane & 31, col_l = (lane >> 5) * 4;
     if constexpr (!std::is_same<T, TC>::value) {
-        // fp32 C from 16-bit operands: a lane's register quad is four consecutive columns of its row, one 16-byte access
+        // fp32 results of 16-bit operands.  A lane owns a row of the tile, so its own stores would be 16 bytes each in 32
+        // different rows; each wavefront passes its tile, 32 rows at a time, through its own slice of LDS (free after
+        // the last barrier) and the lanes then walk the rows: consecutive lanes take consecutive quads of columns, and
+        // whatever the epilogue stores is contiguous along the row.
+        constexpr int CW = 32 * WN, LDC = CW + 4;
+        constexpr int LPR = CW / 4, RPI = 64 / LPR;             // lanes per row, rows per pass
+        constexpr int NIT = (32 + RPI - 1) / RPI;
+        float* cs = reinterpret_cast<float*>(smem_raw) + wave * 32 * LDC;
+        const int rr = lane / LPR, cc = (lane % LPR) * 4;
         const bool vec4 = (N & 3) == 0 && (((uintptr_t)C) & 15) == 0;
 #pragma unroll
-        for (int i = 0; i < WM; i++)
+        for (int i = 0; i < WM; i++) {
 #pragma unroll
-            for (int j = 0; j < WN; j++) {
-                const int r = m0 + wm + i * 32 + row_l;
-                if (r >= M) continue;
+            for (int j = 0; j < WN; j++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int c = n0 + wn + j * 32 + 8 * g + col_l;
-                    float* cp = C + (size_t)r * N + c;
-                    if (vec4 && c + 3 < N) {
-                        float4 o = make_float4(alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1], alpha * acc[i][j][4 * g + 2],
-                                               alpha * acc[i][j][4 * g + 3]);
-                        if (beta != 0.f) {
-                            const float4 old = *(const float4*)cp;
-                            o.x += beta * old.x; o.y += beta * old.y; o.z += beta * old.z; o.w += beta * old.w;
-                        }
-                        *(float4*)cp = o;
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; q++)
-                            if (c + q < N) cp[q] = alpha * acc[i][j][4 * g + q] + (beta != 0.f ? beta * cp[q] : 0.f);
+                for (int g = 0; g < 4; g++)
+                    *(float4*)(cs + row_l * LDC + j * 32 + 8 * g + col_l) =
+                        make_float4(alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1], alpha * acc[i][j][4 * g + 2], alpha * acc[i][j][4 * g + 3]);
+            // same wavefront wrote and reads: LDS operations of one wavefront complete in order
+#pragma unroll 4
+            for (int it = 0; it < NIT; it++) {
+                const int row = it * RPI + rr, r = m0 + wm + i * 32 + row, c = n0 + wn + cc;
+                if (rr >= RPI || row >= 32 || r >= M || c >= N) continue;
+                const float4 v = *(const float4*)(cs + row * LDC + cc);
+                if (EPI != 0) {
+                    // N is a multiple of 4 here: a quad is inside the matrix or outside it
+                    const float a4[4] = {v.x, v.y, v.z, v.w};
+                    if (EPI == 1) prompt_epilogue_swiglu(pe, r, c, a4);
+                    else prompt_epilogue_rope(pe, r, c, a4);
+                    continue;
+                }
+                float* cp = C + (size_t)r * N + c;
+                if (vec4 && c + 3 < N) {
+                    float4 o = v;
+                    if (beta != 0.f) {
+                        const float4 old = *(const float4*)cp;
+                        o.x += beta * old.x; o.y += beta * old.y; o.z += beta * old.z; o.w += beta * old.w;
                     }
+                    *(float4*)cp = o;
+                } else {
+                    const float a4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (c + q < N) cp[q] = a4[q] + (beta != 0.f ? beta * cp[q] : 0.f);
                 }
             }
+        }
         return;
     } else
     if (m0 + BM <= M && n0 + BN <= N && (HEADS || (beta == 0.f && (((uintptr_t)C) & 15) == 0)) && (N % E) == 0) {
@@ -595,10 +689,12 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     }
 }
 
-template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false>
+template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false, int EPI = 0>
 static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C,
-                             const HeadsEpilogue* heads = nullptr)
+                             const HeadsEpilogue* heads = nullptr, const PromptEpilogue* prompt = nullptr)
 {
+    PromptEpilogue pe = {};
+    if (prompt) pe = *prompt;
     HeadsEpilogue he = {};
     if (heads) he = *heads;
     constexpr int E = BigTraits<T>::E;
@@ -607,11 +703,11 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
     if (total > (1ll << 30)) return hipErrorInvalidValue;
     const int per = (int)((total + 7) / 8);
     size_t lds = (size_t)2 * (64 * WM + 64 * WN) * (9 * E) * sizeof(T);
-    const size_t ldsEpilogue = (size_t)4 * 32 * (32 * WN + E) * sizeof(T);
+    const size_t ldsEpilogue = std::is_same<T, TC>::value ? (size_t)4 * 32 * (32 * WN + E) * sizeof(T) : (size_t)4 * 32 * (32 * WN + 4) * sizeof(float);
     if (ldsEpilogue > lds) lds = ldsEpilogue;
     static bool attr = false;   // per instantiation: allow more than the default 64 KB of dynamic LDS
     if (!attr) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         attr = true;
     }
@@ -627,8 +723,8 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
             colBlock = (tn + nb - 1) / nb;   // equal-width blocks
         }
     }
-    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
-                       (TC*)C, tn, (int)total, bandRows, colBlock, he);
+    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT, EPI>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
+                       (TC*)C, tn, (int)total, bandRows, colBlock, he, pe);
     return hipGetLastError();
 }
 
@@ -930,25 +1026,52 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
 // those leave over, and the kernel walks W once for each.  The products are exact and accumulate in fp32, so what is lost
 // is the part of X below its leading sixteen bits: 2^-17 relative, against 2^-9 for activations rounded to bf16.
 // k a multiple of 64, 16-byte aligned operands.
-template <bool SPLIT>
-static hipError_t gemm_bf16_f32_tiles(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* W, float beta, float* C)
+template <bool SPLIT, int EPI>
+static hipError_t gemm_bf16_f32_tiles(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* W, float beta, float* C,
+                                      const PromptEpilogue* pe)
 {
     // Tile shapes as k_gemm picks them for bf16: below 200 tiles of 128 x 128, 64 x 128 tiles where they give every CU
     // one, else 64 x 64 (2048 x 768: 384 tiles of 64 x 64 measure 27.8 us a product, 192 of 64 x 128 30.1 us).
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
     if (t128 < 200) {
         const long long t64x128 = (long long)((m + 63) / 64) * ((n + 127) / 128);
-        if (t64x128 >= 200) return launch_big<bf16_t, 1, 2, 3, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
-        return launch_big<bf16_t, 1, 1, 3, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+        if (t64x128 >= 200) return launch_big<bf16_t, 1, 2, 3, false, float, SPLIT, EPI>(s, m, n, k, alpha, A, W, beta, C, nullptr, pe);
+        return launch_big<bf16_t, 1, 1, 3, false, float, SPLIT, EPI>(s, m, n, k, alpha, A, W, beta, C, nullptr, pe);
     }
-    if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
-    return launch_big<bf16_t, 2, 2, 2, false, float, SPLIT>(s, m, n, k, alpha, A, W, beta, C);
+    if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, false, float, SPLIT, EPI>(s, m, n, k, alpha, A, W, beta, C, nullptr, pe);
+    return launch_big<bf16_t, 2, 2, 2, false, float, SPLIT, EPI>(s, m, n, k, alpha, A, W, beta, C, nullptr, pe);
 }
+static bool bf16_f32_operands_ok(int k, const void* A, const void* W) { return k > 0 && k % 64 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0; }
 hipError_t k_gemm_bf16_f32(hipStream_t s, int m, int n, int k, float alpha, const void* A, bool split, const void* W, float beta, float* C)
 {
     if (m <= 0 || n <= 0) return hipSuccess;
-    if (k <= 0 || k % 64 != 0 || (((uintptr_t)A | (uintptr_t)W) & 15) != 0) return hipErrorInvalidValue;
-    return split ? gemm_bf16_f32_tiles<true>(s, m, n, k, alpha, A, W, beta, C) : gemm_bf16_f32_tiles<false>(s, m, n, k, alpha, A, W, beta, C);
+    if (!bf16_f32_operands_ok(k, A, W)) return hipErrorInvalidValue;
+    return split ? gemm_bf16_f32_tiles<true, 0>(s, m, n, k, alpha, A, W, beta, C, nullptr) : gemm_bf16_f32_tiles<false, 0>(s, m, n, k, alpha, A, W, beta, C, nullptr);
+}
+// out (m x hid) = silu(X W1^T) (X W3^T) for the stacked 16-bit W13 (2 hid x k), as bf16 rows (outSplit: hi | lo rows)
+hipError_t k_gemm_bf16_swiglu(hipStream_t s, int m, int hid, int k, const void* A, bool split, const void* W13, void* out, bool outSplit)
+{
+    if (m <= 0 || hid <= 0) return hipSuccess;
+    if (!bf16_f32_operands_ok(k, A, W13) || (hid & 1) || (((uintptr_t)out) & 3)) return hipErrorInvalidValue;
+    PromptEpilogue pe = {};
+    pe.out = out; pe.hid = hid; pe.split = outSplit ? 1 : 0;
+    return split ? gemm_bf16_f32_tiles<true, 1>(s, m, 2 * hid, k, 1.f, A, W13, 0.f, nullptr, &pe) : gemm_bf16_f32_tiles<false, 1>(s, m, 2 * hid, k, 1.f, A, W13, 0.f, nullptr, &pe);
+}
+// the stacked 16-bit Wqkv ((H + 2 kvH) hs x k) product of B x P rows, rotated and scattered (PromptEpilogue, EPI 2)
+hipError_t k_gemm_bf16_qkv_rope(hipStream_t s, int B, int P, int H, int kvH, int hs, int k, const void* A, bool split, const void* Wqkv,
+                                void* q, void* kh, void* vh, bool heads16, void* kc, void* vc, bool cache16, int seqLen,
+                                const float* fcos, const float* fsin)
+{
+    const int m = B * P, n = (H + 2 * kvH) * hs;
+    if (m <= 0 || n <= 0) return hipSuccess;
+    if (!bf16_f32_operands_ok(k, A, Wqkv) || (hs & 3) || kvH <= 0 || H % kvH != 0) return hipErrorInvalidValue;
+    if ((((uintptr_t)q | (uintptr_t)kh | (uintptr_t)vh | (uintptr_t)kc | (uintptr_t)vc) & 15) != 0) return hipErrorInvalidValue;
+    PromptEpilogue pe = {};
+    pe.q = q; pe.k = kh; pe.v = vh; pe.kc = kc; pe.vc = vc; pe.fcos = fcos; pe.fsin = fsin;
+    pe.P = P; pe.H = H; pe.kvH = kvH; pe.hs = hs; pe.seqLen = seqLen; pe.heads16 = heads16 ? 1 : 0; pe.cache16 = cache16 ? 1 : 0;
+    pe.kvMul = H / kvH; pe.invP = 1.0f / (float)P; pe.invHs = 1.0f / (float)hs;
+    if (m >= (1 << 24) || n >= (1 << 24)) return hipErrorInvalidValue;
+    return split ? gemm_bf16_f32_tiles<true, 2>(s, m, n, k, 1.f, A, Wqkv, 0.f, nullptr, &pe) : gemm_bf16_f32_tiles<false, 2>(s, m, n, k, 1.f, A, Wqkv, 0.f, nullptr, &pe);
 }
 
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,

@@ -107,6 +107,12 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
 // C (fp32) = alpha X W^T + beta C on the bf16 matrix cores: W 16-bit (n x k), k % 64 == 0; A is X as bf16 (m x k) or,
 // split, every row of X as two bf16 rows (nearest bf16, then the bf16 nearest to the remainder; m x 2k)
 hipError_t k_gemm_bf16_f32(hipStream_t s, int m, int n, int k, float alpha, const void* A, bool split, const void* W, float beta, float* C);
+// the same product with the epilogues of the Llama prompt pass: SwiGLU of the stacked W1 | W3 (bf16 rows of hid, or hi | lo
+// rows of 2 hid), and rotation + scatter of the stacked Wq | Wk | Wv into head tensors and caches (gemm.hip, PromptEpilogue)
+hipError_t k_gemm_bf16_swiglu(hipStream_t s, int m, int hid, int k, const void* A, bool split, const void* W13, void* out, bool outSplit);
+hipError_t k_gemm_bf16_qkv_rope(hipStream_t s, int B, int P, int H, int kvH, int hs, int k, const void* A, bool split, const void* Wqkv,
+                                void* q, void* kh, void* vh, bool heads16, void* kc, void* vc, bool cache16, int seqLen,
+                                const float* fcos, const float* fsin);
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
                    int batch);

@@ -774,20 +774,6 @@ __global__ __launch_bounds__(256) void prefill_norm_split_kernel(const float* __
         split_store4<LO>(orow, n, i, v);
     }
 }
-// out[m] = split(silu(h2[m, j]) * h2[m, hid + j]), hid a multiple of 4
-template <bool LO>
-__global__ void prefill_swiglu_split_kernel(const float* __restrict__ h2, bf16_t* __restrict__ out, size_t rows, int hid)
-{
-    const size_t total = rows * hid / 4;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
-        const size_t m = i * 4 / hid;
-        const int j = (int)(i * 4 - m * hid);
-        const float4 a0 = *(const float4*)(h2 + m * 2 * hid + j), a1 = *(const float4*)(h2 + m * 2 * hid + hid + j);
-        auto f = [](float a, float b) { return a * (1.0f / (1.0f + expf(-a))) * b; };
-        split_store4<LO>(out + m * (LO ? 2 : 1) * hid, hid, j, make_float4(f(a0.x, a1.x), f(a0.y, a1.y), f(a0.z, a1.z), f(a0.w, a1.w)));
-    }
-}
-
 // First-max argmax of every logits row (sample_argmax, llama2_sampler.cpp:25-36), one workgroup per row: the id
 // chosen after prompt position p of sequence b goes to out_ids[b][p]; the one after the last prefilled position is
 // also the token the first decode step starts from (next[b]).
@@ -1374,8 +1360,9 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
             return hipGetLastError();
         };
         HIPCHK(norm16(pfX, w.rms_att, dim));
-        HIPCHK(k_gemm_bf16_f32(s, (int)M, ldq, dim, 1.f, a16, split, w.wqkv, 0.f, pfQkv));
-        HIPCHK(rope_scatter(!split));
+        // rotation, head tensors and cache rows leave the QKV product's epilogue
+        HIPCHK(k_gemm_bf16_qkv_rope(s, B, P, H, kvH, hs, dim, a16, split, w.wqkv, pfQ, pfK, pfV, !split, kcl, vcl, state_kv_bf16, cfg.seq_len,
+                                    fcos, fsin));
         if (split) {
             HIPCHK(k_attn_prefill(s, F32, pfQ, pfK, pfV, pfXn, B, H, P, P, hs, scale, nullptr, MASK_CAUSAL, nullptr, true));
             HIPCHK(norm16(pfXn, nullptr, dim));
@@ -1384,11 +1371,9 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         }
         HIPCHK(k_gemm_bf16_f32(s, (int)M, dim, dim, 1.f, a16, split, w.wo, 1.f, pfX));                               // x += Wo att
         HIPCHK(norm16(pfX, w.rms_ffn, dim));
-        HIPCHK(k_gemm_bf16_f32(s, (int)M, 2 * hid, dim, 1.f, a16, split, w.w13, 0.f, pfH2));
-        if (split) hipLaunchKernelGGL(prefill_swiglu_split_kernel<true>, grid_for(M * hid / 4), 256, 0, s, pfH2, a16, M, hid);
-        else hipLaunchKernelGGL(prefill_swiglu_split_kernel<false>, grid_for(M * hid / 4), 256, 0, s, pfH2, a16, M, hid);
-        HIPCHK(hipGetLastError());
-        HIPCHK(k_gemm_bf16_f32(s, (int)M, dim, hid, 1.f, a16, split, w.w2, 1.f, pfX));                               // x += W2 hb
+        // silu(w1 x) (w3 x) leaves the W1 | W3 product's epilogue in the operand form of the next product
+        HIPCHK(k_gemm_bf16_swiglu(s, (int)M, hid, dim, a16, split, w.w13, pfH2, split));
+        HIPCHK(k_gemm_bf16_f32(s, (int)M, dim, hid, 1.f, pfH2, split, w.w2, 1.f, pfX));                              // x += W2 hb
     }
     // The classifier has 250 tiles of 128 x 128 per 128 rows, enough for the tiled GEMM even where the layers' matrices
     // are not: the mat-vec family keeps it only for a handful of rows.
