@@ -281,7 +281,12 @@ enum {
      *                 multiples of 64) keeps its activations to sixteen leading bits - two bf16 numbers a
      *                 value on the bf16 matrix cores, attention in fp32: logits within the fp32 bar of the
      *                 step-per-position loop (0, default) - or rounds them to bf16 and runs the attention
-     *                 in bf16 (1: half the matrix-core work, logits within the 16-bit bar)
+     *                 in bf16 (1: half the matrix-core work, logits within the 16-bit bar); option 11 = where
+     *                 a sampler with a temperature above 0 runs: on the device (1, default: softmax, the
+     *                 xorshift64* coin and the top-p / multinomial choice in one kernel per step, so the
+     *                 steps replay as a captured graph; the id can differ from the host's only where the
+     *                 coin falls within rounding of an edge of the cumulative distribution) or on the host
+     *                 after a copy of the logits, as llama2_gpu.cpp:108 and llama2_sampler.cpp do it (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}
      *                 -> f{batch x nSteps next ids [, logits with option 6]}
      *   QUERY_TIMING  f{hLlm} -> f{ms of the timed span (HIP events), steps in it, 1 if the steps were

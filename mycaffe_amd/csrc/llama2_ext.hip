@@ -588,7 +588,8 @@ template <typename T>
 __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __restrict__ logits, int V, GenState* st, int* ticket,
                                                                const int* __restrict__ prompt, int promptStride, int* next,
                                                                int* out_ids, const T* __restrict__ emb, float* __restrict__ x,
-                                                               int dim, int* cur, const int* __restrict__ given)
+                                                               int dim, int* cur, const int* __restrict__ given,
+                                                               unsigned long long* rng = nullptr)
 {
     __shared__ float sv[16];
     __shared__ int si[16];
@@ -649,8 +650,215 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
             if (gridDim.x > 1) *ticket = 0;
             st->pos = pos + 1;
             st->len = pos + 2;
+            if (rng) {
+                // the device sampler drew one coin per sequence from this step's state (sample_device_kernel)
+                unsigned long long r = *rng;
+                for (unsigned int d = 0; d < gridDim.x; d++) {
+                    r ^= r >> 12;
+                    r ^= r << 25;
+                    r ^= r >> 27;
+                }
+                *rng = r;
+            }
         }
     }
+}
+
+// ---------------------------------------------------------------------------
+// Temperature / top-p sampling on the device (sample, llama2_sampler.cpp:126-151, with sample_mult :38-49 and
+// sample_topp :59-100), one workgroup of 1024 threads per sequence, so that a sampled generation needs no copy of the
+// logits to the host.  The reference's arithmetic is sequential - the softmax denominator and the cumulative sums are
+// running fp32 sums in index order and in sorted order - and with a flat distribution the rounding of those sums moves
+// the chosen id as often as one time in five, so it is kept: what can run in parallel does (maximum, exponentials,
+// division, the sort), the running sums are walked by one lane over LDS in the reference's order.
+//   * The coin is the reference's: xorshift64* (:115-124) on a state kept in device memory; sequence b of a step takes
+//     draw b + 1 from the step's state (the reference flips one coin per forward call, forced positions included), and
+//     the step's tail kernel moves the state on by one draw per sequence.
+//   * exp is taken in double and rounded to float: the host library's expf is correctly rounded for all but a handful of
+//     arguments, the device's single-precision one is not.
+//   * The logits are overwritten by the probabilities, as in the reference.
+//   * Top-p: the candidates (probability >= (1 - topp) / (n - 1)) are gathered in LDS and sorted by value (bitonic,
+//     descending); the order among equal values does not change a sum, only which index a position stands for, and
+//     that is settled afterwards: the m-th of the equal values in the sorted list is the m-th of them by index.
+// Up to 32768 logits (128 KB of LDS); the engine samples longer vocabularies on the host.
+__device__ __forceinline__ unsigned long long xorshift64_next(unsigned long long st)
+{
+    st ^= st >> 12;
+    st ^= st << 25;
+    st ^= st >> 27;
+    return st;
+}
+struct WgScratch { float f[16]; int i[16]; };
+__device__ __forceinline__ float wg_max_1024(float v, WgScratch& sc)
+{
+    v = group_max<64>(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sc.f[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = sc.f[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) t = fmaxf(t, sc.f[w]);
+    return t;
+}
+__device__ __forceinline__ int wg_exclusive_scan_int_1024(int v, WgScratch& sc)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += up;
+    }
+    __syncthreads();
+    if (lane == 63) sc.i[wave] = inc;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; w++) base += sc.i[w];
+    return base + inc - v;
+}
+constexpr int SAMPLE_MAX_VOCAB = 32768;
+// One lane's running sum over buf[0 .. n) in order: acc += buf[i], stopping at the first i where exceeds(acc) holds.
+// Returns that i (n if none) and leaves the sum reached in acc.  The values are not negative, so the sum never falls and
+// `exceeds` - a threshold on it - only has to be asked once per batch of 32 additions; the batch in which it first holds
+// is gone through again.  That leaves one dependent addition per value, and the LDS latency is paid once per batch.
+template <typename F> __device__ __forceinline__ int running_sum_until(const float* buf, int n, float& acc, F exceeds)
+{
+    int i = 0;
+    for (; i + 32 <= n; i += 32) {
+        float4 q[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) q[u] = *(const float4*)(buf + i + 4 * u);
+        float t = acc;
+#pragma unroll
+        for (int u = 0; u < 8; u++) { t += q[u].x; t += q[u].y; t += q[u].z; t += q[u].w; }
+        if (exceeds(t)) break;
+        acc = t;
+    }
+    for (; i < n; i++) {
+        acc += buf[i];
+        if (exceeds(acc)) return i;
+    }
+    return n;
+}
+__global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__ logits, int V, float temperature, float topp,
+                                                             const unsigned long long* __restrict__ rng, int* __restrict__ given)
+{
+    extern __shared__ __attribute__((aligned(16))) float sbuf[];   // V values in index order, later the sorted candidates
+    __shared__ WgScratch sc;
+    __shared__ float sval[2];
+    __shared__ int sint[4];
+    const int tid = threadIdx.x, b = blockIdx.x;
+    float* p = logits + (size_t)b * V;
+    // the coin: draw b + 1 of the step's state (:115-124)
+    unsigned long long st = *rng;
+    for (int d = 0; d <= b; d++) st = xorshift64_next(st);
+    const float coin = (float)((unsigned int)((st * 0x2545F4914F6CDD1Dull) >> 32) >> 8) / 16777216.0f;
+    // probabilities (:131-135; softmax, llama2_cpu.cpp): maximum, exponentials, their sum in index order, division
+    float mx = -INFINITY;
+    for (int i = tid; i < V; i += 1024) {
+        const float v = p[i] / temperature;
+        sbuf[i] = v;
+        mx = fmaxf(mx, v);
+    }
+    mx = wg_max_1024(mx, sc);
+    for (int i = tid; i < V; i += 1024) sbuf[i] = (float)exp((double)(sbuf[i] - mx));
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.f;
+        running_sum_until(sbuf, V, sum, [](float) { return false; });
+        sval[0] = sum;
+    }
+    __syncthreads();
+    const float sum = sval[0];
+    for (int i = tid; i < V; i += 1024) {
+        const float q = sbuf[i] / sum;
+        sbuf[i] = q;
+        p[i] = q;
+    }
+    __syncthreads();
+    if (topp <= 0.f || topp >= 1.f) {
+        // sample_mult: the first index whose running sum exceeds the coin, else the last one
+        if (tid == 0) {
+            float cdf = 0.f;
+            const int hit = running_sum_until(sbuf, V, cdf, [coin](float c) { return coin < c; });
+            given[b] = hit < V ? hit : V - 1;
+        }
+        return;
+    }
+    // candidates into LDS, in any order (this thread's values are in registers of a sort: re-read from memory)
+    const float cutoff = (1.0f - topp) / (float)(V - 1);
+    if (tid == 0) sint[0] = 0;
+    __syncthreads();   // everybody has read its part of the index-ordered values above; the buffer is rewritten now
+    float mine[SAMPLE_MAX_VOCAB / 1024];
+#pragma unroll
+    for (int j = 0; j < SAMPLE_MAX_VOCAB / 1024; j++) {
+        const int i = j * 1024 + tid;
+        mine[j] = i < V ? sbuf[i] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SAMPLE_MAX_VOCAB / 1024; j++)
+        if (mine[j] >= cutoff && j * 1024 + tid < V) sbuf[atomicAdd(&sint[0], 1)] = mine[j];
+    __syncthreads();
+    const int n0 = sint[0];
+    if (n0 == 0) {
+        // the reference would index in front of its list; the largest probability (lowest index) is the sane answer
+        float best = 0.f;
+        for (int i = tid; i < V; i += 1024) best = fmaxf(best, p[i]);
+        best = wg_max_1024(best, sc);
+        if (tid == 0) sint[1] = 0x7fffffff;
+        __syncthreads();
+        for (int i = tid; i < V; i += 1024)
+            if (p[i] == best) atomicMin(&sint[1], i);
+        __syncthreads();
+        if (tid == 0) given[b] = sint[1];
+        return;
+    }
+    int n2 = 1;
+    while (n2 < n0) n2 <<= 1;
+    for (int i = n0 + tid; i < n2; i += 1024) sbuf[i] = 0.f;   // padding sorts behind every candidate
+    __syncthreads();
+    // bitonic sort, descending
+    for (int k = 2; k <= n2; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int t = tid; t < (n2 >> 1); t += 1024) {
+                const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1)), hi = lo | j;
+                const float x = sbuf[lo], y = sbuf[hi];
+                const bool desc = (lo & k) == 0;
+                if (desc ? x < y : x > y) { sbuf[lo] = y; sbuf[hi] = x; }
+            }
+            __syncthreads();
+        }
+    // end of the nucleus (:78-87) and the sampled position (:89-99), running sums in sorted order
+    if (tid == 0) {
+        float cum = 0.f;
+        int last = running_sum_until(sbuf, n0, cum, [topp](float c) { return c > topp; });
+        if (last == n0) last = n0 - 1;
+        const float r = coin * cum;
+        float cdf = 0.f;
+        int pos = running_sum_until(sbuf, last + 1, cdf, [r](float c) { return r < c; });
+        if (pos > last) pos = last;
+        // the position stands for the m-th (by index) of the candidates that share its value
+        const float v = sbuf[pos];
+        int first = pos;
+        while (first > 0 && sbuf[first - 1] == v) first--;
+        sval[1] = v;
+        sint[2] = pos - first + 1;
+        sint[3] = -1;
+    }
+    __syncthreads();
+    const float v = sval[1];
+    const int m = sint[2];
+    const int chunk = (V + 1023) / 1024, i0 = min(tid * chunk, V), i1 = min(i0 + chunk, V);
+    int cnt = 0;
+    for (int i = i0; i < i1; i++) cnt += p[i] == v ? 1 : 0;
+    const int before = wg_exclusive_scan_int_1024(cnt, sc);
+    if (before < m && m <= before + cnt) {
+        int k = before;
+        for (int i = i0; i < i1; i++)
+            if (p[i] == v && ++k == m) sint[3] = i;
+    }
+    __syncthreads();
+    if (tid == 0) given[b] = sint[3];
 }
 
 // ---------------------------------------------------------------------------
@@ -942,6 +1150,7 @@ public:
     bool lastUsedGraph = false;  // whether the last generate replayed a captured graph (false: eager launches)
     bool use_prefill = true;     // prompt positions as one batched pass (false: one decode step per position)
     bool prefill_act16 = false;  // 16-bit weights, many prompt rows: activations of the pass rounded to bf16 (false: kept to sixteen bits)
+    bool device_sampling = true; // temperature / top-p on the device (false: logits to the host every step)
     bool kv_bf16 = false;        // caches stored as bf16 (option 8; takes effect when the run state is next allocated)
     bool state_kv_bf16 = false;  // what the allocated caches hold
     void set_kv_bf16(bool on) { kv_bf16 = on; if (on != state_kv_bf16) { stateB = -1; graphB = -1; } }
@@ -967,7 +1176,8 @@ public:
 
 private:
     template <typename T> long upload(const float* blob);
-    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr, bool deviceArgmax = true);
+    // tail: 1 = first-max argmax on the device, 0 = stop at the logits (the host samples), 2 = temperature / top-p on the device
+    template <typename T> long step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof = nullptr, int tail = 1);
     template <typename T> long advance_given(hipStream_t s, int B);
     long ensure_state(int B, int nSteps);
     long ensure_prefill(size_t rows);
@@ -1004,7 +1214,10 @@ private:
     int *dcount = nullptr, *dticket = nullptr;   // attention merge tickets (B * heads) and the step ticket; zero between launches
     hipGraphExec_t graphExec = nullptr;
     int graphB = 0;
-    bool graphArgmax = true;                     // whether the captured step ends with the device argmax
+    int graphTail = 1;                           // the tail the captured step ends with (see step), and the sampler
+    float graphTemperature = 0.f, graphTopp = 0.f;   // parameters captured with tail 2
+    float sampleTemperature = 1.f, sampleTopp = 0.9f;
+    unsigned long long* drng = nullptr;          // state of the device sampler's random stream
     int* dgiven = nullptr;                       // ids chosen by the host sampler (one per sequence)
     int hostNPrompt = 0;                         // prompt length of the running generation
     float* hLogits = nullptr; int* hGiven = nullptr; size_t hLogitsCount = 0;   // pinned staging of the sampled path
@@ -1240,6 +1453,7 @@ long Engine::ensure_state(int B, int nSteps)
     dnext = (int*)sa(B * 4);
     dcur = (int*)sa(B * 4);
     dgiven = (int*)sa(B * 4);
+    drng = (unsigned long long*)sa(8);
     dout = (int*)sa((size_t)B * cfg.seq_len * 4);
     dcount = (int*)sa(((size_t)B * cfg.n_heads + 1) * 4);
     if (!x || !xb || !qkv || !qc || !hb || !logits || !kc || !vc || !ws || !dstate || !dprompt || !dnext || !dcur || !dout || !dcount)
@@ -1517,7 +1731,7 @@ hipError_t Engine::embed_first(hipStream_t s, int B)
 }
 
 // enqueue one decode step for B sequences at the device-side position
-template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof, bool deviceArgmax)
+template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float* allLogits, StepProfile* prof, int tail)
 {
     const int dim = cfg.dim, hid = cfg.hidden_dim, hs = dim / cfg.n_heads, kvd = hs * cfg.n_kv_heads, V = cfg.vocab_size;
     const int ldq = dim + 2 * kvd;
@@ -1566,10 +1780,26 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
                            dstate, V, nSteps);
         HIPCHK(hipGetLastError());
     }
-    if (deviceArgmax) {
+    if (tail == 1) {
         SPAN_BEGIN(SC_SAMPLE);
         hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
-                           (const T*)emb, x, dim, dcur, (const int*)nullptr);
+                           (const T*)emb, x, dim, dcur, (const int*)nullptr, (unsigned long long*)nullptr);
+        HIPCHK(hipGetLastError());
+        SPAN_END();
+    } else if (tail == 2) {
+        SPAN_BEGIN(SC_SAMPLE);
+        {
+            static bool attr = false;   // 128 KB of dynamic LDS
+            if (!attr) {
+                HIPCHK(hipFuncSetAttribute((const void*)sample_device_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SAMPLE_MAX_VOCAB * 4));
+                attr = true;
+            }
+        }
+        hipLaunchKernelGGL(sample_device_kernel, B, 1024, SAMPLE_MAX_VOCAB * 4, s, logits, V, sampleTemperature, sampleTopp,
+                           (const unsigned long long*)drng, dgiven);
+        HIPCHK(hipGetLastError());
+        hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
+                           (const T*)emb, x, dim, dcur, (const int*)dgiven, drng);
         HIPCHK(hipGetLastError());
         SPAN_END();
     }
@@ -1582,7 +1812,7 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
 template <typename T> long Engine::advance_given(hipStream_t s, int B)
 {
     hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, cfg.vocab_size, dstate, dticket, dprompt, cfg.seq_len, dnext,
-                       dout, (const T*)emb, x, cfg.dim, dcur, (const int*)dgiven);
+                       dout, (const T*)emb, x, cfg.dim, dcur, (const int*)dgiven, (unsigned long long*)nullptr);
     HIPCHK(hipGetLastError());
     return 0;
 }
@@ -1691,7 +1921,15 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     float* const allLogits = sc.allLogits;
     // With a sampler whose temperature is not 0 the id of every step is chosen on the host, as in the reference: the
     // step's kernels stop at the logits, which are copied out, sampled, and the chosen id goes back for the step's tail.
-    const bool hostSample = sampler && !sampler->greedy();
+    const bool sampled = sampler && !sampler->greedy();
+    const bool devSample = sampled && device_sampling && cfg.vocab_size <= SAMPLE_MAX_VOCAB, hostSample = sampled && !devSample;
+    const int tail = hostSample ? 0 : devSample ? 2 : 1;
+    if (devSample) {
+        sampleTemperature = sampler->temperature;
+        sampleTopp = sampler->topp;
+        HIPCHK(hipMemcpyAsync(drng, &sampler->state, 8, hipMemcpyHostToDevice, stream));
+        HIPCHK(hipStreamSynchronize(stream));
+    }
     const size_t V = (size_t)cfg.vocab_size;
     if (hostSample) {
         if (hLogitsCount < (size_t)B * V) {
@@ -1703,15 +1941,15 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         if (!hGiven) HIPCHK(hipHostMalloc((void**)&hGiven, 64 * sizeof(int), hipHostMallocDefault));
     }
     auto enqueue = [&]() -> long {
-        return stored_bf16 ? step<bf16_t>(s, B, nSteps, allLogits, nullptr, !hostSample)
-                            : step<float>(s, B, nSteps, allLogits, nullptr, !hostSample);
+        return stored_bf16 ? step<bf16_t>(s, B, nSteps, allLogits, nullptr, tail)
+                            : step<float>(s, B, nSteps, allLogits, nullptr, tail);
     };
     HIPCHK(hipEventCreate(&sc.evA));
     HIPCHK(hipEventCreate(&sc.evB));
     const hipEvent_t evA = sc.evA, evB = sc.evB;
     const int t0 = timedFrom < 0 ? nPrompt : timedFrom;
     bool graph = use_graph && !wantLogits;
-    if (graph && (!graphExec || graphB != B || graphArgmax != !hostSample)) {
+    if (graph && (!graphExec || graphB != B || graphTail != tail || (tail == 2 && (graphTemperature != sampleTemperature || graphTopp != sampleTopp)))) {
         // one decode step, captured once; position / tokens are device-side so the graph is replayed as is
         if (graphExec) { (void)hipGraphExecDestroy(graphExec); graphExec = nullptr; }
         hipGraph_t g = nullptr;
@@ -1724,13 +1962,15 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         }
         if (e || he != hipSuccess || !graphExec) { graphExec = nullptr; graph = false; e = 0; }
         graphB = B;
-        graphArgmax = !hostSample;
+        graphTail = tail;
+        graphTemperature = sampleTemperature;
+        graphTopp = sampleTopp;
     }
     lastUsedGraph = graph;
     // the forced prompt positions in one batched pass (ids chosen on the host need every position's logits in turn,
     // so a sampled generation keeps the one-step-per-position loop)
     const int nPre = std::min(nPrompt, nSteps);
-    const bool batched = use_prefill && !hostSample && nPre >= 2;
+    const bool batched = use_prefill && !sampled && nPre >= 2;   // a sampled generation flips a coin at every position
     const int start = batched ? nPre : 0;
     lastPrefillMs = 0.f;
     lastPrefillRows = 0;
@@ -1786,6 +2026,11 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
     (void)hipEventRecord(evB, s);
     hipError_t he = hipStreamSynchronize(s);
     if (!e && he != hipSuccess) e = (long)he;
+    if (!e && devSample) {
+        // the host sampler carries the random stream from one generation to the next
+        he = hipMemcpy(&sampler->state, drng, 8, hipMemcpyDeviceToHost);
+        if (he != hipSuccess) e = (long)he;
+    }
     lastTimedMs = 0.f;
     lastTimedSteps = 0;
     if (!e && done > t0 && t0 >= 0 && timing) {
@@ -2005,6 +2250,7 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         else if (opt == 8) m->engine.set_kv_bf16(pIn[2] != 0.f);
         else if (opt == 9) m->engine.set_defer_merge(pIn[2] != 0.f);
         else if (opt == 10) m->engine.prefill_act16 = pIn[2] != 0.f;
+        else if (opt == 11) m->engine.device_sampling = pIn[2] != 0.f;
         else return MCH_ERROR_PARAM_OUT_OF_RANGE;
         return 0;
     }

@@ -231,6 +231,38 @@ def test_llama110m_batch16_bf16_weights_prompt_pass_with_bf16_activations(llm, c
             assert (top2[1] - top2[0]) / np.abs(ref_logits[t]).max() < BF16_RTOL, "sequence %d: id differs at a decisive step %d" % (b, t)
 
 
+@pytest.mark.parametrize("topp", [0.9, 0.0, 0.3])
+def test_llama110m_device_sampler_against_the_host_sampler_at_vocab_32000(c4_model, topp):
+    """Temperature 0.8 at the 110M shape (32000 logits a step): the device sampler (option 11 = 1, default: one kernel per
+    step, the steps replayed as a captured graph) against the host sampler after a copy of the logits (option 11 = 0, the
+    reference's arrangement, itself checked against the C checker in test_gpu_llama.py).  Same seed, same coin stream;
+    single sequence and a batch of three; the second generation continues the stream of the first.  An id may differ only
+    where the coin lies within rounding of an edge of the cumulative distribution: none does for these seeds."""
+    path, _ = c4_model
+    rng = np.random.default_rng(12)
+    prompt = rng.integers(3, C4["vocab_size"], 9)
+    prompts = rng.integers(3, C4["vocab_size"], (3, 9))
+    out = {}
+    for dev in (0, 1):
+        cuda = CudaDnn(0)
+        inf = LlmInference(cuda)
+        inf.Initialize(fTemperature=0.8, fTopp=topp, lSeed=4242)
+        inf.SetOption(5, 1)
+        inf.SetOption(11, dev)
+        inf.Load(path)
+        a = inf.GenerateIds(prompt, 60)
+        graph = inf.LastRunUsedGraph()
+        b = inf.GenerateIds(prompt, 40)          # continues the random stream
+        c = inf.GenerateBatch(prompts, 30)
+        out[dev] = (a, b, c)
+        assert graph                             # either way the step's kernels replay as a graph; the host path stops at the logits
+        inf.CleanUp()
+        cuda.Dispose()
+    for x, y in zip(out[0], out[1]):
+        assert np.array_equal(x, y)
+    assert not np.array_equal(out[1][0][:40], out[1][1])   # a different stretch of the stream, a different text
+
+
 def test_weight_storage_option_after_load_leaves_the_loaded_model_alone(llm, c4_model):
     # option 1 names the storage of the NEXT load: flipping it on a loaded fp32 model changes nothing
     path, blob = c4_model
