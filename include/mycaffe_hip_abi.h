@@ -178,7 +178,9 @@ enum {
      * QKV_PROJ_HEADS replaces the head of CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-557):
      * the fused InnerProduct, its bias GEMM, the three channel copies and the three head transposes become one
      * GEMM whose epilogue adds the bias and writes q, k, v as (batch, heads, T, hs):
-     *   l{batch, T, heads, hs, hX, hWeight (3C x C), hBias (0 = none), hQ, hK, hV}
+     *   l{batch, T, heads, hs, hX, hWeight (3C x C), hBias (0 = none), hQ, hK, hV [, hRope]}
+     * With hRope (a CREATE_ROPE handle of the same heads and hs) the epilogue also rotates q and k, which replaces the
+     * two ROPE_FWD calls the layer makes between the channel copies and the transposes (:538-545).
      * Together with the 11th value of ATTN_FWD (Y written head-merged) the layer forward is four calls:
      * QKV_PROJ_HEADS, ATTN_FWD, GEMM and bias GEMM of the output projection.
      */

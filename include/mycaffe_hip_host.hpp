@@ -401,10 +401,13 @@ public:
     {
         m_cuda.AttnDecodeNoAlloc(m_hKernel, {fScale}, {nBatch, nHeads, nKvHeads, nSize, nLen, hQ, hKCache, hVCache, hY, nStrideBatch, nStrideHead, nStridePos});
     }
-    // fused QKV projection: q, k, v = X W^T + bias written as (B,H,T,hs) (no counterpart in the reference)
-    void QkvProjHeads(int nBatch, int nT, int nHeads, int nSize, long hX, long hWeight, long hBias, long hQ, long hK, long hV)
+    // fused QKV projection: q, k, v = X W^T + bias written as (B,H,T,hs), q and k rotated when hRope is given (no
+    // counterpart in the reference)
+    void QkvProjHeads(int nBatch, int nT, int nHeads, int nSize, long hX, long hWeight, long hBias, long hQ, long hK, long hV,
+                      long hRope = 0)
     {
-        ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV});
+        if (hRope) ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV, hRope});
+        else ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV});
     }
     void RmsNormForward(int nOuter, int nDim, long hX, long hWeight, long hY, float fEps = 1e-5f)
     {

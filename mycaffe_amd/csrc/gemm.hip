@@ -348,7 +348,10 @@ template <> struct BigTraits<float> {
 // N = 3*H*hs columns goes, bias added, to element (b, h, t, d) of tensor `which` (q, k, v), i.e. the layout the
 // attention kernels read, instead of to C[r][c].  Replaces the bias GEMM, the three channel copies and the three head
 // transposes that follow the fused InnerProduct in CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-557).
-struct HeadsEpilogue { const void* bias; void* dst[3]; int T, H, hs; };
+// With fcos / fsin set (tables [seq][hs/2]) the q and k thirds are also rotated, after their rounding to the storage type:
+// adjacent pairs (2i, 2i+1) of row r by the angle of table row r % seq, column i - the rotary embedding that the layer
+// applies to q and k in (B,T,H,hs) layout before the head transposes (CausalSelfAttentionLayer.cs:538-545, rope.cu:785-825).
+struct HeadsEpilogue { const void* bias; void* dst[3]; int T, H, hs; const float* fcos; const float* fsin; int seq; };
 
 template <typename T>
 __device__ __forceinline__ T* heads_dst(const HeadsEpilogue& he, int row, int col)
@@ -357,6 +360,38 @@ __device__ __forceinline__ T* heads_dst(const HeadsEpilogue& he, int row, int co
     const int which = col / Cd, w = col - which * Cd, h = w / he.hs, d = w - h * he.hs;
     const int b = row / he.T, t = row - b * he.T;
     return (T*)he.dst[which] + (((size_t)b * he.H + h) * he.T + t) * he.hs + d;
+}
+
+// (re, im) of one pair of q or k, rotated; the expressions of rope_kernel (ew_kernels.hip)
+__device__ __forceinline__ void heads_rope_pair(float c, float sn, float& re, float& im)
+{
+    const float a = re * c - im * sn, b = re * sn + im * c;
+    re = a; im = b;
+}
+
+// the rotation applied to one 16-byte piece (columns col .. col + 16 / sizeof(T) - 1 of row `row`; whole pairs of one head)
+template <typename T>
+__device__ __forceinline__ u32x4 heads_rope_piece(const HeadsEpilogue& he, int row, int col, u32x4 v)
+{
+    if (!he.fcos || col >= 2 * he.H * he.hs) return v;
+    constexpr int NP = 8 / (int)sizeof(T);
+    const size_t ti = (size_t)(row % he.seq) * (he.hs >> 1) + ((col % he.hs) >> 1);
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        const float c = he.fcos[ti + i], sn = he.fsin[ti + i];
+        if constexpr (sizeof(T) == 4) {
+            float re = __uint_as_float(w[2 * i]), im = __uint_as_float(w[2 * i + 1]);
+            heads_rope_pair(c, sn, re, im);
+            w[2 * i] = __float_as_uint(re); w[2 * i + 1] = __float_as_uint(im);
+        } else {
+            float re = __uint_as_float(w[i] << 16), im = __uint_as_float(w[i] & 0xffff0000u);
+            heads_rope_pair(c, sn, re, im);
+            w[i] = (uint32_t)f32_to_bf16(re) | ((uint32_t)f32_to_bf16(im) << 16);
+        }
+    }
+    u32x4 o; o.x = w[0]; o.y = w[1]; o.z = w[2]; o.w = w[3];
+    return o;
 }
 
 // Epilogues of the prompt pass of the Llama engine (fp32 results of 16-bit operands; llama2_ext.hip), which save the
@@ -655,7 +690,10 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
                 // lanes past RPI * LPR (row widths that do not divide 64) and rows past the block stay idle
                 if (rr < RPI && it * RPI + rr < 32) {
                     const u32x4 v = *(const u32x4*)(cs + (it * RPI + rr) * LDC + cc);
-                    if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + i * 32 + it * RPI + rr, n0 + wn + cc) = v;
+                    if (HEADS) {
+                        const int hr = m0 + wm + i * 32 + it * RPI + rr, hc = n0 + wn + cc;
+                        *(u32x4*)heads_dst<T>(he, hr, hc) = heads_rope_piece<T>(he, hr, hc, v);
+                    }
                     else *(u32x4*)(cg + (size_t)it * RPI * N) = v;
                 }
             }
@@ -670,6 +708,25 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
         for (int j = 0; j < WN; j++) {
             const int r = m0 + wm + i * 32 + row_l;
             if (r >= M) continue;
+            if constexpr (HEADS) {
+                // pairs of adjacent columns (N = 3 H hs with hs even: a pair is inside the matrix or outside it)
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    const int c = n0 + wn + j * 32 + (v >> 2) * 8 + col_l + (v & 3);
+                    if (c >= N) continue;
+                    float o0 = alpha * acc[i][j][v], o1 = alpha * acc[i][j][v + 1];
+                    if (he.bias) { o0 += TR::ld((const T*)he.bias + c); o1 += TR::ld((const T*)he.bias + c + 1); }
+                    T* dp = heads_dst<T>(he, r, c);
+                    if (he.fcos && c < 2 * he.H * he.hs) {
+                        TR::st(dp, o0); TR::st(dp + 1, o1);
+                        o0 = TR::ld(dp); o1 = TR::ld(dp + 1);      // the values as the storage type holds them
+                        const size_t ti = (size_t)(r % he.seq) * (he.hs >> 1) + ((c % he.hs) >> 1);
+                        heads_rope_pair(he.fcos[ti], he.fsin[ti], o0, o1);
+                    }
+                    TR::st(dp, o0); TR::st(dp + 1, o1);
+                }
+                continue;
+            }
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int c = n0 + wn + j * 32 + (v >> 2) * 8 + col_l + (v & 3);
@@ -854,7 +911,7 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_wide_kernel(int M, int N, int 
         for (int it = 0; it < NIT; it++) {
             const int id = it * 64 + lane, r = id / LPR, cc = (id - r * LPR) * E;
             const u32x4 v = *(const u32x4*)(cs + r * LDC + cc);
-            if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + r, n0 + c * CW + cc) = v;
+            if (HEADS) *(u32x4*)heads_dst<T>(he, m0 + wm + r, n0 + c * CW + cc) = heads_rope_piece<T>(he, m0 + wm + r, n0 + c * CW + cc, v);
             else *(u32x4*)(C + (size_t)(m0 + wm + r) * N + n0 + c * CW + cc) = v;
         }
     }
@@ -977,21 +1034,37 @@ __global__ void gemm_rank1_kernel(int m, int n, float alpha, const T* __restrict
 template <typename T>
 __global__ void qkv_split_heads_kernel(const T* __restrict__ tmp, size_t total, int N, HeadsEpilogue he)
 {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)blockDim.x * gridDim.x) {
+    // one pair of adjacent columns per step (hs is even when the rotation is asked for; otherwise N may be odd)
+    const bool pairs = he.fcos != nullptr;
+    const size_t steps = pairs ? total / 2 : total;
+    for (size_t s = (size_t)blockIdx.x * blockDim.x + threadIdx.x; s < steps; s += (size_t)blockDim.x * gridDim.x) {
+        const size_t i = pairs ? 2 * s : s;
         const int r = (int)(i / N), c = (int)(i - (size_t)r * N);
         float o = ldf(tmp, i);
         if (he.bias) o += ldf((const T*)he.bias, c);
-        stf(heads_dst<T>(he, r, c), 0, o);
+        T* dp = heads_dst<T>(he, r, c);
+        if (!pairs) { stf(dp, 0, o); continue; }
+        float o1 = ldf(tmp, i + 1);
+        if (he.bias) o1 += ldf((const T*)he.bias, c + 1);
+        if (c < 2 * he.H * he.hs) {
+            stf(dp, 0, o); stf(dp, 1, o1);
+            o = ldf(dp, 0); o1 = ldf(dp, 1);                       // the values as the storage type holds them
+            const size_t ti = (size_t)(r % he.seq) * (he.hs >> 1) + ((c % he.hs) >> 1);
+            heads_rope_pair(he.fcos[ti], he.fsin[ti], o, o1);
+        }
+        stf(dp, 0, o); stf(dp, 1, o1);
     }
 }
 
 hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
-                            void* q, void* k, void* v, void* tmp)
+                            void* q, void* k, void* v, void* tmp, const float* fcos, const float* fsin, int ropeSeq)
 {
+    if (fcos && (!fsin || ropeSeq < 1 || (hs & 1))) return hipErrorInvalidValue;
     const int m = B * T, C = H * hs, n = 3 * C, kk = C;
     if (m <= 0 || C <= 0) return hipSuccess;
     HeadsEpilogue he;
     he.bias = bias; he.dst[0] = q; he.dst[1] = k; he.dst[2] = v; he.T = T; he.H = H; he.hs = hs;
+    he.fcos = fcos; he.fsin = fcos ? fsin : nullptr; he.seq = fcos ? ropeSeq : 1;
     const int vec = dt == F32 ? 4 : 8;
     const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 == 0) && hs % vec == 0;
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);

@@ -1735,8 +1735,9 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
 
     case MCH_FN_QKV_PROJ_HEADS: {
         // l{batch, T, heads, hs, hX, hW, hBias(0 = none), hQ, hK, hV}: [q|k|v] = X W^T + bias, X (batch*T, C), W (3C, C),
-        // C = heads*hs, each third written as (batch, heads, T, hs)
-        NEED_L(10, 10);
+        // C = heads*hs, each third written as (batch, heads, T, hs).  An eleventh value, hRope != 0, also applies that
+        // handle's rotation to q and k, as ROPE_FWD without an offset does to their (batch, T, heads, hs) form.
+        NEED_L(10, 11);
         const long long B = pl[0], T = pl[1], H = pl[2], hs = pl[3];
         if (B < 1 || T < 1 || H < 1 || hs < 1 || B * T > INT_MAX || 3 * H * hs > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         const long long C = H * hs, M = B * T;
@@ -1755,10 +1756,20 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(Q, 0, M * C);
         RANGE(K, 0, M * C);
         RANGE(V, 0, M * C);
+        RopeState* r = nullptr;
+        if (ll > 10 && pl[10]) {
+            r = m_rope.get((long)pl[10]);
+            if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+            if (r->heads != H || r->hs != hs) {
+                last_detail = "the rope handle was created for other heads or another head size";
+                return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            }
+        }
         void* ws = nullptr;
         ERRCHK(workspace((size_t)(M * 3 * C) * X->esize(), &ws));
         HIPCHK(k_gemm_qkv_heads(s, X->dt(), (int)B, (int)T, (int)H, (int)hs, X->ptr, W->ptr, Bi ? Bi->ptr : nullptr, Q->ptr, K->ptr,
-                                V->ptr, ws));
+                                V->ptr, ws, r ? (const float*)r->dcos.get() : nullptr, r ? (const float*)r->dsin.get() : nullptr,
+                                r ? r->seq : 0));
         m_mem.touch((long)pl[7]);
         m_mem.touch((long)pl[8]);
         m_mem.touch((long)pl[9]);

@@ -678,11 +678,14 @@ class CudaDnn:
             rgl.append(1)
         self._ex2(CUDAFN.CUDA_ATTN_FWD, None, rgl)
 
-    def QkvProjHeads(self, nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV):
+    def QkvProjHeads(self, nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV, hRope=0):
         """Fused QKV projection (no counterpart in the reference: replaces the InnerProduct, bias GEMM, three
         channel copies and three head transposes of CausalSelfAttentionLayer.cs:526-557): q, k, v written as
-        (B,H,T,hs)."""
-        self._ex2(CUDAFN.QKV_PROJ_HEADS, None, [nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV])
+        (B,H,T,hs).  With hRope the two RopeForward calls on q and k (:538-545) are part of it as well."""
+        rgl = [nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV]
+        if hRope:
+            rgl.append(hRope)
+        self._ex2(CUDAFN.QKV_PROJ_HEADS, None, rgl)
 
     def AttnScaledDotProductBackward(self, hCuDnn, hAttn, hQdata, hQdiff, hKdata, hKdiff, hVdata, hVdiff, hMaskdata, hYData, hYdiff):
         """CudaDnn.cs:5695-5701."""

@@ -315,8 +315,8 @@ class CausalSelfAttentionLayer:
                  fused_qkv_heads=False):
         self.training = training
         # four calls per forward instead of seventeen (ids with no counterpart in the reference): the fused QKV
-        # projection writes q, k, v as (B,H,T,hs) and the attention handle writes its output head-merged.  Inference,
-        # fused attention handle, no rotary embedding.
+        # projection writes q, k, v as (B,H,T,hs), rotated where the layer has a rotary embedding, and the attention
+        # handle writes its output head-merged.  Inference, fused attention handle.
         self.fused_qkv_heads = fused_qkv_heads
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
         self.nSize = embed // heads
@@ -368,13 +368,13 @@ class CausalSelfAttentionLayer:
         self._reshape(B, T)
         b, cuda, H, hs = self.b, self.cuda, self.nHeads, self.nSize
         if self.fused_qkv_heads:
-            if not self.enable_sdpa or self.hRope or self.training:
-                raise ValueError("fused_qkv_heads needs the fused attention handle, no rotary embedding, inference mode")
+            if not self.enable_sdpa or self.training:
+                raise ValueError("fused_qkv_heads needs the fused attention handle, inference mode")
             for name in ("Qt", "Kt", "Vt"):
                 b[name].Reshape(B, H, T, hs)
             ip = self.c_attn
             cuda.QkvProjHeads(B, T, H, hs, blobX.gpu_data, ip.blobs[0].gpu_data, ip.blobs[1].gpu_data if ip.bias_term else 0,
-                              b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data)
+                              b["Qt"].gpu_data, b["Kt"].gpu_data, b["Vt"].gpu_data, self.hRope)
             mask = self.blobMask
             if T != self.nBlockSize:
                 if getattr(self, "_sdpa_mask_T", None) != T:

@@ -440,6 +440,64 @@ def test_qkv_proj_heads_against_the_call_sequence_it_replaces(dev, half, B, T, H
 
 
 @pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("B,T,H,hs", [(2, 128, 4, 64), (3, 100, 3, 64), (1, 257, 2, 128), (2, 40, 3, 16), (2, 64, 5, 24)])
+def test_qkv_proj_heads_with_the_rotary_embedding(dev, half, B, T, H, hs):
+    """The eleventh argument: q and k leave the projection rotated, as the two RopeForward calls between the channel
+    copies and the head transposes leave them (CausalSelfAttentionLayer.cs:538-545).  Against the layer's own call
+    sequence (the same products, roundings and tables; the rotation's multiply-adds may contract differently, hence a
+    few ulps and not bit for bit) and against the checker; v must not be touched."""
+    C = H * hs
+    rng = np.random.default_rng(B * 1000 + T + 7)
+    x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    w = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
+    bv = bf16_round((rng.standard_normal(3 * C) * 0.1).astype(np.float32))
+    layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, True, True, enable_rotary_positional_embedding=True, half=half)
+    bottom, top = Blob(dev.cuda, x.shape, half=half), Blob(dev.cuda, half=half)
+    bottom.mutable_cpu_data = x
+    layer.Setup(bottom, w, bv, np.eye(C, dtype=np.float32), np.zeros(C, np.float32))
+    layer.Forward(bottom, top)
+    seq = [layer.b[n].mutable_cpu_data.reshape(B, H, T, hs) for n in ("Qt", "Kt", "Vt")]
+    hx, hw, hb = dev.put(x, half), dev.put(w, half), dev.put(bv, half)
+    hq, hk, hv = (dev.zeros(B * T * C, half) for _ in range(3))
+    dev.cuda.QkvProjHeads(B, T, H, hs, hx, hw, hb, hq, hk, hv, layer.hRope)
+    got = [dev.get(h, (B, H, T, hs)) for h in (hq, hk, hv)]
+    qkv = R.inner_product(x, w, bv, np.float64).reshape(B, T, 3, H, hs)
+    ref = [R.rope_forward(qkv[:, :, i], T, H, hs, dtype=np.float64).reshape(B, T, H, hs) if i < 2 else qkv[:, :, i] for i in range(3)]
+    for i, name in enumerate("qkv"):
+        assert_close(got[i], ref[i].transpose(0, 2, 1, 3), BF16_RTOL if half else FP32_RTOL, name + " vs checker")
+        assert_close(got[i], seq[i], BF16_RTOL if half else 1e-6, name + " vs the call sequence")
+    assert np.array_equal(got[2], seq[2]) or half
+    # the handle has to fit the projection
+    other = dev.cuda.CreateRope(0, 0, B * T * C, B, T, H + 1, hs, 10000.0)
+    with pytest.raises(Exception):
+        dev.cuda.QkvProjHeads(B, T, H, hs, hx, hw, hb, hq, hk, hv, other)
+    dev.cuda.FreeRope(other)
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_causal_self_attention_layer_with_rotary_embedding_as_four_calls(dev, half):
+    B, T, C, H = 2, 128, 256, 4
+    rng = np.random.default_rng(T + 1)
+    x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    wa = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
+    wp = bf16_round((rng.standard_normal((C, C)) * 0.05).astype(np.float32))
+    ba = bf16_round((rng.standard_normal(3 * C) * 0.1).astype(np.float32))
+    bp = bf16_round((rng.standard_normal(C) * 0.1).astype(np.float32))
+    outs = []
+    for fused in (False, True):
+        layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, True, True, enable_rotary_positional_embedding=True, half=half,
+                                         fused_qkv_heads=fused)
+        bottom, top = Blob(dev.cuda, x.shape, half=half), Blob(dev.cuda, half=half)
+        bottom.mutable_cpu_data = x
+        layer.Setup(bottom, wa, ba, wp, bp)
+        layer.Forward(bottom, top)
+        outs.append(top.mutable_cpu_data.copy())
+    ref = R.causal_self_attention(x, wa, ba, wp, bp, H, rope=(T, 10000.0), dtype=np.float64)["y"]
+    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "four-call layer vs checker")
+    assert_close(outs[1], outs[0], BF16_RTOL if half else 1e-5, "four-call layer vs the nineteen-call sequence")
+
+
+@pytest.mark.parametrize("half", [False, True])
 @pytest.mark.parametrize("B,T,C,H", [(2, 128, 256, 4), (1, 200, 192, 3), (2, 96, 256, 2), (2, 50, 48, 3)])
 def test_causal_self_attention_layer_as_four_calls(dev, half, B, T, C, H):
     rng = np.random.default_rng(T)

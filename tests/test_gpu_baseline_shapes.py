@@ -475,6 +475,14 @@ def test_qkv_proj_heads_at_layer_shapes(dev, half, H, hs):
     ref = R.inner_product(x, w, bv, np.float64).reshape(B, T, 3, H, hs).transpose(2, 0, 3, 1, 4)
     for i, (name, h) in enumerate(zip("qkv", (hq, hk, hv))):
         assert_close(dev.get(h, (B, H, T, hs)), ref[i], BF16_RTOL if half else FP32_RTOL, name)
+    # the same with the rotation of q and k in the epilogue (the wide tiles' store path in 16-bit storage)
+    hr = dev.cuda.CreateRope(0, 0, B * T * C, B, T, H, hs, 10000.0)
+    dev.cuda.QkvProjHeads(B, T, H, hs, hx, hw, hb, hq, hk, hv, hr)
+    dev.cuda.FreeRope(hr)
+    qkv = ref.transpose(1, 3, 0, 2, 4)      # (B, T, 3, H, hs)
+    for i, (name, h) in enumerate(zip("qkv", (hq, hk, hv))):
+        want = R.rope_forward(qkv[:, :, i], T, H, hs, dtype=np.float64).reshape(B, T, H, hs) if i < 2 else qkv[:, :, i]
+        assert_close(dev.get(h, (B, H, T, hs)), want.transpose(0, 2, 1, 3), BF16_RTOL if half else FP32_RTOL, name + " rotated")
 
 
 @pytest.mark.parametrize("half", [False, True])
