@@ -101,6 +101,37 @@ def run_decode(cuda, path, bf16, batch, steps, warmup, seed=1, graph=True, kv_bf
     return inf, res
 
 
+def bench_sampled_generation(cuda, path, steps=192):
+    """Temperature 0.8, top-p 0.9 and plain multinomial, fp32 weights, one sequence: the reference samples on the host after
+    a copy of the logits, at every position, the prompt's included (llm.cpp:231, llama2_sampler.cpp:126-151).  Reported
+    per sampler placement: milliseconds per generated position, and the time to get through the 128 prompt positions -
+    one batched pass with the device sampler (every row takes its own draw), one step per position with the host's."""
+    from mycaffe_amd.llm_inference import LlmInference
+    out = {}
+    prompt = np.random.default_rng(17).integers(3, C4["vocab_size"], N_PROMPT)
+    for topp, tag in ((0.9, "top_p_0.9"), (0.0, "multinomial")):
+        for dev in (1, 0):
+            inf = LlmInference(cuda)
+            inf.Initialize(fTemperature=0.8, fTopp=topp, lSeed=1)
+            inf.SetOption(5, 1)
+            inf.SetOption(11, dev)
+            inf.Load(path)
+            inf.GenerateIds(prompt, N_PROMPT + 8)
+            inf.SetOption(2, N_PROMPT)
+            inf.GenerateIds(prompt, N_PROMPT + steps)
+            ms, n = inf.QueryTiming()
+            pre_ms, rows = inf.LastPrefill()
+            if not rows:
+                # the prompt went one step per position: time those steps
+                inf.SetOption(2, 0)
+                inf.GenerateIds(prompt, N_PROMPT)
+                pre_ms = inf.QueryTiming()[0]
+            out["%s_%s" % (tag, "device_sampler" if dev else "host_sampler")] = {
+                "ms_per_position": round(ms / n, 4), "prompt_128_positions_ms": round(pre_ms, 3), "prompt_as_one_pass": bool(rows)}
+            inf.CleanUp()
+    return out
+
+
 def prefill_summary(r, batch, es):
     """The batched prompt pass of one generation: HIP-event time, prompt tokens per second, and the model flops per second
     (2 x matrix parameters x rows, the classifier included, plus the causal half of the attention products) as a fraction
@@ -623,7 +654,7 @@ def main():
     ap.add_argument("--counter-pass", nargs="?", const="all", default=None, metavar="SECTIONS",
                     help="few dispatches of the kernels of the named sections (comma list of %s; default all), for rocprofv3 "
                          "--pmc runs; prints what ran instead of the benchmark line" % ", ".join(COUNTER_SECTIONS))
-    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,prefill,backward,csa_layer,matmul_chain,block_ops,decode_attn,encdec,gemm "
+    ap.add_argument("--only", default="", help="comma list of 'also' sections to run: decode,sampled,prefill,backward,csa_layer,matmul_chain,block_ops,decode_attn,encdec,gemm "
                     "(and copy, the counter-calibration kernel, which only runs when named)")
     args = ap.parse_args()
     if args.no_steady:
@@ -690,6 +721,9 @@ def main():
                 also["decode_" + tag]["prefill_128_tokens_bf16_activations"] = prefill_summary({"prefill_ms": best, "prefill_rows": rows}, batch, 2)
                 log("  with bf16 activations (option 10):", json.dumps(also["decode_" + tag]["prefill_128_tokens_bf16_activations"]))
             i2.CleanUp()
+    if want("sampled"):
+        also["sampled_generation_fp32_b1"] = bench_sampled_generation(cuda, path)
+        log("sampled generation:", json.dumps(also["sampled_generation_fp32_b1"]))
     if want("prefill"):
         also["prefill_attention_B8_T1024_H12x64"] = bench_prefill_attention(cuda, 50)
         log("prefill attention:", json.dumps(also["prefill_attention_B8_T1024_H12x64"]))

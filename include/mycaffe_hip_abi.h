@@ -286,7 +286,8 @@ enum {
      *                 in bf16 (1: half the matrix-core work, logits within the 16-bit bar); option 11 = where
      *                 a sampler with a temperature above 0 runs: on the device (1, default: softmax, the
      *                 xorshift64* coin and the top-p / multinomial choice in one kernel per step, so the
-     *                 steps replay as a captured graph; the id can differ from the host's only where the
+     *                 steps replay as a captured graph, and the prompt stays one batched pass in which
+     *                 every row takes the draw of its position; the id can differ from the host's only where the
      *                 coin falls within rounding of an edge of the cumulative distribution) or on the host
      *                 after a copy of the logits, as llama2_gpu.cpp:108 and llama2_sampler.cpp do it (0)
      *   GENERATE_BATCH f{hLlm, nSteps, batch, nPrompt, ids of seq 0.., seq 1..}

@@ -739,8 +739,13 @@ template <typename F> __device__ __forceinline__ int running_sum_until(const flo
     }
     return n;
 }
+// Rows of a batched prompt pass (P > 0): row row0 + blockIdx.x = (sequence b, position p) of B sequences takes draw
+// p B + b + 1 - the coin the one-position-at-a-time loop would have flipped for it - and its id goes to
+// out_ids[b][p] (and to next[b] after the last position) instead of given[].
 __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__ logits, int V, float temperature, float topp,
-                                                             const unsigned long long* __restrict__ rng, int* __restrict__ given)
+                                                             const unsigned long long* __restrict__ rng, int* __restrict__ given,
+                                                             int row0 = 0, int P = 0, int B = 0, int promptStride = 0,
+                                                             int* __restrict__ out_ids = nullptr, int* __restrict__ next = nullptr)
 {
     extern __shared__ __attribute__((aligned(16))) float sbuf[];   // V values in index order, later the sorted candidates
     __shared__ WgScratch sc;
@@ -748,9 +753,17 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
     __shared__ int sint[4];
     const int tid = threadIdx.x, b = blockIdx.x;
     float* p = logits + (size_t)b * V;
+    const int rowSeq = P > 0 ? (row0 + b) / P : b, rowPos = P > 0 ? (row0 + b) - rowSeq * P : 0;
+    auto emit = [&](int id) {
+        if (P > 0) {
+            out_ids[(size_t)rowSeq * promptStride + rowPos] = id;
+            if (rowPos == P - 1) next[rowSeq] = id;
+        } else given[b] = id;
+    };
     // the coin: draw b + 1 of the step's state (:115-124)
     unsigned long long st = *rng;
-    for (int d = 0; d <= b; d++) st = xorshift64_next(st);
+    const int draws = P > 0 ? rowPos * B + rowSeq : b;
+    for (int d = 0; d <= draws; d++) st = xorshift64_next(st);
     const float coin = (float)((unsigned int)((st * 0x2545F4914F6CDD1Dull) >> 32) >> 8) / 16777216.0f;
     // probabilities (:131-135; softmax, llama2_cpu.cpp): maximum, exponentials, their sum in index order, division
     float mx = -INFINITY;
@@ -780,7 +793,7 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
         if (tid == 0) {
             float cdf = 0.f;
             const int hit = running_sum_until(sbuf, V, cdf, [coin](float c) { return coin < c; });
-            given[b] = hit < V ? hit : V - 1;
+            emit(hit < V ? hit : V - 1);
         }
         return;
     }
@@ -810,7 +823,7 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
         for (int i = tid; i < V; i += 1024)
             if (p[i] == best) atomicMin(&sint[1], i);
         __syncthreads();
-        if (tid == 0) given[b] = sint[1];
+        if (tid == 0) emit(sint[1]);
         return;
     }
     int n2 = 1;
@@ -858,7 +871,25 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
             if (p[i] == v && ++k == m) sint[3] = i;
     }
     __syncthreads();
-    if (tid == 0) given[b] = sint[3];
+    if (tid == 0) emit(sint[3]);
+}
+
+// the random stream moved on by n draws (what a batched prompt pass of n rows used up)
+__global__ void rng_advance_kernel(unsigned long long* rng, int n)
+{
+    unsigned long long st = *rng;
+    for (int d = 0; d < n; d++) st = xorshift64_next(st);
+    *rng = st;
+}
+
+// the sampling kernel keeps a whole vocabulary in LDS: 128 KB of dynamic LDS, allowed once per process
+static hipError_t sample_attr()
+{
+    static bool done = false;
+    if (done) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute((const void*)sample_device_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SAMPLE_MAX_VOCAB * 4);
+    done = e == hipSuccess;
+    return e;
 }
 
 // ---------------------------------------------------------------------------
@@ -1181,7 +1212,7 @@ private:
     template <typename T> long advance_given(hipStream_t s, int B);
     long ensure_state(int B, int nSteps);
     long ensure_prefill(size_t rows);
-    template <typename T> long prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits);
+    template <typename T> long prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits, int tail = 1);
     hipError_t embed_first(hipStream_t s, int B);
 
     hipStream_t stream = nullptr;
@@ -1500,7 +1531,7 @@ long Engine::ensure_prefill(size_t rows)
 // Positions 0 .. P-1 of all B sequences in one pass.  Leaves what P single-token steps leave: the caches of every
 // layer filled up to P - 1, the id chosen after every position in dout, the id after the last one in dnext, and the
 // generation state at position P.
-template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits)
+template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSteps, float* allLogits, int tail)
 {
     const int dim = cfg.dim, hid = cfg.hidden_dim, H = cfg.n_heads, kvH = cfg.n_kv_heads, hs = dim / H, kvd = hs * kvH, V = cfg.vocab_size;
     const int ldq = dim + 2 * kvd;
@@ -1609,8 +1640,10 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
         if (!clsGemm) HIPCHK((launch_matvec_rows<0, true, T>(s, wcls, pfX + r0 * dim, rms_final, pfLogits, V, dim, rows, V, wclsP)));
         else if (!cls16) HIPCHK(k_gemm(s, F32, false, true, rows, V, dim, 1.f, pfXn + r0 * dim, mode == PF_F32 ? wcls : (const void*)pfW, 0.f, pfLogits));
         else HIPCHK(k_gemm_bf16_f32(s, rows, V, dim, 1.f, (bf16_t*)pfW + r0 * a16Row, mode == PF_SPLIT, wcls, 0.f, pfLogits));
-        hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
-        HIPCHK(hipGetLastError());
+        if (tail != 2) {
+            hipLaunchKernelGGL(prefill_argmax_kernel, rows, 256, 0, s, pfLogits, V, (int)r0, P, cfg.seq_len, dout, dnext);
+            HIPCHK(hipGetLastError());
+        }
         if (allLogits) {
             // rows of one sequence are contiguous on both sides: [b][nSteps][V] <- [b*P + p][V]
             for (size_t m = r0; m < r0 + rows;) {
@@ -1621,6 +1654,17 @@ template <typename T> long Engine::prefill(hipStream_t s, int B, int P, int nSte
                 m += n;
             }
         }
+        if (tail == 2) {
+            // the ids of a sampled generation: every row's own draw of the random stream (the logits become probabilities)
+            HIPCHK(sample_attr());
+            hipLaunchKernelGGL(sample_device_kernel, rows, 1024, SAMPLE_MAX_VOCAB * 4, s, pfLogits, V, sampleTemperature, sampleTopp,
+                               (const unsigned long long*)drng, (int*)nullptr, (int)r0, P, B, cfg.seq_len, dout, dnext);
+            HIPCHK(hipGetLastError());
+        }
+    }
+    if (tail == 2) {
+        hipLaunchKernelGGL(rng_advance_kernel, 1, 1, 0, s, drng, B * P);
+        HIPCHK(hipGetLastError());
     }
     GenState st = {P, 0, P + 1, 0};
     st.n_prompt = hostNPrompt;
@@ -1788,15 +1832,9 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
         SPAN_END();
     } else if (tail == 2) {
         SPAN_BEGIN(SC_SAMPLE);
-        {
-            static bool attr = false;   // 128 KB of dynamic LDS
-            if (!attr) {
-                HIPCHK(hipFuncSetAttribute((const void*)sample_device_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SAMPLE_MAX_VOCAB * 4));
-                attr = true;
-            }
-        }
+        HIPCHK(sample_attr());
         hipLaunchKernelGGL(sample_device_kernel, B, 1024, SAMPLE_MAX_VOCAB * 4, s, logits, V, sampleTemperature, sampleTopp,
-                           (const unsigned long long*)drng, dgiven);
+                           (const unsigned long long*)drng, dgiven, 0, 0, 0, 0, (int*)nullptr, (int*)nullptr);
         HIPCHK(hipGetLastError());
         hipLaunchKernelGGL(sample_advance_kernel<T>, B, 1024, 0, s, logits, V, dstate, dticket, dprompt, cfg.seq_len, dnext, dout,
                            (const T*)emb, x, dim, dcur, (const int*)dgiven, drng);
@@ -1967,10 +2005,11 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         graphTopp = sampleTopp;
     }
     lastUsedGraph = graph;
-    // the forced prompt positions in one batched pass (ids chosen on the host need every position's logits in turn,
-    // so a sampled generation keeps the one-step-per-position loop)
+    // The forced prompt positions in one batched pass.  The reference flips a coin at every position, forced ones
+    // included: the device sampler gives every row of the pass the draw its position would have had.  Ids chosen on
+    // the host need every position's logits in turn, so that kind of generation keeps the one-step-per-position loop.
     const int nPre = std::min(nPrompt, nSteps);
-    const bool batched = use_prefill && !sampled && nPre >= 2;   // a sampled generation flips a coin at every position
+    const bool batched = use_prefill && !hostSample && nPre >= 2;
     const int start = batched ? nPre : 0;
     lastPrefillMs = 0.f;
     lastPrefillRows = 0;
@@ -1982,7 +2021,7 @@ long Engine::generate(const int* prompts, int B, int nPrompt, int nSteps, bool w
         HIPCHK(hipEventCreate(&sc.evP0));
         HIPCHK(hipEventCreate(&sc.evP1));
         HIPCHK(hipEventRecord(sc.evP0, s));
-        e = stored_bf16 ? prefill<bf16_t>(s, B, nPre, nSteps, allLogits) : prefill<float>(s, B, nPre, nSteps, allLogits);
+        e = stored_bf16 ? prefill<bf16_t>(s, B, nPre, nSteps, allLogits, tail) : prefill<float>(s, B, nPre, nSteps, allLogits, tail);
         if (e) return e;
         HIPCHK(hipEventRecord(sc.evP1, s));
         HIPCHK(hipEventSynchronize(sc.evP1));
@@ -2380,6 +2419,8 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
             if (t < 0 || t >= m->engine.cfg.vocab_size) e = MCH_ERROR_LLM_GENERATE;   // e.g. a vocabulary without the " " entry
         if (!e) {
             std::vector<int> ids;
+            int endPos = -1;   // the position whose token or sampled id ended the generation
+            const unsigned long long rng0 = m->sampler.state;
             auto onChunk = [&](const int* out, int from, int to) -> bool {
                 for (int pos = from; pos < to; pos++) {
                     const int token = pos < nP ? toks[pos] : out[pos - 1];
@@ -2389,7 +2430,7 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
                         std::lock_guard<std::mutex> g(m->responseLock);
                         m->response += piece;
                     }
-                    if (token == 2 || next == 2) return false;
+                    if (token == 2 || next == 2) { endPos = pos; return false; }
                 }
                 return !m->cancel.load();
             };
@@ -2397,6 +2438,13 @@ MCH_LONG DLL_InvokeFloatCustomExtensionEx(MCH_LONG fn, float* pIn, MCH_LONG lIn,
             // step that draws the end-of-text id and the random stream stays where the reference's would be
             e = m->engine.generate(toks.data(), 1, nP, steps, false, &ids, nullptr, &m->cancel, m->sampler.greedy() ? 32 : 1, onChunk,
                                    &m->sampler);
+            if (!e && !m->sampler.greedy() && endPos >= 0) {
+                // The reference stops on the very position that draws the end-of-text id, one coin per position up to
+                // it.  The batched prompt pass flips the coins of all prompt positions at once: the stream is put
+                // where the reference's would be.
+                m->sampler.state = rng0;
+                for (int d = 0; d <= endPos; d++) (void)m->sampler.random_u32();
+            }
             if (m->cancel.load()) {
                 std::lock_guard<std::mutex> g(m->responseLock);
                 m->response.clear();

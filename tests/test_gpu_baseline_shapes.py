@@ -237,7 +237,10 @@ def test_llama110m_device_sampler_against_the_host_sampler_at_vocab_32000(c4_mod
     step, the steps replayed as a captured graph) against the host sampler after a copy of the logits (option 11 = 0, the
     reference's arrangement, itself checked against the C checker in test_gpu_llama.py).  Same seed, same coin stream;
     single sequence and a batch of three; the second generation continues the stream of the first.  An id may differ only
-    where the coin lies within rounding of an edge of the cumulative distribution: none does for these seeds."""
+    where the coin lies within rounding of an edge of the cumulative distribution: none does for these seeds.  Both runs
+    take the prompt one position per step (option 7 = 0), so that the two samplers see the same logits bit for bit: a
+    random model's 32000 probabilities are nearly equal, and the last bit of a logit - the batched prompt pass sums in
+    another order - moves such a draw to a neighbouring id."""
     path, _ = c4_model
     rng = np.random.default_rng(12)
     prompt = rng.integers(3, C4["vocab_size"], 9)
@@ -248,6 +251,7 @@ def test_llama110m_device_sampler_against_the_host_sampler_at_vocab_32000(c4_mod
         inf = LlmInference(cuda)
         inf.Initialize(fTemperature=0.8, fTopp=topp, lSeed=4242)
         inf.SetOption(5, 1)
+        inf.SetOption(7, 0)
         inf.SetOption(11, dev)
         inf.Load(path)
         a = inf.GenerateIds(prompt, 60)

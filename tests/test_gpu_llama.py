@@ -366,6 +366,85 @@ def test_sampled_text_generation_matches_checker(tmp_path):
     cuda.Dispose()
 
 
+def test_sampled_text_generation_that_draws_end_of_text_inside_the_prompt(tmp_path):
+    """The reference samples at every position, the prompt's included, and stops on the position that draws the
+    end-of-text id (llm.cpp:231-246).  With this seed that happens at prompt position 18 of 27: the batched prompt pass
+    has flipped the coins of all 27 positions by then, and the random stream has to be left where the reference's loop
+    left it - the next generation tells."""
+    from oracle import tokenizer_ref as TK
+    cfg = dict(dim=64, hidden_dim=172, n_layers=2, n_heads=4, n_kv_heads=4, vocab_size=320, seq_len=96)
+    vocab, scores = _vocab(cfg["vocab_size"])
+    tok_path = str(tmp_path / "tok.bin")
+    TK.write_tokenizer(tok_path, vocab, scores)
+    tok = TK.Tokenizer(vocab, scores)
+    blob, _ = O.random_weights(cfg, seed=9, shared_classifier=False, std=0.3)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, cfg, blob, False)
+    text = "the cat, hello? hello world the cat hello"
+    # the checker's loop, position by position, to be sure of the premise
+    probe, toks = O.Sampler(1.5, 0.0, 167), tok.encode(text, True, False)
+    model, stop = O.Llama(cfg, blob, False), None
+    for pos in range(len(toks)):
+        if probe.sample(model.forward(toks[pos], pos)) == 2:
+            stop = pos
+            break
+    assert stop is not None and 1 < stop < len(toks) - 2
+    cuda = CudaDnn(0)
+    inf = LlmInference(cuda)
+    inf.Initialize(fTemperature=1.5, fTopp=0.0, lSeed=167)
+    inf.Load(ckpt, tok_path)
+    ref_sampler = O.Sampler(1.5, 0.0, 167)
+    for t in [text, "hello world"]:
+        ref = TK.generate_text_sampled(O.Llama(cfg, blob, False), tok, t, cfg["seq_len"], ref_sampler)
+        inf.Generate(t)
+        got, end, polls = "", False, 0
+        while not end and polls < 50:
+            part, end = inf.QueryResponse()
+            got += part
+            polls += 1
+        assert end
+        assert got.encode("utf-8") == ref.decode("utf-8", errors="replace").encode("utf-8"), (t, got, ref)
+    inf.CleanUp()
+    cuda.Dispose()
+
+
+@pytest.mark.parametrize("topp", [0.9, 0.0])
+def test_sampled_generation_with_the_batched_prompt_pass(topp, tmp_path):
+    """A sampled generation flips a coin at every position, forced ones included (llm.cpp:231).  With the sampler on the
+    device the prompt still goes through the layers as one pass: row (sequence b, position p) takes the draw the
+    position-by-position loop would have given it.  Same ids as that loop and as the checker's, for one sequence and for
+    a batch, and the stream carries on into the next generation."""
+    cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, seq_len=256)
+    blob, _ = O.random_weights(cfg, seed=33, shared_classifier=False, std=0.08)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, cfg, blob, False)
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(3, cfg["vocab_size"], 100)
+    prompts = rng.integers(3, cfg["vocab_size"], (3, 41))
+    out = {}
+    for pre in (1, 0):
+        cuda = CudaDnn(0)
+        inf = LlmInference(cuda)
+        inf.Initialize(fTemperature=0.8, fTopp=topp, lSeed=77)
+        inf.SetOption(5, 1)
+        inf.SetOption(7, pre)
+        inf.Load(ckpt)
+        a = inf.GenerateIds(prompt, 140)
+        rows = inf.LastPrefill()[1]
+        b = inf.GenerateIds(prompt[:30], 50)
+        c = inf.GenerateBatch(prompts, 60)
+        assert rows == (100 if pre else 0) and inf.LastPrefill()[1] == (3 * 41 if pre else 0)
+        out[pre] = (a, b, c)
+        inf.CleanUp()
+        cuda.Dispose()
+    for x, y in zip(out[0], out[1]):
+        assert np.array_equal(x, y)
+    ref_sampler = O.Sampler(0.8, topp, 77)
+    cpu = O.Llama(cfg, blob, False)
+    assert np.array_equal(out[1][0], cpu.generate_sampled(prompt, 140, ref_sampler))
+    assert np.array_equal(out[1][1], cpu.generate_sampled(prompt[:30], 50, ref_sampler))
+
+
 def test_llama_decode_through_the_layer_call_sequences_matches_the_checker(dev):
     """The route the C# model builder's networks take (TestModelBuilder.cs:745-790: "position" layer option, one token
     per forward): embedding, Llama-style ENCODER transformer blocks (RMSNorm chain, MultiheadAttentionLayer with rotary
