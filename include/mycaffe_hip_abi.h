@@ -302,14 +302,21 @@ enum {
      *   TOKENIZE      Ex: f{hLlm, bos(0|1), eos(0|1)} + text -> f{token ids};
      *                 f{hLlm, -1, prevToken, token} -> the token's piece in szOutput
      *   SAMPLE        f{hLlm, logits...} -> f{id}: one call of the handle's sampler
-     *                 (llama2_sampler.cpp:126-151); advances its random state unless greedy */
+     *                 (llama2_sampler.cpp:126-151); advances its random state unless greedy; runs where the
+     *                 generations sample (option 11: the device kernel for up to 32768 logits, else the host)
+     *   RUNNING_SUM   f{hLlm, threshold, values...} -> f{index, sum}: the device sampler's way of adding up
+     *                 non-negative fp32 values one after the other, every addition rounded (the sums of
+     *                 llama2_sampler.cpp:38-49, 78-99 and of the softmax), stopped at the first index where
+     *                 the sum exceeds the threshold (index = count if it never does); for checking it
+     *                 against a plain loop, up to 32768 values */
     MCH_LLM_GENERATE_IDS = 100,
     MCH_LLM_SET_OPTION = 101,
     MCH_LLM_GENERATE_BATCH = 102,
     MCH_LLM_QUERY_TIMING = 103,
     MCH_LLM_PROFILE_STEP = 104,
     MCH_LLM_TOKENIZE = 105,
-    MCH_LLM_SAMPLE = 106
+    MCH_LLM_SAMPLE = 106,
+    MCH_LLM_RUNNING_SUM = 107
 };
 
 MCH_LONG DLL_InitFloatCustomExtension(void* hParent, MCH_LONG lKernelIdx);

@@ -670,7 +670,8 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
 // logits to the host.  The reference's arithmetic is sequential - the softmax denominator and the cumulative sums are
 // running fp32 sums in index order and in sorted order - and with a flat distribution the rounding of those sums moves
 // the chosen id as often as one time in five, so it is kept: what can run in parallel does (maximum, exponentials,
-// division, the sort), the running sums are walked by one lane over LDS in the reference's order.
+// division, the sort), and the running sums come out bit for bit as the reference's loops leave them
+// (wg_running_sum_until).
 //   * The coin is the reference's: xorshift64* (:115-124) on a state kept in device memory; sequence b of a step takes
 //     draw b + 1 from the step's state (the reference flips one coin per forward call, forced positions included), and
 //     the step's tail kernel moves the state on by one draw per sequence.
@@ -678,8 +679,9 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(const float* __res
 //     arguments, the device's single-precision one is not.
 //   * The logits are overwritten by the probabilities, as in the reference.
 //   * Top-p: the candidates (probability >= (1 - topp) / (n - 1)) are gathered in LDS and sorted by value (bitonic,
-//     descending); the order among equal values does not change a sum, only which index a position stands for, and
-//     that is settled afterwards: the m-th of the equal values in the sorted list is the m-th of them by index.
+//     descending, 32 values per thread in registers); the order among equal values does not change a sum, only which
+//     index a position stands for, and that is settled afterwards: the m-th of the equal values in the sorted list is
+//     the m-th of them by index.
 // Up to 32768 logits (128 KB of LDS); the engine samples longer vocabularies on the host.
 __device__ __forceinline__ unsigned long long xorshift64_next(unsigned long long st)
 {
@@ -716,28 +718,134 @@ __device__ __forceinline__ int wg_exclusive_scan_int_1024(int v, WgScratch& sc)
     return base + inc - v;
 }
 constexpr int SAMPLE_MAX_VOCAB = 32768;
-// One lane's running sum over buf[0 .. n) in order: acc += buf[i], stopping at the first i where exceeds(acc) holds.
-// Returns that i (n if none) and leaves the sum reached in acc.  The values are not negative, so the sum never falls and
-// `exceeds` - a threshold on it - only has to be asked once per batch of 32 additions; the batch in which it first holds
-// is gone through again.  That leaves one dependent addition per value, and the LDS latency is paid once per batch.
-template <typename F> __device__ __forceinline__ int running_sum_until(const float* buf, int n, float& acc, F exceeds)
+// The running sum acc += buf[0], acc += buf[1], ... in fp32, every addition rounded, as the reference's loops do it: the
+// sum after the last value, or the first index at which a threshold on the sum holds.  One lane adding 32000 numbers
+// one after the other is 150000 cycles of dependent additions; this does the same additions, bit for bit, in a
+// fraction of that.  While the sum stays in one binade it is an integer m < 2^24 times u = ulp(sum), and adding
+// x >= 0 gives m + round(x / u) - round to nearest, a tie (x / u = k + 1/2) to the even neighbour, which depends on
+// nothing but the parity of m.  So a run of values is, for a known exponent of the sum, a function of that parity alone:
+// it adds an integer and leaves a parity, and a tie forces the parity to even whatever it was.  Every thread works
+// that function out for its own chunk of 33 consecutive values (stride 33: its LDS reads hit 64 different banks),
+// taking the exponent from an approximate prefix sum; then one lane goes over the chunks in order with a few integer
+// operations each.  A chunk whose guess was wrong (the exact sum has another exponent than the approximate one), in
+// which the sum reaches the next binade, whose prefix is zero, or the one in which the threshold is crossed is added
+// up value by value - a handful of the thousand chunks.  All 1024 threads call it; values must not be negative.
+struct SumChunk { int e, sum0, sum1, meta; };   // meta: bit 0 / 1 parity left for incoming parity 0 / 1, bit 2 usable
+constexpr int SUM_CHUNK = 33;
+static_assert(SAMPLE_MAX_VOCAB <= 1024 * SUM_CHUNK, "one chunk per thread");
+template <typename F>
+__device__ __forceinline__ int wg_running_sum_until(const float* buf, int n, float& acc, F exceeds, SumChunk* tab, WgScratch& sc,
+                                                    int* result)
 {
-    int i = 0;
-    for (; i + 32 <= n; i += 32) {
-        float4 q[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i0 = tid * SUM_CHUNK;
+    const int cnt = min(max(n - i0, 0), SUM_CHUNK);
+    float x[SUM_CHUNK];
+    float part = 0.f;
 #pragma unroll
-        for (int u = 0; u < 8; u++) q[u] = *(const float4*)(buf + i + 4 * u);
-        float t = acc;
+    for (int i = 0; i < SUM_CHUNK; i++) {
+        x[i] = i < cnt ? buf[i0 + i] : 0.f;
+        part += x[i];
+    }
+    // approximate sum in front of this chunk: scan over the lanes, then over the wavefronts
+    float inc = part;
 #pragma unroll
-        for (int u = 0; u < 8; u++) { t += q[u].x; t += q[u].y; t += q[u].z; t += q[u].w; }
-        if (exceeds(t)) break;
-        acc = t;
+    for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += up;
     }
-    for (; i < n; i++) {
-        acc += buf[i];
-        if (exceeds(acc)) return i;
+    __syncthreads();
+    if (lane == 63) sc.f[wave] = inc;
+    __syncthreads();
+    float before = acc;
+    for (int w = 0; w < wave; w++) before += sc.f[w];
+    before += inc - part;
+    {
+        const unsigned int bb = __float_as_uint(before), be = (bb >> 23) & 0xffu;
+        SumChunk t;
+        t.e = (int)be;                                        // biased exponent the sum is expected to have
+        bool ok = cnt == SUM_CHUNK && be >= 1u && be <= 254u;
+        int sum[2] = {0, 0}, par[2] = {0, 1};
+        const int shift = 150 - (int)be;                       // x / u = x * 2^(23 - (be - 127))
+#pragma unroll
+        for (int i = 0; i < SUM_CHUNK; i++) {
+            const float y = __builtin_ldexpf(x[i], shift);
+            ok = ok && y < 16777216.f;
+            const float fl = floorf(y), fr = y - fl;
+            const int k = (int)fminf(fl, 16777216.f);
+            const int up = fr > 0.5f ? 1 : 0;
+            const bool tie = fr == 0.5f;
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                const int q = k + (tie ? ((par[p] ^ k) & 1) : up);
+                par[p] ^= q & 1;
+                sum[p] += q;
+            }
+        }
+        ok = ok && sum[0] < 16777216 && sum[1] < 16777216;
+        t.sum0 = sum[0];
+        t.sum1 = sum[1];
+        t.meta = par[0] | (par[1] << 1) | (ok ? 4 : 0);
+        tab[tid] = t;
     }
-    return n;
+    __syncthreads();
+    if (wave == 0) {
+        // Wavefront 0 goes over the chunks 64 at a time.  The chunks' functions compose (parity in -> integer added,
+        // parity out), so an inclusive scan over the lanes gives every lane the sum after its chunk, all at once; the
+        // first lane whose chunk cannot be taken that way (or behind which the threshold holds) is where the value-by-value
+        // additions take over for one chunk, and the scan resumes behind it.
+        const int nch = (n + SUM_CHUNK - 1) / SUM_CHUNK;
+        unsigned int sb = __float_as_uint(acc);
+        int hit = n, c = 0;
+        while (c < nch) {
+            const int cc = c + lane;
+            const SumChunk t = tab[min(cc, 1023)];
+            unsigned int s0 = (unsigned int)t.sum0, s1 = (unsigned int)t.sum1;
+            int p0 = t.meta & 1, p1 = (t.meta >> 1) & 1;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const unsigned int us0 = __shfl_up(s0, o, 64), us1 = __shfl_up(s1, o, 64);
+                const int up0 = __shfl_up(p0, o, 64), up1 = __shfl_up(p1, o, 64);
+                if (lane >= o) {
+                    // the lanes before, then mine
+                    const unsigned int n0 = us0 + (up0 ? s1 : s0), n1 = us1 + (up1 ? s1 : s0);
+                    const int q0 = up0 ? p1 : p0, q1 = up1 ? p1 : p0;
+                    s0 = n0; s1 = n1; p0 = q0; p1 = q1;
+                }
+            }
+            const unsigned int m = (sb & 0x7fffffu) | 0x800000u;
+            // behind a chunk that cannot be taken the scan's sums mean nothing (and may have wrapped): 64 bits for the compare
+            const unsigned long long tot = (unsigned long long)m + (unsigned long long)((m & 1u) ? s1 : s0);
+            const unsigned int nb = (sb & 0xff800000u) | ((unsigned int)tot & 0x7fffffu);
+            const bool fail = cc >= nch || !(t.meta & 4) || (int)(sb >> 23) != t.e || tot >= 0x1000000ull || exceeds(__uint_as_float(nb));
+            const unsigned long long mask = __ballot(fail);
+            const int f = mask ? __builtin_ctzll(mask) : 64;
+            if (f > 0) sb = (unsigned int)__builtin_amdgcn_readlane((int)nb, f - 1);
+            c += f;
+            if (f < 64 && c < nch) {
+                // value by value (every lane the same additions: the result stays uniform)
+                float a = __uint_as_float(sb);
+                const int j0 = c * SUM_CHUNK, j1 = min(j0 + SUM_CHUNK, n);
+                int j = j0;
+                for (; j < j1; j++) {
+                    a += buf[j];
+                    if (exceeds(a)) break;
+                }
+                sb = __float_as_uint(a);
+                if (j < j1) { hit = j; break; }
+                c++;
+            }
+        }
+        if (lane == 0) {
+            result[0] = hit;
+            result[1] = (int)sb;
+        }
+    }
+    __syncthreads();
+    acc = __uint_as_float((unsigned int)result[1]);
+    const int hit = result[0];
+    __syncthreads();   // result[] may be written again by the next call
+    return hit;
 }
 // Rows of a batched prompt pass (P > 0): row row0 + blockIdx.x = (sequence b, position p) of B sequences takes draw
 // p B + b + 1 - the coin the one-position-at-a-time loop would have flipped for it - and its id goes to
@@ -749,6 +857,8 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
 {
     extern __shared__ __attribute__((aligned(16))) float sbuf[];   // V values in index order, later the sorted candidates
     __shared__ WgScratch sc;
+    __shared__ SumChunk tab[1024];
+    __shared__ int sres[2];
     __shared__ float sval[2];
     __shared__ int sint[4];
     const int tid = threadIdx.x, b = blockIdx.x;
@@ -775,13 +885,8 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
     mx = wg_max_1024(mx, sc);
     for (int i = tid; i < V; i += 1024) sbuf[i] = (float)exp((double)(sbuf[i] - mx));
     __syncthreads();
-    if (tid == 0) {
-        float sum = 0.f;
-        running_sum_until(sbuf, V, sum, [](float) { return false; });
-        sval[0] = sum;
-    }
-    __syncthreads();
-    const float sum = sval[0];
+    float sum = 0.f;
+    wg_running_sum_until(sbuf, V, sum, [](float) { return false; }, tab, sc, sres);
     for (int i = tid; i < V; i += 1024) {
         const float q = sbuf[i] / sum;
         sbuf[i] = q;
@@ -790,27 +895,27 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
     __syncthreads();
     if (topp <= 0.f || topp >= 1.f) {
         // sample_mult: the first index whose running sum exceeds the coin, else the last one
-        if (tid == 0) {
-            float cdf = 0.f;
-            const int hit = running_sum_until(sbuf, V, cdf, [coin](float c) { return coin < c; });
-            emit(hit < V ? hit : V - 1);
-        }
+        float cdf = 0.f;
+        const int hit = wg_running_sum_until(sbuf, V, cdf, [coin](float c) { return coin < c; }, tab, sc, sres);
+        if (tid == 0) emit(hit < V ? hit : V - 1);
         return;
     }
     // candidates into LDS, in any order (this thread's values are in registers of a sort: re-read from memory)
     const float cutoff = (1.0f - topp) / (float)(V - 1);
-    if (tid == 0) sint[0] = 0;
-    __syncthreads();   // everybody has read its part of the index-ordered values above; the buffer is rewritten now
     float mine[SAMPLE_MAX_VOCAB / 1024];
 #pragma unroll
     for (int j = 0; j < SAMPLE_MAX_VOCAB / 1024; j++) {
         const int i = j * 1024 + tid;
         mine[j] = i < V ? sbuf[i] : 0.f;
     }
-    __syncthreads();
+    int keep = 0;
+#pragma unroll
+    for (int j = 0; j < SAMPLE_MAX_VOCAB / 1024; j++) keep += (mine[j] >= cutoff && j * 1024 + tid < V) ? 1 : 0;
+    int at = wg_exclusive_scan_int_1024(keep, sc);   // its barriers also separate the reads above from the writes below
+    if (tid == 1023) sint[0] = at + keep;
 #pragma unroll
     for (int j = 0; j < SAMPLE_MAX_VOCAB / 1024; j++)
-        if (mine[j] >= cutoff && j * 1024 + tid < V) sbuf[atomicAdd(&sint[0], 1)] = mine[j];
+        if (mine[j] >= cutoff && j * 1024 + tid < V) sbuf[at++] = mine[j];
     __syncthreads();
     const int n0 = sint[0];
     if (n0 == 0) {
@@ -826,30 +931,84 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
         if (tid == 0) emit(sint[1]);
         return;
     }
-    int n2 = 1;
+    // Bitonic sort, descending, 32 values per thread in registers: position 32 t + r of the sequence is register r of
+    // thread t.  Exchanges 1 .. 16 apart stay inside a thread, those 32 .. 1024 apart are lane exchanges inside a wavefront,
+    // only the ones 2048 and more apart go through LDS (ten of the 120 steps at 32768 values).  Padding zeros sort behind
+    // every candidate (a candidate is at least the cutoff, which is positive).
+    constexpr int EPT = 32;
+    int n2 = EPT;
     while (n2 < n0) n2 <<= 1;
-    for (int i = n0 + tid; i < n2; i += 1024) sbuf[i] = 0.f;   // padding sorts behind every candidate
-    __syncthreads();
-    // bitonic sort, descending
-    for (int k = 2; k <= n2; k <<= 1)
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int t = tid; t < (n2 >> 1); t += 1024) {
-                const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1)), hi = lo | j;
-                const float x = sbuf[lo], y = sbuf[hi];
-                const bool desc = (lo & k) == 0;
-                if (desc ? x < y : x > y) { sbuf[lo] = y; sbuf[hi] = x; }
+    const int nthr = n2 / EPT;
+    float el[EPT];
+#pragma unroll
+    for (int r = 0; r < EPT; r++) {
+        const int i = r * nthr + tid;
+        el[r] = (tid < nthr && i < n0) ? sbuf[i] : 0.f;
+    }
+    __syncthreads();   // the values are in registers: the buffer is free for the exchanges
+    auto inside = [&](int j, bool desc) {   // compare-exchange of the registers j apart, larger first where desc
+#pragma unroll
+        for (int r = 0; r < EPT; r++)
+            if ((r & j) == 0) {
+                const float mx = fmaxf(el[r], el[r | j]), mn = fminf(el[r], el[r | j]);
+                el[r] = desc ? mx : mn;
+                el[r | j] = desc ? mn : mx;
             }
-            __syncthreads();
+    };
+    // runs of 32 inside each thread, alternating direction from thread to thread as a run of 64 wants them
+#pragma unroll
+    for (int k = 2; k <= EPT; k <<= 1)
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+#pragma unroll
+            for (int r = 0; r < EPT; r++)
+                if ((r & j) == 0) {
+                    const bool desc = k == EPT ? (tid & 1) == 0 : (r & k) == 0;
+                    const float mx = fmaxf(el[r], el[r | j]), mn = fminf(el[r], el[r | j]);
+                    el[r] = desc ? mx : mn;
+                    el[r | j] = desc ? mn : mx;
+                }
         }
+    for (int k = 2 * EPT; k <= n2; k <<= 1) {
+        const bool desc = ((tid * EPT) & k) == 0;
+        for (int j = k >> 1; j >= EPT; j >>= 1) {
+            const int jm = j / EPT;
+            const bool keepmax = ((tid & jm) == 0) == desc;
+            if (jm < 64) {
+#pragma unroll
+                for (int r = 0; r < EPT; r++) {
+                    const float other = __shfl_xor(el[r], jm, 64);
+                    el[r] = keepmax ? fmaxf(el[r], other) : fminf(el[r], other);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < EPT; r++) sbuf[r * 1024 + tid] = el[r];
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < EPT; r++) {
+                    const float other = sbuf[r * 1024 + (tid ^ jm)];
+                    el[r] = keepmax ? fmaxf(el[r], other) : fminf(el[r], other);
+                }
+                __syncthreads();
+            }
+        }
+#pragma unroll
+        for (int j = EPT >> 1; j > 0; j >>= 1) inside(j, desc);
+    }
+    if (tid < nthr) {
+#pragma unroll
+        for (int r = 0; r < EPT; r += 4) *(float4*)(sbuf + tid * EPT + r) = make_float4(el[r], el[r + 1], el[r + 2], el[r + 3]);
+    }
+    __syncthreads();
     // end of the nucleus (:78-87) and the sampled position (:89-99), running sums in sorted order
+    float cum = 0.f;
+    int last = wg_running_sum_until(sbuf, n0, cum, [topp](float c) { return c > topp; }, tab, sc, sres);
+    if (last == n0) last = n0 - 1;
+    const float r = coin * cum;
+    float cdf = 0.f;
+    int pos = wg_running_sum_until(sbuf, last + 1, cdf, [r](float c) { return r < c; }, tab, sc, sres);
+    if (pos > last) pos = last;
     if (tid == 0) {
-        float cum = 0.f;
-        int last = running_sum_until(sbuf, n0, cum, [topp](float c) { return c > topp; });
-        if (last == n0) last = n0 - 1;
-        const float r = coin * cum;
-        float cdf = 0.f;
-        int pos = running_sum_until(sbuf, last + 1, cdf, [r](float c) { return r < c; });
-        if (pos > last) pos = last;
         // the position stands for the m-th (by index) of the candidates that share its value
         const float v = sbuf[pos];
         int first = pos;
@@ -872,6 +1031,21 @@ __global__ __launch_bounds__(1024) void sample_device_kernel(float* __restrict__
     }
     __syncthreads();
     if (tid == 0) emit(sint[3]);
+}
+
+// The sampler's running sum by itself (the RUNNING_SUM entry, for checking it against a plain loop): out[0] = first index
+// at which the sum exceeds `threshold` (n if none), out[1] = bits of the sum reached.
+__global__ __launch_bounds__(1024) void running_sum_kernel(const float* __restrict__ values, int n, float threshold, int* out)
+{
+    extern __shared__ __attribute__((aligned(16))) float sbuf[];
+    __shared__ WgScratch sc;
+    __shared__ SumChunk tab[1024];
+    __shared__ int sres[2];
+    for (int i = threadIdx.x; i < n; i += 1024) sbuf[i] = values[i];
+    __syncthreads();
+    float acc = 0.f;
+    const int hit = wg_running_sum_until(sbuf, n, acc, [threshold](float c) { return c > threshold; }, tab, sc, sres);
+    if (threadIdx.x == 0) { out[0] = hit; out[1] = (int)__float_as_uint(acc); }
 }
 
 // the random stream moved on by n draws (what a batched prompt pass of n rows used up)
@@ -1199,6 +1373,8 @@ public:
 
     ~Engine() { release(); }
     long load(const char* path);
+    long sample_device(float* lg, int n, HostSampler* sampler, int* id);
+    long running_sum_device(const float* values, int n, float threshold, int* out2);
     long generate(const int* prompts, int batch, int nPrompt, int nSteps, bool wantLogits, std::vector<int>* ids,
                   std::vector<float>* logits, std::atomic<bool>* cancel, int chunk = 0,
                   const std::function<bool(const int*, int, int)>& onChunk = nullptr, HostSampler* sampler = nullptr);
@@ -1846,6 +2022,57 @@ template <typename T> long Engine::step(hipStream_t s, int B, int nSteps, float*
     return 0;
 }
 
+// One call of the sampler on the device over n logits given on the host (the SAMPLE entry): the kernel of the decode
+// steps, the handle's random stream, one draw.  The logits come back as probabilities, as the host sampler leaves them.
+long Engine::sample_device(float* lg, int n, HostSampler* sampler, int* id)
+{
+    if (n < 1 || n > SAMPLE_MAX_VOCAB) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    struct Dev {
+        void* p = nullptr;
+        ~Dev() { if (p) (void)hipFree(p); }
+    } d;
+    HIPCHK(hipMalloc(&d.p, (size_t)n * 4 + 16));
+    float* dl = (float*)d.p;
+    unsigned long long* dr = (unsigned long long*)(dl + n + (n & 1));
+    int* dg = (int*)(dr + 1);
+    hipStream_t s = stream;
+    HIPCHK(hipMemcpyAsync(dl, lg, (size_t)n * 4, hipMemcpyHostToDevice, s));
+    HIPCHK(hipMemcpyAsync(dr, &sampler->state, 8, hipMemcpyHostToDevice, s));
+    HIPCHK(sample_attr());
+    hipLaunchKernelGGL(sample_device_kernel, 1, 1024, SAMPLE_MAX_VOCAB * 4, s, dl, n, sampler->temperature, sampler->topp,
+                       (const unsigned long long*)dr, dg, 0, 0, 0, 0, (int*)nullptr, (int*)nullptr);
+    HIPCHK(hipGetLastError());
+    HIPCHK(hipMemcpyAsync(lg, dl, (size_t)n * 4, hipMemcpyDeviceToHost, s));
+    HIPCHK(hipMemcpyAsync(id, dg, 4, hipMemcpyDeviceToHost, s));
+    HIPCHK(hipStreamSynchronize(s));
+    (void)sampler->random_u32();   // the draw the kernel took
+    return 0;
+}
+
+long Engine::running_sum_device(const float* values, int n, float threshold, int* out2)
+{
+    if (n < 1 || n > SAMPLE_MAX_VOCAB) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    struct Dev {
+        void* p = nullptr;
+        ~Dev() { if (p) (void)hipFree(p); }
+    } d;
+    HIPCHK(hipMalloc(&d.p, (size_t)n * 4 + 8));
+    float* dv = (float*)d.p;
+    int* dout2 = (int*)(dv + n);
+    hipStream_t s = stream;
+    HIPCHK(hipMemcpyAsync(dv, values, (size_t)n * 4, hipMemcpyHostToDevice, s));
+    static bool attr = false;
+    if (!attr) {
+        HIPCHK(hipFuncSetAttribute((const void*)running_sum_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SAMPLE_MAX_VOCAB * 4));
+        attr = true;
+    }
+    hipLaunchKernelGGL(running_sum_kernel, 1, 1024, SAMPLE_MAX_VOCAB * 4, s, (const float*)dv, n, threshold, dout2);
+    HIPCHK(hipGetLastError());
+    HIPCHK(hipMemcpyAsync(out2, dout2, 8, hipMemcpyDeviceToHost, s));
+    HIPCHK(hipStreamSynchronize(s));
+    return 0;
+}
+
 // tail of a step whose ids were chosen on the host (dgiven): record, embed the next token, advance the position
 template <typename T> long Engine::advance_given(hipStream_t s, int B)
 {
@@ -2318,7 +2545,29 @@ MCH_LONG DLL_InvokeFloatCustomExtension(MCH_LONG fn, float* pIn, MCH_LONG lIn, f
         if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
         std::lock_guard<std::mutex> run(m->runLock);
         std::vector<float> lg(pIn + 1, pIn + lIn);
+        if (!m->sampler.greedy() && m->engine.device_sampling && (int)lg.size() <= SAMPLE_MAX_VOCAB) {
+            // where the generations sample: on the device (option 11)
+            int id = 0;
+            const long e = m->engine.sample_device(lg.data(), (int)lg.size(), &m->sampler, &id);
+            if (e) return (MCH_LONG)e;
+            return (MCH_LONG)give({(float)id}, ppOut, plOut);
+        }
         return (MCH_LONG)give({(float)m->sampler.sample(lg.data(), (int)lg.size())}, ppOut, plOut);
+    }
+    case MCH_LLM_RUNNING_SUM: {
+        // f{hLlm, threshold, values...} -> f{index, sum}: the device sampler's rounded running sum over the values, stopped at
+        // the first index where it exceeds the threshold (index = count when it never does)
+        if (lIn < 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        std::shared_ptr<Llm> m = find_llm((long)pIn[0]);
+        if (!m) return MCH_ERROR_PARAM;
+        if (!m->loaded.load()) return MCH_ERROR_LLM_GENERATE;
+        std::lock_guard<std::mutex> run(m->runLock);
+        int out2[2] = {0, 0};
+        const long e = m->engine.running_sum_device(pIn + 2, (int)(lIn - 2), pIn[1], out2);
+        if (e) return (MCH_LONG)e;
+        float sum;
+        memcpy(&sum, &out2[1], 4);
+        return (MCH_LONG)give({(float)out2[0], sum}, ppOut, plOut);
     }
     case MCH_LLM_GENERATE_IDS:
     case MCH_LLM_GENERATE_BATCH: {

@@ -26,6 +26,7 @@ class CUDAFN_EXTENSION_LLM:
     PROFILE_STEP = 104
     TOKENIZE = 105
     SAMPLE = 106
+    RUNNING_SUM = 107
 
 
 STEP_CLASSES = ("matvec_qkv", "rope_store", "attn_decode", "matvec_wo", "matvec_w13", "matvec_w2", "matvec_cls", "embed_argmax")
@@ -93,6 +94,13 @@ class LlmInference:
         """One call of the handle's sampler on the given logits (advances its random state unless temperature is 0)."""
         rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.SAMPLE, self.m_rgLlm + [float(v) for v in logits])
         return int(rg[0])
+
+    def RunningSum(self, values, threshold=float("inf")):
+        """The device sampler's rounded running sum over non-negative fp32 ``values``: (first index at which the sum
+        exceeds ``threshold`` or len(values), the sum reached as numpy.float32)."""
+        rg = self.m_cuda.RunExtension(self.m_hExtension, CUDAFN_EXTENSION_LLM.RUNNING_SUM,
+                                      self.m_rgLlm + [float(threshold)] + [float(v) for v in values])
+        return int(rg[0]), np.float32(rg[1])
 
     def GenerateIds(self, prompt_ids, nSteps, want_logits=False, vocab_size=None):
         """Greedy decode from token ids; returns the id sampled after every position

@@ -311,6 +311,59 @@ def test_sampler_entry_matches_checker_on_given_logits():
         cuda.Dispose()
 
 
+def _seq_sum_f32(x, threshold=np.inf):
+    acc = np.float32(0)
+    for i, v in enumerate(np.asarray(x, np.float32)):
+        acc = np.float32(acc + v)
+        if acc > threshold:
+            return i, acc
+    return len(x), acc
+
+
+def test_device_running_sum_is_the_plain_loop_bit_for_bit(tmp_path):
+    """The sampler's sums (softmax denominator, cumulative probabilities in index and in sorted order,
+    llama2_sampler.cpp:38-49, 78-99) are fp32 running sums whose rounding decides ids.  The device adds chunks of values
+    as integers in units of the sum's ulp; this pins that against the plain loop on the cases that can break it: ties
+    (a value that is an odd number of half ulps of the sum), sums that climb through binades, zeros and denormals in
+    front, a threshold crossed in the middle of a chunk, lengths that are not whole chunks."""
+    blob, _ = O.random_weights(TINY, seed=2, std=0.2)
+    ckpt = str(tmp_path / "m.bin")
+    O.write_checkpoint_v1(ckpt, TINY, blob, False)
+    cuda = CudaDnn(0)
+    inf = LlmInference(cuda)
+    inf.Initialize(fTemperature=1.0, fTopp=0.9, lSeed=1)
+    inf.Load(ckpt)
+    rng = np.random.default_rng(5)
+    cases = []
+    for t in range(3):
+        lg = rng.standard_normal(32000).astype(np.float32) * (1 + 2 * t)
+        e = np.exp((lg - lg.max()).astype(np.float64)).astype(np.float32)
+        cases += [("exponentials", e, np.inf), ("sorted probabilities", np.sort(e / e.sum(dtype=np.float32))[::-1], 0.9),
+                  ("probabilities", e / e.sum(dtype=np.float32), float(rng.random()))]
+    x = np.full(32000, 2.0 ** -24, np.float32); x[0] = 1.0
+    cases.append(("half ulps of 1.0", x, np.inf))
+    x = (rng.integers(1, 8, 32000) * 2.0 ** -25).astype(np.float32); x[0] = 1.0
+    cases.append(("quarter and half ulps", x, np.inf))
+    x = (rng.integers(0, 3, 32000) * 2.0 ** -24).astype(np.float32); x[5] = 0.75
+    cases.append(("zeros and ties", x, 0.7502))
+    cases.append(("powers of two", np.exp2(-rng.integers(0, 40, 32000).astype(np.float64)).astype(np.float32), np.inf))
+    cases.append(("tiny", rng.random(32768).astype(np.float32) * np.float32(1e-30), np.inf))
+    cases.append(("denormals", rng.random(5000).astype(np.float32) * np.float32(1e-41), np.inf))
+    x = np.zeros(32000, np.float32); x[31999] = 1
+    cases.append(("zeros", x, 0.5))
+    cases.append(("ones", np.ones(32768, np.float32), 20000.5))
+    cases.append(("flat", np.full(32000, 3.1e-5, np.float32), np.inf))
+    for n in (1, 2, 32, 33, 34, 65, 66, 67, 1000, 4097):
+        cases.append(("n = %d" % n, (rng.random(n) ** 8).astype(np.float32) * np.float32(10.0 ** rng.integers(-20, 3)), np.inf))
+        cases.append(("n = %d with a threshold" % n, rng.random(n).astype(np.float32), float(rng.random()) * n / 2))
+    for name, x, thr in cases:
+        ri, rs = _seq_sum_f32(x, thr)
+        gi, gs = inf.RunningSum(x, thr)
+        assert (gi, gs.tobytes()) == (ri, rs.tobytes()), (name, gi, gs, ri, rs)
+    inf.CleanUp()
+    cuda.Dispose()
+
+
 @pytest.mark.parametrize("topp", [0.9, 0.0])
 def test_sampled_generation_matches_checker(topp, tmp_path):
     """Token-id generation with temperature 0.8: ids equal to the checker's sampled loop with the same seed, graph replay
