@@ -10,9 +10,10 @@
  * pointer to device memory crosses this boundary.
  *
  * Only the function ids listed below are dispatched; every other id returns
- * MCH_ERROR_NOT_IMPLEMENTED with a message naming the id.  The Double entry
- * points exist and return MCH_ERROR_NOT_IMPLEMENTED (the hot path is fp32 and
- * 16-bit storage).
+ * MCH_ERROR_NOT_IMPLEMENTED with a message naming the id.  DLL_InvokeDouble and
+ * DLL_InvokeDoubleEx2 drive a second kernel table whose memory and arithmetic are
+ * double (the reference's Kernel<double>): the ids of the attention path are built
+ * for it, with plain kernels - see the comment at their declarations.
  */
 #ifndef MYCAFFE_HIP_ABI_H
 #define MYCAFFE_HIP_ABI_H
@@ -211,7 +212,15 @@ MCH_LONG DLL_InvokeFloatEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pI
                            MCH_TCHAR* pszInput, float** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr,
                            MCH_LONG lszErrMax);
 
-/* CudaDnnDLL.cpp:494-853: double twins; return MCH_ERROR_NOT_IMPLEMENTED here. */
+/* CudaDnnDLL.cpp:494-853: the double base type.  Kernel indices of these calls are their own table (dllmain.cpp:6-14),
+ * arrays cross the boundary as doubles, device memory holds doubles and every result is computed in double.  Built:
+ * INITIALIZE / CLEANUP / FREEMEM(-1), SETDEVICE, GETDEVICE, SYNCHRONIZEDEVICE, ALLOCMEM (ALLOCMEM_HALF allocates doubles
+ * too), FREEMEM, GETMEM, SETMEM, SET, COPY, GEMM, GEMM2, GEMV, AXPY, SCAL, SCALE, ADD, MUL, MASK, MASK_BATCH, TRANSPOSE,
+ * TRANSPOSE_HW, CHANNEL_COPY, EMBED_FWD, SILU_FWD, CREATE / FREE_CUDNN, CREATE / FREE / SET_TENSORDESC, SOFTMAX_FWD,
+ * ATTN_CREATE / FREE / SET / FWD (no dropout; the tenth and eleventh values of ATTN_FWD as on the float side),
+ * CREATE_ROPE / FREE_ROPE / ROPE_FWD - same packing as the float ids above.  These are one-element-per-thread kernels:
+ * the precision twin of the path, not a fast one.  Any other id, and DLL_InvokeDoubleEx (extensions and blob loaders
+ * are float objects), returns MCH_ERROR_NOT_IMPLEMENTED with the id in the message. */
 MCH_LONG DLL_InvokeDouble(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,
                           double** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
 MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,

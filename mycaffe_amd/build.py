@@ -27,7 +27,7 @@ FLAGS = [
 
 KERNEL_SOURCES = ["ew_kernels.hip", "gemm.hip", "attn_prefill.hip", "attn_flash2.hip", "attn_decode.hip", "attn_backward.hip"]
 LIBS = {
-    "libmycaffe_hip.so": KERNEL_SOURCES + ["library.hip"],
+    "libmycaffe_hip.so": KERNEL_SOURCES + ["library.hip", "library_f64.hip"],
     "libmycaffe_hip_llama2.so": KERNEL_SOURCES + ["llama2_ext.hip"],
 }
 

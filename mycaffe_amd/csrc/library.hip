@@ -2312,21 +2312,15 @@ MCH_LONG DLL_InvokeFloatEx(MCH_LONG k, MCH_LONG fn, float* pIn, MCH_LONG lIn, MC
     return (MCH_LONG)invoke(k, fn, pIn, lIn, nullptr, 0, pszIn, ppOut, plOut, szErr, errMax, true);
 }
 
+// The double base type's own entry points (DLL_InvokeDouble, DLL_InvokeDoubleEx2, Internal_GetPointerDouble) are in
+// library_f64.hip.  What stays unbuilt for it: the string-carrying calls, which only create extensions and blob loaders -
+// the llama2 extension is a float library (a double-typed parent fails cleanly at CREATE_EXTENSION).
 static MCH_LONG double_unsupported(MCH_TCHAR* szErr, MCH_LONG errMax)
 {
-    utf8_to_utf16("The double base type is not built: the attention hot path runs in fp32 and 16-bit storage. (90009)", szErr, errMax);
+    utf8_to_utf16("This call is not built for the double base type: extensions and blob loaders are float objects. (90009)", szErr, errMax);
     return MCH_ERROR_NOT_IMPLEMENTED;
 }
 
-MCH_LONG DLL_InvokeDouble(MCH_LONG, MCH_LONG, double*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR* szErr, MCH_LONG errMax)
-{
-    return double_unsupported(szErr, errMax);
-}
-MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG, MCH_LONG, double*, MCH_LONG, MCH_LONGLONG*, MCH_LONG, double**, MCH_LONG*, MCH_TCHAR* szErr,
-                             MCH_LONG errMax)
-{
-    return double_unsupported(szErr, errMax);
-}
 MCH_LONG DLL_InvokeDoubleEx(MCH_LONG, MCH_LONG, double*, MCH_LONG, MCH_TCHAR*, double**, MCH_LONG*, MCH_TCHAR* szErr, MCH_LONG errMax)
 {
     return double_unsupported(szErr, errMax);
@@ -2384,7 +2378,6 @@ MCH_LONG Internal_GetPointerFloat(int32_t ht, MCH_LONG kIdx, MCH_LONG h, void** 
     if (!k) return MCH_ERROR_PARAM_NULL;
     return (MCH_LONG)k->get_pointer(h, pp);
 }
-MCH_LONG Internal_GetPointerDouble(int32_t, MCH_LONG, MCH_LONG, void**) { return MCH_ERROR_NOT_IMPLEMENTED; }
 
 MCH_LONG Internal_AllocHostFloat(MCH_LONG kIdx, MCH_LONG count, float** dst, float* src, bool srcOnDevice)
 {

@@ -1,0 +1,998 @@
+// The double base type of the C ABI (DLL_InvokeDouble, DLL_InvokeDoubleEx2; CudaDnnDLL.cpp:494-853): a second kernel
+// table whose device memory holds doubles and whose arithmetic is double, as the reference's Kernel<double> instances
+// are (dllmain.cpp:6-14; the reference test base runs every test once per base type, TestBase.cs:107-115).
+//
+// It covers the function ids of the attention path - memory, GEMM / GEMM2 / GEMV and the vector updates, mask, the
+// transposes, channel copy, softmax forward, the attention handle's forward call, rotary embedding forward, embedding
+// lookup, SiLU - with plain kernels: one output element per thread, reductions by one workgroup per row, nothing tiled
+// for the matrix cores.  This is the precision twin of the fp32 path, for hosts that instantiate their layers in
+// double; the fast kernels are the fp32 / bf16 ones.  Every other id returns MCH_ERROR_NOT_IMPLEMENTED with its number
+// in the message.  ALLOCMEM_HALF allocates doubles (no 16-bit storage under this base type).
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "runtime.h"
+
+namespace mch {
+
+#define HIPCHK(x) do { hipError_t _e = (x); if (_e != hipSuccess) return (long)_e; } while (0)
+#define ERRCHK(x) do { long _e = (x); if (_e) return _e; } while (0)
+#define GRID_STRIDE(i, n) for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (n); i += (size_t)blockDim.x * gridDim.x)
+
+static inline int grid_of(size_t n)
+{
+    const size_t g = (n + 255) / 256;
+    return (int)(g < 1 ? 1 : g > 65535 ? 65535 : g);
+}
+
+// ---- kernels ----------------------------------------------------------------------------------------------------
+__global__ void d_set_kernel(size_t n, double* y, double v) { GRID_STRIDE(i, n) y[i] = v; }
+__global__ void d_axpy_kernel(size_t n, double a, const double* x, double* y) { GRID_STRIDE(i, n) y[i] = a * x[i] + y[i]; }
+__global__ void d_scale_kernel(size_t n, double a, const double* x, double* y) { GRID_STRIDE(i, n) y[i] = a * x[i]; }
+__global__ void d_add_kernel(size_t n, const double* a, const double* b, double* y, double alpha) { GRID_STRIDE(i, n) y[i] = a[i] + b[i] * alpha; }
+__global__ void d_mul_kernel(size_t n, const double* a, const double* b, double* y) { GRID_STRIDE(i, n) y[i] = a[i] * b[i]; }
+__global__ void d_silu_kernel(size_t n, const double* x, double* y) { GRID_STRIDE(i, n) y[i] = x[i] * (1.0 / (1.0 + exp(-x[i]))); }
+
+// mask index = i % md1 + (i / dd1) * md1 (math.cu:2995-3002, 3046-3056; the plain mask is the case dd1 = n)
+__global__ void d_mask_kernel(size_t n, size_t md1, size_t dd1, const double* x, const double* mask, double* y, double search, double replace)
+{
+    GRID_STRIDE(i, n) y[i] = mask[i % md1 + (i / dd1) * md1] == search ? replace : x[i];
+}
+
+// C(i,j) = alpha sum_k A(i,k) B(k,j) + beta C(i,j) for any element strides (row-major GEMM and column-major GEMM2 alike),
+// batched over blockIdx.z.  16 x 16 outputs per workgroup, K in slices of 16 through LDS.
+__global__ __launch_bounds__(256) void d_gemm_kernel(int m, int n, int k, double alpha, const double* A, long long ars, long long acs,
+                                                     const double* B, long long brs, long long bcs, double beta, double* C,
+                                                     long long crs, long long ccs, long long sA, long long sB, long long sC)
+{
+    __shared__ double as[16][17], bs[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int i = blockIdx.y * 16 + ty, j = blockIdx.x * 16 + tx;
+    A += (size_t)blockIdx.z * sA;
+    B += (size_t)blockIdx.z * sB;
+    C += (size_t)blockIdx.z * sC;
+    double acc = 0.0;
+    for (int k0 = 0; k0 < k; k0 += 16) {
+        as[ty][tx] = (i < m && k0 + tx < k) ? A[(long long)i * ars + (long long)(k0 + tx) * acs] : 0.0;
+        bs[ty][tx] = (k0 + ty < k && j < n) ? B[(long long)(k0 + ty) * brs + (long long)j * bcs] : 0.0;
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) acc += as[ty][kk] * bs[kk][tx];
+        __syncthreads();
+    }
+    if (i < m && j < n) {
+        double* c = C + (long long)i * crs + (long long)j * ccs;
+        *c = beta == 0.0 ? alpha * acc : alpha * acc + beta * *c;
+    }
+}
+
+struct PermuteD { int axes; long long xs[8], ys[8]; int map[8]; };
+__global__ void d_permute_kernel(size_t n, const double* x, double* y, PermuteD a)
+{
+    GRID_STRIDE(i, n)
+    {
+        long long from[8];
+        size_t rem = i;
+        for (int d = 0; d < a.axes; d++) {
+            from[d] = (long long)(rem / (size_t)a.xs[d]);
+            rem = rem % (size_t)a.xs[d];
+        }
+        size_t to = 0;
+        for (int d = 0; d < a.axes; d++) to += (size_t)from[a.map[d]] * (size_t)a.ys[d];
+        y[to] = x[i];
+    }
+}
+// (nc, h, w) -> (nc, w, h)
+__global__ void d_transpose_hw_kernel(size_t n, int h, int w, const double* x, double* y)
+{
+    GRID_STRIDE(o, n)
+    {
+        const size_t hw = (size_t)h * w, c = o / hw, r = o % hw;
+        const size_t ww = r / h, hh = r % h;
+        y[o] = x[c * hw + hh * w + ww];
+    }
+}
+__global__ void d_channel_copy_kernel(size_t n, int channels, int blocks, int inner, int offset, double* x, double* y, int dir)
+{
+    GRID_STRIDE(i, n)
+    {
+        const size_t nn = i / ((size_t)channels * inner), c = (i % ((size_t)channels * inner)) / inner, b = i % inner;
+        const size_t xi = (nn * channels + c) * (size_t)blocks * inner + (size_t)offset * inner + b;
+        if (dir == 0) y[i] = x[xi];
+        else x[xi] = y[i];
+    }
+}
+__global__ void d_embed_kernel(size_t count, const double* ids, const double* w, int N, double* top)
+{
+    GRID_STRIDE(i, count)
+    {
+        long long wi = (long long)ids[i / N] * N + (long long)(i % N);
+        if (wi < 0) wi = -wi;
+        top[i] = w[wi];
+    }
+}
+// pairs (2p, 2p+1) rotated by the angle of table entry ((p % wrap) / full) * half + p % half + off (rope.cu:725-825)
+__global__ void d_rope_kernel(size_t pairs, const double* x, double* y, const double* fcos, const double* fsin, size_t full,
+                              size_t wrap, int half, int off)
+{
+    GRID_STRIDE(p, pairs)
+    {
+        const size_t base = p % wrap, t = (base / full) * half + base % half + off;
+        const double c = fcos[t], sn = fsin[t], re = x[2 * p], im = x[2 * p + 1];
+        y[2 * p] = re * c - im * sn;
+        y[2 * p + 1] = re * sn + im * c;
+    }
+}
+
+__device__ inline double d_block_reduce(double v, double* red, bool isMax)
+{
+    for (int o = 32; o > 0; o >>= 1) {
+        const double u = __shfl_xor(v, o, 64);
+        v = isMax ? fmax(v, u) : v + u;
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    double r = red[0];
+    for (int w = 1; w < 4; w++) r = isMax ? fmax(r, red[w]) : r + red[w];
+    return r;
+}
+// softmax over `len` values `inner` apart, one workgroup per (outer, inner) pair; logsm: x - max - log(sum)
+__global__ __launch_bounds__(256) void d_softmax_kernel(const double* x, double* y, int len, int inner, bool logsm)
+{
+    __shared__ double red[4];
+    const size_t o = blockIdx.x / inner, in = blockIdx.x % inner, base = o * (size_t)len * inner + in;
+    double mx = -INFINITY;
+    for (int i = threadIdx.x; i < len; i += 256) mx = fmax(mx, x[base + (size_t)i * inner]);
+    mx = d_block_reduce(mx, red, true);
+    double sum = 0.0;
+    for (int i = threadIdx.x; i < len; i += 256) sum += exp(x[base + (size_t)i * inner] - mx);
+    sum = d_block_reduce(sum, red, false);
+    for (int i = threadIdx.x; i < len; i += 256) {
+        const double v = x[base + (size_t)i * inner] - mx;
+        y[base + (size_t)i * inner] = logsm ? v - log(sum) : exp(v) / sum;
+    }
+}
+
+// Attention forward as the reference's chain computes it (attn.cu:518-602): scores = scale q . k, masked ones -1e29,
+// softmax over the keys, y = p V.  One workgroup per (sequence, head, query row); the row of probabilities stays in LDS.
+// kind 0: no mask, 1: mask (Tq,Tk), 2: mask (B,Tk), 3: mask (B,Tq,Tk); merged: y written (B,Tq,H,hs)
+__global__ __launch_bounds__(256) void d_attn_row_kernel(const double* q, const double* k, const double* v, double* y, int H, int Tq,
+                                                         int Tk, int hs, double scale, const double* mask, int kind, bool merged)
+{
+    extern __shared__ double d_smem[];
+    double* p = d_smem;        // Tk
+    double* qs = p + Tk;       // hs
+    __shared__ double red[4];
+    const size_t row = blockIdx.x;
+    const int t = (int)(row % Tq);
+    const size_t bh = row / Tq;
+    const int h = (int)(bh % H);
+    const size_t b = bh / H;
+    const double* qr = q + row * hs;
+    const double* kb = k + bh * Tk * hs;
+    const double* vb = v + bh * Tk * hs;
+    for (int d = threadIdx.x; d < hs; d += 256) qs[d] = qr[d];
+    __syncthreads();
+    double mx = -INFINITY;
+    for (int j = threadIdx.x; j < Tk; j += 256) {
+        double s = 0.0;
+        for (int d = 0; d < hs; d++) s += qs[d] * kb[(size_t)j * hs + d];
+        s *= scale;
+        bool masked = false;
+        if (kind == 1) masked = mask[(size_t)t * Tk + j] == 0.0;
+        else if (kind == 2) masked = mask[b * Tk + j] == 0.0;
+        else if (kind == 3) masked = mask[(b * Tq + t) * Tk + j] == 0.0;
+        if (masked) s = -1e29;
+        p[j] = s;
+        mx = fmax(mx, s);
+    }
+    mx = d_block_reduce(mx, red, true);
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < Tk; j += 256) {
+        const double e = exp(p[j] - mx);
+        p[j] = e;
+        sum += e;
+    }
+    sum = d_block_reduce(sum, red, false);
+    double* yr = merged ? y + ((b * Tq + t) * H + h) * (size_t)hs : y + row * hs;
+    for (int d = threadIdx.x; d < hs; d += 256) {
+        double acc = 0.0;
+        for (int j = 0; j < Tk; j++) acc += p[j] * vb[(size_t)j * hs + d];
+        yr[d] = acc / sum;
+    }
+}
+
+// ---- the kernel object --------------------------------------------------------------------------------------------
+struct MemD { double* ptr = nullptr; size_t count = 0; bool used = false; };
+struct AttnD { bool set = false; int batch = 0, block = 0, heads = 0, hs = 0; double scale = 1.0; };
+struct RopeD { bool set = false; int seq = 0, heads = 0, hs = 0; double* dcos = nullptr; double* dsin = nullptr;
+               ~RopeD() { if (dcos) (void)hipFree(dcos); if (dsin) (void)hipFree(dsin); } };
+
+class KernelD {
+public:
+    ~KernelD()
+    {
+        if (m_stream) (void)hipStreamSynchronize(m_stream);
+        m_rope.clear();
+        for (MemD& m : m_mem)
+            if (m.used && m.ptr) (void)hipFree(m.ptr);
+        for (double* p : m_host) (void)hipHostFree(p);
+        if (m_stream) (void)hipStreamDestroy(m_stream);
+    }
+    long initialize(const double* pf, long n)
+    {
+        // SetDevice: f{deviceId, flags[, seed]} (device.cu:772-795)
+        if (n < 2 || n > 3) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (!pf) return MCH_ERROR_PARAM_NULL;
+        int count = 0;
+        HIPCHK(hipGetDeviceCount(&count));
+        const int dev = (int)pf[0];
+        if (dev < 0 || dev >= count) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        m_device = dev;
+        HIPCHK(hipSetDevice(dev));
+        if (!m_stream) HIPCHK(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking));
+        return 0;
+    }
+    long free_host(double* p)
+    {
+        for (size_t i = 0; i < m_host.size(); i++)
+            if (m_host[i] == p) {
+                m_host.erase(m_host.begin() + i);
+                HIPCHK(hipHostFree(p));
+                return 0;
+            }
+        return MCH_ERROR_MEMORY_NOT_FOUND;
+    }
+    long get_pointer(long h, void** pp)
+    {
+        MemD* it;
+        ERRCHK(mem(h, &it));
+        *pp = it->ptr;
+        return 0;
+    }
+    long run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, long ll, double** ppOut, MCH_LONG* plOut);
+    std::string last_detail;
+
+private:
+    long mem(long h, MemD** it)
+    {
+        if (h <= 0 || (size_t)h >= m_mem.size() || !m_mem[h].used) return MCH_ERROR_MEMORY_NOT_FOUND;
+        *it = &m_mem[h];
+        return 0;
+    }
+    long alloc(size_t count, long* h)
+    {
+        double* p = nullptr;
+        HIPCHK(hipMalloc((void**)&p, (count ? count : 1) * sizeof(double)));
+        hipError_t e = hipMemsetAsync(p, 0, (count ? count : 1) * sizeof(double), m_stream);
+        if (e != hipSuccess) { (void)hipFree(p); return (long)e; }
+        size_t slot = 0;
+        for (size_t i = 1; i < m_mem.size(); i++)
+            if (!m_mem[i].used) { slot = i; break; }
+        if (!slot) { m_mem.emplace_back(); slot = m_mem.size() - 1; }
+        m_mem[slot].ptr = p; m_mem[slot].count = count; m_mem[slot].used = true;
+        *h = (long)slot;
+        return 0;
+    }
+    int m_device = 0;
+    hipStream_t m_stream = nullptr;
+    std::vector<MemD> m_mem{1};
+    std::vector<double*> m_host;
+    HandleTable<CudnnState> m_cudnn;
+    HandleTable<TensorDesc> m_tdesc;
+    HandleTable<AttnD> m_attn;
+    HandleTable<RopeD> m_rope;
+};
+
+static inline long verify_d(long n, const void* p, long lo, long hi)
+{
+    if (n < lo || n > hi) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    if (lo == 0 && hi == 0) return 0;
+    if (!p) return MCH_ERROR_PARAM_NULL;
+    return 0;
+}
+static inline long set_out_d(double v, double** ppOut, MCH_LONG* plOut)
+{
+    if (!plOut || !ppOut || !*ppOut) return MCH_ERROR_PARAM_NULL;
+    if (*plOut < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    *plOut = 1;
+    (*ppOut)[0] = v;
+    return 0;
+}
+
+#define NEED_L(lo, hi) ERRCHK(verify_d(ll, pl, lo, hi))
+#define NEED_F(lo, hi) ERRCHK(verify_d(lf, pf, lo, hi))
+#define RANGE(item, off, n) do { if ((long long)(off) < 0 || (long long)(n) < 0 || (size_t)(off) + (size_t)(n) > (item)->count) { \
+        last_detail = "range exceeds the allocation behind the memory handle"; return MCH_ERROR_MEMORY_RANGE_EXCEEDED; } } while (0)
+#define LAUNCHED() HIPCHK(hipGetLastError())
+
+long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, long ll, double** ppOut, MCH_LONG* plOut)
+{
+    last_detail.clear();
+    hipStream_t s = m_stream;
+    if (!s) return MCH_ERROR_DEVICE_NOT_INITIALIZED;
+    HIPCHK(hipSetDevice(m_device));
+    switch (fn) {
+    case MCH_FN_SETDEVICE:
+        return initialize(pf, lf);
+    case MCH_FN_GETDEVICE:
+        return set_out_d((double)m_device, ppOut, plOut);
+    case MCH_FN_SYNCHRONIZEDEVICE:
+        HIPCHK(hipStreamSynchronize(s));
+        return 0;
+
+    // ---- memory (device.cu:854-1091) ----------------------------------------------------------------------------
+    case MCH_FN_ALLOCMEM:
+    case MCH_FN_ALLOCMEM_HALF: {
+        // l{count[,stream]}; optional f{count,[stream,] data...}
+        NEED_L(1, 2);
+        if (pl[0] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const size_t count = (size_t)pl[0];
+        const double* src = nullptr;
+        if (lf > 1) {
+            if (!pf) return MCH_ERROR_PARAM_NULL;
+            if ((size_t)lf == count + 1) src = pf + 1;
+            else if ((size_t)lf == count + 2) src = pf + 2;
+            else return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        long h = 0;
+        ERRCHK(alloc(count, &h));
+        if (src && count) {
+            hipError_t e = hipMemcpyAsync(m_mem[h].ptr, src, count * 8, hipMemcpyHostToDevice, s);
+            if (e == hipSuccess) e = hipStreamSynchronize(s);
+            if (e != hipSuccess) { (void)hipFree(m_mem[h].ptr); m_mem[h] = MemD(); return (long)e; }
+        }
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_FREEMEM: {
+        NEED_L(1, 1);
+        MemD* it;
+        ERRCHK(mem((long)pl[0], &it));
+        HIPCHK(hipStreamSynchronize(s));
+        HIPCHK(hipFree(it->ptr));
+        *it = MemD();
+        return 0;
+    }
+    case MCH_FN_GETMEM: {
+        // l{h, count(-1 = all)}
+        NEED_L(1, 2);
+        if (!plOut || !ppOut) return MCH_ERROR_PARAM_NULL;
+        MemD* it;
+        ERRCHK(mem((long)pl[0], &it));
+        long long count = ll > 1 ? pl[1] : 0;
+        if (count < 0) count = (long long)it->count;
+        else if ((size_t)count > it->count) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (count > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        double* dst = *ppOut;
+        if (!(count <= *plOut && dst)) {
+            HIPCHK(hipHostMalloc((void**)&dst, (size_t)(count > 0 ? count : 1) * 8, hipHostMallocDefault));
+            m_host.push_back(dst);
+            *ppOut = dst;   // handed back with DLL_FREEMEM
+        }
+        if (count) HIPCHK(hipMemcpyAsync(dst, it->ptr, (size_t)count * 8, hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        *plOut = (MCH_LONG)count;
+        return 0;
+    }
+    case MCH_FN_SETMEM: {
+        // f{h, count, [stream,] data...}, l{h, count}
+        NEED_F(2, INT_MAX);
+        NEED_L(2, 2);
+        if (pl[1] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const size_t count = (size_t)pl[1];
+        const double* data;
+        if (count == (size_t)lf - 2) data = pf + 2;
+        else if (count == (size_t)lf - 3) data = pf + 3;
+        else return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD* it;
+        ERRCHK(mem((long)pl[0], &it));
+        RANGE(it, 0, count);
+        if (count) HIPCHK(hipMemcpyAsync(it->ptr, data, count * 8, hipMemcpyHostToDevice, s));
+        HIPCHK(hipStreamSynchronize(s));
+        return 0;
+    }
+    case MCH_FN_SET: {
+        // f{val}, l{n, h, 0, idx, xOff} (device.h:6038-6061)
+        NEED_F(1, 1);
+        NEED_L(3, 5);
+        const long long n = pl[0], idx = ll > 3 ? pl[3] : -1;
+        long long off = ll > 4 ? pl[4] : 0;
+        MemD* it;
+        ERRCHK(mem((long)pl[1], &it));
+        if (off < 0) off = 0;
+        if (idx >= 0) {
+            RANGE(it, off + idx, 1);
+            hipLaunchKernelGGL(d_set_kernel, 1, 256, 0, s, (size_t)1, it->ptr + off + idx, pf[0]);
+        } else {
+            RANGE(it, off, n);
+            if (n) hipLaunchKernelGGL(d_set_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, it->ptr + off, pf[0]);
+        }
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_COPY: {
+        // l{n, hSrc, hDst, srcOff, dstOff, ...} (device.h:6063-6095)
+        NEED_L(3, 8);
+        const long long n = pl[0];
+        long long so = ll > 3 ? pl[3] : 0, dofs = ll > 4 ? pl[4] : 0;
+        MemD *src, *dst;
+        ERRCHK(mem((long)pl[1], &src));
+        ERRCHK(mem((long)pl[2], &dst));
+        if (so < 0) so = 0;
+        if (dofs < 0) dofs = 0;
+        RANGE(src, so, n);
+        RANGE(dst, dofs, n);
+        if (n) HIPCHK(hipMemcpyAsync(dst->ptr + dofs, src->ptr + so, (size_t)n * 8, hipMemcpyDeviceToDevice, s));
+        return 0;
+    }
+
+    // ---- BLAS-like (device.cu:1636-2051) ----------------------------------------------------------------------------
+    case MCH_FN_GEMM: {
+        // f{alpha,beta}, l{tA,tB,m,n,k,0,hA,hB,0,hC,aOff,bOff,cOff,groups,gA,gB,gC}: row-major C = alpha op(A) op(B) + beta C
+        NEED_F(2, 2);
+        NEED_L(10, 17);
+        const bool tA = pl[0] != 0, tB = pl[1] != 0;
+        const int m = (int)pl[2], n = (int)pl[3], k = (int)pl[4];
+        long long aOff = ll > 10 ? pl[10] : 0, bOff = ll > 11 ? pl[11] : 0, cOff = ll > 12 ? pl[12] : 0;
+        const int groups = ll > 13 ? (int)pl[13] : 1;
+        const long long gA = ll > 14 ? pl[14] : 0, gB = ll > 15 ? pl[15] : 0, gC = ll > 16 ? pl[16] : 0;
+        if (m < 0 || n < 0 || k < 0 || groups < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *A, *B, *C;
+        ERRCHK(mem((long)pl[6], &A));
+        ERRCHK(mem((long)pl[7], &B));
+        ERRCHK(mem((long)pl[9], &C));
+        if (aOff < 0) aOff = 0;
+        if (bOff < 0) bOff = 0;
+        if (cOff < 0) cOff = 0;
+        for (int g = 0; g < groups; g++) {
+            const long long ao = aOff + gA * g, bo = bOff + gB * g, co = cOff + gC * g;
+            RANGE(A, ao, (long long)m * k);
+            RANGE(B, bo, (long long)k * n);
+            RANGE(C, co, (long long)m * n);
+            if (m == 0 || n == 0) continue;
+            hipLaunchKernelGGL(d_gemm_kernel, dim3((n + 15) / 16, (m + 15) / 16, 1), 256, 0, s, m, n, k, pf[0], A->ptr + ao,
+                               tA ? 1ll : (long long)k, tA ? (long long)m : 1ll, B->ptr + bo, tB ? 1ll : (long long)n,
+                               tB ? (long long)k : 1ll, pf[1], C->ptr + co, (long long)n, 1ll, 0ll, 0ll, 0ll);
+            LAUNCHED();
+        }
+        return 0;
+    }
+    case MCH_FN_GEMM2: {
+        // f{alpha,beta}, l{tA,tB,m,n,k,0,hA,hB,0,hC,lda,ldb,ldc[,sA,sB,sC,batch]}: BLAS column-major (device.cu:1691-1726)
+        NEED_F(2, 2);
+        NEED_L(13, 17);
+        if (ll != 13 && ll != 17) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const bool tA = pl[0] != 0, tB = pl[1] != 0;
+        const int m = (int)pl[2], n = (int)pl[3], k = (int)pl[4];
+        const long long lda = pl[10], ldb = pl[11], ldc = pl[12];
+        long long sA = 0, sB = 0, sC = 0;
+        int batch = 1;
+        if (ll == 17) { sA = pl[13]; sB = pl[14]; sC = pl[15]; batch = (int)pl[16]; }
+        if (m < 0 || n < 0 || k < 0 || batch < 1 || batch > 65535 || lda < 1 || ldb < 1 || ldc < 1 || sA < 0 || sB < 0 || sC < 0)
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *A, *B, *C;
+        ERRCHK(mem((long)pl[6], &A));
+        ERRCHK(mem((long)pl[7], &B));
+        ERRCHK(mem((long)pl[9], &C));
+        if (m == 0 || n == 0) return 0;
+        const long long ac = tA ? m : k, bc = tB ? k : n, ar = tA ? k : m, br = tB ? n : k;   // stored columns / rows
+        RANGE(A, 0, (batch - 1) * sA + (ac - 1) * lda + ar);
+        RANGE(B, 0, (batch - 1) * sB + (bc - 1) * ldb + br);
+        RANGE(C, 0, (batch - 1) * sC + (long long)(n - 1) * ldc + m);
+        // column-major: element (i, kk) of op(A) is A[i + kk lda], or A[kk + i lda] when transposed
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((n + 15) / 16, (m + 15) / 16, batch), 256, 0, s, m, n, k, pf[0], A->ptr,
+                           tA ? lda : 1ll, tA ? 1ll : lda, B->ptr, tB ? ldb : 1ll, tB ? 1ll : ldb, pf[1], C->ptr, 1ll, ldc, sA, sB, sC);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_GEMV: {
+        // f{alpha,beta}, l{tA,m,n,0,hA,hX,0,hY,aOff,xOff,yOff}: A row-major (m, n); y = alpha op(A) x + beta y
+        NEED_F(2, 2);
+        NEED_L(8, 11);
+        const bool tA = pl[0] != 0;
+        const int m = (int)pl[1], n = (int)pl[2];
+        long long aOff = ll > 8 ? pl[8] : 0, xOff = ll > 9 ? pl[9] : 0, yOff = ll > 10 ? pl[10] : 0;
+        if (m < 0 || n < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *A, *X, *Y;
+        ERRCHK(mem((long)pl[4], &A));
+        ERRCHK(mem((long)pl[5], &X));
+        ERRCHK(mem((long)pl[7], &Y));
+        if (aOff < 0) aOff = 0;
+        if (xOff < 0) xOff = 0;
+        if (yOff < 0) yOff = 0;
+        RANGE(A, aOff, (long long)m * n);
+        RANGE(X, xOff, tA ? m : n);
+        RANGE(Y, yOff, tA ? n : m);
+        const int rows = tA ? n : m, inner = tA ? m : n;   // y (rows) = op(A) (rows x inner) x (inner)
+        if (rows == 0) return 0;
+        hipLaunchKernelGGL(d_gemm_kernel, dim3(1, (rows + 15) / 16, 1), 256, 0, s, rows, 1, inner, pf[0], A->ptr + aOff,
+                           tA ? 1ll : (long long)n, tA ? (long long)n : 1ll, X->ptr + xOff, 1ll, 1ll, pf[1], Y->ptr + yOff, 1ll, 1ll,
+                           0ll, 0ll, 0ll);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_AXPY: {
+        // f{alpha}, l{n,0,hX,hY,xOff,yOff}
+        NEED_F(1, 1);
+        NEED_L(4, 6);
+        const long long n = pl[0], xo = ll > 4 ? pl[4] : 0, yo = ll > 5 ? pl[5] : 0;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_axpy_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, pf[0], X->ptr + xo, Y->ptr + yo);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_SCAL:
+    case MCH_FN_SCALE: {
+        // SCAL f{alpha}, l{n,0,hX,xOff}; SCALE f{alpha}, l{n,0,hX,hY,xOff,yOff}
+        NEED_F(1, 1);
+        const bool inplace = fn == MCH_FN_SCAL;
+        if (inplace) NEED_L(3, 4); else NEED_L(4, 6);
+        const long long n = pl[0];
+        const long long xo = inplace ? (ll > 3 ? pl[3] : 0) : (ll > 4 ? pl[4] : 0), yo = inplace ? xo : (ll > 5 ? pl[5] : 0);
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[inplace ? 2 : 3], &Y));
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_scale_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, pf[0], X->ptr + xo, Y->ptr + yo);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_ADD: {
+        // [f{alpha}], l{n,hA,hB,hY}: y = a + alpha b (math.cu:3363-3369)
+        if (lf > 0 && pf) NEED_F(1, 1);
+        NEED_L(4, 5);
+        const long long n = pl[0];
+        const double alpha = (lf > 0 && pf) ? pf[0] : 1.0;
+        MemD *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        if (n) hipLaunchKernelGGL(d_add_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, A->ptr, B->ptr, Y->ptr, alpha);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_MUL: {
+        // l{n,hA,hB,hY,aOff,bOff,yOff}
+        NEED_L(4, 7);
+        const long long n = pl[0], ao = ll > 4 ? pl[4] : 0, bo = ll > 5 ? pl[5] : 0, yo = ll > 6 ? pl[6] : 0;
+        MemD *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(A, ao, n);
+        RANGE(B, bo, n);
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_mul_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, A->ptr + ao, B->ptr + bo, Y->ptr + yo);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_SILU_FWD: {
+        // l{count,hBtm,hTop}
+        NEED_L(3, 3);
+        const long long n = pl[0];
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        if (n) hipLaunchKernelGGL(d_silu_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, X->ptr, Y->ptr);
+        LAUNCHED();
+        return 0;
+    }
+
+    // ---- mask, layout (device.cu:2101-2145, 3088-3127, 3730-3748) --------------------------------------------------------
+    case MCH_FN_MASK:
+    case MCH_FN_MASK_BATCH: {
+        // MASK f{search,replace}, l{n,maskDim,0,0,hX,hMask,hY}; MASK_BATCH l{n,batch,maskDim,0,0,hX,hMask,hY}
+        NEED_F(2, 2);
+        const bool batched = fn == MCH_FN_MASK_BATCH;
+        if (batched) NEED_L(8, 8); else NEED_L(7, 7);
+        const long long n = pl[0];
+        const long long batch = batched ? pl[1] : 1, md = batched ? pl[2] : pl[1];
+        if (md < 1 || batch < 1 || md < batch || (batched && n < batch)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const int o = batched ? 5 : 4;
+        MemD *X, *M, *Y;
+        ERRCHK(mem((long)pl[o], &X));
+        ERRCHK(mem((long)pl[o + 1], &M));
+        ERRCHK(mem((long)pl[o + 2], &Y));
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        if (n == 0) return 0;
+        const long long md1 = batched ? md / batch : md, dd1 = batched ? n / batch : n;
+        RANGE(M, 0, batched ? (md1 - 1) + ((n - 1) / dd1) * md1 + 1 : md);
+        hipLaunchKernelGGL(d_mask_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (size_t)md1, (size_t)dd1, X->ptr, M->ptr, Y->ptr,
+                           pf[0], pf[1]);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_TRANSPOSE: {
+        // l{n,hX,hY,hXCounts,hYCounts,hMapping,numAxes,hBuffer}: the three small blobs hold element strides and the axis map
+        NEED_L(8, 8);
+        const long long n = pl[0];
+        const int axes = (int)pl[6];
+        MemD *X, *Y, *XC, *YC, *MP;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        ERRCHK(mem((long)pl[3], &XC));
+        ERRCHK(mem((long)pl[4], &YC));
+        ERRCHK(mem((long)pl[5], &MP));
+        if (axes < 1 || axes > 8) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        RANGE(XC, 0, axes);
+        RANGE(YC, 0, axes);
+        RANGE(MP, 0, axes);
+        double hx[8], hy[8], hm[8];
+        HIPCHK(hipMemcpyAsync(hx, XC->ptr, axes * 8, hipMemcpyDeviceToHost, s));
+        HIPCHK(hipMemcpyAsync(hy, YC->ptr, axes * 8, hipMemcpyDeviceToHost, s));
+        HIPCHK(hipMemcpyAsync(hm, MP->ptr, axes * 8, hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        PermuteD a;
+        a.axes = axes;
+        for (int i = 0; i < axes; i++) {
+            a.xs[i] = (long long)hx[i]; a.ys[i] = (long long)hy[i]; a.map[i] = (int)hm[i];
+            if (a.xs[i] < 1 || a.ys[i] < 1 || a.map[i] < 0 || a.map[i] >= axes) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        if (n) hipLaunchKernelGGL(d_permute_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, X->ptr, Y->ptr, a);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_TRANSPOSE_HW: {
+        // l{n,c,h,w,hSrc,hDst}
+        NEED_L(6, 6);
+        const long long nn = pl[0], c = pl[1], h = pl[2], w = pl[3];
+        if (nn < 0 || c < 0 || h < 0 || w < 0 || h > INT_MAX || w > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        const long long total = nn * c * h * w;
+        RANGE(X, 0, total);
+        RANGE(Y, 0, total);
+        if (total) hipLaunchKernelGGL(d_transpose_hw_kernel, grid_of((size_t)total), 256, 0, s, (size_t)total, (int)h, (int)w, X->ptr, Y->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_COPY: {
+        // l{count,outer,channels,blocks,inner,offset,hX,hY,dir}
+        NEED_L(9, 9);
+        const long long n = pl[0], chn = pl[2], blocks = pl[3], inner = pl[4], off = pl[5];
+        const int dir = (int)pl[8];
+        if (n < 0 || chn < 1 || blocks < 1 || inner < 1 || off < 0 || off >= blocks) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[6], &X));
+        ERRCHK(mem((long)pl[7], &Y));
+        RANGE(Y, 0, n);
+        if (n == 0) return 0;
+        const long long last = n - 1;
+        const long long xi = ((last / (chn * inner)) * chn + (last % (chn * inner)) / inner) * blocks * inner + off * inner + last % inner;
+        RANGE(X, 0, xi + (inner - 1 - last % inner) + 1);
+        hipLaunchKernelGGL(d_channel_copy_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (int)chn, (int)blocks, (int)inner, (int)off,
+                           X->ptr, Y->ptr, dir);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_EMBED_FWD: {
+        // l{count,hBtm,hWeight,M,N,K,hTop} (math.cu:9314-9330)
+        NEED_L(7, 7);
+        const long long n = pl[0], N = pl[4], K = pl[5];
+        if (n < 0 || N < 1 || K < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *I, *W, *T;
+        ERRCHK(mem((long)pl[1], &I));
+        ERRCHK(mem((long)pl[2], &W));
+        ERRCHK(mem((long)pl[6], &T));
+        RANGE(T, 0, n);
+        RANGE(I, 0, (n + N - 1) / N);
+        RANGE(W, 0, K * N);
+        if (n) hipLaunchKernelGGL(d_embed_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, I->ptr, W->ptr, (int)N, T->ptr);
+        LAUNCHED();
+        return 0;
+    }
+
+    // ---- descriptors, softmax (device.h:1201-1262, 4778-4798) -----------------------------------------------------------
+    case MCH_FN_CREATE_CUDNN: {
+        ERRCHK(verify_d(lf, pf, 0, 1));
+        long h;
+        ERRCHK(m_cudnn.create(&h));
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_CUDNN:
+        NEED_F(1, 1);
+        return m_cudnn.free((long)pf[0]);
+    case MCH_FN_CREATE_TENSORDESC: {
+        long h;
+        ERRCHK(m_tdesc.create(&h));
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_TENSORDESC:
+        NEED_F(1, 1);
+        return m_tdesc.free((long)pf[0]);
+    case MCH_FN_SET_TENSORDESC: {
+        // l{h,half,n,c,h,w[,sn,sc,sh,sw]}
+        NEED_L(6, 10);
+        if (ll != 6 && ll != 10) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        TensorDesc* d = m_tdesc.get((long)pl[0]);
+        if (!d) return MCH_ERROR_PARAM_NULL;
+        d->half = false;
+        d->n = (int)pl[2]; d->c = (int)pl[3]; d->h = (int)pl[4]; d->w = (int)pl[5];
+        if (ll == 6) { d->sw = 1; d->sh = d->w; d->sc = d->h * d->sh; d->sn = d->c * d->sc; }
+        else { d->sn = (int)pl[6]; d->sc = (int)pl[7]; d->sh = (int)pl[8]; d->sw = (int)pl[9]; }
+        return 0;
+    }
+    case MCH_FN_SOFTMAX_FWD: {
+        // f{alpha,beta}, l{hCudnn,0,hBtmDesc,hBtm,0,hTopDesc,hTop,alg,mode}
+        NEED_F(2, 2);
+        NEED_L(9, 9);
+        if (!m_cudnn.get((long)pl[0])) return MCH_ERROR_PARAM_NULL;
+        TensorDesc* bd = m_tdesc.get((long)pl[2]);
+        TensorDesc* td = m_tdesc.get((long)pl[5]);
+        if (!bd || !td) return MCH_ERROR_PARAM_NULL;
+        if (pf[0] != 1.0 || pf[1] != 0.0) { last_detail = "softmax supports alpha=1, beta=0 only"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const int alg = (int)pl[7], mode = (int)pl[8];   // alg 0 fast, 1 accurate, 2 log; mode 0 instance, 1 channel
+        if (alg < 0 || alg > 2 || mode < 0 || mode > 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (bd->n != td->n || bd->c != td->c || bd->h != td->h || bd->w != td->w) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const bool packed = bd->sw == 1 && bd->sh == bd->w && bd->sc == bd->h * bd->w && bd->sn == bd->c * bd->h * bd->w &&
+                            td->sw == 1 && td->sh == td->w && td->sc == td->h * td->w && td->sn == td->c * td->h * td->w;
+        if (!packed) { last_detail = "softmax needs fully packed NCHW descriptors"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const long long total = (long long)bd->n * bd->c * bd->h * bd->w;
+        const int len = mode == 0 ? bd->c * bd->h * bd->w : bd->c, inner = mode == 0 ? 1 : bd->h * bd->w;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[3], &X));
+        ERRCHK(mem((long)pl[6], &Y));
+        RANGE(X, 0, total);
+        RANGE(Y, 0, total);
+        const long long rows = (long long)bd->n * inner;
+        if (total == 0) return 0;
+        if (rows > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        hipLaunchKernelGGL(d_softmax_kernel, (int)rows, 256, 0, s, (const double*)X->ptr, Y->ptr, len, inner, alg == 2);
+        LAUNCHED();
+        return 0;
+    }
+
+    // ---- attention handle (device.h:2435-2506, attn.cu:408-602) ------------------------------------------------------------
+    case MCH_FN_ATTN_CREATE: {
+        long h;
+        ERRCHK(m_attn.create(&h));
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_ATTN_FREE:
+        NEED_F(1, 1);
+        return m_attn.free((long)pf[0]);
+    case MCH_FN_ATTN_SET: {
+        // f{dropout}, l{hCudnn,hAttn,gpuId,training,batch,blockSize,heads,hs,seed}
+        NEED_L(9, 9);
+        NEED_F(1, 1);
+        AttnD* st = m_attn.get((long)pl[1]);
+        if (!st) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        if (pl[4] < 1 || pl[5] < 1 || pl[6] < 1 || pl[7] < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (pl[3] != 0 && pf[0] != 0.0) {
+            last_detail = "the double base type runs the attention handle without dropout";
+            return MCH_ERROR_NOT_IMPLEMENTED;
+        }
+        st->batch = (int)pl[4]; st->block = (int)pl[5]; st->heads = (int)pl[6]; st->hs = (int)pl[7];
+        st->scale = 1.0 / sqrt((double)st->hs);   // attn.cu:427
+        st->set = true;
+        return 0;
+    }
+    case MCH_FN_ATTN_FWD: {
+        // l{hCudnn,hAttn,blockSize,hQ,hK,hV,hMask,hY,batchMask[,blockSizeK[,mergedY]]}; the tenth and eleventh values as in the
+        // fp32 library (key length when it differs, Y written head-merged)
+        NEED_L(9, 11);
+        AttnD* st = m_attn.get((long)pl[1]);
+        if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        const int T = (int)pl[2], Tk = ll > 9 ? (int)pl[9] : T;
+        const bool merged = ll > 10 && pl[10] != 0;
+        if (T > st->block || Tk > st->block) return MCH_ERROR_ATTN_INVALID_BLOCK_SIZE;
+        if (T < 1 || Tk < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *Q, *K, *V, *Y, *M = nullptr;
+        ERRCHK(mem((long)pl[3], &Q));
+        ERRCHK(mem((long)pl[4], &K));
+        ERRCHK(mem((long)pl[5], &V));
+        ERRCHK(mem((long)pl[7], &Y));
+        const long long batchMask = pl[8];   // 0: (1,1,T,T); 1: (B,T,1,1); 2: (B,T,T)
+        if (batchMask < 0 || batchMask > 2) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (pl[6]) ERRCHK(mem((long)pl[6], &M));
+        const long long qn = (long long)st->batch * st->heads * T * st->hs, kn = (long long)st->batch * st->heads * Tk * st->hs;
+        if ((long long)Q->count < qn || (long long)Y->count < qn || (long long)K->count < kn || (long long)V->count < kn)
+            return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+        int kind = 0;
+        if (M) {
+            const long long need = batchMask == 2 ? (long long)st->batch * T * Tk : batchMask == 1 ? (long long)st->batch * Tk : (long long)T * Tk;
+            if ((long long)M->count < need) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+            kind = batchMask == 2 ? 3 : batchMask == 1 ? 2 : 1;
+        }
+        const size_t lds = ((size_t)Tk + st->hs) * sizeof(double);
+        if (lds > 60000) { last_detail = "the double attention call keeps a row of scores in LDS: up to about 7000 keys"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const long long rows = (long long)st->batch * st->heads * T;
+        if (rows > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        hipLaunchKernelGGL(d_attn_row_kernel, (int)rows, 256, lds, s, (const double*)Q->ptr, (const double*)K->ptr, (const double*)V->ptr,
+                           Y->ptr, st->heads, T, Tk, st->hs, st->scale, M ? (const double*)M->ptr : nullptr, kind, merged);
+        LAUNCHED();
+        return 0;
+    }
+
+    // ---- rotary embedding (device.h:4201-4263, rope.cu:502-607, 785-825) ----------------------------------------------------
+    case MCH_FN_CREATE_ROPE: {
+        // f{theta}, l{sharedIdx,gpuId,count,batch,seqLen,heads,hs}
+        NEED_F(1, 1);
+        NEED_L(7, 7);
+        const long long seq = pl[4], heads = pl[5], hs = pl[6];
+        if (seq < 1 || heads < 1 || hs < 2 || (hs & 1) || seq * hs > (1ll << 30)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        long h;
+        ERRCHK(m_rope.create(&h));
+        RopeD* r = m_rope.get(h);
+        r->seq = (int)seq; r->heads = (int)heads; r->hs = (int)hs;
+        const int half = (int)hs / 2;
+        // the reference's host tables for T = double (rope.cu:535-553): the power and the cosines are single-precision
+        // library calls on values held in double
+        std::vector<double> freq(half), hc((size_t)seq * half), hsn((size_t)seq * half);
+        for (int i = 0, j = 0; i < (int)hs; i += 2, j++) {
+            double power = (double)(i / (double)hs);
+            power = (double)powf((float)pf[0], (float)power);
+            freq[j] = 1.0 / power;
+        }
+        for (long long pos = 0; pos < seq; pos++)
+            for (int i = 0; i < half; i++) {
+                const double fpos = freq[i] * (double)pos;
+                hc[(size_t)pos * half + i] = (double)cosf((float)fpos);
+                hsn[(size_t)pos * half + i] = (double)sinf((float)fpos);
+            }
+        long e = 0;
+        hipError_t he = hipMalloc((void**)&r->dcos, hc.size() * 8);
+        if (he == hipSuccess) he = hipMalloc((void**)&r->dsin, hsn.size() * 8);
+        if (he == hipSuccess) he = hipMemcpyAsync(r->dcos, hc.data(), hc.size() * 8, hipMemcpyHostToDevice, s);
+        if (he == hipSuccess) he = hipMemcpyAsync(r->dsin, hsn.data(), hsn.size() * 8, hipMemcpyHostToDevice, s);
+        if (he == hipSuccess) he = hipStreamSynchronize(s);
+        if (he != hipSuccess) e = (long)he;
+        if (e) { m_rope.free(h); return e; }
+        r->set = true;
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_ROPE:
+        NEED_F(1, 1);
+        HIPCHK(hipStreamSynchronize(s));
+        return m_rope.free((long)pf[0]);
+    case MCH_FN_ROPE_FWD: {
+        // l{hRope,n,hX,hY[,freqOffset]}
+        NEED_L(4, 5);
+        RopeD* r = m_rope.get((long)pl[0]);
+        if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+        const long long n = pl[1];
+        long long off = ll > 4 ? pl[4] : -1;
+        if (off < 0) off = 0;   // offsets <= 0 mean "no shift" (rope.cu:808-814)
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (n < 0 || (n & 1)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        const long long half = r->hs / 2, full = half * r->heads, wrap = (long long)r->seq * full, pairs = n / 2;
+        const long long maxbase = (pairs < wrap ? pairs : wrap) - 1;
+        if (pairs > 0 && (maxbase / full) * half + (half - 1) + off >= (long long)r->seq * half) {
+            last_detail = "rope table offset reaches past the last position of the table";
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        if (pairs) hipLaunchKernelGGL(d_rope_kernel, grid_of((size_t)pairs), 256, 0, s, (size_t)pairs, (const double*)X->ptr, Y->ptr,
+                                      (const double*)r->dcos, (const double*)r->dsin, (size_t)full, (size_t)wrap, (int)half, (int)off);
+        LAUNCHED();
+        return 0;
+    }
+    default:
+        break;
+    }
+    char buf[160];
+    snprintf(buf, sizeof(buf), "function id %ld is not built for the double base type (the attention path's ids are)", fn);
+    last_detail = buf;
+    return MCH_ERROR_NOT_IMPLEMENTED;
+}
+
+// ---- kernel table and entry points ----------------------------------------------------------------------------------
+static const int MAX_KERNELS_D = 2048;   // CudaDnnDLL/main.h:21
+static KernelD* g_kernelsD[MAX_KERNELS_D];
+static std::mutex g_tableLockD;
+
+static KernelD* kernel_d(long idx)
+{
+    if (idx <= 0 || idx >= MAX_KERNELS_D) return nullptr;
+    std::lock_guard<std::mutex> g(g_tableLockD);
+    return g_kernelsD[idx];
+}
+static void put_error_d(KernelD* k, long e, MCH_TCHAR* szErr, long max)
+{
+    if (!szErr || max <= 0) return;
+    char buf[512];
+    if (k && !k->last_detail.empty()) snprintf(buf, sizeof(buf), "%s (%ld)", k->last_detail.c_str(), e);
+    else if (e > 0 && e < 2000) snprintf(buf, sizeof(buf), "HIP runtime error: %s (%ld)", hipGetErrorString((hipError_t)e), e);
+    else snprintf(buf, sizeof(buf), "error %ld in the double base type's call", e);
+    utf8_to_utf16(buf, szErr, max);
+}
+
+static long invoke_d(long kIdx, long fn, double* pf, long lf, MCH_LONGLONG* pl, long ll, double** ppOut, MCH_LONG* plOut, MCH_TCHAR* szErr,
+                     long errMax)
+{
+    if (szErr && errMax > 0) szErr[0] = 0;
+    if (kIdx < 0 || kIdx >= MAX_KERNELS_D) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    long e = 0;
+    KernelD* k = nullptr;
+    switch (fn) {
+    case MCH_DLL_INITIALIZE: {
+        // creates a kernel, returns its index in (*ppOutput)[0] (CudaDnnDLL.cpp:154-176)
+        if (!ppOut || !*ppOut || !plOut) return MCH_ERROR_PARAM_NULL;
+        k = new KernelD();
+        e = k->initialize(pf, lf);
+        if (e) { put_error_d(k, e, szErr, errMax); delete k; return e; }
+        long slot = -1;
+        {
+            std::lock_guard<std::mutex> g(g_tableLockD);
+            for (int i = 1; i < MAX_KERNELS_D; i++)
+                if (!g_kernelsD[i]) { g_kernelsD[i] = k; slot = i; break; }
+        }
+        if (slot < 0) { delete k; e = MCH_ERROR_MEMORY_OUT; put_error_d(nullptr, e, szErr, errMax); return e; }
+        (*ppOut)[0] = (double)slot;
+        *plOut = 1;
+        return 0;
+    }
+    case MCH_DLL_CLEANUP: {
+        std::lock_guard<std::mutex> g(g_tableLockD);
+        k = g_kernelsD[kIdx];
+        g_kernelsD[kIdx] = nullptr;
+        delete k;
+        return 0;
+    }
+    case MCH_DLL_FREEMEM:
+        if (!(k = kernel_d(kIdx))) { e = MCH_ERROR_PARAM_NULL; put_error_d(nullptr, e, szErr, errMax); return e; }
+        e = k->free_host(pf);
+        if (e) put_error_d(k, e, szErr, errMax);
+        return e;
+    default:
+        break;
+    }
+    if (!(k = kernel_d(kIdx))) { e = MCH_ERROR_PARAM_NULL; put_error_d(nullptr, e, szErr, errMax); return e; }
+    e = k->run(fn, pf, lf, pl, ll, ppOut, plOut);
+    if (e) put_error_d(k, e, szErr, errMax);
+    return e;
+}
+
+}  // namespace mch
+
+using namespace mch;
+
+extern "C" {
+
+MCH_LONG DLL_InvokeDouble(MCH_LONG k, MCH_LONG fn, double* pIn, MCH_LONG lIn, double** ppOut, MCH_LONG* plOut, MCH_TCHAR* szErr,
+                          MCH_LONG errMax)
+{
+    // the legacy entry point forwards no integer array (CudaDnnDLL.cpp:303)
+    return (MCH_LONG)invoke_d(k, fn, pIn, lIn, nullptr, 0, ppOut, plOut, szErr, errMax);
+}
+
+MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG k, MCH_LONG fn, double* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn, double** ppOut,
+                             MCH_LONG* plOut, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
+    return (MCH_LONG)invoke_d(k, fn, pIn, lIn, plIn, llIn, ppOut, plOut, szErr, errMax);
+}
+
+MCH_LONG Internal_GetPointerDouble(int32_t ht, MCH_LONG kIdx, MCH_LONG h, void** pp)
+{
+    if (ht != 0 || !pp) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+    KernelD* k = kernel_d(kIdx);
+    if (!k) return MCH_ERROR_PARAM_NULL;
+    return (MCH_LONG)k->get_pointer(h, pp);
+}
+
+}  // extern "C"

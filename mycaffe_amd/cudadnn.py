@@ -166,6 +166,7 @@ class ERROR:
 
 
 _c_float_p = ctypes.POINTER(ctypes.c_float)
+_c_double_p = ctypes.POINTER(ctypes.c_double)
 _c_long = ctypes.c_int32
 _c_longlong_p = ctypes.POINTER(ctypes.c_int64)
 _c_tchar_p = ctypes.POINTER(ctypes.c_uint16)
@@ -214,7 +215,12 @@ def load_library(path=None):
     lib.DLL_QueryStringFloatEx.argtypes = [_c_long, _c_long, ctypes.POINTER(_c_long), _c_long, _c_tchar_p, _c_long,
                                            _c_tchar_p, _c_long]
     lib.DLL_QueryStringFloatEx.restype = _c_long
+    lib.DLL_InvokeDouble.argtypes = [_c_long, _c_long, _c_double_p, _c_long, ctypes.POINTER(_c_double_p),
+                                     ctypes.POINTER(_c_long), _c_tchar_p, _c_long]
     lib.DLL_InvokeDouble.restype = _c_long
+    lib.DLL_InvokeDoubleEx2.argtypes = [_c_long, _c_long, _c_double_p, _c_long, _c_longlong_p, _c_long,
+                                        ctypes.POINTER(_c_double_p), ctypes.POINTER(_c_long), _c_tchar_p, _c_long]
+    lib.DLL_InvokeDoubleEx2.restype = _c_long
     lib.MCH_TimeInvokeFloatEx2.argtypes = [_c_long, _c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_long, _c_long,
                                            _c_float_p, _c_tchar_p, _c_long]
     lib.MCH_TimeInvokeFloatEx2.restype = _c_long
@@ -236,13 +242,18 @@ def _from_utf16(buf):
 
 
 class CudaDnn:
-    """One kernel (device context) of the native library, float base type.
+    """One kernel (device context) of the native library, float base type (``CudaDnnDouble`` below: double).
 
     CudaDnn.cs:1679-1760: the constructor loads the DLL at ``strPath`` and sends
     INITIALIZE with ``{deviceId, flags}`` to obtain the kernel index.
     """
 
     OUT_CAPACITY = 16
+    # the base type T of CudaDnn<T>: element type of every array that crosses the boundary, and the entry points it uses
+    DTYPE = np.float32
+    _CTYPE = ctypes.c_float
+    _CPTR = _c_float_p
+    _INVOKE, _INVOKE_EX2 = "DLL_InvokeFloat", "DLL_InvokeFloatEx2"
 
     def __init__(self, nDeviceID=0, flags=DEVINIT.CUBLAS | DEVINIT.CURAND, lSeed=None, strPath=None):
         self._lib = load_library(strPath)
@@ -260,13 +271,13 @@ class CudaDnn:
 
     def _out(self, capacity=None):
         cap = capacity or self.OUT_CAPACITY
-        buf = (ctypes.c_float * cap)()
-        return buf, ctypes.cast(buf, _c_float_p), _c_long(cap)
+        buf = (self._CTYPE * cap)()
+        return buf, ctypes.cast(buf, self._CPTR), _c_long(cap)
 
     def _collect(self, buf, pout, nout, hKernel):
         n = nout.value
         if n <= 0:
-            return np.empty(0, np.float32)
+            return np.empty(0, self.DTYPE)
         addr = ctypes.addressof(pout.contents)
         if addr == ctypes.addressof(buf):
             return np.ctypeslib.as_array(buf)[:n].copy()
@@ -274,14 +285,13 @@ class CudaDnn:
         out = np.ctypeslib.as_array(pout, shape=(n,)).copy()
         errbuf = (ctypes.c_uint16 * _ERRMAX)()
         dummy_buf, dummy_p, dummy_n = self._out(4)
-        self._lib.DLL_InvokeFloat(hKernel, CUDAFN.FREEMEM_HOST, pout, 0, ctypes.byref(dummy_p), ctypes.byref(dummy_n), errbuf, _ERRMAX)
+        getattr(self._lib, self._INVOKE)(hKernel, CUDAFN.FREEMEM_HOST, pout, 0, ctypes.byref(dummy_p), ctypes.byref(dummy_n), errbuf, _ERRMAX)
         return out
 
-    @staticmethod
-    def _farr(rg):
+    def _farr(self, rg):
         if rg is None:
             return None, 0
-        a = np.ascontiguousarray(rg, dtype=np.float32).reshape(-1)
+        a = np.ascontiguousarray(rg, dtype=self.DTYPE).reshape(-1)
         return a, a.size
 
     @staticmethod
@@ -295,8 +305,8 @@ class CudaDnn:
         a, n = self._farr(rgf)
         buf, pout, nout = self._out(out_capacity)
         errbuf = (ctypes.c_uint16 * _ERRMAX)()
-        err = self._lib.DLL_InvokeFloat(hKernel, fn, a.ctypes.data_as(_c_float_p) if a is not None else None, n,
-                                        ctypes.byref(pout), ctypes.byref(nout), errbuf, _ERRMAX)
+        err = getattr(self._lib, self._INVOKE)(hKernel, fn, a.ctypes.data_as(self._CPTR) if a is not None else None, n,
+                                               ctypes.byref(pout), ctypes.byref(nout), errbuf, _ERRMAX)
         self._check(err, errbuf)
         return self._collect(buf, pout, nout, hKernel)
 
@@ -305,9 +315,9 @@ class CudaDnn:
         l, ln = self._larr(rgl)
         buf, pout, nout = self._out(out_capacity)
         errbuf = (ctypes.c_uint16 * _ERRMAX)()
-        err = self._lib.DLL_InvokeFloatEx2(hKernel, fn, a.ctypes.data_as(_c_float_p) if a is not None else None, n,
-                                           l.ctypes.data_as(_c_longlong_p) if l is not None else None, ln,
-                                           ctypes.byref(pout), ctypes.byref(nout), errbuf, _ERRMAX)
+        err = getattr(self._lib, self._INVOKE_EX2)(hKernel, fn, a.ctypes.data_as(self._CPTR) if a is not None else None, n,
+                                                   l.ctypes.data_as(_c_longlong_p) if l is not None else None, ln,
+                                                   ctypes.byref(pout), ctypes.byref(nout), errbuf, _ERRMAX)
         self._check(err, errbuf)
         return self._collect(buf, pout, nout, hKernel)
 
@@ -382,11 +392,11 @@ class CudaDnn:
             if src <= 0:
                 raise ValueError("capacity must be positive")
             return int(self._ex2(fn, None, [int(src)])[0])
-        data = np.ascontiguousarray(src, dtype=np.float32).reshape(-1)
+        data = np.ascontiguousarray(src, dtype=self.DTYPE).reshape(-1)
         if data.size == 0:
             raise ValueError("no data")
         head = [data.size] + ([hStream] if hStream > 0 else [])
-        rgf = np.concatenate([np.array(head, np.float32), data])
+        rgf = np.concatenate([np.array(head, self.DTYPE), data])
         return int(self._ex2(fn, rgf, head)[0])
 
     def FreeMemory(self, hMem):
@@ -401,13 +411,13 @@ class CudaDnn:
 
     def SetMemory(self, hMem, src, hStream=0, nCount=-1):
         """CudaDnn.cs:3027-3095: ``f{h, count, [stream,] data}``, ``l{h, count}``."""
-        data = np.ascontiguousarray(src, dtype=np.float32).reshape(-1)
+        data = np.ascontiguousarray(src, dtype=self.DTYPE).reshape(-1)
         if nCount == -1:
             nCount = data.size
         if nCount == 0:
             raise ValueError("There are no data items to set!")
         head = [hMem, nCount] + ([hStream] if hStream > 0 else [])
-        rgf = np.concatenate([np.array(head, np.float32), data[:nCount]])
+        rgf = np.concatenate([np.array(head, self.DTYPE), data[:nCount]])
         self._ex2(CUDAFN.SETMEM, rgf, [hMem, nCount])
 
     def CreateMemoryPointer(self, hData, lOffset, lCount):
@@ -797,3 +807,18 @@ class CudaDnn:
                                                ctypes.byref(ms), errbuf, _ERRMAX)
         self._check(err, errbuf)
         return float(ms.value)
+
+
+class CudaDnnDouble(CudaDnn):
+    """One kernel of the double base type (CudaDnn<double>): every array crosses the boundary as doubles through
+    DLL_InvokeDouble / DLL_InvokeDoubleEx2 (CudaDnnDLL.cpp:494-853), device memory holds doubles and the arithmetic is
+    double.  The library builds the function ids of the attention path for it; any other id raises
+    ``CudaDnnError`` with code NOT_IMPLEMENTED (90009)."""
+
+    DTYPE = np.float64
+    _CTYPE = ctypes.c_double
+    _CPTR = _c_double_p
+    _INVOKE, _INVOKE_EX2 = "DLL_InvokeDouble", "DLL_InvokeDoubleEx2"
+
+    def RunFloatEx(self, hKernel, fn, rgf, strInput):
+        raise CudaDnnError(90009, "extensions and blob loaders are float objects")

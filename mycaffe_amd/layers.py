@@ -74,7 +74,7 @@ class Blob:
 
     @mutable_cpu_diff.setter
     def mutable_cpu_diff(self, values):
-        self.cuda.SetMemory(self.gpu_diff, np.asarray(values, np.float32).reshape(-1), nCount=self.count())
+        self.cuda.SetMemory(self.gpu_diff, np.asarray(values, self.cuda.DTYPE).reshape(-1), nCount=self.count())
 
     @property
     def mutable_cpu_data(self):
@@ -82,7 +82,7 @@ class Blob:
 
     @mutable_cpu_data.setter
     def mutable_cpu_data(self, values):
-        self.cuda.SetMemory(self.gpu_data, np.asarray(values, np.float32).reshape(-1), nCount=self.count())
+        self.cuda.SetMemory(self.gpu_data, np.asarray(values, self.cuda.DTYPE).reshape(-1), nCount=self.count())
 
     def SetData(self, value):
         self.cuda.set(self.count(), self.gpu_data, float(value))

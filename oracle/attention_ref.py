@@ -279,10 +279,18 @@ def rmsnorm_layer_backward(x, weight, dy, eps=1e-5, dtype=np.float32):
 # RoPE, CudaDnnDLL form
 # ----------------------------------------------------------------------------
 
-def rope_tables(seq_len, hs, theta=10000.0):
+def rope_tables(seq_len, hs, theta=10000.0, base_double=False):
     """cos/sin tables [seq_len, hs/2] as RopeDataGpu<float>::Initialize builds
     them on the host (rope.cu:535-553): freq_j = 1/powf(theta, 2j/hs) in fp32,
-    angle = freq_j * pos in fp32, cosf/sinf."""
+    angle = freq_j * pos in fp32, cosf/sinf.  ``base_double``: the T = double
+    instance of the same lines - the exponent, the reciprocal and the angle are
+    held in double, powf / cosf / sinf still take and return floats."""
+    if base_double:
+        j = np.arange(0, hs, 2, dtype=np.float64)
+        power = np.power(np.float32(theta), (j / np.float64(hs)).astype(np.float32), dtype=np.float32).astype(np.float64)
+        freq = 1.0 / power
+        ang = (freq[None, :] * np.arange(seq_len, dtype=np.float64)[:, None]).astype(np.float32)
+        return np.cos(ang).astype(np.float32).astype(np.float64), np.sin(ang).astype(np.float32).astype(np.float64)
     j = np.arange(0, hs, 2, dtype=np.float32)
     power = (j / np.float32(hs)).astype(np.float32)
     freq = (np.float32(1.0) / np.power(np.float32(theta), power, dtype=np.float32)).astype(np.float32)
@@ -291,7 +299,7 @@ def rope_tables(seq_len, hs, theta=10000.0):
     return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
 
 
-def rope_forward(x, seq_len, heads, hs, theta=10000.0, freq_offset=-1, dtype=np.float32):
+def rope_forward(x, seq_len, heads, hs, theta=10000.0, freq_offset=-1, dtype=np.float32, base_double=False):
     """RopeDataGpu<T>::Forward (rope.cu:725-825).
 
     x is flat with an even count; consecutive (even, odd) elements form a pair.
@@ -301,7 +309,7 @@ def rope_forward(x, seq_len, heads, hs, theta=10000.0, freq_offset=-1, dtype=np.
     x = np.asarray(x, dtype).reshape(-1)
     half = hs // 2
     full = half * heads
-    cos, sin = rope_tables(seq_len, hs, theta)
+    cos, sin = rope_tables(seq_len, hs, theta, base_double)
     cos = cos.reshape(-1).astype(dtype)
     sin = sin.reshape(-1).astype(dtype)
     off = freq_offset if freq_offset > 0 else 0

@@ -1,0 +1,270 @@
+"""The double base type of the C ABI (DLL_InvokeDouble / DLL_InvokeDoubleEx2; CudaDnnDLL.cpp:494-853): the function ids of
+the attention path on a kernel whose memory and arithmetic are double, against the checker in float64.  The reference's
+own tests run every case once per base type (TestBase.cs:107-115); the bar here is what double arithmetic gives, 1e-12
+relative, so a path that went through fp32 anywhere (2^-24) cannot pass it.  The rotary tables are the exception: the
+reference builds them with powf / cosf / sinf for either base type (rope.cu:535-553), the checker's library calls may
+differ from the C library's by an ulp of a float."""
+import numpy as np
+import pytest
+
+from tests.conftest import assert_close
+from mycaffe_amd.cudadnn import CUDAFN, CudaDnn, CudaDnnDouble, CudaDnnError
+from mycaffe_amd.layers import Blob, CausalSelfAttentionLayer, InnerProductLayer, SoftmaxLayer, TransposeLayer
+from oracle import attention_ref as R
+
+pytestmark = pytest.mark.gpu
+
+F64_RTOL = 1e-12
+ROPE_RTOL = 2e-6
+
+
+class DevD:
+    def __init__(self):
+        self.cuda = CudaDnnDouble(0)
+
+    def put(self, a):
+        return self.cuda.AllocMemory(np.asarray(a, np.float64))
+
+    def zeros(self, n):
+        return self.cuda.AllocMemory(int(n))
+
+    def get(self, h, shape=None):
+        a = self.cuda.GetMemoryFloat(h)
+        assert a.dtype == np.float64
+        return a.reshape(shape) if shape is not None else a
+
+
+@pytest.fixture()
+def devd():
+    d = DevD()
+    yield d
+    d.cuda.Dispose()
+
+
+def test_double_memory_keeps_every_bit(devd):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(1000), [1.0 + 2.0 ** -52, 1e-300, -1e300, 2.0 ** -1074, np.pi]])
+    h = devd.put(x)
+    assert devd.get(h).tobytes() == x.tobytes()
+    y = rng.standard_normal(x.size)
+    devd.cuda.SetMemory(h, y)
+    assert devd.get(h).tobytes() == y.tobytes()
+    assert devd.cuda.GetMemoryFloat(h, 7).tobytes() == y[:7].tobytes()     # fits the caller's buffer
+    h2 = devd.zeros(x.size)
+    assert not devd.get(h2).any()
+    devd.cuda.copy(100, h, h2, 5, 10)
+    assert np.array_equal(devd.get(h2)[10:110], y[5:105])
+    devd.cuda.set(x.size, h2, 1.0 / 3.0)
+    assert np.all(devd.get(h2) == 1.0 / 3.0)
+    devd.cuda.set(1, h2, 7.0, 3)
+    assert devd.get(h2)[3] == 7.0 and devd.get(h2)[4] == 1.0 / 3.0
+    devd.cuda.FreeMemory(h)
+    with pytest.raises(CudaDnnError):
+        devd.cuda.GetMemoryFloat(h)
+    # the float table does not know the double table's kernels and the other way round: separate index spaces
+    f = CudaDnn(0)
+    hf = f.AllocMemory(np.float32([1, 2, 3]))
+    assert f.GetMemoryFloat(hf).dtype == np.float32
+    f.Dispose()
+
+
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+def test_double_gemm_inline_vectors_and_random(devd, tA, tB):
+    """The 2x3 . 3x4 case of TestCudaDnn.cs:5586-5686 in the four transpose combinations, then a random product."""
+    A = np.arange(1, 7, dtype=np.float64).reshape(2, 3)
+    B = np.arange(1, 13, dtype=np.float64).reshape(3, 4)
+    hA, hB, hC = devd.put(A.T if tA else A), devd.put(B.T if tB else B), devd.zeros(8)
+    devd.cuda.gemm(tA, tB, 2, 4, 3, 1.0, hA, hB, 0.0, hC)
+    assert np.array_equal(devd.get(hC), [38, 44, 50, 56, 83, 98, 113, 128])
+    rng = np.random.default_rng(5)
+    m, n, k = 70, 45, 130
+    A, B, C = rng.standard_normal((m, k)), rng.standard_normal((k, n)), rng.standard_normal((m, n))
+    hA, hB, hC = devd.put(A.T if tA else A), devd.put(B.T if tB else B), devd.put(C)
+    devd.cuda.gemm(tA, tB, m, n, k, 0.7, hA, hB, -1.3, hC)
+    assert_close(devd.get(hC, (m, n)), 0.7 * A @ B - 1.3 * C, F64_RTOL, "gemm")
+
+
+def test_double_gemm_is_double(devd, dev):
+    # the same product on the float base type is off by 2^-24 and more; on the double base type by 2^-50
+    rng = np.random.default_rng(6)
+    A, B = rng.standard_normal((64, 256)), rng.standard_normal((256, 64))
+    ref = A @ B
+    hA, hB, hC = devd.put(A), devd.put(B), devd.zeros(64 * 64)
+    devd.cuda.gemm(False, False, 64, 64, 256, 1.0, hA, hB, 0.0, hC)
+    err_d = np.abs(devd.get(hC, (64, 64)) - ref).max() / np.abs(ref).max()
+    fA, fB, fC = dev.put(A), dev.put(B), dev.zeros(64 * 64)
+    dev.cuda.gemm(False, False, 64, 64, 256, 1.0, fA, fB, 0.0, fC)
+    err_f = np.abs(dev.get(fC, (64, 64)) - ref).max() / np.abs(ref).max()
+    assert err_d < 1e-14 and err_f > 1e-9
+
+
+def test_double_matmul_gemv_and_vector_updates(devd):
+    rng = np.random.default_rng(7)
+    outer, m, n, k = 6, 33, 20, 17
+    A, B = rng.standard_normal((outer, m, k)), rng.standard_normal((outer, k, n))
+    hA, hB, hC = devd.put(A), devd.put(B), devd.zeros(outer * m * n)
+    devd.cuda.matmul(outer, m, n, k, hA, hB, hC, 0.25)
+    assert_close(devd.get(hC, (outer, m, n)), 0.25 * A @ B, F64_RTOL, "matmul")
+    Bt = np.ascontiguousarray(B.transpose(0, 2, 1))
+    hBt = devd.put(Bt)
+    devd.cuda.matmul(outer, m, n, k, hA, hBt, hC, 1.0, False, True)
+    assert_close(devd.get(hC, (outer, m, n)), A @ B, F64_RTOL, "matmul with B transposed")
+    W, x, y = rng.standard_normal((40, 30)), rng.standard_normal(30), rng.standard_normal(40)
+    hW, hx, hy = devd.put(W), devd.put(x), devd.put(y)
+    devd.cuda.gemv(False, 40, 30, 2.0, hW, hx, 0.5, hy)
+    assert_close(devd.get(hy), 2.0 * W @ x + 0.5 * y, F64_RTOL, "gemv")
+    hy2 = devd.zeros(30)
+    devd.cuda.gemv(True, 40, 30, 1.0, hW, hy, 0.0, hy2)
+    assert_close(devd.get(hy2), W.T @ devd.get(hy), F64_RTOL, "gemv transposed")
+    a, b = rng.standard_normal(1001), rng.standard_normal(1001)
+    ha, hb, hc = devd.put(a), devd.put(b), devd.zeros(1001)
+    devd.cuda.axpy(1001, 1.0 / 3.0, ha, hb)
+    b2 = a / 3.0 + b
+    assert_close(devd.get(hb), b2, F64_RTOL, "axpy")
+    devd.cuda.scal(1001, 1.0 / 7.0, hb)
+    assert_close(devd.get(hb), b2 / 7.0, F64_RTOL, "scal")
+    devd.cuda.scale(1001, -2.5, ha, hc)
+    assert np.array_equal(devd.get(hc), -2.5 * a)
+    devd.cuda.add(1001, ha, hb, hc)
+    assert_close(devd.get(hc), a + b2 / 7.0, F64_RTOL, "add")
+    devd.cuda.add(1001, ha, hb, hc, 0.1)
+    assert_close(devd.get(hc), a + 0.1 * (b2 / 7.0), F64_RTOL, "add with a factor")
+    devd.cuda.mul(1001, ha, ha, hc)
+    assert np.array_equal(devd.get(hc), a * a)
+    devd.cuda.silu_fwd(1001, ha, hc)
+    assert_close(devd.get(hc), R.silu(a, np.float64), F64_RTOL, "silu")
+
+
+def test_double_mask_layout_ops_softmax_embed(devd):
+    rng = np.random.default_rng(8)
+    B, H, T = 2, 3, 16
+    x = rng.standard_normal((B, H, T, T))
+    causal = np.tril(np.ones((T, T)))
+    hx, hm, hy = devd.put(x), devd.put(causal), devd.zeros(x.size)
+    devd.cuda.mask(x.size, T * T, 0.0, -1e29, hx, hm, hy)
+    assert np.array_equal(devd.get(hy), R.mask(x.size, T * T, 0.0, -1e29, x, causal, np.float64).reshape(-1))
+    keym = (rng.random((B, T)) > 0.3).astype(np.float64)
+    hk = devd.put(keym)
+    devd.cuda.mask_batch(x.size, B, B * T, 0.0, -1e29, hx, hk, hy)
+    want = R.mask_batch(x.size, B, B * T, 0.0, -1e29, x, keym, np.float64)
+    assert np.array_equal(devd.get(hy), want.reshape(-1))
+    # softmax through the descriptors, over the last axis (rows) and over channels
+    sm = SoftmaxLayer(devd.cuda, -1)
+    bx, by = Blob(devd.cuda, x.shape), Blob(devd.cuda)
+    bx.mutable_cpu_data = want.reshape(x.shape)
+    sm.Forward(bx, by)
+    assert_close(by.mutable_cpu_data, R.softmax_lastaxis(want.reshape(x.shape), np.float64), F64_RTOL, "softmax rows")
+    sm1 = SoftmaxLayer(devd.cuda, 1)
+    bx.mutable_cpu_data = x
+    sm1.Forward(bx, by)
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    assert_close(by.mutable_cpu_data, e / e.sum(axis=1, keepdims=True), F64_RTOL, "softmax over channels")
+    # transposes and channel copy as the layer uses them
+    t = TransposeLayer(devd.cuda, (0, 2, 1, 3))
+    z = rng.standard_normal((2, 5, 3, 4))
+    bz, bt = Blob(devd.cuda, z.shape), Blob(devd.cuda)
+    bz.mutable_cpu_data = z
+    t.Forward(bz, bt)
+    assert np.array_equal(bt.mutable_cpu_data.reshape(2, 3, 5, 4), z.transpose(0, 2, 1, 3))
+    hz, hz2 = devd.put(z), devd.zeros(z.size)
+    devd.cuda.transposeHW(2, 5, 3, 4, hz, hz2)
+    assert np.array_equal(devd.get(hz2, (2, 5, 4, 3)), z.transpose(0, 1, 3, 2))
+    ip = rng.standard_normal((2, 7, 3 * 8))
+    hip_, hq = devd.put(ip), devd.zeros(2 * 7 * 8)
+    devd.cuda.channel_copy(2 * 7 * 8, 2, 7, 3, 8, 1, hip_, hq, 0)
+    assert np.array_equal(devd.get(hq, (2, 7, 8)), ip[:, :, 8:16])
+    ids = rng.integers(0, 11, 9).astype(np.float64)
+    w = rng.standard_normal((11, 6))
+    hi, hw, ht = devd.put(ids), devd.put(w), devd.zeros(9 * 6)
+    devd.cuda.embed_fwd(9 * 6, hi, hw, 9, 6, 11, ht)
+    assert np.array_equal(devd.get(ht, (9, 6)), w[ids.astype(int)])
+
+
+@pytest.mark.parametrize("B,T,H,hs,off", [(2, 16, 3, 8, -1), (1, 9, 2, 64, -1), (1, 1, 2, 16, 5)])
+def test_double_rope_forward(devd, B, T, H, hs, off):
+    S = 16
+    rng = np.random.default_rng(T)
+    x = rng.standard_normal((B, T, H, hs))
+    hr = devd.cuda.CreateRope(0, 0, x.size, B, S, H, hs, 10000.0)
+    hx, hy = devd.put(x), devd.zeros(x.size)
+    devd.cuda.RopeForward(hr, x.size, hx, hy, off)
+    want = R.rope_forward(x, S, H, hs, 10000.0, off, np.float64, base_double=True)
+    assert_close(devd.get(hy), want, ROPE_RTOL, "rope")
+    # the rotation keeps the length of every pair: a property no table error can hide
+    got = devd.get(hy).reshape(-1, 2)
+    assert_close((got ** 2).sum(axis=1), (x.reshape(-1, 2) ** 2).sum(axis=1), 1e-6, "pair norms")
+    devd.cuda.FreeRope(hr)
+
+
+@pytest.mark.parametrize("kind", ["causal", "none", "keys", "per_sequence"])
+def test_double_attention_forward(devd, kind):
+    B, H, T, hs = 2, 3, 40, 16
+    rng = np.random.default_rng(3)
+    q, k, v = (rng.standard_normal((B, H, T, hs)) for _ in range(3))
+    hc, ha = devd.cuda.CreateCuDNN(), devd.cuda.CreateAttn()
+    devd.cuda.SetAttn(hc, ha, 0, False, B, 64, H, hs, 0.0)
+    hq, hk, hv, hy = devd.put(q), devd.put(k), devd.put(v), devd.zeros(q.size)
+    if kind == "causal":
+        m = np.tril(np.ones((T, T)))
+        hm, bm = devd.put(m), 0
+        full = np.broadcast_to(m, (B, H, T, T))
+    elif kind == "none":
+        hm, bm, full = 0, 0, np.ones((B, H, T, T))
+    elif kind == "keys":
+        m = (rng.random((B, T)) > 0.4).astype(np.float64)
+        m[1, :] = 0                                        # a sequence with every key masked: uniform weights
+        hm, bm = devd.put(m), 1
+        full = np.broadcast_to(m[:, None, None, :], (B, H, T, T))
+    else:
+        m = (rng.random((B, T, T)) > 0.4).astype(np.float64)
+        hm, bm = devd.put(m), 2
+        full = np.broadcast_to(m[:, None], (B, H, T, T))
+    devd.cuda.AttnScaledDotProductForward(hc, ha, T, hq, hk, hv, hm, hy, bm)
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) / np.sqrt(hs)
+    s = np.where(full == 0, -1e29, s)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    assert_close(devd.get(hy, q.shape), np.einsum("bhqk,bhkd->bhqd", p, v), F64_RTOL, "attention, " + kind)
+    if kind == "causal":
+        ref, _ = R.attn_forward(q, k, v, R.causal_mask(T, np.float64), False, np.float64)
+        assert_close(devd.get(hy, q.shape), ref, F64_RTOL, "attention vs the checker")
+    devd.cuda.FreeAttn(ha)
+    devd.cuda.FreeCuDNN(hc)
+
+
+@pytest.mark.parametrize("sdpa", [True, False])
+@pytest.mark.parametrize("rope", [False, True])
+def test_double_causal_self_attention_layer(devd, sdpa, rope):
+    """CausalSelfAttentionLayer.forward (CausalSelfAttentionLayer.cs:526-605) on the double base type, through the fused
+    attention handle and through the explicit chain (transposes, MatMul, scale, mask, softmax, MatMul), against the
+    checker in float64."""
+    B, T, C, H = 2, 24, 48, 3
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((B, T, C))
+    wa, wp = rng.standard_normal((3 * C, C)) * 0.1, rng.standard_normal((C, C)) * 0.1
+    ba, bp = rng.standard_normal(3 * C) * 0.1, rng.standard_normal(C) * 0.1
+    layer = CausalSelfAttentionLayer(devd.cuda, H, C, T, True, sdpa, enable_rotary_positional_embedding=rope)
+    bottom, top = Blob(devd.cuda, x.shape), Blob(devd.cuda)
+    bottom.mutable_cpu_data = x
+    layer.Setup(bottom, wa, ba, wp, bp)
+    layer.Forward(bottom, top)
+    y = top.mutable_cpu_data
+    assert y.dtype == np.float64
+    ref = R.causal_self_attention(x, wa, ba, wp, bp, H, rope=(T, 10000.0) if rope else None, dtype=np.float64)["y"]
+    assert_close(y, ref, ROPE_RTOL if rope else F64_RTOL, "layer output")
+
+
+def test_double_ids_outside_the_attention_path_say_so(devd):
+    h = devd.zeros(16)
+    with pytest.raises(CudaDnnError) as e:
+        devd.cuda.powx(16, h, 2.0, h)
+    assert e.value.code == 90009 and "double" in str(e.value)
+    with pytest.raises(CudaDnnError) as e:
+        devd.cuda.CreateExtension("libmycaffe_hip_llama2.so")
+    assert e.value.code == 90009
+    # dropout in the handle is a float-only feature
+    hc, ha = devd.cuda.CreateCuDNN(), devd.cuda.CreateAttn()
+    with pytest.raises(CudaDnnError) as e:
+        devd.cuda.SetAttn(hc, ha, 0, True, 1, 8, 1, 8, 0.1)
+    assert e.value.code == 90009
