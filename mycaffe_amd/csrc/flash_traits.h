@@ -155,6 +155,14 @@ __device__ __forceinline__ int flash_causal_rank(int occ)
 {
     if ((gridDim.x & 7) != 0) return (int)blockIdx.x;
     const int x = blockIdx.x & 7, j = blockIdx.x >> 3, per = gridDim.x >> 3;
+    if (occ == 2 && per > 32 && per < 64) {
+        // Less than two rounds: the XCD's CUs 0 .. per - 33 get a second workgroup, the others stay alone.  The heaviest
+        // blocks go to the CUs that stay alone; the paired CUs take the next heaviest, and as partners the lightest ones,
+        // lightest to the heaviest - so that no CU holds much more than the heaviest single block.
+        const int nPair = per - 32, nLone = 32 - nPair;
+        const int r = j >= 32 ? per - 1 - (j - 32) : j >= nPair ? j - nPair : nLone + j;
+        return (r << 3) + x;
+    }
     const int r = j >> 5, c = j & 31;
     if (!(r & 1) || r >= occ) return (int)blockIdx.x;
     const int rest = per - (r << 5);
