@@ -2,10 +2,11 @@
 // table whose device memory holds doubles and whose arithmetic is double, as the reference's Kernel<double> instances
 // are (dllmain.cpp:6-14; the reference test base runs every test once per base type, TestBase.cs:107-115).
 //
-// It covers the function ids of the attention path - memory, GEMM / GEMM2 / GEMV and the vector updates, mask, the
-// transposes, channel copy, softmax forward, the attention handle's forward call, rotary embedding forward, embedding
-// lookup, SiLU - with plain kernels: one output element per thread, reductions by one workgroup per row, nothing tiled
-// for the matrix cores.  This is the precision twin of the fp32 path, for hosts that instantiate their layers in
+// It covers the function ids of the attention path and of the layers around it - memory, GEMM / GEMM2 / GEMV and the
+// vector updates, mask, the transposes, channel copy and the channel reductions / broadcasts, softmax, the attention
+// handle, rotary embedding, layer norm handle, RMS norm, the activations, each forward and backward, embedding lookup -
+// with plain kernels: one output element per thread, reductions by one workgroup per row, nothing tiled for the matrix
+// cores.  This is the precision twin of the fp32 path, for hosts that instantiate their layers in
 // double; the fast kernels are the fp32 / bf16 ones.  Every other id returns MCH_ERROR_NOT_IMPLEMENTED with its number
 // in the message.  ALLOCMEM_HALF allocates doubles (no 16-bit storage under this base type).
 #include <hip/hip_runtime.h>
@@ -39,6 +40,53 @@ __global__ void d_scale_kernel(size_t n, double a, const double* x, double* y) {
 __global__ void d_add_kernel(size_t n, const double* a, const double* b, double* y, double alpha) { GRID_STRIDE(i, n) y[i] = a[i] + b[i] * alpha; }
 __global__ void d_mul_kernel(size_t n, const double* a, const double* b, double* y) { GRID_STRIDE(i, n) y[i] = a[i] * b[i]; }
 __global__ void d_silu_kernel(size_t n, const double* x, double* y) { GRID_STRIDE(i, n) y[i] = x[i] * (1.0 / (1.0 + exp(-x[i]))); }
+
+__global__ void d_swiglu_kernel(size_t n, const double* a, const double* b, double* y) { GRID_STRIDE(i, n) y[i] = a[i] * (1.0 / (1.0 + exp(-a[i]))) * b[i]; }
+// f(dy, x) = dy s (1 + x (1 - s)) (math.cu:11740-11749)
+__global__ void d_silu_bwd_kernel(size_t n, const double* dy, const double* x, double* dx)
+{
+    GRID_STRIDE(i, n) { const double sg = 1.0 / (1.0 + exp(-x[i])); dx[i] = dy[i] * (sg * (1.0 + x[i] * (1.0 - sg))); }
+}
+// GELU (math.cu:11348-11376) and its gradient with the reference's rounded constants (math.cu:11412-11448)
+__global__ void d_gelu_kernel(size_t n, const double* x, double* y, bool bert)
+{
+    GRID_STRIDE(i, n)
+    {
+        const double v = x[i];
+        y[i] = bert ? 0.5 * v * (1.0 + tanh(0.7978845608028654 * (v + 0.044715 * v * v * v))) : v * (0.5 * (1.0 + erf(v * 0.7071067811865475)));
+    }
+}
+__global__ void d_gelu_bwd_kernel(size_t n, const double* dy, const double* x, double* dx, bool bert)
+{
+    GRID_STRIDE(i, n)
+    {
+        const double v = x[i];
+        double grad;
+        if (bert) {
+            const double x3 = v * v * v, t = tanh(0.797885 * (v + 0.044715 * x3));
+            grad = 0.5 * t + (0.0535161 * x3 + 0.398942 * v) * (1.0 - t * t) + 0.5;
+        } else {
+            grad = 0.5 * (1.0 + erf(v * 0.7071067811865475)) + v * (0.3989422804014327 * exp(-0.5 * v * v));
+        }
+        dx[i] = dy[i] * grad;
+    }
+}
+// ReLU with negative slope (math.cu:12038-12044); its gradient looks at the top data (math.cu:12072-12078)
+__global__ void d_relu_kernel(size_t n, const double* x, double* y, double slope) { GRID_STRIDE(i, n) y[i] = x[i] > 0.0 ? x[i] : x[i] * slope; }
+__global__ void d_relu_bwd_kernel(size_t n, const double* dy, const double* y, double* dx, double slope)
+{
+    GRID_STRIDE(i, n) dx[i] = dy[i] * ((y[i] > 0.0 ? 1.0 : 0.0) + (y[i] <= 0.0 ? 1.0 : 0.0) * slope);
+}
+// the elementwise primitives of the norm chains and of the CAFFE-engine softmax (math.cu:5064-5090, 5681-5687, 5859-5865,
+// 5923-5929, 5955-5961, 6018-6082, 6211-6217)
+__global__ void d_sub_kernel(size_t n, const double* a, const double* b, double* y, size_t nB) { GRID_STRIDE(i, n) y[i] = a[i] - b[nB ? i % nB : i]; }
+__global__ void d_div_kernel(size_t n, const double* a, const double* b, double* y) { GRID_STRIDE(i, n) y[i] = b[i] == 0.0 ? 0.0 : a[i] / b[i]; }
+__global__ void d_add_scalar_kernel(size_t n, double alpha, double* y) { GRID_STRIDE(i, n) y[i] += alpha; }
+__global__ void d_powx_kernel(size_t n, const double* a, double alpha, double* y) { GRID_STRIDE(i, n) y[i] = alpha == 2.0 ? a[i] * a[i] : pow(a[i], alpha); }
+__global__ void d_sqrt_kernel(size_t n, const double* x, double* y, double eps) { GRID_STRIDE(i, n) y[i] = sqrt(x[i] + eps); }
+__global__ void d_invert_kernel(size_t n, const double* x, double* y, double num, double den) { GRID_STRIDE(i, n) y[i] = x[i] == 0.0 ? 0.0 : num / (x[i] * den); }
+__global__ void d_exp_kernel(size_t n, const double* a, double* y, double beta) { GRID_STRIDE(i, n) y[i] = exp(beta * a[i]); }
+__global__ void d_log_kernel(size_t n, const double* a, double* y, double beta, double alpha) { GRID_STRIDE(i, n) y[i] = log(beta * (a[i] + alpha)); }
 
 // mask index = i % md1 + (i / dd1) * md1 (math.cu:2995-3002, 3046-3056; the plain mask is the case dd1 = n)
 __global__ void d_mask_kernel(size_t n, size_t md1, size_t dd1, const double* x, const double* mask, double* y, double search, double replace)
@@ -120,14 +168,79 @@ __global__ void d_embed_kernel(size_t count, const double* ids, const double* w,
 }
 // pairs (2p, 2p+1) rotated by the angle of table entry ((p % wrap) / full) * half + p % half + off (rope.cu:725-825)
 __global__ void d_rope_kernel(size_t pairs, const double* x, double* y, const double* fcos, const double* fsin, size_t full,
-                              size_t wrap, int half, int off)
+                              size_t wrap, int half, int off, double sinSign)
 {
     GRID_STRIDE(p, pairs)
     {
         const size_t base = p % wrap, t = (base / full) * half + base % half + off;
-        const double c = fcos[t], sn = fsin[t], re = x[2 * p], im = x[2 * p + 1];
+        const double c = fcos[t], sn = sinSign * fsin[t], re = x[2 * p], im = x[2 * p + 1];
         y[2 * p] = re * c - im * sn;
         y[2 * p + 1] = re * sn + im * c;
+    }
+}
+
+// MODE 0: y[i] = x[i / spatial]; 1: x[i] = y[i * spatial]; 2: y[i] = x[i % period]; 3: y[i] = x[(i / period) * channels + i % channels]
+// (channel_fillfrom forward / backward, channel_copyall, channel_duplicate: math.cu:7465-7481, 7630-7639, 7667-7676)
+__global__ void d_spread_kernel(int mode, size_t n, size_t spatial, size_t period, size_t channels, double* x, double* y)
+{
+    GRID_STRIDE(i, n)
+    {
+        if (mode == 0) y[i] = x[i / spatial];
+        else if (mode == 1) x[i] = y[i * spatial];
+        else if (mode == 2) y[i] = x[i % period];
+        else y[i] = x[(i / period) * channels + i % channels];
+    }
+}
+// y[row] = scale * sum of the row's `inner` values, one thread per row (channel_mean, channel_sum within a channel)
+__global__ void d_rowsum_kernel(size_t rows, int inner, const double* x, double* y, double scale)
+{
+    GRID_STRIDE(r, rows)
+    {
+        double acc = 0.0;
+        for (int i = 0; i < inner; i++) acc += x[r * inner + i];
+        y[r] = acc * scale;
+    }
+}
+// y[n, s] = sum over c of x[n, c, s] (math.cu:6945-6980), or of x a (channel_dot, math.cu:7335-7351)
+__global__ void d_colsum_kernel(size_t rows, int channels, int spatial, const double* x, const double* a, double* y)
+{
+    GRID_STRIDE(i, rows)
+    {
+        const size_t n = i / spatial, sp = i % spatial, base = n * channels * (size_t)spatial + sp;
+        double acc = 0.0;
+        for (int c = 0; c < channels; c++) acc += a ? x[base + (size_t)c * spatial] * a[base + (size_t)c * spatial] : x[base + (size_t)c * spatial];
+        y[i] = acc;
+    }
+}
+// channel_max across channels or within one, value or first index (math.cu:6697-6810); starts from -DBL_MAX
+__global__ void d_channel_max_kernel(size_t rows, int channels, int spatial, const double* x, double* y, bool idx, bool across)
+{
+    GRID_STRIDE(i, rows)
+    {
+        double val = -1.7976931348623157e308;
+        int at = 0;
+        if (across) {
+            const size_t n = i / spatial, sp = i % spatial;
+            for (int c = 0; c < channels; c++) {
+                const double v = x[n * channels * (size_t)spatial + (size_t)c * spatial + sp];
+                if (v > val) { val = v; at = c; }
+            }
+        } else {
+            for (int j = 0; j < spatial; j++) {
+                const double v = x[i * spatial + j];
+                if (v > val) { val = v; at = j; }
+            }
+        }
+        y[i] = idx ? (double)at : val;
+    }
+}
+// sub: y[i] = a[i] - x[n, s]; div: y[i] /= x[n, s]; i = (n, c, s) (math.cu:6908-6916, 7160-7168)
+__global__ void d_channel_bcast_kernel(size_t count, int channels, int spatial, const double* a, const double* x, double* y, bool sub)
+{
+    GRID_STRIDE(i, count)
+    {
+        const double r = x[(i / channels / spatial) * spatial + i % spatial];
+        y[i] = sub ? a[i] - r : y[i] / r;
     }
 }
 
@@ -161,11 +274,83 @@ __global__ __launch_bounds__(256) void d_softmax_kernel(const double* x, double*
     }
 }
 
+// dx = (dy - sum) y, sum = sum_l dy y over the series (log form: dx = dy - exp(y) sum dy); one workgroup per series
+__global__ __launch_bounds__(256) void d_softmax_bwd_kernel(const double* y, const double* dy, double* dx, int len, int inner, bool logsm)
+{
+    __shared__ double red[4];
+    const size_t o = blockIdx.x / inner, in = blockIdx.x % inner, base = o * (size_t)len * inner + in;
+    double sum = 0.0;
+    for (int l = threadIdx.x; l < len; l += 256) {
+        const size_t i = base + (size_t)l * inner;
+        sum += logsm ? dy[i] : dy[i] * y[i];
+    }
+    sum = d_block_reduce(sum, red, false);
+    for (int l = threadIdx.x; l < len; l += 256) {
+        const size_t i = base + (size_t)l * inner;
+        dx[i] = logsm ? dy[i] - exp(y[i]) * sum : (dy[i] - sum) * y[i];
+    }
+}
+// y = (x - mean) / sqrt(var + eps) per row, the row's sqrt(var + eps) kept (layernorm.cu:219-262)
+__global__ __launch_bounds__(256) void d_layernorm_fwd_kernel(int inner, const double* x, double* y, double* stdev, double eps)
+{
+    __shared__ double red[4];
+    const double* xr = x + (size_t)blockIdx.x * inner;
+    double* yr = y + (size_t)blockIdx.x * inner;
+    double sum = 0.0;
+    for (int i = threadIdx.x; i < inner; i += 256) sum += xr[i];
+    const double mean = d_block_reduce(sum, red, false) / inner;
+    double sq = 0.0;
+    for (int i = threadIdx.x; i < inner; i += 256) sq += (xr[i] - mean) * (xr[i] - mean);
+    const double sd = sqrt(d_block_reduce(sq, red, false) / inner + eps);
+    if (threadIdx.x == 0) stdev[blockIdx.x] = sd;
+    for (int i = threadIdx.x; i < inner; i += 256) yr[i] = (xr[i] - mean) / sd;
+}
+// dx = (dy - (y mean(y dy) + mean(dy))) / divisor (layernorm.cu:268-312); the reference adds eps to the first `rows`
+// entries of its row-expanded stdev array on every backward call: `bump` = eps x (backward calls since the forward)
+__global__ __launch_bounds__(256) void d_layernorm_bwd_kernel(int rows, int inner, const double* y, const double* dy, double* dx,
+                                                              const double* stdev, double bump)
+{
+    __shared__ double red[4];
+    const size_t base = (size_t)blockIdx.x * inner;
+    double a = 0.0, b = 0.0;
+    for (int i = threadIdx.x; i < inner; i += 256) { a += y[base + i] * dy[base + i]; b += dy[base + i]; }
+    const double m1 = d_block_reduce(a, red, false) / inner;
+    const double m2 = d_block_reduce(b, red, false) / inner;
+    const double sd = stdev[blockIdx.x];
+    for (int i = threadIdx.x; i < inner; i += 256) {
+        const double div = base + i < (size_t)rows ? sd + bump : sd;
+        dx[base + i] = (dy[base + i] - (y[base + i] * m1 + m2)) / div;
+    }
+}
+// y = w (x / sqrt(mean(x^2) + eps)), one workgroup per row
+__global__ __launch_bounds__(256) void d_rmsnorm_kernel(int dim, const double* x, const double* w, double* y, double eps)
+{
+    __shared__ double red[4];
+    const double* xr = x + (size_t)blockIdx.x * dim;
+    double* yr = y + (size_t)blockIdx.x * dim;
+    double ss = 0.0;
+    for (int i = threadIdx.x; i < dim; i += 256) ss += xr[i] * xr[i];
+    const double inv = 1.0 / sqrt(d_block_reduce(ss, red, false) / dim + eps);
+    for (int i = threadIdx.x; i < dim; i += 256) yr[i] = w ? w[i] * (inv * xr[i]) : inv * xr[i];
+}
+// dS = P (dP - sum_k P dP) per row, in place in dp (the softmax gradient of attn.cu:608-661)
+__global__ __launch_bounds__(256) void d_attn_ds_kernel(const double* p, double* dp, int Tk)
+{
+    __shared__ double red[4];
+    const size_t base = (size_t)blockIdx.x * Tk;
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < Tk; j += 256) sum += p[base + j] * dp[base + j];
+    sum = d_block_reduce(sum, red, false);
+    for (int j = threadIdx.x; j < Tk; j += 256) dp[base + j] = p[base + j] * (dp[base + j] - sum);
+}
+
 // Attention forward as the reference's chain computes it (attn.cu:518-602): scores = scale q . k, masked ones -1e29,
 // softmax over the keys, y = p V.  One workgroup per (sequence, head, query row); the row of probabilities stays in LDS.
 // kind 0: no mask, 1: mask (Tq,Tk), 2: mask (B,Tk), 3: mask (B,Tq,Tk); merged: y written (B,Tq,H,hs)
+// probs != nullptr: the row's probabilities are written there as well (B, H, Tq, Tk) and y may be null (the backward pass)
 __global__ __launch_bounds__(256) void d_attn_row_kernel(const double* q, const double* k, const double* v, double* y, int H, int Tq,
-                                                         int Tk, int hs, double scale, const double* mask, int kind, bool merged)
+                                                         int Tk, int hs, double scale, const double* mask, int kind, bool merged,
+                                                         double* probs)
 {
     extern __shared__ double d_smem[];
     double* p = d_smem;        // Tk
@@ -202,6 +387,9 @@ __global__ __launch_bounds__(256) void d_attn_row_kernel(const double* q, const 
         sum += e;
     }
     sum = d_block_reduce(sum, red, false);
+    if (probs)
+        for (int j = threadIdx.x; j < Tk; j += 256) probs[row * Tk + j] = p[j] / sum;
+    if (!y) return;
     double* yr = merged ? y + ((b * Tq + t) * H + h) * (size_t)hs : y + row * hs;
     for (int d = threadIdx.x; d < hs; d += 256) {
         double acc = 0.0;
@@ -212,7 +400,10 @@ __global__ __launch_bounds__(256) void d_attn_row_kernel(const double* q, const 
 
 // ---- the kernel object --------------------------------------------------------------------------------------------
 struct MemD { double* ptr = nullptr; size_t count = 0; bool used = false; };
-struct AttnD { bool set = false; int batch = 0, block = 0, heads = 0, hs = 0; double scale = 1.0; };
+struct AttnD { bool set = false; int batch = 0, block = 0, heads = 0, hs = 0; double scale = 1.0;
+               int lastTq = 0, lastTk = 0; long long lastBatchMask = 0; long lastMask = 0; };   // of the last forward call
+struct LayerNormD { bool set = false; int count = 0, outer = 0, channels = 0, inner = 0, backwards = 0; double eps = 1e-10; double* stdev = nullptr;
+                    ~LayerNormD() { if (stdev) (void)hipFree(stdev); } };
 struct RopeD { bool set = false; int seq = 0, heads = 0, hs = 0; double* dcos = nullptr; double* dsin = nullptr;
                ~RopeD() { if (dcos) (void)hipFree(dcos); if (dsin) (void)hipFree(dsin); } };
 
@@ -222,6 +413,8 @@ public:
     {
         if (m_stream) (void)hipStreamSynchronize(m_stream);
         m_rope.clear();
+        m_layernorm.clear();
+        if (m_ws) (void)hipFree(m_ws);
         for (MemD& m : m_mem)
             if (m.used && m.ptr) (void)hipFree(m.ptr);
         for (double* p : m_host) (void)hipHostFree(p);
@@ -290,6 +483,27 @@ private:
     HandleTable<TensorDesc> m_tdesc;
     HandleTable<AttnD> m_attn;
     HandleTable<RopeD> m_rope;
+    HandleTable<LayerNormD> m_layernorm;
+    double* m_ws = nullptr; size_t m_wsCount = 0;   // scratch of the attention backward call
+    long workspace(size_t count, double** p)
+    {
+        if (count > m_wsCount) {
+            if (m_ws) { HIPCHK(hipStreamSynchronize(m_stream)); HIPCHK(hipFree(m_ws)); m_ws = nullptr; m_wsCount = 0; }
+            HIPCHK(hipMalloc((void**)&m_ws, count * sizeof(double)));
+            m_wsCount = count;
+        }
+        *p = m_ws;
+        return 0;
+    }
+    long attn_mask_kind(AttnD* st, MemD* M, long long batchMask, int T, int Tk, int* kind)
+    {
+        *kind = 0;
+        if (!M) return 0;
+        const long long need = batchMask == 2 ? (long long)st->batch * T * Tk : batchMask == 1 ? (long long)st->batch * Tk : (long long)T * Tk;
+        if ((long long)M->count < need) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+        *kind = batchMask == 2 ? 3 : batchMask == 1 ? 2 : 1;
+        return 0;
+    }
 };
 
 static inline long verify_d(long n, const void* p, long lo, long hi)
@@ -764,6 +978,436 @@ long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, lo
         return 0;
     }
 
+    case MCH_FN_SOFTMAX_BWD: {
+        // f{alpha,beta}, l{hCudnn,0,hTopDataDesc,hTopData,hTopDiffDesc,hTopDiff,0,hBtmDiffDesc,hBtmDiff,alg,mode} (device.h:4801-4823)
+        NEED_F(2, 2);
+        NEED_L(11, 11);
+        if (!m_cudnn.get((long)pl[0])) return MCH_ERROR_PARAM_NULL;
+        TensorDesc* yd = m_tdesc.get((long)pl[2]);
+        TensorDesc* gd = m_tdesc.get((long)pl[4]);
+        TensorDesc* bd = m_tdesc.get((long)pl[7]);
+        if (!yd || !gd || !bd) return MCH_ERROR_PARAM_NULL;
+        if (pf[0] != 1.0 || pf[1] != 0.0) { last_detail = "softmax supports alpha=1, beta=0 only"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        const int alg = (int)pl[9], mode = (int)pl[10];
+        if (alg < 0 || alg > 2 || mode < 0 || mode > 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        for (TensorDesc* d : {gd, bd})
+            if (d->n != yd->n || d->c != yd->c || d->h != yd->h || d->w != yd->w) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        for (TensorDesc* d : {yd, gd, bd})
+            if (!(d->sw == 1 && d->sh == d->w && d->sc == d->h * d->w && d->sn == d->c * d->h * d->w)) {
+                last_detail = "softmax needs fully packed NCHW descriptors";
+                return MCH_ERROR_NOT_IMPLEMENTED;
+            }
+        MemD *Y, *G, *X;
+        ERRCHK(mem((long)pl[3], &Y));
+        ERRCHK(mem((long)pl[5], &G));
+        ERRCHK(mem((long)pl[8], &X));
+        const long long total = (long long)yd->n * yd->c * yd->h * yd->w;
+        RANGE(Y, 0, total);
+        RANGE(G, 0, total);
+        RANGE(X, 0, total);
+        const int len = mode == 0 ? yd->c * yd->h * yd->w : yd->c, inner = mode == 0 ? 1 : yd->h * yd->w;
+        const long long series = (long long)yd->n * inner;
+        if (total == 0) return 0;
+        if (series > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        hipLaunchKernelGGL(d_softmax_bwd_kernel, (int)series, 256, 0, s, (const double*)Y->ptr, (const double*)G->ptr, X->ptr, len, inner, alg == 2);
+        LAUNCHED();
+        return 0;
+    }
+
+    // ---- the layers around the attention: activations, norms, the primitives of their chains --------------------------------
+    case MCH_FN_SWIGLU_FWD: {
+        // l{n,hA,hB,hY}: y = silu(a) b
+        NEED_L(4, 4);
+        const long long n = pl[0];
+        MemD *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        if (n) hipLaunchKernelGGL(d_swiglu_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr, (const double*)B->ptr, Y->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_SILU_BWD:
+    case MCH_FN_GELU_BWD: {
+        // l{count,hTopDiff,hTopData,hBtmDiff,hBtmData[,bert]} (device.h:3269-3316)
+        const bool gelu = fn == MCH_FN_GELU_BWD;
+        NEED_L(gelu ? 6 : 5, gelu ? 6 : 5);
+        const long long n = pl[0];
+        MemD *dY, *dX, *X;
+        ERRCHK(mem((long)pl[1], &dY));
+        ERRCHK(mem((long)pl[3], &dX));
+        ERRCHK(mem((long)pl[4], &X));
+        RANGE(dY, 0, n);
+        RANGE(dX, 0, n);
+        RANGE(X, 0, n);
+        if (n && gelu) hipLaunchKernelGGL(d_gelu_bwd_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)dY->ptr, (const double*)X->ptr, dX->ptr, pl[5] != 0);
+        else if (n) hipLaunchKernelGGL(d_silu_bwd_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)dY->ptr, (const double*)X->ptr, dX->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_GELU_FWD:
+    case MCH_FN_RELU_FWD: {
+        // GELU l{count,hBtm,hTop,bert}; ReLU f{negativeSlope}, l{count,hBtm,hTop,0} (device.h:3253-3266, 4925-4940)
+        const bool gelu = fn == MCH_FN_GELU_FWD;
+        if (!gelu) NEED_F(1, 1);
+        NEED_L(4, 4);
+        const long long n = pl[0];
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        if (n && gelu) hipLaunchKernelGGL(d_gelu_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)X->ptr, Y->ptr, pl[3] != 0);
+        else if (n) hipLaunchKernelGGL(d_relu_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)X->ptr, Y->ptr, pf[0]);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_RELU_BWD: {
+        // f{negativeSlope}, l{count,hTopDiff,hTopData,hBtmDiff,0} (device.h:4943-4959)
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        const long long n = pl[0];
+        MemD *dY, *Y, *dX;
+        ERRCHK(mem((long)pl[1], &dY));
+        ERRCHK(mem((long)pl[2], &Y));
+        ERRCHK(mem((long)pl[3], &dX));
+        RANGE(dY, 0, n);
+        RANGE(Y, 0, n);
+        RANGE(dX, 0, n);
+        if (n) hipLaunchKernelGGL(d_relu_bwd_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)dY->ptr, (const double*)Y->ptr, dX->ptr, pf[0]);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CREATE_LAYERNORM: {
+        // f{eps}, l{gpuId,count,outer,channels,inner} (device.h:4123-4147)
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        const long long count = pl[1], outer = pl[2], channels = pl[3], inner = pl[4];
+        if (outer < 1 || channels < 1 || inner < 1 || count > INT_MAX || outer * channels > INT_MAX || count != outer * channels * inner)
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;   // layernorm.cu:141-142
+        long h;
+        ERRCHK(m_layernorm.create(&h));
+        LayerNormD* ln = m_layernorm.get(h);
+        ln->count = (int)count; ln->outer = (int)outer; ln->channels = (int)channels; ln->inner = (int)inner;
+        ln->eps = pf[0];
+        hipError_t e = hipMalloc((void**)&ln->stdev, (size_t)(outer * channels) * sizeof(double));
+        if (e != hipSuccess) { ln->stdev = nullptr; m_layernorm.free(h); return (long)e; }
+        ln->set = true;
+        return set_out_d((double)h, ppOut, plOut);
+    }
+    case MCH_FN_FREE_LAYERNORM:
+        NEED_F(1, 1);
+        HIPCHK(hipStreamSynchronize(s));
+        return m_layernorm.free((long)pf[0]);
+    case MCH_FN_LAYERNORM_FWD: {
+        // l{hLayerNorm,hX,hY} (layernorm.cu:219-262)
+        NEED_L(3, 3);
+        LayerNormD* ln = m_layernorm.get((long)pl[0]);
+        if (!ln || !ln->set) return MCH_ERROR_LAYERNORM_NOT_INITIALIZED;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(X, 0, ln->count);
+        RANGE(Y, 0, ln->count);
+        hipLaunchKernelGGL(d_layernorm_fwd_kernel, ln->outer * ln->channels, 256, 0, s, ln->inner, (const double*)X->ptr, Y->ptr, ln->stdev, ln->eps);
+        LAUNCHED();
+        ln->backwards = 0;
+        return 0;
+    }
+    case MCH_FN_LAYERNORM_BWD: {
+        // l{hLayerNorm,hYdata,hYdiff,hXdiff} (layernorm.cu:268-312)
+        NEED_L(4, 4);
+        LayerNormD* ln = m_layernorm.get((long)pl[0]);
+        if (!ln || !ln->set) return MCH_ERROR_LAYERNORM_NOT_INITIALIZED;
+        MemD *Y, *dY, *dX;
+        ERRCHK(mem((long)pl[1], &Y));
+        ERRCHK(mem((long)pl[2], &dY));
+        ERRCHK(mem((long)pl[3], &dX));
+        RANGE(Y, 0, ln->count);
+        RANGE(dY, 0, ln->count);
+        RANGE(dX, 0, ln->count);
+        ln->backwards++;
+        const int rows = ln->outer * ln->channels;
+        hipLaunchKernelGGL(d_layernorm_bwd_kernel, rows, 256, 0, s, rows, ln->inner, (const double*)Y->ptr, (const double*)dY->ptr, dX->ptr,
+                           (const double*)ln->stdev, ln->eps * (double)ln->backwards);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_RMSNORM_FWD: {
+        // f{eps}, l{outer,dim,hX,hWeight(0 = none),hY}
+        NEED_F(1, 1);
+        NEED_L(5, 5);
+        const long long outer = pl[0], dim = pl[1];
+        if (outer < 0 || dim < 1 || outer > INT_MAX || dim > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *W = nullptr, *Y;
+        ERRCHK(mem((long)pl[2], &X));
+        if (pl[3]) ERRCHK(mem((long)pl[3], &W));
+        ERRCHK(mem((long)pl[4], &Y));
+        RANGE(X, 0, outer * dim);
+        RANGE(Y, 0, outer * dim);
+        if (W) RANGE(W, 0, dim);
+        if (outer) hipLaunchKernelGGL(d_rmsnorm_kernel, (int)outer, 256, 0, s, (int)dim, (const double*)X->ptr, W ? (const double*)W->ptr : nullptr, Y->ptr, pf[0]);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_SUB: {
+        // l{n,hA,hB,hY[,aOff,bOff,yOff,nB]}: y = a - b[i % nB] when nB > 0 (device.cu:2294-2331)
+        NEED_L(4, 8);
+        const long long n = pl[0], ao = ll > 4 ? pl[4] : 0, bo = ll > 5 ? pl[5] : 0, yo = ll > 6 ? pl[6] : 0, nB = ll > 7 ? pl[7] : 0;
+        MemD *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        if (nB < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(A, ao, n);
+        RANGE(B, bo, nB > 0 ? (nB < n ? nB : n) : n);
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_sub_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr + ao, (const double*)B->ptr + bo, Y->ptr + yo, (size_t)nB);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_DIV: {
+        // l{n,hA,hB,hY}: y = b == 0 ? 0 : a / b (device.cu:2492-2505)
+        NEED_L(4, 4);
+        const long long n = pl[0];
+        MemD *A, *B, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &B));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(A, 0, n);
+        RANGE(B, 0, n);
+        RANGE(Y, 0, n);
+        if (n) hipLaunchKernelGGL(d_div_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr, (const double*)B->ptr, Y->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_ADD_SCALAR: {
+        // f{alpha}, l{n,0,hY[,yOff]} (device.cu:2183-2201)
+        NEED_F(1, 1);
+        NEED_L(3, 4);
+        const long long n = pl[0], yo = ll > 3 ? pl[3] : 0;
+        MemD* Y;
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_add_scalar_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, pf[0], Y->ptr + yo);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_POWX: {
+        // f{alpha}, l{n,hA,0,hY[,aOff,yOff]} (device.cu:2595-2618)
+        NEED_F(1, 1);
+        NEED_L(4, 6);
+        const long long n = pl[0], ao = ll > 4 ? pl[4] : 0, yo = ll > 5 ? pl[5] : 0;
+        MemD *A, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[3], &Y));
+        RANGE(A, ao, n);
+        RANGE(Y, yo, n);
+        if (n) hipLaunchKernelGGL(d_powx_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr + ao, pf[0], Y->ptr + yo);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_SQRT: {
+        // [f{epsilon}], l{n,hX,hY}: y = sqrt(x + epsilon) (device.cu:2712-2728)
+        NEED_L(3, 3);
+        const long long n = pl[0];
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(X, 0, n);
+        RANGE(Y, 0, n);
+        if (n) hipLaunchKernelGGL(d_sqrt_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)X->ptr, Y->ptr, (lf > 0 && pf) ? pf[0] : 0.0);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_INVERT: {
+        // [f{numerator, denominator}], l{n,hX,hY[,xOff,yOff]}: 0 stays 0; factors 0 and 1 are ignored (device.cu:2624-2655)
+        NEED_L(3, 5);
+        const long long n = pl[0], xo = ll > 3 ? pl[3] : 0, yo = ll > 4 ? pl[4] : 0;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[1], &X));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(X, xo, n);
+        RANGE(Y, yo, n);
+        const double num = (lf > 0 && pf) ? pf[0] : 1.0, den = (lf > 1 && pf) ? pf[1] : 1.0;
+        if (n) hipLaunchKernelGGL(d_invert_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)X->ptr + xo, Y->ptr + yo,
+                                  (num != 0.0 && num != 1.0) ? num : 1.0, (den != 0.0 && den != 1.0) ? den : 1.0);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_EXP:
+    case MCH_FN_LOG: {
+        // 235 [f{beta}] l{n,hA,hY[,aOff,yOff,0]}: y = exp(beta a); 236 [f{beta[,alpha]}] l{n,hA,hY[,0,0]}: y = log(beta (a + alpha))
+        const bool isExp = fn == MCH_FN_EXP;
+        ERRCHK(verify_d(lf, pf, 0, isExp ? 1 : 2));
+        if (isExp) NEED_L(3, 6); else NEED_L(3, 5);
+        const long long n = pl[0];
+        long long aOff = isExp && ll > 3 ? pl[3] : 0, yOff = isExp && ll > 4 ? pl[4] : 0;
+        if (n < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (aOff < 0) aOff = 0;
+        if (yOff < 0) yOff = 0;
+        const double beta = lf > 0 ? pf[0] : 1.0, alpha = !isExp && lf > 1 ? pf[1] : 0.0;
+        MemD *A, *Y;
+        ERRCHK(mem((long)pl[1], &A));
+        ERRCHK(mem((long)pl[2], &Y));
+        RANGE(A, aOff, n);
+        RANGE(Y, yOff, n);
+        if (n && isExp) hipLaunchKernelGGL(d_exp_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr + aOff, Y->ptr + yOff, beta);
+        else if (n) hipLaunchKernelGGL(d_log_kernel, grid_of((size_t)n), 256, 0, s, (size_t)n, (const double*)A->ptr, Y->ptr, beta, alpha);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_MEAN: {
+        // l{count,outer,channels,inner,hX,hY[,xOff]}: y[outer*channels] = row means (device.cu:3386-3405)
+        NEED_L(6, 7);
+        const long long outer = pl[1], ch = pl[2], inner = pl[3], xo = ll > 6 ? pl[6] : 0;
+        if (outer < 0 || ch < 0 || inner < 1 || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        RANGE(X, xo, outer * ch * inner);
+        RANGE(Y, 0, outer * ch);
+        if (outer * ch) hipLaunchKernelGGL(d_rowsum_kernel, grid_of((size_t)(outer * ch)), 256, 0, s, (size_t)(outer * ch), (int)inner,
+                                           (const double*)X->ptr + xo, Y->ptr, 1.0 / (double)inner);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_MAX: {
+        // l{count,outer,channels,inner,hX,hY,returnIdx[,acrossChannels]} (device.cu:3359-3380)
+        NEED_L(7, 8);
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        const bool idx = pl[6] != 0, across = ll > 7 ? pl[7] != 0 : true;
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (X->ptr == Y->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, across ? outer * ch * inner : outer * inner * inner);
+        RANGE(Y, 0, outer * inner);
+        if (outer * inner) hipLaunchKernelGGL(d_channel_max_kernel, grid_of((size_t)(outer * inner)), 256, 0, s, (size_t)(outer * inner), (int)ch, (int)inner,
+                                              (const double*)X->ptr, Y->ptr, idx, across);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_SUB:
+    case MCH_FN_CHANNEL_DIV: {
+        // 291 l{count,outer,channels,inner,hX,hY[,hA]}: y[n,c,s] = a[n,c,s] - x[n,s], a = y when absent (device.cu:3438-3457)
+        // 293 l{count,outer,channels,inner,hX,hY[,method]}: y[n,c,s] /= x[n,s]; method 2 with count = outer * inner (device.cu:3541-3560)
+        NEED_L(6, 7);
+        const bool sub = fn == MCH_FN_CHANNEL_SUB;
+        long long count = pl[0];
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        if (count < 0 || outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        if (!sub && ll > 6 && pl[6] == 2) {
+            if (count != outer * inner) { last_detail = "channel_div method 2 takes count = outer * inner only"; return MCH_ERROR_PARAM_OUT_OF_RANGE; }
+            count *= ch;
+        }
+        if (count > outer * ch * inner) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y, *A = nullptr;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (sub && ll > 6) ERRCHK(mem((long)pl[6], &A));
+        RANGE(X, 0, outer * inner);
+        RANGE(Y, 0, count);
+        if (A) RANGE(A, 0, count);
+        if (count) hipLaunchKernelGGL(d_channel_bcast_kernel, grid_of((size_t)count), 256, 0, s, (size_t)count, (int)ch, (int)inner,
+                                      (const double*)(A ? A->ptr : Y->ptr), (const double*)X->ptr, Y->ptr, sub);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_DOT: {
+        // l{count,outer,channels,inner,hX,hA,hY}: y[n,s] = sum_c x[n,c,s] a[n,c,s] (device.cu:3638-3654)
+        NEED_L(7, 7);
+        const long long outer = pl[1], ch = pl[2], inner = pl[3];
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *A, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &A));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (Y->ptr == X->ptr || Y->ptr == A->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(X, 0, outer * ch * inner);
+        RANGE(A, 0, outer * ch * inner);
+        RANGE(Y, 0, outer * inner);
+        if (outer * inner) hipLaunchKernelGGL(d_colsum_kernel, grid_of((size_t)(outer * inner)), 256, 0, s, (size_t)(outer * inner), (int)ch, (int)inner,
+                                              (const double*)X->ptr, (const double*)A->ptr, Y->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_SUM:
+    case MCH_FN_CHANNEL_SUM2: {
+        // 292 l{count,outer,channels,inner,hX,hY}: y[outer,inner] = sum over the channels (device.cu:3488-3503)
+        // 309 l{count,outer,channels,inner,hX,hY,acrossChannels[,dir,channelsY]} (device.cu:3510-3534): forward sums across the
+        //     channels or within every channel; backward writes X from Y, every Y value spread over what it was summed from
+        const bool two = fn == MCH_FN_CHANNEL_SUM2;
+        if (two) NEED_L(7, 9); else NEED_L(6, 6);
+        long long outer = pl[1];
+        const long long ch = pl[2], inner = pl[3];
+        const bool across = two ? pl[6] != 0 : true;
+        const int dir = two && ll > 7 ? (int)pl[7] : 0;
+        const long long chY = two && ll > 8 ? pl[8] : -1;
+        if (outer < 0 || ch < 1 || inner < 1 || ch > INT_MAX || inner > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        // RMSNormLayer.cs:198-199 passes its weight gradient (inner values) as Y with outer = batch: only what Y holds is computed
+        if (!two && outer > 1 && (long long)Y->count < outer * inner && (long long)Y->count >= inner) outer = (long long)Y->count / inner;
+        const long long full = outer * ch * inner, reduced = across ? outer * inner : outer * ch;
+        RANGE(X, 0, full);
+        RANGE(Y, 0, reduced);
+        if (dir == 0) {
+            if (X->ptr == Y->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            if (reduced == 0) return 0;
+            if (across) hipLaunchKernelGGL(d_colsum_kernel, grid_of((size_t)reduced), 256, 0, s, (size_t)reduced, (int)ch, (int)inner, (const double*)X->ptr,
+                                           (const double*)nullptr, Y->ptr);
+            else hipLaunchKernelGGL(d_rowsum_kernel, grid_of((size_t)reduced), 256, 0, s, (size_t)reduced, (int)inner, (const double*)X->ptr, Y->ptr, 1.0);
+            LAUNCHED();
+            return 0;
+        }
+        if (chY == 1 && chY != ch) { last_detail = "channel_sum backward with channelsY = 1 is not supported"; return MCH_ERROR_NOT_IMPLEMENTED; }
+        if (full == 0) return 0;
+        if (across) hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)full), 256, 0, s, 3, (size_t)full, (size_t)1, (size_t)(ch * inner), (size_t)inner, Y->ptr, X->ptr);
+        else hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)full), 256, 0, s, 0, (size_t)full, (size_t)inner, (size_t)1, (size_t)1, Y->ptr, X->ptr);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_CHANNEL_FILLFROM:
+    case MCH_FN_CHANNEL_COPYALL:
+    case MCH_FN_CHANNEL_DUP: {
+        // l{count,outer,channels,inner,hX,hY[,dir]} (math.cu:7465-7481, 7630-7639, 7667-7676)
+        const bool fill = fn == MCH_FN_CHANNEL_FILLFROM;
+        NEED_L(fill ? 7 : 6, fill ? 7 : 6);
+        const long long n = pl[0], outer = pl[1], ch = pl[2], inner = pl[3];
+        if (n < 0 || outer < 1 || ch < 1 || inner < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *Y;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &Y));
+        if (fill && pl[6] != 0) {
+            // backward: x[i] = y[i * inner], i < outer * channels
+            RANGE(X, 0, outer * ch);
+            RANGE(Y, 0, (outer * ch - 1) * inner + 1);
+            hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)(outer * ch)), 256, 0, s, 1, (size_t)(outer * ch), (size_t)inner, (size_t)1, (size_t)1, X->ptr, Y->ptr);
+            LAUNCHED();
+            return 0;
+        }
+        RANGE(Y, 0, n);
+        if (n == 0) return 0;
+        if (fill) {
+            RANGE(X, 0, (n - 1) / inner + 1);
+            hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)n), 256, 0, s, 0, (size_t)n, (size_t)inner, (size_t)1, (size_t)1, X->ptr, Y->ptr);
+        } else if (fn == MCH_FN_CHANNEL_COPYALL) {
+            RANGE(X, 0, n < ch * inner ? n : ch * inner);
+            hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)n), 256, 0, s, 2, (size_t)n, (size_t)1, (size_t)(ch * inner), (size_t)1, X->ptr, Y->ptr);
+        } else {
+            RANGE(X, 0, ((n - 1) / (ch * inner)) * ch + ch);
+            hipLaunchKernelGGL(d_spread_kernel, grid_of((size_t)n), 256, 0, s, 3, (size_t)n, (size_t)1, (size_t)(ch * inner), (size_t)ch, X->ptr, Y->ptr);
+        }
+        LAUNCHED();
+        return 0;
+    }
+
     // ---- attention handle (device.h:2435-2506, attn.cu:408-602) ------------------------------------------------------------
     case MCH_FN_ATTN_CREATE: {
         long h;
@@ -811,17 +1455,68 @@ long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, lo
         if ((long long)Q->count < qn || (long long)Y->count < qn || (long long)K->count < kn || (long long)V->count < kn)
             return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
         int kind = 0;
-        if (M) {
-            const long long need = batchMask == 2 ? (long long)st->batch * T * Tk : batchMask == 1 ? (long long)st->batch * Tk : (long long)T * Tk;
-            if ((long long)M->count < need) return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
-            kind = batchMask == 2 ? 3 : batchMask == 1 ? 2 : 1;
-        }
+        ERRCHK(attn_mask_kind(st, M, batchMask, T, Tk, &kind));
         const size_t lds = ((size_t)Tk + st->hs) * sizeof(double);
         if (lds > 60000) { last_detail = "the double attention call keeps a row of scores in LDS: up to about 7000 keys"; return MCH_ERROR_NOT_IMPLEMENTED; }
         const long long rows = (long long)st->batch * st->heads * T;
         if (rows > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
         hipLaunchKernelGGL(d_attn_row_kernel, (int)rows, 256, lds, s, (const double*)Q->ptr, (const double*)K->ptr, (const double*)V->ptr,
-                           Y->ptr, st->heads, T, Tk, st->hs, st->scale, M ? (const double*)M->ptr : nullptr, kind, merged);
+                           Y->ptr, st->heads, T, Tk, st->hs, st->scale, M ? (const double*)M->ptr : nullptr, kind, merged, (double*)nullptr);
+        LAUNCHED();
+        st->lastTq = T; st->lastTk = Tk; st->lastBatchMask = batchMask; st->lastMask = (long)pl[6];
+        return 0;
+    }
+    case MCH_FN_ATTN_BWD: {
+        // l{hCudnn,hAttn,hQ,hdQ,hK,hdK,hV,hdV,hMask,hY,hdY} (attn.cu:608-661): dV = P^T dY, dP = dY V^T, dS = P (dP - sum P dP),
+        // dQ = scale dS K, dK = scale dS^T Q, with the probabilities recomputed under the last forward call's lengths and
+        // mask (the reference reads the ones that call left behind); without a forward call: block size and hMask
+        NEED_L(11, 11);
+        AttnD* st = m_attn.get((long)pl[1]);
+        if (!st || !st->set) return MCH_ERROR_ATTN_NOT_INITIALIZED;
+        const int T = st->lastTq > 0 ? st->lastTq : st->block, Tk = st->lastTq > 0 ? st->lastTk : st->block;
+        const long long batchMask = st->lastTq > 0 ? st->lastBatchMask : 0;
+        MemD *Q, *dQ, *K, *dK, *V, *dV, *dY, *M = nullptr;
+        ERRCHK(mem((long)pl[2], &Q));
+        ERRCHK(mem((long)pl[3], &dQ));
+        ERRCHK(mem((long)pl[4], &K));
+        ERRCHK(mem((long)pl[5], &dK));
+        ERRCHK(mem((long)pl[6], &V));
+        ERRCHK(mem((long)pl[7], &dV));
+        ERRCHK(mem((long)pl[10], &dY));
+        const long hMask = st->lastTq > 0 ? st->lastMask : (long)pl[8];
+        if (hMask) ERRCHK(mem(hMask, &M));
+        const int H = st->heads, hs = st->hs;
+        const long long bh = (long long)st->batch * H, qn = bh * T * hs, kn = bh * Tk * hs;
+        if ((long long)Q->count < qn || (long long)dQ->count < qn || (long long)dY->count < qn || (long long)K->count < kn ||
+            (long long)dK->count < kn || (long long)V->count < kn || (long long)dV->count < kn)
+            return MCH_ERROR_ATTN_INCOMPATIBLE_BLOB_SIZE;
+        int kind = 0;
+        ERRCHK(attn_mask_kind(st, M, batchMask, T, Tk, &kind));
+        const size_t lds = ((size_t)Tk + hs) * sizeof(double);
+        const long long rows = bh * T, pn = rows * Tk;
+        if (lds > 60000 || rows > INT_MAX || bh > 65535 || pn > (1ll << 28)) {
+            last_detail = "the double attention gradient keeps the probabilities of all rows: up to 2^28 of them, about 7000 keys a row";
+            return MCH_ERROR_NOT_IMPLEMENTED;
+        }
+        double* P;
+        ERRCHK(workspace((size_t)pn * 2, &P));
+        double* dP = P + pn;
+        hipLaunchKernelGGL(d_attn_row_kernel, (int)rows, 256, lds, s, (const double*)Q->ptr, (const double*)K->ptr, (const double*)V->ptr,
+                           (double*)nullptr, H, T, Tk, hs, st->scale, M ? (const double*)M->ptr : nullptr, kind, false, P);
+        LAUNCHED();
+        const long long sq = (long long)T * hs, sk = (long long)Tk * hs, sp = (long long)T * Tk;
+        // dV (Tk x hs) = P^T dY
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((hs + 15) / 16, (Tk + 15) / 16, (int)bh), 256, 0, s, Tk, hs, T, 1.0, (const double*)P, 1ll, (long long)Tk,
+                           (const double*)dY->ptr, (long long)hs, 1ll, 0.0, dV->ptr, (long long)hs, 1ll, sp, sq, sk);
+        // dP (T x Tk) = dY V^T
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((Tk + 15) / 16, (T + 15) / 16, (int)bh), 256, 0, s, T, Tk, hs, 1.0, (const double*)dY->ptr, (long long)hs, 1ll,
+                           (const double*)V->ptr, 1ll, (long long)hs, 0.0, dP, (long long)Tk, 1ll, sq, sk, sp);
+        hipLaunchKernelGGL(d_attn_ds_kernel, (int)rows, 256, 0, s, (const double*)P, dP, Tk);
+        // dQ (T x hs) = scale dS K;  dK (Tk x hs) = scale dS^T Q
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((hs + 15) / 16, (T + 15) / 16, (int)bh), 256, 0, s, T, hs, Tk, st->scale, (const double*)dP, (long long)Tk, 1ll,
+                           (const double*)K->ptr, (long long)hs, 1ll, 0.0, dQ->ptr, (long long)hs, 1ll, sp, sk, sq);
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((hs + 15) / 16, (Tk + 15) / 16, (int)bh), 256, 0, s, Tk, hs, T, st->scale, (const double*)dP, 1ll, (long long)Tk,
+                           (const double*)Q->ptr, (long long)hs, 1ll, 0.0, dK->ptr, (long long)hs, 1ll, sp, sq, sk);
         LAUNCHED();
         return 0;
     }
@@ -888,7 +1583,25 @@ long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, lo
             return MCH_ERROR_PARAM_OUT_OF_RANGE;
         }
         if (pairs) hipLaunchKernelGGL(d_rope_kernel, grid_of((size_t)pairs), 256, 0, s, (size_t)pairs, (const double*)X->ptr, Y->ptr,
-                                      (const double*)r->dcos, (const double*)r->dsin, (size_t)full, (size_t)wrap, (int)half, (int)off);
+                                      (const double*)r->dcos, (const double*)r->dsin, (size_t)full, (size_t)wrap, (int)half, (int)off, 1.0);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_ROPE_BWD: {
+        // l{hRope,n,hXdata,hYdiff,hXdiff}: the rotation by the opposite angle, never shifted (rope.cu:832-864)
+        NEED_L(5, 5);
+        RopeD* r = m_rope.get((long)pl[0]);
+        if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+        const long long n = pl[1];
+        MemD *dY, *dX;
+        ERRCHK(mem((long)pl[3], &dY));
+        ERRCHK(mem((long)pl[4], &dX));
+        if (n < 0 || (n & 1)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        RANGE(dY, 0, n);
+        RANGE(dX, 0, n);
+        const long long half = r->hs / 2, full = half * r->heads, wrap = (long long)r->seq * full, pairs = n / 2;
+        if (pairs) hipLaunchKernelGGL(d_rope_kernel, grid_of((size_t)pairs), 256, 0, s, (size_t)pairs, (const double*)dY->ptr, dX->ptr,
+                                      (const double*)r->dcos, (const double*)r->dsin, (size_t)full, (size_t)wrap, (int)half, 0, -1.0);
         LAUNCHED();
         return 0;
     }

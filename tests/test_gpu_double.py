@@ -255,10 +255,152 @@ def test_double_causal_self_attention_layer(devd, sdpa, rope):
     assert_close(y, ref, ROPE_RTOL if rope else F64_RTOL, "layer output")
 
 
-def test_double_ids_outside_the_attention_path_say_so(devd):
+def test_double_activations_softmax_rope_gradients(devd):
+    rng = np.random.default_rng(22)
+    n = 5001
+    x, g = rng.standard_normal(n) * 3, rng.standard_normal(n)
+    hx, hg, hy, hdx = devd.put(x), devd.put(g), devd.zeros(n), devd.zeros(n)
+    for bert in (True, False):
+        devd.cuda.gelu_fwd(n, hx, hy, bert)
+        assert_close(devd.get(hy), R.gelu(x, bert, np.float64), F64_RTOL, "gelu bert=%s" % bert)
+        devd.cuda.gelu_bwd(n, hg, hy, hdx, hx, bert)
+        assert_close(devd.get(hdx), R.gelu_grad(x, g, bert, np.float64), F64_RTOL, "gelu grad bert=%s" % bert)
+    devd.cuda.silu_bwd(n, hg, hy, hdx, hx)
+    assert_close(devd.get(hdx), R.silu_grad(x, g, np.float64), F64_RTOL, "silu grad")
+    for slope in (0.0, 0.1):
+        devd.cuda.relu_fwd(n, hx, hy, slope)
+        y = devd.get(hy)
+        assert_close(y, R.relu(x, slope, np.float64), F64_RTOL, "relu")
+        devd.cuda.relu_bwd(n, hg, hy, hdx, slope)
+        assert_close(devd.get(hdx), R.relu_grad(y, g, slope, np.float64), F64_RTOL, "relu grad")
+    devd.cuda.SwigluForward(n, hx, hg, hy)
+    assert_close(devd.get(hy), R.silu(x, np.float64) * g, F64_RTOL, "swiglu")
+    # softmax gradient through the layer (cuDNN engine ids 111 / 112)
+    z, dz = rng.standard_normal((3, 4, 5, 33)), rng.standard_normal((3, 4, 5, 33))
+    sm = SoftmaxLayer(devd.cuda, -1)
+    bz, bt = Blob(devd.cuda, z.shape), Blob(devd.cuda)
+    bz.mutable_cpu_data = z
+    sm.Forward(bz, bt)
+    bt.mutable_cpu_diff = dz
+    sm.Backward(bt, bz)
+    yy = R.softmax_lastaxis(z, np.float64)
+    assert_close(bz.mutable_cpu_diff, R.softmax_backward(yy, dz, -1, False, np.float64), F64_RTOL, "softmax gradient")
+    # rope backward undoes rope forward
+    B, T, H, hs = 2, 12, 3, 16
+    r = rng.standard_normal((B, T, H, hs))
+    hr = devd.cuda.CreateRope(0, 0, r.size, B, T, H, hs, 10000.0)
+    h1, h2, h3 = devd.put(r), devd.zeros(r.size), devd.zeros(r.size)
+    devd.cuda.RopeForward(hr, r.size, h1, h2)
+    devd.cuda.RopeBackward(hr, r.size, h1, h2, h3)
+    assert_close(devd.get(h3), r, 1e-6, "rope round trip")
+    assert_close(devd.get(h3), R.rope_backward(devd.get(h2), T, H, hs, dtype=np.float64), ROPE_RTOL, "rope gradient")
+
+
+@pytest.mark.parametrize("kind", ["causal", "keys", "cross"])
+def test_double_attention_backward(devd, kind):
+    B, H, hs = 2, 2, 16
+    Tq, Tk = (24, 40) if kind == "cross" else (32, 32)
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal((B, H, Tq, hs))
+    k, v = rng.standard_normal((B, H, Tk, hs)), rng.standard_normal((B, H, Tk, hs))
+    dy = rng.standard_normal((B, H, Tq, hs))
+    hc, ha = devd.cuda.CreateCuDNN(), devd.cuda.CreateAttn()
+    devd.cuda.SetAttn(hc, ha, 0, True, B, 64, H, hs, 0.0)
+    if kind == "causal":
+        m = np.tril(np.ones((Tq, Tk)))
+        hm, bm, full = devd.put(m), 0, np.broadcast_to(m, (B, H, Tq, Tk))
+    elif kind == "keys":
+        m = (rng.random((B, Tk)) > 0.4).astype(np.float64)
+        hm, bm, full = devd.put(m), 1, np.broadcast_to(m[:, None, None, :], (B, H, Tq, Tk))
+    else:
+        hm, bm, full = 0, 0, np.ones((B, H, Tq, Tk))
+    hq, hk, hv, hy, hdy = devd.put(q), devd.put(k), devd.put(v), devd.zeros(q.size), devd.put(dy)
+    hdq, hdk, hdv = devd.zeros(q.size), devd.zeros(k.size), devd.zeros(v.size)
+    devd.cuda.AttnScaledDotProductForward(hc, ha, Tq, hq, hk, hv, hm, hy, bm, Tk)
+    devd.cuda.AttnScaledDotProductBackward(hc, ha, hq, hdq, hk, hdk, hv, hdv, 0, hy, hdy)
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) / np.sqrt(hs)
+    s = np.where(full == 0, -1e29, s)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    dv = np.einsum("bhqk,bhqd->bhkd", p, dy)
+    dp = np.einsum("bhqd,bhkd->bhqk", dy, v)
+    ds = p * (dp - (p * dp).sum(-1, keepdims=True)) / np.sqrt(hs)
+    assert_close(devd.get(hdv, v.shape), dv, F64_RTOL, "dV")
+    assert_close(devd.get(hdq, q.shape), np.einsum("bhqk,bhkd->bhqd", ds, k), 1e-11, "dQ")
+    assert_close(devd.get(hdk, k.shape), np.einsum("bhqk,bhqd->bhkd", ds, q), 1e-11, "dK")
+
+
+@pytest.mark.parametrize("sdpa", [True, False])
+@pytest.mark.parametrize("name,heads", [("gpt-pico-blk3", 3), ("gpt-pico-blk3B", 3)])
+def test_double_transformer_block_forward_and_backward_golden(devd, name, heads, sdpa, golden_dir):
+    """The reference's own dump of a GPT block (layer norm handle, attention, ReLU MLP, residuals): activations and
+    gradients, the C# call sequence replayed on the double base type - what its test base does for T = double."""
+    import os
+    from mycaffe_amd.layers import TransformerBlockLayer
+    from tests.conftest import load_txt
+    d = os.path.join(golden_dir, name)
+    g = os.path.join(d, "iter_0")
+    p = {k: load_txt(os.path.join(d, k + ".txt")) for k in ("attn_weight", "attn_bias", "attn_proj_weight", "attn_proj_bias",
+                                                             "fc_weight", "fc_bias", "proj_weight", "proj_bias")}
+    x = load_txt(os.path.join(d, "1_x.txt"))
+    B, T, C = x.shape
+    layer = TransformerBlockLayer(devd.cuda, heads, C, T, "relu", True, 1e-10, sdpa, training=True)
+    bx, top = Blob(devd.cuda, x.shape), Blob(devd.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    assert_close(top.mutable_cpu_data, load_txt(os.path.join(d, "10_y.txt")), 2e-6, "block y")
+    top.mutable_cpu_diff = load_txt(os.path.join(g, "grad_1_y.txt"))
+    layer.Backward(top, bx)
+    assert_close(layer.b["Norm2"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_6_x_ln2.txt")), 2e-5, "grad ln2 out")
+    assert_close(bx.mutable_cpu_diff, load_txt(os.path.join(g, "grad_10_x.txt")), 5e-5, "grad x")
+    # and against the checker in float64, where the bar is double's
+    ref = R.transformer_block_gpt(x, p, heads, "relu", 1e-10, np.float64)
+    assert_close(top.mutable_cpu_data, ref["y"], 1e-10, "block y vs the float64 checker")
+
+
+@pytest.mark.parametrize("fused_rmsnorm,sdpa", [(False, False), (True, True)])
+def test_double_llama_style_block_and_its_gradient(devd, fused_rmsnorm, sdpa):
+    """The Llama-style block (RMSNorm chain of primitives or the fused id, rotary attention, SiLU-gated MLP) on the double
+    base type: forward against the checker, input gradient against central differences of the checker."""
+    from mycaffe_amd.layers import TransformerBlockLayer
+    rng = np.random.default_rng(85)
+    B, T, C, H = 2, 6, 16, 2
+    layer = TransformerBlockLayer(devd.cuda, H, C, T, "silu", False, 1e-5, sdpa, training=not fused_rmsnorm, enable_llama_style_head=True,
+                                  multiple_of=8, fused_rmsnorm=fused_rmsnorm)
+    hid = layer.fc1.N
+    p = {"rms1_weight": 1 + 0.1 * rng.standard_normal(C), "rms2_weight": 1 + 0.1 * rng.standard_normal(C),
+         "attn_weight": rng.standard_normal((3 * C, C)) * 0.3, "attn_proj_weight": rng.standard_normal((C, C)) * 0.3,
+         "fc_weight": rng.standard_normal((hid, C)) * 0.3, "fc2_weight": rng.standard_normal((hid, C)) * 0.3,
+         "proj_weight": rng.standard_normal((C, hid)) * 0.3}
+    x, dy = rng.standard_normal((B, T, C)), rng.standard_normal((B, T, C))
+    bx, top = Blob(devd.cuda, x.shape), Blob(devd.cuda)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, p)
+    layer.Forward(bx, top)
+    assert_close(top.mutable_cpu_data, R.transformer_block_llama(x, p, H, T, 10000.0, 1e-5, np.float64), ROPE_RTOL, "llama block")
+    if fused_rmsnorm:
+        return
+    top.mutable_cpu_diff = dy
+    layer.Backward(top, bx)
+    got = bx.mutable_cpu_diff.reshape(x.shape)
+
+    def loss(xx):
+        return float((R.transformer_block_llama(xx, p, H, T, 10000.0, 1e-5, np.float64) * dy).sum())
+
+    num, h = np.zeros(x.shape), 1e-6
+    for i in np.ndindex(*x.shape):
+        xp, xm = x.copy(), x.copy()
+        xp[i] += h
+        xm[i] -= h
+        num[i] = (loss(xp) - loss(xm)) / (2 * h)
+    assert_close(got, num, 1e-5, "llama block dx")
+
+
+def test_double_ids_outside_the_built_set_say_so(devd):
     h = devd.zeros(16)
     with pytest.raises(CudaDnnError) as e:
-        devd.cuda.powx(16, h, 2.0, h)
+        devd.cuda.QkvProjHeads(1, 2, 1, 8, h, h, 0, h, h, h)
     assert e.value.code == 90009 and "double" in str(e.value)
     with pytest.raises(CudaDnnError) as e:
         devd.cuda.CreateExtension("libmycaffe_hip_llama2.so")
