@@ -805,6 +805,12 @@ def main():
                 flat[short + "_prefill_ms"] = d["prefill_128_tokens"]["ms"]
             if d.get("prefill_128_tokens_bf16_activations"):
                 flat[short + "_prefill_bf16_activations_ms"] = d["prefill_128_tokens_bf16_activations"]["ms"]
+    sg = also.get("sampled_generation_fp32_b1")
+    if sg:
+        flat["sampled_top_p_device_ms_per_position"] = sg["top_p_0.9_device_sampler"]["ms_per_position"]
+        flat["sampled_top_p_host_ms_per_position"] = sg["top_p_0.9_host_sampler"]["ms_per_position"]
+        flat["sampled_top_p_device_prompt_128_ms"] = sg["top_p_0.9_device_sampler"]["prompt_128_positions_ms"]
+        flat["sampled_top_p_host_prompt_128_ms"] = sg["top_p_0.9_host_sampler"]["prompt_128_positions_ms"]
     roof.update(flat)
 
     line = {
