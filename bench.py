@@ -502,7 +502,7 @@ def csa_layer_compiled_host(reps):
         return {"error": r.stderr.strip()[-300:]}
     d = json.loads(r.stdout.strip().splitlines()[-1])
     flops = 51.5e9
-    for k in ("f32_fused_ms", "f32_explicit_ms", "bf16_fused_ms", "f32_4call_ms", "bf16_4call_ms"):
+    for k in ("f32_fused_ms", "f32_explicit_ms", "bf16_fused_ms", "f32_4call_ms", "bf16_4call_ms", "f32_3call_ms", "bf16_3call_ms"):
         d[k.replace("_ms", "_TFLOPs_causal_useful")] = round(flops / (d[k] / 1e3) / 1e12, 1)
     return d
 

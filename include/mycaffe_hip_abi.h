@@ -184,11 +184,17 @@ enum {
      * two ROPE_FWD calls the layer makes between the channel copies and the transposes (:538-545).
      * Together with the 11th value of ATTN_FWD (Y written head-merged) the layer forward is four calls:
      * QKV_PROJ_HEADS, ATTN_FWD, GEMM and bias GEMM of the output projection.
+     *
+     * LINEAR_FWD replaces the two GEMM calls of InnerProductLayer.forward (InnerProductLayer.cs:372-417: the product
+     * with the transposed weight, then the rank-1 update with the vector of ones) by one GEMM whose epilogue adds
+     * the bias:  l{M, N, K, hX (M x K), hWeight (N x K), hBias (N; 0 = none), hY (M x N)}.
+     * With it the causal self attention layer's forward is three calls.
      */
     MCH_FN_ATTN_DECODE_FWD = 2001,
     MCH_FN_RMSNORM_FWD = 2002,
     MCH_FN_SWIGLU_FWD = 2003,
-    MCH_FN_QKV_PROJ_HEADS = 2004
+    MCH_FN_QKV_PROJ_HEADS = 2004,
+    MCH_FN_LINEAR_FWD = 2005
 };
 
 /* DEVINIT flags (CudaDnnDLL/Cuda Files/device.h:18-22) */

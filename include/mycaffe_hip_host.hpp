@@ -409,6 +409,11 @@ public:
         if (hRope) ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV, hRope});
         else ex2(MCH_FN_QKV_PROJ_HEADS, {}, {nBatch, nT, nHeads, nSize, hX, hWeight, hBias, hQ, hK, hV});
     }
+    // y (M,N) = x (M,K) W^T (N,K) + bias (hBias 0: none) in one GEMM (no counterpart in the reference)
+    void LinearForward(int nM, int nN, int nK, long hX, long hWeight, long hBias, long hY)
+    {
+        ex2(MCH_FN_LINEAR_FWD, {}, {nM, nN, nK, hX, hWeight, hBias, hY});
+    }
     void RmsNormForward(int nOuter, int nDim, long hX, long hWeight, long hY, float fEps = 1e-5f)
     {
         ex2(MCH_FN_RMSNORM_FWD, {fEps}, {nOuter, nDim, hX, hWeight, hY});

@@ -1056,20 +1056,19 @@ __global__ void qkv_split_heads_kernel(const T* __restrict__ tmp, size_t total, 
     }
 }
 
-hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
-                            void* q, void* k, void* v, void* tmp, const float* fcos, const float* fsin, int ropeSeq)
+// X (m x kk) W^T (n x kk) through the tile kernels' HEADS epilogue `he`, or through `tmp` (m x n) and the splitting pass
+// (tiles256: the 256 x 256 tiles may be chosen as k_gemm chooses them)
+static hipError_t gemm_heads_dispatch(hipStream_t s, DType dt, int m, int n, int kk, const void* X, const void* W, const HeadsEpilogue& he,
+                                      int rowUnit, void* tmp, bool tiles256)
 {
-    if (fcos && (!fsin || ropeSeq < 1 || (hs & 1))) return hipErrorInvalidValue;
-    const int m = B * T, C = H * hs, n = 3 * C, kk = C;
-    if (m <= 0 || C <= 0) return hipSuccess;
-    HeadsEpilogue he;
-    he.bias = bias; he.dst[0] = q; he.dst[1] = k; he.dst[2] = v; he.T = T; he.H = H; he.hs = hs;
-    he.fcos = fcos; he.fsin = fcos ? fsin : nullptr; he.seq = fcos ? ropeSeq : 1;
+    const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
+    const bool full256 = tiles256 && (double)t256 / (double)(((t256 + 255) / 256) * 256) >= 0.85;
     const int vec = dt == F32 ? 4 : 8;
-    const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 == 0) && hs % vec == 0;
+    const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)he.dst[0] | (uintptr_t)he.dst[1] | (uintptr_t)he.dst[2]) % 16 == 0) && rowUnit % vec == 0;
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
     if (aligned && dt == F32 && kk % 32 == 0) {
         hipError_t e;
+        if (full256 && kk >= 1024) return launch_big<float, 4, 4, 1, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (launch_small_if_few<float, true>(&e, s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he)) return e;
         if (n % 192 == 0 && t128 <= 512) return launch_big<float, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (short_last_round(t128) && launch_wide_if_fits<float, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
@@ -1077,6 +1076,7 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
     }
     if (aligned && dt == BF16 && kk % 64 == 0) {
         hipError_t e;
+        if (full256 && kk >= 2048) return launch_big<bf16_t, 4, 4, 1, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (launch_wide_if_fits<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
         if (launch_small_if_few<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he)) return e;
         if (n % 192 == 0 && t128 <= 512) return launch_big<bf16_t, 2, 3, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
@@ -1091,6 +1091,30 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
     if (dt == F32) hipLaunchKernelGGL(qkv_split_heads_kernel<float>, grid, 256, 0, s, (const float*)tmp, total, n, he);
     else hipLaunchKernelGGL(qkv_split_heads_kernel<bf16_t>, grid, 256, 0, s, (const bf16_t*)tmp, total, n, he);
     return hipGetLastError();
+}
+
+hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,
+                            void* q, void* k, void* v, void* tmp, const float* fcos, const float* fsin, int ropeSeq)
+{
+    if (fcos && (!fsin || ropeSeq < 1 || (hs & 1))) return hipErrorInvalidValue;
+    const int m = B * T, C = H * hs, n = 3 * C, kk = C;
+    if (m <= 0 || C <= 0) return hipSuccess;
+    HeadsEpilogue he;
+    he.bias = bias; he.dst[0] = q; he.dst[1] = k; he.dst[2] = v; he.T = T; he.H = H; he.hs = hs;
+    he.fcos = fcos; he.fsin = fcos ? fsin : nullptr; he.seq = fcos ? ropeSeq : 1;
+    return gemm_heads_dispatch(s, dt, m, n, kk, X, W, he, hs, tmp, false);
+}
+
+// Y (m x n) = X (m x k) W^T (n x k) + bias (n): the inner product layer's forward in one launch (InnerProductLayer.cs:
+// 372-417 issues the product and a rank-1 update with a vector of ones).  The HEADS epilogue with one head of n values
+// over m positions is the plain row-major layout, so the same kernels serve.
+hipError_t k_gemm_bias(hipStream_t s, DType dt, int m, int n, int k, const void* X, const void* W, const void* bias, void* Y, void* tmp)
+{
+    if (m <= 0 || n <= 0) return hipSuccess;
+    HeadsEpilogue he;
+    he.bias = bias; he.dst[0] = he.dst[1] = he.dst[2] = Y; he.T = m; he.H = 1; he.hs = n;
+    he.fcos = nullptr; he.fsin = nullptr; he.seq = 1;
+    return gemm_heads_dispatch(s, dt, m, n, k, X, W, he, n, tmp, true);
 }
 
 // C (m x n, fp32) = alpha X W^T + beta C for a 16-bit weight matrix W (n x k), on the bf16 matrix cores, C in fp32.

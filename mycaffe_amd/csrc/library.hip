@@ -1776,6 +1776,28 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return 0;
     }
 
+    case MCH_FN_LINEAR_FWD: {
+        // l{M, N, K, hX, hW, hBias(0 = none), hY}: Y (M x N) = X (M x K) W^T (N x K) + bias (N), one launch
+        NEED_L(7, 7);
+        const long long M = pl[0], N = pl[1], K = pl[2];
+        if (M < 1 || N < 1 || K < 1 || M > INT_MAX || N > INT_MAX || K > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemItem *X, *W, *Bi = nullptr, *Y;
+        ERRCHK(mem((long)pl[3], &X));
+        ERRCHK(mem((long)pl[4], &W));
+        if (pl[5]) ERRCHK(mem((long)pl[5], &Bi));
+        ERRCHK(mem((long)pl[6], &Y));
+        if (X->half != W->half || X->half != Y->half || (Bi && Bi->half != X->half)) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        RANGE(X, 0, M * K);
+        RANGE(W, 0, N * K);
+        if (Bi) RANGE(Bi, 0, N);
+        RANGE(Y, 0, M * N);
+        void* ws = nullptr;
+        ERRCHK(workspace((size_t)(M * N) * X->esize(), &ws));
+        HIPCHK(k_gemm_bias(s, X->dt(), (int)M, (int)N, (int)K, X->ptr, W->ptr, Bi ? Bi->ptr : nullptr, Y->ptr, ws));
+        m_mem.touch((long)pl[6]);
+        return 0;
+    }
+
     // ---- RoPE ------------------------------------------------------------------
     case MCH_FN_CREATE_ROPE: {
         // f{theta}, l{sharedIdx,gpuId,count,batch,seqLen,heads,hs} (device.h:4201-4229, rope.cu:502-607)

@@ -115,6 +115,7 @@ class CUDAFN:
     RMSNORM_FWD = 2002
     SWIGLU_FWD = 2003
     QKV_PROJ_HEADS = 2004
+    LINEAR_FWD = 2005
 
 
 class CUDAQRY:
@@ -696,6 +697,11 @@ class CudaDnn:
         if hRope:
             rgl.append(hRope)
         self._ex2(CUDAFN.QKV_PROJ_HEADS, None, rgl)
+
+    def LinearForward(self, nM, nN, nK, hX, hWeight, hBias, hY):
+        """y (M,N) = x (M,K) W^T (N,K) + bias in one GEMM (no counterpart in the reference: replaces the product and
+        the rank-1 bias update of InnerProductLayer.cs:372-417).  hBias 0: no bias."""
+        self._ex2(CUDAFN.LINEAR_FWD, None, [nM, nN, nK, hX, hWeight, hBias, hY])
 
     def AttnScaledDotProductBackward(self, hCuDnn, hAttn, hQdata, hQdiff, hKdata, hKdiff, hVdata, hVdiff, hMaskdata, hYData, hYdiff):
         """CudaDnn.cs:5695-5701."""

@@ -11,6 +11,7 @@
 //   bf16_fused    16-bit storage (ALLOCMEM_HALF), fused attention handle
 //   *_4call       the same forward as four calls: fused QKV projection writing (B,H,T,hs) (id 2004), attention handle
 //                 writing head-merged output, output projection GEMM and its bias GEMM
+//   *_3call       the same with the output projection and its bias as one call (id 2005)
 // Timed region: `reps` forwards between two device synchronisations (steady_clock), after 60 ms of untimed forwards.
 #include <chrono>
 #include <cmath>
@@ -61,7 +62,7 @@ std::vector<float> normal(size_t n, float std, unsigned seed)
     return v;
 }
 
-double run(CudaDnn& cuda, bool half, bool fused, int reps, bool fourCall = false)
+double run(CudaDnn& cuda, bool half, bool fused, int reps, int calls = 0)
 {
     const int B = 8, T = 1024, C = 768, H = 12, hs = C / H, M = B * T;
     const long long MC = (long long)M * C;
@@ -92,9 +93,13 @@ double run(CudaDnn& cuda, bool half, bool fused, int reps, bool fourCall = false
         cuda.SetTensorDesc(hTopDesc, B * H * T, T, 1, 1, half);
     }
     auto forward = [&]() {
-        if (fourCall) {
+        if (calls) {
             cuda.QkvProjHeads(B, T, H, hs, hX, hWa, hBa, hQt, hKt, hVt);
             cuda.AttnScaledDotProductForward(hCudnn, hAttn, T, hQt, hKt, hVt, hMask, hY, 0, true);
+            if (calls == 3) {
+                cuda.LinearForward(M, C, C, hY, hWp, hBp, hTop);
+                return;
+            }
             cuda.gemm(false, true, M, C, C, 1.f, hY, hWp, 0.f, hTop);
             cuda.gemm(false, false, M, C, 1, 1.f, hOnes, hBp, 1.f, hTop);
             return;
@@ -161,10 +166,12 @@ int main(int argc, char** argv)
         const double a = run(cuda, false, true, reps);
         const double b = run(cuda, false, false, reps);
         const double c = run(cuda, true, true, reps);
-        const double d = run(cuda, false, true, reps, true);
-        const double e = run(cuda, true, true, reps, true);
+        const double d = run(cuda, false, true, reps, 4);
+        const double e = run(cuda, true, true, reps, 4);
+        const double f = run(cuda, false, true, reps, 3);
+        const double g = run(cuda, true, true, reps, 3);
         std::printf("{\"reps\": %d, \"f32_fused_ms\": %.4f, \"f32_explicit_ms\": %.4f, \"bf16_fused_ms\": %.4f, \"f32_4call_ms\": %.4f, "
-                    "\"bf16_4call_ms\": %.4f}\n", reps, a, b, c, d, e);
+                    "\"bf16_4call_ms\": %.4f, \"f32_3call_ms\": %.4f, \"bf16_3call_ms\": %.4f}\n", reps, a, b, c, d, e, f, g);
     } catch (const std::exception& e) {
         std::fprintf(stderr, "csa_layer_bench: %s\n", e.what());
         return 1;

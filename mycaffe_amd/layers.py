@@ -140,8 +140,10 @@ class Blob:
 class InnerProductLayer:
     """MyCaffe/layers/InnerProductLayer.cs:372-417.  Weights are (num_output, K)."""
 
-    def __init__(self, cuda, num_output, bias_term=True, axis=2, half=False):
+    def __init__(self, cuda, num_output, bias_term=True, axis=2, half=False, fused_bias=False):
         self.cuda, self.N, self.bias_term, self.axis, self.half = cuda, num_output, bias_term, axis, half
+        # product and bias in one call (an id with no counterpart in the reference) instead of the two GEMM calls
+        self.fused_bias = fused_bias
         self.blobs = []
         self.bias_multiplier = None
 
@@ -161,7 +163,10 @@ class InnerProductLayer:
         M = bottom.count(0, self.axis)
         top.Reshape(*(bottom.shape_[:self.axis] + [self.N]))
         hW = self.blobs[0].gpu_data
-        if M == 1 and not self.half:
+        if self.fused_bias:
+            self.cuda.LinearForward(M, self.N, self.K, bottom.gpu_data, hW, self.blobs[1].gpu_data if self.bias_term else 0,
+                                    top.gpu_data)
+        elif M == 1 and not self.half:
             self.cuda.gemv(False, self.N, self.K, 1.0, hW, bottom.gpu_data, 0.0, top.gpu_data)
             if self.bias_term:
                 self.cuda.axpy(self.N, 1.0, self.blobs[1].gpu_data, top.gpu_data)
@@ -314,9 +319,10 @@ class CausalSelfAttentionLayer:
                  enable_rotary_positional_embedding=False, rope_theta=10000.0, half=False, training=False,
                  fused_qkv_heads=False):
         self.training = training
-        # four calls per forward instead of seventeen (ids with no counterpart in the reference): the fused QKV
-        # projection writes q, k, v as (B,H,T,hs), rotated where the layer has a rotary embedding, and the attention
-        # handle writes its output head-merged.  Inference, fused attention handle.
+        # three calls per forward instead of seventeen (ids with no counterpart in the reference): the fused QKV
+        # projection writes q, k, v as (B,H,T,hs), rotated where the layer has a rotary embedding, the attention
+        # handle writes its output head-merged and the output projection adds its bias in the GEMM's epilogue.
+        # Inference, fused attention handle.
         self.fused_qkv_heads = fused_qkv_heads
         self.cuda, self.nHeads, self.nEmbed, self.nBlockSize = cuda, heads, embed, block_size
         self.nSize = embed // heads
@@ -325,7 +331,7 @@ class CausalSelfAttentionLayer:
         self.enable_rope, self.rope_theta = enable_rotary_positional_embedding, rope_theta
         self.dfIgnoreVal = -1e29
         self.c_attn = InnerProductLayer(cuda, 3 * embed, bias_term, 2, half)
-        self.c_proj = InnerProductLayer(cuda, embed, bias_term, 2, half)
+        self.c_proj = InnerProductLayer(cuda, embed, bias_term, 2, half, fused_bias=fused_qkv_heads)
         self.transpose = TransposeLayer(cuda, (0, 2, 1, 3))
         self.transposeQ = TransposeLayer(cuda, (0, 1, 3, 2))
         self.softmax = SoftmaxLayer(cuda, -1)

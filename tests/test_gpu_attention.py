@@ -475,7 +475,7 @@ def test_qkv_proj_heads_with_the_rotary_embedding(dev, half, B, T, H, hs):
 
 
 @pytest.mark.parametrize("half", [False, True])
-def test_causal_self_attention_layer_with_rotary_embedding_as_four_calls(dev, half):
+def test_causal_self_attention_layer_with_rotary_embedding_as_three_calls(dev, half):
     B, T, C, H = 2, 128, 256, 4
     rng = np.random.default_rng(T + 1)
     x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
@@ -493,13 +493,13 @@ def test_causal_self_attention_layer_with_rotary_embedding_as_four_calls(dev, ha
         layer.Forward(bottom, top)
         outs.append(top.mutable_cpu_data.copy())
     ref = R.causal_self_attention(x, wa, ba, wp, bp, H, rope=(T, 10000.0), dtype=np.float64)["y"]
-    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "four-call layer vs checker")
-    assert_close(outs[1], outs[0], BF16_RTOL if half else 1e-5, "four-call layer vs the nineteen-call sequence")
+    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "three-call layer vs checker")
+    assert_close(outs[1], outs[0], BF16_RTOL if half else 1e-5, "three-call layer vs the nineteen-call sequence")
 
 
 @pytest.mark.parametrize("half", [False, True])
 @pytest.mark.parametrize("B,T,C,H", [(2, 128, 256, 4), (1, 200, 192, 3), (2, 96, 256, 2), (2, 50, 48, 3)])
-def test_causal_self_attention_layer_as_four_calls(dev, half, B, T, C, H):
+def test_causal_self_attention_layer_as_three_calls(dev, half, B, T, C, H):
     rng = np.random.default_rng(T)
     x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
     wa = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
@@ -515,6 +515,6 @@ def test_causal_self_attention_layer_as_four_calls(dev, half, B, T, C, H):
         layer.Forward(bottom, top)
         outs.append(top.mutable_cpu_data.copy())
     ref = R.causal_self_attention(x, wa, ba, wp, bp, H, dtype=np.float64)["y"]
-    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "four-call layer vs checker")
+    assert_close(outs[1], ref, BF16_RTOL if half else FP32_RTOL, "three-call layer vs checker")
     if not half:
-        assert np.array_equal(outs[0], outs[1]), "four-call layer differs from the seventeen-call sequence"
+        assert np.array_equal(outs[0], outs[1]), "three-call layer differs from the seventeen-call sequence"

@@ -185,6 +185,53 @@ def test_gemm_offsets_and_bias_rank1_update(dev):
     assert_close(out[M // 2:], (x @ W.T)[M // 2:], FP32_RTOL, "gemm offsets")
 
 
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("m,n,k", [
+    (96, 80, 64),           # fewer tiles than CUs, ragged edges
+    (300, 200, 128),        # edge tiles in both directions
+    (512, 768, 192),        # 128 x 192 tiles, interior only
+    (2048, 768, 768),       # the attention layer's output projection
+    (1024, 1024, 2048),     # long contraction
+    (1536, 1152, 2048),     # wide tiles in 16-bit storage
+    (4096, 4096, 2048),     # 256 x 256 tiles in both storage types
+    (37, 53, 29),           # no tile kernel takes it: product in the workspace, then one pass
+    (260, 132, 64),
+])
+def test_linear_forward_is_the_inner_product_with_its_bias(dev, half, bias, m, n, k):
+    """Id 2005 against the float64 checker and against the two calls it replaces (InnerProductLayer.cs:372-417)."""
+    rng = np.random.default_rng(m + n + k + 5)
+    x = bf16_round(rng.standard_normal((m, k)).astype(np.float32))
+    W = bf16_round((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+    b = bf16_round(rng.standard_normal(n).astype(np.float32))
+    hx, hW, hb, hy = dev.put(x, half), dev.put(W, half), dev.put(b, half), dev.put(np.full(m * n, 7.0, np.float32), half)
+    dev.cuda.LinearForward(m, n, k, hx, hW, hb if bias else 0, hy)
+    got = dev.get(hy, (m, n))
+    ref = x.astype(np.float64) @ W.astype(np.float64).T + (b.astype(np.float64) if bias else 0.0)
+    assert_close(got, ref, BF16_RTOL if half else FP32_RTOL, "linear forward vs checker")
+    hy2, hones = dev.zeros(m * n, half), dev.put(np.ones(m, np.float32), half)
+    dev.cuda.gemm(False, True, m, n, k, 1.0, hx, hW, 0.0, hy2)
+    if bias:
+        dev.cuda.gemm(False, False, m, n, 1, 1.0, hones, hb, 1.0, hy2)
+    two = dev.get(hy2, (m, n))
+    # 16-bit storage: the two calls round the product and then the sum, the one call rounds once
+    assert_close(got, two, BF16_RTOL if half else 1e-5, "linear forward vs gemm and bias gemm")
+
+
+def test_linear_forward_checks_its_arguments(dev):
+    hx, hW, hb, hy = dev.zeros(64 * 32), dev.zeros(48 * 32), dev.zeros(48), dev.zeros(64 * 48)
+    dev.cuda.LinearForward(64, 48, 32, hx, hW, hb, hy)
+    with pytest.raises(CudaDnnError):
+        dev.cuda.LinearForward(64, 49, 32, hx, hW, hb, hy)          # weight, bias and y are too short
+    with pytest.raises(CudaDnnError):
+        dev.cuda.LinearForward(0, 48, 32, hx, hW, hb, hy)
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.LinearForward(64, 48, 32, hx, hW, dev.zeros(48, half=True), hy)
+    assert e.value.code == ERROR.MEMORY_MIXED_HALF_TYPES
+    with pytest.raises(CudaDnnError):
+        dev.cuda._ex2(2005, None, [64, 48, 32, hx, hW, hb])
+
+
 def test_matmul_batched_is_gemm2_with_swapped_operands(dev):
     rng = np.random.default_rng(4)
     outer, m, n, k = 6, 50, 24, 40
