@@ -185,6 +185,17 @@ def recorded_traffic(key):
     return None
 
 
+def timed_sets(cuda, fn, rgf, rgl_sets, warm, reps):
+    """`timed` over several argument lists taken in turn (operands that do not stay in the caches between repeats)."""
+    if STEADY_MS > 0:
+        est = cuda.TimeFunctionSets(fn, rgf, rgl_sets, 1, 3)
+        chunk = int(min(5000, max(1, 10.0 / max(est, 1e-4))))
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < STEADY_MS:
+            cuda.TimeFunctionSets(fn, rgf, rgl_sets, 0, chunk)
+    return cuda.TimeFunctionSets(fn, rgf, rgl_sets, warm, max(reps, 2 * len(rgl_sets)))
+
+
 def step_roofline(inf, head, steps, warmup):
     """Roofline of the timed unit, one decode step (one replay of the captured graph: 62 dispatches that stream
     every weight once and the KV cache of the current length), from the HIP-event time of the timed region.
@@ -362,11 +373,26 @@ def bench_decode_attention(cuda, reps, warm=5, cases=None):
                 gbs = nbytes / (ms / 1e3) / 1e9
                 # back-to-back dispatches re-read the same cache: below the 256 MB of last-level cache the figure is
                 # not an HBM rate (and the smallest cases are launch bound)
-                out["%s_B%d_L%d" % (name, B, L)] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
-                                                    "us_attention_kernel_alone": round(ms_attn * 1e3, 2),
-                                                    "fits_last_level_cache": bool(nbytes <= 256e6)}
+                case = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                        "us_attention_kernel_alone": round(ms_attn * 1e3, 2), "fits_last_level_cache": bool(nbytes <= 256e6)}
+                extra = []
+                if nbytes < 800e6:
+                    # the same step over copies of the caches taken in turn, 0.8 GB of them (more than three times the
+                    # last-level cache), so that every dispatch reads its cache from HBM
+                    sets = [rgl]
+                    for _ in range(min(127, int(800e6 // nbytes))):
+                        kc2, vc2 = cuda.AllocMemory(n, bHalfSize=half), cuda.AllocMemory(n, bHalfSize=half)
+                        cuda.copy(n, kc, kc2)
+                        cuda.copy(n, vc, vc2)
+                        extra += [kc2, vc2]
+                        sets.append(rgl[:6] + [kc2, vc2] + rgl[8:])
+                    ms_cold = timed_sets(cuda, CUDAFN.ATTN_DECODE_FWD, [0.0], sets, warm, reps)
+                    gbs_cold = nbytes / (ms_cold / 1e3) / 1e9
+                    case.update({"us_caches_from_hbm": round(ms_cold * 1e3, 2), "GBps_caches_from_hbm": round(gbs_cold, 1),
+                                 "frac_hbm_caches_from_hbm": round(gbs_cold / HBM_PEAK_GBS, 4), "cache_copies_taken_in_turn": len(sets)})
+                out["%s_B%d_L%d" % (name, B, L)] = case
                 cuda.FreeRope(hr)
-                for h in (kc, vc, src, q, kn, vn, y):
+                for h in [kc, vc, src, q, kn, vn, y] + extra:
                     cuda.FreeMemory(h)
     if "bf16_B32_L4096" not in out:
         return out

@@ -361,6 +361,12 @@ MCH_LONG DLL_InvokeDoubleCustomExtensionEx(MCH_LONG lfnIdx, double* pInput, MCH_
 MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
                                 MCH_LONGLONG* plInput, MCH_LONG llInput, MCH_LONG nWarmup, MCH_LONG nReps,
                                 float* pfMs, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
+/* The same with `nSets` lists of `llInput` long arguments each, one after the other in plInput: dispatch i takes list
+ * i mod nSets.  With handles of different buffers in the lists, a kernel whose operands would otherwise stay in the
+ * caches from one repeat to the next is timed on operands that come from memory. */
+MCH_LONG MCH_TimeInvokeFloatEx2Sets(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pInput, MCH_LONG lInput,
+                                    MCH_LONGLONG* plInput, MCH_LONG llInput, MCH_LONG nSets, MCH_LONG nWarmup,
+                                    MCH_LONG nReps, float* pfMs, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
 
 /* ---- entry point that allocates nothing (no counterpart in the reference) ----
  * For callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses

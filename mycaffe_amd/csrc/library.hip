@@ -2211,7 +2211,7 @@ static const char* api_name(long fn)
 #define N(x) {MCH_FN_##x, "CUDA_FN_" #x}
     static const struct { long id; const char* name; } table[] = {
         {MCH_DLL_FREEMEM, "CUDA_DLL_FREEMEM"}, {MCH_DLL_INITIALIZE, "CUDA_DLL_INITIALIZE"}, {MCH_DLL_CLEANUP, "CUDA_DLL_CLEANUP"},
-        N(SETDEVICE), N(GETDEVICE), N(SYNCHRONIZEDEVICE), N(CREATE_MEMORYPOINTER), N(FREE_MEMORYPOINTER), N(ALLOCMEM_HALF), N(ALLOCMEM), N(FREEMEM), N(GETMEM), N(SETMEM), N(CREATE_CUDNN), N(FREE_CUDNN), N(CREATE_TENSORDESC), N(FREE_TENSORDESC), N(SET_TENSORDESC), N(CREATE_EXTENSION), N(FREE_EXTENSION), N(EXTENSION_RUN), N(SOFTMAX_FWD), N(SOFTMAX_BWD), N(ATTN_CREATE), N(ATTN_FREE), N(ATTN_SET), N(ATTN_FWD), N(ATTN_BWD), N(SET), N(COPY), N(GEMM2), N(GEMM), N(GEMV), N(AXPY), N(SCAL), N(SCALE), N(ADD_SCALAR), N(ADD), N(SUB), N(MUL), N(DIV), N(EXP), N(LOG), N(POWX), N(SQRT), N(TRANSPOSE), N(MASK), N(MASK_BATCH), N(TRANSPOSE_HW), N(INVERT), N(CHANNEL_MEAN), N(CHANNEL_MAX), N(CHANNEL_SUB), N(CHANNEL_SUM), N(CHANNEL_DIV), N(CHANNEL_DOT), N(CHANNEL_COPY), N(CHANNEL_FILLFROM), N(CHANNEL_COPYALL), N(CHANNEL_DUP), N(CHANNEL_SUM2), N(EMBED_FWD), N(RELU_FWD), N(RELU_BWD), N(GELU_FWD), N(GELU_BWD), N(SILU_FWD), N(SILU_BWD), N(CREATE_LAYERNORM), N(FREE_LAYERNORM), N(LAYERNORM_FWD), N(LAYERNORM_BWD), N(CREATE_ROPE), N(FREE_ROPE), N(ROPE_FWD), N(ROPE_BWD), N(CREATE_BLOBLOADER), N(FREE_BLOBLOADER), N(BLOBLOADER_LOAD), N(BLOBLOADER_RESETOFFSET), N(BLOBLOADER_ADDTOOFFSET), N(ATTN_DECODE_FWD), N(RMSNORM_FWD), N(SWIGLU_FWD), N(QKV_PROJ_HEADS)};
+        N(SETDEVICE), N(GETDEVICE), N(SYNCHRONIZEDEVICE), N(CREATE_MEMORYPOINTER), N(FREE_MEMORYPOINTER), N(ALLOCMEM_HALF), N(ALLOCMEM), N(FREEMEM), N(GETMEM), N(SETMEM), N(CREATE_CUDNN), N(FREE_CUDNN), N(CREATE_TENSORDESC), N(FREE_TENSORDESC), N(SET_TENSORDESC), N(CREATE_EXTENSION), N(FREE_EXTENSION), N(EXTENSION_RUN), N(SOFTMAX_FWD), N(SOFTMAX_BWD), N(ATTN_CREATE), N(ATTN_FREE), N(ATTN_SET), N(ATTN_FWD), N(ATTN_BWD), N(SET), N(COPY), N(GEMM2), N(GEMM), N(GEMV), N(AXPY), N(SCAL), N(SCALE), N(ADD_SCALAR), N(ADD), N(SUB), N(MUL), N(DIV), N(EXP), N(LOG), N(POWX), N(SQRT), N(TRANSPOSE), N(MASK), N(MASK_BATCH), N(TRANSPOSE_HW), N(INVERT), N(CHANNEL_MEAN), N(CHANNEL_MAX), N(CHANNEL_SUB), N(CHANNEL_SUM), N(CHANNEL_DIV), N(CHANNEL_DOT), N(CHANNEL_COPY), N(CHANNEL_FILLFROM), N(CHANNEL_COPYALL), N(CHANNEL_DUP), N(CHANNEL_SUM2), N(EMBED_FWD), N(RELU_FWD), N(RELU_BWD), N(GELU_FWD), N(GELU_BWD), N(SILU_FWD), N(SILU_BWD), N(CREATE_LAYERNORM), N(FREE_LAYERNORM), N(LAYERNORM_FWD), N(LAYERNORM_BWD), N(CREATE_ROPE), N(FREE_ROPE), N(ROPE_FWD), N(ROPE_BWD), N(CREATE_BLOBLOADER), N(FREE_BLOBLOADER), N(BLOBLOADER_LOAD), N(BLOBLOADER_RESETOFFSET), N(BLOBLOADER_ADDTOOFFSET), N(ATTN_DECODE_FWD), N(RMSNORM_FWD), N(SWIGLU_FWD), N(QKV_PROJ_HEADS), N(LINEAR_FWD)};
 #undef N
     for (const auto& t : table)
         if (t.id == fn) return t.name;
@@ -2425,19 +2425,27 @@ MCH_LONG MCH_AttnDecodeForwardNoAlloc(MCH_LONG kIdx, float* pIn, MCH_LONG lIn, M
 MCH_LONG MCH_TimeInvokeFloatEx2(MCH_LONG kIdx, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn,
                                 MCH_LONG nWarmup, MCH_LONG nReps, float* pfMs, MCH_TCHAR* szErr, MCH_LONG errMax)
 {
+    return MCH_TimeInvokeFloatEx2Sets(kIdx, fn, pIn, lIn, plIn, llIn, 1, nWarmup, nReps, pfMs, szErr, errMax);
+}
+
+MCH_LONG MCH_TimeInvokeFloatEx2Sets(MCH_LONG kIdx, MCH_LONG fn, float* pIn, MCH_LONG lIn, MCH_LONGLONG* plIn, MCH_LONG llIn,
+                                    MCH_LONG nSets, MCH_LONG nWarmup, MCH_LONG nReps, float* pfMs, MCH_TCHAR* szErr, MCH_LONG errMax)
+{
     if (szErr && errMax > 0) szErr[0] = 0;
     Kernel* k = kernel_at(kIdx);
-    if (!k || !pfMs || nReps < 1 || nWarmup < 0) return MCH_ERROR_PARAM_NULL;
+    if (!k || !pfMs || nReps < 1 || nWarmup < 0 || nSets < 1 || (nSets > 1 && (!plIn || llIn < 1))) return MCH_ERROR_PARAM_NULL;
     float dummy[4];
     float* po = dummy;
     MCH_LONG lo = 4;
     long e = 0;
-    for (int i = 0; i < nWarmup && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, plIn, llIn, &po, &lo, true); }
+    // dispatch i takes the i-th list of long arguments, round robin over the nSets lists that lie one after the other
+    auto longs = [&](int i) { return plIn ? plIn + (size_t)(i % nSets) * llIn : plIn; };
+    for (int i = 0; i < nWarmup && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, longs(i), llIn, &po, &lo, true); }
     hipEvent_t a = nullptr, b = nullptr;
     if (!e) e = (long)hipEventCreate(&a);
     if (!e) e = (long)hipEventCreate(&b);
     if (!e) e = (long)hipEventRecord(a, k->stream());
-    for (int i = 0; i < nReps && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, plIn, llIn, &po, &lo, true); }
+    for (int i = 0; i < nReps && !e; i++) { po = dummy; lo = 4; e = k->run(fn, pIn, lIn, longs(nWarmup + i), llIn, &po, &lo, true); }
     if (!e) e = (long)hipEventRecord(b, k->stream());
     if (!e) e = (long)hipEventSynchronize(b);
     float ms = 0.f;

@@ -177,7 +177,7 @@ EXPORTS = (
     "DLL_InvokeFloat", "DLL_InvokeDouble", "DLL_QueryString", "DLL_InvokeFloatEx", "DLL_InvokeDoubleEx",
     "DLL_InvokeFloatEx2", "DLL_InvokeDoubleEx2", "Internal_GetPointerFloat", "Internal_GetPointerDouble",
     "Internal_AllocHostFloat", "Internal_AllocHostDouble", "DLL_QueryStringFloatEx", "DLL_QueryStringDoubleEx",
-    "MCH_TimeInvokeFloatEx2", "MCH_AttnDecodeForwardNoAlloc",
+    "MCH_TimeInvokeFloatEx2", "MCH_AttnDecodeForwardNoAlloc", "MCH_TimeInvokeFloatEx2Sets",
 )
 EXTENSION_EXPORTS = (
     "DLL_InitFloatCustomExtension", "DLL_InvokeFloatCustomExtension", "DLL_InvokeFloatCustomExtensionEx",
@@ -225,6 +225,9 @@ def load_library(path=None):
     lib.MCH_TimeInvokeFloatEx2.argtypes = [_c_long, _c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_long, _c_long,
                                            _c_float_p, _c_tchar_p, _c_long]
     lib.MCH_TimeInvokeFloatEx2.restype = _c_long
+    lib.MCH_TimeInvokeFloatEx2Sets.argtypes = [_c_long, _c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_long, _c_long, _c_long,
+                                               _c_float_p, _c_tchar_p, _c_long]
+    lib.MCH_TimeInvokeFloatEx2Sets.restype = _c_long
     lib.MCH_AttnDecodeForwardNoAlloc.argtypes = [_c_long, _c_float_p, _c_long, _c_longlong_p, _c_long, _c_tchar_p, _c_long]
     lib.MCH_AttnDecodeForwardNoAlloc.restype = _c_long
     return lib
@@ -811,6 +814,22 @@ class CudaDnn:
         err = self._lib.MCH_TimeInvokeFloatEx2(self.m_hKernel, fn, a.ctypes.data_as(_c_float_p) if a is not None else None, n,
                                                l.ctypes.data_as(_c_longlong_p) if l is not None else None, ln, nWarmup, nReps,
                                                ctypes.byref(ms), errbuf, _ERRMAX)
+        self._check(err, errbuf)
+        return float(ms.value)
+
+    def TimeFunctionSets(self, fn, rgf, rglSets, nWarmup=3, nReps=20):
+        """As TimeFunction with one list of long arguments per set: dispatch i takes list i mod len(rglSets), so that
+        the operands of one dispatch are not the ones the previous dispatches left in the caches."""
+        a, n = self._farr(rgf)
+        ll = len(rglSets[0])
+        if any(len(r) != ll for r in rglSets):
+            raise ValueError("the argument lists differ in length")
+        l = np.ascontiguousarray(np.asarray(rglSets, np.int64).reshape(-1))
+        ms = ctypes.c_float(0)
+        errbuf = (ctypes.c_uint16 * _ERRMAX)()
+        err = self._lib.MCH_TimeInvokeFloatEx2Sets(self.m_hKernel, fn, a.ctypes.data_as(_c_float_p) if a is not None else None, n,
+                                                   l.ctypes.data_as(_c_longlong_p), ll, len(rglSets), nWarmup, nReps,
+                                                   ctypes.byref(ms), errbuf, _ERRMAX)
         self._check(err, errbuf)
         return float(ms.value)
 
