@@ -221,16 +221,16 @@ MCH_LONG DLL_InvokeFloatEx(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, float* pI
 /* CudaDnnDLL.cpp:494-853: the double base type.  Kernel indices of these calls are their own table (dllmain.cpp:6-14),
  * arrays cross the boundary as doubles, device memory holds doubles and every result is computed in double.  Built:
  * INITIALIZE / CLEANUP / FREEMEM(-1), SETDEVICE, GETDEVICE, SYNCHRONIZEDEVICE, ALLOCMEM (ALLOCMEM_HALF allocates doubles
- * too), FREEMEM, GETMEM, SETMEM, SET, COPY, GEMM, GEMM2, GEMV, AXPY, SCAL, SCALE, ADD, SUB, MUL, DIV, ADD_SCALAR, POWX,
+ * too), FREEMEM, CREATE / FREE_MEMORYPOINTER, GETMEM, SETMEM, SET, COPY, GEMM, GEMM2, GEMV, AXPY, SCAL, SCALE, ADD, SUB, MUL, DIV, ADD_SCALAR, POWX,
  * SQRT, INVERT, EXP, LOG, MASK, MASK_BATCH, TRANSPOSE, TRANSPOSE_HW, CHANNEL_COPY / MEAN / MAX / SUB / DIV / DOT / SUM /
  * SUM2 / FILLFROM / COPYALL / DUP, EMBED_FWD, SILU / GELU / RELU forward and backward, SWIGLU_FWD, RMSNORM_FWD, CREATE /
  * FREE_LAYERNORM and LAYERNORM_FWD / BWD, CREATE / FREE_CUDNN, CREATE / FREE / SET_TENSORDESC, SOFTMAX_FWD / BWD,
  * ATTN_CREATE / FREE / SET / FWD / BWD (no dropout; the tenth and eleventh values of ATTN_FWD as on the float side),
- * CREATE_ROPE / FREE_ROPE / ROPE_FWD / BWD - same packing as the float ids above: what the attention, multi-head
- * attention and transformer block layers call, forward and backward.  These are one-element-per-thread kernels: the
- * precision twin of the path, not a fast one.  Any other id (memory pointers, the fused ids 2001 / 2004, blob loaders),
- * and DLL_InvokeDoubleEx (extensions and blob loaders are float objects), returns MCH_ERROR_NOT_IMPLEMENTED with the id
- * in the message. */
+ * CREATE_ROPE / FREE_ROPE / ROPE_FWD / BWD, and the fused ids ATTN_DECODE_FWD, QKV_PROJ_HEADS (even head sizes) and
+ * LINEAR_FWD - same packing as the float ids above: what the attention, multi-head attention and transformer block layers
+ * call, forward and backward.  These are one-element-per-thread kernels: the precision twin of the path, not a fast
+ * one.  Any other id (blob loaders, extensions), and DLL_InvokeDoubleEx (extensions and blob loaders are float objects),
+ * returns MCH_ERROR_NOT_IMPLEMENTED with the id in the message. */
 MCH_LONG DLL_InvokeDouble(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,
                           double** ppOutput, MCH_LONG* plOutput, MCH_TCHAR* szErr, MCH_LONG lszErrMax);
 MCH_LONG DLL_InvokeDoubleEx2(MCH_LONG lKernelIdx, MCH_LONG lFunctionIdx, double* pInput, MCH_LONG lInput,

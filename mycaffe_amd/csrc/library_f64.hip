@@ -398,8 +398,108 @@ __global__ __launch_bounds__(256) void d_attn_row_kernel(const double* q, const 
     }
 }
 
+// One query row per (sequence, head) against that head's rows of a key / value cache with any strides (id 2001; the loop
+// it replaces: MultiheadAttentionLayer.cs:713-730).  The row of probabilities stays in LDS.
+__global__ __launch_bounds__(256) void d_attn_decode_kernel(const double* q, const double* kc, const double* vc, double* y, int H,
+                                                            int kvMul, int hs, int len, long long sB, long long sH, long long sT,
+                                                            double scale)
+{
+    extern __shared__ double d_smem[];
+    double* p = d_smem;        // len
+    double* qs = p + len;      // hs
+    __shared__ double red[4];
+    const size_t bh = blockIdx.x;
+    const int h = (int)(bh % H);
+    const size_t b = bh / H;
+    const double* kb = kc + b * sB + (size_t)(h / kvMul) * sH;
+    const double* vb = vc + b * sB + (size_t)(h / kvMul) * sH;
+    for (int d = threadIdx.x; d < hs; d += 256) qs[d] = q[bh * hs + d];
+    __syncthreads();
+    double mx = -INFINITY;
+    for (int j = threadIdx.x; j < len; j += 256) {
+        double sc = 0.0;
+        for (int d = 0; d < hs; d++) sc += qs[d] * kb[(size_t)j * sT + d];
+        sc *= scale;
+        p[j] = sc;
+        mx = fmax(mx, sc);
+    }
+    mx = d_block_reduce(mx, red, true);
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < len; j += 256) {
+        const double e = exp(p[j] - mx);
+        p[j] = e;
+        sum += e;
+    }
+    sum = d_block_reduce(sum, red, false);
+    for (int d = threadIdx.x; d < hs; d += 256) {
+        double acc = 0.0;
+        for (int j = 0; j < len; j++) acc += p[j] * vb[(size_t)j * sT + d];
+        y[bh * hs + d] = acc / sum;
+    }
+}
+
+// The step before it when a rope handle and the new key / value come with the call: q and the new key rotated in place
+// at position `pos` (adjacent pairs), the new key and value stored into the caches at that position.
+__global__ void d_rope_append_kernel(double* q, double* knew, const double* vnew, double* kc, double* vc, int B, int H, int kvH, int hs,
+                                     int pos, long long sB, long long sH, long long sT, const double* fcos, const double* fsin)
+{
+    const int half = hs / 2;
+    const size_t nq = (size_t)B * H * half, nk = (size_t)B * kvH * half, nv = (size_t)B * kvH * hs;
+    GRID_STRIDE(i, nq + nk + nv)
+    {
+        if (i < nq + nk) {
+            const bool isq = i < nq;
+            const size_t pr = isq ? i : i - nq;
+            const int j = (int)(pr % half);
+            const double c = fcos ? fcos[(size_t)pos * half + j] : 1.0, sn = fsin ? fsin[(size_t)pos * half + j] : 0.0;
+            double* x = isq ? q : knew;
+            const double re = x[2 * pr], im = x[2 * pr + 1];
+            const double r0 = re * c - im * sn, r1 = re * sn + im * c;
+            x[2 * pr] = r0;
+            x[2 * pr + 1] = r1;
+            if (!isq) {
+                const size_t bh = pr / half;
+                const size_t dst = (bh / kvH) * sB + (bh % kvH) * sH + (size_t)pos * sT + 2 * j;
+                kc[dst] = r0;
+                kc[dst + 1] = r1;
+            }
+        } else {
+            const size_t pv = i - nq - nk;
+            const size_t bh = pv / hs;
+            vc[(bh / kvH) * sB + (bh % kvH) * sH + (size_t)pos * sT + pv % hs] = vnew[pv];
+        }
+    }
+}
+
+// Epilogue of the fused QKV projection (id 2004): the plain product `tmp` (B*T, 3C) gets its bias and goes, head by head,
+// to q, k, v as (B,H,T,hs); q and k are rotated on the way when the tables are given (position = row % seq).
+__global__ void d_qkv_split_kernel(size_t pairs, const double* tmp, const double* bias, double* q, double* k, double* v, int T, int H,
+                                   int hs, const double* fcos, const double* fsin, int seq)
+{
+    const int C = H * hs;
+    GRID_STRIDE(pi, pairs)
+    {
+        const size_t i = 2 * pi;
+        const size_t r = i / (3 * C);
+        const int c = (int)(i - r * 3 * C);
+        double o0 = tmp[i], o1 = tmp[i + 1];
+        if (bias) { o0 += bias[c]; o1 += bias[c + 1]; }
+        const int which = c / C, w = c - which * C, h = w / hs, d = w - h * hs;
+        if (fcos && which < 2) {
+            const size_t ti = (size_t)(r % seq) * (hs >> 1) + (d >> 1);
+            const double cs = fcos[ti], sn = fsin[ti], re = o0, im = o1;
+            o0 = re * cs - im * sn;
+            o1 = re * sn + im * cs;
+        }
+        double* dst = (which == 0 ? q : which == 1 ? k : v) + (((r / T) * H + h) * T + r % T) * hs + d;
+        dst[0] = o0;
+        dst[1] = o1;
+    }
+}
+__global__ void d_add_bias_rows_kernel(size_t n, int N, const double* bias, double* y) { GRID_STRIDE(i, n) y[i] += bias[i % N]; }
+
 // ---- the kernel object --------------------------------------------------------------------------------------------
-struct MemD { double* ptr = nullptr; size_t count = 0; bool used = false; };
+struct MemD { double* ptr = nullptr; size_t count = 0; bool used = false; long base = 0; };   // base != 0: a view into that handle's allocation
 struct AttnD { bool set = false; int batch = 0, block = 0, heads = 0, hs = 0; double scale = 1.0;
                int lastTq = 0, lastTk = 0; long long lastBatchMask = 0; long lastMask = 0; };   // of the last forward call
 struct LayerNormD { bool set = false; int count = 0, outer = 0, channels = 0, inner = 0, backwards = 0; double eps = 1e-10; double* stdev = nullptr;
@@ -416,7 +516,7 @@ public:
         m_layernorm.clear();
         if (m_ws) (void)hipFree(m_ws);
         for (MemD& m : m_mem)
-            if (m.used && m.ptr) (void)hipFree(m.ptr);
+            if (m.used && m.ptr && !m.base) (void)hipFree(m.ptr);
         for (double* p : m_host) (void)hipHostFree(p);
         if (m_stream) (void)hipStreamDestroy(m_stream);
     }
@@ -467,12 +567,31 @@ private:
         HIPCHK(hipMalloc((void**)&p, (count ? count : 1) * sizeof(double)));
         hipError_t e = hipMemsetAsync(p, 0, (count ? count : 1) * sizeof(double), m_stream);
         if (e != hipSuccess) { (void)hipFree(p); return (long)e; }
-        size_t slot = 0;
-        for (size_t i = 1; i < m_mem.size(); i++)
-            if (!m_mem[i].used) { slot = i; break; }
-        if (!slot) { m_mem.emplace_back(); slot = m_mem.size() - 1; }
+        const size_t slot = new_slot();
+        m_mem[slot] = MemD();
         m_mem[slot].ptr = p; m_mem[slot].count = count; m_mem[slot].used = true;
         *h = (long)slot;
+        return 0;
+    }
+    size_t new_slot()
+    {
+        for (size_t i = 1; i < m_mem.size(); i++)
+            if (!m_mem[i].used) return i;
+        m_mem.emplace_back();
+        return m_mem.size() - 1;
+    }
+    // an allocation takes its views with it (device.h:1000-1020: a memory pointer aliases the handle it was made from)
+    long release(long h)
+    {
+        MemD* it;
+        ERRCHK(mem(h, &it));
+        if (!it->base) {
+            HIPCHK(hipStreamSynchronize(m_stream));
+            for (MemD& m : m_mem)
+                if (m.used && m.base == h) m = MemD();
+            HIPCHK(hipFree(it->ptr));
+        }
+        *it = MemD();
         return 0;
     }
     int m_device = 0;
@@ -566,14 +685,23 @@ long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, lo
         }
         return set_out_d((double)h, ppOut, plOut);
     }
-    case MCH_FN_FREEMEM: {
+    case MCH_FN_FREEMEM:
+    case MCH_FN_FREE_MEMORYPOINTER:
         NEED_L(1, 1);
-        MemD* it;
-        ERRCHK(mem((long)pl[0], &it));
-        HIPCHK(hipStreamSynchronize(s));
-        HIPCHK(hipFree(it->ptr));
-        *it = MemD();
-        return 0;
+        return release((long)pl[0]);
+    case MCH_FN_CREATE_MEMORYPOINTER: {
+        // l{hData, offset, count} (device.h:1000-1020)
+        NEED_L(3, 3);
+        if (pl[1] < 0 || pl[2] < 0) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD* b;
+        ERRCHK(mem((long)pl[0], &b));
+        RANGE(b, pl[1], pl[2]);
+        double* ptr = b->ptr + pl[1];
+        const long root = b->base ? b->base : (long)pl[0];
+        const size_t slot = new_slot();   // b may dangle from here on
+        m_mem[slot] = MemD();
+        m_mem[slot].ptr = ptr; m_mem[slot].count = (size_t)pl[2]; m_mem[slot].used = true; m_mem[slot].base = root;
+        return set_out_d((double)slot, ppOut, plOut);
     }
     case MCH_FN_GETMEM: {
         // l{h, count(-1 = all)}
@@ -1602,6 +1730,119 @@ long KernelD::run(long fn, const double* pf, long lf, const MCH_LONGLONG* pl, lo
         const long long half = r->hs / 2, full = half * r->heads, wrap = (long long)r->seq * full, pairs = n / 2;
         if (pairs) hipLaunchKernelGGL(d_rope_kernel, grid_of((size_t)pairs), 256, 0, s, (size_t)pairs, (const double*)dY->ptr, dX->ptr,
                                       (const double*)r->dcos, (const double*)r->dsin, (size_t)full, (size_t)wrap, (int)half, 0, -1.0);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_LINEAR_FWD: {
+        // l{M, N, K, hX, hW, hBias(0 = none), hY}: Y = X W^T + bias
+        NEED_L(7, 7);
+        const long long M = pl[0], N = pl[1], K = pl[2];
+        if (M < 1 || N < 1 || K < 1 || M > INT_MAX || N > INT_MAX || K > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *X, *W, *Bi = nullptr, *Y;
+        ERRCHK(mem((long)pl[3], &X));
+        ERRCHK(mem((long)pl[4], &W));
+        if (pl[5]) ERRCHK(mem((long)pl[5], &Bi));
+        ERRCHK(mem((long)pl[6], &Y));
+        RANGE(X, 0, M * K);
+        RANGE(W, 0, N * K);
+        if (Bi) RANGE(Bi, 0, N);
+        RANGE(Y, 0, M * N);
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), 1), 256, 0, s, (int)M, (int)N, (int)K, 1.0,
+                           (const double*)X->ptr, K, 1ll, (const double*)W->ptr, 1ll, K, 0.0, Y->ptr, N, 1ll, 0ll, 0ll, 0ll);
+        LAUNCHED();
+        if (Bi) {
+            hipLaunchKernelGGL(d_add_bias_rows_kernel, grid_of((size_t)(M * N)), 256, 0, s, (size_t)(M * N), (int)N, (const double*)Bi->ptr, Y->ptr);
+            LAUNCHED();
+        }
+        return 0;
+    }
+    case MCH_FN_QKV_PROJ_HEADS: {
+        // l{batch, T, heads, hs, hX, hW, hBias(0 = none), hQ, hK, hV [, hRope]}
+        NEED_L(10, 11);
+        const long long B = pl[0], T = pl[1], H = pl[2], hs = pl[3];
+        if (B < 1 || T < 1 || H < 1 || hs < 1 || B * T > INT_MAX || 3 * H * hs > INT_MAX) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const long long C = H * hs, M = B * T;
+        MemD *X, *W, *Bi = nullptr, *Q, *K, *V;
+        ERRCHK(mem((long)pl[4], &X));
+        ERRCHK(mem((long)pl[5], &W));
+        if (pl[6]) ERRCHK(mem((long)pl[6], &Bi));
+        ERRCHK(mem((long)pl[7], &Q));
+        ERRCHK(mem((long)pl[8], &K));
+        ERRCHK(mem((long)pl[9], &V));
+        RANGE(X, 0, M * C);
+        RANGE(W, 0, 3 * C * C);
+        if (Bi) RANGE(Bi, 0, 3 * C);
+        RANGE(Q, 0, M * C);
+        RANGE(K, 0, M * C);
+        RANGE(V, 0, M * C);
+        RopeD* r = nullptr;
+        if (ll > 10 && pl[10]) {
+            r = m_rope.get((long)pl[10]);
+            if (!r || !r->set) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+            if (r->heads != H || r->hs != hs) {
+                last_detail = "the rope handle was created for other heads or another head size";
+                return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            }
+        }
+        if (hs & 1) {
+            last_detail = "the double form of the fused QKV projection takes even head sizes";
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        }
+        double* tmp;
+        ERRCHK(workspace((size_t)(M * 3 * C), &tmp));
+        hipLaunchKernelGGL(d_gemm_kernel, dim3((unsigned)((3 * C + 15) / 16), (unsigned)((M + 15) / 16), 1), 256, 0, s, (int)M, (int)(3 * C), (int)C,
+                           1.0, (const double*)X->ptr, C, 1ll, (const double*)W->ptr, 1ll, C, 0.0, tmp, 3 * C, 1ll, 0ll, 0ll, 0ll);
+        LAUNCHED();
+        const size_t pairs = (size_t)(M * 3 * C) / 2;
+        hipLaunchKernelGGL(d_qkv_split_kernel, grid_of(pairs), 256, 0, s, pairs, (const double*)tmp, Bi ? (const double*)Bi->ptr : nullptr,
+                           Q->ptr, K->ptr, V->ptr, (int)T, (int)H, (int)hs, r ? (const double*)r->dcos : nullptr,
+                           r ? (const double*)r->dsin : nullptr, r ? r->seq : 1);
+        LAUNCHED();
+        return 0;
+    }
+    case MCH_FN_ATTN_DECODE_FWD: {
+        // f{scale (0 = 1/sqrt(hs))}, l{batch, heads, kvHeads, hs, len, hQ, hKcache, hVcache, hY, strideKvBatch, strideKvHead,
+        //   strideKvPos [, hRope, hKnew, hVnew]}
+        NEED_F(1, 1);
+        NEED_L(12, 15);
+        if (ll != 12 && ll != 15) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        const long long B = pl[0], H = pl[1], KVH = pl[2], hs = pl[3], len = pl[4];
+        const long long sB = pl[9], sH = pl[10], sT = pl[11];
+        if (B < 1 || H < 1 || KVH < 1 || hs < 1 || len < 1 || H % KVH || sB < 0 || sH < 0 || sT < 1 || (hs & 1) || B * H > INT_MAX)
+            return MCH_ERROR_PARAM_OUT_OF_RANGE;
+        MemD *Q, *KC, *VC, *Y;
+        ERRCHK(mem((long)pl[5], &Q));
+        ERRCHK(mem((long)pl[6], &KC));
+        ERRCHK(mem((long)pl[7], &VC));
+        ERRCHK(mem((long)pl[8], &Y));
+        RANGE(Q, 0, B * H * hs);
+        RANGE(Y, 0, B * H * hs);
+        const long long need = (B - 1) * sB + (KVH - 1) * sH + (len - 1) * sT + hs;
+        RANGE(KC, 0, need);
+        RANGE(VC, 0, need);
+        const double scale = pf[0] != 0.0 ? pf[0] : 1.0 / sqrt((double)hs);
+        const size_t lds = (size_t)(len + hs) * sizeof(double);
+        if (lds > 60000) {
+            last_detail = "the double form of the decode attention keeps a row of probabilities in LDS: up to about 7000 positions";
+            return MCH_ERROR_NOT_IMPLEMENTED;
+        }
+        if (ll == 15 && (pl[12] || pl[13] || pl[14])) {
+            RopeD* rp = pl[12] ? m_rope.get((long)pl[12]) : nullptr;
+            if (pl[12] && (!rp || !rp->set)) return MCH_ERROR_ROPE_NOT_INITIALIZED;
+            if (rp && (rp->hs != hs || len > rp->seq)) return MCH_ERROR_PARAM_OUT_OF_RANGE;
+            MemD *KN, *VN;
+            ERRCHK(mem((long)pl[13], &KN));
+            ERRCHK(mem((long)pl[14], &VN));
+            RANGE(KN, 0, B * KVH * hs);
+            RANGE(VN, 0, B * KVH * hs);
+            const size_t items = (size_t)(B * H * (hs / 2) + B * KVH * (hs / 2) + B * KVH * hs);
+            hipLaunchKernelGGL(d_rope_append_kernel, grid_of(items), 256, 0, s, Q->ptr, KN->ptr, (const double*)VN->ptr, KC->ptr, VC->ptr, (int)B,
+                               (int)H, (int)KVH, (int)hs, (int)len - 1, sB, sH, sT, rp ? (const double*)rp->dcos : nullptr,
+                               rp ? (const double*)rp->dsin : nullptr);
+            LAUNCHED();
+        }
+        hipLaunchKernelGGL(d_attn_decode_kernel, (unsigned)(B * H), 256, lds, s, (const double*)Q->ptr, (const double*)KC->ptr,
+                           (const double*)VC->ptr, Y->ptr, (int)H, (int)(H / KVH), (int)hs, (int)len, sB, sH, sT, scale);
         LAUNCHED();
         return 0;
     }

@@ -397,10 +397,144 @@ def test_double_llama_style_block_and_its_gradient(devd, fused_rmsnorm, sdpa):
     assert_close(got, num, 1e-5, "llama block dx")
 
 
+def test_double_memory_pointers_alias_the_allocation(devd):
+    x = np.arange(100, dtype=np.float64)
+    h = devd.put(x)
+    v = devd.cuda.CreateMemoryPointer(h, 10, 20)
+    assert np.array_equal(devd.get(v), x[10:30])
+    devd.cuda.set(20, v, -1.0)
+    assert np.array_equal(devd.get(h)[10:30], np.full(20, -1.0)) and devd.get(h)[9] == 9 and devd.get(h)[30] == 30
+    v2 = devd.cuda.CreateMemoryPointer(v, 5, 5)              # a view of a view aliases the allocation
+    devd.cuda.set(5, v2, 2.0)
+    assert np.array_equal(devd.get(h)[15:20], np.full(5, 2.0))
+    with pytest.raises(CudaDnnError):
+        devd.cuda.CreateMemoryPointer(h, 90, 20)
+    devd.cuda.FreeMemoryPointer(v2)
+    assert devd.get(h)[15] == 2.0                             # freeing a view frees nothing else
+    devd.cuda.FreeMemory(h)
+    with pytest.raises(CudaDnnError):
+        devd.cuda.GetMemoryFloat(v)                           # views go with their allocation
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("m,n,k", [(37, 53, 29), (128, 96, 64), (1, 7, 300)])
+def test_double_linear_forward(devd, bias, m, n, k):
+    rng = np.random.default_rng(m + n)
+    x, W, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)), rng.standard_normal(n)
+    hx, hW, hb, hy = devd.put(x), devd.put(W), devd.put(b), devd.put(np.full(m * n, 9.0))
+    devd.cuda.LinearForward(m, n, k, hx, hW, hb if bias else 0, hy)
+    assert_close(devd.get(hy, (m, n)), x @ W.T + (b if bias else 0.0), F64_RTOL, "linear forward")
+    with pytest.raises(CudaDnnError):
+        devd.cuda.LinearForward(m, n + 1, k, hx, hW, hb, hy)
+
+
+@pytest.mark.parametrize("rope", [False, True])
+@pytest.mark.parametrize("bias", [True, False])
+def test_double_qkv_proj_heads(devd, rope, bias):
+    B, T, H, hs = 2, 12, 3, 8
+    C = H * hs
+    rng = np.random.default_rng(4)
+    x, W, b = rng.standard_normal((B, T, C)), rng.standard_normal((3 * C, C)) * 0.2, rng.standard_normal(3 * C)
+    hx, hW, hb = devd.put(x), devd.put(W), devd.put(b)
+    hq, hk, hv = (devd.zeros(B * T * C) for _ in range(3))
+    hr = devd.cuda.CreateRope(0, 0, B * T * C, B, T, H, hs, 10000.0) if rope else 0
+    devd.cuda.QkvProjHeads(B, T, H, hs, hx, hW, hb if bias else 0, hq, hk, hv, hr)
+    ip = x.reshape(B * T, C) @ W.T + (b if bias else 0.0)
+    for i, h in enumerate((hq, hk, hv)):
+        part = ip[:, i * C:(i + 1) * C].reshape(B, T, H, hs)
+        if rope and i < 2:
+            part = np.asarray(R.rope_forward(part, T, H, hs, 10000.0, -1, np.float64, base_double=True)).reshape(B, T, H, hs)
+        assert_close(devd.get(h, (B, H, T, hs)), part.transpose(0, 2, 1, 3), ROPE_RTOL if rope else F64_RTOL, "qkv part %d" % i)
+    if rope:
+        other = devd.cuda.CreateRope(0, 0, B * T * C, B, T, H + 1, hs, 10000.0)
+        with pytest.raises(CudaDnnError):
+            devd.cuda.QkvProjHeads(B, T, H, hs, hx, hW, hb, hq, hk, hv, other)
+
+
+def test_double_causal_self_attention_layer_as_three_calls(devd):
+    B, T, C, H = 2, 24, 48, 3
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((B, T, C))
+    wa, wp = rng.standard_normal((3 * C, C)) * 0.1, rng.standard_normal((C, C)) * 0.1
+    ba, bp = rng.standard_normal(3 * C) * 0.1, rng.standard_normal(C) * 0.1
+    for rope in (False, True):
+        layer = CausalSelfAttentionLayer(devd.cuda, H, C, T, True, True, enable_rotary_positional_embedding=rope, fused_qkv_heads=True)
+        bottom, top = Blob(devd.cuda, x.shape), Blob(devd.cuda)
+        bottom.mutable_cpu_data = x
+        layer.Setup(bottom, wa, ba, wp, bp)
+        layer.Forward(bottom, top)
+        ref = R.causal_self_attention(x, wa, ba, wp, bp, H, rope=(T, 10000.0) if rope else None, dtype=np.float64)["y"]
+        assert_close(top.mutable_cpu_data, ref, ROPE_RTOL if rope else F64_RTOL, "three-call layer, double")
+
+
+@pytest.mark.parametrize("kvH", [4, 2])
+@pytest.mark.parametrize("append", [False, True])
+def test_double_attn_decode_forward(devd, kvH, append):
+    """Id 2001 on the double base type: one query per (sequence, head) over a cache with padded strides, grouped heads,
+    with and without the rotate-and-append step, against the plain float64 formulas."""
+    B, H, hs, L, S = 3, 4, 16, 37, 48
+    rng = np.random.default_rng(kvH + 2 * append)
+    sT, sH = hs + 8, S * (hs + 8) + 16
+    sB = kvH * sH + 32
+    kc, vc = rng.standard_normal(B * sB), rng.standard_normal(B * sB)
+    q, kn, vn = rng.standard_normal((B, H, hs)), rng.standard_normal((B, kvH, hs)), rng.standard_normal((B, kvH, hs))
+    hq, hkc, hvc, hy = devd.put(q), devd.put(kc), devd.put(vc), devd.zeros(B * H * hs)
+    hkn, hvn = devd.put(kn), devd.put(vn)
+    hr = devd.cuda.CreateRope(0, 0, B * S * H * hs, B, S, H, hs, 10000.0)
+    if append:
+        devd.cuda.AttnDecodeForward(B, H, kvH, hs, L, hq, hkc, hvc, hy, sB, sH, sT, 0.0, hr, hkn, hvn)
+    else:
+        devd.cuda.AttnDecodeForward(B, H, kvH, hs, L, hq, hkc, hvc, hy, sB, sH, sT)
+    fcos, fsin = R.rope_tables(S, hs, 10000.0, base_double=True)
+
+    def rot(a, pos):
+        a = a.reshape(-1, hs // 2, 2)
+        c, sn = fcos[pos], fsin[pos]
+        return np.stack([a[..., 0] * c - a[..., 1] * sn, a[..., 0] * sn + a[..., 1] * c], -1).reshape(-1, hs)
+
+    qq = q.reshape(B * H, hs)
+    K = np.zeros((B, kvH, L, hs)); V = np.zeros((B, kvH, L, hs))
+    for b in range(B):
+        for g in range(kvH):
+            for t in range(L):
+                o = b * sB + g * sH + t * sT
+                K[b, g, t], V[b, g, t] = kc[o:o + hs], vc[o:o + hs]
+    if append:
+        qq = rot(qq, L - 1)
+        K[:, :, L - 1] = rot(kn.reshape(-1, hs), L - 1).reshape(B, kvH, hs)
+        V[:, :, L - 1] = vn
+    qq = qq.reshape(B, H, hs)
+    want = np.zeros((B, H, hs))
+    for b in range(B):
+        for h in range(H):
+            g = h // (H // kvH)
+            sc = K[b, g] @ qq[b, h] / np.sqrt(hs)
+            p = np.exp(sc - sc.max())
+            want[b, h] = (p / p.sum()) @ V[b, g]
+    assert_close(devd.get(hy, (B, H, hs)), want, ROPE_RTOL if append else F64_RTOL, "decode attention, double")
+    if append:
+        # q and the new key were rotated in place and the caches hold the new rows
+        assert_close(devd.get(hq, (B * H, hs)), rot(q.reshape(-1, hs), L - 1), ROPE_RTOL, "q rotated in place")
+        got_kc, got_vc = devd.get(hkc), devd.get(hvc)
+        o = 1 * sB + (kvH - 1) * sH + (L - 1) * sT
+        assert_close(got_kc[o:o + hs], K[1, kvH - 1, L - 1], ROPE_RTOL, "appended key")
+        assert np.array_equal(got_vc[o:o + hs], vn[1, kvH - 1])
+        untouched = np.ones(B * sB, bool)
+        for b in range(B):
+            for g in range(kvH):
+                o = b * sB + g * sH + (L - 1) * sT
+                untouched[o:o + hs] = False
+        assert np.array_equal(got_kc[untouched], kc[untouched]) and np.array_equal(got_vc[untouched], vc[untouched])
+    with pytest.raises(CudaDnnError):
+        devd.cuda.AttnDecodeForward(B, H, 3, hs, L, hq, hkc, hvc, hy, sB, sH, sT)          # heads not a multiple of kv heads
+    with pytest.raises(CudaDnnError):
+        devd.cuda.AttnDecodeForward(B, H, kvH, hs, S + 40, hq, hkc, hvc, hy, sB, sH, sT)    # past the cache
+
+
 def test_double_ids_outside_the_built_set_say_so(devd):
     h = devd.zeros(16)
     with pytest.raises(CudaDnnError) as e:
-        devd.cuda.QkvProjHeads(1, 2, 1, 8, h, h, 0, h, h, h)
+        devd.cuda._ex2(CUDAFN.CUDA_BLOBLOADER_LOAD, None, [1, 4, h, 0])
     assert e.value.code == 90009 and "double" in str(e.value)
     with pytest.raises(CudaDnnError) as e:
         devd.cuda.CreateExtension("libmycaffe_hip_llama2.so")
