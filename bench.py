@@ -457,26 +457,27 @@ def bench_gemm(cuda, reps):
                                           "traffic": recorded_traffic("gemm_%s_%s" % (tag, name))}
             for h in (a, w, c):
                 cuda.FreeMemory(h)
-    # InnerProductLayer backward of the QKV layer (fp32): bias update of the forward pass (K = 1), data gradient
+    # InnerProductLayer backward of the QKV layer: bias update of the forward pass (K = 1), data gradient
     # dX = dY W (no transposes) and weight gradient dW += dY^T X (A transposed)
     M, N, K = 8192, 2304, 768
-    x = cuda.AllocMemory(rng.standard_normal(M * K).astype(np.float32))
-    w = cuda.AllocMemory((rng.standard_normal(N * K) * 0.02).astype(np.float32))
-    dy = cuda.AllocMemory(rng.standard_normal(M * N).astype(np.float32))
-    dx, dw = cuda.AllocMemory(M * K), cuda.AllocMemory(N * K)
-    ones, bias = cuda.AllocMemory(np.ones(M, np.float32)), cuda.AllocMemory(np.zeros(N, np.float32))
-    for tag, rgf, rgl, fl in (("f32_qkv_bias_rank1", [1.0, 1.0], [0, 0, M, N, 1, 0, ones, bias, 0, dy], None),
-                              ("f32_qkv_data_grad", [1.0, 0.0], [0, 0, M, K, N, 0, dy, w, 0, dx], 2.0 * M * N * K),
-                              ("f32_qkv_weight_grad", [1.0, 1.0], [1, 0, N, K, M, 0, dy, x, 0, dw], 2.0 * M * N * K)):
-        ms = timed(cuda, CUDAFN.CUDA_GEMM, rgf, rgl, 3, reps)
-        if fl is None:
-            gbs = 2.0 * M * N * 4 / (ms / 1e3) / 1e9
-            out[tag] = {"ms": round(ms, 4), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
-        else:
-            tf = fl / (ms / 1e3) / 1e12
-            out[tag] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS["f32"], 4)}
-    for h in (x, w, dy, dx, dw, ones, bias):
-        cuda.FreeMemory(h)
+    for name, half in (("f32", False), ("bf16", True)):
+        x = cuda.AllocMemory(rng.standard_normal(M * K).astype(np.float32), bHalfSize=half)
+        w = cuda.AllocMemory((rng.standard_normal(N * K) * 0.02).astype(np.float32), bHalfSize=half)
+        dy = cuda.AllocMemory(rng.standard_normal(M * N).astype(np.float32), bHalfSize=half)
+        dx, dw = cuda.AllocMemory(M * K, bHalfSize=half), cuda.AllocMemory(N * K, bHalfSize=half)
+        ones, bias = cuda.AllocMemory(np.ones(M, np.float32), bHalfSize=half), cuda.AllocMemory(np.zeros(N, np.float32), bHalfSize=half)
+        for tag, rgf, rgl, fl in ((name + "_qkv_bias_rank1", [1.0, 1.0], [0, 0, M, N, 1, 0, ones, bias, 0, dy], None),
+                                  (name + "_qkv_data_grad", [1.0, 0.0], [0, 0, M, K, N, 0, dy, w, 0, dx], 2.0 * M * N * K),
+                                  (name + "_qkv_weight_grad", [1.0, 1.0], [1, 0, N, K, M, 0, dy, x, 0, dw], 2.0 * M * N * K)):
+            ms = timed(cuda, CUDAFN.CUDA_GEMM, rgf, rgl, 3, reps)
+            if fl is None:
+                gbs = 2.0 * M * N * (2 if half else 4) / (ms / 1e3) / 1e9
+                out[tag] = {"ms": round(ms, 4), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+            else:
+                tf = fl / (ms / 1e3) / 1e12
+                out[tag] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS[name], 4)}
+        for h in (x, w, dy, dx, dw, ones, bias):
+            cuda.FreeMemory(h)
     return out
 
 

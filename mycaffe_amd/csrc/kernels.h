@@ -97,8 +97,11 @@ hipError_t k_channel_dot(hipStream_t s, DType dt, size_t num, int channels, int 
 
 // ---- GEMM family (gemm.hip) ------------------------------------------------
 // row-major C[m,n] = alpha*op(A)*op(B) + beta*C; A, B, C all of storage type dt
+// ws: k_gemm_workspace_bytes(...) bytes of scratch for the transpose combinations that run as "transpose the operand that
+// lies the other way, then the A B^T kernels" (without it they take the strided kernels)
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
-                  const void* B, float beta, void* C);
+                  const void* B, float beta, void* C, void* ws = nullptr, size_t wsBytes = 0);
+size_t k_gemm_workspace_bytes(DType dt, bool tA, bool tB, int m, int n, int k);
 // Fused QKV projection of CausalSelfAttentionLayer: [q|k|v] = X W^T + bias with X (B*T, C), W (3C, C), C = H*hs, written
 // straight into three (B,H,T,hs) tensors.  tmp: (B*T, 3C) scratch, only used for shapes the fused kernel does not take.
 hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs, const void* X, const void* W, const void* bias,

@@ -672,7 +672,11 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             RANGE(A, ao, (long long)m * k);
             RANGE(B, bo, (long long)k * n);
             RANGE(C, co, (long long)m * n);
-            HIPCHK(k_gemm(s, A->dt(), tA, tB, m, n, k, pf[0], PTR(A, ao), PTR(B, bo), pf[1], PTR(C, co)));
+            // the transpose combinations of the layers' backward passes turn an operand in scratch memory
+            void* ws = nullptr;
+            const size_t wsb = k_gemm_workspace_bytes(A->dt(), tA, tB, m, n, k);
+            if (wsb) ERRCHK(workspace(wsb, &ws));
+            HIPCHK(k_gemm(s, A->dt(), tA, tB, m, n, k, pf[0], PTR(A, ao), PTR(B, bo), pf[1], PTR(C, co), ws, wsb));
         }
         m_mem.touch((long)pl[9]);
         return 0;

@@ -168,6 +168,29 @@ def test_gemm_bf16_large_tile_paths(dev, m, n, k, alpha, beta):
     assert_close(dev.get(hC, (m, n)), ref, BF16_RTOL, "gemm bf16 large tiles")
 
 
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k,beta", [
+    (1024, 768, 512, 0.0),      # data gradient shape: large enough in fp32 for the operand to be turned in scratch memory
+    (768, 512, 2048, 1.0),      # weight gradient shape, accumulated into the result (beta = 1)
+    (264, 200, 136, 0.5),       # ragged tiles, multiples of eight
+    (260, 132, 72, 0.0),        # multiples of four only: 16-bit storage keeps the strided kernel
+])
+def test_gemm_backward_transpose_combinations(dev, half, tA, tB, m, n, k, beta):
+    """The transpose combinations of InnerProductLayer.backward (InnerProductLayer.cs:429-494) at sizes where an operand
+    is turned in scratch memory and the product runs on the A B^T kernels, against the float64 checker."""
+    rng = np.random.default_rng(m + n + k + 2 * tA + tB)
+    A = bf16_round(rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32))
+    B = bf16_round((rng.standard_normal((n, k) if tB else (k, n)) * 0.05).astype(np.float32))
+    C0 = bf16_round(rng.standard_normal((m, n)).astype(np.float32))
+    hA, hB, hC = dev.put(A, half), dev.put(B, half), dev.put(C0, half)
+    dev.cuda.gemm(tA, tB, m, n, k, 1.0, hA, hB, beta, hC)
+    ref = R.gemm(tA, tB, m, n, k, 1.0, A, B, beta, C0, dtype=np.float64)
+    assert_close(dev.get(hC, (m, n)), ref, BF16_RTOL if half else FP32_RTOL, "gemm, transposed operands")
+    # the operands are left as they were
+    assert np.array_equal(dev.get(hA), A.reshape(-1)) and np.array_equal(dev.get(hB), B.reshape(-1))
+
+
 def test_gemm_offsets_and_bias_rank1_update(dev):
     # InnerProductLayer.cs:411-415: y = x W^T, then y += ones(M,1) * bias(1,N) through gemm with K = 1
     rng = np.random.default_rng(3)
