@@ -469,8 +469,14 @@ template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC =
 __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int K, float alpha, const T* __restrict__ A,
                                                                const T* __restrict__ B, float beta, TC* __restrict__ C, int tilesN,
                                                                int tilesTotal, int bandRows, int colBlock, HeadsEpilogue he,
-                                                               PromptEpilogue pe)
+                                                               PromptEpilogue pe, int ld)
 {
+    // K: the contraction length of this launch's products, ld: the distance between rows of A and of B.  With a second
+    // grid dimension, workgroup row y multiplies columns y K .. y K + K - 1 of the operands into the y-th M x N matrix
+    // behind C (partial products of a long contraction, added up by splitk_reduce_kernel).
+    A += (size_t)blockIdx.y * K;
+    B += (size_t)blockIdx.y * K;
+    C += (size_t)blockIdx.y * M * N;
     static_assert(EPI == 0 || !std::is_same<T, TC>::value, "the prompt epilogues take the fp32 results of 16-bit operands");
     static_assert(std::is_same<T, TC>::value || (!HEADS && std::is_same<TC, float>::value), "C is of the operands' type, or fp32");
     static_assert(!SPLIT || !std::is_same<T, TC>::value, "the split product writes fp32");
@@ -521,11 +527,11 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
     const T* ga[PA];
     const T* gb[PB];
 #pragma unroll
-    for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * (SPLIT ? 2 * K : K) + lc;
+    for (int p = 0; p < PA; p++) ga[p] = A + (size_t)min(m0 + lr + p * RPP, M - 1) * (SPLIT ? 2 * K : ld) + lc;
 #pragma unroll
     for (int p = 0; p < PB; p++) {
         const int c = min(n0 + lr + p * RPP, N - 1);
-        gb[p] = B + (size_t)(EPI == 1 ? (c & 1) * pe.hid + (c >> 1) : c) * K + lc;
+        gb[p] = B + (size_t)(EPI == 1 ? (c & 1) * pe.hid + (c >> 1) : c) * ld + lc;
     }
     T* sa = As + lr * LDK + lc;
     T* sb = Bs + lr * LDK + lc;
@@ -748,8 +754,11 @@ __global__ __launch_bounds__(256, OCC) void gemm_nt_big_kernel(int M, int N, int
 
 template <typename T, int WM, int WN, int OCC, bool HEADS = false, typename TC = T, bool SPLIT = false, int EPI = 0>
 static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, const void* A, const void* B, float beta, void* C,
-                             const HeadsEpilogue* heads = nullptr, const PromptEpilogue* prompt = nullptr)
+                             const HeadsEpilogue* heads = nullptr, const PromptEpilogue* prompt = nullptr, int ksplits = 1)
 {
+    // ksplits > 1: the contraction in ksplits equal parts, part y into the y-th m x n matrix behind C
+    const int ld = k;
+    k /= ksplits;
     PromptEpilogue pe = {};
     if (prompt) pe = *prompt;
     HeadsEpilogue he = {};
@@ -780,8 +789,8 @@ static hipError_t launch_big(hipStream_t s, int m, int n, int k, float alpha, co
             colBlock = (tn + nb - 1) / nb;   // equal-width blocks
         }
     }
-    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT, EPI>), dim3(per * 8), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
-                       (TC*)C, tn, (int)total, bandRows, colBlock, he, pe);
+    hipLaunchKernelGGL((gemm_nt_big_kernel<T, WM, WN, OCC, HEADS, TC, SPLIT, EPI>), dim3(per * 8, ksplits), 256, lds, s, m, n, k, alpha, (const T*)A, (const T*)B, beta,
+                       (TC*)C, tn, (int)total, bandRows, colBlock, he, pe, ld);
     return hipGetLastError();
 }
 
@@ -1218,6 +1227,38 @@ static hipError_t transpose2d(hipStream_t s, DType dt, const void* x, void* y, i
 // storage that replaces the strided scalar kernel (8192 x 768 x 2304: 604 -> 3x us, the weight gradient 1778 -> 5x us),
 // in fp32 the strided MFMA kernel where the product is large enough to pay for the pass over the operand.
 static size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// A long contraction with few tiles (weight gradients: K is the token count) is cut into 2 .. 16 equal parts, one row of
+// workgroups of 128 x 128 tiles each, until the launch has some 400 workgroups; every part stays 512 long at least.
+static int gemm_ksplits(DType dt, int m, int n, int k)
+{
+    const int bk = dt == F32 ? 32 : 64;
+    const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+    if (t128 >= 200 || k < 2048 || ((long long)m * n) % 4) return 1;
+    int S = 1;
+    while (S < 16 && t128 * S < 400 && k % (2 * S * bk) == 0 && k / (2 * S) >= 512) S *= 2;
+    return S;
+}
+// C = sum of the S partial products (fp32, alpha already applied) + beta C
+template <typename T>
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, int S, size_t total4, float beta, T* __restrict__ C)
+{
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total4; e += (size_t)blockDim.x * gridDim.x) {
+        float4 a = *(const float4*)(part + 4 * e);
+        for (int z = 1; z < S; z++) {
+            const float4 b = *(const float4*)(part + (size_t)z * total4 * 4 + 4 * e);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        float v[4] = {a.x, a.y, a.z, a.w};
+        if (beta != 0.f) {
+            float c[4];
+            Quad<T>::load(C + 4 * e, c);
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[q] += beta * c[q];
+        }
+        Quad<T>::store(C + 4 * e, v);
+    }
+}
 static bool gemm_turns_operands(DType dt, bool tA, bool tB, int m, int n, int k)
 {
     if (!tA && tB) return false;
@@ -1228,11 +1269,18 @@ static bool gemm_turns_operands(DType dt, bool tA, bool tB, int m, int n, int k)
     // fp32: 136 against 88 TFLOP/s for the product, about 3 TB/s (read + write) for the pass over an operand
     return (double)m * n * k * 8.0e-15 > 1.5 * turned * 8.0 / 3.0e12;
 }
-size_t k_gemm_workspace_bytes(DType dt, bool tA, bool tB, int m, int n, int k)
+static size_t gemm_turned_bytes(DType dt, bool tA, bool tB, int m, int n, int k)
 {
-    if (m <= 0 || n <= 0 || k <= 0 || !gemm_turns_operands(dt, tA, tB, m, n, k)) return 0;
     const size_t es = dt == F32 ? 4 : 2;
     return (tA ? round256((size_t)m * k * es) : 0) + (!tB ? round256((size_t)n * k * es) : 0);
+}
+size_t k_gemm_workspace_bytes(DType dt, bool tA, bool tB, int m, int n, int k)
+{
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const bool nt = !tA && tB;
+    if (!nt && !gemm_turns_operands(dt, tA, tB, m, n, k)) return 0;
+    const int S = k % (dt == F32 ? 4 : 8) == 0 ? gemm_ksplits(dt, m, n, k) : 1;
+    return (nt ? 0 : gemm_turned_bytes(dt, tA, tB, m, n, k)) + (S > 1 ? (size_t)S * m * n * sizeof(float) : 0);
 }
 
 hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k, float alpha, const void* A,
@@ -1254,8 +1302,9 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
             hipError_t e = transpose2d(s, dt, B, w, k, n);
             if (e != hipSuccess) return e;
             b2 = w;
+            w += round256((size_t)n * k * es);
         }
-        return k_gemm(s, dt, false, true, m, n, k, alpha, a2, b2, beta, C);
+        return k_gemm(s, dt, false, true, m, n, k, alpha, a2, b2, beta, C, w, wsBytes - (size_t)(w - (char*)ws));
     }
     if (k == 1) {
         const size_t es = dt == F32 ? 4 : 2;
@@ -1283,6 +1332,17 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
         const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
         const double fill = (double)t256 / (double)(((t256 + 255) / 256) * 256);
         const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
+        const int S = ws && (((uintptr_t)ws | (uintptr_t)C) % 16 == 0) ? gemm_ksplits(dt, m, n, k) : 1;
+        if (S > 1 && wsBytes >= (size_t)S * m * n * sizeof(float)) {
+            hipError_t e = dt == F32 ? launch_big<float, 2, 2, 2>(s, m, n, k, alpha, A, B, 0.f, ws, nullptr, nullptr, S)
+                                     : launch_big<bf16_t, 2, 2, 2, false, float>(s, m, n, k, alpha, A, B, 0.f, ws, nullptr, nullptr, S);
+            if (e != hipSuccess) return e;
+            const size_t total4 = (size_t)m * n / 4;
+            const int g = (int)std::min<size_t>((total4 + 255) / 256, 4096);
+            if (dt == F32) hipLaunchKernelGGL(splitk_reduce_kernel<float>, g, 256, 0, s, (const float*)ws, S, total4, beta, (float*)C);
+            else hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, g, 256, 0, s, (const float*)ws, S, total4, beta, (bf16_t*)C);
+            return hipGetLastError();
+        }
         if (dt == F32) {
             if (k % 32 == 0) {
                 if (k >= 1024 && fill >= 0.85) return launch_big<float, 4, 4, 1>(s, m, n, k, alpha, A, B, beta, C);

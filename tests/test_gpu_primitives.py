@@ -191,6 +191,32 @@ def test_gemm_backward_transpose_combinations(dev, half, tA, tB, m, n, k, beta):
     assert np.array_equal(dev.get(hA), A.reshape(-1)) and np.array_equal(dev.get(hB), B.reshape(-1))
 
 
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("tA,tB", [(False, True), (True, False)])
+@pytest.mark.parametrize("m,n,k,alpha,beta", [
+    (768, 512, 4096, 1.0, 0.0),     # 24 tiles of 128 x 128: eight parts of 512
+    (300, 260, 2048, 0.5, 1.0),     # ragged tiles, two parts, both scalars
+    (1536, 1152, 2048, 1.0, 1.0),   # 108 tiles: two parts
+])
+def test_gemm_long_contraction_split_over_workgroups(dev, half, tA, tB, m, n, k, alpha, beta):
+    """Weight-gradient shapes (few tiles, the token count as the contraction): partial products of equal slices of K by
+    rows of workgroups, summed in fp32 by a second kernel; against the float64 checker."""
+    rng = np.random.default_rng(m + n + k + tA)
+    A = bf16_round(rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32))
+    B = bf16_round((rng.standard_normal((n, k) if tB else (k, n)) * 0.05).astype(np.float32))
+    C0 = bf16_round(rng.standard_normal((m, n)).astype(np.float32))
+    hA, hB, hC = dev.put(A, half), dev.put(B, half), dev.put(C0, half)
+    dev.cuda.gemm(tA, tB, m, n, k, alpha, hA, hB, beta, hC)
+    ref = R.gemm(tA, tB, m, n, k, alpha, A, B, beta, C0, dtype=np.float64)
+    assert_close(dev.get(hC, (m, n)), ref, BF16_RTOL if half else FP32_RTOL, "gemm, split contraction")
+    # The same call again gives the same bits: the parts are summed in a fixed order.  (An fp32 product too small to pay
+    # for turning its operands stays on the strided kernel, which adds its parts with atomics.)
+    if half or not tA:
+        hC2 = dev.put(C0, half)
+        dev.cuda.gemm(tA, tB, m, n, k, alpha, hA, hB, beta, hC2)
+        assert np.array_equal(dev.get(hC2), dev.get(hC))
+
+
 def test_gemm_offsets_and_bias_rank1_update(dev):
     # InnerProductLayer.cs:411-415: y = x W^T, then y += ones(M,1) * bias(1,N) through gemm with K = 1
     rng = np.random.default_rng(3)
