@@ -736,13 +736,21 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         ERRCHK(mem((long)pl[4], &A));
         ERRCHK(mem((long)pl[5], &X));
         ERRCHK(mem((long)pl[7], &Y));
-        if (X->half || Y->half) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
+        // vectors in 16-bit storage: with a 16-bit matrix the call is the product with a one-column matrix (the bias
+        // gradient of an inner product kept in 16-bit storage); the reference reads such memory as floats (math.cu:2155-2185)
+        const bool all16 = A->half && X->half && Y->half;
+        if ((X->half || Y->half) && !all16) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
         if (aOff < 0) aOff = 0;
         if (xOff < 0) xOff = 0;
         if (yOff < 0) yOff = 0;
         RANGE(A, aOff, (long long)m * n);
         RANGE(X, xOff, tA ? m : n);
         RANGE(Y, yOff, tA ? n : m);
+        if (all16) {
+            HIPCHK(k_gemm(s, BF16, tA, false, tA ? n : m, 1, tA ? m : n, pf[0], PTR(A, aOff), PTR(X, xOff), pf[1], PTR(Y, yOff)));
+            m_mem.touch((long)pl[7]);
+            return 0;
+        }
         HIPCHK(k_gemv(s, A->dt(), tA, m, n, pf[0], PTR(A, aOff), (const float*)PTR(X, xOff), pf[1], (float*)PTR(Y, yOff)));
         m_mem.touch((long)pl[7]);
         return 0;

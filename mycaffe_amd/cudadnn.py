@@ -153,6 +153,7 @@ class ERROR:
     NOT_IMPLEMENTED = 90009
     MEMORY_RANGE_EXCEEDED = 90010
     MEMORY_MIXED_HALF_TYPES = 90011
+    MEMORY_HALF_TYPE_NOT_SUPPORTED = 90012
     MEMORY_NOT_FOUND = 90014
     LAYERNORM_NOT_INITIALIZED = 90161
     ROPE_NOT_INITIALIZED = 90201

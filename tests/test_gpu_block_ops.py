@@ -253,6 +253,47 @@ def test_causal_self_attention_layer_backward_golden(dev, name, heads, sdpa):
         assert_close(layer.b["Kt1"].mutable_cpu_diff, load_txt(os.path.join(g, "grad_kt1.txt")), 2e-5, "grad k^T")
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_causal_self_attention_layer_backward_at_a_tiled_shape(dev, half):
+    """Forward and backward of the layer at B = 2, T = 256, C = 256, four heads, in fp32 and in 16-bit storage, where the
+    attention gradient runs on the tiled kernels and the inner products' data and weight gradients (InnerProductLayer.cs:
+    429-494) on the A B^T kernels with a turned operand; against the float64 formulas of the same layer."""
+    from mycaffe_amd.layers import CausalSelfAttentionLayer
+    B, T, C, H = 2, 256, 256, 4
+    hs = C // H
+    rng = np.random.default_rng(77)
+    x = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    wa = bf16_round((rng.standard_normal((3 * C, C)) * 0.05).astype(np.float32))
+    wp = bf16_round((rng.standard_normal((C, C)) * 0.05).astype(np.float32))
+    ba = bf16_round((rng.standard_normal(3 * C) * 0.1).astype(np.float32))
+    bp = bf16_round((rng.standard_normal(C) * 0.1).astype(np.float32))
+    dy = bf16_round(rng.standard_normal((B, T, C)).astype(np.float32))
+    layer = CausalSelfAttentionLayer(dev.cuda, H, C, T, True, True, half=half, training=True)
+    bx, top = Blob(dev.cuda, x.shape, half=half), Blob(dev.cuda, half=half)
+    bx.mutable_cpu_data = x
+    layer.Setup(bx, wa, ba, wp, bp)
+    layer.Forward(bx, top)
+    f = R.causal_self_attention(x, wa, ba, wp, bp, H, dtype=np.float64)
+    tol = BF16_RTOL if half else 2e-5
+    assert_close(top.mutable_cpu_data, f["y"], tol, "y")
+    top.mutable_cpu_diff = dy
+    layer.Backward(top, bx)
+    # the layer's gradients in float64
+    d = dy.astype(np.float64).reshape(B * T, C)
+    merged = f["work"].transpose(0, 2, 1, 3).reshape(B * T, C)
+    dwp, dbp = d.T @ merged, d.sum(0)
+    dwork = (d @ wp.astype(np.float64)).reshape(B, T, H, hs).transpose(0, 2, 1, 3)
+    dq, dk, dv = R.attn_backward(f["qt"], f["kt"], f["vt"], f["att"], dwork, np.float64)
+    dqkv = np.concatenate([g.transpose(0, 2, 1, 3).reshape(B * T, C) for g in (dq, dk, dv)], axis=1)
+    dwa, dba = dqkv.T @ x.astype(np.float64).reshape(B * T, C), dqkv.sum(0)
+    dx = (dqkv @ wa.astype(np.float64)).reshape(B, T, C)
+    assert_close(bx.mutable_cpu_diff, dx, tol, "grad x")
+    assert_close(layer.c_attn.blobs[0].mutable_cpu_diff, dwa, tol, "grad w_attn")
+    assert_close(layer.c_attn.blobs[1].mutable_cpu_diff, dba, tol, "grad b_attn")
+    assert_close(layer.c_proj.blobs[0].mutable_cpu_diff, dwp, tol, "grad w_proj")
+    assert_close(layer.c_proj.blobs[1].mutable_cpu_diff, dbp, tol, "grad b_proj")
+
+
 @pytest.mark.parametrize("sdpa", [True, False])
 @pytest.mark.parametrize("name,heads", [("gpt-pico-blk", 1), ("gpt-pico-blk3", 3), ("gpt-pico-blk3B", 3)])
 def test_transformer_block_backward_golden(dev, name, heads, sdpa):

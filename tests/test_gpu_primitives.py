@@ -370,6 +370,24 @@ def test_gemv_decode_shapes(dev, half):
         assert_close(dev.get(hx2), W.astype(np.float64).T @ dev.get(hy), FP32_RTOL, "gemv transposed")
 
 
+@pytest.mark.parametrize("tA", [False, True])
+def test_gemv_in_16_bit_storage(dev, tA):
+    """Matrix and both vectors in 16-bit storage (the bias gradient of an inner product kept that way); a 16-bit vector with
+    an fp32 matrix stays refused."""
+    m, n = 300, 136
+    rng = np.random.default_rng(9 + tA)
+    A = bf16_round(rng.standard_normal((m, n)).astype(np.float32))
+    x = bf16_round(rng.standard_normal(m if tA else n).astype(np.float32))
+    y0 = bf16_round(rng.standard_normal(n if tA else m).astype(np.float32))
+    hA, hx, hy = dev.put(A, True), dev.put(x, True), dev.put(y0, True)
+    dev.cuda.gemv(tA, m, n, 0.5, hA, hx, 1.0, hy)
+    want = 0.5 * ((A.T if tA else A).astype(np.float64) @ x) + y0
+    assert_close(dev.get(hy), want, BF16_RTOL, "gemv, 16-bit storage")
+    with pytest.raises(CudaDnnError) as e:
+        dev.cuda.gemv(tA, m, n, 1.0, dev.put(A), hx, 0.0, hy)
+    assert e.value.code == ERROR.MEMORY_HALF_TYPE_NOT_SUPPORTED
+
+
 def test_mask_inline_vectors(dev):
     x = np.array(INL["mask"]["x"], np.float32)
     n = x.size
