@@ -1066,16 +1066,31 @@ __global__ void qkv_split_heads_kernel(const T* __restrict__ tmp, size_t total, 
 }
 
 // X (m x kk) W^T (n x kk) through the tile kernels' HEADS epilogue `he`, or through `tmp` (m x n) and the splitting pass
+// whether a product with these operands goes through the scratch matrix (shapes and addresses the tile kernels do not take)
+static bool gemm_heads_through_tmp(DType dt, int kk, int rowUnit, const void* X, const void* W, const void* d0, const void* d1, const void* d2)
+{
+    const int vec = dt == F32 ? 4 : 8;
+    const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)d0 | (uintptr_t)d1 | (uintptr_t)d2) % 16 == 0) && rowUnit % vec == 0;
+    return !(aligned && kk % (dt == F32 ? 32 : 64) == 0);
+}
+bool k_gemm_bias_needs_tmp(DType dt, int n, int k, const void* X, const void* W, const void* Y)
+{
+    return gemm_heads_through_tmp(dt, k, n, X, W, Y, Y, Y);
+}
+bool k_gemm_qkv_heads_needs_tmp(DType dt, int H, int hs, const void* X, const void* W, const void* q, const void* k, const void* v)
+{
+    return gemm_heads_through_tmp(dt, H * hs, hs, X, W, q, k, v);
+}
+
 // (tiles256: the 256 x 256 tiles may be chosen as k_gemm chooses them)
 static hipError_t gemm_heads_dispatch(hipStream_t s, DType dt, int m, int n, int kk, const void* X, const void* W, const HeadsEpilogue& he,
                                       int rowUnit, void* tmp, bool tiles256)
 {
     const long long t256 = (long long)((m + 255) / 256) * ((n + 255) / 256);
     const bool full256 = tiles256 && (double)t256 / (double)(((t256 + 255) / 256) * 256) >= 0.85;
-    const int vec = dt == F32 ? 4 : 8;
-    const bool aligned = (((uintptr_t)X | (uintptr_t)W | (uintptr_t)he.dst[0] | (uintptr_t)he.dst[1] | (uintptr_t)he.dst[2]) % 16 == 0) && rowUnit % vec == 0;
+    const bool aligned = !gemm_heads_through_tmp(dt, kk, rowUnit, X, W, he.dst[0], he.dst[1], he.dst[2]);   // and K in whole stages
     const long long t128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-    if (aligned && dt == F32 && kk % 32 == 0) {
+    if (aligned && dt == F32) {
         hipError_t e;
         if (full256 && kk >= 1024) return launch_big<float, 4, 4, 1, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (launch_small_if_few<float, true>(&e, s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he)) return e;
@@ -1083,7 +1098,7 @@ static hipError_t gemm_heads_dispatch(hipStream_t s, DType dt, int m, int n, int
         if (short_last_round(t128) && launch_wide_if_fits<float, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;
         return launch_big<float, 2, 2, 2, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
     }
-    if (aligned && dt == BF16 && kk % 64 == 0) {
+    if (aligned && dt == BF16) {
         hipError_t e;
         if (full256 && kk >= 2048) return launch_big<bf16_t, 4, 4, 1, true>(s, m, n, kk, 1.f, X, W, 0.f, nullptr, &he);
         if (launch_wide_if_fits<bf16_t, true>(&e, s, m, n, kk, 1.f, X, W, nullptr, &he)) return e;

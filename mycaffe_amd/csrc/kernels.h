@@ -109,6 +109,9 @@ hipError_t k_gemm_qkv_heads(hipStream_t s, DType dt, int B, int T, int H, int hs
                             int ropeSeq = 0);
 // Y (m x n) = X (m x k) W^T + bias: product and bias in one launch; tmp: m x n scratch for shapes the tile kernels do not take
 hipError_t k_gemm_bias(hipStream_t s, DType dt, int m, int n, int k, const void* X, const void* W, const void* bias, void* Y, void* tmp);
+// whether these operands make k_gemm_bias / k_gemm_qkv_heads use their scratch matrix (tmp may be null otherwise)
+bool k_gemm_bias_needs_tmp(DType dt, int n, int k, const void* X, const void* W, const void* Y);
+bool k_gemm_qkv_heads_needs_tmp(DType dt, int H, int hs, const void* X, const void* W, const void* q, const void* k, const void* v);
 // column-major strided batched gemm with BLAS semantics (fp32)
 // C (fp32) = alpha X W^T + beta C on the bf16 matrix cores: W 16-bit (n x k), k % 64 == 0; A is X as bf16 (m x k) or,
 // split, every row of X as two bf16 rows (nearest bf16, then the bf16 nearest to the remainder; m x 2k)

@@ -1778,7 +1778,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             }
         }
         void* ws = nullptr;
-        ERRCHK(workspace((size_t)(M * 3 * C) * X->esize(), &ws));
+        if (k_gemm_qkv_heads_needs_tmp(X->dt(), (int)H, (int)hs, X->ptr, W->ptr, Q->ptr, K->ptr, V->ptr))
+            ERRCHK(workspace((size_t)(M * 3 * C) * X->esize(), &ws));
         HIPCHK(k_gemm_qkv_heads(s, X->dt(), (int)B, (int)T, (int)H, (int)hs, X->ptr, W->ptr, Bi ? Bi->ptr : nullptr, Q->ptr, K->ptr,
                                 V->ptr, ws, r ? (const float*)r->dcos.get() : nullptr, r ? (const float*)r->dsin.get() : nullptr,
                                 r ? r->seq : 0));
@@ -1804,7 +1805,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         if (Bi) RANGE(Bi, 0, N);
         RANGE(Y, 0, M * N);
         void* ws = nullptr;
-        ERRCHK(workspace((size_t)(M * N) * X->esize(), &ws));
+        if (k_gemm_bias_needs_tmp(X->dt(), (int)N, (int)K, X->ptr, W->ptr, Y->ptr)) ERRCHK(workspace((size_t)(M * N) * X->esize(), &ws));
         HIPCHK(k_gemm_bias(s, X->dt(), (int)M, (int)N, (int)K, X->ptr, W->ptr, Bi ? Bi->ptr : nullptr, Y->ptr, ws));
         m_mem.touch((long)pl[6]);
         return 0;
