@@ -125,6 +125,21 @@ static void csa_golden(CudaDnn& cuda, const std::string& dir, int heads)
     std::vector<float> out = cuda.GetMemoryFloat(hTop, (long long)M * C);
     const double err = max_rel_err(out, y.data);
     report(("causal self attention layer vs " + dir.substr(dir.find_last_of('/') + 1) + "/y.txt").c_str(), err <= 1e-4, err);
+    // the same forward as three calls (ids with no counterpart in the reference: fused QKV projection written head by
+    // head, attention output written merged, output projection with its bias), on an inference-mode handle
+    {
+        long hAttn2 = cuda.CreateAttn();
+        cuda.SetAttn(hCudnn, hAttn2, 0, false, B, T, heads, hs, 0.f);
+        for (long h : {hQt, hKt, hVt, hY, hTop}) cuda.set((long long)M * C, h, 0.f);
+        cuda.QkvProjHeads(B, T, heads, hs, hX, hWa, hBa, hQt, hKt, hVt);
+        cuda.AttnScaledDotProductForward(hCudnn, hAttn2, T, hQt, hKt, hVt, hMask, hY, 0, true);
+        cuda.LinearForward(M, C, C, hY, hWp, hBp, hTop);
+        const double e3 = max_rel_err(cuda.GetMemoryFloat(hTop, (long long)M * C), y.data);
+        report(("the layer as three calls vs " + dir.substr(dir.find_last_of('/') + 1) + "/y.txt").c_str(), e3 <= 1e-4, e3);
+        cuda.FreeAttn(hAttn2);
+        // the training-mode handle's forward state is what the gradient below uses: run it again
+        cuda.AttnScaledDotProductForward(hCudnn, hAttn, T, hQt, hKt, hVt, hMask, hWork, 0);
+    }
     // gradients of the attention core against the reference's dump of the same layer (iter_0): dY (B,H,T,hs) -> dQ, dK, dV
     {
         Tensor gy = load_txt(dir + "/iter_0/grad_y_pre_transpose.txt");

@@ -33,7 +33,7 @@ def test_cpp_host_parity_program(tmp_path):
     print(r.stdout)
     assert r.returncode == 0, r.stdout
     lines = r.stdout.splitlines()
-    assert sum(l.startswith("PASS") for l in lines) == 15 and not any(l.startswith("FAIL") for l in lines)
+    assert sum(l.startswith("PASS") for l in lines) == 19 and not any(l.startswith("FAIL") for l in lines)
     ids = [int(t) for t in next(l for l in lines if l.startswith("IDS")).split()[1:]]
     ref = O.Llama(cfg, blob, False).generate_greedy(np.array(prompt), n_steps)
     assert ids == list(ref)
