@@ -388,6 +388,25 @@ def test_gemv_in_16_bit_storage(dev, tA):
     assert e.value.code == ERROR.MEMORY_HALF_TYPE_NOT_SUPPORTED
 
 
+def test_timed_dispatch_over_argument_sets_takes_them_in_turn(dev):
+    """MCH_TimeInvokeFloatEx2Sets: dispatch i runs with the i-th list of long arguments (modulo the number of lists)."""
+    from mycaffe_amd.cudadnn import CUDAFN
+    n = 1000
+    src = dev.put(np.arange(n, dtype=np.float32))
+    dsts = [dev.zeros(n) for _ in range(3)]
+    sets = [[n, src, d, 0, 0, -1, -1, -1] for d in dsts]
+    ms = dev.cuda.TimeFunctionSets(CUDAFN.CUDA_COPY, None, sets, 0, 2)      # two dispatches: sets 0 and 1
+    assert ms > 0
+    assert np.array_equal(dev.get(dsts[0]), np.arange(n)) and np.array_equal(dev.get(dsts[1]), np.arange(n))
+    assert not dev.get(dsts[2]).any()
+    dev.cuda.TimeFunctionSets(CUDAFN.CUDA_COPY, None, sets, 1, 2)           # one warm-up and two timed: sets 0, 1, 2
+    assert np.array_equal(dev.get(dsts[2]), np.arange(n))
+    with pytest.raises(ValueError):
+        dev.cuda.TimeFunctionSets(CUDAFN.CUDA_COPY, None, [sets[0], sets[1][:5]], 0, 1)
+    # one list is the plain timing call
+    assert dev.cuda.TimeFunctionSets(CUDAFN.CUDA_COPY, None, sets[:1], 1, 3) > 0
+
+
 def test_mask_inline_vectors(dev):
     x = np.array(INL["mask"]["x"], np.float32)
     n = x.size
