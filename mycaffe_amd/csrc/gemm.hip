@@ -1282,6 +1282,10 @@ static bool gemm_turns_operands(DType dt, bool tA, bool tB, int m, int n, int k)
     const double turned = (tA ? (double)m * k : 0.0) + (!tB ? (double)n * k : 0.0);
     if (dt == BF16) return (double)m * n >= 64.0 * 64.0;
     // fp32: 136 against 88 TFLOP/s for the product, about 3 TB/s (read + write) for the pass over an operand
+    // Also where the strided kernel would split a long contraction over workgroups that add their parts with atomics
+    // (few tiles, K of 2048 and more): here the parts are summed in a fixed order, so a weight gradient comes out the
+    // same bits every run, at the same speed to within a few per cent.
+    if ((long long)((m + 127) / 128) * ((n + 127) / 128) < 256 && k >= 2048) return true;
     return (double)m * n * k * 8.0e-15 > 1.5 * turned * 8.0 / 3.0e12;
 }
 static size_t gemm_turned_bytes(DType dt, bool tA, bool tB, int m, int n, int k)

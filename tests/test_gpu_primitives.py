@@ -209,12 +209,10 @@ def test_gemm_long_contraction_split_over_workgroups(dev, half, tA, tB, m, n, k,
     dev.cuda.gemm(tA, tB, m, n, k, alpha, hA, hB, beta, hC)
     ref = R.gemm(tA, tB, m, n, k, alpha, A, B, beta, C0, dtype=np.float64)
     assert_close(dev.get(hC, (m, n)), ref, BF16_RTOL if half else FP32_RTOL, "gemm, split contraction")
-    # The same call again gives the same bits: the parts are summed in a fixed order.  (An fp32 product too small to pay
-    # for turning its operands stays on the strided kernel, which adds its parts with atomics.)
-    if half or not tA:
-        hC2 = dev.put(C0, half)
-        dev.cuda.gemm(tA, tB, m, n, k, alpha, hA, hB, beta, hC2)
-        assert np.array_equal(dev.get(hC2), dev.get(hC))
+    # the same call again gives the same bits: the parts are summed in a fixed order
+    hC2 = dev.put(C0, half)
+    dev.cuda.gemm(tA, tB, m, n, k, alpha, hA, hB, beta, hC2)
+    assert np.array_equal(dev.get(hC2), dev.get(hC))
 
 
 def test_gemm_offsets_and_bias_rank1_update(dev):
