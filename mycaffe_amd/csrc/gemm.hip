@@ -1561,6 +1561,142 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
         }
 }
 
+// The same product for a short contraction (K = KC of at most 128: Q K^T of the explicit attention chain, K = head size)
+// with A(i,k) i-fast and B(k,j) k-fast.  A tile of such a product is all prologue and epilogue for the kernel above: one
+// trip to memory for the operands, a few MFMAs, 64 KB of C to write.  Here a workgroup keeps its 128 rows of B (the j
+// panel) in registers as MFMA operands for its whole life and walks `tilesPerWg` tiles of 128 i: the next tile's slice of
+// A is requested before the current tile is multiplied, and the stores of one pair of 32 x 32 blocks drain under the
+// MFMAs of the next (the loads are older than the stores, so waiting for them does not wait for the stores).
+template <int KC>
+__global__ __launch_bounds__(256, 2) void gemm2_panel_f32_kernel(int M, int N, float alpha, const float* __restrict__ A,
+                                                              const float* __restrict__ B, float beta, float* __restrict__ C,
+                                                              GemmStrides st, int iChunks, int tilesPerWg)
+{
+    constexpr int LDI = 128 + 4, NP = KC * 128 / 4 / 256;       // [k][i] row stride; float4 per thread and tile of A
+    extern __shared__ __attribute__((aligned(16))) float panel_smem[];   // two stages of KC x LDI
+    A += (size_t)blockIdx.y * st.sA;
+    B += (size_t)blockIdx.y * st.sB;
+    C += (size_t)blockIdx.y * st.sC;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int jp = blockIdx.x / iChunks, ic = blockIdx.x % iChunks;
+    const int j0 = jp * 128, wj = (wave >> 1) * 64, wi = (wave & 1) * 64;
+    const int fr = lane & 31, fg = (lane >> 5) * 4;
+    const int t0 = ic * tilesPerWg, nT = (M + 127) / 128, t1 = min(nT, t0 + tilesPerWg);
+    if (t0 >= t1) return;
+
+    // B fragments: block a holds rows j0 + wj + 32 a + fr, this lane's four k of every eight
+    float4 qf[2][KC / 8];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const int j = j0 + wj + a * 32 + fr;
+        const float* bp = B + (size_t)min(j, N - 1) * st.bj + fg;
+#pragma unroll
+        for (int q = 0; q < KC / 8; q++) qf[a][q] = *(const float4*)(bp + 8 * q);
+    }
+    float4 ra[NP];
+    // whole: the tile lies inside the matrix (wavefront-uniform), so nothing is masked
+    auto gload = [&](int t, bool whole) {
+        const int i0 = t * 128;
+        if (whole) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int e = tid + p * 256, ig = e & 31, k = e >> 5;
+                ra[p] = *(const float4*)(A + (size_t)(i0 + 4 * ig) + (size_t)k * st.ak);
+            }
+            return;
+        }
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int e = tid + p * 256, ig = e & 31, k = e >> 5;
+            ra[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (i0 + 4 * ig < M) ra[p] = *(const float4*)(A + (size_t)(i0 + 4 * ig) + (size_t)k * st.ak);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int e = tid + p * 256, ig = e & 31, k = e >> 5;
+            *(float4*)(&panel_smem[buf * KC * LDI + k * LDI + 4 * ig]) = ra[p];
+        }
+    };
+    const bool jWhole = j0 + 128 <= N;
+    gload(t0, t0 * 128 + 128 <= M);
+    sstore(0);
+    __syncthreads();
+    for (int t = t0; t < t1; t++) {
+        const int buf = (t - t0) & 1;
+        if (t + 1 < t1) gload(t + 1, (t + 1) * 128 + 128 <= M);
+        const float* as = panel_smem + buf * KC * LDI;
+        const bool plain = jWhole && t * 128 + 128 <= M && beta == 0.f;   // wavefront-uniform
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            floatx16 acc[2];
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[a][v] = 0.f;
+#pragma unroll
+            for (int q = 0; q < KC / 8; q++) {
+                const float* ap = as + (8 * q + fg) * LDI + wi + b * 32 + fr;
+                const float fi[4] = {ap[0], ap[LDI], ap[2 * LDI], ap[3 * LDI]};
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(((const float*)&qf[a][q])[e], fi[e], acc[a], 0, 0, 0);
+            }
+            // accumulator register v of a block: j = 8 (v / 4) + 4 (lane / 32) + v % 4, i = lane % 32
+            const int i = t * 128 + wi + b * 32 + fr;
+            if (plain) {
+#pragma unroll
+                for (int a = 0; a < 2; a++) {
+                    float* cp = C + (size_t)i + (size_t)(j0 + wj + a * 32 + fg) * st.cj;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) cp[(size_t)((v >> 2) * 8 + (v & 3)) * st.cj] = alpha * acc[a][v];
+                }
+            } else if (i < M) {
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int j = j0 + wj + a * 32 + (v >> 2) * 8 + fg + (v & 3);
+                        if (j < N) {
+                            const size_t ci = (size_t)i + (size_t)j * st.cj;
+                            float o = alpha * acc[a][v];
+                            if (beta != 0.f) o += beta * C[ci];
+                            C[ci] = o;
+                        }
+                    }
+            }
+        }
+        if (t + 1 < t1) sstore(buf ^ 1);
+        // LDS only: a full __syncthreads() would also wait for this tile's stores of C
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+}
+
+template <int KC>
+static hipError_t launch_gemm2_panel(hipStream_t s, int M, int N, float alpha, const float* A, const float* B, float beta, float* C,
+                                     const GemmStrides& st, int batch)
+{
+    const int jPanels = (N + 127) / 128, nT = (M + 127) / 128;
+    // enough workgroups for two rounds of two per CU, as long as a workgroup keeps two tiles
+    int iChunks = 1;
+    while ((long long)jPanels * iChunks * batch < 1024 && nT / (2 * iChunks) >= 2) iChunks *= 2;
+    const int tilesPerWg = (nT + iChunks - 1) / iChunks;
+    constexpr int lds = 2 * KC * (128 + 4) * 4;
+    static bool attr = false;
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm2_panel_f32_kernel<KC>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    dim3 grid(jPanels * iChunks, batch);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gemm2_panel_f32_kernel<KC>, grid, 256, lds, s, M, N, alpha, A, B, beta, C, st, iChunks, tilesPerWg);
+    return hipGetLastError();
+}
+
 template <typename T> __global__ void gemm_prescale_kernel(T* c, size_t n, float beta)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)blockDim.x * gridDim.x)
@@ -1612,6 +1748,12 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
     const bool aOk = tA ? (k % 4 == 0) : (m % 4 == 0);
     const bool bOk = tB ? (n % 4 == 0) : (k % 4 == 0);
     if (aligned && aOk && bOk && k > 0 && (long long)m * n >= 1024) {
+        if (!tA && !tB && m >= 256 && n >= 128 && (long long)m * n * batch >= (1ll << 22)) {
+            // a short contraction over large matrices (Q K^T of the attention chain): the j panel stays in registers
+            if (k == 32) return launch_gemm2_panel<32>(s, m, n, alpha, A, B, beta, C, st, batch);
+            if (k == 64) return launch_gemm2_panel<64>(s, m, n, alpha, A, B, beta, C, st, batch);
+            if (k == 128) return launch_gemm2_panel<128>(s, m, n, alpha, A, B, beta, C, st, batch);
+        }
         if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
         if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
         if (tA && !tB) return launch_gemm2_mfma<false, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);

@@ -349,6 +349,26 @@ def test_matmul_attention_chain_shapes(dev):
     assert_close(dev.get(hy), att @ v, FP32_RTOL, "att @ v")
 
 
+@pytest.mark.parametrize("hs", [32, 64, 128])
+@pytest.mark.parametrize("Tq,Tk", [(512, 512), (300, 260), (129, 1028)])
+def test_matmul_scores_of_the_attention_chain_with_the_query_panel_in_registers(dev, hs, Tq, Tk):
+    """Q K^T of the explicit attention chain (CausalSelfAttentionLayer.cs:583-590: MatMul of q with the transposed keys)
+    at sizes that take the kernel built for short contractions: whole and ragged tiles, the three head sizes, then the
+    BLAS form of the same call with both scalars."""
+    rng = np.random.default_rng(hs + Tq)
+    outer = 64
+    q, kt = rng.standard_normal((outer, Tq, hs)).astype(np.float32), rng.standard_normal((outer, hs, Tk)).astype(np.float32)
+    hq, hkt, hatt = dev.put(q), dev.put(kt), dev.put(np.full(outer * Tq * Tk, 3.0, np.float32))
+    dev.cuda.matmul(outer, Tq, Tk, hs, hq, hkt, hatt)
+    want = q.astype(np.float64) @ kt.astype(np.float64)
+    assert_close(dev.get(hatt, want.shape), want, FP32_RTOL, "q @ k^T")
+    # C = alpha A B + beta C through id 219 itself (column-major: C^T = K^T-operand first)
+    c0 = rng.standard_normal((outer, Tq, Tk)).astype(np.float32)
+    hc = dev.put(c0)
+    dev.cuda._ex2(219, [0.5, -2.0], [0, 0, Tk, Tq, hs, 0, hkt, hq, 0, hc, Tk, hs, Tk, hs * Tk, Tq * hs, Tq * Tk, outer])
+    assert_close(dev.get(hc, want.shape), 0.5 * want - 2.0 * c0, FP32_RTOL, "gemm2 with both scalars")
+
+
 @pytest.mark.parametrize("half", [False, True])
 def test_gemv_decode_shapes(dev, half):
     rng = np.random.default_rng(5)
