@@ -783,7 +783,7 @@ hipError_t k_layernorm_bwd(hipStream_t s, DType dt, int rows, int inner, const v
 // multiples of the row length, so a row maps to one run of mask values).
 // causalT != 0: the mask is known to keep exactly the lower triangle of a (causalT, causalT) square and rows are causalT
 // long, so it is not read, and neither are the chunks of x that lie wholly above the diagonal.
-struct SoftmaxMask { const void* mask; size_t md1, dd1; float search, replace, xscale; int causalT; };
+struct SoftmaxMask { const void* mask; size_t md1, dd1; float search, replace, xscale; int causalT; int* zeroFlag; int epoch; };
 
 template <typename T, int R, bool MASKED>
 __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int len, const T* x, T* y, bool logsm, SoftmaxMask mk)
@@ -833,6 +833,9 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(size_t rows, int 
         }
     }
     mx = wave_max(mx);
+    // a later product over this row may skip the masked entries if every one of them comes out as an exact zero
+    if (MASKED && mk.causalT && mk.zeroFlag && lane == 0 && qrow + 1 < len && (logsm || expf(mk.replace - mx) != 0.f))
+        *mk.zeroFlag = mk.epoch;
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -876,19 +879,19 @@ static bool softmax_fwd_wave_launch_t(hipStream_t s, DType dt, const void* x, vo
 }
 static bool softmax_fwd_wave_launch(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm)
 {
-    return softmax_fwd_wave_launch_t<false>(s, dt, x, y, rows, len, logsm, SoftmaxMask());
+    return softmax_fwd_wave_launch_t<false>(s, dt, x, y, rows, len, logsm, SoftmaxMask{});
 }
 
 // Softmax over rows of `len` of a tensor whose mask call (with its folded-in scaling) has been held back: one pass
 // instead of two.  Returns hipErrorNotSupported when the shape does not fit the one-wavefront-per-row kernel or a row
 // would straddle a wrap of the mask; the caller then runs the mask call first.
 hipError_t k_softmax_masked(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, const void* mask,
-                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal)
+                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal, int* zeroFlag, int epoch)
 {
     if (rows == 0 || len <= 0) return hipSuccess;
     if (md1 == 0 || dd1 == 0 || md1 % (size_t)len != 0 || dd1 % (size_t)len != 0) return hipErrorNotSupported;
     if (causal && (md1 != (size_t)len * len || dd1 % md1 != 0)) return hipErrorInvalidValue;
-    SoftmaxMask mk{mask, md1, dd1, search, replace, xscale, causal ? len : 0};
+    SoftmaxMask mk{mask, md1, dd1, search, replace, xscale, causal ? len : 0, causal ? zeroFlag : nullptr, epoch};
     if (!softmax_fwd_wave_launch_t<true>(s, dt, x, y, rows, len, logsm, mk)) return hipErrorNotSupported;
     return hipGetLastError();
 }

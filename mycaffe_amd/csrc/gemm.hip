@@ -1414,8 +1414,22 @@ hipError_t k_gemm(hipStream_t s, DType dt, bool tA, bool tB, int m, int n, int k
 template <bool A_IFAST, bool B_KFAST, int TI, int TJ>
 __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K, float alpha, const float* __restrict__ A,
                                                              const float* __restrict__ B, float beta, float* __restrict__ C,
-                                                             GemmStrides st, int splits, int kChunk)
+                                                             GemmStrides st, int splits, int kChunk, const int* causalFlag, int epoch)
 {
+    // B(k,j) known to be zero for k > j (the probabilities of a causal softmax, unless the flag carries this launch's
+    // epoch): the contraction of this tile of columns stops at its last column
+    // Tiles of columns then differ in length.  Consecutive workgroups go to consecutive dies, and workgroup i shares its CU
+    // with i + 256, i + 512, ... (all are resident at once): the tile a workgroup takes is rotated by its batch index, so
+    // that no die is left with the long ones, and every other round of 256 takes them in reverse, so that a long tile
+    // meets a short one on its CU.
+    int jTile = blockIdx.y;
+    if (causalFlag) {
+        // (decided per batch index, so that the tiles of one batch entry are still each taken once)
+        const unsigned first = gridDim.x * gridDim.y * blockIdx.z;
+        jTile = (int)((blockIdx.y + blockIdx.z) % gridDim.y);
+        if ((first >> 8) & 1) jTile = (int)gridDim.y - 1 - jTile;
+    }
+    if (causalFlag && *causalFlag != epoch) K = min(K, (jTile + 1) * TJ);
     constexpr int BK = 16, LDK = BK + 4;
     constexpr int LDI = TI + 4, LDJ = TJ + 4;        // row strides of the [k][row] layouts
     constexpr int NI = TI / 64, NJ = TJ / 64;        // 32x32 blocks per wavefront along i and j
@@ -1431,7 +1445,7 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
     C += (size_t)batchIdx * st.sC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave & 1) * (TI / 2), wj = (wave >> 1) * (TJ / 2);
-    const int i0 = blockIdx.x * TI, j0 = blockIdx.y * TJ;
+    const int i0 = blockIdx.x * TI, j0 = jTile * TJ;
     const long long lda = A_IFAST ? st.ak : st.ai, ldb = B_KFAST ? st.bj : st.bk;
 
     floatx16 acc[NJ][NI];
@@ -1705,7 +1719,7 @@ template <typename T> __global__ void gemm_prescale_kernel(T* c, size_t n, float
 
 template <bool A_IFAST, bool B_KFAST>
 static hipError_t launch_gemm2_mfma(hipStream_t s, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
-                                    float* C, const GemmStrides& st, int batch)
+                                    float* C, const GemmStrides& st, int batch, const int* causalFlag = nullptr, int epoch = 0)
 {
     const bool si = M <= 64, sj = N <= 64;
     const int gi = (M + (si ? 63 : 127)) / (si ? 64 : 128), gj = (N + (sj ? 63 : 127)) / (sj ? 64 : 128);
@@ -1726,16 +1740,18 @@ static hipError_t launch_gemm2_mfma(hipStream_t s, int M, int N, int K, float al
     }
     dim3 grid(gi, gj, batch * splits);
     if (grid.y > 65535 || grid.z > 65535) return hipErrorInvalidValue;
-    if (si && sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
-    else if (si) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
-    else if (sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
-    else hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk);
+    if (si && sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk, splits > 1 ? nullptr : causalFlag, epoch);
+    else if (si) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 64, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk, splits > 1 ? nullptr : causalFlag, epoch);
+    else if (sj) hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 64>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk, splits > 1 ? nullptr : causalFlag, epoch);
+    else hipLaunchKernelGGL((gemm2_f32_mfma_kernel<A_IFAST, B_KFAST, 128, 128>), grid, 256, 0, s, M, N, K, alpha, A, B, beta, C, st, splits, kChunk, splits > 1 ? nullptr : causalFlag, epoch);
     return hipGetLastError();
 }
 
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
-                   float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch)
+                   float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch,
+                   const int* causalFlag, int epoch)
 {
+    if (causalFlag && (tA || tB || n != k)) return hipErrorInvalidValue;
     // column-major: op(A)(i,kk) = tA ? A[kk + i*lda] : A[i + kk*lda]
     GemmStrides st;
     st.ai = tA ? lda : 1;  st.ak = tA ? 1 : lda;
@@ -1754,7 +1770,7 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
             if (k == 64) return launch_gemm2_panel<64>(s, m, n, alpha, A, B, beta, C, st, batch);
             if (k == 128) return launch_gemm2_panel<128>(s, m, n, alpha, A, B, beta, C, st, batch);
         }
-        if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+        if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch, causalFlag, epoch);
         if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
         if (tA && !tB) return launch_gemm2_mfma<false, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
         return launch_gemm2_mfma<false, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);

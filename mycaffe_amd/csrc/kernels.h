@@ -57,8 +57,10 @@ hipError_t k_embed(hipStream_t s, DType wdt, size_t count, const float* ids, con
 hipError_t k_softmax(hipStream_t s, DType dt, const void* x, void* y, size_t outer, int len, int inner, bool logsm);
 // softmax of mask(x) in one pass (mask semantics of k_mask / k_mask_batch with md1 = maskDim / batch, dd1 = n / batch);
 // hipErrorNotSupported when the shape does not fit
+// zeroFlag (causal only): a row whose masked entries do not all come out as exact zeros writes `epoch` there
 hipError_t k_softmax_masked(hipStream_t s, DType dt, const void* x, void* y, size_t rows, int len, bool logsm, const void* mask,
-                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal = false);
+                            size_t md1, size_t dd1, float search, float replace, float xscale, bool causal = false,
+                            int* zeroFlag = nullptr, int epoch = 0);
 // gradient with respect to the softmax input from the output y and its gradient dy (dx may alias dy)
 hipError_t k_softmax_bwd(hipStream_t s, DType dt, const void* y, const void* dy, void* dx, size_t outer, int len, int inner, bool logsm);
 // adjacent-pair rotary embedding with the CudaDnnDLL index rule; x == y allowed
@@ -122,9 +124,11 @@ hipError_t k_gemm_bf16_swiglu(hipStream_t s, int m, int hid, int k, const void* 
 hipError_t k_gemm_bf16_qkv_rope(hipStream_t s, int B, int P, int H, int kvH, int hs, int k, const void* A, bool split, const void* Wqkv,
                                 void* q, void* kh, void* vh, bool heads16, void* kc, void* vc, bool cache16, int seqLen,
                                 const float* fcos, const float* fsin);
+// causalFlag != nullptr (no transposes, n == k): B(k,j) is known to be exactly zero for k > j unless *causalFlag == epoch,
+// and the contraction of a tile of columns stops at its last column
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
-                   int batch);
+                   int batch, const int* causalFlag = nullptr, int epoch = 0);
 // A row-major (m,n) of type adt; x, y fp32.  y = alpha*A*x + beta*y, or with tA y = alpha*A^T*x + beta*y
 hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x,
                   float beta, float* y);

@@ -218,6 +218,7 @@ Kernel::~Kernel()
     m_layernorm.clear();
     m_mem.free_all();
     if (m_ws) (void)hipFree(m_ws);
+    if (m_zeroFlag) (void)hipFree(m_zeroFlag);
     if (m_tickets) (void)hipFree(m_tickets);
     if (m_stage) (void)hipHostFree(m_stage);
     for (float* p : m_hostAllocs) (void)hipHostFree(p);
@@ -718,8 +719,16 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             C->pending = 1.f;
             if (m_pendingMask.hX == (long)pl[9]) m_pendingMask = PendingMask();
         }
+        // The second operand is the output of a softmax with a causal mask folded in (the P V product of the explicit
+        // attention chain): its entries above the diagonal are exact zeros - the softmax kernel raises a flag on the
+        // device if a row's are not - and the contraction stops at the diagonal.
+        const int* zeroFlag = nullptr;
+        if (m_zeroHandle && (long)pl[7] == m_zeroHandle && (long)pl[9] != m_zeroHandle && !tA && !tB && n == k && k == m_zeroLen &&
+            ldb == k && (batch == 1 || sB == (long long)k * n) && (unsigned long long)batch * n <= m_zeroRows &&
+            m_mem.version(m_zeroHandle) == m_zeroVersion && !B->view && !B->exposed)
+            zeroFlag = m_zeroFlag;
         HIPCHK(k_gemm2(s, tA, tB, m, n, k, pf[0], (const float*)A->ptr, (const float*)B->ptr, pf[1], (float*)C->ptr, lda,
-                       ldb, ldc, sA, sB, sC, batch));
+                       ldb, ldc, sA, sB, sC, batch, zeroFlag, m_zeroEpoch));
         m_mem.touch((long)pl[9]);
         return 0;
     }
@@ -1515,9 +1524,19 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 // a (len,len) lower-triangle mask with search == 0 is not read at all, and neither are the scores above the diagonal
                 const bool causal = p.batch == 0 && !X->half && p.search == 0.f && md1 == (size_t)len * len && dd1 % md1 == 0 &&
                                     held_mask_is_causal(p.hM, M, len);
-                hipError_t e = k_softmax_masked(s, X->dt(), X->ptr, Y->ptr, outer, len, alg == 2, M->ptr, md1, dd1, p.search, p.replace, p.xscale, causal);
+                // a causal pass over fp32 probabilities leaves word of whether every masked entry came out as an exact zero
+                const bool tag = causal && alg != 2 && !Y->view && !Y->exposed;
+                if (tag && !m_zeroFlag) {
+                    HIPCHK(hipMalloc((void**)&m_zeroFlag, sizeof(int)));
+                    HIPCHK(hipMemsetAsync(m_zeroFlag, 0, sizeof(int), s));
+                }
+                m_zeroHandle = 0;
+                if (tag) m_zeroEpoch = m_zeroEpoch == INT_MAX ? 1 : m_zeroEpoch + 1;
+                hipError_t e = k_softmax_masked(s, X->dt(), X->ptr, Y->ptr, outer, len, alg == 2, M->ptr, md1, dd1, p.search, p.replace, p.xscale, causal,
+                                                tag ? m_zeroFlag : nullptr, m_zeroEpoch);
                 if (e == hipSuccess) {
                     m_mem.touch((long)pl[6]);
+                    if (tag) { m_zeroHandle = (long)pl[6]; m_zeroVersion = m_mem.version((long)pl[6]); m_zeroLen = len; m_zeroRows = outer; }
                     return 0;
                 }
                 if (e != hipErrorNotSupported) return (long)e;

@@ -170,6 +170,10 @@ private:
     bool tril_scan(MemItem* mask, int T, bool* causal);
     bool held_mask_is_causal(long hMask, MemItem* mask, int T);
     long m_heldMaskHandle = 0; uint64_t m_heldMaskVersion = 0; int m_heldMaskT = 0; bool m_heldMaskCausal = false;
+    // the last output of a softmax with a causal mask folded in: (handle, content version) of the tensor, its row length
+    // and row count; m_zeroFlag (device) holds m_zeroEpoch if one of its rows has a masked entry that is not exactly zero
+    int* m_zeroFlag = nullptr; int m_zeroEpoch = 0;
+    long m_zeroHandle = 0; uint64_t m_zeroVersion = 0; int m_zeroLen = 0; size_t m_zeroRows = 0;
 
     int m_device = 0;
     hipStream_t m_stream = nullptr;

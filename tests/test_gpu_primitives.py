@@ -232,6 +232,50 @@ def test_gemm_offsets_and_bias_rank1_update(dev):
     assert_close(out[M // 2:], (x @ W.T)[M // 2:], FP32_RTOL, "gemm offsets")
 
 
+@pytest.mark.parametrize("replace", [-1e29, -3.0])
+def test_matmul_after_a_causal_softmax_stops_at_the_diagonal_only_when_the_masked_weights_are_zero(dev, replace):
+    """The explicit attention chain (CausalSelfAttentionLayer.cs:583-603): scale, mask, softmax, MatMul with v.  The softmax
+    pass that folds the causal mask in leaves word that the weights above the diagonal are exact zeros, and the MatMul
+    then stops each block of queries at its diagonal.  With a replacement value that leaves those weights non-zero
+    (-3), or after anything else has written to the weights, the whole contraction runs.  Either way against numpy."""
+    rng = np.random.default_rng(5)
+    cuda = dev.cuda
+    outer, T, hs = 6, 512, 64
+    n = outer * T * T
+    sc = rng.standard_normal((outer, T, T)).astype(np.float32) * 3
+    v = rng.standard_normal((outer, T, hs)).astype(np.float32)
+    tril = np.tril(np.ones((T, T), np.float32))
+    hm, hv = dev.put(tril), dev.put(v)
+    hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+    cuda.SetTensorDesc(d, outer * T, T, 1, 1, False)
+    masked = np.where(tril == 0, np.float64(replace), sc.astype(np.float64) * 0.125)
+    p = np.exp(masked - masked.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+
+    def weights():
+        h, hp = dev.put(sc), dev.zeros(n)
+        cuda.scal(n, 0.125, h)
+        cuda.mask(n, T * T, 0.0, replace, h, hm, h)
+        cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, h, 0.0, d, hp)
+        return hp
+
+    hp, hy = weights(), dev.zeros(outer * T * hs)
+    cuda.matmul(outer, T, hs, T, hp, hv, hy)
+    assert_close(dev.get(hy, v.shape), p @ v, FP32_RTOL, "weights @ v")
+    assert_close(dev.get(hp, p.shape), p, FP32_RTOL, "weights")
+    # the weights are written to before the MatMul (one of them above the diagonal set to one): the whole row counts
+    hp = weights()
+    cuda.set(1, hp, 1.0, 5 * T + 300)          # sequence 0, query 5, key 300
+    p2 = p.copy()
+    p2[0, 5, 300] = 1.0
+    cuda.matmul(outer, T, hs, T, hp, hv, hy)
+    assert_close(dev.get(hy, v.shape), p2 @ v, FP32_RTOL, "changed weights @ v")
+    # a product with other operands of the same shape is untouched by the record
+    hq = dev.put(rng.standard_normal((outer, T, T)).astype(np.float32))
+    cuda.matmul(outer, T, hs, T, hq, hv, hy)
+    assert_close(dev.get(hy, v.shape), dev.get(hq, p.shape).astype(np.float64) @ v, FP32_RTOL, "other weights @ v")
+
+
 @pytest.mark.parametrize("half", [False, True])
 @pytest.mark.parametrize("bias", [True, False])
 @pytest.mark.parametrize("m,n,k", [
