@@ -1584,7 +1584,7 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
 template <int KC>
 __global__ __launch_bounds__(256, 2) void gemm2_panel_f32_kernel(int M, int N, float alpha, const float* __restrict__ A,
                                                               const float* __restrict__ B, float beta, float* __restrict__ C,
-                                                              GemmStrides st, int iChunks, int tilesPerWg)
+                                                              GemmStrides st, int iChunks, int tilesPerWg, int causal)
 {
     constexpr int LDI = 128 + 4, NP = KC * 128 / 4 / 256;       // [k][i] row stride; float4 per thread and tile of A
     extern __shared__ __attribute__((aligned(16))) float panel_smem[];   // two stages of KC x LDI
@@ -1592,10 +1592,20 @@ __global__ __launch_bounds__(256, 2) void gemm2_panel_f32_kernel(int M, int N, f
     B += (size_t)blockIdx.y * st.sB;
     C += (size_t)blockIdx.y * st.sC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int jp = blockIdx.x / iChunks, ic = blockIdx.x % iChunks;
+    int jp = blockIdx.x / iChunks;
+    const int ic = blockIdx.x % iChunks;
+    if (causal) {
+        // One workgroup per j panel (iChunks == 1), which walks the tiles up to its diagonal: 1 to gridDim.x of them.
+        // Panels are rotated by the batch index and taken in reverse in every other round of 256 workgroups, so that
+        // neither a die (workgroup i goes to die i mod 8) nor a CU (i and i + 256 share one) collects the long ones.
+        jp = (int)((blockIdx.x + blockIdx.y) % gridDim.x);
+        if (((gridDim.x * blockIdx.y) >> 8) & 1) jp = (int)gridDim.x - 1 - jp;
+    }
     const int j0 = jp * 128, wj = (wave >> 1) * 64, wi = (wave & 1) * 64;
     const int fr = lane & 31, fg = (lane >> 5) * 4;
-    const int t0 = ic * tilesPerWg, nT = (M + 127) / 128, t1 = min(nT, t0 + tilesPerWg);
+    const int t0 = ic * tilesPerWg, nT = (M + 127) / 128;
+    int t1 = min(nT, t0 + tilesPerWg);
+    if (causal) t1 = min(t1, jp + 1);   // tile t holds i >= 128 t, the panel j <= 128 jp + 127
     if (t0 >= t1) return;
 
     // B fragments: block a holds rows j0 + wj + 32 a + fr, this lane's four k of every eight
@@ -1691,12 +1701,12 @@ __global__ __launch_bounds__(256, 2) void gemm2_panel_f32_kernel(int M, int N, f
 
 template <int KC>
 static hipError_t launch_gemm2_panel(hipStream_t s, int M, int N, float alpha, const float* A, const float* B, float beta, float* C,
-                                     const GemmStrides& st, int batch)
+                                     const GemmStrides& st, int batch, bool causal)
 {
     const int jPanels = (N + 127) / 128, nT = (M + 127) / 128;
     // enough workgroups for two rounds of two per CU, as long as a workgroup keeps two tiles
     int iChunks = 1;
-    while ((long long)jPanels * iChunks * batch < 1024 && nT / (2 * iChunks) >= 2) iChunks *= 2;
+    while (!causal && (long long)jPanels * iChunks * batch < 1024 && nT / (2 * iChunks) >= 2) iChunks *= 2;
     const int tilesPerWg = (nT + iChunks - 1) / iChunks;
     constexpr int lds = 2 * KC * (128 + 4) * 4;
     static bool attr = false;
@@ -1707,7 +1717,7 @@ static hipError_t launch_gemm2_panel(hipStream_t s, int M, int N, float alpha, c
     }
     dim3 grid(jPanels * iChunks, batch);
     if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(gemm2_panel_f32_kernel<KC>, grid, 256, lds, s, M, N, alpha, A, B, beta, C, st, iChunks, tilesPerWg);
+    hipLaunchKernelGGL(gemm2_panel_f32_kernel<KC>, grid, 256, lds, s, M, N, alpha, A, B, beta, C, st, iChunks, tilesPerWg, causal ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -1749,9 +1759,10 @@ static hipError_t launch_gemm2_mfma(hipStream_t s, int M, int N, int K, float al
 
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch,
-                   const int* causalFlag, int epoch)
+                   const int* causalFlag, int epoch, bool skipAboveDiagonal)
 {
     if (causalFlag && (tA || tB || n != k)) return hipErrorInvalidValue;
+    if (skipAboveDiagonal && (tA || tB || m != n || beta != 0.f)) return hipErrorInvalidValue;
     // column-major: op(A)(i,kk) = tA ? A[kk + i*lda] : A[i + kk*lda]
     GemmStrides st;
     st.ai = tA ? lda : 1;  st.ak = tA ? 1 : lda;
@@ -1766,9 +1777,9 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
     if (aligned && aOk && bOk && k > 0 && (long long)m * n >= 1024) {
         if (!tA && !tB && m >= 256 && n >= 128 && (long long)m * n * batch >= (1ll << 22)) {
             // a short contraction over large matrices (Q K^T of the attention chain): the j panel stays in registers
-            if (k == 32) return launch_gemm2_panel<32>(s, m, n, alpha, A, B, beta, C, st, batch);
-            if (k == 64) return launch_gemm2_panel<64>(s, m, n, alpha, A, B, beta, C, st, batch);
-            if (k == 128) return launch_gemm2_panel<128>(s, m, n, alpha, A, B, beta, C, st, batch);
+            if (k == 32) return launch_gemm2_panel<32>(s, m, n, alpha, A, B, beta, C, st, batch, skipAboveDiagonal);
+            if (k == 64) return launch_gemm2_panel<64>(s, m, n, alpha, A, B, beta, C, st, batch, skipAboveDiagonal);
+            if (k == 128) return launch_gemm2_panel<128>(s, m, n, alpha, A, B, beta, C, st, batch, skipAboveDiagonal);
         }
         if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch, causalFlag, epoch);
         if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);

@@ -128,7 +128,9 @@ hipError_t k_gemm_bf16_qkv_rope(hipStream_t s, int B, int P, int H, int kvH, int
 // and the contraction of a tile of columns stops at its last column
 hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float alpha, const float* A, const float* B,
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC,
-                   int batch, const int* causalFlag = nullptr, int epoch = 0);
+                   int batch, const int* causalFlag = nullptr, int epoch = 0, bool skipAboveDiagonal = false);
+// skipAboveDiagonal (no transposes, m == n, short contraction): entries C(i,j) of tiles that lie wholly at i > j need not
+// be computed (their memory is left as it is); other shapes ignore the request
 // A row-major (m,n) of type adt; x, y fp32.  y = alpha*A*x + beta*y, or with tA y = alpha*A^T*x + beta*y
 hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x,
                   float beta, float* y);

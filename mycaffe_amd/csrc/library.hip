@@ -319,8 +319,33 @@ long Kernel::free_host(float* p)
     return MCH_ERROR_MEMORY_NOT_FOUND;
 }
 
+// The held-back product, in full or (causal) up to the diagonal tiles.  Its operands were resolved when the call was
+// recorded; every later call that names one of them runs it first (mem / mem_lazy), so they still hold what the call saw.
+long Kernel::flush_pending_product(bool causal)
+{
+    const PendingProduct p = m_pendingProduct;
+    m_pendingProduct = PendingProduct();
+    if (!p.hC) return 0;
+    MemItem *A, *B, *C;
+    if (m_mem.get(p.hA, &A) || m_mem.get(p.hB, &B) || m_mem.get(p.hC, &C)) return 0;   // an operand is gone
+    HIPCHK(k_gemm2(m_stream, false, false, p.m, p.n, p.k, p.alpha, (const float*)A->ptr, (const float*)B->ptr, 0.f, (float*)C->ptr,
+                   p.lda, p.ldb, p.ldc, p.sA, p.sB, p.sC, p.batch, nullptr, 0, causal));
+    return 0;
+}
+
+long Kernel::mem_lazy(long h, MemItem** it)
+{
+    ERRCHK(m_mem.get(h, it));
+    if (m_pendingProduct.hC) {
+        const long hr = (*it)->view ? (*it)->base : h;
+        if (hr == m_pendingProduct.hA || hr == m_pendingProduct.hB) ERRCHK(flush_pending_product());
+    }
+    return 0;
+}
+
 long Kernel::flush_pending_mask()
 {
+    if (m_pendingProduct.hC && m_pendingProduct.hC == m_pendingMask.hX) ERRCHK(flush_pending_product());
     const PendingMask p = m_pendingMask;
     m_pendingMask = PendingMask();
     if (!p.hX) return 0;
@@ -347,6 +372,10 @@ long Kernel::mem(long h, MemItem** it)
 {
     ERRCHK(m_mem.get(h, it));
     MemItem* root = *it;
+    if (m_pendingProduct.hC) {
+        const long hr = root->view ? root->base : h;
+        if (hr == m_pendingProduct.hA || hr == m_pendingProduct.hB || hr == m_pendingProduct.hC) ERRCHK(flush_pending_product());
+    }
     if (m_pendingMask.hX) {
         const long hr = root->view ? root->base : h;
         if (hr == m_pendingMask.hX || hr == m_pendingMask.hM) ERRCHK(flush_pending_mask());
@@ -369,6 +398,12 @@ long Kernel::mask_operands(long hX, long hM, long hY, long long n, MemItem** X, 
     ERRCHK(mem(hM, M));
     MemItem* x;
     ERRCHK(mem_lazy(hX, &x));
+    if (m_pendingProduct.hC == hX && hX == hY && n > 0 && (size_t)n == x->count) {
+        // the result of a held-back product, masked in place as a whole: the caller either holds the mask back as well
+        // or runs the product first
+        *X = *Y = x;
+        return 0;
+    }
     if (!x->view && x->pending != 1.f && hX == hY && n > 0 && (size_t)n == x->count) {
         *xscale = x->pending;   // the caller clears `pending` once its kernel is launched
         *X = *Y = x;
@@ -532,6 +567,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
 
     case MCH_FN_FREEMEM:
         NEED_L(1, 1);
+        if (m_pendingProduct.hC == (long)pl[0]) m_pendingProduct = PendingProduct();   // the result goes: nothing to compute
+        else if (m_pendingProduct.hA == (long)pl[0] || m_pendingProduct.hB == (long)pl[0]) ERRCHK(flush_pending_product());
         if (m_pendingMask.hX == (long)pl[0]) m_pendingMask = PendingMask();       // the tensor goes: nothing to apply
         else if (m_pendingMask.hM == (long)pl[0]) ERRCHK(flush_pending_mask());   // the mask blob goes: apply it now
         HIPCHK(hipStreamSynchronize(s));
@@ -718,6 +755,21 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         if (overwrite) {
             C->pending = 1.f;
             if (m_pendingMask.hX == (long)pl[9]) m_pendingMask = PendingMask();
+            if (m_pendingProduct.hC == (long)pl[9]) m_pendingProduct = PendingProduct();
+            // Q K^T of the explicit attention chain (square result per batch entry, contraction = head size, everything
+            // contiguous): held back until the calls that follow show what is needed of it
+            if (!timing && !tA && !tB && m == n && m >= 256 && (k == 32 || k == 64 || k == 128) && lda == m && ldb == k &&
+                (batch == 1 || (sA == (long long)m * k && sB == (long long)n * k)) && (long long)m * n * batch >= (1ll << 22) &&
+                !A->view && !B->view && !A->exposed && !B->exposed && !C->exposed && C->views == 0 && (long)pl[6] != (long)pl[7] &&
+                (((uintptr_t)A->ptr | (uintptr_t)B->ptr) & 15) == 0) {
+                if (m_pendingProduct.hC) ERRCHK(flush_pending_product());   // one at a time
+                PendingProduct& pp = m_pendingProduct;
+                pp.hA = (long)pl[6]; pp.hB = (long)pl[7]; pp.hC = (long)pl[9];
+                pp.m = m; pp.n = n; pp.k = k; pp.lda = lda; pp.ldb = ldb; pp.ldc = ldc; pp.batch = batch;
+                pp.sA = sA; pp.sB = sB; pp.sC = sC; pp.alpha = pf[0];
+                m_mem.touch((long)pl[9]);
+                return 0;
+            }
         }
         // The second operand is the output of a softmax with a causal mask folded in (the P V product of the explicit
         // attention chain): its entries above the diagonal are exact zeros - the softmax kernel raises a flag on the
@@ -787,6 +839,11 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         NEED_L(3, 4);
         long long n = pl[0], xo = ll > 3 ? pl[3] : 0;
         MemItem* X;
+        if (m_pendingProduct.hC == (long)pl[2] && !timing && xo == 0 && !m_mem.get((long)pl[2], &X) && (size_t)n == X->count) {
+            m_pendingProduct.alpha *= pf[0];   // the scaling of a held-back product's whole result becomes its alpha
+            m_mem.touch((long)pl[2]);
+            return 0;
+        }
         ERRCHK(mem((long)pl[2], &X));
         RANGE(X, xo, n);
         if (!timing && !X->view && X->views == 0 && !X->exposed && xo == 0 && (size_t)n == X->count && n >= (1 << 20)) {
@@ -1146,6 +1203,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             m_mem.touch((long)pl[6]);
             return 0;
         }
+        if (m_pendingProduct.hC == (long)pl[4]) ERRCHK(flush_pending_product());
         HIPCHK(k_mask(s, X->dt(), (size_t)n, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
         if (xscale != 1.f) X->pending = 1.f;
         m_mem.touch((long)pl[6]);
@@ -1175,6 +1233,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             m_mem.touch((long)pl[7]);
             return 0;
         }
+        if (m_pendingProduct.hC == (long)pl[5]) ERRCHK(flush_pending_product());
         HIPCHK(k_mask_batch(s, X->dt(), (size_t)n, batch, md, pf[0], pf[1], X->ptr, M->ptr, Y->ptr, xscale));
         if (xscale != 1.f) X->pending = 1.f;
         m_mem.touch((long)pl[7]);
@@ -1524,6 +1583,11 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 // a (len,len) lower-triangle mask with search == 0 is not read at all, and neither are the scores above the diagonal
                 const bool causal = p.batch == 0 && !X->half && p.search == 0.f && md1 == (size_t)len * len && dd1 % md1 == 0 &&
                                     held_mask_is_causal(p.hM, M, len);
+                // the scores themselves may still be a held-back product: under the causal mask only the tiles that touch
+                // the lower triangle are computed (the pass below reads nothing else, and the mask call, whenever it is
+                // applied to the tensor, overwrites the rest)
+                if (m_pendingProduct.hC == (long)pl[3])
+                    ERRCHK(flush_pending_product(causal && m_pendingProduct.m == len && (long long)m_pendingProduct.batch * len == (long long)outer));
                 // a causal pass over fp32 probabilities leaves word of whether every masked entry came out as an exact zero
                 const bool tag = causal && alg != 2 && !Y->view && !Y->exposed;
                 if (tag && !m_zeroFlag) {

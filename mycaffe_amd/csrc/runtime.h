@@ -126,6 +126,15 @@ struct PendingMask {
     int md = 0, batch = 0;      // batch 0: plain mask (index i % md); else mask_batch
     float search = 0.f, replace = 0.f, xscale = 1.f;
 };
+// A GEMM2 call held back: the Q K^T product of the explicit attention chain, which the calls that follow scale, mask and
+// put through a softmax.  If the mask turns out to be the causal one, the tiles wholly above the diagonal are never
+// computed (the softmax does not read them and the mask call, whenever it is applied, overwrites them).
+struct PendingProduct {
+    long hA = 0, hB = 0, hC = 0;
+    int m = 0, n = 0, k = 0, lda = 0, ldb = 0, ldc = 0, batch = 0;
+    long long sA = 0, sB = 0, sC = 0;
+    float alpha = 1.f;
+};
 struct PermuteCacheEntry { uint64_t key[6]; int axes; PermuteArgs args; };
 struct ExtensionState {
     void* lib = nullptr;
@@ -160,7 +169,9 @@ private:
     long staging(size_t bytes, void** p);
     long tickets(size_t count, int** p);
     long mem(long h, MemItem** it);                                            // with any deferred scaling applied
-    long mem_lazy(long h, MemItem** it) { return m_mem.get(h, it); }           // as it is; the caller deals with `pending`
+    long mem_lazy(long h, MemItem** it);                                       // as it is; the caller deals with `pending`
+    PendingProduct m_pendingProduct;
+    long flush_pending_product(bool causal = false);
     long mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale);
     long flush_pending_mask();
     bool defer_mask(long hX, long hM, long hY, MemItem* X, MemItem* M, long long n, int md, int batch, float search, float replace,

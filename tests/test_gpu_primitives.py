@@ -232,6 +232,83 @@ def test_gemm_offsets_and_bias_rank1_update(dev):
     assert_close(out[M // 2:], (x @ W.T)[M // 2:], FP32_RTOL, "gemm offsets")
 
 
+def test_scores_product_is_held_back_without_changing_any_result(dev):
+    """Q K^T of the explicit attention chain (CausalSelfAttentionLayer.cs:583-603) waits for the calls that follow it: the
+    scaling becomes its alpha and, under a causal mask, the softmax pass has only the tiles that touch the lower triangle
+    computed.  Whatever reads or changes the scores, or an operand, in between sees what the immediate calls would have
+    left.  Every variant against numpy."""
+    rng = np.random.default_rng(8)
+    cuda = dev.cuda
+    outer, T, hs = 16, 512, 64
+    n = outer * T * T
+    q = rng.standard_normal((outer, T, hs)).astype(np.float32)
+    kt = rng.standard_normal((outer, hs, T)).astype(np.float32)
+    tril = np.tril(np.ones((T, T), np.float32))
+    hm = dev.put(tril)
+    hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+    cuda.SetTensorDesc(d, outer * T, T, 1, 1, False)
+    sc = q.astype(np.float64) @ kt.astype(np.float64)
+    masked = np.where(tril == 0, -1e29, sc * 0.125)
+    p = np.exp(masked - masked.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+
+    def chain(hq, hkt, hatt, mask=hm):
+        cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+        cuda.scal(n, 0.125, hatt)
+        cuda.mask(n, T * T, 0.0, -1e29, hatt, mask, hatt)
+
+    # the whole chain: probabilities, and afterwards the scores tensor itself (masked and scaled, also where no tile was computed)
+    hq, hkt, hatt, hp = dev.put(q), dev.put(kt), dev.put(np.full(n, 7.0, np.float32)), dev.zeros(n)
+    chain(hq, hkt, hatt)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hatt, 0.0, d, hp)
+    assert_close(dev.get(hp, p.shape), p, FP32_RTOL, "probabilities")
+    got = dev.get(hatt, sc.shape)
+    assert np.all(got[:, tril == 0] == np.float32(-1e29))
+    assert_close(got[:, tril == 1], (sc * 0.125)[:, tril == 1], FP32_RTOL, "masked, scaled scores")
+    # read right after the product, after the scaling, after the mask
+    hatt = dev.zeros(n)
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    assert_close(dev.get(hatt, sc.shape), sc, FP32_RTOL, "scores")
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    cuda.scal(n, 0.125, hatt)
+    assert_close(dev.get(hatt, sc.shape), sc * 0.125, FP32_RTOL, "scaled scores")
+    chain(hq, hkt, hatt)
+    assert_close(dev.get(hatt, sc.shape), np.where(tril == 0, -1e29, sc * 0.125), FP32_RTOL, "masked scores")
+    # an operand changes, or goes, while the product waits: the values of the moment of the call count
+    hq2 = dev.put(q)
+    cuda.matmul(outer, T, T, hs, hq2, hkt, hatt)
+    cuda.set(q.size, hq2, 0.0)
+    assert_close(dev.get(hatt, sc.shape), sc, FP32_RTOL, "scores after q was overwritten")
+    hq3 = dev.put(q)
+    chain(hq3, hkt, hatt)
+    cuda.FreeMemory(hq3)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hatt, 0.0, d, hp)
+    assert_close(dev.get(hp, p.shape), p, FP32_RTOL, "probabilities after q was freed")
+    # a mask that is not the causal one: the whole product
+    m2 = (rng.random((T, T)) > 0.3).astype(np.float32)
+    m2[:, 0] = 1
+    hm2 = dev.put(m2)
+    chain(hq, hkt, hatt, hm2)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hatt, 0.0, d, hp)
+    mk2 = np.where(m2 == 0, -1e29, sc * 0.125)
+    p2 = np.exp(mk2 - mk2.max(-1, keepdims=True))
+    p2 /= p2.sum(-1, keepdims=True)
+    assert_close(dev.get(hp, p.shape), p2, FP32_RTOL, "probabilities under another mask")
+    # softmax with no mask call in between
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    cuda.SoftmaxForward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hatt, 0.0, d, hp)
+    p3 = np.exp(sc - sc.max(-1, keepdims=True))
+    p3 /= p3.sum(-1, keepdims=True)
+    assert_close(dev.get(hp, p.shape), p3, FP32_RTOL, "probabilities without a mask")
+    # a second product into the same tensor replaces the first; the result freed while its product waits
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt, 2.0)
+    assert_close(dev.get(hatt, sc.shape), 2.0 * sc, FP32_RTOL, "second product")
+    cuda.matmul(outer, T, T, hs, hq, hkt, hatt)
+    cuda.FreeMemory(hatt)
+    assert_close(dev.get(hq, q.shape), q, 0.0, "q untouched")
+
+
 @pytest.mark.parametrize("replace", [-1e29, -3.0])
 def test_matmul_after_a_causal_softmax_stops_at_the_diagonal_only_when_the_masked_weights_are_zero(dev, replace):
     """The explicit attention chain (CausalSelfAttentionLayer.cs:583-603): scale, mask, softmax, MatMul with v.  The softmax
