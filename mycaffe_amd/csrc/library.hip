@@ -328,6 +328,10 @@ long Kernel::flush_pending_product(bool causal)
     if (!p.hC) return 0;
     MemItem *A, *B, *C;
     if (m_mem.get(p.hA, &A) || m_mem.get(p.hB, &B) || m_mem.get(p.hC, &C)) return 0;   // an operand is gone
+    if (p.kind == 1) {
+        HIPCHK(k_gemm(m_stream, F32, false, true, p.m, p.n, p.k, p.alpha, A->ptr, B->ptr, 0.f, C->ptr));
+        return 0;
+    }
     HIPCHK(k_gemm2(m_stream, false, false, p.m, p.n, p.k, p.alpha, (const float*)A->ptr, (const float*)B->ptr, 0.f, (float*)C->ptr,
                    p.lda, p.ldb, p.ldc, p.sA, p.sB, p.sC, p.batch, nullptr, 0, causal));
     return 0;
@@ -398,7 +402,7 @@ long Kernel::mask_operands(long hX, long hM, long hY, long long n, MemItem** X, 
     ERRCHK(mem(hM, M));
     MemItem* x;
     ERRCHK(mem_lazy(hX, &x));
-    if (m_pendingProduct.hC == hX && hX == hY && n > 0 && (size_t)n == x->count) {
+    if (m_pendingProduct.hC == hX && m_pendingProduct.kind == 0 && hX == hY && n > 0 && (size_t)n == x->count) {
         // the result of a held-back product, masked in place as a whole: the caller either holds the mask back as well
         // or runs the product first
         *X = *Y = x;
@@ -485,6 +489,35 @@ bool Kernel::tril_scan(MemItem* mask, int T, bool* causal)
     if (hipStreamSynchronize(m_stream) != hipSuccess) return false;
     *causal = (bad == 0);
     return true;
+}
+
+__global__ void check_ones_kernel(const float* v, int n, int* bad)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += blockDim.x * gridDim.x)
+        if (v[i] != 1.f) *bad = 1;
+}
+
+bool Kernel::vector_is_ones(long h, MemItem* v, int n)
+{
+    if (v->half || v->view || v->exposed || v->count < (size_t)n) return false;
+    const uint64_t ver = m_mem.version(h);
+    for (const OnesCacheEntry& e : m_onesCache)
+        if (e.handle == h && e.version == ver && e.n >= n && e.ones) return true;
+        else if (e.handle == h && e.version == ver && e.n <= n && !e.ones) return false;
+    void* ws;
+    if (workspace(256, &ws)) return false;
+    int* flag = (int*)ws;
+    if (hipMemsetAsync(flag, 0, sizeof(int), m_stream) != hipSuccess) return false;
+    int grid = (n + 255) / 256;
+    if (grid > 1024) grid = 1024;
+    hipLaunchKernelGGL(check_ones_kernel, grid, 256, 0, m_stream, (const float*)v->ptr, n, flag);
+    int bad = 1;
+    if (hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, m_stream) != hipSuccess) return false;
+    if (hipStreamSynchronize(m_stream) != hipSuccess) return false;
+    OnesCacheEntry& e = m_onesCache[m_onesNext];
+    m_onesNext = (m_onesNext + 1) % 16;
+    e.handle = h; e.version = ver; e.n = n; e.ones = (bad == 0);
+    return e.ones;
 }
 
 // the same question for the mask blob of a held-back mask call (no attention handle to keep the answer on): cached per
@@ -697,14 +730,59 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         int groups = ll > 13 ? (int)pl[13] : 1;
         long long gA = ll > 14 ? pl[14] : 0, gB = ll > 15 ? pl[15] : 0, gC = ll > 16 ? pl[16] : 0;
         if (m < 0 || n < 0 || k < 0 || groups < 1) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-        MemItem *A, *B, *C;
-        ERRCHK(mem((long)pl[6], &A));
-        ERRCHK(mem((long)pl[7], &B));
-        ERRCHK(mem((long)pl[9], &C));
-        if (A->half != B->half || A->half != C->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
         if (aOff < 0) aOff = 0;
         if (bOff < 0) bOff = 0;
         if (cOff < 0) cOff = 0;
+        MemItem *A, *B, *C;
+        const long hA = (long)pl[6], hB = (long)pl[7], hC = (long)pl[9];
+        // The bias of an inner product layer: ones (m) times bias (n) added to the held-back product X W^T.  Both run as one
+        // launch that adds the bias where the tile is stored.
+        if (m_pendingProduct.kind == 1 && m_pendingProduct.hC == hC && !tA && !tB && k == 1 && m == m_pendingProduct.m &&
+            n == m_pendingProduct.n && pf[0] == 1.f && pf[1] == 1.f && groups == 1 && aOff == 0 && bOff == 0 && cOff == 0 &&
+            hA != hC && hB != hC && hA != m_pendingProduct.hA && hA != m_pendingProduct.hB && hB != m_pendingProduct.hA &&
+            hB != m_pendingProduct.hB) {
+            ERRCHK(mem(hA, &A));
+            ERRCHK(mem(hB, &B));
+            if (m_pendingProduct.kind == 1 && m_pendingProduct.hC == hC && !A->half && !B->half && !B->view && B->count >= (size_t)n &&
+                vector_is_ones(hA, A, m)) {
+                const PendingProduct p = m_pendingProduct;
+                MemItem *X, *W;
+                if (!m_mem.get(p.hA, &X) && !m_mem.get(p.hB, &W) && !m_mem.get(p.hC, &C)) {
+                    m_pendingProduct = PendingProduct();
+                    void* ws = nullptr;
+                    if (k_gemm_bias_needs_tmp(F32, p.n, p.k, X->ptr, W->ptr, C->ptr)) ERRCHK(workspace((size_t)p.m * p.n * 4, &ws));
+                    HIPCHK(k_gemm_bias(s, F32, p.m, p.n, p.k, X->ptr, W->ptr, B->ptr, C->ptr, ws));
+                    m_mem.touch(hC);
+                    return 0;
+                }
+            }
+        }
+        ERRCHK(mem(hA, &A));
+        ERRCHK(mem(hB, &B));
+        // a product written over the whole of C leaves nothing of a held-back product into C to compute
+        bool whole = false;
+        if (hC != hA && hC != hB && pf[1] == 0.f && groups == 1 && cOff == 0 && !mem_lazy(hC, &C) && !C->view && C->views == 0 &&
+            (size_t)m * n == C->count && C->pending == 1.f && m_pendingMask.hX != hC && m_pendingMask.hM != hC)
+            whole = true;
+        else
+            ERRCHK(mem(hC, &C));
+        if (A->half != B->half || A->half != C->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
+        if (whole) {
+            RANGE(A, aOff, (long long)m * k);
+            RANGE(B, bOff, (long long)k * n);
+            if (m_pendingProduct.hC == hC) m_pendingProduct = PendingProduct();
+            // Y = X W^T of an inner product layer, large enough for the saved pass to matter and not one whose contraction
+            // the library would split over workgroups (that sum has another order than the fused launch's)
+            if (!timing && !tA && tB && !A->half && pf[0] == 1.f && aOff == 0 && bOff == 0 && m >= 256 && n >= 64 && k >= 32 &&
+                (long long)m * n >= (1ll << 20) && !A->view && !B->view && !A->exposed && !B->exposed && !C->exposed &&
+                k_gemm_workspace_bytes(F32, false, true, m, n, k) == 0) {
+                if (m_pendingProduct.hC) ERRCHK(flush_pending_product());   // one at a time
+                PendingProduct& pp = m_pendingProduct;
+                pp.kind = 1; pp.hA = hA; pp.hB = hB; pp.hC = hC; pp.m = m; pp.n = n; pp.k = k; pp.alpha = 1.f;
+                m_mem.touch(hC);
+                return 0;
+            }
+        }
         for (int g = 0; g < groups; g++) {
             long long ao = aOff + gA * g, bo = bOff + gB * g, co = cOff + gC * g;
             RANGE(A, ao, (long long)m * k);
@@ -839,8 +917,10 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         NEED_L(3, 4);
         long long n = pl[0], xo = ll > 3 ? pl[3] : 0;
         MemItem* X;
-        if (m_pendingProduct.hC == (long)pl[2] && !timing && xo == 0 && !m_mem.get((long)pl[2], &X) && (size_t)n == X->count) {
-            m_pendingProduct.alpha *= pf[0];   // the scaling of a held-back product's whole result becomes its alpha
+        if (m_pendingProduct.hC == (long)pl[2] && m_pendingProduct.kind == 0 && m_pendingProduct.alpha == 1.f && !timing && xo == 0 &&
+            !m_mem.get((long)pl[2], &X) && (size_t)n == X->count) {
+            // the scaling of a held-back product's whole result becomes its alpha (one rounding either way, alpha being 1)
+            m_pendingProduct.alpha = pf[0];
             m_mem.touch((long)pl[2]);
             return 0;
         }
@@ -1587,7 +1667,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 // the lower triangle are computed (the pass below reads nothing else, and the mask call, whenever it is
                 // applied to the tensor, overwrites the rest)
                 if (m_pendingProduct.hC == (long)pl[3])
-                    ERRCHK(flush_pending_product(causal && m_pendingProduct.m == len && (long long)m_pendingProduct.batch * len == (long long)outer));
+                    ERRCHK(flush_pending_product(causal && m_pendingProduct.kind == 0 && m_pendingProduct.m == len && (long long)m_pendingProduct.batch * len == (long long)outer));
                 // a causal pass over fp32 probabilities leaves word of whether every masked entry came out as an exact zero
                 const bool tag = causal && alg != 2 && !Y->view && !Y->exposed;
                 if (tag && !m_zeroFlag) {

@@ -129,12 +129,19 @@ struct PendingMask {
 // A GEMM2 call held back: the Q K^T product of the explicit attention chain, which the calls that follow scale, mask and
 // put through a softmax.  If the mask turns out to be the causal one, the tiles wholly above the diagonal are never
 // computed (the softmax does not read them and the mask call, whenever it is applied, overwrites them).
+//
+// kind 1 is a GEMM call held back the same way: the product of an inner product layer, Y = X W^T written over the whole of
+// Y in fp32.  When the next call on Y is the rank-1 update that adds the bias to every row (ones (m) times bias (n), alpha =
+// beta = 1), both run as one launch with the bias added where the tile is stored - the sum is rounded once either way, so
+// no result changes.  lda/ldb/ldc, the strides and batch are unused then.
 struct PendingProduct {
+    int kind = 0;
     long hA = 0, hB = 0, hC = 0;
     int m = 0, n = 0, k = 0, lda = 0, ldb = 0, ldc = 0, batch = 0;
     long long sA = 0, sB = 0, sC = 0;
     float alpha = 1.f;
 };
+struct OnesCacheEntry { long handle = 0; uint64_t version = 0; int n = 0; bool ones = false; };
 struct PermuteCacheEntry { uint64_t key[6]; int axes; PermuteArgs args; };
 struct ExtensionState {
     void* lib = nullptr;
@@ -180,6 +187,10 @@ private:
     bool mask_is_causal(AttnState* st, long hMask, MemItem* mask, int T);
     bool tril_scan(MemItem* mask, int T, bool* causal);
     bool held_mask_is_causal(long hMask, MemItem* mask, int T);
+    // whether the first n entries of an fp32 blob are all 1.0 (the bias multiplier of an inner product layer): one scan and
+    // host read-back per (handle, content version), a few blobs remembered
+    bool vector_is_ones(long h, MemItem* v, int n);
+    OnesCacheEntry m_onesCache[16]; int m_onesNext = 0;
     long m_heldMaskHandle = 0; uint64_t m_heldMaskVersion = 0; int m_heldMaskT = 0; bool m_heldMaskCausal = false;
     // the last output of a softmax with a causal mask folded in: (handle, content version) of the tensor, its row length
     // and row count; m_zeroFlag (device) holds m_zeroEpoch if one of its rows has a masked entry that is not exactly zero

@@ -309,6 +309,104 @@ def test_scores_product_is_held_back_without_changing_any_result(dev):
     assert_close(dev.get(hq, q.shape), q, 0.0, "q untouched")
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 768, 768), (1024, 1024, 96), (4096, 264, 40), (512, 2304, 8192)])
+def test_inner_product_and_its_bias_update_run_as_one_launch_without_changing_any_result(dev, M, N, K):
+    """The forward pass of an inner product layer (InnerProductLayer.cs:372-417) is two gemm calls: Y = X W^T, then the rank-1
+    update ones (M) x bias (N) added to Y.  The first waits for the second and both run as one launch; with Y read in
+    between, a multiplier that is not all ones, other factors, or an operand changed while the product waits, the calls
+    run as they are.  Every variant against numpy, and the fused result bit for bit against the two-launch one."""
+    rng = np.random.default_rng(M + N + K)
+    cuda = dev.cuda
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    hx, hw, hb, hy, hone = dev.put(x), dev.put(w), dev.put(b), dev.put(np.full(M * N, 3.0, np.float32)), dev.put(np.ones(M, np.float32))
+
+    def product(hy=hy, hx=hx):
+        cuda.gemm(False, True, M, N, K, 1.0, hx, hw, 0.0, hy)
+
+    def bias(hone=hone, alpha=1.0, beta=1.0, hy=hy):
+        cuda.gemm(False, False, M, N, 1, alpha, hone, hb, beta, hy)
+
+    # two launches: the result is read in between
+    product()
+    assert_close(dev.get(hy, ref.shape), ref, FP32_RTOL, "product")
+    bias()
+    two = dev.get(hy, ref.shape)
+    assert_close(two, ref + b, FP32_RTOL, "product + bias, two launches")
+    # one launch, twice over (the second time the multiplier is known to be ones)
+    for _ in range(2):
+        cuda.set(M * N, hy, 5.0)
+        product()
+        bias()
+        assert np.array_equal(dev.get(hy, ref.shape), two)
+    # the product alone, read later
+    product()
+    cuda.set(N, hb, 0.0)
+    assert_close(dev.get(hy, ref.shape), ref, FP32_RTOL, "product read after another blob was written")
+    cuda.SetMemory(hb, b)
+    # a multiplier that is not all ones, or becomes ones only later
+    m2 = np.ones(M, np.float32)
+    m2[M // 3] = 0.5
+    hm2 = dev.put(m2)
+    product()
+    bias(hm2)
+    assert_close(dev.get(hy, ref.shape), ref + np.outer(m2, b), FP32_RTOL, "multiplier with another entry")
+    cuda.SetMemory(hm2, np.ones(M, np.float32))
+    product()
+    bias(hm2)
+    assert np.array_equal(dev.get(hy, ref.shape), two)
+    cuda.SetMemory(hm2, m2)
+    product()
+    bias(hm2)
+    assert_close(dev.get(hy, ref.shape), ref + np.outer(m2, b), FP32_RTOL, "multiplier changed back")
+    # other factors on the update
+    product()
+    bias(alpha=2.0)
+    assert_close(dev.get(hy, ref.shape), ref + 2 * b, FP32_RTOL, "alpha 2")
+    product()
+    bias(beta=0.5)
+    assert_close(dev.get(hy, ref.shape), 0.5 * ref + b, FP32_RTOL, "beta 0.5")
+    # the input changes, or goes, while the product waits: the values of the moment of the call count
+    hx2 = dev.put(x)
+    product(hx=hx2)
+    cuda.set(M * K, hx2, 0.0)
+    bias()
+    assert_close(dev.get(hy, ref.shape), ref + b, FP32_RTOL, "input overwritten before the bias call")
+    hx3 = dev.put(x)
+    product(hx=hx3)
+    cuda.FreeMemory(hx3)
+    bias()
+    assert_close(dev.get(hy, ref.shape), ref + b, FP32_RTOL, "input freed before the bias call")
+    # the update on another tensor leaves the waiting product alone; a second product replaces the first
+    hy2 = dev.put(np.zeros(M * N, np.float32))
+    product()
+    bias(hy=hy2)
+    assert_close(dev.get(hy2, ref.shape), np.broadcast_to(b, ref.shape), FP32_RTOL, "update of another tensor")
+    assert_close(dev.get(hy, ref.shape), ref, FP32_RTOL, "product after an update elsewhere")
+    product()
+    product()
+    bias()
+    assert np.array_equal(dev.get(hy, ref.shape), two)
+    # the result is the input of the next product (two layers in a row, N == K only for the first shape)
+    if N == K:
+        product()
+        bias()
+        hy3 = dev.zeros(M * N)
+        product(hy=hy3, hx=hy)
+        bias(hy=hy3)
+        y1 = (ref + b).astype(np.float32).astype(np.float64)
+        assert_close(dev.get(hy3, ref.shape), y1 @ w.astype(np.float64).T + b, 5e-4, "second layer on the first one's result")
+    # the result freed while its product waits
+    hy4 = dev.zeros(M * N)
+    product(hy=hy4)
+    cuda.FreeMemory(hy4)
+    cuda.SynchronizeDevice()
+    for h in (hx, hw, hb, hy, hone, hm2, hx2, hy2):
+        cuda.FreeMemory(h)
+
+
 @pytest.mark.parametrize("replace", [-1e29, -3.0])
 def test_matmul_after_a_causal_softmax_stops_at_the_diagonal_only_when_the_masked_weights_are_zero(dev, replace):
     """The explicit attention chain (CausalSelfAttentionLayer.cs:583-603): scale, mask, softmax, MatMul with v.  The softmax
