@@ -555,6 +555,9 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         return set_out((float)m_device, ppOut, plOut);
 
     case MCH_FN_SYNCHRONIZEDEVICE:
+        // a held-back product runs now, so that a host that times a section between two of these calls sees all of its work
+        // (a held-back mask stays: after the softmax pass that applied it on the fly it may never be needed in memory)
+        if (m_pendingProduct.hC) ERRCHK(flush_pending_product());
         HIPCHK(hipStreamSynchronize(s));
         return 0;
 
