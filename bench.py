@@ -476,6 +476,10 @@ def bench_gemm(cuda, reps):
             else:
                 tf = fl / (ms / 1e3) / 1e12
                 out[tag] = {"ms": round(ms, 4), "TFLOPs": round(tf, 2), "frac_mfma": round(tf / MFMA_PEAK_TFLOPS[name], 4)}
+        # bias gradient db += dY^T ones (InnerProductLayer.cs:473-478): a transposed mat-vec over the M rows
+        ms = timed(cuda, CUDAFN.CUDA_GEMV, [1.0, 1.0], [1, M, N, 0, dy, ones, 0, bias, 0, 0, 0], 3, reps)
+        gbs = M * N * (2 if half else 4) / (ms / 1e3) / 1e9
+        out[name + "_qkv_bias_grad"] = {"ms": round(ms, 4), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
         for h in (x, w, dy, dx, dw, ones, bias):
             cuda.FreeMemory(h)
     return out

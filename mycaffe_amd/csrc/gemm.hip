@@ -1856,8 +1856,93 @@ __global__ void gemv_t_kernel(int m, int n, float alpha, const T* __restrict__ A
     y[j] = v;
 }
 
+// The transposed product over many rows (the bias gradient of an inner product layer: A = dY (rows x outputs), x = ones):
+// the rows are dealt over workgroups, each leaves one partial row of sums, and a second launch adds the partials in the
+// order of their rows - the same sum on every run.  A workgroup is 16 x 16 threads: 16 V columns (V = 4: 256 bytes of a
+// row), sixteen rows at a time.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void gemv_t_part_kernel(int m, int n, int rowsPer, const T* __restrict__ A,
+                                                          const float* __restrict__ x, float* __restrict__ part)
+{
+    __shared__ float red[16][16 * V + 1];
+    const int cl = threadIdx.x & 15, rl = threadIdx.x >> 4;
+    const int j = (blockIdx.x * 16 + cl) * V;
+    const int r0 = blockIdx.y * rowsPer, r1 = min(m, r0 + rowsPer);
+    float acc[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = 0.f;
+    if (j < n) {
+#pragma unroll 8
+        for (int i = r0 + rl; i < r1; i += 16) {
+            const float xi = x[i];
+            const T* a = A + (size_t)i * n + j;
+            if (V == 4) {
+                float av[4];
+                if (sizeof(T) == 4) {
+                    const float4 t = *(const float4*)a;
+                    av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w;
+                } else {
+                    const uint2 t = *(const uint2*)a;
+                    av[0] = __uint_as_float(t.x << 16); av[1] = __uint_as_float(t.x & 0xffff0000u);
+                    av[2] = __uint_as_float(t.y << 16); av[3] = __uint_as_float(t.y & 0xffff0000u);
+                }
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] = __builtin_fmaf(av[v], xi, acc[v]);
+            } else {
+                acc[0] = __builtin_fmaf(ldf(a, 0), xi, acc[0]);
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < V; v++) red[rl][cl * V + v] = acc[v];
+    __syncthreads();
+    if (threadIdx.x < 16 * V) {
+        const int jj = blockIdx.x * 16 * V + threadIdx.x;
+        if (jj < n) {
+            float t = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) t += red[r][threadIdx.x];
+            part[(size_t)blockIdx.y * n + jj] = t;
+        }
+    }
+}
+
+__global__ void gemv_t_sum_kernel(int n, int chunks, float alpha, const float* __restrict__ part, float beta, float* __restrict__ y)
+{
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int c = 0; c < chunks; c++) acc += part[(size_t)c * n + j];
+    float v = alpha * acc;
+    if (beta != 0.f) v += beta * y[j];
+    y[j] = v;
+}
+
+// how the rows of a transposed product are dealt: (columns per thread, rows per workgroup, workgroups along the rows)
+static inline int gemv_t_chunks(int m, int colBlocks)
+{
+    int c = std::max(1, std::min(64, 4096 / colBlocks));
+    return std::min(c, (m + 31) / 32);
+}
+static inline void gemv_t_split(DType adt, int m, int n, const void* A, int* V, int* rowsPer, int* chunks)
+{
+    const size_t es = adt == F32 ? 4 : 2;
+    *V = (n % 4 == 0 && ((uintptr_t)A % (4 * es)) == 0) ? 4 : 1;
+    const int c = gemv_t_chunks(m, (n + 16 * *V - 1) / (16 * *V));
+    *rowsPer = (m + c - 1) / c;
+    *chunks = (m + *rowsPer - 1) / *rowsPer;
+}
+
+size_t k_gemv_workspace_bytes(bool tA, int m, int n)
+{
+    if (!tA || m < 256 || n <= 0) return 0;
+    // whichever column count per thread the alignment allows
+    return (size_t)std::max(gemv_t_chunks(m, (n + 63) / 64), gemv_t_chunks(m, (n + 15) / 16)) * n * sizeof(float);
+}
+
 hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x, float beta,
-                  float* y)
+                  float* y, void* ws, size_t wsBytes)
 {
     if (m <= 0 || n <= 0) return hipSuccess;
     if (!tA) {
@@ -1866,6 +1951,20 @@ hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, 
             hipLaunchKernelGGL(gemv_n_kernel<float>, grid, 256, 0, s, m, n, alpha, (const float*)A, x, beta, y);
         else
             hipLaunchKernelGGL(gemv_n_kernel<bf16_t>, grid, 256, 0, s, m, n, alpha, (const bf16_t*)A, x, beta, y);
+    } else if (ws && m >= 256) {
+        int V, rowsPer, chunks;
+        gemv_t_split(adt, m, n, A, &V, &rowsPer, &chunks);
+        if (wsBytes < (size_t)chunks * n * sizeof(float)) return hipErrorInvalidValue;
+        float* part = (float*)ws;
+        const dim3 grid((n + 16 * V - 1) / (16 * V), chunks);
+        if (adt == F32) {
+            if (V == 4) hipLaunchKernelGGL((gemv_t_part_kernel<float, 4>), grid, 256, 0, s, m, n, rowsPer, (const float*)A, x, part);
+            else hipLaunchKernelGGL((gemv_t_part_kernel<float, 1>), grid, 256, 0, s, m, n, rowsPer, (const float*)A, x, part);
+        } else {
+            if (V == 4) hipLaunchKernelGGL((gemv_t_part_kernel<bf16_t, 4>), grid, 256, 0, s, m, n, rowsPer, (const bf16_t*)A, x, part);
+            else hipLaunchKernelGGL((gemv_t_part_kernel<bf16_t, 1>), grid, 256, 0, s, m, n, rowsPer, (const bf16_t*)A, x, part);
+        }
+        hipLaunchKernelGGL(gemv_t_sum_kernel, (n + 63) / 64, 64, 0, s, n, chunks, alpha, part, beta, y);
     } else {
         int grid = (n + 255) / 256;
         if (adt == F32)

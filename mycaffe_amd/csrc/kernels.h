@@ -132,8 +132,9 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
 // skipAboveDiagonal (no transposes, m == n, short contraction): entries C(i,j) of tiles that lie wholly at i > j need not
 // be computed (their memory is left as it is); other shapes ignore the request
 // A row-major (m,n) of type adt; x, y fp32.  y = alpha*A*x + beta*y, or with tA y = alpha*A^T*x + beta*y
+size_t k_gemv_workspace_bytes(bool tA, int m, int n);   // scratch for the partial sums of a transposed product over many rows
 hipError_t k_gemv(hipStream_t s, DType adt, bool tA, int m, int n, float alpha, const void* A, const float* x,
-                  float beta, float* y);
+                  float beta, float* y, void* ws = nullptr, size_t wsBytes = 0);
 
 // ---- attention (attn_prefill.hip, attn_decode.hip) --------------------------
 enum MaskKind { MASK_NONE = 0, MASK_QK = 1, MASK_KEY = 2, MASK_BQK = 3, MASK_CAUSAL = 4 };

@@ -393,6 +393,36 @@ long Kernel::mem(long h, MemItem** it)
     return 0;
 }
 
+static inline bool power_of_two(float f)
+{
+    int e;
+    return f > 0.f && std::isfinite(f) && frexpf(f, &e) == 0.5f && e > -100 && e < 100;
+}
+
+long Kernel::mem_factor(long h, MemItem** it, float* fold)
+{
+    ERRCHK(m_mem.get(h, it));
+    MemItem* r = *it;
+    if (r->view || r->pending == 1.f || !power_of_two(r->pending) || m_pendingMask.hX == h || m_pendingMask.hM == h ||
+        m_pendingProduct.hC == h)
+        return mem(h, it);
+    if (m_pendingProduct.hC && (h == m_pendingProduct.hA || h == m_pendingProduct.hB)) ERRCHK(flush_pending_product());
+    *fold *= r->pending;
+    return 0;
+}
+
+long Kernel::mem_overwritten(long h, MemItem** it, long long count)
+{
+    ERRCHK(m_mem.get(h, it));
+    MemItem* r = *it;
+    if (r->view || count < 0 || (size_t)count != r->count || m_pendingMask.hM == h) return mem(h, it);
+    if (m_pendingProduct.hC == h) m_pendingProduct = PendingProduct();
+    else if (m_pendingProduct.hA == h || m_pendingProduct.hB == h) ERRCHK(flush_pending_product());
+    if (m_pendingMask.hX == h) m_pendingMask = PendingMask();
+    r->pending = 1.f;
+    return 0;
+}
+
 // Operands of a mask call.  When X carries a deferred scaling and the call masks the whole tensor in place, the factor
 // is handed to the mask kernel (*xscale) instead of being applied in a pass of its own.
 long Kernel::mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale)
@@ -815,8 +845,15 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         if (m < 0 || n < 0 || k < 0 || batch < 1 || lda < 1 || ldb < 1 || ldc < 1 || sA < 0 || sB < 0 || sC < 0)
             return MCH_ERROR_PARAM_OUT_OF_RANGE;
         MemItem *A, *B, *C;
-        ERRCHK(mem((long)pl[6], &A));
-        ERRCHK(mem((long)pl[7], &B));
+        float fold = 1.f;   // deferred power-of-two scalings of the operands (MatMulGrad scales a gradient, then multiplies by it twice)
+        if (timing || (long)pl[9] == (long)pl[6] || (long)pl[9] == (long)pl[7]) {
+            ERRCHK(mem((long)pl[6], &A));
+            ERRCHK(mem((long)pl[7], &B));
+        } else {
+            ERRCHK(mem_factor((long)pl[6], &A, &fold));
+            ERRCHK(mem_factor((long)pl[7], &B, &fold));
+        }
+        const float alpha2 = pf[0] * fold;
         // When every element of C is overwritten, a held-back scaling or mask call on C has nothing left to act on and is
         // cancelled (once the arguments have passed their checks) instead of being run first.
         bool overwrite = false;
@@ -847,7 +884,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
                 PendingProduct& pp = m_pendingProduct;
                 pp.hA = (long)pl[6]; pp.hB = (long)pl[7]; pp.hC = (long)pl[9];
                 pp.m = m; pp.n = n; pp.k = k; pp.lda = lda; pp.ldb = ldb; pp.ldc = ldc; pp.batch = batch;
-                pp.sA = sA; pp.sB = sB; pp.sC = sC; pp.alpha = pf[0];
+                pp.sA = sA; pp.sB = sB; pp.sC = sC; pp.alpha = alpha2;
                 m_mem.touch((long)pl[9]);
                 return 0;
             }
@@ -860,7 +897,7 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             ldb == k && (batch == 1 || sB == (long long)k * n) && (unsigned long long)batch * n <= m_zeroRows &&
             m_mem.version(m_zeroHandle) == m_zeroVersion && !B->view && !B->exposed)
             zeroFlag = m_zeroFlag;
-        HIPCHK(k_gemm2(s, tA, tB, m, n, k, pf[0], (const float*)A->ptr, (const float*)B->ptr, pf[1], (float*)C->ptr, lda,
+        HIPCHK(k_gemm2(s, tA, tB, m, n, k, alpha2, (const float*)A->ptr, (const float*)B->ptr, pf[1], (float*)C->ptr, lda,
                        ldb, ldc, sA, sB, sC, batch, zeroFlag, m_zeroEpoch));
         m_mem.touch((long)pl[9]);
         return 0;
@@ -888,12 +925,25 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(A, aOff, (long long)m * n);
         RANGE(X, xOff, tA ? m : n);
         RANGE(Y, yOff, tA ? n : m);
+        void* ws = nullptr;
+        const size_t wsb = (k_gemv_workspace_bytes(tA, m, n) + 255) / 256 * 256;
         if (all16) {
-            HIPCHK(k_gemm(s, BF16, tA, false, tA ? n : m, 1, tA ? m : n, pf[0], PTR(A, aOff), PTR(X, xOff), pf[1], PTR(Y, yOff)));
+            // the vectors widened into scratch memory (a few KB), the matrix read as it is stored, the result rounded once
+            if (m == 0 || n == 0) return 0;
+            const size_t nx = tA ? m : n, ny = tA ? n : m;
+            const size_t xb = (nx * 4 + 255) / 256 * 256;
+            ERRCHK(workspace(wsb + xb + ny * 4, &ws));
+            float* xf = (float*)((char*)ws + wsb);
+            float* yf = (float*)((char*)ws + wsb + xb);
+            HIPCHK(k_convert(s, BF16, PTR(X, xOff), F32, xf, nx));
+            if (pf[1] != 0.f) HIPCHK(k_convert(s, BF16, PTR(Y, yOff), F32, yf, ny));
+            HIPCHK(k_gemv(s, BF16, tA, m, n, pf[0], PTR(A, aOff), xf, pf[1], yf, wsb ? ws : nullptr, wsb));
+            HIPCHK(k_convert(s, F32, yf, BF16, PTR(Y, yOff), ny));
             m_mem.touch((long)pl[7]);
             return 0;
         }
-        HIPCHK(k_gemv(s, A->dt(), tA, m, n, pf[0], PTR(A, aOff), (const float*)PTR(X, xOff), pf[1], (float*)PTR(Y, yOff)));
+        if (wsb) ERRCHK(workspace(wsb, &ws));
+        HIPCHK(k_gemv(s, A->dt(), tA, m, n, pf[0], PTR(A, aOff), (const float*)PTR(X, xOff), pf[1], (float*)PTR(Y, yOff), ws, wsb));
         m_mem.touch((long)pl[7]);
         return 0;
     }
@@ -1722,11 +1772,12 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
             }
         }
         MemItem *Y, *G, *X;
+        long long total = (long long)yd->n * yd->c * yd->h * yd->w;
         ERRCHK(mem((long)pl[3], &Y));
         ERRCHK(mem((long)pl[5], &G));
-        ERRCHK(mem((long)pl[8], &X));
+        if (pl[8] != pl[3] && pl[8] != pl[5]) ERRCHK(mem_overwritten((long)pl[8], &X, total));
+        else ERRCHK(mem((long)pl[8], &X));
         if (Y->half != G->half || Y->half != X->half) return MCH_ERROR_MEMORY_MIXED_HALF_TYPES;
-        long long total = (long long)yd->n * yd->c * yd->h * yd->w;
         RANGE(Y, 0, total);
         RANGE(G, 0, total);
         RANGE(X, 0, total);

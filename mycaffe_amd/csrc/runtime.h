@@ -177,6 +177,11 @@ private:
     long tickets(size_t count, int** p);
     long mem(long h, MemItem** it);                                            // with any deferred scaling applied
     long mem_lazy(long h, MemItem** it);                                       // as it is; the caller deals with `pending`
+    // an operand of a product: a deferred scaling by a power of two stays deferred and goes into *fold (the product's alpha
+    // takes it: every partial product and sum is the same number times that power, so no bit changes)
+    long mem_factor(long h, MemItem** it, float* fold);
+    // the target of a call that writes all `count` elements without reading any: what was held back for it is dropped
+    long mem_overwritten(long h, MemItem** it, long long count);
     PendingProduct m_pendingProduct;
     long flush_pending_product(bool causal = false);
     long mask_operands(long hX, long hM, long hY, long long n, MemItem** X, MemItem** M, MemItem** Y, float* xscale);

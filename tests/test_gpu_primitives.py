@@ -309,6 +309,59 @@ def test_scores_product_is_held_back_without_changing_any_result(dev):
     assert_close(dev.get(hq, q.shape), q, 0.0, "q untouched")
 
 
+@pytest.mark.parametrize("scale", [0.125, 0.3])
+def test_matmul_by_a_tensor_whose_scaling_is_held_back(dev, scale):
+    """Blob.MatMulGrad (Blob.cs:4304-4311) scales a gradient and multiplies by it twice.  The scaling of a large tensor
+    waits; a power of two then goes into the products' alpha and keeps waiting - every partial product and sum is the
+    same number times that power, so the products come out bit for bit as with the tensor scaled in memory - and any
+    other factor is applied before the first product.  Reading the tensor, or overwriting it through the softmax
+    gradient, afterwards shows the scaled values, or the new ones."""
+    from mycaffe_amd.cudadnn import SOFTMAX_ALGORITHM, SOFTMAX_MODE
+    rng = np.random.default_rng(3)
+    cuda = dev.cuda
+    outer, T, hs = 8, 512, 64
+    n = outer * T * T
+    assert n >= 1 << 20
+    g = rng.standard_normal((outer, T, T)).astype(np.float32)
+    kt = rng.standard_normal((outer, hs, T)).astype(np.float32)
+    q = rng.standard_normal((outer, T, hs)).astype(np.float32)
+
+    def products(hg, immediate):
+        hdq, hdkt = dev.zeros(outer * T * hs), dev.zeros(outer * T * hs)
+        cuda.scal(n, scale, hg)
+        if immediate:
+            dev.get(hg)          # a read in between: the scaling is applied in memory first
+        # dq = dS k (dS times kt transposed), dkt = q^T dS
+        cuda.matmul(outer, T, hs, T, hg, hkt_, hdq, 1.0, False, True)
+        cuda.matmul(outer, hs, T, T, hq_, hg, hdkt, 1.0, True, False)
+        return dev.get(hdq, (outer, T, hs)), dev.get(hdkt, (outer, hs, T))
+
+    hkt_, hq_ = dev.put(kt), dev.put(q)
+    a1, b1 = products(dev.put(g), True)
+    hg = dev.put(g)
+    a2, b2 = products(hg, False)
+    gs = g.astype(np.float64) * np.float32(scale)
+    assert_close(a1, gs @ kt.astype(np.float64).transpose(0, 2, 1), FP32_RTOL, "dS k")
+    assert_close(b1, q.astype(np.float64).transpose(0, 2, 1) @ gs, FP32_RTOL, "q^T dS")
+    if scale == 0.125:
+        assert np.array_equal(a1, a2) and np.array_equal(b1, b2)
+    else:
+        assert_close(a2, a1, FP32_RTOL, "dS k, factor applied first")
+        assert_close(b2, b1, FP32_RTOL, "q^T dS, factor applied first")
+    assert np.array_equal(dev.get(hg, g.shape), g * np.float32(scale))
+    # the scaled tensor overwritten by a softmax gradient: nothing of the old factor is left on it
+    cuda.scal(n, scale, hg)
+    y = rng.random((outer * T, T)).astype(np.float32)
+    y /= y.sum(-1, keepdims=True)
+    dy = rng.standard_normal((outer * T, T)).astype(np.float32)
+    hy, hdy = dev.put(y), dev.put(dy)
+    hc, d = cuda.CreateCuDNN(), cuda.CreateTensorDesc()
+    cuda.SetTensorDesc(d, outer * T, T, 1, 1, False)
+    cuda.SoftmaxBackward(hc, SOFTMAX_ALGORITHM.ACCURATE, SOFTMAX_MODE.INSTANCE, 1.0, d, hy, d, hdy, 0.0, d, hg)
+    want = y.astype(np.float64) * (dy - (y.astype(np.float64) * dy).sum(-1, keepdims=True))
+    assert_close(dev.get(hg, want.shape), want, FP32_RTOL, "softmax gradient over a tensor with a factor outstanding")
+
+
 @pytest.mark.parametrize("M,N,K", [(2048, 768, 768), (1024, 1024, 96), (4096, 264, 40), (512, 2304, 8192)])
 def test_inner_product_and_its_bias_update_run_as_one_launch_without_changing_any_result(dev, M, N, K):
     """The forward pass of an inner product layer (InnerProductLayer.cs:372-417) is two gemm calls: Y = X W^T, then the rank-1
@@ -605,6 +658,35 @@ def test_gemv_decode_shapes(dev, half):
         hx2 = dev.zeros(n)
         dev.cuda.gemv(True, d, n, 1.0, hW, hy, 0.0, hx2)
         assert_close(dev.get(hx2), W.astype(np.float64).T @ dev.get(hy), FP32_RTOL, "gemv transposed")
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("m,n", [(8192, 2304), (4096, 770), (1000, 52), (256, 4), (5000, 1)])
+def test_gemv_transposed_over_many_rows(dev, half, m, n):
+    """y = alpha A^T x + beta y with many rows (the bias gradient of an inner product layer, InnerProductLayer.cs:473-478:
+    A = the output gradient, x = ones): rows dealt over workgroups, partial sums added in a fixed order, so two runs give
+    the same bits.  Column counts that allow 16-byte loads and ones that do not; matrix in fp32 and in 16-bit storage."""
+    rng = np.random.default_rng(m + n)
+    A = rng.standard_normal((m, n)).astype(np.float32)
+    if half:
+        A = bf16_round(A)
+    x = rng.standard_normal(m).astype(np.float32)
+    y0 = rng.standard_normal(n).astype(np.float32)
+    hA, hx = dev.put(A, half), dev.put(x)
+    ref = A.astype(np.float64).T @ x
+    # sums of m products of N(0,1) numbers: compare on the scale of the sum's terms
+    tol = 2e-6 * np.sqrt(m) * 4
+    outs = []
+    for _ in range(2):
+        hy = dev.put(y0)
+        dev.cuda.gemv(True, m, n, 0.5, hA, hx, 2.0, hy)
+        got = dev.get(hy)
+        assert np.max(np.abs(got - (0.5 * ref + 2.0 * y0))) < tol * 0.5 + 1e-5
+        outs.append(got)
+    assert np.array_equal(outs[0], outs[1])
+    hy = dev.put(y0)
+    dev.cuda.gemv(True, m, n, 1.0, hA, dev.put(np.ones(m, np.float32)), 0.0, hy)
+    assert np.max(np.abs(dev.get(hy) - A.astype(np.float64).sum(0))) < tol
 
 
 @pytest.mark.parametrize("tA", [False, True])
