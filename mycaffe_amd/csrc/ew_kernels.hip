@@ -1187,10 +1187,44 @@ __global__ void channel_max_kernel(size_t rows, int channels, int spatial, const
         st(y, i, IDX ? (float)idx : val);
     }
 }
+// the same over a softmax axis that is the last one (spatial = 1, rows of `channels` consecutive values): one wavefront
+// a row, four rows per workgroup; among equal maxima the first index, as the loop above finds it
+template <typename T, bool IDX>
+__global__ __launch_bounds__(256) void channel_rowmax_kernel(size_t rows, int channels, const T* __restrict__ x, T* __restrict__ y)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * channels;
+    float val = -3.402823466e+38f;
+    int idx = 0;
+    for (int c = lane; c < channels; c += 64) {
+        const float v = ld(xr, c);
+        if (v > val) { val = v; idx = c; }
+    }
+    if (IDX) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(val, o, 64);
+            const int oi = __shfl_xor(idx, o, 64);
+            if (ov > val || (ov == val && oi < idx)) { val = ov; idx = oi; }
+        }
+    } else {
+        val = wave_max(val);
+    }
+    if (lane == 0) st(y, row, IDX ? (float)idx : val);
+}
+
 hipError_t k_channel_max(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, void* y, bool idx, bool across)
 {
     const size_t rows = num * spatial;
     if (rows == 0) return hipSuccess;
+    if (across && spatial == 1 && channels >= 64 && (rows + 3) / 4 <= 0x7fffffffu) {
+        const int g = (int)((rows + 3) / 4);
+        if (idx) DISPATCH_DT(dt, hipLaunchKernelGGL((channel_rowmax_kernel<T, true>), g, 256, 0, s, rows, channels, (const T*)x, (T*)y));
+        else DISPATCH_DT(dt, hipLaunchKernelGGL((channel_rowmax_kernel<T, false>), g, 256, 0, s, rows, channels, (const T*)x, (T*)y));
+        return hipGetLastError();
+    }
 #define CMAX(I, A) DISPATCH_DT(dt, hipLaunchKernelGGL((channel_max_kernel<T, I, A>), grid_for(rows), TPB, 0, s, rows, channels, spatial, (const T*)x, (T*)y))
     if (idx) { if (across) CMAX(true, true); else CMAX(true, false); }
     else { if (across) CMAX(false, true); else CMAX(false, false); }
@@ -1209,15 +1243,50 @@ __global__ void channel_bcast_kernel(size_t count, int channels, int spatial, co
         st(y, i, MODE == 0 ? ld(a, i) - r : ld(y, i) / r);
     }
 }
+// whole rows of `channels` consecutive values (spatial = 1): one wavefront a row, no division per element
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void channel_rowbcast_kernel(size_t rows, int channels, const T* __restrict__ a, const T* __restrict__ x, T* y)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float r = ld(x, row);
+    const T* ar = MODE == 0 ? a + row * channels : nullptr;
+    T* yr = y + row * channels;
+    if (sizeof(T) == 4 && channels % 4 == 0 && (((uintptr_t)y | (MODE == 0 ? (uintptr_t)a : 0)) & 15) == 0) {
+        for (int c = lane * 4; c < channels; c += 256) {
+            float4 v = *(const float4*)(MODE == 0 ? (const float*)ar + c : (const float*)yr + c);
+            if (MODE == 0) { v.x -= r; v.y -= r; v.z -= r; v.w -= r; }
+            else { v.x /= r; v.y /= r; v.z /= r; v.w /= r; }
+            *(float4*)((float*)yr + c) = v;
+        }
+        return;
+    }
+    for (int c = lane; c < channels; c += 64) st(yr, c, MODE == 0 ? ld(ar, c) - r : ld(yr, c) / r);
+}
+static inline bool channel_rows_whole(size_t count, int channels, int spatial)
+{
+    return spatial == 1 && channels >= 64 && count % channels == 0 && (count / channels + 3) / 4 <= 0x7fffffffu;
+}
 hipError_t k_channel_sub(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* a, const void* x, void* y)
 {
     if (count == 0) return hipSuccess;
+    if (channel_rows_whole(count, channels, spatial)) {
+        const size_t rows = count / channels;
+        DISPATCH_DT(dt, hipLaunchKernelGGL((channel_rowbcast_kernel<T, 0>), (int)((rows + 3) / 4), 256, 0, s, rows, channels, (const T*)a, (const T*)x, (T*)y));
+        return hipGetLastError();
+    }
     DISPATCH_DT(dt, hipLaunchKernelGGL((channel_bcast_kernel<T, 0>), grid_for(count), TPB, 0, s, count, channels, spatial, (const T*)a, (const T*)x, (T*)y));
     return hipGetLastError();
 }
 hipError_t k_channel_div(hipStream_t s, DType dt, size_t count, int channels, int spatial, const void* x, void* y)
 {
     if (count == 0) return hipSuccess;
+    if (channel_rows_whole(count, channels, spatial)) {
+        const size_t rows = count / channels;
+        DISPATCH_DT(dt, hipLaunchKernelGGL((channel_rowbcast_kernel<T, 1>), (int)((rows + 3) / 4), 256, 0, s, rows, channels, (const T*)nullptr, (const T*)x, (T*)y));
+        return hipGetLastError();
+    }
     DISPATCH_DT(dt, hipLaunchKernelGGL((channel_bcast_kernel<T, 1>), grid_for(count), TPB, 0, s, count, channels, spatial, (const T*)nullptr, (const T*)x, (T*)y));
     return hipGetLastError();
 }
@@ -1240,10 +1309,28 @@ __global__ void channel_dot_kernel(size_t rows, int channels, int spatial, const
         st(y, i, v0 + v1);
     }
 }
+// rows of `channels` consecutive values (spatial = 1): one wavefront a row
+template <typename T>
+__global__ __launch_bounds__(256) void channel_rowdot_kernel(size_t rows, int channels, const T* __restrict__ x, const T* __restrict__ a, T* __restrict__ y)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * channels;
+    const T* ar = a + row * channels;
+    float acc = 0.f;
+    for (int c = lane; c < channels; c += 64) acc += ld(xr, c) * ld(ar, c);
+    acc = wave_sum(acc);
+    if (lane == 0) st(y, row, acc);
+}
 hipError_t k_channel_dot(hipStream_t s, DType dt, size_t num, int channels, int spatial, const void* x, const void* a, void* y)
 {
     const size_t rows = num * spatial;
     if (rows == 0) return hipSuccess;
+    if (spatial == 1 && channels >= 64 && (rows + 3) / 4 <= 0x7fffffffu) {
+        DISPATCH_DT(dt, hipLaunchKernelGGL(channel_rowdot_kernel<T>, (int)((rows + 3) / 4), 256, 0, s, rows, channels, (const T*)x, (const T*)a, (T*)y));
+        return hipGetLastError();
+    }
     DISPATCH_DT(dt, hipLaunchKernelGGL(channel_dot_kernel<T>, grid_for(rows), TPB, 0, s, rows, channels, spatial, (const T*)x, (const T*)a, (T*)y));
     return hipGetLastError();
 }

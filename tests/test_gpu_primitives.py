@@ -1213,10 +1213,15 @@ def test_in_place_mask_is_held_back_for_the_softmax_without_changing_any_result(
 # ---- CAFFE-engine softmax chain: exp, log, channel_max / sub / div / dot ----------------------
 
 @pytest.mark.parametrize("half", [False, True])
-def test_channel_primitives_of_the_softmax_chain(dev, half):
+@pytest.mark.parametrize("num,ch,sp", [(5, 37, 19), (33, 200, 1), (7, 1024, 1), (9, 67, 1)])
+def test_channel_primitives_of_the_softmax_chain(dev, half, num, ch, sp):
+    """Channel axis in the middle, and as the last axis (spatial = 1: rows of consecutive values, which take the
+    one-wavefront-a-row kernels from 64 channels on), with ties for the index of the maximum."""
     rng = np.random.default_rng(3)
-    num, ch, sp = 5, 37, 19
     x = bf16_round(rng.standard_normal((num, ch, sp)).astype(np.float32))
+    x[0, ch // 3] = x[0, ch - 1] = x[0].max(0) + 1        # equal maxima: the first index counts
+    x[1, 0] = x[1, ch // 2] = x[1].max(0) + 1
+    x = bf16_round(x)
     a = bf16_round(rng.standard_normal((num, ch, sp)).astype(np.float32))
     r = bf16_round((rng.random((num, sp)) + 0.5).astype(np.float32))
     tol = BF16_RTOL if half else 1e-6
@@ -1226,7 +1231,8 @@ def test_channel_primitives_of_the_softmax_chain(dev, half):
     dev.cuda.channel_max(n, num, ch, sp, hx, hy)
     assert np.array_equal(dev.get(hy), R.channel_max(x, num, ch, sp))
     dev.cuda.channel_max(n, num, ch, sp, hx, hy, True)
-    assert np.array_equal(dev.get(hy), R.channel_max(x, num, ch, sp, return_idx=True))
+    want_idx = R.channel_max(x, num, ch, sp, return_idx=True)
+    assert np.array_equal(dev.get(hy), bf16_round(want_idx) if half else want_idx)     # the index is stored as a number
     dev.cuda.channel_max(n, num, 1, sp, hx, hy, False, False)                      # within-channel index rule
     assert np.array_equal(dev.get(hy), R.channel_max(x, num, 1, sp, across=False))
     dev.cuda.channel_sub(full, num, ch, sp, hr, hfull, ha)
@@ -1249,8 +1255,15 @@ def test_channel_primitives_of_the_softmax_chain(dev, half):
     with pytest.raises(CudaDnnError) as ei:
         dev.cuda.channel_div(n - sp, num, ch, sp, hr, hfull, 2)
     assert ei.value.code == ERROR.PARAM_OUT_OF_RANGE
+    dev.cuda.copy(full, hx, hfull)
+    part = (num - 1) * ch * sp - 3                       # not a whole number of rows
+    dev.cuda.channel_sub(part, num, ch, sp, hr, hfull)
+    want = R.channel_sub(x, r, num, ch, sp).reshape(-1).copy()
+    want[part:] = x.reshape(-1)[part:]
+    assert_close(dev.get(hfull), want, tol, "channel_sub in place, partial count")
     dev.cuda.channel_dot(n, num, ch, sp, hx, ha, hy)
-    assert_close(dev.get(hy), R.channel_dot(x, a, num, ch, sp), BF16_RTOL if half else 1e-5, "channel_dot")
+    ref_dot = R.channel_dot(x, a, num, ch, sp)
+    assert np.max(np.abs(dev.get(hy).reshape(ref_dot.shape) - ref_dot)) < (2e-2 if half else 1e-5) * np.sqrt(ch)
     dev.cuda.exp(full, hx, hfull, 0, 0, 0.5)
     assert_close(dev.get(hfull), np.exp(0.5 * x.astype(np.float64)).reshape(-1), tol, "exp")
     dev.cuda.log(n, hr, hy, 2.0, 0.25)
