@@ -1429,7 +1429,10 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
         jTile = (int)((blockIdx.y + blockIdx.z) % gridDim.y);
         if ((first >> 8) & 1) jTile = (int)gridDim.y - 1 - jTile;
     }
-    if (causalFlag && *causalFlag != epoch) K = min(K, (jTile + 1) * TJ);
+    // (B given transposed, B(k,j) stored as [k][j]: the same tensor read the other way, zero for k < j - the product with the
+    // transposed probabilities in the backward pass - and the contraction begins at the tile's first column instead)
+    const bool causal = causalFlag && *causalFlag != epoch;
+    if (causal && B_KFAST) K = min(K, (jTile + 1) * TJ);
     constexpr int BK = 16, LDK = BK + 4;
     constexpr int LDI = TI + 4, LDJ = TJ + 4;        // row strides of the [k][row] layouts
     constexpr int NI = TI / 64, NJ = TJ / 64;        // 32x32 blocks per wavefront along i and j
@@ -1438,7 +1441,7 @@ __global__ __launch_bounds__(256) void gemm2_f32_mfma_kernel(int M, int N, int K
     // blockIdx.z = batch * splits + split; with splits > 1 every workgroup covers kChunk of the contraction and adds its
     // part to C with float atomics (C holds beta * C already)
     const int batchIdx = blockIdx.z / splits, split = blockIdx.z % splits;
-    const int kBegin = split * kChunk;
+    const int kBegin = (causal && !B_KFAST) ? min(K, jTile * TJ) : split * kChunk;
     if (splits > 1) K = min(K, kBegin + kChunk);
     A += (size_t)batchIdx * st.sA;
     B += (size_t)batchIdx * st.sB;
@@ -1761,7 +1764,7 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
                    float beta, float* C, int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch,
                    const int* causalFlag, int epoch, bool skipAboveDiagonal)
 {
-    if (causalFlag && (tA || tB || n != k)) return hipErrorInvalidValue;
+    if (causalFlag && (tA || n != k)) return hipErrorInvalidValue;
     if (skipAboveDiagonal && (tA || tB || m != n || beta != 0.f)) return hipErrorInvalidValue;
     // column-major: op(A)(i,kk) = tA ? A[kk + i*lda] : A[i + kk*lda]
     GemmStrides st;
@@ -1782,7 +1785,7 @@ hipError_t k_gemm2(hipStream_t s, bool tA, bool tB, int m, int n, int k, float a
             if (k == 128) return launch_gemm2_panel<128>(s, m, n, alpha, A, B, beta, C, st, batch, skipAboveDiagonal);
         }
         if (!tA && !tB) return launch_gemm2_mfma<true, true>(s, m, n, k, alpha, A, B, beta, C, st, batch, causalFlag, epoch);
-        if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
+        if (!tA && tB) return launch_gemm2_mfma<true, false>(s, m, n, k, alpha, A, B, beta, C, st, batch, causalFlag, epoch);
         if (tA && !tB) return launch_gemm2_mfma<false, true>(s, m, n, k, alpha, A, B, beta, C, st, batch);
         return launch_gemm2_mfma<false, false>(s, m, n, k, alpha, A, B, beta, C, st, batch);
     }

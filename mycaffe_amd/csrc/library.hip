@@ -893,7 +893,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         // attention chain): its entries above the diagonal are exact zeros - the softmax kernel raises a flag on the
         // device if a row's are not - and the contraction stops at the diagonal.
         const int* zeroFlag = nullptr;
-        if (m_zeroHandle && (long)pl[7] == m_zeroHandle && (long)pl[9] != m_zeroHandle && !tA && !tB && n == k && k == m_zeroLen &&
+        // (given transposed - the product P^T dY of the backward pass - the same zeros let it begin at the diagonal)
+        if (m_zeroHandle && (long)pl[7] == m_zeroHandle && (long)pl[9] != m_zeroHandle && !tA && n == k && k == m_zeroLen &&
             ldb == k && (batch == 1 || sB == (long long)k * n) && (unsigned long long)batch * n <= m_zeroRows &&
             m_mem.version(m_zeroHandle) == m_zeroVersion && !B->view && !B->exposed)
             zeroFlag = m_zeroFlag;

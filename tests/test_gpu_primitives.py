@@ -502,6 +502,16 @@ def test_matmul_after_a_causal_softmax_stops_at_the_diagonal_only_when_the_maske
     hq = dev.put(rng.standard_normal((outer, T, T)).astype(np.float32))
     cuda.matmul(outer, T, hs, T, hq, hv, hy)
     assert_close(dev.get(hy, v.shape), dev.get(hq, p.shape).astype(np.float64) @ v, FP32_RTOL, "other weights @ v")
+    # the backward pass multiplies by the transposed weights (Blob.MatMulGrad, Blob.cs:4304-4311: v' = weights^T y'): that
+    # contraction, over the queries, begins at the diagonal; with an entry above the diagonal written, the whole column counts
+    hp = weights()
+    cuda.matmul(outer, T, hs, T, hp, hv, hy, 1.0, True, False)
+    assert_close(dev.get(hy, v.shape), p.transpose(0, 2, 1) @ v, FP32_RTOL, "weights^T @ y'")
+    cuda.set(1, hp, 1.0, 5 * T + 300)
+    cuda.matmul(outer, T, hs, T, hp, hv, hy, 1.0, True, False)
+    assert_close(dev.get(hy, v.shape), p2.transpose(0, 2, 1) @ v, FP32_RTOL, "changed weights^T @ y'")
+    cuda.matmul(outer, T, hs, T, hq, hv, hy, 1.0, True, False)
+    assert_close(dev.get(hy, v.shape), dev.get(hq, p.shape).astype(np.float64).transpose(0, 2, 1) @ v, FP32_RTOL, "other weights^T @ y'")
 
 
 @pytest.mark.parametrize("half", [False, True])
