@@ -1877,7 +1877,7 @@ __global__ __launch_bounds__(256) void gemv_t_part_kernel(int m, int n, int rows
     if (j < n) {
 #pragma unroll 8
         for (int i = r0 + rl; i < r1; i += 16) {
-            const float xi = x[i];
+            const float xi = x ? x[i] : 1.f;   // no vector: the plain sum of every column
             const T* a = A + (size_t)i * n + j;
             if (V == 4) {
                 float av[4];

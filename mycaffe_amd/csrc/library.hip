@@ -1268,7 +1268,14 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         RANGE(Y, 0, reduced);
         if (dir == 0) {
             if (X->ptr == Y->ptr) return MCH_ERROR_PARAM_OUT_OF_RANGE;
-            if (across) HIPCHK(k_channel_colsum(s, X->dt(), (size_t)outer, (int)ch, (int)inner, X->ptr, Y->ptr));
+            // one tensor of many channels and few columns (a norm layer's weight gradient: 8192 rows of 768): the rows are
+            // dealt over workgroups as for a transposed mat-vec, partial sums added in a fixed order
+            const size_t wsb = (!X->half && outer == 1 && (inner + 63) / 64 < 256) ? k_gemv_workspace_bytes(true, (int)ch, (int)inner) : 0;
+            if (across && wsb) {
+                void* ws;
+                ERRCHK(workspace(wsb, &ws));
+                HIPCHK(k_gemv(s, F32, true, (int)ch, (int)inner, 1.f, X->ptr, nullptr, 0.f, (float*)Y->ptr, ws, wsb));
+            } else if (across) HIPCHK(k_channel_colsum(s, X->dt(), (size_t)outer, (int)ch, (int)inner, X->ptr, Y->ptr));
             else HIPCHK(k_channel_rowsum(s, X->dt(), (size_t)(outer * ch), (int)inner, X->ptr, Y->ptr, 1.0f));
             m_mem.touch((long)pl[5]);
             return 0;

@@ -381,7 +381,7 @@ def test_channel_sum_forms_vs_numpy(dev, half):
     rng = np.random.default_rng(83)
     cuda = dev.cuda
     tol = BF16_RTOL if half else 1e-6
-    for outer, ch, inner in [(3, 5, 48), (2, 1024, 70), (4, 7, 1), (1, 1, 300), (2, 130, 64)]:
+    for outer, ch, inner in [(3, 5, 48), (2, 1024, 70), (4, 7, 1), (1, 1, 300), (2, 130, 64), (1, 4096, 768), (1, 300, 70), (1, 1000, 36)]:
         n = outer * ch * inner
         x = bf16_round(rng.standard_normal((outer, ch, inner)).astype(np.float32))
         hx, ha, hw = dev.put(x, half), dev.zeros(outer * inner, half), dev.zeros(outer * ch, half)
