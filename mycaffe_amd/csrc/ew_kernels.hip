@@ -1077,7 +1077,17 @@ template <typename T> __global__ __launch_bounds__(256) void channel_rowsum_kern
     if (row >= rows) return;
     const T* xr = x + row * inner;
     float acc = 0.f;
-    for (int i = lane; i < inner; i += 64) acc += ld(xr, i);
+    if (sizeof(T) == 4 && inner % 4 == 0 && ((uintptr_t)x & 15) == 0) {
+        float a1 = 0.f;
+        for (int i = lane * 4; i < inner; i += 256) {
+            const float4 v = *(const float4*)((const float*)xr + i);
+            acc += v.x + v.y;
+            a1 += v.z + v.w;
+        }
+        acc += a1;
+    } else {
+        for (int i = lane; i < inner; i += 64) acc += ld(xr, i);
+    }
     acc = wave_sum(acc);
     if (lane == 0) st(y, row, acc * scale);
 }
@@ -1198,9 +1208,20 @@ __global__ __launch_bounds__(256) void channel_rowmax_kernel(size_t rows, int ch
     const T* xr = x + row * channels;
     float val = -3.402823466e+38f;
     int idx = 0;
-    for (int c = lane; c < channels; c += 64) {
-        const float v = ld(xr, c);
-        if (v > val) { val = v; idx = c; }
+    if (!IDX && sizeof(T) == 4 && channels % 4 == 0 && ((uintptr_t)x & 15) == 0) {
+        for (int c = lane * 4; c < channels; c += 256) {
+            const float4 v = *(const float4*)((const float*)xr + c);
+            // (a NaN never replaces the running maximum, as in the one-value loop)
+            if (v.x > val) val = v.x;
+            if (v.y > val) val = v.y;
+            if (v.z > val) val = v.z;
+            if (v.w > val) val = v.w;
+        }
+    } else {
+        for (int c = lane; c < channels; c += 64) {
+            const float v = ld(xr, c);
+            if (v > val) { val = v; idx = c; }
+        }
     }
     if (IDX) {
 #pragma unroll
