@@ -916,8 +916,8 @@ long Kernel::run(long fn, float* pf, long lf, MCH_LONGLONG* pl, long ll, float**
         ERRCHK(mem((long)pl[4], &A));
         ERRCHK(mem((long)pl[5], &X));
         ERRCHK(mem((long)pl[7], &Y));
-        // vectors in 16-bit storage: with a 16-bit matrix the call is the product with a one-column matrix (the bias
-        // gradient of an inner product kept in 16-bit storage); the reference reads such memory as floats (math.cu:2155-2185)
+        // vectors in 16-bit storage are taken with a 16-bit matrix only (the bias gradient of an inner product kept in 16-bit
+        // storage): they are widened into scratch memory below; the reference reads such memory as floats (math.cu:2155-2185)
         const bool all16 = A->half && X->half && Y->half;
         if ((X->half || Y->half) && !all16) return MCH_ERROR_MEMORY_HALF_TYPE_NOT_SUPPORTED;
         if (aOff < 0) aOff = 0;
